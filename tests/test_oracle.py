@@ -1,0 +1,252 @@
+"""Pins the CPU oracle: brute force on small inputs, closed forms, library routines and
+hand-worked examples.  None of these tests re-types the oracle's own formula."""
+
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from evox_amd import workloads
+from oracle import brute_force as bf
+from oracle import eager_restatement as er
+from tests.cases import as_np, edge_cases
+
+EDGE = edge_cases()
+IDS = [c[0] for c in EDGE]
+
+
+def same_float(a, b):
+    """Equal including inf signs and NaN positions."""
+    a, b = as_np(a), as_np(b)
+    return a.shape == b.shape and np.array_equal(a, b, equal_nan=True)
+
+
+# ---------------------------------------------------------------- dominance
+
+
+def dominance_pure_python(rows):
+    n = len(rows)
+    out = [[False] * n for _ in range(n)]
+    for i, j in itertools.product(range(n), range(n)):
+        le = all(a <= b for a, b in zip(rows[i], rows[j]))
+        lt = any(a < b for a, b in zip(rows[i], rows[j]))
+        out[i][j] = le and lt
+    return np.array(out, dtype=bool).reshape(n, n)
+
+
+@pytest.mark.parametrize("name,f,ks", EDGE, ids=IDS)
+def test_dominance_matches_pure_python_and_numpy(name, f, ks):
+    got = as_np(er.pareto_dominance(f, f))
+    assert np.array_equal(got, bf.dominates_matrix(as_np(f)))
+    if f.size(0) <= 65:
+        assert np.array_equal(got, dominance_pure_python(f.tolist()))
+
+
+@pytest.mark.parametrize("name,f,ks", EDGE, ids=IDS)
+def test_dominance_is_a_strict_partial_order(name, f, ks):
+    a = as_np(er.pareto_dominance(f, f))
+    assert not a.diagonal().any()  # irreflexive
+    assert not (a & a.T).any()  # antisymmetric
+    reach = (a.astype(np.int64) @ a.astype(np.int64)) > 0
+    assert not (reach & ~a).any()  # transitive
+    nan_rows = np.isnan(as_np(f)).any(axis=1)
+    assert not a[nan_rows].any() and not a[:, nan_rows].any()
+
+
+def test_dominance_density_uniform():
+    f = workloads.uniform_population(2000, 3, 0, seed=5)[0]
+    dens = as_np(er.pareto_dominance(f, f)).mean()
+    assert abs(dens - 0.125) < 0.01  # P(all three coordinates smaller) = 2^-3
+
+
+# --------------------------------------------------------------------- rank
+
+
+@pytest.mark.parametrize("name,f,ks", EDGE, ids=IDS)
+def test_rank_three_definitions_agree(name, f, ks):
+    r = as_np(er.ranks_by_peeling(f))
+    assert r.dtype == np.int32
+    assert np.array_equal(r, bf.rank_longest_chain(as_np(f)))
+    assert np.array_equal(r, bf.rank_deb(as_np(f)))
+
+
+def test_rank_closed_forms():
+    chain = torch.arange(9, dtype=torch.float32)[:, None].repeat(1, 3)
+    assert as_np(er.ranks_by_peeling(chain)).tolist() == list(range(9))
+    assert as_np(er.ranks_by_peeling(chain.flip(0))).tolist() == list(range(8, -1, -1))
+    assert as_np(er.ranks_by_peeling(torch.full((7, 4), 3.0))).tolist() == [0] * 7
+    # M = 1: rank is the dense rank of the value, ties share a rank
+    v = torch.tensor([3.0, 1.0, 2.0, 1.0, 5.0, 3.0, 2.0])[:, None]
+    assert as_np(er.ranks_by_peeling(v)).tolist() == [2, 0, 1, 0, 3, 2, 1]
+    # a mutually non-dominated anti-diagonal is one front
+    t = torch.arange(6, dtype=torch.float32)
+    assert as_np(er.ranks_by_peeling(torch.stack([t, 5 - t], 1))).tolist() == [0] * 6
+    # rows holding a NaN are isolated: rank 0, and they do not push anyone down
+    f = torch.tensor([[0.0, 0.0], [float("nan"), -1.0], [1.0, 1.0]])
+    assert as_np(er.ranks_by_peeling(f)).tolist() == [0, 0, 1]
+
+
+@pytest.mark.parametrize("permute", [False, True])
+def test_rank_layered_construction(permute):
+    """C2: layer l lies on f1 + f2 = l + 1, so its rank is at least... exactly l when every layer
+    has a point dominating each point of the next; checked here against the two independent
+    definitions and against the construction's own bound rank <= layer."""
+    w = workloads.c2(seed=0, permute=permute)
+    r = as_np(er.ranks_by_peeling(w.f))
+    assert np.array_equal(r, bf.rank_longest_chain(as_np(w.f)))
+    layer = np.round(as_np(w.f).sum(axis=1)).astype(np.int64) - 1
+    assert (r <= layer).all()
+    assert r.max() == 19  # 20 fronts, as BASELINE.md records for this generator
+
+
+def test_rank_c1_and_medium_random():
+    for f in (workloads.c1().f, workloads.uniform_population(700, 3, 0, seed=9)[0],
+              workloads.sphere_shell_population((512,), 3, 0.1, seed=1000)):
+        r = as_np(er.ranks_by_peeling(f))
+        assert np.array_equal(r, bf.rank_longest_chain(as_np(f)))
+    assert as_np(er.ranks_by_peeling(workloads.c1().f)).max() + 1 == 11  # F = 11
+
+
+def test_rank_batched_equals_per_population():
+    f = workloads.sphere_shell_population((6, 40), 3, 0.1, seed=3)
+    f[2] = torch.arange(40, dtype=torch.float32)[:, None].repeat(1, 3)  # one deep chain among shallow ones
+    got = er.ranks_by_peeling_batched(f)
+    for b in range(f.size(0)):
+        assert torch.equal(got[b], er.ranks_by_peeling(f[b]))
+
+
+# ------------------------------------------------------------------ lexsort
+
+
+def test_chained_argsort_is_numpy_lexsort():
+    g = torch.Generator("cpu").manual_seed(77)
+    for n in (1, 2, 17, 200):
+        k0 = torch.randint(0, 4, (n,), generator=g).float()
+        k1 = torch.randint(0, 3, (n,), generator=g).float()
+        k2 = torch.randint(0, 2, (n,), generator=g)
+        got = as_np(er.chained_stable_argsort([k0, k1, k2]))
+        assert np.array_equal(got, np.lexsort((as_np(k0), as_np(k1), as_np(k2))))
+    # NaN keys sort after every number, for x and for -x alike; signed zeros tie
+    x = torch.tensor([0.0, float("nan"), -0.0, 1.0, float("inf"), -float("inf"), 0.0])
+    assert as_np(er.chained_stable_argsort([x])).tolist() == [5, 0, 2, 6, 3, 4, 1]
+    assert as_np(er.chained_stable_argsort([-x])).tolist() == [4, 3, 0, 2, 6, 5, 1]
+    # column-wise form used by the crowding distance
+    c = torch.rand(50, 3, generator=g)
+    m = (torch.rand(50, generator=g) < 0.5).float()[:, None].expand(-1, 3)
+    got = as_np(er.chained_stable_argsort([c, m], dim=0))
+    for k in range(3):
+        assert np.array_equal(got[:, k], np.lexsort((as_np(c[:, k]), as_np(m[:, k]))))
+
+
+# ----------------------------------------------------------------- crowding
+
+
+def test_crowding_hand_worked():
+    inf = float("inf")
+    # five points on a line: interior gaps are 2/4 per objective
+    f = torch.tensor([[0.0, 4.0], [1.0, 3.0], [2.0, 2.0], [3.0, 1.0], [4.0, 0.0]])
+    assert as_np(er.crowding(f, None)).tolist() == [inf, 1.0, 1.0, 1.0, inf]
+    # uneven spacing: f1 = 0,1,4,9,10 and f2 reversed
+    f = torch.tensor([[0.0, 10.0], [1.0, 9.0], [4.0, 6.0], [9.0, 1.0], [10.0, 0.0]])
+    want = [inf, 0.4 + 0.4, 0.8 + 0.8, 0.6 + 0.6, inf]
+    np.testing.assert_allclose(as_np(er.crowding(f, None)), want, rtol=1e-6)
+    # mask: rows 1..3 only -> 1 and 3 are boundary rows, row 2 spans the whole range
+    mask = torch.tensor([False, True, True, True, False])
+    assert as_np(er.crowding(f, mask)).tolist() == [-inf, inf, 2.0, inf, -inf]
+    # a row that is extreme in one objective only is still +inf overall
+    f = torch.tensor([[0.0, 5.0], [1.0, 1.0], [2.0, 9.0], [3.0, 4.0]])
+    d = as_np(er.crowding(f, None))
+    assert d[0] == inf and d[3] == inf and d[1] == inf and d[2] == inf  # 1 is min of f2, 2 is max of f2
+    # ties: equal costs keep index order, lowest index is the low boundary, highest the high one
+    f = torch.tensor([[1.0], [1.0], [2.0], [3.0], [3.0]])
+    assert as_np(er.crowding(f, None)).tolist() == [inf, 0.5, 1.0, 0.5, inf]
+    # zero range: interior rows are 0/0
+    f = torch.tensor([[2.0, 0.0], [2.0, 1.0], [2.0, 2.0], [2.0, 3.0]])
+    d = as_np(er.crowding(f, None))
+    assert d[0] == inf and d[3] == inf and np.isnan(d[1]) and np.isnan(d[2])
+    # one or two valid rows are all boundary
+    f = torch.rand(6, 3, generator=torch.Generator("cpu").manual_seed(1))
+    assert as_np(er.crowding(f, torch.tensor([0, 0, 1, 0, 0, 0], dtype=torch.bool))).tolist() == [-inf, -inf, inf, -inf, -inf, -inf]
+    assert as_np(er.crowding(f, torch.tensor([1, 0, 0, 0, 0, 1], dtype=torch.bool))).tolist() == [inf, -inf, -inf, -inf, -inf, inf]
+    assert as_np(er.crowding(f, torch.zeros(6, dtype=torch.bool))).tolist() == [-inf] * 6
+
+
+def _masks_for(f, seed):
+    n = f.size(0)
+    g = torch.Generator("cpu").manual_seed(seed)
+    masks = [None, torch.ones(n, dtype=torch.bool), torch.rand(n, generator=g) < 0.5, torch.rand(n, generator=g) < 0.15]
+    one = torch.zeros(n, dtype=torch.bool)
+    one[n // 2] = True
+    masks.append(one)
+    return masks
+
+
+@pytest.mark.parametrize("name,f,ks", EDGE, ids=IDS)
+def test_crowding_matches_brute_force(name, f, ks):
+    for mask in _masks_for(f, 11):
+        got = er.crowding(f, mask)
+        assert got.dtype == torch.float32
+        want = bf.crowding_brute(as_np(f), None if mask is None else as_np(mask))
+        assert same_float(got, want), (name, mask)
+
+
+def test_crowding_invariants_on_a_front():
+    f = workloads.sphere_shell_population((300,), 3, 0.1, seed=2)
+    rank = er.ranks_by_peeling(f)
+    mask = rank == 0
+    d = as_np(er.crowding(f, mask))
+    m = as_np(mask)
+    assert np.isneginf(d[~m]).all()
+    assert (d[m] >= 0).all()
+    fm = as_np(f)[m]
+    extreme = np.zeros(m.sum(), dtype=bool)
+    for k in range(3):
+        extreme |= fm[:, k] == fm[:, k].min()
+        extreme |= fm[:, k] == fm[:, k].max()
+    assert np.isposinf(d[m][extreme]).all()  # no ties in this population: extremes are exactly the +inf rows
+    assert np.isfinite(d[m][~extreme]).all()
+    # finite part is bounded by M (each objective contributes at most the whole range once)
+    assert d[m][~extreme].max() <= 3.0
+
+
+# ---------------------------------------------------------------- selection
+
+
+@pytest.mark.parametrize("name,f,ks", EDGE, ids=IDS)
+def test_selection_matches_brute_force(name, f, ks):
+    x = torch.arange(f.size(0), dtype=torch.float32)[:, None].repeat(1, 2)
+    for k in ks:
+        (xs, fs, rs, ds), rank, dist, order = er.environmental_selection(x, f, k, return_all=True)
+        b_order, b_rank, b_dist = bf.selection_brute(as_np(f), k)
+        assert np.array_equal(as_np(rank), b_rank)
+        assert same_float(dist, b_dist)
+        assert np.array_equal(as_np(order), b_order)
+        assert same_float(fs, as_np(f)[b_order]) and np.array_equal(as_np(xs)[:, 0].astype(np.int64), b_order)
+        assert np.array_equal(as_np(rs), b_rank[b_order]) and same_float(ds, b_dist[b_order])
+
+
+def test_selection_structure_c1_c2():
+    for w in (workloads.c1(), workloads.c2(), workloads.c2(permute=True)):
+        x = w.x if w.x is not None else w.f
+        _, rank, dist, order = er.environmental_selection(x, w.f, w.topk, return_all=True)
+        rank, dist, order = as_np(rank), as_np(dist), as_np(order)
+        b_order, b_rank, b_dist = bf.selection_brute(as_np(w.f), w.topk)
+        assert np.array_equal(rank, b_rank) and same_float(dist, b_dist) and np.array_equal(order, b_order)
+        sel_rank = rank[order]
+        assert (np.diff(sel_rank) >= 0).all()
+        worst = sel_rank[-1]
+        better = np.flatnonzero(rank < worst)
+        assert np.array_equal(order[: better.size], better[np.argsort(rank[better], kind="stable")])
+        tail = order[better.size:]
+        assert (rank[tail] == worst).all()
+        assert (dist[tail][1:] <= dist[tail][:-1]).all() or np.isnan(dist[tail]).any()
+        assert np.isneginf(dist[rank != worst]).all()
+
+
+def test_selection_errors():
+    f = torch.rand(5, 2)
+    with pytest.raises(RuntimeError):
+        er.environmental_selection(f, f, 6)
+    with pytest.raises(IndexError):
+        er.environmental_selection(f, f, 0)
