@@ -1,0 +1,12 @@
+"""MI355X-native multi-objective environmental selection with EvoX's operator signatures.
+
+    from evox_amd.operators.selection import non_dominate_rank, crowding_distance, nd_environmental_selection
+
+The package holds only this hot path: HIP kernels for gfx950 behind a C ABI (``csrc/``,
+``include/evox_hip.h``), the ``evox_amd::`` torch custom operators and the three Python functions.
+"""
+
+__all__ = ["operators", "ops", "runtime", "workloads", "install_into_evox"]
+
+from . import operators, ops, runtime, workloads
+from .compat import install_into_evox

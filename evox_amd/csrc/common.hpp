@@ -1,0 +1,42 @@
+// Shared definitions for the gfx950 selection kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace evx {
+
+constexpr int kWave = 64;
+
+// Error codes returned through the C ABI (0 = ok, positive = hipError_t passed through).
+constexpr int kErrBadArg = -1;
+constexpr int kErrWorkspace = -2;
+constexpr int kErrBarrierTimeout = -3;
+
+__host__ __device__ inline int64_t round_up(int64_t v, int64_t q) { return (v + q - 1) / q * q; }
+
+// Order-preserving map float -> uint32 with torch's sort conventions: -0.0 and +0.0 share a key,
+// every NaN (either sign) maps to the largest key so that it sorts after +inf.
+__device__ inline uint32_t ordered_key(float v) {
+  uint32_t u = __float_as_uint(v);
+  if (v != v) return 0xFFFFFFFFu;
+  if (v == 0.0f) u = 0u;
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Device control block shared by the peel / crowding / selection kernels of one call.
+struct Ctrl {
+  int err;          // 0, or kErrBarrierTimeout when a bounded grid-barrier wait ran out
+  int nfronts;      // number of fronts peeled so far (ranks 0 .. nfronts-1 are final)
+  int worst;        // rank of the front that contains the stop_count-th row
+  int worst_start;  // rows ranked strictly better than `worst`
+  int nv;           // size of front `worst`
+  int need;         // rows to take from front `worst` (stop_count - worst_start)
+  int passes;       // sweep passes executed
+  int reserved[9];
+  unsigned release;  // grid barrier: generation published by block 0
+  unsigned pad[15];
+  unsigned arrive[1];  // grid barrier: one slot per block (allocated to the grid size)
+};
+
+}  // namespace evx

@@ -1,0 +1,154 @@
+// Pairwise Pareto dominance -> bit matrix.
+//
+// Reference semantics (src/evox/operators/selection/non_dominate.py:6-26):
+//   A[i, j] = all_k(x[i,k] <= x[j,k]) and any_k(x[i,k] < x[j,k])      (any NaN makes the pair False)
+//
+// Layout produced here ("dominated-by" rows): dom[j * wstride + w] holds, in bit b, A[64*w + b, j].
+// Row j therefore lists the dominators of j; its popcount is the domination count of
+// non_dominate.py:188 and one peel pass is popcount(row & front) (non_dominate.py:29-59).
+//
+// Work split: lane = j (fitness of 64 rows held in VGPRs), loop over i with x[i, :] fetched by
+// scalar loads (the index is wave-uniform), so every `<=` is one v_cmp_le_f32 with an SGPR operand
+// whose result is a 64-lane mask in an SGPR pair; the per-objective masks are ANDed on the scalar
+// unit.  "any strictly less" is replaced by one 64-bit compare: with key(i) = sum_k ordered_key(x[i,k])
+// and all_k(x[i,k] <= x[j,k]) already true (which rules out NaN on both sides), the rows differ in
+// some objective exactly when key(i) != key(j), because the per-objective keys are ordered the same
+// way as the floats and sum without overflow.  The lane mask is then shifted into the lane's own
+// 32-bit accumulator with v_addc_co_u32 (acc = acc + acc + carry), which performs the transpose from
+// "mask over j" to "word over i" at one VALU instruction per 64 pairs.
+#pragma once
+
+#include "common.hpp"
+
+namespace evx {
+
+// Fitness in structure-of-arrays form, padded with NaN to a multiple of 128 rows, plus the 64-bit row key.
+struct Prepared {
+  const float* xs;       // [m][npad]
+  const uint64_t* key;   // [npad]
+  int n;
+  int npad;
+};
+
+// One kernel turns the caller's strided (n, m) fitness into Prepared and clears the small state
+// arrays that later kernels accumulate into.
+__global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ f, int64_t stride_row, int64_t stride_col,
+                                                      int n, int m, int npad, float* __restrict__ xs,
+                                                      uint64_t* __restrict__ key, uint32_t* __restrict__ zero_words,
+                                                      int64_t n_zero_words) {
+  const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = tid; i < npad; i += nthreads) {
+    uint64_t s = 0;
+    for (int k = 0; k < m; ++k) {
+      const float v = i < n ? f[i * stride_row + k * stride_col] : __uint_as_float(0x7FC00000u);
+      xs[(int64_t)k * npad + i] = v;
+      s += ordered_key(v);
+    }
+    key[i] = s;
+  }
+  for (int64_t i = tid; i < n_zero_words; i += nthreads) zero_words[i] = 0u;
+}
+
+// acc = (acc << 1) | bit, with the bit taken from a 64-lane mask: one v_addc_co_u32.
+__device__ inline uint32_t shift_in(uint32_t acc, uint64_t mask) {
+  uint32_t r;
+  uint64_t carry_out;
+  asm("v_addc_co_u32_e64 %0, %1, %2, %2, %3" : "=v"(r), "=s"(carry_out) : "v"(acc), "s"(mask));
+  return r;
+}
+
+enum DomVariant { kDomKey64 = 0, kDomTwoCompares = 1 };
+
+// grid.x = ceil(npad / 256) blocks of four 64-row groups, grid.y = ceil(nwords / IW) column tiles.
+template <int M, int IW, int VARIANT>
+__global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
+                                                        uint64_t* __restrict__ dom, int n, int npad, int64_t wstride,
+                                                        int nwords) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int j = (blockIdx.x * 4 + wave) * 64 + lane;
+  if (j - lane >= npad) return;  // whole wave past the padded population
+  const int w0 = blockIdx.y * IW;
+  float xj[M];
+#pragma unroll
+  for (int k = 0; k < M; ++k) xj[k] = xs[(int64_t)k * npad + j];
+  const uint64_t kj = key[j];
+  uint64_t* __restrict__ out = dom + (int64_t)j * wstride;
+  const int wend = (w0 + IW < nwords) ? w0 + IW : nwords;  // nwords = npad / 64 is even, and so is IW
+#pragma unroll 1
+  for (int w = w0; w < wend; w += 2) {
+    uint32_t half[4];
+#pragma unroll
+    for (int h = 3; h >= 0; --h) {
+      const int ib = w * 64 + h * 32;
+      uint32_t acc = 0;
+#pragma unroll
+      for (int t = 31; t >= 0; --t) {
+        const int i = ib + t;
+        // each comparison is balloted on its own so that it stays a v_cmp writing an SGPR pair and the
+        // combination runs on the scalar unit
+        uint64_t c = ~0ull;
+#pragma unroll
+        for (int k = 0; k < M; ++k) c &= __builtin_amdgcn_ballot_w64(xs[(int64_t)k * npad + i] <= xj[k]);
+        if (VARIANT == kDomKey64) {
+          c &= __builtin_amdgcn_ballot_w64(key[i] != kj);
+        } else {
+          uint64_t lt = 0ull;
+#pragma unroll
+          for (int k = 0; k < M; ++k) lt |= __builtin_amdgcn_ballot_w64(xs[(int64_t)k * npad + i] < xj[k]);
+          c &= lt;
+        }
+        acc = shift_in(acc, c);
+      }
+      half[h] = acc;
+    }
+    if (j < n) {
+      // two words = one 16-byte store; rows are 128-byte aligned and w is even.  Bits of padding rows
+      // (i >= n) are zero because their fitness is NaN.
+      const uint64_t lo = ((uint64_t)half[1] << 32) | half[0];
+      const uint64_t hi = ((uint64_t)half[3] << 32) | half[2];
+      *reinterpret_cast<ulonglong2*>(out + w) = make_ulonglong2(lo, hi);
+    }
+  }
+}
+
+// Any number of objectives (used above 8): same scheme, with the lane's own fitness re-read from
+// memory for every objective instead of living in registers.
+template <int IW>
+__global__ __launch_bounds__(256) void dominance_any_m_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
+                                                              uint64_t* __restrict__ dom, int n, int npad, int64_t wstride,
+                                                              int nwords, int m) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int j = (blockIdx.x * 4 + wave) * 64 + lane;
+  if (j - lane >= npad) return;
+  const int w0 = blockIdx.y * IW;
+  const uint64_t kj = key[j];
+  uint64_t* __restrict__ out = dom + (int64_t)j * wstride;
+  const int wend = (w0 + IW < nwords) ? w0 + IW : nwords;
+#pragma unroll 1
+  for (int w = w0; w < wend; w += 2) {
+    uint32_t half[4];
+#pragma unroll
+    for (int h = 3; h >= 0; --h) {
+      const int ib = w * 64 + h * 32;
+      uint32_t acc = 0;
+#pragma unroll 4
+      for (int t = 31; t >= 0; --t) {
+        const int i = ib + t;
+        uint64_t c = __builtin_amdgcn_ballot_w64(key[i] != kj);
+        for (int k = 0; k < m; ++k) c &= __builtin_amdgcn_ballot_w64(xs[(int64_t)k * npad + i] <= xs[(int64_t)k * npad + j]);
+        acc = shift_in(acc, c);
+      }
+      half[h] = acc;
+    }
+    if (j < n) {
+      const uint64_t lo = ((uint64_t)half[1] << 32) | half[0];
+      const uint64_t hi = ((uint64_t)half[3] << 32) | half[2];
+      *reinterpret_cast<ulonglong2*>(out + w) = make_ulonglong2(lo, hi);
+    }
+  }
+}
+
+}  // namespace evx

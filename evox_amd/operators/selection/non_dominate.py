@@ -1,0 +1,52 @@
+"""Drop-in replacements for the three selection operators of
+``evox.operators.selection.non_dominate`` (src/evox/operators/selection/non_dominate.py),
+with the same names, positional arguments, return arity, dtypes and devices.  The work is done by
+hand-written gfx950 kernels reached through the ``evox_amd::`` custom operators; there is no
+PyTorch or CPU implementation behind them.
+"""
+
+from typing import Optional, Tuple
+
+import torch
+
+from ... import ops
+
+
+def non_dominate_rank(x: torch.Tensor) -> torch.Tensor:
+    """Non-domination rank of every row of ``x`` (minimisation).
+
+    Same contract as the reference's ``non_dominate_rank`` (non_dominate.py:172-195):
+    ``x`` is ``(N, M)``; the result is ``int32 (N,)`` on ``x.device``; rank 0 is the Pareto front,
+    rank r + 1 the front of what remains after removing ranks 0..r.  Rows holding a NaN neither
+    dominate nor are dominated (rank 0); identical rows do not dominate each other.
+    """
+    return ops.nd_rank(x)
+
+
+def crowding_distance(costs: torch.Tensor, mask: Optional[torch.Tensor]) -> torch.Tensor:
+    """Crowding distance of the rows selected by ``mask`` (all rows when ``mask`` is ``None``).
+
+    Same contract as the reference's ``crowding_distance`` (non_dominate.py:198-231): per objective
+    the selected rows are sorted by (cost, row index) with NaN last; the first and last row of any
+    objective get ``+inf``; every other selected row gets the sum over objectives of
+    ``(next - previous) / (last - first)``; unselected rows get ``-inf``.  The result has torch's
+    default float dtype, and, as in the reference (its scatter at :224-225), ``costs`` must have that
+    dtype too.
+    """
+    if costs.dtype != torch.get_default_dtype():
+        raise RuntimeError(
+            f"crowding_distance: expected costs.dtype to be the default dtype {torch.get_default_dtype()}, got {costs.dtype}"
+        )
+    return ops.crowding(costs, mask)
+
+
+def nd_environmental_selection(x: torch.Tensor, f: torch.Tensor, topk: int) -> Tuple[torch.Tensor, ...]:
+    """NSGA-II environmental selection of ``topk`` rows.
+
+    Same contract as the reference's ``nd_environmental_selection`` (non_dominate.py:234-254):
+    returns ``(x[order], f[order], rank[order], crowding_dis[order])`` where ``order`` sorts by rank
+    ascending, then by the crowding distance within the last admitted front descending (NaN last),
+    then by row index; the distance of rows in better fronts is ``-inf``.  ``topk > N`` raises
+    ``RuntimeError`` and ``topk < 1`` raises ``IndexError`` as ``torch.topk`` / indexing do there.
+    """
+    return ops.nd_select(x, f, int(topk))

@@ -1,0 +1,190 @@
+"""torch.library custom operators backed by the HIP kernels.
+
+The reference wraps its peeling loop in a custom operator with a fake (shape-only) implementation
+and vmap rules for two nesting levels (src/evox/utils/op_register.py:54-132, used at
+src/evox/operators/selection/non_dominate.py:151-169).  The operators here follow the same pattern
+in a namespace of their own (``evox_amd::``): each has a fake implementation so that it traces
+under ``torch.compile(fullgraph=True)``, and a vmap rule that moves the mapped dimension to the
+front; the operators themselves accept any number of leading batch dimensions, so nested vmaps
+need no extra registrations.
+"""
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib, runtime
+
+
+def _as_f32(t: torch.Tensor, what: str) -> torch.Tensor:
+    if t.dtype == torch.float32:
+        return t
+    if t.dtype in (torch.float16, torch.bfloat16):
+        return t.float()  # exact and order preserving
+    raise TypeError(f"{what} must be float32 (float16 / bfloat16 are widened exactly); got {t.dtype}")
+
+
+def _rank_one(f: torch.Tensor, out: torch.Tensor) -> None:
+    n, m = f.shape
+    ws = runtime.workspace(n, m, f.device)
+    stream = runtime.stream_handle(f.device)
+    _lib.call("evox_hip_non_dominate_rank", f.data_ptr(), n, m, f.stride(0), f.stride(1), out.data_ptr(), ws.data_ptr(),
+              ws.numel(), stream)
+    runtime.note_call(ws, stream)
+
+
+@torch.library.custom_op("evox_amd::nd_rank", mutates_args=())
+def nd_rank(f: torch.Tensor) -> torch.Tensor:
+    """(..., N, M) fitness -> (..., N) int32 non-domination rank."""
+    runtime.require_gpu_tensor(f, "fitness")
+    if f.dim() < 2:
+        raise ValueError("fitness must have shape (..., N, M)")
+    f32 = _as_f32(f, "fitness")
+    n, m = f32.shape[-2:]
+    out = torch.empty(f32.shape[:-1], dtype=torch.int32, device=f.device)
+    if n == 0 or out.numel() == 0:
+        return out
+    if m == 0:
+        return out.zero_()
+    with torch.cuda.device(f.device):
+        flat_f = f32.reshape(-1, n, m)
+        flat_out = out.view(-1, n)
+        for b in range(flat_f.size(0)):
+            _rank_one(flat_f[b], flat_out[b])
+    return out
+
+
+@nd_rank.register_fake
+def _(f):
+    return f.new_empty(f.shape[:-1], dtype=torch.int32)
+
+
+def _nd_rank_vmap(info, in_dims, f):
+    return nd_rank(f.movedim(in_dims[0], 0)), 0
+
+
+torch.library.register_vmap(nd_rank, _nd_rank_vmap)
+
+
+@torch.library.custom_op("evox_amd::crowding", mutates_args=())
+def crowding(costs: torch.Tensor, mask: Optional[torch.Tensor]) -> torch.Tensor:
+    """(..., N, M) costs, optional (..., N) bool mask -> (..., N) float32 crowding distance."""
+    runtime.require_gpu_tensor(costs, "costs")
+    if costs.dim() < 2:
+        raise ValueError("costs must have shape (..., N, M)")
+    c32 = _as_f32(costs, "costs")
+    n, m = c32.shape[-2:]
+    out = torch.empty(c32.shape[:-1], dtype=torch.float32, device=costs.device)
+    if mask is not None:
+        runtime.require_gpu_tensor(mask, "mask")
+        if mask.dtype != torch.bool:
+            raise TypeError(f"mask must be a bool tensor; got {mask.dtype}")
+        if mask.shape != out.shape:
+            raise ValueError(f"mask shape {tuple(mask.shape)} does not match costs {tuple(costs.shape)}")
+    if n == 0 or out.numel() == 0:
+        return out
+    if m == 0:
+        raise ValueError("costs must have at least one objective")
+    with torch.cuda.device(costs.device):
+        flat_c = c32.reshape(-1, n, m)
+        flat_out = out.view(-1, n)
+        flat_mask = None if mask is None else mask.reshape(-1, n)
+        stream = runtime.stream_handle(costs.device)
+        ws = runtime.workspace(n, m, costs.device)
+        for b in range(flat_c.size(0)):
+            c = flat_c[b]
+            mk = None if flat_mask is None else flat_mask[b]
+            _lib.call("evox_hip_crowding_distance", c.data_ptr(), n, m, c.stride(0), c.stride(1),
+                      None if mk is None else mk.data_ptr(), 0 if mk is None else mk.stride(0), flat_out[b].data_ptr(),
+                      ws.data_ptr(), ws.numel(), stream)
+        runtime.note_call(ws, stream)
+    return out
+
+
+@crowding.register_fake
+def _(costs, mask):
+    return costs.new_empty(costs.shape[:-1], dtype=torch.float32)
+
+
+def _crowding_vmap(info, in_dims, costs, mask):
+    cd, md = in_dims
+    costs = costs.movedim(cd, 0) if cd is not None else costs.unsqueeze(0).expand(info.batch_size, *costs.shape)
+    if mask is not None:
+        mask = mask.movedim(md, 0) if md is not None else mask.unsqueeze(0).expand(info.batch_size, *mask.shape)
+    return crowding(costs, mask), 0
+
+
+torch.library.register_vmap(crowding, _crowding_vmap)
+
+
+@torch.library.custom_op("evox_amd::nd_select", mutates_args=())
+def nd_select(x: torch.Tensor, f: torch.Tensor, topk: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """x (..., N, *D), f (..., N, M), topk -> (x, f, rank, crowding distance) of the topk survivors."""
+    runtime.require_gpu_tensor(f, "fitness")
+    runtime.require_gpu_tensor(x, "decision vectors")
+    if f.dim() < 2:
+        raise ValueError("fitness must have shape (..., N, M)")
+    bd = f.dim() - 2
+    n, m = f.shape[-2:]
+    if x.dim() < bd + 1 or x.shape[: bd + 1] != f.shape[: bd + 1]:
+        raise ValueError(f"decision vectors {tuple(x.shape)} and fitness {tuple(f.shape)} disagree on the leading dimensions")
+    if x.device != f.device:
+        raise RuntimeError("decision vectors and fitness are on different devices")
+    if topk > n:
+        raise RuntimeError(f"selected index k out of range: topk={topk} exceeds the population size {n}")
+    if topk < 1:
+        raise IndexError(f"topk must be at least 1; got {topk}")
+    if m == 0:
+        raise ValueError("fitness must have at least one objective")
+    f32 = _as_f32(f, "fitness")
+    batch = f.shape[:bd]
+    tail = x.shape[bd + 1:]
+    out_x = torch.empty(*batch, topk, *tail, dtype=x.dtype, device=x.device)
+    out_f = torch.empty(*batch, topk, m, dtype=torch.float32, device=f.device)
+    out_rank = torch.empty(*batch, topk, dtype=torch.int32, device=f.device)
+    out_dist = torch.empty(*batch, topk, dtype=torch.float32, device=f.device)
+    if out_rank.numel() == 0:
+        return out_x, out_f.to(f.dtype), out_rank, out_dist
+    with torch.cuda.device(f.device):
+        flat_f = f32.reshape(-1, n, m)
+        flat_x = x.reshape(flat_f.size(0), n, -1)
+        if flat_x.stride(-1) != 1 and flat_x.size(-1) > 1:
+            flat_x = flat_x.contiguous()
+        row_bytes = flat_x.size(-1) * flat_x.element_size()
+        fo_x = out_x.view(flat_f.size(0), topk, -1)
+        fo_f = out_f.view(-1, topk, m)
+        fo_r = out_rank.view(-1, topk)
+        fo_d = out_dist.view(-1, topk)
+        stream = runtime.stream_handle(f.device)
+        ws = runtime.workspace(n, m, f.device)
+        for b in range(flat_f.size(0)):
+            fb, xb = flat_f[b], flat_x[b]
+            has_x = row_bytes > 0
+            _lib.call("evox_hip_nd_environmental_selection", xb.data_ptr() if has_x else None, row_bytes,
+                      xb.stride(0) * xb.element_size(), fb.data_ptr(), n, m, fb.stride(0), fb.stride(1), topk,
+                      fo_x[b].data_ptr() if has_x else None, fo_f[b].data_ptr(), fo_r[b].data_ptr(), fo_d[b].data_ptr(),
+                      None, ws.data_ptr(), ws.numel(), stream)
+        runtime.note_call(ws, stream)
+    return out_x, out_f.to(f.dtype), out_rank, out_dist
+
+
+@nd_select.register_fake
+def _(x, f, topk):
+    bd = f.dim() - 2
+    batch = f.shape[:bd]
+    return (
+        x.new_empty(*batch, topk, *x.shape[bd + 1:]),
+        f.new_empty(*batch, topk, f.shape[-1]),
+        f.new_empty(*batch, topk, dtype=torch.int32),
+        f.new_empty(*batch, topk, dtype=torch.float32),
+    )
+
+
+def _nd_select_vmap(info, in_dims, x, f, topk):
+    xd, fd, _ = in_dims
+    x = x.movedim(xd, 0) if xd is not None else x.unsqueeze(0).expand(info.batch_size, *x.shape)
+    f = f.movedim(fd, 0) if fd is not None else f.unsqueeze(0).expand(info.batch_size, *f.shape)
+    return nd_select(x, f, topk), (0, 0, 0, 0)
+
+
+torch.library.register_vmap(nd_select, _nd_select_vmap)

@@ -1,0 +1,96 @@
+"""Host-side plumbing between torch tensors and the C ABI: workspaces, streams, status."""
+
+import ctypes
+import os
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+_last: Optional[Tuple[torch.Tensor, int]] = None  # (workspace, stream handle) of the latest call
+
+CHECK_STATUS = os.environ.get("EVOX_AMD_CHECK_STATUS", "0") not in ("", "0")
+
+
+def require_gpu_tensor(t: torch.Tensor, what: str) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{what} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"{what} is on {t.device}: evox_amd runs on an AMD GPU only (HIP kernels, no CPU fallback); "
+            "move the tensors to the 'cuda' device"
+        )
+
+
+def stream_handle(device: torch.device) -> int:
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def workspace(n: int, m: int, device: torch.device) -> torch.Tensor:
+    """A uint8 tensor of at least evox_hip_workspace_bytes(n, m) bytes, cached per (device, stream):
+    calls on one stream are ordered, so they can share it."""
+    need = int(_lib.lib().evox_hip_workspace_bytes(n, m))
+    if need == 0:
+        raise ValueError(f"unsupported population shape n={n}, m={m}")
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_handle(device))
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        _workspaces.pop(key, None)
+        ws = None
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        assert ws.data_ptr() % 256 == 0
+        _workspaces[key] = ws
+    return ws
+
+
+def release_workspaces() -> None:
+    _workspaces.clear()
+
+
+def note_call(ws: torch.Tensor, stream: int) -> None:
+    global _last
+    _last = (ws, stream)
+    if CHECK_STATUS:
+        last_status()
+
+
+def last_status() -> dict:
+    """Waits for the latest call and returns its control block; raises if the device reported an error."""
+    if _last is None:
+        return {}
+    ws, stream = _last
+    out = (ctypes.c_int32 * 8)()
+    code = _lib.lib().evox_hip_read_status(ws.data_ptr(), stream, out)
+    if code != 0:
+        raise _lib.EvoxHipError("evox_hip_read_status", code)
+    keys = ("error", "fronts", "worst_rank", "better_rows", "last_front_size", "taken_from_last", "passes")
+    return dict(zip(keys, list(out)[:7]))
+
+
+def set_option(name: str, value: int) -> None:
+    _lib.call("evox_hip_set_option", name.encode(), int(value))
+
+
+def workspace_views(ws: torch.Tensor, n: int, m: int) -> dict:
+    """Typed views of the workspace regions (for tests and tools)."""
+    out = (ctypes.c_int64 * 10)()
+    _lib.call("evox_hip_workspace_layout", n, m, out)
+    dom_off, wstride, nwords, count, rank, dist, perm, fstart, order, ctrl = list(out)
+
+    def view(off, count_, dtype):
+        size = torch.empty((), dtype=dtype).element_size()
+        return ws[off: off + count_ * size].view(dtype)
+
+    return {
+        "dom": view(dom_off, n * wstride, torch.int64).view(n, wstride),
+        "nwords": nwords,
+        "count": view(count, n, torch.int32),
+        "rank": view(rank, n, torch.int32),
+        "dist": view(dist, n, torch.float32),
+        "perm": view(perm, n, torch.int32),
+        "fstart": view(fstart, n + 2, torch.int32),
+        "order": view(order, n, torch.int32),
+        "ctrl": view(ctrl, 16, torch.int32),
+    }

@@ -1,0 +1,109 @@
+/* C ABI of libevox_hip.so: MI355X (gfx950) kernels for EvoX's multi-objective environmental
+ * selection.  Plain pointers and sizes only; every pointer is DEVICE memory unless said otherwise.
+ *
+ * Conventions
+ *   - Return value: 0 on success, a negative library code (EVOX_HIP_E_*) or a positive hipError_t.
+ *     No exceptions cross the boundary and nothing aborts.
+ *   - The caller owns every buffer, including the workspace; the library allocates no device memory
+ *     and synchronises only in evox_hip_read_status().  All work is enqueued on `stream`
+ *     (a hipStream_t passed as void*).
+ *   - Fitness `f` is float32, addressed as f[i * stride_row + k * stride_col] (strides in elements),
+ *     minimisation, n rows (individuals) by m columns (objectives).
+ *   - The workspace must hold evox_hip_workspace_bytes(n, m) bytes, 256-byte aligned.  Calls that
+ *     share a workspace must be ordered on one stream.
+ */
+#ifndef EVOX_HIP_H
+#define EVOX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EVOX_HIP_ABI_VERSION 1
+
+#define EVOX_HIP_E_BAD_ARG (-1)         /* null pointer, n < 1, m < 1, topk outside [1, n], ... */
+#define EVOX_HIP_E_WORKSPACE (-2)       /* workspace too small or misaligned */
+#define EVOX_HIP_E_BARRIER_TIMEOUT (-3) /* reported by evox_hip_read_status(): a bounded device-side wait ran out */
+
+int evox_hip_abi_version(void);
+
+/* Bytes of workspace needed by every entry point below for an (n, m) population.  0 if the
+ * arguments are invalid. */
+size_t evox_hip_workspace_bytes(int64_t n, int64_t m);
+
+/* rank_out[j] (int32, n entries) = non-domination rank of row j.
+ * Replaces evox.operators.selection.non_dominate_rank
+ * (src/evox/operators/selection/non_dominate.py:172-195, with dominate_relation :6-26,
+ * the column sum :188 and the peeling loop :29-59, :161-169). */
+int evox_hip_non_dominate_rank(const float* f, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col,
+                               int32_t* rank_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* dist_out[j] (float32, n entries) = crowding distance of row j among the rows with mask[j] != 0,
+ * -inf for the others.  `mask` is a byte per row at mask[j * mask_stride]; NULL selects every row.
+ * Replaces evox.operators.selection.crowding_distance
+ * (src/evox/operators/selection/non_dominate.py:198-231; ordering rules of
+ * src/evox/utils/jit_fix_operator.py:246-252). */
+int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col,
+                               const uint8_t* mask, int64_t mask_stride, float* dist_out, void* workspace,
+                               size_t workspace_bytes, void* stream);
+
+/* NSGA-II survivor selection: ranks f, takes the topk best rows by (rank ascending, crowding
+ * distance within the last admitted front descending, row index ascending) and gathers them.
+ *   x            decision vectors as raw bytes, row i at x + i * x_row_stride_bytes, x_row_bytes each
+ *                (may be NULL together with out_x when only f / rank / distance are wanted)
+ *   out_x        topk rows of x_row_bytes, contiguous
+ *   out_f        (topk, m) float32 contiguous
+ *   out_rank     topk int32
+ *   out_dist     topk float32 (crowding distance; -inf for rows of better fronts than the last one)
+ *   out_order    optional (may be NULL): the topk selected row indices, int32
+ * Replaces evox.operators.selection.nd_environmental_selection
+ * (src/evox/operators/selection/non_dominate.py:234-254). */
+int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes, const float* f,
+                                        int64_t n, int64_t m, int64_t stride_row, int64_t stride_col, int64_t topk,
+                                        void* out_x, float* out_f, int32_t* out_rank, float* out_dist,
+                                        int32_t* out_order, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- stages of the calls above, exposed so that each kernel can be tested and timed alone.
+ * They operate on the state left in the workspace by the previous stage, in this order:
+ *   dominance -> count -> peel -> (crowding -> order -> gather).                                   */
+
+/* Fitness -> structure-of-arrays copy + row keys, clears the small state, then the pairwise
+ * dominance bit matrix (non_dominate.py:6-26).  variant 0 = production kernel, 1 = check kernel that
+ * evaluates both `<=` and `<` per objective as the reference does. */
+int evox_hip_stage_dominance(const float* f, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col, int variant,
+                             void* workspace, size_t workspace_bytes, void* stream);
+/* Domination counts by row popcount (non_dominate.py:188) and front 0 (:192). */
+int evox_hip_stage_count(int64_t n, int64_t m, void* workspace, size_t workspace_bytes, void* stream);
+/* Front peeling (non_dominate.py:29-59, :161-169) until stop_count rows are ranked (stop_count = n
+ * ranks every row).  rank_out may be NULL (ranks stay in the workspace). */
+int evox_hip_stage_peel(int64_t n, int64_t m, int64_t stop_count, int32_t* rank_out, void* workspace,
+                        size_t workspace_bytes, void* stream);
+/* Crowding distance of the last peeled front (non_dominate.py:198-231 with mask = rank == worst). */
+int evox_hip_stage_crowding(int64_t n, int64_t m, void* workspace, size_t workspace_bytes, void* stream);
+/* Index-stable top-k on the last front + listing of the better fronts (non_dominate.py:253). */
+int evox_hip_stage_order(int64_t n, int64_t m, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Byte offsets of the workspace regions, for tests and tools:
+ *   out[0] dominance bit matrix (uint64, row j at + j * out[1] words)   out[1] row stride in words
+ *   out[2] words per row in use      out[3] count (int32 n)             out[4] rank (int32 n)
+ *   out[5] distance (float32 n)      out[6] rank-ordered listing (int32 n)
+ *   out[7] front starts (int32 n+2)  out[8] selected order (int32 n)    out[9] control block      */
+int evox_hip_workspace_layout(int64_t n, int64_t m, int64_t* out10);
+
+/* Waits for `stream`, then copies the control block's eight leading ints to HOST memory:
+ * out[0] error (0 or EVOX_HIP_E_BARRIER_TIMEOUT), out[1] fronts peeled, out[2] last front's rank,
+ * out[3] rows in better fronts, out[4] last front's size, out[5] rows taken from it, out[6] sweep passes.
+ * Returns out[0] when it is non-zero. */
+int evox_hip_read_status(const void* workspace, void* stream, int32_t* host_out8);
+
+/* Tunables (process-wide): "peel_blocks_per_cu" (default 2), "spin_limit" (polls before a device-side
+ * wait gives up, default 4000000), "dominance_tile_words" (16). */
+int evox_hip_set_option(const char* name, int64_t value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EVOX_HIP_H */

@@ -1,0 +1,63 @@
+"""CPU-side checks of the C ABI: the library builds, loads and exports every symbol that
+include/evox_hip.h declares; argument validation works without a GPU."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from evox_amd import _lib
+from evox_amd.build import LIB_PATH, build_library
+
+HEADER = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "evox_hip.h")
+
+
+@pytest.fixture(scope="module")
+def handle():
+    if not os.path.exists(LIB_PATH):
+        build_library()
+    return _lib.lib()
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(evox_hip_\w+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert declared_symbols() == sorted(_lib.EXPORTED_SYMBOLS)
+
+
+def test_every_declared_symbol_is_exported(handle):
+    raw = ctypes.CDLL(LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(raw, name), name
+    assert handle.evox_hip_abi_version() == 1
+
+
+def test_workspace_size_and_layout(handle):
+    assert handle.evox_hip_workspace_bytes(0, 3) == 0
+    assert handle.evox_hip_workspace_bytes(10, 0) == 0
+    b = handle.evox_hip_workspace_bytes(20000, 3)
+    # dominated by the bit matrix: 20000 rows x 320 words (313 rounded up to a 128-byte multiple)
+    assert 20000 * 320 * 8 <= b <= 20000 * 320 * 8 + 4 * 2**20
+    b5 = handle.evox_hip_workspace_bytes(200000, 8)
+    assert 5.0e9 < b5 < 5.3e9
+    out = (ctypes.c_int64 * 10)()
+    assert handle.evox_hip_workspace_layout(20000, 3, out) == 0
+    assert out[1] == 320 and out[2] == 314 and out[0] % 256 == 0 and out[9] == 0
+
+
+def test_argument_validation_without_gpu(handle):
+    # null / misaligned / short workspaces and bad sizes are rejected before anything is launched
+    assert handle.evox_hip_non_dominate_rank(None, 10, 3, 3, 1, None, None, 0, None) == _lib.E_BAD_ARG
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    assert handle.evox_hip_non_dominate_rank(p, 10, 3, 3, 1, p, None, 0, None) == _lib.E_WORKSPACE
+    assert handle.evox_hip_non_dominate_rank(p, 10, 3, 3, 1, p, p, 64, None) == _lib.E_WORKSPACE
+    assert handle.evox_hip_non_dominate_rank(p, 0, 3, 3, 1, p, p, 64, None) == _lib.E_BAD_ARG
+    assert handle.evox_hip_nd_environmental_selection(None, 0, 0, p, 10, 3, 3, 1, 11, None, p, p, p, None, p, 64, None) == _lib.E_BAD_ARG
+    assert handle.evox_hip_set_option(b"no_such_option", 1) == _lib.E_BAD_ARG
+    assert handle.evox_hip_set_option(b"peel_blocks_per_cu", 2) == 0
