@@ -1,0 +1,222 @@
+#!/usr/bin/env python3
+"""Benchmark of the environmental-selection hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3|C2|C1|C5] [--no-cpu]
+
+One step = one `nd_environmental_selection` call on the workload (default C3: N=20000, M=3,
+D=100, topk=10000, fitness i.i.d. U[0,1) from seed 0), inputs and outputs resident in HBM.
+Prints ONE JSON line.  `value` is ordered pair comparisons per second through the whole step
+(N^2 / step time); the dominance kernel's own rate, the per-stage times, the roofline of the
+dominant kernel and a host-CPU baseline (the CPU oracle on a bounded sample) ride along.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+VALU_CMP_PEAK_GOPS = 39321.6  # 256 CU x 64 lanes/clk x 2.4 GHz: issue peak of v_cmp_*_f32 (not packable)
+FP32_VECTOR_PEAK_GFLOPS = 157300.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C5"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
+    ap.add_argument("--cpu-sample", type=int, default=16000, help="rows of the workload timed on the CPU")
+    return ap.parse_args()
+
+
+def median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def event_time_us(fn, reps):
+    """Median duration of fn() in microseconds, HIP events on the current stream."""
+    out = []
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        b.synchronize()
+        out.append(a.elapsed_time(b) * 1e3)
+    return median(out)
+
+
+def stage_profile(w, f, reps):
+    """Times every stage alone through the stage entry points (same kernels, same stream)."""
+    from evox_amd import _lib, runtime
+
+    n, m = f.shape
+    ws = runtime.workspace(n, m, f.device)
+    s = runtime.stream_handle(f.device)
+    tail = (ws.data_ptr(), ws.numel(), s)
+
+    def dom():
+        _lib.call("evox_hip_stage_dominance", f.data_ptr(), n, m, f.stride(0), f.stride(1), 0, *tail)
+
+    def count():
+        _lib.call("evox_hip_stage_count", n, m, *tail)
+
+    def peel():
+        _lib.call("evox_hip_stage_peel", n, m, w.topk, None, *tail)
+
+    def crowd():
+        _lib.call("evox_hip_stage_crowding", n, m, *tail)
+
+    def order():
+        _lib.call("evox_hip_stage_order", n, m, *tail)
+
+    times = {}
+    dom(); count(); peel(); crowd(); order()
+    torch.cuda.synchronize()
+    times["dominance_us"] = event_time_us(dom, reps)
+    times["count_us"] = event_time_us(count, reps)
+    # the peel consumes the counts, so each repetition re-runs count first and subtracts it
+    both = event_time_us(lambda: (count(), peel()), reps)
+    times["peel_us"] = max(both - times["count_us"], 0.0)
+    times["crowding_us"] = event_time_us(crowd, reps)
+    times["order_us"] = event_time_us(order, reps)
+    count(); peel()
+    runtime.note_call(ws, s)
+    status = runtime.last_status()
+    views = runtime.workspace_views(ws, n, m)
+    rank = views["rank"].clone()
+    return times, status, rank, views["nwords"]
+
+
+def cpu_baseline(w, sample_rows):
+    """The CPU oracle (torch restatement of the reference's eager path) on the first `sample_rows`
+    rows of the workload, all host threads.  Only this leg touches oracle/."""
+    from oracle import eager_restatement as er
+
+    n = min(sample_rows, w.f.size(0))
+    f = w.f[:n].contiguous()
+    x = (w.x if w.x is not None else w.f)[:n].contiguous()
+    k = max(1, n // 2)
+    torch.set_num_threads(os.cpu_count() or 1)
+    t0 = time.perf_counter()
+    er.environmental_selection(x, f, k)
+    dt = time.perf_counter() - t0
+    return {
+        "value": n * n / dt,
+        "unit": "comparisons/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"first {n} rows of {w.name} (topk={k}), one nd_environmental_selection call, {dt:.2f} s; "
+                  f"torch-CPU restatement of the reference's eager path",
+        "seconds": dt,
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs the selection path on ONE GPU (asked for {args.gpus}); "
+              "the path is not sharded across GPUs, so there is no multi-GPU figure to report.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X (torch.cuda.is_available() is False)", file=sys.stderr)
+        sys.exit(2)
+
+    from evox_amd import workloads
+    from evox_amd.operators.selection import nd_environmental_selection
+
+    w = {"C1": workloads.c1, "C2": workloads.c2, "C3": workloads.c3, "C5": workloads.c5}[args.workload]()
+    dev = torch.device("cuda", 0)
+    f = w.f.to(dev)
+    x = (w.x if w.x is not None else w.f).to(dev)
+    n, m = f.shape
+
+    def step():
+        return nd_environmental_selection(x, f, w.topk)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+
+    times, status, rank, nwords = stage_profile(w, f, max(5, min(args.steps, 30)))
+
+    pairs = float(n) * n
+    compares = 2.0 * m * pairs  # the reference's `<=` and `<` per objective and ordered pair
+    row_bytes = nwords * 8
+    # peel: rows still unranked at the start of pass r are read once in pass r (sweep formulation),
+    # plus count read/write and rank write per touched row and the front bitmap per pass
+    passes = status["passes"]
+    rank_cpu = rank.cpu()
+    alive_rows = sum(int((rank_cpu > r).sum()) for r in range(passes))
+    peel_bytes = alive_rows * (row_bytes + 12) + passes * (nwords * 8)
+    dom_bytes = n * m * 4 + n * row_bytes
+    count_bytes = n * row_bytes + n * 8
+    phases = {
+        "dominance": {"us": times["dominance_us"], "bound": "valu", "achieved": compares / times["dominance_us"] / 1e3,
+                      "peak": VALU_CMP_PEAK_GOPS, "unit": "Gcompare/s",
+                      "hbm_GBs": dom_bytes / times["dominance_us"] / 1e3},
+        "count": {"us": times["count_us"], "bound": "hbm", "achieved": count_bytes / times["count_us"] / 1e3,
+                  "peak": HBM_PEAK_GBS, "unit": "GB/s"},
+        "peel": {"us": times["peel_us"], "bound": "hbm", "achieved": peel_bytes / max(times["peel_us"], 1e-9) / 1e3,
+                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "passes": passes, "bytes": peel_bytes},
+        "crowding": {"us": times["crowding_us"]},
+        "order": {"us": times["order_us"]},
+    }
+    for p in phases.values():
+        if "achieved" in p:
+            p["frac"] = p["achieved"] / p["peak"]
+    dominant = max(("dominance", "count", "peel"), key=lambda k: phases[k]["us"])
+    d = phases[dominant]
+    roofline = {
+        "kernel": {"dominance": "dominance_kernel", "count": "count_kernel", "peel": "peel_kernel"}[dominant],
+        "bound": "hbm" if d["bound"] == "hbm" else "valu",
+        "achieved": d["achieved"], "peak": d["peak"], "unit": d["unit"], "frac": d["frac"], "traffic": None,
+    }
+
+    out = {
+        "metric": "dominance comparisons/sec through nd_environmental_selection (N^2 ordered pairs per step)",
+        "value": pairs / (ms_per_step * 1e-3),
+        "unit": "comparisons/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{w.name}: nd_environmental_selection N={n} M={m} D={x.shape[1] if x.dim() > 1 else 1} "
+                               f"topk={w.topk}, fitness U[0,1) seed {w.seed}" if w.name in ("C1", "C3") else
+                               f"{w.name}: nd_environmental_selection N={n} M={m} topk={w.topk} seed {w.seed}"},
+        "latency_ms": ms_per_step,
+        "dominance_kernel_comparisons_per_s": pairs / (times["dominance_us"] * 1e-6),
+        "dominance_kernel_scalar_compares_per_s": compares / (times["dominance_us"] * 1e-6),
+        "fronts_peeled": status["fronts"],
+        "roofline": roofline,
+        "phases": phases,
+    }
+    if not args.no_cpu:
+        base = cpu_baseline(w, args.cpu_sample)
+        out["cpu_baseline"] = base
+        out["speedup_vs_cpu_baseline"] = out["value"] / base["value"]
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -276,6 +276,12 @@ int evox_hip_stage_dominance(const float* f, int64_t n, int64_t m, int64_t sr, i
 int evox_hip_stage_count(int64_t n, int64_t m, void* ws, size_t ws_bytes, void* stream) {
   Ws w;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
+  // as a stage of its own it may be repeated on one dominance matrix: start from a clean state
+  const int64_t zero_words = (int64_t)((w.L.zero_end - w.L.ctrl) / 4);
+  int blocks = (int)((zero_words + 255) / 256);
+  if (blocks > 1024) blocks = 1024;
+  hipLaunchKernelGGL(reset_state_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, w.at<uint32_t>(w.L.ctrl), zero_words);
+  EVX_LAUNCH_CHECK();
   return stage_count(w, true, (hipStream_t)stream);
 }
 

@@ -27,6 +27,12 @@ namespace evx {
 constexpr int kPeelThreads = 256;
 constexpr int kRankUnset = 0x7FFFFFFF;
 
+// Clears the control block, the front sizes and the front bitmaps (one contiguous region).
+__global__ __launch_bounds__(256) void reset_state_kernel(uint32_t* __restrict__ words, int64_t n_words) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_words; i += (int64_t)gridDim.x * blockDim.x)
+    words[i] = 0u;
+}
+
 // ------------------------------------------------------------------ counts
 
 // One wave per row: popcount of the row.  Rows with no dominator are rank 0 and form front 0.
@@ -63,47 +69,58 @@ __global__ __launch_bounds__(256) void count_kernel(const uint64_t* __restrict__
 
 // ------------------------------------------------------------ grid barrier
 
+// Relaxed agent-scope accesses: they go to the level that all XCDs share (each XCD has an L2 of
+// its own), one location at a time, without the whole-cache write-back / invalidate that an
+// agent-scope fence costs.  Everything that one block writes and another block reads during the
+// kernel (front bitmaps, front sizes, barrier flags) is accessed only through these.
+template <class T>
+__device__ inline T coherent_load(const T* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <class T>
+__device__ inline void coherent_store(T* p, T v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Flag-array barrier: every block publishes the generation in its own slot, block 0 waits for all
 // slots and then publishes the generation in `release`, the others wait for that.  No
-// read-modify-write contention; every wait is bounded by `spin_limit` polls, after which the
-// error flag is set and the caller leaves its loop, so all waves always finish.
+// read-modify-write contention.  __syncthreads() makes every wave wait for its own outstanding
+// memory operations (it carries a workgroup-scope fence) before the block's flag is written, and
+// the data exchanged across the barrier is accessed coherently (see above), so no cache-wide fence
+// is needed.  Every wait is bounded by `spin_limit` polls, after which the error flag is set and the
+// caller leaves its loop, so all waves always finish.
 __device__ inline bool grid_barrier(Ctrl* ctrl, unsigned gen, unsigned spin_limit) {
-  __threadfence();
   __syncthreads();
-  bool ok = true;
   if (blockIdx.x == 0) {
+    bool ok = true;
     for (unsigned b = 1 + threadIdx.x; b < gridDim.x; b += blockDim.x) {
       unsigned spins = 0;
-      while (__hip_atomic_load(&ctrl->arrive[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < gen) {
-        __builtin_amdgcn_s_sleep(2);
+      while (coherent_load(&ctrl->arrive[b]) < gen) {
         if (++spins > spin_limit) {
           ok = false;
           break;
         }
+        __builtin_amdgcn_s_sleep(1);
       }
     }
-    if (!ok) __hip_atomic_store(&ctrl->err, kErrBarrierTimeout, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!ok) coherent_store(&ctrl->err, kErrBarrierTimeout);
     __syncthreads();
-    if (threadIdx.x == 0) {
-      __threadfence();
-      __hip_atomic_store(&ctrl->release, gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    if (threadIdx.x == 0) coherent_store(&ctrl->release, gen);
   } else {
     if (threadIdx.x == 0) {
-      __hip_atomic_store(&ctrl->arrive[blockIdx.x], gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      coherent_store(&ctrl->arrive[blockIdx.x], gen);
       unsigned spins = 0;
-      while (__hip_atomic_load(&ctrl->release, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < gen) {
-        __builtin_amdgcn_s_sleep(2);
+      while (coherent_load(&ctrl->release) < gen) {
         if (++spins > spin_limit) {
-          __hip_atomic_store(&ctrl->err, kErrBarrierTimeout, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          coherent_store(&ctrl->err, kErrBarrierTimeout);
           break;
         }
+        __builtin_amdgcn_s_sleep(1);
       }
     }
   }
   __syncthreads();
-  __threadfence();
-  return __hip_atomic_load(&ctrl->err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
+  return coherent_load(&ctrl->err) == 0;
 }
 
 // -------------------------------------------------------------- one sweep
@@ -196,11 +213,11 @@ __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __re
     uint64_t* cur = fronts + (int64_t)(level % 3) * nwords;
     uint64_t* nxt = fronts + (int64_t)((level + 1) % 3) * nwords;
     uint64_t* old = fronts + (int64_t)((level + 2) % 3) * nwords;
-    const int size = fsize[level];
+    const int size = coherent_load(&fsize[level]);
     if (size <= 0) break;  // cannot happen for 1 <= stop_count <= n: a finite partial order has minimal rows
     const bool last = ranked + size >= stop_count;
     if (!last || blockIdx.x == 0) {
-      for (int w = threadIdx.x; w < nwords; w += blockDim.x) front_lds[w] = cur[w];
+      for (int w = threadIdx.x; w < nwords; w += blockDim.x) front_lds[w] = coherent_load(&cur[w]);
       __syncthreads();
     }
     if (blockIdx.x == 0) {
@@ -218,7 +235,7 @@ __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __re
         }
       }
       if (!last)
-        for (int w = threadIdx.x; w < nwords; w += blockDim.x) old[w] = 0;
+        for (int w = threadIdx.x; w < nwords; w += blockDim.x) coherent_store(&old[w], (uint64_t)0);
     }
     if (last) break;
     if (blockIdx.x != 0) {

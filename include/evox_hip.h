@@ -75,7 +75,8 @@ int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int6
  * evaluates both `<=` and `<` per objective as the reference does. */
 int evox_hip_stage_dominance(const float* f, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col, int variant,
                              void* workspace, size_t workspace_bytes, void* stream);
-/* Domination counts by row popcount (non_dominate.py:188) and front 0 (:192). */
+/* Domination counts by row popcount (non_dominate.py:188) and front 0 (:192).  Resets the peeling
+ * state first, so count -> peel can be repeated on one dominance matrix. */
 int evox_hip_stage_count(int64_t n, int64_t m, void* workspace, size_t workspace_bytes, void* stream);
 /* Front peeling (non_dominate.py:29-59, :161-169) until stop_count rows are ranked (stop_count = n
  * ranks every row).  rank_out may be NULL (ranks stay in the workspace). */
