@@ -7,6 +7,7 @@
 #include "common.hpp"
 #include "crowd.hpp"
 #include "dominance.hpp"
+#include "order.hpp"
 #include "peel.hpp"
 
 namespace evx {
@@ -15,16 +16,18 @@ constexpr int kMaxGrid = 4096;  // slots of the grid barrier
 
 struct Options {
   int peel_blocks_per_cu = 2;
+  int peel_witness = 1;
   unsigned spin_limit = 4000000u;
-  int dominance_tile_words = 16;
+  int dominance_tile_words = 4;
 };
 static Options g_opt;
 
 struct Layout {
-  int n, m, npad, nwords, kstride;
+  int n, m, npad, nwords, kstride, buckets, prep_blocks;
   int64_t wstride;
   // byte offsets
-  size_t ctrl, fsize, fronts, zero_end, fstart, xs, key, count, rank, dist, perm, order, ukey, pos, scost, dkey, dom, total;
+  size_t ctrl, fsize, fronts_slot, fronts_orig, hist, zero_end, fstart, xs, key, partials, sortparam, bstart, bcursor,
+      members, xs_sorted, key_sorted, orig_of, count, witness, rank, dist, perm, order, ukey, pos, scost, dkey, dom, total;
 };
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
@@ -37,25 +40,41 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->nwords = L->npad / 64;
   L->wstride = round_up(L->nwords, 16);
   L->kstride = (int)round_up(n, 64);
+  // buckets of the slot sort: a power of two near 4 n, between 1024 and 65536
+  int buckets = 1024;
+  while (buckets < 65536 && buckets < 4 * n) buckets <<= 1;
+  L->buckets = buckets;
+  L->prep_blocks = (int)((L->npad + 255) / 256 < 1024 ? (L->npad + 255) / 256 : 1024);
   size_t o = 0;
-  // --- cleared by prepare_kernel on every call: control block, front sizes, front bitmaps
-  L->ctrl = o;   o = align_up(o + sizeof(Ctrl) + sizeof(unsigned) * kMaxGrid);
-  L->fsize = o;  o = align_up(o + sizeof(int) * (size_t)(n + 2));
-  L->fronts = o; o = align_up(o + sizeof(uint64_t) * 3 * (size_t)L->nwords);
+  // --- cleared on every call: control block, front sizes, front bitmaps, sort histogram
+  L->ctrl = o;        o = align_up(o + sizeof(Ctrl) + sizeof(unsigned long long) * kMaxGrid);
+  L->fsize = o;       o = align_up(o + sizeof(int) * (size_t)(n + 2));
+  L->fronts_slot = o; o = align_up(o + sizeof(uint64_t) * kFrontBuffers * kFrontStride * (size_t)L->nwords);
+  L->fronts_orig = o; o = align_up(o + sizeof(uint64_t) * kFrontBuffers * kFrontStride * (size_t)L->nwords);
+  L->hist = o;        o = align_up(o + sizeof(int) * (size_t)buckets);
   L->zero_end = o;
-  L->fstart = o; o = align_up(o + sizeof(int) * (size_t)(n + 2));
-  L->xs = o;     o = align_up(o + sizeof(float) * (size_t)m * L->npad);
-  L->key = o;    o = align_up(o + sizeof(uint64_t) * (size_t)L->npad);
-  L->count = o;  o = align_up(o + sizeof(int) * (size_t)n);
-  L->rank = o;   o = align_up(o + sizeof(int) * (size_t)n);
-  L->dist = o;   o = align_up(o + sizeof(float) * (size_t)n);
-  L->perm = o;   o = align_up(o + sizeof(int) * (size_t)n);
-  L->order = o;  o = align_up(o + sizeof(int) * (size_t)n);
-  L->ukey = o;   o = align_up(o + sizeof(uint32_t) * (size_t)m * L->kstride);
-  L->pos = o;    o = align_up(o + sizeof(int) * (size_t)m * L->kstride);
-  L->scost = o;  o = align_up(o + sizeof(float) * (size_t)m * L->kstride);
-  L->dkey = o;   o = align_up(o + sizeof(uint32_t) * (size_t)L->kstride);
-  L->dom = o;    o = align_up(o + sizeof(uint64_t) * (size_t)n * (size_t)L->wstride);
+  L->fstart = o;     o = align_up(o + sizeof(int) * (size_t)(n + 2));
+  L->xs = o;         o = align_up(o + sizeof(float) * (size_t)m * L->npad);
+  L->key = o;        o = align_up(o + sizeof(uint64_t) * (size_t)L->npad);
+  L->partials = o;   o = align_up(o + sizeof(unsigned long long) * 2 * (size_t)L->prep_blocks);
+  L->sortparam = o;  o = align_up(o + sizeof(SortParam));
+  L->bstart = o;     o = align_up(o + sizeof(int) * (size_t)(buckets + 1));
+  L->bcursor = o;    o = align_up(o + sizeof(int) * (size_t)buckets);
+  L->members = o;    o = align_up(o + sizeof(int) * (size_t)n);
+  L->xs_sorted = o;  o = align_up(o + sizeof(float) * (size_t)m * L->npad);
+  L->key_sorted = o; o = align_up(o + sizeof(uint64_t) * (size_t)L->npad);
+  L->orig_of = o;    o = align_up(o + sizeof(int) * (size_t)L->npad);
+  L->count = o;      o = align_up(o + sizeof(int) * (size_t)n);
+  L->witness = o;    o = align_up(o + sizeof(int) * (size_t)n);
+  L->rank = o;       o = align_up(o + sizeof(int) * (size_t)n);
+  L->dist = o;       o = align_up(o + sizeof(float) * (size_t)n);
+  L->perm = o;       o = align_up(o + sizeof(int) * (size_t)n);
+  L->order = o;      o = align_up(o + sizeof(int) * (size_t)n);
+  L->ukey = o;       o = align_up(o + sizeof(uint32_t) * (size_t)m * L->kstride);
+  L->pos = o;        o = align_up(o + sizeof(int) * (size_t)m * L->kstride);
+  L->scost = o;      o = align_up(o + sizeof(float) * (size_t)m * L->kstride);
+  L->dkey = o;       o = align_up(o + sizeof(uint32_t) * (size_t)L->kstride);
+  L->dom = o;        o = align_up(o + sizeof(uint64_t) * (size_t)n * (size_t)L->wstride);
   L->total = o;
   return true;
 }
@@ -102,11 +121,11 @@ static void launch_dominance_m(const Ws& w, int variant, hipStream_t s) {
   const Layout& L = w.L;
   dim3 grid((L.npad + 255) / 256, (L.nwords + IW - 1) / IW);
   if (variant == kDomTwoCompares)
-    hipLaunchKernelGGL((dominance_kernel<M, IW, kDomTwoCompares>), grid, dim3(256), 0, s, w.at<float>(L.xs),
-                       w.at<uint64_t>(L.key), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords);
+    hipLaunchKernelGGL((dominance_kernel<M, IW, kDomTwoCompares>), grid, dim3(256), 0, s, w.at<float>(L.xs_sorted),
+                       w.at<uint64_t>(L.key_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords);
   else
-    hipLaunchKernelGGL((dominance_kernel<M, IW, kDomKey64>), grid, dim3(256), 0, s, w.at<float>(L.xs),
-                       w.at<uint64_t>(L.key), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords);
+    hipLaunchKernelGGL((dominance_kernel<M, IW, kDomKey64>), grid, dim3(256), 0, s, w.at<float>(L.xs_sorted),
+                       w.at<uint64_t>(L.key_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords);
 }
 
 template <int IW>
@@ -123,25 +142,48 @@ static void launch_dominance(const Ws& w, int variant, hipStream_t s) {
     case 8: launch_dominance_m<8, IW>(w, variant, s); break;
     default: {
       dim3 grid((L.npad + 255) / 256, (L.nwords + IW - 1) / IW);
-      hipLaunchKernelGGL((dominance_any_m_kernel<IW>), grid, dim3(256), 0, s, w.at<float>(L.xs), w.at<uint64_t>(L.key),
-                         w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords, L.m);
+      hipLaunchKernelGGL((dominance_any_m_kernel<IW>), grid, dim3(256), 0, s, w.at<float>(L.xs_sorted),
+                         w.at<uint64_t>(L.key_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords, L.m);
     }
   }
 }
 
-static int stage_dominance(const Ws& w, const float* f, int64_t sr, int64_t sc, int variant, hipStream_t s) {
+// Fitness -> structure of arrays + keys, state reset, then the slot sort (order.hpp).
+static int stage_prepare(const Ws& w, const float* f, int64_t sr, int64_t sc, bool with_sort, hipStream_t s) {
   const Layout& L = w.L;
   if (f == nullptr) return kErrBadArg;
   const int64_t zero_words = (int64_t)((L.zero_end - L.ctrl) / 4);
-  int blocks = (int)((L.npad + 255) / 256);
-  const int64_t zb = (zero_words + 255) / 256;
-  if (zb > blocks) blocks = (int)(zb > 2048 ? 2048 : zb);
-  hipLaunchKernelGGL(prepare_kernel, dim3(blocks), dim3(256), 0, s, f, sr, sc, L.n, L.m, L.npad, w.at<float>(L.xs),
-                     w.at<uint64_t>(L.key), w.at<uint32_t>(L.ctrl), zero_words);
+  hipLaunchKernelGGL(prepare_kernel, dim3(L.prep_blocks), dim3(256), 0, s, f, sr, sc, L.n, L.m, L.npad, w.at<float>(L.xs),
+                     w.at<uint64_t>(L.key), w.at<unsigned long long>(L.partials), w.at<uint32_t>(L.ctrl), zero_words);
   EVX_LAUNCH_CHECK();
-  // small populations get narrower tiles so that the grid still has many blocks
-  int tile = g_opt.dominance_tile_words;
-  if ((int64_t)((L.npad + 255) / 256) * ((L.nwords + 15) / 16) < 2 * device_cus()) tile = 4;
+  if (!with_sort) return 0;
+  int blocks = (L.n + 255) / 256;
+  if (blocks > 2048) blocks = 2048;
+  hipLaunchKernelGGL(bucket_hist_kernel, dim3(blocks), dim3(256), 0, s, w.at<uint64_t>(L.key), L.n,
+                     w.at<unsigned long long>(L.partials), L.prep_blocks, L.buckets, w.at<int>(L.hist),
+                     w.at<SortParam>(L.sortparam));
+  EVX_LAUNCH_CHECK();
+  hipLaunchKernelGGL(bucket_scan_kernel, dim3(1), dim3(1024), 0, s, w.at<int>(L.hist), L.buckets, w.at<int>(L.bstart),
+                     w.at<int>(L.bcursor));
+  EVX_LAUNCH_CHECK();
+  hipLaunchKernelGGL(bucket_scatter_kernel, dim3(blocks), dim3(256), 0, s, w.at<uint64_t>(L.key), L.n,
+                     w.at<SortParam>(L.sortparam), w.at<int>(L.bcursor), w.at<int>(L.members));
+  EVX_LAUNCH_CHECK();
+  int pblocks = (L.npad + 255) / 256;
+  if (pblocks > 2048) pblocks = 2048;
+  hipLaunchKernelGGL(bucket_place_kernel, dim3(pblocks), dim3(256), 0, s, w.at<uint64_t>(L.key), w.at<float>(L.xs), L.n, L.m,
+                     L.npad, w.at<SortParam>(L.sortparam), w.at<int>(L.bstart), w.at<int>(L.members),
+                     w.at<uint64_t>(L.key_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of));
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+static int stage_dominance(const Ws& w, const float* f, int64_t sr, int64_t sc, int variant, hipStream_t s) {
+  const Layout& L = w.L;
+  if (int e = stage_prepare(w, f, sr, sc, true, s)) return e;
+  // (the lower triangle in tiles of 4 words keeps every SIMD busy with several waves; 16 is kept for
+  // measurements)
+  const int tile = g_opt.dominance_tile_words;
   if (tile >= 16)
     launch_dominance<16>(w, variant, s);
   else
@@ -155,37 +197,76 @@ static int stage_count(const Ws& w, bool fill_dist, hipStream_t s) {
   int blocks = (L.n + 3) / 4;
   const int cap = device_cus() * 8;
   if (blocks > cap) blocks = cap;
-  hipLaunchKernelGGL(count_kernel, dim3(blocks), dim3(256), 0, s, w.at<uint64_t>(L.dom), L.wstride, L.nwords, L.n,
-                     w.at<int>(L.count), w.at<int>(L.rank), w.at<uint64_t>(L.fronts), w.at<int>(L.fsize),
+  hipLaunchKernelGGL(count_kernel, dim3(blocks), dim3(256), 0, s, w.at<uint64_t>(L.dom), L.wstride, L.n,
+                     w.at<int>(L.orig_of), w.at<int>(L.count), w.at<int>(L.rank), w.at<int>(L.witness),
+                     w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
                      fill_dist ? w.at<float>(L.dist) : (float*)nullptr);
   EVX_LAUNCH_CHECK();
   return 0;
 }
 
-static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s) {
-  const Layout& L = w.L;
-  if (stop_count < 1 || stop_count > L.n) return kErrBadArg;
-  const size_t lds = sizeof(uint64_t) * (size_t)L.nwords;
-  if (lds > 160 * 1024 - 4096) return kErrBadArg;
+// Resident blocks per CU of the peel kernel for a dynamic-LDS size (cached: the query is not free).
+// Returns a negative library code or positive hipError_t through *err and 0 on failure.
+static int peel_blocks_per_cu(size_t lds, int* err) {
+  struct Entry { size_t lds; int dev; int per_cu; };
+  static Entry cache[16];
+  static int used = 0;
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  for (int i = 0; i < used; ++i)
+    if (cache[i].lds == lds && cache[i].dev == dev) return cache[i].per_cu;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(peel_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
+    if (e != hipSuccess) { *err = (int)e; return 0; }
   }
   int per_cu = 0;
   hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, peel_kernel, kPeelThreads, lds);
-  if (e != hipSuccess) return (int)e;
-  if (per_cu < 1) return kErrBadArg;
-  if (per_cu > g_opt.peel_blocks_per_cu) per_cu = g_opt.peel_blocks_per_cu;
-  // every block must be resident at once: the grid never exceeds what the device holds
-  int blocks = device_cus() * per_cu;
-  if (blocks > kMaxGrid) blocks = kMaxGrid;
-  const int useful = 1 + (L.n + 3) / 4;  // block 0 + one wave per row
-  if (blocks > useful) blocks = useful;
+  if (e != hipSuccess) { *err = (int)e; return 0; }
+  if (per_cu < 1) { *err = kErrBadArg; return 0; }
+  if (used < 16) cache[used++] = Entry{lds, dev, per_cu};
+  return per_cu;
+}
+
+static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s) {
+  const Layout& L = w.L;
+  if (stop_count < 1 || stop_count > L.n) return kErrBadArg;
+  const size_t lds_limit = 160 * 1024 - 4096;
+  const size_t bitmap = sizeof(uint64_t) * (size_t)L.nwords;
+  const int cus = device_cus();
+  // The grid never exceeds what the device holds at once (the blocks wait for one another).
+  auto grid_for = [&](size_t lds, int* err) -> int {
+    int per_cu = peel_blocks_per_cu(lds, err);
+    if (per_cu > g_opt.peel_blocks_per_cu) per_cu = g_opt.peel_blocks_per_cu;
+    int64_t blocks = (int64_t)cus * per_cu;
+    if (blocks > kMaxGrid) blocks = kMaxGrid;
+    const int64_t wpb = kPeelThreads / 64;
+    const int64_t useful = kFirstSweeper + ((int64_t)L.n + wpb - 1) / wpb;  // master, lister + one wave per row
+    return (int)(blocks < useful ? blocks : useful);
+  };
+  // The witness pass keeps two bitmaps in LDS and at most kWitnessChunks * 64 rows per sweeping
+  // wave; populations too large for that use the sweep pass.
+  int err = 0;
+  int use_witness = g_opt.peel_witness && 2 * bitmap <= lds_limit;
+  int blocks = 0;
+  if (use_witness) {
+    blocks = grid_for(2 * bitmap, &err);
+    if (err) return err;
+    const int64_t waves = (int64_t)(blocks - kFirstSweeper) * (kPeelThreads / 64);
+    if (blocks <= kFirstSweeper || (L.n + waves - 1) / waves > kWitnessChunks * 64) use_witness = 0;
+  }
+  if (!use_witness) {
+    if (bitmap > lds_limit) return kErrBadArg;
+    blocks = grid_for(bitmap, &err);
+    if (err) return err;
+  }
+  if (blocks <= kFirstSweeper) return kErrBadArg;
+  const size_t lds = bitmap * (use_witness ? 2 : 1);
   hipLaunchKernelGGL(peel_kernel, dim3(blocks), dim3(kPeelThreads), lds, s, w.at<uint64_t>(L.dom), L.wstride, L.nwords,
-                     L.n, w.at<int>(L.count), w.at<int>(L.rank), w.at<uint64_t>(L.fronts), w.at<int>(L.fsize),
+                     L.n, w.at<int>(L.orig_of), w.at<int>(L.count), w.at<int>(L.rank), w.at<uint64_t>(L.fronts_slot),
+                     w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
                      want_perm ? w.at<int>(L.perm) : (int*)nullptr, w.at<int>(L.fstart), w.ctrl(), (int)stop_count,
-                     g_opt.spin_limit);
+                     g_opt.spin_limit, w.at<int>(L.witness), use_witness);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -249,6 +330,7 @@ int evox_hip_workspace_layout(int64_t n, int64_t m, int64_t* out) {
   out[7] = (int64_t)L.fstart;
   out[8] = (int64_t)L.order;
   out[9] = (int64_t)L.ctrl;
+  out[10] = (int64_t)L.orig_of;
   return 0;
 }
 
@@ -256,6 +338,8 @@ int evox_hip_set_option(const char* name, int64_t value) {
   if (name == nullptr) return kErrBadArg;
   if (!strcmp(name, "peel_blocks_per_cu") && value >= 1 && value <= 16) {
     g_opt.peel_blocks_per_cu = (int)value;
+  } else if (!strcmp(name, "peel_witness") && (value == 0 || value == 1)) {
+    g_opt.peel_witness = (int)value;
   } else if (!strcmp(name, "spin_limit") && value >= 1 && value <= 0x7FFFFFFFll) {
     g_opt.spin_limit = (unsigned)value;
   } else if (!strcmp(name, "dominance_tile_words") && (value == 4 || value == 16)) {
@@ -325,10 +409,7 @@ int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   const Layout& L = w.L;
   hipStream_t s = (hipStream_t)stream;
-  const int64_t zero_words = (int64_t)((L.zero_end - L.ctrl) / 4);
-  hipLaunchKernelGGL(prepare_kernel, dim3((L.npad + 255) / 256), dim3(256), 0, s, costs, sr, sc, L.n, L.m, L.npad,
-                     w.at<float>(L.xs), w.at<uint64_t>(L.key), w.at<uint32_t>(L.ctrl), zero_words);
-  EVX_LAUNCH_CHECK();
+  if (int e = stage_prepare(w, costs, sr, sc, false, s)) return e;
   hipLaunchKernelGGL(compact_mask_kernel, dim3(1), dim3(1024), 0, s, mask, mask_stride, L.n, w.at<int>(L.perm),
                      w.at<float>(L.dist), w.ctrl());
   EVX_LAUNCH_CHECK();

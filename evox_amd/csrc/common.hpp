@@ -33,10 +33,13 @@ struct Ctrl {
   int nv;           // size of front `worst`
   int need;         // rows to take from front `worst` (stop_count - worst_start)
   int passes;       // sweep passes executed
-  int reserved[9];
-  unsigned release;  // grid barrier: generation published by block 0
-  unsigned pad[15];
-  unsigned arrive[1];  // grid barrier: one slot per block (allocated to the grid size)
+  int listed;       // front bitmaps 0 .. listed-1 have been listed and cleared; polled by the barrier master
+  int reserved[8];
+  // grid barrier: block 0 publishes (generation << 32 | rows found by all blocks) in `release`,
+  // every other block publishes (generation << 32 | rows it found) in its own `arrive` slot
+  unsigned long long release;
+  unsigned long long pad[7];
+  unsigned long long arrive[1];  // one slot per block (allocated to the grid size)
 };
 
 }  // namespace evx

@@ -6,6 +6,9 @@
 // Layout produced here ("dominated-by" rows): dom[j * wstride + w] holds, in bit b, A[64*w + b, j].
 // Row j therefore lists the dominators of j; its popcount is the domination count of
 // non_dominate.py:188 and one peel pass is popcount(row & front) (non_dominate.py:29-59).
+// Rows and columns are SLOTS: the population relabelled by ascending row key (order.hpp), which makes
+// the matrix strictly lower triangular; word pairs that lie wholly above the diagonal are stored as
+// zeros without being evaluated.
 //
 // Work split: lane = j (fitness of 64 rows held in VGPRs), loop over i with x[i, :] fetched by
 // scalar loads (the index is wave-uniform), so every `<=` is one v_cmp_le_f32 with an SGPR operand
@@ -22,22 +25,18 @@
 
 namespace evx {
 
-// Fitness in structure-of-arrays form, padded with NaN to a multiple of 128 rows, plus the 64-bit row key.
-struct Prepared {
-  const float* xs;       // [m][npad]
-  const uint64_t* key;   // [npad]
-  int n;
-  int npad;
-};
-
-// One kernel turns the caller's strided (n, m) fitness into Prepared and clears the small state
-// arrays that later kernels accumulate into.
+// One kernel turns the caller's strided (n, m) fitness into structure-of-arrays form in original
+// order (padded with NaN to npad, a multiple of 128 rows) plus the 64-bit row keys, leaves the
+// (min, max) key of each block in `partials` for the slot sort, and clears the state arrays that
+// later kernels accumulate into.
 __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ f, int64_t stride_row, int64_t stride_col,
                                                       int n, int m, int npad, float* __restrict__ xs,
-                                                      uint64_t* __restrict__ key, uint32_t* __restrict__ zero_words,
-                                                      int64_t n_zero_words) {
+                                                      uint64_t* __restrict__ key, unsigned long long* __restrict__ partials,
+                                                      uint32_t* __restrict__ zero_words, int64_t n_zero_words) {
+  __shared__ unsigned long long red[2][4];
   const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+  unsigned long long lo = ~0ull, hi = 0ull;
   for (int64_t i = tid; i < npad; i += nthreads) {
     uint64_t s = 0;
     for (int k = 0; k < m; ++k) {
@@ -46,6 +45,29 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
       s += ordered_key(v);
     }
     key[i] = s;
+    if (i < n) {
+      lo = s < lo ? s : lo;
+      hi = s > hi ? s : hi;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned long long a = __shfl_xor(lo, off), b = __shfl_xor(hi, off);
+    lo = a < lo ? a : lo;
+    hi = b > hi ? b : hi;
+  }
+  if ((threadIdx.x & 63) == 0) {
+    red[0][threadIdx.x >> 6] = lo;
+    red[1][threadIdx.x >> 6] = hi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int v = 1; v < 4; ++v) {
+      lo = red[0][v] < lo ? red[0][v] : lo;
+      hi = red[1][v] > hi ? red[1][v] : hi;
+    }
+    partials[2 * blockIdx.x] = lo;      // a block without rows leaves (all-ones, 0): neutral
+    partials[2 * blockIdx.x + 1] = hi;
   }
   for (int64_t i = tid; i < n_zero_words; i += nthreads) zero_words[i] = 0u;
 }
@@ -76,8 +98,14 @@ __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict_
   const uint64_t kj = key[j];
   uint64_t* __restrict__ out = dom + (int64_t)j * wstride;
   const int wend = (w0 + IW < nwords) ? w0 + IW : nwords;  // nwords = npad / 64 is even, and so is IW
+  const int jlast = j - lane + 63;  // last row of this wave
 #pragma unroll 1
   for (int w = w0; w < wend; w += 2) {
+    if (w * 64 > jlast) {
+      // both words lie above the diagonal: no row of a larger slot dominates these rows
+      if (j < n) *reinterpret_cast<ulonglong2*>(out + w) = make_ulonglong2(0ull, 0ull);
+      continue;
+    }
     uint32_t half[4];
 #pragma unroll
     for (int h = 3; h >= 0; --h) {
@@ -127,8 +155,13 @@ __global__ __launch_bounds__(256) void dominance_any_m_kernel(const float* __res
   const uint64_t kj = key[j];
   uint64_t* __restrict__ out = dom + (int64_t)j * wstride;
   const int wend = (w0 + IW < nwords) ? w0 + IW : nwords;
+  const int jlast = j - lane + 63;
 #pragma unroll 1
   for (int w = w0; w < wend; w += 2) {
+    if (w * 64 > jlast) {
+      if (j < n) *reinterpret_cast<ulonglong2*>(out + w) = make_ulonglong2(0ull, 0ull);
+      continue;
+    }
     uint32_t half[4];
 #pragma unroll
     for (int h = 3; h >= 0; --h) {

@@ -1,0 +1,169 @@
+// Relabelling of the population by ascending row key ("slots").
+//
+// key(i) = sum_k ordered_key(x[i,k]) is strictly smaller for a dominator than for the row it
+// dominates (every term is <=, one is <, and NaN rows dominate nothing), so after sorting the rows by
+// (key, original index) every dominance pair has slot(i) < slot(j): the bit matrix built in slot
+// space is strictly lower triangular.  That halves the dominance work, bounds every row scan by the
+// row's own slot, and makes "the highest unranked dominator" a near-perfect witness for the peel
+// (rows of large key lie in deep fronts).  Results never depend on the labelling: ranks are written
+// back by original index and fronts are listed in original-index order.
+//
+// The sort is an exact bucket sort in four small kernels: histogram of a monotone quantisation of the
+// key, exclusive scan of the histogram, unordered scatter of the rows into their bucket ranges
+// (atomics), and an exact placement inside each bucket by counting the members that precede the row in
+// (key, original index) order.  The outcome is deterministic although the scatter is not.
+#pragma once
+
+#include "common.hpp"
+
+namespace evx {
+
+struct SortParam {
+  unsigned long long kmin;
+  int shift;
+  int buckets;
+};
+
+__device__ inline int bucket_of(uint64_t key, const SortParam& p) { return (int)((key - p.kmin) >> p.shift); }
+
+// Reduces the per-block (min, max) key partials written by prepare_kernel and derives the
+// quantisation: (key - kmin) >> shift < buckets.  Every block of the histogram kernel calls it.
+__device__ inline SortParam make_sort_param(const unsigned long long* __restrict__ partials, int nparts, int buckets,
+                                            unsigned long long* lds2) {
+  if (threadIdx.x < 64) {
+    unsigned long long lo = ~0ull, hi = 0ull;
+    for (int p = threadIdx.x; p < nparts; p += 64) {
+      const unsigned long long a = partials[2 * p], b = partials[2 * p + 1];
+      lo = a < lo ? a : lo;
+      hi = b > hi ? b : hi;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const unsigned long long a = __shfl_xor(lo, off), b = __shfl_xor(hi, off);
+      lo = a < lo ? a : lo;
+      hi = b > hi ? b : hi;
+    }
+    if (threadIdx.x == 0) {
+      lds2[0] = lo;
+      lds2[1] = hi;
+    }
+  }
+  __syncthreads();
+  SortParam sp;
+  sp.kmin = lds2[0];
+  sp.buckets = buckets;
+  const unsigned long long span = lds2[1] >= lds2[0] ? lds2[1] - lds2[0] : 0ull;
+  int shift = 0;
+  while (shift < 63 && (span >> shift) >= (unsigned long long)buckets) ++shift;
+  sp.shift = shift;
+  return sp;
+}
+
+__global__ __launch_bounds__(256) void bucket_hist_kernel(const uint64_t* __restrict__ key, int n,
+                                                          const unsigned long long* __restrict__ partials, int nparts,
+                                                          int buckets, int* __restrict__ hist, SortParam* __restrict__ param_out) {
+  __shared__ unsigned long long lds2[2];
+  const SortParam sp = make_sort_param(partials, nparts, buckets, lds2);
+  if (blockIdx.x == 0 && threadIdx.x == 0) *param_out = sp;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
+    atomicAdd(&hist[bucket_of(key[i], sp)], 1);
+}
+
+// One block: start[b] = exclusive prefix of hist, start[buckets] = n; cursor = copy of start.
+// Thread t owns the bins [t * per, (t + 1) * per), per = buckets / 1024 (a multiple of 4, at most
+// 64): it loads them with independent 16-byte loads, scans them in registers, and the 1024 thread
+// totals are scanned by wave shuffles.
+__global__ __launch_bounds__(1024) void bucket_scan_kernel(const int* __restrict__ hist, int buckets, int* __restrict__ start,
+                                                           int* __restrict__ cursor) {
+  __shared__ int wave_tot[16];
+  const int per = buckets / 1024;  // 1, 2, 4, ..., 64
+  const int b0 = threadIdx.x * per;
+  int4 v[16];
+  int mine = 0;
+  if (per >= 4) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) v[q] = q * 4 < per ? *reinterpret_cast<const int4*>(hist + b0 + q * 4) : make_int4(0, 0, 0, 0);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) mine += v[q].x + v[q].y + v[q].z + v[q].w;
+  } else {
+    v[0] = make_int4(hist[b0], per > 1 ? hist[b0 + 1] : 0, 0, 0);
+    mine = v[0].x + v[0].y;
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = mine;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
+  }
+  if (lane == 63) wave_tot[wave] = incl;
+  __syncthreads();
+  int run = incl - mine;
+  for (int w = 0; w < wave; ++w) run += wave_tot[w];
+  if (per >= 4) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      if (q * 4 < per) {
+        int4 o;
+        o.x = run; run += v[q].x;
+        o.y = run; run += v[q].y;
+        o.z = run; run += v[q].z;
+        o.w = run; run += v[q].w;
+        *reinterpret_cast<int4*>(start + b0 + q * 4) = o;
+        *reinterpret_cast<int4*>(cursor + b0 + q * 4) = o;
+      }
+    }
+  } else {
+    start[b0] = run;
+    cursor[b0] = run;
+    run += v[0].x;
+    if (per > 1) {
+      start[b0 + 1] = run;
+      cursor[b0 + 1] = run;
+      run += v[0].y;
+    }
+  }
+  if (threadIdx.x == 1023) start[buckets] = run;
+}
+
+__global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint64_t* __restrict__ key, int n,
+                                                             const SortParam* __restrict__ param, int* __restrict__ cursor,
+                                                             int* __restrict__ members) {
+  const SortParam sp = *param;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
+    members[atomicAdd(&cursor[bucket_of(key[i], sp)], 1)] = i;
+}
+
+// Exact slot of every row: bucket start + number of bucket members that precede it by (key, index).
+// Writes the slot-ordered copies of the fitness (structure of arrays, NaN padding up to npad), of
+// the keys (all-ones padding) and the slot -> original index table (-1 padding).
+__global__ __launch_bounds__(256) void bucket_place_kernel(const uint64_t* __restrict__ key, const float* __restrict__ xs, int n,
+                                                           int m, int npad, const SortParam* __restrict__ param,
+                                                           const int* __restrict__ start, const int* __restrict__ members,
+                                                           uint64_t* __restrict__ key_sorted, float* __restrict__ xs_sorted,
+                                                           int* __restrict__ orig_of) {
+  const SortParam sp = *param;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < npad; i += gridDim.x * blockDim.x) {
+    if (i < n) {
+      const uint64_t ki = key[i];
+      const int b = bucket_of(ki, sp);
+      const int lo = start[b], hi = start[b + 1];
+      int before = 0;
+      for (int p = lo; p < hi; ++p) {
+        const int e = members[p];
+        const uint64_t ke = key[e];
+        before += (ke < ki) || (ke == ki && e < i);
+      }
+      const int slot = lo + before;
+      orig_of[slot] = i;
+      key_sorted[slot] = ki;
+      for (int k = 0; k < m; ++k) xs_sorted[(int64_t)k * npad + slot] = xs[(int64_t)k * npad + i];
+    } else {
+      orig_of[i] = -1;
+      key_sorted[i] = ~0ull;
+      for (int k = 0; k < m; ++k) xs_sorted[(int64_t)k * npad + i] = __uint_as_float(0x7FC00000u);
+    }
+  }
+}
+
+}  // namespace evx

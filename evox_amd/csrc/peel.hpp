@@ -7,59 +7,157 @@
 //     rank[front] = level; count -= sum_{i in front} A[i, :]; count -= front (non_dominate.py:29-59)
 //     level += 1; front = count == 0
 //
-// Here row j of the matrix is the dominator set of j, so count[j] = popcount(row j) and one pass
-// is count[j] -= popcount(row j & front).  A row whose count reaches 0 is ranked at once and enters
-// the next front; ranked rows have count 0 forever and are skipped, which is the reference's
-// "count -= front" (its ranked rows sit at -1 so they never test == 0 again).
+// Row j of the matrix (slot space, see order.hpp) is the dominator set of j, so count[j] =
+// popcount(row j) and a row enters the next front exactly when no unranked row dominates it any more.
+// Two interchangeable passes implement that:
+//   * the sweep pass keeps the counts: count[j] -= popcount(row j & front) for every unranked row;
+//   * the witness pass keeps, per unranked row, one word of its row that still holds an unranked
+//     dominator, and touches memory only when that word has none left.
+// Because the matrix is strictly lower triangular, only words 0 .. j/64 of row j are ever read.
 //
-// The pass loop runs inside ONE persistent kernel: blocks meet at a grid barrier after every
-// pass and read the size of the next front from device memory, so the host never waits for a
-// front.  Block 0 does the bookkeeping of a pass while the others sweep: it lists the members of
-// the current front in ascending row order into `perm` (a stable ordering by rank, which is what
-// the final selection needs for every rank better than the last one) and clears the front
-// buffer that the pass after next will fill.
+// The pass loop runs inside ONE persistent kernel: the sweeping blocks meet at a grid barrier after
+// every pass and learn the size of the next front from the barrier itself, so the host never waits
+// for a front.  A separate block lists every finished front in ascending original row index into
+// `perm` (a stable ordering by rank, which is what the final selection needs for every rank better
+// than the last one) off the critical path.
 #pragma once
 
 #include "common.hpp"
+
+// Hooks for development builds; they compile to nothing in the library.
+#ifndef EVX_TRACE
+#define EVX_TRACE(level, slot)
+#endif
+#ifndef EVX_RESCAN
+#define EVX_RESCAN(level, rows, rounds)
+#endif
 
 namespace evx {
 
 constexpr int kPeelThreads = 256;
 constexpr int kRankUnset = 0x7FFFFFFF;
+// Words of a front bitmap in global memory are kFrontStride words apart (one per 128-byte line): the
+// rows of a front are published by many waves at the same moment, and atomics that share a line
+// serialise.
+constexpr int kFrontStride = 16;
 
-// Clears the control block, the front sizes and the front bitmaps (one contiguous region).
+// Clears the control block, the front sizes, the front bitmaps and the sort histogram (one region).
 __global__ __launch_bounds__(256) void reset_state_kernel(uint32_t* __restrict__ words, int64_t n_words) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_words; i += (int64_t)gridDim.x * blockDim.x)
     words[i] = 0u;
 }
 
+// Words of row j that can hold a dominator (slots below j), rounded up to a whole 16-byte pair.
+__device__ inline int row_words(int j) { return ((j >> 6) + 2) & ~1; }
+
+// ---------------------------------------------------------------- row scan
+
+// Wave-cooperative scan of R bit rows at once (optionally ANDed with a bitmap in LDS).  Every lane
+// takes pairs of words 128 apart; the loads of a U*128-word stretch of all R rows are issued before
+// any of them is used, so a scan costs about one memory latency however many rows are scanned
+// together.  Per row it returns the popcount, the highest non-empty word (-1 when the row is empty)
+// and that word's unmasked value, identical in every lane.
+struct RowScan {
+  int total;
+  int last_word;
+  uint64_t last_bits;
+};
+
+template <bool MASKED, int R, int U>
+__device__ inline void scan_rows(const uint64_t* const (&row)[R], const int (&nw)[R], const uint64_t* mask_lds,
+                                 RowScan (&out)[R]) {
+  const int lane = threadIdx.x & 63;
+  int total[R], last_w[R];
+  uint64_t last_v[R];
+  int nw_max = 0;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    total[r] = 0;
+    last_w[r] = -1;
+    last_v[r] = 0;
+    nw_max = nw[r] > nw_max ? nw[r] : nw_max;
+  }
+  for (int w0 = lane * 2; w0 < nw_max; w0 += U * 128) {
+    ulonglong2 v[R][U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int w = w0 + u * 128;
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        v[r][u] = w < nw[r] ? *reinterpret_cast<const ulonglong2*>(row[r] + w) : make_ulonglong2(0ull, 0ull);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int w = w0 + u * 128;
+      if (w < nw_max) {
+        const uint64_t mx = MASKED ? mask_lds[w] : ~0ull;
+        const uint64_t my = MASKED ? mask_lds[w + 1] : ~0ull;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const uint64_t ax = v[r][u].x & mx, ay = v[r][u].y & my;
+          total[r] += __popcll(ax) + __popcll(ay);
+          if (ax) { last_w[r] = w; last_v[r] = v[r][u].x; }
+          if (ay) { last_w[r] = w + 1; last_v[r] = v[r][u].y; }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    int t = total[r];
+    int hi = last_w[r];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      t += __shfl_xor(t, off);
+      const int other = __shfl_xor(hi, off);
+      hi = other > hi ? other : hi;
+    }
+    out[r].total = t;
+    out[r].last_word = hi;
+    // word w is held by lane (w / 2) % 64; that lane's own highest non-empty word is then w
+    out[r].last_bits = hi < 0 ? 0ull : (uint64_t)__shfl((long long)last_v[r], (hi >> 1) & 63);
+  }
+}
+
+template <bool MASKED>
+__device__ inline RowScan scan_row(const uint64_t* __restrict__ row, int nw, const uint64_t* mask_lds) {
+  const uint64_t* const rows[1] = {row};
+  const int nws[1] = {nw};
+  RowScan out[1];
+  if (nw <= 512)
+    scan_rows<MASKED, 1, 4>(rows, nws, mask_lds, out);
+  else
+    scan_rows<MASKED, 1, 8>(rows, nws, mask_lds, out);
+  return out[0];
+}
+
 // ------------------------------------------------------------------ counts
 
-// One wave per row: popcount of the row.  Rows with no dominator are rank 0 and form front 0.
-// Also fills the crowding-distance output with -inf when one is given.
-__global__ __launch_bounds__(256) void count_kernel(const uint64_t* __restrict__ dom, int64_t wstride, int nwords, int n,
-                                                    int* __restrict__ count, int* __restrict__ rank,
-                                                    uint64_t* __restrict__ front0, int* __restrict__ fsize,
-                                                    float* __restrict__ dist_fill) {
+// One wave per row (slot): popcount of the row = the domination count.  Rows with no dominator
+// are rank 0 and form front 0, published both in slot space (for the passes) and in original-index
+// space (for the listing).  witness[j] = the highest non-empty word of row j (-1 for ranked rows).
+// Also fills the crowding-distance output with -inf when one is given.  Ranks are stored by
+// original index.
+__global__ __launch_bounds__(256) void count_kernel(const uint64_t* __restrict__ dom, int64_t wstride, int n,
+                                                    const int* __restrict__ orig_of, int* __restrict__ count,
+                                                    int* __restrict__ rank, int* __restrict__ witness,
+                                                    uint64_t* __restrict__ front0_slot, uint64_t* __restrict__ front0_orig,
+                                                    int* __restrict__ fsize, float* __restrict__ dist_fill) {
   const int lane = threadIdx.x & 63;
   const int wave_in_block = threadIdx.x >> 6;
   const int waves = gridDim.x * (blockDim.x >> 6);
   int found = 0;
   for (int j = blockIdx.x * (blockDim.x >> 6) + wave_in_block; j < n; j += waves) {
-    const uint64_t* __restrict__ row = dom + (int64_t)j * wstride;
-    int c = 0;
-    for (int w = lane * 2; w < nwords; w += 128) {
-      const ulonglong2 v = *reinterpret_cast<const ulonglong2*>(row + w);
-      c += __popcll(v.x) + __popcll(v.y);
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
+    const RowScan r = scan_row<false>(dom + (int64_t)j * wstride, row_words(j), nullptr);
     if (lane == 0) {
-      count[j] = c;
-      rank[j] = c == 0 ? 0 : kRankUnset;
-      if (dist_fill) dist_fill[j] = -INFINITY;
-      if (c == 0) {
-        atomicOr(reinterpret_cast<unsigned long long*>(front0 + (j >> 6)), 1ull << (j & 63));
+      const int o = orig_of[j];
+      count[j] = r.total;
+      rank[o] = r.total == 0 ? 0 : kRankUnset;
+      witness[j] = r.last_word;
+      if (dist_fill) dist_fill[o] = -INFINITY;
+      if (r.total == 0) {
+        atomicOr(reinterpret_cast<unsigned long long*>(front0_slot + (int64_t)(j >> 6) * kFrontStride), 1ull << (j & 63));
+        atomicOr(reinterpret_cast<unsigned long long*>(front0_orig + (int64_t)(o >> 6) * kFrontStride), 1ull << (o & 63));
         ++found;
       }
     }
@@ -69,10 +167,10 @@ __global__ __launch_bounds__(256) void count_kernel(const uint64_t* __restrict__
 
 // ------------------------------------------------------------ grid barrier
 
-// Relaxed agent-scope accesses: they go to the level that all XCDs share (each XCD has an L2 of
-// its own), one location at a time, without the whole-cache write-back / invalidate that an
-// agent-scope fence costs.  Everything that one block writes and another block reads during the
-// kernel (front bitmaps, front sizes, barrier flags) is accessed only through these.
+// Relaxed agent-scope accesses: one location at a time, coherent across the whole device, without
+// the cache-wide write-back / invalidate that an agent-scope fence costs.  Everything that one
+// block writes and another block reads during the kernel (front bitmaps, front sizes, barrier
+// flags) is accessed only through these or through atomics.
 template <class T>
 __device__ inline T coherent_load(const T* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -82,100 +180,252 @@ __device__ inline void coherent_store(T* p, T v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Flag-array barrier: every block publishes the generation in its own slot, block 0 waits for all
-// slots and then publishes the generation in `release`, the others wait for that.  No
-// read-modify-write contention.  __syncthreads() makes every wave wait for its own outstanding
-// memory operations (it carries a workgroup-scope fence) before the block's flag is written, and
-// the data exchanged across the barrier is accessed coherently (see above), so no cache-wide fence
-// is needed.  Every wait is bounded by `spin_limit` polls, after which the error flag is set and the
-// caller leaves its loop, so all waves always finish.
-__device__ inline bool grid_barrier(Ctrl* ctrl, unsigned gen, unsigned spin_limit) {
-  __syncthreads();
-  if (blockIdx.x == 0) {
-    bool ok = true;
-    for (unsigned b = 1 + threadIdx.x; b < gridDim.x; b += blockDim.x) {
-      unsigned spins = 0;
-      while (coherent_load(&ctrl->arrive[b]) < gen) {
-        if (++spins > spin_limit) {
-          ok = false;
-          break;
-        }
-        __builtin_amdgcn_s_sleep(1);
-      }
-    }
-    if (!ok) coherent_store(&ctrl->err, kErrBarrierTimeout);
-    __syncthreads();
-    if (threadIdx.x == 0) coherent_store(&ctrl->release, gen);
-  } else {
-    if (threadIdx.x == 0) {
-      coherent_store(&ctrl->arrive[blockIdx.x], gen);
-      unsigned spins = 0;
-      while (coherent_load(&ctrl->release) < gen) {
-        if (++spins > spin_limit) {
-          coherent_store(&ctrl->err, kErrBarrierTimeout);
-          break;
-        }
-        __builtin_amdgcn_s_sleep(1);
-      }
-    }
+// Grid synchronisation with three roles, all through flag words and bounded polling:
+//   block 0 ("master")   waits for the tally of every sweeping block, adds them up and publishes
+//                        (generation << 32 | total) in `release`: one round trip both synchronises the
+//                        sweepers and tells them the size of the front they just built;
+//   block 1 ("lister")   follows `release` at its own pace (see peel_kernel) and is never waited for
+//                        inside a pass;
+//   blocks 2.. ("sweepers") publish (generation << 32 | rows found) in their own `arrive` slot and wait
+//                        for `release`.
+// No read-modify-write contention.  __syncthreads() makes every wave wait for its own outstanding
+// memory operations (it carries a workgroup-scope fence) before the block's flag is written, and the
+// data exchanged across the barrier is accessed coherently (see above), so no cache-wide fence is
+// needed.  Every wait is bounded by `spin_limit` polls, after which the error flag is set and every
+// role leaves its loop, so all waves always finish.
+constexpr int kFirstSweeper = 2;
+constexpr int kFrontBuffers = 8;  // front bitmaps in rotation: the lister may lag the sweepers by 6 fronts
+
+template <class Pred>
+__device__ inline bool bounded_wait(Pred done, unsigned spin_limit) {
+  unsigned spins = 0;
+  while (!done()) {
+    if (++spins > spin_limit) return false;
+    __builtin_amdgcn_s_sleep(1);
   }
-  __syncthreads();
-  return coherent_load(&ctrl->err) == 0;
+  return true;
 }
 
-// -------------------------------------------------------------- one sweep
+// Sweeper side.  Returns false after a timeout (here or elsewhere); *total_out = size of the new front.
+__device__ inline bool sweeper_barrier(Ctrl* ctrl, unsigned gen, int block_tally, int* total_out, unsigned spin_limit,
+                                       int* scratch) {
+  __syncthreads();
+  const unsigned long long want = (unsigned long long)gen << 32;
+  if (threadIdx.x == 0) {
+    coherent_store(&ctrl->arrive[blockIdx.x], want | (unsigned)block_tally);
+    unsigned long long v = 0;
+    if (!bounded_wait([&] { return (v = coherent_load(&ctrl->release)) >= want; }, spin_limit))
+      coherent_store(&ctrl->err, kErrBarrierTimeout);
+    scratch[0] = (int)(unsigned)(v & 0xFFFFFFFFull);
+    scratch[1] = coherent_load(&ctrl->err);
+  }
+  __syncthreads();
+  *total_out = scratch[0];
+  const bool fine = scratch[1] == 0;
+  __syncthreads();  // scratch is reused by the caller
+  return fine;
+}
+
+// Master side: gathers the tallies of generation `gen`, waits until the lister has cleared the bitmap
+// that the coming pass will fill (`listed_needed` fronts cleared), then releases the sweepers.
+__device__ inline bool master_barrier(Ctrl* ctrl, unsigned gen, int listed_needed, int* total_out, unsigned spin_limit,
+                                      int* scratch) {
+  const unsigned long long want = (unsigned long long)gen << 32;
+  const int lane = threadIdx.x & 63;
+  bool ok = true;
+  int sum = 0;
+  for (unsigned b = kFirstSweeper + threadIdx.x; b < gridDim.x; b += blockDim.x) {
+    unsigned long long v = 0;
+    ok &= bounded_wait([&] { return (v = coherent_load(&ctrl->arrive[b])) >= want; }, spin_limit);
+    sum += (int)(unsigned)(v & 0xFFFFFFFFull);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+  if (lane == 0) scratch[threadIdx.x >> 6] = sum;
+  if (!ok) coherent_store(&ctrl->err, kErrBarrierTimeout);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int total = 0;
+    for (int v = 0; v < (int)(blockDim.x >> 6); ++v) total += scratch[v];
+    if (!bounded_wait([&] { return coherent_load(&ctrl->listed) >= listed_needed; }, spin_limit))
+      coherent_store(&ctrl->err, kErrBarrierTimeout);
+    coherent_store(&ctrl->release, want | (unsigned)total);
+    scratch[40] = total;
+    scratch[41] = coherent_load(&ctrl->err);
+  }
+  __syncthreads();
+  *total_out = scratch[40];
+  const bool fine = scratch[41] == 0;
+  __syncthreads();
+  return fine;
+}
+
+// What the passes share: the matrix, the slot -> original index table, the output ranks (by
+// original index) and the two bitmaps of the front being built.
+struct PassCtx {
+  const uint64_t* dom;
+  int64_t wstride;
+  int n;
+  const int* orig_of;
+  int* rank;
+  uint64_t* next_slot;
+  uint64_t* next_orig;
+  int next_level;
+};
+
+__device__ inline void publish_ranked(const PassCtx& c, int slot, int orig) {
+  c.rank[orig] = c.next_level;
+  atomicOr(reinterpret_cast<unsigned long long*>(c.next_slot + (int64_t)(slot >> 6) * kFrontStride), 1ull << (slot & 63));
+  atomicOr(reinterpret_cast<unsigned long long*>(c.next_orig + (int64_t)(orig >> 6) * kFrontStride), 1ull << (orig & 63));
+}
+
+// -------------------------------------------------------------- sweep pass
 
 // count[j] -= popcount(row j & front) for every row of this wave's share that is still unranked.
-// `front_lds` is the current front copied to LDS.  Returns the number of rows this thread moved
-// into the next front (non-zero on lane 0 only).
-__device__ inline int sweep_rows(const uint64_t* __restrict__ dom, int64_t wstride, int nwords, int n,
-                                 const uint64_t* front_lds, int* __restrict__ count, int* __restrict__ rank,
-                                 uint64_t* __restrict__ next_front, int next_level, int first_row, int row_step) {
+// `front_lds` is the current front (slot space) copied to LDS.  Returns the number of rows this
+// wave moved into the next front (in every lane).
+__device__ inline int sweep_rows(const PassCtx& c, const uint64_t* front_lds, int* __restrict__ count, int first_row,
+                                 int row_step) {
   const int lane = threadIdx.x & 63;
   int found = 0;
-  for (int j = first_row; j < n; j += row_step) {
+  for (int j = first_row; j < c.n; j += row_step) {
     const int cj = count[j];  // wave-uniform
     if (cj <= 0) continue;
-    const uint64_t* __restrict__ row = dom + (int64_t)j * wstride;
-    int c = 0;
-    for (int w = lane * 2; w < nwords; w += 128) {
-      const ulonglong2 v = *reinterpret_cast<const ulonglong2*>(row + w);
-      c += __popcll(v.x & front_lds[w]) + __popcll(v.y & front_lds[w + 1]);
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
-    if (lane == 0 && c) {
-      const int left = cj - c;
-      count[j] = left;
-      if (left == 0) {
-        rank[j] = next_level;
-        atomicOr(reinterpret_cast<unsigned long long*>(next_front + (j >> 6)), 1ull << (j & 63));
-        ++found;
+    const RowScan r = scan_row<true>(c.dom + (int64_t)j * c.wstride, row_words(j), front_lds);
+    if (r.total) {
+      const int left = cj - r.total;
+      if (lane == 0) {
+        count[j] = left;
+        if (left == 0) publish_ranked(c, j, c.orig_of[j]);
       }
+      found += left == 0;
     }
   }
   return found;
 }
 
+// ------------------------------------------------------------ witness pass
+
+// Every unranked row remembers the highest word of its row that held an unranked dominator when it
+// was last looked at (the "witness": word index + word value, kept in the registers of the lane that
+// owns the row, so the common case touches no memory at all).  A pass only tests that word against
+// the bitmap of unranked rows; when none of its dominators is left the wave rescans the row against
+// the bitmap and either finds the new highest word or ranks the row.  In slot order the highest
+// dominator is almost always the one ranked last, so nearly every rescan is the one that ranks the
+// row.  Same results as the count formulation.
+constexpr int kWitnessChunks = 4;  // a wave owns up to 4 x 64 rows
+
+struct WitnessState {
+  int word[kWitnessChunks];        // witness word index, -1 = ranked (or no row)
+  int orig[kWitnessChunks];        // original index of the row
+  uint64_t bits[kWitnessChunks];   // that word of the row
+};
+
+// Rows are dealt to the sweeping waves round-robin (row = wave + index * waves): rows of
+// neighbouring slots enter the same fronts, and this keeps each front's rescans spread over all waves.
+__device__ inline void witness_load(WitnessState& st, const PassCtx& c, const int* __restrict__ witness, int first_row,
+                                    int row_step) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int ch = 0; ch < kWitnessChunks; ++ch) {
+    const int64_t j64 = (int64_t)first_row + (int64_t)(ch * 64 + lane) * row_step;
+    const bool have = j64 < c.n;
+    const int j = have ? (int)j64 : 0;
+    st.word[ch] = have ? witness[j] : -1;
+    st.orig[ch] = have ? c.orig_of[j] : 0;
+    st.bits[ch] = st.word[ch] >= 0 ? c.dom[(int64_t)j * c.wstride + st.word[ch]] : 0ull;
+  }
+}
+
+__device__ inline int witness_rows(WitnessState& st, const PassCtx& c, const uint64_t* alive_lds, int first_row,
+                                   int row_step) {
+  const int lane = threadIdx.x & 63;
+  int found = 0;
+  int stat_rows = 0, stat_rounds = 0;
+#pragma unroll
+  for (int ch = 0; ch < kWitnessChunks; ++ch) {
+    const bool need = st.word[ch] >= 0 && (st.bits[ch] & alive_lds[st.word[ch] < 0 ? 0 : st.word[ch]]) == 0;
+    uint64_t todo = __builtin_amdgcn_ballot_w64(need);
+    while (todo) {
+      // up to four rows per round: their loads overlap
+      int l[4], jrow[4], nws[4];
+      const uint64_t* rows[4];
+      int cnt = 0;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const bool have = todo != 0;
+        if (have) {
+          l[q] = __ffsll((unsigned long long)todo) - 1;
+          todo &= todo - 1;
+          ++cnt;
+        } else {
+          l[q] = l[0];
+        }
+        jrow[q] = first_row + (ch * 64 + l[q]) * row_step;
+        rows[q] = c.dom + (int64_t)jrow[q] * c.wstride;
+        nws[q] = row_words(jrow[q]);
+      }
+      stat_rows += cnt;
+      ++stat_rounds;
+      RowScan r[4];
+      const bool short_rows = nws[0] <= 512 && nws[1] <= 512 && nws[2] <= 512 && nws[3] <= 512;
+      if (cnt > 2 && short_rows) {
+        const uint64_t* const four[4] = {rows[0], rows[1], rows[2], rows[3]};
+        scan_rows<true, 4, 4>(four, nws, alive_lds, r);
+      } else {
+        for (int q0 = 0; q0 < cnt; q0 += 2) {
+          const uint64_t* const two[2] = {rows[q0], rows[q0 + 1]};
+          const int nw2[2] = {nws[q0], nws[q0 + 1]};
+          RowScan r2[2];
+          if (short_rows)
+            scan_rows<true, 2, 4>(two, nw2, alive_lds, r2);
+          else
+            scan_rows<true, 2, 8>(two, nw2, alive_lds, r2);
+          r[q0] = r2[0];
+          r[q0 + 1] = r2[1];
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (q < cnt) {
+          if (lane == l[q]) {
+            st.word[ch] = r[q].last_word;
+            st.bits[ch] = r[q].last_bits;
+            if (r[q].last_word < 0) publish_ranked(c, jrow[q], st.orig[ch]);
+          }
+          found += r[q].last_word < 0;
+        }
+      }
+    }
+  }
+  EVX_RESCAN(c.next_level - 1, stat_rows, stat_rounds);
+  (void)stat_rows;
+  (void)stat_rounds;
+  return found;
+}
+
 // Block-wide listing of the set bits of `front` (nwords words, LDS) in ascending order into
-// perm[base ...].  `scratch` holds blockDim.x ints.
+// perm[base ...].  `scratch` holds at least blockDim.x / 64 ints.
 __device__ inline void list_front(const uint64_t* front_lds, int nwords, int* __restrict__ perm, int base, int* scratch) {
   // each thread owns a contiguous slice of words so that the order is ascending
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
   const int per = (nwords + blockDim.x - 1) / blockDim.x;
   const int w_begin = threadIdx.x * per;
   const int w_end = min(nwords, w_begin + per);
   int mine = 0;
   for (int w = w_begin; w < w_end; ++w) mine += __popcll(front_lds[w]);
-  scratch[threadIdx.x] = mine;
-  __syncthreads();
-  // inclusive scan over blockDim.x partial sums (Hillis-Steele)
-  for (int off = 1; off < (int)blockDim.x; off <<= 1) {
-    const int add = threadIdx.x >= (unsigned)off ? scratch[threadIdx.x - off] : 0;
-    __syncthreads();
-    scratch[threadIdx.x] += add;
-    __syncthreads();
+  // inclusive scan inside the wave, then across the (few) waves through LDS
+  int incl = mine;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
   }
-  int pos = base + scratch[threadIdx.x] - mine;
+  if (lane == 63) scratch[wave] = incl;
+  __syncthreads();
+  int pos = base + incl - mine;
+  for (int v = 0; v < wave; ++v) pos += scratch[v];
   for (int w = w_begin; w < w_end; ++w) {
     uint64_t bits = front_lds[w];
     while (bits) {
@@ -189,43 +439,86 @@ __device__ inline void list_front(const uint64_t* front_lds, int nwords, int* __
 
 // --------------------------------------------------------- persistent peel
 
-// fronts: three buffers of nwords words (front of the pass, front being built, buffer being cleared).
-// fsize[r]: size of front r (fsize[0] and fronts[0] come from count_kernel; the rest must be zero).
-// perm / fstart may be null when only ranks are wanted.
-// Stops as soon as the fronts listed so far hold stop_count rows (stop_count = n ranks everything).
+// fronts_slot / fronts_orig: kFrontBuffers bitmaps of nwords words each (kFrontStride apart); front r lives in buffer
+// r % kFrontBuffers of both (slot space for the passes, original-index space for the listing).
+// fsize[0] and buffer 0 come from count_kernel; the other buffers must be zero.
+// perm may be null when only ranks are wanted.
+// Stops as soon as the fronts built so far hold stop_count rows (stop_count = n ranks everything).
+// use_witness selects the witness pass (needs 2 * nwords words of LDS and at most
+// kWitnessChunks * 64 rows per sweeping wave) instead of the popcount sweep (nwords words of LDS).
+// The host launches at least three blocks (master, lister, one sweeper), all resident at once.
 __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __restrict__ dom, int64_t wstride, int nwords,
-                                                             int n, int* __restrict__ count, int* __restrict__ rank,
-                                                             uint64_t* __restrict__ fronts, int* __restrict__ fsize,
+                                                             int n, const int* __restrict__ orig_of, int* __restrict__ count,
+                                                             int* __restrict__ rank, uint64_t* __restrict__ fronts_slot,
+                                                             uint64_t* __restrict__ fronts_orig, int* __restrict__ fsize,
                                                              int* __restrict__ perm, int* __restrict__ fstart,
-                                                             Ctrl* __restrict__ ctrl, int stop_count, unsigned spin_limit) {
-  extern __shared__ uint64_t front_lds[];  // nwords words (nwords is even: rows are padded to 128)
+                                                             Ctrl* __restrict__ ctrl, int stop_count, unsigned spin_limit,
+                                                             const int* __restrict__ witness, int use_witness) {
+  extern __shared__ uint64_t front_lds[];  // nwords words (nwords is even: rows are padded to 128),
+                                           // followed by nwords more (unranked rows) in witness mode
   __shared__ int scratch[kPeelThreads];
-  const int waves_per_block = blockDim.x >> 6;
-  // block 0 keeps the books, blocks 1 .. gridDim.x-1 sweep (the host launches at least two blocks)
-  const int sweep_blocks = gridDim.x - 1;
-  const int sweep_block = (int)blockIdx.x - 1;
-  const int row_step = sweep_blocks * waves_per_block;
-  const int first_row = sweep_block * waves_per_block + (threadIdx.x >> 6);
 
-  int level = 0;
-  int ranked = 0;  // rows in fronts 0 .. level-1
-  for (;;) {
-    uint64_t* cur = fronts + (int64_t)(level % 3) * nwords;
-    uint64_t* nxt = fronts + (int64_t)((level + 1) % 3) * nwords;
-    uint64_t* old = fronts + (int64_t)((level + 2) % 3) * nwords;
-    const int size = coherent_load(&fsize[level]);
-    if (size <= 0) break;  // cannot happen for 1 <= stop_count <= n: a finite partial order has minimal rows
-    const bool last = ranked + size >= stop_count;
-    if (!last || blockIdx.x == 0) {
-      for (int w = threadIdx.x; w < nwords; w += blockDim.x) front_lds[w] = coherent_load(&cur[w]);
-      __syncthreads();
+  if (blockIdx.x == 0) {
+    // ---- master: nothing but the barrier
+    int level = 0, ranked = 0;
+    int size = coherent_load(&fsize[0]);
+    for (;;) {
+      if (size <= 0 || ranked + size >= stop_count) break;
+      ranked += size;
+      ++level;
+      // pass `level` fills the bitmaps that held front level + 1 - kFrontBuffers: that front and all
+      // before it must have been listed and cleared
+      if (!master_barrier(ctrl, (unsigned)level, level + 2 - kFrontBuffers, &size, spin_limit, scratch)) break;
     }
-    if (blockIdx.x == 0) {
+    return;
+  }
+
+  if (blockIdx.x == 1) {
+    // ---- lister: for each finished front, in order: list its rows (ascending original index) into
+    // perm, which makes perm a stable ordering by rank; record where the front starts; clear the
+    // bitmaps of the front before it for reuse.
+    int ranked = 0;
+    for (int level = 0;; ++level) {
+      if (level > 0) {
+        const unsigned long long want = (unsigned long long)level << 32;
+        if (threadIdx.x == 0) {
+          if (!bounded_wait([&] { return coherent_load(&ctrl->release) >= want || coherent_load(&ctrl->err) != 0; }, spin_limit))
+            coherent_store(&ctrl->err, kErrBarrierTimeout);
+          scratch[48] = coherent_load(&ctrl->err);
+        }
+        __syncthreads();
+        const bool bad = scratch[48] != 0;
+        __syncthreads();
+        if (bad) return;
+        // The sweepers have now finished the pass that read front level-1: its bitmaps can be cleared.
+        uint64_t* prev_slot = fronts_slot + (int64_t)((level - 1) % kFrontBuffers) * nwords * kFrontStride;
+        uint64_t* prev_orig = fronts_orig + (int64_t)((level - 1) % kFrontBuffers) * nwords * kFrontStride;
+        for (int w = threadIdx.x; w < nwords; w += blockDim.x) {
+          coherent_store(&prev_slot[(int64_t)w * kFrontStride], (uint64_t)0);
+          coherent_store(&prev_orig[(int64_t)w * kFrontStride], (uint64_t)0);
+        }
+      }
+      const uint64_t* cur = fronts_orig + (int64_t)(level % kFrontBuffers) * nwords * kFrontStride;
+      int mine = 0;
+      for (int w = threadIdx.x; w < nwords; w += blockDim.x) {
+        const uint64_t fw = coherent_load(&cur[(int64_t)w * kFrontStride]);
+        front_lds[w] = fw;
+        mine += __popcll(fw);
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) mine += __shfl_xor(mine, off);
+      if ((threadIdx.x & 63) == 0) scratch[32 + (threadIdx.x >> 6)] = mine;
+      __syncthreads();  // also waits for the clearing stores of this block's waves
+      int size = 0;
+      for (int v = 0; v < (int)(blockDim.x >> 6); ++v) size += scratch[32 + v];
+      if (threadIdx.x == 0) coherent_store(&ctrl->listed, level);  // fronts 0 .. level-1 are cleared
       if (perm) list_front(front_lds, nwords, perm, ranked, scratch);
+      const bool last = size <= 0 || ranked + size >= stop_count;
       if (threadIdx.x == 0) {
-        if (fstart) fstart[level] = ranked;
+        fstart[level] = ranked;
+        if (level > 0) fsize[level] = size;
         if (last) {
-          if (fstart) fstart[level + 1] = ranked + size;
+          fstart[level + 1] = ranked + size;
           ctrl->nfronts = level + 1;
           ctrl->worst = level;
           ctrl->worst_start = ranked;
@@ -234,25 +527,64 @@ __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __re
           ctrl->passes = level;
         }
       }
-      if (!last)
-        for (int w = threadIdx.x; w < nwords; w += blockDim.x) coherent_store(&old[w], (uint64_t)0);
-    }
-    if (last) break;
-    if (blockIdx.x != 0) {
-      const int found = sweep_rows(dom, wstride, nwords, n, front_lds, count, rank, nxt, level + 1, first_row, row_step);
-      // lane 0 of each wave holds that wave's tally: one atomic per block
+      if (last) return;
+      ranked += size;
       __syncthreads();
-      scratch[threadIdx.x] = found;
-      __syncthreads();
-      if (threadIdx.x == 0) {
-        int total = 0;
-        for (int t = 0; t < (int)blockDim.x; t += 64) total += scratch[t];
-        if (total) atomicAdd(&fsize[level + 1], total);
-      }
     }
+  }
+
+  // ---- sweepers
+  uint64_t* alive_lds = front_lds + nwords;
+  const int waves_per_block = blockDim.x >> 6;
+  const int sweep_blocks = gridDim.x - kFirstSweeper;
+  const int sweep_block = (int)blockIdx.x - kFirstSweeper;
+  const int row_step = sweep_blocks * waves_per_block;
+  const int first_row = sweep_block * waves_per_block + (threadIdx.x >> 6);
+  PassCtx c;
+  c.dom = dom;
+  c.wstride = wstride;
+  c.n = n;
+  c.orig_of = orig_of;
+  c.rank = rank;
+  WitnessState st;
+  if (use_witness) {
+    witness_load(st, c, witness, first_row, row_step);
+    for (int w = threadIdx.x; w < nwords; w += blockDim.x) {
+      const int lo = w * 64;
+      alive_lds[w] = lo + 64 <= n ? ~0ull : (lo >= n ? 0ull : ((1ull << (n - lo)) - 1ull));
+    }
+  }
+  int level = 0;
+  int ranked = 0;                        // rows in fronts 0 .. level-1
+  int size = coherent_load(&fsize[0]);   // size of front `level`
+  for (;;) {
+    EVX_TRACE(level, 0);
+    if (size <= 0 || ranked + size >= stop_count) break;  // size 0 cannot happen for 1 <= stop_count <= n
+    const uint64_t* cur = fronts_slot + (int64_t)(level % kFrontBuffers) * nwords * kFrontStride;
+    c.next_slot = fronts_slot + (int64_t)((level + 1) % kFrontBuffers) * nwords * kFrontStride;
+    c.next_orig = fronts_orig + (int64_t)((level + 1) % kFrontBuffers) * nwords * kFrontStride;
+    c.next_level = level + 1;
+    for (int w = threadIdx.x; w < nwords; w += blockDim.x) {
+      const uint64_t fw = coherent_load(&cur[(int64_t)w * kFrontStride]);
+      if (use_witness)
+        alive_lds[w] &= ~fw;
+      else
+        front_lds[w] = fw;
+    }
+    __syncthreads();
+    EVX_TRACE(level, 1);
+    const int found = use_witness ? witness_rows(st, c, alive_lds, first_row, row_step)
+                                  : sweep_rows(c, front_lds, count, first_row, row_step);
+    EVX_TRACE(level, 2);
+    // every lane of a wave holds that wave's tally
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = found;
+    __syncthreads();
+    int tally = 0;
+    for (int v = 0; v < waves_per_block; ++v) tally += scratch[v];
+    EVX_TRACE(level, 3);
     ranked += size;
     ++level;
-    if (!grid_barrier(ctrl, (unsigned)level, spin_limit)) break;
+    if (!sweeper_barrier(ctrl, (unsigned)level, tally, &size, spin_limit, scratch + 64)) break;
   }
 }
 

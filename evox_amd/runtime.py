@@ -75,9 +75,9 @@ def set_option(name: str, value: int) -> None:
 
 def workspace_views(ws: torch.Tensor, n: int, m: int) -> dict:
     """Typed views of the workspace regions (for tests and tools)."""
-    out = (ctypes.c_int64 * 10)()
+    out = (ctypes.c_int64 * 11)()
     _lib.call("evox_hip_workspace_layout", n, m, out)
-    dom_off, wstride, nwords, count, rank, dist, perm, fstart, order, ctrl = list(out)
+    dom_off, wstride, nwords, count, rank, dist, perm, fstart, order, ctrl, orig_of = list(out)
 
     def view(off, count_, dtype):
         size = torch.empty((), dtype=dtype).element_size()
@@ -93,4 +93,5 @@ def workspace_views(ws: torch.Tensor, n: int, m: int) -> dict:
         "fstart": view(fstart, n + 2, torch.int32),
         "order": view(order, n, torch.int32),
         "ctrl": view(ctrl, 16, torch.int32),
+        "orig_of": view(orig_of, n, torch.int32),
     }

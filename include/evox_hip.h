@@ -70,8 +70,8 @@ int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int6
  * They operate on the state left in the workspace by the previous stage, in this order:
  *   dominance -> count -> peel -> (crowding -> order -> gather).                                   */
 
-/* Fitness -> structure-of-arrays copy + row keys, clears the small state, then the pairwise
- * dominance bit matrix (non_dominate.py:6-26).  variant 0 = production kernel, 1 = check kernel that
+/* Fitness -> structure-of-arrays copy + row keys, clears the small state, sorts the rows into slots
+ * by key, then the pairwise dominance bit matrix (non_dominate.py:6-26).  variant 0 = production kernel, 1 = check kernel that
  * evaluates both `<=` and `<` per objective as the reference does. */
 int evox_hip_stage_dominance(const float* f, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col, int variant,
                              void* workspace, size_t workspace_bytes, void* stream);
@@ -91,8 +91,12 @@ int evox_hip_stage_order(int64_t n, int64_t m, void* workspace, size_t workspace
  *   out[0] dominance bit matrix (uint64, row j at + j * out[1] words)   out[1] row stride in words
  *   out[2] words per row in use      out[3] count (int32 n)             out[4] rank (int32 n)
  *   out[5] distance (float32 n)      out[6] rank-ordered listing (int32 n)
- *   out[7] front starts (int32 n+2)  out[8] selected order (int32 n)    out[9] control block      */
-int evox_hip_workspace_layout(int64_t n, int64_t m, int64_t* out10);
+ *   out[7] front starts (int32 n+2)  out[8] selected order (int32 n)    out[9] control block
+ *   out[10] slot -> original row index (int32 n)
+ * The bit matrix and the counts are indexed by SLOT (rows relabelled by ascending row key, which makes
+ * the matrix strictly lower triangular): bit b of word w of row s says that the row in slot 64 w + b
+ * dominates the row in slot s.  Ranks, distances, listings and the order use original row indices. */
+int evox_hip_workspace_layout(int64_t n, int64_t m, int64_t* out11);
 
 /* Waits for `stream`, then copies the control block's eight leading ints to HOST memory:
  * out[0] error (0 or EVOX_HIP_E_BARRIER_TIMEOUT), out[1] fronts peeled, out[2] last front's rank,
@@ -100,8 +104,8 @@ int evox_hip_workspace_layout(int64_t n, int64_t m, int64_t* out10);
  * Returns out[0] when it is non-zero. */
 int evox_hip_read_status(const void* workspace, void* stream, int32_t* host_out8);
 
-/* Tunables (process-wide): "peel_blocks_per_cu" (default 2), "spin_limit" (polls before a device-side
- * wait gives up, default 4000000), "dominance_tile_words" (16). */
+/* Tunables (process-wide): "peel_blocks_per_cu" (default 2), "peel_witness" (1 = witness pass, 0 = popcount sweep), "spin_limit" (polls before a device-side
+ * wait gives up, default 4000000), "dominance_tile_words" (4 or 16, default 4). */
 int evox_hip_set_option(const char* name, int64_t value);
 
 #ifdef __cplusplus

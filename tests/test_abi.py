@@ -42,10 +42,10 @@ def test_workspace_size_and_layout(handle):
     assert handle.evox_hip_workspace_bytes(10, 0) == 0
     b = handle.evox_hip_workspace_bytes(20000, 3)
     # dominated by the bit matrix: 20000 rows x 320 words (313 rounded up to a 128-byte multiple)
-    assert 20000 * 320 * 8 <= b <= 20000 * 320 * 8 + 4 * 2**20
+    assert 20000 * 320 * 8 <= b <= 20000 * 320 * 8 + 6 * 2**20
     b5 = handle.evox_hip_workspace_bytes(200000, 8)
     assert 5.0e9 < b5 < 5.3e9
-    out = (ctypes.c_int64 * 10)()
+    out = (ctypes.c_int64 * 11)()
     assert handle.evox_hip_workspace_layout(20000, 3, out) == 0
     assert out[1] == 320 and out[2] == 314 and out[0] % 256 == 0 and out[9] == 0
 
