@@ -27,7 +27,7 @@ struct Layout {
   int64_t wstride;
   // byte offsets
   size_t ctrl, fsize, fronts_slot, fronts_orig, hist, zero_end, fstart, xs, key, partials, sortparam, bstart, bcursor,
-      members, xs_sorted, key_sorted, orig_of, count, witness, rank, dist, perm, order, ukey, pos, scost, dkey, dom, total;
+      scanflags, members, xs_sorted, key_sorted, orig_of, count, witness, rank, dist, perm, order, ukey, pos, scost, dkey, dom, total;
 };
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
@@ -52,6 +52,7 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->fronts_slot = o; o = align_up(o + sizeof(uint64_t) * kFrontBuffers * kFrontStride * (size_t)L->nwords);
   L->fronts_orig = o; o = align_up(o + sizeof(uint64_t) * kFrontBuffers * kFrontStride * (size_t)L->nwords);
   L->hist = o;        o = align_up(o + sizeof(int) * (size_t)buckets);
+  L->scanflags = o;   o = align_up(o + sizeof(unsigned long long) * 64);
   L->zero_end = o;
   L->fstart = o;     o = align_up(o + sizeof(int) * (size_t)(n + 2));
   L->xs = o;         o = align_up(o + sizeof(float) * (size_t)m * L->npad);
@@ -163,8 +164,8 @@ static int stage_prepare(const Ws& w, const float* f, int64_t sr, int64_t sc, bo
                      w.at<unsigned long long>(L.partials), L.prep_blocks, L.buckets, w.at<int>(L.hist),
                      w.at<SortParam>(L.sortparam));
   EVX_LAUNCH_CHECK();
-  hipLaunchKernelGGL(bucket_scan_kernel, dim3(1), dim3(1024), 0, s, w.at<int>(L.hist), L.buckets, w.at<int>(L.bstart),
-                     w.at<int>(L.bcursor));
+  hipLaunchKernelGGL(bucket_scan_kernel, dim3(L.buckets / 1024), dim3(256), 0, s, w.at<int>(L.hist), L.buckets,
+                     w.at<int>(L.bstart), w.at<int>(L.bcursor), w.at<unsigned long long>(L.scanflags), g_opt.spin_limit);
   EVX_LAUNCH_CHECK();
   hipLaunchKernelGGL(bucket_scatter_kernel, dim3(blocks), dim3(256), 0, s, w.at<uint64_t>(L.key), L.n,
                      w.at<SortParam>(L.sortparam), w.at<int>(L.bcursor), w.at<int>(L.members));
@@ -277,11 +278,8 @@ static int stage_crowding(const Ws& w, const int* list, bool want_dkey, hipStrea
   const Layout& L = w.L;
   int qblocks = (L.kstride + 255) / 256;
   if (qblocks > 4096) qblocks = 4096;
-  hipLaunchKernelGGL(crowd_keys_kernel, dim3(qblocks, L.m), dim3(256), 0, s, w.at<float>(L.xs), L.npad, list, w.ctrl(),
-                     w.at<uint32_t>(L.ukey), L.kstride);
-  EVX_LAUNCH_CHECK();
   hipLaunchKernelGGL(crowd_rank_kernel, dim3(qblocks, L.m), dim3(256), 0, s, w.at<float>(L.xs), L.npad, list, w.ctrl(),
-                     w.at<uint32_t>(L.ukey), L.kstride, w.at<int>(L.pos), w.at<float>(L.scost));
+                     L.kstride, w.at<int>(L.pos), w.at<float>(L.scost));
   EVX_LAUNCH_CHECK();
   hipLaunchKernelGGL(crowd_dist_kernel, dim3(qblocks), dim3(256), 0, s, list, w.ctrl(), L.m, w.at<int>(L.pos),
                      w.at<float>(L.scost), L.kstride, w.at<float>(L.dist),

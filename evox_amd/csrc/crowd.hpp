@@ -11,22 +11,13 @@
 // (ordered_key(cost), position in L): that is torch's stable ascending sort with NaN last and signed
 // zeros tied, restricted to the masked rows, which the reference puts first (non_dominate.py:215-221).
 // The ordering is computed as a rank by counting, pos(q) = #{q' : (key', q') < (key, q)}: every
-// candidate is compared with every other one with the partner's key coming from scalar loads, the
-// same lane = row / scalar = partner structure as the dominance kernel.  The counts give the sorted
-// position directly, with no passes that depend on one another.
+// candidate is compared with every other one, the partners streaming through LDS in tiles.  The
+// counts give the sorted position directly, with no passes that depend on one another.
 #pragma once
 
 #include "common.hpp"
 
 namespace evx {
-
-// acc += bit, the bit taken from a 64-lane mask.
-__device__ inline uint32_t add_bit(uint32_t acc, uint64_t mask) {
-  uint32_t r;
-  uint64_t carry_out;
-  asm("v_addc_co_u32_e64 %0, %1, %2, 0, %3" : "=v"(r), "=s"(carry_out) : "v"(acc), "s"(mask));
-  return r;
-}
 
 // Stable compaction of a boolean mask into an ascending list (one block; n is at most a few 10^5).
 // mask == nullptr selects every row.  Also fills dist with -inf and publishes nv in ctrl.
@@ -65,45 +56,52 @@ __global__ __launch_bounds__(1024) void compact_mask_kernel(const uint8_t* __res
   }
 }
 
-// ukey[k][q] = ordered_key(cost of candidate q in objective k); padding up to a multiple of 64 gets
-// the largest key so that it never counts as smaller.  grid = (blocks over q, m).
-__global__ __launch_bounds__(256) void crowd_keys_kernel(const float* __restrict__ xs, int npad, const int* __restrict__ list_base,
-                                                         const Ctrl* __restrict__ ctrl, uint32_t* __restrict__ ukey,
-                                                         int kstride) {
-  const int nv = ctrl->nv;
-  const int* __restrict__ list = list_base + ctrl->worst_start;
-  const int k = blockIdx.y;
-  const int nv_pad = (int)round_up(nv, 64);
-  for (int q = blockIdx.x * blockDim.x + threadIdx.x; q < nv_pad; q += gridDim.x * blockDim.x)
-    ukey[(int64_t)k * kstride + q] = q < nv ? ordered_key(xs[(int64_t)k * npad + list[q]]) : 0xFFFFFFFFu;
+// Position of a candidate among nv candidates ordered by (key, candidate index): the number of
+// candidates whose (key, index) pair is smaller.  The block's 256 candidates each hold their own pair
+// in a register; the pairs of all candidates stream through LDS in tiles of kRankTile, loaded
+// cooperatively by `load_pair(q)`, and every thread compares its pair with the whole tile (LDS
+// broadcast reads, one 64-bit compare per partner).
+constexpr int kRankTile = 1024;
+
+template <class LoadPair>
+__device__ inline int rank_by_counting(uint64_t mine, int nv, LoadPair load_pair, uint64_t* tile_lds) {
+  int smaller = 0;
+  for (int t0 = 0; t0 < nv; t0 += kRankTile) {
+    __syncthreads();
+    for (int e = threadIdx.x; e < kRankTile; e += blockDim.x) tile_lds[e] = t0 + e < nv ? load_pair(t0 + e) : ~0ull;
+    __syncthreads();
+    // 16 partners per step, their LDS reads issued together (entries past nv hold all-ones)
+    const int lim = min(kRankTile, (int)round_up(nv - t0, 16));
+    for (int e = 0; e < lim; e += 16) {
+      ulonglong2 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const ulonglong2*>(tile_lds + e + 2 * u);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) smaller += (v[u].x < mine) + (v[u].y < mine);
+    }
+  }
+  return smaller;
 }
 
 // pos[k][q] = sorted position of candidate q in objective k; sorted_cost[k][pos] = its cost.
-// grid = (blocks over q, m); waves whose 64 candidates lie past nv leave at once.
+// grid = (blocks over q, m); blocks whose candidates lie past nv leave at once.
 __global__ __launch_bounds__(256) void crowd_rank_kernel(const float* __restrict__ xs, int npad, const int* __restrict__ list_base,
-                                                         const Ctrl* __restrict__ ctrl, const uint32_t* __restrict__ ukey,
-                                                         int kstride, int* __restrict__ pos, float* __restrict__ sorted_cost) {
+                                                         const Ctrl* __restrict__ ctrl, int kstride, int* __restrict__ pos,
+                                                         float* __restrict__ sorted_cost) {
+  __shared__ uint64_t tile_lds[kRankTile];
   const int nv = ctrl->nv;
   const int* __restrict__ list = list_base + ctrl->worst_start;
   const int k = blockIdx.y;
-  const uint32_t* __restrict__ keys = ukey + (int64_t)k * kstride;
-  const int nv_pad = (int)round_up(nv, 64);
-  const int waves = gridDim.x * (blockDim.x >> 6);
-  const int lane = threadIdx.x & 63;
-  for (int q0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 64; q0 < nv; q0 += waves * 64) {
-    const int q = q0 + lane;
-    const uint64_t mine = ((uint64_t)keys[q] << 32) | (uint32_t)q;  // q < nv_pad: keys are padded
-    uint32_t smaller = 0;
-    for (int p0 = 0; p0 < nv_pad; p0 += 8) {
-#pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        const uint64_t other = ((uint64_t)keys[p0 + t] << 32) | (uint32_t)(p0 + t);
-        smaller = add_bit(smaller, __builtin_amdgcn_ballot_w64(other < mine));
-      }
-    }
+  const float* __restrict__ col = xs + (int64_t)k * npad;
+  auto pair_of = [&](int q) { return ((uint64_t)ordered_key(col[list[q]]) << 32) | (uint32_t)q; };
+  for (int q0 = blockIdx.x * blockDim.x; q0 < nv; q0 += gridDim.x * blockDim.x) {
+    const int q = q0 + threadIdx.x;
+    const float cost = q < nv ? col[list[q]] : 0.0f;
+    const uint64_t mine = q < nv ? (((uint64_t)ordered_key(cost) << 32) | (uint32_t)q) : 0ull;
+    const int p = rank_by_counting(mine, nv, pair_of, tile_lds);
     if (q < nv) {
-      pos[(int64_t)k * kstride + q] = (int)smaller;
-      sorted_cost[(int64_t)k * kstride + smaller] = xs[(int64_t)k * npad + list[q]];
+      pos[(int64_t)k * kstride + q] = p;
+      sorted_cost[(int64_t)k * kstride + p] = cost;
     }
   }
 }
@@ -146,29 +144,21 @@ __global__ __launch_bounds__(256) void crowd_dist_kernel(const int* __restrict__
 // Index-stable top-k on the last front: candidate q goes to place #{q' : (dkey', q') < (dkey, q)}
 // (distance descending, NaN after every number, then row index; jit_fix_operator.py:246-252 applied
 // to non_dominate.py:253) and is kept when that place is below `need`.  The better fronts are copied
-// from the rank-ordered listing.  grid.x covers max(n / 64 waves, copy work).
+// from the rank-ordered listing.
 __global__ __launch_bounds__(256) void final_order_kernel(const int* __restrict__ perm, const Ctrl* __restrict__ ctrl,
                                                           const uint32_t* __restrict__ dkey, int* __restrict__ order) {
+  __shared__ uint64_t tile_lds[kRankTile];
   const int nv = ctrl->nv;
   const int start = ctrl->worst_start;
   const int need = ctrl->need;
   const int* __restrict__ list = perm + start;
-  const int nv_pad = (int)round_up(nv, 64);
-  const int waves = gridDim.x * (blockDim.x >> 6);
-  const int lane = threadIdx.x & 63;
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < start; i += gridDim.x * blockDim.x) order[i] = perm[i];
-  for (int q0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 64; q0 < nv; q0 += waves * 64) {
-    const int q = q0 + lane;
-    const uint64_t mine = ((uint64_t)dkey[q] << 32) | (uint32_t)q;
-    uint32_t smaller = 0;
-    for (int p0 = 0; p0 < nv_pad; p0 += 8) {
-#pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        const uint64_t other = ((uint64_t)dkey[p0 + t] << 32) | (uint32_t)(p0 + t);
-        smaller = add_bit(smaller, __builtin_amdgcn_ballot_w64(other < mine));
-      }
-    }
-    if (q < nv && (int)smaller < need) order[start + smaller] = list[q];
+  auto pair_of = [&](int q) { return ((uint64_t)dkey[q] << 32) | (uint32_t)q; };
+  for (int q0 = blockIdx.x * blockDim.x; q0 < nv; q0 += gridDim.x * blockDim.x) {
+    const int q = q0 + threadIdx.x;
+    const uint64_t mine = q < nv ? pair_of(q) : 0ull;
+    const int p = rank_by_counting(mine, nv, pair_of, tile_lds);
+    if (q < nv && p < need) order[start + p] = list[q];
   }
 }
 

@@ -69,27 +69,19 @@ __global__ __launch_bounds__(256) void bucket_hist_kernel(const uint64_t* __rest
     atomicAdd(&hist[bucket_of(key[i], sp)], 1);
 }
 
-// One block: start[b] = exclusive prefix of hist, start[buckets] = n; cursor = copy of start.
-// Thread t owns the bins [t * per, (t + 1) * per), per = buckets / 1024 (a multiple of 4, at most
-// 64): it loads them with independent 16-byte loads, scans them in registers, and the 1024 thread
-// totals are scanned by wave shuffles.
-__global__ __launch_bounds__(1024) void bucket_scan_kernel(const int* __restrict__ hist, int buckets, int* __restrict__ start,
-                                                           int* __restrict__ cursor) {
-  __shared__ int wave_tot[16];
-  const int per = buckets / 1024;  // 1, 2, 4, ..., 64
-  const int b0 = threadIdx.x * per;
-  int4 v[16];
-  int mine = 0;
-  if (per >= 4) {
-#pragma unroll
-    for (int q = 0; q < 16; ++q) v[q] = q * 4 < per ? *reinterpret_cast<const int4*>(hist + b0 + q * 4) : make_int4(0, 0, 0, 0);
-#pragma unroll
-    for (int q = 0; q < 16; ++q) mine += v[q].x + v[q].y + v[q].z + v[q].w;
-  } else {
-    v[0] = make_int4(hist[b0], per > 1 ? hist[b0 + 1] : 0, 0, 0);
-    mine = v[0].x + v[0].y;
-  }
+// start[b] = exclusive prefix of hist, start[buckets] = n; cursor = copy of start.
+// One block of 256 threads per 1024 bins (at most 64 blocks, all resident): each block adds up its
+// bins, publishes (1 << 32 | total) in its flag, adds the totals of the blocks before it as they appear
+// (bounded polling; the flags start at zero), and then scans its own bins.
+__global__ __launch_bounds__(256) void bucket_scan_kernel(const int* __restrict__ hist, int buckets, int* __restrict__ start,
+                                                          int* __restrict__ cursor, unsigned long long* __restrict__ flags,
+                                                          unsigned spin_limit) {
+  __shared__ int wave_tot[4];
+  __shared__ int base_lds;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int b0 = blockIdx.x * 1024 + threadIdx.x * 4;
+  const int4 v = *reinterpret_cast<const int4*>(hist + b0);
+  const int mine = v.x + v.y + v.z + v.w;
   int incl = mine;
 #pragma unroll
   for (int off = 1; off < 64; off <<= 1) {
@@ -98,32 +90,36 @@ __global__ __launch_bounds__(1024) void bucket_scan_kernel(const int* __restrict
   }
   if (lane == 63) wave_tot[wave] = incl;
   __syncthreads();
-  int run = incl - mine;
-  for (int w = 0; w < wave; ++w) run += wave_tot[w];
-  if (per >= 4) {
-#pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      if (q * 4 < per) {
-        int4 o;
-        o.x = run; run += v[q].x;
-        o.y = run; run += v[q].y;
-        o.z = run; run += v[q].z;
-        o.w = run; run += v[q].w;
-        *reinterpret_cast<int4*>(start + b0 + q * 4) = o;
-        *reinterpret_cast<int4*>(cursor + b0 + q * 4) = o;
+  const int block_total = wave_tot[0] + wave_tot[1] + wave_tot[2] + wave_tot[3];
+  if (threadIdx.x == 0)
+    __hip_atomic_store(&flags[blockIdx.x], (1ull << 32) | (unsigned)block_total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // the first wave gathers the totals of the preceding blocks (at most 63)
+  if (wave == 0) {
+    int before = 0;
+    if (lane < (int)blockIdx.x) {
+      unsigned long long f = 0;
+      unsigned spins = 0;
+      while (((f = __hip_atomic_load(&flags[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) == 0) {
+        if (++spins > spin_limit) break;  // cannot happen: every block is resident and publishes first
+        __builtin_amdgcn_s_sleep(1);
       }
+      before = (int)(unsigned)(f & 0xFFFFFFFFull);
     }
-  } else {
-    start[b0] = run;
-    cursor[b0] = run;
-    run += v[0].x;
-    if (per > 1) {
-      start[b0 + 1] = run;
-      cursor[b0 + 1] = run;
-      run += v[0].y;
-    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off);
+    if (lane == 0) base_lds = before;
   }
-  if (threadIdx.x == 1023) start[buckets] = run;
+  __syncthreads();
+  int run = base_lds + incl - mine;
+  for (int w = 0; w < wave; ++w) run += wave_tot[w];
+  int4 o;
+  o.x = run; run += v.x;
+  o.y = run; run += v.y;
+  o.z = run; run += v.z;
+  o.w = run; run += v.w;
+  *reinterpret_cast<int4*>(start + b0) = o;
+  *reinterpret_cast<int4*>(cursor + b0) = o;
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 255) start[buckets] = run;
 }
 
 __global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint64_t* __restrict__ key, int n,
