@@ -34,6 +34,9 @@ def parse():
     ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C5"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--cpu-sample", type=int, default=16000, help="rows of the workload timed on the CPU")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run a plain 512 MiB device copy three times, so that a rocprofv3 --pmc run of this "
+                         "command holds a kernel of known traffic next to the selection kernels")
     return ap.parse_args()
 
 
@@ -42,16 +45,18 @@ def median(xs):
     return xs[len(xs) // 2]
 
 
-def event_time_us(fn, reps):
-    """Median duration of fn() in microseconds, HIP events on the current stream."""
+def event_time_us(fn, reps, inner=4):
+    """Median duration of fn() in microseconds: HIP events on the current stream around `inner`
+    back-to-back calls, so that the launch latency of the first one is amortised."""
     out = []
     for _ in range(reps):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
-        fn()
+        for _ in range(inner):
+            fn()
         b.record()
         b.synchronize()
-        out.append(a.elapsed_time(b) * 1e3)
+        out.append(a.elapsed_time(b) * 1e3 / inner)
     return median(out)
 
 
@@ -64,8 +69,11 @@ def stage_profile(w, f, reps):
     s = runtime.stream_handle(f.device)
     tail = (ws.data_ptr(), ws.numel(), s)
 
+    def prep():
+        _lib.call("evox_hip_stage_prepare", f.data_ptr(), n, m, f.stride(0), f.stride(1), *tail)
+
     def dom():
-        _lib.call("evox_hip_stage_dominance", f.data_ptr(), n, m, f.stride(0), f.stride(1), 0, *tail)
+        _lib.call("evox_hip_stage_dominance", n, m, 0, *tail)
 
     def count():
         _lib.call("evox_hip_stage_count", n, m, *tail)
@@ -80,8 +88,9 @@ def stage_profile(w, f, reps):
         _lib.call("evox_hip_stage_order", n, m, *tail)
 
     times = {}
-    dom(); count(); peel(); crowd(); order()
+    prep(); dom(); count(); peel(); crowd(); order()
     torch.cuda.synchronize()
+    times["prepare_us"] = event_time_us(prep, reps)
     times["dominance_us"] = event_time_us(dom, reps)
     times["count_us"] = event_time_us(count, reps)
     # the peel consumes the counts, so each repetition re-runs count first and subtracts it
@@ -142,6 +151,14 @@ def main():
     x = (w.x if w.x is not None else w.f).to(dev)
     n, m = f.shape
 
+    if args.pmc_calibration:
+        src = torch.empty(512 * 2**20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     def step():
         return nd_environmental_selection(x, f, w.topk)
 
@@ -173,6 +190,7 @@ def main():
     dom_bytes = n * m * 4 + n * row_bytes
     count_bytes = int(row_read.sum()) + n * 12
     phases = {
+        "prepare_and_slot_sort": {"us": times["prepare_us"]},
         "dominance": {"us": times["dominance_us"], "bound": "valu", "achieved": compares / times["dominance_us"] / 1e3,
                       "peak": VALU_CMP_PEAK_GOPS, "unit": "Gcompare/s",
                       "hbm_GBs": dom_bytes / times["dominance_us"] / 1e3},

@@ -27,7 +27,8 @@ _SIGNATURES = {
     "evox_hip_nd_environmental_selection": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                                     c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                     c_size_t, c_void_p]),
-    "evox_hip_stage_dominance": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
+    "evox_hip_stage_prepare": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
+    "evox_hip_stage_dominance": (c_int, [c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
     "evox_hip_stage_count": (c_int, [c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "evox_hip_stage_peel": (c_int, [c_int64, c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "evox_hip_stage_crowding": (c_int, [c_int64, c_int64, c_void_p, c_size_t, c_void_p]),

@@ -179,9 +179,7 @@ static int stage_prepare(const Ws& w, const float* f, int64_t sr, int64_t sc, bo
   return 0;
 }
 
-static int stage_dominance(const Ws& w, const float* f, int64_t sr, int64_t sc, int variant, hipStream_t s) {
-  const Layout& L = w.L;
-  if (int e = stage_prepare(w, f, sr, sc, true, s)) return e;
+static int stage_dominance(const Ws& w, int variant, hipStream_t s) {
   // (the lower triangle in tiles of 4 words keeps every SIMD busy with several waves; 16 is kept for
   // measurements)
   const int tile = g_opt.dominance_tile_words;
@@ -348,11 +346,17 @@ int evox_hip_set_option(const char* name, int64_t value) {
   return 0;
 }
 
-int evox_hip_stage_dominance(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, int variant, void* ws,
-                             size_t ws_bytes, void* stream) {
+int evox_hip_stage_prepare(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, void* ws, size_t ws_bytes,
+                           void* stream) {
   Ws w;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
-  return stage_dominance(w, f, sr, sc, variant, (hipStream_t)stream);
+  return stage_prepare(w, f, sr, sc, true, (hipStream_t)stream);
+}
+
+int evox_hip_stage_dominance(int64_t n, int64_t m, int variant, void* ws, size_t ws_bytes, void* stream) {
+  Ws w;
+  if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
+  return stage_dominance(w, variant, (hipStream_t)stream);
 }
 
 int evox_hip_stage_count(int64_t n, int64_t m, void* ws, size_t ws_bytes, void* stream) {
@@ -394,7 +398,8 @@ int evox_hip_non_dominate_rank(const float* f, int64_t n, int64_t m, int64_t sr,
   if (rank_out == nullptr) return kErrBadArg;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   hipStream_t s = (hipStream_t)stream;
-  if (int e = stage_dominance(w, f, sr, sc, kDomKey64, s)) return e;
+  if (int e = stage_prepare(w, f, sr, sc, true, s)) return e;
+  if (int e = stage_dominance(w, kDomKey64, s)) return e;
   if (int e = stage_count(w, false, s)) return e;
   if (int e = stage_peel(w, n, false, s)) return e;
   return copy_async(rank_out, w.at<int>(w.L.rank), sizeof(int) * (size_t)n, s);
@@ -426,7 +431,8 @@ int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int6
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   const Layout& L = w.L;
   hipStream_t s = (hipStream_t)stream;
-  if (int e = stage_dominance(w, f, sr, sc, kDomKey64, s)) return e;
+  if (int e = stage_prepare(w, f, sr, sc, true, s)) return e;
+  if (int e = stage_dominance(w, kDomKey64, s)) return e;
   if (int e = stage_count(w, true, s)) return e;
   if (int e = stage_peel(w, topk, true, s)) return e;
   if (int e = stage_crowding(w, w.at<int>(L.perm), true, s)) return e;

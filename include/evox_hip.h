@@ -68,13 +68,15 @@ int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int6
 
 /* ---- stages of the calls above, exposed so that each kernel can be tested and timed alone.
  * They operate on the state left in the workspace by the previous stage, in this order:
- *   dominance -> count -> peel -> (crowding -> order -> gather).                                   */
+ *   prepare -> dominance -> count -> peel -> (crowding -> order -> gather).                                 */
 
 /* Fitness -> structure-of-arrays copy + row keys, clears the small state, sorts the rows into slots
- * by key, then the pairwise dominance bit matrix (non_dominate.py:6-26).  variant 0 = production kernel, 1 = check kernel that
- * evaluates both `<=` and `<` per objective as the reference does. */
-int evox_hip_stage_dominance(const float* f, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col, int variant,
-                             void* workspace, size_t workspace_bytes, void* stream);
+ * by key (a relabelling under which every dominator precedes the rows it dominates). */
+int evox_hip_stage_prepare(const float* f, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col, void* workspace,
+                           size_t workspace_bytes, void* stream);
+/* The pairwise dominance bit matrix (non_dominate.py:6-26) in slot space.  variant 0 = production
+ * kernel, 1 = check kernel that evaluates both `<=` and `<` per objective as the reference does. */
+int evox_hip_stage_dominance(int64_t n, int64_t m, int variant, void* workspace, size_t workspace_bytes, void* stream);
 /* Domination counts by row popcount (non_dominate.py:188) and front 0 (:192).  Resets the peeling
  * state first, so count -> peel can be repeated on one dominance matrix. */
 int evox_hip_stage_count(int64_t n, int64_t m, void* workspace, size_t workspace_bytes, void* stream);

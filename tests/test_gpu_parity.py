@@ -42,7 +42,8 @@ def run_stages(f, topk, variant=0):
     n, m = f.shape
     ws = runtime.workspace(n, m, f.device)
     s = runtime.stream_handle(f.device)
-    _lib.call("evox_hip_stage_dominance", f.data_ptr(), n, m, f.stride(0), f.stride(1), variant, ws.data_ptr(), ws.numel(), s)
+    _lib.call("evox_hip_stage_prepare", f.data_ptr(), n, m, f.stride(0), f.stride(1), ws.data_ptr(), ws.numel(), s)
+    _lib.call("evox_hip_stage_dominance", n, m, variant, ws.data_ptr(), ws.numel(), s)
     _lib.call("evox_hip_stage_count", n, m, ws.data_ptr(), ws.numel(), s)
     _lib.call("evox_hip_stage_peel", n, m, topk, None, ws.data_ptr(), ws.numel(), s)
     runtime.note_call(ws, s)
@@ -76,7 +77,8 @@ def test_dominance_bits_edge(name, f, ks, variant):
     n, m = f.shape
     ws = runtime.workspace(n, m, fd.device)
     s = runtime.stream_handle(fd.device)
-    _lib.call("evox_hip_stage_dominance", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), variant, ws.data_ptr(), ws.numel(), s)
+    _lib.call("evox_hip_stage_prepare", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), ws.data_ptr(), ws.numel(), s)
+    _lib.call("evox_hip_stage_dominance", n, m, variant, ws.data_ptr(), ws.numel(), s)
     _lib.call("evox_hip_stage_count", n, m, ws.data_ptr(), ws.numel(), s)
     torch.cuda.synchronize()
     views = runtime.workspace_views(ws, n, m)
@@ -102,8 +104,8 @@ def test_dominance_bits_all_m(m):
     s = runtime.stream_handle(fd.device)
     want = as_np(er.pareto_dominance(f, f)).T
     for variant in ([0, 1] if m <= 8 else [0]):
-        _lib.call("evox_hip_stage_dominance", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), variant, ws.data_ptr(),
-                  ws.numel(), s)
+        _lib.call("evox_hip_stage_prepare", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), ws.data_ptr(), ws.numel(), s)
+        _lib.call("evox_hip_stage_dominance", n, m, variant, ws.data_ptr(), ws.numel(), s)
         torch.cuda.synchronize()
         got = unpack_bits(runtime.workspace_views(ws, n, m), n)
         assert np.array_equal(got, want), (m, variant)
@@ -118,8 +120,8 @@ def test_dominance_variants_agree_c3():
     s = runtime.stream_handle(fd.device)
     doms = []
     for variant in (0, 1):
-        _lib.call("evox_hip_stage_dominance", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), variant, ws.data_ptr(),
-                  ws.numel(), s)
+        _lib.call("evox_hip_stage_prepare", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), ws.data_ptr(), ws.numel(), s)
+        _lib.call("evox_hip_stage_dominance", n, m, variant, ws.data_ptr(), ws.numel(), s)
         v = runtime.workspace_views(ws, n, m)
         doms.append(v["dom"][:, : v["nwords"]].clone())
     assert torch.equal(doms[0], doms[1])
