@@ -4,6 +4,7 @@
 #include <string.h>
 
 #include "../../include/evox_hip.h"
+#include "batched.hpp"
 #include "common.hpp"
 #include "crowd.hpp"
 #include "dominance.hpp"
@@ -300,6 +301,48 @@ static int copy_async(void* dst, const void* src, size_t bytes, hipStream_t s) {
   return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s);
 }
 
+template <int M>
+static int launch_batched_m(const BatchedArgs& a, int64_t batch, hipStream_t s) {
+  const int nt = (int)round_up(a.n, 64);
+  const size_t lds = batched_lds_bytes(nt);
+  static size_t granted = 0;
+  if (lds > 48 * 1024 && lds > granted) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(batched_kernel<M>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    granted = lds;
+  }
+  // grid.x carries the batch; very large batches go in slices
+  for (int64_t b0 = 0; b0 < batch; b0 += 0x40000000ll) {
+    BatchedArgs part = a;
+    const int64_t nb = batch - b0 < 0x40000000ll ? batch - b0 : 0x40000000ll;
+    part.f += b0 * a.f_stride_b;
+    if (part.rank_all) part.rank_all += b0 * a.n;
+    if (part.x) part.x += b0 * a.x_stride_b;
+    if (part.out_x) part.out_x += b0 * a.stop_count * a.x_row_bytes;
+    if (part.out_f) part.out_f += b0 * a.stop_count * a.m;
+    if (part.out_rank) part.out_rank += b0 * a.stop_count;
+    if (part.out_dist) part.out_dist += b0 * a.stop_count;
+    hipLaunchKernelGGL(batched_kernel<M>, dim3((unsigned)nb), dim3(nt), lds, s, part);
+    EVX_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+static int launch_batched(const BatchedArgs& a, int64_t batch, hipStream_t s) {
+  switch (a.m) {
+    case 1: return launch_batched_m<1>(a, batch, s);
+    case 2: return launch_batched_m<2>(a, batch, s);
+    case 3: return launch_batched_m<3>(a, batch, s);
+    case 4: return launch_batched_m<4>(a, batch, s);
+    case 5: return launch_batched_m<5>(a, batch, s);
+    case 6: return launch_batched_m<6>(a, batch, s);
+    case 7: return launch_batched_m<7>(a, batch, s);
+    case 8: return launch_batched_m<8>(a, batch, s);
+    default: return kErrBadArg;
+  }
+}
+
 }  // namespace evx
 
 using namespace evx;
@@ -452,6 +495,56 @@ int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int6
   EVX_LAUNCH_CHECK();
   if (out_order) return copy_async(out_order, w.at<int>(L.order), sizeof(int) * (size_t)topk, s);
   return 0;
+}
+
+int64_t evox_hip_batched_max_rows(int64_t m) { return (m >= 1 && m <= 8) ? kBatchedMaxRows : 0; }
+
+int evox_hip_batched_non_dominate_rank(const float* f, int64_t batch, int64_t n, int64_t m, int64_t stride_batch,
+                                       int64_t stride_row, int64_t stride_col, int32_t* rank_out, void* stream) {
+  if (f == nullptr || rank_out == nullptr || batch < 1 || n < 1 || n > kBatchedMaxRows || m < 1 || m > 8) return kErrBadArg;
+  BatchedArgs a = {};
+  a.f = f;
+  a.f_stride_b = stride_batch;
+  a.f_stride_row = stride_row;
+  a.f_stride_col = stride_col;
+  a.n = (int)n;
+  a.m = (int)m;
+  a.stop_count = (int)n;
+  a.rank_all = rank_out;
+  return launch_batched(a, batch, (hipStream_t)stream);
+}
+
+int evox_hip_batched_nd_environmental_selection(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes,
+                                                int64_t x_batch_stride_bytes, const float* f, int64_t batch, int64_t n,
+                                                int64_t m, int64_t stride_batch, int64_t stride_row, int64_t stride_col,
+                                                int64_t topk, void* out_x, float* out_f, int32_t* out_rank, float* out_dist,
+                                                void* stream) {
+  if (f == nullptr || out_f == nullptr || out_rank == nullptr || out_dist == nullptr) return kErrBadArg;
+  if (batch < 1 || n < 1 || n > kBatchedMaxRows || m < 1 || m > 8 || topk < 1 || topk > n) return kErrBadArg;
+  if ((x == nullptr) != (out_x == nullptr) || (x != nullptr && (x_row_bytes < 0 || x_row_stride_bytes < 0))) return kErrBadArg;
+  BatchedArgs a = {};
+  a.f = f;
+  a.f_stride_b = stride_batch;
+  a.f_stride_row = stride_row;
+  a.f_stride_col = stride_col;
+  a.n = (int)n;
+  a.m = (int)m;
+  a.stop_count = (int)topk;
+  a.x = static_cast<const uint8_t*>(x);
+  a.x_stride_b = x_batch_stride_bytes;
+  a.x_row_stride = x_row_stride_bytes;
+  a.x_row_bytes = x_row_bytes;
+  a.out_x = static_cast<uint8_t*>(out_x);
+  a.out_f = out_f;
+  a.out_rank = out_rank;
+  a.out_dist = out_dist;
+  a.x_unit = 1;
+  if (x != nullptr) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out_x) | (uintptr_t)x_row_bytes |
+                           (uintptr_t)x_row_stride_bytes | (uintptr_t)x_batch_stride_bytes;
+    a.x_unit = (bits % 16 == 0) ? 16 : (bits % 4 == 0) ? 4 : 1;
+  }
+  return launch_batched(a, batch, (hipStream_t)stream);
 }
 
 int evox_hip_read_status(const void* ws, void* stream, int32_t* host_out8) {

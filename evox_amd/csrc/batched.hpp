@@ -1,0 +1,234 @@
+// Many small populations at once: one workgroup per population, everything in LDS.
+//
+// This is the batched form of the same path (what the reference reaches through vmap:
+// src/evox/operators/selection/non_dominate.py:107-125 for the peeling, :198-254 under vmap for
+// the rest).  Per population the result is identical to the single-population kernels.
+//
+// Thread j owns row j of its population (blockDim.x = rows rounded up to 64, at most 1024).
+//   * dominance: lane = dominated row j, loop over dominators i whose fitness comes from scalar loads
+//     (wave-uniform address), `<=` and `<` per objective exactly as non_dominate.py:20-24, masks
+//     combined on the scalar unit and shifted into the lane's word with v_addc_co_u32; the 64-bit
+//     words of row j go to LDS (row stride W + 1 words against bank conflicts);
+//   * counts = popcount of the row; peeling = count -= popcount(row & front) with the front bitmap in
+//     LDS and two block barriers per pass; fronts are listed in ascending row order as they appear;
+//   * crowding distance and the index-stable top-k on the last front by counting ranks over LDS tiles;
+//   * the selected rows are gathered by the whole block.
+#pragma once
+
+#include "common.hpp"
+#include "dominance.hpp"
+
+namespace evx {
+
+constexpr int kBatchedMaxRows = 1024;
+
+struct BatchedArgs {
+  const float* f;          // (batch, n, m) with strides in elements
+  int64_t f_stride_b, f_stride_row, f_stride_col;
+  int n, m;
+  int stop_count;          // rows to rank before stopping (n = rank everything)
+  int* rank_all;           // (batch, n) ranks of all rows, or null
+  // selection outputs (all null in rank-only mode)
+  const uint8_t* x;        // (batch, n, row_bytes) raw rows, or null
+  int64_t x_stride_b, x_row_stride, x_row_bytes;
+  int x_unit;              // 16, 4 or 1: copy granularity that pointers, strides and row size allow
+  uint8_t* out_x;          // (batch, topk, row_bytes)
+  float* out_f;            // (batch, topk, m)
+  int* out_rank;           // (batch, topk)
+  float* out_dist;         // (batch, topk)
+};
+
+// Number of elements of `tile` (nv entries, (key << 32 | index) pairs) that are smaller than `mine`.
+__device__ inline int count_smaller(const uint64_t* tile, int nv, uint64_t mine) {
+  int smaller = 0;
+  const int lim = (nv + 3) & ~3;  // the tile is padded with all-ones up to a multiple of 4
+  for (int e = 0; e < lim; e += 4) {
+    const ulonglong2 a = *reinterpret_cast<const ulonglong2*>(tile + e);
+    const ulonglong2 b = *reinterpret_cast<const ulonglong2*>(tile + e + 2);
+    smaller += (a.x < mine) + (a.y < mine) + (b.x < mine) + (b.y < mine);
+  }
+  return smaller;
+}
+
+// Row stride of the LDS matrix in words: one word of padding against bank conflicts, except at the
+// largest size, where the padding would not fit.
+__host__ __device__ inline int batched_row_stride(int nt) { return nt == 1024 ? 16 : nt / 64 + 1; }
+
+// Dynamic LDS layout (nt = blockDim.x):
+//   uint64 dom[nt][row stride] | uint64 tile[nt + 4] | uint64 front[2][16] | float scost[nt] | float dist[nt] |
+//   int perm[nt] | int order[nt] | int rank[nt]
+__host__ __device__ inline size_t batched_lds_bytes(int nt) {
+  return sizeof(uint64_t) * ((size_t)nt * batched_row_stride(nt) + (nt + 4) + 32) + sizeof(float) * 2 * (size_t)nt +
+         sizeof(int) * 3 * (size_t)nt;
+}
+
+template <int M>
+__global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
+  extern __shared__ uint64_t lds64[];
+  const int nt = blockDim.x;
+  const int W = nt >> 6;
+  const int rs = batched_row_stride(nt);
+  uint64_t* dom = lds64;
+  uint64_t* tile = dom + (size_t)nt * rs;
+  uint64_t* front = tile + (nt + 4);
+  float* scost = reinterpret_cast<float*>(front + 32);
+  float* dist = scost + nt;
+  int* perm = reinterpret_cast<int*>(dist + nt);
+  int* order = perm + nt;
+  int* rank_lds = order + nt;
+
+  const int n = a.n;
+  const int j = threadIdx.x;
+  const int lane = j & 63;
+  const int wave = j >> 6;
+  const bool valid = j < n;
+  const float* __restrict__ f = a.f + (int64_t)blockIdx.x * a.f_stride_b;
+  const float nan = __uint_as_float(0x7FC00000u);
+
+  float xj[M];
+#pragma unroll
+  for (int k = 0; k < M; ++k) xj[k] = valid ? f[(int64_t)j * a.f_stride_row + k * a.f_stride_col] : nan;
+
+  // ---- dominance: word w of row j = which rows 64 w .. 64 w + 63 dominate row j
+  int cnt = 0;
+  for (int w = 0; w < W; ++w) {
+    uint32_t half[2];
+#pragma unroll
+    for (int h = 1; h >= 0; --h) {
+      uint32_t acc = 0;
+#pragma unroll 8
+      for (int t = 31; t >= 0; --t) {
+        const int i = w * 64 + h * 32 + t;  // wave-uniform
+        const int ic = i < n ? i : 0;
+        uint64_t le = i < n ? ~0ull : 0ull;
+        uint64_t lt = 0ull;
+#pragma unroll
+        for (int k = 0; k < M; ++k) {
+          const float xi = f[(int64_t)ic * a.f_stride_row + k * a.f_stride_col];
+          le &= __builtin_amdgcn_ballot_w64(xi <= xj[k]);
+          lt |= __builtin_amdgcn_ballot_w64(xi < xj[k]);
+        }
+        acc = shift_in(acc, le & lt);
+      }
+      half[h] = acc;
+    }
+    const uint64_t word = valid ? (((uint64_t)half[1] << 32) | half[0]) : 0ull;
+    dom[(size_t)j * rs + w] = word;
+    cnt += __popcll(word);
+  }
+
+  // ---- peeling (non_dominate.py:29-59, :107-125), fronts listed in ascending row order
+  int rank = valid ? kRankUnset : -1;
+  int level = 0, ranked = 0;
+  int worst_start = 0, nv = 0;
+  {
+    const uint64_t b = __builtin_amdgcn_ballot_w64(valid && cnt == 0);
+    if (lane == 0) front[wave] = b;
+    if (valid && cnt == 0) rank = 0;
+  }
+  for (;;) {
+    __syncthreads();
+    const uint64_t* cur = front + (level & 1) * 16;
+    uint64_t* nxt = front + ((level + 1) & 1) * 16;
+    int size = 0, before = 0;
+    for (int w = 0; w < W; ++w) {
+      const int c = __popcll(cur[w]);
+      size += c;
+      if (w < wave) before += c;
+    }
+    if (rank == level) perm[ranked + before + __popcll(cur[wave] & ((1ull << lane) - 1ull))] = j;
+    if (size == 0 || ranked + size >= a.stop_count) {
+      worst_start = ranked;
+      nv = size;
+      break;
+    }
+    bool newly = false;
+    if (rank == kRankUnset) {
+      int c = 0;
+      for (int w = 0; w < W; ++w) c += __popcll(dom[(size_t)j * rs + w] & cur[w]);
+      cnt -= c;
+      newly = cnt == 0;
+      if (newly) rank = level + 1;
+    }
+    const uint64_t b = __builtin_amdgcn_ballot_w64(newly);
+    if (lane == 0) nxt[wave] = b;
+    ranked += size;
+    ++level;
+  }
+  if (a.rank_all && valid) a.rank_all[(int64_t)blockIdx.x * n + j] = rank;
+  if (a.out_f == nullptr) return;  // rank-only mode
+
+  // ---- crowding distance of the last front (non_dominate.py:198-231 with mask = rank == worst)
+  const int topk = a.stop_count;
+  const int need = topk - worst_start;
+  rank_lds[j] = rank;
+  dist[j] = -INFINITY;
+  __syncthreads();
+  const bool cand = j < nv;                      // thread q = candidate q of the last front
+  const int row = cand ? perm[worst_start + j] : 0;
+  bool boundary = false;
+  float acc = 0.0f;
+  for (int k = 0; k < M; ++k) {
+    const float cost = cand ? f[(int64_t)row * a.f_stride_row + k * a.f_stride_col] : 0.0f;
+    const uint64_t mine = ((uint64_t)ordered_key(cost) << 32) | (uint32_t)j;
+    __syncthreads();
+    if (j < nv + 4) tile[j] = cand ? mine : ~0ull;
+    if (j < 4 && nv + j >= nt) tile[nv + j] = ~0ull;  // padding past the thread count
+    __syncthreads();
+    const int p = cand ? count_smaller(tile, nv, mine) : 0;
+    if (cand) scost[p] = cost;
+    __syncthreads();
+    if (cand) {
+      if (p == 0 || p == nv - 1) {
+        boundary = true;
+      } else {
+        const float term = (scost[p + 1] - scost[p - 1]) / (scost[nv - 1] - scost[0]);
+        acc = k == 0 ? term : acc + term;
+      }
+    }
+  }
+  const float d = boundary ? INFINITY : acc;
+  if (cand) dist[row] = d;
+
+  // ---- index-stable top-k on the last front by (-distance, row index) (non_dominate.py:253)
+  {
+    const uint64_t mine = ((uint64_t)ordered_key(-d) << 32) | (uint32_t)j;
+    __syncthreads();
+    if (j < nv + 4) tile[j] = cand ? mine : ~0ull;
+    if (j < 4 && nv + j >= nt) tile[nv + j] = ~0ull;
+    __syncthreads();
+    const int p = cand ? count_smaller(tile, nv, mine) : 0;
+    if (cand && p < need) order[worst_start + p] = row;
+    if (j < worst_start) order[j] = perm[j];
+  }
+  __syncthreads();
+
+  // ---- gather the topk selected rows
+  const int64_t ob = (int64_t)blockIdx.x * topk;
+  for (int p = j; p < topk; p += nt) {
+    const int src = order[p];
+    a.out_rank[ob + p] = rank_lds[src];
+    a.out_dist[ob + p] = dist[src];
+    for (int k = 0; k < M; ++k) a.out_f[(ob + p) * M + k] = f[(int64_t)src * a.f_stride_row + k * a.f_stride_col];
+  }
+  if (a.x != nullptr) {
+    const uint8_t* __restrict__ xb = a.x + (int64_t)blockIdx.x * a.x_stride_b;
+    uint8_t* __restrict__ dst = a.out_x + ob * a.x_row_bytes;
+    const int waves = nt >> 6;
+    for (int p = wave; p < topk; p += waves) {
+      const uint8_t* __restrict__ s = xb + (int64_t)order[p] * a.x_row_stride;
+      uint8_t* __restrict__ dp = dst + (int64_t)p * a.x_row_bytes;
+      if (a.x_unit == 16) {
+        for (int64_t b = lane * 16; b < a.x_row_bytes; b += 64 * 16)
+          *reinterpret_cast<uint4*>(dp + b) = *reinterpret_cast<const uint4*>(s + b);
+      } else if (a.x_unit == 4) {
+        for (int64_t b = lane * 4; b < a.x_row_bytes; b += 64 * 4)
+          *reinterpret_cast<uint32_t*>(dp + b) = *reinterpret_cast<const uint32_t*>(s + b);
+      } else {
+        for (int64_t b = lane; b < a.x_row_bytes; b += 64) dp[b] = s[b];
+      }
+    }
+  }
+}
+
+}  // namespace evx

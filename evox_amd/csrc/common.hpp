@@ -13,6 +13,8 @@ constexpr int kErrBadArg = -1;
 constexpr int kErrWorkspace = -2;
 constexpr int kErrBarrierTimeout = -3;
 
+constexpr int kRankUnset = 0x7FFFFFFF;  // rank of a row that has not been peeled (yet)
+
 __host__ __device__ inline int64_t round_up(int64_t v, int64_t q) { return (v + q - 1) / q * q; }
 
 // Order-preserving map float -> uint32 with torch's sort conventions: -0.0 and +0.0 share a key,

@@ -35,7 +35,6 @@
 namespace evx {
 
 constexpr int kPeelThreads = 256;
-constexpr int kRankUnset = 0x7FFFFFFF;
 // Words of a front bitmap in global memory are kFrontStride words apart (one per 128-byte line): the
 // rows of a front are published by many waves at the same moment, and atomics that share a line
 // serialise.

@@ -49,8 +49,13 @@ def nd_rank(f: torch.Tensor) -> torch.Tensor:
     with torch.cuda.device(f.device):
         flat_f = f32.reshape(-1, n, m)
         flat_out = out.view(-1, n)
-        for b in range(flat_f.size(0)):
-            _rank_one(flat_f[b], flat_out[b])
+        if runtime.small_population_kernel_fits(n, m, flat_f.size(0)):
+            _lib.call("evox_hip_batched_non_dominate_rank", flat_f.data_ptr(), flat_f.size(0), n, m, flat_f.stride(0),
+                      flat_f.stride(1), flat_f.stride(2), flat_out.data_ptr(), runtime.stream_handle(f.device))
+            runtime.note_small_kernel_call()
+        else:
+            for b in range(flat_f.size(0)):
+                _rank_one(flat_f[b], flat_out[b])
     return out
 
 
@@ -156,10 +161,18 @@ def nd_select(x: torch.Tensor, f: torch.Tensor, topk: int) -> Tuple[torch.Tensor
         fo_r = out_rank.view(-1, topk)
         fo_d = out_dist.view(-1, topk)
         stream = runtime.stream_handle(f.device)
+        has_x = row_bytes > 0
+        if runtime.small_population_kernel_fits(n, m, flat_f.size(0)):
+            es = flat_x.element_size()
+            _lib.call("evox_hip_batched_nd_environmental_selection", flat_x.data_ptr() if has_x else None, row_bytes,
+                      flat_x.stride(1) * es, flat_x.stride(0) * es, flat_f.data_ptr(), flat_f.size(0), n, m, flat_f.stride(0),
+                      flat_f.stride(1), flat_f.stride(2), topk, fo_x.data_ptr() if has_x else None, fo_f.data_ptr(),
+                      fo_r.data_ptr(), fo_d.data_ptr(), stream)
+            runtime.note_small_kernel_call()
+            return out_x, out_f.to(f.dtype), out_rank, out_dist
         ws = runtime.workspace(n, m, f.device)
         for b in range(flat_f.size(0)):
             fb, xb = flat_f[b], flat_x[b]
-            has_x = row_bytes > 0
             _lib.call("evox_hip_nd_environmental_selection", xb.data_ptr() if has_x else None, row_bytes,
                       xb.stride(0) * xb.element_size(), fb.data_ptr(), n, m, fb.stride(0), fb.stride(1), topk,
                       fo_x[b].data_ptr() if has_x else None, fo_f[b].data_ptr(), fo_r[b].data_ptr(), fo_d[b].data_ptr(),

@@ -13,6 +13,23 @@ _last: Optional[Tuple[torch.Tensor, int]] = None  # (workspace, stream handle) o
 
 CHECK_STATUS = os.environ.get("EVOX_AMD_CHECK_STATUS", "0") not in ("", "0")
 
+# Populations of at most evox_hip_batched_max_rows(m) rows can run in the one-workgroup-per-population
+# kernel, larger ones need the bit-matrix pipeline.  None = choose by size (a lone population above
+# 384 rows is faster in the pipeline, which spreads it over the whole device; measured cross-over
+# between 200 and 512 rows); True / False force the choice where it is possible (tests use that to
+# drive small inputs through both).
+use_small_population_kernel = None
+
+
+def small_population_kernel_fits(n: int, m: int, batch: int) -> bool:
+    if use_small_population_kernel is False:
+        return False
+    if not 1 <= n <= int(_lib.lib().evox_hip_batched_max_rows(m)):
+        return False
+    if use_small_population_kernel is True:
+        return True
+    return n <= 384 or batch >= 3
+
 
 def require_gpu_tensor(t: torch.Tensor, what: str) -> None:
     if not isinstance(t, torch.Tensor):
@@ -56,10 +73,17 @@ def note_call(ws: torch.Tensor, stream: int) -> None:
         last_status()
 
 
+def note_small_kernel_call() -> None:
+    """The one-workgroup-per-population kernel has no control block and no device-side waits."""
+    global _last
+    _last = None
+
+
 def last_status() -> dict:
-    """Waits for the latest call and returns its control block; raises if the device reported an error."""
+    """Waits for the latest call and returns its control block; raises if the device reported an error.
+    Calls served by the small-population kernel have no control block: {"error": 0}."""
     if _last is None:
-        return {}
+        return {"error": 0}
     ws, stream = _last
     out = (ctypes.c_int32 * 8)()
     code = _lib.lib().evox_hip_read_status(ws.data_ptr(), stream, out)

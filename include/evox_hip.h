@@ -66,6 +66,20 @@ int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int6
                                         void* out_x, float* out_f, int32_t* out_rank, float* out_dist,
                                         int32_t* out_order, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- many small populations at once (what the reference reaches through vmap: non_dominate.py:107-125
+ * for the peeling, the rest of the path batching natively).  One workgroup per population, no workspace.
+ * n <= evox_hip_batched_max_rows(m) (1024 rows for m <= 8, 0 = unsupported); f is addressed as
+ * f[b * stride_batch + i * stride_row + k * stride_col]; outputs are contiguous (batch, ...) arrays.
+ * Per population the results equal those of the single-population entry points. */
+int64_t evox_hip_batched_max_rows(int64_t m);
+int evox_hip_batched_non_dominate_rank(const float* f, int64_t batch, int64_t n, int64_t m, int64_t stride_batch,
+                                       int64_t stride_row, int64_t stride_col, int32_t* rank_out, void* stream);
+int evox_hip_batched_nd_environmental_selection(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes,
+                                                int64_t x_batch_stride_bytes, const float* f, int64_t batch, int64_t n,
+                                                int64_t m, int64_t stride_batch, int64_t stride_row, int64_t stride_col,
+                                                int64_t topk, void* out_x, float* out_f, int32_t* out_rank, float* out_dist,
+                                                void* stream);
+
 /* ---- stages of the calls above, exposed so that each kernel can be tested and timed alone.
  * They operate on the state left in the workspace by the previous stage, in this order:
  *   prepare -> dominance -> count -> peel -> (crowding -> order -> gather).                                 */
