@@ -10,10 +10,12 @@
 #include "dominance.hpp"
 #include "order.hpp"
 #include "peel.hpp"
+#include "radix.hpp"
 
 namespace evx {
 
 constexpr int kMaxGrid = 4096;  // slots of the grid barrier
+constexpr int kRadixMaxWorkers = 510;
 
 struct Options {
   int peel_blocks_per_cu = 2;
@@ -28,7 +30,7 @@ struct Layout {
   int64_t wstride;
   // byte offsets
   size_t ctrl, fsize, fronts_slot, fronts_orig, hist, zero_end, fstart, xs, key, partials, sortparam, bstart, bcursor,
-      scanflags, members, xs_sorted, key_sorted, orig_of, count, witness, rank, dist, perm, order, ukey, pos, scost, dkey, dom, total;
+      scanflags, members, xs_sorted, key_sorted, orig_of, count, witness, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
 };
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
@@ -72,7 +74,12 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->dist = o;       o = align_up(o + sizeof(float) * (size_t)n);
   L->perm = o;       o = align_up(o + sizeof(int) * (size_t)n);
   L->order = o;      o = align_up(o + sizeof(int) * (size_t)n);
-  L->ukey = o;       o = align_up(o + sizeof(uint32_t) * (size_t)m * L->kstride);
+  // radix sort of large fronts: only populations that can have one get the buffers
+  const size_t rseg = n > kRadixMinCandidates ? (size_t)m * L->kstride : 0;
+  L->rpairs0 = o;    o = align_up(o + sizeof(unsigned long long) * rseg);
+  L->rpairs1 = o;    o = align_up(o + sizeof(unsigned long long) * rseg);
+  L->rtable = o;     o = align_up(o + (rseg ? sizeof(int) * (size_t)m * 256 * kRadixMaxWorkers : 0));
+  L->rtotals = o;    o = align_up(o + (rseg ? sizeof(int) * (size_t)m * 256 : 0));
   L->pos = o;        o = align_up(o + sizeof(int) * (size_t)m * L->kstride);
   L->scost = o;      o = align_up(o + sizeof(float) * (size_t)m * L->kstride);
   L->dkey = o;       o = align_up(o + sizeof(uint32_t) * (size_t)L->kstride);
@@ -166,16 +173,16 @@ static int stage_prepare(const Ws& w, const float* f, int64_t sr, int64_t sc, bo
                      w.at<SortParam>(L.sortparam));
   EVX_LAUNCH_CHECK();
   hipLaunchKernelGGL(bucket_scan_kernel, dim3(L.buckets / 1024), dim3(256), 0, s, w.at<int>(L.hist), L.buckets,
-                     w.at<int>(L.bstart), w.at<int>(L.bcursor), w.at<unsigned long long>(L.scanflags), g_opt.spin_limit);
+                     w.at<int>(L.bstart), w.at<int>(L.bcursor), w.at<unsigned long long>(L.scanflags), w.ctrl());
   EVX_LAUNCH_CHECK();
   hipLaunchKernelGGL(bucket_scatter_kernel, dim3(blocks), dim3(256), 0, s, w.at<uint64_t>(L.key), L.n,
-                     w.at<SortParam>(L.sortparam), w.at<int>(L.bcursor), w.at<int>(L.members));
+                     w.at<SortParam>(L.sortparam), w.at<int>(L.bcursor), w.at<int>(L.members), w.ctrl());
   EVX_LAUNCH_CHECK();
   int pblocks = (L.npad + 255) / 256;
   if (pblocks > 2048) pblocks = 2048;
   hipLaunchKernelGGL(bucket_place_kernel, dim3(pblocks), dim3(256), 0, s, w.at<uint64_t>(L.key), w.at<float>(L.xs), L.n, L.m,
                      L.npad, w.at<SortParam>(L.sortparam), w.at<int>(L.bstart), w.at<int>(L.members),
-                     w.at<uint64_t>(L.key_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of));
+                     w.at<uint64_t>(L.key_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of), w.ctrl());
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -200,7 +207,7 @@ static int stage_count(const Ws& w, bool fill_dist, hipStream_t s) {
   hipLaunchKernelGGL(count_kernel, dim3(blocks), dim3(256), 0, s, w.at<uint64_t>(L.dom), L.wstride, L.n,
                      w.at<int>(L.orig_of), w.at<int>(L.count), w.at<int>(L.rank), w.at<int>(L.witness),
                      w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
-                     fill_dist ? w.at<float>(L.dist) : (float*)nullptr);
+                     fill_dist ? w.at<float>(L.dist) : (float*)nullptr, w.ctrl());
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -271,15 +278,50 @@ static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream
   return 0;
 }
 
+static RadixBuffers radix_buffers(const Ws& w) {
+  RadixBuffers b;
+  b.pairs[0] = w.at<unsigned long long>(w.L.rpairs0);
+  b.pairs[1] = w.at<unsigned long long>(w.L.rpairs1);
+  b.table = w.at<int>(w.L.rtable);
+  b.totals = w.at<int>(w.L.rtotals);
+  b.kstride = w.L.kstride;
+  return b;
+}
+
+// Blocks of a radix kernel: master + idle slot + one worker per 1024 candidates, all resident.
+static int radix_grid(const Layout& L) {
+  int workers = (L.n + 1023) / 1024;
+  const int cap = device_cus() * 2 - kFirstSweeper;
+  if (workers > cap) workers = cap;
+  if (workers > kRadixMaxWorkers) workers = kRadixMaxWorkers;
+  if (workers < 1) workers = 1;
+  return workers + kFirstSweeper;
+}
+
 // Crowding distance of the candidates list[ctrl.worst_start ... + ctrl.nv); dkey filled when the
 // final ordering follows.
 static int stage_crowding(const Ws& w, const int* list, bool want_dkey, hipStream_t s) {
   const Layout& L = w.L;
   int qblocks = (L.kstride + 255) / 256;
   if (qblocks > 4096) qblocks = 4096;
+  // fronts of at most kRadixMinCandidates rows are ordered by counting, larger ones by the radix sort;
+  // the front size is only known on the device, so both are launched and one of them returns at once
+  const bool may_be_large = L.n > kRadixMinCandidates;
   hipLaunchKernelGGL(crowd_rank_kernel, dim3(qblocks, L.m), dim3(256), 0, s, w.at<float>(L.xs), L.npad, list, w.ctrl(),
-                     L.kstride, w.at<int>(L.pos), w.at<float>(L.scost));
+                     L.kstride, w.at<int>(L.pos), w.at<float>(L.scost), may_be_large ? kRadixMinCandidates : L.n);
   EVX_LAUNCH_CHECK();
+  if (may_be_large) {
+    const size_t lds = sizeof(int) * (size_t)L.m * 4 * 256;
+    if (lds > 150 * 1024) return kErrBadArg;
+    if (lds > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(crowd_radix_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL(crowd_radix_kernel, dim3(radix_grid(L)), dim3(kRadixThreads), lds, s, w.at<float>(L.xs), L.npad, list,
+                       w.ctrl(), L.m, radix_buffers(w), w.at<int>(L.pos), w.at<float>(L.scost), g_opt.spin_limit);
+    EVX_LAUNCH_CHECK();
+  }
   hipLaunchKernelGGL(crowd_dist_kernel, dim3(qblocks), dim3(256), 0, s, list, w.ctrl(), L.m, w.at<int>(L.pos),
                      w.at<float>(L.scost), L.kstride, w.at<float>(L.dist),
                      want_dkey ? w.at<uint32_t>(L.dkey) : (uint32_t*)nullptr);
@@ -291,9 +333,16 @@ static int stage_order(const Ws& w, hipStream_t s) {
   const Layout& L = w.L;
   int blocks = (L.n + 255) / 256;
   if (blocks > 4096) blocks = 4096;
+  const bool may_be_large = L.n > kRadixMinCandidates;
   hipLaunchKernelGGL(final_order_kernel, dim3(blocks), dim3(256), 0, s, w.at<int>(L.perm), w.ctrl(), w.at<uint32_t>(L.dkey),
-                     w.at<int>(L.order));
+                     w.at<int>(L.order), may_be_large ? kRadixMinCandidates : L.n);
   EVX_LAUNCH_CHECK();
+  if (may_be_large) {
+    hipLaunchKernelGGL(order_radix_kernel, dim3(radix_grid(L)), dim3(kRadixThreads), sizeof(int) * 4 * 256, s,
+                       w.at<int>(L.perm), w.ctrl(), w.at<uint32_t>(L.dkey), radix_buffers(w), w.at<int>(L.order),
+                       g_opt.spin_limit);
+    EVX_LAUNCH_CHECK();
+  }
   return 0;
 }
 
@@ -491,7 +540,7 @@ int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int6
   if (blocks > cap) blocks = cap;
   hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(256), 0, s, w.at<int>(L.order), (int)topk,
                      static_cast<const uint8_t*>(x), x_row_stride_bytes, x_row_bytes, static_cast<uint8_t*>(out_x), unit, f,
-                     sr, sc, L.m, out_f, w.at<int>(L.rank), out_rank, w.at<float>(L.dist), out_dist);
+                     sr, sc, L.m, out_f, w.at<int>(L.rank), out_rank, w.at<float>(L.dist), out_dist, w.ctrl());
   EVX_LAUNCH_CHECK();
   if (out_order) return copy_async(out_order, w.at<int>(L.order), sizeof(int) * (size_t)topk, s);
   return 0;

@@ -36,7 +36,8 @@ struct Ctrl {
   int need;         // rows to take from front `worst` (stop_count - worst_start)
   int passes;       // sweep passes executed
   int listed;       // front bitmaps 0 .. listed-1 have been listed and cleared; polled by the barrier master
-  int reserved[8];
+  int radix_epoch;  // runs of a radix sort kernel so far: each takes a fresh range of barrier generations
+  int reserved[7];
   // grid barrier: block 0 publishes (generation << 32 | rows found by all blocks) in `release`,
   // every other block publishes (generation << 32 | rows it found) in its own `arrive` slot
   unsigned long long release;

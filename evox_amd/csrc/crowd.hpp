@@ -87,9 +87,10 @@ __device__ inline int rank_by_counting(uint64_t mine, int nv, LoadPair load_pair
 // grid = (blocks over q, m); blocks whose candidates lie past nv leave at once.
 __global__ __launch_bounds__(256) void crowd_rank_kernel(const float* __restrict__ xs, int npad, const int* __restrict__ list_base,
                                                          const Ctrl* __restrict__ ctrl, int kstride, int* __restrict__ pos,
-                                                         float* __restrict__ sorted_cost) {
+                                                         float* __restrict__ sorted_cost, int radix_above) {
   __shared__ uint64_t tile_lds[kRankTile];
   const int nv = ctrl->nv;
+  if (nv > radix_above || ctrl->err != 0) return;  // large fronts: radix sort kernel; error: nothing is valid
   const int* __restrict__ list = list_base + ctrl->worst_start;
   const int k = blockIdx.y;
   const float* __restrict__ col = xs + (int64_t)k * npad;
@@ -114,6 +115,7 @@ __global__ __launch_bounds__(256) void crowd_rank_kernel(const float* __restrict
 __global__ __launch_bounds__(256) void crowd_dist_kernel(const int* __restrict__ list_base, const Ctrl* __restrict__ ctrl, int m,
                                                          const int* __restrict__ pos, const float* __restrict__ sorted_cost,
                                                          int kstride, float* __restrict__ dist, uint32_t* __restrict__ dkey) {
+  if (ctrl->err != 0) return;
   const int nv = ctrl->nv;
   const int* __restrict__ list = list_base + ctrl->worst_start;
   const int nv_pad = (int)round_up(nv, 64);
@@ -146,9 +148,11 @@ __global__ __launch_bounds__(256) void crowd_dist_kernel(const int* __restrict__
 // to non_dominate.py:253) and is kept when that place is below `need`.  The better fronts are copied
 // from the rank-ordered listing.
 __global__ __launch_bounds__(256) void final_order_kernel(const int* __restrict__ perm, const Ctrl* __restrict__ ctrl,
-                                                          const uint32_t* __restrict__ dkey, int* __restrict__ order) {
+                                                          const uint32_t* __restrict__ dkey, int* __restrict__ order,
+                                                          int radix_above) {
   __shared__ uint64_t tile_lds[kRankTile];
   const int nv = ctrl->nv;
+  if (nv > radix_above || ctrl->err != 0) return;  // large fronts: radix sort kernel; error: nothing is valid
   const int start = ctrl->worst_start;
   const int need = ctrl->need;
   const int* __restrict__ list = perm + start;
@@ -169,7 +173,9 @@ __global__ __launch_bounds__(256) void gather_kernel(const int* __restrict__ ord
                                                      int unit, const float* __restrict__ f, int64_t f_stride_row,
                                                      int64_t f_stride_col, int m, float* __restrict__ out_f,
                                                      const int* __restrict__ rank, int* __restrict__ out_rank,
-                                                     const float* __restrict__ dist, float* __restrict__ out_dist) {
+                                                     const float* __restrict__ dist, float* __restrict__ out_dist,
+                                                     const Ctrl* __restrict__ ctrl) {
+  if (ctrl->err != 0) return;  // `order` was not produced: the outputs stay as the caller left them
   const int lane = threadIdx.x & 63;
   const int waves = gridDim.x * (blockDim.x >> 6);
   for (int p = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); p < topk; p += waves) {

@@ -72,10 +72,15 @@ __global__ __launch_bounds__(256) void bucket_hist_kernel(const uint64_t* __rest
 // start[b] = exclusive prefix of hist, start[buckets] = n; cursor = copy of start.
 // One block of 256 threads per 1024 bins (at most 64 blocks, all resident): each block adds up its
 // bins, publishes (1 << 32 | total) in its flag, adds the totals of the blocks before it as they appear
-// (bounded polling; the flags start at zero), and then scans its own bins.
+// (the flags start at zero), and then scans its own bins.  A block only ever waits for blocks of
+// lower index, which are dispatched before it and wait for nobody above them, so the wait ends; it is
+// bounded all the same (kScanSpinLimit polls), and running out sets the error flag, on which every
+// later kernel of the call returns without touching the half-built tables.
+constexpr unsigned kScanSpinLimit = 1u << 24;
+
 __global__ __launch_bounds__(256) void bucket_scan_kernel(const int* __restrict__ hist, int buckets, int* __restrict__ start,
                                                           int* __restrict__ cursor, unsigned long long* __restrict__ flags,
-                                                          unsigned spin_limit) {
+                                                          Ctrl* __restrict__ ctrl) {
   __shared__ int wave_tot[4];
   __shared__ int base_lds;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -100,7 +105,10 @@ __global__ __launch_bounds__(256) void bucket_scan_kernel(const int* __restrict_
       unsigned long long f = 0;
       unsigned spins = 0;
       while (((f = __hip_atomic_load(&flags[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) == 0) {
-        if (++spins > spin_limit) break;  // cannot happen: every block is resident and publishes first
+        if (++spins > kScanSpinLimit) {
+          __hip_atomic_store(&ctrl->err, kErrBarrierTimeout, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
         __builtin_amdgcn_s_sleep(1);
       }
       before = (int)(unsigned)(f & 0xFFFFFFFFull);
@@ -124,7 +132,8 @@ __global__ __launch_bounds__(256) void bucket_scan_kernel(const int* __restrict_
 
 __global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint64_t* __restrict__ key, int n,
                                                              const SortParam* __restrict__ param, int* __restrict__ cursor,
-                                                             int* __restrict__ members) {
+                                                             int* __restrict__ members, const Ctrl* __restrict__ ctrl) {
+  if (ctrl->err != 0) return;
   const SortParam sp = *param;
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
     members[atomicAdd(&cursor[bucket_of(key[i], sp)], 1)] = i;
@@ -137,7 +146,8 @@ __global__ __launch_bounds__(256) void bucket_place_kernel(const uint64_t* __res
                                                            int m, int npad, const SortParam* __restrict__ param,
                                                            const int* __restrict__ start, const int* __restrict__ members,
                                                            uint64_t* __restrict__ key_sorted, float* __restrict__ xs_sorted,
-                                                           int* __restrict__ orig_of) {
+                                                           int* __restrict__ orig_of, const Ctrl* __restrict__ ctrl) {
+  if (ctrl->err != 0) return;
   const SortParam sp = *param;
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < npad; i += gridDim.x * blockDim.x) {
     if (i < n) {

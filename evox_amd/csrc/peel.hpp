@@ -141,7 +141,9 @@ __global__ __launch_bounds__(256) void count_kernel(const uint64_t* __restrict__
                                                     const int* __restrict__ orig_of, int* __restrict__ count,
                                                     int* __restrict__ rank, int* __restrict__ witness,
                                                     uint64_t* __restrict__ front0_slot, uint64_t* __restrict__ front0_orig,
-                                                    int* __restrict__ fsize, float* __restrict__ dist_fill) {
+                                                    int* __restrict__ fsize, float* __restrict__ dist_fill,
+                                                    const Ctrl* __restrict__ ctrl) {
+  if (ctrl->err != 0) return;  // the slot tables are not valid: leave front 0 empty, nothing gets peeled
   const int lane = threadIdx.x & 63;
   const int wave_in_block = threadIdx.x >> 6;
   const int waves = gridDim.x * (blockDim.x >> 6);
@@ -456,6 +458,7 @@ __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __re
   extern __shared__ uint64_t front_lds[];  // nwords words (nwords is even: rows are padded to 128),
                                            // followed by nwords more (unranked rows) in witness mode
   __shared__ int scratch[kPeelThreads];
+  if (coherent_load(&ctrl->err) != 0) return;  // an earlier kernel of this call gave up
 
   if (blockIdx.x == 0) {
     // ---- master: nothing but the barrier

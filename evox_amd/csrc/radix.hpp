@@ -1,0 +1,227 @@
+// Segmented LSD radix sort of (32-bit key, candidate index) pairs for large fronts.
+//
+// Used for the per-objective ordering inside the crowding distance and for the final ordering by
+// distance when the last front has more than kRadixMinCandidates rows (below that, ranking by
+// counting in crowd.hpp is one pass with no dependent steps and is faster).  The result is the same
+// ordering: ascending key, ties by ascending candidate index (torch's stable sort,
+// src/evox/utils/jit_fix_operator.py:246-252).
+//
+// One persistent kernel sorts all segments together, four 8-bit passes, three grid barriers per pass
+// (the barrier of peel.hpp: block 0 is the master, block 1 stays out, blocks 2.. work):
+//   1. every wave histograms the digits of its contiguous share of each segment (LDS); the block
+//      totals go to table[segment][digit][block];
+//   2. for every (segment, digit) one wave turns the per-block counts into exclusive prefixes and
+//      leaves the digit total;
+//   3. every block scans the 256 digit totals, derives the first destination of each of its waves for
+//      each digit, and the waves move their pairs in order: inside a group of 64 pairs the rank among
+//      equal digits comes from eight ballots, so every pass is stable.
+// Pairs travel between blocks through relaxed agent-scope loads and stores (no cache-wide fences).
+// The sizes are read from device memory, so the host launches this unconditionally; when the front is
+// small the kernel returns at once.
+#pragma once
+
+#include "common.hpp"
+#include "peel.hpp"
+
+namespace evx {
+
+constexpr int kRadixMinCandidates = 4096;
+constexpr int kRadixThreads = 256;
+
+struct RadixBuffers {
+  unsigned long long* pairs[2];  // [segments][kstride] each: (key << 32) | candidate index
+  int* table;                    // [segments][256][workers]
+  int* totals;                   // [segments][256]
+  int kstride;
+};
+
+// Sorts `nseg` segments of nv pairs; pair e of segment k is initial(k, e) (candidate order), the
+// result is left in buf.pairs[0] (four passes: initial -> pairs[1] -> pairs[0] -> pairs[1] -> pairs[0]).
+// Must be called by every thread of every block with blockIdx.x >= kFirstSweeper; block 0 must run
+// radix_master().  `hist` = LDS, nseg * 4 * 256 ints; `base` = LDS, 256 ints.
+template <class Initial>
+__device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, int nv, Initial initial, Ctrl* ctrl,
+                                           unsigned gen0, unsigned spin_limit, int* hist, int* base, int* scratch) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int workers = gridDim.x - kFirstSweeper;
+  const int wb = (int)blockIdx.x - kFirstSweeper;
+  const int chunk = (int)round_up((nv + workers - 1) / workers, 256);
+  const int sub = chunk / 4;
+  const int w_begin = min(nv, wb * chunk + wave * sub);
+  const int w_end = min(nv, w_begin + sub);
+  unsigned gen = gen0;
+  int dummy = 0;
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 8 * pass;
+    const unsigned long long* __restrict__ in = buf.pairs[pass & 1];
+    unsigned long long* __restrict__ out = buf.pairs[(pass + 1) & 1];
+    // ---- 1. digit histograms
+    for (int t = threadIdx.x; t < nseg * 4 * 256; t += blockDim.x) hist[t] = 0;
+    __syncthreads();
+    for (int k = 0; k < nseg; ++k) {
+      int* h = hist + (k * 4 + wave) * 256;
+      for (int e = w_begin + lane; e < w_end; e += 64) {
+        const unsigned long long p = pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]);
+        atomicAdd(&h[(int)((p >> (32 + shift)) & 255ull)], 1);
+      }
+    }
+    __syncthreads();
+    for (int k = 0; k < nseg; ++k) {
+      const int d = threadIdx.x;  // blockDim.x == 256
+      const int tot = hist[(k * 4 + 0) * 256 + d] + hist[(k * 4 + 1) * 256 + d] + hist[(k * 4 + 2) * 256 + d] +
+                      hist[(k * 4 + 3) * 256 + d];
+      coherent_store(&buf.table[((int64_t)k * 256 + d) * workers + wb], tot);
+    }
+    if (!sweeper_barrier(ctrl, ++gen, 0, &dummy, spin_limit, scratch)) return false;
+    // ---- 2. per (segment, digit): exclusive prefix over the blocks, digit total
+    for (int item = wb * 4 + wave; item < nseg * 256; item += workers * 4) {
+      int* row = buf.table + (int64_t)item * workers;
+      int carry = 0;
+      for (int b0 = 0; b0 < workers; b0 += 64) {
+        const int b = b0 + lane;
+        const int v = b < workers ? coherent_load(&row[b]) : 0;
+        int incl = v;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+          const int up = __shfl_up(incl, off);
+          if (lane >= off) incl += up;
+        }
+        if (b < workers) coherent_store(&row[b], carry + incl - v);
+        carry += __shfl(incl, 63);
+      }
+      if (lane == 0) coherent_store(&buf.totals[item], carry);
+    }
+    if (!sweeper_barrier(ctrl, ++gen, 0, &dummy, spin_limit, scratch)) return false;
+    // ---- 3. destinations and the stable move
+    for (int k = 0; k < nseg; ++k) {
+      const int d = threadIdx.x;
+      const int tot = coherent_load(&buf.totals[k * 256 + d]);
+      int incl = tot;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
+      }
+      if (lane == 63) base[wave] = incl;
+      __syncthreads();
+      int first = incl - tot;
+      for (int v = 0; v < wave; ++v) first += base[v];
+      __syncthreads();
+      // first destination of digit d for wave 0 of this block, then for waves 1..3
+      int r = first + coherent_load(&buf.table[((int64_t)k * 256 + d) * workers + wb]);
+      for (int v = 0; v < 4; ++v) {
+        const int c = hist[(k * 4 + v) * 256 + d];
+        hist[(k * 4 + v) * 256 + d] = r;
+        r += c;
+      }
+    }
+    __syncthreads();
+    for (int k = 0; k < nseg; ++k) {
+      int* h = hist + (k * 4 + wave) * 256;
+      for (int e0 = w_begin; e0 < w_end; e0 += 64) {
+        const int e = e0 + lane;
+        const bool have = e < w_end;
+        const unsigned long long p =
+            !have ? 0ull : (pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]));
+        const int d = (int)((p >> (32 + shift)) & 255ull);
+        // lanes of this group that hold the same digit
+        uint64_t same = __builtin_amdgcn_ballot_w64(have);
+#pragma unroll
+        for (int bit = 0; bit < 8; ++bit) {
+          const uint64_t b = __builtin_amdgcn_ballot_w64((d >> bit) & 1);
+          same &= ((d >> bit) & 1) ? b : ~b;
+        }
+        const int leader = __ffsll((unsigned long long)same) - 1;
+        const int rank = __popcll(same & ((1ull << lane) - 1ull));
+        int start = 0;
+        if (have && lane == leader) {
+          start = h[d];
+          h[d] = start + __popcll(same);
+        }
+        start = __shfl(start, leader < 0 ? 0 : leader);
+        if (have) coherent_store(&out[(int64_t)k * buf.kstride + start + rank], p);
+      }
+    }
+    if (!sweeper_barrier(ctrl, ++gen, 0, &dummy, spin_limit, scratch)) return false;
+  }
+  return true;
+}
+
+// Block 0 of a radix kernel: the barrier master for the 12 generations of one sort.
+__device__ inline void radix_master(Ctrl* ctrl, unsigned gen0, unsigned spin_limit, int* scratch) {
+  int dummy = 0;
+  for (unsigned g = 1; g <= 12; ++g)
+    if (!master_barrier(ctrl, gen0 + g, 0, &dummy, spin_limit, scratch)) return;
+}
+
+// Barrier generations of the sorts start above every generation the peel can reach, and every run of
+// a radix kernel takes a fresh range (the epoch counter lives in the control block).
+__device__ inline unsigned radix_generation_base(const Ctrl* ctrl) { return 0x80000000u + 16u * (unsigned)ctrl->radix_epoch; }
+
+// Per-objective ordering of the last front for the crowding distance: fills pos[k][q] and
+// sorted_cost[k][p] exactly like crowd_rank_kernel, for fronts above kRadixMinCandidates rows.
+__global__ __launch_bounds__(kRadixThreads) void crowd_radix_kernel(const float* __restrict__ xs, int npad,
+                                                                    const int* __restrict__ list_base, Ctrl* __restrict__ ctrl,
+                                                                    int m, RadixBuffers buf, int* __restrict__ pos,
+                                                                    float* __restrict__ sorted_cost, unsigned spin_limit) {
+  extern __shared__ int radix_lds[];  // m * 4 * 256 ints of histograms
+  __shared__ int base[256];
+  __shared__ int scratch[kRadixThreads];
+  const int nv = ctrl->nv;
+  if (nv <= kRadixMinCandidates || coherent_load(&ctrl->err) != 0) return;
+  const unsigned gen0 = radix_generation_base(ctrl);
+  if (blockIdx.x == 0) {
+    radix_master(ctrl, gen0, spin_limit, scratch);
+    if (threadIdx.x == 0) ctrl->radix_epoch += 1;  // nobody reads it again in this kernel
+    return;
+  }
+  if (blockIdx.x < kFirstSweeper) return;
+  const int* __restrict__ list = list_base + ctrl->worst_start;
+  const int workers = gridDim.x - kFirstSweeper;
+  const int wb = (int)blockIdx.x - kFirstSweeper;
+  auto initial = [&](int k, int q) {
+    return ((unsigned long long)ordered_key(xs[(int64_t)k * npad + list[q]]) << 32) | (unsigned)q;
+  };
+  if (!radix_sort_segments(buf, m, nv, initial, ctrl, gen0, spin_limit, radix_lds, base, scratch)) return;
+  for (int k = 0; k < m; ++k)
+    for (int p = wb * blockDim.x + threadIdx.x; p < nv; p += workers * blockDim.x) {
+      const unsigned long long pr = coherent_load(&buf.pairs[0][(int64_t)k * buf.kstride + p]);
+      const int q = (int)(unsigned)(pr & 0xFFFFFFFFull);
+      pos[(int64_t)k * buf.kstride + q] = p;
+      sorted_cost[(int64_t)k * buf.kstride + p] = xs[(int64_t)k * npad + list[q]];
+    }
+}
+
+// Final ordering of the last front by (distance key, candidate index) for large fronts: the first
+// `need` candidates in that order follow the better fronts in `order`.
+__global__ __launch_bounds__(kRadixThreads) void order_radix_kernel(const int* __restrict__ perm, Ctrl* __restrict__ ctrl,
+                                                                    const uint32_t* __restrict__ dkey, RadixBuffers buf,
+                                                                    int* __restrict__ order, unsigned spin_limit) {
+  extern __shared__ int radix_lds[];
+  __shared__ int base[256];
+  __shared__ int scratch[kRadixThreads];
+  const int nv = ctrl->nv;
+  if (nv <= kRadixMinCandidates || coherent_load(&ctrl->err) != 0) return;
+  const unsigned gen0 = radix_generation_base(ctrl);
+  if (blockIdx.x == 0) {
+    radix_master(ctrl, gen0, spin_limit, scratch);
+    if (threadIdx.x == 0) ctrl->radix_epoch += 1;
+    return;
+  }
+  if (blockIdx.x < kFirstSweeper) return;
+  const int start = ctrl->worst_start;
+  const int need = ctrl->need;
+  const int* __restrict__ list = perm + start;
+  const int workers = gridDim.x - kFirstSweeper;
+  const int wb = (int)blockIdx.x - kFirstSweeper;
+  for (int i = wb * blockDim.x + threadIdx.x; i < start; i += workers * blockDim.x) order[i] = perm[i];
+  auto initial = [&](int, int q) { return ((unsigned long long)dkey[q] << 32) | (unsigned)q; };
+  if (!radix_sort_segments(buf, 1, nv, initial, ctrl, gen0, spin_limit, radix_lds, base, scratch)) return;
+  for (int p = wb * blockDim.x + threadIdx.x; p < need; p += workers * blockDim.x) {
+    const unsigned long long pr = coherent_load(&buf.pairs[0][p]);
+    order[start + p] = list[(int)(unsigned)(pr & 0xFFFFFFFFull)];
+  }
+}
+
+}  // namespace evx

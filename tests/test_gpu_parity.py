@@ -263,6 +263,24 @@ def test_crowding_medium_against_oracle():
         assert_dist_close(crowding_distance(grid.to(DEV), mask.to(DEV)), er.crowding(grid, mask), "grid")
 
 
+def test_large_front_uses_radix_sort():
+    """Fronts above 4096 rows are ordered by the segmented radix sort instead of counting: a
+    many-objective population whose first front holds most rows, and the crowding distance of a
+    whole 9000-row population with heavy ties."""
+    say("large_front_radix")
+    f = workloads.sphere_shell_population((9000,), 6, 0.05, seed=12)
+    x = torch.arange(9000, dtype=torch.float32)[:, None].repeat(1, 3)
+    (_, _, _, _), rank, dist, order = er.environmental_selection(x, f, 4500, return_all=True)
+    assert int((rank == 0).sum()) > 4096  # the last admitted front is front 0 and it is large
+    check_selection(f, x, 4500, as_np(rank), as_np(dist), as_np(order), "sphere 9000x6")
+    assert runtime.last_status()["last_front_size"] > 4096
+    g = torch.Generator("cpu").manual_seed(99)
+    ties = (torch.randint(0, 50, (9000, 3), generator=g).float() / 50.0).contiguous()
+    assert_dist_close(crowding_distance(ties.to(DEV), None), er.crowding(ties, None), "ties 9000x3")
+    mask = torch.rand(9000, generator=g) < 0.7
+    assert_dist_close(crowding_distance(ties.to(DEV), mask.to(DEV)), er.crowding(ties, mask), "ties masked")
+
+
 def test_crowding_dtype_rule():
     with pytest.raises(RuntimeError):
         crowding_distance(torch.rand(8, 2, dtype=torch.float64, device=DEV), None)
