@@ -72,6 +72,8 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
   for (int64_t i = tid; i < n_zero_words; i += nthreads) zero_words[i] = 0u;
 }
 
+enum DomVariant { kDomKey64 = 0, kDomTwoCompares = 1 };
+
 // acc = (acc << 1) | bit, with the bit taken from a 64-lane mask: one v_addc_co_u32.
 __device__ inline uint32_t shift_in(uint32_t acc, uint64_t mask) {
   uint32_t r;
@@ -80,7 +82,69 @@ __device__ inline uint32_t shift_in(uint32_t acc, uint64_t mask) {
   return r;
 }
 
-enum DomVariant { kDomKey64 = 0, kDomTwoCompares = 1 };
+// 32 consecutive dominators ib .. ib+31 against the lane's row: bit t of the result says that
+// dominator ib + t dominates the row.  The dominators' fitness and keys sit in SGPRs (M + 2 per
+// dominator); from M = 4 on they are fetched G at a time with one scalar load per array, G shrinking
+// as M grows, because once
+// the SGPR file overflows the compiler spills through v_writelane / v_readlane, which is VALU work
+// (measured: 3.5x the VALU instructions at M = 8 with 32 dominators in flight).
+template <int M, int VARIANT>
+__device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, const uint64_t* __restrict__ key, int npad,
+                                               int ib, const float (&xj)[M], uint64_t kj) {
+  uint32_t acc = 0;
+  if constexpr (M <= 3) {
+    // few enough values per dominator for the compiler to schedule the scalar loads of all 32 itself
+#pragma unroll
+    for (int t = 31; t >= 0; --t) {
+      const int i = ib + t;
+      uint64_t c = ~0ull;
+#pragma unroll
+      for (int k = 0; k < M; ++k) c &= __builtin_amdgcn_ballot_w64(xs[(int64_t)k * npad + i] <= xj[k]);
+      if (VARIANT == kDomKey64) {
+        c &= __builtin_amdgcn_ballot_w64(key[i] != kj);
+      } else {
+        uint64_t lt = 0ull;
+#pragma unroll
+        for (int k = 0; k < M; ++k) lt |= __builtin_amdgcn_ballot_w64(xs[(int64_t)k * npad + i] < xj[k]);
+        c &= lt;
+      }
+      acc = shift_in(acc, c);
+    }
+  } else {
+    constexpr int G = M <= 5 ? 8 : 4;
+#pragma unroll 1
+    for (int g = 32 / G - 1; g >= 0; --g) {
+      const int i0 = ib + g * G;  // wave-uniform
+      float xi[M][G];
+      uint64_t ki[G];
+#pragma unroll
+      for (int k = 0; k < M; ++k)
+#pragma unroll
+        for (int u = 0; u < G; ++u) xi[k][u] = xs[(int64_t)k * npad + i0 + u];
+      if (VARIANT == kDomKey64) {
+#pragma unroll
+        for (int u = 0; u < G; ++u) ki[u] = key[i0 + u];
+      }
+#pragma unroll
+      for (int u = G - 1; u >= 0; --u) {
+        uint64_t c = ~0ull;
+#pragma unroll
+        for (int k = 0; k < M; ++k) c &= __builtin_amdgcn_ballot_w64(xi[k][u] <= xj[k]);
+        if (VARIANT == kDomKey64) {
+          c &= __builtin_amdgcn_ballot_w64(ki[u] != kj);
+        } else {
+          uint64_t lt = 0ull;
+#pragma unroll
+          for (int k = 0; k < M; ++k) lt |= __builtin_amdgcn_ballot_w64(xi[k][u] < xj[k]);
+          c &= lt;
+        }
+        acc = shift_in(acc, c);
+      }
+    }
+  }
+  return acc;
+}
+
 
 // grid.x = ceil(npad / 256) blocks of four 64-row groups, grid.y = ceil(nwords / IW) column tiles.
 template <int M, int IW, int VARIANT>
@@ -109,27 +173,7 @@ __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict_
     uint32_t half[4];
 #pragma unroll
     for (int h = 3; h >= 0; --h) {
-      const int ib = w * 64 + h * 32;
-      uint32_t acc = 0;
-#pragma unroll
-      for (int t = 31; t >= 0; --t) {
-        const int i = ib + t;
-        // each comparison is balloted on its own so that it stays a v_cmp writing an SGPR pair and the
-        // combination runs on the scalar unit
-        uint64_t c = ~0ull;
-#pragma unroll
-        for (int k = 0; k < M; ++k) c &= __builtin_amdgcn_ballot_w64(xs[(int64_t)k * npad + i] <= xj[k]);
-        if (VARIANT == kDomKey64) {
-          c &= __builtin_amdgcn_ballot_w64(key[i] != kj);
-        } else {
-          uint64_t lt = 0ull;
-#pragma unroll
-          for (int k = 0; k < M; ++k) lt |= __builtin_amdgcn_ballot_w64(xs[(int64_t)k * npad + i] < xj[k]);
-          c &= lt;
-        }
-        acc = shift_in(acc, c);
-      }
-      half[h] = acc;
+      half[h] = dominance_half_word<M, VARIANT>(xs, key, npad, w * 64 + h * 32, xj, kj);
     }
     if (j < n) {
       // two words = one 16-byte store; rows are 128-byte aligned and w is even.  Bits of padding rows

@@ -418,6 +418,32 @@ def test_properties_at_full_size_c3():
     assert torch.equal(again, rank[keep])
 
 
+def test_c5_full_size_against_c_checker(population_path):
+    """The large-scale configuration (N = 200000, M = 8, 5 GB bit matrix): ranks, distances and the
+    selected order against the plain-C checker (the dense restatement cannot allocate here)."""
+    if population_path == "small-kernel":
+        pytest.skip("one run is enough: populations of this size always take the pipeline")
+    from oracle import c_oracle
+
+    say("c5_full_size")
+    w = workloads.c5()
+    n = w.f.size(0)
+    order, rank, dist, fronts = c_oracle.select(as_np(w.f), w.topk)
+    say("c5 checker done", fronts, "fronts")
+    fd = w.f.to(DEV)
+    got_rank = non_dominate_rank(fd)
+    assert np.array_equal(as_np(got_rank), rank)
+    assert runtime.last_status()["fronts"] == fronts
+    x = torch.arange(n, dtype=torch.int32, device=DEV)[:, None].repeat(1, 2)
+    xs, fs, rs, ds = nd_environmental_selection(x, fd, w.topk)
+    assert runtime.last_status()["error"] == 0
+    assert np.array_equal(as_np(xs)[:, 0].astype(np.int64), order)
+    assert np.array_equal(as_np(rs), rank[order])
+    assert_dist_close(ds, dist[order], "C5")
+    assert np.array_equal(as_np(fs), as_np(w.f)[order])
+    runtime.release_workspaces()
+
+
 def test_stop_early_matches_full_ranking(peel_algorithm):
     say("stop_early", peel_algorithm)
     f = workloads.uniform_population(4000, 3, 0, 21)[0]
