@@ -188,11 +188,19 @@ def main():
     ranked_in_passes = (rank >= 1) & (rank <= passes)
     peel_bytes = int(row_read[ranked_in_passes].sum()) + passes * nwords * 8
     dom_bytes = n * m * 4 + n * row_bytes
+    slots = torch.arange(n, device=rank.device)
+    evaluated_pairs = float(((((slots >> 6) << 6) + 63) // 256 * 256 + 256).clamp(max=nwords * 64).sum())
+    executed_valu = (m + 2) * evaluated_pairs
     count_bytes = int(row_read.sum()) + n * 12
     phases = {
         "prepare_and_slot_sort": {"us": times["prepare_us"]},
+        # achieved: the reference's 2*M*N^2 compares over the kernel time (the algorithmic figure);
+        # executed: the VALU lane-instructions this kernel issues, (M + 2) per ordered pair of the lower
+        # triangle (tiles of 64 rows x 256 columns on or below the diagonal), over the same time
         "dominance": {"us": times["dominance_us"], "bound": "valu", "achieved": compares / times["dominance_us"] / 1e3,
                       "peak": VALU_CMP_PEAK_GOPS, "unit": "Gcompare/s",
+                      "executed_valu_Gops": executed_valu / times["dominance_us"] / 1e3,
+                      "executed_valu_frac": executed_valu / times["dominance_us"] / 1e3 / VALU_CMP_PEAK_GOPS,
                       "hbm_GBs": dom_bytes / times["dominance_us"] / 1e3},
         "count": {"us": times["count_us"], "bound": "hbm", "achieved": count_bytes / times["count_us"] / 1e3,
                   "peak": HBM_PEAK_GBS, "unit": "GB/s"},

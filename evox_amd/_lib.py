@@ -33,6 +33,8 @@ _SIGNATURES = {
     "evox_hip_batched_nd_environmental_selection": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                                             c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                                             c_void_p, c_void_p, c_void_p]),
+    "evox_hip_tournament_pick": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p,
+                                         c_void_p]),
     "evox_hip_stage_prepare": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "evox_hip_stage_dominance": (c_int, [c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
     "evox_hip_stage_count": (c_int, [c_int64, c_int64, c_void_p, c_size_t, c_void_p]),

@@ -8,10 +8,16 @@ src/evox/workflows/eval_monitor.py:12), before its extension loader runs
 
 import importlib
 
-from .operators.selection import crowding_distance, nd_environmental_selection, non_dominate_rank
+from .operators.selection import (
+    crowding_distance,
+    nd_environmental_selection,
+    non_dominate_rank,
+    tournament_selection_multifit,
+)
 
 _TARGETS = (
     "evox.operators.selection.non_dominate",
+    "evox.operators.selection.tournament_selection",
     "evox.operators.selection",
     "evox.operators",
     "evox.algorithms.mo.nsga2",
@@ -24,6 +30,7 @@ _FUNCS = {
     "non_dominate_rank": non_dominate_rank,
     "crowding_distance": crowding_distance,
     "nd_environmental_selection": nd_environmental_selection,
+    "tournament_selection_multifit": tournament_selection_multifit,
 }
 
 

@@ -596,6 +596,21 @@ int evox_hip_batched_nd_environmental_selection(const void* x, int64_t x_row_byt
   return launch_batched(a, batch, (hipStream_t)stream);
 }
 
+int evox_hip_tournament_pick(const int64_t* parents, int64_t n_round, int64_t tournament_size, const float* fit,
+                             int64_t n_candidates, int64_t n_keys, int64_t stride_row, int64_t stride_col, int64_t* out,
+                             void* stream) {
+  if (parents == nullptr || fit == nullptr || out == nullptr) return kErrBadArg;
+  if (n_round < 0 || tournament_size < 1 || tournament_size > 0x7FFFFFFF || n_candidates < 1 || n_keys < 1 || n_keys > 0x7FFFFFFF)
+    return kErrBadArg;
+  if (n_round == 0) return 0;
+  int64_t blocks = (n_round + 255) / 256;
+  if (blocks > 65535) blocks = 65535;
+  hipLaunchKernelGGL(tournament_pick_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, parents, n_round,
+                     (int)tournament_size, fit, stride_row, stride_col, (int)n_keys, out);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
 int evox_hip_read_status(const void* ws, void* stream, int32_t* host_out8) {
   if (ws == nullptr || host_out8 == nullptr) return kErrBadArg;
   // the control block is the first region of the workspace

@@ -201,4 +201,33 @@ __global__ __launch_bounds__(256) void gather_kernel(const int* __restrict__ ord
   }
 }
 
+// Winner of every tournament: the candidate that comes first when the tournament's candidates are
+// ordered by the LAST key, ties by the key before it, ..., ties by position in the tournament, with NaN
+// after every number and signed zeros tied (src/evox/operators/selection/tournament_selection.py:8-29:
+// lexsort over the unbound key columns, then column 0).  One thread per tournament.
+// fit is (candidates, nkeys) with strides in elements; parents is (n_round, tsize) int64, contiguous.
+__global__ __launch_bounds__(256) void tournament_pick_kernel(const int64_t* __restrict__ parents, int64_t n_round, int tsize,
+                                                              const float* __restrict__ fit, int64_t stride_row,
+                                                              int64_t stride_col, int nkeys, int64_t* __restrict__ out) {
+  for (int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; r < n_round; r += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t* __restrict__ row = parents + r * tsize;
+    int64_t best = row[0];
+    for (int t = 1; t < tsize; ++t) {
+      const int64_t cand = row[t];
+      // strictly better than the current best? (equal on every key keeps the earlier position)
+      bool better = false;
+      for (int k = nkeys - 1; k >= 0; --k) {
+        const uint32_t a = ordered_key(fit[cand * stride_row + k * stride_col]);
+        const uint32_t b = ordered_key(fit[best * stride_row + k * stride_col]);
+        if (a != b) {
+          better = a < b;
+          break;
+        }
+      }
+      if (better) best = cand;
+    }
+    out[r] = best;
+  }
+}
+
 }  // namespace evx

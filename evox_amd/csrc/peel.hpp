@@ -289,17 +289,41 @@ __device__ inline int sweep_rows(const PassCtx& c, const uint64_t* front_lds, in
                                  int row_step) {
   const int lane = threadIdx.x & 63;
   int found = 0;
-  for (int j = first_row; j < c.n; j += row_step) {
-    const int cj = count[j];  // wave-uniform
-    if (cj <= 0) continue;
-    const RowScan r = scan_row<true>(c.dom + (int64_t)j * c.wstride, row_words(j), front_lds);
-    if (r.total) {
-      const int left = cj - r.total;
-      if (lane == 0) {
-        count[j] = left;
-        if (left == 0) publish_ranked(c, j, c.orig_of[j]);
+  int j = first_row;
+  for (;;) {
+    // the next two unranked rows of this wave's share: their loads are issued together
+    int jr[2], cr[2];
+    int have = 0;
+    for (; j < c.n && have < 2; j += row_step) {
+      const int cj = count[j];  // wave-uniform
+      if (cj > 0) {
+        jr[have] = j;
+        cr[have] = cj;
+        ++have;
       }
-      found += left == 0;
+    }
+    if (have == 0) break;
+    if (have == 1) {
+      jr[1] = jr[0];
+      cr[1] = 0;
+    }
+    const uint64_t* const rows[2] = {c.dom + (int64_t)jr[0] * c.wstride, c.dom + (int64_t)jr[1] * c.wstride};
+    const int nws[2] = {row_words(jr[0]), have == 2 ? row_words(jr[1]) : 0};
+    RowScan r[2];
+    if (nws[0] <= 512 && nws[1] <= 512)
+      scan_rows<true, 2, 4>(rows, nws, front_lds, r);
+    else
+      scan_rows<true, 2, 8>(rows, nws, front_lds, r);
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      if (q < have && r[q].total) {
+        const int left = cr[q] - r[q].total;
+        if (lane == 0) {
+          count[jr[q]] = left;
+          if (left == 0) publish_ranked(c, jr[q], c.orig_of[jr[q]]);
+        }
+        found += left == 0;
+      }
     }
   }
   return found;

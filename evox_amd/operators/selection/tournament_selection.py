@@ -1,0 +1,24 @@
+"""Drop-in replacement for ``evox.operators.selection.tournament_selection_multifit``
+(src/evox/operators/selection/tournament_selection.py:8-29), the consumer of the rank and crowding
+distance that ``nd_environmental_selection`` returns (src/evox/algorithms/mo/nsga2.py:94).
+"""
+
+from typing import List
+
+import torch
+
+from ... import ops
+
+
+def tournament_selection_multifit(n_round: int, fitnesses: List[torch.Tensor], tournament_size: int = 2) -> torch.Tensor:
+    """Indices of the winners of ``n_round`` random tournaments of ``tournament_size`` candidates.
+
+    Same contract as the reference: candidates are drawn with ``torch.randint`` on the fitness
+    device (so a seeded generator gives the same tournaments as the reference), and each tournament
+    is won by the candidate that sorts first by the LAST tensor of ``fitnesses``, ties by the one
+    before it, ..., ties by position in the tournament (NaN last).  The result is squeezed, as there.
+    """
+    fitness_tensor = torch.stack(fitnesses, dim=1)
+    num_candidates = fitness_tensor.size(0)
+    parents = torch.randint(0, num_candidates, (n_round, tournament_size), device=fitnesses[0].device)
+    return ops.tournament_pick(parents, fitness_tensor).squeeze()

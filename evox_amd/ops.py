@@ -201,3 +201,24 @@ def _nd_select_vmap(info, in_dims, x, f, topk):
 
 
 torch.library.register_vmap(nd_select, _nd_select_vmap)
+
+
+@torch.library.custom_op("evox_amd::tournament_pick", mutates_args=())
+def tournament_pick(parents: torch.Tensor, fitness: torch.Tensor) -> torch.Tensor:
+    """parents (n_round, t) int64 candidate indices, fitness (candidates, keys) float32 -> (n_round,) int64 winners."""
+    runtime.require_gpu_tensor(parents, "parents")
+    runtime.require_gpu_tensor(fitness, "fitness")
+    if parents.dim() != 2 or fitness.dim() != 2 or parents.dtype != torch.int64:
+        raise ValueError("parents must be (n_round, tournament_size) int64 and fitness (candidates, keys)")
+    fit = _as_f32(fitness, "fitness")
+    par = parents.contiguous()
+    out = torch.empty(par.size(0), dtype=torch.int64, device=parents.device)
+    with torch.cuda.device(parents.device):
+        _lib.call("evox_hip_tournament_pick", par.data_ptr(), par.size(0), par.size(1), fit.data_ptr(), fit.size(0), fit.size(1),
+                  fit.stride(0), fit.stride(1), out.data_ptr(), runtime.stream_handle(parents.device))
+    return out
+
+
+@tournament_pick.register_fake
+def _(parents, fitness):
+    return parents.new_empty(parents.shape[0])

@@ -80,6 +80,17 @@ int evox_hip_batched_nd_environmental_selection(const void* x, int64_t x_row_byt
                                                 int64_t topk, void* out_x, float* out_f, int32_t* out_rank, float* out_dist,
                                                 void* stream);
 
+/* out[r] (int64) = the winner of tournament r: among parents[r * tournament_size + 0 .. tournament_size-1]
+ * (int64 candidate indices, values in [0, n_candidates)) the one that sorts first by the LAST key column of
+ * fit, ties by the column before it, ..., ties by position in the tournament; NaN after every number.
+ * fit is float32 (n_candidates, n_keys) addressed as fit[c * stride_row + k * stride_col].
+ * Replaces the ordering step of evox.operators.selection.tournament_selection_multifit
+ * (src/evox/operators/selection/tournament_selection.py:21-27; the random draw of `parents`, :21, stays in
+ * torch so that the caller's generator is consumed exactly as before). */
+int evox_hip_tournament_pick(const int64_t* parents, int64_t n_round, int64_t tournament_size, const float* fit,
+                             int64_t n_candidates, int64_t n_keys, int64_t stride_row, int64_t stride_col, int64_t* out,
+                             void* stream);
+
 /* ---- stages of the calls above, exposed so that each kernel can be tested and timed alone.
  * They operate on the state left in the workspace by the previous stage, in this order:
  *   prepare -> dominance -> count -> peel -> (crowding -> order -> gather).                                 */

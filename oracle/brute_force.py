@@ -116,3 +116,19 @@ def selection_brute(f: np.ndarray, topk: int):
     worst = np.sort(rank, kind="stable")[topk - 1]
     dist = crowding_brute(f, rank == worst)
     return selection_order_brute(rank, dist, topk), rank, dist
+
+
+def tournament_winners_brute(parents: np.ndarray, keys: np.ndarray) -> np.ndarray:
+    """Winner of each tournament by an explicit comparison of tuples (last key first, NaN as +inf plus
+    one, then position).  parents: (n_round, t) ints; keys: (candidates, nkeys) floats."""
+    out = np.empty(parents.shape[0], dtype=np.int64)
+    for r, row in enumerate(parents):
+        def sort_key(pos_cand):
+            pos, cand = pos_cand
+            parts = []
+            for k in range(keys.shape[1] - 1, -1, -1):
+                v = float(keys[cand, k])
+                parts.append((1, 0.0) if v != v else (0, v + 0.0))
+            return (tuple(parts), pos)
+        out[r] = min(enumerate(row), key=sort_key)[1]
+    return out

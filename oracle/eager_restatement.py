@@ -13,6 +13,7 @@ the reference's multi-objective environmental selection, on torch CPU tensors:
   chained_stable_argsort    <- src/evox/utils/jit_fix_operator.py:246-252
   crowding                  <- src/evox/operators/selection/non_dominate.py:198-231
   environmental_selection   <- src/evox/operators/selection/non_dominate.py:234-254
+  tournament_winners        <- src/evox/operators/selection/tournament_selection.py:18-27
 
 How each function is pinned (tests/test_oracle.py):
   * dominance / ranks: tiny-input brute force, longest-dominator-chain definition, Deb's fast
@@ -127,3 +128,12 @@ def environmental_selection(x: torch.Tensor, f: torch.Tensor, topk: int, return_
     if return_all:
         return picked, rank, dist, order
     return picked
+
+
+def tournament_winners(parents: torch.Tensor, fitnesses: List[torch.Tensor]) -> torch.Tensor:
+    """Winner of each row of ``parents`` (n_round, t): tournament_selection.py:18-27 without the random
+    draw (:21), which the caller supplies so that the checker and the GPU path see the same tournaments."""
+    table = torch.stack(fitnesses, dim=1)
+    keys = table[parents]
+    ordering = chained_stable_argsort(keys.unbind(-1))
+    return torch.gather(parents, 1, ordering[:, 0].unsqueeze(1)).squeeze()

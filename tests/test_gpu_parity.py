@@ -478,6 +478,70 @@ def test_barrier_timeout_is_reported_not_hung():
     assert np.array_equal(as_np(non_dominate_rank(f)), as_np(er.ranks_by_peeling(f.cpu())))
 
 
+# ------------------------------------------------------------------ tournament (consumer of rank / distance)
+
+
+def _tournament_case(seed, n_cand, n_round, tsize):
+    g = torch.Generator("cpu").manual_seed(seed)
+    rank = torch.randint(0, 3, (n_cand,), generator=g, dtype=torch.int32)
+    dist = torch.randint(0, 4, (n_cand,), generator=g).float() / 2
+    dist[torch.rand(n_cand, generator=g) < 0.15] = float("inf")
+    dist[torch.rand(n_cand, generator=g) < 0.15] = -float("inf")
+    dist[torch.rand(n_cand, generator=g) < 0.1] = float("nan")
+    dist[torch.rand(n_cand, generator=g) < 0.1] = -0.0
+    parents = torch.randint(0, n_cand, (n_round, tsize), generator=g)
+    return parents, [-dist, rank]
+
+
+@pytest.mark.parametrize("tsize", [1, 2, 3, 5])
+def test_tournament_pick_against_oracle(tsize, population_path):
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd import ops
+
+    for seed, n_cand, n_round in ((1, 1, 5), (2, 6, 64), (3, 50, 3000), (4, 10000, 100000)):
+        say("tournament", tsize, seed, n_cand, n_round)
+        parents, fits = _tournament_case(seed, n_cand, n_round, tsize)
+        want = as_np(er.tournament_winners(parents, fits)).reshape(-1)
+        table = torch.stack([k.to(DEV) for k in fits], dim=1)
+        got = as_np(ops.tournament_pick(parents.to(DEV), table))
+        assert np.array_equal(got, want), (tsize, seed)
+        # a transposed (column-major) key table goes through the strides, not through a copy
+        table_t = torch.stack([k.to(DEV).float() for k in fits], dim=0).t()
+        assert n_cand == 1 or not table_t.is_contiguous()
+        assert np.array_equal(as_np(ops.tournament_pick(parents.to(DEV), table_t)), want)
+
+
+def test_tournament_selection_multifit_follows_the_generator(population_path):
+    """Same seed, same tournaments as the reference draws them (torch.randint on the fitness device),
+    so the winners are those the restatement finds for that draw."""
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd.operators.selection import tournament_selection_multifit
+
+    say("tournament_multifit")
+    w = workloads.c1()
+    xs, fs, rank, dist = nd_environmental_selection(w.x.to(DEV), w.f.to(DEV), w.topk)
+    for n_round, tsize in ((100, 2), (1, 2), (37, 4)):
+        torch.manual_seed(123)
+        got = tournament_selection_multifit(n_round, [-dist, rank], tsize)
+        torch.manual_seed(123)
+        parents = torch.randint(0, rank.size(0), (n_round, tsize), device=DEV)
+        want = er.tournament_winners(parents.cpu(), [-dist.cpu(), rank.cpu()])
+        assert got.shape == want.shape and got.dtype == torch.int64 and got.device.type == "cuda"
+        assert torch.equal(got.cpu(), want)
+    compiled = torch.compile(lambda p, t: ops_tournament(p, t), fullgraph=True)
+    parents = torch.randint(0, rank.size(0), (64, 2), device=DEV)
+    table = torch.stack([-dist, rank], dim=1)
+    assert torch.equal(compiled(parents, table), ops_tournament(parents, table))
+
+
+def ops_tournament(parents, table):
+    from evox_amd import ops
+
+    return ops.tournament_pick(parents, table)
+
+
 def test_abi_symbols_resolve():
     handle = ctypes.CDLL(_lib.LIB_PATH)
     for name in _lib.EXPORTED_SYMBOLS:

@@ -250,3 +250,53 @@ def test_selection_errors():
         er.environmental_selection(f, f, 6)
     with pytest.raises(IndexError):
         er.environmental_selection(f, f, 0)
+
+
+# --------------------------------------------------------------- tournament
+
+
+def _tournament_inputs(seed, n_cand, n_round, tsize):
+    g = torch.Generator("cpu").manual_seed(seed)
+    # the caller's shape: [-distance, rank]; few distinct values so that ties on both keys occur
+    rank = torch.randint(0, 3, (n_cand,), generator=g, dtype=torch.int32)
+    dist = torch.randint(0, 4, (n_cand,), generator=g).float() / 2
+    dist[torch.rand(n_cand, generator=g) < 0.15] = float("inf")
+    dist[torch.rand(n_cand, generator=g) < 0.15] = -float("inf")
+    dist[torch.rand(n_cand, generator=g) < 0.1] = float("nan")
+    dist[torch.rand(n_cand, generator=g) < 0.1] = -0.0
+    parents = torch.randint(0, n_cand, (n_round, tsize), generator=g)
+    return parents, [-dist, rank]
+
+
+@pytest.mark.parametrize("tsize", [1, 2, 3, 4, 7])
+def test_tournament_matches_tuple_comparison(tsize):
+    for seed, n_cand, n_round in ((1, 1, 5), (2, 6, 64), (3, 50, 300), (4, 200, 2)):
+        parents, fits = _tournament_inputs(seed, n_cand, n_round, tsize)
+        got = as_np(er.tournament_winners(parents, fits)).reshape(-1)
+        keys = np.stack([as_np(k).astype(np.float32) for k in fits], axis=1)
+        want = bf.tournament_winners_brute(as_np(parents), keys)
+        assert np.array_equal(got, want), (tsize, seed)
+        # the same through numpy.lexsort, one tournament at a time (NaN sorts last there too)
+        for r in range(parents.size(0)):
+            row = as_np(parents[r])
+            first = np.lexsort((np.arange(tsize),) + tuple(keys[row, k] + 0.0 for k in range(keys.shape[1])))[0]
+            assert want[r] == row[first]
+
+
+def test_tournament_hand_worked():
+    neg_dist = torch.tensor([-1.0, -2.0, -float("inf"), float("inf"), float("nan"), 0.0, -0.0])
+    rank = torch.tensor([0, 0, 1, 0, 0, 1, 1], dtype=torch.int32)
+    parents = torch.tensor([
+        [0, 1],  # same rank: larger distance (1) wins
+        [2, 0],  # lower rank wins whatever the distance
+        [3, 4],  # same rank, +inf key against NaN key: the number wins
+        [4, 3],
+        [5, 6],  # +0 and -0 tie: the first position wins
+        [6, 5],
+        [1, 1],  # the same candidate twice
+        [4, 2],  # NaN key but lower rank: rank is the primary key
+    ])
+    got = er.tournament_winners(parents, [neg_dist, rank]).tolist()
+    assert got == [1, 0, 3, 3, 5, 6, 1, 4]
+    # one round comes back 0-d, as the reference's squeeze() leaves it
+    assert er.tournament_winners(parents[:1], [neg_dist, rank]).dim() == 0
