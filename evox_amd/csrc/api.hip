@@ -30,7 +30,7 @@ struct Layout {
   int64_t wstride;
   // byte offsets
   size_t ctrl, fsize, fronts_slot, fronts_orig, hist, zero_end, fstart, xs, key, partials, sortparam, bstart, bcursor,
-      scanflags, members, xs_sorted, key_sorted, orig_of, count, witness, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
+      scanflags, members, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
 };
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
@@ -67,6 +67,7 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->members = o;    o = align_up(o + sizeof(int) * (size_t)n);
   L->xs_sorted = o;  o = align_up(o + sizeof(float) * (size_t)m * L->npad);
   L->key_sorted = o; o = align_up(o + sizeof(uint64_t) * (size_t)L->npad);
+  L->kid_sorted = o; o = align_up(o + sizeof(uint32_t) * (size_t)L->npad);
   L->orig_of = o;    o = align_up(o + sizeof(int) * (size_t)L->npad);
   L->count = o;      o = align_up(o + sizeof(int) * (size_t)n);
   L->witness = o;    o = align_up(o + sizeof(int) * (size_t)n);
@@ -131,10 +132,16 @@ static void launch_dominance_m(const Ws& w, int variant, hipStream_t s) {
   dim3 grid((L.npad + 255) / 256, (L.nwords + IW - 1) / IW);
   if (variant == kDomTwoCompares)
     hipLaunchKernelGGL((dominance_kernel<M, IW, kDomTwoCompares>), grid, dim3(256), 0, s, w.at<float>(L.xs_sorted),
-                       w.at<uint64_t>(L.key_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords);
-  else
+                       w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad,
+                       L.wstride, L.nwords);
+  else if (variant == kDomKey64)
     hipLaunchKernelGGL((dominance_kernel<M, IW, kDomKey64>), grid, dim3(256), 0, s, w.at<float>(L.xs_sorted),
-                       w.at<uint64_t>(L.key_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords);
+                       w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad,
+                       L.wstride, L.nwords);
+  else
+    hipLaunchKernelGGL((dominance_kernel<M, IW, kDomKey32>), grid, dim3(256), 0, s, w.at<float>(L.xs_sorted),
+                       w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad,
+                       L.wstride, L.nwords);
 }
 
 template <int IW>
@@ -152,7 +159,7 @@ static void launch_dominance(const Ws& w, int variant, hipStream_t s) {
     default: {
       dim3 grid((L.npad + 255) / 256, (L.nwords + IW - 1) / IW);
       hipLaunchKernelGGL((dominance_any_m_kernel<IW>), grid, dim3(256), 0, s, w.at<float>(L.xs_sorted),
-                         w.at<uint64_t>(L.key_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords, L.m);
+                         w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords, L.m);
     }
   }
 }
@@ -182,7 +189,8 @@ static int stage_prepare(const Ws& w, const float* f, int64_t sr, int64_t sc, bo
   if (pblocks > 2048) pblocks = 2048;
   hipLaunchKernelGGL(bucket_place_kernel, dim3(pblocks), dim3(256), 0, s, w.at<uint64_t>(L.key), w.at<float>(L.xs), L.n, L.m,
                      L.npad, w.at<SortParam>(L.sortparam), w.at<int>(L.bstart), w.at<int>(L.members),
-                     w.at<uint64_t>(L.key_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of), w.ctrl());
+                     w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of),
+                     w.ctrl());
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -193,6 +201,8 @@ static int stage_dominance(const Ws& w, int variant, hipStream_t s) {
   const int tile = g_opt.dominance_tile_words;
   if (tile >= 16)
     launch_dominance<16>(w, variant, s);
+  else if (tile >= 8)
+    launch_dominance<8>(w, variant, s);
   else
     launch_dominance<4>(w, variant, s);
   EVX_LAUNCH_CHECK();
@@ -430,7 +440,7 @@ int evox_hip_set_option(const char* name, int64_t value) {
     g_opt.peel_witness = (int)value;
   } else if (!strcmp(name, "spin_limit") && value >= 1 && value <= 0x7FFFFFFFll) {
     g_opt.spin_limit = (unsigned)value;
-  } else if (!strcmp(name, "dominance_tile_words") && (value == 4 || value == 16)) {
+  } else if (!strcmp(name, "dominance_tile_words") && (value == 4 || value == 8 || value == 16)) {
     g_opt.dominance_tile_words = (int)value;
   } else {
     return kErrBadArg;

@@ -7,16 +7,18 @@
 // Row j therefore lists the dominators of j; its popcount is the domination count of
 // non_dominate.py:188 and one peel pass is popcount(row & front) (non_dominate.py:29-59).
 // Rows and columns are SLOTS: the population relabelled by ascending row key (order.hpp), which makes
-// the matrix strictly lower triangular; word pairs that lie wholly above the diagonal are stored as
-// zeros without being evaluated.
+// the matrix strictly lower triangular; word pairs that lie wholly above the diagonal are neither
+// evaluated nor stored, and no reader looks at them (row j is defined up to word 2 * (j / 128) + 1).
 //
 // Work split: lane = j (fitness of 64 rows held in VGPRs), loop over i with x[i, :] fetched by
 // scalar loads (the index is wave-uniform), so every `<=` is one v_cmp_le_f32 with an SGPR operand
 // whose result is a 64-lane mask in an SGPR pair; the per-objective masks are ANDed on the scalar
-// unit.  "any strictly less" is replaced by one 64-bit compare: with key(i) = sum_k ordered_key(x[i,k])
+// unit.  "any strictly less" is replaced by one integer compare: with key(i) = sum_k ordered_key(x[i,k])
 // and all_k(x[i,k] <= x[j,k]) already true (which rules out NaN on both sides), the rows differ in
 // some objective exactly when key(i) != key(j), because the per-objective keys are ordered the same
-// way as the floats and sum without overflow.  The lane mask is then shifted into the lane's own
+// way as the floats and sum without overflow.  The compare is made on a 32-bit stand-in for the key,
+// kid(slot) = first slot that holds the same key (equal ids <=> equal keys), which halves the scalar
+// bytes per dominator and is one full-rate v_cmp_ne_u32.  The lane mask is then shifted into the lane's own
 // 32-bit accumulator with v_addc_co_u32 (acc = acc + acc + carry), which performs the transpose from
 // "mask over j" to "word over i" at one VALU instruction per 64 pairs.
 #pragma once
@@ -72,7 +74,7 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
   for (int64_t i = tid; i < n_zero_words; i += nthreads) zero_words[i] = 0u;
 }
 
-enum DomVariant { kDomKey64 = 0, kDomTwoCompares = 1 };
+enum DomVariant { kDomKey32 = 0, kDomTwoCompares = 1, kDomKey64 = 2 };
 
 // acc = (acc << 1) | bit, with the bit taken from a 64-lane mask: one v_addc_co_u32.
 __device__ inline uint32_t shift_in(uint32_t acc, uint64_t mask) {
@@ -89,8 +91,9 @@ __device__ inline uint32_t shift_in(uint32_t acc, uint64_t mask) {
 // the SGPR file overflows the compiler spills through v_writelane / v_readlane, which is VALU work
 // (measured: 3.5x the VALU instructions at M = 8 with 32 dominators in flight).
 template <int M, int VARIANT>
-__device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, const uint64_t* __restrict__ key, int npad,
-                                               int ib, const float (&xj)[M], uint64_t kj) {
+__device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, const uint64_t* __restrict__ key,
+                                               const uint32_t* __restrict__ kid, int npad, int ib, const float (&xj)[M],
+                                               uint64_t kj, uint32_t idj) {
   uint32_t acc = 0;
   if constexpr (M <= 3) {
     // few enough values per dominator for the compiler to schedule the scalar loads of all 32 itself
@@ -102,6 +105,8 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
       for (int k = 0; k < M; ++k) c &= __builtin_amdgcn_ballot_w64(xs[(int64_t)k * npad + i] <= xj[k]);
       if (VARIANT == kDomKey64) {
         c &= __builtin_amdgcn_ballot_w64(key[i] != kj);
+      } else if (VARIANT == kDomKey32) {
+        c &= __builtin_amdgcn_ballot_w64(kid[i] != idj);
       } else {
         uint64_t lt = 0ull;
 #pragma unroll
@@ -117,6 +122,7 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
       const int i0 = ib + g * G;  // wave-uniform
       float xi[M][G];
       uint64_t ki[G];
+      uint32_t idi[G];
 #pragma unroll
       for (int k = 0; k < M; ++k)
 #pragma unroll
@@ -125,6 +131,10 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
 #pragma unroll
         for (int u = 0; u < G; ++u) ki[u] = key[i0 + u];
       }
+      if (VARIANT == kDomKey32) {
+#pragma unroll
+        for (int u = 0; u < G; ++u) idi[u] = kid[i0 + u];
+      }
 #pragma unroll
       for (int u = G - 1; u >= 0; --u) {
         uint64_t c = ~0ull;
@@ -132,6 +142,8 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
         for (int k = 0; k < M; ++k) c &= __builtin_amdgcn_ballot_w64(xi[k][u] <= xj[k]);
         if (VARIANT == kDomKey64) {
           c &= __builtin_amdgcn_ballot_w64(ki[u] != kj);
+        } else if (VARIANT == kDomKey32) {
+          c &= __builtin_amdgcn_ballot_w64(idi[u] != idj);
         } else {
           uint64_t lt = 0ull;
 #pragma unroll
@@ -149,8 +161,8 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
 // grid.x = ceil(npad / 256) blocks of four 64-row groups, grid.y = ceil(nwords / IW) column tiles.
 template <int M, int IW, int VARIANT>
 __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
-                                                        uint64_t* __restrict__ dom, int n, int npad, int64_t wstride,
-                                                        int nwords) {
+                                                        const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom, int n,
+                                                        int npad, int64_t wstride, int nwords) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int j = (blockIdx.x * 4 + wave) * 64 + lane;
@@ -160,27 +172,38 @@ __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict_
 #pragma unroll
   for (int k = 0; k < M; ++k) xj[k] = xs[(int64_t)k * npad + j];
   const uint64_t kj = key[j];
+  const uint32_t idj = kid[j];
   uint64_t* __restrict__ out = dom + (int64_t)j * wstride;
   const int wend = (w0 + IW < nwords) ? w0 + IW : nwords;  // nwords = npad / 64 is even, and so is IW
   const int jlast = j - lane + 63;  // last row of this wave
+  // Word pairs wholly above the diagonal (no row of a larger slot dominates these rows) are neither
+  // evaluated nor stored: every reader bounds its scan of row j by the words up to j's own.
+  // The results of the tile are kept in registers and stored together at the end, so that the 16-byte
+  // pieces of one row reach the cache back to back and leave it as whole sectors.
+  ulonglong2 res[IW / 2];
+#pragma unroll
+  for (int q = 0; q < IW / 2; ++q) res[q] = make_ulonglong2(0ull, 0ull);
 #pragma unroll 1
-  for (int w = w0; w < wend; w += 2) {
-    if (w * 64 > jlast) {
-      // both words lie above the diagonal: no row of a larger slot dominates these rows
-      if (j < n) *reinterpret_cast<ulonglong2*>(out + w) = make_ulonglong2(0ull, 0ull);
-      continue;
-    }
+  for (int p = 0; p < IW / 2; ++p) {
+    const int w = w0 + 2 * p;
+    if (w >= wend || w * 64 > jlast) break;
     uint32_t half[4];
 #pragma unroll
     for (int h = 3; h >= 0; --h) {
-      half[h] = dominance_half_word<M, VARIANT>(xs, key, npad, w * 64 + h * 32, xj, kj);
+      half[h] = dominance_half_word<M, VARIANT>(xs, key, kid, npad, w * 64 + h * 32, xj, kj, idj);
     }
-    if (j < n) {
-      // two words = one 16-byte store; rows are 128-byte aligned and w is even.  Bits of padding rows
-      // (i >= n) are zero because their fitness is NaN.
-      const uint64_t lo = ((uint64_t)half[1] << 32) | half[0];
-      const uint64_t hi = ((uint64_t)half[3] << 32) | half[2];
-      *reinterpret_cast<ulonglong2*>(out + w) = make_ulonglong2(lo, hi);
+    // bits of padding rows (i >= n) are zero because their fitness is NaN
+    const uint64_t lo = ((uint64_t)half[1] << 32) | half[0];
+    const uint64_t hi = ((uint64_t)half[3] << 32) | half[2];
+#pragma unroll
+    for (int q = 0; q < IW / 2; ++q)
+      if (q == p) res[q] = make_ulonglong2(lo, hi);
+  }
+  if (j < n) {
+#pragma unroll
+    for (int q = 0; q < IW / 2; ++q) {
+      const int w = w0 + 2 * q;  // rows are 128-byte aligned and w is even: one 16-byte store per pair
+      if (w < wend && w * 64 <= jlast) *reinterpret_cast<ulonglong2*>(out + w) = res[q];
     }
   }
 }
@@ -188,7 +211,7 @@ __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict_
 // Any number of objectives (used above 8): same scheme, with the lane's own fitness re-read from
 // memory for every objective instead of living in registers.
 template <int IW>
-__global__ __launch_bounds__(256) void dominance_any_m_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
+__global__ __launch_bounds__(256) void dominance_any_m_kernel(const float* __restrict__ xs, const uint32_t* __restrict__ kid,
                                                               uint64_t* __restrict__ dom, int n, int npad, int64_t wstride,
                                                               int nwords, int m) {
   const int lane = threadIdx.x & 63;
@@ -196,16 +219,13 @@ __global__ __launch_bounds__(256) void dominance_any_m_kernel(const float* __res
   const int j = (blockIdx.x * 4 + wave) * 64 + lane;
   if (j - lane >= npad) return;
   const int w0 = blockIdx.y * IW;
-  const uint64_t kj = key[j];
+  const uint32_t idj = kid[j];
   uint64_t* __restrict__ out = dom + (int64_t)j * wstride;
   const int wend = (w0 + IW < nwords) ? w0 + IW : nwords;
   const int jlast = j - lane + 63;
 #pragma unroll 1
   for (int w = w0; w < wend; w += 2) {
-    if (w * 64 > jlast) {
-      if (j < n) *reinterpret_cast<ulonglong2*>(out + w) = make_ulonglong2(0ull, 0ull);
-      continue;
-    }
+    if (w * 64 > jlast) break;  // above the diagonal: never read
     uint32_t half[4];
 #pragma unroll
     for (int h = 3; h >= 0; --h) {
@@ -214,7 +234,7 @@ __global__ __launch_bounds__(256) void dominance_any_m_kernel(const float* __res
 #pragma unroll 4
       for (int t = 31; t >= 0; --t) {
         const int i = ib + t;
-        uint64_t c = __builtin_amdgcn_ballot_w64(key[i] != kj);
+        uint64_t c = __builtin_amdgcn_ballot_w64(kid[i] != idj);
         for (int k = 0; k < m; ++k) c &= __builtin_amdgcn_ballot_w64(xs[(int64_t)k * npad + i] <= xs[(int64_t)k * npad + j]);
         acc = shift_in(acc, c);
       }

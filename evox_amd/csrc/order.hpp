@@ -145,8 +145,9 @@ __global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint64_t* __r
 __global__ __launch_bounds__(256) void bucket_place_kernel(const uint64_t* __restrict__ key, const float* __restrict__ xs, int n,
                                                            int m, int npad, const SortParam* __restrict__ param,
                                                            const int* __restrict__ start, const int* __restrict__ members,
-                                                           uint64_t* __restrict__ key_sorted, float* __restrict__ xs_sorted,
-                                                           int* __restrict__ orig_of, const Ctrl* __restrict__ ctrl) {
+                                                           uint64_t* __restrict__ key_sorted, uint32_t* __restrict__ kid_sorted,
+                                                           float* __restrict__ xs_sorted, int* __restrict__ orig_of,
+                                                           const Ctrl* __restrict__ ctrl) {
   if (ctrl->err != 0) return;
   const SortParam sp = *param;
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < npad; i += gridDim.x * blockDim.x) {
@@ -154,19 +155,22 @@ __global__ __launch_bounds__(256) void bucket_place_kernel(const uint64_t* __res
       const uint64_t ki = key[i];
       const int b = bucket_of(ki, sp);
       const int lo = start[b], hi = start[b + 1];
-      int before = 0;
+      int before = 0, smaller = 0;
       for (int p = lo; p < hi; ++p) {
         const int e = members[p];
         const uint64_t ke = key[e];
+        smaller += ke < ki;
         before += (ke < ki) || (ke == ki && e < i);
       }
       const int slot = lo + before;
       orig_of[slot] = i;
       key_sorted[slot] = ki;
+      kid_sorted[slot] = (uint32_t)(lo + smaller);  // first slot holding this key: equal ids <=> equal keys
       for (int k = 0; k < m; ++k) xs_sorted[(int64_t)k * npad + slot] = xs[(int64_t)k * npad + i];
     } else {
       orig_of[i] = -1;
       key_sorted[i] = ~0ull;
+      kid_sorted[i] = (uint32_t)i;
       for (int k = 0; k < m; ++k) xs_sorted[(int64_t)k * npad + i] = __uint_as_float(0x7FC00000u);
     }
   }
