@@ -99,9 +99,11 @@ struct Ws {
   Ctrl* ctrl() const { return at<Ctrl>(L.ctrl); }
 };
 
-static int open_ws(int64_t n, int64_t m, void* ws, size_t bytes, Ws* out) {
+// The bit matrix is the last region: entry points that never build it need only the bytes before it.
+static int open_ws(int64_t n, int64_t m, void* ws, size_t bytes, Ws* out, bool with_matrix = true) {
   if (!make_layout(n, m, &out->L)) return kErrBadArg;
-  if (ws == nullptr || bytes < out->L.total || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return kErrWorkspace;
+  const size_t need = with_matrix ? out->L.total : out->L.dom;
+  if (ws == nullptr || bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return kErrWorkspace;
   out->base = static_cast<uint8_t*>(ws);
   return 0;
 }
@@ -162,6 +164,14 @@ static void launch_dominance(const Ws& w, int variant, hipStream_t s) {
                          w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords, L.m);
     }
   }
+}
+
+template <int M>
+static void launch_first_front(const Ws& w, uint8_t* mask, hipStream_t s) {
+  const Layout& L = w.L;
+  hipLaunchKernelGGL((first_front_kernel<M>), dim3((L.n + 255) / 256), dim3(256), 0, s, w.at<float>(L.xs_sorted),
+                     w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<int>(L.orig_of), L.n, L.npad, mask,
+                     w.ctrl());
 }
 
 // Fitness -> structure of arrays + keys, state reset, then the slot sort (order.hpp).
@@ -501,10 +511,40 @@ int evox_hip_non_dominate_rank(const float* f, int64_t n, int64_t m, int64_t sr,
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   hipStream_t s = (hipStream_t)stream;
   if (int e = stage_prepare(w, f, sr, sc, true, s)) return e;
-  if (int e = stage_dominance(w, kDomKey64, s)) return e;
+  if (int e = stage_dominance(w, kDomKey32, s)) return e;
   if (int e = stage_count(w, false, s)) return e;
   if (int e = stage_peel(w, n, false, s)) return e;
   return copy_async(rank_out, w.at<int>(w.L.rank), sizeof(int) * (size_t)n, s);
+}
+
+size_t evox_hip_first_front_workspace_bytes(int64_t n, int64_t m) {
+  Layout L;
+  return make_layout(n, m, &L) ? L.dom : 0;
+}
+
+int evox_hip_first_front_mask(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, uint8_t* mask_out, void* ws,
+                              size_t ws_bytes, void* stream) {
+  Ws w;
+  if (mask_out == nullptr) return kErrBadArg;
+  if (int e = open_ws(n, m, ws, ws_bytes, &w, false)) return e;
+  const Layout& L = w.L;
+  hipStream_t s = (hipStream_t)stream;
+  if (int e = stage_prepare(w, f, sr, sc, true, s)) return e;
+  switch (L.m) {
+    case 1: launch_first_front<1>(w, mask_out, s); break;
+    case 2: launch_first_front<2>(w, mask_out, s); break;
+    case 3: launch_first_front<3>(w, mask_out, s); break;
+    case 4: launch_first_front<4>(w, mask_out, s); break;
+    case 5: launch_first_front<5>(w, mask_out, s); break;
+    case 6: launch_first_front<6>(w, mask_out, s); break;
+    case 7: launch_first_front<7>(w, mask_out, s); break;
+    case 8: launch_first_front<8>(w, mask_out, s); break;
+    default:
+      hipLaunchKernelGGL(first_front_any_m_kernel, dim3((L.n + 255) / 256), dim3(256), 0, s, w.at<float>(L.xs_sorted),
+                         w.at<uint32_t>(L.kid_sorted), w.at<int>(L.orig_of), L.n, L.npad, L.m, mask_out, w.ctrl());
+  }
+  EVX_LAUNCH_CHECK();
+  return 0;
 }
 
 int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t sr, int64_t sc, const uint8_t* mask,
@@ -534,7 +574,7 @@ int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int6
   const Layout& L = w.L;
   hipStream_t s = (hipStream_t)stream;
   if (int e = stage_prepare(w, f, sr, sc, true, s)) return e;
-  if (int e = stage_dominance(w, kDomKey64, s)) return e;
+  if (int e = stage_dominance(w, kDomKey32, s)) return e;
   if (int e = stage_count(w, true, s)) return e;
   if (int e = stage_peel(w, topk, true, s)) return e;
   if (int e = stage_crowding(w, w.at<int>(L.perm), true, s)) return e;

@@ -248,4 +248,63 @@ __global__ __launch_bounds__(256) void dominance_any_m_kernel(const float* __res
   }
 }
 
+// ------------------------------------------------------------------ first front only
+
+// mask[orig_of[j]] = 1 when no row dominates slot j, 0 otherwise: `non_dominate_rank(f) == 0`, the
+// only thing src/evox/workflows/eval_monitor.py:301-302 and :333-335 keep of the ranks.  No matrix is
+// built: a lane holds one row, the candidate dominators (slots below the end of the wave's own 64
+// rows, since a dominator has a smaller key) stream past it 32 at a time in slot order, and the wave
+// stops as soon as every one of its rows has met a dominator.  Rows of small key lie near the front and
+// dominate most of the population, so almost every wave ends after its first few steps; a wave that
+// holds a non-dominated row scans all the slots below it.
+template <int M>
+__global__ __launch_bounds__(256) void first_front_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
+                                                          const uint32_t* __restrict__ kid, const int* __restrict__ orig_of,
+                                                          int n, int npad, uint8_t* __restrict__ mask,
+                                                          const Ctrl* __restrict__ ctrl) {
+  if (ctrl->err != 0) return;  // the slot sort failed: nothing is valid
+  const int lane = threadIdx.x & 63;
+  const int j = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 64 + lane;
+  if (j - lane >= n) return;  // npad is a multiple of 128: every row touched below exists
+  float xj[M];
+#pragma unroll
+  for (int k = 0; k < M; ++k) xj[k] = xs[(int64_t)k * npad + j];
+  const uint32_t idj = kid[j];
+  bool dominated = j >= n;  // padding rows never hold the wave back
+  const int iend = j - lane + 64;
+#pragma unroll 1
+  for (int ib = 0; ib < iend; ib += 32) {
+    dominated |= dominance_half_word<M, kDomKey32>(xs, key, kid, npad, ib, xj, 0ull, idj) != 0u;
+    if (__builtin_amdgcn_ballot_w64(!dominated) == 0ull) break;
+  }
+  if (j < n) mask[orig_of[j]] = dominated ? 0 : 1;
+}
+
+// Any number of objectives (used above 8).
+__global__ __launch_bounds__(256) void first_front_any_m_kernel(const float* __restrict__ xs, const uint32_t* __restrict__ kid,
+                                                                const int* __restrict__ orig_of, int n, int npad, int m,
+                                                                uint8_t* __restrict__ mask, const Ctrl* __restrict__ ctrl) {
+  if (ctrl->err != 0) return;
+  const int lane = threadIdx.x & 63;
+  const int j = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 64 + lane;
+  if (j - lane >= n) return;
+  const uint32_t idj = kid[j];
+  bool dominated = j >= n;
+  const int iend = j - lane + 64;
+#pragma unroll 1
+  for (int ib = 0; ib < iend; ib += 32) {
+    uint64_t any = 0ull;
+#pragma unroll 4
+    for (int t = 0; t < 32; ++t) {
+      const int i = ib + t;
+      uint64_t c = __builtin_amdgcn_ballot_w64(kid[i] != idj);
+      for (int k = 0; k < m; ++k) c &= __builtin_amdgcn_ballot_w64(xs[(int64_t)k * npad + i] <= xs[(int64_t)k * npad + j]);
+      any |= c;
+    }
+    dominated |= ((any >> lane) & 1ull) != 0ull;
+    if (__builtin_amdgcn_ballot_w64(!dominated) == 0ull) break;
+  }
+  if (j < n) mask[orig_of[j]] = dominated ? 0 : 1;
+}
+
 }  // namespace evx

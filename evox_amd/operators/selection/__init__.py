@@ -1,4 +1,10 @@
-__all__ = ["crowding_distance", "nd_environmental_selection", "non_dominate_rank", "tournament_selection_multifit"]
+__all__ = [
+    "crowding_distance",
+    "nd_environmental_selection",
+    "non_dominate_rank",
+    "non_dominated_mask",
+    "tournament_selection_multifit",
+]
 
-from .non_dominate import crowding_distance, nd_environmental_selection, non_dominate_rank
+from .non_dominate import crowding_distance, nd_environmental_selection, non_dominate_rank, non_dominated_mask
 from .tournament_selection import tournament_selection_multifit

@@ -23,6 +23,17 @@ def non_dominate_rank(x: torch.Tensor) -> torch.Tensor:
     return ops.nd_rank(x)
 
 
+def non_dominated_mask(x: torch.Tensor) -> torch.Tensor:
+    """``non_dominate_rank(x) == 0`` without ranking anything else: bool ``(N,)`` on ``x.device``.
+
+    Not a name of the reference; it replaces the two statements with which ``EvalMonitor.get_pf_fitness``
+    and ``get_pf`` (src/evox/workflows/eval_monitor.py:301-302, :333-335) rank the whole evaluation
+    history only to keep the rows of rank 0.  No dominance matrix is built, so memory stays linear in
+    ``N`` and a history of millions of rows can be filtered.
+    """
+    return ops.nd_first_front(x)
+
+
 def crowding_distance(costs: torch.Tensor, mask: Optional[torch.Tensor]) -> torch.Tensor:
     """Crowding distance of the rows selected by ``mask`` (all rows when ``mask`` is ``None``).
 

@@ -71,6 +71,44 @@ def _nd_rank_vmap(info, in_dims, f):
 torch.library.register_vmap(nd_rank, _nd_rank_vmap)
 
 
+@torch.library.custom_op("evox_amd::nd_first_front", mutates_args=())
+def nd_first_front(f: torch.Tensor) -> torch.Tensor:
+    """(..., N, M) fitness -> (..., N) bool, True for the rows that no row dominates (rank 0)."""
+    runtime.require_gpu_tensor(f, "fitness")
+    if f.dim() < 2:
+        raise ValueError("fitness must have shape (..., N, M)")
+    f32 = _as_f32(f, "fitness")
+    n, m = f32.shape[-2:]
+    out = torch.empty(f32.shape[:-1], dtype=torch.bool, device=f.device)
+    if n == 0 or out.numel() == 0:
+        return out
+    if m == 0:
+        return out.fill_(True)
+    with torch.cuda.device(f.device):
+        flat_f = f32.reshape(-1, n, m)
+        flat_out = out.view(-1, n)
+        ws = runtime.workspace(n, m, f.device, with_matrix=False)
+        stream = runtime.stream_handle(f.device)
+        for b in range(flat_f.size(0)):
+            fb = flat_f[b]
+            _lib.call("evox_hip_first_front_mask", fb.data_ptr(), n, m, fb.stride(0), fb.stride(1), flat_out[b].data_ptr(),
+                      ws.data_ptr(), ws.numel(), stream)
+        runtime.note_call(ws, stream)
+    return out
+
+
+@nd_first_front.register_fake
+def _(f):
+    return f.new_empty(f.shape[:-1], dtype=torch.bool)
+
+
+def _nd_first_front_vmap(info, in_dims, f):
+    return nd_first_front(f.movedim(in_dims[0], 0)), 0
+
+
+torch.library.register_vmap(nd_first_front, _nd_first_front_vmap)
+
+
 @torch.library.custom_op("evox_amd::crowding", mutates_args=())
 def crowding(costs: torch.Tensor, mask: Optional[torch.Tensor]) -> torch.Tensor:
     """(..., N, M) costs, optional (..., N) bool mask -> (..., N) float32 crowding distance."""

@@ -45,10 +45,12 @@ def stream_handle(device: torch.device) -> int:
     return int(torch.cuda.current_stream(device).cuda_stream)
 
 
-def workspace(n: int, m: int, device: torch.device) -> torch.Tensor:
+def workspace(n: int, m: int, device: torch.device, with_matrix: bool = True) -> torch.Tensor:
     """A uint8 tensor of at least evox_hip_workspace_bytes(n, m) bytes, cached per (device, stream):
-    calls on one stream are ordered, so they can share it."""
-    need = int(_lib.lib().evox_hip_workspace_bytes(n, m))
+    calls on one stream are ordered, so they can share it.  ``with_matrix=False`` asks only for the
+    bytes that the entry points without a dominance matrix need."""
+    query = _lib.lib().evox_hip_workspace_bytes if with_matrix else _lib.lib().evox_hip_first_front_workspace_bytes
+    need = int(query(n, m))
     if need == 0:
         raise ValueError(f"unsupported population shape n={n}, m={m}")
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream_handle(device))

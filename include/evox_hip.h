@@ -41,6 +41,16 @@ size_t evox_hip_workspace_bytes(int64_t n, int64_t m);
 int evox_hip_non_dominate_rank(const float* f, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col,
                                int32_t* rank_out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* mask_out[j] (one byte per row, n entries) = 1 when no row dominates row j, else 0: the rows of rank 0,
+ * without building the dominance matrix or peeling.  Replaces the pair
+ * `rank = non_dominate_rank(all_fitness); ... [rank == 0]` of EvalMonitor.get_pf_fitness / get_pf
+ * (src/evox/workflows/eval_monitor.py:301-302 and :333-335), which ranks the whole evaluation history only
+ * to keep its first front.  Needs evox_hip_first_front_workspace_bytes(n, m) bytes of workspace (a few
+ * arrays of n entries; a workspace of evox_hip_workspace_bytes(n, m) is also accepted). */
+size_t evox_hip_first_front_workspace_bytes(int64_t n, int64_t m);
+int evox_hip_first_front_mask(const float* f, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col,
+                              uint8_t* mask_out, void* workspace, size_t workspace_bytes, void* stream);
+
 /* dist_out[j] (float32, n entries) = crowding distance of row j among the rows with mask[j] != 0,
  * -inf for the others.  `mask` is a byte per row at mask[j * mask_stride]; NULL selects every row.
  * Replaces evox.operators.selection.crowding_distance

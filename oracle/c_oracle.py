@@ -24,6 +24,8 @@ def lib():
         h.oracle_select.restype = ctypes.c_int
         h.oracle_select.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int64, ctypes.c_void_p,
                                     ctypes.c_void_p, ctypes.c_void_p]
+        h.oracle_first_front.restype = ctypes.c_int
+        h.oracle_first_front.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
         _lib = h
     return _lib
 
@@ -60,3 +62,10 @@ def select(f, topk):
     if fronts < 0:
         raise RuntimeError(f"oracle_select failed ({fronts})")
     return order, rank, dist, fronts
+
+
+def first_front(f):
+    f = _f32(f)
+    mask = np.empty(f.shape[0], dtype=np.uint8)
+    lib().oracle_first_front(f.ctypes.data, f.shape[0], f.shape[1], mask.ctypes.data)
+    return mask.astype(bool)

@@ -14,11 +14,14 @@ the reference's multi-objective environmental selection, on torch CPU tensors:
   crowding                  <- src/evox/operators/selection/non_dominate.py:198-231
   environmental_selection   <- src/evox/operators/selection/non_dominate.py:234-254
   tournament_winners        <- src/evox/operators/selection/tournament_selection.py:18-27
+  first_front_mask          <- src/evox/workflows/eval_monitor.py:301-302 (= :333-334)
 
 How each function is pinned (tests/test_oracle.py):
   * dominance / ranks: tiny-input brute force, longest-dominator-chain definition, Deb's fast
     non-dominated sort, closed forms (chain, all-equal, M=1 dense rank, layered construction).
   * chained_stable_argsort: numpy.lexsort on the same keys.
+  * first_front_mask: the independent definition "no row dominates it" (brute_force.dominates_matrix).
+  * tournament_winners: explicit tuple comparison and numpy.lexsort per tournament.
   * crowding / environmental_selection: independent numpy brute force, hand-worked examples, and
     the golden vectors under tests/golden/ (written once from the reference itself).
 """
@@ -137,3 +140,9 @@ def tournament_winners(parents: torch.Tensor, fitnesses: List[torch.Tensor]) -> 
     keys = table[parents]
     ordering = chained_stable_argsort(keys.unbind(-1))
     return torch.gather(parents, 1, ordering[:, 0].unsqueeze(1)).squeeze()
+
+
+def first_front_mask(f: torch.Tensor) -> torch.Tensor:
+    """bool (N,): the rows that EvalMonitor.get_pf_fitness / get_pf keep (eval_monitor.py:301-302, :333-335):
+    the whole history is ranked and only ``rank == 0`` is used."""
+    return ranks_by_peeling(f) == 0

@@ -11,6 +11,7 @@
  *               last row of any objective, (next - prev) / (last - first) summed over objectives for the
  *               others, -inf outside the mask                                         non_dominate.py:198-231
  *   selection   order by (rank, -distance with NaN last, index), first topk          non_dominate.py:234-254
+ *   first front rank == 0, i.e. "no row dominates it"                                 eval_monitor.py:301-302
  *
  * Pinned by tests/test_oracle_c.py against the torch restatement (itself pinned by brute force and by
  * the reference's golden vectors) on every small case.  Only tests/ may load this library.
@@ -80,6 +81,19 @@ int oracle_nd_rank(const float* f, int64_t n, int m, int32_t* rank) {
   }
   free(bits); free(count); free(front);
   return level;
+}
+
+/* mask[j] = 1 when no row dominates row j (the rows of rank 0: all that
+ * src/evox/workflows/eval_monitor.py:301-302 keeps of the ranking), by direct search.  No matrix. */
+int oracle_first_front(const float* f, int64_t n, int m, uint8_t* mask) {
+#pragma omp parallel for schedule(dynamic, 256)
+  for (int64_t j = 0; j < n; ++j) {
+    uint8_t free_row = 1;
+    for (int64_t i = 0; i < n && free_row; ++i)
+      if (dominates(f + i * m, f + j * m, m)) free_row = 0;
+    mask[j] = free_row;
+  }
+  return 0;
 }
 
 /* ---- stable ordering helpers: torch.argsort(stable=True) puts NaN last and ties by index */

@@ -45,6 +45,10 @@ def test_workspace_size_and_layout(handle):
     assert 20000 * 320 * 8 <= b <= 20000 * 320 * 8 + 6 * 2**20
     b5 = handle.evox_hip_workspace_bytes(200000, 8)
     assert 5.0e9 < b5 < 5.3e9
+    # the first-front entry builds no matrix: a few arrays of n entries
+    assert handle.evox_hip_first_front_workspace_bytes(0, 3) == 0
+    assert 0 < handle.evox_hip_first_front_workspace_bytes(20000, 3) < 8 * 2**20
+    assert handle.evox_hip_first_front_workspace_bytes(200000, 8) == b5 - 200000 * 3136 * 8
     out = (ctypes.c_int64 * 11)()
     assert handle.evox_hip_workspace_layout(20000, 3, out) == 0
     assert out[1] == 320 and out[2] == 314 and out[0] % 256 == 0 and out[9] == 0
@@ -59,5 +63,9 @@ def test_argument_validation_without_gpu(handle):
     assert handle.evox_hip_non_dominate_rank(p, 10, 3, 3, 1, p, p, 64, None) == _lib.E_WORKSPACE
     assert handle.evox_hip_non_dominate_rank(p, 0, 3, 3, 1, p, p, 64, None) == _lib.E_BAD_ARG
     assert handle.evox_hip_nd_environmental_selection(None, 0, 0, p, 10, 3, 3, 1, 11, None, p, p, p, None, p, 64, None) == _lib.E_BAD_ARG
+    assert handle.evox_hip_first_front_mask(p, 10, 3, 3, 1, None, p, 64, None) == _lib.E_BAD_ARG
+    assert handle.evox_hip_first_front_mask(p, 10, 3, 3, 1, p, p, 64, None) == _lib.E_WORKSPACE
+    assert handle.evox_hip_tournament_pick(None, 4, 2, p, 10, 2, 2, 1, p, None) == _lib.E_BAD_ARG
+    assert handle.evox_hip_tournament_pick(p, 4, 0, p, 10, 2, 2, 1, p, None) == _lib.E_BAD_ARG
     assert handle.evox_hip_set_option(b"no_such_option", 1) == _lib.E_BAD_ARG
     assert handle.evox_hip_set_option(b"peel_blocks_per_cu", 2) == 0

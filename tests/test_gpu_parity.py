@@ -488,6 +488,79 @@ def test_barrier_timeout_is_reported_not_hung():
     assert np.array_equal(as_np(non_dominate_rank(f)), as_np(er.ranks_by_peeling(f.cpu())))
 
 
+# ------------------------------------------------------------------ first front only (rank == 0)
+
+
+@pytest.mark.parametrize("name,f,ks", EDGE, ids=IDS)
+def test_first_front_edge(name, f, ks, population_path):
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd.operators.selection import non_dominated_mask
+
+    say("first_front", name, tuple(f.shape))
+    got = non_dominated_mask(f.to(DEV))
+    assert got.dtype == torch.bool and got.shape == (f.size(0),)
+    assert np.array_equal(as_np(got), as_np(er.first_front_mask(f)))
+    assert runtime.last_status()["error"] == 0
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8, 9, 12])
+def test_first_front_all_m(m, population_path):
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd.operators.selection import non_dominated_mask
+
+    say("first_front_all_m", m)
+    g = torch.Generator("cpu").manual_seed(140 + m)
+    for n in (333, 1500):
+        f = (torch.randint(0, 3 + m, (n, m), generator=g).float() / 4.0).contiguous()
+        f[::17] = f[1::17][: f[::17].size(0)]  # duplicate rows
+        f[5, 0] = float("nan")
+        assert np.array_equal(as_np(non_dominated_mask(f.to(DEV))), as_np(er.first_front_mask(f))), (m, n)
+        ft = f.t().contiguous().t()  # column-major strides
+        assert np.array_equal(as_np(non_dominated_mask(ft.to(DEV))), as_np(er.first_front_mask(f))), (m, n)
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C2p", "C3"])
+def test_first_front_configs_golden(name, population_path):
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd.operators.selection import non_dominated_mask
+
+    say("first_front_golden", name)
+    w, gold = golden_io.config(name)
+    got = as_np(non_dominated_mask(w.f.to(DEV)))
+    assert np.array_equal(got, gold["rank"] == 0)
+
+
+def test_first_front_large_history_and_batch(population_path):
+    """The monitor's use: a long evaluation history.  200 000 rows x 3 objectives need 0.5 TB as a
+    matrix; here the first front comes from the linear-memory entry point and is checked against the
+    plain-C checker.  Then C5 (nearly everything non-dominated: the worst case, every wave scans all
+    the slots below it) against the full ranking."""
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd.operators.selection import non_dominated_mask
+    from oracle import c_oracle
+
+    say("first_front_large")
+    f = workloads.uniform_population(200000, 3, 0, 31)[0]
+    got = as_np(non_dominated_mask(f.to(DEV)))
+    want = c_oracle.first_front(as_np(f))
+    assert np.array_equal(got, want)
+    w = workloads.c5()
+    fd = w.f.to(DEV)
+    got5 = non_dominated_mask(fd)
+    assert torch.equal(got5, non_dominate_rank(fd) == 0)
+    runtime.release_workspaces()
+    # leading batch dimensions and vmap
+    fb = torch.stack([workloads.uniform_population(700, 3, 0, 50 + b)[0] for b in range(4)]).to(DEV)
+    want_b = torch.stack([er.first_front_mask(fb[b].cpu()) for b in range(4)])
+    assert torch.equal(non_dominated_mask(fb).cpu(), want_b)
+    assert torch.equal(torch.vmap(non_dominated_mask)(fb).cpu(), want_b)
+    assert torch.equal(torch.compile(non_dominated_mask, fullgraph=True)(fb[0]).cpu(), want_b[0])
+
+
 # ------------------------------------------------------------------ tournament (consumer of rank / distance)
 
 

@@ -300,3 +300,13 @@ def test_tournament_hand_worked():
     assert got == [1, 0, 3, 3, 5, 6, 1, 4]
     # one round comes back 0-d, as the reference's squeeze() leaves it
     assert er.tournament_winners(parents[:1], [neg_dist, rank]).dim() == 0
+
+
+# -------------------------------------------------------------- first front
+
+
+@pytest.mark.parametrize("name,f,ks", EDGE, ids=IDS)
+def test_first_front_is_the_undominated_set(name, f, ks):
+    got = as_np(er.first_front_mask(f))
+    assert np.array_equal(got, ~bf.dominates_matrix(as_np(f)).any(axis=0))
+    assert got.any()  # a finite population always has a first front

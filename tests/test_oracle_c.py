@@ -23,6 +23,7 @@ def test_edge_cases(name, f, ks):
     rank, fronts = c_oracle.nd_rank(as_np(f))
     want = as_np(er.ranks_by_peeling(f))
     assert np.array_equal(rank, want) and fronts == want.max() + 1
+    assert np.array_equal(c_oracle.first_front(as_np(f)), want == 0)
     g = torch.Generator("cpu").manual_seed(11)
     for mask in (None, torch.rand(f.size(0), generator=g) < 0.5, torch.zeros(f.size(0), dtype=torch.bool)):
         assert same_float(c_oracle.crowding(as_np(f), None if mask is None else as_np(mask)), er.crowding(f, mask)), name
@@ -38,6 +39,7 @@ def test_configs_and_many_objectives():
         _, rank_t, dist_t, order_t = er.environmental_selection(w.f, w.f, w.topk, return_all=True)
         order, rank_c, dist_c, _ = c_oracle.select(as_np(w.f), w.topk)
         assert np.array_equal(order, as_np(order_t)) and np.array_equal(rank_c, as_np(rank_t)) and same_float(dist_c, dist_t)
+        assert np.array_equal(c_oracle.first_front(as_np(w.f)), as_np(rank_t) == 0)
     f = workloads.sphere_shell_population((1500,), 8, 0.05, seed=4)
     _, rank_t, dist_t, order_t = er.environmental_selection(f, f, 750, return_all=True)
     order, rank_c, dist_c, _ = c_oracle.select(as_np(f), 750)
