@@ -29,6 +29,10 @@ _SIGNATURES = {
     "evox_hip_nd_environmental_selection": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                                     c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                     c_size_t, c_void_p]),
+    "evox_hip_nd_environmental_selection_two_part": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64,
+                                                             c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                                             c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                             c_void_p, c_size_t, c_void_p]),
     "evox_hip_batched_max_rows": (c_int64, [c_int64]),
     "evox_hip_batched_non_dominate_rank": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p,
                                                    c_void_p]),

@@ -175,12 +175,24 @@ static void launch_first_front(const Ws& w, uint8_t* mask, hipStream_t s) {
 }
 
 // Fitness -> structure of arrays + keys, state reset, then the slot sort (order.hpp).
-static int stage_prepare(const Ws& w, const float* f, int64_t sr, int64_t sc, bool with_sort, hipStream_t s) {
+// A population given in one part (n_first == n, second part unused) or in two.
+struct Fitness {
+  const float* f;
+  int64_t sr, sc;
+  int64_t n_first;
+  const float* f2;
+  int64_t sr2, sc2;
+};
+
+static Fitness one_part(const float* f, int64_t n, int64_t sr, int64_t sc) { return Fitness{f, sr, sc, n, f, sr, sc}; }
+
+static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStream_t s) {
   const Layout& L = w.L;
-  if (f == nullptr) return kErrBadArg;
+  if (src.f == nullptr || src.f2 == nullptr || src.n_first < 0 || src.n_first > L.n) return kErrBadArg;
   const int64_t zero_words = (int64_t)((L.zero_end - L.ctrl) / 4);
-  hipLaunchKernelGGL(prepare_kernel, dim3(L.prep_blocks), dim3(256), 0, s, f, sr, sc, L.n, L.m, L.npad, w.at<float>(L.xs),
-                     w.at<uint64_t>(L.key), w.at<unsigned long long>(L.partials), w.at<uint32_t>(L.ctrl), zero_words);
+  hipLaunchKernelGGL(prepare_kernel, dim3(L.prep_blocks), dim3(256), 0, s, src.f, src.sr, src.sc, (int)src.n_first, src.f2,
+                     src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs), w.at<uint64_t>(L.key),
+                     w.at<unsigned long long>(L.partials), w.at<uint32_t>(L.ctrl), zero_words);
   EVX_LAUNCH_CHECK();
   if (!with_sort) return 0;
   int blocks = (L.n + 255) / 256;
@@ -462,7 +474,7 @@ int evox_hip_stage_prepare(const float* f, int64_t n, int64_t m, int64_t sr, int
                            void* stream) {
   Ws w;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
-  return stage_prepare(w, f, sr, sc, true, (hipStream_t)stream);
+  return stage_prepare(w, one_part(f, n, sr, sc), true, (hipStream_t)stream);
 }
 
 int evox_hip_stage_dominance(int64_t n, int64_t m, int variant, void* ws, size_t ws_bytes, void* stream) {
@@ -510,7 +522,7 @@ int evox_hip_non_dominate_rank(const float* f, int64_t n, int64_t m, int64_t sr,
   if (rank_out == nullptr) return kErrBadArg;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   hipStream_t s = (hipStream_t)stream;
-  if (int e = stage_prepare(w, f, sr, sc, true, s)) return e;
+  if (int e = stage_prepare(w, one_part(f, n, sr, sc), true, s)) return e;
   if (int e = stage_dominance(w, kDomKey32, s)) return e;
   if (int e = stage_count(w, false, s)) return e;
   if (int e = stage_peel(w, n, false, s)) return e;
@@ -529,7 +541,7 @@ int evox_hip_first_front_mask(const float* f, int64_t n, int64_t m, int64_t sr, 
   if (int e = open_ws(n, m, ws, ws_bytes, &w, false)) return e;
   const Layout& L = w.L;
   hipStream_t s = (hipStream_t)stream;
-  if (int e = stage_prepare(w, f, sr, sc, true, s)) return e;
+  if (int e = stage_prepare(w, one_part(f, n, sr, sc), true, s)) return e;
   switch (L.m) {
     case 1: launch_first_front<1>(w, mask_out, s); break;
     case 2: launch_first_front<2>(w, mask_out, s); break;
@@ -554,7 +566,7 @@ int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   const Layout& L = w.L;
   hipStream_t s = (hipStream_t)stream;
-  if (int e = stage_prepare(w, costs, sr, sc, false, s)) return e;
+  if (int e = stage_prepare(w, one_part(costs, n, sr, sc), false, s)) return e;
   hipLaunchKernelGGL(compact_mask_kernel, dim3(1), dim3(1024), 0, s, mask, mask_stride, L.n, w.at<int>(L.perm),
                      w.at<float>(L.dist), w.ctrl());
   EVX_LAUNCH_CHECK();
@@ -562,18 +574,21 @@ int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t
   return copy_async(dist_out, w.at<float>(L.dist), sizeof(float) * (size_t)n, s);
 }
 
-int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes, const float* f,
-                                        int64_t n, int64_t m, int64_t sr, int64_t sc, int64_t topk, void* out_x,
-                                        float* out_f, int32_t* out_rank, float* out_dist, int32_t* out_order, void* ws,
-                                        size_t ws_bytes, void* stream) {
+}  // extern "C"
+
+// Shared body of the two selection entry points: the population is one part or two.
+static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes, const void* x2,
+                       int64_t x2_row_stride_bytes, const Fitness& fit, int64_t n, int64_t m, int64_t topk, void* out_x,
+                       float* out_f, int32_t* out_rank, float* out_dist, int32_t* out_order, void* ws, size_t ws_bytes,
+                       hipStream_t s) {
   Ws w;
   if (out_f == nullptr || out_rank == nullptr || out_dist == nullptr) return kErrBadArg;
-  if ((x == nullptr) != (out_x == nullptr) || (x != nullptr && (x_row_bytes < 0 || x_row_stride_bytes < 0))) return kErrBadArg;
+  if ((x == nullptr) != (out_x == nullptr) || (x == nullptr) != (x2 == nullptr)) return kErrBadArg;
+  if (x != nullptr && (x_row_bytes < 0 || x_row_stride_bytes < 0 || x2_row_stride_bytes < 0)) return kErrBadArg;
   if (topk < 1 || topk > n) return kErrBadArg;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   const Layout& L = w.L;
-  hipStream_t s = (hipStream_t)stream;
-  if (int e = stage_prepare(w, f, sr, sc, true, s)) return e;
+  if (int e = stage_prepare(w, fit, true, s)) return e;
   if (int e = stage_dominance(w, kDomKey32, s)) return e;
   if (int e = stage_count(w, true, s)) return e;
   if (int e = stage_peel(w, topk, true, s)) return e;
@@ -581,19 +596,54 @@ int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int6
   if (int e = stage_order(w, s)) return e;
   int unit = 1;
   if (x != nullptr) {
-    const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out_x) | (uintptr_t)x_row_bytes |
-                           (uintptr_t)x_row_stride_bytes;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(x2) | reinterpret_cast<uintptr_t>(out_x) |
+                           (uintptr_t)x_row_bytes | (uintptr_t)x_row_stride_bytes | (uintptr_t)x2_row_stride_bytes;
     unit = (bits % 16 == 0) ? 16 : (bits % 4 == 0) ? 4 : 1;
   }
   int blocks = (int)((topk + 3) / 4);
   const int cap = device_cus() * 8;
   if (blocks > cap) blocks = cap;
   hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(256), 0, s, w.at<int>(L.order), (int)topk,
-                     static_cast<const uint8_t*>(x), x_row_stride_bytes, x_row_bytes, static_cast<uint8_t*>(out_x), unit, f,
-                     sr, sc, L.m, out_f, w.at<int>(L.rank), out_rank, w.at<float>(L.dist), out_dist, w.ctrl());
+                     static_cast<const uint8_t*>(x), x_row_stride_bytes, x_row_bytes, static_cast<uint8_t*>(out_x), unit, fit.f,
+                     fit.sr, fit.sc, (int)fit.n_first, static_cast<const uint8_t*>(x2), x2_row_stride_bytes, fit.f2, fit.sr2,
+                     fit.sc2, L.m, out_f, w.at<int>(L.rank), out_rank, w.at<float>(L.dist), out_dist, w.ctrl());
   EVX_LAUNCH_CHECK();
   if (out_order) return copy_async(out_order, w.at<int>(L.order), sizeof(int) * (size_t)topk, s);
   return 0;
+}
+
+extern "C" {
+
+int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes, const float* f,
+                                        int64_t n, int64_t m, int64_t sr, int64_t sc, int64_t topk, void* out_x,
+                                        float* out_f, int32_t* out_rank, float* out_dist, int32_t* out_order, void* ws,
+                                        size_t ws_bytes, void* stream) {
+  if (f == nullptr) return kErrBadArg;
+  return select_rows(x, x_row_bytes, x_row_stride_bytes, x, x_row_stride_bytes, one_part(f, n, sr, sc), n, m, topk, out_x,
+                     out_f, out_rank, out_dist, out_order, ws, ws_bytes, (hipStream_t)stream);
+}
+
+int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_row_stride_bytes, const void* x_b,
+                                                 int64_t x_b_row_stride_bytes, int64_t x_row_bytes, const float* f_a,
+                                                 int64_t n_a, int64_t f_a_stride_row, int64_t f_a_stride_col,
+                                                 const float* f_b, int64_t n_b, int64_t f_b_stride_row,
+                                                 int64_t f_b_stride_col, int64_t m, int64_t topk, void* out_x, float* out_f,
+                                                 int32_t* out_rank, float* out_dist, int32_t* out_order, void* ws,
+                                                 size_t ws_bytes, void* stream) {
+  if (n_a < 0 || n_b < 0 || n_a > 0x7FFFFF00ll || n_b > 0x7FFFFF00ll) return kErrBadArg;
+  // a part without rows may come with null pointers: it is never read, the other part stands in for it
+  if (n_a == 0) {
+    f_a = f_b;
+    x_a = x_b;
+  }
+  if (n_b == 0) {
+    f_b = f_a;
+    x_b = x_a;
+  }
+  if (f_a == nullptr || f_b == nullptr) return kErrBadArg;
+  const Fitness fit{f_a, f_a_stride_row, f_a_stride_col, n_a, f_b, f_b_stride_row, f_b_stride_col};
+  return select_rows(x_a, x_row_bytes, x_a_row_stride_bytes, x_b, x_b_row_stride_bytes, fit, n_a + n_b, m, topk, out_x, out_f,
+                     out_rank, out_dist, out_order, ws, ws_bytes, (hipStream_t)stream);
 }
 
 int64_t evox_hip_batched_max_rows(int64_t m) { return (m >= 1 && m <= 8) ? kBatchedMaxRows : 0; }

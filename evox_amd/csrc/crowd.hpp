@@ -167,21 +167,25 @@ __global__ __launch_bounds__(256) void final_order_kernel(const int* __restrict_
 }
 
 // out[p, :] = src[order[p], :] for the decision vectors (raw bytes, any dtype), the fitness, the rank
-// and the distance.  One wave per output row; rows are copied in 16-, 4- or 1-byte units.
+// and the distance.  Rows from n_first on are read from the second part (x2, f2) of a two-part population.
+// One wave per output row; rows are copied in 16-, 4- or 1-byte units.
 __global__ __launch_bounds__(256) void gather_kernel(const int* __restrict__ order, int topk, const uint8_t* __restrict__ x,
                                                      int64_t x_row_stride, int64_t x_row_bytes, uint8_t* __restrict__ out_x,
                                                      int unit, const float* __restrict__ f, int64_t f_stride_row,
-                                                     int64_t f_stride_col, int m, float* __restrict__ out_f,
-                                                     const int* __restrict__ rank, int* __restrict__ out_rank,
-                                                     const float* __restrict__ dist, float* __restrict__ out_dist,
-                                                     const Ctrl* __restrict__ ctrl) {
+                                                     int64_t f_stride_col, int n_first, const uint8_t* __restrict__ x2,
+                                                     int64_t x2_row_stride, const float* __restrict__ f2,
+                                                     int64_t f2_stride_row, int64_t f2_stride_col, int m,
+                                                     float* __restrict__ out_f, const int* __restrict__ rank,
+                                                     int* __restrict__ out_rank, const float* __restrict__ dist,
+                                                     float* __restrict__ out_dist, const Ctrl* __restrict__ ctrl) {
   if (ctrl->err != 0) return;  // `order` was not produced: the outputs stay as the caller left them
   const int lane = threadIdx.x & 63;
   const int waves = gridDim.x * (blockDim.x >> 6);
   for (int p = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); p < topk; p += waves) {
     const int64_t src = order[p];
+    const bool second = src >= n_first;  // rows of the second part of a two-part population
     if (x) {
-      const uint8_t* __restrict__ s = x + src * x_row_stride;
+      const uint8_t* __restrict__ s = second ? x2 + (src - n_first) * x2_row_stride : x + src * x_row_stride;
       uint8_t* __restrict__ d = out_x + (int64_t)p * x_row_bytes;
       if (unit == 16) {
         for (int64_t b = lane * 16; b < x_row_bytes; b += 64 * 16)
@@ -193,7 +197,9 @@ __global__ __launch_bounds__(256) void gather_kernel(const int* __restrict__ ord
         for (int64_t b = lane; b < x_row_bytes; b += 64) d[b] = s[b];
       }
     }
-    for (int k = lane; k < m; k += 64) out_f[(int64_t)p * m + k] = f[src * f_stride_row + k * f_stride_col];
+    for (int k = lane; k < m; k += 64)
+      out_f[(int64_t)p * m + k] =
+          second ? f2[(src - n_first) * f2_stride_row + k * f2_stride_col] : f[src * f_stride_row + k * f_stride_col];
     if (lane == 0) {
       out_rank[p] = rank[src];
       out_dist[p] = dist[src];

@@ -31,8 +31,11 @@ namespace evx {
 // order (padded with NaN to npad, a multiple of 128 rows) plus the 64-bit row keys, leaves the
 // (min, max) key of each block in `partials` for the slot sort, and clears the state arrays that
 // later kernels accumulate into.
+// The population may come in two parts (rows 0..n_first-1 from f, the rest from f2: parents and
+// offspring that the caller never concatenates, src/evox/algorithms/mo/nsga2.py:99-100).
 __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ f, int64_t stride_row, int64_t stride_col,
-                                                      int n, int m, int npad, float* __restrict__ xs,
+                                                      int n_first, const float* __restrict__ f2, int64_t stride_row2,
+                                                      int64_t stride_col2, int n, int m, int npad, float* __restrict__ xs,
                                                       uint64_t* __restrict__ key, unsigned long long* __restrict__ partials,
                                                       uint32_t* __restrict__ zero_words, int64_t n_zero_words) {
   __shared__ unsigned long long red[2][4];
@@ -42,7 +45,9 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
   for (int64_t i = tid; i < npad; i += nthreads) {
     uint64_t s = 0;
     for (int k = 0; k < m; ++k) {
-      const float v = i < n ? f[i * stride_row + k * stride_col] : __uint_as_float(0x7FC00000u);
+      const float v = i < n_first ? f[i * stride_row + k * stride_col]
+                      : i < n     ? f2[(i - n_first) * stride_row2 + k * stride_col2]
+                                  : __uint_as_float(0x7FC00000u);
       xs[(int64_t)k * npad + i] = v;
       s += ordered_key(v);
     }

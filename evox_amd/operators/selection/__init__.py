@@ -1,10 +1,17 @@
 __all__ = [
     "crowding_distance",
     "nd_environmental_selection",
+    "nd_environmental_selection_two_part",
     "non_dominate_rank",
     "non_dominated_mask",
     "tournament_selection_multifit",
 ]
 
-from .non_dominate import crowding_distance, nd_environmental_selection, non_dominate_rank, non_dominated_mask
+from .non_dominate import (
+    crowding_distance,
+    nd_environmental_selection,
+    nd_environmental_selection_two_part,
+    non_dominate_rank,
+    non_dominated_mask,
+)
 from .tournament_selection import tournament_selection_multifit

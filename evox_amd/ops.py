@@ -241,6 +241,70 @@ def _nd_select_vmap(info, in_dims, x, f, topk):
 torch.library.register_vmap(nd_select, _nd_select_vmap)
 
 
+@torch.library.custom_op("evox_amd::nd_select_two_part", mutates_args=())
+def nd_select_two_part(x_a: torch.Tensor, f_a: torch.Tensor, x_b: torch.Tensor, f_b: torch.Tensor,
+                       topk: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """nd_select on the concatenation of (x_a, f_a) and (x_b, f_b) along the rows, without making it.
+    x_* (N_*, *D), f_* (N_*, M); one population (no leading batch dimensions)."""
+    for t, what in ((f_a, "fitness"), (f_b, "fitness"), (x_a, "decision vectors"), (x_b, "decision vectors")):
+        runtime.require_gpu_tensor(t, what)
+    if f_a.dim() != 2 or f_b.dim() != 2 or f_a.size(1) != f_b.size(1):
+        raise ValueError(f"fitness parts must be (N_a, M) and (N_b, M); got {tuple(f_a.shape)} and {tuple(f_b.shape)}")
+    if x_a.dim() < 1 or x_b.dim() < 1 or x_a.shape[1:] != x_b.shape[1:] or x_a.dtype != x_b.dtype:
+        raise ValueError("the decision vectors of the two parts differ in row shape or dtype")
+    if x_a.size(0) != f_a.size(0) or x_b.size(0) != f_b.size(0):
+        raise ValueError("decision vectors and fitness disagree on the number of rows")
+    if len({x_a.device, x_b.device, f_a.device, f_b.device}) != 1:
+        raise RuntimeError("the parts are on different devices")
+    if f_a.dtype != f_b.dtype:
+        raise TypeError("the fitness parts differ in dtype")
+    n_a, n_b, m = f_a.size(0), f_b.size(0), f_a.size(1)
+    n = n_a + n_b
+    if topk > n:
+        raise RuntimeError(f"selected index k out of range: topk={topk} exceeds the population size {n}")
+    if topk < 1:
+        raise IndexError(f"topk must be at least 1; got {topk}")
+    if m == 0:
+        raise ValueError("fitness must have at least one objective")
+    fa32, fb32 = _as_f32(f_a, "fitness"), _as_f32(f_b, "fitness")
+    tail = x_a.shape[1:]
+    out_x = torch.empty(topk, *tail, dtype=x_a.dtype, device=x_a.device)
+    out_f = torch.empty(topk, m, dtype=torch.float32, device=f_a.device)
+    out_rank = torch.empty(topk, dtype=torch.int32, device=f_a.device)
+    out_dist = torch.empty(topk, dtype=torch.float32, device=f_a.device)
+    with torch.cuda.device(f_a.device):
+        width = 1
+        for d in tail:
+            width *= d
+        xa, xb = x_a.reshape(n_a, width), x_b.reshape(n_b, width)
+        if xa.size(1) > 1 and xa.stride(1) != 1:
+            xa = xa.contiguous()
+        if xb.size(1) > 1 and xb.stride(1) != 1:
+            xb = xb.contiguous()
+        es = xa.element_size()
+        row_bytes = xa.size(1) * es
+        has_x = row_bytes > 0
+        ws = runtime.workspace(n, m, f_a.device)
+        stream = runtime.stream_handle(f_a.device)
+        _lib.call("evox_hip_nd_environmental_selection_two_part", xa.data_ptr() if has_x else None, xa.stride(0) * es,
+                  xb.data_ptr() if has_x else None, xb.stride(0) * es, row_bytes, fa32.data_ptr(), n_a, fa32.stride(0),
+                  fa32.stride(1), fb32.data_ptr(), n_b, fb32.stride(0), fb32.stride(1), m, topk,
+                  out_x.data_ptr() if has_x else None, out_f.data_ptr(), out_rank.data_ptr(), out_dist.data_ptr(), None,
+                  ws.data_ptr(), ws.numel(), stream)
+        runtime.note_call(ws, stream)
+    return out_x, out_f.to(f_a.dtype), out_rank, out_dist
+
+
+@nd_select_two_part.register_fake
+def _(x_a, f_a, x_b, f_b, topk):
+    return (
+        x_a.new_empty(topk, *x_a.shape[1:]),
+        f_a.new_empty(topk, f_a.shape[-1]),
+        f_a.new_empty(topk, dtype=torch.int32),
+        f_a.new_empty(topk, dtype=torch.float32),
+    )
+
+
 @torch.library.custom_op("evox_amd::tournament_pick", mutates_args=())
 def tournament_pick(parents: torch.Tensor, fitness: torch.Tensor) -> torch.Tensor:
     """parents (n_round, t) int64 candidate indices, fitness (candidates, keys) float32 -> (n_round,) int64 winners."""

@@ -76,6 +76,22 @@ int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int6
                                         void* out_x, float* out_f, int32_t* out_rank, float* out_dist,
                                         int32_t* out_order, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same selection over a population that is given in two parts (rows 0..n_a-1 = part a, rows n_a.. = part
+ * b), with the results exactly those of the entry point above on their concatenation.  Replaces, together
+ * with it, the merge step of NSGA-II
+ *     merge_pop = torch.cat([self.pop, offspring]); merge_fit = torch.cat([self.fit, off_fit])
+ *     ... = nd_environmental_selection(merge_pop, merge_fit, self.pop_size)
+ * (src/evox/algorithms/mo/nsga2.py:99-102): parents and offspring are read where they lie and the
+ * concatenated copies are never made.  A part with no rows may pass NULL pointers.
+ * Workspace: evox_hip_workspace_bytes(n_a + n_b, m). */
+int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_row_stride_bytes, const void* x_b,
+                                                 int64_t x_b_row_stride_bytes, int64_t x_row_bytes, const float* f_a,
+                                                 int64_t n_a, int64_t f_a_stride_row, int64_t f_a_stride_col,
+                                                 const float* f_b, int64_t n_b, int64_t f_b_stride_row,
+                                                 int64_t f_b_stride_col, int64_t m, int64_t topk, void* out_x, float* out_f,
+                                                 int32_t* out_rank, float* out_dist, int32_t* out_order, void* workspace,
+                                                 size_t workspace_bytes, void* stream);
+
 /* ---- many small populations at once (what the reference reaches through vmap: non_dominate.py:107-125
  * for the peeling, the rest of the path batching natively).  One workgroup per population, no workspace.
  * n <= evox_hip_batched_max_rows(m) (1024 rows for m <= 8, 0 = unsupported); f is addressed as

@@ -15,6 +15,7 @@ the reference's multi-objective environmental selection, on torch CPU tensors:
   environmental_selection   <- src/evox/operators/selection/non_dominate.py:234-254
   tournament_winners        <- src/evox/operators/selection/tournament_selection.py:18-27
   first_front_mask          <- src/evox/workflows/eval_monitor.py:301-302 (= :333-334)
+  merged_selection          <- src/evox/algorithms/mo/nsga2.py:99-102
 
 How each function is pinned (tests/test_oracle.py):
   * dominance / ranks: tiny-input brute force, longest-dominator-chain definition, Deb's fast
@@ -146,3 +147,8 @@ def first_front_mask(f: torch.Tensor) -> torch.Tensor:
     """bool (N,): the rows that EvalMonitor.get_pf_fitness / get_pf keep (eval_monitor.py:301-302, :333-335):
     the whole history is ranked and only ``rank == 0`` is used."""
     return ranks_by_peeling(f) == 0
+
+
+def merged_selection(x_a, f_a, x_b, f_b, topk: int, return_all: bool = False):
+    """The merge step of NSGA-II, nsga2.py:99-102: concatenate parents and offspring, then select."""
+    return environmental_selection(torch.cat([x_a, x_b], dim=0), torch.cat([f_a, f_b], dim=0), topk, return_all)

@@ -67,5 +67,11 @@ def test_argument_validation_without_gpu(handle):
     assert handle.evox_hip_first_front_mask(p, 10, 3, 3, 1, p, p, 64, None) == _lib.E_WORKSPACE
     assert handle.evox_hip_tournament_pick(None, 4, 2, p, 10, 2, 2, 1, p, None) == _lib.E_BAD_ARG
     assert handle.evox_hip_tournament_pick(p, 4, 0, p, 10, 2, 2, 1, p, None) == _lib.E_BAD_ARG
+    assert handle.evox_hip_nd_environmental_selection_two_part(None, 0, None, 0, 0, p, 5, 3, 1, p, 5, 3, 1, 3, 11, None, p, p, p,
+                                                               None, p, 64, None) == _lib.E_BAD_ARG  # topk > n_a + n_b
+    assert handle.evox_hip_nd_environmental_selection_two_part(None, 0, None, 0, 0, p, 5, 3, 1, None, 5, 3, 1, 3, 4, None, p, p,
+                                                               p, None, p, 64, None) == _lib.E_BAD_ARG  # missing part
+    assert handle.evox_hip_nd_environmental_selection_two_part(None, 0, None, 0, 0, p, 5, 3, 1, p, 5, 3, 1, 3, 4, None, p, p, p,
+                                                               None, p, 64, None) == _lib.E_WORKSPACE
     assert handle.evox_hip_set_option(b"no_such_option", 1) == _lib.E_BAD_ARG
     assert handle.evox_hip_set_option(b"peel_blocks_per_cu", 2) == 0

@@ -561,6 +561,68 @@ def test_first_front_large_history_and_batch(population_path):
     assert torch.equal(torch.compile(non_dominated_mask, fullgraph=True)(fb[0]).cpu(), want_b[0])
 
 
+# ------------------------------------------------------------------ parents + offspring given as two parts
+
+
+@pytest.mark.parametrize("name", ["C1", "C2p", "C3"])
+def test_two_part_selection_golden(name, population_path):
+    if population_path != "pipeline":
+        pytest.skip("the two-part entry always takes the pipeline")
+    from evox_amd.operators.selection import nd_environmental_selection_two_part
+
+    w, gold = golden_io.config(name)
+    n = w.f.size(0)
+    x = w.x if w.x is not None else torch.arange(n, dtype=torch.float32)[:, None].repeat(1, 3)
+    fd, xd = w.f.to(DEV), x.to(DEV)
+    order = gold["order"]
+    for cut in (n // 2, 1, n - 1, 0, n, 129):
+        say("two_part", name, cut)
+        xs, fs, rs, ds = nd_environmental_selection_two_part(xd[:cut], fd[:cut], xd[cut:], fd[cut:], w.topk)
+        assert np.array_equal(as_np(rs), gold["rank"][order])
+        assert np.array_equal(as_np(fs), as_np(w.f)[order]) and np.array_equal(as_np(xs), as_np(x)[order])
+        assert_dist_close(ds, gold["dist"][order], f"{name} cut {cut}")
+    # parts with strides of their own: column-major fitness in one, padded rows of x in the other
+    cut = n // 3
+    fa = fd[:cut].t().contiguous().t()
+    xb = torch.zeros(n - cut, x.size(1) + 5, device=DEV)[:, : x.size(1)]
+    xb.copy_(xd[cut:])
+    xs, fs, rs, ds = nd_environmental_selection_two_part(xd[:cut], fa, xb, fd[cut:], w.topk)
+    assert np.array_equal(as_np(rs), gold["rank"][order]) and np.array_equal(as_np(xs), as_np(x)[order])
+
+
+def test_two_part_selection_edge_and_errors(edge_golden, population_path):
+    if population_path != "pipeline":
+        pytest.skip("the two-part entry always takes the pipeline")
+    from evox_amd.operators.selection import nd_environmental_selection_two_part
+
+    for name, f, ks in EDGE:
+        n = f.size(0)
+        x = torch.arange(n, dtype=torch.float64)[:, None, None].repeat(1, 2, 2)  # any dtype, any row shape
+        for k in ks:
+            for cut in sorted({0, n // 2, n}):
+                say("two_part_edge", name, k, cut)
+                want, _, _, order = er.merged_selection(x[:cut], f[:cut], x[cut:], f[cut:], k, return_all=True)
+                assert np.array_equal(as_np(order), edge_golden[f"{name}/order@{k}"])
+                got = nd_environmental_selection_two_part(x[:cut].to(DEV), f[:cut].to(DEV), x[cut:].to(DEV), f[cut:].to(DEV), k)
+                assert np.array_equal(as_np(got[0]), as_np(want[0])) and np.array_equal(as_np(got[2]), as_np(want[2]))
+                assert np.array_equal(as_np(got[1]), as_np(want[1]), equal_nan=True)
+                assert_dist_close(got[3], as_np(want[3]), f"{name}@{k}")
+    f = torch.rand(6, 2, device=DEV)
+    x = torch.rand(6, 4, device=DEV)
+    with pytest.raises(RuntimeError):
+        nd_environmental_selection_two_part(x[:3], f[:3], x[3:], f[3:], 7)
+    with pytest.raises(IndexError):
+        nd_environmental_selection_two_part(x[:3], f[:3], x[3:], f[3:], 0)
+    with pytest.raises(ValueError):
+        nd_environmental_selection_two_part(x[:3], f[:3], x[3:, :2], f[3:], 2)
+    with pytest.raises(ValueError):
+        nd_environmental_selection_two_part(x[:3], f[:3], x[3:], f[3:, :1], 2)
+    compiled = torch.compile(nd_environmental_selection_two_part, fullgraph=True)
+    a = compiled(x[:3], f[:3], x[3:], f[3:], 4)
+    b = nd_environmental_selection(x, f, 4)
+    assert all(torch.equal(p, q) for p, q in zip(a, b))
+
+
 # ------------------------------------------------------------------ tournament (consumer of rank / distance)
 
 
