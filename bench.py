@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the environmental-selection hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3|C2|C1|C5] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3|C2|C1|C5] [--no-cpu] [--next-rows]
 
 One step = one `nd_environmental_selection` call on the workload (default C3: N=20000, M=3,
 D=100, topk=10000, fitness i.i.d. U[0,1) from seed 0), inputs and outputs resident in HBM.
@@ -25,6 +25,15 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 VALU_CMP_PEAK_GOPS = 39321.6  # 256 CU x 64 lanes/clk x 2.4 GHz: issue peak of v_cmp_*_f32 (not packable)
 FP32_VECTOR_PEAK_GFLOPS = 157300.0
 
+# HBM bytes per launch from rocprofv3 counter runs of this script (FETCH_SIZE and WRITE_SIZE in runs of
+# their own, scaled by what the same counters read for a 512 MiB copy: x2.0 and x1.0); the summaries
+# with the commands are kept under profiles/.  Keyed by (workload, kernel); absent = not measured.
+MEASURED_TRAFFIC_BYTES = {
+    ("C3", "peel_kernel"): 19.12e6 + 6.17e6,
+    ("C3", "dominance_kernel"): 3.19e6 + 25.44e6,
+    ("C3", "count_kernel"): 26.99e6 + 1.31e6,
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -37,6 +46,9 @@ def parse():
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 512 MiB device copy three times, so that a rocprofv3 --pmc run of this "
                          "command holds a kernel of known traffic next to the selection kernels")
+    ap.add_argument("--next-rows", action="store_true",
+                    help="also time the entry points around the hot path (first-front mask, two-part selection, "
+                         "tournament) and add them to the JSON line under \"next_rows\"")
     return ap.parse_args()
 
 
@@ -132,6 +144,42 @@ def cpu_baseline(w, sample_rows):
     }
 
 
+def next_rows(dev, reps):
+    """Times of the entry points either side of the hot path, on inputs resident in HBM."""
+    from evox_amd import workloads
+    from evox_amd.operators.selection import (nd_environmental_selection, nd_environmental_selection_two_part,
+                                              non_dominate_rank, non_dominated_mask, tournament_selection_multifit)
+
+    out = {}
+    # first front of a long evaluation history (what the monitor asks for) against ranking all of it
+    for n, m in ((20000, 3), (200000, 3), (1000000, 3)):
+        f = workloads.uniform_population(n, m, 0, 7)[0].to(dev)
+        non_dominated_mask(f)
+        t = event_time_us(lambda: non_dominated_mask(f), reps, inner=2)
+        row = {"first_front_us": t, "front_rows": int(non_dominated_mask(f).sum())}
+        if n <= 200000:
+            non_dominate_rank(f)
+            row["full_rank_us"] = event_time_us(lambda: non_dominate_rank(f), max(3, reps // 4), inner=1)
+        out[f"first_front N={n} M={m}"] = row
+        del f
+    # parents + offspring: two-part entry against cat + selection (C3 split in halves)
+    w = workloads.c3()
+    f, x = w.f.to(dev), w.x.to(dev)
+    h = f.size(0) // 2
+    xa, fa, xb, fb = x[:h].clone(), f[:h].clone(), x[h:].clone(), f[h:].clone()
+    nd_environmental_selection_two_part(xa, fa, xb, fb, w.topk)
+    out["two_part C3"] = {
+        "two_part_us": event_time_us(lambda: nd_environmental_selection_two_part(xa, fa, xb, fb, w.topk), reps),
+        "cat_then_select_us": event_time_us(
+            lambda: nd_environmental_selection(torch.cat([xa, xb]), torch.cat([fa, fb]), w.topk), reps),
+    }
+    # mating selection on the survivors' rank and distance (10000 binary tournaments)
+    _, _, rank, dist = nd_environmental_selection(x, f, w.topk)
+    tournament_selection_multifit(w.topk, [-dist, rank])
+    out["tournament 10000 x 2"] = {"us": event_time_us(lambda: tournament_selection_multifit(w.topk, [-dist, rank]), reps)}
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -178,7 +226,7 @@ def main():
     compares = 2.0 * m * pairs  # the reference's `<=` and `<` per objective and ordered pair
     # Bytes that the algorithm must move.  Rows live in slots (sorted by key) and only words 0..slot/64
     # of a row can be non-zero, so a row read costs row_words(slot) * 8 bytes.
-    #   dominance: fitness in, the full matrix out (the upper triangle is stored as zeros)
+    #   dominance: fitness in, the words of the lower triangle out (nothing above the diagonal is stored)
     #   count:     every row read once
     #   peel:      witness pass: a row is rescanned at least once, in the pass that ranks it; plus the
     #              front bitmap (one word per 128-byte line) read by the sweepers each pass
@@ -187,7 +235,7 @@ def main():
     passes = status["passes"]
     ranked_in_passes = (rank >= 1) & (rank <= passes)
     peel_bytes = int(row_read[ranked_in_passes].sum()) + passes * nwords * 8
-    dom_bytes = n * m * 4 + n * row_bytes
+    dom_bytes = n * m * 4 + int(row_read.sum())
     slots = torch.arange(n, device=rank.device)
     evaluated_pairs = float(((((slots >> 6) << 6) + 63) // 256 * 256 + 256).clamp(max=nwords * 64).sum())
     executed_valu = (m + 2) * evaluated_pairs
@@ -221,6 +269,7 @@ def main():
         "bound": "hbm" if d["bound"] == "hbm" else "valu",
         "achieved": d["achieved"], "peak": d["peak"], "unit": d["unit"], "frac": d["frac"], "traffic": None,
     }
+    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get((args.workload, roofline["kernel"]))
 
     out = {
         "metric": "dominance comparisons/sec through nd_environmental_selection (N^2 ordered pairs per step)",
@@ -245,6 +294,8 @@ def main():
         "roofline": roofline,
         "phases": phases,
     }
+    if args.next_rows:
+        out["next_rows"] = next_rows(dev, max(5, min(args.steps, 20)))
     if not args.no_cpu:
         base = cpu_baseline(w, args.cpu_sample)
         out["cpu_baseline"] = base

@@ -38,11 +38,16 @@ struct Ctrl {
   int listed;       // front bitmaps 0 .. listed-1 have been listed and cleared; polled by the barrier master
   int radix_epoch;  // runs of a radix sort kernel so far: each takes a fresh range of barrier generations
   int reserved[7];
-  // grid barrier: block 0 publishes (generation << 32 | rows found by all blocks) in `release`,
-  // every other block publishes (generation << 32 | rows it found) in its own `arrive` slot
+  // grid barrier: block 0 publishes (generation << 32 | rows found by all blocks) in `release` and in
+  // kReleaseCopies copies of it, one per 128-byte line, so that the waiting blocks do not all poll one
+  // address; all-ones means "give up" (a bounded wait ran out).  Every other block publishes
+  // (generation << 32 | rows it found) in its own `arrive` slot.
   unsigned long long release;
-  unsigned long long pad[7];
+  unsigned long long pad[15];
+  unsigned long long release_copy[32 * 16];
   unsigned long long arrive[1];  // one slot per block (allocated to the grid size)
 };
+constexpr int kReleaseCopies = 32;
+constexpr unsigned long long kReleaseGiveUp = ~0ull;
 
 }  // namespace evx

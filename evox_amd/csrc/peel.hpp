@@ -214,27 +214,33 @@ __device__ inline bool sweeper_barrier(Ctrl* ctrl, unsigned gen, int block_tally
   const unsigned long long want = (unsigned long long)gen << 32;
   if (threadIdx.x == 0) {
     coherent_store(&ctrl->arrive[blockIdx.x], want | (unsigned)block_tally);
+    const unsigned long long* mine = &ctrl->release_copy[(blockIdx.x % kReleaseCopies) * 16];
     unsigned long long v = 0;
-    if (!bounded_wait([&] { return (v = coherent_load(&ctrl->release)) >= want; }, spin_limit))
-      coherent_store(&ctrl->err, kErrBarrierTimeout);
+    const bool seen = bounded_wait([&] { return (v = coherent_load(mine)) >= want; }, spin_limit);
+    if (!seen) coherent_store(&ctrl->err, kErrBarrierTimeout);
     scratch[0] = (int)(unsigned)(v & 0xFFFFFFFFull);
-    scratch[1] = coherent_load(&ctrl->err);
+    scratch[1] = seen && v != kReleaseGiveUp;
   }
   __syncthreads();
   *total_out = scratch[0];
-  const bool fine = scratch[1] == 0;
+  const bool fine = scratch[1] != 0;
   __syncthreads();  // scratch is reused by the caller
   return fine;
 }
 
-// Master side: gathers the tallies of generation `gen`, waits until the lister has cleared the bitmap
-// that the coming pass will fill (`listed_needed` fronts cleared), then releases the sweepers.
+// Master side: gathers the tallies of generation `gen` while one thread waits until the lister has
+// cleared the bitmap that the coming pass will fill (`listed_needed` fronts cleared), then releases the
+// sweepers.  After a timeout it releases them with the give-up word, so that nobody waits on.
 __device__ inline bool master_barrier(Ctrl* ctrl, unsigned gen, int listed_needed, int* total_out, unsigned spin_limit,
                                       int* scratch) {
   const unsigned long long want = (unsigned long long)gen << 32;
   const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int waves = blockDim.x >> 6;
   bool ok = true;
   int sum = 0;
+  if (threadIdx.x == blockDim.x - 1)
+    ok &= bounded_wait([&] { return coherent_load(&ctrl->listed) >= listed_needed; }, spin_limit);
   for (unsigned b = kFirstSweeper + threadIdx.x; b < gridDim.x; b += blockDim.x) {
     unsigned long long v = 0;
     ok &= bounded_wait([&] { return (v = coherent_load(&ctrl->arrive[b])) >= want; }, spin_limit);
@@ -242,22 +248,26 @@ __device__ inline bool master_barrier(Ctrl* ctrl, unsigned gen, int listed_neede
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-  if (lane == 0) scratch[threadIdx.x >> 6] = sum;
-  if (!ok) coherent_store(&ctrl->err, kErrBarrierTimeout);
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int total = 0;
-    for (int v = 0; v < (int)(blockDim.x >> 6); ++v) total += scratch[v];
-    if (!bounded_wait([&] { return coherent_load(&ctrl->listed) >= listed_needed; }, spin_limit))
-      coherent_store(&ctrl->err, kErrBarrierTimeout);
-    coherent_store(&ctrl->release, want | (unsigned)total);
-    scratch[40] = total;
-    scratch[41] = coherent_load(&ctrl->err);
+  const bool wave_ok = __builtin_amdgcn_ballot_w64(!ok) == 0ull;
+  if (lane == 0) {
+    scratch[wave] = sum;
+    scratch[16 + wave] = wave_ok;
   }
   __syncthreads();
-  *total_out = scratch[40];
-  const bool fine = scratch[41] == 0;
-  __syncthreads();
+  int total = 0;
+  bool fine = true;
+  for (int v = 0; v < waves; ++v) {
+    total += scratch[v];
+    fine &= scratch[16 + v] != 0;
+  }
+  const unsigned long long word = fine ? (want | (unsigned)total) : kReleaseGiveUp;
+  if (threadIdx.x < kReleaseCopies) coherent_store(&ctrl->release_copy[threadIdx.x * 16], word);
+  if (threadIdx.x == kReleaseCopies) {
+    if (!fine) coherent_store(&ctrl->err, kErrBarrierTimeout);
+    coherent_store(&ctrl->release, word);
+  }
+  __syncthreads();  // scratch is reused by the next call
+  *total_out = total;
   return fine;
 }
 
@@ -508,9 +518,11 @@ __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __re
       if (level > 0) {
         const unsigned long long want = (unsigned long long)level << 32;
         if (threadIdx.x == 0) {
-          if (!bounded_wait([&] { return coherent_load(&ctrl->release) >= want || coherent_load(&ctrl->err) != 0; }, spin_limit))
+          unsigned long long v = 0;
+          if (!bounded_wait([&] { return (v = coherent_load(&ctrl->release)) >= want || coherent_load(&ctrl->err) != 0; },
+                            spin_limit))
             coherent_store(&ctrl->err, kErrBarrierTimeout);
-          scratch[48] = coherent_load(&ctrl->err);
+          scratch[48] = coherent_load(&ctrl->err) | (v == kReleaseGiveUp);
         }
         __syncthreads();
         const bool bad = scratch[48] != 0;
@@ -573,6 +585,8 @@ __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __re
   c.orig_of = orig_of;
   c.rank = rank;
   WitnessState st;
+  int size = coherent_load(&fsize[0]);  // size of front `level`
+  if (size <= 0 || size >= stop_count) return;  // front 0 already holds every row asked for: no pass
   if (use_witness) {
     witness_load(st, c, witness, first_row, row_step);
     for (int w = threadIdx.x; w < nwords; w += blockDim.x) {
@@ -581,8 +595,7 @@ __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __re
     }
   }
   int level = 0;
-  int ranked = 0;                        // rows in fronts 0 .. level-1
-  int size = coherent_load(&fsize[0]);   // size of front `level`
+  int ranked = 0;  // rows in fronts 0 .. level-1
   for (;;) {
     EVX_TRACE(level, 0);
     if (size <= 0 || ranked + size >= stop_count) break;  // size 0 cannot happen for 1 <= stop_count <= n
@@ -590,12 +603,24 @@ __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __re
     c.next_slot = fronts_slot + (int64_t)((level + 1) % kFrontBuffers) * nwords * kFrontStride;
     c.next_orig = fronts_orig + (int64_t)((level + 1) % kFrontBuffers) * nwords * kFrontStride;
     c.next_level = level + 1;
-    for (int w = threadIdx.x; w < nwords; w += blockDim.x) {
-      const uint64_t fw = coherent_load(&cur[(int64_t)w * kFrontStride]);
-      if (use_witness)
-        alive_lds[w] &= ~fw;
-      else
-        front_lds[w] = fw;
+    // the words of the front just finished, four per thread in flight at once
+    for (int w0 = threadIdx.x; w0 < nwords; w0 += 4 * blockDim.x) {
+      uint64_t fw[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int w = w0 + u * blockDim.x;
+        fw[u] = w < nwords ? coherent_load(&cur[(int64_t)w * kFrontStride]) : 0ull;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int w = w0 + u * blockDim.x;
+        if (w < nwords) {
+          if (use_witness)
+            alive_lds[w] &= ~fw[u];
+          else
+            front_lds[w] = fw[u];
+        }
+      }
     }
     __syncthreads();
     EVX_TRACE(level, 1);
