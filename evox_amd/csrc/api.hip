@@ -15,11 +15,14 @@
 namespace evx {
 
 constexpr int kMaxGrid = 4096;  // slots of the grid barrier
+constexpr int kRecordsMaxRows = 65534;  // largest population peeled with the record protocol
 constexpr int kRadixMaxWorkers = 510;
 
 struct Options {
   int peel_blocks_per_cu = 2;
   int peel_witness = 1;
+  int peel_record_blocks = 128;  // sweeping blocks of the record protocol, 16 .. 255 (plus the lister)
+  int peel_records = 1;  // record protocol (all-to-all, no master) for populations up to kRecordsMaxRows
   unsigned spin_limit = 4000000u;
   int dominance_tile_words = 4;
 };
@@ -30,7 +33,7 @@ struct Layout {
   int64_t wstride;
   // byte offsets
   size_t ctrl, fsize, fronts_slot, fronts_orig, hist, zero_end, fstart, xs, key, partials, sortparam, bstart, bcursor,
-      scanflags, members, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
+      scanflags, records, members, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
 };
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
@@ -56,6 +59,7 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->fronts_orig = o; o = align_up(o + sizeof(uint64_t) * kFrontBuffers * kFrontStride * (size_t)L->nwords);
   L->hist = o;        o = align_up(o + sizeof(int) * (size_t)buckets);
   L->scanflags = o;   o = align_up(o + sizeof(unsigned long long) * 64);
+  L->records = o;     o = align_up(o + (n <= kRecordsMaxRows ? sizeof(unsigned long long) * kRecRing * kRecUnits : 0));
   L->zero_end = o;
   L->fstart = o;     o = align_up(o + sizeof(int) * (size_t)(n + 2));
   L->xs = o;         o = align_up(o + sizeof(float) * (size_t)m * L->npad);
@@ -300,6 +304,26 @@ static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream
     if (err) return err;
   }
   if (blocks <= kFirstSweeper) return kErrBadArg;
+  if (use_witness && g_opt.peel_records && L.n <= kRecordsMaxRows) {
+    // all-to-all records: 1 lister + a power of two of sweeping blocks, all resident at once
+    const int sweepers = cus >= 64 ? g_opt.peel_record_blocks : 16;
+    const int wpb = kRecThreads / 64;
+    const int list_capacity = wpb * ((L.n + sweepers * wpb - 1) / (sweepers * wpb));
+    const size_t rec_lds = bitmap + 24 * (size_t)list_capacity;  // queue (8 + 4 + 4) and ranked pairs (2 x 4) per row
+    // every block waits for every other one: all of them must be resident at once
+    int rec_per_cu = 0;
+    const hipError_t oe = hipOccupancyMaxActiveBlocksPerMultiprocessor(&rec_per_cu, peel_records_kernel, kRecThreads, rec_lds);
+    if (oe != hipSuccess) return (int)oe;
+    if ((int64_t)rec_per_cu * cus >= sweepers + 1) {
+    hipLaunchKernelGGL(peel_records_kernel, dim3(sweepers + 1), dim3(kRecThreads), rec_lds, s, w.at<uint64_t>(L.dom), L.wstride,
+                       L.nwords, L.n, w.at<int>(L.orig_of), w.at<int>(L.rank), w.at<uint64_t>(L.fronts_slot),
+                       w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize), want_perm ? w.at<int>(L.perm) : (int*)nullptr,
+                       w.at<int>(L.fstart), w.ctrl(), (int)stop_count, g_opt.spin_limit, w.at<int>(L.witness),
+                       w.at<unsigned long long>(L.records), sweepers, list_capacity);
+    EVX_LAUNCH_CHECK();
+    return 0;
+    }  // otherwise: the master protocol below, whose grid is sized to what fits
+  }
   const size_t lds = bitmap * (use_witness ? 2 : 1);
   hipLaunchKernelGGL(peel_kernel, dim3(blocks), dim3(kPeelThreads), lds, s, w.at<uint64_t>(L.dom), L.wstride, L.nwords,
                      L.n, w.at<int>(L.orig_of), w.at<int>(L.count), w.at<int>(L.rank), w.at<uint64_t>(L.fronts_slot),
@@ -460,6 +484,10 @@ int evox_hip_set_option(const char* name, int64_t value) {
     g_opt.peel_blocks_per_cu = (int)value;
   } else if (!strcmp(name, "peel_witness") && (value == 0 || value == 1)) {
     g_opt.peel_witness = (int)value;
+  } else if (!strcmp(name, "peel_record_blocks") && value >= 16 && value <= 255) {
+    g_opt.peel_record_blocks = (int)value;
+  } else if (!strcmp(name, "peel_records") && (value == 0 || value == 1)) {
+    g_opt.peel_records = (int)value;
   } else if (!strcmp(name, "spin_limit") && value >= 1 && value <= 0x7FFFFFFFll) {
     g_opt.spin_limit = (unsigned)value;
   } else if (!strcmp(name, "dominance_tile_words") && (value == 4 || value == 8 || value == 16)) {

@@ -40,6 +40,10 @@ constexpr int kPeelThreads = 256;
 // serialise.
 constexpr int kFrontStride = 16;
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
+// global load of the wave, which a pass of the persistent kernels has no reason to wait for.
+__device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // Clears the control block, the front sizes, the front bitmaps and the sort histogram (one region).
 __global__ __launch_bounds__(256) void reset_state_kernel(uint32_t* __restrict__ words, int64_t n_words) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_words; i += (int64_t)gridDim.x * blockDim.x)
@@ -372,8 +376,33 @@ __device__ inline void witness_load(WitnessState& st, const PassCtx& c, const in
   }
 }
 
+// Rescan of up to four rows against the bitmap of unranked rows, all loads in flight together.
+// Entries from `cnt` on repeat entry 0 and are ignored.
+__device__ inline void scan_up_to_four(const uint64_t* const (&rows)[4], const int (&nws)[4], int cnt, const uint64_t* alive_lds,
+                                       RowScan (&r)[4]) {
+  const bool short_rows = nws[0] <= 512 && nws[1] <= 512 && nws[2] <= 512 && nws[3] <= 512;
+  if (cnt > 2 && short_rows) {
+    scan_rows<true, 4, 4>(rows, nws, alive_lds, r);
+  } else {
+    for (int q0 = 0; q0 < cnt; q0 += 2) {
+      const uint64_t* const two[2] = {rows[q0], rows[q0 + 1]};
+      const int nw2[2] = {nws[q0], nws[q0 + 1]};
+      RowScan r2[2];
+      if (short_rows)
+        scan_rows<true, 2, 4>(two, nw2, alive_lds, r2);
+      else
+        scan_rows<true, 2, 8>(two, nw2, alive_lds, r2);
+      r[q0] = r2[0];
+      r[q0 + 1] = r2[1];
+    }
+  }
+}
+
+// `on_ranked(slot, original index)` is called, by the lane that owns the row, for every row that enters the
+// front being built.
+template <class OnRanked>
 __device__ inline int witness_rows(WitnessState& st, const PassCtx& c, const uint64_t* alive_lds, int first_row,
-                                   int row_step) {
+                                   int row_step, OnRanked on_ranked) {
   const int lane = threadIdx.x & 63;
   int found = 0;
   int stat_rows = 0, stat_rounds = 0;
@@ -403,30 +432,14 @@ __device__ inline int witness_rows(WitnessState& st, const PassCtx& c, const uin
       stat_rows += cnt;
       ++stat_rounds;
       RowScan r[4];
-      const bool short_rows = nws[0] <= 512 && nws[1] <= 512 && nws[2] <= 512 && nws[3] <= 512;
-      if (cnt > 2 && short_rows) {
-        const uint64_t* const four[4] = {rows[0], rows[1], rows[2], rows[3]};
-        scan_rows<true, 4, 4>(four, nws, alive_lds, r);
-      } else {
-        for (int q0 = 0; q0 < cnt; q0 += 2) {
-          const uint64_t* const two[2] = {rows[q0], rows[q0 + 1]};
-          const int nw2[2] = {nws[q0], nws[q0 + 1]};
-          RowScan r2[2];
-          if (short_rows)
-            scan_rows<true, 2, 4>(two, nw2, alive_lds, r2);
-          else
-            scan_rows<true, 2, 8>(two, nw2, alive_lds, r2);
-          r[q0] = r2[0];
-          r[q0 + 1] = r2[1];
-        }
-      }
+      scan_up_to_four(rows, nws, cnt, alive_lds, r);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         if (q < cnt) {
           if (lane == l[q]) {
             st.word[ch] = r[q].last_word;
             st.bits[ch] = r[q].last_bits;
-            if (r[q].last_word < 0) publish_ranked(c, jrow[q], st.orig[ch]);
+            if (r[q].last_word < 0) on_ranked(jrow[q], st.orig[ch]);
           }
           found += r[q].last_word < 0;
         }
@@ -437,6 +450,65 @@ __device__ inline int witness_rows(WitnessState& st, const PassCtx& c, const uin
   (void)stat_rows;
   (void)stat_rounds;
   return found;
+}
+
+// The same pass with the rescans of a whole block pooled: the rows that lost their witness are queued
+// in LDS and dealt to the block's waves four at a time, so that a wave that owns five such rows does not
+// take two rounds while its neighbours idle (with 20 rows per wave that happens somewhere in almost
+// every pass, and everybody waits for the slowest wave).  q_row / q_word / q_bits hold one entry per
+// queued row; *q_n must be zero on entry.
+template <class OnRanked>
+__device__ inline void witness_rows_pooled(WitnessState& st, const PassCtx& c, const uint64_t* alive_lds, int first_row,
+                                           int row_step, int* q_n, int* q_row, int* q_word, uint64_t* q_bits, int q_capacity,
+                                           OnRanked on_ranked) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int waves = blockDim.x >> 6;
+  int mine[kWitnessChunks];
+#pragma unroll
+  for (int ch = 0; ch < kWitnessChunks; ++ch) {
+    const bool need = st.word[ch] >= 0 && (st.bits[ch] & alive_lds[st.word[ch] < 0 ? 0 : st.word[ch]]) == 0;
+    mine[ch] = -1;
+    if (need) {
+      const int idx = atomicAdd(q_n, 1);
+      if (idx < q_capacity) {
+        q_row[idx] = first_row + (ch * 64 + lane) * row_step;
+        mine[ch] = idx;
+      }
+    }
+  }
+  lds_barrier();
+  const int total = min(*q_n, q_capacity);
+  for (int base = wave * 4; base < total; base += waves * 4) {
+    const int cnt = min(4, total - base);
+    int jrow[4], nws[4];
+    const uint64_t* rows[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      jrow[q] = q_row[base + (q < cnt ? q : 0)];
+      rows[q] = c.dom + (int64_t)jrow[q] * c.wstride;
+      nws[q] = row_words(jrow[q]);
+    }
+    RowScan r[4];
+    const uint64_t* const four[4] = {rows[0], rows[1], rows[2], rows[3]};
+    scan_up_to_four(four, nws, cnt, alive_lds, r);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (q < cnt && lane == q) {
+        q_word[base + q] = r[q].last_word;
+        q_bits[base + q] = r[q].last_bits;
+      }
+    }
+  }
+  lds_barrier();
+#pragma unroll
+  for (int ch = 0; ch < kWitnessChunks; ++ch) {
+    if (mine[ch] >= 0) {
+      st.word[ch] = q_word[mine[ch]];
+      st.bits[ch] = q_bits[mine[ch]];
+      if (st.word[ch] < 0) on_ranked(first_row + (ch * 64 + lane) * row_step, st.orig[ch]);
+    }
+  }
 }
 
 // Block-wide listing of the set bits of `front` (nwords words, LDS) in ascending order into
@@ -624,7 +696,8 @@ __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __re
     }
     __syncthreads();
     EVX_TRACE(level, 1);
-    const int found = use_witness ? witness_rows(st, c, alive_lds, first_row, row_step)
+    const int found = use_witness ? witness_rows(st, c, alive_lds, first_row, row_step,
+                                                 [&](int slot, int orig) { publish_ranked(c, slot, orig); })
                                   : sweep_rows(c, front_lds, count, first_row, row_step);
     EVX_TRACE(level, 2);
     // every lane of a wave holds that wave's tally
@@ -636,6 +709,282 @@ __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __re
     ranked += size;
     ++level;
     if (!sweeper_barrier(ctrl, (unsigned)level, tally, &size, spin_limit, scratch + 64)) break;
+  }
+}
+
+// ------------------------------------------- persistent peel, record protocol
+
+// A pass of peel_kernel is a chain of dependent device-coherent exchanges (front bitmap load, rescan,
+// publish, arrive -> master, release -> sweepers).  This kernel removes three of them for populations
+// of moderate size: every sweeping block announces the rows it has just ranked in a RECORD of its own,
+// and every block reads the records of all blocks.  A record is a row of 8-byte units, each written and
+// read with one relaxed atomic access and each carrying the low 16 bits of the pass number in its top
+// bits, so a unit says by itself whether it belongs to the pass awaited: unit 0 holds the number of rows
+// and two slots, the others three slots each (16-bit slots, kRecNil for none), and a writer always
+// writes all its units.  Seeing every unit of a generation is therefore both the grid barrier and the
+// exchange of the new front, in one hop, with no master.  The units of one generation are few (8 KB):
+// a block that polls more than that per round waits on its own uncached loads.  A block that ranks more
+// rows than fit its record publishes them through the front bitmaps (as peel_kernel does), waits for
+// those atomics and flags the overflow in unit 0; in such a pass the readers also load the bitmap.
+// Records live in a ring of kRecRing generations; the lister (block 0) follows at its own pace, builds
+// each front in original-index space from the records, lists it into perm and recycles bitmaps;
+// `listed` keeps the sweepers from lapping it.  All waits are bounded.
+constexpr int kRecThreads = 512;
+constexpr int kRecUnits = 1024;  // units of one generation = sweepers x units per record
+constexpr int kRecRing = 8;      // == kFrontBuffers: a generation's record slot and bitmap buffer recycle together
+constexpr int kRecLoads = kRecUnits / kRecThreads;
+constexpr uint32_t kRecNil = 0xFFFFu;       // no slot (populations have fewer than 65535 rows)
+constexpr uint32_t kRecOverflow = 0x8000u;  // in the count field: the rows are in the bitmaps, not in the record
+static_assert(kRecRing == kFrontBuffers, "records and bitmaps are recycled by the same counter");
+
+__device__ inline unsigned long long record_unit(unsigned gen, uint32_t a, uint32_t b, uint32_t c) {
+  return ((unsigned long long)(gen & 0xFFFFu) << 48) | ((unsigned long long)(a & 0xFFFFu) << 32) | ((b & 0xFFFFu) << 16) | (c & 0xFFFFu);
+}
+// Slots that a record of `units` units can carry.
+__device__ inline int record_capacity(int units) { return 2 + 3 * (units - 1); }
+// The unit that thread i (< units) of the writer stores: list = (slot, original index) pairs, cnt of them.
+__device__ inline unsigned long long record_unit_for(unsigned gen, int i, const int* list, int cnt, bool overflow) {
+  auto slot_at = [&](int k) { return (!overflow && k < cnt) ? (uint32_t)list[2 * k] : kRecNil; };
+  if (i == 0) return record_unit(gen, overflow ? (kRecOverflow | (uint32_t)cnt) : (uint32_t)cnt, slot_at(0), slot_at(1));
+  return record_unit(gen, slot_at(3 * i - 1), slot_at(3 * i), slot_at(3 * i + 1));
+}
+// Calls on_count(count, overflow) for a unit 0 and on_slot(slot) for every slot a unit carries.
+template <class OnCount, class OnSlot>
+__device__ inline void record_unit_read(unsigned long long v, bool is_first, OnCount on_count, OnSlot on_slot) {
+  const uint32_t a = (uint32_t)(v >> 32) & 0xFFFFu, b = (uint32_t)(v >> 16) & 0xFFFFu, c = (uint32_t)v & 0xFFFFu;
+  if (is_first)
+    on_count((int)(a & ~kRecOverflow), (a & kRecOverflow) != 0u);
+  else if (a != kRecNil)
+    on_slot((int)a);
+  if (b != kRecNil) on_slot((int)b);
+  if (c != kRecNil) on_slot((int)c);
+}
+
+// Waits until the kRecLoads units of generation `gen` that this thread reads are all present (and, for
+// the thread that is given a counter, until *listed >= listed_needed).  False after a timeout or when
+// another block has given up.  Only what is still missing is loaded again: a block's uncached loads are
+// served one after the other, so every extra polling load delays the one that matters (two rounds in
+// flight at once, or records four times this size, each cost more than a microsecond per pass).
+__device__ inline bool poll_record_units(const unsigned long long* gen_units, unsigned gen, unsigned long long (&v)[kRecLoads],
+                                         const int* listed, int listed_needed, const int* err, unsigned spin_limit) {
+  const unsigned long long* mine = gen_units + threadIdx.x;
+  unsigned pending = (1u << kRecLoads) - 1u;
+  bool waiting_listed = listed != nullptr;
+  for (unsigned spins = 0;; ++spins) {
+    int seen_listed = 0;
+#pragma unroll
+    for (int k = 0; k < kRecLoads; ++k)
+      if (pending & (1u << k)) v[k] = coherent_load(&mine[k * kRecThreads]);
+    if (waiting_listed) seen_listed = coherent_load(listed);
+#pragma unroll
+    for (int k = 0; k < kRecLoads; ++k)
+      if ((pending & (1u << k)) && (unsigned)(v[k] >> 48) == (gen & 0xFFFFu)) pending &= ~(1u << k);
+    if (waiting_listed && seen_listed >= listed_needed) waiting_listed = false;
+    if (pending == 0u && !waiting_listed) return true;
+    if (spins > spin_limit) return false;
+    if ((spins & 63u) == 63u && coherent_load(err) != 0) return false;
+  }
+}
+
+__global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
+    const uint64_t* __restrict__ dom, int64_t wstride, int nwords, int n, const int* __restrict__ orig_of,
+    int* __restrict__ rank, uint64_t* __restrict__ fronts_slot, uint64_t* __restrict__ fronts_orig, int* __restrict__ fsize,
+    int* __restrict__ perm, int* __restrict__ fstart, Ctrl* __restrict__ ctrl, int stop_count, unsigned spin_limit,
+    const int* __restrict__ witness, unsigned long long* __restrict__ records, int sweepers, int list_capacity) {
+  extern __shared__ uint64_t rec_lds[];  // nwords words: unranked rows (sweepers) / the front being listed (lister);
+                                         // then, per row a block can own (list_capacity): the rescan queue
+                                         // (result bits, row, result word) and the (slot, original index) pairs
+                                         // of the rows just ranked
+  __shared__ int sh[32];
+  if (coherent_load(&ctrl->err) != 0) return;
+  int units = 1;  // per record: the largest power of two that gives every sweeper a record
+  while (units * 2 * sweepers <= kRecUnits) units *= 2;
+  const int tid = threadIdx.x;
+
+  if (blockIdx.x == 0) {
+    // ---- lister
+    uint64_t* front_lds = rec_lds;
+    int ranked = 0;
+    for (int level = 0;; ++level) {
+      int size = 0;
+      if (level == 0) {
+        const uint64_t* cur = fronts_orig;  // buffer 0, filled by count_kernel
+        int mine = 0;
+        for (int w = tid; w < nwords; w += blockDim.x) {
+          const uint64_t fw = coherent_load(&cur[(int64_t)w * kFrontStride]);
+          front_lds[w] = fw;
+          mine += __popcll(fw);
+        }
+        if (tid == 0) sh[1] = 0;
+        __syncthreads();
+        if (mine) atomicAdd(&sh[1], mine);
+        __syncthreads();
+        size = sh[1];
+      } else {
+        for (int w = tid; w < nwords; w += blockDim.x) front_lds[w] = 0ull;
+        if (tid == 0) {
+          sh[1] = 0;
+          sh[2] = 0;
+        }
+        __syncthreads();
+        unsigned long long v[kRecLoads];
+        const unsigned gen = (unsigned)level;
+        if (!poll_record_units(records + (size_t)(gen % kRecRing) * kRecUnits, gen, v, nullptr, 0, &ctrl->err, spin_limit)) {
+          coherent_store(&ctrl->err, kErrBarrierTimeout);
+          atomicOr(&sh[2], 2);
+        } else {
+#pragma unroll
+          for (int k = 0; k < kRecLoads; ++k) {
+            const int i = (tid + k * kRecThreads) & (units - 1);
+            record_unit_read(
+                v[k], i == 0,
+                [&](int count, bool overflow) {
+                  atomicAdd(&sh[1], count);
+                  if (overflow) atomicOr(&sh[2], 1);
+                },
+                [&](int slot) {
+                  const int o = orig_of[slot];
+                  atomicOr(reinterpret_cast<unsigned long long*>(&front_lds[o >> 6]), 1ull << (o & 63));
+                });
+          }
+        }
+        __syncthreads();
+        if (sh[2] & 2) return;
+        size = sh[1];
+        if (sh[2] & 1) {
+          const uint64_t* cur = fronts_orig + (int64_t)(level % kFrontBuffers) * nwords * kFrontStride;
+          for (int w = tid; w < nwords; w += blockDim.x) front_lds[w] |= coherent_load(&cur[(int64_t)w * kFrontStride]);
+        }
+        // every sweeper has published generation `level`, so it has finished with the bitmaps of front level-1
+        uint64_t* prev_slot = fronts_slot + (int64_t)((level - 1) % kFrontBuffers) * nwords * kFrontStride;
+        uint64_t* prev_orig = fronts_orig + (int64_t)((level - 1) % kFrontBuffers) * nwords * kFrontStride;
+        for (int w = tid; w < nwords; w += blockDim.x) {
+          coherent_store(&prev_slot[(int64_t)w * kFrontStride], (uint64_t)0);
+          coherent_store(&prev_orig[(int64_t)w * kFrontStride], (uint64_t)0);
+        }
+      }
+      __syncthreads();  // also waits for the clearing stores of this block's waves
+      if (tid == 0) coherent_store(&ctrl->listed, level);  // records <= level consumed, bitmaps < level cleared
+      if (perm) list_front(front_lds, nwords, perm, ranked, sh + 8);
+      const bool last = size <= 0 || ranked + size >= stop_count;
+      if (tid == 0) {
+        fstart[level] = ranked;
+        if (level > 0) fsize[level] = size;
+        if (last) {
+          fstart[level + 1] = ranked + size;
+          ctrl->nfronts = level + 1;
+          ctrl->worst = level;
+          ctrl->worst_start = ranked;
+          ctrl->nv = size;
+          ctrl->need = stop_count - ranked;
+          ctrl->passes = level;
+        }
+      }
+      if (last) return;
+      ranked += size;
+      __syncthreads();
+    }
+  }
+
+  // ---- sweepers
+  uint64_t* alive_lds = rec_lds;
+  uint64_t* q_bits = rec_lds + nwords;
+  int* found = reinterpret_cast<int*>(q_bits + list_capacity);
+  int* q_row = found + 2 * list_capacity;
+  int* q_word = q_row + list_capacity;
+  const int waves_per_block = blockDim.x >> 6;
+  const int sb = (int)blockIdx.x - 1;
+  const int row_step = sweepers * waves_per_block;
+  const int first_row = sb * waves_per_block + (tid >> 6);
+  PassCtx c;
+  c.dom = dom;
+  c.wstride = wstride;
+  c.n = n;
+  c.orig_of = orig_of;
+  c.rank = rank;
+  int size = coherent_load(&fsize[0]);  // size of front `level`
+  if (size <= 0 || size >= stop_count) return;  // front 0 already holds every row asked for: no pass
+  WitnessState st;
+  witness_load(st, c, witness, first_row, row_step);
+  for (int w = tid; w < nwords; w += blockDim.x) {
+    const int lo = w * 64;
+    const uint64_t all = lo + 64 <= n ? ~0ull : (lo >= n ? 0ull : ((1ull << (n - lo)) - 1ull));
+    alive_lds[w] = all & ~coherent_load(&fronts_slot[(int64_t)w * kFrontStride]);  // minus front 0 (buffer 0)
+  }
+  __syncthreads();
+  int level = 0;
+  int ranked = 0;  // rows in fronts 0 .. level-1
+  for (;;) {
+    if (size <= 0 || ranked + size >= stop_count) break;
+    ranked += size;
+    ++level;  // this pass builds front `level`
+    const unsigned gen = (unsigned)level;
+    c.next_slot = fronts_slot + (int64_t)(level % kFrontBuffers) * nwords * kFrontStride;
+    c.next_orig = fronts_orig + (int64_t)(level % kFrontBuffers) * nwords * kFrontStride;
+    c.next_level = level;
+    if (tid == 0) {
+      sh[0] = 0;  // rows this block ranks in the pass
+      sh[1] = 0;  // rows all blocks rank
+      sh[2] = 0;  // bit 0: some block overflowed its record, bit 1: give up
+      sh[3] = 0;  // rows queued for a rescan
+    }
+    lds_barrier();
+    EVX_TRACE(level - 1, 0);
+    witness_rows_pooled(st, c, alive_lds, first_row, row_step, &sh[3], q_row, q_word, q_bits, list_capacity, [&](int slot, int orig) {
+      rank[orig] = level;
+      const int k = atomicAdd(&sh[0], 1);
+      if (k < list_capacity) {
+        found[2 * k] = slot;
+        found[2 * k + 1] = orig;
+      }
+    });
+    lds_barrier();  // the list of ranked rows is complete (the rank stores need not be)
+    EVX_TRACE(level - 1, 1);
+    const int cnt = sh[0];
+    unsigned long long* mine = records + (size_t)(gen % kRecRing) * kRecUnits + (size_t)sb * units;
+    if (cnt <= record_capacity(units)) {
+      if (tid < units) coherent_store(&mine[tid], record_unit_for(gen, tid, found, cnt, false));
+    } else {
+      for (int e = tid; e < cnt; e += blockDim.x) {
+        const int slot = found[2 * e], orig = found[2 * e + 1];
+        atomicOr(reinterpret_cast<unsigned long long*>(c.next_slot + (int64_t)(slot >> 6) * kFrontStride), 1ull << (slot & 63));
+        atomicOr(reinterpret_cast<unsigned long long*>(c.next_orig + (int64_t)(orig >> 6) * kFrontStride), 1ull << (orig & 63));
+      }
+      __syncthreads();  // every wave has waited for its own atomics
+      if (tid < units) coherent_store(&mine[tid], record_unit_for(gen, tid, found, cnt, true));
+    }
+    // the records of everybody: barrier and front exchange in one.  Thread 0 also makes sure that the
+    // lister has recycled what generation level + 1 will overwrite.
+    EVX_TRACE(level - 1, 2);
+    unsigned long long v[kRecLoads];
+    const bool fine = poll_record_units(records + (size_t)(gen % kRecRing) * kRecUnits, gen, v, tid == 0 ? &ctrl->listed : nullptr,
+                                        level + 2 - kRecRing, &ctrl->err, spin_limit);
+    EVX_TRACE(level - 1, 3);
+    if (!fine) {
+      coherent_store(&ctrl->err, kErrBarrierTimeout);
+      atomicOr(&sh[2], 2);
+    } else {
+#pragma unroll
+      for (int k = 0; k < kRecLoads; ++k) {
+        const int i = (tid + k * kRecThreads) & (units - 1);
+        record_unit_read(
+            v[k], i == 0,
+            [&](int count, bool overflow) {
+              atomicAdd(&sh[1], count);
+              if (overflow) atomicOr(&sh[2], 1);
+            },
+            [&](int slot) { atomicAnd(reinterpret_cast<unsigned long long*>(&alive_lds[slot >> 6]), ~(1ull << (slot & 63))); });
+      }
+    }
+    lds_barrier();
+    const int flags = sh[2];
+    size = sh[1];
+    if (flags & 2) break;
+    if (flags & 1) {
+      const uint64_t* cur = c.next_slot;
+      for (int w = tid; w < nwords; w += blockDim.x) alive_lds[w] &= ~coherent_load(&cur[(int64_t)w * kFrontStride]);
+    }
+    lds_barrier();  // sh is reset at the top of the next pass
   }
 }
 

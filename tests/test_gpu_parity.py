@@ -178,12 +178,15 @@ def test_rank_strided_and_half_inputs():
     assert np.array_equal(as_np(non_dominate_rank(h.to(DEV))), as_np(er.ranks_by_peeling(h.float())))
 
 
-@pytest.fixture(params=["witness", "sweep"])
+@pytest.fixture(params=["witness-records", "witness-master", "sweep"])
 def peel_algorithm(request):
-    """Both peeling passes: the witness pass (default) and the popcount-decrement sweep."""
-    runtime.set_option("peel_witness", 1 if request.param == "witness" else 0)
+    """The peeling variants: witness pass with the record protocol (default), witness pass with the
+    master barrier and front bitmaps, and the popcount-decrement sweep (master barrier)."""
+    runtime.set_option("peel_witness", 0 if request.param == "sweep" else 1)
+    runtime.set_option("peel_records", 1 if request.param == "witness-records" else 0)
     yield request.param
     runtime.set_option("peel_witness", 1)
+    runtime.set_option("peel_records", 1)
 
 
 @pytest.mark.parametrize("name", ["C1", "C2", "C2p", "C3"])
