@@ -106,6 +106,19 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
     for (int t = 31; t >= 0; --t) {
       const int i = ib + t;
       uint64_t c = ~0ull;
+      if (VARIANT == kDomKey32) {
+        // all compares first, then a tree of ANDs: independent instructions for the scheduler
+        uint64_t mk[M + 1];
+#pragma unroll
+        for (int k = 0; k < M; ++k) mk[k] = __builtin_amdgcn_ballot_w64(xs[(int64_t)k * npad + i] <= xj[k]);
+        mk[M] = __builtin_amdgcn_ballot_w64(kid[i] != idj);
+#pragma unroll
+        for (int span = 1; span <= M; span *= 2)
+#pragma unroll
+          for (int k = 0; k + span <= M; k += 2 * span) mk[k] &= mk[k + span];
+        acc = shift_in(acc, mk[0]);
+        continue;
+      }
 #pragma unroll
       for (int k = 0; k < M; ++k) c &= __builtin_amdgcn_ballot_w64(xs[(int64_t)k * npad + i] <= xj[k]);
       if (VARIANT == kDomKey64) {
