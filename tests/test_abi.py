@@ -42,7 +42,7 @@ def test_workspace_size_and_layout(handle):
     assert handle.evox_hip_workspace_bytes(10, 0) == 0
     b = handle.evox_hip_workspace_bytes(20000, 3)
     # dominated by the bit matrix: 20000 rows x 320 words (313 rounded up to a 128-byte multiple)
-    assert 20000 * 320 * 8 <= b <= 20000 * 320 * 8 + 6 * 2**20
+    assert 20000 * 320 * 8 <= b <= 20000 * 320 * 8 + 8 * 2**20
     b5 = handle.evox_hip_workspace_bytes(200000, 8)
     assert 5.0e9 < b5 < 5.3e9
     # the first-front entry builds no matrix: a few arrays of n entries
