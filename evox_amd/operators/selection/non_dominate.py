@@ -18,7 +18,9 @@ def non_dominate_rank(x: torch.Tensor) -> torch.Tensor:
     Same contract as the reference's ``non_dominate_rank`` (non_dominate.py:172-195):
     ``x`` is ``(N, M)``; the result is ``int32 (N,)`` on ``x.device``; rank 0 is the Pareto front,
     rank r + 1 the front of what remains after removing ranks 0..r.  Rows holding a NaN neither
-    dominate nor are dominated (rank 0); identical rows do not dominate each other.
+    dominate nor are dominated (rank 0); identical rows do not dominate each other.  Any real dtype is
+    accepted, as in the reference: float32 (and float16 / bfloat16, widened exactly) goes to the kernels
+    as it is, other dtypes through per-objective dense ranks, which keep every comparison.
     """
     return ops.nd_rank(x)
 
@@ -60,6 +62,11 @@ def nd_environmental_selection(x: torch.Tensor, f: torch.Tensor, topk: int) -> T
     then by row index; the distance of rows in better fronts is ``-inf``.  ``topk > N`` raises
     ``RuntimeError`` and ``topk < 1`` raises ``IndexError`` as ``torch.topk`` / indexing do there.
     """
+    if f.is_floating_point() and f.dtype not in (torch.float16, torch.bfloat16) and f.dtype != torch.get_default_dtype():
+        # the reference fails in the scatter of its crowding distance (non_dominate.py:224-225)
+        raise RuntimeError(
+            f"nd_environmental_selection: expected f.dtype to be the default dtype {torch.get_default_dtype()}, got {f.dtype}"
+        )
     return ops.nd_select(x, f, int(topk))
 
 

@@ -24,6 +24,33 @@ def _as_f32(t: torch.Tensor, what: str) -> torch.Tensor:
     raise TypeError(f"{what} must be float32 (float16 / bfloat16 are widened exactly); got {t.dtype}")
 
 
+def _order_preserving_f32(t: torch.Tensor, what: str) -> torch.Tensor:
+    """A float32 tensor with the same `<=` / `<` relations inside every objective (column) as ``t``.
+
+    Dominance only looks at the order of the values within one objective, so fitness of a dtype that
+    the kernels do not read (float64, integers) is replaced, objective by objective, by the dense rank
+    of each value among the values of that objective (``torch.unique`` on the device: equal values get
+    equal ranks, -0.0 and 0.0 tie, NaN stays NaN).  Dense ranks below 2**24 are exact in float32.
+    Used for ranking only: crowding distances depend on the values themselves.
+    """
+    if t.dtype in (torch.float32, torch.float16, torch.bfloat16):
+        return _as_f32(t, what)
+    if t.is_complex() or t.dtype == torch.bool:
+        raise TypeError(f"{what} must be a real numeric tensor; got {t.dtype}")
+    if t.shape[-2] >= 2**24:
+        raise ValueError(f"{what} of dtype {t.dtype} is limited to 2**24 rows per population")
+    flat = t.reshape(-1, t.shape[-2], t.shape[-1])
+    out = torch.empty(flat.shape, dtype=torch.float32, device=t.device)
+    for b in range(flat.size(0)):
+        for k in range(flat.size(2)):
+            col = flat[b, :, k]
+            dense = torch.unique(col, sorted=True, return_inverse=True)[1].to(torch.float32)
+            if col.is_floating_point():
+                dense = torch.where(torch.isnan(col), torch.full_like(dense, float("nan")), dense)
+            out[b, :, k] = dense
+    return out.reshape(t.shape)
+
+
 def _rank_one(f: torch.Tensor, out: torch.Tensor) -> None:
     n, m = f.shape
     ws = runtime.workspace(n, m, f.device)
@@ -39,7 +66,7 @@ def nd_rank(f: torch.Tensor) -> torch.Tensor:
     runtime.require_gpu_tensor(f, "fitness")
     if f.dim() < 2:
         raise ValueError("fitness must have shape (..., N, M)")
-    f32 = _as_f32(f, "fitness")
+    f32 = _order_preserving_f32(f, "fitness") if f.shape[-2] > 0 and f.shape[-1] > 0 else f.float()
     n, m = f32.shape[-2:]
     out = torch.empty(f32.shape[:-1], dtype=torch.int32, device=f.device)
     if n == 0 or out.numel() == 0:
@@ -77,7 +104,7 @@ def nd_first_front(f: torch.Tensor) -> torch.Tensor:
     runtime.require_gpu_tensor(f, "fitness")
     if f.dim() < 2:
         raise ValueError("fitness must have shape (..., N, M)")
-    f32 = _as_f32(f, "fitness")
+    f32 = _order_preserving_f32(f, "fitness") if f.shape[-2] > 0 and f.shape[-1] > 0 else f.float()
     n, m = f32.shape[-2:]
     out = torch.empty(f32.shape[:-1], dtype=torch.bool, device=f.device)
     if n == 0 or out.numel() == 0:

@@ -384,6 +384,40 @@ def test_selection_x_dtypes_and_shapes():
         assert xs.dtype == x.dtype and np.array_equal(as_np(xs), as_np(x)[order])
 
 
+@pytest.mark.parametrize("name,f,ks", EDGE, ids=IDS)
+def test_rank_of_other_dtypes_edge(name, f, ks):
+    """float64 and integer fitness is ranked through per-objective dense ranks, which keep every
+    `<=` and `<` of the original values (the reference ranks any dtype, non_dominate.py:172-195)."""
+    from evox_amd.operators.selection import non_dominated_mask
+
+    say("rank_f64", name)
+    want = as_np(er.ranks_by_peeling(f.double()))
+    assert np.array_equal(want, as_np(er.ranks_by_peeling(f)))  # widening float32 keeps the order
+    assert np.array_equal(as_np(non_dominate_rank(f.double().to(DEV))), want)
+    assert np.array_equal(as_np(non_dominated_mask(f.double().to(DEV))), want == 0)
+
+
+def test_rank_of_other_dtypes_values_beyond_float32():
+    say("rank_dtypes")
+    g = torch.Generator("cpu").manual_seed(77)
+    # float64 values that collapse when rounded to float32, and 64-bit integers beyond 2**24
+    f64 = 1.0 + torch.randint(0, 50, (700, 3), generator=g).double() * 1e-12
+    f64[5, 1] = float("nan")
+    f64[6] = f64[7]
+    f64[8, 0], f64[9, 0] = 0.0, -0.0
+    i64 = (2**40 + torch.randint(0, 40, (500, 2), generator=g)).long()
+    i32 = torch.randint(-5, 5, (400, 4), generator=g, dtype=torch.int32)
+    for t in (f64, i64, i32):
+        want = as_np(er.ranks_by_peeling(t))
+        assert want.max() > 3
+        assert np.array_equal(as_np(non_dominate_rank(t.to(DEV))), want), t.dtype
+    assert not np.array_equal(as_np(er.ranks_by_peeling(f64.float())), as_np(er.ranks_by_peeling(f64)))
+    stacked = torch.stack([f64, f64.flip(0)])
+    assert np.array_equal(as_np(non_dominate_rank(stacked.to(DEV))), np.stack([as_np(er.ranks_by_peeling(x)) for x in stacked]))
+    with pytest.raises(TypeError):
+        non_dominate_rank(torch.zeros(4, 2, dtype=torch.bool, device=DEV))
+
+
 def test_selection_errors():
     f = torch.rand(5, 2, device=DEV)
     with pytest.raises(RuntimeError):
