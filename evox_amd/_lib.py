@@ -22,6 +22,8 @@ _SIGNATURES = {
     "evox_hip_abi_version": (c_int, []),
     "evox_hip_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "evox_hip_non_dominate_rank": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "evox_hip_non_dominate_rank_until": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_size_t,
+                                                 c_void_p]),
     "evox_hip_first_front_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "evox_hip_first_front_mask": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "evox_hip_crowding_distance": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p,

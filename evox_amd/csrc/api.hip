@@ -544,17 +544,22 @@ int evox_hip_stage_order(int64_t n, int64_t m, void* ws, size_t ws_bytes, void* 
   return stage_order(w, (hipStream_t)stream);
 }
 
-int evox_hip_non_dominate_rank(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, int32_t* rank_out, void* ws,
-                               size_t ws_bytes, void* stream) {
+int evox_hip_non_dominate_rank_until(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, int64_t stop_count,
+                                     int32_t* rank_out, void* ws, size_t ws_bytes, void* stream) {
   Ws w;
-  if (rank_out == nullptr) return kErrBadArg;
+  if (rank_out == nullptr || stop_count < 1 || stop_count > n) return kErrBadArg;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   hipStream_t s = (hipStream_t)stream;
   if (int e = stage_prepare(w, one_part(f, n, sr, sc), true, s)) return e;
   if (int e = stage_dominance(w, kDomKey32, s)) return e;
   if (int e = stage_count(w, false, s)) return e;
-  if (int e = stage_peel(w, n, false, s)) return e;
+  if (int e = stage_peel(w, stop_count, false, s)) return e;
   return copy_async(rank_out, w.at<int>(w.L.rank), sizeof(int) * (size_t)n, s);
+}
+
+int evox_hip_non_dominate_rank(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, int32_t* rank_out, void* ws,
+                               size_t ws_bytes, void* stream) {
+  return evox_hip_non_dominate_rank_until(f, n, m, sr, sc, n, rank_out, ws, ws_bytes, stream);
 }
 
 size_t evox_hip_first_front_workspace_bytes(int64_t n, int64_t m) {

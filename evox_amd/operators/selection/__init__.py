@@ -3,6 +3,7 @@ __all__ = [
     "nd_environmental_selection",
     "nd_environmental_selection_two_part",
     "non_dominate_rank",
+    "non_dominate_rank_until",
     "non_dominated_mask",
     "tournament_selection_multifit",
 ]
@@ -12,6 +13,7 @@ from .non_dominate import (
     nd_environmental_selection,
     nd_environmental_selection_two_part,
     non_dominate_rank,
+    non_dominate_rank_until,
     non_dominated_mask,
 )
 from .tournament_selection import tournament_selection_multifit

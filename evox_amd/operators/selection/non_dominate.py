@@ -25,6 +25,19 @@ def non_dominate_rank(x: torch.Tensor) -> torch.Tensor:
     return ops.nd_rank(x)
 
 
+def non_dominate_rank_until(x: torch.Tensor, count: int) -> torch.Tensor:
+    """``non_dominate_rank(x)`` peeled only as far as the front that holds the ``count``-th best row.
+
+    Rows of that front and of the better ones get their rank; every other row gets ``2**31 - 1``.  Not a name
+    of the reference; it serves its callers that rank a merged population only to cut it at a front --
+    ``worst = torch.topk(rank, k, largest=False)[0][-1]; keep = rank <= worst`` in NSGA-III
+    (src/evox/algorithms/mo/nsga3.py:169-171) and the argsort form of the same in HypE
+    (src/evox/algorithms/mo/hype.py:135-138) -- which read the same ``worst`` and ``keep`` from the
+    truncated ranks without the fronts behind the cut ever being peeled.
+    """
+    return ops.nd_rank_until(x, int(count))
+
+
 def non_dominated_mask(x: torch.Tensor) -> torch.Tensor:
     """``non_dominate_rank(x) == 0`` without ranking anything else: bool ``(N,)`` on ``x.device``.
 

@@ -98,6 +98,52 @@ def _nd_rank_vmap(info, in_dims, f):
 torch.library.register_vmap(nd_rank, _nd_rank_vmap)
 
 
+RANK_UNSET = 0x7FFFFFFF
+
+
+@torch.library.custom_op("evox_amd::nd_rank_until", mutates_args=())
+def nd_rank_until(f: torch.Tensor, count: int) -> torch.Tensor:
+    """(..., N, M) fitness -> (..., N) int32 rank, peeled only as far as the front that holds the
+    count-th best row; rows of later fronts get RANK_UNSET."""
+    runtime.require_gpu_tensor(f, "fitness")
+    if f.dim() < 2:
+        raise ValueError("fitness must have shape (..., N, M)")
+    n, m = f.shape[-2:]
+    if count > n:
+        raise RuntimeError(f"selected index k out of range: count={count} exceeds the population size {n}")
+    if count < 1:
+        raise IndexError(f"count must be at least 1; got {count}")
+    if m == 0:
+        raise ValueError("fitness must have at least one objective")
+    f32 = _order_preserving_f32(f, "fitness")
+    out = torch.empty(f32.shape[:-1], dtype=torch.int32, device=f.device)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(f.device):
+        flat_f = f32.reshape(-1, n, m)
+        flat_out = out.view(-1, n)
+        ws = runtime.workspace(n, m, f.device)
+        stream = runtime.stream_handle(f.device)
+        for b in range(flat_f.size(0)):
+            fb = flat_f[b]
+            _lib.call("evox_hip_non_dominate_rank_until", fb.data_ptr(), n, m, fb.stride(0), fb.stride(1), count,
+                      flat_out[b].data_ptr(), ws.data_ptr(), ws.numel(), stream)
+        runtime.note_call(ws, stream)
+    return out
+
+
+@nd_rank_until.register_fake
+def _(f, count):
+    return f.new_empty(f.shape[:-1], dtype=torch.int32)
+
+
+def _nd_rank_until_vmap(info, in_dims, f, count):
+    return nd_rank_until(f.movedim(in_dims[0], 0), count), 0
+
+
+torch.library.register_vmap(nd_rank_until, _nd_rank_until_vmap)
+
+
 @torch.library.custom_op("evox_amd::nd_first_front", mutates_args=())
 def nd_first_front(f: torch.Tensor) -> torch.Tensor:
     """(..., N, M) fitness -> (..., N) bool, True for the rows that no row dominates (rank 0)."""

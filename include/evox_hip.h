@@ -41,6 +41,17 @@ size_t evox_hip_workspace_bytes(int64_t n, int64_t m);
 int evox_hip_non_dominate_rank(const float* f, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col,
                                int32_t* rank_out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same ranking, stopped after the front that holds the stop_count-th best row: rows of that front and of
+ * the better ones get their rank, all others EVOX_HIP_RANK_UNSET.  It serves the callers that rank a merged
+ * population only to cut it at a front, `worst = topk(rank, k, largest=False)[0][-1]; keep = rank <= worst`
+ * (src/evox/algorithms/mo/nsga3.py:169-171 with k = pop_size + 1, src/evox/algorithms/mo/hype.py:135-138 with
+ * k = pop_size): both statements give the same result on the truncated ranks, and the fronts behind the cut are
+ * never peeled (C3 shape: 24 of 61 fronts). */
+#define EVOX_HIP_RANK_UNSET 0x7FFFFFFF
+int evox_hip_non_dominate_rank_until(const float* f, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col,
+                                     int64_t stop_count, int32_t* rank_out, void* workspace, size_t workspace_bytes,
+                                     void* stream);
+
 /* mask_out[j] (one byte per row, n entries) = 1 when no row dominates row j, else 0: the rows of rank 0,
  * without building the dominance matrix or peeling.  Replaces the pair
  * `rank = non_dominate_rank(all_fitness); ... [rank == 0]` of EvalMonitor.get_pf_fitness / get_pf

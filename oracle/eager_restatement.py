@@ -16,6 +16,7 @@ the reference's multi-objective environmental selection, on torch CPU tensors:
   tournament_winners        <- src/evox/operators/selection/tournament_selection.py:18-27
   first_front_mask          <- src/evox/workflows/eval_monitor.py:301-302 (= :333-334)
   merged_selection          <- src/evox/algorithms/mo/nsga2.py:99-102
+  front_cut                 <- src/evox/algorithms/mo/nsga3.py:169-171 (hype.py:135-138 is the argsort form)
 
 How each function is pinned (tests/test_oracle.py):
   * dominance / ranks: tiny-input brute force, longest-dominator-chain definition, Deb's fast
@@ -152,3 +153,11 @@ def first_front_mask(f: torch.Tensor) -> torch.Tensor:
 def merged_selection(x_a, f_a, x_b, f_b, topk: int, return_all: bool = False):
     """The merge step of NSGA-II, nsga2.py:99-102: concatenate parents and offspring, then select."""
     return environmental_selection(torch.cat([x_a, x_b], dim=0), torch.cat([f_a, f_b], dim=0), topk, return_all)
+
+
+def front_cut(f: torch.Tensor, count: int):
+    """(worst_rank, keep mask, rank) of nsga3.py:169-171: rank everything, find the rank of the count-th
+    best row, keep the rows up to that front."""
+    rank = ranks_by_peeling(f)
+    worst = torch.topk(rank, count, largest=False)[0][-1]
+    return worst, rank <= worst, rank

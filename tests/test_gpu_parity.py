@@ -525,6 +525,47 @@ def test_barrier_timeout_is_reported_not_hung():
     assert np.array_equal(as_np(non_dominate_rank(f)), as_np(er.ranks_by_peeling(f.cpu())))
 
 
+# ------------------------------------------------------------------ ranks up to the cut front only
+
+
+@pytest.mark.parametrize("name,f,ks", EDGE, ids=IDS)
+def test_rank_until_edge(name, f, ks, peel_algorithm):
+    from evox_amd.operators.selection import non_dominate_rank_until
+
+    for k in sorted(set(ks) | {1, f.size(0)}):
+        say("rank_until", name, k, peel_algorithm)
+        worst, keep, rank = er.front_cut(f, k)
+        got = non_dominate_rank_until(f.to(DEV), k).cpu()
+        # the caller's own statements on the truncated ranks (nsga3.py:170-171)
+        assert torch.equal(torch.topk(got, k, largest=False)[0][-1], worst)
+        assert torch.equal(got <= worst, keep)
+        assert torch.equal(got[keep], rank[keep]) and bool((got[~keep] == 2**31 - 1).all())
+
+
+def test_rank_until_c3_and_batch(peel_algorithm):
+    from evox_amd.operators.selection import non_dominate_rank_until
+
+    say("rank_until_c3", peel_algorithm)
+    w, gold = golden_io.config("C3")
+    rank = torch.from_numpy(gold["rank"])
+    for k in (1, 31, 10001, 20000):
+        worst = torch.topk(rank, k, largest=False)[0][-1]
+        got = non_dominate_rank_until(w.f.to(DEV), k).cpu()
+        assert torch.equal(got <= worst, rank <= worst) and torch.equal(got[rank <= worst], rank[rank <= worst])
+        assert bool((got[rank > worst] == 2**31 - 1).all())
+        assert runtime.last_status()["fronts"] == int(worst) + 1
+    fb = torch.stack([workloads.uniform_population(500, 3, 0, 90 + b)[0] for b in range(3)])
+    got = non_dominate_rank_until(fb.to(DEV), 100).cpu()
+    for b in range(3):
+        worst, keep, r = er.front_cut(fb[b], 100)
+        assert torch.equal(got[b] <= worst, keep) and torch.equal(got[b][keep], r[keep])
+    assert torch.equal(torch.vmap(lambda t: non_dominate_rank_until(t, 100))(fb.to(DEV)).cpu(), got)
+    with pytest.raises(RuntimeError):
+        non_dominate_rank_until(fb[0].to(DEV), 501)
+    with pytest.raises(IndexError):
+        non_dominate_rank_until(fb[0].to(DEV), 0)
+
+
 # ------------------------------------------------------------------ first front only (rank == 0)
 
 
