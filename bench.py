@@ -148,7 +148,9 @@ def next_rows(dev, reps):
     """Times of the entry points either side of the hot path, on inputs resident in HBM."""
     from evox_amd import workloads
     from evox_amd.operators.selection import (nd_environmental_selection, nd_environmental_selection_two_part,
-                                              non_dominate_rank, non_dominated_mask, tournament_selection_multifit)
+                                              non_dominate_rank, non_dominate_rank_until, non_dominated_mask,
+                                              tournament_selection_multifit)
+    from evox_amd.utils import lexsort
 
     out = {}
     # first front of a long evaluation history (what the monitor asks for) against ranking all of it
@@ -173,6 +175,17 @@ def next_rows(dev, reps):
         "cat_then_select_us": event_time_us(
             lambda: nd_environmental_selection(torch.cat([xa, xb]), torch.cat([fa, fb]), w.topk), reps),
     }
+    # the cut that NSGA-III / HypE make: ranks only up to the front of the (topk+1)-th row, against all ranks
+    non_dominate_rank_until(f, w.topk + 1)
+    out["rank_until C3"] = {
+        "rank_until_us": event_time_us(lambda: non_dominate_rank_until(f, w.topk + 1), reps),
+        "full_rank_us": event_time_us(lambda: non_dominate_rank(f), reps),
+    }
+    # lexsort as a function of its own: HypE's lexsort([-dis, rank]) over the merged population
+    full_rank = non_dominate_rank(f)
+    key = torch.rand(f.size(0), device=dev)
+    lexsort([key, full_rank])
+    out["lexsort 2 keys x 20000"] = {"us": event_time_us(lambda: lexsort([key, full_rank]), reps)}
     # mating selection on the survivors' rank and distance (10000 binary tournaments)
     _, _, rank, dist = nd_environmental_selection(x, f, w.topk)
     tournament_selection_multifit(w.topk, [-dist, rank])

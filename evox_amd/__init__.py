@@ -3,10 +3,11 @@
     from evox_amd.operators.selection import non_dominate_rank, crowding_distance, nd_environmental_selection
 
 The package holds only this hot path: HIP kernels for gfx950 behind a C ABI (``csrc/``,
-``include/evox_hip.h``), the ``evox_amd::`` torch custom operators and the three Python functions.
+``include/evox_hip.h``), the ``evox_amd::`` torch custom operators and the Python functions around them
+(``operators.selection``, ``utils.lexsort``).
 """
 
-__all__ = ["operators", "ops", "runtime", "workloads", "install_into_evox"]
+__all__ = ["operators", "ops", "runtime", "utils", "workloads", "install_into_evox"]
 
-from . import operators, ops, runtime, workloads
+from . import operators, ops, runtime, utils, workloads
 from .compat import install_into_evox

@@ -609,6 +609,67 @@ int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t
 
 }  // extern "C"
 
+// Workspace of the standalone stable argsort: control block with barrier slots, two pair buffers, the
+// per-block digit table and the digit totals.
+struct SortLayout {
+  int n, kstride, workers;
+  size_t ctrl, pairs0, pairs1, table, totals, total;
+};
+
+static bool make_sort_layout(int64_t n, SortLayout* L) {
+  if (n < 1 || n > 0x7FFFFF00ll) return false;
+  L->n = (int)n;
+  L->kstride = (int)round_up(n, 64);
+  int workers = (int)((n + 1023) / 1024);
+  if (workers > kRadixMaxWorkers) workers = kRadixMaxWorkers;
+  L->workers = workers;
+  size_t o = 0;
+  L->ctrl = o;    o = align_up(o + sizeof(Ctrl) + sizeof(unsigned long long) * kMaxGrid);
+  L->pairs0 = o;  o = align_up(o + sizeof(unsigned long long) * (size_t)L->kstride);
+  L->pairs1 = o;  o = align_up(o + sizeof(unsigned long long) * (size_t)L->kstride);
+  L->table = o;   o = align_up(o + sizeof(int) * 256 * (size_t)kRadixMaxWorkers);
+  L->totals = o;  o = align_up(o + sizeof(int) * 256);
+  L->total = o;
+  return true;
+}
+
+extern "C" {
+
+size_t evox_hip_argsort_workspace_bytes(int64_t n) {
+  SortLayout L;
+  return make_sort_layout(n, &L) ? L.total : 0;
+}
+
+int evox_hip_stable_argsort_step(const void* key, int kind, int64_t stride, int64_t n, const int32_t* prev_order,
+                                 int32_t* order_out, void* ws, size_t ws_bytes, void* stream) {
+  SortLayout L;
+  if (key == nullptr || order_out == nullptr || kind < 0 || kind > 2) return kErrBadArg;
+  if (!make_sort_layout(n, &L)) return kErrBadArg;
+  if (ws == nullptr || ws_bytes < L.total || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return kErrWorkspace;
+  hipStream_t s = (hipStream_t)stream;
+  uint8_t* base = static_cast<uint8_t*>(ws);
+  // every call starts from a cleared control block: barrier generations restart
+  const int64_t zero_words = (int64_t)((L.pairs0 - L.ctrl) / 4);
+  hipLaunchKernelGGL(reset_state_kernel, dim3(16), dim3(256), 0, s, reinterpret_cast<uint32_t*>(base + L.ctrl), zero_words);
+  EVX_LAUNCH_CHECK();
+  RadixBuffers b;
+  b.pairs[0] = reinterpret_cast<unsigned long long*>(base + L.pairs0);
+  b.pairs[1] = reinterpret_cast<unsigned long long*>(base + L.pairs1);
+  b.table = reinterpret_cast<int*>(base + L.table);
+  b.totals = reinterpret_cast<int*>(base + L.totals);
+  b.kstride = L.kstride;
+  int workers = L.workers;
+  const int cap = device_cus() * 2 - kFirstSweeper;  // all blocks resident at once
+  if (workers > cap) workers = cap;
+  if (workers < 1) workers = 1;
+  hipLaunchKernelGGL(argsort_step_kernel, dim3(workers + kFirstSweeper), dim3(kRadixThreads), sizeof(int) * 4 * 256, s, key, kind,
+                     stride, L.n, prev_order, reinterpret_cast<Ctrl*>(base + L.ctrl), b, order_out, g_opt.spin_limit);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"
+
 // Shared body of the two selection entry points: the population is one part or two.
 static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes, const void* x2,
                        int64_t x2_row_stride_bytes, const Fitness& fit, int64_t n, int64_t m, int64_t topk, void* out_x,

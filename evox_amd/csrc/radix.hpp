@@ -224,4 +224,45 @@ __global__ __launch_bounds__(kRadixThreads) void order_radix_kernel(const int* _
   }
 }
 
+// One step of the reference's lexsort (src/evox/utils/jit_fix_operator.py:246-250): positions ordered by
+// key[prev[e]] ascending (NaN last, signed zeros tied), ties by position e, mapped back through prev --
+//     sorted_key = key.gather(dim, sorted_indices); step = argsort(sorted_key, stable=True);
+//     sorted_indices = sorted_indices.gather(dim, step)
+// -- and the first step with prev == nullptr (the identity).  The caller chains one launch per key.
+// kind 0: float32 keys, 1: int32 keys, 2: uint32 keys; `stride` in elements.
+enum KeyKind { kKeyFloat32 = 0, kKeyInt32 = 1, kKeyUint32 = 2 };
+
+__global__ __launch_bounds__(kRadixThreads) void argsort_step_kernel(const void* __restrict__ key, int kind, int64_t stride,
+                                                                     int n, const int* __restrict__ prev,
+                                                                     Ctrl* __restrict__ ctrl, RadixBuffers buf,
+                                                                     int* __restrict__ order_out, unsigned spin_limit) {
+  extern __shared__ int radix_lds[];
+  __shared__ int base[256];
+  __shared__ int scratch[kRadixThreads];
+  if (coherent_load(&ctrl->err) != 0) return;
+  const unsigned gen0 = radix_generation_base(ctrl);
+  if (blockIdx.x == 0) {
+    radix_master(ctrl, gen0, spin_limit, scratch);
+    if (threadIdx.x == 0) ctrl->radix_epoch += 1;  // nobody reads it again in this kernel
+    return;
+  }
+  if (blockIdx.x < kFirstSweeper) return;
+  const int workers = gridDim.x - kFirstSweeper;
+  const int wb = (int)blockIdx.x - kFirstSweeper;
+  auto initial = [&](int, int e) {
+    const int idx = prev ? prev[e] : e;
+    uint32_t k;
+    if (kind == kKeyFloat32)
+      k = ordered_key(static_cast<const float*>(key)[(int64_t)idx * stride]);
+    else if (kind == kKeyInt32)
+      k = static_cast<const uint32_t*>(key)[(int64_t)idx * stride] ^ 0x80000000u;
+    else
+      k = static_cast<const uint32_t*>(key)[(int64_t)idx * stride];
+    return ((unsigned long long)k << 32) | (unsigned)idx;
+  };
+  if (!radix_sort_segments(buf, 1, n, initial, ctrl, gen0, spin_limit, radix_lds, base, scratch)) return;
+  for (int p = wb * blockDim.x + threadIdx.x; p < n; p += workers * blockDim.x)
+    order_out[p] = (int)(unsigned)(coherent_load(&buf.pairs[0][p]) & 0xFFFFFFFFull);
+}
+
 }  // namespace evx

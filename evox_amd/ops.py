@@ -378,6 +378,39 @@ def _(x_a, f_a, x_b, f_b, topk):
     )
 
 
+@torch.library.custom_op("evox_amd::stable_argsort_step", mutates_args=())
+def stable_argsort_step(key: torch.Tensor, kind: int, prev: Optional[torch.Tensor]) -> torch.Tensor:
+    """One step of lexsort on a 1-D key of 4-byte elements: ``prev`` (int32 order, or None for the
+    identity) rearranged by a stable ascending sort of ``key[prev]``.  kind 0: float32, 1: int32,
+    2: uint32 bit patterns held in an int32 tensor.  Returns an int32 order."""
+    runtime.require_gpu_tensor(key, "key")
+    if key.dim() != 1 or key.element_size() != 4 or kind not in (0, 1, 2):
+        raise ValueError("key must be one-dimensional with 4-byte elements and kind 0, 1 or 2")
+    if (kind == 0) != (key.dtype == torch.float32):
+        raise TypeError(f"kind {kind} does not fit a key of dtype {key.dtype}")
+    n = key.size(0)
+    out = torch.empty(n, dtype=torch.int32, device=key.device)
+    if n == 0:
+        return out
+    if prev is not None:
+        runtime.require_gpu_tensor(prev, "prev")
+        if prev.dtype != torch.int32 or prev.shape != (n,):
+            raise ValueError("prev must be an int32 order of the same length as the key")
+        prev = prev.contiguous()
+    with torch.cuda.device(key.device):
+        ws = runtime.sort_workspace(n, key.device)
+        stream = runtime.stream_handle(key.device)
+        _lib.call("evox_hip_stable_argsort_step", key.data_ptr(), kind, key.stride(0), n,
+                  None if prev is None else prev.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
+        runtime.note_call(ws, stream)
+    return out
+
+
+@stable_argsort_step.register_fake
+def _(key, kind, prev):
+    return key.new_empty(key.shape, dtype=torch.int32)
+
+
 @torch.library.custom_op("evox_amd::tournament_pick", mutates_args=())
 def tournament_pick(parents: torch.Tensor, fitness: torch.Tensor) -> torch.Tensor:
     """parents (n_round, t) int64 candidate indices, fitness (candidates, keys) float32 -> (n_round,) int64 winners."""

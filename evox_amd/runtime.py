@@ -64,6 +64,22 @@ def workspace(n: int, m: int, device: torch.device, with_matrix: bool = True) ->
     return ws
 
 
+def sort_workspace(n: int, device: torch.device) -> torch.Tensor:
+    """Workspace of the standalone stable argsort; shares the per-(device, stream) buffer of `workspace`
+    (every call initialises the parts it uses)."""
+    need = int(_lib.lib().evox_hip_argsort_workspace_bytes(n))
+    if need == 0:
+        raise ValueError(f"unsupported sort length n={n}")
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_handle(device))
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        _workspaces.pop(key, None)
+        ws = None
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
 def release_workspaces() -> None:
     _workspaces.clear()
 

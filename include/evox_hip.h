@@ -128,6 +128,16 @@ int evox_hip_tournament_pick(const int64_t* parents, int64_t n_round, int64_t to
                              int64_t n_candidates, int64_t n_keys, int64_t stride_row, int64_t stride_col, int64_t* out,
                              void* stream);
 
+/* One step of evox.utils.lexsort (src/evox/utils/jit_fix_operator.py:246-250): order_out = prev_order
+ * rearranged by a stable ascending sort of key[prev_order[.]] (NaN after every number, -0.0 and 0.0 tied);
+ * prev_order == NULL is the identity (the first key, :246).  Chaining one call per key, in the order of the
+ * list, gives lexsort(keys) for a one-dimensional sort: the last key is primary, ties fall to the earlier
+ * keys and then to the index.  kind: 0 float32 keys, 1 int32 keys, 2 uint32 keys; stride in elements;
+ * order_out must not alias prev_order.  Workspace: evox_hip_argsort_workspace_bytes(n). */
+size_t evox_hip_argsort_workspace_bytes(int64_t n);
+int evox_hip_stable_argsort_step(const void* key, int kind, int64_t stride, int64_t n, const int32_t* prev_order,
+                                 int32_t* order_out, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- stages of the calls above, exposed so that each kernel can be tested and timed alone.
  * They operate on the state left in the workspace by the previous stage, in this order:
  *   prepare -> dominance -> count -> peel -> (crowding -> order -> gather).                                 */

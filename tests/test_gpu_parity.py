@@ -701,6 +701,54 @@ def test_two_part_selection_edge_and_errors(edge_golden, population_path):
     assert all(torch.equal(p, q) for p, q in zip(a, b))
 
 
+# ------------------------------------------------------------------ lexsort as a function of its own
+
+
+def test_lexsort_matches_numpy_and_the_restatement(population_path):
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd.utils import lexsort
+
+    g = torch.Generator("cpu").manual_seed(5)
+    for n in (1, 2, 63, 64, 65, 1000, 5000, 70000):
+        say("lexsort", n)
+        k_f32 = torch.randint(0, 7, (n,), generator=g).float() / 2 - 1
+        k_f32[torch.rand(n, generator=g) < 0.05] = float("nan")
+        k_f32[torch.rand(n, generator=g) < 0.05] = -0.0
+        k_f32[torch.rand(n, generator=g) < 0.05] = float("inf")
+        k_f32[torch.rand(n, generator=g) < 0.05] = -float("inf")
+        k_i32 = torch.randint(-3, 3, (n,), generator=g, dtype=torch.int32)
+        k_i64 = torch.randint(-2, 2, (n,), generator=g) * (2**40) + torch.randint(0, 2, (n,), generator=g)
+        k_f64 = 1.0 + torch.randint(0, 4, (n,), generator=g).double() * 1e-13
+        k_f64[torch.rand(n, generator=g) < 0.05] = float("nan")
+        k_u8 = torch.randint(0, 3, (n,), generator=g, dtype=torch.uint8)
+        for keys in ([k_f32], [k_i32], [k_i64], [k_f64], [k_u8, k_f32], [k_f32, k_i32, k_u8], [k_f64, k_i64], [k_f32.half(), k_i32]):
+            want = er.chained_stable_argsort([k.float() if k.dtype == torch.float16 else k for k in keys])
+            got = lexsort([k.to(DEV) for k in keys])
+            assert got.dtype == torch.int64 and torch.equal(got.cpu(), want), (n, [k.dtype for k in keys])
+        # numpy's lexsort on keys without NaN (same convention: last key primary, stable)
+        assert np.array_equal(as_np(lexsort([k_i32.to(DEV), k_u8.to(DEV)])), np.lexsort((as_np(k_i32), as_np(k_u8))))
+    # along a dimension of a matrix, as the crowding distance uses it (non_dominate.py:221)
+    c = torch.rand(300, 4, generator=g)
+    m = (torch.rand(300, generator=g) < 0.5).float()[:, None].expand(-1, 4).contiguous()
+    assert torch.equal(lexsort([c.to(DEV), m.to(DEV)], dim=0).cpu(), er.chained_stable_argsort([c, m], dim=0))
+    assert torch.equal(lexsort([c.t().contiguous().to(DEV)], dim=-1).cpu(), er.chained_stable_argsort([c.t().contiguous()], dim=-1))
+
+
+def test_lexsort_gives_the_selection_order(population_path):
+    """HypE's `lexsort([-dis, rank])[:pop_size]` (hype.py:143) and the selection's own final ordering
+    (non_dominate.py:253) on the golden rank and distance of C3."""
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd.utils import lexsort
+
+    w, gold = golden_io.config("C3")
+    rank = torch.from_numpy(gold["rank"]).to(DEV)
+    dist = torch.from_numpy(gold["dist"]).to(DEV)
+    got = lexsort([-dist, rank])[: w.topk]
+    assert np.array_equal(as_np(got), gold["order"])
+
+
 # ------------------------------------------------------------------ tournament (consumer of rank / distance)
 
 
