@@ -144,6 +144,48 @@ def cpu_baseline(w, sample_rows):
     }
 
 
+def sweep_pass_bandwidth(dev, n, m):
+    """Time of the peel kernel with one sweep pass minus its time with none, over the bytes that pass reads."""
+    from evox_amd import _lib, runtime, workloads
+
+    f = workloads.uniform_population(n, m, 0, 3)[0].to(dev)
+    ws = runtime.workspace(n, m, dev)
+    s = runtime.stream_handle(dev)
+    tail = (ws.data_ptr(), ws.numel(), s)
+    runtime.set_option("peel_witness", 0)
+    try:
+        _lib.call("evox_hip_stage_prepare", f.data_ptr(), n, m, f.stride(0), f.stride(1), *tail)
+        _lib.call("evox_hip_stage_dominance", n, m, 0, *tail)
+        _lib.call("evox_hip_stage_count", n, m, *tail)
+        _lib.call("evox_hip_stage_peel", n, m, 1, None, *tail)
+        runtime.note_call(ws, s)
+        front0 = runtime.last_status()["last_front_size"]
+
+        def timed(stop):
+            ts = []
+            for _ in range(5):
+                _lib.call("evox_hip_stage_count", n, m, *tail)
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                _lib.call("evox_hip_stage_peel", n, m, stop, None, *tail)
+                b.record()
+                b.synchronize()
+                ts.append(a.elapsed_time(b) * 1e3)
+            return median(ts)
+
+        t_none, t_one = timed(1), timed(front0 + 1)
+        views = runtime.workspace_views(ws, n, m)
+        slot_of = torch.empty(n, dtype=torch.int64, device=dev)
+        slot_of[views["orig_of"].long()] = torch.arange(n, device=dev)
+        read = int(((((slot_of >> 6) + 2) & ~1) * 8)[views["rank"] >= 1].sum())
+    finally:
+        runtime.set_option("peel_witness", 1)
+        runtime.release_workspaces()
+    gbs = read / max(t_one - t_none, 1e-9) / 1e3
+    return {"pass_us": t_one - t_none, "kernel_us_with_no_pass": t_none, "bytes": read, "bound": "hbm", "achieved": gbs,
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS}
+
+
 def next_rows(dev, reps):
     """Times of the entry points either side of the hot path, on inputs resident in HBM."""
     from evox_amd import workloads
@@ -153,6 +195,9 @@ def next_rows(dev, reps):
     from evox_amd.utils import lexsort
 
     out = {}
+    # one sweep pass of the popcount-decrement formulation over a population where a pass is HBM-bound:
+    # every row outside front 0 is read once (row_words(slot) * 8 bytes each)
+    out["sweep pass N=200000 M=3"] = sweep_pass_bandwidth(dev, 200000, 3)
     # first front of a long evaluation history (what the monitor asks for) against ranking all of it
     for n, m in ((20000, 3), (200000, 3), (1000000, 3)):
         f = workloads.uniform_population(n, m, 0, 7)[0].to(dev)

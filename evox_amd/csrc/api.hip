@@ -8,6 +8,7 @@
 #include "common.hpp"
 #include "crowd.hpp"
 #include "dominance.hpp"
+#include "finish.hpp"
 #include "order.hpp"
 #include "peel.hpp"
 #include "radix.hpp"
@@ -354,51 +355,44 @@ static int radix_grid(const Layout& L) {
   return workers + kFirstSweeper;
 }
 
-// Crowding distance of the candidates list[ctrl.worst_start ... + ctrl.nv); dkey filled when the
-// final ordering follows.
-static int stage_crowding(const Ws& w, const int* list, bool want_dkey, hipStream_t s) {
-  const Layout& L = w.L;
-  int qblocks = (L.kstride + 255) / 256;
-  if (qblocks > 4096) qblocks = 4096;
-  // fronts of at most kRadixMinCandidates rows are ordered by counting, larger ones by the radix sort;
-  // the front size is only known on the device, so both are launched and one of them returns at once
-  const bool may_be_large = L.n > kRadixMinCandidates;
-  hipLaunchKernelGGL(crowd_rank_kernel, dim3(qblocks, L.m), dim3(256), 0, s, w.at<float>(L.xs), L.npad, list, w.ctrl(),
-                     L.kstride, w.at<int>(L.pos), w.at<float>(L.scost), may_be_large ? kRadixMinCandidates : L.n);
-  EVX_LAUNCH_CHECK();
-  if (may_be_large) {
-    const size_t lds = sizeof(int) * (size_t)L.m * 4 * 256;
-    if (lds > 150 * 1024) return kErrBadArg;
-    if (lds > 48 * 1024) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(crowd_radix_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess) return (int)e;
-    }
-    hipLaunchKernelGGL(crowd_radix_kernel, dim3(radix_grid(L)), dim3(kRadixThreads), lds, s, w.at<float>(L.xs), L.npad, list,
-                       w.ctrl(), L.m, radix_buffers(w), w.at<int>(L.pos), w.at<float>(L.scost), g_opt.spin_limit);
-    EVX_LAUNCH_CHECK();
+// Grid of the two kernels that order the last front (finish.hpp): the radix grid when a front of this
+// population can exceed kRadixMinCandidates rows (they then synchronise across blocks), else one block
+// per 256 candidates and objective.
+static int finish_grid(const Layout& L, int per_candidate_block) {
+  if (L.n > kRadixMinCandidates) return radix_grid(L);
+  int blocks = ((L.n + 255) / 256) * per_candidate_block;
+  return blocks < 1 ? 1 : blocks;
+}
+
+static int grant_dynamic_lds(const void* kernel, size_t lds) {
+  if (lds > 150 * 1024) return kErrBadArg;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL(crowd_dist_kernel, dim3(qblocks), dim3(256), 0, s, list, w.ctrl(), L.m, w.at<int>(L.pos),
-                     w.at<float>(L.scost), L.kstride, w.at<float>(L.dist),
-                     want_dkey ? w.at<uint32_t>(L.dkey) : (uint32_t*)nullptr);
+  return 0;
+}
+
+// Per-objective ordering of the candidates list[ctrl.worst_start ... + ctrl.nv).
+static int stage_crowd_sort(const Ws& w, const int* list, hipStream_t s) {
+  const Layout& L = w.L;
+  size_t lds = sizeof(uint64_t) * kRankTile;
+  if (L.n > kRadixMinCandidates && sizeof(int) * (size_t)L.m * 4 * 256 > lds) lds = sizeof(int) * (size_t)L.m * 4 * 256;
+  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(crowd_sort_kernel), lds)) return e;
+  hipLaunchKernelGGL(crowd_sort_kernel, dim3(finish_grid(L, L.m)), dim3(kRadixThreads), lds, s, w.at<float>(L.xs), L.npad, list,
+                     w.ctrl(), L.m, L.kstride, w.at<int>(L.pos), w.at<float>(L.scost), radix_buffers(w), g_opt.spin_limit);
   EVX_LAUNCH_CHECK();
   return 0;
 }
 
-static int stage_order(const Ws& w, hipStream_t s) {
+// Crowding distances of those candidates and, with want_order, the selection order.
+static int stage_crowd_finish(const Ws& w, const int* list, bool want_order, hipStream_t s) {
   const Layout& L = w.L;
-  int blocks = (L.n + 255) / 256;
-  if (blocks > 4096) blocks = 4096;
-  const bool may_be_large = L.n > kRadixMinCandidates;
-  hipLaunchKernelGGL(final_order_kernel, dim3(blocks), dim3(256), 0, s, w.at<int>(L.perm), w.ctrl(), w.at<uint32_t>(L.dkey),
-                     w.at<int>(L.order), may_be_large ? kRadixMinCandidates : L.n);
+  const size_t lds = sizeof(uint32_t) * kRadixMinCandidates + sizeof(uint64_t) * kRankTile;
+  hipLaunchKernelGGL(crowd_finish_kernel, dim3(finish_grid(L, 1)), dim3(kRadixThreads), lds, s, list, w.ctrl(), L.m,
+                     w.at<int>(L.pos), w.at<float>(L.scost), L.kstride, w.at<float>(L.dist), w.at<uint32_t>(L.dkey),
+                     w.at<int>(L.order), radix_buffers(w), g_opt.spin_limit, want_order ? 1 : 0);
   EVX_LAUNCH_CHECK();
-  if (may_be_large) {
-    hipLaunchKernelGGL(order_radix_kernel, dim3(radix_grid(L)), dim3(kRadixThreads), sizeof(int) * 4 * 256, s,
-                       w.at<int>(L.perm), w.ctrl(), w.at<uint32_t>(L.dkey), radix_buffers(w), w.at<int>(L.order),
-                       g_opt.spin_limit);
-    EVX_LAUNCH_CHECK();
-  }
   return 0;
 }
 
@@ -535,13 +529,14 @@ int evox_hip_stage_peel(int64_t n, int64_t m, int64_t stop_count, int32_t* rank_
 int evox_hip_stage_crowding(int64_t n, int64_t m, void* ws, size_t ws_bytes, void* stream) {
   Ws w;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
-  return stage_crowding(w, w.at<int>(w.L.perm), true, (hipStream_t)stream);
+  if (int e = stage_crowd_sort(w, w.at<int>(w.L.perm), (hipStream_t)stream)) return e;
+  return stage_crowd_finish(w, w.at<int>(w.L.perm), false, (hipStream_t)stream);
 }
 
 int evox_hip_stage_order(int64_t n, int64_t m, void* ws, size_t ws_bytes, void* stream) {
   Ws w;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
-  return stage_order(w, (hipStream_t)stream);
+  return stage_crowd_finish(w, w.at<int>(w.L.perm), true, (hipStream_t)stream);
 }
 
 int evox_hip_non_dominate_rank_until(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, int64_t stop_count,
@@ -603,7 +598,8 @@ int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t
   hipLaunchKernelGGL(compact_mask_kernel, dim3(1), dim3(1024), 0, s, mask, mask_stride, L.n, w.at<int>(L.perm),
                      w.at<float>(L.dist), w.ctrl());
   EVX_LAUNCH_CHECK();
-  if (int e = stage_crowding(w, w.at<int>(L.perm), false, s)) return e;
+  if (int e = stage_crowd_sort(w, w.at<int>(L.perm), s)) return e;
+  if (int e = stage_crowd_finish(w, w.at<int>(L.perm), false, s)) return e;
   return copy_async(dist_out, w.at<float>(L.dist), sizeof(float) * (size_t)n, s);
 }
 
@@ -686,8 +682,8 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   if (int e = stage_dominance(w, kDomKey32, s)) return e;
   if (int e = stage_count(w, true, s)) return e;
   if (int e = stage_peel(w, topk, true, s)) return e;
-  if (int e = stage_crowding(w, w.at<int>(L.perm), true, s)) return e;
-  if (int e = stage_order(w, s)) return e;
+  if (int e = stage_crowd_sort(w, w.at<int>(L.perm), s)) return e;
+  if (int e = stage_crowd_finish(w, w.at<int>(L.perm), true, s)) return e;
   int unit = 1;
   if (x != nullptr) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(x2) | reinterpret_cast<uintptr_t>(out_x) |

@@ -1,5 +1,6 @@
-// Crowding distance over a candidate list, the index-stable top-k on the last front, and the
-// fused row gather.
+// Building blocks of the crowding distance and the selection: mask compaction, ranking by counting,
+// the distance formula, the fused row gather and the tournament pick (the kernels that order the last
+// front are in finish.hpp).
 //
 // Reference semantics:
 //   crowding_distance            src/evox/operators/selection/non_dominate.py:198-231
@@ -83,87 +84,26 @@ __device__ inline int rank_by_counting(uint64_t mine, int nv, LoadPair load_pair
   return smaller;
 }
 
-// pos[k][q] = sorted position of candidate q in objective k; sorted_cost[k][pos] = its cost.
-// grid = (blocks over q, m); blocks whose candidates lie past nv leave at once.
-__global__ __launch_bounds__(256) void crowd_rank_kernel(const float* __restrict__ xs, int npad, const int* __restrict__ list_base,
-                                                         const Ctrl* __restrict__ ctrl, int kstride, int* __restrict__ pos,
-                                                         float* __restrict__ sorted_cost, int radix_above) {
-  __shared__ uint64_t tile_lds[kRankTile];
-  const int nv = ctrl->nv;
-  if (nv > radix_above || ctrl->err != 0) return;  // large fronts: radix sort kernel; error: nothing is valid
-  const int* __restrict__ list = list_base + ctrl->worst_start;
-  const int k = blockIdx.y;
-  const float* __restrict__ col = xs + (int64_t)k * npad;
-  auto pair_of = [&](int q) { return ((uint64_t)ordered_key(col[list[q]]) << 32) | (uint32_t)q; };
-  for (int q0 = blockIdx.x * blockDim.x; q0 < nv; q0 += gridDim.x * blockDim.x) {
-    const int q = q0 + threadIdx.x;
-    const float cost = q < nv ? col[list[q]] : 0.0f;
-    const uint64_t mine = q < nv ? (((uint64_t)ordered_key(cost) << 32) | (uint32_t)q) : 0ull;
-    const int p = rank_by_counting(mine, nv, pair_of, tile_lds);
-    if (q < nv) {
-      pos[(int64_t)k * kstride + q] = p;
-      sorted_cost[(int64_t)k * kstride + p] = cost;
+// Crowding distance of candidate q from the per-objective sorted positions: the sum over objectives of
+// (next - previous) / (last - first) in sorted order, +inf for a candidate that is first or last in any
+// objective (non_dominate.py:223-229).  Objectives are added in column order starting from the first
+// term, which is what torch's row sum does for the small M of this workload.
+__device__ inline float crowding_distance_of(int q, int nv, int m, const int* __restrict__ pos,
+                                             const float* __restrict__ sorted_cost, int kstride) {
+  bool boundary = false;
+  float acc = 0.0f;
+  for (int k = 0; k < m; ++k) {
+    const float* __restrict__ sc = sorted_cost + (int64_t)k * kstride;
+    const int p = pos[(int64_t)k * kstride + q];
+    if (p == 0 || p == nv - 1) {
+      boundary = true;
+    } else {
+      const float span = sc[nv - 1] - sc[0];
+      const float term = (sc[p + 1] - sc[p - 1]) / span;
+      acc = k == 0 ? term : acc + term;
     }
   }
-}
-
-// One thread per candidate: sum over objectives of (next - previous) / (last - first) in sorted
-// order, +inf for a candidate that is first or last in any objective (non_dominate.py:223-229).
-// Objectives are added in column order starting from the first term, which is what torch's row
-// sum does for the small M of this workload.  Writes the distance of row L[q] and the key of its
-// negation for the final ordering.
-__global__ __launch_bounds__(256) void crowd_dist_kernel(const int* __restrict__ list_base, const Ctrl* __restrict__ ctrl, int m,
-                                                         const int* __restrict__ pos, const float* __restrict__ sorted_cost,
-                                                         int kstride, float* __restrict__ dist, uint32_t* __restrict__ dkey) {
-  if (ctrl->err != 0) return;
-  const int nv = ctrl->nv;
-  const int* __restrict__ list = list_base + ctrl->worst_start;
-  const int nv_pad = (int)round_up(nv, 64);
-  for (int q = blockIdx.x * blockDim.x + threadIdx.x; q < nv_pad; q += gridDim.x * blockDim.x) {
-    if (q >= nv) {
-      if (dkey) dkey[q] = 0xFFFFFFFFu;
-      continue;
-    }
-    bool boundary = false;
-    float acc = 0.0f;
-    for (int k = 0; k < m; ++k) {
-      const float* __restrict__ sc = sorted_cost + (int64_t)k * kstride;
-      const int p = pos[(int64_t)k * kstride + q];
-      if (p == 0 || p == nv - 1) {
-        boundary = true;
-      } else {
-        const float span = sc[nv - 1] - sc[0];
-        const float term = (sc[p + 1] - sc[p - 1]) / span;
-        acc = k == 0 ? term : acc + term;
-      }
-    }
-    const float d = boundary ? INFINITY : acc;
-    dist[list[q]] = d;
-    if (dkey) dkey[q] = ordered_key(-d);
-  }
-}
-
-// Index-stable top-k on the last front: candidate q goes to place #{q' : (dkey', q') < (dkey, q)}
-// (distance descending, NaN after every number, then row index; jit_fix_operator.py:246-252 applied
-// to non_dominate.py:253) and is kept when that place is below `need`.  The better fronts are copied
-// from the rank-ordered listing.
-__global__ __launch_bounds__(256) void final_order_kernel(const int* __restrict__ perm, const Ctrl* __restrict__ ctrl,
-                                                          const uint32_t* __restrict__ dkey, int* __restrict__ order,
-                                                          int radix_above) {
-  __shared__ uint64_t tile_lds[kRankTile];
-  const int nv = ctrl->nv;
-  if (nv > radix_above || ctrl->err != 0) return;  // large fronts: radix sort kernel; error: nothing is valid
-  const int start = ctrl->worst_start;
-  const int need = ctrl->need;
-  const int* __restrict__ list = perm + start;
-  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < start; i += gridDim.x * blockDim.x) order[i] = perm[i];
-  auto pair_of = [&](int q) { return ((uint64_t)dkey[q] << 32) | (uint32_t)q; };
-  for (int q0 = blockIdx.x * blockDim.x; q0 < nv; q0 += gridDim.x * blockDim.x) {
-    const int q = q0 + threadIdx.x;
-    const uint64_t mine = q < nv ? pair_of(q) : 0ull;
-    const int p = rank_by_counting(mine, nv, pair_of, tile_lds);
-    if (q < nv && p < need) order[start + p] = list[q];
-  }
+  return boundary ? INFINITY : acc;
 }
 
 // out[p, :] = src[order[p], :] for the decision vectors (raw bytes, any dtype), the fitness, the rank

@@ -148,81 +148,16 @@ __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, in
   return true;
 }
 
-// Block 0 of a radix kernel: the barrier master for the 12 generations of one sort.
-__device__ inline void radix_master(Ctrl* ctrl, unsigned gen0, unsigned spin_limit, int* scratch) {
+// Block 0 of a radix kernel: the barrier master for `generations` barriers (12 per sort).
+__device__ inline void radix_master(Ctrl* ctrl, unsigned gen0, unsigned generations, unsigned spin_limit, int* scratch) {
   int dummy = 0;
-  for (unsigned g = 1; g <= 12; ++g)
+  for (unsigned g = 1; g <= generations; ++g)
     if (!master_barrier(ctrl, gen0 + g, 0, &dummy, spin_limit, scratch)) return;
 }
 
 // Barrier generations of the sorts start above every generation the peel can reach, and every run of
 // a radix kernel takes a fresh range (the epoch counter lives in the control block).
 __device__ inline unsigned radix_generation_base(const Ctrl* ctrl) { return 0x80000000u + 16u * (unsigned)ctrl->radix_epoch; }
-
-// Per-objective ordering of the last front for the crowding distance: fills pos[k][q] and
-// sorted_cost[k][p] exactly like crowd_rank_kernel, for fronts above kRadixMinCandidates rows.
-__global__ __launch_bounds__(kRadixThreads) void crowd_radix_kernel(const float* __restrict__ xs, int npad,
-                                                                    const int* __restrict__ list_base, Ctrl* __restrict__ ctrl,
-                                                                    int m, RadixBuffers buf, int* __restrict__ pos,
-                                                                    float* __restrict__ sorted_cost, unsigned spin_limit) {
-  extern __shared__ int radix_lds[];  // m * 4 * 256 ints of histograms
-  __shared__ int base[256];
-  __shared__ int scratch[kRadixThreads];
-  const int nv = ctrl->nv;
-  if (nv <= kRadixMinCandidates || coherent_load(&ctrl->err) != 0) return;
-  const unsigned gen0 = radix_generation_base(ctrl);
-  if (blockIdx.x == 0) {
-    radix_master(ctrl, gen0, spin_limit, scratch);
-    if (threadIdx.x == 0) ctrl->radix_epoch += 1;  // nobody reads it again in this kernel
-    return;
-  }
-  if (blockIdx.x < kFirstSweeper) return;
-  const int* __restrict__ list = list_base + ctrl->worst_start;
-  const int workers = gridDim.x - kFirstSweeper;
-  const int wb = (int)blockIdx.x - kFirstSweeper;
-  auto initial = [&](int k, int q) {
-    return ((unsigned long long)ordered_key(xs[(int64_t)k * npad + list[q]]) << 32) | (unsigned)q;
-  };
-  if (!radix_sort_segments(buf, m, nv, initial, ctrl, gen0, spin_limit, radix_lds, base, scratch)) return;
-  for (int k = 0; k < m; ++k)
-    for (int p = wb * blockDim.x + threadIdx.x; p < nv; p += workers * blockDim.x) {
-      const unsigned long long pr = coherent_load(&buf.pairs[0][(int64_t)k * buf.kstride + p]);
-      const int q = (int)(unsigned)(pr & 0xFFFFFFFFull);
-      pos[(int64_t)k * buf.kstride + q] = p;
-      sorted_cost[(int64_t)k * buf.kstride + p] = xs[(int64_t)k * npad + list[q]];
-    }
-}
-
-// Final ordering of the last front by (distance key, candidate index) for large fronts: the first
-// `need` candidates in that order follow the better fronts in `order`.
-__global__ __launch_bounds__(kRadixThreads) void order_radix_kernel(const int* __restrict__ perm, Ctrl* __restrict__ ctrl,
-                                                                    const uint32_t* __restrict__ dkey, RadixBuffers buf,
-                                                                    int* __restrict__ order, unsigned spin_limit) {
-  extern __shared__ int radix_lds[];
-  __shared__ int base[256];
-  __shared__ int scratch[kRadixThreads];
-  const int nv = ctrl->nv;
-  if (nv <= kRadixMinCandidates || coherent_load(&ctrl->err) != 0) return;
-  const unsigned gen0 = radix_generation_base(ctrl);
-  if (blockIdx.x == 0) {
-    radix_master(ctrl, gen0, spin_limit, scratch);
-    if (threadIdx.x == 0) ctrl->radix_epoch += 1;
-    return;
-  }
-  if (blockIdx.x < kFirstSweeper) return;
-  const int start = ctrl->worst_start;
-  const int need = ctrl->need;
-  const int* __restrict__ list = perm + start;
-  const int workers = gridDim.x - kFirstSweeper;
-  const int wb = (int)blockIdx.x - kFirstSweeper;
-  for (int i = wb * blockDim.x + threadIdx.x; i < start; i += workers * blockDim.x) order[i] = perm[i];
-  auto initial = [&](int, int q) { return ((unsigned long long)dkey[q] << 32) | (unsigned)q; };
-  if (!radix_sort_segments(buf, 1, nv, initial, ctrl, gen0, spin_limit, radix_lds, base, scratch)) return;
-  for (int p = wb * blockDim.x + threadIdx.x; p < need; p += workers * blockDim.x) {
-    const unsigned long long pr = coherent_load(&buf.pairs[0][p]);
-    order[start + p] = list[(int)(unsigned)(pr & 0xFFFFFFFFull)];
-  }
-}
 
 // One step of the reference's lexsort (src/evox/utils/jit_fix_operator.py:246-250): positions ordered by
 // key[prev[e]] ascending (NaN last, signed zeros tied), ties by position e, mapped back through prev --
@@ -242,7 +177,7 @@ __global__ __launch_bounds__(kRadixThreads) void argsort_step_kernel(const void*
   if (coherent_load(&ctrl->err) != 0) return;
   const unsigned gen0 = radix_generation_base(ctrl);
   if (blockIdx.x == 0) {
-    radix_master(ctrl, gen0, spin_limit, scratch);
+    radix_master(ctrl, gen0, 12, spin_limit, scratch);
     if (threadIdx.x == 0) ctrl->radix_epoch += 1;  // nobody reads it again in this kernel
     return;
   }
