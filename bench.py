@@ -29,9 +29,9 @@ FP32_VECTOR_PEAK_GFLOPS = 157300.0
 # their own, scaled by what the same counters read for a 512 MiB copy: x2.0 and x1.0); the summaries
 # with the commands are kept under profiles/.  Keyed by (workload, kernel); absent = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("C3", "peel_kernel"): 19.12e6 + 6.17e6,
-    ("C3", "dominance_kernel"): 3.19e6 + 25.44e6,
-    ("C3", "count_kernel"): 26.99e6 + 1.31e6,
+    ("C3", "peel_records_kernel"): 13.42e6 + 2.18e6,
+    ("C3", "dominance_kernel"): 2.89e6 + 25.36e6,
+    ("C3", "count_kernel"): 26.99e6 + 1.29e6,
 }
 
 
@@ -313,7 +313,7 @@ def main():
         "peel": {"us": times["peel_us"], "bound": "hbm", "achieved": peel_bytes / max(times["peel_us"], 1e-9) / 1e3,
                  "peak": HBM_PEAK_GBS, "unit": "GB/s", "passes": passes, "bytes": peel_bytes,
                  "us_per_pass": times["peel_us"] / max(passes, 1),
-                 "note": "latency-bound: each pass is one grid barrier plus one dependent row read"},
+                 "note": "latency-bound: each pass is one dependent row read plus one exchange between all blocks"},
         "crowding": {"us": times["crowding_us"]},
         "order": {"us": times["order_us"]},
     }
@@ -323,7 +323,9 @@ def main():
     dominant = max(("dominance", "count", "peel"), key=lambda k: phases[k]["us"])
     d = phases[dominant]
     roofline = {
-        "kernel": {"dominance": "dominance_kernel", "count": "count_kernel", "peel": "peel_kernel"}[dominant],
+        # populations below 65535 rows are peeled by the record-protocol kernel, larger ones by peel_kernel
+        "kernel": {"dominance": "dominance_kernel", "count": "count_kernel",
+                   "peel": "peel_records_kernel" if n < 65535 else "peel_kernel"}[dominant],
         "bound": "hbm" if d["bound"] == "hbm" else "valu",
         "achieved": d["achieved"], "peak": d["peak"], "unit": d["unit"], "frac": d["frac"], "traffic": None,
     }
