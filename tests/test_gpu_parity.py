@@ -525,6 +525,30 @@ def test_barrier_timeout_is_reported_not_hung():
     assert np.array_equal(as_np(non_dominate_rank(f)), as_np(er.ranks_by_peeling(f.cpu())))
 
 
+def test_fronts_of_thousands_of_rows(peel_algorithm):
+    """Every pass ranks about 3000 rows at once: with the record protocol most blocks then hold more
+    rows than their record carries and publish through the front bitmaps, and the lister merges both
+    sources.  Checked against the plain-C checker."""
+    from oracle import c_oracle
+
+    say("big_fronts", peel_algorithm)
+    f = workloads.layered_grid_population(10, 3000, seed=3, permute=True)
+    n = f.size(0)
+    want_rank, fronts = c_oracle.nd_rank(as_np(f))
+    assert fronts >= 10
+    fd = f.to(DEV)
+    assert np.array_equal(as_np(non_dominate_rank(fd)), want_rank)
+    st = runtime.last_status()
+    assert st["error"] == 0 and st["fronts"] == fronts
+    x = torch.arange(n, dtype=torch.float32)[:, None].repeat(1, 2)
+    for topk in (n // 2, 2999, n):
+        order, rank, dist, _ = c_oracle.select(as_np(f), topk)
+        xs, fs, rs, ds = nd_environmental_selection(x.to(DEV), fd, topk)
+        assert np.array_equal(as_np(xs)[:, 0].astype(np.int64), order), topk
+        assert np.array_equal(as_np(rs), rank[order])
+        assert_dist_close(ds, dist[order], f"big fronts topk {topk}")
+
+
 # ------------------------------------------------------------------ ranks up to the cut front only
 
 
