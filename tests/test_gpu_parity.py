@@ -145,7 +145,7 @@ def test_dominance_variants_agree_c3():
         keep = torch.from_numpy(defined_words(n, v["nwords"])).to(DEV).bool()
         doms.append(torch.where(keep, v["dom"][:, : v["nwords"]], 0))
     assert torch.equal(doms[0], doms[1]) and torch.equal(doms[0], doms[2])
-    # popcount of the whole matrix = dominated ordered pairs; 12.3% of N^2
+    # popcount of the whole matrix = dominated ordered pairs; 12.3% of N^2 (2^-3 for three independent uniform objectives)
     sample = doms[0][::50]  # every 50th slot
     dens = float(sum(bin(int(x) & (2**64 - 1)).count("1") for x in sample.flatten().tolist())) / (sample.size(0) * n)
     assert abs(dens - 0.125) < 0.02

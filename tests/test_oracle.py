@@ -97,7 +97,7 @@ def test_rank_layered_construction(permute):
     assert np.array_equal(r, bf.rank_longest_chain(as_np(w.f)))
     layer = np.round(as_np(w.f).sum(axis=1)).astype(np.int64) - 1
     assert (r <= layer).all()
-    assert r.max() == 19  # 20 fronts, as BASELINE.md records for this generator
+    assert r.max() == 19  # 20 fronts: one per layer of the construction
 
 
 def test_rank_c1_and_medium_random():
@@ -105,7 +105,7 @@ def test_rank_c1_and_medium_random():
               workloads.sphere_shell_population((512,), 3, 0.1, seed=1000)):
         r = as_np(er.ranks_by_peeling(f))
         assert np.array_equal(r, bf.rank_longest_chain(as_np(f)))
-    assert as_np(er.ranks_by_peeling(workloads.c1().f)).max() + 1 == 11  # F = 11
+    assert as_np(er.ranks_by_peeling(workloads.c1().f)).max() + 1 == 11  # 11 fronts for this seed (the reference gives the same, see the golden vectors)
 
 
 def test_rank_batched_equals_per_population():
