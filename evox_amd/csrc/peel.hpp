@@ -456,7 +456,8 @@ __device__ inline int witness_rows(WitnessState& st, const PassCtx& c, const uin
 // in LDS and dealt to the block's waves four at a time, so that a wave that owns five such rows does not
 // take two rounds while its neighbours idle (with 20 rows per wave that happens somewhere in almost
 // every pass, and everybody waits for the slowest wave).  q_row / q_word / q_bits hold one entry per
-// queued row; *q_n must be zero on entry.
+// queued row (q_word: in, the number of leading words to scan; out, the new witness word); *q_n must be
+// zero on entry.
 template <class OnRanked>
 __device__ inline void witness_rows_pooled(WitnessState& st, const PassCtx& c, const uint64_t* alive_lds, int first_row,
                                            int row_step, int* q_n, int* q_row, int* q_word, uint64_t* q_bits, int q_capacity,
@@ -473,6 +474,7 @@ __device__ inline void witness_rows_pooled(WitnessState& st, const PassCtx& c, c
       const int idx = atomicAdd(q_n, 1);
       if (idx < q_capacity) {
         q_row[idx] = first_row + (ch * 64 + lane) * row_step;
+        q_word[idx] = st.word[ch];  // words from the dead witness upwards hold no unranked dominator
         mine[ch] = idx;
       }
     }
@@ -487,7 +489,7 @@ __device__ inline void witness_rows_pooled(WitnessState& st, const PassCtx& c, c
     for (int q = 0; q < 4; ++q) {
       jrow[q] = q_row[base + (q < cnt ? q : 0)];
       rows[q] = c.dom + (int64_t)jrow[q] * c.wstride;
-      nws[q] = row_words(jrow[q]);
+      nws[q] = q_word[base + (q < cnt ? q : 0)];  // scan below the dead witness word only
     }
     RowScan r[4];
     const uint64_t* const four[4] = {rows[0], rows[1], rows[2], rows[3]};
