@@ -4,7 +4,7 @@ There is no fallback: if the library is missing or a call fails, an exception is
 
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+from ctypes import c_float, c_char_p, c_int, c_int64, c_size_t, c_void_p
 
 from .build import LIB_PATH
 
@@ -45,6 +45,9 @@ _SIGNATURES = {
                                          c_void_p]),
     "evox_hip_argsort_workspace_bytes": (c_size_t, [c_int64]),
     "evox_hip_stable_argsort_step": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "evox_hip_hv_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "evox_hip_hv_contributions": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p, c_void_p,
+                                          c_size_t, c_void_p]),
     "evox_hip_stage_prepare": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "evox_hip_stage_dominance": (c_int, [c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
     "evox_hip_stage_count": (c_int, [c_int64, c_int64, c_void_p, c_size_t, c_void_p]),

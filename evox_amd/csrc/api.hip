@@ -9,6 +9,7 @@
 #include "crowd.hpp"
 #include "dominance.hpp"
 #include "finish.hpp"
+#include "hv.hpp"
 #include "order.hpp"
 #include "peel.hpp"
 #include "radix.hpp"
@@ -797,6 +798,34 @@ int evox_hip_tournament_pick(const int64_t* parents, int64_t n_round, int64_t to
   if (blocks > 65535) blocks = 65535;
   hipLaunchKernelGGL(tournament_pick_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, parents, n_round,
                      (int)tournament_size, fit, stride_row, stride_col, (int)n_keys, out);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+size_t evox_hip_hv_workspace_bytes(int64_t n, int64_t n_sample) {
+  if (n < 1 || n_sample < 1 || n > 0x7FFFFF00ll || n_sample > 0x7FFFFF00ll) return 0;
+  const size_t chunks = (size_t)((n_sample + kHvChunk - 1) / kHvChunk);
+  return align_up(sizeof(float) * (size_t)n_sample) + align_up(sizeof(float) * chunks * (size_t)n);
+}
+
+int evox_hip_hv_contributions(const float* fit_t, const float* samples_t, const float* alpha, int64_t n, int64_t m,
+                              int64_t n_sample, float scale, float* out, void* ws, size_t ws_bytes, void* stream) {
+  if (fit_t == nullptr || samples_t == nullptr || alpha == nullptr || out == nullptr || m < 1 || m > 65535) return kErrBadArg;
+  const size_t need = evox_hip_hv_workspace_bytes(n, n_sample);
+  if (need == 0) return kErrBadArg;
+  if (ws == nullptr || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return kErrWorkspace;
+  hipStream_t s = (hipStream_t)stream;
+  float* weight = static_cast<float*>(ws);
+  float* partial = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + align_up(sizeof(float) * (size_t)n_sample));
+  const int chunks = (int)((n_sample + kHvChunk - 1) / kHvChunk);
+  hipLaunchKernelGGL(hv_sample_weight_kernel, dim3((unsigned)((n_sample + 255) / 256)), dim3(256), 0, s, fit_t, samples_t, alpha,
+                     (int)n, (int)m, (int)n_sample, weight);
+  EVX_LAUNCH_CHECK();
+  if (chunks > 65535) return kErrBadArg;
+  hipLaunchKernelGGL(hv_point_partial_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)chunks), dim3(256), 0, s, fit_t,
+                     samples_t, weight, (int)n, (int)m, (int)n_sample, partial);
+  EVX_LAUNCH_CHECK();
+  hipLaunchKernelGGL(hv_point_total_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, partial, (int)n, chunks, scale, out);
   EVX_LAUNCH_CHECK();
   return 0;
 }

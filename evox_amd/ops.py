@@ -411,6 +411,35 @@ def _(key, kind, prev):
     return key.new_empty(key.shape, dtype=torch.int32)
 
 
+@torch.library.custom_op("evox_amd::hv_contributions", mutates_args=())
+def hv_contributions(fit: torch.Tensor, samples: torch.Tensor, alpha: torch.Tensor, scale: float) -> torch.Tensor:
+    """fit (N, M), samples (S, M), alpha (N,) float32 -> (N,) float32:
+    scale * sum over the samples s that point i covers of alpha[max(c_s - 1, 0)], c_s = points covering s."""
+    for t, what in ((fit, "fitness"), (samples, "samples"), (alpha, "alpha")):
+        runtime.require_gpu_tensor(t, what)
+    if fit.dim() != 2 or samples.dim() != 2 or fit.size(1) != samples.size(1) or alpha.shape != (fit.size(0),):
+        raise ValueError("expected fit (N, M), samples (S, M) and alpha (N,)")
+    n, m = fit.shape
+    n_sample = samples.size(0)
+    out = torch.zeros(n, dtype=torch.float32, device=fit.device)
+    if n == 0 or n_sample == 0 or m == 0:
+        return out
+    with torch.cuda.device(fit.device):
+        fit_t = _as_f32(fit, "fitness").t().contiguous()
+        samples_t = _as_f32(samples, "samples").t().contiguous()
+        alpha32 = _as_f32(alpha, "alpha").contiguous()
+        need = int(_lib.lib().evox_hip_hv_workspace_bytes(n, n_sample))
+        ws = torch.empty(need, dtype=torch.uint8, device=fit.device)
+        _lib.call("evox_hip_hv_contributions", fit_t.data_ptr(), samples_t.data_ptr(), alpha32.data_ptr(), n, m, n_sample,
+                  float(scale), out.data_ptr(), ws.data_ptr(), ws.numel(), runtime.stream_handle(fit.device))
+    return out
+
+
+@hv_contributions.register_fake
+def _(fit, samples, alpha, scale):
+    return fit.new_empty(fit.shape[0], dtype=torch.float32)
+
+
 @torch.library.custom_op("evox_amd::tournament_pick", mutates_args=())
 def tournament_pick(parents: torch.Tensor, fitness: torch.Tensor) -> torch.Tensor:
     """parents (n_round, t) int64 candidate indices, fitness (candidates, keys) float32 -> (n_round,) int64 winners."""

@@ -138,6 +138,16 @@ size_t evox_hip_argsort_workspace_bytes(int64_t n);
 int evox_hip_stable_argsort_step(const void* key, int kind, int64_t stride, int64_t n, const int32_t* prev_order,
                                  int32_t* order_out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Monte-Carlo hypervolume contributions of HypE (src/evox/algorithms/mo/hype.py:29-39, the part of cal_hv
+ * after the samples are drawn): out[i] = scale * sum over the samples s that point i covers
+ * (all_k fit[i,k] <= sample[s,k]) of alpha[max(c_s - 1, 0)], c_s = the number of points that cover s.
+ * fit_t is (m, n) row-major (objectives by points), samples_t is (m, n_sample), alpha has n entries
+ * (hype.py:14-24), scale = prod(ref - f_min) / n_sample (:38).  Workspace: evox_hip_hv_workspace_bytes. */
+size_t evox_hip_hv_workspace_bytes(int64_t n, int64_t n_sample);
+int evox_hip_hv_contributions(const float* fit_t, const float* samples_t, const float* alpha, int64_t n, int64_t m,
+                              int64_t n_sample, float scale, float* out, void* workspace, size_t workspace_bytes,
+                              void* stream);
+
 /* ---- stages of the calls above, exposed so that each kernel can be tested and timed alone.
  * They operate on the state left in the workspace by the previous stage, in this order:
  *   prepare -> dominance -> count -> peel -> (crowding -> order -> gather).                                 */

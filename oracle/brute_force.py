@@ -132,3 +132,26 @@ def tournament_winners_brute(parents: np.ndarray, keys: np.ndarray) -> np.ndarra
             return (tuple(parts), pos)
         out[r] = min(enumerate(row), key=sort_key)[1]
     return out
+
+
+def hv_contributions_brute(fit: np.ndarray, ref: np.ndarray, pop_size: int, uniform: np.ndarray) -> np.ndarray:
+    """HypE's sampled hypervolume contributions by explicit loops, in float64: a sample inside the box
+    [min fit, ref] that is covered by c >= 1 points gives each of them alpha[c - 1], with
+    alpha[j] = prod_{l=1..j} (pop_size - l) / (n - l) / (j + 1); the sums are scaled by box volume / samples."""
+    fit = np.asarray(fit, dtype=np.float32)
+    n, m = fit.shape
+    alpha = np.zeros(n)
+    for j in range(n):
+        a = 1.0
+        for l in range(1, j + 1):
+            a *= (pop_size - l) / (n - l)
+        alpha[j] = a / (j + 1)
+    f_min = fit.min(axis=0)
+    box = (np.asarray(ref, dtype=np.float32) - f_min).astype(np.float32)
+    samples = (np.asarray(uniform, dtype=np.float32) * box + f_min).astype(np.float32)
+    out = np.zeros(n)
+    for s in range(samples.shape[0]):
+        covering = [i for i in range(n) if all(fit[i, k] <= samples[s, k] for k in range(m))]
+        for i in covering:
+            out[i] += alpha[len(covering) - 1]
+    return out * float(np.prod(box.astype(np.float64))) / samples.shape[0]

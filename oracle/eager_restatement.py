@@ -17,6 +17,7 @@ the reference's multi-objective environmental selection, on torch CPU tensors:
   first_front_mask          <- src/evox/workflows/eval_monitor.py:301-302 (= :333-334)
   merged_selection          <- src/evox/algorithms/mo/nsga2.py:99-102
   front_cut                 <- src/evox/algorithms/mo/nsga3.py:169-171 (hype.py:135-138 is the argsort form)
+  hv_contributions          <- src/evox/algorithms/mo/hype.py:12-39 (cal_hv, with the uniform draws handed in)
 
 How each function is pinned (tests/test_oracle.py):
   * dominance / ranks: tiny-input brute force, longest-dominator-chain definition, Deb's fast
@@ -24,6 +25,8 @@ How each function is pinned (tests/test_oracle.py):
   * chained_stable_argsort: numpy.lexsort on the same keys.
   * first_front_mask: the independent definition "no row dominates it" (brute_force.dominates_matrix).
   * tournament_winners: explicit tuple comparison and numpy.lexsort per tournament.
+  * hv_contributions: an explicit loop over samples and points (brute_force.hv_contributions_brute) and the
+    closed form for a single point (its contribution is the whole sampled box).
   * crowding / environmental_selection: independent numpy brute force, hand-worked examples, and
     the golden vectors under tests/golden/ (written once from the reference itself).
 """
@@ -161,3 +164,23 @@ def front_cut(f: torch.Tensor, count: int):
     rank = ranks_by_peeling(f)
     worst = torch.topk(rank, count, largest=False)[0][-1]
     return worst, rank <= worst, rank
+
+
+def hv_contributions(fit: torch.Tensor, ref: torch.Tensor, pop_size, uniform: torch.Tensor) -> torch.Tensor:
+    """cal_hv of hype.py:12-39 with the draws of its torch.rand (:28) supplied as ``uniform`` (n_sample, m)."""
+    n, m = fit.size()
+    n_sample = uniform.size(0)
+    alpha = torch.cumprod(
+        torch.cat([torch.ones(1), (pop_size - torch.arange(1, n)) / (n - torch.arange(1, n))]), dim=0
+    ) / torch.arange(1, n + 1)
+    alpha = torch.nan_to_num(alpha)
+    f_min = torch.min(fit, dim=0).values
+    samples = uniform * (ref - f_min) + f_min
+    ds = torch.zeros(n_sample, dtype=torch.int64)
+    pds = (fit.unsqueeze(0).expand(n_sample, -1, -1) - samples.unsqueeze(1).expand(-1, n, -1) <= 0).all(dim=2)
+    ds = torch.sum(torch.where(pds, ds.unsqueeze(1) + 1, ds.unsqueeze(1)), dim=1)
+    ds = torch.where(ds == 0, ds, ds - 1)
+    temp = torch.where(pds.T, ds.unsqueeze(0), -1)
+    value = torch.where(temp != -1, alpha[temp], torch.tensor(0, dtype=torch.float32))
+    f = torch.sum(value, dim=1)
+    return f * torch.prod(ref - f_min) / n_sample

@@ -773,6 +773,41 @@ def test_lexsort_gives_the_selection_order(population_path):
     assert np.array_equal(as_np(got), gold["order"])
 
 
+# ------------------------------------------------------------------ hypervolume contributions (HypE)
+
+
+def test_hv_contributions_against_oracle(population_path):
+    """Tolerance 1e-5 relative: the per-point sums run over the samples in another order than torch's."""
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd import ops
+    from evox_amd.hype import cal_hv, hv_alpha
+
+    g = torch.Generator("cpu").manual_seed(19)
+    for n, m, pop, ns in ((1, 2, 1, 100), (7, 2, 3, 333), (200, 3, 100, 10000), (1000, 5, 400, 5000), (64, 9, 64, 1025)):
+        say("hv", n, m, pop, ns)
+        fit = torch.rand(n, m, generator=g)
+        if n > 3:
+            fit[1] = fit[0]
+        ref = torch.full((m,), 1.2)
+        u = torch.rand(ns, m, generator=g)
+        want = er.hv_contributions(fit, ref, pop, u)
+        f_min = fit.min(dim=0).values
+        samples = u * (ref - f_min) + f_min  # the same float32 values as the restatement forms
+        alpha = hv_alpha(n, pop, DEV)
+        got = ops.hv_contributions(fit.to(DEV), samples.to(DEV), alpha, 1.0).cpu() * torch.prod(ref - f_min) / ns
+        assert torch.allclose(got, want, rtol=1e-5, atol=1e-9), (n, m)
+    # the function with the reference's signature draws its samples itself
+    fit = torch.rand(300, 3, generator=g).to(DEV)
+    ref = torch.full((3,), 1.1, device=DEV)
+    torch.manual_seed(7)
+    got = cal_hv(fit, ref, 150, 4000)
+    torch.manual_seed(7)
+    u = torch.rand(4000, 3, device=DEV)
+    want = er.hv_contributions(fit.cpu(), ref.cpu(), 150, u.cpu())
+    assert got.shape == (300,) and torch.allclose(got.cpu(), want, rtol=1e-5, atol=1e-9)
+
+
 # ------------------------------------------------------------------ tournament (consumer of rank / distance)
 
 

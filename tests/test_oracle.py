@@ -310,3 +310,24 @@ def test_first_front_is_the_undominated_set(name, f, ks):
     got = as_np(er.first_front_mask(f))
     assert np.array_equal(got, ~bf.dominates_matrix(as_np(f)).any(axis=0))
     assert got.any()  # a finite population always has a first front
+
+
+# ----------------------------------------------------- hypervolume contributions (HypE)
+
+
+def test_hv_contributions_match_explicit_loops():
+    g = torch.Generator("cpu").manual_seed(9)
+    for n, m, pop, ns in ((1, 2, 1, 50), (5, 2, 3, 200), (12, 3, 6, 400), (30, 4, 10, 300)):
+        fit = torch.rand(n, m, generator=g)
+        if n > 3:
+            fit[1] = fit[0]  # duplicate points share every sample
+        ref = torch.full((m,), 1.2)
+        u = torch.rand(ns, m, generator=g)
+        got = as_np(er.hv_contributions(fit, ref, pop, u)).astype(np.float64)
+        want = bf.hv_contributions_brute(as_np(fit), as_np(ref), pop, as_np(u))
+        assert np.allclose(got, want, rtol=2e-5, atol=1e-7), (n, m)
+    # closed form: a single point covers every sample of its own box, so it gets the whole volume
+    fit = torch.tensor([[0.25, 0.5, 0.75]])
+    ref = torch.tensor([1.0, 2.0, 1.0])
+    got = er.hv_contributions(fit, ref, 1, torch.rand(100, 3, generator=g))
+    assert abs(float(got[0]) - 0.75 * 1.5 * 0.25) < 1e-6
