@@ -767,10 +767,19 @@ __device__ inline void record_unit_read(unsigned long long v, bool is_first, OnC
 // another block has given up.  Only what is still missing is loaded again: a block's uncached loads are
 // served one after the other, so every extra polling load delays the one that matters (two rounds in
 // flight at once, or records four times this size, each cost more than a microsecond per pass).
-__device__ inline bool poll_record_units(const unsigned long long* gen_units, unsigned gen, unsigned long long (&v)[kRecLoads],
-                                         const int* listed, int listed_needed, const int* err, unsigned spin_limit) {
+__device__ inline bool poll_record_units(const unsigned long long* gen_units, int used_units, unsigned gen,
+                                         unsigned long long (&v)[kRecLoads], const int* listed, int listed_needed,
+                                         const int* err, unsigned spin_limit) {
   const unsigned long long* mine = gen_units + threadIdx.x;
-  unsigned pending = (1u << kRecLoads) - 1u;
+  unsigned pending = 0u;
+#pragma unroll
+  for (int k = 0; k < kRecLoads; ++k) {
+    // units past the last record are never written: they read as "no slot"
+    if ((int)threadIdx.x + k * kRecThreads < used_units)
+      pending |= 1u << k;
+    else
+      v[k] = ~0ull;
+  }
   bool waiting_listed = listed != nullptr;
   for (unsigned spins = 0;; ++spins) {
     int seen_listed = 0;
@@ -831,12 +840,14 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
         __syncthreads();
         unsigned long long v[kRecLoads];
         const unsigned gen = (unsigned)level;
-        if (!poll_record_units(records + (size_t)(gen % kRecRing) * kRecUnits, gen, v, nullptr, 0, &ctrl->err, spin_limit)) {
+        if (!poll_record_units(records + (size_t)(gen % kRecRing) * kRecUnits, sweepers * units, gen, v, nullptr, 0, &ctrl->err,
+                               spin_limit)) {
           coherent_store(&ctrl->err, kErrBarrierTimeout);
           atomicOr(&sh[2], 2);
         } else {
 #pragma unroll
           for (int k = 0; k < kRecLoads; ++k) {
+            if (tid + k * kRecThreads >= sweepers * units) continue;  // past the last record
             const int i = (tid + k * kRecThreads) & (units - 1);
             record_unit_read(
                 v[k], i == 0,
@@ -959,8 +970,8 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
     // lister has recycled what generation level + 1 will overwrite.
     EVX_TRACE(level - 1, 2);
     unsigned long long v[kRecLoads];
-    const bool fine = poll_record_units(records + (size_t)(gen % kRecRing) * kRecUnits, gen, v, tid == 0 ? &ctrl->listed : nullptr,
-                                        level + 2 - kRecRing, &ctrl->err, spin_limit);
+    const bool fine = poll_record_units(records + (size_t)(gen % kRecRing) * kRecUnits, sweepers * units, gen, v,
+                                        tid == 0 ? &ctrl->listed : nullptr, level + 2 - kRecRing, &ctrl->err, spin_limit);
     EVX_TRACE(level - 1, 3);
     if (!fine) {
       coherent_store(&ctrl->err, kErrBarrierTimeout);
@@ -968,7 +979,8 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
     } else {
 #pragma unroll
       for (int k = 0; k < kRecLoads; ++k) {
-        const int i = (tid + k * kRecThreads) & (units - 1);
+        if (tid + k * kRecThreads >= sweepers * units) continue;  // past the last record
+            const int i = (tid + k * kRecThreads) & (units - 1);
         record_unit_read(
             v[k], i == 0,
             [&](int count, bool overflow) {

@@ -549,6 +549,39 @@ def test_fronts_of_thousands_of_rows(peel_algorithm):
         assert_dist_close(ds, dist[order], f"big fronts topk {topk}")
 
 
+def test_rank_at_the_protocol_boundary(population_path):
+    """65534 rows is the largest population that the record protocol peels (16-bit slots), 65535 the first
+    one that goes to the master protocol: both against the plain-C checker."""
+    if population_path != "pipeline":
+        pytest.skip("single large populations always take the pipeline")
+    from oracle import c_oracle
+
+    f = workloads.uniform_population(65535, 3, 0, 77)[0]
+    for n in (65534, 65535):
+        say("protocol_boundary", n)
+        want, fronts = c_oracle.nd_rank(as_np(f[:n]))
+        got = non_dominate_rank(f[:n].to(DEV))
+        assert np.array_equal(as_np(got), want)
+        st = runtime.last_status()
+        assert st["error"] == 0 and st["fronts"] == fronts
+    runtime.release_workspaces()
+
+
+def test_record_protocol_with_other_block_counts():
+    """The number of sweeping blocks of the record protocol is a tunable; records need not fill the unit
+    array (100 blocks x 8 units) and may be long (16 blocks x 64 units)."""
+    say("record_blocks")
+    f = workloads.uniform_population(6000, 3, 0, 12)[0]
+    want = as_np(er.ranks_by_peeling(f))
+    try:
+        for blocks in (16, 37, 100, 128, 200):
+            runtime.set_option("peel_record_blocks", blocks)
+            assert np.array_equal(as_np(non_dominate_rank(f.to(DEV))), want), blocks
+            assert runtime.last_status()["error"] == 0
+    finally:
+        runtime.set_option("peel_record_blocks", 128)
+
+
 # ------------------------------------------------------------------ ranks up to the cut front only
 
 
