@@ -8,6 +8,7 @@ src/evox/workflows/eval_monitor.py:12), before its extension loader runs
 
 import importlib
 
+from .hype import cal_hv
 from .operators.selection import (
     crowding_distance,
     nd_environmental_selection,
@@ -31,12 +32,13 @@ _FUNCS = {
     "crowding_distance": crowding_distance,
     "nd_environmental_selection": nd_environmental_selection,
     "tournament_selection_multifit": tournament_selection_multifit,
+    "cal_hv": cal_hv,  # only evox.algorithms.mo.hype holds this name
 }
 
 
 def install_into_evox() -> list:
-    """Replaces EvoX's three selection operators, wherever a module already holds them, by the
-    HIP-backed ones.  Returns the list of ``module.name`` bindings that were changed."""
+    """Replaces EvoX's selection operators (and HypE's ``cal_hv``), wherever a module already holds
+    them, by the HIP-backed ones.  Returns the list of ``module.name`` bindings that were changed."""
     changed = []
     for target in _TARGETS:
         try:
