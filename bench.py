@@ -72,6 +72,25 @@ def event_time_us(fn, reps, inner=4):
     return median(out)
 
 
+def valu_issue_rates(dev):
+    """Vector issue rates that the device sustains right now, in G lane-ops/s: plain v_add_f32, v_cmp_le_f32 with
+    the mask written to SGPRs (every compare of the dominance kernel), and the dominance kernel's own
+    three-objective instruction mix (vector instructions only)."""
+    from evox_amd import _lib, runtime
+
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    s = runtime.stream_handle(dev)
+    blocks, iters = 2048, 2000  # 8 waves per SIMD on 256 CUs; about half a millisecond per launch
+    out = {}
+    for kind, name, valu_per_iter in ((0, "v_add_f32", 16), (1, "v_cmp_to_sgpr", 16), (2, "dominance_unit_m3", 10)):
+        def launch():
+            _lib.call("evox_hip_calibration_launch", kind, blocks, iters, sink.data_ptr(), s)
+        launch()
+        us = event_time_us(launch, 5, inner=1)
+        out[name] = blocks * 4 * iters * valu_per_iter * 64 / us / 1e3
+    return out
+
+
 def stage_profile(w, f, reps):
     """Times every stage alone through the stage entry points (same kernels, same stream)."""
     from evox_amd import _lib, runtime
@@ -320,6 +339,12 @@ def main():
     for p in phases.values():
         if "achieved" in p:
             p["frac"] = p["achieved"] / p["peak"]
+    # the same executed lane-ops against what the vector unit sustains for mask-writing compares on this
+    # device at the clock of the moment (the datasheet peak assumes the boost clock)
+    rates = valu_issue_rates(dev)
+    phases["dominance"]["measured_issue_rates_Gops"] = rates
+    phases["dominance"]["executed_valu_frac_of_measured_compare_rate"] = (
+        phases["dominance"]["executed_valu_Gops"] / rates["v_cmp_to_sgpr"])
     dominant = max(("dominance", "count", "peel"), key=lambda k: phases[k]["us"])
     d = phases[dominant]
     roofline = {

@@ -5,6 +5,7 @@
 
 #include "../../include/evox_hip.h"
 #include "batched.hpp"
+#include "calibrate.hpp"
 #include "common.hpp"
 #include "crowd.hpp"
 #include "dominance.hpp"
@@ -826,6 +827,21 @@ int evox_hip_hv_contributions(const float* fit_t, const float* samples_t, const 
                      samples_t, weight, (int)n, (int)m, (int)n_sample, partial);
   EVX_LAUNCH_CHECK();
   hipLaunchKernelGGL(hv_point_total_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, partial, (int)n, chunks, scale, out);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+int evox_hip_calibration_launch(int kind, int64_t blocks, int64_t iterations, float* scratch_out, void* stream) {
+  if (scratch_out == nullptr || kind < 0 || kind > 2 || blocks < 1 || blocks > 65535 || iterations < 1 || iterations > 10000000)
+    return kErrBadArg;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)blocks), block(256);
+  if (kind == 0)
+    hipLaunchKernelGGL(calibrate_kernel<0>, grid, block, 0, s, scratch_out, (int)iterations, 1.0f, 2.0f);
+  else if (kind == 1)
+    hipLaunchKernelGGL(calibrate_kernel<1>, grid, block, 0, s, scratch_out, (int)iterations, 1.0f, 2.0f);
+  else
+    hipLaunchKernelGGL(calibrate_kernel<2>, grid, block, 0, s, scratch_out, (int)iterations, 1.0f, 2.0f);
   EVX_LAUNCH_CHECK();
   return 0;
 }
