@@ -67,7 +67,7 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->fstart = o;     o = align_up(o + sizeof(int) * (size_t)(n + 2));
   L->xs = o;         o = align_up(o + sizeof(float) * (size_t)m * L->npad);
   L->key = o;        o = align_up(o + sizeof(uint64_t) * (size_t)L->npad);
-  L->partials = o;   o = align_up(o + sizeof(unsigned long long) * 2 * (size_t)L->prep_blocks);
+  L->partials = o;   o = align_up(o + sizeof(unsigned long long) * 3 * (size_t)L->prep_blocks);
   L->sortparam = o;  o = align_up(o + sizeof(SortParam));
   L->bstart = o;     o = align_up(o + sizeof(int) * (size_t)(buckets + 1));
   L->bcursor = o;    o = align_up(o + sizeof(int) * (size_t)buckets);
@@ -139,18 +139,17 @@ template <int M, int IW>
 static void launch_dominance_m(const Ws& w, int variant, hipStream_t s) {
   const Layout& L = w.L;
   dim3 grid((L.npad + 255) / 256, (L.nwords + IW - 1) / IW);
-  if (variant == kDomTwoCompares)
-    hipLaunchKernelGGL((dominance_kernel<M, IW, kDomTwoCompares>), grid, dim3(256), 0, s, w.at<float>(L.xs_sorted),
-                       w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad,
-                       L.wstride, L.nwords);
-  else if (variant == kDomKey64)
-    hipLaunchKernelGGL((dominance_kernel<M, IW, kDomKey64>), grid, dim3(256), 0, s, w.at<float>(L.xs_sorted),
-                       w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad,
-                       L.wstride, L.nwords);
-  else
-    hipLaunchKernelGGL((dominance_kernel<M, IW, kDomKey32>), grid, dim3(256), 0, s, w.at<float>(L.xs_sorted),
-                       w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad,
-                       L.wstride, L.nwords);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, w.at<float>(L.xs_sorted), w.at<uint64_t>(L.key_sorted),
+                       w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords,
+                       w.at<SortParam>(L.sortparam));
+  };
+  switch (variant) {
+    case kDomTwoCompares: launch(dominance_kernel<M, IW, kDomTwoCompares>); break;
+    case kDomKey64: launch(dominance_kernel<M, IW, kDomKey64>); break;
+    case kDomKey32: launch(dominance_kernel<M, IW, kDomKey32>); break;
+    default: launch(dominance_kernel<M, IW, kDomAuto>); break;
+  }
 }
 
 template <int IW>
@@ -548,7 +547,7 @@ int evox_hip_non_dominate_rank_until(const float* f, int64_t n, int64_t m, int64
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   hipStream_t s = (hipStream_t)stream;
   if (int e = stage_prepare(w, one_part(f, n, sr, sc), true, s)) return e;
-  if (int e = stage_dominance(w, kDomKey32, s)) return e;
+  if (int e = stage_dominance(w, kDomAuto, s)) return e;
   if (int e = stage_count(w, false, s)) return e;
   if (int e = stage_peel(w, stop_count, false, s)) return e;
   return copy_async(rank_out, w.at<int>(w.L.rank), sizeof(int) * (size_t)n, s);
@@ -681,7 +680,7 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   const Layout& L = w.L;
   if (int e = stage_prepare(w, fit, true, s)) return e;
-  if (int e = stage_dominance(w, kDomKey32, s)) return e;
+  if (int e = stage_dominance(w, kDomAuto, s)) return e;
   if (int e = stage_count(w, true, s)) return e;
   if (int e = stage_peel(w, topk, true, s)) return e;
   if (int e = stage_crowd_sort(w, w.at<int>(L.perm), s)) return e;

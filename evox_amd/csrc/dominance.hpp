@@ -21,16 +21,27 @@
 // bytes per dominator and is one full-rate v_cmp_ne_u32.  The lane mask is then shifted into the lane's own
 // 32-bit accumulator with v_addc_co_u32 (acc = acc + acc + carry), which performs the transpose from
 // "mask over j" to "word over i" at one VALU instruction per 64 pairs.
+//
+// Faster still when every value is finite (the usual case; the slot sort reports it): the test is done in
+// VGPR arithmetic, which this hardware issues at twice the rate of compares that write a lane mask.
+// With d_k = x[j,k] - x[i,k] (exact in sign, zero only for equal values once -0.0 is stored as +0.0; an
+// overflow to infinity keeps the sign), i dominates j exactly when no d_k is negative and some d_k is not
+// zero, i.e. when the bitwise OR of the d_k, read as a signed integer, is positive: M v_sub_f32 with a
+// scalar operand, (M-1)/2 v_or3_b32, one v_med3_i32 (clamp to 0..1) and one v_lshl_or_b32 into the lane's
+// accumulator -- 6 full-rate instructions for M = 3 instead of 5 half-rate ones and 3 scalar ANDs
+// (measured in a bare loop: 8.6 against 5.9 T pairs/s).  NaN and infinities would break the sign argument
+// (inf - inf), so populations that hold any keep the compare form.
 #pragma once
 
 #include "common.hpp"
+#include "order.hpp"
 
 namespace evx {
 
 // One kernel turns the caller's strided (n, m) fitness into structure-of-arrays form in original
 // order (padded with NaN to npad, a multiple of 128 rows) plus the 64-bit row keys, leaves the
 // (min, max) key of each block in `partials` for the slot sort, and clears the state arrays that
-// later kernels accumulate into.
+// later kernels accumulate into.  The third partial of a block says whether it met a NaN or an infinity.
 // The population may come in two parts (rows 0..n_first-1 from f, the rest from f2: parents and
 // offspring that the caller never concatenates, src/evox/algorithms/mo/nsga2.py:99-100).
 __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ f, int64_t stride_row, int64_t stride_col,
@@ -39,6 +50,10 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
                                                       uint64_t* __restrict__ key, unsigned long long* __restrict__ partials,
                                                       uint32_t* __restrict__ zero_words, int64_t n_zero_words) {
   __shared__ unsigned long long red[2][4];
+  __shared__ int any_bad;
+  if (threadIdx.x == 0) any_bad = 0;
+  __syncthreads();
+  bool bad = false;
   const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
   unsigned long long lo = ~0ull, hi = 0ull;
@@ -50,6 +65,7 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
                                   : __uint_as_float(0x7FC00000u);
       xs[(int64_t)k * npad + i] = v;
       s += ordered_key(v);
+      bad |= i < n && !(fabsf(v) <= 3.4028234663852886e38f);  // NaN or infinite
     }
     key[i] = s;
     if (i < n) {
@@ -67,25 +83,37 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
     red[0][threadIdx.x >> 6] = lo;
     red[1][threadIdx.x >> 6] = hi;
   }
+  if (bad) any_bad = 1;
   __syncthreads();
   if (threadIdx.x == 0) {
     for (int v = 1; v < 4; ++v) {
       lo = red[0][v] < lo ? red[0][v] : lo;
       hi = red[1][v] > hi ? red[1][v] : hi;
     }
-    partials[2 * blockIdx.x] = lo;      // a block without rows leaves (all-ones, 0): neutral
-    partials[2 * blockIdx.x + 1] = hi;
+    partials[3 * blockIdx.x] = lo;      // a block without rows leaves (all-ones, 0, 0): neutral
+    partials[3 * blockIdx.x + 1] = hi;
+    partials[3 * blockIdx.x + 2] = (unsigned long long)any_bad;
   }
   for (int64_t i = tid; i < n_zero_words; i += nthreads) zero_words[i] = 0u;
 }
 
-enum DomVariant { kDomKey32 = 0, kDomTwoCompares = 1, kDomKey64 = 2 };
+enum DomVariant { kDomAuto = 0, kDomTwoCompares = 1, kDomKey64 = 2, kDomKey32 = 3, kDomArith = 4 };
 
 // acc = (acc << 1) | bit, with the bit taken from a 64-lane mask: one v_addc_co_u32.
 __device__ inline uint32_t shift_in(uint32_t acc, uint64_t mask) {
   uint32_t r;
   uint64_t carry_out;
   asm("v_addc_co_u32_e64 %0, %1, %2, %2, %3" : "=v"(r), "=s"(carry_out) : "v"(acc), "s"(mask));
+  return r;
+}
+
+// acc = (acc << 1) | (o read as a signed integer is positive): v_med3_i32 clamps to 0..1, v_lshl_or_b32
+// shifts it in.  Written out because the compiler turns the clamp into a compare and a select, and a
+// compare that writes a lane mask issues at half the rate.
+__device__ inline uint32_t shift_in_positive(uint32_t acc, uint32_t o) {
+  uint32_t bit, r;
+  asm("v_med3_i32 %0, %1, 0, 1" : "=v"(bit) : "v"(o));
+  asm("v_lshl_or_b32 %0, %1, 1, %2" : "=v"(r) : "v"(acc), "v"(bit));
   return r;
 }
 
@@ -106,6 +134,13 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
     for (int t = 31; t >= 0; --t) {
       const int i = ib + t;
       uint64_t c = ~0ull;
+      if (VARIANT == kDomArith) {
+        uint32_t o = 0u;
+#pragma unroll
+        for (int k = 0; k < M; ++k) o |= __float_as_uint(xj[k] - xs[(int64_t)k * npad + i]);
+        acc = shift_in_positive(acc, o);
+        continue;
+      }
       if (VARIANT == kDomKey32) {
         // all compares first, then a tree of ANDs: independent instructions for the scheduler
         uint64_t mk[M + 1];
@@ -155,6 +190,13 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
       }
 #pragma unroll
       for (int u = G - 1; u >= 0; --u) {
+        if (VARIANT == kDomArith) {
+          uint32_t o = 0u;
+#pragma unroll
+          for (int k = 0; k < M; ++k) o |= __float_as_uint(xj[k] - xi[k][u]);
+          acc = shift_in_positive(acc, o);
+          continue;
+        }
         uint64_t c = ~0ull;
 #pragma unroll
         for (int k = 0; k < M; ++k) c &= __builtin_amdgcn_ballot_w64(xi[k][u] <= xj[k]);
@@ -180,7 +222,8 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
 template <int M, int IW, int VARIANT>
 __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
                                                         const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom, int n,
-                                                        int npad, int64_t wstride, int nwords) {
+                                                        int npad, int64_t wstride, int nwords,
+                                                        const SortParam* __restrict__ param) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int j = (blockIdx.x * 4 + wave) * 64 + lane;
@@ -191,6 +234,7 @@ __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict_
   for (int k = 0; k < M; ++k) xj[k] = xs[(int64_t)k * npad + j];
   const uint64_t kj = key[j];
   const uint32_t idj = kid[j];
+  const bool all_finite = VARIANT == kDomAuto && param->nonfinite == 0;  // wave-uniform
   uint64_t* __restrict__ out = dom + (int64_t)j * wstride;
   const int wend = (w0 + IW < nwords) ? w0 + IW : nwords;  // nwords = npad / 64 is even, and so is IW
   const int jlast = j - lane + 63;  // last row of this wave
@@ -206,9 +250,27 @@ __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict_
     const int w = w0 + 2 * p;
     if (w >= wend || w * 64 > jlast) break;
     uint32_t half[4];
+    if (VARIANT == kDomAuto) {
+      if (all_finite) {
 #pragma unroll
-    for (int h = 3; h >= 0; --h) {
-      half[h] = dominance_half_word<M, VARIANT>(xs, key, kid, npad, w * 64 + h * 32, xj, kj, idj);
+        for (int h = 3; h >= 0; --h) half[h] = dominance_half_word<M, kDomArith>(xs, key, kid, npad, w * 64 + h * 32, xj, kj, idj);
+        // padding dominators (i >= n) are NaN and give a NaN difference, whose sign is arbitrary: cleared here
+        if (w * 64 + 128 > n) {
+#pragma unroll
+          for (int h = 0; h < 4; ++h) {
+            const int first = w * 64 + h * 32;
+            half[h] = first >= n ? 0u : (first + 32 > n ? half[h] & ((1u << (n - first)) - 1u) : half[h]);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int h = 3; h >= 0; --h) half[h] = dominance_half_word<M, kDomKey32>(xs, key, kid, npad, w * 64 + h * 32, xj, kj, idj);
+      }
+    } else {
+#pragma unroll
+      for (int h = 3; h >= 0; --h) {
+        half[h] = dominance_half_word<M, VARIANT>(xs, key, kid, npad, w * 64 + h * 32, xj, kj, idj);
+      }
     }
     // bits of padding rows (i >= n) are zero because their fitness is NaN
     const uint64_t lo = ((uint64_t)half[1] << 32) | half[0];

@@ -22,21 +22,25 @@ struct SortParam {
   unsigned long long kmin;
   int shift;
   int buckets;
+  int nonfinite;  // some fitness value of the population is NaN or infinite
+  int reserved;
 };
 
 __device__ inline int bucket_of(uint64_t key, const SortParam& p) { return (int)((key - p.kmin) >> p.shift); }
 
-// Reduces the per-block (min, max) key partials written by prepare_kernel and derives the
+// Reduces the per-block (min key, max key, non-finite flag) partials written by prepare_kernel and derives the
 // quantisation: (key - kmin) >> shift < buckets.  Every block of the histogram kernel calls it.
 __device__ inline SortParam make_sort_param(const unsigned long long* __restrict__ partials, int nparts, int buckets,
                                             unsigned long long* lds2) {
   if (threadIdx.x < 64) {
-    unsigned long long lo = ~0ull, hi = 0ull;
+    unsigned long long lo = ~0ull, hi = 0ull, bad = 0ull;
     for (int p = threadIdx.x; p < nparts; p += 64) {
-      const unsigned long long a = partials[2 * p], b = partials[2 * p + 1];
+      const unsigned long long a = partials[3 * p], b = partials[3 * p + 1];
       lo = a < lo ? a : lo;
       hi = b > hi ? b : hi;
+      bad |= partials[3 * p + 2];
     }
+    bad = __builtin_amdgcn_ballot_w64(bad != 0ull);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
       const unsigned long long a = __shfl_xor(lo, off), b = __shfl_xor(hi, off);
@@ -46,12 +50,15 @@ __device__ inline SortParam make_sort_param(const unsigned long long* __restrict
     if (threadIdx.x == 0) {
       lds2[0] = lo;
       lds2[1] = hi;
+      lds2[2] = bad;
     }
   }
   __syncthreads();
   SortParam sp;
   sp.kmin = lds2[0];
   sp.buckets = buckets;
+  sp.nonfinite = lds2[2] != 0ull;
+  sp.reserved = 0;
   const unsigned long long span = lds2[1] >= lds2[0] ? lds2[1] - lds2[0] : 0ull;
   int shift = 0;
   while (shift < 63 && (span >> shift) >= (unsigned long long)buckets) ++shift;
@@ -62,7 +69,7 @@ __device__ inline SortParam make_sort_param(const unsigned long long* __restrict
 __global__ __launch_bounds__(256) void bucket_hist_kernel(const uint64_t* __restrict__ key, int n,
                                                           const unsigned long long* __restrict__ partials, int nparts,
                                                           int buckets, int* __restrict__ hist, SortParam* __restrict__ param_out) {
-  __shared__ unsigned long long lds2[2];
+  __shared__ unsigned long long lds2[3];
   const SortParam sp = make_sort_param(partials, nparts, buckets, lds2);
   if (blockIdx.x == 0 && threadIdx.x == 0) *param_out = sp;
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
@@ -166,7 +173,8 @@ __global__ __launch_bounds__(256) void bucket_place_kernel(const uint64_t* __res
       orig_of[slot] = i;
       key_sorted[slot] = ki;
       kid_sorted[slot] = (uint32_t)(lo + smaller);  // first slot holding this key: equal ids <=> equal keys
-      for (int k = 0; k < m; ++k) xs_sorted[(int64_t)k * npad + slot] = xs[(int64_t)k * npad + i];
+      // -0.0 is stored as +0.0: every comparison reads the same, and differences of equal values are +0.0
+      for (int k = 0; k < m; ++k) xs_sorted[(int64_t)k * npad + slot] = xs[(int64_t)k * npad + i] + 0.0f;
     } else {
       orig_of[i] = -1;
       key_sorted[i] = ~0ull;

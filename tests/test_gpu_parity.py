@@ -88,7 +88,7 @@ def unpack_bits(views, n):
 # ------------------------------------------------------------ dominance bits
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
 @pytest.mark.parametrize("name,f,ks", EDGE, ids=IDS)
 def test_dominance_bits_edge(name, f, ks, variant):
     say("dominance_bits", name, "variant", variant, tuple(f.shape))
@@ -122,12 +122,41 @@ def test_dominance_bits_all_m(m):
     ws = runtime.workspace(n, m, fd.device)
     s = runtime.stream_handle(fd.device)
     want = as_np(er.pareto_dominance(f, f)).T
-    for variant in ([0, 1, 2] if m <= 8 else [0]):
+    for variant in ([0, 1, 2, 3] if m <= 8 else [0]):
         _lib.call("evox_hip_stage_prepare", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), ws.data_ptr(), ws.numel(), s)
         _lib.call("evox_hip_stage_dominance", n, m, variant, ws.data_ptr(), ws.numel(), s)
         torch.cuda.synchronize()
         got = unpack_bits(runtime.workspace_views(ws, n, m), n)
         assert np.array_equal(got, want), (m, variant)
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 8])
+def test_dominance_arithmetic_form_corner_values(m):
+    """A population of finite values takes the arithmetic form of the dominance test (signs of differences):
+    denormal differences, differences that overflow, signed zeros, huge and tiny magnitudes, duplicates."""
+    say("dominance_arith", m)
+    g = torch.Generator("cpu").manual_seed(60 + m)
+    tiny = torch.tensor([0.0, -0.0, 1.4e-45, -1.4e-45, 2.8e-45, 1.17549435e-38, 1.17549421e-38, -1.17549435e-38])
+    huge = torch.tensor([3.4028235e38, -3.4028235e38, 3.4028233e38, 1e38, -1e38, 1.0, -1.0, 1.0000001])
+    pool = torch.cat([tiny, huge])
+    f = pool[torch.randint(0, pool.numel(), (700, m), generator=g)].contiguous()
+    assert bool(torch.isfinite(f).all())
+    n = f.size(0)
+    fd = f.to(DEV)
+    ws = runtime.workspace(n, m, fd.device)
+    s = runtime.stream_handle(fd.device)
+    want = as_np(er.pareto_dominance(f, f)).T
+    for variant in (0, 1):
+        _lib.call("evox_hip_stage_prepare", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), ws.data_ptr(), ws.numel(), s)
+        _lib.call("evox_hip_stage_dominance", n, m, variant, ws.data_ptr(), ws.numel(), s)
+        torch.cuda.synchronize()
+        assert np.array_equal(unpack_bits(runtime.workspace_views(ws, n, m), n), want), (m, variant)
+    assert np.array_equal(as_np(non_dominate_rank(fd)), as_np(er.ranks_by_peeling(f)))
+    # one infinity anywhere switches the whole population to the compare form: same answers
+    f2 = f.clone()
+    f2[3, 0] = float("inf")
+    f2[9, m - 1] = -float("inf")
+    assert np.array_equal(as_np(non_dominate_rank(f2.to(DEV))), as_np(er.ranks_by_peeling(f2)))
 
 
 def test_dominance_variants_agree_c3():
@@ -138,13 +167,13 @@ def test_dominance_variants_agree_c3():
     ws = runtime.workspace(n, m, fd.device)
     s = runtime.stream_handle(fd.device)
     doms = []
-    for variant in (0, 1, 2):
+    for variant in (0, 1, 2, 3):
         _lib.call("evox_hip_stage_prepare", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), ws.data_ptr(), ws.numel(), s)
         _lib.call("evox_hip_stage_dominance", n, m, variant, ws.data_ptr(), ws.numel(), s)
         v = runtime.workspace_views(ws, n, m)
         keep = torch.from_numpy(defined_words(n, v["nwords"])).to(DEV).bool()
         doms.append(torch.where(keep, v["dom"][:, : v["nwords"]], 0))
-    assert torch.equal(doms[0], doms[1]) and torch.equal(doms[0], doms[2])
+    assert torch.equal(doms[0], doms[1]) and torch.equal(doms[0], doms[2]) and torch.equal(doms[0], doms[3])
     # popcount of the whole matrix = dominated ordered pairs; 12.3% of N^2 (2^-3 for three independent uniform objectives)
     sample = doms[0][::50]  # every 50th slot
     dens = float(sum(bin(int(x) & (2**64 - 1)).count("1") for x in sample.flatten().tolist())) / (sample.size(0) * n)
