@@ -177,7 +177,7 @@ static void launch_first_front(const Ws& w, uint8_t* mask, hipStream_t s) {
   const Layout& L = w.L;
   hipLaunchKernelGGL((first_front_kernel<M>), dim3((L.n + 255) / 256), dim3(256), 0, s, w.at<float>(L.xs_sorted),
                      w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<int>(L.orig_of), L.n, L.npad, mask,
-                     w.ctrl());
+                     w.ctrl(), w.at<SortParam>(L.sortparam));
 }
 
 // Fitness -> structure of arrays + keys, state reset, then the slot sort (order.hpp).

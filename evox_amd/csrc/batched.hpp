@@ -89,26 +89,48 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
 #pragma unroll
   for (int k = 0; k < M; ++k) xj[k] = valid ? f[(int64_t)j * a.f_stride_row + k * a.f_stride_col] : nan;
 
-  // ---- dominance: word w of row j = which rows 64 w .. 64 w + 63 dominate row j
+  // ---- dominance: word w of row j = which rows 64 w .. 64 w + 63 dominate row j.  When every value of
+  // the population is finite the test is the arithmetic one of dominance.hpp (signs of the differences
+  // x[j,k] - x[i,k]; the lane's own values with -0.0 turned into +0.0, which is all that form needs).
+  bool finite_row = true;
+  float xz[M];
+#pragma unroll
+  for (int k = 0; k < M; ++k) {
+    finite_row &= !valid || fabsf(xj[k]) <= 3.4028234663852886e38f;
+    xz[k] = xj[k] + 0.0f;
+  }
+  const bool all_finite = __syncthreads_and(finite_row) != 0;
   int cnt = 0;
   for (int w = 0; w < W; ++w) {
     uint32_t half[2];
 #pragma unroll
     for (int h = 1; h >= 0; --h) {
       uint32_t acc = 0;
+      if (all_finite) {
 #pragma unroll 8
-      for (int t = 31; t >= 0; --t) {
-        const int i = w * 64 + h * 32 + t;  // wave-uniform
-        const int ic = i < n ? i : 0;
-        uint64_t le = i < n ? ~0ull : 0ull;
-        uint64_t lt = 0ull;
+        for (int t = 31; t >= 0; --t) {
+          const int i = w * 64 + h * 32 + t;  // wave-uniform
+          const int ic = i < n ? i : 0;
+          uint32_t o = 0u;
 #pragma unroll
-        for (int k = 0; k < M; ++k) {
-          const float xi = f[(int64_t)ic * a.f_stride_row + k * a.f_stride_col];
-          le &= __builtin_amdgcn_ballot_w64(xi <= xj[k]);
-          lt |= __builtin_amdgcn_ballot_w64(xi < xj[k]);
+          for (int k = 0; k < M; ++k) o |= __float_as_uint(xz[k] - f[(int64_t)ic * a.f_stride_row + k * a.f_stride_col]);
+          acc = shift_in_positive(acc, i < n ? o : 0u);
         }
-        acc = shift_in(acc, le & lt);
+      } else {
+#pragma unroll 8
+        for (int t = 31; t >= 0; --t) {
+          const int i = w * 64 + h * 32 + t;  // wave-uniform
+          const int ic = i < n ? i : 0;
+          uint64_t le = i < n ? ~0ull : 0ull;
+          uint64_t lt = 0ull;
+#pragma unroll
+          for (int k = 0; k < M; ++k) {
+            const float xi = f[(int64_t)ic * a.f_stride_row + k * a.f_stride_col];
+            le &= __builtin_amdgcn_ballot_w64(xi <= xj[k]);
+            lt |= __builtin_amdgcn_ballot_w64(xi < xj[k]);
+          }
+          acc = shift_in(acc, le & lt);
+        }
       }
       half[h] = acc;
     }

@@ -341,7 +341,7 @@ template <int M>
 __global__ __launch_bounds__(256) void first_front_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
                                                           const uint32_t* __restrict__ kid, const int* __restrict__ orig_of,
                                                           int n, int npad, uint8_t* __restrict__ mask,
-                                                          const Ctrl* __restrict__ ctrl) {
+                                                          const Ctrl* __restrict__ ctrl, const SortParam* __restrict__ param) {
   if (ctrl->err != 0) return;  // the slot sort failed: nothing is valid
   const int lane = threadIdx.x & 63;
   const int j = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 64 + lane;
@@ -350,11 +350,20 @@ __global__ __launch_bounds__(256) void first_front_kernel(const float* __restric
 #pragma unroll
   for (int k = 0; k < M; ++k) xj[k] = xs[(int64_t)k * npad + j];
   const uint32_t idj = kid[j];
+  const bool all_finite = param->nonfinite == 0;  // wave-uniform: the arithmetic form of the test applies
   bool dominated = j >= n;  // padding rows never hold the wave back
   const int iend = j - lane + 64;
 #pragma unroll 1
   for (int ib = 0; ib < iend; ib += 32) {
-    dominated |= dominance_half_word<M, kDomKey32>(xs, key, kid, npad, ib, xj, 0ull, idj) != 0u;
+    uint32_t h;
+    if (all_finite) {
+      h = dominance_half_word<M, kDomArith>(xs, key, kid, npad, ib, xj, 0ull, idj);
+      // padding dominators (NaN) give differences of arbitrary sign
+      if (ib + 32 > n) h = ib >= n ? 0u : h & ((1u << (n - ib)) - 1u);
+    } else {
+      h = dominance_half_word<M, kDomKey32>(xs, key, kid, npad, ib, xj, 0ull, idj);
+    }
+    dominated |= h != 0u;
     if (__builtin_amdgcn_ballot_w64(!dominated) == 0ull) break;
   }
   if (j < n) mask[orig_of[j]] = dominated ? 0 : 1;

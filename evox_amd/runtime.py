@@ -15,9 +15,9 @@ CHECK_STATUS = os.environ.get("EVOX_AMD_CHECK_STATUS", "0") not in ("", "0")
 
 # Populations of at most evox_hip_batched_max_rows(m) rows can run in the one-workgroup-per-population
 # kernel, larger ones need the bit-matrix pipeline.  None = choose by size (a lone population above
-# 384 rows is faster in the pipeline, which spreads it over the whole device; measured cross-over
-# between 200 and 512 rows); True / False force the choice where it is possible (tests use that to
-# drive small inputs through both).
+# 576 rows is faster in the pipeline, which spreads it over the whole device; measured: 84 against
+# 106 us at 512 rows, 227 against 113 us at 1024 rows); True / False force the choice where it is
+# possible (tests use that to drive small inputs through both).
 use_small_population_kernel = None
 
 
@@ -28,7 +28,7 @@ def small_population_kernel_fits(n: int, m: int, batch: int) -> bool:
         return False
     if use_small_population_kernel is True:
         return True
-    return n <= 384 or batch >= 3
+    return n <= 576 or batch >= 3
 
 
 def require_gpu_tensor(t: torch.Tensor, what: str) -> None:
