@@ -23,6 +23,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 VALU_CMP_PEAK_GOPS = 39321.6  # 256 CU x 64 lanes/clk x 2.4 GHz: issue peak of v_cmp_*_f32 (not packable)
+VALU_FP32_PEAK_GOPS = 78643.2  # 256 CU x 128 lanes/clk x 2.4 GHz: non-packed fp32 vector ops (157.3 TFLOP/s / 2)
 FP32_VECTOR_PEAK_GFLOPS = 157300.0
 
 # HBM bytes per launch from rocprofv3 counter runs of this script (FETCH_SIZE and WRITE_SIZE in runs of
@@ -74,15 +75,16 @@ def event_time_us(fn, reps, inner=4):
 
 def valu_issue_rates(dev):
     """Vector issue rates that the device sustains right now, in G lane-ops/s: plain v_add_f32, v_cmp_le_f32 with
-    the mask written to SGPRs (every compare of the dominance kernel), and the dominance kernel's own
-    three-objective instruction mix (vector instructions only)."""
+    the mask written to SGPRs, and the three-objective instruction mixes of the dominance kernel's two forms
+    (vector instructions only)."""
     from evox_amd import _lib, runtime
 
     sink = torch.zeros(1, dtype=torch.float32, device=dev)
     s = runtime.stream_handle(dev)
     blocks, iters = 2048, 2000  # 8 waves per SIMD on 256 CUs; about half a millisecond per launch
     out = {}
-    for kind, name, valu_per_iter in ((0, "v_add_f32", 16), (1, "v_cmp_to_sgpr", 16), (2, "dominance_unit_m3", 10)):
+    for kind, name, valu_per_iter in ((0, "v_add_f32", 16), (1, "v_cmp_to_sgpr", 16), (2, "compare_form_unit_m3", 10),
+                                      (3, "arithmetic_form_unit_m3", 12)):
         def launch():
             _lib.call("evox_hip_calibration_launch", kind, blocks, iters, sink.data_ptr(), s)
         launch()
@@ -315,17 +317,24 @@ def main():
     dom_bytes = n * m * 4 + int(row_read.sum())
     slots = torch.arange(n, device=rank.device)
     evaluated_pairs = float(((((slots >> 6) << 6) + 63) // 256 * 256 + 256).clamp(max=nwords * 64).sum())
-    executed_valu = (m + 2) * evaluated_pairs
+    # finite populations take the arithmetic form: m subtractions, (m - 1) ORs three at a time, clamp, shift-in,
+    # all issued at the full vector rate; others the compare form: m + 2 mask-writing instructions
+    finite = bool(torch.isfinite(f).all())
+    valu_per_pair = m + (m // 2) + 2 if finite else m + 2
+    executed_valu = valu_per_pair * evaluated_pairs
+    executed_peak = VALU_FP32_PEAK_GOPS if finite else VALU_CMP_PEAK_GOPS
     count_bytes = int(row_read.sum()) + n * 12
     phases = {
         "prepare_and_slot_sort": {"us": times["prepare_us"]},
-        # achieved: the reference's 2*M*N^2 compares over the kernel time (the algorithmic figure);
-        # executed: the VALU lane-instructions this kernel issues, (M + 2) per ordered pair of the lower
-        # triangle (tiles of 64 rows x 256 columns on or below the diagonal), over the same time
+        # achieved: the reference's 2*M*N^2 compares over the kernel time (the algorithmic figure), against the
+        # issue peak of compares; executed: the VALU lane-instructions this kernel issues per ordered pair of the
+        # lower triangle (tiles of 64 rows x 256 columns on or below the diagonal), over the same time, against
+        # the peak of the instruction kind it uses
         "dominance": {"us": times["dominance_us"], "bound": "valu", "achieved": compares / times["dominance_us"] / 1e3,
                       "peak": VALU_CMP_PEAK_GOPS, "unit": "Gcompare/s",
                       "executed_valu_Gops": executed_valu / times["dominance_us"] / 1e3,
-                      "executed_valu_frac": executed_valu / times["dominance_us"] / 1e3 / VALU_CMP_PEAK_GOPS,
+                      "executed_form": "arithmetic" if finite else "compare", "executed_valu_peak_Gops": executed_peak,
+                      "executed_valu_frac": executed_valu / times["dominance_us"] / 1e3 / executed_peak,
                       "hbm_GBs": dom_bytes / times["dominance_us"] / 1e3},
         "count": {"us": times["count_us"], "bound": "hbm", "achieved": count_bytes / times["count_us"] / 1e3,
                   "peak": HBM_PEAK_GBS, "unit": "GB/s"},
@@ -343,8 +352,8 @@ def main():
     # device at the clock of the moment (the datasheet peak assumes the boost clock)
     rates = valu_issue_rates(dev)
     phases["dominance"]["measured_issue_rates_Gops"] = rates
-    phases["dominance"]["executed_valu_frac_of_measured_compare_rate"] = (
-        phases["dominance"]["executed_valu_Gops"] / rates["v_cmp_to_sgpr"])
+    phases["dominance"]["executed_valu_frac_of_measured_rate"] = (
+        phases["dominance"]["executed_valu_Gops"] / (rates["v_add_f32"] if finite else rates["v_cmp_to_sgpr"]))
     dominant = max(("dominance", "count", "peel"), key=lambda k: phases[k]["us"])
     d = phases[dominant]
     roofline = {

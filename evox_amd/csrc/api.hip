@@ -831,7 +831,7 @@ int evox_hip_hv_contributions(const float* fit_t, const float* samples_t, const 
 }
 
 int evox_hip_calibration_launch(int kind, int64_t blocks, int64_t iterations, float* scratch_out, void* stream) {
-  if (scratch_out == nullptr || kind < 0 || kind > 2 || blocks < 1 || blocks > 65535 || iterations < 1 || iterations > 10000000)
+  if (scratch_out == nullptr || kind < 0 || kind > 3 || blocks < 1 || blocks > 65535 || iterations < 1 || iterations > 10000000)
     return kErrBadArg;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)blocks), block(256);
@@ -839,8 +839,10 @@ int evox_hip_calibration_launch(int kind, int64_t blocks, int64_t iterations, fl
     hipLaunchKernelGGL(calibrate_kernel<0>, grid, block, 0, s, scratch_out, (int)iterations, 1.0f, 2.0f);
   else if (kind == 1)
     hipLaunchKernelGGL(calibrate_kernel<1>, grid, block, 0, s, scratch_out, (int)iterations, 1.0f, 2.0f);
-  else
+  else if (kind == 2)
     hipLaunchKernelGGL(calibrate_kernel<2>, grid, block, 0, s, scratch_out, (int)iterations, 1.0f, 2.0f);
+  else
+    hipLaunchKernelGGL(calibrate_kernel<3>, grid, block, 0, s, scratch_out, (int)iterations, 1.0f, 2.0f);
   EVX_LAUNCH_CHECK();
   return 0;
 }

@@ -6,7 +6,9 @@
 //           kernel is); v_addc_co_u32 with SGPR carries runs at the same rate
 //   kind 2: the dominance kernel's unit for three objectives -- three v_cmp_le_f32, one v_cmp_ne_u32,
 //           three s_and_b64, one v_addc_co_u32 -- twice, on two sets of SGPRs
-// Every iteration issues 16 VALU instructions for kinds 0 and 1 and 10 for kind 2.
+//   kind 3: the unit of the arithmetic form for three objectives -- three v_sub_f32 with a scalar operand,
+//           v_or3_b32, v_med3_i32, v_lshl_or_b32 -- twice
+// Every iteration issues 16 VALU instructions for kinds 0 and 1, 10 for kind 2 and 12 for kind 3.
 #pragma once
 
 #include "common.hpp"
@@ -38,6 +40,15 @@ __global__ __launch_bounds__(256) void calibrate_kernel(float* out, int iters, f
           :
           : "v"(x), "v"(y)
           : "s20", "s21", "s22", "s23", "s24", "s25", "s26", "s27", "s28", "s29", "s30", "s31", "s32", "s33", "s34", "s35");
+    } else if (KIND == 3) {
+      asm volatile(
+          "v_sub_f32 %2, %6, s20\n v_sub_f32 %3, %7, s21\n v_sub_f32 %4, %6, s22\n v_or3_b32 %2, %2, %3, %4\n"
+          "v_med3_i32 %2, %2, 0, 1\n v_lshl_or_b32 %0, %0, 1, %2\n"
+          "v_sub_f32 %5, %6, s23\n v_sub_f32 %3, %7, s24\n v_sub_f32 %4, %6, s25\n v_or3_b32 %5, %5, %3, %4\n"
+          "v_med3_i32 %5, %5, 0, 1\n v_lshl_or_b32 %1, %1, 1, %5\n"
+          : "+v"(acc0), "+v"(acc1), "=&v"(z0), "=&v"(z1), "=&v"(z2), "=&v"(z3)
+          : "v"(x), "v"(y)
+          : "s20", "s21", "s22", "s23", "s24", "s25");
     } else {
       // s_and_b64 writes SCC: declared, or the loop's own compare would be carried across this block
       asm volatile(

@@ -149,9 +149,10 @@ int evox_hip_hv_contributions(const float* fit_t, const float* samples_t, const 
                               void* stream);
 
 /* No counterpart in the reference: launches `blocks` workgroups of 256 threads that issue, `iterations` times,
- * 16 independent v_add_f32 (kind 0), 16 independent v_cmp_le_f32 with SGPR results (kind 1), or twice the
- * dominance kernel's three-objective unit, 10 vector and 6 scalar instructions (kind 2).  The benchmark times
- * it to report the vector issue rate that the device sustains for the instruction kind of the dominance kernel.
+ * 16 independent v_add_f32 (kind 0), 16 independent v_cmp_le_f32 with SGPR results (kind 1), twice the
+ * three-objective unit of the dominance kernel's compare form, 10 vector and 6 scalar instructions (kind 2), or
+ * twice that of its arithmetic form, 12 vector instructions (kind 3).  The benchmark times it to report the
+ * vector issue rates that the device sustains for the instruction kinds of the dominance kernel.
  * scratch_out: one float of device memory (never written in practice). */
 int evox_hip_calibration_launch(int kind, int64_t blocks, int64_t iterations, float* scratch_out, void* stream);
 
