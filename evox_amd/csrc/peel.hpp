@@ -376,22 +376,72 @@ __device__ inline void witness_load(WitnessState& st, const PassCtx& c, const in
   }
 }
 
+// The witness passes only need the highest word of a row that still holds an unranked dominator, and
+// that word: found with one lane-mask per 128 words (which lanes saw an unranked dominator), the highest
+// lane of the highest non-empty mask, and three lane reads -- no cross-lane reduction through the LDS
+// permute unit, whose six dependent steps per row made the rescan the longest part of a pass.
+// Lane l holds words 2 l + 128 u and 2 l + 128 u + 1, so later lanes and later u mean higher words.
+template <int R, int U>
+__device__ inline void scan_rows_highest(const uint64_t* const (&row)[R], const int (&nw)[R], const uint64_t* mask_lds,
+                                         RowScan (&out)[R]) {
+  const int lane = threadIdx.x & 63;
+  int nw_max = 0;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    out[r].total = 0;  // not computed here
+    out[r].last_word = -1;
+    out[r].last_bits = 0ull;
+    nw_max = nw[r] > nw_max ? nw[r] : nw_max;
+  }
+  for (int w0 = lane * 2; w0 - lane * 2 < nw_max; w0 += U * 128) {  // wave-uniform trip count
+    ulonglong2 v[R][U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int w = w0 + u * 128;
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        v[r][u] = w < nw[r] ? *reinterpret_cast<const ulonglong2*>(row[r] + w) : make_ulonglong2(0ull, 0ull);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int w = w0 + u * 128;
+      const bool inside = w < nw_max;
+      const uint64_t mx = inside ? mask_lds[w] : 0ull;
+      const uint64_t my = inside ? mask_lds[w + 1] : 0ull;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const uint64_t ax = v[r][u].x & mx, ay = v[r][u].y & my;
+        const uint64_t seen = __builtin_amdgcn_ballot_w64((ax | ay) != 0ull);
+        if (seen != 0ull) {  // wave-uniform; a later (r, u) of the same row overrides an earlier one
+          const int top = 63 - __builtin_clzll(seen);
+          const int cand_word = ay != 0ull ? w + 1 : w;
+          const uint64_t cand_bits = ay != 0ull ? v[r][u].y : v[r][u].x;
+          out[r].last_word = __builtin_amdgcn_readlane(cand_word, top);
+          const uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)cand_bits, top);
+          const uint32_t hi = __builtin_amdgcn_readlane((int)(uint32_t)(cand_bits >> 32), top);
+          out[r].last_bits = ((uint64_t)hi << 32) | lo;
+        }
+      }
+    }
+  }
+}
+
 // Rescan of up to four rows against the bitmap of unranked rows, all loads in flight together.
 // Entries from `cnt` on repeat entry 0 and are ignored.
 __device__ inline void scan_up_to_four(const uint64_t* const (&rows)[4], const int (&nws)[4], int cnt, const uint64_t* alive_lds,
                                        RowScan (&r)[4]) {
   const bool short_rows = nws[0] <= 512 && nws[1] <= 512 && nws[2] <= 512 && nws[3] <= 512;
   if (cnt > 2 && short_rows) {
-    scan_rows<true, 4, 4>(rows, nws, alive_lds, r);
+    scan_rows_highest<4, 4>(rows, nws, alive_lds, r);
   } else {
     for (int q0 = 0; q0 < cnt; q0 += 2) {
       const uint64_t* const two[2] = {rows[q0], rows[q0 + 1]};
       const int nw2[2] = {nws[q0], nws[q0 + 1]};
       RowScan r2[2];
       if (short_rows)
-        scan_rows<true, 2, 4>(two, nw2, alive_lds, r2);
+        scan_rows_highest<2, 4>(two, nw2, alive_lds, r2);
       else
-        scan_rows<true, 2, 8>(two, nw2, alive_lds, r2);
+        scan_rows_highest<2, 8>(two, nw2, alive_lds, r2);
       r[q0] = r2[0];
       r[q0 + 1] = r2[1];
     }
