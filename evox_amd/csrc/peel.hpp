@@ -66,6 +66,28 @@ struct RowScan {
   uint64_t last_bits;
 };
 
+// Wave-wide sum and maximum through DPP row shifts and row broadcasts (vector ALU, a few clocks per
+// step) instead of six dependent steps through the LDS permute unit.  The result is the same in all lanes.
+__device__ inline int wave_sum(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xe, true);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xc, true);   // row_shr:8: lane 15 of a row holds the row's sum
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+  return __builtin_amdgcn_readlane(v, 63);
+}
+__device__ inline int wave_max(int v) {
+  constexpr int lowest = -2147483647 - 1;
+  v = max(v, __builtin_amdgcn_update_dpp(lowest, v, 0x111, 0xf, 0xf, false));
+  v = max(v, __builtin_amdgcn_update_dpp(lowest, v, 0x112, 0xf, 0xf, false));
+  v = max(v, __builtin_amdgcn_update_dpp(lowest, v, 0x114, 0xf, 0xe, false));
+  v = max(v, __builtin_amdgcn_update_dpp(lowest, v, 0x118, 0xf, 0xc, false));
+  v = max(v, __builtin_amdgcn_update_dpp(lowest, v, 0x142, 0xa, 0xf, false));
+  v = max(v, __builtin_amdgcn_update_dpp(lowest, v, 0x143, 0xc, 0xf, false));
+  return __builtin_amdgcn_readlane(v, 63);
+}
+
 template <bool MASKED, int R, int U>
 __device__ inline void scan_rows(const uint64_t* const (&row)[R], const int (&nw)[R], const uint64_t* mask_lds,
                                  RowScan (&out)[R]) {
@@ -107,18 +129,14 @@ __device__ inline void scan_rows(const uint64_t* const (&row)[R], const int (&nw
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    int t = total[r];
-    int hi = last_w[r];
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      t += __shfl_xor(t, off);
-      const int other = __shfl_xor(hi, off);
-      hi = other > hi ? other : hi;
-    }
-    out[r].total = t;
+    const int hi = wave_max(last_w[r]);
+    out[r].total = wave_sum(total[r]);
     out[r].last_word = hi;
     // word w is held by lane (w / 2) % 64; that lane's own highest non-empty word is then w
-    out[r].last_bits = hi < 0 ? 0ull : (uint64_t)__shfl((long long)last_v[r], (hi >> 1) & 63);
+    const int holder = hi < 0 ? 0 : (hi >> 1) & 63;
+    const uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)last_v[r], holder);
+    const uint32_t up = __builtin_amdgcn_readlane((int)(uint32_t)(last_v[r] >> 32), holder);
+    out[r].last_bits = hi < 0 ? 0ull : (((uint64_t)up << 32) | lo);
   }
 }
 
