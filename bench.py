@@ -256,6 +256,21 @@ def next_rows(dev, reps):
     _, _, rank, dist = nd_environmental_selection(x, f, w.topk)
     tournament_selection_multifit(w.topk, [-dist, rank])
     out["tournament 10000 x 2"] = {"us": event_time_us(lambda: tournament_selection_multifit(w.topk, [-dist, rank]), reps)}
+    # Monte-Carlo hypervolume: contributions of HypE (cal_hv) and the metric (100000 samples against a front)
+    from evox_amd.hype import cal_hv
+    from evox_amd.metrics import hv
+    front = f[non_dominated_mask(f)]
+    ref = torch.full((f.size(1),), 1.1, device=dev)
+    cal_hv(f[:2000], ref, 1000, 10000)
+    out["cal_hv 2000 points x 10000 samples"] = {"us": event_time_us(lambda: cal_hv(f[:2000], ref, 1000, 10000), reps)}
+    from evox_amd import ops
+    for pts, what in ((front, "first front"), (f, "whole population")):
+        points = torch.abs(pts - ref)
+        samples = torch.rand(100000, f.size(1), device=dev) * points.max(dim=0).values
+        ops.hv_covered_count(points, samples)
+        out[f"hv metric {what}: {pts.size(0)} points x 100000 samples"] = {
+            "count_us": event_time_us(lambda: ops.hv_covered_count(points, samples), reps),
+            "with_draws_on_default_device_us": event_time_us(lambda: hv(pts, ref), max(3, reps // 4))}
     return out
 
 

@@ -48,6 +48,8 @@ _SIGNATURES = {
     "evox_hip_hv_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "evox_hip_hv_contributions": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p, c_void_p,
                                           c_size_t, c_void_p]),
+    "evox_hip_hv_covered_workspace_bytes": (c_size_t, [c_int64]),
+    "evox_hip_hv_covered_count": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "evox_hip_calibration_launch": (c_int, [c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "evox_hip_stage_prepare": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "evox_hip_stage_dominance": (c_int, [c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),

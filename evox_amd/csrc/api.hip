@@ -804,8 +804,11 @@ int evox_hip_tournament_pick(const int64_t* parents, int64_t n_round, int64_t to
 
 size_t evox_hip_hv_workspace_bytes(int64_t n, int64_t n_sample) {
   if (n < 1 || n_sample < 1 || n > 0x7FFFFF00ll || n_sample > 0x7FFFFF00ll) return 0;
-  const size_t chunks = (size_t)((n_sample + kHvChunk - 1) / kHvChunk);
-  return align_up(sizeof(float) * (size_t)n_sample) + align_up(sizeof(float) * chunks * (size_t)n);
+  const int point_chunk = hv_chunk_length(n, kHvPointChunk), sample_chunk = hv_chunk_length(n_sample, kHvChunk);
+  const size_t point_chunks = (size_t)((n + point_chunk - 1) / point_chunk);
+  const size_t sample_chunks = (size_t)((n_sample + sample_chunk - 1) / sample_chunk);
+  return align_up(sizeof(float) * (size_t)n_sample) + align_up(sizeof(int32_t) * point_chunks * (size_t)n_sample) +
+         align_up(sizeof(float) * sample_chunks * (size_t)n);
 }
 
 int evox_hip_hv_contributions(const float* fit_t, const float* samples_t, const float* alpha, int64_t n, int64_t m,
@@ -815,17 +818,55 @@ int evox_hip_hv_contributions(const float* fit_t, const float* samples_t, const 
   if (need == 0) return kErrBadArg;
   if (ws == nullptr || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return kErrWorkspace;
   hipStream_t s = (hipStream_t)stream;
-  float* weight = static_cast<float*>(ws);
-  float* partial = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + align_up(sizeof(float) * (size_t)n_sample));
-  const int chunks = (int)((n_sample + kHvChunk - 1) / kHvChunk);
-  hipLaunchKernelGGL(hv_sample_weight_kernel, dim3((unsigned)((n_sample + 255) / 256)), dim3(256), 0, s, fit_t, samples_t, alpha,
-                     (int)n, (int)m, (int)n_sample, weight);
+  const int point_chunk = hv_chunk_length(n, kHvPointChunk), sample_chunk = hv_chunk_length(n_sample, kHvChunk);
+  const int point_chunks = (int)((n + point_chunk - 1) / point_chunk);
+  const int sample_chunks = (int)((n_sample + sample_chunk - 1) / sample_chunk);
+  uint8_t* base = static_cast<uint8_t*>(ws);
+  float* weight = reinterpret_cast<float*>(base);
+  int32_t* cover = reinterpret_cast<int32_t*>(base + align_up(sizeof(float) * (size_t)n_sample));
+  float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(cover) +
+                                            align_up(sizeof(int32_t) * (size_t)point_chunks * (size_t)n_sample));
+  const unsigned sample_blocks = (unsigned)((n_sample + 255) / 256), point_blocks = (unsigned)((n + 255) / 256);
+  hipLaunchKernelGGL(hv_cover_count_kernel, dim3(sample_blocks, (unsigned)point_chunks), dim3(256), 0, s, fit_t, samples_t, (int)n,
+                     (int)m, (int)n_sample, point_chunk, cover);
   EVX_LAUNCH_CHECK();
-  if (chunks > 65535) return kErrBadArg;
-  hipLaunchKernelGGL(hv_point_partial_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)chunks), dim3(256), 0, s, fit_t,
-                     samples_t, weight, (int)n, (int)m, (int)n_sample, partial);
+  hipLaunchKernelGGL(hv_sample_weight_kernel, dim3(sample_blocks), dim3(256), 0, s, cover, alpha, point_chunks, (int)n_sample,
+                     weight);
   EVX_LAUNCH_CHECK();
-  hipLaunchKernelGGL(hv_point_total_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, partial, (int)n, chunks, scale, out);
+  hipLaunchKernelGGL(hv_point_partial_kernel, dim3(point_blocks, (unsigned)sample_chunks), dim3(256), 0, s, fit_t, samples_t, weight,
+                     (int)n, (int)m, (int)n_sample, sample_chunk, partial);
+  EVX_LAUNCH_CHECK();
+  hipLaunchKernelGGL(hv_point_total_kernel, dim3(point_blocks), dim3(256), 0, s, partial, (int)n, sample_chunks, scale, out);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+size_t evox_hip_hv_covered_workspace_bytes(int64_t n_sample) {
+  if (n_sample < 1 || n_sample > 0x7FFFFF00ll) return 0;
+  return align_up(sizeof(uint32_t) * (size_t)n_sample);
+}
+
+int evox_hip_hv_covered_count(const float* points_t, const float* samples_t, int64_t n, int64_t m, int64_t n_sample,
+                              int64_t* out_count, void* ws, size_t ws_bytes, void* stream) {
+  if (points_t == nullptr || samples_t == nullptr || out_count == nullptr || n < 1 || n > 0x7FFFFF00ll || m < 1 || m > 65535)
+    return kErrBadArg;
+  const size_t need = evox_hip_hv_covered_workspace_bytes(n_sample);
+  if (need == 0) return kErrBadArg;
+  if (ws == nullptr || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return kErrWorkspace;
+  const int64_t point_chunks = (n + kHvCoverChunk - 1) / kHvCoverChunk;
+  if (point_chunks > 65535) return kErrBadArg;
+  hipStream_t s = (hipStream_t)stream;
+  uint32_t* flag = static_cast<uint32_t*>(ws);
+  hipLaunchKernelGGL(reset_state_kernel, dim3(64), dim3(256), 0, s, flag, n_sample);
+  EVX_LAUNCH_CHECK();
+  hipLaunchKernelGGL(reset_state_kernel, dim3(1), dim3(64), 0, s, reinterpret_cast<uint32_t*>(out_count), (int64_t)2);
+  EVX_LAUNCH_CHECK();
+  const unsigned sample_blocks = (unsigned)((n_sample + 255) / 256);
+  hipLaunchKernelGGL(hv_covered_kernel, dim3(sample_blocks, (unsigned)point_chunks), dim3(256), 0, s, points_t, samples_t, (int)n,
+                     (int)m, (int)n_sample, flag);
+  EVX_LAUNCH_CHECK();
+  hipLaunchKernelGGL(hv_covered_total_kernel, dim3(sample_blocks < 64u ? sample_blocks : 64u), dim3(256), 0, s, flag, (int)n_sample,
+                     reinterpret_cast<unsigned long long*>(out_count));
   EVX_LAUNCH_CHECK();
   return 0;
 }

@@ -440,6 +440,36 @@ def _(fit, samples, alpha, scale):
     return fit.new_empty(fit.shape[0], dtype=torch.float32)
 
 
+@torch.library.custom_op("evox_amd::hv_covered_count", mutates_args=())
+def hv_covered_count(points: torch.Tensor, samples: torch.Tensor) -> torch.Tensor:
+    """points (N, M), samples (S, M) float32 -> 0-d int64: the number of samples that some point exceeds
+    strictly in every objective."""
+    runtime.require_gpu_tensor(points, "points")
+    runtime.require_gpu_tensor(samples, "samples")
+    if points.dim() != 2 or samples.dim() != 2 or points.size(1) != samples.size(1):
+        raise ValueError("expected points (N, M) and samples (S, M)")
+    n, m = points.shape
+    n_sample = samples.size(0)
+    out = torch.zeros((), dtype=torch.int64, device=points.device)
+    if n == 0 or n_sample == 0:
+        return out
+    if m == 0:  # an empty conjunction holds: every sample is covered (torch.all over an empty dimension)
+        return out + n_sample
+    with torch.cuda.device(points.device):
+        points_t = _as_f32(points, "points").t().contiguous()
+        samples_t = _as_f32(samples, "samples").t().contiguous()
+        need = int(_lib.lib().evox_hip_hv_covered_workspace_bytes(n_sample))
+        ws = torch.empty(need, dtype=torch.uint8, device=points.device)
+        _lib.call("evox_hip_hv_covered_count", points_t.data_ptr(), samples_t.data_ptr(), n, m, n_sample, out.data_ptr(),
+                  ws.data_ptr(), ws.numel(), runtime.stream_handle(points.device))
+    return out
+
+
+@hv_covered_count.register_fake
+def _(points, samples):
+    return points.new_empty((), dtype=torch.int64)
+
+
 @torch.library.custom_op("evox_amd::tournament_pick", mutates_args=())
 def tournament_pick(parents: torch.Tensor, fitness: torch.Tensor) -> torch.Tensor:
     """parents (n_round, t) int64 candidate indices, fitness (candidates, keys) float32 -> (n_round,) int64 winners."""

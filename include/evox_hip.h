@@ -148,6 +148,15 @@ int evox_hip_hv_contributions(const float* fit_t, const float* samples_t, const 
                               int64_t n_sample, float scale, float* out, void* workspace, size_t workspace_bytes,
                               void* stream);
 
+/* Monte-Carlo hypervolume metric (src/evox/metrics/hv.py:18, the sample-against-points test after the samples
+ * are drawn): out_count[0] = the number of samples s with some point i strictly greater in every objective
+ * (all_k samples[s,k] < points[i,k]; a NaN on either side compares false).  points_t is (m, n) row-major,
+ * samples_t is (m, n_sample); hv.py:19 turns the count into the estimate count / n_sample * prod(bound).
+ * Workspace: evox_hip_hv_covered_workspace_bytes(n_sample). */
+size_t evox_hip_hv_covered_workspace_bytes(int64_t n_sample);
+int evox_hip_hv_covered_count(const float* points_t, const float* samples_t, int64_t n, int64_t m, int64_t n_sample,
+                              int64_t* out_count, void* workspace, size_t workspace_bytes, void* stream);
+
 /* No counterpart in the reference: launches `blocks` workgroups of 256 threads that issue, `iterations` times,
  * 16 independent v_add_f32 (kind 0), 16 independent v_cmp_le_f32 with SGPR results (kind 1), twice the
  * three-objective unit of the dominance kernel's compare form, 10 vector and 6 scalar instructions (kind 2), or

@@ -155,3 +155,28 @@ def hv_contributions_brute(fit: np.ndarray, ref: np.ndarray, pop_size: int, unif
         for i in covering:
             out[i] += alpha[len(covering) - 1]
     return out * float(np.prod(box.astype(np.float64))) / samples.shape[0]
+
+
+def hv_covered_brute(points: np.ndarray, samples: np.ndarray) -> int:
+    """Number of samples that some point exceeds strictly in every objective, by explicit loops."""
+    count = 0
+    for s in range(samples.shape[0]):
+        hit = False
+        for i in range(points.shape[0]):
+            if all(samples[s, k] < points[i, k] for k in range(points.shape[1])):
+                hit = True
+                break
+        count += int(hit)
+    return count
+
+
+def staircase_area_2d(points: np.ndarray) -> float:
+    """Exact area of the union of the boxes [0, p] over 2-D points p >= 0 (a staircase), in float64:
+    sweep the points by descending first coordinate and add the strips that raise the running height."""
+    pts = sorted(((float(p[0]), float(p[1])) for p in points), reverse=True)
+    area, height = 0.0, 0.0
+    for a, b in pts:
+        if b > height:
+            area += a * (b - height)
+            height = b
+    return area

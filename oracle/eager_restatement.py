@@ -184,3 +184,13 @@ def hv_contributions(fit: torch.Tensor, ref: torch.Tensor, pop_size, uniform: to
     value = torch.where(temp != -1, alpha[temp], torch.tensor(0, dtype=torch.float32))
     f = torch.sum(value, dim=1)
     return f * torch.prod(ref - f_min) / n_sample
+
+
+def hv_estimate(objs: torch.Tensor, ref: torch.Tensor, uniform: torch.Tensor) -> torch.Tensor:
+    """hv of metrics/hv.py:13-20 with the draws of its torch.rand (:17) supplied as ``uniform`` (num_sample, m)."""
+    points = torch.abs(objs - ref)
+    bound = torch.max(points, dim=0).values
+    max_vol = torch.prod(bound)
+    samples = uniform * bound
+    in_hypercube = torch.any(torch.all(samples.unsqueeze(1) < points.unsqueeze(0), dim=2), dim=1)
+    return in_hypercube.sum() / uniform.size(0) * max_vol

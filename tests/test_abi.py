@@ -72,6 +72,9 @@ def test_argument_validation_without_gpu(handle):
     assert handle.evox_hip_hv_workspace_bytes(0, 10) == 0 and handle.evox_hip_hv_workspace_bytes(100, 5000) >= 4 * (5000 + 5 * 100)
     assert handle.evox_hip_hv_contributions(p, p, p, 10, 0, 100, 1.0, p, p, 64, None) == _lib.E_BAD_ARG
     assert handle.evox_hip_hv_contributions(p, p, p, 10, 3, 100, 1.0, p, p, 64, None) == _lib.E_WORKSPACE
+    assert handle.evox_hip_hv_covered_workspace_bytes(0) == 0 and handle.evox_hip_hv_covered_workspace_bytes(100000) >= 4 * 391
+    assert handle.evox_hip_hv_covered_count(p, p, 10, 0, 100, p, p, 1 << 20, None) == _lib.E_BAD_ARG
+    assert handle.evox_hip_hv_covered_count(p, p, 10, 3, 100000, p, p, 64, None) == _lib.E_WORKSPACE
     assert handle.evox_hip_first_front_mask(p, 10, 3, 3, 1, None, p, 64, None) == _lib.E_BAD_ARG
     assert handle.evox_hip_first_front_mask(p, 10, 3, 3, 1, p, p, 64, None) == _lib.E_WORKSPACE
     assert handle.evox_hip_tournament_pick(None, 4, 2, p, 10, 2, 2, 1, p, None) == _lib.E_BAD_ARG

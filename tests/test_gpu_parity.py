@@ -870,6 +870,58 @@ def test_hv_contributions_against_oracle(population_path):
     assert got.shape == (300,) and torch.allclose(got.cpu(), want, rtol=1e-5, atol=1e-9)
 
 
+def test_hv_metric_against_oracle(population_path):
+    """Counts are integers, so the estimate equals the restatement's bit for bit on the same samples."""
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd import ops
+    from evox_amd.metrics import hv
+
+    g = torch.Generator("cpu").manual_seed(23)
+    for n, m, ns in ((1, 2, 100), (7, 2, 333), (200, 3, 10000), (1000, 5, 5000), (64, 9, 1025), (3000, 3, 100000)):
+        say("hv metric", n, m, ns)
+        objs = torch.rand(n, m, generator=g)
+        if n > 3:
+            objs[1] = objs[0]
+        if n == 1000:
+            objs[5, 0] = float("nan")   # the bound, every sample and the estimate become NaN (torch.max propagates)
+        ref = torch.full((m,), 1.2)
+        u = torch.rand(ns, m, generator=g)
+        want = er.hv_estimate(objs, ref, u)
+        points = torch.abs(objs - ref)
+        samples = u * points.max(dim=0).values
+        covered = ops.hv_covered_count(points.to(DEV), samples.to(DEV))
+        exact = int(torch.any(torch.all(samples.unsqueeze(1) < points.unsqueeze(0), dim=2), dim=1).sum()) if n * ns <= 5e6 else None
+        if exact is not None:
+            assert int(covered) == exact, (n, m)
+        got = covered.cpu() / ns * torch.prod(points.max(dim=0).values)  # hv.py:19 on the CPU, like the restatement
+        assert torch.equal(got, want) or (torch.isnan(got) and torch.isnan(want)), (n, m, float(got), float(want))
+    # the count itself with non-finite points among finite samples (NaN compares false, +inf exceeds everything)
+    points = torch.rand(500, 3, generator=g)
+    points[::7, 0] = float("nan")
+    points[::11, 1] = float("inf")
+    points[::13, 2] = -float("inf")
+    samples = torch.rand(4000, 3, generator=g) * 1.05
+    samples[::17, 1] = float("nan")
+    samples[::19, 2] = float("inf")
+    exact = int(torch.any(torch.all(samples.unsqueeze(1) < points.unsqueeze(0), dim=2), dim=1).sum())
+    assert 0 < exact < 4000 and int(ops.hv_covered_count(points.to(DEV), samples.to(DEV))) == exact
+    # strictness: a sample on a face of the only box is outside
+    points = torch.tensor([[1.0, 2.0]], device=DEV)
+    samples = torch.tensor([[0.5, 1.0], [1.0, 1.0], [0.5, 2.0], [0.0, 0.0]], device=DEV)
+    assert int(ops.hv_covered_count(points, samples)) == 2
+    # the function with the reference's signature draws its samples itself, on the default device
+    objs = torch.rand(300, 3, generator=g)
+    ref = torch.full((3,), 1.1)
+    torch.manual_seed(11)
+    got = hv(objs.to(DEV), ref.to(DEV), 20000)
+    torch.manual_seed(11)
+    want = er.hv_estimate(objs, ref, torch.rand(20000, 3))
+    # hv.py:19 runs on the GPU here: torch's division and product there may differ from the CPU's in the last bit
+    assert got.shape == () and got.device.type == "cuda" and float(got) == pytest.approx(float(want), rel=1e-6)
+    assert float(hv(objs.to(DEV), ref.to(DEV))) == pytest.approx(float(want), rel=0.02)  # default: 100000 samples
+
+
 # ------------------------------------------------------------------ tournament (consumer of rank / distance)
 
 

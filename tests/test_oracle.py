@@ -331,3 +331,38 @@ def test_hv_contributions_match_explicit_loops():
     ref = torch.tensor([1.0, 2.0, 1.0])
     got = er.hv_contributions(fit, ref, 1, torch.rand(100, 3, generator=g))
     assert abs(float(got[0]) - 0.75 * 1.5 * 0.25) < 1e-6
+
+
+def test_hv_estimate_matches_explicit_loops_and_exact_areas():
+    g = torch.Generator("cpu").manual_seed(21)
+    for n, m, ns in ((1, 2, 64), (6, 2, 300), (15, 3, 500), (40, 5, 300)):
+        objs = torch.rand(n, m, generator=g)
+        if n > 3:
+            objs[2] = objs[0]
+        ref = torch.full((m,), 1.3)
+        u = torch.rand(ns, m, generator=g)
+        points = torch.abs(objs - ref)
+        bound = points.max(dim=0).values
+        covered = bf.hv_covered_brute(as_np(points), as_np(u * bound))
+        want = np.float32(covered) / np.float32(ns) * np.float32(torch.prod(bound))
+        assert float(er.hv_estimate(objs, ref, u)) == pytest.approx(float(want), rel=1e-6), (n, m)
+    # one point: every sample lies strictly inside its box (a draw is below 1), so the estimate is the volume
+    objs = torch.tensor([[0.25, 0.5, 0.75]])
+    ref = torch.tensor([1.0, 2.0, 1.0])
+    assert float(er.hv_estimate(objs, ref, torch.rand(200, 3, generator=g) * 0.999)) == pytest.approx(0.75 * 1.5 * 0.25, rel=1e-6)
+    # 2-D staircase: the estimate converges on the exact union area (binomial standard error)
+    objs = torch.rand(25, 2, generator=g)
+    ref = torch.tensor([1.5, 1.5])
+    ns = 200000
+    est = float(er.hv_estimate(objs, ref, torch.rand(ns, 2, generator=g)))
+    points = as_np(torch.abs(objs - ref)).astype(np.float64)
+    exact = bf.staircase_area_2d(points)
+    box = float(points[:, 0].max() * points[:, 1].max())
+    p = exact / box
+    assert abs(est - exact) < 5 * box * np.sqrt(p * (1 - p) / ns)
+    # a NaN coordinate removes its point, strictness removes samples on a face
+    objs = torch.tensor([[0.0, float("nan")], [0.5, 0.5]])
+    ref = torch.tensor([1.0, 1.0])
+    u = torch.tensor([[0.1, 0.1], [0.5, 0.1], [0.75, 0.2]])  # bound = [1.0, nan] -> samples' 2nd coordinate is NaN
+    assert torch.isnan(er.hv_estimate(objs, ref, u))
+
