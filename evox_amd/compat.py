@@ -9,6 +9,7 @@ src/evox/workflows/eval_monitor.py:12), before its extension loader runs
 import importlib
 
 from .hype import cal_hv
+from .metrics.hv import hv
 from .operators.selection import (
     crowding_distance,
     nd_environmental_selection,
@@ -26,6 +27,8 @@ _TARGETS = (
     "evox.algorithms.mo.hype",
     "evox.algorithms.mo.rveaa",
     "evox.workflows.eval_monitor",
+    "evox.metrics.hv",
+    "evox.metrics",
 )
 _FUNCS = {
     "non_dominate_rank": non_dominate_rank,
@@ -33,12 +36,13 @@ _FUNCS = {
     "nd_environmental_selection": nd_environmental_selection,
     "tournament_selection_multifit": tournament_selection_multifit,
     "cal_hv": cal_hv,  # only evox.algorithms.mo.hype holds this name
+    "hv": hv,  # the function that evox.metrics and evox.metrics.hv hold (src/evox/metrics/__init__.py:4), not the module
 }
 
 
 def install_into_evox() -> list:
-    """Replaces EvoX's selection operators (and HypE's ``cal_hv``), wherever a module already holds
-    them, by the HIP-backed ones.  Returns the list of ``module.name`` bindings that were changed."""
+    """Replaces EvoX's selection operators (and HypE's ``cal_hv``, and the ``hv`` metric), wherever a module
+    already holds them, by the HIP-backed ones.  Returns the list of ``module.name`` bindings that were changed."""
     changed = []
     for target in _TARGETS:
         try:
@@ -46,7 +50,7 @@ def install_into_evox() -> list:
         except ImportError:
             continue
         for name, fn in _FUNCS.items():
-            if hasattr(module, name):
+            if callable(getattr(module, name, None)):
                 setattr(module, name, fn)
                 changed.append(f"{target}.{name}")
     return changed

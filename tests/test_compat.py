@@ -13,7 +13,7 @@ def _fake_evox():
         "evox", "evox.operators", "evox.operators.selection", "evox.operators.selection.non_dominate",
         "evox.operators.selection.tournament_selection", "evox.algorithms", "evox.algorithms.mo",
         "evox.algorithms.mo.nsga2", "evox.algorithms.mo.nsga3", "evox.algorithms.mo.hype", "evox.algorithms.mo.rveaa",
-        "evox.workflows", "evox.workflows.eval_monitor",
+        "evox.workflows", "evox.workflows.eval_monitor", "evox.metrics", "evox.metrics.hv", "evox.metrics.igd",
     ]
     mods = {n: types.ModuleType(n) for n in names}
     for n, m in mods.items():
@@ -41,6 +41,8 @@ def _fake_evox():
     mods["evox.algorithms.mo.rveaa"].non_dominate_rank = original
     mods["evox.workflows.eval_monitor"].non_dominate_rank = original
     mods["evox.workflows.eval_monitor"].unrelated = original
+    mods["evox.metrics.hv"].hv = original
+    mods["evox.metrics"].hv = original  # the package's `from .hv import hv` shadows the sub-module (metrics/__init__.py:4)
     return mods, original
 
 
@@ -57,7 +59,9 @@ def test_install_rebinds_every_early_bound_name(monkeypatch):
     assert mods["evox.operators.selection"].crowding_distance is hip_selection.crowding_distance
     assert mods["evox.algorithms.mo.hype"].cal_hv is evox_amd.hype.cal_hv
     assert mods["evox.workflows.eval_monitor"].unrelated is original  # nothing else is touched
-    assert "evox.algorithms.mo.nsga2.nd_environmental_selection" in changed and len(changed) == 17
+    assert mods["evox.metrics"].hv is evox_amd.metrics.hv and mods["evox.metrics.hv"].hv is evox_amd.metrics.hv
+    assert isinstance(mods["evox.metrics"].igd, types.ModuleType)  # sub-modules stay what they are
+    assert "evox.algorithms.mo.nsga2.nd_environmental_selection" in changed and len(changed) == 19
 
 
 def test_install_without_evox_changes_nothing():
