@@ -18,9 +18,16 @@
 #include "common.hpp"
 #include "dominance.hpp"
 
+// Hook for timing builds (a tool defines it to store a time stamp per workgroup and phase); nothing otherwise.
+#ifndef EVX_BATCH_TRACE
+#define EVX_BATCH_TRACE(slot)
+#endif
+
 namespace evx {
 
 constexpr int kBatchedMaxRows = 1024;
+
+typedef const float __attribute__((address_space(4))) * ConstFloatPtr;
 
 struct BatchedArgs {
   const float* f;          // (batch, n, m) with strides in elements
@@ -51,8 +58,9 @@ __device__ inline int count_smaller(const uint64_t* tile, int nv, uint64_t mine)
 }
 
 // Row stride of the LDS matrix in words: one word of padding against bank conflicts, except at the
-// largest size, where the padding would not fit.
-__host__ __device__ inline int batched_row_stride(int nt) { return nt == 1024 ? 16 : nt / 64 + 1; }
+// largest size, where the padding would not fit; at least five words (an odd stride again), because
+// after the peeling the matrix's LDS holds the fitness, up to eight floats per row.
+__host__ __device__ inline int batched_row_stride(int nt) { return nt == 1024 ? 16 : (nt / 64 + 1 < 5 ? 5 : nt / 64 + 1); }
 
 // Dynamic LDS layout (nt = blockDim.x):
 //   uint64 dom[nt][row stride] | uint64 tile[nt + 4] | uint64 front[2][16] | float scost[nt] | float dist[nt] |
@@ -85,6 +93,7 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
   const float* __restrict__ f = a.f + (int64_t)blockIdx.x * a.f_stride_b;
   const float nan = __uint_as_float(0x7FC00000u);
 
+  EVX_BATCH_TRACE(0);
   float xj[M];
 #pragma unroll
   for (int k = 0; k < M; ++k) xj[k] = valid ? f[(int64_t)j * a.f_stride_row + k * a.f_stride_col] : nan;
@@ -100,20 +109,40 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
     xz[k] = xj[k] + 0.0f;
   }
   const bool all_finite = __syncthreads_and(finite_row) != 0;
+  const bool packed_rows = a.f_stride_col == 1 && a.f_stride_row == M;
+  // Dominators are read at wave-uniform addresses through the constant address space: the fitness is never
+  // written here, and only loads known to be invariant are issued as scalar loads.
+  const ConstFloatPtr fc = (ConstFloatPtr)f;
   int cnt = 0;
   for (int w = 0; w < W; ++w) {
     uint32_t half[2];
 #pragma unroll
     for (int h = 1; h >= 0; --h) {
       uint32_t acc = 0;
-      if (all_finite) {
+      if (all_finite && packed_rows && w * 64 + h * 32 + 32 <= n) {
+        // rows of M consecutive floats: eight dominators are 8 M consecutive scalars, fetched by wide scalar loads
+#pragma unroll 1
+        for (int g = 3; g >= 0; --g) {
+          const ConstFloatPtr p = fc + (int64_t)(w * 64 + h * 32 + g * 8) * M;  // wave-uniform
+          float v[8 * M];
+#pragma unroll
+          for (int e = 0; e < 8 * M; ++e) v[e] = p[e];
+#pragma unroll
+          for (int u = 7; u >= 0; --u) {
+            uint32_t o = 0u;
+#pragma unroll
+            for (int k = 0; k < M; ++k) o |= __float_as_uint(xz[k] - v[u * M + k]);
+            acc = shift_in_positive(acc, o);
+          }
+        }
+      } else if (all_finite) {
 #pragma unroll 8
         for (int t = 31; t >= 0; --t) {
           const int i = w * 64 + h * 32 + t;  // wave-uniform
           const int ic = i < n ? i : 0;
           uint32_t o = 0u;
 #pragma unroll
-          for (int k = 0; k < M; ++k) o |= __float_as_uint(xz[k] - f[(int64_t)ic * a.f_stride_row + k * a.f_stride_col]);
+          for (int k = 0; k < M; ++k) o |= __float_as_uint(xz[k] - fc[(int64_t)ic * a.f_stride_row + k * a.f_stride_col]);
           acc = shift_in_positive(acc, i < n ? o : 0u);
         }
       } else {
@@ -125,7 +154,7 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
           uint64_t lt = 0ull;
 #pragma unroll
           for (int k = 0; k < M; ++k) {
-            const float xi = f[(int64_t)ic * a.f_stride_row + k * a.f_stride_col];
+            const float xi = fc[(int64_t)ic * a.f_stride_row + k * a.f_stride_col];
             le &= __builtin_amdgcn_ballot_w64(xi <= xj[k]);
             lt |= __builtin_amdgcn_ballot_w64(xi < xj[k]);
           }
@@ -139,6 +168,7 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
     cnt += __popcll(word);
   }
 
+  EVX_BATCH_TRACE(1);
   // ---- peeling (non_dominate.py:29-59, :107-125), fronts listed in ascending row order
   int rank = valid ? kRankUnset : -1;
   int level = 0, ranked = 0;
@@ -180,18 +210,26 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
   if (a.rank_all && valid) a.rank_all[(int64_t)blockIdx.x * n + j] = rank;
   if (a.out_f == nullptr) return;  // rank-only mode
 
+  EVX_BATCH_TRACE(2);
   // ---- crowding distance of the last front (non_dominate.py:198-231 with mask = rank == worst)
   const int topk = a.stop_count;
   const int need = topk - worst_start;
   rank_lds[j] = rank;
   dist[j] = -INFINITY;
+  // The matrix is not needed any more: its LDS now holds the fitness by objective (fit_lds[k * nt + row]), so
+  // that candidates and the final gather read other rows' values from LDS instead of from memory again.
+  __syncthreads();
+  float* fit_lds = reinterpret_cast<float*>(dom);
+#pragma unroll
+  for (int k = 0; k < M; ++k) fit_lds[k * nt + j] = xj[k];
   __syncthreads();
   const bool cand = j < nv;                      // thread q = candidate q of the last front
   const int row = cand ? perm[worst_start + j] : 0;
   bool boundary = false;
   float acc = 0.0f;
+#pragma unroll
   for (int k = 0; k < M; ++k) {
-    const float cost = cand ? f[(int64_t)row * a.f_stride_row + k * a.f_stride_col] : 0.0f;
+    const float cost = cand ? fit_lds[k * nt + row] : 0.0f;
     const uint64_t mine = ((uint64_t)ordered_key(cost) << 32) | (uint32_t)j;
     __syncthreads();
     if (j < nv + 4) tile[j] = cand ? mine : ~0ull;
@@ -212,6 +250,7 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
   const float d = boundary ? INFINITY : acc;
   if (cand) dist[row] = d;
 
+  EVX_BATCH_TRACE(3);
   // ---- index-stable top-k on the last front by (-distance, row index) (non_dominate.py:253)
   {
     const uint64_t mine = ((uint64_t)ordered_key(-d) << 32) | (uint32_t)j;
@@ -225,13 +264,15 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
   }
   __syncthreads();
 
+  EVX_BATCH_TRACE(4);
   // ---- gather the topk selected rows
   const int64_t ob = (int64_t)blockIdx.x * topk;
   for (int p = j; p < topk; p += nt) {
     const int src = order[p];
     a.out_rank[ob + p] = rank_lds[src];
     a.out_dist[ob + p] = dist[src];
-    for (int k = 0; k < M; ++k) a.out_f[(ob + p) * M + k] = f[(int64_t)src * a.f_stride_row + k * a.f_stride_col];
+#pragma unroll
+    for (int k = 0; k < M; ++k) a.out_f[(ob + p) * M + k] = fit_lds[k * nt + src];
   }
   if (a.x != nullptr) {
     const uint8_t* __restrict__ xb = a.x + (int64_t)blockIdx.x * a.x_stride_b;
@@ -251,6 +292,7 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
       }
     }
   }
+  EVX_BATCH_TRACE(5);
 }
 
 }  // namespace evx
