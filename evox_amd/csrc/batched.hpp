@@ -58,32 +58,90 @@ __device__ inline int count_smaller(const uint64_t* tile, int nv, uint64_t mine)
 }
 
 // Row stride of the LDS matrix in words: one word of padding against bank conflicts, except at the
-// largest size, where the padding would not fit; at least five words (an odd stride again), because
-// after the peeling the matrix's LDS holds the fitness, up to eight floats per row.
-__host__ __device__ inline int batched_row_stride(int nt) { return nt == 1024 ? 16 : (nt / 64 + 1 < 5 ? 5 : nt / 64 + 1); }
+// largest size, where the padding would not fit; at least nine words, because after the peeling the
+// matrix's LDS is reused for everything that the rest of the kernel needs (up to 60 bytes per row).
+__host__ __device__ inline int batched_row_stride(int nt) { return nt == 1024 ? 16 : (nt / 64 + 1 < 9 ? 9 : nt / 64 + 1); }
 
 // Dynamic LDS layout (nt = blockDim.x):
-//   uint64 dom[nt][row stride] | uint64 tile[nt + 4] | uint64 front[2][16] | float scost[nt] | float dist[nt] |
-//   int perm[nt] | int order[nt] | int rank[nt]
+//   uint64 dom[nt][row stride] | uint64 front[2][16] | int perm[nt]
+// and, once the peeling is over, inside dom:
+//   float fit[8][nt] | uint64 tile[nt + 4] | float scost[nt] | float dist[nt] | int order[nt] | int rank[nt] | int below[nt]
+// 512 rows take 39.2 KB, so that four workgroups share a compute unit's 160 KB.
 __host__ __device__ inline size_t batched_lds_bytes(int nt) {
-  return sizeof(uint64_t) * ((size_t)nt * batched_row_stride(nt) + (nt + 4) + 32) + sizeof(float) * 2 * (size_t)nt +
-         sizeof(int) * 3 * (size_t)nt;
+  return sizeof(uint64_t) * ((size_t)nt * batched_row_stride(nt) + 32) + sizeof(int) * (size_t)nt;
 }
 
+// Position of every candidate among the nv (key << 32 | index) pairs of `tile`, by counting the smaller
+// ones; the count of candidate q is split over `parts` threads (q + nvq * part, nvq = nv rounded up to whole
+// waves), which add their shares in `below`.  Every thread of the block calls it; returns the position
+// for threads below nv.  tile must be padded with all-ones up to a multiple of 4 entries.
+__device__ inline int position_by_counting(const uint64_t* tile, int* below, int nv, int j, int nt) {
+  const int nvq = (nv + 63) & ~63;
+  const int parts = nt / nvq;  // >= 1: nv <= n <= nt
+  if (parts == 1) {
+    __syncthreads();
+    return j < nv ? count_smaller(tile, nv, tile[j]) : 0;
+  }
+  if (j < nv) below[j] = 0;
+  __syncthreads();
+  const int part = j / nvq, q = j - part * nvq;
+  if (part < parts && q < nv) {
+    const int chunk = (((nv + parts - 1) / parts) + 3) & ~3;
+    const int e0 = part * chunk;
+    const int e1 = min(e0 + chunk, (nv + 3) & ~3);
+    const uint64_t mine = tile[q];
+    int smaller = 0;
+    for (int e = e0; e < e1; e += 4) {
+      const ulonglong2 u = *reinterpret_cast<const ulonglong2*>(tile + e);
+      const ulonglong2 v = *reinterpret_cast<const ulonglong2*>(tile + e + 2);
+      smaller += (u.x < mine) + (u.y < mine) + (v.x < mine) + (v.y < mine);
+    }
+    if (smaller) atomicAdd(&below[q], smaller);
+  }
+  __syncthreads();
+  return j < nv ? below[j] : 0;
+}
+
+// The selected rows of x as one flat array of units of type T (4 or 16 bytes): unit e of the output is unit
+// e % row_units of input row order[e / row_units].  Four units per thread are in flight: a load that waits
+// for the store before it costs a memory round trip per unit.
+template <class T>
+__device__ inline void gather_units(const uint8_t* __restrict__ xb, uint8_t* __restrict__ dst, const int* order,
+                                    int64_t x_row_stride, uint32_t row_units, uint32_t total, int j, int nt) {
+  for (uint32_t e = j; e < total; e += 4u * nt) {
+    const uint32_t e1 = e + nt, e2 = e + 2u * nt, e3 = e + 3u * nt;
+    const uint32_t c0 = e, c1 = e1 < total ? e1 : e, c2 = e2 < total ? e2 : e, c3 = e3 < total ? e3 : e;
+    const uint32_t p0 = c0 / row_units, p1 = c1 / row_units, p2 = c2 / row_units, p3 = c3 / row_units;
+    const T v0 = *reinterpret_cast<const T*>(xb + (int64_t)order[p0] * x_row_stride + (int64_t)(c0 - p0 * row_units) * sizeof(T));
+    const T v1 = *reinterpret_cast<const T*>(xb + (int64_t)order[p1] * x_row_stride + (int64_t)(c1 - p1 * row_units) * sizeof(T));
+    const T v2 = *reinterpret_cast<const T*>(xb + (int64_t)order[p2] * x_row_stride + (int64_t)(c2 - p2 * row_units) * sizeof(T));
+    const T v3 = *reinterpret_cast<const T*>(xb + (int64_t)order[p3] * x_row_stride + (int64_t)(c3 - p3 * row_units) * sizeof(T));
+    *reinterpret_cast<T*>(dst + (int64_t)c0 * sizeof(T)) = v0;
+    if (e1 < total) *reinterpret_cast<T*>(dst + (int64_t)e1 * sizeof(T)) = v1;
+    if (e2 < total) *reinterpret_cast<T*>(dst + (int64_t)e2 * sizeof(T)) = v2;
+    if (e3 < total) *reinterpret_cast<T*>(dst + (int64_t)e3 * sizeof(T)) = v3;
+  }
+}
+
+// Registers are capped for eight waves per SIMD (at most 64 VGPRs and 96 SGPRs): populations of 512 rows
+// then run four workgroups to a compute unit, which their LDS allows.
 template <int M>
-__global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void batched_kernel(BatchedArgs a) {
   extern __shared__ uint64_t lds64[];
   const int nt = blockDim.x;
   const int W = nt >> 6;
   const int rs = batched_row_stride(nt);
   uint64_t* dom = lds64;
-  uint64_t* tile = dom + (size_t)nt * rs;
-  uint64_t* front = tile + (nt + 4);
-  float* scost = reinterpret_cast<float*>(front + 32);
+  uint64_t* front = dom + (size_t)nt * rs;
+  int* perm = reinterpret_cast<int*>(front + 32);
+  // valid only after the peeling (they lie inside dom)
+  float* fit_lds = reinterpret_cast<float*>(dom);
+  uint64_t* tile = reinterpret_cast<uint64_t*>(fit_lds + 8 * (size_t)nt);
+  float* scost = reinterpret_cast<float*>(tile + (nt + 4));
   float* dist = scost + nt;
-  int* perm = reinterpret_cast<int*>(dist + nt);
-  int* order = perm + nt;
+  int* order = reinterpret_cast<int*>(dist + nt);
   int* rank_lds = order + nt;
+  int* below = rank_lds + nt;
 
   const int n = a.n;
   const int j = threadIdx.x;
@@ -212,14 +270,13 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
 
   EVX_BATCH_TRACE(2);
   // ---- crowding distance of the last front (non_dominate.py:198-231 with mask = rank == worst)
+  // Every thread is past its last read of the matrix (the loop above leaves after a barrier): its LDS now
+  // holds the fitness by objective (fit_lds[k * nt + row]) and the arrays of the steps below, so that
+  // candidates and the final gather read other rows' values from LDS instead of from memory again.
   const int topk = a.stop_count;
   const int need = topk - worst_start;
   rank_lds[j] = rank;
   dist[j] = -INFINITY;
-  // The matrix is not needed any more: its LDS now holds the fitness by objective (fit_lds[k * nt + row]), so
-  // that candidates and the final gather read other rows' values from LDS instead of from memory again.
-  __syncthreads();
-  float* fit_lds = reinterpret_cast<float*>(dom);
 #pragma unroll
   for (int k = 0; k < M; ++k) fit_lds[k * nt + j] = xj[k];
   __syncthreads();
@@ -230,12 +287,9 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
 #pragma unroll
   for (int k = 0; k < M; ++k) {
     const float cost = cand ? fit_lds[k * nt + row] : 0.0f;
-    const uint64_t mine = ((uint64_t)ordered_key(cost) << 32) | (uint32_t)j;
-    __syncthreads();
-    if (j < nv + 4) tile[j] = cand ? mine : ~0ull;
+    if (j < nv + 4) tile[j] = cand ? ((uint64_t)ordered_key(cost) << 32) | (uint32_t)j : ~0ull;
     if (j < 4 && nv + j >= nt) tile[nv + j] = ~0ull;  // padding past the thread count
-    __syncthreads();
-    const int p = cand ? count_smaller(tile, nv, mine) : 0;
+    const int p = position_by_counting(tile, below, nv, j, nt);
     if (cand) scost[p] = cost;
     __syncthreads();
     if (cand) {
@@ -246,6 +300,7 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
         acc = k == 0 ? term : acc + term;
       }
     }
+    // (the barriers inside the next position_by_counting separate these reads from the next writes of scost)
   }
   const float d = boundary ? INFINITY : acc;
   if (cand) dist[row] = d;
@@ -253,12 +308,9 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
   EVX_BATCH_TRACE(3);
   // ---- index-stable top-k on the last front by (-distance, row index) (non_dominate.py:253)
   {
-    const uint64_t mine = ((uint64_t)ordered_key(-d) << 32) | (uint32_t)j;
-    __syncthreads();
-    if (j < nv + 4) tile[j] = cand ? mine : ~0ull;
+    if (j < nv + 4) tile[j] = cand ? ((uint64_t)ordered_key(-d) << 32) | (uint32_t)j : ~0ull;
     if (j < 4 && nv + j >= nt) tile[nv + j] = ~0ull;
-    __syncthreads();
-    const int p = cand ? count_smaller(tile, nv, mine) : 0;
+    const int p = position_by_counting(tile, below, nv, j, nt);
     if (cand && p < need) order[worst_start + p] = row;
     if (j < worst_start) order[j] = perm[j];
   }
@@ -277,18 +329,27 @@ __global__ __launch_bounds__(1024) void batched_kernel(BatchedArgs a) {
   if (a.x != nullptr) {
     const uint8_t* __restrict__ xb = a.x + (int64_t)blockIdx.x * a.x_stride_b;
     uint8_t* __restrict__ dst = a.out_x + ob * a.x_row_bytes;
-    const int waves = nt >> 6;
-    for (int p = wave; p < topk; p += waves) {
-      const uint8_t* __restrict__ s = xb + (int64_t)order[p] * a.x_row_stride;
-      uint8_t* __restrict__ dp = dst + (int64_t)p * a.x_row_bytes;
-      if (a.x_unit == 16) {
-        for (int64_t b = lane * 16; b < a.x_row_bytes; b += 64 * 16)
-          *reinterpret_cast<uint4*>(dp + b) = *reinterpret_cast<const uint4*>(s + b);
-      } else if (a.x_unit == 4) {
-        for (int64_t b = lane * 4; b < a.x_row_bytes; b += 64 * 4)
-          *reinterpret_cast<uint32_t*>(dp + b) = *reinterpret_cast<const uint32_t*>(s + b);
-      } else {
-        for (int64_t b = lane; b < a.x_row_bytes; b += 64) dp[b] = s[b];
+    const int64_t row_units = a.x_row_bytes / a.x_unit;
+    const int64_t total = row_units * topk;
+    if (a.x_unit >= 4 && total < (1ll << 31)) {
+      if (a.x_unit == 16)
+        gather_units<uint4>(xb, dst, order, a.x_row_stride, (uint32_t)row_units, (uint32_t)total, j, nt);
+      else
+        gather_units<uint32_t>(xb, dst, order, a.x_row_stride, (uint32_t)row_units, (uint32_t)total, j, nt);
+    } else {
+      const int waves = nt >> 6;
+      for (int p = wave; p < topk; p += waves) {
+        const uint8_t* __restrict__ sp = xb + (int64_t)order[p] * a.x_row_stride;
+        uint8_t* __restrict__ dp = dst + (int64_t)p * a.x_row_bytes;
+        if (a.x_unit == 16) {
+          for (int64_t b = lane * 16; b < a.x_row_bytes; b += 64 * 16)
+            *reinterpret_cast<uint4*>(dp + b) = *reinterpret_cast<const uint4*>(sp + b);
+        } else if (a.x_unit == 4) {
+          for (int64_t b = lane * 4; b < a.x_row_bytes; b += 64 * 4)
+            *reinterpret_cast<uint32_t*>(dp + b) = *reinterpret_cast<const uint32_t*>(sp + b);
+        } else {
+          for (int64_t b = lane; b < a.x_row_bytes; b += 64) dp[b] = sp[b];
+        }
       }
     }
   }
