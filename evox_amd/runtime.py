@@ -14,10 +14,10 @@ _last: Optional[Tuple[torch.Tensor, int]] = None  # (workspace, stream handle) o
 CHECK_STATUS = os.environ.get("EVOX_AMD_CHECK_STATUS", "0") not in ("", "0")
 
 # Populations of at most evox_hip_batched_max_rows(m) rows can run in the one-workgroup-per-population
-# kernel, larger ones need the bit-matrix pipeline.  None = choose by size (a lone population above
-# 576 rows is faster in the pipeline, which spreads it over the whole device; measured: 84 against
-# 106 us at 512 rows, 227 against 113 us at 1024 rows); True / False force the choice where it is
-# possible (tests use that to drive small inputs through both).
+# kernel, larger ones need the bit-matrix pipeline.  None = choose by size (a lone population of more
+# than 960 rows is faster in the pipeline, which spreads it over the whole device; measured: 55 against
+# 105 us at 576 rows, 96 against 104 us at 960 rows, 114 against 111 us at 1024 rows); True / False
+# force the choice where it is possible (tests use that to drive small inputs through both).
 use_small_population_kernel = None
 
 
@@ -28,7 +28,7 @@ def small_population_kernel_fits(n: int, m: int, batch: int) -> bool:
         return False
     if use_small_population_kernel is True:
         return True
-    return n <= 576 or batch >= 3
+    return n <= 960 or batch >= 2
 
 
 def require_gpu_tensor(t: torch.Tensor, what: str) -> None:
