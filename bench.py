@@ -332,8 +332,10 @@ def main():
     dom_bytes = n * m * 4 + int(row_read.sum())
     slots = torch.arange(n, device=rank.device)
     evaluated_pairs = float(((((slots >> 6) << 6) + 63) // 256 * 256 + 256).clamp(max=nwords * 64).sum())
-    # finite populations take the arithmetic form: m subtractions, (m - 1) ORs three at a time, clamp, shift-in,
-    # all issued at the full vector rate; others the compare form: m + 2 mask-writing instructions
+    # finite populations take the arithmetic form: m subtractions (scalar operand), (m - 1) ORs three at a time,
+    # clamp, shift-in; others the compare form: m + 2 mask-writing instructions.  Measured alone, two-operand
+    # vector-register instructions issue at about 50 T lane-ops/s and three-operand, min/max and scalar-operand
+    # ones at about 32 T; mixed as in the arithmetic form they sustain about 52 T (calibration kind 3)
     finite = bool(torch.isfinite(f).all())
     valu_per_pair = m + (m // 2) + 2 if finite else m + 2
     executed_valu = valu_per_pair * evaluated_pairs
