@@ -401,6 +401,44 @@ def test_c4_full_batch_one_launch():
         runtime.use_small_population_kernel = keep
 
 
+@pytest.mark.parametrize("n,m", [(33, 1), (64, 2), (95, 3), (130, 4), (257, 5), (500, 6), (777, 7), (1024, 8), (1000, 3)])
+def test_batched_selection_shapes_layouts_and_row_units(n, m, population_path):
+    """The one-workgroup kernel over ragged sizes, every objective count, packed and strided fitness (its
+    dominator loads take different paths), non-finite values (the compare form) and rows of x whose size
+    allows 16-byte, 4-byte or single-byte units; every population against the CPU restatement."""
+    if population_path != "small-kernel":
+        pytest.skip("about the one-workgroup kernel")
+    say("batched_shapes", n, m)
+    g = torch.Generator("cpu").manual_seed(100 * n + m)
+    batch, topk = 3, max(1, n // 3)
+    f = torch.rand(batch, n, m, generator=g)
+    f[0, : n // 4] = (f[0, : n // 4] * 4).round() / 4        # ties and duplicate rows
+    f[1, 1] = f[1, 0]
+    f_strided = f.transpose(1, 2).contiguous().transpose(1, 2)  # same values, objective-major memory
+    f_bad = f.clone()
+    f_bad[2, 0, 0] = float("nan")
+    f_bad[2, n - 1, m - 1] = float("inf")
+    f_bad[1, n // 2, 0] = -float("inf")
+    xs = [torch.rand(batch, n, 8, generator=g),                                  # 32-byte rows: 16-byte units
+          torch.rand(batch, n, 5, generator=g),                                  # 20-byte rows: 4-byte units
+          torch.randint(0, 255, (batch, n, 7), generator=g, dtype=torch.uint8),  # 7-byte rows: single bytes
+          torch.rand(batch, n, 300, generator=g)]                                # several units per lane and row
+    for fit in (f, f_strided, f_bad):
+        assert m == 1 or fit.is_contiguous() == (fit is not f_strided)
+        want = [er.environmental_selection(fit[b], fit[b], topk, return_all=True) for b in range(batch)]
+        ranks = non_dominate_rank(fit.to(DEV))
+        for b in range(batch):
+            assert np.array_equal(as_np(ranks[b]), as_np(want[b][1])), b
+        for x in xs:
+            ox, of, orank, odist = nd_environmental_selection(x.to(DEV), fit.to(DEV), topk)
+            for b in range(batch):
+                order = as_np(want[b][3])
+                assert np.array_equal(as_np(ox[b]), as_np(x[b])[order]), (b, tuple(x.shape))
+                assert np.array_equal(as_np(of[b]), as_np(fit[b])[order], equal_nan=True), b
+                assert np.array_equal(as_np(orank[b]), as_np(want[b][0][2])), b
+                assert_dist_close(odist[b], as_np(want[b][0][3]))
+
+
 def test_selection_x_dtypes_and_shapes():
     say("selection_x_dtypes")
     f = workloads.uniform_population(300, 3, 0, 8)[0]
