@@ -439,6 +439,42 @@ def test_batched_selection_shapes_layouts_and_row_units(n, m, population_path):
                 assert_dist_close(odist[b], as_np(want[b][0][3]))
 
 
+@pytest.mark.parametrize("n,m,d,topk", [(200, 3, 30, 100), (5000, 3, 16, 2500)])
+def test_selection_captured_in_a_graph_replays_correctly(n, m, d, topk, population_path):
+    """The whole selection (no allocation by the library, no host synchronisation, state cleared by kernels)
+    can be captured in a HIP graph; every replay, with eager calls in between, must equal the eager result."""
+    if population_path == "small-kernel" and n > 1024:
+        pytest.skip("population too large for the one-workgroup kernel")
+    say("graph", n, m, population_path)
+    g = torch.Generator("cpu").manual_seed(n)
+    fs = [torch.rand(n, m, generator=g) for _ in range(3)]
+    xs = [torch.rand(n, d, generator=g) for _ in range(3)]
+    f_static, x_static = fs[0].to(DEV).clone(), xs[0].to(DEV).clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on a side stream, as torch asks before a capture
+        for _ in range(2):
+            nd_environmental_selection(x_static, f_static, topk)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = nd_environmental_selection(x_static, f_static, topk)
+    for rep in range(5):
+        i = rep % 3
+        f_static.copy_(fs[i].to(DEV))
+        x_static.copy_(xs[i].to(DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in out]
+        want = nd_environmental_selection(xs[i].to(DEV), fs[i].to(DEV), topk)  # eager work between the replays
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert np.array_equal(as_np(a), as_np(b), equal_nan=a.dtype.is_floating_point), rep
+    del graph
+    runtime.release_workspaces()  # the workspace of the capture stream lives in the graph's private pool
+
+
 def test_selection_x_dtypes_and_shapes():
     say("selection_x_dtypes")
     f = workloads.uniform_population(300, 3, 0, 8)[0]
