@@ -14,6 +14,7 @@ from .operators.selection import (
     crowding_distance,
     nd_environmental_selection,
     non_dominate_rank,
+    tournament_selection,
     tournament_selection_multifit,
 )
 
@@ -35,6 +36,7 @@ _FUNCS = {
     "crowding_distance": crowding_distance,
     "nd_environmental_selection": nd_environmental_selection,
     "tournament_selection_multifit": tournament_selection_multifit,
+    "tournament_selection": tournament_selection,
     "cal_hv": cal_hv,  # only evox.algorithms.mo.hype holds this name
     "hv": hv,  # the function that evox.metrics and evox.metrics.hv hold (src/evox/metrics/__init__.py:4), not the module
 }

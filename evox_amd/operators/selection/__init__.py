@@ -5,6 +5,7 @@ __all__ = [
     "non_dominate_rank",
     "non_dominate_rank_until",
     "non_dominated_mask",
+    "tournament_selection",
     "tournament_selection_multifit",
 ]
 
@@ -16,4 +17,4 @@ from .non_dominate import (
     non_dominate_rank_until,
     non_dominated_mask,
 )
-from .tournament_selection import tournament_selection_multifit
+from .tournament_selection import tournament_selection, tournament_selection_multifit

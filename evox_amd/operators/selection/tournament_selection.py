@@ -1,6 +1,7 @@
-"""Drop-in replacement for ``evox.operators.selection.tournament_selection_multifit``
+"""Drop-in replacements for ``evox.operators.selection.tournament_selection_multifit``
 (src/evox/operators/selection/tournament_selection.py:8-29), the consumer of the rank and crowding
-distance that ``nd_environmental_selection`` returns (src/evox/algorithms/mo/nsga2.py:94).
+distance that ``nd_environmental_selection`` returns (src/evox/algorithms/mo/nsga2.py:94), and for its
+single-fitness sibling ``tournament_selection`` (tournament_selection.py:32-54).
 """
 
 from typing import List
@@ -22,3 +23,14 @@ def tournament_selection_multifit(n_round: int, fitnesses: List[torch.Tensor], t
     num_candidates = fitness_tensor.size(0)
     parents = torch.randint(0, num_candidates, (n_round, tournament_size), device=fitnesses[0].device)
     return ops.tournament_pick(parents, fitness_tensor).squeeze()
+
+
+def tournament_selection(n_round: int, fitness: torch.Tensor, tournament_size: int = 2) -> torch.Tensor:
+    """Indices of the winners of ``n_round`` random tournaments on one fitness tensor: the candidate of
+    least fitness, the first of them on ties, and -- as ``torch.argmin`` has it (tournament_selection.py:50) --
+    a NaN before every number.  Candidates are drawn as the reference draws them (:47)."""
+    num_candidates = fitness.size(0)
+    parents = torch.randint(0, num_candidates, (n_round, tournament_size), device=fitness.device)
+    # the kernel orders by the last column first and puts NaN last: "is a number" as the last column puts NaN first
+    keys = torch.stack([fitness, (~torch.isnan(fitness)).to(fitness.dtype)], dim=1)
+    return ops.tournament_pick(parents, keys).squeeze()

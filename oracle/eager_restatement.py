@@ -147,6 +147,14 @@ def tournament_winners(parents: torch.Tensor, fitnesses: List[torch.Tensor]) -> 
     return torch.gather(parents, 1, ordering[:, 0].unsqueeze(1)).squeeze()
 
 
+def tournament_winners_single(parents: torch.Tensor, fitness: torch.Tensor) -> torch.Tensor:
+    """Winner of each row of ``parents`` (n_round, t) on one fitness tensor: tournament_selection.py:48-54
+    without the random draw (:47)."""
+    candidates_fitness = fitness[parents]
+    winner_indices = torch.argmin(candidates_fitness, dim=1)
+    return torch.gather(parents, 1, winner_indices.unsqueeze(1)).squeeze()
+
+
 def first_front_mask(f: torch.Tensor) -> torch.Tensor:
     """bool (N,): the rows that EvalMonitor.get_pf_fitness / get_pf keep (eval_monitor.py:301-302, :333-335):
     the whole history is ranked and only ``rank == 0`` is used."""

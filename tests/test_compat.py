@@ -30,7 +30,9 @@ def _fake_evox():
         for f in ("non_dominate_rank", "crowding_distance", "nd_environmental_selection"):
             setattr(mods[n], f, original)
     mods["evox.operators.selection.tournament_selection"].tournament_selection_multifit = original
+    mods["evox.operators.selection.tournament_selection"].tournament_selection = original
     mods["evox.operators.selection"].tournament_selection_multifit = original
+    mods["evox.operators.selection"].tournament_selection = original  # the function shadows the sub-module (__init__.py:14)
     mods["evox.operators"].non_dominate_rank = original
     mods["evox.operators"].crowding_distance = original
     mods["evox.algorithms.mo.nsga2"].nd_environmental_selection = original
@@ -58,10 +60,11 @@ def test_install_rebinds_every_early_bound_name(monkeypatch):
         assert mods[n].non_dominate_rank is hip_selection.non_dominate_rank, n
     assert mods["evox.operators.selection"].crowding_distance is hip_selection.crowding_distance
     assert mods["evox.algorithms.mo.hype"].cal_hv is evox_amd.hype.cal_hv
+    assert mods["evox.operators.selection"].tournament_selection is hip_selection.tournament_selection
     assert mods["evox.workflows.eval_monitor"].unrelated is original  # nothing else is touched
     assert mods["evox.metrics"].hv is evox_amd.metrics.hv and mods["evox.metrics.hv"].hv is evox_amd.metrics.hv
     assert isinstance(mods["evox.metrics"].igd, types.ModuleType)  # sub-modules stay what they are
-    assert "evox.algorithms.mo.nsga2.nd_environmental_selection" in changed and len(changed) == 19
+    assert "evox.algorithms.mo.nsga2.nd_environmental_selection" in changed and len(changed) == 21
 
 
 def test_install_without_evox_changes_nothing():

@@ -1054,6 +1054,27 @@ def test_tournament_selection_multifit_follows_the_generator(population_path):
     assert torch.equal(compiled(parents, table), ops_tournament(parents, table))
 
 
+def test_tournament_selection_single_fitness(population_path):
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd.operators.selection import tournament_selection
+
+    say("tournament_single")
+    g = torch.Generator("cpu").manual_seed(41)
+    fit = torch.randint(0, 50, (500,), generator=g).float() / 4
+    fit[torch.rand(500, generator=g) < 0.1] = float("nan")
+    fit[torch.rand(500, generator=g) < 0.05] = -float("inf")
+    fit[torch.rand(500, generator=g) < 0.05] = -0.0
+    fd = fit.to(DEV)
+    for n_round, tsize in ((1000, 2), (1, 2), (333, 5)):
+        torch.manual_seed(77)
+        got = tournament_selection(n_round, fd, tsize)
+        torch.manual_seed(77)
+        parents = torch.randint(0, 500, (n_round, tsize), device=DEV)
+        want = er.tournament_winners_single(parents.cpu(), fit)
+        assert got.shape == want.shape and got.dtype == torch.int64 and torch.equal(got.cpu(), want)
+
+
 def ops_tournament(parents, table):
     from evox_amd import ops
 

@@ -283,6 +283,23 @@ def test_tournament_matches_tuple_comparison(tsize):
             assert want[r] == row[first]
 
 
+def test_single_fitness_tournament_is_first_least_with_nan_first():
+    g = torch.Generator("cpu").manual_seed(31)
+    fit = torch.randint(0, 5, (40,), generator=g).float()
+    fit[torch.rand(40, generator=g) < 0.2] = float("nan")
+    fit[torch.rand(40, generator=g) < 0.1] = -0.0
+    parents = torch.randint(0, 40, (300, 3), generator=g)
+    got = er.tournament_winners_single(parents, fit)
+    for r in range(300):
+        vals = [float(fit[c]) for c in parents[r]]
+        nan_at = [t for t, v in enumerate(vals) if v != v]
+        t_best = nan_at[0] if nan_at else min(range(3), key=lambda t: (vals[t], t))
+        assert int(got[r]) == int(parents[r, t_best]), r
+    # the same winners from the multi-key ordering with "is a number" as the primary key
+    keys = [fit, (~torch.isnan(fit)).float()]
+    assert torch.equal(er.tournament_winners(parents, keys), got)
+
+
 def test_tournament_hand_worked():
     neg_dist = torch.tensor([-1.0, -2.0, -float("inf"), float("inf"), float("nan"), 0.0, -0.0])
     rank = torch.tensor([0, 0, 1, 0, 0, 1, 1], dtype=torch.int32)
