@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the environmental-selection hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3|C2|C1|C5] [--no-cpu] [--next-rows]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3|C2|C1|C4|C5] [--no-cpu] [--next-rows]
 
 One step = one `nd_environmental_selection` call on the workload (default C3: N=20000, M=3,
 D=100, topk=10000, fitness i.i.d. U[0,1) from seed 0), inputs and outputs resident in HBM.
@@ -41,7 +41,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C5"])
+    ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--cpu-sample", type=int, default=16000, help="rows of the workload timed on the CPU")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -274,6 +274,76 @@ def next_rows(dev, reps):
     return out
 
 
+def batched_line(args, dev):
+    """C4: 1024 populations of 512 rows in one call of the one-workgroup-per-population kernel.  There are no
+    stages to time apart: the line carries the whole kernel, against the vector unit's issue rate."""
+    from evox_amd import workloads
+    from evox_amd.operators.selection import nd_environmental_selection
+
+    w = workloads.c4()
+    f = w.f.to(dev)
+    batch, n, m = f.shape
+    x = torch.rand(batch, n, 30, generator=torch.Generator("cpu").manual_seed(w.seed)).to(dev)
+
+    def step():
+        return nd_environmental_selection(x, f, w.topk)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    # kernel time by HIP events around back-to-back launches through the C ABI on the launch stream (a ctypes call
+    # costs a few microseconds, so the launches queue up and the interval per launch is the kernel's duration)
+    from evox_amd import _lib, runtime
+
+    ox, of, orank, odist = step()
+    stream = runtime.stream_handle(dev)
+
+    def launch():
+        _lib.call("evox_hip_batched_nd_environmental_selection", x.data_ptr(), x.size(2) * 4, x.stride(1) * 4, x.stride(0) * 4,
+                  f.data_ptr(), batch, n, m, f.stride(0), f.stride(1), f.stride(2), w.topk, ox.data_ptr(), of.data_ptr(),
+                  orank.data_ptr(), odist.data_ptr(), stream)
+
+    kernel_us = event_time_us(launch, max(5, min(args.steps, 30)), inner=8)
+    pairs = float(batch) * n * n
+    # every row is tested against all rows of its population (no slot order inside a workgroup):
+    # m subtractions, (m - 1) ORs three at a time, clamp, shift-in per pair
+    executed = (m + m // 2 + 2) * pairs
+    rates = valu_issue_rates(dev)
+    roofline = {"kernel": "batched_kernel", "bound": "valu", "achieved": executed / kernel_us / 1e3,
+                "peak": VALU_FP32_PEAK_GOPS, "unit": "Gop/s", "frac": executed / kernel_us / 1e3 / VALU_FP32_PEAK_GOPS,
+                "traffic": None, "kernel_us": kernel_us, "measured_issue_rates_Gops": rates,
+                "frac_of_measured_rate": executed / kernel_us / 1e3 / rates["arithmetic_form_unit_m3"]}
+    out = {
+        "metric": "dominance comparisons/sec through nd_environmental_selection (N^2 ordered pairs per population and step)",
+        "value": pairs / (ms_per_step * 1e-3), "unit": "comparisons/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"C4: nd_environmental_selection of {batch} populations, N={n} M={m} D=30 topk={w.topk} "
+                               f"each, one launch, seed {w.seed}"},
+        "latency_ms": ms_per_step, "roofline": roofline,
+    }
+    if not args.no_cpu:
+        from oracle import eager_restatement as er
+
+        sample = batch  # the whole workload: a few seconds of CPU work
+        torch.set_num_threads(os.cpu_count() or 1)
+        t0 = time.perf_counter()
+        for b in range(sample):
+            er.environmental_selection(x[b].cpu(), w.f[b], w.topk)
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": sample * n * n / dt, "unit": "comparisons/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "seconds": dt,
+                               "sample": f"first {sample} populations of C4, one nd_environmental_selection call each, "
+                                         f"{dt:.2f} s; torch-CPU restatement of the reference's eager path"}
+        out["speedup_vs_cpu_baseline"] = out["value"] / out["cpu_baseline"]["value"]
+    print(json.dumps(out))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -287,8 +357,11 @@ def main():
     from evox_amd import workloads
     from evox_amd.operators.selection import nd_environmental_selection
 
-    w = {"C1": workloads.c1, "C2": workloads.c2, "C3": workloads.c3, "C5": workloads.c5}[args.workload]()
     dev = torch.device("cuda", 0)
+    if args.workload == "C4":
+        batched_line(args, dev)
+        return
+    w = {"C1": workloads.c1, "C2": workloads.c2, "C3": workloads.c3, "C5": workloads.c5}[args.workload]()
     f = w.f.to(dev)
     x = (w.x if w.x is not None else w.f).to(dev)
     n, m = f.shape
