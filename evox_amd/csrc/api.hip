@@ -405,12 +405,15 @@ template <int M>
 static int launch_batched_m(const BatchedArgs& a, int64_t batch, hipStream_t s) {
   const int nt = (int)round_up(a.n, 64);
   const size_t lds = batched_lds_bytes(nt);
-  static size_t granted = 0;
-  if (lds > 48 * 1024 && lds > granted) {
+  // the attribute belongs to the (kernel, device) pair: remembered per device
+  static size_t granted[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+  if (lds > 48 * 1024 && (dev < 0 || lds > granted[dev])) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(batched_kernel<M>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
-    granted = lds;
+    if (dev >= 0) granted[dev] = lds;
   }
   // grid.x carries the batch; very large batches go in slices
   for (int64_t b0 = 0; b0 < batch; b0 += 0x40000000ll) {
