@@ -682,7 +682,7 @@ def test_record_protocol_with_other_block_counts():
             assert np.array_equal(as_np(non_dominate_rank(f.to(DEV))), want), blocks
             assert runtime.last_status()["error"] == 0
     finally:
-        runtime.set_option("peel_record_blocks", 128)
+        runtime.set_option("peel_record_blocks", 0)
 
 
 # ------------------------------------------------------------------ ranks up to the cut front only
