@@ -28,6 +28,7 @@ struct Options {
   int peel_records = 1;  // record protocol (all-to-all, no master) for populations up to kRecordsMaxRows
   unsigned spin_limit = 4000000u;
   int dominance_tile_words = 4;
+  int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
 };
 static Options g_opt;
 
@@ -196,6 +197,14 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
   const Layout& L = w.L;
   if (src.f == nullptr || src.f2 == nullptr || src.n_first < 0 || src.n_first > L.n) return kErrBadArg;
   const int64_t zero_words = (int64_t)((L.zero_end - L.ctrl) / 4);
+  if (with_sort && L.n <= kSmallSortRows && (int64_t)L.n * L.m <= kSmallSortValues && g_opt.small_sort) {
+    hipLaunchKernelGGL(small_sort_kernel, dim3(L.npad / kSmallSortGroup), dim3(kSmallSortThreads), sizeof(double) * (size_t)L.npad, s, src.f,
+                       src.sr, src.sc, (int)src.n_first, src.f2, src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs),
+                       w.at<SortParam>(L.sortparam), w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted),
+                       w.at<float>(L.xs_sorted), w.at<int>(L.orig_of), w.at<uint32_t>(L.ctrl), zero_words);
+    EVX_LAUNCH_CHECK();
+    return 0;
+  }
   hipLaunchKernelGGL(prepare_kernel, dim3(L.prep_blocks), dim3(256), 0, s, src.f, src.sr, src.sc, (int)src.n_first, src.f2,
                      src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs), w.at<uint64_t>(L.key),
                      w.at<unsigned long long>(L.partials), w.at<uint32_t>(L.ctrl), zero_words);
@@ -493,6 +502,8 @@ int evox_hip_set_option(const char* name, int64_t value) {
     g_opt.spin_limit = (unsigned)value;
   } else if (!strcmp(name, "dominance_tile_words") && (value == 4 || value == 8 || value == 16)) {
     g_opt.dominance_tile_words = (int)value;
+  } else if (!strcmp(name, "small_sort") && (value == 0 || value == 1)) {
+    g_opt.small_sort = (int)value;
   } else {
     return kErrBadArg;
   }

@@ -97,6 +97,162 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
   for (int64_t i = tid; i < n_zero_words; i += nthreads) zero_words[i] = 0u;
 }
 
+// Populations of at most kSmallSortRows rows: prepare_kernel and the four kernels of the bucket sort in one
+// launch, with no dependence between workgroups.  Every workgroup computes the keys of all rows into LDS as
+// composites (key << 12 | original index; keys are below 2^35 and indices below 2^12), then places its own
+// sixteen rows by counting: the count of a row is split over the four quarters of a wave's lanes and the
+// sixteen waves, each part counting over a sixty-fourth of the composites, and the first wave adds the
+// shares up (a few thousand rows thus spread over the whole device: 10 against 20 us at 4096 x 3, 7 against
+// 19 us at 2000 x 2).  slot = number of smaller
+// composites, kid = number of smaller keys = first slot that holds the key; the outputs are those of
+// prepare_kernel (xs, the state cleared) and of bucket_place_kernel (slot-ordered arrays, NaN / all-ones / -1
+// padding up to npad), and the flag that says whether a NaN or an infinity was met.
+constexpr int kSmallSortRows = 4096;
+constexpr int kSmallSortValues = 28672;  // and at most this many fitness values (every workgroup reads all of them:
+                                         // measured 14.8 against 21.3 us at 4096 x 7, 22.7 against 21.8 us at 4096 x 8)
+constexpr int kSmallSortThreads = 1024;
+constexpr int kSmallSortGroup = 16;  // rows placed by one workgroup
+
+__global__ __launch_bounds__(kSmallSortThreads) void small_sort_kernel(
+    const float* __restrict__ f, int64_t stride_row, int64_t stride_col, int n_first, const float* __restrict__ f2,
+    int64_t stride_row2, int64_t stride_col2, int n, int m, int npad, float* __restrict__ xs, SortParam* __restrict__ param_out,
+    uint64_t* __restrict__ key_sorted, uint32_t* __restrict__ kid_sorted, float* __restrict__ xs_sorted, int* __restrict__ orig_of,
+    uint32_t* __restrict__ zero_words, int64_t n_zero_words) {
+  // npad composites, held as doubles (they are below 2^47, so exact): the hardware compares doubles at the
+  // rate of 32-bit values, 64-bit integers several times slower; +inf for the padding rows
+  extern __shared__ double comp[];
+  __shared__ int share[2][16 * (64 / kSmallSortGroup)][kSmallSortGroup];
+  const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;
+  auto value = [&](int i, int k) {
+    return i < n_first ? f[(int64_t)i * stride_row + k * stride_col] : f2[(int64_t)(i - n_first) * stride_row2 + k * stride_col2];
+  };
+  bool bad = false;
+  {
+    // every row of the population, kRowsPerThread per thread; the loads of one objective for all of a thread's
+    // rows are independent and in flight together (a load per row and round trip would cost a memory latency
+    // per 1024 rows)
+    constexpr int kRowsPerThread = (kSmallSortRows + 127) / kSmallSortThreads + 1;
+    uint64_t sum[kRowsPerThread];
+#pragma unroll
+    for (int t = 0; t < kRowsPerThread; ++t) sum[t] = 0;
+    // rows of m consecutive floats are read four values at a time (the compiler merges them into one 16-byte
+    // load per lane: with a separate load per objective every lane would use 4 bytes of each 32-byte sector)
+    const bool packed = stride_col == 1 && stride_row == m && stride_col2 == 1 && stride_row2 == m;
+    int k0 = 0;
+    if (packed) {
+      for (; k0 + 4 <= m; k0 += 4) {
+        float v[kRowsPerThread][4];
+#pragma unroll
+        for (int t = 0; t < kRowsPerThread; ++t) {
+          const int i = (int)threadIdx.x + t * kSmallSortThreads;
+          const float* __restrict__ p = i < n_first ? f + (int64_t)i * m + k0 : f2 + (int64_t)(i - n_first) * m + k0;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) v[t][u] = i < n ? p[u] : 0.0f;
+        }
+#pragma unroll
+        for (int t = 0; t < kRowsPerThread; ++t)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            sum[t] += ordered_key(v[t][u]);
+            bad |= !(fabsf(v[t][u]) <= 3.4028234663852886e38f);  // NaN or infinite
+          }
+      }
+    }
+    for (int k = k0; k < m; ++k) {
+      float v[kRowsPerThread];
+#pragma unroll
+      for (int t = 0; t < kRowsPerThread; ++t) {
+        const int i = (int)threadIdx.x + t * kSmallSortThreads;
+        v[t] = i < n ? value(i, k) : 0.0f;
+      }
+#pragma unroll
+      for (int t = 0; t < kRowsPerThread; ++t) {
+        sum[t] += ordered_key(v[t]);
+        bad |= !(fabsf(v[t]) <= 3.4028234663852886e38f);  // NaN or infinite
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < kRowsPerThread; ++t) {
+      const int i = (int)threadIdx.x + t * kSmallSortThreads;
+      if (i < npad) comp[i] = i < n ? (double)((sum[t] << 12) | (uint64_t)i) : (double)INFINITY;
+    }
+  }
+  const int any_bad = __syncthreads_or(bad);  // also the barrier after the composites
+  // kSmallSortGroup rows per workgroup (so that a few thousand rows spread over the whole device); a row's count
+  // is split over 64 parts: the four sixteenths of a wave's lanes times the sixteen waves
+  const int row_in_group = lane & (kSmallSortGroup - 1);
+  const int split = part * (64 / kSmallSortGroup) + lane / kSmallSortGroup;
+  constexpr int kParts = 16 * (64 / kSmallSortGroup);
+  for (int r0 = blockIdx.x * kSmallSortGroup; r0 < npad; r0 += gridDim.x * kSmallSortGroup) {
+    const int i = r0 + row_in_group;  // below npad: npad is a multiple of 128
+    const double mine = comp[i];
+    const double floor = mine - (double)(i & 0xFFF);  // the smallest composite of this key (unused for padding rows)
+    // this part's share of the composites, in pairs (16-byte LDS reads)
+    const int per = (((n + kParts - 1) / kParts) + 1) & ~1;
+    const int e0 = split * per;
+    const int e1 = min(e0 + per, (n + 1) & ~1);  // an odd n reads one composite of the padding: +inf
+    int before = 0, smaller = 0;
+#pragma unroll 8
+    for (int e = e0; e < e1; e += 2) {
+      const double2 c = *reinterpret_cast<const double2*>(comp + e);
+      before += (c.x < mine) + (c.y < mine);
+      smaller += (c.x < floor) + (c.y < floor);
+    }
+    share[0][split][row_in_group] = before;
+    share[1][split][row_in_group] = smaller;
+    __syncthreads();
+    if (part == 0) {
+      // lane = (row, quarter of the parts); the quarters are added across the lanes
+      before = 0;
+      smaller = 0;
+      const int q0 = (lane / kSmallSortGroup) * (kParts / (64 / kSmallSortGroup));
+#pragma unroll
+      for (int p = 0; p < kParts / (64 / kSmallSortGroup); ++p) {
+        before += share[0][q0 + p][row_in_group];
+        smaller += share[1][q0 + p][row_in_group];
+      }
+#pragma unroll
+      for (int off = kSmallSortGroup; off < 64; off <<= 1) {
+        before += __shfl_xor(before, off);
+        smaller += __shfl_xor(smaller, off);
+      }
+      if (lane < kSmallSortGroup) {
+        if (i < n) {
+          orig_of[before] = i;
+          key_sorted[before] = (uint64_t)mine >> 12;
+          kid_sorted[before] = (uint32_t)smaller;
+          for (int k = 0; k < m; ++k) {
+            const float v = value(i, k);
+            xs[(int64_t)k * npad + i] = v;
+            // -0.0 is stored as +0.0: every comparison reads the same, and differences of equal values are +0.0
+            xs_sorted[(int64_t)k * npad + before] = v + 0.0f;
+          }
+        } else {
+          orig_of[i] = -1;
+          key_sorted[i] = ~0ull;
+          kid_sorted[i] = (uint32_t)i;
+          for (int k = 0; k < m; ++k) {
+            xs[(int64_t)k * npad + i] = __uint_as_float(0x7FC00000u);
+            xs_sorted[(int64_t)k * npad + i] = __uint_as_float(0x7FC00000u);
+          }
+        }
+      }
+    }
+    __syncthreads();  // the shares are rewritten by the next row group
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    SortParam sp;
+    sp.kmin = 0ull;
+    sp.shift = 0;
+    sp.buckets = 0;
+    sp.nonfinite = any_bad != 0;
+    sp.reserved = 0;
+    *param_out = sp;
+  }
+  const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (int64_t w = tid; w < n_zero_words; w += (int64_t)gridDim.x * blockDim.x) zero_words[w] = 0u;
+}
+
 enum DomVariant { kDomAuto = 0, kDomTwoCompares = 1, kDomKey64 = 2, kDomKey32 = 3, kDomArith = 4 };
 
 // acc = (acc << 1) | bit, with the bit taken from a 64-lane mask: one v_addc_co_u32.
