@@ -992,6 +992,11 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
     const uint64_t all = lo + 64 <= n ? ~0ull : (lo >= n ? 0ull : ((1ull << (n - lo)) - 1ull));
     alive_lds[w] = all & ~coherent_load(&fronts_slot[(int64_t)w * kFrontStride]);  // minus front 0 (buffer 0)
   }
+  // The counters of a pass live in sh[4 p .. 4 p + 3], p = the parity of the pass: [0] rows this block ranks,
+  // [1] rows all blocks rank, [2] bit 0: some block overflowed its record, bit 1: give up, [3] rows queued
+  // for a rescan.  Those of the next pass are cleared in the middle of this one (between two barriers that
+  // the pass needs anyway), so that a pass neither starts nor ends with a barrier of its own.
+  if (tid < 8) sh[tid] = 0;
   __syncthreads();
   int level = 0;
   int ranked = 0;  // rows in fronts 0 .. level-1
@@ -1003,17 +1008,12 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
     c.next_slot = fronts_slot + (int64_t)(level % kFrontBuffers) * nwords * kFrontStride;
     c.next_orig = fronts_orig + (int64_t)(level % kFrontBuffers) * nwords * kFrontStride;
     c.next_level = level;
-    if (tid == 0) {
-      sh[0] = 0;  // rows this block ranks in the pass
-      sh[1] = 0;  // rows all blocks rank
-      sh[2] = 0;  // bit 0: some block overflowed its record, bit 1: give up
-      sh[3] = 0;  // rows queued for a rescan
-    }
-    lds_barrier();
+    int* const cnts = sh + 4 * (level & 1);
+    int* const next_cnts = sh + 4 * ((level + 1) & 1);
     EVX_TRACE(level - 1, 0);
-    witness_rows_pooled(st, c, alive_lds, first_row, row_step, &sh[3], q_row, q_word, q_bits, list_capacity, [&](int slot, int orig) {
+    witness_rows_pooled(st, c, alive_lds, first_row, row_step, &cnts[3], q_row, q_word, q_bits, list_capacity, [&](int slot, int orig) {
       rank[orig] = level;
-      const int k = atomicAdd(&sh[0], 1);
+      const int k = atomicAdd(&cnts[0], 1);
       if (k < list_capacity) {
         found[2 * k] = slot;
         found[2 * k + 1] = orig;
@@ -1021,7 +1021,8 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
     });
     lds_barrier();  // the list of ranked rows is complete (the rank stores need not be)
     EVX_TRACE(level - 1, 1);
-    const int cnt = sh[0];
+    const int cnt = cnts[0];
+    if (tid < 4) next_cnts[tid] = 0;  // last read before the barrier above, first used after the one below
     unsigned long long* mine = records + (size_t)(gen % kRecRing) * kRecUnits + (size_t)sb * units;
     if (cnt <= record_capacity(units)) {
       if (tid < units) coherent_store(&mine[tid], record_unit_for(gen, tid, found, cnt, false));
@@ -1043,30 +1044,30 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
     EVX_TRACE(level - 1, 3);
     if (!fine) {
       coherent_store(&ctrl->err, kErrBarrierTimeout);
-      atomicOr(&sh[2], 2);
+      atomicOr(&cnts[2], 2);
     } else {
 #pragma unroll
       for (int k = 0; k < kRecLoads; ++k) {
         if (tid + k * kRecThreads >= sweepers * units) continue;  // past the last record
-            const int i = (tid + k * kRecThreads) & (units - 1);
+        const int i = (tid + k * kRecThreads) & (units - 1);
         record_unit_read(
             v[k], i == 0,
             [&](int count, bool overflow) {
-              atomicAdd(&sh[1], count);
-              if (overflow) atomicOr(&sh[2], 1);
+              atomicAdd(&cnts[1], count);
+              if (overflow) atomicOr(&cnts[2], 1);
             },
             [&](int slot) { atomicAnd(reinterpret_cast<unsigned long long*>(&alive_lds[slot >> 6]), ~(1ull << (slot & 63))); });
       }
     }
-    lds_barrier();
-    const int flags = sh[2];
-    size = sh[1];
+    lds_barrier();  // the bitmap of unranked rows and the counters of the pass are complete
+    const int flags = cnts[2];
+    size = cnts[1];
     if (flags & 2) break;
-    if (flags & 1) {
+    if (flags & 1) {  // the same in every thread
       const uint64_t* cur = c.next_slot;
       for (int w = tid; w < nwords; w += blockDim.x) alive_lds[w] &= ~coherent_load(&cur[(int64_t)w * kFrontStride]);
+      lds_barrier();
     }
-    lds_barrier();  // sh is reset at the top of the next pass
   }
 }
 
