@@ -28,6 +28,9 @@
 #ifndef EVX_TRACE
 #define EVX_TRACE(level, slot)
 #endif
+#ifndef EVX_TRACE_POOL
+#define EVX_TRACE_POOL(level, slot)
+#endif
 #ifndef EVX_RESCAN
 #define EVX_RESCAN(level, rows, rounds)
 #endif
@@ -548,6 +551,7 @@ __device__ inline void witness_rows_pooled(WitnessState& st, const PassCtx& c, c
     }
   }
   lds_barrier();
+  EVX_TRACE_POOL(c.next_level - 1, 2);
   const int total = min(*q_n, q_capacity);
   for (int base = wave * 4; base < total; base += waves * 4) {
     const int cnt = min(4, total - base);
@@ -570,6 +574,7 @@ __device__ inline void witness_rows_pooled(WitnessState& st, const PassCtx& c, c
       }
     }
   }
+  EVX_TRACE_POOL(c.next_level - 1, 3);
   lds_barrier();
 #pragma unroll
   for (int ch = 0; ch < kWitnessChunks; ++ch) {
