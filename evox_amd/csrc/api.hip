@@ -661,6 +661,14 @@ int evox_hip_stable_argsort_step(const void* key, int kind, int64_t stride, int6
   if (!make_sort_layout(n, &L)) return kErrBadArg;
   if (ws == nullptr || ws_bytes < L.total || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return kErrWorkspace;
   hipStream_t s = (hipStream_t)stream;
+  if (n <= kSmallArgsortRows) {
+    const int npad = ((int)n + 127) & ~127;
+    if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(small_argsort_kernel), sizeof(double) * (size_t)npad)) return e;
+    hipLaunchKernelGGL(small_argsort_kernel, dim3(npad / kSmallArgsortGroup), dim3(kSmallArgsortThreads),
+                       sizeof(double) * (size_t)npad, s, key, kind, stride, (int)n, prev_order, order_out);
+    EVX_LAUNCH_CHECK();
+    return 0;
+  }
   uint8_t* base = static_cast<uint8_t*>(ws);
   // every call starts from a cleared control block: barrier generations restart
   const int64_t zero_words = (int64_t)((L.pairs0 - L.ctrl) / 4);

@@ -200,4 +200,66 @@ __global__ __launch_bounds__(kRadixThreads) void argsort_step_kernel(const void*
     order_out[p] = (int)(unsigned)(coherent_load(&buf.pairs[0][p]) & 0xFFFFFFFFull);
 }
 
+// The same step for at most kSmallArgsortRows positions in one launch, with no dependence between
+// workgroups: every workgroup builds all composites (key << 14 | position, below 2^46, held as doubles:
+// exact, and compared at the rate of 32-bit values) in LDS and places its own sixteen positions by counting
+// the smaller composites, the count of a position split over 64 parts (the four quarters of a wave's lanes
+// times the sixteen waves).  Same ordering as the radix sort: key ascending, ties by position.
+constexpr int kSmallArgsortRows = 8192;  // measured per step: 30 us up to 8192 positions (radix sort: 90), 75 us at 16384
+constexpr int kSmallArgsortThreads = 1024;
+constexpr int kSmallArgsortGroup = 16;
+
+__global__ __launch_bounds__(kSmallArgsortThreads) void small_argsort_kernel(const void* __restrict__ key, int kind, int64_t stride,
+                                                                             int n, const int* __restrict__ prev,
+                                                                             int* __restrict__ order_out) {
+  extern __shared__ double argsort_comp[];  // n rounded up to a multiple of 128 entries, +inf past n
+  __shared__ int share[16 * (64 / kSmallArgsortGroup)][kSmallArgsortGroup];
+  const int npad = (n + 127) & ~127;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int e = threadIdx.x; e < npad; e += kSmallArgsortThreads) {
+    double c = (double)INFINITY;
+    if (e < n) {
+      const int idx = prev ? prev[e] : e;
+      uint32_t k;
+      if (kind == kKeyFloat32)
+        k = ordered_key(static_cast<const float*>(key)[(int64_t)idx * stride]);
+      else if (kind == kKeyInt32)
+        k = static_cast<const uint32_t*>(key)[(int64_t)idx * stride] ^ 0x80000000u;
+      else
+        k = static_cast<const uint32_t*>(key)[(int64_t)idx * stride];
+      c = (double)(((uint64_t)k << 14) | (uint64_t)e);
+    }
+    argsort_comp[e] = c;
+  }
+  __syncthreads();
+  constexpr int kParts = 16 * (64 / kSmallArgsortGroup);
+  const int in_group = lane & (kSmallArgsortGroup - 1);
+  const int split = wave * (64 / kSmallArgsortGroup) + lane / kSmallArgsortGroup;
+  for (int e0 = blockIdx.x * kSmallArgsortGroup; e0 < npad; e0 += gridDim.x * kSmallArgsortGroup) {
+    const int e = e0 + in_group;
+    const double mine = argsort_comp[e];
+    const int per = (((n + kParts - 1) / kParts) + 1) & ~1;
+    const int b0 = split * per;
+    const int b1 = min(b0 + per, (n + 1) & ~1);  // an odd n reads one entry of the padding: +inf
+    int before = 0;
+#pragma unroll 8
+    for (int b = b0; b < b1; b += 2) {
+      const double2 c = *reinterpret_cast<const double2*>(argsort_comp + b);
+      before += (c.x < mine) + (c.y < mine);
+    }
+    share[split][in_group] = before;
+    __syncthreads();
+    if (wave == 0) {
+      before = 0;
+      const int q0 = (lane / kSmallArgsortGroup) * (kParts / (64 / kSmallArgsortGroup));
+#pragma unroll
+      for (int p = 0; p < kParts / (64 / kSmallArgsortGroup); ++p) before += share[q0 + p][in_group];
+#pragma unroll
+      for (int off = kSmallArgsortGroup; off < 64; off <<= 1) before += __shfl_xor(before, off);
+      if (lane < kSmallArgsortGroup && e < n) order_out[before] = prev ? prev[e] : e;
+    }
+    __syncthreads();
+  }
+}
+
 }  // namespace evx
