@@ -197,7 +197,7 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
   const Layout& L = w.L;
   if (src.f == nullptr || src.f2 == nullptr || src.n_first < 0 || src.n_first > L.n) return kErrBadArg;
   const int64_t zero_words = (int64_t)((L.zero_end - L.ctrl) / 4);
-  if (with_sort && L.n <= kSmallSortRows && (int64_t)L.n * L.m <= kSmallSortValues && g_opt.small_sort) {
+  if (with_sort && L.n <= kSmallSortRows && L.m <= kSmallSortObjectives && (int64_t)L.n * L.m <= kSmallSortValues && g_opt.small_sort) {
     hipLaunchKernelGGL(small_sort_kernel, dim3(L.npad / kSmallSortGroup), dim3(kSmallSortThreads), sizeof(double) * (size_t)L.npad, s, src.f,
                        src.sr, src.sc, (int)src.n_first, src.f2, src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs),
                        w.at<SortParam>(L.sortparam), w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted),

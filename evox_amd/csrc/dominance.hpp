@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
 
 // Populations of at most kSmallSortRows rows: prepare_kernel and the four kernels of the bucket sort in one
 // launch, with no dependence between workgroups.  Every workgroup computes the keys of all rows into LDS as
-// composites (key << 12 | original index; keys are below 2^35 and indices below 2^12), then places its own
+// composites (key << 12 | original index; keys are below 2^40 and indices below 2^12), then places its own
 // sixteen rows by counting: the count of a row is split over the four quarters of a wave's lanes and the
 // sixteen waves, each part counting over a sixty-fourth of the composites, and the first wave adds the
 // shares up (a few thousand rows thus spread over the whole device: 10 against 20 us at 4096 x 3, 7 against
@@ -110,6 +110,7 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
 constexpr int kSmallSortRows = 4096;
 constexpr int kSmallSortValues = 28672;  // and at most this many fitness values (every workgroup reads all of them:
                                          // measured 14.8 against 21.3 us at 4096 x 7, 22.7 against 21.8 us at 4096 x 8)
+constexpr int kSmallSortObjectives = 256;  // keys stay below 2^40, composites below 2^52: exact as doubles
 constexpr int kSmallSortThreads = 1024;
 constexpr int kSmallSortGroup = 16;  // rows placed by one workgroup
 

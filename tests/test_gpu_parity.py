@@ -204,6 +204,8 @@ def test_both_slot_sorts_on_small_and_mid_size_inputs(population_path):
     cases.append(("c2", workloads.c2().f))
     cases.append(("uniform-4096x4", workloads.uniform_population(4096, 4, 0, 21)[0]))
     cases.append(("uniform-4097x2", workloads.uniform_population(4097, 2, 0, 22)[0]))
+    cases.append(("wide-60x200", workloads.uniform_population(60, 200, 0, 23)[0]))   # keys near 2^40
+    cases.append(("wide-40x300", workloads.uniform_population(40, 300, 0, 24)[0]))   # too wide for the one-kernel sort
     try:
         for small_sort in (0, 1):
             runtime.set_option("small_sort", small_sort)
