@@ -220,6 +220,8 @@ __device__ inline void coherent_store(T* p, T v) {
 // needed.  Every wait is bounded by `spin_limit` polls, after which the error flag is set and every
 // role leaves its loop, so all waves always finish.
 constexpr int kFirstSweeper = 2;
+constexpr int kSharedListingRows = 8192;   // a final front 0 of more rows is listed by many blocks
+constexpr int kSharedListingBlocks = 64;
 constexpr int kFrontBuffers = 8;  // front bitmaps in rotation: the lister may lag the sweepers by 6 fronts
 
 template <class Pred>
@@ -587,8 +589,10 @@ __device__ inline void witness_rows_pooled(WitnessState& st, const PassCtx& c, c
 }
 
 // Block-wide listing of the set bits of `front` (nwords words, LDS) in ascending order into
-// perm[base ...].  `scratch` holds at least blockDim.x / 64 ints.
-__device__ inline void list_front(const uint64_t* front_lds, int nwords, int* __restrict__ perm, int base, int* scratch) {
+// perm[base ...]; the words are words first_word ... of the whole bitmap.  `scratch` holds at least
+// blockDim.x / 64 ints.
+__device__ inline void list_front(const uint64_t* front_lds, int nwords, int* __restrict__ perm, int base, int* scratch,
+                                  int first_word = 0) {
   // each thread owns a contiguous slice of words so that the order is ascending
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -612,7 +616,7 @@ __device__ inline void list_front(const uint64_t* front_lds, int nwords, int* __
     uint64_t bits = front_lds[w];
     while (bits) {
       const int b = __ffsll((unsigned long long)bits) - 1;
-      perm[pos++] = w * 64 + b;
+      perm[pos++] = (first_word + w) * 64 + b;
       bits &= bits - 1;
     }
   }
@@ -697,8 +701,11 @@ __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __re
       int size = 0;
       for (int v = 0; v < (int)(blockDim.x >> 6); ++v) size += scratch[32 + v];
       if (threadIdx.x == 0) coherent_store(&ctrl->listed, level);  // fronts 0 .. level-1 are cleared
-      if (perm) list_front(front_lds, nwords, perm, ranked, scratch);
       const bool last = size <= 0 || ranked + size >= stop_count;
+      // a front 0 that ends the peel is listed by the sweepers together (they have nothing else to do, and it
+      // may hold most of a large population)
+      const bool shared_listing = level == 0 && last && size > kSharedListingRows && gridDim.x > kFirstSweeper;
+      if (perm && !shared_listing) list_front(front_lds, nwords, perm, ranked, scratch);
       if (threadIdx.x == 0) {
         fstart[level] = ranked;
         if (level > 0) fsize[level] = size;
@@ -733,7 +740,34 @@ __global__ __launch_bounds__(kPeelThreads) void peel_kernel(const uint64_t* __re
   c.rank = rank;
   WitnessState st;
   int size = coherent_load(&fsize[0]);  // size of front `level`
-  if (size <= 0 || size >= stop_count) return;  // front 0 already holds every row asked for: no pass
+  if (size <= 0 || size >= stop_count) {  // front 0 already holds every row asked for: no pass
+    if (perm && size > kSharedListingRows) {
+      // list it: the first sweeping blocks take a slice of the bitmap (original-index space) each, after adding
+      // up the rows of the words before their slice
+      const int listers = min(sweep_blocks, kSharedListingBlocks);
+      if (sweep_block < listers) {
+        const int per = (nwords + listers - 1) / listers;
+        const int w_begin = min(nwords, sweep_block * per), w_end = min(nwords, w_begin + per);
+        int before = 0;
+        for (int w = threadIdx.x; w < w_end; w += blockDim.x) {
+          const uint64_t fw = coherent_load(&fronts_orig[(int64_t)w * kFrontStride]);
+          if (w < w_begin)
+            before += __popcll(fw);
+          else
+            front_lds[w - w_begin] = fw;
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off);
+        if ((threadIdx.x & 63) == 0) scratch[32 + (threadIdx.x >> 6)] = before;
+        __syncthreads();
+        before = 0;
+        for (int v = 0; v < (int)(blockDim.x >> 6); ++v) before += scratch[32 + v];
+        __syncthreads();
+        list_front(front_lds, w_end - w_begin, perm, before, scratch, w_begin);
+      }
+    }
+    return;
+  }
   if (use_witness) {
     witness_load(st, c, witness, first_row, row_step);
     for (int w = threadIdx.x; w < nwords; w += blockDim.x) {
