@@ -166,6 +166,25 @@ static void launch_dominance(const Ws& w, int variant, hipStream_t s) {
     case 7: launch_dominance_m<7, IW>(w, variant, s); break;
     case 8: launch_dominance_m<8, IW>(w, variant, s); break;
     default: {
+      // nine to sixteen objectives: the register kernel in its production form (tiles of four words, form chosen
+      // on the device); the other tile sizes and the check variants, and more objectives, take the generic kernel
+      if (IW == 4 && variant == kDomAuto && L.m <= 16) {
+        auto wide = [&](auto kernel) {
+          hipLaunchKernelGGL(kernel, dim3((L.npad + 255) / 256, (L.nwords + 3) / 4), dim3(256), 0, s, w.at<float>(L.xs_sorted),
+                             w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad,
+                             L.wstride, L.nwords, w.at<SortParam>(L.sortparam));
+        };
+        switch (L.m) {
+          case 9: wide(dominance_kernel<9, 4, kDomAuto>); return;
+          case 10: wide(dominance_kernel<10, 4, kDomAuto>); return;
+          case 11: wide(dominance_kernel<11, 4, kDomAuto>); return;
+          case 12: wide(dominance_kernel<12, 4, kDomAuto>); return;
+          case 13: wide(dominance_kernel<13, 4, kDomAuto>); return;
+          case 14: wide(dominance_kernel<14, 4, kDomAuto>); return;
+          case 15: wide(dominance_kernel<15, 4, kDomAuto>); return;
+          default: wide(dominance_kernel<16, 4, kDomAuto>); return;
+        }
+      }
       dim3 grid((L.npad + 255) / 256, (L.nwords + IW - 1) / IW);
       hipLaunchKernelGGL((dominance_any_m_kernel<IW>), grid, dim3(256), 0, s, w.at<float>(L.xs_sorted),
                          w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords, L.m);
@@ -597,6 +616,14 @@ int evox_hip_first_front_mask(const float* f, int64_t n, int64_t m, int64_t sr, 
     case 6: launch_first_front<6>(w, mask_out, s); break;
     case 7: launch_first_front<7>(w, mask_out, s); break;
     case 8: launch_first_front<8>(w, mask_out, s); break;
+    case 9: launch_first_front<9>(w, mask_out, s); break;
+    case 10: launch_first_front<10>(w, mask_out, s); break;
+    case 11: launch_first_front<11>(w, mask_out, s); break;
+    case 12: launch_first_front<12>(w, mask_out, s); break;
+    case 13: launch_first_front<13>(w, mask_out, s); break;
+    case 14: launch_first_front<14>(w, mask_out, s); break;
+    case 15: launch_first_front<15>(w, mask_out, s); break;
+    case 16: launch_first_front<16>(w, mask_out, s); break;
     default:
       hipLaunchKernelGGL(first_front_any_m_kernel, dim3((L.n + 255) / 256), dim3(256), 0, s, w.at<float>(L.xs_sorted),
                          w.at<uint32_t>(L.kid_sorted), w.at<int>(L.orig_of), L.n, L.npad, L.m, mask_out, w.ctrl());

@@ -326,7 +326,7 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
       acc = shift_in(acc, c);
     }
   } else {
-    constexpr int G = M <= 5 ? 8 : 4;
+    constexpr int G = M <= 5 ? 8 : (M <= 8 ? 4 : 2);
 #pragma unroll 1
     for (int g = 32 / G - 1; g >= 0; --g) {
       const int i0 = ib + g * G;  // wave-uniform

@@ -113,25 +113,30 @@ def test_dominance_bits_edge(name, f, ks, variant):
     assert np.array_equal(as_np(views["rank"]), as_np(er.ranks_by_peeling(f)))
 
 
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8, 9, 12])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 16, 17])
 def test_dominance_bits_all_m(m):
     say("dominance_bits_all_m", m)
     g = torch.Generator("cpu").manual_seed(40 + m)
-    f = (torch.randint(0, 3 + m, (333, m), generator=g).float() / 4.0).contiguous()
-    n = f.size(0)
-    fd = f.to(DEV)
-    ws = runtime.workspace(n, m, fd.device)
-    s = runtime.stream_handle(fd.device)
-    want = as_np(er.pareto_dominance(f, f)).T
-    for variant in ([0, 1, 2, 3] if m <= 8 else [0]):
-        _lib.call("evox_hip_stage_prepare", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), ws.data_ptr(), ws.numel(), s)
-        _lib.call("evox_hip_stage_dominance", n, m, variant, ws.data_ptr(), ws.numel(), s)
-        torch.cuda.synchronize()
-        got = unpack_bits(runtime.workspace_views(ws, n, m), n)
-        assert np.array_equal(got, want), (m, variant)
+    finite = (torch.randint(0, 3 + m, (333, m), generator=g).float() / 4.0).contiguous()
+    other = finite.clone()  # with values that are not finite: the kernels then take the compare form
+    other[torch.rand(333, m, generator=g) < 0.02] = float("nan")
+    other[torch.rand(333, m, generator=g) < 0.02] = float("inf")
+    other[torch.rand(333, m, generator=g) < 0.02] = -float("inf")
+    for f in (finite, other):
+        n = f.size(0)
+        fd = f.to(DEV)
+        ws = runtime.workspace(n, m, fd.device)
+        s = runtime.stream_handle(fd.device)
+        want = as_np(er.pareto_dominance(f, f)).T
+        for variant in ([0, 1, 2, 3] if m <= 8 else [0, 1]):
+            _lib.call("evox_hip_stage_prepare", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), ws.data_ptr(), ws.numel(), s)
+            _lib.call("evox_hip_stage_dominance", n, m, variant, ws.data_ptr(), ws.numel(), s)
+            torch.cuda.synchronize()
+            got = unpack_bits(runtime.workspace_views(ws, n, m), n)
+            assert np.array_equal(got, want), (m, variant, bool(torch.isfinite(f).all()))
 
 
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 8])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 8, 11, 16])
 def test_dominance_arithmetic_form_corner_values(m):
     """A population of finite values takes the arithmetic form of the dominance test (signs of differences):
     denormal differences, differences that overflow, signed zeros, huge and tiny magnitudes, duplicates."""
@@ -775,7 +780,7 @@ def test_first_front_edge(name, f, ks, population_path):
     assert runtime.last_status()["error"] == 0
 
 
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8, 9, 12])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 16, 17])
 def test_first_front_all_m(m, population_path):
     if population_path != "pipeline":
         pytest.skip("does not depend on the population path")
