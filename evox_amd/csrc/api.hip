@@ -435,7 +435,7 @@ static int copy_async(void* dst, const void* src, size_t bytes, hipStream_t s) {
 template <int M>
 static int launch_batched_m(const BatchedArgs& a, int64_t batch, hipStream_t s) {
   const int nt = (int)round_up(a.n, 64);
-  const size_t lds = batched_lds_bytes(nt);
+  const size_t lds = batched_lds_bytes(nt, M);
   // the attribute belongs to the (kernel, device) pair: remembered per device
   static size_t granted[64] = {0};
   int dev = 0;
@@ -473,6 +473,14 @@ static int launch_batched(const BatchedArgs& a, int64_t batch, hipStream_t s) {
     case 6: return launch_batched_m<6>(a, batch, s);
     case 7: return launch_batched_m<7>(a, batch, s);
     case 8: return launch_batched_m<8>(a, batch, s);
+    case 9: return launch_batched_m<9>(a, batch, s);
+    case 10: return launch_batched_m<10>(a, batch, s);
+    case 11: return launch_batched_m<11>(a, batch, s);
+    case 12: return launch_batched_m<12>(a, batch, s);
+    case 13: return launch_batched_m<13>(a, batch, s);
+    case 14: return launch_batched_m<14>(a, batch, s);
+    case 15: return launch_batched_m<15>(a, batch, s);
+    case 16: return launch_batched_m<16>(a, batch, s);
     default: return kErrBadArg;
   }
 }
@@ -789,11 +797,11 @@ int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_ro
                      out_rank, out_dist, out_order, ws, ws_bytes, (hipStream_t)stream);
 }
 
-int64_t evox_hip_batched_max_rows(int64_t m) { return (m >= 1 && m <= 8) ? kBatchedMaxRows : 0; }
+int64_t evox_hip_batched_max_rows(int64_t m) { return (m >= 1 && m <= kBatchedMaxObjectives) ? kBatchedMaxRows : 0; }
 
 int evox_hip_batched_non_dominate_rank(const float* f, int64_t batch, int64_t n, int64_t m, int64_t stride_batch,
                                        int64_t stride_row, int64_t stride_col, int32_t* rank_out, void* stream) {
-  if (f == nullptr || rank_out == nullptr || batch < 1 || n < 1 || n > kBatchedMaxRows || m < 1 || m > 8) return kErrBadArg;
+  if (f == nullptr || rank_out == nullptr || batch < 1 || n < 1 || n > kBatchedMaxRows || m < 1 || m > kBatchedMaxObjectives) return kErrBadArg;
   BatchedArgs a = {};
   a.f = f;
   a.f_stride_b = stride_batch;
@@ -812,7 +820,7 @@ int evox_hip_batched_nd_environmental_selection(const void* x, int64_t x_row_byt
                                                 int64_t topk, void* out_x, float* out_f, int32_t* out_rank, float* out_dist,
                                                 void* stream) {
   if (f == nullptr || out_f == nullptr || out_rank == nullptr || out_dist == nullptr) return kErrBadArg;
-  if (batch < 1 || n < 1 || n > kBatchedMaxRows || m < 1 || m > 8 || topk < 1 || topk > n) return kErrBadArg;
+  if (batch < 1 || n < 1 || n > kBatchedMaxRows || m < 1 || m > kBatchedMaxObjectives || topk < 1 || topk > n) return kErrBadArg;
   if ((x == nullptr) != (out_x == nullptr) || (x != nullptr && (x_row_bytes < 0 || x_row_stride_bytes < 0))) return kErrBadArg;
   BatchedArgs a = {};
   a.f = f;

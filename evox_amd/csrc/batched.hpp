@@ -26,6 +26,7 @@
 namespace evx {
 
 constexpr int kBatchedMaxRows = 1024;
+constexpr int kBatchedMaxObjectives = 16;
 
 typedef const float __attribute__((address_space(4))) * ConstFloatPtr;
 
@@ -58,17 +59,21 @@ __device__ inline int count_smaller(const uint64_t* tile, int nv, uint64_t mine)
 }
 
 // Row stride of the LDS matrix in words: one word of padding against bank conflicts, except at the
-// largest size, where the padding would not fit; at least nine words, because after the peeling the
-// matrix's LDS is reused for everything that the rest of the kernel needs (up to 60 bytes per row).
-__host__ __device__ inline int batched_row_stride(int nt) { return nt == 1024 ? 16 : (nt / 64 + 1 < 9 ? 9 : nt / 64 + 1); }
+// largest size, where the padding would not fit; at least nine words (thirteen above eight objectives),
+// because after the peeling the matrix's LDS is reused for everything that the rest of the kernel needs
+// (4 bytes per objective, rounded up to eight objectives, plus 28 bytes per row).
+__host__ __device__ inline int batched_row_stride(int nt, int m) {
+  const int least = m <= 8 ? 9 : 13;
+  return nt == 1024 ? 16 : (nt / 64 + 1 < least ? least : nt / 64 + 1);
+}
 
-// Dynamic LDS layout (nt = blockDim.x):
+// Dynamic LDS layout (nt = blockDim.x, M8 = the objectives rounded up to a multiple of eight):
 //   uint64 dom[nt][row stride] | uint64 front[2][16] | int perm[nt]
 // and, once the peeling is over, inside dom:
-//   float fit[8][nt] | uint64 tile[nt + 4] | float scost[nt] | float dist[nt] | int order[nt] | int rank[nt] | int below[nt]
-// 512 rows take 39.2 KB, so that four workgroups share a compute unit's 160 KB.
-__host__ __device__ inline size_t batched_lds_bytes(int nt) {
-  return sizeof(uint64_t) * ((size_t)nt * batched_row_stride(nt) + 32) + sizeof(int) * (size_t)nt;
+//   float fit[M8][nt] | uint64 tile[nt + 4] | float scost[nt] | float dist[nt] | int order[nt] | int rank[nt] | int below[nt]
+// 512 rows of up to eight objectives take 39.2 KB, so that four workgroups share a compute unit's 160 KB.
+__host__ __device__ inline size_t batched_lds_bytes(int nt, int m) {
+  return sizeof(uint64_t) * ((size_t)nt * batched_row_stride(nt, m) + 32) + sizeof(int) * (size_t)nt;
 }
 
 // Position of every candidate among the nv (key << 32 | index) pairs of `tile`, by counting the smaller
@@ -124,19 +129,19 @@ __device__ inline void gather_units(const uint8_t* __restrict__ xb, uint8_t* __r
 }
 
 // Registers are capped for eight waves per SIMD (at most 64 VGPRs and 96 SGPRs): populations of 512 rows
-// then run four workgroups to a compute unit, which their LDS allows.
+// then run four workgroups to a compute unit, which their LDS allows (three above eight objectives).
 template <int M>
-__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void batched_kernel(BatchedArgs a) {
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(M <= 12 ? 8 : 4, 8))) void batched_kernel(BatchedArgs a) {
   extern __shared__ uint64_t lds64[];
   const int nt = blockDim.x;
   const int W = nt >> 6;
-  const int rs = batched_row_stride(nt);
+  const int rs = batched_row_stride(nt, M);
   uint64_t* dom = lds64;
   uint64_t* front = dom + (size_t)nt * rs;
   int* perm = reinterpret_cast<int*>(front + 32);
   // valid only after the peeling (they lie inside dom)
   float* fit_lds = reinterpret_cast<float*>(dom);
-  uint64_t* tile = reinterpret_cast<uint64_t*>(fit_lds + 8 * (size_t)nt);
+  uint64_t* tile = reinterpret_cast<uint64_t*>(fit_lds + ((M + 7) / 8 * 8) * (size_t)nt);
   float* scost = reinterpret_cast<float*>(tile + (nt + 4));
   float* dist = scost + nt;
   int* order = reinterpret_cast<int*>(dist + nt);
@@ -168,6 +173,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
   }
   const bool all_finite = __syncthreads_and(finite_row) != 0;
   const bool packed_rows = a.f_stride_col == 1 && a.f_stride_row == M;
+  constexpr int GP = M <= 8 ? 8 : 4;  // dominators per group of scalar loads (at most 64 scalars)
   // Dominators are read at wave-uniform addresses through the constant address space: the fitness is never
   // written here, and only loads known to be invariant are issued as scalar loads.
   const ConstFloatPtr fc = (ConstFloatPtr)f;
@@ -178,15 +184,15 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
     for (int h = 1; h >= 0; --h) {
       uint32_t acc = 0;
       if (all_finite && packed_rows && w * 64 + h * 32 + 32 <= n) {
-        // rows of M consecutive floats: eight dominators are 8 M consecutive scalars, fetched by wide scalar loads
+        // rows of M consecutive floats: GP dominators are GP M consecutive scalars, fetched by wide scalar loads
 #pragma unroll 1
-        for (int g = 3; g >= 0; --g) {
-          const ConstFloatPtr p = fc + (int64_t)(w * 64 + h * 32 + g * 8) * M;  // wave-uniform
-          float v[8 * M];
+        for (int g = 32 / GP - 1; g >= 0; --g) {
+          const ConstFloatPtr p = fc + (int64_t)(w * 64 + h * 32 + g * GP) * M;  // wave-uniform
+          float v[GP * M];
 #pragma unroll
-          for (int e = 0; e < 8 * M; ++e) v[e] = p[e];
+          for (int e = 0; e < GP * M; ++e) v[e] = p[e];
 #pragma unroll
-          for (int u = 7; u >= 0; --u) {
+          for (int u = GP - 1; u >= 0; --u) {
             uint32_t o = 0u;
 #pragma unroll
             for (int k = 0; k < M; ++k) o |= __float_as_uint(xz[k] - v[u * M + k]);

@@ -105,7 +105,7 @@ int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_ro
 
 /* ---- many small populations at once (what the reference reaches through vmap: non_dominate.py:107-125
  * for the peeling, the rest of the path batching natively).  One workgroup per population, no workspace.
- * n <= evox_hip_batched_max_rows(m) (1024 rows for m <= 8, 0 = unsupported); f is addressed as
+ * n <= evox_hip_batched_max_rows(m) (1024 rows for m <= 16, 0 = unsupported); f is addressed as
  * f[b * stride_batch + i * stride_row + k * stride_col]; outputs are contiguous (batch, ...) arrays.
  * Per population the results equal those of the single-population entry points. */
 int64_t evox_hip_batched_max_rows(int64_t m);

@@ -30,7 +30,7 @@ def say(*a):
 
 @pytest.fixture(autouse=True, params=["pipeline", "small-kernel"])
 def population_path(request):
-    """Every test runs twice: with small populations (<= 1024 rows, <= 8 objectives) served by the
+    """Every test runs twice: with small populations (<= 1024 rows, <= 16 objectives) served by the
     one-workgroup-per-population kernel, as in production, and with everything forced through the
     bit-matrix pipeline."""
     runtime.use_small_population_kernel = request.param == "small-kernel"
@@ -439,7 +439,8 @@ def test_c4_full_batch_one_launch():
         runtime.use_small_population_kernel = keep
 
 
-@pytest.mark.parametrize("n,m", [(33, 1), (64, 2), (95, 3), (130, 4), (257, 5), (500, 6), (777, 7), (1024, 8), (1000, 3)])
+@pytest.mark.parametrize("n,m", [(33, 1), (64, 2), (95, 3), (130, 4), (257, 5), (500, 6), (777, 7), (1024, 8), (1000, 3), (300, 9),
+                                 (512, 12), (200, 13), (1024, 16)])
 def test_batched_selection_shapes_layouts_and_row_units(n, m, population_path):
     """The one-workgroup kernel over ragged sizes, every objective count, packed and strided fitness (its
     dominator loads take different paths), non-finite values (the compare form) and rows of x whose size
