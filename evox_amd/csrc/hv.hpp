@@ -22,7 +22,7 @@ constexpr int kHvChunk = 256;        // samples per partial sum of the contribut
 constexpr int kHvPointChunk = 128;   // points per partial cover count of the contributions, at least
 constexpr int kHvMaxChunks = 64;     // chunks of either kind, at most (bounds the workspace)
 constexpr int kHvCoverChunk = 1024;  // points per block of the metric
-constexpr int kHvRegs = 8;           // objectives held in registers; more are re-read from memory
+constexpr int kHvRegs = 16;          // objectives held in registers; more are re-read from memory
 
 // Length of the chunks that cut `count` items into at most kHvMaxChunks pieces of at least `least` items
 // (a multiple of eight, the streaming unit).

@@ -959,7 +959,8 @@ def test_hv_contributions_against_oracle(population_path):
     from evox_amd.hype import cal_hv, hv_alpha
 
     g = torch.Generator("cpu").manual_seed(19)
-    for n, m, pop, ns in ((1, 2, 1, 100), (7, 2, 3, 333), (200, 3, 100, 10000), (1000, 5, 400, 5000), (64, 9, 64, 1025)):
+    for n, m, pop, ns in ((1, 2, 1, 100), (7, 2, 3, 333), (200, 3, 100, 10000), (1000, 5, 400, 5000), (64, 9, 64, 1025),
+                          (50, 17, 20, 700)):
         say("hv", n, m, pop, ns)
         fit = torch.rand(n, m, generator=g)
         if n > 3:
@@ -991,7 +992,7 @@ def test_hv_metric_against_oracle(population_path):
     from evox_amd.metrics import hv
 
     g = torch.Generator("cpu").manual_seed(23)
-    for n, m, ns in ((1, 2, 100), (7, 2, 333), (200, 3, 10000), (1000, 5, 5000), (64, 9, 1025), (3000, 3, 100000)):
+    for n, m, ns in ((1, 2, 100), (7, 2, 333), (200, 3, 10000), (1000, 5, 5000), (64, 9, 1025), (50, 17, 700), (3000, 3, 100000)):
         say("hv metric", n, m, ns)
         objs = torch.rand(n, m, generator=g)
         if n > 3:
