@@ -169,6 +169,9 @@ __global__ __launch_bounds__(256) void count_kernel(const uint64_t* __restrict__
                                                     int* __restrict__ fsize, float* __restrict__ dist_fill,
                                                     const Ctrl* __restrict__ ctrl) {
   if (ctrl->err != 0) return;  // the slot tables are not valid: leave front 0 empty, nothing gets peeled
+  __shared__ int block_found;
+  if (threadIdx.x == 0) block_found = 0;
+  __syncthreads();
   const int lane = threadIdx.x & 63;
   const int wave_in_block = threadIdx.x >> 6;
   const int waves = gridDim.x * (blockDim.x >> 6);
@@ -188,7 +191,10 @@ __global__ __launch_bounds__(256) void count_kernel(const uint64_t* __restrict__
       }
     }
   }
-  if (lane == 0 && found) atomicAdd(fsize, found);
+  // one addition per block: a front 0 of thousands of rows would otherwise queue thousands of atomics on one word
+  if (lane == 0 && found) atomicAdd(&block_found, found);
+  __syncthreads();
+  if (threadIdx.x == 0 && block_found) atomicAdd(fsize, block_found);
 }
 
 // ------------------------------------------------------------ grid barrier

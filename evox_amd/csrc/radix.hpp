@@ -25,7 +25,7 @@
 
 namespace evx {
 
-constexpr int kRadixMinCandidates = 4096;
+constexpr int kRadixMinCandidates = 8192;
 constexpr int kRadixThreads = 256;
 
 struct RadixBuffers {

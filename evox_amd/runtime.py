@@ -14,11 +14,24 @@ _last: Optional[Tuple[torch.Tensor, int]] = None  # (workspace, stream handle) o
 CHECK_STATUS = os.environ.get("EVOX_AMD_CHECK_STATUS", "0") not in ("", "0")
 
 # Populations of at most evox_hip_batched_max_rows(m) rows can run in the one-workgroup-per-population
-# kernel, larger ones need the bit-matrix pipeline.  None = choose by size (a lone population of more
-# than 960 rows is faster in the pipeline, which spreads it over the whole device; measured: 55 against
-# 105 us at 576 rows, 96 against 104 us at 960 rows, 114 against 111 us at 1024 rows); True / False
-# force the choice where it is possible (tests use that to drive small inputs through both).
+# kernel, larger ones need the bit-matrix pipeline.  None = choose by size: a lone population is faster in
+# the pipeline, which spreads it over the whole device, from a size on that shrinks as the objectives grow
+# (measured, one-workgroup kernel against pipeline, in us: 3 objectives 48/75 at 704 rows and 86/81 at 960;
+# 5 objectives 60/71 at 704, 94/80 at 960; 8 objectives 65/68 at 256, 85/76 at 384; 16 objectives 67/77 at 128,
+# 119/101 at 256); two or three populations up to twice that size, and four or more always, take the
+# one-workgroup kernel, which runs them side by side.  True / False force the choice where it is possible
+# (tests use that to drive small inputs through both).
 use_small_population_kernel = None
+
+
+def _lone_population_limit(m: int) -> int:
+    if m <= 3:
+        return 896
+    if m <= 5:
+        return 768
+    if m <= 8:
+        return 288
+    return 160
 
 
 def small_population_kernel_fits(n: int, m: int, batch: int) -> bool:
@@ -28,7 +41,9 @@ def small_population_kernel_fits(n: int, m: int, batch: int) -> bool:
         return False
     if use_small_population_kernel is True:
         return True
-    return n <= 960 or batch >= 2
+    if batch >= 4:
+        return True
+    return n <= _lone_population_limit(m) * (1 if batch == 1 else 2)
 
 
 def require_gpu_tensor(t: torch.Tensor, what: str) -> None:
