@@ -447,9 +447,9 @@ def main():
     dominant = max(("dominance", "count", "peel"), key=lambda k: phases[k]["us"])
     d = phases[dominant]
     roofline = {
-        # populations below 65535 rows are peeled by the record-protocol kernel, larger ones by peel_kernel
+        # populations up to 262144 rows are peeled by the record-protocol kernel, larger ones by peel_kernel
         "kernel": {"dominance": "dominance_kernel", "count": "count_kernel",
-                   "peel": "peel_records_kernel" if n < 65535 else "peel_kernel"}[dominant],
+                   "peel": "peel_records_kernel" if n <= 262144 else "peel_kernel"}[dominant],
         "bound": "hbm" if d["bound"] == "hbm" else "valu",
         "achieved": d["achieved"], "peak": d["peak"], "unit": d["unit"], "frac": d["frac"], "traffic": None,
     }

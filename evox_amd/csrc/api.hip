@@ -18,14 +18,16 @@
 namespace evx {
 
 constexpr int kMaxGrid = 4096;  // slots of the grid barrier
-constexpr int kRecordsMaxRows = 65534;  // largest population peeled with the record protocol
+constexpr int kRecordsMaxRows = 65534;       // largest population whose record units hold three 16-bit slots
+constexpr int kRecordsMaxRowsWide = 262144;  // largest population peeled with the record protocol at all (two
+                                             // 24-bit slots per unit; 128 blocks of 8 waves own 256 rows per wave)
 constexpr int kRadixMaxWorkers = 510;
 
 struct Options {
   int peel_blocks_per_cu = 2;
   int peel_witness = 1;
   int peel_record_blocks = 0;  // sweeping blocks of the record protocol, 16 .. 255 (plus the lister); 0 = by size
-  int peel_records = 1;  // record protocol (all-to-all, no master) for populations up to kRecordsMaxRows
+  int peel_records = 1;  // record protocol (all-to-all, no master) for populations up to kRecordsMaxRowsWide
   unsigned spin_limit = 4000000u;
   int dominance_tile_words = 4;
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
@@ -63,7 +65,7 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->fronts_orig = o; o = align_up(o + sizeof(uint64_t) * kFrontBuffers * kFrontStride * (size_t)L->nwords);
   L->hist = o;        o = align_up(o + sizeof(int) * (size_t)buckets);
   L->scanflags = o;   o = align_up(o + sizeof(unsigned long long) * 64);
-  L->records = o;     o = align_up(o + (n <= kRecordsMaxRows ? sizeof(unsigned long long) * kRecRing * kRecUnits : 0));
+  L->records = o;     o = align_up(o + (n <= kRecordsMaxRowsWide ? sizeof(unsigned long long) * kRecRing * kRecUnits : 0));
   L->zero_end = o;
   L->fstart = o;     o = align_up(o + sizeof(int) * (size_t)(n + 2));
   L->xs = o;         o = align_up(o + sizeof(float) * (size_t)m * L->npad);
@@ -301,6 +303,15 @@ static int peel_blocks_per_cu(size_t lds, int* err) {
   return per_cu;
 }
 
+static int grant_dynamic_lds(const void* kernel, size_t lds) {
+  if (lds > 150 * 1024) return kErrBadArg;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+  }
+  return 0;
+}
+
 static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s) {
   const Layout& L = w.L;
   if (stop_count < 1 || stop_count > L.n) return kErrBadArg;
@@ -334,7 +345,7 @@ static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream
     if (err) return err;
   }
   if (blocks <= kFirstSweeper) return kErrBadArg;
-  if (use_witness && g_opt.peel_records && L.n <= kRecordsMaxRows) {
+  if (use_witness && g_opt.peel_records && L.n <= kRecordsMaxRowsWide) {
     // all-to-all records: 1 lister + a power of two of sweeping blocks, all resident at once
     // by size: 64 blocks up to 32768 rows, 128 above (measured at 20000 rows: 221 us per selection with 64
     // blocks, 225 with 128, 228 with 32, 238 with 192; between 1200 and 6000 rows the count hardly matters)
@@ -345,10 +356,17 @@ static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream
     const size_t rec_lds = bitmap + 24 * (size_t)list_capacity;  // queue (8 + 4 + 4) and ranked pairs (2 x 4) per row
     // every block waits for every other one: all of them must be resident at once
     int rec_per_cu = 0;
-    const hipError_t oe = hipOccupancyMaxActiveBlocksPerMultiprocessor(&rec_per_cu, peel_records_kernel, kRecThreads, rec_lds);
+    const bool wide = L.n > kRecordsMaxRows;
+    const void* kernel = wide ? reinterpret_cast<const void*>(peel_records_kernel<true>)
+                              : reinterpret_cast<const void*>(peel_records_kernel<false>);
+    const bool rows_fit = (int64_t)list_capacity <= (int64_t)wpb * kWitnessChunks * 64;  // what the waves' registers hold
+    if (rows_fit && rec_lds <= 150 * 1024)
+      if (int e = grant_dynamic_lds(kernel, rec_lds)) return e;
+    const hipError_t oe = wide ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&rec_per_cu, peel_records_kernel<true>, kRecThreads, rec_lds)
+                               : hipOccupancyMaxActiveBlocksPerMultiprocessor(&rec_per_cu, peel_records_kernel<false>, kRecThreads, rec_lds);
     if (oe != hipSuccess) return (int)oe;
-    if ((int64_t)rec_per_cu * cus >= sweepers + 1) {
-    hipLaunchKernelGGL(peel_records_kernel, dim3(sweepers + 1), dim3(kRecThreads), rec_lds, s, w.at<uint64_t>(L.dom), L.wstride,
+    if (rows_fit && rec_lds <= 150 * 1024 && (int64_t)rec_per_cu * cus >= sweepers + 1) {
+    hipLaunchKernelGGL(wide ? peel_records_kernel<true> : peel_records_kernel<false>, dim3(sweepers + 1), dim3(kRecThreads), rec_lds, s, w.at<uint64_t>(L.dom), L.wstride,
                        L.nwords, L.n, w.at<int>(L.orig_of), w.at<int>(L.rank), w.at<uint64_t>(L.fronts_slot),
                        w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize), want_perm ? w.at<int>(L.perm) : (int*)nullptr,
                        w.at<int>(L.fstart), w.ctrl(), (int)stop_count, g_opt.spin_limit, w.at<int>(L.witness),
@@ -405,15 +423,6 @@ static int finish_grid(const Layout& L, int per_candidate_block) {
   }
   int blocks = ((L.n + 255) / 256) * per_candidate_block;
   return blocks < 1 ? 1 : blocks;
-}
-
-static int grant_dynamic_lds(const void* kernel, size_t lds) {
-  if (lds > 150 * 1024) return kErrBadArg;
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-  }
-  return 0;
 }
 
 // Per-objective ordering of the candidates list[ctrl.worst_start ... + ctrl.nv).

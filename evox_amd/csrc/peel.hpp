@@ -848,32 +848,54 @@ constexpr int kRecThreads = 512;
 constexpr int kRecUnits = 1024;  // units of one generation = sweepers x units per record
 constexpr int kRecRing = 8;      // == kFrontBuffers: a generation's record slot and bitmap buffer recycle together
 constexpr int kRecLoads = kRecUnits / kRecThreads;
-constexpr uint32_t kRecNil = 0xFFFFu;       // no slot (populations have fewer than 65535 rows)
-constexpr uint32_t kRecOverflow = 0x8000u;  // in the count field: the rows are in the bitmaps, not in the record
+constexpr uint32_t kRecOverflowNarrow = 0x8000u;  // in the count field: the rows are in the bitmaps, not in the record
 static_assert(kRecRing == kFrontBuffers, "records and bitmaps are recycled by the same counter");
 
-__device__ inline unsigned long long record_unit(unsigned gen, uint32_t a, uint32_t b, uint32_t c) {
-  return ((unsigned long long)(gen & 0xFFFFu) << 48) | ((unsigned long long)(a & 0xFFFFu) << 32) | ((b & 0xFFFFu) << 16) | (c & 0xFFFFu);
-}
-// Slots that a record of `units` units can carry.
-__device__ inline int record_capacity(int units) { return 2 + 3 * (units - 1); }
-// The unit that thread i (< units) of the writer stores: list = (slot, original index) pairs, cnt of them.
-__device__ inline unsigned long long record_unit_for(unsigned gen, int i, const int* list, int cnt, bool overflow) {
-  auto slot_at = [&](int k) { return (!overflow && k < cnt) ? (uint32_t)list[2 * k] : kRecNil; };
-  if (i == 0) return record_unit(gen, overflow ? (kRecOverflow | (uint32_t)cnt) : (uint32_t)cnt, slot_at(0), slot_at(1));
-  return record_unit(gen, slot_at(3 * i - 1), slot_at(3 * i), slot_at(3 * i + 1));
-}
-// Calls on_count(count, overflow) for a unit 0 and on_slot(slot) for every slot a unit carries.
-template <class OnCount, class OnSlot>
-__device__ inline void record_unit_read(unsigned long long v, bool is_first, OnCount on_count, OnSlot on_slot) {
-  const uint32_t a = (uint32_t)(v >> 32) & 0xFFFFu, b = (uint32_t)(v >> 16) & 0xFFFFu, c = (uint32_t)v & 0xFFFFu;
-  if (is_first)
-    on_count((int)(a & ~kRecOverflow), (a & kRecOverflow) != 0u);
-  else if (a != kRecNil)
-    on_slot((int)a);
-  if (b != kRecNil) on_slot((int)b);
-  if (c != kRecNil) on_slot((int)c);
-}
+// Two layouts of a unit.  Narrow (populations of fewer than 65535 rows): generation : 16 | three 16-bit fields;
+// wide (fewer than 2^24 - 1 rows): generation : 16 | two 24-bit fields.  Unit 0 of a record carries the count
+// (with the overflow flag in its top bit) in its first field, every other field is a slot or "none" (all ones).
+template <bool WIDE>
+struct RecFormat {
+  static constexpr int kFields = WIDE ? 2 : 3;
+  static constexpr int kBits = WIDE ? 24 : 16;
+  static constexpr uint32_t kMask = (1u << kBits) - 1u;
+  static constexpr uint32_t kNil = kMask;
+  static constexpr uint32_t kOverflow = 1u << (kBits - 1);
+  // Slots that a record of `units` units can carry.
+  __device__ static int capacity(int units) { return kFields - 1 + kFields * (units - 1); }
+  __device__ static unsigned long long pack(unsigned gen, const uint32_t (&f)[3]) {
+    unsigned long long v = (unsigned long long)(gen & 0xFFFFu) << 48;
+#pragma unroll
+    for (int k = 0; k < kFields; ++k) v |= (unsigned long long)(f[k] & kMask) << (kBits * (kFields - 1 - k));
+    return v;
+  }
+  // The unit that thread i (< units) of the writer stores: list = (slot, original index) pairs, cnt of them.
+  __device__ static unsigned long long unit_for(unsigned gen, int i, const int* list, int cnt, bool overflow) {
+    auto slot_at = [&](int k) { return (!overflow && k < cnt) ? (uint32_t)list[2 * k] : kNil; };
+    uint32_t f[3] = {kNil, kNil, kNil};
+    if (i == 0) {
+      f[0] = overflow ? (kOverflow | (uint32_t)cnt) : (uint32_t)cnt;
+#pragma unroll
+      for (int k = 1; k < kFields; ++k) f[k] = slot_at(k - 1);
+    } else {
+#pragma unroll
+      for (int k = 0; k < kFields; ++k) f[k] = slot_at(kFields * i - 1 + k);
+    }
+    return pack(gen, f);
+  }
+  // Calls on_count(count, overflow) for a unit 0 and on_slot(slot) for every slot a unit carries.
+  template <class OnCount, class OnSlot>
+  __device__ static void read(unsigned long long v, bool is_first, OnCount on_count, OnSlot on_slot) {
+#pragma unroll
+    for (int k = 0; k < kFields; ++k) {
+      const uint32_t field = (uint32_t)(v >> (kBits * (kFields - 1 - k))) & kMask;
+      if (k == 0 && is_first)
+        on_count((int)(field & ~kOverflow), (field & kOverflow) != 0u);
+      else if (field != kNil)
+        on_slot((int)field);
+    }
+  }
+};
 
 // Waits until the kRecLoads units of generation `gen` that this thread reads are all present (and, for
 // the thread that is given a counter, until *listed >= listed_needed).  False after a timeout or when
@@ -910,6 +932,7 @@ __device__ inline bool poll_record_units(const unsigned long long* gen_units, in
   }
 }
 
+template <bool WIDE>
 __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
     const uint64_t* __restrict__ dom, int64_t wstride, int nwords, int n, const int* __restrict__ orig_of,
     int* __restrict__ rank, uint64_t* __restrict__ fronts_slot, uint64_t* __restrict__ fronts_orig, int* __restrict__ fsize,
@@ -962,7 +985,7 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
           for (int k = 0; k < kRecLoads; ++k) {
             if (tid + k * kRecThreads >= sweepers * units) continue;  // past the last record
             const int i = (tid + k * kRecThreads) & (units - 1);
-            record_unit_read(
+            RecFormat<WIDE>::read(
                 v[k], i == 0,
                 [&](int count, bool overflow) {
                   atomicAdd(&sh[1], count);
@@ -991,8 +1014,10 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
       }
       __syncthreads();  // also waits for the clearing stores of this block's waves
       if (tid == 0) coherent_store(&ctrl->listed, level);  // records <= level consumed, bitmaps < level cleared
-      if (perm) list_front(front_lds, nwords, perm, ranked, sh + 8);
       const bool last = size <= 0 || ranked + size >= stop_count;
+      // a front 0 that ends the peel is listed by the sweepers together (see peel_kernel)
+      const bool shared_listing = level == 0 && last && size > kSharedListingRows;
+      if (perm && !shared_listing) list_front(front_lds, nwords, perm, ranked, sh + 8);
       if (tid == 0) {
         fstart[level] = ranked;
         if (level > 0) fsize[level] = size;
@@ -1029,7 +1054,31 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
   c.orig_of = orig_of;
   c.rank = rank;
   int size = coherent_load(&fsize[0]);  // size of front `level`
-  if (size <= 0 || size >= stop_count) return;  // front 0 already holds every row asked for: no pass
+  if (size <= 0 || size >= stop_count) {  // front 0 already holds every row asked for: no pass
+    if (perm && size > kSharedListingRows) {
+      // list it: the first sweeping blocks take a slice of the bitmap (original-index space) each, after adding
+      // up the rows of the words before their slice
+      const int listers = min(sweepers, kSharedListingBlocks);
+      if (sb < listers) {
+        const int per = (nwords + listers - 1) / listers;
+        const int w_begin = min(nwords, sb * per), w_end = min(nwords, w_begin + per);
+        int before = 0;
+        for (int w = tid; w < w_end; w += blockDim.x) {
+          const uint64_t fw = coherent_load(&fronts_orig[(int64_t)w * kFrontStride]);
+          if (w < w_begin)
+            before += __popcll(fw);
+          else
+            rec_lds[w - w_begin] = fw;
+        }
+        if (tid == 0) sh[0] = 0;
+        __syncthreads();
+        if (before) atomicAdd(&sh[0], before);
+        __syncthreads();
+        list_front(rec_lds, w_end - w_begin, perm, sh[0], sh + 8, w_begin);
+      }
+    }
+    return;
+  }
   WitnessState st;
   witness_load(st, c, witness, first_row, row_step);
   for (int w = tid; w < nwords; w += blockDim.x) {
@@ -1069,8 +1118,8 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
     const int cnt = cnts[0];
     if (tid < 4) next_cnts[tid] = 0;  // last read before the barrier above, first used after the one below
     unsigned long long* mine = records + (size_t)(gen % kRecRing) * kRecUnits + (size_t)sb * units;
-    if (cnt <= record_capacity(units)) {
-      if (tid < units) coherent_store(&mine[tid], record_unit_for(gen, tid, found, cnt, false));
+    if (cnt <= RecFormat<WIDE>::capacity(units)) {
+      if (tid < units) coherent_store(&mine[tid], RecFormat<WIDE>::unit_for(gen, tid, found, cnt, false));
     } else {
       for (int e = tid; e < cnt; e += blockDim.x) {
         const int slot = found[2 * e], orig = found[2 * e + 1];
@@ -1078,7 +1127,7 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
         atomicOr(reinterpret_cast<unsigned long long*>(c.next_orig + (int64_t)(orig >> 6) * kFrontStride), 1ull << (orig & 63));
       }
       __syncthreads();  // every wave has waited for its own atomics
-      if (tid < units) coherent_store(&mine[tid], record_unit_for(gen, tid, found, cnt, true));
+      if (tid < units) coherent_store(&mine[tid], RecFormat<WIDE>::unit_for(gen, tid, found, cnt, true));
     }
     // the records of everybody: barrier and front exchange in one.  Thread 0 also makes sure that the
     // lister has recycled what generation level + 1 will overwrite.
@@ -1095,7 +1144,7 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
       for (int k = 0; k < kRecLoads; ++k) {
         if (tid + k * kRecThreads >= sweepers * units) continue;  // past the last record
         const int i = (tid + k * kRecThreads) & (units - 1);
-        record_unit_read(
+        RecFormat<WIDE>::read(
             v[k], i == 0,
             [&](int count, bool overflow) {
               atomicAdd(&cnts[1], count);
