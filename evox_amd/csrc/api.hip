@@ -21,7 +21,6 @@ constexpr int kMaxGrid = 4096;  // slots of the grid barrier
 constexpr int kRecordsMaxRows = 65534;       // largest population whose record units hold three 16-bit slots
 constexpr int kRecordsMaxRowsWide = 262144;  // largest population peeled with the record protocol at all (two
                                              // 24-bit slots per unit; 128 blocks of 8 waves own 256 rows per wave)
-constexpr int kRadixMaxWorkers = 510;
 
 struct Options {
   int peel_blocks_per_cu = 2;

@@ -27,6 +27,8 @@ namespace evx {
 
 constexpr int kRadixMinCandidates = 8192;
 constexpr int kRadixThreads = 256;
+constexpr int kRadixBatch = 4;  // pairs per lane fetched together
+constexpr int kRadixMaxWorkers = 510;  // working blocks of a radix kernel, at most (columns of the digit table)
 
 struct RadixBuffers {
   unsigned long long* pairs[2];  // [segments][kstride] each: (key << 32) | candidate index
@@ -59,11 +61,20 @@ __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, in
     // ---- 1. digit histograms
     for (int t = threadIdx.x; t < nseg * 4 * 256; t += blockDim.x) hist[t] = 0;
     __syncthreads();
+    // (kRadixBatch pairs per lane are fetched before any is used: the coherent loads of a wave are then in flight
+    // together instead of costing a memory round trip each)
     for (int k = 0; k < nseg; ++k) {
       int* h = hist + (k * 4 + wave) * 256;
-      for (int e = w_begin + lane; e < w_end; e += 64) {
-        const unsigned long long p = pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]);
-        atomicAdd(&h[(int)((p >> (32 + shift)) & 255ull)], 1);
+      for (int e0 = w_begin + lane; e0 < w_end; e0 += 64 * kRadixBatch) {
+        unsigned long long p[kRadixBatch];
+#pragma unroll
+        for (int u = 0; u < kRadixBatch; ++u) {
+          const int e = e0 + 64 * u;
+          p[u] = e >= w_end ? 0ull : (pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]));
+        }
+#pragma unroll
+        for (int u = 0; u < kRadixBatch; ++u)
+          if (e0 + 64 * u < w_end) atomicAdd(&h[(int)((p[u] >> (32 + shift)) & 255ull)], 1);
       }
     }
     __syncthreads();
@@ -78,9 +89,19 @@ __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, in
     for (int item = wb * 4 + wave; item < nseg * 256; item += workers * 4) {
       int* row = buf.table + (int64_t)item * workers;
       int carry = 0;
-      for (int b0 = 0; b0 < workers; b0 += 64) {
+      constexpr int kChunks = (kRadixMaxWorkers + 63) / 64;  // all counts of the item are fetched together
+      int vals[kChunks];
+#pragma unroll
+      for (int c = 0; c < kChunks; ++c) {
+        const int b = c * 64 + lane;
+        vals[c] = b < workers ? coherent_load(&row[b]) : 0;
+      }
+#pragma unroll
+      for (int c = 0; c < kChunks; ++c) {
+        const int b0 = c * 64;
+        if (b0 >= workers) break;  // wave-uniform
         const int b = b0 + lane;
-        const int v = b < workers ? coherent_load(&row[b]) : 0;
+        const int v = vals[c];
         int incl = v;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
@@ -119,11 +140,20 @@ __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, in
     __syncthreads();
     for (int k = 0; k < nseg; ++k) {
       int* h = hist + (k * 4 + wave) * 256;
-      for (int e0 = w_begin; e0 < w_end; e0 += 64) {
+      for (int b0 = w_begin; b0 < w_end; b0 += 64 * kRadixBatch) {
+        unsigned long long batch[kRadixBatch];
+#pragma unroll
+        for (int u = 0; u < kRadixBatch; ++u) {
+          const int e = b0 + 64 * u + lane;
+          batch[u] = e >= w_end ? 0ull : (pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]));
+        }
+#pragma unroll
+        for (int u = 0; u < kRadixBatch; ++u) {
+        const int e0 = b0 + 64 * u;
+        if (e0 >= w_end) break;  // wave-uniform
         const int e = e0 + lane;
         const bool have = e < w_end;
-        const unsigned long long p =
-            !have ? 0ull : (pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]));
+        const unsigned long long p = batch[u];
         const int d = (int)((p >> (32 + shift)) & 255ull);
         // lanes of this group that hold the same digit
         uint64_t same = __builtin_amdgcn_ballot_w64(have);
@@ -141,6 +171,7 @@ __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, in
         }
         start = __shfl(start, leader < 0 ? 0 : leader);
         if (have) coherent_store(&out[(int64_t)k * buf.kstride + start + rank], p);
+        }
       }
     }
     if (!sweeper_barrier(ctrl, ++gen, 0, &dummy, spin_limit, scratch)) return false;
