@@ -45,6 +45,8 @@ _SIGNATURES = {
                                          c_void_p]),
     "evox_hip_argsort_workspace_bytes": (c_size_t, [c_int64]),
     "evox_hip_stable_argsort_step": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "evox_hip_stable_argsort_step_batched": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+                                                     c_void_p, c_size_t, c_void_p]),
     "evox_hip_hv_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "evox_hip_hv_contributions": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p, c_void_p,
                                           c_size_t, c_void_p]),

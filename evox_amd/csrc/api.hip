@@ -701,15 +701,8 @@ static bool make_sort_layout(int64_t n, SortLayout* L) {
   return true;
 }
 
-extern "C" {
-
-size_t evox_hip_argsort_workspace_bytes(int64_t n) {
-  SortLayout L;
-  return make_sort_layout(n, &L) ? L.total : 0;
-}
-
-int evox_hip_stable_argsort_step(const void* key, int kind, int64_t stride, int64_t n, const int32_t* prev_order,
-                                 int32_t* order_out, void* ws, size_t ws_bytes, void* stream) {
+static int argsort_step(const void* key, int kind, int64_t stride, int64_t n, const int32_t* prev_order, int32_t* order_out,
+                        void* ws, size_t ws_bytes, void* stream) {
   SortLayout L;
   if (key == nullptr || order_out == nullptr || kind < 0 || kind > 2) return kErrBadArg;
   if (!make_sort_layout(n, &L)) return kErrBadArg;
@@ -741,6 +734,76 @@ int evox_hip_stable_argsort_step(const void* key, int kind, int64_t stride, int6
   hipLaunchKernelGGL(argsort_step_kernel, dim3(workers + kFirstSweeper), dim3(kRadixThreads), sizeof(int) * 4 * 256, s, key, kind,
                      stride, L.n, prev_order, reinterpret_cast<Ctrl*>(base + L.ctrl), b, order_out, g_opt.spin_limit);
   EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+// `batch` sorts of n <= kSmallArgsortRows positions in one launch: a workgroup per sort, or several sorts per
+// workgroup when they are short.
+template <int T, int R>
+static int launch_rows_argsort(const void* key, int kind, int64_t batch_stride, int64_t stride, int64_t batch, int n,
+                               const int32_t* prev_order, int32_t* order_out, hipStream_t s) {
+  int group = 1;
+  while (group * R < n) group <<= 1;  // threads per sort, a power of two
+  if (group > T) return kErrBadArg;
+  const int rows_per_block = T / group;
+  const int row_stride = rows_per_block > 1 ? (n | 1) : n;
+  const size_t lds = sizeof(double) * (size_t)rows_per_block * (size_t)row_stride;
+  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(rows_argsort_kernel<T, R>), lds)) return e;
+  int64_t blocks = (batch + rows_per_block - 1) / rows_per_block;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL((rows_argsort_kernel<T, R>), dim3((unsigned)blocks), dim3(T), lds, s, key, kind, batch_stride, stride, batch, n,
+                     rows_per_block, row_stride, prev_order, order_out);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+static int launch_rows_bitonic(const void* key, int kind, int64_t batch_stride, int64_t stride, int64_t batch, int n,
+                               const int32_t* prev_order, int32_t* order_out, hipStream_t s) {
+  int npad = kRowsBitonicMin;
+  while (npad < n) npad <<= 1;
+  if (npad > kRowsArgsortMax) return kErrBadArg;
+  const int threads = npad / 8 < 1024 ? npad / 8 : 1024;  // eight entries per thread and pass
+  const size_t lds = sizeof(double) * (size_t)npad;
+  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(rows_bitonic_argsort_kernel), lds)) return e;
+  const int64_t blocks = batch < 65536 ? batch : 65536;
+  hipLaunchKernelGGL(rows_bitonic_argsort_kernel, dim3((unsigned)blocks), dim3(threads), lds, s, key, kind, batch_stride, stride,
+                     batch, n, npad, prev_order, order_out);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" {
+
+size_t evox_hip_argsort_workspace_bytes(int64_t n) {
+  SortLayout L;
+  return make_sort_layout(n, &L) ? L.total : 0;
+}
+
+int evox_hip_stable_argsort_step(const void* key, int kind, int64_t stride, int64_t n, const int32_t* prev_order,
+                                 int32_t* order_out, void* ws, size_t ws_bytes, void* stream) {
+  return argsort_step(key, kind, stride, n, prev_order, order_out, ws, ws_bytes, stream);
+}
+
+int evox_hip_stable_argsort_step_batched(const void* key, int kind, int64_t batch_stride, int64_t stride, int64_t batch,
+                                         int64_t n, const int32_t* prev_order, int32_t* order_out, void* ws, size_t ws_bytes,
+                                         void* stream) {
+  SortLayout L;
+  if (key == nullptr || order_out == nullptr || kind < 0 || kind > 2 || batch < 1) return kErrBadArg;
+  if (!make_sort_layout(n, &L)) return kErrBadArg;
+  if (ws == nullptr || ws_bytes < L.total || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return kErrWorkspace;
+  hipStream_t s = (hipStream_t)stream;
+  // all sorts in one launch when a sort fits the LDS of a workgroup: by counting up to 256 positions (several
+  // sorts per workgroup), through a bitonic network above that
+  if (batch >= 2 && n <= kRowsArgsortMax) {
+    if (n <= 256) return launch_rows_argsort<256, 1>(key, kind, batch_stride, stride, batch, (int)n, prev_order, order_out, s);
+    return launch_rows_bitonic(key, kind, batch_stride, stride, batch, (int)n, prev_order, order_out, s);
+  }
+  const size_t key_bytes = 4;
+  for (int64_t b = 0; b < batch; ++b) {
+    const void* kb = static_cast<const uint8_t*>(key) + (size_t)(b * batch_stride) * key_bytes;
+    if (int e = argsort_step(kb, kind, stride, n, prev_order ? prev_order + b * n : nullptr, order_out + b * n, ws, ws_bytes, stream))
+      return e;
+  }
   return 0;
 }
 

@@ -293,4 +293,171 @@ __global__ __launch_bounds__(kSmallArgsortThreads) void small_argsort_kernel(con
   }
 }
 
+// Many independent steps at once: `batch` sorts of n <= kSmallArgsortRows positions each, sort b reading
+// key[b * batch_stride + idx * stride], prev[b * n + .] and writing order_out[b * n + .].  A workgroup of T
+// threads takes `rows_per_block` sorts at a time (a power of two; T / rows_per_block threads each) with the
+// composites of its sorts in LDS; a thread keeps up to R positions of one sort in registers and counts, in one
+// pass over that sort's composites, how many of them precede each of its own.  Needs
+// n <= R * T / rows_per_block.  LDS: rows_per_block * row_stride doubles, row_stride >= n (odd when several
+// sorts share a workgroup, so that their reads fall into different banks).
+template <int T, int R>
+__global__ __launch_bounds__(T) void rows_argsort_kernel(const void* __restrict__ key, int kind, int64_t batch_stride, int64_t stride,
+                                                         int64_t batch, int n, int rows_per_block, int row_stride,
+                                                         const int* __restrict__ prev, int* __restrict__ order_out) {
+  extern __shared__ double rows_comp[];
+  const int group = T / rows_per_block;
+  const int local_row = threadIdx.x / group;
+  const int in_group = threadIdx.x - local_row * group;
+  for (int64_t row0 = (int64_t)blockIdx.x * rows_per_block; row0 < batch; row0 += (int64_t)gridDim.x * rows_per_block) {
+    const int64_t row = row0 + local_row;
+    const bool live = row < batch;
+    double* const comp = rows_comp + (size_t)local_row * row_stride;
+    const int* const prev_row = prev ? prev + row * n : nullptr;
+    if (live) {
+      for (int e = in_group; e < n; e += group) {
+        const int idx = prev_row ? prev_row[e] : e;
+        const int64_t at = row * batch_stride + (int64_t)idx * stride;
+        uint32_t k;
+        if (kind == kKeyFloat32)
+          k = ordered_key(static_cast<const float*>(key)[at]);
+        else if (kind == kKeyInt32)
+          k = static_cast<const uint32_t*>(key)[at] ^ 0x80000000u;
+        else
+          k = static_cast<const uint32_t*>(key)[at];
+        comp[e] = (double)(((uint64_t)k << 14) | (uint64_t)e);
+      }
+    }
+    __syncthreads();
+    double mine[R];
+    int before[R];
+#pragma unroll
+    for (int q = 0; q < R; ++q) {
+      const int e = in_group + q * group;
+      mine[q] = (live && e < n) ? comp[e] : 0.0;  // nothing precedes zero: idle positions count nothing
+      before[q] = 0;
+    }
+    if (live) {
+#pragma unroll 8
+      for (int b = 0; b < n; ++b) {
+        const double c = comp[b];
+#pragma unroll
+        for (int q = 0; q < R; ++q) before[q] += c < mine[q] ? 1 : 0;
+      }
+#pragma unroll
+      for (int q = 0; q < R; ++q) {
+        const int e = in_group + q * group;
+        if (e < n) order_out[row * n + before[q]] = prev_row ? prev_row[e] : e;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// Longer sorts of a batch, one workgroup per sort: the composites (key << 14 | position, distinct, so any
+// sorting network gives the stable order) go through a bitonic network in LDS, padded with +inf to npad, a
+// power of two from 512 to kRowsArgsortMax.  A thread takes eight entries at a time into registers and runs up
+// to three stages of the network on them before they go back, so a sort of 8192 makes 33 passes over LDS for
+// its 91 stages: entries 8t .. 8t+7 are sorted outright first (the phases of length 2, 4 and 8), and the
+// stages of a later phase are grouped by the index bits they pair, {2,1,0}, {5,4,3}, {8,7,6}, ..., the top
+// group taking what is left.  Entry e lives at e ^ swizzle(e), which keeps the 32 lanes of a half wave on 32
+// different banks in every full group.  O(n log^2 n) compare-exchanges per sort, where counting needs n^2
+// comparisons.
+constexpr int kRowsArgsortMax = 16384;  // positions per sort (14 bits of a composite), 128 KB of LDS
+constexpr int kRowsBitonicMin = 512;    // smallest padded length (one wave, eight entries per lane)
+
+__device__ inline int bitonic_slot(int e) { return e ^ ((e >> 5) & 7) ^ (((e >> 6) & 3) << 3); }
+
+__device__ inline void compare_exchange(double& a, double& b) {
+  const double lo = __builtin_fmin(a, b), hi = __builtin_fmax(a, b);
+  a = lo;
+  b = hi;
+}
+
+// The stages of phase k that pair entries differing in one of the S index bits low_log .. low_log + S - 1.
+template <int S>
+__device__ inline void bitonic_pass(double* comp, int npad, int k, int low_log) {
+  constexpr int E = 1 << S;
+  const int units = npad >> S;
+  for (int u = threadIdx.x; u < units; u += blockDim.x) {
+    const int base = ((u >> low_log) << (low_log + S)) | (u & ((1 << low_log) - 1));
+    const int flip = (base & k) ? E - 1 : 0;  // a descending run is an ascending one read backwards
+    double v[E];
+#pragma unroll
+    for (int c = 0; c < E; ++c) v[c] = comp[bitonic_slot(base + ((c ^ flip) << low_log))];
+#pragma unroll
+    for (int d = E >> 1; d > 0; d >>= 1)
+#pragma unroll
+      for (int c = 0; c < E; ++c)
+        if ((c & d) == 0) compare_exchange(v[c], v[c | d]);
+#pragma unroll
+    for (int c = 0; c < E; ++c) comp[bitonic_slot(base + ((c ^ flip) << low_log))] = v[c];
+  }
+}
+
+__global__ __launch_bounds__(1024) void rows_bitonic_argsort_kernel(const void* __restrict__ key, int kind, int64_t batch_stride,
+                                                                    int64_t stride, int64_t batch, int n, int npad,
+                                                                    const int* __restrict__ prev, int* __restrict__ order_out) {
+  extern __shared__ double bitonic_comp[];
+  double* const comp = bitonic_comp;
+  for (int64_t row = blockIdx.x; row < batch; row += gridDim.x) {
+    const int* const prev_row = prev ? prev + row * n : nullptr;
+    for (int e = threadIdx.x; e < npad; e += blockDim.x) {
+      double c = (double)INFINITY;
+      if (e < n) {
+        const int idx = prev_row ? prev_row[e] : e;
+        const int64_t at = row * batch_stride + (int64_t)idx * stride;
+        uint32_t k;
+        if (kind == kKeyFloat32)
+          k = ordered_key(static_cast<const float*>(key)[at]);
+        else if (kind == kKeyInt32)
+          k = static_cast<const uint32_t*>(key)[at] ^ 0x80000000u;
+        else
+          k = static_cast<const uint32_t*>(key)[at];
+        c = (double)(((uint64_t)k << 14) | (uint64_t)e);
+      }
+      comp[bitonic_slot(e)] = c;
+    }
+    __syncthreads();
+    // phases 2, 4 and 8: eight neighbours sorted in registers, every second run of eight descending
+    for (int u = threadIdx.x; u < (npad >> 3); u += blockDim.x) {
+      const int base = u << 3;
+      const int flip = (base & 8) ? 7 : 0;
+      double v[8];
+#pragma unroll
+      for (int c = 0; c < 8; ++c) v[c] = comp[bitonic_slot(base + (c ^ flip))];
+      compare_exchange(v[0], v[1]); compare_exchange(v[3], v[2]); compare_exchange(v[4], v[5]); compare_exchange(v[7], v[6]);
+      compare_exchange(v[0], v[2]); compare_exchange(v[1], v[3]); compare_exchange(v[6], v[4]); compare_exchange(v[7], v[5]);
+      compare_exchange(v[0], v[1]); compare_exchange(v[2], v[3]); compare_exchange(v[5], v[4]); compare_exchange(v[7], v[6]);
+#pragma unroll
+      for (int d = 4; d > 0; d >>= 1)
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+          if ((c & d) == 0) compare_exchange(v[c], v[c | d]);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) comp[bitonic_slot(base + (c ^ flip))] = v[c];
+    }
+    __syncthreads();
+    for (int k = 16, top = 3; k <= npad; k <<= 1, ++top) {  // top = the highest index bit that phase k pairs
+      int low_log = (top / 3) * 3;
+      const int first = top - low_log + 1;
+      if (first == 1)
+        bitonic_pass<1>(comp, npad, k, low_log);
+      else if (first == 2)
+        bitonic_pass<2>(comp, npad, k, low_log);
+      else
+        bitonic_pass<3>(comp, npad, k, low_log);
+      __syncthreads();
+      for (low_log -= 3; low_log >= 0; low_log -= 3) {
+        bitonic_pass<3>(comp, npad, k, low_log);
+        __syncthreads();
+      }
+    }
+    for (int e = threadIdx.x; e < n; e += blockDim.x) {
+      const int pos = (int)((uint64_t)comp[bitonic_slot(e)] & 16383ull);
+      order_out[row * n + e] = prev_row ? prev_row[pos] : pos;
+    }
+    __syncthreads();
+  }
+}
+
 }  // namespace evx

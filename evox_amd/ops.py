@@ -411,6 +411,41 @@ def _(key, kind, prev):
     return key.new_empty(key.shape, dtype=torch.int32)
 
 
+@torch.library.custom_op("evox_amd::stable_argsort_rows", mutates_args=())
+def stable_argsort_rows(key: torch.Tensor, kind: int, prev: Optional[torch.Tensor]) -> torch.Tensor:
+    """``stable_argsort_step`` for every row of a 2-D key at once: ``prev`` (int32 orders, one per row, or
+    None for the identity) rearranged, row by row, by a stable ascending sort of ``key[r, prev[r]]``.
+    The key may have any strides; ``prev`` is made contiguous.  Returns int32 orders of the key's shape."""
+    runtime.require_gpu_tensor(key, "key")
+    if key.dim() != 2 or key.element_size() != 4 or kind not in (0, 1, 2):
+        raise ValueError("key must be two-dimensional with 4-byte elements and kind 0, 1 or 2")
+    if (kind == 0) != (key.dtype == torch.float32):
+        raise TypeError(f"kind {kind} does not fit a key of dtype {key.dtype}")
+    batch, n = key.shape
+    out = torch.empty((batch, n), dtype=torch.int32, device=key.device)
+    if batch == 0 or n == 0:
+        return out
+    if prev is not None:
+        runtime.require_gpu_tensor(prev, "prev")
+        if prev.dtype != torch.int32 or prev.shape != (batch, n):
+            raise ValueError("prev must hold one int32 order per row of the key")
+        prev = prev.contiguous()
+    if key.stride(0) < 0 or key.stride(1) < 0:
+        key = key.contiguous()
+    with torch.cuda.device(key.device):
+        ws = runtime.sort_workspace(n, key.device)
+        stream = runtime.stream_handle(key.device)
+        _lib.call("evox_hip_stable_argsort_step_batched", key.data_ptr(), kind, key.stride(0), key.stride(1), batch, n,
+                  None if prev is None else prev.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
+        runtime.note_call(ws, stream)
+    return out
+
+
+@stable_argsort_rows.register_fake
+def _(key, kind, prev):
+    return key.new_empty(key.shape, dtype=torch.int32)
+
+
 @torch.library.custom_op("evox_amd::hv_contributions", mutates_args=())
 def hv_contributions(fit: torch.Tensor, samples: torch.Tensor, alpha: torch.Tensor, scale: float) -> torch.Tensor:
     """fit (N, M), samples (S, M), alpha (N,) float32 -> (N,) float32:

@@ -1,8 +1,9 @@
 """Drop-in replacement for ``evox.utils.lexsort`` (src/evox/utils/jit_fix_operator.py:213-252) on the GPU.
 
-The reference chains one stable ``torch.argsort`` per key; here every link of that chain is one launch of
-the segmented LSD radix sort that also orders large fronts inside the selection path
-(``evox_amd::stable_argsort_step``).
+The reference chains one stable ``torch.argsort`` per key; here every link of that chain is one stable
+argsort step on the GPU (``evox_amd::stable_argsort_step`` for a one-dimensional sort: a counting kernel up
+to 8192 positions, above that the segmented LSD radix sort that also orders large fronts inside the
+selection path; ``evox_amd::stable_argsort_rows`` for many sorts along one dimension at once).
 """
 
 from typing import List, Sequence, Tuple
@@ -49,14 +50,21 @@ def lexsort(keys: Sequence[torch.Tensor], dim: int = -1) -> torch.Tensor:
         raise ValueError("lexsort: all keys must have the same shape")
     if keys[0].dim() == 0:
         raise IndexError("lexsort: keys must have at least one dimension")
+    if keys[0].numel() == 0:
+        keys[0].size(dim)  # an IndexError for a dimension the keys do not have
+        return torch.empty(shape, dtype=torch.int64, device=keys[0].device)
     moved = [k.movedim(dim, -1) for k in keys]
     n = moved[0].shape[-1]
     rows = [m.reshape(-1, n) for m in moved]
-    out = torch.empty(rows[0].shape, dtype=torch.int64, device=keys[0].device)
-    for r in range(rows[0].size(0)):
-        order = None
+    order = None
+    if rows[0].size(0) == 1:
         for key_rows in rows:
-            for part, kind in _key_parts(key_rows[r]):
+            for part, kind in _key_parts(key_rows[0]):
                 order = ops.stable_argsort_step(part, kind, order)
-        out[r] = order.to(torch.int64)
+        out = order.to(torch.int64)
+    else:  # every row in the same launches
+        for key_rows in rows:
+            for part, kind in _key_parts(key_rows):
+                order = ops.stable_argsort_rows(part, kind, order)
+        out = order.to(torch.int64)
     return out.reshape(moved[0].shape).movedim(-1, dim)

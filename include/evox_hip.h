@@ -138,6 +138,16 @@ size_t evox_hip_argsort_workspace_bytes(int64_t n);
 int evox_hip_stable_argsort_step(const void* key, int kind, int64_t stride, int64_t n, const int32_t* prev_order,
                                  int32_t* order_out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same step for `batch` independent sorts of n positions each, which is lexsort along one dimension of
+ * keys with more dimensions (jit_fix_operator.py:246-250 with dim, the shape tournament selection sorts in,
+ * src/evox/operators/selection/tournament_selection.py:26): sort b reads key[b * batch_stride + i * stride]
+ * (strides in elements; batch_stride may be negative only if the addressed elements stay inside the buffer),
+ * prev_order + b * n and writes order_out + b * n.  Sorts of up to 8192 positions run together in one launch;
+ * longer ones run one after the other on the stream.  Workspace: evox_hip_argsort_workspace_bytes(n). */
+int evox_hip_stable_argsort_step_batched(const void* key, int kind, int64_t batch_stride, int64_t stride, int64_t batch,
+                                         int64_t n, const int32_t* prev_order, int32_t* order_out, void* workspace,
+                                         size_t workspace_bytes, void* stream);
+
 /* Monte-Carlo hypervolume contributions of HypE (src/evox/algorithms/mo/hype.py:29-39, the part of cal_hv
  * after the samples are drawn): out[i] = scale * sum over the samples s that point i covers
  * (all_k fit[i,k] <= sample[s,k]) of alpha[max(c_s - 1, 0)], c_s = the number of points that cover s.

@@ -69,6 +69,8 @@ def test_argument_validation_without_gpu(handle):
     assert handle.evox_hip_argsort_workspace_bytes(0) == 0 and handle.evox_hip_argsort_workspace_bytes(1000) > 16000
     assert handle.evox_hip_stable_argsort_step(p, 3, 1, 10, None, p, p, 64, None) == _lib.E_BAD_ARG
     assert handle.evox_hip_stable_argsort_step(p, 0, 1, 10, None, p, p, 64, None) == _lib.E_WORKSPACE
+    assert handle.evox_hip_stable_argsort_step_batched(p, 0, 10, 1, 0, 10, None, p, p, 1 << 20, None) == _lib.E_BAD_ARG
+    assert handle.evox_hip_stable_argsort_step_batched(p, 0, 10, 1, 4, 10, None, p, p, 64, None) == _lib.E_WORKSPACE
     assert handle.evox_hip_hv_workspace_bytes(0, 10) == 0 and handle.evox_hip_hv_workspace_bytes(100, 5000) >= 4 * (5000 + 5 * 100)
     assert handle.evox_hip_hv_contributions(p, p, p, 10, 0, 100, 1.0, p, p, 64, None) == _lib.E_BAD_ARG
     assert handle.evox_hip_hv_contributions(p, p, p, 10, 3, 100, 1.0, p, p, 64, None) == _lib.E_WORKSPACE

@@ -934,6 +934,41 @@ def test_lexsort_matches_numpy_and_the_restatement(population_path):
     assert torch.equal(lexsort([c.t().contiguous().to(DEV)], dim=-1).cpu(), er.chained_stable_argsort([c.t().contiguous()], dim=-1))
 
 
+def test_lexsort_along_a_dimension_of_many_sorts(population_path):
+    """Keys with more than one dimension (jit_fix_operator.py:246-250 with `dim`): every sort of the batch
+    in the same launches for up to 16384 positions, one after the other above that."""
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd.utils import lexsort
+
+    g = torch.Generator("cpu").manual_seed(15)
+    shapes = [(5, 1), (4000, 2), (130, 3), (9, 64), (37, 200), (3, 256), (3, 257), (5, 300), (2, 1000), (4, 1024), (3, 1025),
+              (2, 4096), (3, 4097), (9, 5000), (8, 8192), (2, 8192), (2, 8193), (2, 16384), (2, 16385), (3, 20000), (300, 2048), (0, 7), (6, 0)]
+    for batch, n in shapes:
+        say("lexsort rows", batch, n)
+        k_f32 = torch.randint(0, 9, (batch, n), generator=g).float() / 4 - 1
+        k_f32[torch.rand(batch, n, generator=g) < 0.03] = float("nan")
+        k_f32[torch.rand(batch, n, generator=g) < 0.03] = -0.0
+        k_i32 = torch.randint(-3, 3, (batch, n), generator=g, dtype=torch.int32)
+        k_f64 = 1.0 + torch.randint(0, 4, (batch, n), generator=g).double() * 1e-13
+        for keys in ([k_f32], [k_f32, k_i32], [k_f64, k_f32]):
+            want = er.chained_stable_argsort(keys, dim=-1)
+            got = lexsort([k.to(DEV) for k in keys], dim=-1)
+            assert got.dtype == torch.int64 and got.shape == want.shape and torch.equal(got.cpu(), want), (batch, n)
+    # a middle dimension, keys that are views, and the tournament's shape (tournament_selection.py:26)
+    a = torch.randint(0, 5, (6, 50, 7), generator=g).float()
+    b = torch.randint(0, 3, (6, 50, 7), generator=g, dtype=torch.int32)
+    for dim in (0, 1, 2, -2):
+        assert torch.equal(lexsort([a.to(DEV), b.to(DEV)], dim=dim).cpu(), er.chained_stable_argsort([a, b], dim=dim)), dim
+    at = a.to(DEV).transpose(0, 2)
+    assert torch.equal(lexsort([at, b.to(DEV).transpose(0, 2)], dim=1).cpu(),
+                       er.chained_stable_argsort([a.transpose(0, 2), b.transpose(0, 2)], dim=1))
+    wide = torch.rand(2, 8192, generator=g)[:, ::2]  # strided within the sort
+    assert torch.equal(lexsort([wide.to(DEV)[:, :]], dim=1).cpu(), er.chained_stable_argsort([wide], dim=1))
+    flipped = torch.rand(4, 33, generator=g)
+    assert torch.equal(lexsort([flipped.to(DEV).flip(0)], dim=1).cpu(), er.chained_stable_argsort([flipped.flip(0)], dim=1))
+
+
 def test_lexsort_gives_the_selection_order(population_path):
     """HypE's `lexsort([-dis, rank])[:pop_size]` (hype.py:143) and the selection's own final ordering
     (non_dominate.py:253) on the golden rank and distance of C3."""
