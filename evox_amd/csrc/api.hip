@@ -13,6 +13,7 @@
 #include "hv.hpp"
 #include "order.hpp"
 #include "peel.hpp"
+#include "prefix.hpp"
 #include "radix.hpp"
 
 namespace evx {
@@ -30,6 +31,9 @@ struct Options {
   unsigned spin_limit = 4000000u;
   int dominance_tile_words = 4;
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
+  int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 8 objectives (twice as
+                                    // many rows with 2) get their matrix from the per-objective orders (prefix.hpp);
+                                    // 0 = never
 };
 static Options g_opt;
 
@@ -48,6 +52,9 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->n = (int)n;
   L->m = (int)m;
   L->npad = (int)round_up(n, 128);
+  // the objectives are columns npad floats apart: at a multiple of 16 KB the same row of six or more columns
+  // competes for one set of the scalar cache (pairwise matrix of 65536 rows x 8: 1.19 ms, of 49152 rows: 0.42 ms)
+  if (L->npad % 4096 == 0 && n >= 16384) L->npad += 128;
   L->nwords = L->npad / 64;
   L->wstride = round_up(L->nwords, 16);
   L->kstride = (int)round_up(n, 64);
@@ -252,7 +259,17 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
   return 0;
 }
 
+// Measured (prefix against pairwise, us): 65536 x 3: 264 / 300, x 4: 301 / 391, x 8: 487 / 674; 49152 x 8: 391 / 417;
+// 32768 x 8: 355 / 221; 65536 x 2: 321 / 246; 131072 x 2: 818 / 1390; 200000 x 8: 2270 / 5310.
+static bool prefix_dominance_applies(const Layout& L) {
+  if (g_opt.prefix_min_rows <= 0 || L.m < 2 || L.m > kPrefixMaxObjectives) return false;
+  const int64_t least = L.m == 2 ? 2 * g_opt.prefix_min_rows : g_opt.prefix_min_rows;  // two objectives are cheap pair by pair
+  return L.n >= least && L.n > kRadixMinCandidates && L.n <= kPrefixMaxRows;
+}
+static int stage_dominance_prefix(const Ws& w, hipStream_t s);
+
 static int stage_dominance(const Ws& w, int variant, hipStream_t s) {
+  if (variant == kDomAuto && prefix_dominance_applies(w.L)) return stage_dominance_prefix(w, s);
   // (the lower triangle in tiles of 4 words keeps every SIMD busy with several waves; 16 is kept for
   // measurements)
   const int tile = g_opt.dominance_tile_words;
@@ -424,6 +441,57 @@ static int finish_grid(const Layout& L, int per_candidate_block) {
   return blocks < 1 ? 1 : blocks;
 }
 
+template <int M>
+static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
+  const Layout& L = w.L;
+  const int shift = prefix_bucket_shift(L.n);
+  const int buckets = ((L.n - 1) >> shift) + 1;
+  const size_t lds = prefix_lds_bytes(M, buckets);
+  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(dominance_prefix_kernel<M>), lds)) return e;
+  const int tiles = (int)round_up((L.nwords + kPrefixTileWords - 1) / kPrefixTileWords, 32);
+  // shorter stretches for smaller populations, so that the workgroups still outnumber the compute units
+  const int chunk = L.n >= 131072 ? kPrefixRowChunk : (L.n >= 65536 ? kPrefixRowChunk / 2 : kPrefixRowChunk / 4);
+  const int stretches = (L.n + chunk - 1) / chunk;
+  hipLaunchKernelGGL(dominance_prefix_kernel<M>, dim3(tiles, stretches), dim3(kPrefixThreads), lds, s, w.at<int>(L.pos),
+                     w.at<int>(L.scost), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.kstride, L.wstride, L.nwords,
+                     shift, buckets, chunk, w.at<SortParam>(L.sortparam));
+  EVX_LAUNCH_CHECK();
+  // a population with a NaN or an infinity: the pairwise kernel, on a grid that costs nothing when it has nothing to do
+  hipLaunchKernelGGL(dominance_nonfinite_kernel<M>, dim3(device_cus() * 8), dim3(256), 0, s, w.at<float>(L.xs_sorted),
+                     w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride,
+                     L.nwords, w.at<SortParam>(L.sortparam));
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+// The matrix of a large finite population from the order of its rows in every objective (prefix.hpp).  The
+// buffers of the crowding stage (radix pairs, pos, scost) are free until then and carry the orders.
+static int stage_dominance_prefix(const Ws& w, hipStream_t s) {
+  const Layout& L = w.L;
+  const size_t lds = sizeof(int) * (size_t)L.m * 4 * 256;
+  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(objective_order_kernel), lds)) return e;
+  hipLaunchKernelGGL(objective_order_kernel, dim3(radix_grid(L)), dim3(kRadixThreads), lds, s, w.at<float>(L.xs_sorted), L.npad, L.n,
+                     L.m, w.at<SortParam>(L.sortparam), w.ctrl(), w.at<int>(L.pos), w.at<int>(L.scost), radix_buffers(w),
+                     g_opt.spin_limit);
+  EVX_LAUNCH_CHECK();
+  // the barrier words of the control block restart from zero for the kernels that follow (the sort counted its
+  // generations from a high base)
+  const size_t first = offsetof(Ctrl, release);
+  const int64_t words = (int64_t)((sizeof(Ctrl) + sizeof(unsigned long long) * kMaxGrid - first) / 4);
+  hipLaunchKernelGGL(reset_state_kernel, dim3(16), dim3(256), 0, s, reinterpret_cast<uint32_t*>(w.base + L.ctrl + first), words);
+  EVX_LAUNCH_CHECK();
+  switch (L.m) {
+    case 2: return launch_dominance_prefix<2>(w, s);
+    case 3: return launch_dominance_prefix<3>(w, s);
+    case 4: return launch_dominance_prefix<4>(w, s);
+    case 5: return launch_dominance_prefix<5>(w, s);
+    case 6: return launch_dominance_prefix<6>(w, s);
+    case 7: return launch_dominance_prefix<7>(w, s);
+    case 8: return launch_dominance_prefix<8>(w, s);
+    default: return kErrBadArg;
+  }
+}
+
 // Per-objective ordering of the candidates list[ctrl.worst_start ... + ctrl.nv).
 static int stage_crowd_sort(const Ws& w, const int* list, hipStream_t s) {
   const Layout& L = w.L;
@@ -550,6 +618,8 @@ int evox_hip_set_option(const char* name, int64_t value) {
     g_opt.dominance_tile_words = (int)value;
   } else if (!strcmp(name, "small_sort") && (value == 0 || value == 1)) {
     g_opt.small_sort = (int)value;
+  } else if (!strcmp(name, "prefix_min_rows") && value >= 0) {
+    g_opt.prefix_min_rows = value;
   } else {
     return kErrBadArg;
   }

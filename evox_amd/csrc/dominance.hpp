@@ -375,17 +375,17 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
 }
 
 
-// grid.x = ceil(npad / 256) blocks of four 64-row groups, grid.y = ceil(nwords / IW) column tiles.
+// The tile of block (bx, by): bx = one of ceil(npad / 256) groups of four 64-row waves, by = one of
+// ceil(nwords / IW) column tiles.
 template <int M, int IW, int VARIANT>
-__global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
-                                                        const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom, int n,
-                                                        int npad, int64_t wstride, int nwords,
-                                                        const SortParam* __restrict__ param) {
+__device__ inline void dominance_tile(int bx, int by, const float* __restrict__ xs, const uint64_t* __restrict__ key,
+                                      const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom, int n, int npad,
+                                      int64_t wstride, int nwords, const SortParam* __restrict__ param) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int j = (blockIdx.x * 4 + wave) * 64 + lane;
+  const int j = (bx * 4 + wave) * 64 + lane;
   if (j - lane >= npad) return;  // whole wave past the padded population
-  const int w0 = blockIdx.y * IW;
+  const int w0 = by * IW;
   float xj[M];
 #pragma unroll
   for (int k = 0; k < M; ++k) xj[k] = xs[(int64_t)k * npad + j];
@@ -443,6 +443,29 @@ __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict_
       if (w < wend && w * 64 <= jlast) *reinterpret_cast<ulonglong2*>(out + w) = res[q];
     }
   }
+}
+
+// grid.x = ceil(npad / 256) blocks of four 64-row groups, grid.y = ceil(nwords / IW) column tiles.
+template <int M, int IW, int VARIANT>
+__global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
+                                                        const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom, int n,
+                                                        int npad, int64_t wstride, int nwords,
+                                                        const SortParam* __restrict__ param) {
+  dominance_tile<M, IW, VARIANT>((int)blockIdx.x, (int)blockIdx.y, xs, key, kid, dom, n, npad, wstride, nwords, param);
+}
+
+// The same matrix for a population that holds a NaN or an infinity, launched beside the kernels of prefix.hpp,
+// which only handle finite populations: any grid, every block takes tiles in turn; nothing to do (and nothing
+// done) when the population is finite.
+template <int M>
+__global__ __launch_bounds__(256) void dominance_nonfinite_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
+                                                                  const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom,
+                                                                  int n, int npad, int64_t wstride, int nwords,
+                                                                  const SortParam* __restrict__ param) {
+  if (param->nonfinite == 0) return;
+  const int gx = (npad + 255) / 256, gy = (nwords + 3) / 4;
+  for (int64_t t = blockIdx.x; t < (int64_t)gx * gy; t += gridDim.x)
+    dominance_tile<M, 4, kDomKey32>((int)(t % gx), (int)(t / gx), xs, key, kid, dom, n, npad, wstride, nwords, param);
 }
 
 // Any number of objectives (used above 8): same scheme, with the lane's own fitness re-read from

@@ -136,6 +136,59 @@ def test_dominance_bits_all_m(m):
             assert np.array_equal(got, want), (m, variant, bool(torch.isfinite(f).all()))
 
 
+def _matrix_words(f, variant, views_out=None):
+    """Raw words of the bit matrix (slot space) that readers look at, after prepare + dominance."""
+    n, m = f.shape
+    fd = f.to(DEV)
+    ws = runtime.workspace(n, m, fd.device)
+    s = runtime.stream_handle(fd.device)
+    _lib.call("evox_hip_stage_prepare", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), ws.data_ptr(), ws.numel(), s)
+    _lib.call("evox_hip_stage_dominance", n, m, variant, ws.data_ptr(), ws.numel(), s)
+    torch.cuda.synchronize()
+    views = runtime.workspace_views(ws, n, m)
+    words = np.ascontiguousarray(as_np(views["dom"])[:, : views["nwords"]]).view(np.uint64).copy()
+    words[defined_words(words.shape[0], words.shape[1]) == 0] = 0
+    return words
+
+
+@pytest.mark.parametrize("m", [2, 3, 4, 5, 6, 7, 8])
+def test_matrix_from_objective_orders_equals_the_pairwise_matrix(m):
+    """Large finite populations get their matrix from the order of the rows in every objective; it must be
+    the matrix of the pairwise test, word for word: ties, duplicate rows, constant objectives, a population
+    whose rows are all equal, signed zeros; and a NaN or an infinity hands the work back to the pairwise kernel."""
+    g = torch.Generator("cpu").manual_seed(700 + m)
+    cases = {}
+    cases["uniform"] = torch.rand(12345, m, generator=g)
+    cases["ties"] = torch.randint(0, 40, (9000, m), generator=g).float() / 8 - 2
+    dup = torch.rand(3000, m, generator=g)
+    cases["duplicates"] = dup[torch.randint(0, 3000, (8500,), generator=g)]
+    cases["all_equal"] = torch.full((8300, m), 1.5)
+    const = torch.rand(8400, m, generator=g)
+    const[:, m - 1] = -0.0
+    const[::3, m - 1] = 0.0
+    cases["constant_objective_signed_zeros"] = const
+    front = torch.rand(8200, m, generator=g)
+    front = front / front.sum(dim=1, keepdim=True)
+    cases["one_front"] = front
+    chain = torch.arange(8193, dtype=torch.float32)[:, None].repeat(1, m)
+    cases["chain"] = chain[torch.randperm(8193, generator=g)]
+    nan = torch.rand(8600, m, generator=g)
+    nan[17, 0] = float("nan")
+    nan[4000, m - 1] = float("inf")
+    cases["nonfinite"] = nan
+    cases["large"] = torch.rand(40000, m, generator=g)
+    try:
+        for name, f in cases.items():
+            say("prefix_matrix", m, name, tuple(f.shape))
+            runtime.set_option("prefix_min_rows", 4097)  # (twice as many rows with two objectives)
+            got = _matrix_words(f.contiguous(), 0)
+            runtime.set_option("prefix_min_rows", 0)
+            want = _matrix_words(f.contiguous(), 0)
+            assert np.array_equal(got, want), (m, name, int((got != want).sum()))
+    finally:
+        runtime.set_option("prefix_min_rows", 65536)
+
+
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 8, 11, 16])
 def test_dominance_arithmetic_form_corner_values(m):
     """A population of finite values takes the arithmetic form of the dominance test (signs of differences):
