@@ -448,7 +448,7 @@ static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
   const int buckets = ((L.n - 1) >> shift) + 1;
   const size_t lds = prefix_lds_bytes(M, buckets);
   if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(dominance_prefix_kernel<M>), lds)) return e;
-  const int tiles = (int)round_up((L.nwords + kPrefixTileWords - 1) / kPrefixTileWords, 32);
+  const int tiles = (int)round_up((L.nwords + kPrefixTileWords - 1) / kPrefixTileWords, 16);
   // shorter stretches for smaller populations, so that the workgroups still outnumber the compute units
   const int chunk = L.n >= 131072 ? kPrefixRowChunk : (L.n >= 65536 ? kPrefixRowChunk / 2 : kPrefixRowChunk / 4);
   const int stretches = (L.n + chunk - 1) / chunk;

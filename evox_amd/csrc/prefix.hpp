@@ -11,14 +11,15 @@
 //
 //  1. objective_order_kernel: one segmented radix sort orders the slots by every objective (radix.hpp) and
 //     leaves pos[k][slot] and upper[k][slot].
-//  2. dominance_prefix_kernel: a workgroup takes a tile of kPrefixTileSlots dominator slots (4 matrix words)
-//     and a stretch of rows below it.  Restricted to the tile, the prefix of objective k that belongs to row j
-//     is one of only 257 bit sets: the tile's own slots sorted by pos_k, the first t of them, where
-//     t = how many of them lie before upper_k(j).  The workgroup builds these tables in LDS (8 KB per
-//     objective) together with a coarse index from position to t; a lane then needs, per row and objective, one
-//     look-up of t (the coarse index, then a step or two along the tile's sorted positions) and one 32-byte read
-//     of the bit set, ANDed over the objectives: about 20 instructions per objective and 256 pairs, where the
-//     pairwise test needs 320.
+//  2. dominance_prefix_kernel: a workgroup takes a tile of kPrefixTileSlots dominator slots (8 matrix words,
+//     64 bytes of every row) and a stretch of rows below it.  Restricted to one word of the tile, the prefix of
+//     objective k that belongs to row j is one of only 65 bit sets: the word's own slots sorted by pos_k, the
+//     first c of them.  The workgroup builds in LDS, per objective: the tile's 512 positions in ascending
+//     order (mp), a coarse index from position to the number t of them that lie before it, for every t the
+//     eight counts c (how many of the first t fall into each word), and the 8 x 65 bit sets.  A lane then
+//     needs, per row and objective, one look-up of t (the coarse index, then a comparison or two along mp),
+//     one 8-byte read of the counts and eight 8-byte reads of bit sets, ANDed over the objectives: about
+//     55 instructions per objective and 512 pairs, where the pairwise test needs 640.
 #pragma once
 
 #include "common.hpp"
@@ -28,20 +29,25 @@
 
 namespace evx {
 
-constexpr int kPrefixTileWords = 4;
+constexpr int kPrefixTileWords = 8;
 constexpr int kPrefixTileSlots = 64 * kPrefixTileWords;
-constexpr int kPrefixMaxObjectives = 8;   // 8224 bytes of bit sets per objective
-constexpr int kPrefixBuckets = 512;       // entries of the coarse index per objective, at most (plus two)
+constexpr int kPrefixMaxObjectives = 8;   // 14.4 KB of LDS per objective
+constexpr int kPrefixBuckets = 1024;      // entries of the coarse index per objective, at most (plus two)
 constexpr int kPrefixThreads = 1024;
 constexpr int kPrefixRowChunk = 32768;    // rows per workgroup, at most (`chunk`, a multiple of 64)
 constexpr int kPrefixMaxRows = 1 << 22;   // a position and a slot of the tile share one int
 
-// LDS of dominance_prefix_kernel<M>.
+// LDS of dominance_prefix_kernel<M>, per objective: bit sets and counts (the scratch of the build lies over
+// them), sorted positions, the sorted (position, slot) pairs of the build, and the coarse index.
 __host__ __device__ inline size_t prefix_lds_bytes(int m, int buckets) {
-  const size_t sets = sizeof(uint64_t) * (size_t)m * (kPrefixTileSlots + 1) * kPrefixTileWords;  // also the histogram
-  const size_t members = sizeof(int) * (size_t)m * kPrefixTileSlots * 2;
-  const size_t index = (sizeof(uint32_t) * (size_t)m * (buckets + 2) + 15) & ~(size_t)15;
-  return sets + members + index;
+  const size_t sets = sizeof(uint64_t) * kPrefixTileWords * 65;
+  const size_t counts = sizeof(uint64_t) * (kPrefixTileSlots + 1);
+  const size_t scratch = sizeof(int) * (size_t)(buckets + 2) + sizeof(int) * kPrefixTileSlots;  // histogram, claimed
+  const size_t over = sets + counts > scratch ? sets + counts : scratch;
+  const size_t positions = sizeof(int) * (kPrefixTileSlots + 8);
+  const size_t sorted = sizeof(int) * kPrefixTileSlots;
+  const size_t index = (sizeof(uint16_t) * (size_t)(buckets + 2) + 7) & ~(size_t)7;
+  return (size_t)m * (over + positions + sorted + index);
 }
 
 // Positions are cut into at most kPrefixBuckets buckets of 2^shift positions.
@@ -101,10 +107,10 @@ __global__ __launch_bounds__(kRadixThreads) void objective_order_kernel(const fl
   }
 }
 
-// grid.x = the ceil(nwords / kPrefixTileWords) tiles of dominator slots, rounded up to a multiple of 32,
-// grid.y = stretches of `chunk` rows, counted from the first row of the tile (rows above it have no
-// word there).  Dynamic LDS:
-// prefix_lds_bytes(M, buckets).  Writes words 4 * blockIdx.x .. + 3 of every row of the stretch.
+// grid.x = the ceil(nwords / kPrefixTileWords) tiles of dominator slots, rounded up to a multiple of 16,
+// grid.y = stretches of `chunk` rows, counted from the first row of the tile (rows above it have no word
+// there).  Dynamic LDS: prefix_lds_bytes(M, buckets).  Writes the eight words of the tile in every row of the
+// stretch.
 template <int M>
 __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const int* __restrict__ pos, const int* __restrict__ upper,
                                                                           const uint32_t* __restrict__ kid,
@@ -114,13 +120,13 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
   constexpr int WW = kPrefixTileWords, TS = kPrefixTileSlots, T = kPrefixThreads;
   extern __shared__ uint64_t prefix_lds[];
   if (param->nonfinite != 0) return;
-  // Workgroups go to the eight dies in turn (linear index modulo 8), and a die has its own L2.  The four tiles
+  // Workgroups go to the eight dies in turn (linear index modulo 8), and a die has its own L2.  The two tiles
   // that share the 128-byte lines of the matrix are given to consecutive workgroups of one die, which run
-  // side by side over the same rows: their 32-byte pieces of a line then meet in that L2 and leave as one line.
+  // side by side over the same rows: their halves of a line then meet in that L2 and leave as one line.
   const int64_t linear = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
   const int die = (int)(linear & 7);
   const int seq = (int)blockIdx.x >> 3;  // this workgroup among those of its die in this row of the grid
-  const int tile = 4 * ((seq >> 2) * 8 + die) + (seq & 3);
+  const int tile = 2 * ((seq >> 1) * 8 + die) + (seq & 1);
   if (tile * WW >= nwords) return;
   const int w0 = tile * WW;
   const int slot0 = w0 * 64;
@@ -129,16 +135,25 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
   const int r0 = (int)first_row;
   const int r1 = (int)(first_row + chunk < n ? first_row + chunk : n);
   const int HB = buckets + 2;  // entries of the coarse index per objective
-  uint64_t* const sets = prefix_lds;                                          // [M][TS + 1][WW]
-  int* const hist = reinterpret_cast<int*>(sets);                             // [M][HB] while the tables are built
-  int* const member = reinterpret_cast<int*>(sets + (size_t)M * (TS + 1) * WW);  // [M][TS]: position << 8 | slot in tile, ascending
-  int* const claimed = member + M * TS;                                       // [M][TS]: the same, unordered inside a bucket
-  uint32_t* const index = reinterpret_cast<uint32_t*>(claimed + M * TS);      // [M][HB]: members before the bucket | members in it << 16
+  // per objective k (all arrays [M][...]):
+  constexpr int kSetWords = WW * 65;                 // sets[k][w][c]: the slots of the first c members of word w
+  constexpr int kOver = kSetWords + TS + 1;          // ... then counts[k][t]: eight byte counts, members of each word among the first t
+  const int scratch_words = (HB + TS + 1) / 2;       // histogram and claimed pairs of the build, in the same place
+  const int over = kOver > scratch_words ? kOver : scratch_words;
+  uint64_t* const sets = prefix_lds;
+  uint64_t* const counts = sets + kSetWords;
+  int* const mp = reinterpret_cast<int*>(prefix_lds + (size_t)M * over);  // [M][TS + 8]: positions ascending, then INT_MAX
+  int* const sorted = mp + M * (TS + 8);                                     // [M][TS]: position << 9 | slot in tile, ascending
+  uint16_t* const index = reinterpret_cast<uint16_t*>(sorted + M * TS);      // [M][HB]: members in earlier buckets
+  auto hist_of = [&](int k) { return reinterpret_cast<int*>(prefix_lds + (size_t)k * over); };  // [HB]
+  auto claimed_of = [&](int k) { return hist_of(k) + HB; };                                        // [TS]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int live = n - slot0 < TS ? n - slot0 : TS;  // slots of the tile that hold a row
+  const int index_stride = (HB + 3) & ~3;
 
   // ---- the tile's slots by position, objective by objective
-  for (int t = threadIdx.x; t < M * HB; t += T) hist[t] = 0;
+  for (int t = threadIdx.x; t < M * HB; t += T) hist_of(t / HB)[t % HB] = 0;
+  for (int t = threadIdx.x; t < M * (TS + 8); t += T) mp[t] = 0x7FFFFFFF;
   __syncthreads();
   constexpr int PER = (M * TS + T - 1) / T;
   int mine[PER];
@@ -149,8 +164,8 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
     mine[u] = -1;
     if (item < M * TS && i < live) {
       const int p = pos[(int64_t)k * kstride + slot0 + i];
-      mine[u] = (p << 8) | i;
-      atomicAdd(&hist[k * HB + (p >> shift)], 1);
+      mine[u] = (p << 9) | i;
+      atomicAdd(&hist_of(k)[p >> shift], 1);
     }
   }
   __syncthreads();
@@ -158,14 +173,14 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
     int carry = 0;
     for (int b0 = 0; b0 < HB; b0 += 64) {
       const int b = b0 + lane;
-      const int v = b < HB ? hist[wave * HB + b] : 0;
+      const int v = b < HB ? hist_of(wave)[b] : 0;
       int incl = v;
 #pragma unroll
       for (int off = 1; off < 64; off <<= 1) {
         const int up = __shfl_up(incl, off);
         if (lane >= off) incl += up;
       }
-      if (b < HB) index[wave * HB + b] = (uint32_t)(carry + incl - v) | ((uint32_t)v << 16);
+      if (b < HB) index[wave * index_stride + b] = (uint16_t)(carry + incl - v);
       carry += __shfl(incl, 63);
     }
   }
@@ -174,9 +189,9 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
   for (int u = 0; u < PER; ++u) {
     if (mine[u] >= 0) {
       const int k = (threadIdx.x + u * T) / TS;
-      const int b = (mine[u] >> 8) >> shift;
-      const int r = atomicSub(&hist[k * HB + b], 1) - 1;
-      claimed[k * TS + (int)(index[k * HB + b] & 0xFFFFu) + r] = mine[u];
+      const int b = (mine[u] >> 9) >> shift;
+      const int r = atomicSub(&hist_of(k)[b], 1) - 1;
+      claimed_of(k)[(int)index[k * index_stride + b] + r] = mine[u];
     }
   }
   __syncthreads();
@@ -184,41 +199,62 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
   for (int u = 0; u < PER; ++u) {
     if (mine[u] >= 0) {
       const int k = (threadIdx.x + u * T) / TS;
-      const int b = (mine[u] >> 8) >> shift;
-      const uint32_t entry = index[k * HB + b];
-      const int t0 = (int)(entry & 0xFFFFu), t1 = t0 + (int)(entry >> 16);
+      const int b = (mine[u] >> 9) >> shift;
+      const int t0 = index[k * index_stride + b], t1 = index[k * index_stride + b + 1];
       int before = 0;
-      for (int t = t0; t < t1; ++t) before += claimed[k * TS + t] < mine[u] ? 1 : 0;
-      member[k * TS + t0 + before] = mine[u];
+      for (int t = t0; t < t1; ++t) before += claimed_of(k)[t] < mine[u] ? 1 : 0;
+      sorted[k * TS + t0 + before] = mine[u];
+      mp[k * (TS + 8) + t0 + before] = mine[u] >> 9;
     }
   }
   __syncthreads();
-  // ---- sets[k][t] = the slots of the first t members of objective k; a wave per (objective, word)
+  // ---- counts[k][t] and the single bits of sets[k][w][c + 1]; a wave per objective, a lane per eight members
+  for (int t = threadIdx.x; t < M * kSetWords; t += T) sets[(size_t)(t / kSetWords) * over + t % kSetWords] = 0ull;
+  __syncthreads();
+  for (int k = wave; k < M; k += T / 64) {
+    uint64_t one[8];
+    uint64_t sum = 0ull;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const int t = 8 * lane + c;
+      one[c] = t < live ? 1ull << (8 * ((sorted[k * TS + t] & (TS - 1)) >> 6)) : 0ull;
+      sum += one[c];
+    }
+    uint64_t incl = sum;  // byte-wise counts: at most 64 per byte, no carry between bytes
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const uint64_t up = __shfl_up(incl, off);
+      if (lane >= off) incl += up;
+    }
+    uint64_t run = incl - sum;  // members before this lane's eight
+    uint64_t* const cnt = counts + (size_t)k * over;
+    uint64_t* const set = sets + (size_t)k * over;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const int t = 8 * lane + c;
+      cnt[t] = run;
+      if (t < live) {
+        const int i = sorted[k * TS + t] & (TS - 1);
+        const int w = i >> 6;
+        const int rank_in_word = (int)((run >> (8 * w)) & 255ull);
+        set[w * 65 + rank_in_word + 1] = 1ull << (i & 63);
+      }
+      run += one[c];
+    }
+    if (lane == 63) cnt[TS] = run;
+  }
+  __syncthreads();
+  // ---- sets[k][w][c] = OR of the single bits up to c; a wave per (objective, word)
   for (int item = wave; item < M * WW; item += T / 64) {
     const int k = item / WW, w = item - k * WW;
-    uint64_t bits[4];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int t = 4 * lane + c;
-      const int ent = t < live ? member[k * TS + t] : -1;
-      const int i = ent & 255;
-      bits[c] = (ent >= 0 && (i >> 6) == w) ? 1ull << (i & 63) : 0ull;
-    }
-    const uint64_t b0 = bits[0], b1 = b0 | bits[1], b2 = b1 | bits[2], b3 = b2 | bits[3];
-    uint64_t incl = b3;
+    uint64_t* const col = sets + (size_t)k * over + w * 65;
+    uint64_t incl = col[lane + 1];
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
       const uint64_t up = __shfl_up(incl, off);
       if (lane >= off) incl |= up;
     }
-    uint64_t excl = __shfl_up(incl, 1);
-    if (lane == 0) excl = 0ull;
-    uint64_t* const col = sets + (size_t)k * (TS + 1) * WW + w;
-    col[(size_t)(4 * lane + 0) * WW] = excl;
-    col[(size_t)(4 * lane + 1) * WW] = excl | b0;
-    col[(size_t)(4 * lane + 2) * WW] = excl | b1;
-    col[(size_t)(4 * lane + 3) * WW] = excl | b2;
-    if (lane == 63) col[(size_t)TS * WW] = excl | b3;
+    col[lane + 1] = incl;
   }
   __syncthreads();
 
@@ -242,53 +278,33 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
     for (int k = 0; k < M; ++k) e[k] = e_next[k];
     const int same_from = same_next;  // slots from here on hold rows with the key of row j, or larger keys
     if (g + T / 64 < groups) fetch(g + T / 64);
-    // t[k] = members of objective k that lie before upper_k(j): those of the earlier buckets, then a step or
-    // two inside the bucket (the look-ups of all objectives are in flight together)
-    int t[M], t1[M];
-#pragma unroll
-    for (int k = 0; k < M; ++k) {
-      const uint32_t entry = index[k * HB + (e[k] >> shift)];
-      t[k] = (int)(entry & 0xFFFFu);
-      t1[k] = t[k] + (int)(entry >> 16);
-    }
+    // t[k] = members of objective k that lie before upper_k(j): those of the earlier buckets plus those of the
+    // bucket itself that do (positions ascend, so the members from t on that lie before it are consecutive)
+    int t[M];
     bool more = false;
 #pragma unroll
-    for (int step = 0; step < 2; ++step) {
-      int first[M];
+    for (int k = 0; k < M; ++k) t[k] = index[k * index_stride + (e[k] >> shift)];
 #pragma unroll
-      for (int k = 0; k < M; ++k) first[k] = member[k * TS + (t[k] < TS ? t[k] : TS - 1)];
-#pragma unroll
-      for (int k = 0; k < M; ++k) {
-        const bool advance = t[k] < t1[k] && (first[k] >> 8) < e[k];
-        t[k] += advance ? 1 : 0;
-        if (step == 1) more |= advance && t[k] < t1[k];
-      }
+    for (int k = 0; k < M; ++k) {
+      const int m0 = mp[k * (TS + 8) + t[k]], m1 = mp[k * (TS + 8) + t[k] + 1];
+      const int a0 = m0 < e[k] ? 1 : 0, a1 = m1 < e[k] ? 1 : 0;
+      t[k] += a0 + a1;
+      more |= a1 != 0;
     }
-    if (__builtin_amdgcn_ballot_w64(more) != 0ull) {  // a bucket with three or more members of the tile: rare
+    if (__builtin_amdgcn_ballot_w64(more) != 0ull) {  // three or more members of the tile in one bucket: rare
 #pragma unroll
       for (int k = 0; k < M; ++k)
-        while (t[k] < t1[k] && (member[k * TS + t[k]] >> 8) < e[k]) ++t[k];
+        while (mp[k * (TS + 8) + t[k]] < e[k]) ++t[k];
     }
     uint64_t d[WW];
-    {
-      ulonglong2 lo[M], hi[M];
 #pragma unroll
-      for (int k = 0; k < M; ++k) {
-        const ulonglong2* const set = reinterpret_cast<const ulonglong2*>(sets + ((size_t)k * (TS + 1) + t[k]) * WW);
-        lo[k] = set[0];
-        hi[k] = set[1];
-      }
-      d[0] = lo[0].x;
-      d[1] = lo[0].y;
-      d[2] = hi[0].x;
-      d[3] = hi[0].y;
+    for (int w = 0; w < WW; ++w) d[w] = ~0ull;
 #pragma unroll
-      for (int k = 1; k < M; ++k) {
-        d[0] &= lo[k].x;
-        d[1] &= lo[k].y;
-        d[2] &= hi[k].x;
-        d[3] &= hi[k].y;
-      }
+    for (int k = 0; k < M; ++k) {
+      const uint64_t c8 = counts[(size_t)k * over + t[k]];
+      const uint64_t* const set = sets + (size_t)k * over;
+#pragma unroll
+      for (int w = 0; w < WW; ++w) d[w] &= set[w * 65 + (int)((c8 >> (8 * w)) & 255ull)];
     }
 #pragma unroll
     for (int w = 0; w < WW; ++w) {
@@ -300,8 +316,8 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
     }
     if (j < n) {
       ulonglong2* const out = reinterpret_cast<ulonglong2*>(dom + (int64_t)j * wstride + w0);
-      out[0] = make_ulonglong2(d[0], d[1]);
-      out[1] = make_ulonglong2(d[2], d[3]);
+#pragma unroll
+      for (int q = 0; q < WW / 2; ++q) out[q] = make_ulonglong2(d[2 * q], d[2 * q + 1]);
     }
   }
 }
