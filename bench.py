@@ -411,8 +411,8 @@ def main():
     # ones at about 32 T; mixed as in the arithmetic form they sustain about 52 T (calibration kind 3)
     finite = bool(torch.isfinite(f).all())
     # large finite populations get the matrix from the order of the rows in every objective instead (the library's
-    # rule: at least 65536 rows with 3 to 8 objectives, 131072 with 2): no pairwise test is executed at all
-    from_orders = finite and ((3 <= m <= 8 and n >= 65536) or (m == 2 and n >= 131072))
+    # rule: at least 65536 rows with 3 to 10 objectives, 81920 with 2): no pairwise test is executed at all
+    from_orders = finite and ((3 <= m <= 10 and n >= 65536) or (m == 2 and n >= 81920))
     valu_per_pair = m + (m // 2) + 2 if finite else m + 2
     executed_valu = valu_per_pair * evaluated_pairs
     executed_peak = VALU_FP32_PEAK_GOPS if finite else VALU_CMP_PEAK_GOPS
@@ -439,7 +439,7 @@ def main():
         "order": {"us": times["order_us"]},
     }
     if from_orders:
-        # bound by the stores of the matrix (32-byte pieces of rows that lie kilobytes apart); the reference's
+        # bound by the stores of the matrix (64-byte pieces of rows that lie kilobytes apart); the reference's
         # compares over the same time stay as the algorithmic figure
         phases["dominance"] = {"us": times["dominance_us"], "bound": "hbm", "achieved": dom_bytes / times["dominance_us"] / 1e3,
                                "peak": HBM_PEAK_GBS, "unit": "GB/s", "executed_form": "objective orders",

@@ -31,8 +31,8 @@ struct Options {
   unsigned spin_limit = 4000000u;
   int dominance_tile_words = 4;
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
-  int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 8 objectives (twice as
-                                    // many rows with 2) get their matrix from the per-objective orders (prefix.hpp);
+  int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 10 objectives (a quarter
+                                    // more rows with 2) get their matrix from the per-objective orders (prefix.hpp);
                                     // 0 = never
 };
 static Options g_opt;
@@ -259,11 +259,12 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
   return 0;
 }
 
-// Measured (prefix against pairwise, us): 65536 x 3: 264 / 300, x 4: 301 / 391, x 8: 487 / 674; 49152 x 8: 391 / 417;
-// 32768 x 8: 355 / 221; 65536 x 2: 321 / 246; 131072 x 2: 818 / 1390; 200000 x 8: 2270 / 5310.
+// Measured (matrix from the orders against pairwise, us): 49152 x 8: 373 / 373; 65536 x 2: 239 / 227, x 3: 277 / 287,
+// x 4: 305 / 366, x 8: 451 / 637; 100000 x 2: 370 / 558, x 3: 408 / 709; 200000 x 3: 1268 / 2622, x 8: 1624 / 5340.
 static bool prefix_dominance_applies(const Layout& L) {
   if (g_opt.prefix_min_rows <= 0 || L.m < 2 || L.m > kPrefixMaxObjectives) return false;
-  const int64_t least = L.m == 2 ? 2 * g_opt.prefix_min_rows : g_opt.prefix_min_rows;  // two objectives are cheap pair by pair
+  // (two objectives are cheap pair by pair: a quarter more rows before the orders pay)
+  const int64_t least = L.m == 2 ? g_opt.prefix_min_rows + g_opt.prefix_min_rows / 4 : g_opt.prefix_min_rows;
   return L.n >= least && L.n > kRadixMinCandidates && L.n <= kPrefixMaxRows;
 }
 static int stage_dominance_prefix(const Ws& w, hipStream_t s);
@@ -488,6 +489,8 @@ static int stage_dominance_prefix(const Ws& w, hipStream_t s) {
     case 6: return launch_dominance_prefix<6>(w, s);
     case 7: return launch_dominance_prefix<7>(w, s);
     case 8: return launch_dominance_prefix<8>(w, s);
+    case 9: return launch_dominance_prefix<9>(w, s);
+    case 10: return launch_dominance_prefix<10>(w, s);
     default: return kErrBadArg;
   }
 }

@@ -31,7 +31,7 @@ namespace evx {
 
 constexpr int kPrefixTileWords = 8;
 constexpr int kPrefixTileSlots = 64 * kPrefixTileWords;
-constexpr int kPrefixMaxObjectives = 8;   // 14.4 KB of LDS per objective
+constexpr int kPrefixMaxObjectives = 10;  // 14.4 KB of LDS per objective
 constexpr int kPrefixBuckets = 1024;      // entries of the coarse index per objective, at most (plus two)
 constexpr int kPrefixThreads = 1024;
 constexpr int kPrefixRowChunk = 32768;    // rows per workgroup, at most (`chunk`, a multiple of 64)
@@ -254,7 +254,8 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
       const uint64_t up = __shfl_up(incl, off);
       if (lane >= off) incl |= up;
     }
-    col[lane + 1] = incl;
+    col[lane + 1] = ~incl;  // kept complemented: a row ORs the complements of its M sets (three-input ORs) and
+    if (lane == 0) col[0] = ~0ull;  // complements once
   }
   __syncthreads();
 
@@ -296,23 +297,28 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
       for (int k = 0; k < M; ++k)
         while (mp[k * (TS + 8) + t[k]] < e[k]) ++t[k];
     }
-    uint64_t d[WW];
+    uint64_t d[WW];  // slots that are worse than row j in some objective
 #pragma unroll
-    for (int w = 0; w < WW; ++w) d[w] = ~0ull;
+    for (int w = 0; w < WW; ++w) d[w] = 0ull;
 #pragma unroll
     for (int k = 0; k < M; ++k) {
       const uint64_t c8 = counts[(size_t)k * over + t[k]];
       const uint64_t* const set = sets + (size_t)k * over;
 #pragma unroll
-      for (int w = 0; w < WW; ++w) d[w] &= set[w * 65 + (int)((c8 >> (8 * w)) & 255ull)];
+      for (int w = 0; w < WW; ++w) d[w] |= set[w * 65 + (int)((c8 >> (8 * w)) & 255ull)];
     }
 #pragma unroll
-    for (int w = 0; w < WW; ++w) {
-      const int first = (w0 + w) * 64;
-      if (same_from <= first)
-        d[w] = 0ull;
-      else if (same_from < first + 64)
-        d[w] &= (1ull << (same_from - first)) - 1ull;
+    for (int w = 0; w < WW; ++w) d[w] = ~d[w];
+    // rows identical to j and everything after them: only near the diagonal (wave-uniform test)
+    if (__builtin_amdgcn_ballot_w64(same_from < slot0 + TS) != 0ull) {
+#pragma unroll
+      for (int w = 0; w < WW; ++w) {
+        const int first = (w0 + w) * 64;
+        if (same_from <= first)
+          d[w] = 0ull;
+        else if (same_from < first + 64)
+          d[w] &= (1ull << (same_from - first)) - 1ull;
+      }
     }
     if (j < n) {
       ulonglong2* const out = reinterpret_cast<ulonglong2*>(dom + (int64_t)j * wstride + w0);

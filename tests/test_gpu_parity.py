@@ -151,7 +151,7 @@ def _matrix_words(f, variant, views_out=None):
     return words
 
 
-@pytest.mark.parametrize("m", [2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("m", [2, 3, 4, 5, 6, 7, 8, 9, 10])
 def test_matrix_from_objective_orders_equals_the_pairwise_matrix(m):
     """Large finite populations get their matrix from the order of the rows in every objective; it must be
     the matrix of the pairwise test, word for word: ties, duplicate rows, constant objectives, a population
@@ -180,7 +180,7 @@ def test_matrix_from_objective_orders_equals_the_pairwise_matrix(m):
     try:
         for name, f in cases.items():
             say("prefix_matrix", m, name, tuple(f.shape))
-            runtime.set_option("prefix_min_rows", 4097)  # (twice as many rows with two objectives)
+            runtime.set_option("prefix_min_rows", 4097)  # (a quarter more rows with two objectives)
             got = _matrix_words(f.contiguous(), 0)
             runtime.set_option("prefix_min_rows", 0)
             want = _matrix_words(f.contiguous(), 0)
