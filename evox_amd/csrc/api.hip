@@ -267,10 +267,12 @@ static bool prefix_dominance_applies(const Layout& L) {
   const int64_t least = L.m == 2 ? g_opt.prefix_min_rows + g_opt.prefix_min_rows / 4 : g_opt.prefix_min_rows;
   return L.n >= least && L.n > kRadixMinCandidates && L.n <= kPrefixMaxRows;
 }
-static int stage_dominance_prefix(const Ws& w, hipStream_t s);
+static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s);
 
 static int stage_dominance(const Ws& w, int variant, hipStream_t s) {
-  if (variant == kDomAuto && prefix_dominance_applies(w.L)) return stage_dominance_prefix(w, s);
+  // (kDomOrdersOnly: the first half of the path below alone, for measurements of the second)
+  if (variant == kDomOrdersOnly) return prefix_dominance_applies(w.L) ? stage_dominance_prefix(w, true, s) : kErrBadArg;
+  if (variant == kDomAuto && prefix_dominance_applies(w.L)) return stage_dominance_prefix(w, false, s);
   // (the lower triangle in tiles of 4 words keeps every SIMD busy with several waves; 16 is kept for
   // measurements)
   const int tile = g_opt.dominance_tile_words;
@@ -467,7 +469,7 @@ static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
 
 // The matrix of a large finite population from the order of its rows in every objective (prefix.hpp).  The
 // buffers of the crowding stage (radix pairs, pos, scost) are free until then and carry the orders.
-static int stage_dominance_prefix(const Ws& w, hipStream_t s) {
+static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) {
   const Layout& L = w.L;
   const size_t lds = sizeof(int) * (size_t)L.m * 4 * 256;
   if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(objective_order_kernel), lds)) return e;
@@ -481,6 +483,7 @@ static int stage_dominance_prefix(const Ws& w, hipStream_t s) {
   const int64_t words = (int64_t)((sizeof(Ctrl) + sizeof(unsigned long long) * kMaxGrid - first) / 4);
   hipLaunchKernelGGL(reset_state_kernel, dim3(16), dim3(256), 0, s, reinterpret_cast<uint32_t*>(w.base + L.ctrl + first), words);
   EVX_LAUNCH_CHECK();
+  if (orders_only) return 0;
   switch (L.m) {
     case 2: return launch_dominance_prefix<2>(w, s);
     case 3: return launch_dominance_prefix<3>(w, s);

@@ -254,7 +254,7 @@ __global__ __launch_bounds__(kSmallSortThreads) void small_sort_kernel(
   for (int64_t w = tid; w < n_zero_words; w += (int64_t)gridDim.x * blockDim.x) zero_words[w] = 0u;
 }
 
-enum DomVariant { kDomAuto = 0, kDomTwoCompares = 1, kDomKey64 = 2, kDomKey32 = 3, kDomArith = 4 };
+enum DomVariant { kDomAuto = 0, kDomTwoCompares = 1, kDomKey64 = 2, kDomKey32 = 3, kDomArith = 4, kDomOrdersOnly = 5 };
 
 // acc = (acc << 1) | bit, with the bit taken from a 64-lane mask: one v_addc_co_u32.
 __device__ inline uint32_t shift_in(uint32_t acc, uint64_t mask) {

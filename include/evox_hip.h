@@ -184,9 +184,11 @@ int evox_hip_calibration_launch(int kind, int64_t blocks, int64_t iterations, fl
 int evox_hip_stage_prepare(const float* f, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col, void* workspace,
                            size_t workspace_bytes, void* stream);
 /* The pairwise dominance bit matrix (non_dominate.py:6-26) in slot space.  variant 0 = production
- * kernel (signs of differences when every value is finite, else compares plus "differs somewhere" from a 32-bit
- * stand-in of the row key), 1 = check kernel that evaluates both `<=` and `<` per objective as the reference
- * does, 2 = the compare form on the 64-bit row keys themselves, 3 = the compare form whatever the values. */
+ * path (large finite populations: from the order of the rows in every objective; else pair by pair, by the signs
+ * of differences when every value is finite, else by compares plus "differs somewhere" from a 32-bit stand-in of
+ * the row key), 1 = check kernel that evaluates both `<=` and `<` per objective as the reference does, 2 = the
+ * compare form on the 64-bit row keys themselves, 3 = the compare form whatever the values, 5 = only the
+ * per-objective orders of the production path (an error where that path does not apply; for measurements). */
 int evox_hip_stage_dominance(int64_t n, int64_t m, int variant, void* workspace, size_t workspace_bytes, void* stream);
 /* Domination counts by row popcount (non_dominate.py:188) and front 0 (:192).  Resets the peeling
  * state first, so count -> peel can be repeated on one dominance matrix. */
