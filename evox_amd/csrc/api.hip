@@ -42,7 +42,7 @@ struct Layout {
   int64_t wstride;
   // byte offsets
   size_t ctrl, fsize, fronts_slot, fronts_orig, hist, zero_end, fstart, xs, key, partials, sortparam, bstart, bcursor,
-      scanflags, records, members, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
+      scanflags, records, members, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, total0, witness0, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
 };
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
@@ -87,6 +87,10 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->orig_of = o;    o = align_up(o + sizeof(int) * (size_t)L->npad);
   L->count = o;      o = align_up(o + sizeof(int) * (size_t)n);
   L->witness = o;    o = align_up(o + sizeof(int) * (size_t)n);
+  // popcount and highest non-empty word of every row as the order-based dominance kernel leaves them (kept apart
+  // from count / witness, which the peel consumes, so that the count stage can be repeated)
+  L->total0 = o;     o = align_up(o + sizeof(int) * (size_t)n);
+  L->witness0 = o;   o = align_up(o + sizeof(int) * (size_t)n);
   L->rank = o;       o = align_up(o + sizeof(int) * (size_t)n);
   L->dist = o;       o = align_up(o + sizeof(float) * (size_t)n);
   L->perm = o;       o = align_up(o + sizeof(int) * (size_t)n);
@@ -294,8 +298,17 @@ static int stage_count(const Ws& w, bool fill_dist, hipStream_t s) {
   hipLaunchKernelGGL(count_kernel, dim3(blocks), dim3(256), 0, s, w.at<uint64_t>(L.dom), L.wstride, L.n,
                      w.at<int>(L.orig_of), w.at<int>(L.count), w.at<int>(L.rank), w.at<int>(L.witness),
                      w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
-                     fill_dist ? w.at<float>(L.dist) : (float*)nullptr, w.ctrl());
+                     fill_dist ? w.at<float>(L.dist) : (float*)nullptr, w.ctrl(), w.at<SortParam>(L.sortparam));
   EVX_LAUNCH_CHECK();
+  if (prefix_dominance_applies(L)) {
+    // the order-based dominance kernel has left the popcounts: count_kernel above returned at once (the choice is
+    // made on the device: a population with a NaN or an infinity went through the pairwise kernel and is counted there)
+    hipLaunchKernelGGL(count_from_totals_kernel, dim3((L.n + 255) / 256), dim3(256), 0, s, w.at<int>(L.total0),
+                       w.at<int>(L.witness0), L.n, w.at<int>(L.orig_of), w.at<int>(L.count), w.at<int>(L.rank),
+                       w.at<int>(L.witness), w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
+                       fill_dist ? w.at<float>(L.dist) : (float*)nullptr, w.ctrl(), w.at<SortParam>(L.sortparam));
+    EVX_LAUNCH_CHECK();
+  }
   return 0;
 }
 
@@ -457,7 +470,7 @@ static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
   const int stretches = (L.n + chunk - 1) / chunk;
   hipLaunchKernelGGL(dominance_prefix_kernel<M>, dim3(tiles, stretches), dim3(kPrefixThreads), lds, s, w.at<int>(L.pos),
                      w.at<int>(L.scost), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.kstride, L.wstride, L.nwords,
-                     shift, buckets, chunk, w.at<SortParam>(L.sortparam));
+                     shift, buckets, chunk, w.at<int>(L.total0), w.at<int>(L.witness0), w.at<SortParam>(L.sortparam));
   EVX_LAUNCH_CHECK();
   // a population with a NaN or an infinity: the pairwise kernel, on a grid that costs nothing when it has nothing to do
   hipLaunchKernelGGL(dominance_nonfinite_kernel<M>, dim3(device_cus() * 8), dim3(256), 0, s, w.at<float>(L.xs_sorted),
@@ -474,8 +487,8 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) 
   const size_t lds = sizeof(int) * (size_t)L.m * 4 * 256;
   if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(objective_order_kernel), lds)) return e;
   hipLaunchKernelGGL(objective_order_kernel, dim3(radix_grid(L)), dim3(kRadixThreads), lds, s, w.at<float>(L.xs_sorted), L.npad, L.n,
-                     L.m, w.at<SortParam>(L.sortparam), w.ctrl(), w.at<int>(L.pos), w.at<int>(L.scost), radix_buffers(w),
-                     g_opt.spin_limit);
+                     L.m, w.at<SortParam>(L.sortparam), w.ctrl(), w.at<int>(L.pos), w.at<int>(L.scost), w.at<int>(L.total0),
+                     w.at<int>(L.witness0), radix_buffers(w), g_opt.spin_limit);
   EVX_LAUNCH_CHECK();
   // the barrier words of the control block restart from zero for the kernels that follow (the sort counted its
   // generations from a high base)

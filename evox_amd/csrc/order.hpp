@@ -23,7 +23,7 @@ struct SortParam {
   int shift;
   int buckets;
   int nonfinite;  // some fitness value of the population is NaN or infinite
-  int reserved;
+  int totals_valid;  // the dominance stage has left popcount and highest word of every row (zero after the slot sort)
 };
 
 __device__ inline int bucket_of(uint64_t key, const SortParam& p) { return (int)((key - p.kmin) >> p.shift); }
@@ -58,7 +58,7 @@ __device__ inline SortParam make_sort_param(const unsigned long long* __restrict
   sp.kmin = lds2[0];
   sp.buckets = buckets;
   sp.nonfinite = lds2[2] != 0ull;
-  sp.reserved = 0;
+  sp.totals_valid = 0;
   const unsigned long long span = lds2[1] >= lds2[0] ? lds2[1] - lds2[0] : 0ull;
   int shift = 0;
   while (shift < 63 && (span >> shift) >= (unsigned long long)buckets) ++shift;

@@ -167,8 +167,9 @@ __global__ __launch_bounds__(256) void count_kernel(const uint64_t* __restrict__
                                                     int* __restrict__ rank, int* __restrict__ witness,
                                                     uint64_t* __restrict__ front0_slot, uint64_t* __restrict__ front0_orig,
                                                     int* __restrict__ fsize, float* __restrict__ dist_fill,
-                                                    const Ctrl* __restrict__ ctrl) {
+                                                    const Ctrl* __restrict__ ctrl, const SortParam* __restrict__ param) {
   if (ctrl->err != 0) return;  // the slot tables are not valid: leave front 0 empty, nothing gets peeled
+  if (param->totals_valid != 0) return;  // count_from_totals_kernel does the work from what the dominance stage left
   __shared__ int block_found;
   if (threadIdx.x == 0) block_found = 0;
   __syncthreads();
@@ -193,6 +194,42 @@ __global__ __launch_bounds__(256) void count_kernel(const uint64_t* __restrict__
   }
   // one addition per block: a front 0 of thousands of rows would otherwise queue thousands of atomics on one word
   if (lane == 0 && found) atomicAdd(&block_found, found);
+  __syncthreads();
+  if (threadIdx.x == 0 && block_found) atomicAdd(fsize, block_found);
+}
+
+// The same outputs from total0[j] = popcount of row j and witness0[j] = its highest non-empty word (-1: none), which
+// the order-based dominance kernel (prefix.hpp) accumulates while it builds the matrix: one thread per row, no row
+// is read again.  Does nothing unless that kernel has run for this population.
+__global__ __launch_bounds__(256) void count_from_totals_kernel(const int* __restrict__ total0, const int* __restrict__ witness0,
+                                                                int n, const int* __restrict__ orig_of, int* __restrict__ count,
+                                                                int* __restrict__ rank, int* __restrict__ witness,
+                                                                uint64_t* __restrict__ front0_slot,
+                                                                uint64_t* __restrict__ front0_orig, int* __restrict__ fsize,
+                                                                float* __restrict__ dist_fill, const Ctrl* __restrict__ ctrl,
+                                                                const SortParam* __restrict__ param) {
+  if (ctrl->err != 0 || param->totals_valid == 0) return;
+  __shared__ int block_found;
+  if (threadIdx.x == 0) block_found = 0;
+  __syncthreads();
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  bool first = false;
+  if (j < n) {
+    const int total = total0[j];
+    const int o = orig_of[j];
+    count[j] = total;
+    rank[o] = total == 0 ? 0 : kRankUnset;
+    witness[j] = witness0[j];
+    if (dist_fill) dist_fill[o] = -INFINITY;
+    first = total == 0;
+    if (first) atomicOr(reinterpret_cast<unsigned long long*>(front0_orig + (int64_t)(o >> 6) * kFrontStride), 1ull << (o & 63));
+  }
+  // the 64 rows of a wave share one word of the slot bitmap: one store instead of up to 64 atomics
+  const uint64_t members = __builtin_amdgcn_ballot_w64(first);
+  if ((threadIdx.x & 63) == 0 && members != 0ull) {
+    front0_slot[(int64_t)(j >> 6) * kFrontStride] = members;
+    atomicAdd(&block_found, __popcll(members));
+  }
   __syncthreads();
   if (threadIdx.x == 0 && block_found) atomicAdd(fsize, block_found);
 }

@@ -64,7 +64,8 @@ __host__ __device__ inline int prefix_bucket_shift(int n) {
 __global__ __launch_bounds__(kRadixThreads) void objective_order_kernel(const float* __restrict__ xs, int npad, int n, int m,
                                                                         const SortParam* __restrict__ param,
                                                                         Ctrl* __restrict__ ctrl, int* __restrict__ pos,
-                                                                        int* __restrict__ upper, RadixBuffers buf,
+                                                                        int* __restrict__ upper, int* __restrict__ total0,
+                                                                        int* __restrict__ witness0, RadixBuffers buf,
                                                                         unsigned spin_limit) {
   extern __shared__ int order_lds[];
   __shared__ int base[256];
@@ -80,6 +81,11 @@ __global__ __launch_bounds__(kRadixThreads) void objective_order_kernel(const fl
   if (blockIdx.x < kFirstSweeper) return;
   const int workers = gridDim.x - kFirstSweeper;
   const int wb = (int)blockIdx.x - kFirstSweeper;
+  // the row totals that dominance_prefix_kernel accumulates start from nothing
+  for (int j = wb * blockDim.x + threadIdx.x; j < n; j += workers * blockDim.x) {
+    total0[j] = 0;
+    witness0[j] = -1;
+  }
   auto initial = [&](int k, int e) { return ((unsigned long long)ordered_key(xs[(int64_t)k * npad + e]) << 32) | (unsigned)e; };
   if (!radix_sort_segments(buf, m, n, initial, ctrl, gen0, spin_limit, order_lds, base, scratch)) return;
   for (int k = 0; k < m; ++k) {
@@ -116,10 +122,12 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
                                                                           const uint32_t* __restrict__ kid,
                                                                           uint64_t* __restrict__ dom, int n, int kstride,
                                                                           int64_t wstride, int nwords, int shift, int buckets,
-                                                                          int chunk, const SortParam* __restrict__ param) {
+                                                                          int chunk, int* __restrict__ total0,
+                                                                          int* __restrict__ witness0, SortParam* __restrict__ param) {
   constexpr int WW = kPrefixTileWords, TS = kPrefixTileSlots, T = kPrefixThreads;
   extern __shared__ uint64_t prefix_lds[];
   if (param->nonfinite != 0) return;
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) param->totals_valid = 1;  // for the count stage
   // Workgroups go to the eight dies in turn (linear index modulo 8), and a die has its own L2.  The two tiles
   // that share the 128-byte lines of the matrix are given to consecutive workgroups of one die, which run
   // side by side over the same rows: their halves of a line then meet in that L2 and leave as one line.
@@ -324,6 +332,17 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
       ulonglong2* const out = reinterpret_cast<ulonglong2*>(dom + (int64_t)j * wstride + w0);
 #pragma unroll
       for (int q = 0; q < WW / 2; ++q) out[q] = make_ulonglong2(d[2 * q], d[2 * q + 1]);
+      // what the count stage wants to know of the row, so that it does not have to read it again
+      int dominators = 0, highest = -1;
+#pragma unroll
+      for (int w = 0; w < WW; ++w) {
+        dominators += __popcll(d[w]);
+        highest = d[w] != 0ull ? w0 + w : highest;
+      }
+      if (dominators != 0) {
+        atomicAdd(&total0[j], dominators);
+        atomicMax(&witness0[j], highest);
+      }
     }
   }
 }

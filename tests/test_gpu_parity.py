@@ -144,10 +144,13 @@ def _matrix_words(f, variant, views_out=None):
     s = runtime.stream_handle(fd.device)
     _lib.call("evox_hip_stage_prepare", fd.data_ptr(), n, m, fd.stride(0), fd.stride(1), ws.data_ptr(), ws.numel(), s)
     _lib.call("evox_hip_stage_dominance", n, m, variant, ws.data_ptr(), ws.numel(), s)
+    _lib.call("evox_hip_stage_count", n, m, ws.data_ptr(), ws.numel(), s)
     torch.cuda.synchronize()
     views = runtime.workspace_views(ws, n, m)
     words = np.ascontiguousarray(as_np(views["dom"])[:, : views["nwords"]]).view(np.uint64).copy()
     words[defined_words(words.shape[0], words.shape[1]) == 0] = 0
+    if views_out is not None:
+        views_out.update({k: as_np(views[k]).copy() for k in ("count", "rank")})
     return words
 
 
@@ -181,10 +184,21 @@ def test_matrix_from_objective_orders_equals_the_pairwise_matrix(m):
         for name, f in cases.items():
             say("prefix_matrix", m, name, tuple(f.shape))
             runtime.set_option("prefix_min_rows", 4097)  # (a quarter more rows with two objectives)
-            got = _matrix_words(f.contiguous(), 0)
+            got_state, want_state = {}, {}
+            got = _matrix_words(f.contiguous(), 0, got_state)
             runtime.set_option("prefix_min_rows", 0)
-            want = _matrix_words(f.contiguous(), 0)
+            want = _matrix_words(f.contiguous(), 0, want_state)
             assert np.array_equal(got, want), (m, name, int((got != want).sum()))
+            # the counts and front 0 that the count stage derives from what the order-based kernel left behind
+            assert np.array_equal(got_state["count"], want_state["count"]), (m, name)
+            assert np.array_equal(got_state["count"], np.bitwise_count(want).sum(axis=1)), (m, name)
+            assert np.array_equal(got_state["rank"], want_state["rank"]), (m, name)
+            if name in ("ties", "duplicates", "large"):  # and the whole ranking on top of them (the passes start from
+                fd = f.contiguous().to(DEV)              # the highest non-empty word of every row)
+                runtime.set_option("prefix_min_rows", 4097)
+                ranks = non_dominate_rank(fd)
+                runtime.set_option("prefix_min_rows", 0)
+                assert torch.equal(ranks, non_dominate_rank(fd)), (m, name)
     finally:
         runtime.set_option("prefix_min_rows", 65536)
 
