@@ -136,6 +136,27 @@ def test_dominance_bits_all_m(m):
             assert np.array_equal(got, want), (m, variant, bool(torch.isfinite(f).all()))
 
 
+@pytest.mark.parametrize("n,m", [(65535, 3), (65536, 3), (65537, 4), (65664, 8), (81919, 2), (81920, 2), (70001, 10), (66000, 11)])
+def test_ranks_across_the_switch_to_the_order_based_matrix(n, m):
+    """Populations just below and above the size at which the matrix comes from the per-objective orders (and 65536
+    rows, where the padded column length steps off a multiple of 4096): same ranks and same selection whichever
+    kernel builds the matrix."""
+    say("switch", n, m)
+    g = torch.Generator("cpu").manual_seed(n + m)
+    f = (torch.randint(0, 1 << 12, (n, m), generator=g).float() / 64).to(DEV)  # ties in every objective
+    x = torch.arange(n, dtype=torch.int32, device=DEV)[:, None]
+    try:
+        got_rank = non_dominate_rank(f)
+        got = nd_environmental_selection(x, f, n // 2)
+        runtime.set_option("prefix_min_rows", 0)
+        assert torch.equal(got_rank, non_dominate_rank(f))
+        want = nd_environmental_selection(x, f, n // 2)
+        assert all(torch.equal(a, b) for a, b in zip(got, want))
+    finally:
+        runtime.set_option("prefix_min_rows", 65536)
+        runtime.release_workspaces()
+
+
 def _matrix_words(f, variant, views_out=None):
     """Raw words of the bit matrix (slot space) that readers look at, after prepare + dominance."""
     n, m = f.shape
