@@ -31,7 +31,7 @@ struct Options {
   unsigned spin_limit = 4000000u;
   int dominance_tile_words = 4;
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
-  int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 10 objectives (a quarter
+  int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 16 objectives (a quarter
                                     // more rows with 2) get their matrix from the per-objective orders (prefix.hpp);
                                     // 0 = never
 };
@@ -459,16 +459,17 @@ static int finish_grid(const Layout& L, int per_candidate_block) {
 
 template <int M>
 static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
+  constexpr int WW = M <= kPrefixWideObjectives ? 8 : 4;  // words per tile: what the LDS holds tables for
   const Layout& L = w.L;
   const int shift = prefix_bucket_shift(L.n);
   const int buckets = ((L.n - 1) >> shift) + 1;
-  const size_t lds = prefix_lds_bytes(M, buckets);
-  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(dominance_prefix_kernel<M>), lds)) return e;
-  const int tiles = (int)round_up((L.nwords + kPrefixTileWords - 1) / kPrefixTileWords, 16);
+  const size_t lds = prefix_lds_bytes(M, WW, buckets);
+  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(dominance_prefix_kernel<M, WW>), lds)) return e;
+  const int tiles = (int)round_up((L.nwords + WW - 1) / WW, 128 / WW);
   // shorter stretches for smaller populations, so that the workgroups still outnumber the compute units
   const int chunk = L.n >= 131072 ? kPrefixRowChunk : (L.n >= 65536 ? kPrefixRowChunk / 2 : kPrefixRowChunk / 4);
   const int stretches = (L.n + chunk - 1) / chunk;
-  hipLaunchKernelGGL(dominance_prefix_kernel<M>, dim3(tiles, stretches), dim3(kPrefixThreads), lds, s, w.at<int>(L.pos),
+  hipLaunchKernelGGL((dominance_prefix_kernel<M, WW>), dim3(tiles, stretches), dim3(kPrefixThreads), lds, s, w.at<int>(L.pos),
                      w.at<int>(L.scost), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.kstride, L.wstride, L.nwords,
                      shift, buckets, chunk, w.at<int>(L.total0), w.at<int>(L.witness0), w.at<SortParam>(L.sortparam));
   EVX_LAUNCH_CHECK();
@@ -507,6 +508,12 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) 
     case 8: return launch_dominance_prefix<8>(w, s);
     case 9: return launch_dominance_prefix<9>(w, s);
     case 10: return launch_dominance_prefix<10>(w, s);
+    case 11: return launch_dominance_prefix<11>(w, s);
+    case 12: return launch_dominance_prefix<12>(w, s);
+    case 13: return launch_dominance_prefix<13>(w, s);
+    case 14: return launch_dominance_prefix<14>(w, s);
+    case 15: return launch_dominance_prefix<15>(w, s);
+    case 16: return launch_dominance_prefix<16>(w, s);
     default: return kErrBadArg;
   }
 }

@@ -11,8 +11,9 @@
 //
 //  1. objective_order_kernel: one segmented radix sort orders the slots by every objective (radix.hpp) and
 //     leaves pos[k][slot] and upper[k][slot].
-//  2. dominance_prefix_kernel: a workgroup takes a tile of kPrefixTileSlots dominator slots (8 matrix words,
-//     64 bytes of every row) and a stretch of rows below it.  Restricted to one word of the tile, the prefix of
+//  2. dominance_prefix_kernel: a workgroup takes a tile of 512 dominator slots (8 matrix words, 64 bytes of
+//     every row; 256 slots above ten objectives, where the tables of 512 no longer fit the LDS) and a stretch
+//     of rows below it.  Restricted to one word of the tile, the prefix of
 //     objective k that belongs to row j is one of only 65 bit sets: the word's own slots sorted by pos_k, the
 //     first c of them.  The workgroup builds in LDS, per objective: the tile's 512 positions in ascending
 //     order (mp), a coarse index from position to the number t of them that lie before it, for every t the
@@ -29,23 +30,23 @@
 
 namespace evx {
 
-constexpr int kPrefixTileWords = 8;
-constexpr int kPrefixTileSlots = 64 * kPrefixTileWords;
-constexpr int kPrefixMaxObjectives = 10;  // 14.4 KB of LDS per objective
-constexpr int kPrefixBuckets = 1024;      // entries of the coarse index per objective, at most (plus two)
+constexpr int kPrefixMaxObjectives = 16;
+constexpr int kPrefixWideObjectives = 10;  // up to here tiles of 8 words (14.4 KB of LDS per objective), above it of 4 (9.3 KB)
+constexpr int kPrefixBuckets = 1024;       // entries of the coarse index per objective, at most (plus two)
 constexpr int kPrefixThreads = 1024;
-constexpr int kPrefixRowChunk = 32768;    // rows per workgroup, at most (`chunk`, a multiple of 64)
-constexpr int kPrefixMaxRows = 1 << 22;   // a position and a slot of the tile share one int
+constexpr int kPrefixRowChunk = 32768;     // rows per workgroup, at most (`chunk`, a multiple of 64)
+constexpr int kPrefixMaxRows = 1 << 22;    // a position and a slot of the tile share one int
 
-// LDS of dominance_prefix_kernel<M>, per objective: bit sets and counts (the scratch of the build lies over
+// LDS of dominance_prefix_kernel<M, WW>, per objective: bit sets and counts (the scratch of the build lies over
 // them), sorted positions, the sorted (position, slot) pairs of the build, and the coarse index.
-__host__ __device__ inline size_t prefix_lds_bytes(int m, int buckets) {
-  const size_t sets = sizeof(uint64_t) * kPrefixTileWords * 65;
-  const size_t counts = sizeof(uint64_t) * (kPrefixTileSlots + 1);
-  const size_t scratch = sizeof(int) * (size_t)(buckets + 2) + sizeof(int) * kPrefixTileSlots;  // histogram, claimed
+__host__ __device__ inline size_t prefix_lds_bytes(int m, int tile_words, int buckets) {
+  const int tile_slots = 64 * tile_words;
+  const size_t sets = sizeof(uint64_t) * tile_words * 65;
+  const size_t counts = sizeof(uint64_t) * (tile_slots + 1);
+  const size_t scratch = (sizeof(int) * (size_t)(buckets + 2 + tile_slots) + 7) & ~(size_t)7;  // histogram, claimed
   const size_t over = sets + counts > scratch ? sets + counts : scratch;
-  const size_t positions = sizeof(int) * (kPrefixTileSlots + 8);
-  const size_t sorted = sizeof(int) * kPrefixTileSlots;
+  const size_t positions = sizeof(int) * (tile_slots + 8);
+  const size_t sorted = sizeof(int) * tile_slots;
   const size_t index = (sizeof(uint16_t) * (size_t)(buckets + 2) + 7) & ~(size_t)7;
   return (size_t)m * (over + positions + sorted + index);
 }
@@ -113,28 +114,30 @@ __global__ __launch_bounds__(kRadixThreads) void objective_order_kernel(const fl
   }
 }
 
-// grid.x = the ceil(nwords / kPrefixTileWords) tiles of dominator slots, rounded up to a multiple of 16,
+// grid.x = the ceil(nwords / WW) tiles of dominator slots, rounded up to a multiple of 128 / WW,
 // grid.y = stretches of `chunk` rows, counted from the first row of the tile (rows above it have no word
-// there).  Dynamic LDS: prefix_lds_bytes(M, buckets).  Writes the eight words of the tile in every row of the
+// there).  Dynamic LDS: prefix_lds_bytes(M, WW, buckets).  Writes the WW words of the tile in every row of the
 // stretch.
-template <int M>
+template <int M, int WW>
 __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const int* __restrict__ pos, const int* __restrict__ upper,
                                                                           const uint32_t* __restrict__ kid,
                                                                           uint64_t* __restrict__ dom, int n, int kstride,
                                                                           int64_t wstride, int nwords, int shift, int buckets,
                                                                           int chunk, int* __restrict__ total0,
                                                                           int* __restrict__ witness0, SortParam* __restrict__ param) {
-  constexpr int WW = kPrefixTileWords, TS = kPrefixTileSlots, T = kPrefixThreads;
+  constexpr int TS = 64 * WW, T = kPrefixThreads;
+  constexpr int TPL = 16 / WW;  // tiles that share a 128-byte line of the matrix
+  constexpr int MPL = TS / 64;  // members of the tile per lane when a wave walks through them
   extern __shared__ uint64_t prefix_lds[];
   if (param->nonfinite != 0) return;
   if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) param->totals_valid = 1;  // for the count stage
-  // Workgroups go to the eight dies in turn (linear index modulo 8), and a die has its own L2.  The two tiles
+  // Workgroups go to the eight dies in turn (linear index modulo 8), and a die has its own L2.  The tiles
   // that share the 128-byte lines of the matrix are given to consecutive workgroups of one die, which run
-  // side by side over the same rows: their halves of a line then meet in that L2 and leave as one line.
+  // side by side over the same rows: their pieces of a line then meet in that L2 and leave as one line.
   const int64_t linear = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
   const int die = (int)(linear & 7);
   const int seq = (int)blockIdx.x >> 3;  // this workgroup among those of its die in this row of the grid
-  const int tile = 2 * ((seq >> 1) * 8 + die) + (seq & 1);
+  const int tile = TPL * ((seq / TPL) * 8 + die) + seq % TPL;
   if (tile * WW >= nwords) return;
   const int w0 = tile * WW;
   const int slot0 = w0 * 64;
@@ -216,15 +219,15 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
     }
   }
   __syncthreads();
-  // ---- counts[k][t] and the single bits of sets[k][w][c + 1]; a wave per objective, a lane per eight members
+  // ---- counts[k][t] and the single bits of sets[k][w][c + 1]; a wave per objective, a lane per MPL members
   for (int t = threadIdx.x; t < M * kSetWords; t += T) sets[(size_t)(t / kSetWords) * over + t % kSetWords] = 0ull;
   __syncthreads();
   for (int k = wave; k < M; k += T / 64) {
-    uint64_t one[8];
+    uint64_t one[MPL];
     uint64_t sum = 0ull;
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-      const int t = 8 * lane + c;
+    for (int c = 0; c < MPL; ++c) {
+      const int t = MPL * lane + c;
       one[c] = t < live ? 1ull << (8 * ((sorted[k * TS + t] & (TS - 1)) >> 6)) : 0ull;
       sum += one[c];
     }
@@ -238,8 +241,8 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
     uint64_t* const cnt = counts + (size_t)k * over;
     uint64_t* const set = sets + (size_t)k * over;
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-      const int t = 8 * lane + c;
+    for (int c = 0; c < MPL; ++c) {
+      const int t = MPL * lane + c;
       cnt[t] = run;
       if (t < live) {
         const int i = sorted[k * TS + t] & (TS - 1);

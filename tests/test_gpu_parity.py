@@ -136,7 +136,7 @@ def test_dominance_bits_all_m(m):
             assert np.array_equal(got, want), (m, variant, bool(torch.isfinite(f).all()))
 
 
-@pytest.mark.parametrize("n,m", [(65535, 3), (65536, 3), (65537, 4), (65664, 8), (81919, 2), (81920, 2), (70001, 10), (66000, 11)])
+@pytest.mark.parametrize("n,m", [(65535, 3), (65536, 3), (65537, 4), (65664, 8), (81919, 2), (81920, 2), (70001, 10), (66000, 11), (65536, 16), (66000, 17)])
 def test_ranks_across_the_switch_to_the_order_based_matrix(n, m):
     """Populations just below and above the size at which the matrix comes from the per-objective orders (and 65536
     rows, where the padded column length steps off a multiple of 4096): same ranks and same selection whichever
@@ -175,7 +175,7 @@ def _matrix_words(f, variant, views_out=None):
     return words
 
 
-@pytest.mark.parametrize("m", [2, 3, 4, 5, 6, 7, 8, 9, 10])
+@pytest.mark.parametrize("m", [2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 13, 16])
 def test_matrix_from_objective_orders_equals_the_pairwise_matrix(m):
     """Large finite populations get their matrix from the order of the rows in every objective; it must be
     the matrix of the pairwise test, word for word: ties, duplicate rows, constant objectives, a population
