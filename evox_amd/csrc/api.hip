@@ -31,8 +31,8 @@ struct Options {
   unsigned spin_limit = 4000000u;
   int dominance_tile_words = 4;
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
-  int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 16 objectives (a quarter
-                                    // more rows with 2) get their matrix from the per-objective orders (prefix.hpp);
+  int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 8 objectives (a quarter
+                                    // more rows with 2, a quarter fewer with 9 to 16) get their matrix from the per-objective orders (prefix.hpp);
                                     // 0 = never
 };
 static Options g_opt;
@@ -267,8 +267,10 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
 // x 4: 305 / 366, x 8: 451 / 637; 100000 x 2: 370 / 558, x 3: 408 / 709; 200000 x 3: 1268 / 2622, x 8: 1624 / 5340.
 static bool prefix_dominance_applies(const Layout& L) {
   if (g_opt.prefix_min_rows <= 0 || L.m < 2 || L.m > kPrefixMaxObjectives) return false;
-  // (two objectives are cheap pair by pair: a quarter more rows before the orders pay)
-  const int64_t least = L.m == 2 ? g_opt.prefix_min_rows + g_opt.prefix_min_rows / 4 : g_opt.prefix_min_rows;
+  // (two objectives are cheap pair by pair: a quarter more rows before the orders pay; nine or more are dear: a
+  // quarter fewer -- 49152 x 9: 419 / 563, x 16: 675 / 933; 32768 x 9: 365 / 271, x 16: 622 / 464)
+  const int64_t q = g_opt.prefix_min_rows / 4;
+  const int64_t least = L.m == 2 ? g_opt.prefix_min_rows + q : (L.m >= 9 ? g_opt.prefix_min_rows - q : g_opt.prefix_min_rows);
   return L.n >= least && L.n > kRadixMinCandidates && L.n <= kPrefixMaxRows;
 }
 static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s);

@@ -136,7 +136,7 @@ def test_dominance_bits_all_m(m):
             assert np.array_equal(got, want), (m, variant, bool(torch.isfinite(f).all()))
 
 
-@pytest.mark.parametrize("n,m", [(65535, 3), (65536, 3), (65537, 4), (65664, 8), (81919, 2), (81920, 2), (70001, 10), (66000, 11), (65536, 16), (66000, 17)])
+@pytest.mark.parametrize("n,m", [(65535, 3), (65536, 3), (65537, 4), (65664, 8), (81919, 2), (81920, 2), (70001, 10), (49151, 9), (49152, 16), (66000, 17)])
 def test_ranks_across_the_switch_to_the_order_based_matrix(n, m):
     """Populations just below and above the size at which the matrix comes from the per-objective orders (and 65536
     rows, where the padded column length steps off a multiple of 4096): same ranks and same selection whichever
