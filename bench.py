@@ -30,7 +30,7 @@ FP32_VECTOR_PEAK_GFLOPS = 157300.0
 # their own, scaled by what the same counters read for a 512 MiB copy: x2.0 and x1.0); the summaries
 # with the commands are kept under profiles/.  Keyed by (workload, kernel); absent = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("C5", "dominance_prefix_kernel"): 1148.16e6 + 2589.61e6,  # profiles/c5_selection_hbm_traffic.md: read + written
+    ("C5", "dominance_prefix_kernel"): 1156.56e6 + 2602.48e6,  # profiles/c5_selection_hbm_traffic.md: read + written
     ("C3", "peel_records_kernel"): 11.33e6 + 2.03e6,
     ("C3", "dominance_kernel"): 3.54e6 + 25.36e6,
     ("C3", "count_kernel"): 27.00e6 + 1.30e6,

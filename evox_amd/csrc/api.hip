@@ -489,7 +489,12 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) 
   const Layout& L = w.L;
   const size_t lds = sizeof(int) * (size_t)L.m * 4 * 256;
   if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(objective_order_kernel), lds)) return e;
-  hipLaunchKernelGGL(objective_order_kernel, dim3(radix_grid(L)), dim3(kRadixThreads), lds, s, w.at<float>(L.xs_sorted), L.npad, L.n,
+  // more workers than one per 1024 rows: every one of them handles its share of all m segments
+  int workers = (int)(((int64_t)L.n * L.m + 2047) / 2048);
+  const int cap = (device_cus() * 2 < kRadixMaxWorkers + kFirstSweeper ? device_cus() * 2 : kRadixMaxWorkers + kFirstSweeper) - kFirstSweeper;
+  if (workers > cap) workers = cap;
+  if (workers + kFirstSweeper < radix_grid(L)) workers = radix_grid(L) - kFirstSweeper;
+  hipLaunchKernelGGL(objective_order_kernel, dim3(workers + kFirstSweeper), dim3(kRadixThreads), lds, s, w.at<float>(L.xs_sorted), L.npad, L.n,
                      L.m, w.at<SortParam>(L.sortparam), w.ctrl(), w.at<int>(L.pos), w.at<int>(L.scost), w.at<int>(L.total0),
                      w.at<int>(L.witness0), radix_buffers(w), g_opt.spin_limit);
   EVX_LAUNCH_CHECK();
