@@ -27,7 +27,8 @@ namespace evx {
 
 constexpr int kRadixMinCandidates = 8192;
 constexpr int kRadixThreads = 256;
-constexpr int kRadixBatch = 4;  // pairs per lane fetched together
+constexpr int kRadixBatch = 4;  // pairs per lane and segment fetched together
+constexpr int kRadixSegments = 4;  // segments whose pairs are fetched together
 constexpr int kRadixMaxWorkers = 510;  // working blocks of a radix kernel, at most (columns of the digit table)
 
 struct RadixBuffers {
@@ -63,18 +64,27 @@ __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, in
     __syncthreads();
     // (kRadixBatch pairs per lane are fetched before any is used: the coherent loads of a wave are then in flight
     // together instead of costing a memory round trip each)
-    for (int k = 0; k < nseg; ++k) {
-      int* h = hist + (k * 4 + wave) * 256;
+    // (and the pairs of kRadixSegments segments together: a wave's share of one segment is often a single batch)
+    for (int k0 = 0; k0 < nseg; k0 += kRadixSegments) {
       for (int e0 = w_begin + lane; e0 < w_end; e0 += 64 * kRadixBatch) {
-        unsigned long long p[kRadixBatch];
+        unsigned long long p[kRadixSegments][kRadixBatch];
 #pragma unroll
-        for (int u = 0; u < kRadixBatch; ++u) {
-          const int e = e0 + 64 * u;
-          p[u] = e >= w_end ? 0ull : (pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]));
+        for (int kk = 0; kk < kRadixSegments; ++kk) {
+          const int k = k0 + kk < nseg ? k0 + kk : nseg - 1;
+#pragma unroll
+          for (int u = 0; u < kRadixBatch; ++u) {
+            const int e = e0 + 64 * u;
+            p[kk][u] = e >= w_end ? 0ull : (pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]));
+          }
         }
 #pragma unroll
-        for (int u = 0; u < kRadixBatch; ++u)
-          if (e0 + 64 * u < w_end) atomicAdd(&h[(int)((p[u] >> (32 + shift)) & 255ull)], 1);
+        for (int kk = 0; kk < kRadixSegments; ++kk) {
+          if (k0 + kk >= nseg) break;  // wave-uniform
+          int* h = hist + ((k0 + kk) * 4 + wave) * 256;
+#pragma unroll
+          for (int u = 0; u < kRadixBatch; ++u)
+            if (e0 + 64 * u < w_end) atomicAdd(&h[(int)((p[kk][u] >> (32 + shift)) & 255ull)], 1);
+        }
       }
     }
     __syncthreads();
@@ -138,22 +148,30 @@ __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, in
       }
     }
     __syncthreads();
-    for (int k = 0; k < nseg; ++k) {
-      int* h = hist + (k * 4 + wave) * 256;
+    for (int k0 = 0; k0 < nseg; k0 += kRadixSegments) {
       for (int b0 = w_begin; b0 < w_end; b0 += 64 * kRadixBatch) {
-        unsigned long long batch[kRadixBatch];
+        unsigned long long batch[kRadixSegments][kRadixBatch];
 #pragma unroll
-        for (int u = 0; u < kRadixBatch; ++u) {
-          const int e = b0 + 64 * u + lane;
-          batch[u] = e >= w_end ? 0ull : (pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]));
+        for (int kk = 0; kk < kRadixSegments; ++kk) {
+          const int k = k0 + kk < nseg ? k0 + kk : nseg - 1;
+#pragma unroll
+          for (int u = 0; u < kRadixBatch; ++u) {
+            const int e = b0 + 64 * u + lane;
+            batch[kk][u] = e >= w_end ? 0ull : (pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]));
+          }
         }
+#pragma unroll
+        for (int kk = 0; kk < kRadixSegments; ++kk) {
+        if (k0 + kk >= nseg) break;  // wave-uniform
+        const int k = k0 + kk;
+        int* h = hist + (k * 4 + wave) * 256;
 #pragma unroll
         for (int u = 0; u < kRadixBatch; ++u) {
         const int e0 = b0 + 64 * u;
         if (e0 >= w_end) break;  // wave-uniform
         const int e = e0 + lane;
         const bool have = e < w_end;
-        const unsigned long long p = batch[u];
+        const unsigned long long p = batch[kk][u];
         const int d = (int)((p >> (32 + shift)) & 255ull);
         // lanes of this group that hold the same digit
         uint64_t same = __builtin_amdgcn_ballot_w64(have);
@@ -171,6 +189,7 @@ __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, in
         }
         start = __shfl(start, leader < 0 ? 0 : leader);
         if (have) coherent_store(&out[(int64_t)k * buf.kstride + start + rank], p);
+        }
         }
       }
     }
