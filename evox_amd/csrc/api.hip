@@ -528,12 +528,21 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) 
 // Per-objective ordering of the candidates list[ctrl.worst_start ... + ctrl.nv).
 static int stage_crowd_sort(const Ws& w, const int* list, hipStream_t s) {
   const Layout& L = w.L;
-  size_t lds = sizeof(uint64_t) * kRankTile;
-  if (L.n > kRadixMinCandidates && sizeof(int) * (size_t)L.m * 4 * 256 > lds) lds = sizeof(int) * (size_t)L.m * 4 * 256;
-  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(crowd_sort_kernel), lds)) return e;
-  hipLaunchKernelGGL(crowd_sort_kernel, dim3(finish_grid(L, L.m)), dim3(kRadixThreads), lds, s, w.at<float>(L.xs), L.npad, list,
-                     w.ctrl(), L.m, L.kstride, w.at<int>(L.pos), w.at<float>(L.scost), radix_buffers(w), g_opt.spin_limit);
-  EVX_LAUNCH_CHECK();
+  // The radix path keeps a 4 KB digit table per objective in LDS, and its grid (two workgroups per compute unit, all
+  // resident: they wait for one another) leaves a workgroup half the LDS: populations that can take that path are
+  // ordered at most kCrowdSortObjectives objectives per launch (the sort buffers are used again by the next launch).
+  constexpr int kCrowdSortObjectives = 16;
+  const int per_launch = L.n > kRadixMinCandidates && L.m > kCrowdSortObjectives ? kCrowdSortObjectives : L.m;
+  for (int k0 = 0; k0 < L.m; k0 += per_launch) {
+    const int mc = L.m - k0 < per_launch ? L.m - k0 : per_launch;
+    size_t lds = sizeof(uint64_t) * kRankTile;
+    if (L.n > kRadixMinCandidates && sizeof(int) * (size_t)mc * 4 * 256 > lds) lds = sizeof(int) * (size_t)mc * 4 * 256;
+    if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(crowd_sort_kernel), lds)) return e;
+    hipLaunchKernelGGL(crowd_sort_kernel, dim3(finish_grid(L, mc)), dim3(kRadixThreads), lds, s, w.at<float>(L.xs) + (size_t)k0 * L.npad,
+                       L.npad, list, w.ctrl(), mc, L.kstride, w.at<int>(L.pos) + (size_t)k0 * L.kstride,
+                       w.at<float>(L.scost) + (size_t)k0 * L.kstride, radix_buffers(w), g_opt.spin_limit);
+    EVX_LAUNCH_CHECK();
+  }
   return 0;
 }
 

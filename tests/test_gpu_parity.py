@@ -449,6 +449,35 @@ def test_large_front_uses_radix_sort():
     assert_dist_close(crowding_distance(ties.to(DEV), mask.to(DEV)), er.crowding(ties, mask), "ties masked")
 
 
+def test_large_front_with_more_objectives_than_one_sort_launch_takes():
+    """The radix path orders at most 16 objectives per launch: 17 to 70 objectives on 9000 rows, whole
+    population and a masked part, and a selection whose last front is large."""
+    say("large_front_many_objectives")
+    g = torch.Generator("cpu").manual_seed(123)
+    for m in (17, 24, 33, 70):
+        f = (torch.randint(0, 200, (9000, m), generator=g).float() / 16.0).contiguous()
+        assert_dist_close(crowding_distance(f.to(DEV), None), er.crowding(f, None), f"9000x{m}")
+        mask = torch.rand(9000, generator=g) < 0.95
+        assert_dist_close(crowding_distance(f.to(DEV), mask.to(DEV)), er.crowding(f, mask), f"9000x{m} masked")
+    # a selection out of one large front.  The sum of 40 terms is associated differently from torch's (tolerance
+    # 1e-5 on the distance), so rows whose distances nearly tie may swap: the order is checked through what defines it
+    f = torch.rand(9000, 40, generator=g)
+    x = torch.arange(9000, dtype=torch.float32)[:, None]
+    (_, _, _, _), rank, dist, order = er.environmental_selection(x, f, 8500, return_all=True)
+    xs, fs, rs, ds = nd_environmental_selection(x.to(DEV), f.to(DEV), 8500)
+    assert runtime.last_status()["error"] == 0 and runtime.last_status()["last_front_size"] > 8192
+    picked = as_np(xs)[:, 0].astype(np.int64)
+    assert len(set(picked.tolist())) == 8500
+    assert np.array_equal(as_np(rs), as_np(rank)[picked]) and np.array_equal(as_np(fs), as_np(f)[picked])
+    assert_dist_close(ds, as_np(dist)[picked], "uniform 9000x40")
+    got_d = as_np(ds).astype(np.float64)
+    key = np.where(np.isnan(got_d), -np.inf, got_d)
+    assert np.array_equal(picked, picked[np.lexsort((picked, -key, as_np(rs)))])  # rank, distance descending, index
+    left_out = np.setdiff1d(np.arange(9000), picked)
+    cut = as_np(dist)[picked].min()
+    assert (as_np(dist)[left_out] <= cut * (1 + 1e-5)).all()  # nothing clearly better than the worst taken row is left out
+
+
 def test_crowding_dtype_rule():
     with pytest.raises(RuntimeError):
         crowding_distance(torch.rand(8, 2, dtype=torch.float64, device=DEV), None)
