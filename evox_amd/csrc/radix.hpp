@@ -125,29 +125,44 @@ __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, in
     }
     if (!sweeper_barrier(ctrl, ++gen, 0, &dummy, spin_limit, scratch)) return false;
     // ---- 3. destinations and the stable move
-    for (int k = 0; k < nseg; ++k) {
+    // (the digit totals and this block's prefixes of kRadixSegments segments are fetched together, and their
+    // scans share the two barriers)
+    for (int k0 = 0; k0 < nseg; k0 += kRadixSegments) {
       const int d = threadIdx.x;
-      const int tot = coherent_load(&buf.totals[k * 256 + d]);
-      int incl = tot;
+      int tot[kRadixSegments], mine[kRadixSegments], incl[kRadixSegments];
 #pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const int up = __shfl_up(incl, off);
-        if (lane >= off) incl += up;
+      for (int kk = 0; kk < kRadixSegments; ++kk) {
+        const int k = k0 + kk < nseg ? k0 + kk : nseg - 1;
+        tot[kk] = coherent_load(&buf.totals[k * 256 + d]);
+        mine[kk] = coherent_load(&buf.table[((int64_t)k * 256 + d) * workers + wb]);
       }
-      if (lane == 63) base[wave] = incl;
-      __syncthreads();
-      int first = incl - tot;
-      for (int v = 0; v < wave; ++v) first += base[v];
-      __syncthreads();
-      // first destination of digit d for wave 0 of this block, then for waves 1..3
-      int r = first + coherent_load(&buf.table[((int64_t)k * 256 + d) * workers + wb]);
-      for (int v = 0; v < 4; ++v) {
-        const int c = hist[(k * 4 + v) * 256 + d];
-        hist[(k * 4 + v) * 256 + d] = r;
-        r += c;
+#pragma unroll
+      for (int kk = 0; kk < kRadixSegments; ++kk) {
+        incl[kk] = tot[kk];
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+          const int up = __shfl_up(incl[kk], off);
+          if (lane >= off) incl[kk] += up;
+        }
+        if (lane == 63) base[kk * 4 + wave] = incl[kk];
       }
+      __syncthreads();
+#pragma unroll
+      for (int kk = 0; kk < kRadixSegments; ++kk) {
+        if (k0 + kk >= nseg) break;  // block-uniform
+        const int k = k0 + kk;
+        int first = incl[kk] - tot[kk];
+        for (int v = 0; v < wave; ++v) first += base[kk * 4 + v];
+        // first destination of digit d for wave 0 of this block, then for waves 1..3
+        int r = first + mine[kk];
+        for (int v = 0; v < 4; ++v) {
+          const int c = hist[(k * 4 + v) * 256 + d];
+          hist[(k * 4 + v) * 256 + d] = r;
+          r += c;
+        }
+      }
+      __syncthreads();
     }
-    __syncthreads();
     for (int k0 = 0; k0 < nseg; k0 += kRadixSegments) {
       for (int b0 = w_begin; b0 < w_end; b0 += 64 * kRadixBatch) {
         unsigned long long batch[kRadixSegments][kRadixBatch];
