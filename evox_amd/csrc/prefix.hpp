@@ -13,14 +13,16 @@
 //     leaves pos[k][slot] and upper[k][slot].
 //  2. dominance_prefix_kernel: a workgroup takes a tile of 512 dominator slots (8 matrix words, 64 bytes of
 //     every row; 256 slots above ten objectives, where the tables of 512 no longer fit the LDS) and a stretch
-//     of rows below it.  Restricted to one word of the tile, the prefix of
-//     objective k that belongs to row j is one of only 65 bit sets: the word's own slots sorted by pos_k, the
-//     first c of them.  The workgroup builds in LDS, per objective: the tile's 512 positions in ascending
-//     order (mp), a coarse index from position to the number t of them that lie before it, for every t the
-//     eight counts c (how many of the first t fall into each word), and the 8 x 65 bit sets.  A lane then
-//     needs, per row and objective, one look-up of t (the coarse index, then a comparison or two along mp),
-//     one 8-byte read of the counts and eight 8-byte reads of bit sets, ANDed over the objectives: about
-//     55 instructions per objective and 512 pairs, where the pairwise test needs 640.
+//     of rows below it.  Restricted to one word of the tile, the prefix of objective k that belongs to row j is
+//     one of only 65 bit sets: the word's own slots sorted by pos_k, the first c of them.  The workgroup builds
+//     in LDS, per objective: the tile's positions in ascending order (mp), a coarse index from position to the
+//     number t of them that lie before it, for every t the byte counts c (how many of the first t fall into each
+//     word), and the 65 bit sets of every word, kept complemented.  A lane then needs, per row and objective, one
+//     look-up of t (the coarse index, then a comparison or two along mp), one 8-byte read of the counts and one
+//     8-byte read of a bit set per word, ORed over the objectives and complemented once: about 55 instructions
+//     per objective and 512 pairs, where the pairwise test needs 640.  While it holds the words of a row it also
+//     leaves their popcount and the highest non-empty word for the count stage (peel.hpp), which then reads no
+//     row again.
 #pragma once
 
 #include "common.hpp"
@@ -117,7 +119,8 @@ __global__ __launch_bounds__(kRadixThreads) void objective_order_kernel(const fl
 // grid.x = the ceil(nwords / WW) tiles of dominator slots, rounded up to a multiple of 128 / WW,
 // grid.y = stretches of `chunk` rows, counted from the first row of the tile (rows above it have no word
 // there).  Dynamic LDS: prefix_lds_bytes(M, WW, buckets).  Writes the WW words of the tile in every row of the
-// stretch.
+// stretch and adds their popcount to total0[row]; witness0[row] = the highest non-empty word so far (both start
+// from objective_order_kernel's 0 and -1).  Sets param->totals_valid.
 template <int M, int WW>
 __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const int* __restrict__ pos, const int* __restrict__ upper,
                                                                           const uint32_t* __restrict__ kid,
