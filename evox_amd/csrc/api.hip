@@ -487,7 +487,7 @@ static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
 // buffers of the crowding stage (radix pairs, pos, scost) are free until then and carry the orders.
 static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) {
   const Layout& L = w.L;
-  const size_t lds = sizeof(int) * (size_t)L.m * 4 * 256;
+  const size_t lds = kRadixLdsBytes;
   if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(objective_order_kernel), lds)) return e;
   // more workers than one per 1024 rows: every one of them handles its share of all m segments
   int workers = (int)(((int64_t)L.n * L.m + 2047) / 2048);
@@ -528,28 +528,20 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) 
 // Per-objective ordering of the candidates list[ctrl.worst_start ... + ctrl.nv).
 static int stage_crowd_sort(const Ws& w, const int* list, hipStream_t s) {
   const Layout& L = w.L;
-  // The radix path keeps a 4 KB digit table per objective in LDS, and its grid (two workgroups per compute unit, all
-  // resident: they wait for one another) leaves a workgroup half the LDS: populations that can take that path are
-  // ordered at most kCrowdSortObjectives objectives per launch (the sort buffers are used again by the next launch).
-  constexpr int kCrowdSortObjectives = 16;
-  const int per_launch = L.n > kRadixMinCandidates && L.m > kCrowdSortObjectives ? kCrowdSortObjectives : L.m;
-  for (int k0 = 0; k0 < L.m; k0 += per_launch) {
-    const int mc = L.m - k0 < per_launch ? L.m - k0 : per_launch;
-    size_t lds = sizeof(uint64_t) * kRankTile;
-    if (L.n > kRadixMinCandidates && sizeof(int) * (size_t)mc * 4 * 256 > lds) lds = sizeof(int) * (size_t)mc * 4 * 256;
-    if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(crowd_sort_kernel), lds)) return e;
-    hipLaunchKernelGGL(crowd_sort_kernel, dim3(finish_grid(L, mc)), dim3(kRadixThreads), lds, s, w.at<float>(L.xs) + (size_t)k0 * L.npad,
-                       L.npad, list, w.ctrl(), mc, L.kstride, w.at<int>(L.pos) + (size_t)k0 * L.kstride,
-                       w.at<float>(L.scost) + (size_t)k0 * L.kstride, radix_buffers(w), g_opt.spin_limit);
-    EVX_LAUNCH_CHECK();
-  }
+  size_t lds = sizeof(uint64_t) * kRankTile;
+  if (L.n > kRadixMinCandidates && kRadixLdsBytes > lds) lds = kRadixLdsBytes;
+  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(crowd_sort_kernel), lds)) return e;
+  hipLaunchKernelGGL(crowd_sort_kernel, dim3(finish_grid(L, L.m)), dim3(kRadixThreads), lds, s, w.at<float>(L.xs), L.npad, list,
+                     w.ctrl(), L.m, L.kstride, w.at<int>(L.pos), w.at<float>(L.scost), radix_buffers(w), g_opt.spin_limit);
+  EVX_LAUNCH_CHECK();
   return 0;
 }
 
 // Crowding distances of those candidates and, with want_order, the selection order.
 static int stage_crowd_finish(const Ws& w, const int* list, bool want_order, hipStream_t s) {
   const Layout& L = w.L;
-  const size_t lds = sizeof(uint32_t) * kRadixMinCandidates + sizeof(uint64_t) * kRankTile;
+  size_t lds = sizeof(uint32_t) * kRadixMinCandidates + sizeof(uint64_t) * kRankTile;
+  if (L.n > kRadixMinCandidates && kRadixLdsBytes > lds) lds = kRadixLdsBytes;
   hipLaunchKernelGGL(crowd_finish_kernel, dim3(finish_grid(L, 1)), dim3(kRadixThreads), lds, s, list, w.ctrl(), L.m,
                      w.at<int>(L.pos), w.at<float>(L.scost), L.kstride, w.at<float>(L.dist), w.at<uint32_t>(L.dkey),
                      w.at<int>(L.order), radix_buffers(w), g_opt.spin_limit, want_order ? 1 : 0);
@@ -843,7 +835,7 @@ static int argsort_step(const void* key, int kind, int64_t stride, int64_t n, co
   const int cap = device_cus() * 2 - kFirstSweeper;  // all blocks resident at once
   if (workers > cap) workers = cap;
   if (workers < 1) workers = 1;
-  hipLaunchKernelGGL(argsort_step_kernel, dim3(workers + kFirstSweeper), dim3(kRadixThreads), sizeof(int) * 4 * 256, s, key, kind,
+  hipLaunchKernelGGL(argsort_step_kernel, dim3(workers + kFirstSweeper), dim3(kRadixThreads), kRadixLdsBytes, s, key, kind,
                      stride, L.n, prev_order, reinterpret_cast<Ctrl*>(base + L.ctrl), b, order_out, g_opt.spin_limit);
   EVX_LAUNCH_CHECK();
   return 0;

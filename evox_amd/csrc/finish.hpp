@@ -21,7 +21,7 @@ namespace evx {
 // Per-objective sorted position of every candidate of the last front: pos[k][q], sorted_cost[k][pos].
 // Grid: the radix grid (master, idle block, workers; all resident) when the population can have a
 // front above kRadixMinCandidates rows, any grid otherwise.  Dynamic LDS: max(kRankTile * 8,
-// m * 4 * 256 * 4) bytes.
+// kRadixLdsBytes) bytes.
 __global__ __launch_bounds__(kRadixThreads) void crowd_sort_kernel(const float* __restrict__ xs, int npad,
                                                                    const int* __restrict__ list_base, Ctrl* __restrict__ ctrl,
                                                                    int m, int kstride, int* __restrict__ pos,

@@ -62,7 +62,7 @@ __host__ __device__ inline int prefix_bucket_shift(int n) {
 
 // pos[k * kstride + slot] = position of the slot in the ascending order of objective k (ties in any order);
 // upper[k * kstride + slot] = number of slots whose value in objective k is at most this slot's.
-// Grid: the radix grid (all blocks resident).  Dynamic LDS: m * 4 * 256 ints.  Nothing is done for a
+// Grid: the radix grid (all blocks resident).  Dynamic LDS: kRadixLdsBytes.  Nothing is done for a
 // population with a NaN or an infinity.
 __global__ __launch_bounds__(kRadixThreads) void objective_order_kernel(const float* __restrict__ xs, int npad, int n, int m,
                                                                         const SortParam* __restrict__ param,

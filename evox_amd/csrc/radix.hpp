@@ -8,13 +8,13 @@
 //
 // One persistent kernel sorts all segments together, four 8-bit passes, three grid barriers per pass
 // (the barrier of peel.hpp: block 0 is the master, block 1 stays out, blocks 2.. work):
-//   1. every wave histograms the digits of its contiguous share of each segment (LDS); the block
-//      totals go to table[segment][digit][block];
-//   2. for every (segment, digit) one wave turns the per-block counts into exclusive prefixes and
+//   1. every block counts the digits of its chunks (LDS); the counts go to table[segment][digit][chunk];
+//   2. for every (segment, digit) one wave turns the per-chunk counts into exclusive prefixes and
 //      leaves the digit total;
-//   3. every block scans the 256 digit totals, derives the first destination of each of its waves for
-//      each digit, and the waves move their pairs in order: inside a group of 64 pairs the rank among
-//      equal digits comes from eight ballots, so every pass is stable.
+//   3. every block scans the 256 digit totals of its chunk's segment, derives the destination of the chunk's
+//      pairs of each digit, and moves the pairs tile by tile through LDS: inside a group of 64 pairs the rank
+//      among equal digits comes from eight ballots, the waves and groups follow one another, so every pass is
+//      stable.
 // Pairs travel between blocks through relaxed agent-scope loads and stores (no cache-wide fences).
 // The sizes are read from device memory, so the host launches this unconditionally; when the front is
 // small the kernel returns at once.
@@ -27,13 +27,12 @@ namespace evx {
 
 constexpr int kRadixMinCandidates = 8192;
 constexpr int kRadixThreads = 256;
-constexpr int kRadixBatch = 4;  // pairs per lane and segment fetched together
-constexpr int kRadixSegments = 4;  // segments whose pairs are fetched together
+constexpr int kRadixBatch = 4;  // pairs per lane fetched together when the digits are counted
 constexpr int kRadixMaxWorkers = 510;  // working blocks of a radix kernel, at most (columns of the digit table)
 
 struct RadixBuffers {
   unsigned long long* pairs[2];  // [segments][kstride] each: (key << 32) | candidate index
-  int* table;                    // [segments][256][workers]
+  int* table;                    // [segments][256][chunks], chunks <= kRadixMaxWorkers
   int* totals;                   // [segments][256]
   int kstride;
 };
@@ -41,171 +40,172 @@ struct RadixBuffers {
 // Sorts `nseg` segments of nv pairs; pair e of segment k is initial(k, e) (candidate order), the
 // result is left in buf.pairs[0] (four passes: initial -> pairs[1] -> pairs[0] -> pairs[1] -> pairs[0]).
 // Must be called by every thread of every block with blockIdx.x >= kFirstSweeper; block 0 must run
-// radix_master().  `hist` = LDS, nseg * 4 * 256 ints; `base` = LDS, 256 ints.
+// radix_master().  `lds` = kRadixLdsBytes of LDS; `base` = LDS, 256 ints; `scratch` as for the barrier.
+//
+// A segment is cut into chunks (as many pairs as gives every working block about one chunk, a multiple of 256), and
+// a block takes whole chunks: all pairs that it moves in a pass belong to one segment and lie side by side.  It
+// stages them in LDS, a tile of kRadixTile at a time, in the order of their destinations, so that the pairs of one
+// digit leave as one run of neighbouring addresses instead of one 8-byte store each.
+constexpr int kRadixTile = 4096;
+constexpr size_t kRadixLdsBytes = sizeof(int) * 6 * 256 + sizeof(unsigned long long) * kRadixTile;
+
 template <class Initial>
 __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, int nv, Initial initial, Ctrl* ctrl,
-                                           unsigned gen0, unsigned spin_limit, int* hist, int* base, int* scratch) {
+                                           unsigned gen0, unsigned spin_limit, int* lds, int* base, int* scratch) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
+  const int tid = threadIdx.x;  // blockDim.x == 256
   const int workers = gridDim.x - kFirstSweeper;
   const int wb = (int)blockIdx.x - kFirstSweeper;
-  const int chunk = (int)round_up((nv + workers - 1) / workers, 256);
-  const int sub = chunk / 4;
-  const int w_begin = min(nv, wb * chunk + wave * sub);
-  const int w_end = min(nv, w_begin + sub);
+  int64_t per = ((int64_t)nv * nseg + workers - 1) / workers;
+  const int64_t least = ((int64_t)nv + kRadixMaxWorkers - 1) / kRadixMaxWorkers;  // the digit table has kRadixMaxWorkers columns
+  if (per < least) per = least;
+  const int chunk = (int)round_up(per < 256 ? 256 : per, 256);
+  const int chunks = (nv + chunk - 1) / chunk;
+  const int items = nseg * chunks;
+  int* const hw = lds;               // [4][256]: digit counts of a tile per wave, then the waves' cursors
+  int* const lstart = lds + 4 * 256;  // [256]: first staged position of every digit of the tile
+  int* const gstart = lds + 5 * 256;  // [256]: destination of the next pair of every digit of the chunk
+  unsigned long long* const stage = reinterpret_cast<unsigned long long*>(lds + 6 * 256);  // [kRadixTile]
+  // exclusive prefix over the 256 threads of the block (two barriers)
+  auto exclusive256 = [&](int v) {
+    int incl = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(incl, off);
+      if (lane >= off) incl += up;
+    }
+    if (lane == 63) base[wave] = incl;
+    __syncthreads();
+    int r = incl - v;
+    for (int x = 0; x < wave; ++x) r += base[x];
+    __syncthreads();
+    return r;
+  };
   unsigned gen = gen0;
   int dummy = 0;
   for (int pass = 0; pass < 4; ++pass) {
     const int shift = 8 * pass;
     const unsigned long long* __restrict__ in = buf.pairs[pass & 1];
     unsigned long long* __restrict__ out = buf.pairs[(pass + 1) & 1];
-    // ---- 1. digit histograms
-    for (int t = threadIdx.x; t < nseg * 4 * 256; t += blockDim.x) hist[t] = 0;
-    __syncthreads();
-    // (kRadixBatch pairs per lane are fetched before any is used: the coherent loads of a wave are then in flight
-    // together instead of costing a memory round trip each)
-    // (and the pairs of kRadixSegments segments together: a wave's share of one segment is often a single batch)
-    for (int k0 = 0; k0 < nseg; k0 += kRadixSegments) {
-      for (int e0 = w_begin + lane; e0 < w_end; e0 += 64 * kRadixBatch) {
-        unsigned long long p[kRadixSegments][kRadixBatch];
+    auto fetch = [&](int k, int e) { return pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]); };
+    // ---- 1. digit counts of every chunk (kRadixBatch pairs per lane are fetched before any is used: the coherent
+    // loads of a wave are then in flight together instead of costing a memory round trip each)
+    for (int item = wb; item < items; item += workers) {
+      const int k = item / chunks, c = item - k * chunks;
+      const int begin = c * chunk, end = min(nv, begin + chunk);
+      hw[tid] = 0;
+      __syncthreads();
+      for (int e0 = begin + tid; e0 < end; e0 += 256 * kRadixBatch) {
+        unsigned long long p[kRadixBatch];
 #pragma unroll
-        for (int kk = 0; kk < kRadixSegments; ++kk) {
-          const int k = k0 + kk < nseg ? k0 + kk : nseg - 1;
+        for (int u = 0; u < kRadixBatch; ++u) p[u] = e0 + 256 * u < end ? fetch(k, e0 + 256 * u) : 0ull;
 #pragma unroll
-          for (int u = 0; u < kRadixBatch; ++u) {
-            const int e = e0 + 64 * u;
-            p[kk][u] = e >= w_end ? 0ull : (pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]));
-          }
-        }
-#pragma unroll
-        for (int kk = 0; kk < kRadixSegments; ++kk) {
-          if (k0 + kk >= nseg) break;  // wave-uniform
-          int* h = hist + ((k0 + kk) * 4 + wave) * 256;
-#pragma unroll
-          for (int u = 0; u < kRadixBatch; ++u)
-            if (e0 + 64 * u < w_end) atomicAdd(&h[(int)((p[kk][u] >> (32 + shift)) & 255ull)], 1);
-        }
+        for (int u = 0; u < kRadixBatch; ++u)
+          if (e0 + 256 * u < end) atomicAdd(&hw[(int)((p[u] >> (32 + shift)) & 255ull)], 1);
       }
-    }
-    __syncthreads();
-    for (int k = 0; k < nseg; ++k) {
-      const int d = threadIdx.x;  // blockDim.x == 256
-      const int tot = hist[(k * 4 + 0) * 256 + d] + hist[(k * 4 + 1) * 256 + d] + hist[(k * 4 + 2) * 256 + d] +
-                      hist[(k * 4 + 3) * 256 + d];
-      coherent_store(&buf.table[((int64_t)k * 256 + d) * workers + wb], tot);
+      __syncthreads();
+      coherent_store(&buf.table[((int64_t)k * 256 + tid) * chunks + c], hw[tid]);
     }
     if (!sweeper_barrier(ctrl, ++gen, 0, &dummy, spin_limit, scratch)) return false;
-    // ---- 2. per (segment, digit): exclusive prefix over the blocks, digit total
+    // ---- 2. per (segment, digit): exclusive prefix over the chunks, digit total
     for (int item = wb * 4 + wave; item < nseg * 256; item += workers * 4) {
-      int* row = buf.table + (int64_t)item * workers;
+      int* row = buf.table + (int64_t)item * chunks;
       int carry = 0;
       constexpr int kChunks = (kRadixMaxWorkers + 63) / 64;  // all counts of the item are fetched together
       int vals[kChunks];
 #pragma unroll
-      for (int c = 0; c < kChunks; ++c) {
-        const int b = c * 64 + lane;
-        vals[c] = b < workers ? coherent_load(&row[b]) : 0;
+      for (int q = 0; q < kChunks; ++q) {
+        const int b = q * 64 + lane;
+        vals[q] = b < chunks ? coherent_load(&row[b]) : 0;
       }
 #pragma unroll
-      for (int c = 0; c < kChunks; ++c) {
-        const int b0 = c * 64;
-        if (b0 >= workers) break;  // wave-uniform
+      for (int q = 0; q < kChunks; ++q) {
+        const int b0 = q * 64;
+        if (b0 >= chunks) break;  // wave-uniform
         const int b = b0 + lane;
-        const int v = vals[c];
+        const int v = vals[q];
         int incl = v;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
           const int up = __shfl_up(incl, off);
           if (lane >= off) incl += up;
         }
-        if (b < workers) coherent_store(&row[b], carry + incl - v);
+        if (b < chunks) coherent_store(&row[b], carry + incl - v);
         carry += __shfl(incl, 63);
       }
       if (lane == 0) coherent_store(&buf.totals[item], carry);
     }
     if (!sweeper_barrier(ctrl, ++gen, 0, &dummy, spin_limit, scratch)) return false;
-    // ---- 3. destinations and the stable move
-    // (the digit totals and this block's prefixes of kRadixSegments segments are fetched together, and their
-    // scans share the two barriers)
-    for (int k0 = 0; k0 < nseg; k0 += kRadixSegments) {
-      const int d = threadIdx.x;
-      int tot[kRadixSegments], mine[kRadixSegments], incl[kRadixSegments];
-#pragma unroll
-      for (int kk = 0; kk < kRadixSegments; ++kk) {
-        const int k = k0 + kk < nseg ? k0 + kk : nseg - 1;
-        tot[kk] = coherent_load(&buf.totals[k * 256 + d]);
-        mine[kk] = coherent_load(&buf.table[((int64_t)k * 256 + d) * workers + wb]);
+    // ---- 3. the stable move, chunk by chunk and tile by tile
+    for (int item = wb; item < items; item += workers) {
+      const int k = item / chunks, c = item - k * chunks;
+      const int begin = c * chunk, end = min(nv, begin + chunk);
+      {  // destination of the chunk's first pair of every digit: the smaller digits of the segment, then the earlier chunks
+        const int total = coherent_load(&buf.totals[k * 256 + tid]);
+        const int before = coherent_load(&buf.table[((int64_t)k * 256 + tid) * chunks + c]);
+        gstart[tid] = exclusive256(total) + before;
       }
+      for (int t0 = begin; t0 < end; t0 += kRadixTile) {
+        const int count = min(end - t0, kRadixTile);
+        const int sub = ((count + 255) / 256) * 64;  // a wave takes a quarter of the tile, whole groups of 64 pairs
+        const int w_begin = min(count, wave * sub), w_end = min(count, w_begin + sub);
+        constexpr int kGroups = kRadixTile / 4 / 64;
+        unsigned long long pr[kGroups];
 #pragma unroll
-      for (int kk = 0; kk < kRadixSegments; ++kk) {
-        incl[kk] = tot[kk];
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-          const int up = __shfl_up(incl[kk], off);
-          if (lane >= off) incl[kk] += up;
+        for (int g = 0; g < kGroups; ++g) {
+          const int e = w_begin + g * 64 + lane;
+          pr[g] = e < w_end ? fetch(k, t0 + e) : 0ull;
         }
-        if (lane == 63) base[kk * 4 + wave] = incl[kk];
-      }
-      __syncthreads();
 #pragma unroll
-      for (int kk = 0; kk < kRadixSegments; ++kk) {
-        if (k0 + kk >= nseg) break;  // block-uniform
-        const int k = k0 + kk;
-        int first = incl[kk] - tot[kk];
-        for (int v = 0; v < wave; ++v) first += base[kk * 4 + v];
-        // first destination of digit d for wave 0 of this block, then for waves 1..3
-        int r = first + mine[kk];
-        for (int v = 0; v < 4; ++v) {
-          const int c = hist[(k * 4 + v) * 256 + d];
-          hist[(k * 4 + v) * 256 + d] = r;
-          r += c;
-        }
-      }
-      __syncthreads();
-    }
-    for (int k0 = 0; k0 < nseg; k0 += kRadixSegments) {
-      for (int b0 = w_begin; b0 < w_end; b0 += 64 * kRadixBatch) {
-        unsigned long long batch[kRadixSegments][kRadixBatch];
+        for (int x = 0; x < 4; ++x) hw[x * 256 + tid] = 0;
+        __syncthreads();
 #pragma unroll
-        for (int kk = 0; kk < kRadixSegments; ++kk) {
-          const int k = k0 + kk < nseg ? k0 + kk : nseg - 1;
+        for (int g = 0; g < kGroups; ++g)
+          if (w_begin + g * 64 + lane < w_end) atomicAdd(&hw[wave * 256 + (int)((pr[g] >> (32 + shift)) & 255ull)], 1);
+        __syncthreads();
+        // staged position of the first pair of every digit, and from there the first pair of every wave
+        const int c0 = hw[tid], c1 = hw[256 + tid], c2 = hw[512 + tid], c3 = hw[768 + tid];
+        const int digit_total = c0 + c1 + c2 + c3;
+        const int first = exclusive256(digit_total);
+        lstart[tid] = first;
+        hw[tid] = first;
+        hw[256 + tid] = first + c0;
+        hw[512 + tid] = first + c0 + c1;
+        hw[768 + tid] = first + c0 + c1 + c2;
+        __syncthreads();
+        int* const cursor = hw + wave * 256;
 #pragma unroll
-          for (int u = 0; u < kRadixBatch; ++u) {
-            const int e = b0 + 64 * u + lane;
-            batch[kk][u] = e >= w_end ? 0ull : (pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]));
+        for (int g = 0; g < kGroups; ++g) {
+          if (w_begin + g * 64 >= w_end) break;  // wave-uniform
+          const bool have = w_begin + g * 64 + lane < w_end;
+          const unsigned long long p = pr[g];
+          const int d = (int)((p >> (32 + shift)) & 255ull);
+          // lanes of this group that hold the same digit: the rank among them keeps the pass stable
+          uint64_t same = __builtin_amdgcn_ballot_w64(have);
+#pragma unroll
+          for (int bit = 0; bit < 8; ++bit) {
+            const uint64_t b = __builtin_amdgcn_ballot_w64((d >> bit) & 1);
+            same &= ((d >> bit) & 1) ? b : ~b;
           }
+          const int leader = __ffsll((unsigned long long)same) - 1;
+          const int rank = __popcll(same & ((1ull << lane) - 1ull));
+          int start = 0;
+          if (have && lane == leader) {
+            start = cursor[d];
+            cursor[d] = start + __popcll(same);
+          }
+          start = __shfl(start, leader < 0 ? 0 : leader);
+          if (have) stage[start + rank] = p;
         }
-#pragma unroll
-        for (int kk = 0; kk < kRadixSegments; ++kk) {
-        if (k0 + kk >= nseg) break;  // wave-uniform
-        const int k = k0 + kk;
-        int* h = hist + (k * 4 + wave) * 256;
-#pragma unroll
-        for (int u = 0; u < kRadixBatch; ++u) {
-        const int e0 = b0 + 64 * u;
-        if (e0 >= w_end) break;  // wave-uniform
-        const int e = e0 + lane;
-        const bool have = e < w_end;
-        const unsigned long long p = batch[kk][u];
-        const int d = (int)((p >> (32 + shift)) & 255ull);
-        // lanes of this group that hold the same digit
-        uint64_t same = __builtin_amdgcn_ballot_w64(have);
-#pragma unroll
-        for (int bit = 0; bit < 8; ++bit) {
-          const uint64_t b = __builtin_amdgcn_ballot_w64((d >> bit) & 1);
-          same &= ((d >> bit) & 1) ? b : ~b;
+        __syncthreads();
+        for (int t = tid; t < count; t += 256) {
+          const unsigned long long p = stage[t];
+          const int d = (int)((p >> (32 + shift)) & 255ull);
+          coherent_store(&out[(int64_t)k * buf.kstride + gstart[d] + (t - lstart[d])], p);
         }
-        const int leader = __ffsll((unsigned long long)same) - 1;
-        const int rank = __popcll(same & ((1ull << lane) - 1ull));
-        int start = 0;
-        if (have && lane == leader) {
-          start = h[d];
-          h[d] = start + __popcll(same);
-        }
-        start = __shfl(start, leader < 0 ? 0 : leader);
-        if (have) coherent_store(&out[(int64_t)k * buf.kstride + start + rank], p);
-        }
-        }
+        __syncthreads();
+        gstart[tid] += digit_total;  // read again after the barriers of the next tile, or not at all
       }
     }
     if (!sweeper_barrier(ctrl, ++gen, 0, &dummy, spin_limit, scratch)) return false;
