@@ -116,6 +116,44 @@ __global__ __launch_bounds__(kRadixThreads) void objective_order_kernel(const fl
   }
 }
 
+// d[2p], d[2p+1] = the p-th 16-byte piece of this lane's row.  Afterwards they hold piece (lane & 3) of the row of
+// lane (lane & ~3) + p: the 4 x 4 transpose of the pieces among four neighbouring lanes, in two exchanges (with the
+// lane one away, then with the lane two away), every dword moved by one DPP quad permutation.
+__device__ inline void quad_transpose_pieces(uint64_t (&d)[8], int lane) {
+  int v[16];
+#pragma unroll
+  for (int w = 0; w < 8; ++w) {
+    v[2 * w] = (int)(uint32_t)d[w];
+    v[2 * w + 1] = (int)(uint32_t)(d[w] >> 32);
+  }
+  const bool odd = (lane & 1) != 0, high = (lane & 2) != 0;
+  // piece p occupies v[4p .. 4p+3]
+#pragma unroll
+  for (int h = 0; h < 2; ++h)  // pieces 2h and 2h+1 against the lane one away
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      int& even = v[4 * (2 * h) + x];
+      int& oddp = v[4 * (2 * h + 1) + x];
+      const int send = odd ? even : oddp;
+      const int recv = __builtin_amdgcn_mov_dpp(send, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+      even = odd ? recv : even;
+      oddp = odd ? oddp : recv;
+    }
+#pragma unroll
+  for (int h = 0; h < 2; ++h)  // pieces h and h+2 against the lane two away
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      int& low = v[4 * h + x];
+      int& hi = v[4 * (h + 2) + x];
+      const int send = high ? low : hi;
+      const int recv = __builtin_amdgcn_mov_dpp(send, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+      low = high ? recv : low;
+      hi = high ? hi : recv;
+    }
+#pragma unroll
+  for (int w = 0; w < 8; ++w) d[w] = (uint64_t)(uint32_t)v[2 * w] | ((uint64_t)(uint32_t)v[2 * w + 1] << 32);
+}
+
 // grid.x = the ceil(nwords / WW) tiles of dominator slots, rounded up to a multiple of 128 / WW,
 // grid.y = stretches of `chunk` rows, counted from the first row of the tile (rows above it have no word
 // there).  Dynamic LDS: prefix_lds_bytes(M, WW, buckets).  Writes the WW words of the tile in every row of the
@@ -335,9 +373,6 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
       }
     }
     if (j < n) {
-      ulonglong2* const out = reinterpret_cast<ulonglong2*>(dom + (int64_t)j * wstride + w0);
-#pragma unroll
-      for (int q = 0; q < WW / 2; ++q) out[q] = make_ulonglong2(d[2 * q], d[2 * q + 1]);
       // what the count stage wants to know of the row, so that it does not have to read it again
       int dominators = 0, highest = -1;
 #pragma unroll
@@ -349,6 +384,22 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
         atomicAdd(&total0[j], dominators);
         atomicMax(&witness0[j], highest);
       }
+    }
+    if constexpr (WW == 8) {
+      // Four neighbouring lanes exchange their 16-byte pieces (a 4 x 4 transpose through DPP moves), so that a
+      // store instruction writes the whole 64 bytes of a row from four lanes side by side -- one request per row
+      // to the memory system instead of four requests of 16 bytes from four instructions.
+      quad_transpose_pieces(d, lane);
+      const int jq = j - (lane & 3);  // the first row of this lane's four
+#pragma unroll
+      for (int p = 0; p < 4; ++p)
+        if (jq + p < n)
+          *reinterpret_cast<ulonglong2*>(dom + (int64_t)(jq + p) * wstride + w0 + 2 * (lane & 3)) =
+              make_ulonglong2(d[2 * p], d[2 * p + 1]);
+    } else if (j < n) {
+      ulonglong2* const out = reinterpret_cast<ulonglong2*>(dom + (int64_t)j * wstride + w0);
+#pragma unroll
+      for (int q = 0; q < WW / 2; ++q) out[q] = make_ulonglong2(d[2 * q], d[2 * q + 1]);
     }
   }
 }
