@@ -116,6 +116,13 @@ __global__ __launch_bounds__(kRadixThreads) void objective_order_kernel(const fl
   }
 }
 
+// The value that the neighbouring lane (lane ^ 1) passes in, by two DPP quad permutations.
+__device__ inline uint64_t pair_exchange(uint64_t v) {
+  const int lo = __builtin_amdgcn_mov_dpp((int)(uint32_t)v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+  const int hi = __builtin_amdgcn_mov_dpp((int)(uint32_t)(v >> 32), 0xB1, 0xF, 0xF, true);
+  return (uint64_t)(uint32_t)lo | ((uint64_t)(uint32_t)hi << 32);
+}
+
 // d[2p], d[2p+1] = the p-th 16-byte piece of this lane's row.  Afterwards they hold piece (lane & 3) of the row of
 // lane (lane & ~3) + p: the 4 x 4 transpose of the pieces among four neighbouring lanes, in two exchanges (with the
 // lane one away, then with the lane two away), every dword moved by one DPP quad permutation.
@@ -164,7 +171,7 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
                                                                           const uint32_t* __restrict__ kid,
                                                                           uint64_t* __restrict__ dom, int n, int kstride,
                                                                           int64_t wstride, int nwords, int shift, int buckets,
-                                                                          int chunk, int* __restrict__ total0,
+                                                                          int chunk, int bands, int* __restrict__ total0,
                                                                           int* __restrict__ witness0, SortParam* __restrict__ param) {
   constexpr int TS = 64 * WW, T = kPrefixThreads;
   constexpr int TPL = 16 / WW;  // tiles that share a 128-byte line of the matrix
@@ -182,10 +189,15 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
   if (tile * WW >= nwords) return;
   const int w0 = tile * WW;
   const int slot0 = w0 * 64;
-  const int64_t first_row = (int64_t)slot0 + (int64_t)blockIdx.y * chunk;
-  if (first_row >= n) return;
+  int64_t first_row = (int64_t)slot0 + (int64_t)blockIdx.y * chunk, end_row = first_row + chunk;
+  if (bands) {  // the same rows for all tiles of a grid row: the tiles left of the diagonal in rows y * chunk ...
+    first_row = (int64_t)blockIdx.y * chunk;
+    end_row = first_row + chunk;
+    if (first_row < slot0) first_row = slot0;
+  }
+  if (first_row >= n || first_row >= end_row) return;
   const int r0 = (int)first_row;
-  const int r1 = (int)(first_row + chunk < n ? first_row + chunk : n);
+  const int r1 = (int)(end_row < n ? end_row : n);
   const int HB = buckets + 2;  // entries of the coarse index per objective
   // per objective k (all arrays [M][...]):
   constexpr int kSetWords = WW * 65;                 // sets[k][w][c]: the slots of the first c members of word w
@@ -396,10 +408,18 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
         if (jq + p < n)
           *reinterpret_cast<ulonglong2*>(dom + (int64_t)(jq + p) * wstride + w0 + 2 * (lane & 3)) =
               make_ulonglong2(d[2 * p], d[2 * p + 1]);
-    } else if (j < n) {
-      ulonglong2* const out = reinterpret_cast<ulonglong2*>(dom + (int64_t)j * wstride + w0);
-#pragma unroll
-      for (int q = 0; q < WW / 2; ++q) out[q] = make_ulonglong2(d[2 * q], d[2 * q + 1]);
+    } else {
+      // tiles of four words: two neighbouring lanes exchange one piece each, a store writes the 32 bytes of a row
+      static_assert(WW == 4, "tiles of four or eight words");
+      const bool odd = (lane & 1) != 0;
+      const uint64_t s0 = odd ? d[0] : d[2], s1 = odd ? d[1] : d[3];
+      const uint64_t g0 = pair_exchange(s0), g1 = pair_exchange(s1);
+      const uint64_t a0 = odd ? g0 : d[0], a1 = odd ? g1 : d[1];  // piece (lane & 1) of the even lane's row
+      const uint64_t b0 = odd ? d[2] : g0, b1 = odd ? d[3] : g1;  // piece (lane & 1) of the odd lane's row
+      const int jp = j - (lane & 1);
+      if (jp < n) *reinterpret_cast<ulonglong2*>(dom + (int64_t)jp * wstride + w0 + 2 * (lane & 1)) = make_ulonglong2(a0, a1);
+      if (jp + 1 < n)
+        *reinterpret_cast<ulonglong2*>(dom + (int64_t)(jp + 1) * wstride + w0 + 2 * (lane & 1)) = make_ulonglong2(b0, b1);
     }
   }
 }
