@@ -34,6 +34,7 @@ struct Options {
   int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 8 objectives (a quarter
                                     // more rows with 2, a quarter fewer with 9 to 16) get their matrix from the per-objective orders (prefix.hpp);
                                     // 0 = never
+  int prefix_mode = 3;  // measurements: 1 = popcounts only, 2 = matrix only
   int prefix_bands = 1;  // stretches of the order-based matrix: 1 = bands of rows counted from row 0, 0 = from each tile's diagonal
 };
 static Options g_opt;
@@ -477,7 +478,7 @@ static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
   const int bands = g_opt.prefix_bands != 0 && L.n >= 98304 ? 1 : 0;
   hipLaunchKernelGGL((dominance_prefix_kernel<M, WW>), dim3(tiles, stretches), dim3(kPrefixThreads), lds, s, w.at<int>(L.pos),
                      w.at<int>(L.scost), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.kstride, L.wstride, L.nwords,
-                     shift, buckets, chunk, bands, w.at<int>(L.total0), w.at<int>(L.witness0),
+                     shift, buckets, chunk, bands, g_opt.prefix_mode, w.at<int>(L.total0), w.at<int>(L.witness0),
                      w.at<SortParam>(L.sortparam));
   EVX_LAUNCH_CHECK();
   // a population with a NaN or an infinity: the pairwise kernel, on a grid that costs nothing when it has nothing to do
@@ -659,6 +660,8 @@ int evox_hip_set_option(const char* name, int64_t value) {
     g_opt.small_sort = (int)value;
   } else if (!strcmp(name, "prefix_min_rows") && value >= 0) {
     g_opt.prefix_min_rows = value;
+  } else if (!strcmp(name, "prefix_mode") && value >= 1 && value <= 3) {
+    g_opt.prefix_mode = (int)value;
   } else if (!strcmp(name, "prefix_bands") && (value == 0 || value == 1)) {
     g_opt.prefix_bands = (int)value;
   } else {

@@ -171,7 +171,7 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
                                                                           const uint32_t* __restrict__ kid,
                                                                           uint64_t* __restrict__ dom, int n, int kstride,
                                                                           int64_t wstride, int nwords, int shift, int buckets,
-                                                                          int chunk, int bands, int* __restrict__ total0,
+                                                                          int chunk, int bands, int mode, int* __restrict__ total0,
                                                                           int* __restrict__ witness0, SortParam* __restrict__ param) {
   constexpr int TS = 64 * WW, T = kPrefixThreads;
   constexpr int TPL = 16 / WW;  // tiles that share a 128-byte line of the matrix
@@ -384,7 +384,7 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
           d[w] &= (1ull << (same_from - first)) - 1ull;
       }
     }
-    if (j < n) {
+    if (j < n && (mode & 1)) {
       // what the count stage wants to know of the row, so that it does not have to read it again
       int dominators = 0, highest = -1;
 #pragma unroll
@@ -397,6 +397,7 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
         atomicMax(&witness0[j], highest);
       }
     }
+    if (!(mode & 2)) continue;
     if constexpr (WW == 8) {
       // Four neighbouring lanes exchange their 16-byte pieces (a 4 x 4 transpose through DPP moves), so that a
       // store instruction writes the whole 64 bytes of a row from four lanes side by side -- one request per row
