@@ -44,7 +44,7 @@ struct Layout {
   int64_t wstride;
   // byte offsets
   size_t ctrl, fsize, fronts_slot, fronts_orig, hist, zero_end, fstart, xs, key, partials, sortparam, bstart, bcursor,
-      scanflags, records, members, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, total0, witness0, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
+      scanflags, records, members, member_key, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, total0, witness0, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
 };
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
@@ -83,6 +83,7 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->bstart = o;     o = align_up(o + sizeof(int) * (size_t)(buckets + 1));
   L->bcursor = o;    o = align_up(o + sizeof(int) * (size_t)buckets);
   L->members = o;    o = align_up(o + sizeof(int) * (size_t)n);
+  L->member_key = o; o = align_up(o + sizeof(uint64_t) * (size_t)n);
   L->xs_sorted = o;  o = align_up(o + sizeof(float) * (size_t)m * L->npad);
   L->key_sorted = o; o = align_up(o + sizeof(uint64_t) * (size_t)L->npad);
   L->kid_sorted = o; o = align_up(o + sizeof(uint32_t) * (size_t)L->npad);
@@ -253,12 +254,13 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
                      w.at<int>(L.bstart), w.at<int>(L.bcursor), w.at<unsigned long long>(L.scanflags), w.ctrl());
   EVX_LAUNCH_CHECK();
   hipLaunchKernelGGL(bucket_scatter_kernel, dim3(blocks), dim3(256), 0, s, w.at<uint64_t>(L.key), L.n,
-                     w.at<SortParam>(L.sortparam), w.at<int>(L.bcursor), w.at<int>(L.members), w.ctrl());
+                     w.at<SortParam>(L.sortparam), w.at<int>(L.bcursor), w.at<int>(L.members), w.at<uint64_t>(L.member_key),
+                     w.ctrl());
   EVX_LAUNCH_CHECK();
   int pblocks = (L.npad + 255) / 256;
   if (pblocks > 2048) pblocks = 2048;
   hipLaunchKernelGGL(bucket_place_kernel, dim3(pblocks), dim3(256), 0, s, w.at<uint64_t>(L.key), w.at<float>(L.xs), L.n, L.m,
-                     L.npad, w.at<SortParam>(L.sortparam), w.at<int>(L.bstart), w.at<int>(L.members),
+                     L.npad, w.at<SortParam>(L.sortparam), w.at<int>(L.bstart), w.at<int>(L.members), w.at<uint64_t>(L.member_key),
                      w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of),
                      w.ctrl());
   EVX_LAUNCH_CHECK();

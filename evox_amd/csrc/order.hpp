@@ -139,11 +139,16 @@ __global__ __launch_bounds__(256) void bucket_scan_kernel(const int* __restrict_
 
 __global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint64_t* __restrict__ key, int n,
                                                              const SortParam* __restrict__ param, int* __restrict__ cursor,
-                                                             int* __restrict__ members, const Ctrl* __restrict__ ctrl) {
+                                                             int* __restrict__ members, uint64_t* __restrict__ member_key,
+                                                             const Ctrl* __restrict__ ctrl) {
   if (ctrl->err != 0) return;
   const SortParam sp = *param;
-  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
-    members[atomicAdd(&cursor[bucket_of(key[i], sp)], 1)] = i;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+    const uint64_t ki = key[i];
+    const int p = atomicAdd(&cursor[bucket_of(ki, sp)], 1);
+    members[p] = i;
+    member_key[p] = ki;  // beside the index, so that the placing kernel reads a bucket without a dependent load
+  }
 }
 
 // Exact slot of every row: bucket start + number of bucket members that precede it by (key, index).
@@ -152,22 +157,38 @@ __global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint64_t* __r
 __global__ __launch_bounds__(256) void bucket_place_kernel(const uint64_t* __restrict__ key, const float* __restrict__ xs, int n,
                                                            int m, int npad, const SortParam* __restrict__ param,
                                                            const int* __restrict__ start, const int* __restrict__ members,
+                                                           const uint64_t* __restrict__ member_key,
                                                            uint64_t* __restrict__ key_sorted, uint32_t* __restrict__ kid_sorted,
                                                            float* __restrict__ xs_sorted, int* __restrict__ orig_of,
                                                            const Ctrl* __restrict__ ctrl) {
   if (ctrl->err != 0) return;
   const SortParam sp = *param;
-  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < npad; i += gridDim.x * blockDim.x) {
-    if (i < n) {
-      const uint64_t ki = key[i];
+  // A thread takes the row at its position in the bucket-ordered member list, not the row of its own index: the
+  // lanes of a wave then walk through the same one or two buckets (their loads fall into the same lines instead of
+  // 64 lists apart) and write neighbouring slots; only the reads of the row's fitness are scattered.
+  for (int t = blockIdx.x * blockDim.x + threadIdx.x; t < npad; t += gridDim.x * blockDim.x) {
+    if (t < n) {
+      const int i = members[t];
+      const uint64_t ki = member_key[t];
       const int b = bucket_of(ki, sp);
       const int lo = start[b], hi = start[b + 1];
       int before = 0, smaller = 0;
-      for (int p = lo; p < hi; ++p) {
-        const int e = members[p];
-        const uint64_t ke = key[e];
-        smaller += ke < ki;
-        before += (ke < ki) || (ke == ki && e < i);
+      // eight members at a time, all loads before any use: a bucket of a clustered population holds dozens of rows,
+      // and one dependent pair of loads per member made this the longest kernel of the slot sort
+      for (int p0 = lo; p0 < hi; p0 += 8) {
+        int e[8];
+        uint64_t ke[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const bool in = p0 + u < hi;
+          e[u] = in ? members[p0 + u] : 0x7FFFFFFF;
+          ke[u] = in ? member_key[p0 + u] : ~0ull;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          smaller += ke[u] < ki;
+          before += (ke[u] < ki) || (ke[u] == ki && e[u] < i);
+        }
       }
       const int slot = lo + before;
       orig_of[slot] = i;
@@ -176,10 +197,10 @@ __global__ __launch_bounds__(256) void bucket_place_kernel(const uint64_t* __res
       // -0.0 is stored as +0.0: every comparison reads the same, and differences of equal values are +0.0
       for (int k = 0; k < m; ++k) xs_sorted[(int64_t)k * npad + slot] = xs[(int64_t)k * npad + i] + 0.0f;
     } else {
-      orig_of[i] = -1;
-      key_sorted[i] = ~0ull;
-      kid_sorted[i] = (uint32_t)i;
-      for (int k = 0; k < m; ++k) xs_sorted[(int64_t)k * npad + i] = __uint_as_float(0x7FC00000u);
+      orig_of[t] = -1;
+      key_sorted[t] = ~0ull;
+      kid_sorted[t] = (uint32_t)t;
+      for (int k = 0; k < m; ++k) xs_sorted[(int64_t)k * npad + t] = __uint_as_float(0x7FC00000u);
     }
   }
 }
