@@ -44,7 +44,7 @@ struct Layout {
   int64_t wstride;
   // byte offsets
   size_t ctrl, fsize, fronts_slot, fronts_orig, hist, zero_end, fstart, xs, key, partials, sortparam, bstart, bcursor,
-      scanflags, records, members, member_key, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, total0, witness0, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
+      scanflags, records, members, member_key, slot_of, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, total0, witness0, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
 };
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
@@ -88,6 +88,7 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->key_sorted = o; o = align_up(o + sizeof(uint64_t) * (size_t)L->npad);
   L->kid_sorted = o; o = align_up(o + sizeof(uint32_t) * (size_t)L->npad);
   L->orig_of = o;    o = align_up(o + sizeof(int) * (size_t)L->npad);
+  L->slot_of = o;    o = align_up(o + sizeof(int) * (size_t)n);
   L->count = o;      o = align_up(o + sizeof(int) * (size_t)n);
   L->witness = o;    o = align_up(o + sizeof(int) * (size_t)n);
   // popcount and highest non-empty word of every row as the order-based dominance kernel leaves them (kept apart
@@ -261,7 +262,7 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
   if (pblocks > 2048) pblocks = 2048;
   hipLaunchKernelGGL(bucket_place_kernel, dim3(pblocks), dim3(256), 0, s, w.at<uint64_t>(L.key), w.at<float>(L.xs), L.n, L.m,
                      L.npad, w.at<SortParam>(L.sortparam), w.at<int>(L.bstart), w.at<int>(L.members), w.at<uint64_t>(L.member_key),
-                     w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of),
+                     w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of), w.at<int>(L.slot_of),
                      w.ctrl());
   EVX_LAUNCH_CHECK();
   return 0;
@@ -502,8 +503,8 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) 
   const int cap = (device_cus() * 2 < kRadixMaxWorkers + kFirstSweeper ? device_cus() * 2 : kRadixMaxWorkers + kFirstSweeper) - kFirstSweeper;
   if (workers > cap) workers = cap;
   if (workers + kFirstSweeper < radix_grid(L)) workers = radix_grid(L) - kFirstSweeper;
-  hipLaunchKernelGGL(objective_order_kernel, dim3(workers + kFirstSweeper), dim3(kRadixThreads), lds, s, w.at<float>(L.xs_sorted), L.npad, L.n,
-                     L.m, w.at<SortParam>(L.sortparam), w.ctrl(), w.at<int>(L.pos), w.at<int>(L.scost), w.at<int>(L.total0),
+  hipLaunchKernelGGL(objective_order_kernel, dim3(workers + kFirstSweeper), dim3(kRadixThreads), lds, s, w.at<float>(L.xs), L.npad, L.n,
+                     L.m, w.at<int>(L.slot_of), w.at<SortParam>(L.sortparam), w.ctrl(), w.at<int>(L.pos), w.at<int>(L.scost), w.at<int>(L.total0),
                      w.at<int>(L.witness0), radix_buffers(w), g_opt.spin_limit);
   EVX_LAUNCH_CHECK();
   // the barrier words of the control block restart from zero for the kernels that follow (the sort counted its
@@ -534,13 +535,33 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) 
 }
 
 // Per-objective ordering of the candidates list[ctrl.worst_start ... + ctrl.nv).
-static int stage_crowd_sort(const Ws& w, const int* list, hipStream_t s) {
+static int stage_crowd_sort(const Ws& w, const int* list, bool use_orders, hipStream_t s) {
   const Layout& L = w.L;
+  use_orders = use_orders && prefix_dominance_applies(L);
+  if (use_orders) {
+    // a large front of a population whose matrix came from the per-objective orders: its own orders are read off
+    // those (finish.hpp); the three kernels and the one below choose on the device which of them has work
+    const RadixBuffers b = radix_buffers(w);
+    const int spans = (L.n + kFrontOrderSpan - 1) / kFrontOrderSpan;
+    int* const number = reinterpret_cast<int*>(w.at<uint32_t>(L.dkey));  // free until the distances are known
+    int* const per_span = b.table;
+    hipLaunchKernelGGL(front_number_kernel, dim3((L.n + 1023) / 1024), dim3(256), 0, s, list, w.ctrl(),
+                       w.at<SortParam>(L.sortparam), number);
+    EVX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(front_order_count_kernel, dim3(spans, L.m), dim3(256), 0, s, b.pairs[0], b.kstride, L.n, w.at<int>(L.rank),
+                       w.ctrl(), w.at<SortParam>(L.sortparam), per_span);
+    EVX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(front_order_place_kernel, dim3(spans, L.m), dim3(256), 0, s, b.pairs[0], b.kstride, L.n,
+                       w.at<int>(L.rank), w.ctrl(), w.at<SortParam>(L.sortparam), per_span, number, w.at<float>(L.xs), L.npad,
+                       w.at<int>(L.pos), w.at<float>(L.scost));
+    EVX_LAUNCH_CHECK();
+  }
   size_t lds = sizeof(uint64_t) * kRankTile;
   if (L.n > kRadixMinCandidates && kRadixLdsBytes > lds) lds = kRadixLdsBytes;
   if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(crowd_sort_kernel), lds)) return e;
   hipLaunchKernelGGL(crowd_sort_kernel, dim3(finish_grid(L, L.m)), dim3(kRadixThreads), lds, s, w.at<float>(L.xs), L.npad, list,
-                     w.ctrl(), L.m, L.kstride, w.at<int>(L.pos), w.at<float>(L.scost), radix_buffers(w), g_opt.spin_limit);
+                     w.ctrl(), L.m, L.kstride, w.at<int>(L.pos), w.at<float>(L.scost), radix_buffers(w), g_opt.spin_limit,
+                     w.at<SortParam>(L.sortparam), use_orders ? 1 : 0);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -552,7 +573,7 @@ static int stage_crowd_finish(const Ws& w, const int* list, bool want_order, hip
   if (L.n > kRadixMinCandidates && kRadixLdsBytes > lds) lds = kRadixLdsBytes;
   hipLaunchKernelGGL(crowd_finish_kernel, dim3(finish_grid(L, 1)), dim3(kRadixThreads), lds, s, list, w.ctrl(), L.m,
                      w.at<int>(L.pos), w.at<float>(L.scost), L.kstride, w.at<float>(L.dist), w.at<uint32_t>(L.dkey),
-                     w.at<int>(L.order), radix_buffers(w), g_opt.spin_limit, want_order ? 1 : 0);
+                     w.at<int>(L.order), radix_buffers(w), g_opt.spin_limit, want_order ? 1 : 0, w.at<SortParam>(L.sortparam));
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -709,7 +730,7 @@ int evox_hip_stage_peel(int64_t n, int64_t m, int64_t stop_count, int32_t* rank_
 int evox_hip_stage_crowding(int64_t n, int64_t m, void* ws, size_t ws_bytes, void* stream) {
   Ws w;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
-  if (int e = stage_crowd_sort(w, w.at<int>(w.L.perm), (hipStream_t)stream)) return e;
+  if (int e = stage_crowd_sort(w, w.at<int>(w.L.perm), true, (hipStream_t)stream)) return e;
   return stage_crowd_finish(w, w.at<int>(w.L.perm), false, (hipStream_t)stream);
 }
 
@@ -786,7 +807,7 @@ int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t
   hipLaunchKernelGGL(compact_mask_kernel, dim3(1), dim3(1024), 0, s, mask, mask_stride, L.n, w.at<int>(L.perm),
                      w.at<float>(L.dist), w.ctrl());
   EVX_LAUNCH_CHECK();
-  if (int e = stage_crowd_sort(w, w.at<int>(L.perm), s)) return e;
+  if (int e = stage_crowd_sort(w, w.at<int>(L.perm), false, s)) return e;
   if (int e = stage_crowd_finish(w, w.at<int>(L.perm), false, s)) return e;
   return copy_async(dist_out, w.at<float>(L.dist), sizeof(float) * (size_t)n, s);
 }
@@ -941,7 +962,7 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   if (int e = stage_dominance(w, kDomAuto, s)) return e;
   if (int e = stage_count(w, true, s)) return e;
   if (int e = stage_peel(w, topk, true, s)) return e;
-  if (int e = stage_crowd_sort(w, w.at<int>(L.perm), s)) return e;
+  if (int e = stage_crowd_sort(w, w.at<int>(L.perm), true, s)) return e;
   if (int e = stage_crowd_finish(w, w.at<int>(L.perm), true, s)) return e;
   int unit = 1;
   if (x != nullptr) {

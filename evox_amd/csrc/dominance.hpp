@@ -248,6 +248,7 @@ __global__ __launch_bounds__(kSmallSortThreads) void small_sort_kernel(
     sp.buckets = 0;
     sp.nonfinite = any_bad != 0;
     sp.totals_valid = 0;
+    sp.orders_valid = 0;
     *param_out = sp;
   }
   const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;

@@ -14,6 +14,7 @@
 #pragma once
 
 #include "crowd.hpp"
+#include "order.hpp"
 #include "radix.hpp"
 
 namespace evx {
@@ -26,13 +27,16 @@ __global__ __launch_bounds__(kRadixThreads) void crowd_sort_kernel(const float* 
                                                                    const int* __restrict__ list_base, Ctrl* __restrict__ ctrl,
                                                                    int m, int kstride, int* __restrict__ pos,
                                                                    float* __restrict__ sorted_cost, RadixBuffers buf,
-                                                                   unsigned spin_limit) {
+                                                                   unsigned spin_limit, SortParam* __restrict__ param,
+                                                                   int use_orders) {
   extern __shared__ uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
   if (coherent_load(&ctrl->err) != 0) return;
   const int nv = ctrl->nv;
   const int* __restrict__ list = list_base + ctrl->worst_start;
+  // a large front of a population whose per-objective orders are at hand is ordered by front_order_*_kernel
+  if (nv > kRadixMinCandidates && use_orders && param->orders_valid != 0) return;
   if (nv <= kRadixMinCandidates) {
     // ranking by counting: one work item per (256 candidates, objective)
     const int qblocks = (nv + (int)blockDim.x - 1) / (int)blockDim.x;
@@ -55,7 +59,10 @@ __global__ __launch_bounds__(kRadixThreads) void crowd_sort_kernel(const float* 
   const unsigned gen0 = radix_generation_base(ctrl);
   if (blockIdx.x == 0) {
     radix_master(ctrl, gen0, 12, spin_limit, scratch);
-    if (threadIdx.x == 0) ctrl->radix_epoch += 1;  // nobody reads it again in this kernel
+    if (threadIdx.x == 0) {
+      ctrl->radix_epoch += 1;  // nobody reads it again in this kernel
+      param->orders_valid = 0;  // the sort has taken the buffer that held them (read at the start of this kernel only)
+    }
     return;
   }
   if (blockIdx.x < kFirstSweeper) return;
@@ -74,6 +81,106 @@ __global__ __launch_bounds__(kRadixThreads) void crowd_sort_kernel(const float* 
     }
 }
 
+// ---- The same per-objective order of a large last front, taken from the orders of the whole population that
+// objective_order_kernel has left in the radix buffer: the candidates of the front, in the order in which they appear
+// among all rows of objective k (value ascending, equal values by original index = by candidate number), are the
+// front in its own order; a candidate's position is the number of candidates before it.  Three launches with no
+// dependence between workgroups inside a launch; each does nothing unless the front is large and the orders are valid.
+constexpr int kFrontOrderSpan = 1024;  // positions per workgroup
+
+__device__ inline bool front_orders_apply(const Ctrl* ctrl, const SortParam* param) {
+  return ctrl->err == 0 && param->orders_valid != 0 && ctrl->nv > kRadixMinCandidates;
+}
+
+// number[list[q]] = q: the candidate number of every row of the front.
+__global__ __launch_bounds__(256) void front_number_kernel(const int* __restrict__ list_base, const Ctrl* __restrict__ ctrl,
+                                                           const SortParam* __restrict__ param, int* __restrict__ number) {
+  if (!front_orders_apply(ctrl, param)) return;
+  const int nv = ctrl->nv;
+  const int* __restrict__ list = list_base + ctrl->worst_start;
+  for (int q = blockIdx.x * blockDim.x + threadIdx.x; q < nv; q += gridDim.x * blockDim.x) number[list[q]] = q;
+}
+
+// per_span[k * gridDim.x + b] = candidates among positions b * kFrontOrderSpan ... of objective k = blockIdx.y.
+__global__ __launch_bounds__(256) void front_order_count_kernel(const unsigned long long* __restrict__ sorted, int kstride, int n,
+                                                                const int* __restrict__ rank, const Ctrl* __restrict__ ctrl,
+                                                                const SortParam* __restrict__ param, int* __restrict__ per_span) {
+  __shared__ int total;
+  if (!front_orders_apply(ctrl, param)) return;
+  const int worst = ctrl->worst;
+  const int k = blockIdx.y;
+  if (threadIdx.x == 0) total = 0;
+  __syncthreads();
+  int mine = 0;
+#pragma unroll
+  for (int u = 0; u < kFrontOrderSpan / 256; ++u) {
+    const int p = blockIdx.x * kFrontOrderSpan + u * 256 + (int)threadIdx.x;
+    if (p < n) mine += rank[(int)(unsigned)(sorted[(int64_t)k * kstride + p] & 0xFFFFFFFFull)] == worst ? 1 : 0;
+  }
+  mine = wave_sum(mine);
+  if ((threadIdx.x & 63) == 0 && mine != 0) atomicAdd(&total, mine);
+  __syncthreads();
+  if (threadIdx.x == 0) per_span[k * gridDim.x + blockIdx.x] = total;
+}
+
+// pos[k][number] and sorted_cost[k][position] of the candidates among the positions of this workgroup.
+__global__ __launch_bounds__(256) void front_order_place_kernel(const unsigned long long* __restrict__ sorted, int kstride, int n,
+                                                                const int* __restrict__ rank, const Ctrl* __restrict__ ctrl,
+                                                                const SortParam* __restrict__ param,
+                                                                const int* __restrict__ per_span, const int* __restrict__ number,
+                                                                const float* __restrict__ xs, int npad, int* __restrict__ pos,
+                                                                float* __restrict__ sorted_cost) {
+  __shared__ int before_span;
+  __shared__ int wave_count[kFrontOrderSpan / 256][4];
+  if (!front_orders_apply(ctrl, param)) return;
+  const int worst = ctrl->worst;
+  const int k = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr int U = kFrontOrderSpan / 256;
+  // the rows at this thread's positions and whether they are candidates: all loads of a step before any use
+  int row[U];
+  bool is[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int p = blockIdx.x * kFrontOrderSpan + u * 256 + (int)threadIdx.x;
+    row[u] = p < n ? (int)(unsigned)(sorted[(int64_t)k * kstride + p] & 0xFFFFFFFFull) : -1;
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) is[u] = row[u] >= 0 && rank[row[u]] == worst;
+  if (threadIdx.x == 0) before_span = 0;
+  __syncthreads();
+  int mine = 0;
+  for (int b = threadIdx.x; b < (int)blockIdx.x; b += 256) mine += per_span[k * gridDim.x + b];
+  mine = wave_sum(mine);
+  if (lane == 0 && mine != 0) atomicAdd(&before_span, mine);
+  int in_wave[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const uint64_t members = __builtin_amdgcn_ballot_w64(is[u]);
+    in_wave[u] = __popcll(members & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_count[u][wave] = __popcll(members);
+  }
+  __syncthreads();
+  int number_of[U];
+  float cost[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    number_of[u] = is[u] ? number[row[u]] : 0;
+    cost[u] = is[u] ? xs[(int64_t)k * npad + row[u]] : 0.0f;
+  }
+  int running = before_span;  // candidates before the 256 positions of step u
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    int place = running + in_wave[u];
+    for (int v = 0; v < wave; ++v) place += wave_count[u][v];
+    if (is[u]) {
+      pos[(int64_t)k * kstride + number_of[u]] = place;
+      sorted_cost[(int64_t)k * kstride + place] = cost[u];
+    }
+    running += wave_count[u][0] + wave_count[u][1] + wave_count[u][2] + wave_count[u][3];
+  }
+}
+
 // Crowding distance of every candidate of the last front (written by original index) and, when
 // `want_order` is set, the selection order: the better fronts as listed, then the `need` candidates
 // that come first by (distance descending, NaN after every number, row index) -- jit_fix_operator.py:246-252
@@ -84,7 +191,8 @@ __global__ __launch_bounds__(kRadixThreads) void crowd_finish_kernel(const int* 
                                                                      const float* __restrict__ sorted_cost, int kstride,
                                                                      float* __restrict__ dist, uint32_t* __restrict__ dkey,
                                                                      int* __restrict__ order, RadixBuffers buf,
-                                                                     unsigned spin_limit, int want_order) {
+                                                                     unsigned spin_limit, int want_order,
+                                                                     SortParam* __restrict__ param) {
   extern __shared__ uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
@@ -121,7 +229,10 @@ __global__ __launch_bounds__(kRadixThreads) void crowd_finish_kernel(const int* 
   if (blockIdx.x == 0) {
     if (want_order) {
       radix_master(ctrl, gen0, 13, spin_limit, scratch);
-      if (threadIdx.x == 0) ctrl->radix_epoch += 1;
+      if (threadIdx.x == 0) {
+        ctrl->radix_epoch += 1;
+        param->orders_valid = 0;  // the sort of the distance keys has taken the buffer that held the orders
+      }
     }
     return;
   }

@@ -24,6 +24,7 @@ struct SortParam {
   int buckets;
   int nonfinite;  // some fitness value of the population is NaN or infinite
   int totals_valid;  // the dominance stage has left popcount and highest word of every row (zero after the slot sort)
+  int orders_valid;  // the radix buffer holds every objective's (key, original index) pairs in ascending order (zero after the slot sort)
 };
 
 __device__ inline int bucket_of(uint64_t key, const SortParam& p) { return (int)((key - p.kmin) >> p.shift); }
@@ -59,6 +60,7 @@ __device__ inline SortParam make_sort_param(const unsigned long long* __restrict
   sp.buckets = buckets;
   sp.nonfinite = lds2[2] != 0ull;
   sp.totals_valid = 0;
+  sp.orders_valid = 0;
   const unsigned long long span = lds2[1] >= lds2[0] ? lds2[1] - lds2[0] : 0ull;
   int shift = 0;
   while (shift < 63 && (span >> shift) >= (unsigned long long)buckets) ++shift;
@@ -153,14 +155,14 @@ __global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint64_t* __r
 
 // Exact slot of every row: bucket start + number of bucket members that precede it by (key, index).
 // Writes the slot-ordered copies of the fitness (structure of arrays, NaN padding up to npad), of
-// the keys (all-ones padding) and the slot -> original index table (-1 padding).
+// the keys (all-ones padding), the slot -> original index table (-1 padding) and its inverse.
 __global__ __launch_bounds__(256) void bucket_place_kernel(const uint64_t* __restrict__ key, const float* __restrict__ xs, int n,
                                                            int m, int npad, const SortParam* __restrict__ param,
                                                            const int* __restrict__ start, const int* __restrict__ members,
                                                            const uint64_t* __restrict__ member_key,
                                                            uint64_t* __restrict__ key_sorted, uint32_t* __restrict__ kid_sorted,
                                                            float* __restrict__ xs_sorted, int* __restrict__ orig_of,
-                                                           const Ctrl* __restrict__ ctrl) {
+                                                           int* __restrict__ slot_of, const Ctrl* __restrict__ ctrl) {
   if (ctrl->err != 0) return;
   const SortParam sp = *param;
   // A thread takes the row at its position in the bucket-ordered member list, not the row of its own index: the
@@ -192,6 +194,7 @@ __global__ __launch_bounds__(256) void bucket_place_kernel(const uint64_t* __res
       }
       const int slot = lo + before;
       orig_of[slot] = i;
+      slot_of[i] = slot;
       key_sorted[slot] = ki;
       kid_sorted[slot] = (uint32_t)(lo + smaller);  // first slot holding this key: equal ids <=> equal keys
       // -0.0 is stored as +0.0: every comparison reads the same, and differences of equal values are +0.0

@@ -60,12 +60,17 @@ __host__ __device__ inline int prefix_bucket_shift(int n) {
   return shift;
 }
 
-// pos[k * kstride + slot] = position of the slot in the ascending order of objective k (ties in any order);
-// upper[k * kstride + slot] = number of slots whose value in objective k is at most this slot's.
+// pos[k * kstride + slot] = position of the slot's row in the ascending order of objective k, equal values in the
+// order of the original row index (the order of a stable sort of the population as the caller holds it, which the
+// ordering of the last front takes over: front_order_kernels below);
+// upper[k * kstride + slot] = number of rows whose value in objective k is at most this slot's.
+// `xs` = the fitness by original index, `slot_of` = original index -> slot.  The sorted (key, original index) pairs
+// stay in buf.pairs[0] and param->orders_valid says so.
 // Grid: the radix grid (all blocks resident).  Dynamic LDS: kRadixLdsBytes.  Nothing is done for a
 // population with a NaN or an infinity.
 __global__ __launch_bounds__(kRadixThreads) void objective_order_kernel(const float* __restrict__ xs, int npad, int n, int m,
-                                                                        const SortParam* __restrict__ param,
+                                                                        const int* __restrict__ slot_of,
+                                                                        SortParam* __restrict__ param,
                                                                         Ctrl* __restrict__ ctrl, int* __restrict__ pos,
                                                                         int* __restrict__ upper, int* __restrict__ total0,
                                                                         int* __restrict__ witness0, RadixBuffers buf,
@@ -96,7 +101,7 @@ __global__ __launch_bounds__(kRadixThreads) void objective_order_kernel(const fl
     for (int p = wb * blockDim.x + threadIdx.x; p < n; p += workers * blockDim.x) {
       const unsigned long long pr = coherent_load(&sorted[p]);
       const uint32_t key = (uint32_t)(pr >> 32);
-      const int slot = (int)(unsigned)(pr & 0xFFFFFFFFull);
+      const int slot = slot_of[(int)(unsigned)(pr & 0xFFFFFFFFull)];
       int e = p + 1;
       if (e < n && (uint32_t)(coherent_load(&sorted[e]) >> 32) == key) {
         // a run of equal values: its end by bisection (the first position whose key is larger, or n)
@@ -114,6 +119,7 @@ __global__ __launch_bounds__(kRadixThreads) void objective_order_kernel(const fl
       upper[(int64_t)k * buf.kstride + slot] = e;
     }
   }
+  if (wb == 0 && threadIdx.x == 0) param->orders_valid = 1;
 }
 
 // The value that the neighbouring lane (lane ^ 1) passes in, by two DPP quad permutations.

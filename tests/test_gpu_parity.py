@@ -750,6 +750,28 @@ def test_c5_full_size_against_c_checker(population_path):
     runtime.release_workspaces()
 
 
+def test_large_front_ordered_from_the_objective_orders_with_ties():
+    """A population large enough for the order-based matrix, whose cut front is large: that front's per-objective
+    order is read off the orders of the whole population.  Values on a coarse grid, so that every objective has long
+    runs of equal values (which a stable sort keeps in index order) and duplicate rows; against the plain-C checker."""
+    from oracle import c_oracle
+
+    say("large_front_from_orders_ties")
+    for n, m, scale, topk, seed in ((70000, 8, 32.0, 35000, 5), (70000, 4, 8.0, 60000, 6)):  # the second: 66806 duplicate rows
+        f = (workloads.sphere_shell_population((n,), m, 0.05, seed=seed) * scale).round() / scale
+        f = f.contiguous()
+        order, rank, dist, fronts = c_oracle.select(as_np(f), topk)
+        x = torch.arange(n, dtype=torch.int32, device=DEV)[:, None]
+        xs, fs, rs, ds = nd_environmental_selection(x, f.to(DEV), topk)
+        st = runtime.last_status()
+        assert st["error"] == 0 and st["last_front_size"] > 8192, st
+        assert np.array_equal(as_np(xs)[:, 0].astype(np.int64), order)
+        assert np.array_equal(as_np(rs), rank[order])
+        assert_dist_close(ds, dist[order], f"ties {n}x{m}")
+        assert np.array_equal(as_np(fs), as_np(f)[order])
+        runtime.release_workspaces()
+
+
 def test_stop_early_matches_full_ranking(peel_algorithm):
     say("stop_early", peel_algorithm)
     f = workloads.uniform_population(4000, 3, 0, 21)[0]
