@@ -772,6 +772,30 @@ def test_large_front_ordered_from_the_objective_orders_with_ties():
         runtime.release_workspaces()
 
 
+def test_large_front_ordered_from_the_objective_orders_twelve_objectives():
+    """The same with twelve objectives (tiles of four words, the lower row limit of the order-based matrix).  The
+    distance is a sum of twelve terms, associated differently from the checker's (tolerance 1e-5), so rows whose
+    distances nearly tie may swap: the order is checked through what defines it."""
+    from oracle import c_oracle
+
+    say("large_front_from_orders_m12")
+    n, m, topk = 52000, 12, 30000
+    f = ((workloads.sphere_shell_population((n,), m, 0.05, seed=8) * 64.0).round() / 64.0).contiguous()
+    order, rank, dist, fronts = c_oracle.select(as_np(f), topk)
+    x = torch.arange(n, dtype=torch.int32, device=DEV)[:, None]
+    xs, fs, rs, ds = nd_environmental_selection(x, f.to(DEV), topk)
+    st = runtime.last_status()
+    assert st["error"] == 0 and st["last_front_size"] > 8192, st
+    picked = as_np(xs)[:, 0].astype(np.int64)
+    assert len(set(picked.tolist())) == topk
+    assert np.array_equal(as_np(rs), rank[picked]) and np.array_equal(as_np(fs), as_np(f)[picked])
+    assert_dist_close(ds, dist[picked], "ties 52000x12")
+    got_d = as_np(ds).astype(np.float64)
+    key = np.where(np.isnan(got_d), -np.inf, got_d)
+    assert np.array_equal(picked, picked[np.lexsort((picked, -key, as_np(rs)))])  # rank, distance descending, index
+    runtime.release_workspaces()
+
+
 def test_stop_early_matches_full_ranking(peel_algorithm):
     say("stop_early", peel_algorithm)
     f = workloads.uniform_population(4000, 3, 0, 21)[0]
