@@ -422,7 +422,8 @@ def main():
     # large finite populations get the matrix from the order of the rows in every objective instead (the library's
     # rule: at least 65536 rows with 3 to 8 objectives, 81920 with 2, 49152 with 9 to 16): no pairwise test is executed at all
     from_orders = finite and ((3 <= m <= 8 and n >= 65536) or (m == 2 and n >= 81920) or (9 <= m <= 16 and n >= 49152))
-    valu_per_pair = m + (m // 2) + 2 if finite else m + 2
+    # (up to three objectives the sign of the OR is shifted in by one v_alignbit_b32 and the word complemented at the end)
+    valu_per_pair = (m + (m // 2) + (1 if m <= 3 else 2)) if finite else m + 2
     executed_valu = valu_per_pair * evaluated_pairs
     executed_peak = VALU_FP32_PEAK_GOPS if finite else VALU_CMP_PEAK_GOPS
     count_bytes = int(row_read.sum()) + n * 12
