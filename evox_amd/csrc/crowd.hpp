@@ -108,7 +108,7 @@ __device__ inline float crowding_distance_of(int q, int nv, int m, const int* __
 
 // out[p, :] = src[order[p], :] for the decision vectors (raw bytes, any dtype), the fitness, the rank
 // and the distance.  Rows from n_first on are read from the second part (x2, f2) of a two-part population.
-// One wave per output row; rows are copied in 16-, 4- or 1-byte units.
+// Rows are copied in 16-, 4- or 1-byte units, a row by 4 to 64 lanes of a wave.
 __global__ __launch_bounds__(256) void gather_kernel(const int* __restrict__ order, int topk, const uint8_t* __restrict__ x,
                                                      int64_t x_row_stride, int64_t x_row_bytes, uint8_t* __restrict__ out_x,
                                                      int unit, const float* __restrict__ f, int64_t f_stride_row,
@@ -119,26 +119,33 @@ __global__ __launch_bounds__(256) void gather_kernel(const int* __restrict__ ord
                                                      int* __restrict__ out_rank, const float* __restrict__ dist,
                                                      float* __restrict__ out_dist, const Ctrl* __restrict__ ctrl) {
   if (ctrl->err != 0) return;  // `order` was not produced: the outputs stay as the caller left them
-  const int lane = threadIdx.x & 63;
-  const int waves = gridDim.x * (blockDim.x >> 6);
-  for (int p = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); p < topk; p += waves) {
+  // A row is copied by g lanes, g = the smallest power of two (4 .. 64) that holds the row's units and its m
+  // fitness values: short rows share a wave (a row of 400 bytes in 16-byte units took 25 of 64 lanes).
+  const int64_t units = (x ? x_row_bytes : 0) / unit;
+  int g = 64;
+  while (g > 4 && (g >> 1) >= units && (g >> 1) >= m) g >>= 1;
+  const int per_wave = 64 / g;
+  const int lane = (threadIdx.x & 63) % g, sub = (threadIdx.x & 63) / g;
+  const int64_t waves = (int64_t)gridDim.x * (blockDim.x >> 6);
+  for (int64_t p = ((int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * per_wave + sub; p < topk;
+       p += waves * per_wave) {
     const int64_t src = order[p];
     const bool second = src >= n_first;  // rows of the second part of a two-part population
     if (x) {
       const uint8_t* __restrict__ s = second ? x2 + (src - n_first) * x2_row_stride : x + src * x_row_stride;
-      uint8_t* __restrict__ d = out_x + (int64_t)p * x_row_bytes;
+      uint8_t* __restrict__ d = out_x + p * x_row_bytes;
       if (unit == 16) {
-        for (int64_t b = lane * 16; b < x_row_bytes; b += 64 * 16)
+        for (int64_t b = lane * 16; b < x_row_bytes; b += g * 16)
           *reinterpret_cast<uint4*>(d + b) = *reinterpret_cast<const uint4*>(s + b);
       } else if (unit == 4) {
-        for (int64_t b = lane * 4; b < x_row_bytes; b += 64 * 4)
+        for (int64_t b = lane * 4; b < x_row_bytes; b += g * 4)
           *reinterpret_cast<uint32_t*>(d + b) = *reinterpret_cast<const uint32_t*>(s + b);
       } else {
-        for (int64_t b = lane; b < x_row_bytes; b += 64) d[b] = s[b];
+        for (int64_t b = lane; b < x_row_bytes; b += g) d[b] = s[b];
       }
     }
-    for (int k = lane; k < m; k += 64)
-      out_f[(int64_t)p * m + k] =
+    for (int k = lane; k < m; k += g)
+      out_f[p * m + k] =
           second ? f2[(src - n_first) * f2_stride_row + k * f2_stride_col] : f[src * f_stride_row + k * f_stride_col];
     if (lane == 0) {
       out_rank[p] = rank[src];
