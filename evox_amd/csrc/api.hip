@@ -34,6 +34,8 @@ struct Options {
   int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 8 objectives (a quarter
                                     // more rows with 2, a quarter fewer with 9 to 16) get their matrix from the per-objective orders (prefix.hpp);
                                     // 0 = never
+  int64_t prefix_double_tile = 131072;  // order-based matrix, up to four objectives: from this many rows on a workgroup
+                                        // takes both tiles of a 128-byte line; 0 = never
   int prefix_mode = 3;  // measurements: 1 = popcounts only, 2 = matrix only
   int prefix_bands = 1;  // stretches of the order-based matrix: 1 = bands of rows counted from row 0, 0 = from each tile's diagonal
 };
@@ -467,23 +469,34 @@ static int finish_grid(const Layout& L, int per_candidate_block) {
 template <int M>
 static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
   constexpr int WW = M <= kPrefixWideObjectives ? 8 : 4;  // words per tile: what the LDS holds tables for
+  // up to four objectives the tables of two tiles fit: a workgroup then builds whole 128-byte lines of the matrix
+  constexpr int TT = M <= 4 ? 2 : 1;
   const Layout& L = w.L;
   const int shift = prefix_bucket_shift(L.n);
   const int buckets = ((L.n - 1) >> shift) + 1;
-  const size_t lds = prefix_lds_bytes(M, WW, buckets);
-  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(dominance_prefix_kernel<M, WW>), lds)) return e;
-  const int tiles = (int)round_up((L.nwords + WW - 1) / WW, 128 / WW);
+  const int bands_wanted = g_opt.prefix_bands;
+  // bands of rows shared by all tiles (their stores then fall into the same rows at about the same time) pay from
+  // about 100 000 rows on: 200 000 x 8 1203 -> 1156 us, 100 000 x 8 441 -> 424, but 65536 x 3 181 -> 190
+  const int bands = bands_wanted != 0 && L.n >= 98304 ? 1 : 0;
   // shorter stretches for smaller populations, so that the workgroups still outnumber the compute units
   const int chunk = L.n >= 131072 ? kPrefixRowChunk : (L.n >= 65536 ? kPrefixRowChunk / 2 : kPrefixRowChunk / 4);
   const int stretches = (L.n + chunk - 1) / chunk;
-  // bands of rows shared by all tiles (their stores then fall into the same rows at about the same time) pay from
-  // about 100 000 rows on: 200 000 x 8 1203 -> 1156 us, 100 000 x 8 441 -> 424, but 65536 x 3 181 -> 190
-  const int bands = g_opt.prefix_bands != 0 && L.n >= 98304 ? 1 : 0;
-  hipLaunchKernelGGL((dominance_prefix_kernel<M, WW>), dim3(tiles, stretches), dim3(kPrefixThreads), lds, s, w.at<int>(L.pos),
-                     w.at<int>(L.scost), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.kstride, L.wstride, L.nwords,
-                     shift, buckets, chunk, bands, g_opt.prefix_mode, w.at<int>(L.total0), w.at<int>(L.witness0),
-                     w.at<SortParam>(L.sortparam));
-  EVX_LAUNCH_CHECK();
+  auto launch = [&](auto kernel, int tt) -> int {
+    const size_t lds = (size_t)tt * prefix_lds_bytes(M, WW, buckets);
+    if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(kernel), lds)) return e;
+    const int tiles = (int)round_up((L.nwords + WW * tt - 1) / (WW * tt), 128 / (WW * tt));
+    hipLaunchKernelGGL(kernel, dim3(tiles, stretches), dim3(kPrefixThreads), lds, s, w.at<int>(L.pos), w.at<int>(L.scost),
+                       w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.kstride, L.wstride, L.nwords, shift, buckets,
+                       chunk, bands, g_opt.prefix_mode, w.at<int>(L.total0), w.at<int>(L.witness0), w.at<SortParam>(L.sortparam));
+    EVX_LAUNCH_CHECK();
+    return 0;
+  };
+  // (200 000 x 3: 957 -> 769 us, x 4: 972 -> 797; 100 000 x 3: 319 -> 317; 65536 x 3: 184 -> 220: half as many workgroups)
+  if (TT == 2 && g_opt.prefix_double_tile > 0 && L.n >= g_opt.prefix_double_tile) {
+    if (int e = launch(dominance_prefix_kernel<M, WW, TT>, TT)) return e;
+  } else {
+    if (int e = launch(dominance_prefix_kernel<M, WW, 1>, 1)) return e;
+  }
   // a population with a NaN or an infinity: the pairwise kernel, on a grid that costs nothing when it has nothing to do
   hipLaunchKernelGGL(dominance_nonfinite_kernel<M>, dim3(device_cus() * 8), dim3(256), 0, s, w.at<float>(L.xs_sorted),
                      w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride,
@@ -683,6 +696,8 @@ int evox_hip_set_option(const char* name, int64_t value) {
     g_opt.small_sort = (int)value;
   } else if (!strcmp(name, "prefix_min_rows") && value >= 0) {
     g_opt.prefix_min_rows = value;
+  } else if (!strcmp(name, "prefix_double_tile") && value >= 0) {
+    g_opt.prefix_double_tile = value;
   } else if (!strcmp(name, "prefix_mode") && value >= 1 && value <= 3) {
     g_opt.prefix_mode = (int)value;
   } else if (!strcmp(name, "prefix_bands") && (value == 0 || value == 1)) {

@@ -167,12 +167,14 @@ __device__ inline void quad_transpose_pieces(uint64_t (&d)[8], int lane) {
   for (int w = 0; w < 8; ++w) d[w] = (uint64_t)(uint32_t)v[2 * w] | ((uint64_t)(uint32_t)v[2 * w + 1] << 32);
 }
 
-// grid.x = the ceil(nwords / WW) tiles of dominator slots, rounded up to a multiple of 128 / WW,
-// grid.y = stretches of `chunk` rows, counted from the first row of the tile (rows above it have no word
-// there).  Dynamic LDS: prefix_lds_bytes(M, WW, buckets).  Writes the WW words of the tile in every row of the
-// stretch and adds their popcount to total0[row]; witness0[row] = the highest non-empty word so far (both start
-// from objective_order_kernel's 0 and -1).  Sets param->totals_valid.
-template <int M, int WW>
+// A workgroup takes TT neighbouring tiles of WW words (TT = 2 with WW = 8: the whole 128-byte line of every row).
+// grid.x = the ceil(nwords / (WW * TT)) tile groups of dominator slots, rounded up to a multiple of 128 / (WW * TT),
+// grid.y = stretches of `chunk` rows, counted from the first row of the tile or (bands) from row 0 (rows above the
+// tile have no word there).  Dynamic LDS: TT * prefix_lds_bytes(M, WW, buckets).  Writes the words of its tiles in
+// every row of the stretch and adds their popcount to total0[row]; witness0[row] = the highest non-empty word so far
+// (both start from objective_order_kernel's 0 and -1).  Sets param->totals_valid.  mode: bit 0 = the row totals,
+// bit 1 = the matrix.
+template <int M, int WW, int TT>
 __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const int* __restrict__ pos, const int* __restrict__ upper,
                                                                           const uint32_t* __restrict__ kid,
                                                                           uint64_t* __restrict__ dom, int n, int kstride,
@@ -180,7 +182,7 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
                                                                           int chunk, int bands, int mode, int* __restrict__ total0,
                                                                           int* __restrict__ witness0, SortParam* __restrict__ param) {
   constexpr int TS = 64 * WW, T = kPrefixThreads;
-  constexpr int TPL = 16 / WW;  // tiles that share a 128-byte line of the matrix
+  constexpr int TPL = 16 / (WW * TT);  // workgroups that share a 128-byte line of the matrix
   constexpr int MPL = TS / 64;  // members of the tile per lane when a wave walks through them
   extern __shared__ uint64_t prefix_lds[];
   if (param->nonfinite != 0) return;
@@ -192,8 +194,8 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
   const int die = (int)(linear & 7);
   const int seq = (int)blockIdx.x >> 3;  // this workgroup among those of its die in this row of the grid
   const int tile = TPL * ((seq / TPL) * 8 + die) + seq % TPL;
-  if (tile * WW >= nwords) return;
-  const int w0 = tile * WW;
+  if (tile * WW * TT >= nwords) return;
+  const int w0 = tile * WW * TT;  // the first word of the workgroup's TT tiles (tile `sub` starts WW * sub words on)
   const int slot0 = w0 * 64;
   int64_t first_row = (int64_t)slot0 + (int64_t)blockIdx.y * chunk, end_row = first_row + chunk;
   if (bands) {  // the same rows for all tiles of a grid row: the tiles left of the diagonal in rows y * chunk ...
@@ -210,17 +212,34 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
   constexpr int kOver = kSetWords + TS + 1;          // ... then counts[k][t]: eight byte counts, members of each word among the first t
   const int scratch_words = (HB + TS + 1) / 2;       // histogram and claimed pairs of the build, in the same place
   const int over = kOver > scratch_words ? kOver : scratch_words;
-  uint64_t* const sets = prefix_lds;
-  uint64_t* const counts = sets + kSetWords;
-  int* const mp = reinterpret_cast<int*>(prefix_lds + (size_t)M * over);  // [M][TS + 8]: positions ascending, then INT_MAX
-  int* const sorted = mp + M * (TS + 8);                                     // [M][TS]: position << 9 | slot in tile, ascending
-  uint16_t* const index = reinterpret_cast<uint16_t*>(sorted + M * TS);      // [M][HB]: members in earlier buckets
-  auto hist_of = [&](int k) { return reinterpret_cast<int*>(prefix_lds + (size_t)k * over); };  // [HB]
-  auto claimed_of = [&](int k) { return hist_of(k) + HB; };                                        // [TS]
+  // the tables of tile `sub` of the workgroup (TT = 2: the two tiles of a 128-byte line, so that the workgroup writes
+  // whole lines; their tables fit the LDS up to four objectives)
+  const size_t tile_lds_words = prefix_lds_bytes(M, WW, buckets) / sizeof(uint64_t);
+  uint64_t* tile_lds = prefix_lds;
+  uint64_t* sets = nullptr;
+  uint64_t* counts = nullptr;
+  int* mp = nullptr;           // [M][TS + 8]: positions ascending, then INT_MAX
+  int* sorted = nullptr;       // [M][TS]: position << 9 | slot in tile, ascending
+  uint16_t* index = nullptr;   // [M][HB]: members in earlier buckets
+  int live = 0;                // slots of the tile that hold a row
+  int tile_slot0 = slot0;
+  auto select_tile = [&](int sub) {
+    tile_lds = prefix_lds + (size_t)sub * tile_lds_words;
+    sets = tile_lds;
+    counts = sets + kSetWords;
+    mp = reinterpret_cast<int*>(tile_lds + (size_t)M * over);
+    sorted = mp + M * (TS + 8);
+    index = reinterpret_cast<uint16_t*>(sorted + M * TS);
+    tile_slot0 = slot0 + sub * TS;
+    live = n - tile_slot0 < TS ? n - tile_slot0 : TS;
+  };
+  auto hist_of = [&](int k) { return reinterpret_cast<int*>(tile_lds + (size_t)k * over); };  // [HB]
+  auto claimed_of = [&](int k) { return hist_of(k) + HB; };                                      // [TS]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int live = n - slot0 < TS ? n - slot0 : TS;  // slots of the tile that hold a row
   const int index_stride = (HB + 3) & ~3;
 
+  for (int sub = 0; sub < TT; ++sub) {
+  select_tile(sub);
   // ---- the tile's slots by position, objective by objective
   for (int t = threadIdx.x; t < M * HB; t += T) hist_of(t / HB)[t % HB] = 0;
   for (int t = threadIdx.x; t < M * (TS + 8); t += T) mp[t] = 0x7FFFFFFF;
@@ -233,7 +252,7 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
     const int k = item / TS, i = item - k * TS;
     mine[u] = -1;
     if (item < M * TS && i < live) {
-      const int p = pos[(int64_t)k * kstride + slot0 + i];
+      const int p = pos[(int64_t)k * kstride + tile_slot0 + i];
       mine[u] = (p << 9) | i;
       atomicAdd(&hist_of(k)[p >> shift], 1);
     }
@@ -329,6 +348,8 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
   }
   __syncthreads();
 
+  }  // tiles of the workgroup
+
   // ---- the rows of the stretch, 64 at a time per wave; the inputs of a wave's next rows are fetched while it
   // works on the present ones
   const int groups = (r1 - r0 + 63) / 64;
@@ -349,84 +370,123 @@ __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const 
     for (int k = 0; k < M; ++k) e[k] = e_next[k];
     const int same_from = same_next;  // slots from here on hold rows with the key of row j, or larger keys
     if (g + T / 64 < groups) fetch(g + T / 64);
-    // t[k] = members of objective k that lie before upper_k(j): those of the earlier buckets plus those of the
-    // bucket itself that do (positions ascend, so the members from t on that lie before it are consecutive)
-    int t[M];
-    bool more = false;
+    uint64_t dd[TT][WW];  // per tile: slots that are worse than row j in some objective, then its dominators
+    int dominators = 0, highest = -1;
 #pragma unroll
-    for (int k = 0; k < M; ++k) t[k] = index[k * index_stride + (e[k] >> shift)];
+    for (int sub = 0; sub < TT; ++sub) {
+      select_tile(sub);
+      const int tw0 = w0 + sub * WW;
+      uint64_t(&d)[WW] = dd[sub];
+      // t[k] = members of objective k that lie before upper_k(j): those of the earlier buckets plus those of the
+      // bucket itself that do (positions ascend, so the members from t on that lie before it are consecutive)
+      int t[M];
+      bool more = false;
 #pragma unroll
-    for (int k = 0; k < M; ++k) {
-      const int m0 = mp[k * (TS + 8) + t[k]], m1 = mp[k * (TS + 8) + t[k] + 1];
-      const int a0 = m0 < e[k] ? 1 : 0, a1 = m1 < e[k] ? 1 : 0;
-      t[k] += a0 + a1;
-      more |= a1 != 0;
-    }
-    if (__builtin_amdgcn_ballot_w64(more) != 0ull) {  // three or more members of the tile in one bucket: rare
+      for (int k = 0; k < M; ++k) t[k] = index[k * index_stride + (e[k] >> shift)];
 #pragma unroll
-      for (int k = 0; k < M; ++k)
-        while (mp[k * (TS + 8) + t[k]] < e[k]) ++t[k];
-    }
-    uint64_t d[WW];  // slots that are worse than row j in some objective
-#pragma unroll
-    for (int w = 0; w < WW; ++w) d[w] = 0ull;
-#pragma unroll
-    for (int k = 0; k < M; ++k) {
-      const uint64_t c8 = counts[(size_t)k * over + t[k]];
-      const uint64_t* const set = sets + (size_t)k * over;
-#pragma unroll
-      for (int w = 0; w < WW; ++w) d[w] |= set[w * 65 + (int)((c8 >> (8 * w)) & 255ull)];
-    }
-#pragma unroll
-    for (int w = 0; w < WW; ++w) d[w] = ~d[w];
-    // rows identical to j and everything after them: only near the diagonal (wave-uniform test)
-    if (__builtin_amdgcn_ballot_w64(same_from < slot0 + TS) != 0ull) {
-#pragma unroll
-      for (int w = 0; w < WW; ++w) {
-        const int first = (w0 + w) * 64;
-        if (same_from <= first)
-          d[w] = 0ull;
-        else if (same_from < first + 64)
-          d[w] &= (1ull << (same_from - first)) - 1ull;
+      for (int k = 0; k < M; ++k) {
+        const int m0 = mp[k * (TS + 8) + t[k]], m1 = mp[k * (TS + 8) + t[k] + 1];
+        const int a0 = m0 < e[k] ? 1 : 0, a1 = m1 < e[k] ? 1 : 0;
+        t[k] += a0 + a1;
+        more |= a1 != 0;
       }
-    }
-    if (j < n && (mode & 1)) {
+      if (__builtin_amdgcn_ballot_w64(more) != 0ull) {  // three or more members of the tile in one bucket: rare
+#pragma unroll
+        for (int k = 0; k < M; ++k)
+          while (mp[k * (TS + 8) + t[k]] < e[k]) ++t[k];
+      }
+#pragma unroll
+      for (int w = 0; w < WW; ++w) d[w] = 0ull;
+#pragma unroll
+      for (int k = 0; k < M; ++k) {
+        const uint64_t c8 = counts[(size_t)k * over + t[k]];
+        const uint64_t* const set = sets + (size_t)k * over;
+#pragma unroll
+        for (int w = 0; w < WW; ++w) d[w] |= set[w * 65 + (int)((c8 >> (8 * w)) & 255ull)];
+      }
+#pragma unroll
+      for (int w = 0; w < WW; ++w) d[w] = ~d[w];
+      // rows identical to j and everything after them: only near the diagonal (wave-uniform test)
+      if (__builtin_amdgcn_ballot_w64(same_from < tile_slot0 + TS) != 0ull) {
+#pragma unroll
+        for (int w = 0; w < WW; ++w) {
+          const int first = (tw0 + w) * 64;
+          if (same_from <= first)
+            d[w] = 0ull;
+          else if (same_from < first + 64)
+            d[w] &= (1ull << (same_from - first)) - 1ull;
+        }
+      }
       // what the count stage wants to know of the row, so that it does not have to read it again
-      int dominators = 0, highest = -1;
 #pragma unroll
       for (int w = 0; w < WW; ++w) {
         dominators += __popcll(d[w]);
-        highest = d[w] != 0ull ? w0 + w : highest;
-      }
-      if (dominators != 0) {
-        atomicAdd(&total0[j], dominators);
-        atomicMax(&witness0[j], highest);
+        highest = d[w] != 0ull ? tw0 + w : highest;
       }
     }
+    if (j < n && (mode & 1) && dominators != 0) {
+      atomicAdd(&total0[j], dominators);
+      atomicMax(&witness0[j], highest);
+    }
     if (!(mode & 2)) continue;
-    if constexpr (WW == 8) {
-      // Four neighbouring lanes exchange their 16-byte pieces (a 4 x 4 transpose through DPP moves), so that a
-      // store instruction writes the whole 64 bytes of a row from four lanes side by side -- one request per row
-      // to the memory system instead of four requests of 16 bytes from four instructions.
-      quad_transpose_pieces(d, lane);
-      const int jq = j - (lane & 3);  // the first row of this lane's four
+    if constexpr (WW == 8 && TT == 2) {
+      // Eight neighbouring lanes transpose the eight 16-byte pieces of their rows' lines (four of each tile): inside
+      // the quads as below, then the lower quad hands its pieces of the second tile to the upper quad for the upper
+      // quad's pieces of the first.  A store instruction then writes the whole 128-byte line of a row from eight
+      // lanes side by side: one request of a line to memory instead of two of half a line.
+      quad_transpose_pieces(dd[0], lane);
+      quad_transpose_pieces(dd[1], lane);
+      const bool upper_quad = (lane & 4) != 0;
+      uint64_t other[8];  // piece (lane & 7) of the rows of the other quad
 #pragma unroll
-      for (int p = 0; p < 4; ++p)
-        if (jq + p < n)
-          *reinterpret_cast<ulonglong2*>(dom + (int64_t)(jq + p) * wstride + w0 + 2 * (lane & 3)) =
-              make_ulonglong2(d[2 * p], d[2 * p + 1]);
-    } else {
-      // tiles of four words: two neighbouring lanes exchange one piece each, a store writes the 32 bytes of a row
-      static_assert(WW == 4, "tiles of four or eight words");
-      const bool odd = (lane & 1) != 0;
-      const uint64_t s0 = odd ? d[0] : d[2], s1 = odd ? d[1] : d[3];
-      const uint64_t g0 = pair_exchange(s0), g1 = pair_exchange(s1);
-      const uint64_t a0 = odd ? g0 : d[0], a1 = odd ? g1 : d[1];  // piece (lane & 1) of the even lane's row
-      const uint64_t b0 = odd ? d[2] : g0, b1 = odd ? d[3] : g1;  // piece (lane & 1) of the odd lane's row
-      const int jp = j - (lane & 1);
-      if (jp < n) *reinterpret_cast<ulonglong2*>(dom + (int64_t)jp * wstride + w0 + 2 * (lane & 1)) = make_ulonglong2(a0, a1);
-      if (jp + 1 < n)
-        *reinterpret_cast<ulonglong2*>(dom + (int64_t)(jp + 1) * wstride + w0 + 2 * (lane & 1)) = make_ulonglong2(b0, b1);
+      for (int x = 0; x < 8; ++x) {
+        const uint64_t send = upper_quad ? dd[0][x] : dd[1][x];
+        const int lo = __shfl_xor((int)(uint32_t)send, 4);
+        const int hi = __shfl_xor((int)(uint32_t)(send >> 32), 4);
+        other[x] = (uint64_t)(uint32_t)lo | ((uint64_t)(uint32_t)hi << 32);
+      }
+      const int j8 = j - (lane & 7);  // the first row of this lane's eight
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        // rows 0..3 of the eight belong to the lower quad, rows 4..7 to the upper one
+        const int q = p & 3;
+        const bool own = (p >= 4) == upper_quad;
+        const uint64_t a = own ? (upper_quad ? dd[1][2 * q] : dd[0][2 * q]) : other[2 * q];
+        const uint64_t b = own ? (upper_quad ? dd[1][2 * q + 1] : dd[0][2 * q + 1]) : other[2 * q + 1];
+        if (j8 + p < n)
+          *reinterpret_cast<ulonglong2*>(dom + (int64_t)(j8 + p) * wstride + w0 + 2 * (lane & 7)) = make_ulonglong2(a, b);
+      }
+      continue;
+    }
+#pragma unroll
+    for (int sub = 0; sub < TT; ++sub) {
+      const int tw0 = w0 + sub * WW;
+      uint64_t(&d)[WW] = dd[sub];
+      if constexpr (WW == 8) {
+        // Four neighbouring lanes exchange their 16-byte pieces (a 4 x 4 transpose through DPP moves), so that a
+        // store instruction writes the whole 64 bytes of a row from four lanes side by side -- one request per row
+        // to the memory system instead of four requests of 16 bytes from four instructions.  With two tiles per
+        // workgroup the two halves of a row's line follow one another and leave the cache as one line.
+        quad_transpose_pieces(d, lane);
+        const int jq = j - (lane & 3);  // the first row of this lane's four
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+          if (jq + p < n)
+            *reinterpret_cast<ulonglong2*>(dom + (int64_t)(jq + p) * wstride + tw0 + 2 * (lane & 3)) =
+                make_ulonglong2(d[2 * p], d[2 * p + 1]);
+      } else {
+        // tiles of four words: two neighbouring lanes exchange one piece each, a store writes the 32 bytes of a row
+        static_assert(WW == 4, "tiles of four or eight words");
+        const bool odd = (lane & 1) != 0;
+        const uint64_t s0 = odd ? d[0] : d[2], s1 = odd ? d[1] : d[3];
+        const uint64_t g0 = pair_exchange(s0), g1 = pair_exchange(s1);
+        const uint64_t a0 = odd ? g0 : d[0], a1 = odd ? g1 : d[1];  // piece (lane & 1) of the even lane's row
+        const uint64_t b0 = odd ? d[2] : g0, b1 = odd ? d[3] : g1;  // piece (lane & 1) of the odd lane's row
+        const int jp = j - (lane & 1);
+        if (jp < n) *reinterpret_cast<ulonglong2*>(dom + (int64_t)jp * wstride + tw0 + 2 * (lane & 1)) = make_ulonglong2(a0, a1);
+        if (jp + 1 < n)
+          *reinterpret_cast<ulonglong2*>(dom + (int64_t)(jp + 1) * wstride + tw0 + 2 * (lane & 1)) = make_ulonglong2(b0, b1);
+      }
     }
   }
 }

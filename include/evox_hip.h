@@ -223,7 +223,7 @@ int evox_hip_read_status(const void* workspace, void* stream, int32_t* host_out8
  * protocol, 0 = master barrier and front bitmaps), "peel_record_blocks" (0 = by size, or 16 .. 255), "spin_limit" (polls before a device-side
  * wait gives up, default 4000000), "dominance_tile_words" (4, 8 or 16, default 4), "small_sort" (1 = one-kernel slot sort up to 4096 rows),
  * "prefix_min_rows" (default 65536: smallest finite population whose matrix is built from the per-objective orders, 0 = never),
- * "prefix_bands" (default 1), "prefix_mode" (default 3; 1 and 2 build only half of that kernel's output, for measurements).
+ * "prefix_bands" (default 1), "prefix_double_tile" (default 131072 rows, 0 = never), "prefix_mode" (default 3; 1 and 2 build only half of that kernel's output, for measurements).
  * Returns EVOX_HIP_E_BAD_ARG for an unknown name or a value out of range. */
 int evox_hip_set_option(const char* name, int64_t value);
 

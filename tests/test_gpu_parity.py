@@ -204,12 +204,19 @@ def test_matrix_from_objective_orders_equals_the_pairwise_matrix(m):
     try:
         for name, f in cases.items():
             say("prefix_matrix", m, name, tuple(f.shape))
-            runtime.set_option("prefix_min_rows", 4097)  # (a quarter more rows with two objectives)
-            got_state, want_state = {}, {}
-            got = _matrix_words(f.contiguous(), 0, got_state)
+            want_state = {}
             runtime.set_option("prefix_min_rows", 0)
             want = _matrix_words(f.contiguous(), 0, want_state)
-            assert np.array_equal(got, want), (m, name, int((got != want).sum()))
+            # up to four objectives also with both tiles of a 128-byte line in one workgroup (by default from 131072 rows on)
+            for double_from in (131072, 1) if m <= 4 else (131072,):
+                runtime.set_option("prefix_min_rows", 4097)  # (a quarter more rows with two objectives)
+                runtime.set_option("prefix_double_tile", double_from)
+                got_state = {}
+                got = _matrix_words(f.contiguous(), 0, got_state)
+                assert np.array_equal(got, want), (m, name, double_from, int((got != want).sum()))
+                if double_from == 1:
+                    assert np.array_equal(got_state["count"], want_state["count"]), (m, name)
+            runtime.set_option("prefix_double_tile", 131072)
             # the counts and front 0 that the count stage derives from what the order-based kernel left behind
             assert np.array_equal(got_state["count"], want_state["count"]), (m, name)
             assert np.array_equal(got_state["count"], np.bitwise_count(want).sum(axis=1)), (m, name)
@@ -222,6 +229,7 @@ def test_matrix_from_objective_orders_equals_the_pairwise_matrix(m):
                 assert torch.equal(ranks, non_dominate_rank(fd)), (m, name)
     finally:
         runtime.set_option("prefix_min_rows", 65536)
+        runtime.set_option("prefix_double_tile", 131072)
 
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 8, 11, 16])
