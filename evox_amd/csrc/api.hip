@@ -312,8 +312,8 @@ static int stage_count(const Ws& w, bool fill_dist, hipStream_t s) {
   if (prefix_dominance_applies(L)) {
     // the order-based dominance kernel has left the popcounts: count_kernel above returned at once (the choice is
     // made on the device: a population with a NaN or an infinity went through the pairwise kernel and is counted there)
-    hipLaunchKernelGGL(count_from_totals_kernel, dim3((L.n + 255) / 256), dim3(256), 0, s, w.at<int>(L.total0),
-                       w.at<int>(L.witness0), L.n, w.at<int>(L.orig_of), w.at<int>(L.count), w.at<int>(L.rank),
+    hipLaunchKernelGGL(count_from_totals_kernel, dim3((L.n + 255) / 256 < 128 ? (L.n + 255) / 256 : 128), dim3(256), 0, s, w.at<int>(L.total0),
+                       w.at<int>(L.witness0), L.n, w.at<int>(L.slot_of), w.at<int>(L.count), w.at<int>(L.rank),
                        w.at<int>(L.witness), w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
                        fill_dist ? w.at<float>(L.dist) : (float*)nullptr, w.ctrl(), w.at<SortParam>(L.sortparam));
     EVX_LAUNCH_CHECK();

@@ -200,9 +200,11 @@ __global__ __launch_bounds__(256) void count_kernel(const uint64_t* __restrict__
 
 // The same outputs from total0[j] = popcount of row j and witness0[j] = its highest non-empty word (-1: none), which
 // the order-based dominance kernel (prefix.hpp) accumulates while it builds the matrix: one thread per row, no row
-// is read again.  Does nothing unless that kernel has run for this population.
+// is read again.  Does nothing unless that kernel has run for this population.  A thread is slot j for what is
+// kept by slot and original index j for what is kept by original index (through slot_of, the inverse of orig_of):
+// both bitmaps of front 0 are then written a whole word per wave, with no atomics.
 __global__ __launch_bounds__(256) void count_from_totals_kernel(const int* __restrict__ total0, const int* __restrict__ witness0,
-                                                                int n, const int* __restrict__ orig_of, int* __restrict__ count,
+                                                                int n, const int* __restrict__ slot_of, int* __restrict__ count,
                                                                 int* __restrict__ rank, int* __restrict__ witness,
                                                                 uint64_t* __restrict__ front0_slot,
                                                                 uint64_t* __restrict__ front0_orig, int* __restrict__ fsize,
@@ -212,24 +214,30 @@ __global__ __launch_bounds__(256) void count_from_totals_kernel(const int* __res
   __shared__ int block_found;
   if (threadIdx.x == 0) block_found = 0;
   __syncthreads();
-  const int j = blockIdx.x * blockDim.x + threadIdx.x;
-  bool first = false;
-  if (j < n) {
-    const int total = total0[j];
-    const int o = orig_of[j];
-    count[j] = total;
-    rank[o] = total == 0 ? 0 : kRankUnset;
-    witness[j] = witness0[j];
-    if (dist_fill) dist_fill[o] = -INFINITY;
-    first = total == 0;
-    if (first) atomicOr(reinterpret_cast<unsigned long long*>(front0_orig + (int64_t)(o >> 6) * kFrontStride), 1ull << (o & 63));
+  // (few blocks, each walking through many rows: the blocks queue on the one word that holds the size of front 0)
+  int found = 0;
+  for (int j0 = blockIdx.x * blockDim.x + (threadIdx.x & ~63); j0 < n; j0 += gridDim.x * blockDim.x) {  // wave-uniform
+    const int j = j0 + (threadIdx.x & 63);
+    bool first = false, first_orig = false;
+    if (j < n) {
+      const int total = total0[j];
+      count[j] = total;
+      witness[j] = witness0[j];
+      first = total == 0;
+      first_orig = total0[slot_of[j]] == 0;  // the row whose original index is j
+      rank[j] = first_orig ? 0 : kRankUnset;
+      if (dist_fill) dist_fill[j] = -INFINITY;
+    }
+    const uint64_t members_orig = __builtin_amdgcn_ballot_w64(first_orig);
+    // the 64 rows of a wave share one word of a bitmap: one store instead of up to 64 atomics
+    const uint64_t members = __builtin_amdgcn_ballot_w64(first);
+    if ((threadIdx.x & 63) == 0) {
+      if (members_orig != 0ull) front0_orig[(int64_t)(j0 >> 6) * kFrontStride] = members_orig;
+      if (members != 0ull) front0_slot[(int64_t)(j0 >> 6) * kFrontStride] = members;
+      found += __popcll(members);
+    }
   }
-  // the 64 rows of a wave share one word of the slot bitmap: one store instead of up to 64 atomics
-  const uint64_t members = __builtin_amdgcn_ballot_w64(first);
-  if ((threadIdx.x & 63) == 0 && members != 0ull) {
-    front0_slot[(int64_t)(j >> 6) * kFrontStride] = members;
-    atomicAdd(&block_found, __popcll(members));
-  }
+  if ((threadIdx.x & 63) == 0 && found) atomicAdd(&block_found, found);
   __syncthreads();
   if (threadIdx.x == 0 && block_found) atomicAdd(fsize, block_found);
 }
