@@ -262,7 +262,7 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
   EVX_LAUNCH_CHECK();
   int pblocks = (L.npad + 255) / 256;
   if (pblocks > 2048) pblocks = 2048;
-  hipLaunchKernelGGL(bucket_place_kernel, dim3(pblocks), dim3(256), 0, s, w.at<uint64_t>(L.key), w.at<float>(L.xs), L.n, L.m,
+  hipLaunchKernelGGL(bucket_place_kernel, dim3(pblocks), dim3(256), 0, s, w.at<float>(L.xs), L.n, L.m,
                      L.npad, w.at<SortParam>(L.sortparam), w.at<int>(L.bstart), w.at<int>(L.members), w.at<uint64_t>(L.member_key),
                      w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of), w.at<int>(L.slot_of),
                      w.ctrl());

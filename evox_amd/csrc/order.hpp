@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint64_t* __r
 // Exact slot of every row: bucket start + number of bucket members that precede it by (key, index).
 // Writes the slot-ordered copies of the fitness (structure of arrays, NaN padding up to npad), of
 // the keys (all-ones padding), the slot -> original index table (-1 padding) and its inverse.
-__global__ __launch_bounds__(256) void bucket_place_kernel(const uint64_t* __restrict__ key, const float* __restrict__ xs, int n,
+__global__ __launch_bounds__(256) void bucket_place_kernel(const float* __restrict__ xs, int n,
                                                            int m, int npad, const SortParam* __restrict__ param,
                                                            const int* __restrict__ start, const int* __restrict__ members,
                                                            const uint64_t* __restrict__ member_key,
@@ -175,8 +175,7 @@ __global__ __launch_bounds__(256) void bucket_place_kernel(const uint64_t* __res
       const int b = bucket_of(ki, sp);
       const int lo = start[b], hi = start[b + 1];
       int before = 0, smaller = 0;
-      // eight members at a time, all loads before any use: a bucket of a clustered population holds dozens of rows,
-      // and one dependent pair of loads per member made this the longest kernel of the slot sort
+      // eight members at a time, all loads before any use (a bucket of a clustered population holds dozens of rows)
       for (int p0 = lo; p0 < hi; p0 += 8) {
         int e[8];
         uint64_t ke[8];
