@@ -13,6 +13,7 @@
 #include "hv.hpp"
 #include "order.hpp"
 #include "peel.hpp"
+#include "peel_lds.hpp"
 #include "prefix.hpp"
 #include "radix.hpp"
 
@@ -28,6 +29,8 @@ struct Options {
   int peel_witness = 1;
   int peel_record_blocks = 0;  // sweeping blocks of the record protocol, 16 .. 255 (plus the lister); 0 = by size
   int peel_records = 1;  // record protocol (all-to-all, no master) for populations up to kRecordsMaxRowsWide
+  int peel_lds = 1;      // populations whose lower triangle fits the LDS of the device are peeled from LDS (peel_lds.hpp)
+  int peel_lds_blocks = 0;  // sweeping workgroups of that kernel, 0 = by size
   unsigned spin_limit = 4000000u;
   int dominance_tile_words = 4;
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
@@ -75,7 +78,7 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->fronts_orig = o; o = align_up(o + sizeof(uint64_t) * kFrontBuffers * kFrontStride * (size_t)L->nwords);
   L->hist = o;        o = align_up(o + sizeof(int) * (size_t)buckets);
   L->scanflags = o;   o = align_up(o + sizeof(unsigned long long) * 64);
-  L->records = o;     o = align_up(o + (n <= kRecordsMaxRowsWide ? sizeof(unsigned long long) * kRecRing * kRecUnits : 0));
+  L->records = o;     o = align_up(o + (n <= 32768 ? sizeof(unsigned long long) * kLdsPeelRecordUnits : (n <= kRecordsMaxRowsWide ? sizeof(unsigned long long) * kRecRing * kRecUnits : 0)));
   L->zero_end = o;
   L->fstart = o;     o = align_up(o + sizeof(int) * (size_t)(n + 2));
   L->xs = o;         o = align_up(o + sizeof(float) * (size_t)m * L->npad);
@@ -351,6 +354,67 @@ static int grant_dynamic_lds(const void* kernel, size_t lds) {
     if (e != hipSuccess) return (int)e;
   }
   return 0;
+}
+
+// Sweeping workgroups of the LDS-resident peel for this population and the dynamic LDS each needs; 0 when the
+// population does not fit (or the option is off).  Every workgroup takes a compute unit of its own.
+constexpr size_t kLdsPeelBudget = 160 * 1024 - 512;
+static int lds_peel_plan(const Layout& L, size_t* lds_out) {
+  if (!g_opt.peel_lds || L.n > 32768 || L.nwords > kRecThreads) return 0;  // (the lister keeps original indices in 16 bits and takes a bitmap word per thread)
+  const int most = device_cus() - 1 < 255 ? device_cus() - 1 : 255;  // + the lister; a record holds at least 4 units
+  if (most < 8) return 0;
+  auto fits = [&](int sweepers) {
+    const size_t b = lds_peel_bytes(L.n, L.nwords, sweepers);
+    return b != 0 && b <= kLdsPeelBudget;
+  };
+  if (!fits(most)) return 0;
+  int sweepers = g_opt.peel_lds_blocks;
+  if (sweepers == 0) {
+    // by size: about 64 rows per workgroup, at least 32 workgroups
+    sweepers = L.n / 64 < 32 ? 32 : L.n / 64;
+  }
+  if (sweepers > most) sweepers = most;
+  while (sweepers < most && !fits(sweepers)) sweepers = sweepers + 8 < most ? sweepers + 8 : most;
+  *lds_out = lds_peel_bytes(L.n, L.nwords, sweepers);
+  return sweepers;
+}
+
+static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool fill_dist, int sweepers, size_t lds, hipStream_t s) {
+  const Layout& L = w.L;
+  if (stop_count < 1 || stop_count > L.n) return kErrBadArg;
+  // the attribute belongs to the (kernel, device) pair; every workgroup waits for every other one, so the grid
+  // must be resident at once: checked once per device for the largest LDS size
+  static int resident[64] = {0};  // 0 unknown, else workgroups per compute unit + 1
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return kErrBadArg;
+  if (resident[dev] == 0) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(peel_lds_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)kLdsPeelBudget);
+    if (e != hipSuccess) return (int)e;
+    int per_cu = 0;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, peel_lds_kernel, kRecThreads, kLdsPeelBudget);
+    if (e != hipSuccess) return (int)e;
+    resident[dev] = per_cu + 1;
+  }
+  if ((int64_t)(resident[dev] - 1) * device_cus() < sweepers + 1) return kErrBadArg;
+  hipLaunchKernelGGL(peel_lds_kernel, dim3(sweepers + 1), dim3(kRecThreads), lds, s, w.at<uint64_t>(L.dom), L.wstride, L.nwords, L.n,
+                     w.at<int>(L.orig_of), w.at<int>(L.rank), fill_dist ? w.at<float>(L.dist) : (float*)nullptr,
+                     w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
+                     want_perm ? w.at<int>(L.perm) : (int*)nullptr, w.at<int>(L.fstart), w.ctrl(), (int)stop_count, g_opt.spin_limit,
+                     w.at<unsigned long long>(L.records), sweepers);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+// Counts and peeling for the entry points: one kernel when the matrix fits the LDS of the device, else the count
+// pass over the matrix followed by a peel kernel that rescans rows in memory.
+static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s);
+static int stage_count(const Ws& w, bool fill_dist, hipStream_t s);
+static int count_and_peel(const Ws& w, int64_t stop_count, bool want_perm, bool fill_dist, hipStream_t s) {
+  size_t lds = 0;
+  if (const int sweepers = lds_peel_plan(w.L, &lds)) return launch_lds_peel(w, stop_count, want_perm, fill_dist, sweepers, lds, s);
+  if (int e = stage_count(w, fill_dist, s)) return e;
+  return stage_peel(w, stop_count, want_perm, s);
 }
 
 static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s) {
@@ -688,6 +752,10 @@ int evox_hip_set_option(const char* name, int64_t value) {
     g_opt.peel_record_blocks = (int)value;
   } else if (!strcmp(name, "peel_records") && (value == 0 || value == 1)) {
     g_opt.peel_records = (int)value;
+  } else if (!strcmp(name, "peel_lds") && (value == 0 || value == 1)) {
+    g_opt.peel_lds = (int)value;
+  } else if (!strcmp(name, "peel_lds_blocks") && (value == 0 || (value >= 8 && value <= 255))) {
+    g_opt.peel_lds_blocks = (int)value;
   } else if (!strcmp(name, "spin_limit") && value >= 1 && value <= 0x7FFFFFFFll) {
     g_opt.spin_limit = (unsigned)value;
   } else if (!strcmp(name, "dominance_tile_words") && (value == 4 || value == 8 || value == 16)) {
@@ -737,7 +805,13 @@ int evox_hip_stage_peel(int64_t n, int64_t m, int64_t stop_count, int32_t* rank_
                         void* stream) {
   Ws w;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
-  if (int e = stage_peel(w, stop_count, true, (hipStream_t)stream)) return e;
+  // (the kernel that peels from LDS counts for itself; after stage_count it finds the same front 0 again)
+  size_t lds = 0;
+  if (const int sweepers = lds_peel_plan(w.L, &lds)) {
+    if (int e = launch_lds_peel(w, stop_count, true, true, sweepers, lds, (hipStream_t)stream)) return e;
+  } else if (int e = stage_peel(w, stop_count, true, (hipStream_t)stream)) {
+    return e;
+  }
   if (rank_out) return copy_async(rank_out, w.at<int>(w.L.rank), sizeof(int) * (size_t)n, (hipStream_t)stream);
   return 0;
 }
@@ -763,8 +837,7 @@ int evox_hip_non_dominate_rank_until(const float* f, int64_t n, int64_t m, int64
   hipStream_t s = (hipStream_t)stream;
   if (int e = stage_prepare(w, one_part(f, n, sr, sc), true, s)) return e;
   if (int e = stage_dominance(w, kDomAuto, s)) return e;
-  if (int e = stage_count(w, false, s)) return e;
-  if (int e = stage_peel(w, stop_count, false, s)) return e;
+  if (int e = count_and_peel(w, stop_count, false, false, s)) return e;
   return copy_async(rank_out, w.at<int>(w.L.rank), sizeof(int) * (size_t)n, s);
 }
 
@@ -975,8 +1048,7 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   const Layout& L = w.L;
   if (int e = stage_prepare(w, fit, true, s)) return e;
   if (int e = stage_dominance(w, kDomAuto, s)) return e;
-  if (int e = stage_count(w, true, s)) return e;
-  if (int e = stage_peel(w, topk, true, s)) return e;
+  if (int e = count_and_peel(w, topk, true, true, s)) return e;
   if (int e = stage_crowd_sort(w, w.at<int>(L.perm), true, s)) return e;
   if (int e = stage_crowd_finish(w, w.at<int>(L.perm), true, s)) return e;
   int unit = 1;

@@ -642,6 +642,7 @@ __device__ inline void witness_rows_pooled(WitnessState& st, const PassCtx& c, c
 // Block-wide listing of the set bits of `front` (nwords words, LDS) in ascending order into
 // perm[base ...]; the words are words first_word ... of the whole bitmap.  `scratch` holds at least
 // blockDim.x / 64 ints.
+template <bool LDS_BARRIERS = false>  // true: the barriers inside order LDS traffic only (see lds_barrier)
 __device__ inline void list_front(const uint64_t* front_lds, int nwords, int* __restrict__ perm, int base, int* scratch,
                                   int first_word = 0) {
   // each thread owns a contiguous slice of words so that the order is ascending
@@ -660,7 +661,7 @@ __device__ inline void list_front(const uint64_t* front_lds, int nwords, int* __
     if (lane >= off) incl += up;
   }
   if (lane == 63) scratch[wave] = incl;
-  __syncthreads();
+  if (LDS_BARRIERS) lds_barrier(); else __syncthreads();
   int pos = base + incl - mine;
   for (int v = 0; v < wave; ++v) pos += scratch[v];
   for (int w = w_begin; w < w_end; ++w) {
@@ -671,7 +672,7 @@ __device__ inline void list_front(const uint64_t* front_lds, int nwords, int* __
       bits &= bits - 1;
     }
   }
-  __syncthreads();
+  if (LDS_BARRIERS) lds_barrier(); else __syncthreads();
 }
 
 // --------------------------------------------------------- persistent peel

@@ -341,13 +341,16 @@ def test_rank_strided_and_half_inputs():
     assert np.array_equal(as_np(non_dominate_rank(h.to(DEV))), as_np(er.ranks_by_peeling(h.float())))
 
 
-@pytest.fixture(params=["witness-records", "witness-master", "sweep"])
+@pytest.fixture(params=["lds", "witness-records", "witness-master", "sweep"])
 def peel_algorithm(request):
-    """The peeling variants: witness pass with the record protocol (default), witness pass with the
-    master barrier and front bitmaps, and the popcount-decrement sweep (master barrier)."""
+    """The peeling variants: matrix rows resident in LDS (default where the matrix fits), and the three that rescan
+    rows in memory: witness pass with the record protocol, witness pass with the master barrier and front
+    bitmaps, and the popcount-decrement sweep (master barrier)."""
+    runtime.set_option("peel_lds", 1 if request.param == "lds" else 0)
     runtime.set_option("peel_witness", 0 if request.param == "sweep" else 1)
     runtime.set_option("peel_records", 1 if request.param == "witness-records" else 0)
     yield request.param
+    runtime.set_option("peel_lds", 1)
     runtime.set_option("peel_witness", 1)
     runtime.set_option("peel_records", 1)
 
