@@ -11,11 +11,13 @@ from .build import LIB_PATH
 E_BAD_ARG = -1
 E_WORKSPACE = -2
 E_BARRIER_TIMEOUT = -3
+E_STATIC_LIMIT = -4
 
 _MESSAGES = {
     E_BAD_ARG: "invalid argument",
     E_WORKSPACE: "workspace too small or misaligned",
     E_BARRIER_TIMEOUT: "a device-side wait ran out of polls (grid barrier timeout)",
+    E_STATIC_LIMIT: "the population needs more scratch memory than the library's own buffer holds",
 }
 
 _SIGNATURES = {
@@ -35,6 +37,8 @@ _SIGNATURES = {
                                                              c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                                              c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                              c_void_p, c_size_t, c_void_p]),
+    "evox_hip_nd_environmental_selection_static": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                                           c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "evox_hip_batched_max_rows": (c_int64, [c_int64]),
     "evox_hip_batched_non_dominate_rank": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p,
                                                    c_void_p]),

@@ -3,6 +3,8 @@
 // evox_hip_read_status().
 #include <string.h>
 
+#include <atomic>
+
 #include "../../include/evox_hip.h"
 #include "batched.hpp"
 #include "calibrate.hpp"
@@ -1101,6 +1103,48 @@ int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_ro
   const Fitness fit{f_a, f_a_stride_row, f_a_stride_col, n_a, f_b, f_b_stride_row, f_b_stride_col};
   return select_rows(x_a, x_row_bytes, x_a_row_stride_bytes, x_b, x_b_row_stride_bytes, fit, n_a + n_b, m, topk, out_x, out_f,
                      out_rank, out_dist, out_order, ws, ws_bytes, (hipStream_t)stream);
+}
+
+}  // extern "C"
+
+// Scratch memory of the entry point that allocates nothing: part of the device image, one copy per GPU.  In host
+// code the array's name stands for the symbol, not for device memory: its address on the current GPU comes from
+// hipGetSymbolAddress, looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[EVOX_HIP_STATIC_SCRATCH_BYTES];
+static std::atomic<void*> g_scratch_ptr[64];
+
+static int static_scratch(void** out) {
+  int dev = 0;
+  const hipError_t de = hipGetDevice(&dev);
+  if (de != hipSuccess) return (int)de;
+  if (dev < 0 || dev >= 64) return kErrBadArg;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (p == nullptr || (reinterpret_cast<uintptr_t>(p) & 255u) != 0) return kErrWorkspace;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // (two first calls at once look up the same address)
+  }
+  *out = p;
+  return 0;
+}
+
+extern "C" {
+
+int evox_hip_nd_environmental_selection_static(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes,
+                                               const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, int64_t topk,
+                                               void* out_x, float* out_f, int32_t* out_rank, float* out_dist,
+                                               int32_t* out_order, void* stream) {
+  if (f == nullptr) return kErrBadArg;
+  const size_t need = evox_hip_workspace_bytes(n, m);
+  if (need == 0) return kErrBadArg;
+  if (need > (size_t)EVOX_HIP_STATIC_SCRATCH_BYTES) return kErrStaticLimit;
+  void* ws = nullptr;
+  if (int e = static_scratch(&ws)) return e;
+  // every call clears the part of the buffer that must start from zero (stage_prepare), whatever the call before
+  // left there
+  return select_rows(x, x_row_bytes, x_row_stride_bytes, x, x_row_stride_bytes, one_part(f, n, sr, sc), n, m, topk, out_x,
+                     out_f, out_rank, out_dist, out_order, ws, (size_t)EVOX_HIP_STATIC_SCRATCH_BYTES, (hipStream_t)stream);
 }
 
 int64_t evox_hip_batched_max_rows(int64_t m) { return (m >= 1 && m <= kBatchedMaxObjectives) ? kBatchedMaxRows : 0; }

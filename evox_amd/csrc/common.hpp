@@ -12,6 +12,7 @@ constexpr int kWave = 64;
 constexpr int kErrBadArg = -1;
 constexpr int kErrWorkspace = -2;
 constexpr int kErrBarrierTimeout = -3;
+constexpr int kErrStaticLimit = -4;
 
 constexpr int kRankUnset = 0x7FFFFFFF;  // rank of a row that has not been peeled (yet)
 

@@ -5,7 +5,8 @@
  *   - Return value: 0 on success, a negative library code (EVOX_HIP_E_*) or a positive hipError_t.
  *     No exceptions cross the boundary and nothing aborts.
  *   - The caller owns every buffer, including the workspace; the library allocates no device memory
- *     and synchronises only in evox_hip_read_status().  All work is enqueued on `stream`
+ *     and synchronises only in evox_hip_read_status().  (One entry point brings its own scratch memory
+ *     instead of taking a workspace: evox_hip_nd_environmental_selection_static.)  All work is enqueued on `stream`
  *     (a hipStream_t passed as void*).
  *   - Fitness `f` is float32, addressed as f[i * stride_row + k * stride_col] (strides in elements),
  *     minimisation, n rows (individuals) by m columns (objectives).
@@ -27,6 +28,7 @@ extern "C" {
 #define EVOX_HIP_E_BAD_ARG (-1)         /* null pointer, n < 1, m < 1, topk outside [1, n], ... */
 #define EVOX_HIP_E_WORKSPACE (-2)       /* workspace too small or misaligned */
 #define EVOX_HIP_E_BARRIER_TIMEOUT (-3) /* reported by evox_hip_read_status(): a bounded device-side wait ran out */
+#define EVOX_HIP_E_STATIC_LIMIT (-4)    /* the population needs more scratch than the library's own buffer holds */
 
 int evox_hip_abi_version(void);
 
@@ -102,6 +104,20 @@ int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_ro
                                                  int64_t f_b_stride_col, int64_t m, int64_t topk, void* out_x, float* out_f,
                                                  int32_t* out_rank, float* out_dist, int32_t* out_order, void* workspace,
                                                  size_t workspace_bytes, void* stream);
+
+/* The same selection for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): no counterpart in the reference.  It takes no workspace: the scratch
+ * memory is a buffer of EVOX_HIP_STATIC_SCRATCH_BYTES bytes that is part of the library's device image, one copy per
+ * GPU, held until the process ends.  The call allocates and frees nothing.  Results are those of
+ * evox_hip_nd_environmental_selection.  A population with evox_hip_workspace_bytes(n, m) >
+ * EVOX_HIP_STATIC_SCRATCH_BYTES (about 14 000 rows of 3 objectives, 11 000 of 16) is refused with
+ * EVOX_HIP_E_STATIC_LIMIT.  All calls on one GPU share the buffer: calls on different streams of one GPU that
+ * overlap in time race, the caller must order them. */
+#define EVOX_HIP_STATIC_SCRATCH_BYTES (32u << 20)
+int evox_hip_nd_environmental_selection_static(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes,
+                                               const float* f, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col,
+                                               int64_t topk, void* out_x, float* out_f, int32_t* out_rank, float* out_dist,
+                                               int32_t* out_order, void* stream);
 
 /* ---- many small populations at once (what the reference reaches through vmap: non_dominate.py:107-125
  * for the peeling, the rest of the path batching natively).  One workgroup per population, no workspace.
