@@ -7,7 +7,7 @@ The package holds only this hot path: HIP kernels for gfx950 behind a C ABI (``c
 (``operators.selection``, ``utils.lexsort``).
 """
 
-__all__ = ["hype", "metrics", "operators", "ops", "runtime", "utils", "workloads", "install_into_evox"]
+__all__ = ["hype", "metrics", "operators", "ops", "runtime", "utils", "workloads", "install_into_evox", "uninstall_from_evox"]
 
 from . import hype, metrics, operators, ops, runtime, utils, workloads
-from .compat import install_into_evox
+from .compat import install_into_evox, uninstall_from_evox

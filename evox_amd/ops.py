@@ -16,6 +16,19 @@ import torch
 from . import _lib, runtime
 
 
+def _batched_first(info, dims, tensors):
+    """The tensors of a vmap rule with the mapped dimension in front; those that are not mapped are expanded."""
+    out = []
+    for t, d in zip(tensors, dims):
+        if t is None:
+            out.append(None)
+        elif d is None:
+            out.append(t.unsqueeze(0).expand(info.batch_size, *t.shape))
+        else:
+            out.append(t.movedim(d, 0))
+    return out
+
+
 def _as_f32(t: torch.Tensor, what: str) -> torch.Tensor:
     if t.dtype == torch.float32:
         return t
@@ -378,6 +391,16 @@ def _(x_a, f_a, x_b, f_b, topk):
     )
 
 
+def _nd_select_two_part_vmap(info, in_dims, x_a, f_a, x_b, f_b, topk):
+    # populations side by side: the concatenation is the definition of the result, and the batched operator
+    # takes small populations through the one-workgroup kernel
+    x_a, f_a, x_b, f_b = _batched_first(info, in_dims[:4], (x_a, f_a, x_b, f_b))
+    return nd_select(torch.cat([x_a, x_b], dim=1), torch.cat([f_a, f_b], dim=1), topk), (0, 0, 0, 0)
+
+
+torch.library.register_vmap(nd_select_two_part, _nd_select_two_part_vmap)
+
+
 @torch.library.custom_op("evox_amd::stable_argsort_step", mutates_args=())
 def stable_argsort_step(key: torch.Tensor, kind: int, prev: Optional[torch.Tensor]) -> torch.Tensor:
     """One step of lexsort on a 1-D key of 4-byte elements: ``prev`` (int32 order, or None for the
@@ -446,6 +469,21 @@ def _(key, kind, prev):
     return key.new_empty(key.shape, dtype=torch.int32)
 
 
+def _stable_argsort_step_vmap(info, in_dims, key, kind, prev):
+    key, prev = _batched_first(info, (in_dims[0], in_dims[2]), (key, prev))
+    return stable_argsort_rows(key, kind, prev), 0  # one sort per row
+
+
+def _stable_argsort_rows_vmap(info, in_dims, key, kind, prev):
+    key, prev = _batched_first(info, (in_dims[0], in_dims[2]), (key, prev))
+    flat_prev = None if prev is None else prev.reshape(-1, prev.shape[-1])
+    return stable_argsort_rows(key.reshape(-1, key.shape[-1]), kind, flat_prev).view(key.shape), 0
+
+
+torch.library.register_vmap(stable_argsort_step, _stable_argsort_step_vmap)
+torch.library.register_vmap(stable_argsort_rows, _stable_argsort_rows_vmap)
+
+
 @torch.library.custom_op("evox_amd::hv_contributions", mutates_args=())
 def hv_contributions(fit: torch.Tensor, samples: torch.Tensor, alpha: torch.Tensor, scale: float) -> torch.Tensor:
     """fit (N, M), samples (S, M), alpha (N,) float32 -> (N,) float32:
@@ -473,6 +511,14 @@ def hv_contributions(fit: torch.Tensor, samples: torch.Tensor, alpha: torch.Tens
 @hv_contributions.register_fake
 def _(fit, samples, alpha, scale):
     return fit.new_empty(fit.shape[0], dtype=torch.float32)
+
+
+def _hv_contributions_vmap(info, in_dims, fit, samples, alpha, scale):
+    fit, samples, alpha = _batched_first(info, in_dims[:3], (fit, samples, alpha))
+    return torch.stack([hv_contributions(fit[b], samples[b], alpha[b], scale) for b in range(info.batch_size)]), 0
+
+
+torch.library.register_vmap(hv_contributions, _hv_contributions_vmap)
 
 
 @torch.library.custom_op("evox_amd::hv_covered_count", mutates_args=())
@@ -505,6 +551,14 @@ def _(points, samples):
     return points.new_empty((), dtype=torch.int64)
 
 
+def _hv_covered_count_vmap(info, in_dims, points, samples):
+    points, samples = _batched_first(info, in_dims, (points, samples))
+    return torch.stack([hv_covered_count(points[b], samples[b]) for b in range(info.batch_size)]), 0
+
+
+torch.library.register_vmap(hv_covered_count, _hv_covered_count_vmap)
+
+
 @torch.library.custom_op("evox_amd::tournament_pick", mutates_args=())
 def tournament_pick(parents: torch.Tensor, fitness: torch.Tensor) -> torch.Tensor:
     """parents (n_round, t) int64 candidate indices, fitness (candidates, keys) float32 -> (n_round,) int64 winners."""
@@ -524,3 +578,15 @@ def tournament_pick(parents: torch.Tensor, fitness: torch.Tensor) -> torch.Tenso
 @tournament_pick.register_fake
 def _(parents, fitness):
     return parents.new_empty(parents.shape[0])
+
+
+def _tournament_pick_vmap(info, in_dims, parents, fitness):
+    # tournaments of all the mapped populations in one launch: population b's candidates are rows b * candidates ...
+    parents, fitness = _batched_first(info, in_dims, (parents, fitness))
+    batch, candidates = fitness.shape[0], fitness.shape[1]
+    offset = (torch.arange(batch, device=parents.device, dtype=torch.int64) * candidates).view(batch, 1, 1)
+    flat = tournament_pick((parents + offset).reshape(-1, parents.shape[-1]), fitness.reshape(batch * candidates, -1))
+    return flat.view(batch, -1) - offset.view(batch, 1), 0
+
+
+torch.library.register_vmap(tournament_pick, _tournament_pick_vmap)
