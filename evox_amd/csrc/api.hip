@@ -657,9 +657,19 @@ static int stage_crowd_finish(const Ws& w, const int* list, bool want_order, hip
   return 0;
 }
 
-static int copy_async(void* dst, const void* src, size_t bytes, hipStream_t s) {
-  return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s);
+// The copy of a result of 4-byte elements out of the workspace, as the last kernel of an entry point: the result, or
+// `poison` in every element when a device-side wait of the call ran out.
+static int copy_out(const Ctrl* ctrl, void* dst, const void* src, int64_t n, uint32_t poison, hipStream_t s) {
+  int64_t blocks = (n + 1023) / 1024;
+  if (blocks > 1024) blocks = 1024;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(copy_or_poison_kernel, dim3((unsigned)blocks), dim3(256), 0, s, ctrl, static_cast<const uint32_t*>(src),
+                     static_cast<uint32_t*>(dst), n, poison);
+  EVX_LAUNCH_CHECK();
+  return 0;
 }
+constexpr uint32_t kPoisonIndex = 0xFFFFFFFFu;  // -1 as a rank or an order
+constexpr uint32_t kPoisonFloat = 0x7FC00000u;  // NaN as a distance
 
 template <int M>
 static int launch_batched_m(const BatchedArgs& a, int64_t batch, hipStream_t s) {
@@ -814,7 +824,7 @@ int evox_hip_stage_peel(int64_t n, int64_t m, int64_t stop_count, int32_t* rank_
   } else if (int e = stage_peel(w, stop_count, true, (hipStream_t)stream)) {
     return e;
   }
-  if (rank_out) return copy_async(rank_out, w.at<int>(w.L.rank), sizeof(int) * (size_t)n, (hipStream_t)stream);
+  if (rank_out) return copy_out(w.ctrl(), rank_out, w.at<int>(w.L.rank), n, kPoisonIndex, (hipStream_t)stream);
   return 0;
 }
 
@@ -840,7 +850,7 @@ int evox_hip_non_dominate_rank_until(const float* f, int64_t n, int64_t m, int64
   if (int e = stage_prepare(w, one_part(f, n, sr, sc), true, s)) return e;
   if (int e = stage_dominance(w, kDomAuto, s)) return e;
   if (int e = count_and_peel(w, stop_count, false, false, s)) return e;
-  return copy_async(rank_out, w.at<int>(w.L.rank), sizeof(int) * (size_t)n, s);
+  return copy_out(w.ctrl(), rank_out, w.at<int>(w.L.rank), n, kPoisonIndex, s);
 }
 
 int evox_hip_non_dominate_rank(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, int32_t* rank_out, void* ws,
@@ -899,7 +909,7 @@ int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t
   EVX_LAUNCH_CHECK();
   if (int e = stage_crowd_sort(w, w.at<int>(L.perm), false, s)) return e;
   if (int e = stage_crowd_finish(w, w.at<int>(L.perm), false, s)) return e;
-  return copy_async(dist_out, w.at<float>(L.dist), sizeof(float) * (size_t)n, s);
+  return copy_out(w.ctrl(), dist_out, w.at<float>(L.dist), n, kPoisonFloat, s);
 }
 
 }  // extern "C"
@@ -961,7 +971,8 @@ static int argsort_step(const void* key, int kind, int64_t stride, int64_t n, co
   hipLaunchKernelGGL(argsort_step_kernel, dim3(workers + kFirstSweeper), dim3(kRadixThreads), kRadixLdsBytes, s, key, kind,
                      stride, L.n, prev_order, reinterpret_cast<Ctrl*>(base + L.ctrl), b, order_out, g_opt.spin_limit);
   EVX_LAUNCH_CHECK();
-  return 0;
+  // (an order of -1 everywhere when one of the sort's grid barriers ran out)
+  return copy_out(reinterpret_cast<const Ctrl*>(base + L.ctrl), order_out, nullptr, n, kPoisonIndex, s);
 }
 
 // `batch` sorts of n <= kSmallArgsortRows positions in one launch: a workgroup per sort, or several sorts per
@@ -1065,9 +1076,8 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(256), 0, s, w.at<int>(L.order), (int)topk,
                      static_cast<const uint8_t*>(x), x_row_stride_bytes, x_row_bytes, static_cast<uint8_t*>(out_x), unit, fit.f,
                      fit.sr, fit.sc, (int)fit.n_first, static_cast<const uint8_t*>(x2), x2_row_stride_bytes, fit.f2, fit.sr2,
-                     fit.sc2, L.m, out_f, w.at<int>(L.rank), out_rank, w.at<float>(L.dist), out_dist, w.ctrl());
+                     fit.sc2, L.m, out_f, w.at<int>(L.rank), out_rank, w.at<float>(L.dist), out_dist, out_order, w.ctrl());
   EVX_LAUNCH_CHECK();
-  if (out_order) return copy_async(out_order, w.at<int>(L.order), sizeof(int) * (size_t)topk, s);
   return 0;
 }
 

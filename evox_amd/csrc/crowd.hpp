@@ -117,8 +117,22 @@ __global__ __launch_bounds__(256) void gather_kernel(const int* __restrict__ ord
                                                      int64_t f2_stride_row, int64_t f2_stride_col, int m,
                                                      float* __restrict__ out_f, const int* __restrict__ rank,
                                                      int* __restrict__ out_rank, const float* __restrict__ dist,
-                                                     float* __restrict__ out_dist, const Ctrl* __restrict__ ctrl) {
-  if (ctrl->err != 0) return;  // `order` was not produced: the outputs stay as the caller left them
+                                                     float* __restrict__ out_dist, int* __restrict__ out_order,
+                                                     const Ctrl* __restrict__ ctrl) {
+  if (ctrl->err != 0) {
+    // a device-side wait ran out and `order` was not produced: no partial result leaves the call -- rank -1,
+    // distance and fitness NaN, order -1, decision vectors all-ones bytes (NaN as floats)
+    const int64_t threads = (int64_t)gridDim.x * blockDim.x, t0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (int64_t p = t0; p < topk; p += threads) {
+      out_rank[p] = -1;
+      out_dist[p] = __uint_as_float(0x7FC00000u);
+      if (out_order) out_order[p] = -1;
+    }
+    for (int64_t e = t0; e < (int64_t)topk * m; e += threads) out_f[e] = __uint_as_float(0x7FC00000u);
+    if (x)
+      for (int64_t b = t0; b < (int64_t)topk * x_row_bytes; b += threads) out_x[b] = 0xFF;
+    return;
+  }
   // A row is copied by g lanes, g = the smallest power of two (4 .. 64) that holds the row's units and its m
   // fitness values: short rows share a wave (a row of 400 bytes in 16-byte units took 25 of 64 lanes).
   const int64_t units = (x ? x_row_bytes : 0) / unit;
@@ -150,6 +164,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const int* __restrict__ ord
     if (lane == 0) {
       out_rank[p] = rank[src];
       out_dist[p] = dist[src];
+      if (out_order) out_order[p] = (int)src;
     }
   }
 }

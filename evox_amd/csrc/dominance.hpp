@@ -546,9 +546,12 @@ __global__ __launch_bounds__(256) void first_front_kernel(const float* __restric
                                                           const uint32_t* __restrict__ kid, const int* __restrict__ orig_of,
                                                           int n, int npad, uint8_t* __restrict__ mask,
                                                           const Ctrl* __restrict__ ctrl, const SortParam* __restrict__ param) {
-  if (ctrl->err != 0) return;  // the slot sort failed: nothing is valid
   const int lane = threadIdx.x & 63;
   const int j = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 64 + lane;
+  if (ctrl->err != 0) {  // the slot sort failed, nothing is valid: no row is reported (the status carries the error)
+    if (j < n) mask[j] = 0;
+    return;
+  }
   if (j - lane >= n) return;  // npad is a multiple of 128: every row touched below exists
   float xj[M];
 #pragma unroll
@@ -577,9 +580,12 @@ __global__ __launch_bounds__(256) void first_front_kernel(const float* __restric
 __global__ __launch_bounds__(256) void first_front_any_m_kernel(const float* __restrict__ xs, const uint32_t* __restrict__ kid,
                                                                 const int* __restrict__ orig_of, int n, int npad, int m,
                                                                 uint8_t* __restrict__ mask, const Ctrl* __restrict__ ctrl) {
-  if (ctrl->err != 0) return;
   const int lane = threadIdx.x & 63;
   const int j = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 64 + lane;
+  if (ctrl->err != 0) {
+    if (j < n) mask[j] = 0;
+    return;
+  }
   if (j - lane >= n) return;
   const uint32_t idj = kid[j];
   bool dominated = j >= n;

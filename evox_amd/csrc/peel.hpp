@@ -53,6 +53,17 @@ __global__ __launch_bounds__(256) void reset_state_kernel(uint32_t* __restrict__
     words[i] = 0u;
 }
 
+// dst[i] = src[i] (4-byte elements), or `poison` everywhere when a device-side wait of the call ran out: the last
+// kernel of an entry point, so that a caller who never reads the status still cannot take a partial result for a
+// result (ranks -1, distances NaN, orders -1).  src == nullptr only poisons.
+__global__ __launch_bounds__(256) void copy_or_poison_kernel(const Ctrl* __restrict__ ctrl, const uint32_t* __restrict__ src,
+                                                             uint32_t* __restrict__ dst, int64_t n, uint32_t poison) {
+  const bool failed = ctrl->err != 0;
+  if (!failed && src == nullptr) return;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = failed ? poison : src[i];
+}
+
 // Words of row j that can hold a dominator (slots below j), rounded up to a whole 16-byte pair.
 __device__ inline int row_words(int j) { return ((j >> 6) + 2) & ~1; }
 

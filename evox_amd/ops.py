@@ -112,6 +112,8 @@ torch.library.register_vmap(nd_rank, _nd_rank_vmap)
 
 
 RANK_UNSET = 0x7FFFFFFF
+_SMALL_ARGSORT_ROWS = 8192  # longest one-dimensional sort that takes the counting kernel (no device-side waits)
+_ROWS_ARGSORT_MAX = 16384  # longest sort of a batch that runs inside one workgroup
 
 
 @torch.library.custom_op("evox_amd::nd_rank_until", mutates_args=())
@@ -425,7 +427,11 @@ def stable_argsort_step(key: torch.Tensor, kind: int, prev: Optional[torch.Tenso
         stream = runtime.stream_handle(key.device)
         _lib.call("evox_hip_stable_argsort_step", key.data_ptr(), kind, key.stride(0), n,
                   None if prev is None else prev.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
-        runtime.note_call(ws, stream)
+        # only the radix sort of long keys waits on the device and keeps a control block
+        if n > _SMALL_ARGSORT_ROWS:
+            runtime.note_call(ws, stream)
+        else:
+            runtime.note_small_kernel_call()
     return out
 
 
@@ -460,7 +466,10 @@ def stable_argsort_rows(key: torch.Tensor, kind: int, prev: Optional[torch.Tenso
         stream = runtime.stream_handle(key.device)
         _lib.call("evox_hip_stable_argsort_step_batched", key.data_ptr(), kind, key.stride(0), key.stride(1), batch, n,
                   None if prev is None else prev.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
-        runtime.note_call(ws, stream)
+        if n > (_ROWS_ARGSORT_MAX if batch >= 2 else _SMALL_ARGSORT_ROWS):
+            runtime.note_call(ws, stream)
+        else:
+            runtime.note_small_kernel_call()
     return out
 
 

@@ -27,7 +27,9 @@ extern "C" {
 
 #define EVOX_HIP_E_BAD_ARG (-1)         /* null pointer, n < 1, m < 1, topk outside [1, n], ... */
 #define EVOX_HIP_E_WORKSPACE (-2)       /* workspace too small or misaligned */
-#define EVOX_HIP_E_BARRIER_TIMEOUT (-3) /* reported by evox_hip_read_status(): a bounded device-side wait ran out */
+#define EVOX_HIP_E_BARRIER_TIMEOUT (-3) /* reported by evox_hip_read_status(): a bounded device-side wait ran out; the call's
+                                           outputs then hold no partial result: ranks and orders -1, distances and fitness NaN,
+                                           decision vectors all-ones bytes, first-front masks 0 */
 #define EVOX_HIP_E_STATIC_LIMIT (-4)    /* the population needs more scratch than the library's own buffer holds */
 
 int evox_hip_abi_version(void);

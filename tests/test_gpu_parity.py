@@ -825,20 +825,43 @@ def test_barrier_timeout_is_reported_not_hung():
     """A spin limit of one poll makes the bounded device-side wait give up: the kernel must end and
     the status must carry the error."""
     say("barrier_timeout")
-    f = workloads.uniform_population(3000, 3, 0, 5)[0].to(DEV)
-    runtime.set_option("spin_limit", 1)
-    try:
-        got_error = False
+    f, x = workloads.uniform_population(3000, 3, 4, 5)
+    f, x = f.to(DEV), x.to(DEV)
+    want = as_np(er.ranks_by_peeling(f.cpu()))
+
+    def failed():
         try:
-            non_dominate_rank(f)
             runtime.last_status()
         except _lib.EvoxHipError as e:
-            got_error = e.code == _lib.E_BARRIER_TIMEOUT
+            assert e.code == _lib.E_BARRIER_TIMEOUT
+            return True
+        return False
+
+    runtime.set_option("spin_limit", 1)
+    try:
+        # with one poll a wait may still succeed when the other blocks are already there: either the result is
+        # right and the status clean, or the status carries the error and NO partial result is handed out --
+        # every rank -1, every distance NaN, the rows all-ones bytes
+        rank = non_dominate_rank(f)
+        if failed():
+            say("barrier_timeout: the ranking gave up")
+            assert (as_np(rank) == -1).all()
+        else:
+            assert np.array_equal(as_np(rank), want)
+        xs, fs, rs, ds = nd_environmental_selection(x, f, 1500)
+        if failed():
+            say("barrier_timeout: the selection gave up")
+            assert (as_np(rs) == -1).all() and np.isnan(as_np(ds)).all() and np.isnan(as_np(fs)).all()
+            assert np.isnan(as_np(xs)).all()
+        else:
+            assert np.array_equal(as_np(rs), np.sort(want)[:1500])
+        dist = crowding_distance(f, None)
+        if failed():
+            assert np.isnan(as_np(dist)).all()
     finally:
         runtime.set_option("spin_limit", 4000000)
-    # with one poll the wait may still succeed when the other blocks are already there
-    assert got_error or np.array_equal(as_np(non_dominate_rank(f)), as_np(er.ranks_by_peeling(f.cpu())))
-    assert np.array_equal(as_np(non_dominate_rank(f)), as_np(er.ranks_by_peeling(f.cpu())))
+    assert np.array_equal(as_np(non_dominate_rank(f)), want)
+    assert not failed()
 
 
 def test_fronts_of_thousands_of_rows(peel_algorithm):
