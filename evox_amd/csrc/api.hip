@@ -33,6 +33,7 @@ struct Options {
   int peel_records = 1;  // record protocol (all-to-all, no master) for populations up to kRecordsMaxRowsWide
   int peel_lds = 1;      // populations whose lower triangle fits the LDS of the device are peeled from LDS (peel_lds.hpp)
   int peel_lds_blocks = 0;  // sweeping workgroups of that kernel, 0 = by size
+  int peel_tail = 1;        // that kernel also orders a small last front (0: always the kernels of finish.hpp)
   unsigned spin_limit = 4000000u;
   int dominance_tile_words = 4;
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
@@ -51,7 +52,7 @@ struct Layout {
   int64_t wstride;
   // byte offsets
   size_t ctrl, fsize, fronts_slot, fronts_orig, hist, zero_end, fstart, xs, key, partials, sortparam, bstart, bcursor,
-      scanflags, records, members, member_key, slot_of, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, total0, witness0, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
+      scanflags, tailbuf, records, members, member_key, slot_of, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, total0, witness0, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
 };
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
@@ -80,6 +81,7 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->fronts_orig = o; o = align_up(o + sizeof(uint64_t) * kFrontBuffers * kFrontStride * (size_t)L->nwords);
   L->hist = o;        o = align_up(o + sizeof(int) * (size_t)buckets);
   L->scanflags = o;   o = align_up(o + sizeof(unsigned long long) * 64);
+  L->tailbuf = o;     o = align_up(o + (n <= 32768 ? sizeof(unsigned long long) * kTailRows : 0));
   L->records = o;     o = align_up(o + (n <= 32768 ? sizeof(unsigned long long) * kLdsPeelRecordUnits : (n <= kRecordsMaxRowsWide ? sizeof(unsigned long long) * kRecRing * kRecUnits : 0)));
   L->zero_end = o;
   L->fstart = o;     o = align_up(o + sizeof(int) * (size_t)(n + 2));
@@ -381,9 +383,26 @@ static int lds_peel_plan(const Layout& L, size_t* lds_out) {
   return sweepers;
 }
 
-static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool fill_dist, int sweepers, size_t lds, hipStream_t s) {
+static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool fill_dist, int sweepers, size_t lds, hipStream_t s,
+                           bool order_last_front = false) {
   const Layout& L = w.L;
   if (stop_count < 1 || stop_count > L.n) return kErrBadArg;
+  PeelTail tail;
+  tail.mode = 0;
+  tail.m = L.m;
+  tail.npad = L.npad;
+  tail.xs_sorted = w.at<float>(L.xs_sorted);
+  tail.dist = w.at<float>(L.dist);
+  tail.order = w.at<int>(L.order);
+  tail.buffer = w.at<unsigned long long>(L.tailbuf);
+  if (order_last_front && g_opt.peel_tail) {
+    // a small last front is ordered by the peel kernel itself; its LDS must hold the candidates
+    const size_t need = peel_tail_lds_bytes(L.n, L.m);
+    if (need != 0 && need <= kLdsPeelBudget) {
+      tail.mode = 2;
+      if (lds < need) lds = need;
+    }
+  }
   // the attribute belongs to the (kernel, device) pair; every workgroup waits for every other one, so the grid
   // must be resident at once: checked once per device for the largest LDS size
   static int resident[64] = {0};  // 0 unknown, else workgroups per compute unit + 1
@@ -403,7 +422,7 @@ static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool
                      w.at<int>(L.orig_of), w.at<int>(L.rank), fill_dist ? w.at<float>(L.dist) : (float*)nullptr,
                      w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
                      want_perm ? w.at<int>(L.perm) : (int*)nullptr, w.at<int>(L.fstart), w.ctrl(), (int)stop_count, g_opt.spin_limit,
-                     w.at<unsigned long long>(L.records), sweepers);
+                     w.at<unsigned long long>(L.records), sweepers, tail);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -412,9 +431,11 @@ static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool
 // pass over the matrix followed by a peel kernel that rescans rows in memory.
 static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s);
 static int stage_count(const Ws& w, bool fill_dist, hipStream_t s);
-static int count_and_peel(const Ws& w, int64_t stop_count, bool want_perm, bool fill_dist, hipStream_t s) {
+static int count_and_peel(const Ws& w, int64_t stop_count, bool want_perm, bool fill_dist, hipStream_t s,
+                          bool order_last_front = false) {
   size_t lds = 0;
-  if (const int sweepers = lds_peel_plan(w.L, &lds)) return launch_lds_peel(w, stop_count, want_perm, fill_dist, sweepers, lds, s);
+  if (const int sweepers = lds_peel_plan(w.L, &lds))
+    return launch_lds_peel(w, stop_count, want_perm, fill_dist, sweepers, lds, s, order_last_front);
   if (int e = stage_count(w, fill_dist, s)) return e;
   return stage_peel(w, stop_count, want_perm, s);
 }
@@ -614,12 +635,34 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) 
 }
 
 // Per-objective ordering of the candidates list[ctrl.worst_start ... + ctrl.nv).
-static int stage_crowd_sort(const Ws& w, const int* list, bool use_orders, hipStream_t s) {
+// fused: 0 = the two kernels as stages of their own; 1 / 2 = a small front gets its distances (2: and the selection
+// order) inside crowd_sort_kernel, and crowd_finish_kernel, given the same value, leaves it alone.
+static CrowdArgs crowd_args(const Ws& w, const int* list, bool use_orders, int fused) {
   const Layout& L = w.L;
-  use_orders = use_orders && prefix_dominance_applies(L);
-  if (use_orders) {
-    // a large front of a population whose matrix came from the per-objective orders: its own orders are read off
-    // those (finish.hpp); the three kernels and the one below choose on the device which of them has work
+  CrowdArgs a;
+  a.xs = w.at<float>(L.xs);
+  a.npad = L.npad;
+  a.list_base = list;
+  a.ctrl = w.ctrl();
+  a.m = L.m;
+  a.kstride = L.kstride;
+  a.pos = w.at<int>(L.pos);
+  a.sorted_cost = w.at<float>(L.scost);
+  a.buf = radix_buffers(w);
+  a.spin_limit = g_opt.spin_limit;
+  a.param = w.at<SortParam>(L.sortparam);
+  a.use_orders = use_orders ? 1 : 0;
+  a.fused = fused;
+  a.dist = w.at<float>(L.dist);
+  a.dkey = w.at<uint32_t>(L.dkey);
+  a.order = w.at<int>(L.order);
+  return a;
+}
+
+// The three launches that read the orders of a large last front off the orders of the whole population.
+static int stage_front_orders(const Ws& w, const int* list, hipStream_t s) {
+  const Layout& L = w.L;
+  {
     const RadixBuffers b = radix_buffers(w);
     const int spans = (L.n + kFrontOrderSpan - 1) / kFrontOrderSpan;
     int* const number = reinterpret_cast<int*>(w.at<uint32_t>(L.dkey));  // free until the distances are known
@@ -635,24 +678,42 @@ static int stage_crowd_sort(const Ws& w, const int* list, bool use_orders, hipSt
                        w.at<int>(L.pos), w.at<float>(L.scost));
     EVX_LAUNCH_CHECK();
   }
-  size_t lds = sizeof(uint64_t) * kRankTile;
+  return 0;
+}
+
+static size_t crowd_lds_bytes(const Layout& L, int fused) {
+  size_t lds = sizeof(uint32_t) * kRadixMinCandidates + sizeof(uint64_t) * kRankTile;
   if (L.n > kRadixMinCandidates && kRadixLdsBytes > lds) lds = kRadixLdsBytes;
+  if (fused != 0 && kFusedFrontLdsBytes > lds) lds = kFusedFrontLdsBytes;
+  return lds;
+}
+
+static int stage_crowd_sort(const Ws& w, const int* list, bool use_orders, int fused, hipStream_t s) {
+  const Layout& L = w.L;
+  use_orders = use_orders && prefix_dominance_applies(L);
+  // a large front of a population whose matrix came from the per-objective orders: its own orders are read off
+  // those (finish.hpp); the three kernels and the one below choose on the device which of them has work
+  if (use_orders)
+    if (int e = stage_front_orders(w, list, s)) return e;
+  const size_t lds = crowd_lds_bytes(L, fused);
   if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(crowd_sort_kernel), lds)) return e;
-  hipLaunchKernelGGL(crowd_sort_kernel, dim3(finish_grid(L, L.m)), dim3(kRadixThreads), lds, s, w.at<float>(L.xs), L.npad, list,
-                     w.ctrl(), L.m, L.kstride, w.at<int>(L.pos), w.at<float>(L.scost), radix_buffers(w), g_opt.spin_limit,
-                     w.at<SortParam>(L.sortparam), use_orders ? 1 : 0);
+  // (the fused path ends with a barrier between all blocks: the grid must be resident at once, which a grid of at
+  // most two blocks of 256 threads per compute unit is)
+  int grid = finish_grid(L, L.m);
+  if (fused != 0 && grid > device_cus() * 2) grid = device_cus() * 2;
+  hipLaunchKernelGGL(crowd_sort_kernel, dim3(grid), dim3(kRadixThreads), lds, s, crowd_args(w, list, use_orders, fused));
   EVX_LAUNCH_CHECK();
   return 0;
 }
 
 // Crowding distances of those candidates and, with want_order, the selection order.
-static int stage_crowd_finish(const Ws& w, const int* list, bool want_order, hipStream_t s) {
+static int stage_crowd_finish(const Ws& w, const int* list, bool want_order, int fused, hipStream_t s) {
   const Layout& L = w.L;
-  size_t lds = sizeof(uint32_t) * kRadixMinCandidates + sizeof(uint64_t) * kRankTile;
-  if (L.n > kRadixMinCandidates && kRadixLdsBytes > lds) lds = kRadixLdsBytes;
-  hipLaunchKernelGGL(crowd_finish_kernel, dim3(finish_grid(L, 1)), dim3(kRadixThreads), lds, s, list, w.ctrl(), L.m,
-                     w.at<int>(L.pos), w.at<float>(L.scost), L.kstride, w.at<float>(L.dist), w.at<uint32_t>(L.dkey),
-                     w.at<int>(L.order), radix_buffers(w), g_opt.spin_limit, want_order ? 1 : 0, w.at<SortParam>(L.sortparam));
+  // (no front of this population is too large for the fused path of crowd_sort_kernel: nothing is left to do)
+  if (fused != 0 && L.n <= kFusedFrontRows && (int64_t)L.n * L.m <= kFusedFrontValues && L.m <= kFusedFrontObjectives) return 0;
+  const size_t lds = crowd_lds_bytes(L, 0);
+  hipLaunchKernelGGL(crowd_finish_kernel, dim3(finish_grid(L, 1)), dim3(kRadixThreads), lds, s, crowd_args(w, list, false, fused),
+                     want_order ? 1 : 0);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -766,6 +827,8 @@ int evox_hip_set_option(const char* name, int64_t value) {
     g_opt.peel_records = (int)value;
   } else if (!strcmp(name, "peel_lds") && (value == 0 || value == 1)) {
     g_opt.peel_lds = (int)value;
+  } else if (!strcmp(name, "peel_tail") && (value == 0 || value == 1)) {
+    g_opt.peel_tail = (int)value;
   } else if (!strcmp(name, "peel_lds_blocks") && (value == 0 || (value >= 8 && value <= 255))) {
     g_opt.peel_lds_blocks = (int)value;
   } else if (!strcmp(name, "spin_limit") && value >= 1 && value <= 0x7FFFFFFFll) {
@@ -831,14 +894,14 @@ int evox_hip_stage_peel(int64_t n, int64_t m, int64_t stop_count, int32_t* rank_
 int evox_hip_stage_crowding(int64_t n, int64_t m, void* ws, size_t ws_bytes, void* stream) {
   Ws w;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
-  if (int e = stage_crowd_sort(w, w.at<int>(w.L.perm), true, (hipStream_t)stream)) return e;
-  return stage_crowd_finish(w, w.at<int>(w.L.perm), false, (hipStream_t)stream);
+  if (int e = stage_crowd_sort(w, w.at<int>(w.L.perm), true, 0, (hipStream_t)stream)) return e;
+  return stage_crowd_finish(w, w.at<int>(w.L.perm), false, 0, (hipStream_t)stream);
 }
 
 int evox_hip_stage_order(int64_t n, int64_t m, void* ws, size_t ws_bytes, void* stream) {
   Ws w;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
-  return stage_crowd_finish(w, w.at<int>(w.L.perm), true, (hipStream_t)stream);
+  return stage_crowd_finish(w, w.at<int>(w.L.perm), true, 0, (hipStream_t)stream);
 }
 
 int evox_hip_non_dominate_rank_until(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, int64_t stop_count,
@@ -907,8 +970,8 @@ int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t
   hipLaunchKernelGGL(compact_mask_kernel, dim3(1), dim3(1024), 0, s, mask, mask_stride, L.n, w.at<int>(L.perm),
                      w.at<float>(L.dist), w.ctrl());
   EVX_LAUNCH_CHECK();
-  if (int e = stage_crowd_sort(w, w.at<int>(L.perm), false, s)) return e;
-  if (int e = stage_crowd_finish(w, w.at<int>(L.perm), false, s)) return e;
+  if (int e = stage_crowd_sort(w, w.at<int>(L.perm), false, 1, s)) return e;
+  if (int e = stage_crowd_finish(w, w.at<int>(L.perm), false, 1, s)) return e;
   return copy_out(w.ctrl(), dist_out, w.at<float>(L.dist), n, kPoisonFloat, s);
 }
 
@@ -1061,22 +1124,53 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   const Layout& L = w.L;
   if (int e = stage_prepare(w, fit, true, s)) return e;
   if (int e = stage_dominance(w, kDomAuto, s)) return e;
-  if (int e = count_and_peel(w, topk, true, true, s)) return e;
-  if (int e = stage_crowd_sort(w, w.at<int>(L.perm), true, s)) return e;
-  if (int e = stage_crowd_finish(w, w.at<int>(L.perm), true, s)) return e;
+  if (int e = count_and_peel(w, topk, true, true, s, true)) return e;
   int unit = 1;
   if (x != nullptr) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(x2) | reinterpret_cast<uintptr_t>(out_x) |
                            (uintptr_t)x_row_bytes | (uintptr_t)x_row_stride_bytes | (uintptr_t)x2_row_stride_bytes;
     unit = (bits % 16 == 0) ? 16 : (bits % 4 == 0) ? 4 : 1;
   }
-  int blocks = (int)((topk + 3) / 4);
-  const int cap = device_cus() * 8;
-  if (blocks > cap) blocks = cap;
-  hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(256), 0, s, w.at<int>(L.order), (int)topk,
-                     static_cast<const uint8_t*>(x), x_row_stride_bytes, x_row_bytes, static_cast<uint8_t*>(out_x), unit, fit.f,
-                     fit.sr, fit.sc, (int)fit.n_first, static_cast<const uint8_t*>(x2), x2_row_stride_bytes, fit.f2, fit.sr2,
-                     fit.sc2, L.m, out_f, w.at<int>(L.rank), out_rank, w.at<float>(L.dist), out_dist, out_order, w.ctrl());
+  GatherArgs g;
+  g.order = w.at<int>(L.order);
+  g.listed = w.at<int>(L.perm);
+  g.topk = (int)topk;
+  g.x = static_cast<const uint8_t*>(x);
+  g.x_row_stride = x_row_stride_bytes;
+  g.x_row_bytes = x_row_bytes;
+  g.out_x = static_cast<uint8_t*>(out_x);
+  g.unit = unit;
+  g.f = fit.f;
+  g.f_stride_row = fit.sr;
+  g.f_stride_col = fit.sc;
+  g.n_first = (int)fit.n_first;
+  g.x2 = static_cast<const uint8_t*>(x2);
+  g.x2_row_stride = x2_row_stride_bytes;
+  g.f2 = fit.f2;
+  g.f2_stride_row = fit.sr2;
+  g.f2_stride_col = fit.sc2;
+  g.m = L.m;
+  g.out_f = out_f;
+  g.rank = w.at<int>(L.rank);
+  g.out_rank = out_rank;
+  g.dist = w.at<float>(L.dist);
+  g.out_dist = out_dist;
+  g.out_order = out_order;
+  g.ctrl = w.ctrl();
+  // the ordering of the last front (where the peel kernel has not left it) and the gather, in one launch
+  const bool use_orders = prefix_dominance_applies(L);
+  if (use_orders)
+    if (int e = stage_front_orders(w, w.at<int>(L.perm), s)) return e;
+  const size_t lds = crowd_lds_bytes(L, 2);
+  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(tail_kernel), lds)) return e;
+  // the radix grid (all blocks resident: they wait for one another), widened to what the gather can use
+  int grid = finish_grid(L, L.m);
+  const int wide = (int)((topk + 15) / 16);
+  if (grid < wide) grid = wide;
+  int most = device_cus() * 2;
+  if (most > kRadixMaxWorkers + kFirstSweeper) most = kRadixMaxWorkers + kFirstSweeper;
+  if (grid > most) grid = most;
+  hipLaunchKernelGGL(tail_kernel, dim3(grid), dim3(kRadixThreads), lds, s, crowd_args(w, w.at<int>(L.perm), use_orders, 2), g);
   EVX_LAUNCH_CHECK();
   return 0;
 }

@@ -38,7 +38,8 @@ struct Ctrl {
   int passes;       // sweep passes executed
   int listed;       // front bitmaps 0 .. listed-1 have been listed and cleared; polled by the barrier master
   int radix_epoch;  // runs of a radix sort kernel so far: each takes a fresh range of barrier generations
-  int reserved[7];
+  int tail_done;    // the peel kernel has also left the crowding distances and the order of the last front
+  int reserved[6];  // [0], [1]: arrival counters of the barriers inside the kernels that order the last front
   // grid barrier: block 0 publishes (generation << 32 | rows found by all blocks) in `release` and in
   // kReleaseCopies copies of it, one per 128-byte line, so that the waiting blocks do not all poll one
   // address; all-ones means "give up" (a bounded wait ran out).  Every other block publishes

@@ -109,20 +109,47 @@ __device__ inline float crowding_distance_of(int q, int nv, int m, const int* __
 // out[p, :] = src[order[p], :] for the decision vectors (raw bytes, any dtype), the fitness, the rank
 // and the distance.  Rows from n_first on are read from the second part (x2, f2) of a two-part population.
 // Rows are copied in 16-, 4- or 1-byte units, a row by 4 to 64 lanes of a wave.
-__global__ __launch_bounds__(256) void gather_kernel(const int* __restrict__ order, int topk, const uint8_t* __restrict__ x,
-                                                     int64_t x_row_stride, int64_t x_row_bytes, uint8_t* __restrict__ out_x,
-                                                     int unit, const float* __restrict__ f, int64_t f_stride_row,
-                                                     int64_t f_stride_col, int n_first, const uint8_t* __restrict__ x2,
-                                                     int64_t x2_row_stride, const float* __restrict__ f2,
-                                                     int64_t f2_stride_row, int64_t f2_stride_col, int m,
-                                                     float* __restrict__ out_f, const int* __restrict__ rank,
-                                                     int* __restrict__ out_rank, const float* __restrict__ dist,
-                                                     float* __restrict__ out_dist, int* __restrict__ out_order,
-                                                     const Ctrl* __restrict__ ctrl) {
-  if (ctrl->err != 0) {
+struct GatherArgs {
+  const int* order;  // selected rows from position `listed_until` on ...
+  const int* listed;  // ... and before it (the rows of the better fronts as the peel listed them) when listed_until > 0
+  int topk;
+  const uint8_t* x;
+  int64_t x_row_stride, x_row_bytes;
+  uint8_t* out_x;
+  int unit;
+  const float* f;
+  int64_t f_stride_row, f_stride_col;
+  int n_first;
+  const uint8_t* x2;
+  int64_t x2_row_stride;
+  const float* f2;
+  int64_t f2_stride_row, f2_stride_col;
+  int m;
+  float* out_f;
+  const int* rank;
+  int* out_rank;
+  const float* dist;
+  float* out_dist;
+  int* out_order;
+  const Ctrl* ctrl;
+};
+
+// Called by every thread of `blocks` blocks of 256 threads (`block` = the caller's index among them).
+// listed_until: positions below it take their row from a.listed instead of a.order.
+__device__ inline void gather_body(const GatherArgs& a, int block, int blocks, int listed_until) {
+  const int topk = a.topk, m = a.m, unit = a.unit, n_first = a.n_first;
+  const uint8_t* __restrict__ x = a.x;
+  const uint8_t* __restrict__ x2 = a.x2;
+  uint8_t* __restrict__ out_x = a.out_x;
+  const int64_t x_row_bytes = a.x_row_bytes;
+  float* __restrict__ out_f = a.out_f;
+  int* __restrict__ out_rank = a.out_rank;
+  float* __restrict__ out_dist = a.out_dist;
+  int* __restrict__ out_order = a.out_order;
+  if (a.ctrl->err != 0) {
     // a device-side wait ran out and `order` was not produced: no partial result leaves the call -- rank -1,
     // distance and fitness NaN, order -1, decision vectors all-ones bytes (NaN as floats)
-    const int64_t threads = (int64_t)gridDim.x * blockDim.x, t0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t threads = (int64_t)blocks * blockDim.x, t0 = (int64_t)block * blockDim.x + threadIdx.x;
     for (int64_t p = t0; p < topk; p += threads) {
       out_rank[p] = -1;
       out_dist[p] = __uint_as_float(0x7FC00000u);
@@ -140,13 +167,13 @@ __global__ __launch_bounds__(256) void gather_kernel(const int* __restrict__ ord
   while (g > 4 && (g >> 1) >= units && (g >> 1) >= m) g >>= 1;
   const int per_wave = 64 / g;
   const int lane = (threadIdx.x & 63) % g, sub = (threadIdx.x & 63) / g;
-  const int64_t waves = (int64_t)gridDim.x * (blockDim.x >> 6);
-  for (int64_t p = ((int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * per_wave + sub; p < topk;
+  const int64_t waves = (int64_t)blocks * (blockDim.x >> 6);
+  for (int64_t p = ((int64_t)block * (blockDim.x >> 6) + (threadIdx.x >> 6)) * per_wave + sub; p < topk;
        p += waves * per_wave) {
-    const int64_t src = order[p];
+    const int64_t src = p < listed_until ? a.listed[p] : a.order[p];
     const bool second = src >= n_first;  // rows of the second part of a two-part population
     if (x) {
-      const uint8_t* __restrict__ s = second ? x2 + (src - n_first) * x2_row_stride : x + src * x_row_stride;
+      const uint8_t* __restrict__ s = second ? x2 + (src - n_first) * a.x2_row_stride : x + src * a.x_row_stride;
       uint8_t* __restrict__ d = out_x + p * x_row_bytes;
       if (unit == 16) {
         for (int64_t b = lane * 16; b < x_row_bytes; b += g * 16)
@@ -159,11 +186,11 @@ __global__ __launch_bounds__(256) void gather_kernel(const int* __restrict__ ord
       }
     }
     for (int k = lane; k < m; k += g)
-      out_f[p * m + k] =
-          second ? f2[(src - n_first) * f2_stride_row + k * f2_stride_col] : f[src * f_stride_row + k * f_stride_col];
+      out_f[p * m + k] = second ? a.f2[(src - n_first) * a.f2_stride_row + k * a.f2_stride_col]
+                                : a.f[src * a.f_stride_row + k * a.f_stride_col];
     if (lane == 0) {
-      out_rank[p] = rank[src];
-      out_dist[p] = dist[src];
+      out_rank[p] = a.rank[src];
+      out_dist[p] = a.dist[src];
       if (out_order) out_order[p] = (int)src;
     }
   }

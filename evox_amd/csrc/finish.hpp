@@ -19,21 +19,174 @@
 
 namespace evx {
 
+// ---- A small last front in one launch.  With a few hundred candidates the two kernels below cost two launches and
+// three chains of dependent loads (positions, sorted costs, distance keys) for a few microseconds of work.  Here the
+// candidates' (key, candidate) composites and costs of every objective sit in LDS of every workgroup, a candidate is
+// taken by sixteen lanes that scan all candidates once per objective for its two neighbours in the objective's order
+// (the largest composite below its own, the smallest above: no positions, no sorted array), and the order of the
+// distances follows after one grid-wide counter barrier.  Same results as the two kernels: the neighbours of a
+// candidate in the stable order by (cost, row index), the span between the first and the last cost, terms added in
+// column order.
+constexpr int kFusedFrontRows = 2048;
+constexpr int kFusedFrontValues = 4096;  // candidates x objectives held in LDS: 12 bytes each
+constexpr int kFusedFrontObjectives = 64;
+constexpr size_t kFusedFrontLdsBytes = 12 * (size_t)kFusedFrontValues + 4 * (size_t)kFusedFrontRows + 16 * kFusedFrontObjectives;
+
+__device__ inline bool fused_front_applies(int nv, int m) {
+  return nv <= kFusedFrontRows && (int64_t)nv * m <= kFusedFrontValues && m <= kFusedFrontObjectives;
+}
+
+// mode 1: distances only; mode 2: distances and the selection order.  Called by every thread of every block;
+// blockDim.x == kRadixThreads.  lds: kFusedFrontLdsBytes.
+__device__ inline void crowd_small_front(const float* __restrict__ xs, int npad, const int* __restrict__ list_base,
+                                         Ctrl* __restrict__ ctrl, int m, float* __restrict__ dist, uint32_t* __restrict__ dkey,
+                                         int* __restrict__ order, unsigned spin_limit, int mode, uint64_t* lds, int* scratch) {
+  const int nv = ctrl->nv, start = ctrl->worst_start, need = ctrl->need;
+  const int* __restrict__ list = list_base + start;
+  const int tid = threadIdx.x, sub = tid & 15;
+  unsigned long long* comp = reinterpret_cast<unsigned long long*>(lds);  // [m][nv]
+  float* cost = reinterpret_cast<float*>(comp + kFusedFrontValues);  // [m][nv]
+  int* lst = reinterpret_cast<int*>(cost + kFusedFrontValues);       // [nv]
+  unsigned long long* ends = reinterpret_cast<unsigned long long*>(lst + kFusedFrontRows);  // [m][2]: first, last composite
+  for (int e = tid; e < nv; e += blockDim.x) lst[e] = list[e];
+  if (mode == 2)  // the better fronts keep the order in which they are listed
+    for (int i = blockIdx.x * blockDim.x + tid; i < start; i += gridDim.x * blockDim.x) order[i] = list_base[i];
+  __syncthreads();
+  for (int i = tid; i < nv * m; i += blockDim.x) {
+    const int k = i / nv, e = i - k * nv;
+    const float c = xs[(int64_t)k * npad + lst[e]];
+    cost[i] = c;
+    comp[i] = ((unsigned long long)ordered_key(c) << 32) | (unsigned)e;
+  }
+  __syncthreads();
+  // first and last composite of every objective: a wave per objective
+  for (int k = tid >> 6; k < m; k += blockDim.x >> 6) {
+    unsigned long long lo = ~0ull, hi = 0ull;
+    for (int e = tid & 63; e < nv; e += 64) {
+      const unsigned long long c = comp[k * nv + e];
+      lo = c < lo ? c : lo;
+      hi = c > hi ? c : hi;
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned long long a = ((unsigned long long)__shfl_xor((unsigned)(lo >> 32), off) << 32) | __shfl_xor((unsigned)lo, off);
+      const unsigned long long b = ((unsigned long long)__shfl_xor((unsigned)(hi >> 32), off) << 32) | __shfl_xor((unsigned)hi, off);
+      lo = a < lo ? a : lo;
+      hi = b > hi ? b : hi;
+    }
+    if ((tid & 63) == 0) {
+      ends[2 * k] = lo;
+      ends[2 * k + 1] = hi;
+    }
+  }
+  __syncthreads();
+  const int groups = gridDim.x * (blockDim.x >> 4);
+  for (int q = blockIdx.x * (blockDim.x >> 4) + (tid >> 4); q < nv; q += groups) {
+    bool boundary = false;
+    float acc = 0.0f;
+    for (int k = 0; k < m; ++k) {
+      const unsigned long long* row = comp + k * nv;
+      const unsigned long long mine = row[q];
+      unsigned long long below = 0ull, above = ~0ull;  // no composite is zero or all ones
+      for (int e0 = sub; e0 < nv; e0 += 8 * 16) {  // eight partners per step, their LDS reads in flight together
+        unsigned long long c[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) c[u] = e0 + 16 * u < nv ? row[e0 + 16 * u] : mine;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (c[u] < mine) below = c[u] > below ? c[u] : below;
+          if (c[u] > mine) above = c[u] < above ? c[u] : above;
+        }
+      }
+      below = group16_max(below);
+      above = group16_min(above);
+      if (below == 0ull || above == ~0ull) {
+        boundary = true;  // first or last of this objective (non_dominate.py:226-227)
+      } else {
+        const float* ck = cost + k * nv;
+        const float span = ck[(int)(unsigned)ends[2 * k + 1]] - ck[(int)(unsigned)ends[2 * k]];
+        const float term = (ck[(int)(unsigned)above] - ck[(int)(unsigned)below]) / span;
+        acc = k == 0 ? term : acc + term;
+      }
+    }
+    if (sub == 0) {
+      const float d = boundary ? INFINITY : acc;
+      dist[lst[q]] = d;
+      if (mode == 2) coherent_store(&dkey[q], ordered_key(-d));
+    }
+  }
+  if (mode != 2) return;
+  // every block has stored its distance keys: one counter, bounded wait
+  __syncthreads();
+  if (tid == 0) {
+    __hip_atomic_fetch_add(&ctrl->reserved[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool seen = bounded_wait([&] { return coherent_load(&ctrl->reserved[0]) >= (int)gridDim.x || coherent_load(&ctrl->err) != 0; },
+                                   spin_limit);
+    if (!seen) coherent_store(&ctrl->err, kErrBarrierTimeout);
+    scratch[0] = seen && coherent_load(&ctrl->err) == 0;
+  }
+  __syncthreads();
+  if (scratch[0] == 0) return;
+  for (int e = tid; e < nv; e += blockDim.x) comp[e] = ((unsigned long long)coherent_load(&dkey[e]) << 32) | (unsigned)e;
+  __syncthreads();
+  for (int q = blockIdx.x * (blockDim.x >> 4) + (tid >> 4); q < nv; q += groups) {
+    const unsigned long long mine = comp[q];
+    int smaller = 0;
+    for (int e0 = sub; e0 < nv; e0 += 8 * 16) {
+      unsigned long long c[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) c[u] = e0 + 16 * u < nv ? comp[e0 + 16 * u] : ~0ull;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) smaller += c[u] < mine;
+    }
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) smaller += __shfl_xor(smaller, off);
+    if (sub == 0 && smaller < need) order[start + smaller] = lst[q];
+  }
+}
+
 // Per-objective sorted position of every candidate of the last front: pos[k][q], sorted_cost[k][pos].
 // Grid: the radix grid (master, idle block, workers; all resident) when the population can have a
 // front above kRadixMinCandidates rows, any grid otherwise.  Dynamic LDS: max(kRankTile * 8,
 // kRadixLdsBytes) bytes.
-__global__ __launch_bounds__(kRadixThreads) void crowd_sort_kernel(const float* __restrict__ xs, int npad,
-                                                                   const int* __restrict__ list_base, Ctrl* __restrict__ ctrl,
-                                                                   int m, int kstride, int* __restrict__ pos,
-                                                                   float* __restrict__ sorted_cost, RadixBuffers buf,
-                                                                   unsigned spin_limit, SortParam* __restrict__ param,
-                                                                   int use_orders) {
-  extern __shared__ uint64_t finish_lds[];
-  __shared__ int base[256];
-  __shared__ int scratch[kRadixThreads];
+struct CrowdArgs {
+  const float* xs;  // fitness, structure of arrays in original row order, columns npad apart
+  int npad;
+  const int* list_base;  // the rows ordered by (rank, row index) as far as peeled
+  Ctrl* ctrl;
+  int m, kstride;
+  int* pos;
+  float* sorted_cost;
+  RadixBuffers buf;
+  unsigned spin_limit;
+  SortParam* param;
+  int use_orders, fused;
+  float* dist;
+  uint32_t* dkey;
+  int* order;
+};
+
+// `epochs`: how many epochs of radix barrier generations the control block's counter moves on when the radix path
+// has run (1 when the kernel ends after this body; the merged tail kernel passes 0 and moves the counter itself).
+__device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int epochs, uint64_t* finish_lds, int* base, int* scratch) {
+  const float* __restrict__ xs = a.xs;
+  const int npad = a.npad, m = a.m, kstride = a.kstride, use_orders = a.use_orders, fused = a.fused;
+  const int* __restrict__ list_base = a.list_base;
+  Ctrl* __restrict__ ctrl = a.ctrl;
+  int* __restrict__ pos = a.pos;
+  float* __restrict__ sorted_cost = a.sorted_cost;
+  const RadixBuffers buf = a.buf;
+  const unsigned spin_limit = a.spin_limit;
+  SortParam* __restrict__ param = a.param;
+  float* __restrict__ dist = a.dist;
+  uint32_t* __restrict__ dkey = a.dkey;
+  int* __restrict__ order = a.order;
   if (coherent_load(&ctrl->err) != 0) return;
   const int nv = ctrl->nv;
+  if (fused != 0 && fused_front_applies(nv, m)) {  // a small front: distances (and order) right here
+    crowd_small_front(xs, npad, list_base, ctrl, m, dist, dkey, order, spin_limit, fused, finish_lds, scratch);
+    return;
+  }
   const int* __restrict__ list = list_base + ctrl->worst_start;
   // a large front of a population whose per-objective orders are at hand is ordered by front_order_*_kernel
   if (nv > kRadixMinCandidates && use_orders && param->orders_valid != 0) return;
@@ -56,12 +209,11 @@ __global__ __launch_bounds__(kRadixThreads) void crowd_sort_kernel(const float* 
     return;
   }
   // radix sort, one segment per objective (the host gave this launch the radix grid)
-  const unsigned gen0 = radix_generation_base(ctrl);
   if (blockIdx.x == 0) {
     radix_master(ctrl, gen0, 12, spin_limit, scratch);
     if (threadIdx.x == 0) {
-      ctrl->radix_epoch += 1;  // nobody reads it again in this kernel
-      param->orders_valid = 0;  // the sort has taken the buffer that held them (read at the start of this kernel only)
+      ctrl->radix_epoch += epochs;  // nobody reads it again in this kernel
+      param->orders_valid = 0;  // the sort has taken the buffer that held them (read at the start of this body only)
     }
     return;
   }
@@ -79,6 +231,13 @@ __global__ __launch_bounds__(kRadixThreads) void crowd_sort_kernel(const float* 
       pos[(int64_t)k * buf.kstride + q] = p;
       sorted_cost[(int64_t)k * buf.kstride + p] = xs[(int64_t)k * npad + list[q]];
     }
+}
+
+__global__ __launch_bounds__(kRadixThreads) void crowd_sort_kernel(CrowdArgs a) {
+  extern __shared__ uint64_t finish_lds[];
+  __shared__ int base[256];
+  __shared__ int scratch[kRadixThreads];
+  crowd_sort_body(a, radix_generation_base(a.ctrl), 1, finish_lds, base, scratch);
 }
 
 // ---- The same per-objective order of a large last front, taken from the orders of the whole population that
@@ -186,18 +345,22 @@ __global__ __launch_bounds__(256) void front_order_place_kernel(const unsigned l
 // that come first by (distance descending, NaN after every number, row index) -- jit_fix_operator.py:246-252
 // applied to non_dominate.py:253.  Same grid rule as crowd_sort_kernel.  Dynamic LDS:
 // kRadixMinCandidates * 4 + kRankTile * 8 bytes.
-__global__ __launch_bounds__(kRadixThreads) void crowd_finish_kernel(const int* __restrict__ list_base, Ctrl* __restrict__ ctrl,
-                                                                     int m, const int* __restrict__ pos,
-                                                                     const float* __restrict__ sorted_cost, int kstride,
-                                                                     float* __restrict__ dist, uint32_t* __restrict__ dkey,
-                                                                     int* __restrict__ order, RadixBuffers buf,
-                                                                     unsigned spin_limit, int want_order,
-                                                                     SortParam* __restrict__ param) {
-  extern __shared__ uint64_t finish_lds[];
-  __shared__ int base[256];
-  __shared__ int scratch[kRadixThreads];
+__device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, unsigned gen0, int epochs, uint64_t* finish_lds,
+                                         int* base, int* scratch) {
+  const int m = a.m, kstride = a.kstride, fused = a.fused;
+  const int* __restrict__ list_base = a.list_base;
+  Ctrl* __restrict__ ctrl = a.ctrl;
+  const int* __restrict__ pos = a.pos;
+  const float* __restrict__ sorted_cost = a.sorted_cost;
+  const RadixBuffers buf = a.buf;
+  const unsigned spin_limit = a.spin_limit;
+  SortParam* __restrict__ param = a.param;
+  float* __restrict__ dist = a.dist;
+  uint32_t* __restrict__ dkey = a.dkey;
+  int* __restrict__ order = a.order;
   if (coherent_load(&ctrl->err) != 0) return;
   const int nv = ctrl->nv;
+  if (fused != 0 && fused_front_applies(nv, m)) return;  // crowd_sort_kernel has done it all
   const int start = ctrl->worst_start;
   const int need = ctrl->need;
   const int* __restrict__ list = list_base + start;
@@ -225,12 +388,11 @@ __global__ __launch_bounds__(kRadixThreads) void crowd_finish_kernel(const int* 
     return;
   }
   // large front: distances by stripes, then (for the order) a grid barrier and the radix sort of their keys
-  const unsigned gen0 = radix_generation_base(ctrl);
   if (blockIdx.x == 0) {
     if (want_order) {
       radix_master(ctrl, gen0, 13, spin_limit, scratch);
       if (threadIdx.x == 0) {
-        ctrl->radix_epoch += 1;
+        ctrl->radix_epoch += epochs;
         param->orders_valid = 0;  // the sort of the distance keys has taken the buffer that held the orders
       }
     }
@@ -254,6 +416,62 @@ __global__ __launch_bounds__(kRadixThreads) void crowd_finish_kernel(const int* 
     const unsigned long long pr = coherent_load(&buf.pairs[0][p]);
     order[start + p] = list[(int)(unsigned)(pr & 0xFFFFFFFFull)];
   }
+}
+
+__global__ __launch_bounds__(kRadixThreads) void crowd_finish_kernel(CrowdArgs a, int want_order) {
+  extern __shared__ uint64_t finish_lds[];
+  __shared__ int base[256];
+  __shared__ int scratch[kRadixThreads];
+  crowd_finish_body(a, want_order, radix_generation_base(a.ctrl), 1, finish_lds, base, scratch);
+}
+
+// ---- Everything after the peeling in one launch: the ordering of the last front, unless the peel kernel has done
+// it already (Ctrl.tail_done: a small front is ordered by the workgroups that peeled it, while its rows are still
+// at hand), then the gather of the selected rows.  A launch that finds nothing to do still costs as much as a small
+// kernel (about 4.7 us on this device), so the stages that choose their algorithm on the device share one launch
+// instead of queueing one launch per algorithm.  Grid: the radix grid (master, idle block, workers), resident at
+// once; the bodies are separated by a counter barrier of all blocks.
+__device__ inline bool tail_barrier(Ctrl* ctrl, int target, unsigned spin_limit, int* scratch) {
+  // The bodies on either side exchange their results (positions, sorted costs, distances, the order) through plain
+  // stores and loads, which are coherent between kernels but not between the dies of one kernel: every thread writes
+  // its die's L2 back before it arrives and drops what its caches hold after it leaves.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __hip_atomic_fetch_add(&ctrl->reserved[1], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool seen = bounded_wait([&] { return coherent_load(&ctrl->reserved[1]) >= target; }, spin_limit);
+    if (!seen) coherent_store(&ctrl->err, kErrBarrierTimeout);
+    scratch[0] = seen;
+  }
+  __syncthreads();
+  const bool fine = scratch[0] != 0;
+  __syncthreads();  // scratch is reused
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  return fine;
+}
+
+__global__ __launch_bounds__(kRadixThreads) void tail_kernel(CrowdArgs a, GatherArgs g) {
+  extern __shared__ uint64_t finish_lds[];
+  __shared__ int base[256];
+  __shared__ int scratch[kRadixThreads];
+  Ctrl* ctrl = a.ctrl;
+  int listed_until = 0;
+  if (coherent_load(&ctrl->err) == 0) {
+    if (ctrl->tail_done != 0) {
+      listed_until = ctrl->worst_start;  // the peel kernel has left the order of the last front only
+    } else {
+      const unsigned gen0 = radix_generation_base(ctrl);
+      crowd_sort_body(a, gen0, 0, finish_lds, base, scratch);
+      bool fine = tail_barrier(ctrl, (int)gridDim.x, a.spin_limit, scratch);
+      if (fine) {
+        crowd_finish_body(a, 1, gen0 + 16u, 0, finish_lds, base, scratch);
+        fine = tail_barrier(ctrl, 2 * (int)gridDim.x, a.spin_limit, scratch);
+      }
+      (void)fine;  // the gather looks at the error flag itself
+      if (blockIdx.x == 0 && threadIdx.x == 0) ctrl->radix_epoch += 2;  // both bodies may have run a radix sort
+    }
+  }
+  gather_body(g, blockIdx.x, gridDim.x, listed_until);
 }
 
 }  // namespace evx

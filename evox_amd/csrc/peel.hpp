@@ -102,6 +102,59 @@ __device__ inline int wave_max(int v) {
   return __builtin_amdgcn_readlane(v, 63);
 }
 
+// Maximum, minimum and sum over the sixteen lanes of a group (lanes 16 g .. 16 g + 15), the same in every lane of
+// the group: four rotations inside the DPP row (row_ror 8, 4, 2, 1), no trip through the LDS permute unit.
+__device__ inline unsigned long long row16_rotate(unsigned long long v, int ctrl_index) {
+  unsigned lo = (unsigned)v, hi = (unsigned)(v >> 32);
+  switch (ctrl_index) {  // (the DPP control is an immediate)
+    case 8:
+      lo = __builtin_amdgcn_update_dpp(0, lo, 0x128, 0xf, 0xf, false);
+      hi = __builtin_amdgcn_update_dpp(0, hi, 0x128, 0xf, 0xf, false);
+      break;
+    case 4:
+      lo = __builtin_amdgcn_update_dpp(0, lo, 0x124, 0xf, 0xf, false);
+      hi = __builtin_amdgcn_update_dpp(0, hi, 0x124, 0xf, 0xf, false);
+      break;
+    case 2:
+      lo = __builtin_amdgcn_update_dpp(0, lo, 0x122, 0xf, 0xf, false);
+      hi = __builtin_amdgcn_update_dpp(0, hi, 0x122, 0xf, 0xf, false);
+      break;
+    default:
+      lo = __builtin_amdgcn_update_dpp(0, lo, 0x121, 0xf, 0xf, false);
+      hi = __builtin_amdgcn_update_dpp(0, hi, 0x121, 0xf, 0xf, false);
+      break;
+  }
+  return ((unsigned long long)hi << 32) | lo;
+}
+__device__ inline unsigned long long group16_max(unsigned long long v) {
+#pragma unroll
+  for (int r = 8; r >= 1; r >>= 1) {
+    const unsigned long long o = row16_rotate(v, r);
+    v = o > v ? o : v;
+  }
+  return v;
+}
+__device__ inline unsigned long long group16_min(unsigned long long v) {
+#pragma unroll
+  for (int r = 8; r >= 1; r >>= 1) {
+    const unsigned long long o = row16_rotate(v, r);
+    v = o < v ? o : v;
+  }
+  return v;
+}
+__device__ inline int group16_sum(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x124, 0xf, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x122, 0xf, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x121, 0xf, 0xf, false);
+  return v;
+}
+// The cost behind an ordered_key (common.hpp): zero comes back as +0.0, every NaN as the canonical one.
+__device__ inline float cost_of_key(uint32_t key) {
+  if (key == 0xFFFFFFFFu) return __uint_as_float(0x7FC00000u);
+  return __uint_as_float((key & 0x80000000u) ? key ^ 0x80000000u : ~key);
+}
+
 template <bool MASKED, int R, int U>
 __device__ inline void scan_rows(const uint64_t* const (&row)[R], const int (&nw)[R], const uint64_t* mask_lds,
                                  RowScan (&out)[R]) {

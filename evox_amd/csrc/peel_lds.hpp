@@ -157,6 +157,42 @@ __device__ inline void list_front_words(const uint64_t* front_lds, int nwords, i
   lds_barrier();
 }
 
+// ---- The crowding distances and the order of a small last front, by the workgroups that have just peeled it.
+// When the peeling stops, every sweeping workgroup holds the units of the last level in registers: the slots of
+// the last front.  Ordering that front in a kernel of its own costs the launch (about 4.7 us on this device) and three
+// chains of dependent loads (the control block, the listing, the costs); here the candidates get a number from the
+// records (the same in every workgroup), their costs and original indices are fetched once, every workgroup works
+// out the distances of its share (candidate e belongs to workgroup e mod sweepers; sixteen lanes scan all candidates
+// for the two neighbours in every objective's order, see crowd_small_front in finish.hpp), publishes them as
+// (distance key, original index) composites in a buffer that all workgroups poll -- a zero entry is one that has
+// not arrived -- and places its candidates by counting the smaller composites.  Same results as the kernels of
+// finish.hpp, except that the costs are read back from their order-preserving keys, under which -0.0 is +0.0 (the
+// sign of a distance of zero can differ) and every NaN is the same NaN.
+constexpr int kTailRows = 2048;        // candidates (four per thread in the poll of the buffer)
+constexpr int kTailValues = 4096;      // candidates x objectives: 12 bytes of LDS each
+constexpr int kTailObjectives = 64;
+
+__host__ __device__ inline bool peel_tail_applies(int64_t nv, int m) {
+  return nv >= 1 && nv <= kTailRows && nv * m <= kTailValues && m <= kTailObjectives;
+}
+// Bytes of LDS that the tail needs at most for a population of n rows (0: it never applies).
+__host__ inline size_t peel_tail_lds_bytes(int n, int m) {
+  if (m > kTailObjectives) return 0;
+  int64_t rows = n < kTailRows ? n : kTailRows;
+  if (rows * m > kTailValues) rows = kTailValues / m;
+  if (rows < 1) return 0;
+  return (size_t)(12 * rows * m + 8 * rows + 16 * m + 8 * 256 + 64);
+}
+
+struct PeelTail {
+  int mode;  // 0: ranks only; 2: crowding distances and selection order of the last front
+  int m, npad;
+  const float* xs_sorted;  // fitness by slot, structure of arrays, columns npad apart
+  float* dist;             // by original index
+  int* order;              // selection order
+  unsigned long long* buffer;  // kTailRows entries, zero at the start of the call
+};
+
 // Grid: 1 lister + `sweepers` sweeping workgroups of kRecThreads threads, all resident at once (every workgroup
 // waits for every other one).  Dynamic LDS: lds_peel_bytes().  The matrix must be complete in `dom`; rank, the
 // crowding-distance fill, the front sizes and listings and the control block are written as by count_kernel +
@@ -165,7 +201,8 @@ __global__ __launch_bounds__(kRecThreads) void peel_lds_kernel(
     const uint64_t* __restrict__ dom, int64_t wstride, int nwords, int n, const int* __restrict__ orig_of,
     int* __restrict__ rank, float* __restrict__ dist_fill, uint64_t* __restrict__ fronts_slot,
     uint64_t* __restrict__ fronts_orig, int* __restrict__ fsize, int* __restrict__ perm, int* __restrict__ fstart,
-    Ctrl* __restrict__ ctrl, int stop_count, unsigned spin_limit, unsigned long long* __restrict__ records, int sweepers) {
+    Ctrl* __restrict__ ctrl, int stop_count, unsigned spin_limit, unsigned long long* __restrict__ records, int sweepers,
+    PeelTail tail) {
   extern __shared__ __attribute__((aligned(16))) uint64_t lds[];  // the rows are read 16 bytes at a time
   __shared__ int sh[48];
   if (coherent_load(&ctrl->err) != 0) return;
@@ -390,7 +427,9 @@ __global__ __launch_bounds__(kRecThreads) void peel_lds_kernel(
   }
   if (have_row) {
     rank[st_orig] = st_word < 0 ? 0 : kRankUnset;
-    if (dist_fill) dist_fill[st_orig] = -INFINITY;
+    // (written through: the distance of a row of the last front is stored again at the end of this kernel by
+    // another workgroup, maybe on another die, whose store must not be overtaken by this one's write-back)
+    if (dist_fill) coherent_store(&dist_fill[st_orig], -INFINITY);
   }
   EVX_TRACE(62, 3);
 
@@ -466,7 +505,203 @@ __global__ __launch_bounds__(kRecThreads) void peel_lds_kernel(
       for (int w = tid; w < nwords; w += blockDim.x) alive_lds[w] &= ~coherent_load(&cur[(int64_t)w * kFrontStride]);
       lds_barrier();
     }
-    if (size <= 0 || ranked + size >= stop_count) break;
+    if (size <= 0 || ranked + size >= stop_count) {
+      // front `level` is the last one: a small one is ordered right here (the overflow path leaves no slots in v)
+      if (tail.mode == 2 && (flags & 1) == 0 && peel_tail_applies(size, tail.m)) {
+        const int nv = size, start = ranked, want = stop_count - ranked, m = tail.m;
+        unsigned long long* comp = reinterpret_cast<unsigned long long*>(lds);  // [m][nv], then the distance composites
+        unsigned long long* ends = comp + (size_t)nv * m;                        // [m][2]
+        int* t_slot = reinterpret_cast<int*>(ends + 2 * m);                      // [nv]
+        int* t_orig = t_slot + nv;                                               // [nv]
+        int* rec_cnt = t_orig + nv;                                              // [256] rows per record, then their prefix
+        EVX_TRACE(61, 0);
+        lds_barrier();  // nobody reads the bitmap or the rows any more
+        // number the candidates: record by record, in the order of the record's slots
+        const int n_rec = sweepers;
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+          const int u = 2 * tid + k;
+          if (u < sweepers * units && (u & (units - 1)) == 0)
+            rec_cnt[u / units] = (int)((uint32_t)(v[k] >> (Rec::kBits * (Rec::kFields - 1))) & Rec::kMask & ~Rec::kOverflow);
+        }
+        lds_barrier();
+        if (wave == 0) {  // exclusive prefix over at most 255 records: four per lane
+          int c[4], sum = 0;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            c[q] = 4 * lane + q < n_rec ? rec_cnt[4 * lane + q] : 0;
+            sum += c[q];
+          }
+          int incl = sum;
+#pragma unroll
+          for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(incl, off);
+            if (lane >= off) incl += up;
+          }
+          int run = incl - sum;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            if (4 * lane + q < n_rec) rec_cnt[4 * lane + q] = run;
+            run += c[q];
+          }
+        }
+        lds_barrier();
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+          const int u = 2 * tid + k;
+          if (u >= sweepers * units) continue;
+          const int b = u / units, i = u & (units - 1);
+          // unit 0 carries the count and the record's first kFields - 1 slots, unit i the slots from kFields * i - 1 on
+#pragma unroll
+          for (int fld = 0; fld < Rec::kFields; ++fld) {
+            if (i == 0 && fld == 0) continue;
+            const uint32_t field = (uint32_t)(v[k] >> (Rec::kBits * (Rec::kFields - 1 - fld))) & Rec::kMask;
+            if (field != Rec::kNil) t_slot[rec_cnt[b] + (i == 0 ? fld - 1 : Rec::kFields * i - 1 + fld)] = (int)field;
+          }
+        }
+        lds_barrier();
+        // (cost key, original index) of every candidate in every objective: one round trip to memory
+        for (int idx = tid; idx < nv * m; idx += blockDim.x) {
+          const int k = idx / nv, e = idx - k * nv;
+          const int slot = t_slot[e];
+          const int orig = orig_of[slot];
+          const float c = tail.xs_sorted[(int64_t)k * tail.npad + slot];
+          comp[idx] = ((unsigned long long)ordered_key(c) << 32) | (unsigned)orig;
+          if (k == 0) t_orig[e] = orig;
+        }
+        lds_barrier();
+        EVX_TRACE(61, 1);
+        for (int k = wave; k < m; k += kWaves) {  // first and last composite of every objective
+          unsigned long long lo = ~0ull, hi = 0ull;
+          for (int e = lane; e < nv; e += 64) {
+            const unsigned long long c = comp[k * nv + e];
+            lo = c < lo ? c : lo;
+            hi = c > hi ? c : hi;
+          }
+#pragma unroll
+          for (int off = 1; off < 64; off <<= 1) {
+            const unsigned long long a = ((unsigned long long)__shfl_xor((unsigned)(lo >> 32), off) << 32) | __shfl_xor((unsigned)lo, off);
+            const unsigned long long b = ((unsigned long long)__shfl_xor((unsigned)(hi >> 32), off) << 32) | __shfl_xor((unsigned)hi, off);
+            lo = a < lo ? a : lo;
+            hi = b > hi ? b : hi;
+          }
+          if (lane == 0) {
+            ends[2 * k] = lo;
+            ends[2 * k + 1] = hi;
+          }
+        }
+        lds_barrier();
+        EVX_TRACE(59, 0);
+        const int sub = tid & 15;
+        // this workgroup's candidates are e = sb, sb + sweepers, ...; a group of sixteen lanes takes one (candidate,
+        // objective) pair, so that the objectives of a candidate are scanned side by side, and leaves the term of
+        // the distance (NaN bit pattern 0xFFFFFFFF for "first or last of the objective") in LDS
+        const int groups = kRecThreads >> 4;
+        const int mine_n = sb < nv ? (nv - 1 - sb) / sweepers + 1 : 0;
+        float* term_lds = reinterpret_cast<float*>(rec_cnt + 256);  // [candidates of this workgroup][m]
+        constexpr uint32_t kBoundaryTerm = 0xFFFFFFFFu;
+        for (int it = tid >> 4; it < mine_n * m; it += groups) {  // (whole groups leave the loop together)
+          const int j = it / m, k = it - j * m;
+          const int e = sb + j * sweepers;
+          const unsigned long long* row = comp + (size_t)k * nv;
+          const unsigned long long mine = row[e];
+          unsigned long long below = 0ull, above = ~0ull;  // no composite is zero or all ones
+          for (int p0 = sub; p0 < nv; p0 += 8 * 16) {  // eight partners per step, their LDS reads in flight together
+            unsigned long long c[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) c[u] = p0 + 16 * u < nv ? row[p0 + 16 * u] : mine;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+              if (c[u] < mine) below = c[u] > below ? c[u] : below;
+              if (c[u] > mine) above = c[u] < above ? c[u] : above;
+            }
+          }
+          below = group16_max(below);
+          above = group16_min(above);
+          if (sub == 0) {
+            float term = __uint_as_float(kBoundaryTerm);  // first or last of this objective (non_dominate.py:226-227)
+            if (below != 0ull && above != ~0ull) {
+              const float span = cost_of_key((uint32_t)(ends[2 * k + 1] >> 32)) - cost_of_key((uint32_t)(ends[2 * k] >> 32));
+              term = (cost_of_key((uint32_t)(above >> 32)) - cost_of_key((uint32_t)(below >> 32))) / span;
+            }
+            term_lds[it] = term;
+          }
+        }
+        lds_barrier();
+        EVX_TRACE(59, 1);
+        for (int j = tid; j < mine_n; j += blockDim.x) {
+          const int e = sb + j * sweepers;
+          bool boundary = false;
+          float acc = 0.0f;
+          for (int k = 0; k < m; ++k) {
+            const float term = term_lds[j * m + k];
+            if (__float_as_uint(term) == kBoundaryTerm)
+              boundary = true;
+            else
+              acc = k == 0 ? term : acc + term;
+          }
+          const float d = boundary ? INFINITY : acc;
+          coherent_store(&tail.dist[t_orig[e]], d);
+          coherent_store(&tail.buffer[e], ((unsigned long long)ordered_key(-d) << 32) | (unsigned)t_orig[e]);
+        }
+        EVX_TRACE(61, 2);
+        lds_barrier();  // the composites of the objectives are no longer needed
+        // everybody's distance composites: entries 4 t .. 4 t + 3 are this thread's
+        {
+          typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+          const int e0 = 4 * tid;
+          bool pending0 = e0 < nv, pending1 = e0 + 2 < nv, fine_poll = true;
+          for (unsigned spins = 0; pending0 || pending1; ++spins) {
+            if (pending0) {
+              u32x4 r;
+              asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(r) : "v"(tail.buffer + e0) : "memory");
+              const unsigned long long a = ((unsigned long long)r.y << 32) | r.x, b = ((unsigned long long)r.w << 32) | r.z;
+              if (a != 0ull && (e0 + 1 >= nv || b != 0ull)) {
+                comp[e0] = a;
+                if (e0 + 1 < nv) comp[e0 + 1] = b;
+                pending0 = false;
+              }
+            }
+            if (pending1) {
+              u32x4 r;
+              asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(r) : "v"(tail.buffer + e0 + 2) : "memory");
+              const unsigned long long a = ((unsigned long long)r.y << 32) | r.x, b = ((unsigned long long)r.w << 32) | r.z;
+              if (a != 0ull && (e0 + 3 >= nv || b != 0ull)) {
+                comp[e0 + 2] = a;
+                if (e0 + 3 < nv) comp[e0 + 3] = b;
+                pending1 = false;
+              }
+            }
+            if (spins > spin_limit || ((spins & 63u) == 63u && coherent_load(&ctrl->err) != 0)) {
+              fine_poll = false;
+              break;
+            }
+          }
+          if (!fine_poll) coherent_store(&ctrl->err, kErrBarrierTimeout);
+        }
+        EVX_TRACE(61, 3);
+        lds_barrier();
+        if (coherent_load(&ctrl->err) == 0) {
+          for (int j = tid >> 4; j < mine_n; j += groups) {
+            const int e = sb + j * sweepers;
+            const unsigned long long mine = comp[e];
+            int smaller = 0;
+            for (int p0 = sub; p0 < nv; p0 += 8 * 16) {
+              unsigned long long c[8];
+#pragma unroll
+              for (int u = 0; u < 8; ++u) c[u] = p0 + 16 * u < nv ? comp[p0 + 16 * u] : ~0ull;
+#pragma unroll
+              for (int u = 0; u < 8; ++u) smaller += c[u] < mine;
+            }
+            smaller = group16_sum(smaller);
+            if (sub == 0 && smaller < want) tail.order[start + smaller] = (int)(unsigned)mine;
+          }
+          if (sb == 0 && tid == 0) ctrl->tail_done = 1;
+          EVX_TRACE(60, 0);
+        }
+      }
+      break;
+    }
     ranked += size;
     ++level;  // now building front `level`
     int* const build = sh + 4 * (level & 1);
