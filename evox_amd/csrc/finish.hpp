@@ -233,10 +233,12 @@ __device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int ep
     }
 }
 
-__global__ __launch_bounds__(kRadixThreads) void crowd_sort_kernel(CrowdArgs a) {
+// after_peel_tail: the peel kernel may have ordered the last front already (Ctrl.tail_done).
+__global__ __launch_bounds__(kRadixThreads) void crowd_sort_kernel(CrowdArgs a, int after_peel_tail) {
   extern __shared__ uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
+  if (after_peel_tail != 0 && a.ctrl->tail_done != 0) return;
   crowd_sort_body(a, radix_generation_base(a.ctrl), 1, finish_lds, base, scratch);
 }
 
@@ -370,6 +372,12 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
     uint32_t* dkey_lds = reinterpret_cast<uint32_t*>(finish_lds);
     uint64_t* tile_lds = finish_lds + kRadixMinCandidates / 2;
     if (!want_order && blockIdx.x != 0) return;
+    if (blockIdx.x != 0 && (int64_t)blockIdx.x * blockDim.x >= nv) {
+      // no candidate of its own to place: this block only helps to copy the listing of the better fronts (the
+      // distance keys below are derived by every block that uses them: a larger grid must not multiply that)
+      for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < start; i += gridDim.x * blockDim.x) order[i] = list_base[i];
+      return;
+    }
     for (int q = threadIdx.x; q < nv; q += blockDim.x) {
       const float d = crowding_distance_of(q, nv, m, pos, sorted_cost, kstride);
       if (blockIdx.x == 0) dist[list[q]] = d;
@@ -418,19 +426,19 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
   }
 }
 
-__global__ __launch_bounds__(kRadixThreads) void crowd_finish_kernel(CrowdArgs a, int want_order) {
+__global__ __launch_bounds__(kRadixThreads) void crowd_finish_kernel(CrowdArgs a, int want_order, int after_peel_tail) {
   extern __shared__ uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
+  if (after_peel_tail != 0 && a.ctrl->tail_done != 0) return;
   crowd_finish_body(a, want_order, radix_generation_base(a.ctrl), 1, finish_lds, base, scratch);
 }
 
-// ---- Everything after the peeling in one launch: the ordering of the last front, unless the peel kernel has done
-// it already (Ctrl.tail_done: a small front is ordered by the workgroups that peeled it, while its rows are still
-// at hand), then the gather of the selected rows.  A launch that finds nothing to do still costs as much as a small
-// kernel (about 4.7 us on this device), so the stages that choose their algorithm on the device share one launch
-// instead of queueing one launch per algorithm.  Grid: the radix grid (master, idle block, workers), resident at
-// once; the bodies are separated by a counter barrier of all blocks.
+// ---- The ordering of the last front in one launch, for populations whose peel kernel orders a small last front
+// itself (Ctrl.tail_done says whether it has: then nothing is left to do here).  A launch that finds nothing to do
+// still costs as much as a small kernel (about 4.7 us on this device), so the two stages share one launch; they are
+// separated by a counter barrier of all blocks.  Grid: that of crowd_sort_kernel (the radix grid: master, idle
+// block, workers), resident at once.
 __device__ inline bool tail_barrier(Ctrl* ctrl, int target, unsigned spin_limit, int* scratch) {
   // The bodies on either side exchange their results (positions, sorted costs, distances, the order) through plain
   // stores and loads, which are coherent between kernels but not between the dies of one kernel: every thread writes
@@ -450,28 +458,24 @@ __device__ inline bool tail_barrier(Ctrl* ctrl, int target, unsigned spin_limit,
   return fine;
 }
 
-__global__ __launch_bounds__(kRadixThreads) void tail_kernel(CrowdArgs a, GatherArgs g) {
+__global__ __launch_bounds__(256) void gather_kernel(GatherArgs g) { gather_body(g, blockIdx.x, gridDim.x, 0); }
+
+// listed: the rows of the better fronts as the peel listed them; positions below Ctrl.worst_start take their row
+// from there when the peel kernel has ordered the last front (it then leaves only that front's part of `order`).
+__global__ __launch_bounds__(256) void gather_after_peel_kernel(GatherArgs g) {
+  gather_body(g, blockIdx.x, gridDim.x, g.ctrl->err == 0 && g.ctrl->tail_done != 0 ? g.ctrl->worst_start : 0);
+}
+
+__global__ __launch_bounds__(kRadixThreads) void crowd_kernel(CrowdArgs a) {
   extern __shared__ uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
   Ctrl* ctrl = a.ctrl;
-  int listed_until = 0;
-  if (coherent_load(&ctrl->err) == 0) {
-    if (ctrl->tail_done != 0) {
-      listed_until = ctrl->worst_start;  // the peel kernel has left the order of the last front only
-    } else {
-      const unsigned gen0 = radix_generation_base(ctrl);
-      crowd_sort_body(a, gen0, 0, finish_lds, base, scratch);
-      bool fine = tail_barrier(ctrl, (int)gridDim.x, a.spin_limit, scratch);
-      if (fine) {
-        crowd_finish_body(a, 1, gen0 + 16u, 0, finish_lds, base, scratch);
-        fine = tail_barrier(ctrl, 2 * (int)gridDim.x, a.spin_limit, scratch);
-      }
-      (void)fine;  // the gather looks at the error flag itself
-      if (blockIdx.x == 0 && threadIdx.x == 0) ctrl->radix_epoch += 2;  // both bodies may have run a radix sort
-    }
-  }
-  gather_body(g, blockIdx.x, gridDim.x, listed_until);
+  if (coherent_load(&ctrl->err) != 0 || ctrl->tail_done != 0) return;
+  const unsigned gen0 = radix_generation_base(ctrl);
+  crowd_sort_body(a, gen0, 0, finish_lds, base, scratch);
+  if (tail_barrier(ctrl, (int)gridDim.x, a.spin_limit, scratch)) crowd_finish_body(a, 1, gen0 + 16u, 0, finish_lds, base, scratch);
+  if (blockIdx.x == 0 && threadIdx.x == 0) ctrl->radix_epoch += 2;  // both bodies may have run a radix sort
 }
 
 }  // namespace evx
