@@ -365,7 +365,7 @@ static int grant_dynamic_lds(const void* kernel, size_t lds) {
 // population does not fit (or the option is off).  Every workgroup takes a compute unit of its own.
 constexpr size_t kLdsPeelBudget = 160 * 1024 - 512;
 static int lds_peel_plan(const Layout& L, size_t* lds_out) {
-  if (!g_opt.peel_lds || L.n > 32768 || L.nwords > kRecThreads) return 0;  // (the lister keeps original indices in 16 bits and takes a bitmap word per thread)
+  if (!g_opt.peel_lds || L.n > 32768 || L.nwords > kLdsPeelThreads) return 0;  // (the lister keeps original indices in 16 bits and takes a bitmap word per thread)
   const int most = device_cus() - 1 < 255 ? device_cus() - 1 : 255;  // + the lister; a record holds at least 4 units
   if (most < 8) return 0;
   auto fits = [&](int sweepers) {
@@ -414,12 +414,12 @@ static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool
                                        (int)kLdsPeelBudget);
     if (e != hipSuccess) return (int)e;
     int per_cu = 0;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, peel_lds_kernel, kRecThreads, kLdsPeelBudget);
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, peel_lds_kernel, kLdsPeelThreads, kLdsPeelBudget);
     if (e != hipSuccess) return (int)e;
     resident[dev] = per_cu + 1;
   }
   if ((int64_t)(resident[dev] - 1) * device_cus() < sweepers + 1) return kErrBadArg;
-  hipLaunchKernelGGL(peel_lds_kernel, dim3(sweepers + 1), dim3(kRecThreads), lds, s, w.at<uint64_t>(L.dom), L.wstride, L.nwords, L.n,
+  hipLaunchKernelGGL(peel_lds_kernel, dim3(sweepers + 1), dim3(kLdsPeelThreads), lds, s, w.at<uint64_t>(L.dom), L.wstride, L.nwords, L.n,
                      w.at<int>(L.orig_of), w.at<int>(L.rank), fill_dist ? w.at<float>(L.dist) : (float*)nullptr,
                      w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
                      want_perm ? w.at<int>(L.perm) : (int*)nullptr, w.at<int>(L.fstart), w.ctrl(), (int)stop_count, g_opt.spin_limit,
@@ -1426,6 +1426,17 @@ int evox_hip_calibration_launch(int kind, int64_t blocks, int64_t iterations, fl
   else
     hipLaunchKernelGGL(calibrate_kernel<3>, grid, block, 0, s, scratch_out, (int)iterations, 1.0f, 2.0f);
   EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+int evox_hip_peel_plan(int64_t n, int64_t m, int64_t* out3) {
+  Layout L;
+  if (out3 == nullptr || !make_layout(n, m, &L)) return kErrBadArg;
+  size_t lds = 0;
+  const int sweepers = prefix_dominance_applies(L) ? 0 : lds_peel_plan(L, &lds);
+  out3[0] = sweepers != 0;
+  out3[1] = sweepers;
+  out3[2] = (int64_t)lds;
   return 0;
 }
 

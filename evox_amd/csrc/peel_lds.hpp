@@ -23,13 +23,14 @@
 
 namespace evx {
 
+constexpr int kLdsPeelThreads = 512;  // (1024 threads: the rows are copied 2 us sooner, the first exchange takes 2 us longer)
 constexpr int kLdsPeelRowsPerWave = 64;  // one row per lane
-constexpr int kLdsPeelMaxRowsPerBlock = kLdsPeelRowsPerWave * (kRecThreads / 64);
+constexpr int kLdsPeelMaxRowsPerBlock = kLdsPeelRowsPerWave * (kLdsPeelThreads / 64);
 
 // Bytes of dynamic LDS for a grid of `sweepers` sweeping workgroups (an upper bound over the workgroups: as if
 // every wave's k-th row were the longest k-th row of any wave), 0 when a wave would own more than 64 rows.
 __host__ inline size_t lds_peel_bytes(int n, int nwords, int sweepers) {
-  const int waves = kRecThreads / 64;
+  const int waves = kLdsPeelThreads / 64;
   const int64_t step = (int64_t)sweepers * waves;
   const int64_t per_wave = (n + step - 1) / step;
   if (per_wave > kLdsPeelRowsPerWave) return 0;
@@ -117,7 +118,7 @@ __device__ inline void lds_row_highest(const uint64_t* row, int nw, const uint64
 // Lists the set bits of a front bitmap of at most blockDim.x words (LDS) in ascending order into perm[base ...].  A
 // thread takes a word; when some word is dense (a front of neighbouring rows: 64 stores from one thread, one after
 // the other, made a level of the listing slower than a level of the peeling) the words are instead taken by whole
-// waves, a lane per bit.  word_base: nwords ints of LDS; scratch: 16 ints.  The barriers order LDS traffic only.
+// waves, a lane per bit.  word_base: nwords ints of LDS; scratch: 32 ints.  The barriers order LDS traffic only.
 __device__ inline void list_front_words(const uint64_t* front_lds, int nwords, int* __restrict__ perm, int base,
                                         int* word_base, int* scratch) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
@@ -132,13 +133,13 @@ __device__ inline void list_front_words(const uint64_t* front_lds, int nwords, i
   const int densest = wave_max(mine);
   if (lane == 63) {
     scratch[wave] = incl;
-    scratch[8 + wave] = densest;
+    scratch[16 + wave] = densest;
   }
   lds_barrier();
   int pos = base + incl - mine, heavy = 0;
   for (int v = 0; v < waves; ++v) {
     if (v < wave) pos += scratch[v];
-    heavy = max(heavy, scratch[8 + v]);
+    heavy = max(heavy, scratch[16 + v]);
   }
   if (heavy <= 12) {
     uint64_t left = bits;
@@ -193,11 +194,11 @@ struct PeelTail {
   unsigned long long* buffer;  // kTailRows entries, zero at the start of the call
 };
 
-// Grid: 1 lister + `sweepers` sweeping workgroups of kRecThreads threads, all resident at once (every workgroup
+// Grid: 1 lister + `sweepers` sweeping workgroups of kLdsPeelThreads threads, all resident at once (every workgroup
 // waits for every other one).  Dynamic LDS: lds_peel_bytes().  The matrix must be complete in `dom`; rank, the
 // crowding-distance fill, the front sizes and listings and the control block are written as by count_kernel +
 // peel_records_kernel.  Stops as soon as the fronts built so far hold stop_count rows.
-__global__ __launch_bounds__(kRecThreads) void peel_lds_kernel(
+__global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
     const uint64_t* __restrict__ dom, int64_t wstride, int nwords, int n, const int* __restrict__ orig_of,
     int* __restrict__ rank, float* __restrict__ dist_fill, uint64_t* __restrict__ fronts_slot,
     uint64_t* __restrict__ fronts_orig, int* __restrict__ fsize, int* __restrict__ perm, int* __restrict__ fstart,
@@ -210,7 +211,7 @@ __global__ __launch_bounds__(kRecThreads) void peel_lds_kernel(
   while (units * 2 * sweepers <= kRecUnits && units < 32) units *= 2;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  constexpr int kWaves = kRecThreads / 64;
+  constexpr int kWaves = kLdsPeelThreads / 64;
   using Rec = RecFormat<false>;
 
   if (blockIdx.x == 0) {
@@ -596,7 +597,7 @@ __global__ __launch_bounds__(kRecThreads) void peel_lds_kernel(
         // this workgroup's candidates are e = sb, sb + sweepers, ...; a group of sixteen lanes takes one (candidate,
         // objective) pair, so that the objectives of a candidate are scanned side by side, and leaves the term of
         // the distance (NaN bit pattern 0xFFFFFFFF for "first or last of the objective") in LDS
-        const int groups = kRecThreads >> 4;
+        const int groups = kLdsPeelThreads >> 4;
         const int mine_n = sb < nv ? (nv - 1 - sb) / sweepers + 1 : 0;
         float* term_lds = reinterpret_cast<float*>(rec_cnt + 256);  // [candidates of this workgroup][m]
         constexpr uint32_t kBoundaryTerm = 0xFFFFFFFFu;

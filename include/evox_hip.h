@@ -231,13 +231,22 @@ int evox_hip_stage_order(int64_t n, int64_t m, void* workspace, size_t workspace
  * dominates the row in slot s.  Ranks, distances, listings and the order use original row indices. */
 int evox_hip_workspace_layout(int64_t n, int64_t m, int64_t* out11);
 
+/* How a population of this shape is peeled, for tools and benchmarks: out[0] = 1 when every sweeping workgroup keeps
+ * its rows of the bit matrix in LDS (the matrix fits the LDS of the device; counts and peeling are then one kernel),
+ * 0 when rows are rescanned in memory; out[1] = sweeping workgroups of that kernel, out[2] = bytes of LDS of each
+ * (both 0 when out[0] is 0).  Depends on the device that is current and on the tunables. */
+int evox_hip_peel_plan(int64_t n, int64_t m, int64_t* out3);
+
 /* Waits for `stream`, then copies the control block's eight leading ints to HOST memory:
  * out[0] error (0 or EVOX_HIP_E_BARRIER_TIMEOUT), out[1] fronts peeled, out[2] last front's rank,
  * out[3] rows in better fronts, out[4] last front's size, out[5] rows taken from it, out[6] sweep passes.
  * Returns out[0] when it is non-zero. */
 int evox_hip_read_status(const void* workspace, void* stream, int32_t* host_out8);
 
-/* Tunables (process-wide): "peel_blocks_per_cu" (default 2), "peel_witness" (1 = witness pass, 0 = popcount sweep), "peel_records" (1 = record
+/* Tunables (process-wide): "peel_lds" (1 = populations whose bit matrix fits the LDS of the device are peeled from LDS), "peel_lds_blocks"
+ * (0 = by size, or 8 .. 255 sweeping workgroups of that kernel), "peel_tail" (1 = that kernel also orders a small last front), "tail_merged"
+ * (1 = after such a peel the two ordering stages share one launch, up to three objectives),
+ * "peel_blocks_per_cu" (default 2), "peel_witness" (1 = witness pass, 0 = popcount sweep), "peel_records" (1 = record
  * protocol, 0 = master barrier and front bitmaps), "peel_record_blocks" (0 = by size, or 16 .. 255), "spin_limit" (polls before a device-side
  * wait gives up, default 4000000), "dominance_tile_words" (4, 8 or 16, default 4), "small_sort" (1 = one-kernel slot sort up to 4096 rows),
  * "prefix_min_rows" (default 65536: smallest finite population whose matrix is built from the per-objective orders, 0 = never),
