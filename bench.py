@@ -26,15 +26,34 @@ VALU_CMP_PEAK_GOPS = 39321.6  # 256 CU x 64 lanes/clk x 2.4 GHz: issue peak of v
 VALU_FP32_PEAK_GOPS = 78643.2  # 256 CU x 128 lanes/clk x 2.4 GHz: non-packed fp32 vector ops (157.3 TFLOP/s / 2)
 FP32_VECTOR_PEAK_GFLOPS = 157300.0
 
-# HBM bytes per launch from rocprofv3 counter runs of this script (FETCH_SIZE and WRITE_SIZE in runs of
-# their own, scaled by what the same counters read for a 512 MiB copy: x2.0 and x1.0); the summaries
-# with the commands are kept under profiles/.  Keyed by (workload, kernel); absent = not measured.
-MEASURED_TRAFFIC_BYTES = {
-    ("C5", "dominance_prefix_kernel"): 1156.56e6 + 2602.48e6,  # profiles/c5_selection_hbm_traffic.md: read + written
-    ("C3", "peel_records_kernel"): 11.33e6 + 2.03e6,
-    ("C3", "dominance_kernel"): 3.54e6 + 25.36e6,
-    ("C3", "count_kernel"): 27.00e6 + 1.30e6,
-}
+
+
+def profile_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` as the committed counter summary of this workload holds them
+    (profiles/<workload>_selection_hbm_traffic.md: FETCH_SIZE and WRITE_SIZE runs of this script, scaled by what the
+    same counters read for a 512 MiB copy); None where the summary has no row for the kernel."""
+    path = os.path.join(ROOT, "profiles", f"{workload.lower()}_selection_hbm_traffic.md")
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) == 6 and cells[0].startswith("evx::" + kernel) and cells[0][len("evx::" + kernel):][:1] in ("", "<"):
+            try:
+                return {"bytes": (float(cells[4]) + float(cells[5])) * 1e6, "read_MB": float(cells[4]),
+                        "written_MB": float(cells[5]), "source": os.path.relpath(path, ROOT)}
+            except ValueError:
+                continue
+    return None
+
+
+def host_cpu():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def parse():
@@ -44,7 +63,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
-    ap.add_argument("--cpu-sample", type=int, default=16000, help="rows of the workload timed on the CPU")
+    ap.add_argument("--cpu-sample", type=int, default=0, help="rows of the workload timed on the CPU (0 = all of them)")
+    ap.add_argument("--cpu-runs", type=int, default=1, help="runs of the CPU leg (the median is reported)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 512 MiB device copy three times, so that a rocprofv3 --pmc run of this "
                          "command holds a kernel of known traffic next to the selection kernels")
@@ -94,14 +114,29 @@ def valu_issue_rates(dev):
     return out
 
 
-def stage_profile(w, f, reps):
-    """Times every stage alone through the stage entry points (same kernels, same stream)."""
+def peel_plan(n, m):
+    """(peeled from LDS?, sweeping workgroups, bytes of LDS each) as the library decides for this shape."""
+    import ctypes
+
+    from evox_amd import _lib
+
+    out = (ctypes.c_int64 * 3)()
+    _lib.call("evox_hip_peel_plan", n, m, out)
+    return bool(out[0]), int(out[1]), int(out[2])
+
+
+def stage_profile(w, x, f, reps):
+    """Where the time of a step goes: the step's stages are run as ever longer prefixes of the pipeline, back to back
+    on the launch stream (same kernels as the step's), and a stage's time is the difference between two prefixes, so
+    the gaps between launches are counted where the step pays them.  The whole step is the last prefix: the selection
+    entry point called through the C ABI with outputs allocated beforehand."""
     from evox_amd import _lib, runtime
 
     n, m = f.shape
     ws = runtime.workspace(n, m, f.device)
     s = runtime.stream_handle(f.device)
     tail = (ws.data_ptr(), ws.numel(), s)
+    from_lds = peel_plan(n, m)[0]
 
     def prep():
         _lib.call("evox_hip_stage_prepare", f.data_ptr(), n, m, f.stride(0), f.stride(1), *tail)
@@ -115,32 +150,58 @@ def stage_profile(w, f, reps):
     def peel():
         _lib.call("evox_hip_stage_peel", n, m, w.topk, None, *tail)
 
-    def crowd():
-        _lib.call("evox_hip_stage_crowding", n, m, *tail)
+    xr = x if x.dim() > 1 else x.unsqueeze(1)
+    out_x = torch.empty(w.topk, xr.size(1), dtype=xr.dtype, device=f.device)
+    out_f = torch.empty(w.topk, m, dtype=torch.float32, device=f.device)
+    out_rank = torch.empty(w.topk, dtype=torch.int32, device=f.device)
+    out_dist = torch.empty(w.topk, dtype=torch.float32, device=f.device)
 
-    def order():
-        _lib.call("evox_hip_stage_order", n, m, *tail)
+    def whole():
+        _lib.call("evox_hip_nd_environmental_selection", xr.data_ptr(), xr.size(1) * xr.element_size(),
+                  xr.stride(0) * xr.element_size(), f.data_ptr(), n, m, f.stride(0), f.stride(1), w.topk, out_x.data_ptr(),
+                  out_f.data_ptr(), out_rank.data_ptr(), out_dist.data_ptr(), None, *tail)
 
-    times = {}
-    prep(); dom(); count(); peel(); crowd(); order()
+    def upto_dom():
+        prep(); dom()
+
+    def upto_count():
+        prep(); dom(); count()
+
+    def upto_peel():
+        prep(); dom()
+        if not from_lds:  # (the kernel that peels from LDS counts for itself)
+            count()
+        peel()
+
+    times = {"peel_from_lds": from_lds}
+    whole(); upto_peel()
     torch.cuda.synchronize()
-    times["prepare_us"] = event_time_us(prep, reps)
-    times["dominance_us"] = event_time_us(dom, reps)
+    t_prep = event_time_us(prep, reps)
+    t_dom = event_time_us(upto_dom, reps)
+    t_peel = event_time_us(upto_peel, reps)
+    t_whole = event_time_us(whole, reps)
+    times["prepare_us"] = t_prep
+    times["dominance_us"] = t_dom - t_prep
+    if from_lds:
+        times["count_us"] = None
+        times["peel_us"] = t_peel - t_dom
+    else:
+        t_count = event_time_us(upto_count, reps)
+        times["count_us"] = t_count - t_dom
+        times["peel_us"] = t_peel - t_count
+    times["order_and_gather_us"] = t_whole - t_peel
+    times["step_us"] = t_whole
+    # the dominance stage alone, back to back (it reads what stage_prepare left and can be repeated)
+    prep(); dom()
+    times["dominance_alone_us"] = event_time_us(dom, reps)
     try:  # where the matrix comes from the per-objective orders: the ordering alone (an error elsewhere)
         def orders():
             _lib.call("evox_hip_stage_dominance", n, m, 5, *tail)
         orders()
         times["dominance_orders_us"] = event_time_us(orders, reps)
-        dom()
     except _lib.EvoxHipError:
         times["dominance_orders_us"] = None
-    times["count_us"] = event_time_us(count, reps)
-    # the peel consumes the counts, so each repetition re-runs count first and subtracts it
-    both = event_time_us(lambda: (count(), peel()), reps)
-    times["peel_us"] = max(both - times["count_us"], 0.0)
-    times["crowding_us"] = event_time_us(crowd, reps)
-    times["order_us"] = event_time_us(order, reps)
-    count(); peel()
+    upto_peel()
     runtime.note_call(ws, s)
     status = runtime.last_status()
     views = runtime.workspace_views(ws, n, m)
@@ -150,27 +211,49 @@ def stage_profile(w, f, reps):
     return times, status, rank, slot_of, views["nwords"]
 
 
-def cpu_baseline(w, sample_rows):
-    """The CPU oracle (torch restatement of the reference's eager path) on the first `sample_rows`
-    rows of the workload, all host threads.  Only this leg touches oracle/."""
-    from oracle import eager_restatement as er
-
-    n = min(sample_rows, w.f.size(0))
+def cpu_baseline(w, sample_rows, runs):
+    """The CPU leg, on the host's cores.  Populations whose dense relation fits host memory: the torch restatement of
+    the reference's eager path, all host threads.  C5 (the reference's formulation would need 40 GB for the relation
+    and two temporaries of 320 GB): the plain-C checker (OpenMP over rows), which is NOT the reference's algorithm
+    (the relation as a bit matrix, peeling by counts).  Only this leg touches oracle/."""
+    n = w.f.size(0) if sample_rows <= 0 else min(sample_rows, w.f.size(0))
     f = w.f[:n].contiguous()
     x = (w.x if w.x is not None else w.f)[:n].contiguous()
-    k = max(1, n // 2)
-    torch.set_num_threads(os.cpu_count() or 1)
-    t0 = time.perf_counter()
-    er.environmental_selection(x, f, k)
-    dt = time.perf_counter() - t0
+    k = w.topk if n == w.f.size(0) else max(1, n // 2)
+    what = f"all {n} rows of {w.name}" if n == w.f.size(0) else f"first {n} rows of {w.name}"
+    dense_bytes = n * n * (2 * f.size(1) + 2)  # the relation, its two (N, N, M) temporaries, one peel temporary
+    secs = []
+    if dense_bytes <= 24 * 2**30:
+        from oracle import eager_restatement as er
+
+        torch.set_num_threads(os.cpu_count() or 1)
+        cores = torch.get_num_threads()
+        for _ in range(max(1, runs)):
+            t0 = time.perf_counter()
+            er.environmental_selection(x, f, k)
+            secs.append(time.perf_counter() - t0)
+        how = "torch-CPU restatement of the reference's eager path"
+    else:
+        from oracle import c_oracle
+
+        cores = c_oracle.threads()
+        fn = f.numpy()
+        for _ in range(max(1, runs)):
+            t0 = time.perf_counter()
+            c_oracle.select(fn, k)
+            secs.append(time.perf_counter() - t0)
+        how = (f"plain-C checker on {cores} threads: NOT the reference's algorithm (the reference's dense formulation cannot "
+               "allocate at this size)")
+    dt = median(secs)
     return {
         "value": n * n / dt,
         "unit": "comparisons/s",
-        "cores": torch.get_num_threads(),
+        "cores": cores,
+        "cpu": host_cpu(),
         "kind": "port",
-        "sample": f"first {n} rows of {w.name} (topk={k}), one nd_environmental_selection call, {dt:.2f} s; "
-                  f"torch-CPU restatement of the reference's eager path",
+        "sample": f"{what} (topk={k}), one nd_environmental_selection call, median of {len(secs)} run(s): {dt:.2f} s; {how}",
         "seconds": dt,
+        "runs": secs,
     }
 
 
@@ -396,21 +479,26 @@ def main():
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
 
-    times, status, rank, slot_of, nwords = stage_profile(w, f, max(5, min(args.steps, 30)))
+    times, status, rank, slot_of, nwords = stage_profile(w, x, f, max(5, min(args.steps, 30)))
+    from_lds = times["peel_from_lds"]
 
     pairs = float(n) * n
     compares = 2.0 * m * pairs  # the reference's `<=` and `<` per objective and ordered pair
     # Bytes that the algorithm must move.  Rows live in slots (sorted by key) and only words 0..slot/64
     # of a row can be non-zero, so a row read costs row_words(slot) * 8 bytes.
     #   dominance: fitness in, the words of the lower triangle out (nothing above the diagonal is stored)
-    #   count:     every row read once
-    #   peel:      witness pass: a row is rescanned at least once, in the pass that ranks it; plus the
+    #   count:     every row read once (no such stage where the rows are peeled from LDS)
+    #   peel from LDS: every row read once into LDS, slot -> index table in, rank / distance fill / listing out,
+    #              and one front bitmap per level
+    #   peel from memory (witness pass): a row is rescanned at least once, in the pass that ranks it; plus the
     #              front bitmap (one word per 128-byte line) read by the sweepers each pass
-    row_bytes = nwords * 8
     row_read = (((slot_of >> 6) + 2) & ~1) * 8
     passes = status["passes"]
     ranked_in_passes = (rank >= 1) & (rank <= passes)
-    peel_bytes = int(row_read[ranked_in_passes].sum()) + passes * nwords * 8
+    if from_lds:
+        peel_bytes = int(row_read.sum()) + 4 * n * 4 + (passes + 1) * nwords * 8
+    else:
+        peel_bytes = int(row_read[ranked_in_passes].sum()) + passes * nwords * 8
     dom_bytes = n * m * 4 + int(row_read.sum())
     slots = torch.arange(n, device=rank.device)
     evaluated_pairs = float(((((slots >> 6) << 6) + 63) // 256 * 256 + 256).clamp(max=nwords * 64).sum())
@@ -427,38 +515,38 @@ def main():
     executed_valu = valu_per_pair * evaluated_pairs
     executed_peak = VALU_FP32_PEAK_GOPS if finite else VALU_CMP_PEAK_GOPS
     count_bytes = int(row_read.sum()) + n * 12
+    dom_us = times["dominance_alone_us"]  # the kernel by itself, back to back; "us" is its share of the step
     phases = {
         "prepare_and_slot_sort": {"us": times["prepare_us"]},
-        # achieved: the reference's 2*M*N^2 compares over the kernel time (the algorithmic figure), against the
-        # issue peak of compares; executed: the VALU lane-instructions this kernel issues per ordered pair of the
-        # lower triangle (tiles of 64 rows x 256 columns on or below the diagonal), over the same time, against
-        # the peak of the instruction kind it uses
-        "dominance": {"us": times["dominance_us"], "bound": "valu", "achieved": compares / times["dominance_us"] / 1e3,
-                      "peak": VALU_CMP_PEAK_GOPS, "unit": "Gcompare/s",
-                      "executed_valu_Gops": executed_valu / times["dominance_us"] / 1e3,
-                      "executed_form": "arithmetic" if finite else "compare", "executed_valu_peak_Gops": executed_peak,
-                      "executed_valu_frac": executed_valu / times["dominance_us"] / 1e3 / executed_peak,
-                      "hbm_GBs": dom_bytes / times["dominance_us"] / 1e3},
-        "count": {"us": times["count_us"], "bound": "hbm", "achieved": count_bytes / times["count_us"] / 1e3,
-                  "peak": HBM_PEAK_GBS, "unit": "GB/s"},
+        # achieved / frac: the VALU lane-instructions this kernel issues per ordered pair of the lower triangle (tiles
+        # of 64 rows x 256 columns on or below the diagonal) over the kernel's time, against the peak of the
+        # instruction kind it uses.  The reference's 2*M*N^2 compares over the same time ride along as a rate only:
+        # the kernel does not execute them, so no fraction of a peak is formed from them.
+        "dominance": {"us": times["dominance_us"], "kernel_alone_us": dom_us, "bound": "valu",
+                      "achieved": executed_valu / dom_us / 1e3, "peak": executed_peak, "unit": "G lane-ops/s",
+                      "executed_form": "arithmetic" if finite else "compare",
+                      "reference_compares_rate_Gcompare_s": compares / dom_us / 1e3,
+                      "hbm_GBs": dom_bytes / dom_us / 1e3},
         "peel": {"us": times["peel_us"], "bound": "hbm", "achieved": peel_bytes / max(times["peel_us"], 1e-9) / 1e3,
                  "peak": HBM_PEAK_GBS, "unit": "GB/s", "passes": passes, "bytes": peel_bytes,
                  "us_per_pass": times["peel_us"] / max(passes, 1),
-                 "note": "latency-bound: each pass is one dependent row read plus one exchange between all blocks"},
-        "crowding": {"us": times["crowding_us"]},
-        "order": {"us": times["order_us"]},
+                 "note": ("one kernel: rows copied to LDS and counted on the way, then one exchange between all workgroups per "
+                          "front, then the order of the last front; latency-bound, not bandwidth-bound") if from_lds else
+                         "latency-bound: each pass is one dependent row read plus one exchange between all blocks"},
+        "order_and_gather": {"us": times["order_and_gather_us"]},
     }
+    if not from_lds:
+        phases["count"] = {"us": times["count_us"], "bound": "hbm", "achieved": count_bytes / times["count_us"] / 1e3,
+                           "peak": HBM_PEAK_GBS, "unit": "GB/s"}
     if from_orders:
-        # bound by the stores of the matrix (64-byte pieces of rows that lie kilobytes apart); the reference's
-        # compares over the same time stay as the algorithmic figure
+        # bound by the stores of the matrix (64-byte pieces of rows that lie kilobytes apart)
         # (the stage = the ordering of the rows in every objective, then dominance_prefix_kernel: `achieved` is that
         # kernel's, its time being the stage less the ordering)
-        kernel_us = times["dominance_us"] - (times.get("dominance_orders_us") or 0.0)
-        phases["dominance"] = {"us": times["dominance_us"], "orders_us": times.get("dominance_orders_us"),
+        kernel_us = dom_us - (times.get("dominance_orders_us") or 0.0)
+        phases["dominance"] = {"us": times["dominance_us"], "kernel_alone_us": dom_us, "orders_us": times.get("dominance_orders_us"),
                                "prefix_kernel_us": kernel_us, "bound": "hbm", "achieved": dom_bytes / kernel_us / 1e3,
                                "peak": HBM_PEAK_GBS, "unit": "GB/s", "executed_form": "objective orders",
-                               "algorithmic_Gcompare_s": compares / times["dominance_us"] / 1e3,
-                               "hbm_GBs": dom_bytes / kernel_us / 1e3}
+                               "reference_compares_rate_Gcompare_s": compares / dom_us / 1e3}
     for p in phases.values():
         if "achieved" in p:
             p["frac"] = p["achieved"] / p["peak"]
@@ -467,18 +555,23 @@ def main():
     if not from_orders:
         rates = valu_issue_rates(dev)
         phases["dominance"]["measured_issue_rates_Gops"] = rates
-        phases["dominance"]["executed_valu_frac_of_measured_rate"] = (
-            phases["dominance"]["executed_valu_Gops"] / (rates["v_add_f32"] if finite else rates["v_cmp_to_sgpr"]))
-    dominant = max(("dominance", "count", "peel"), key=lambda k: phases[k]["us"])
+        phases["dominance"]["frac_of_measured_rate"] = (
+            phases["dominance"]["achieved"] / (rates["v_add_f32"] if finite else rates["v_cmp_to_sgpr"]))
+    dominant = max((k for k in ("dominance", "count", "peel") if k in phases), key=lambda k: phases[k]["us"])
     d = phases[dominant]
     roofline = {
-        # populations up to 262144 rows are peeled by the record-protocol kernel, larger ones by peel_kernel
+        # populations whose matrix fits the LDS of the device are peeled from there; others up to 262144 rows by the
+        # record-protocol kernel, larger ones by peel_kernel
         "kernel": {"dominance": "dominance_prefix_kernel" if from_orders else "dominance_kernel", "count": "count_kernel",
-                   "peel": "peel_records_kernel" if n <= 262144 else "peel_kernel"}[dominant],
+                   "peel": "peel_lds_kernel" if from_lds else ("peel_records_kernel" if n <= 262144 else "peel_kernel")}[dominant],
         "bound": "hbm" if d["bound"] == "hbm" else "valu",
         "achieved": d["achieved"], "peak": d["peak"], "unit": d["unit"], "frac": d["frac"], "traffic": None,
+        "kernel_us": d.get("prefix_kernel_us", d.get("kernel_alone_us", d["us"])),
     }
-    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get((args.workload, roofline["kernel"]))
+    measured = profile_traffic(args.workload, roofline["kernel"])
+    if measured is not None:
+        roofline["traffic"] = measured["bytes"]
+        roofline["traffic_source"] = measured["source"]
 
     out = {
         "metric": "dominance comparisons/sec through nd_environmental_selection (N^2 ordered pairs per step)",
@@ -497,8 +590,9 @@ def main():
                                f"topk={w.topk}, fitness U[0,1) seed {w.seed}" if w.name in ("C1", "C3") else
                                f"{w.name}: nd_environmental_selection N={n} M={m} topk={w.topk} seed {w.seed}"},
         "latency_ms": ms_per_step,
-        "dominance_kernel_comparisons_per_s": pairs / (times["dominance_us"] * 1e-6),
-        "dominance_kernel_scalar_compares_per_s": compares / (times["dominance_us"] * 1e-6),
+        "step_us_by_events": times["step_us"],
+        "dominance_kernel_comparisons_per_s": pairs / (times["dominance_alone_us"] * 1e-6),
+        "dominance_kernel_scalar_compares_per_s": compares / (times["dominance_alone_us"] * 1e-6),
         "fronts_peeled": status["fronts"],
         "roofline": roofline,
         "phases": phases,
@@ -506,7 +600,7 @@ def main():
     if args.next_rows:
         out["next_rows"] = next_rows(dev, max(5, min(args.steps, 20)))
     if not args.no_cpu:
-        base = cpu_baseline(w, args.cpu_sample)
+        base = cpu_baseline(w, args.cpu_sample, args.cpu_runs)
         out["cpu_baseline"] = base
         out["speedup_vs_cpu_baseline"] = out["value"] / base["value"]
     print(json.dumps(out))

@@ -888,10 +888,12 @@ int evox_hip_stage_peel(int64_t n, int64_t m, int64_t stop_count, int32_t* rank_
                         void* stream) {
   Ws w;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
-  // (the kernel that peels from LDS counts for itself; after stage_count it finds the same front 0 again)
+  // (the kernel that peels from LDS counts for itself; after stage_count it finds the same front 0 again.  As in the
+  // selection it also orders a small last front: that part reads memory which stage_prepare clears, so a timing
+  // of it repeats the stages from stage_prepare on)
   size_t lds = 0;
   if (const int sweepers = lds_peel_plan(w.L, &lds)) {
-    if (int e = launch_lds_peel(w, stop_count, true, true, sweepers, lds, (hipStream_t)stream)) return e;
+    if (int e = launch_lds_peel(w, stop_count, true, true, sweepers, lds, (hipStream_t)stream, true)) return e;
   } else if (int e = stage_peel(w, stop_count, true, (hipStream_t)stream)) {
     return e;
   }

@@ -26,8 +26,15 @@ def lib():
                                     ctypes.c_void_p, ctypes.c_void_p]
         h.oracle_first_front.restype = ctypes.c_int
         h.oracle_first_front.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+        h.oracle_threads.restype = ctypes.c_int
+        h.oracle_threads.argtypes = []
         _lib = h
     return _lib
+
+
+def threads() -> int:
+    """Threads that the checker's parallel loops run on."""
+    return int(lib().oracle_threads())
 
 
 def _f32(f):

@@ -17,11 +17,15 @@
  * the reference's golden vectors) on every small case.  Only tests/ may load this library.
  */
 #include <math.h>
+#include <omp.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
 
 typedef uint64_t u64;
+
+/* Threads that the parallel loops below run on (for reports of timings). */
+int oracle_threads(void) { return omp_get_max_threads(); }
 
 static int dominates(const float* a, const float* b, int m) {
   int lt = 0;

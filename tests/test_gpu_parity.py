@@ -140,14 +140,22 @@ def test_dominance_bits_all_m(m):
 def test_ranks_across_the_switch_to_the_order_based_matrix(n, m):
     """Populations just below and above the size at which the matrix comes from the per-objective orders (and 65536
     rows, where the padded column length steps off a multiple of 4096): same ranks and same selection whichever
-    kernel builds the matrix."""
+    kernel builds the matrix, and both the ranks and the selection of the plain-C checker."""
+    from oracle import c_oracle
+
     say("switch", n, m)
     g = torch.Generator("cpu").manual_seed(n + m)
-    f = (torch.randint(0, 1 << 12, (n, m), generator=g).float() / 64).to(DEV)  # ties in every objective
+    f_cpu = torch.randint(0, 1 << 12, (n, m), generator=g).float() / 64  # ties in every objective
+    f = f_cpu.to(DEV)
     x = torch.arange(n, dtype=torch.int32, device=DEV)[:, None]
     try:
         got_rank = non_dominate_rank(f)
         got = nd_environmental_selection(x, f, n // 2)
+        order, rank, dist, _ = c_oracle.select(as_np(f_cpu), n // 2)
+        assert np.array_equal(as_np(got_rank), rank)
+        assert np.array_equal(as_np(got[0])[:, 0].astype(np.int64), order)
+        assert np.array_equal(as_np(got[2]), rank[order])
+        assert_dist_close(got[3], dist[order])
         runtime.set_option("prefix_min_rows", 0)
         assert torch.equal(got_rank, non_dominate_rank(f))
         want = nd_environmental_selection(x, f, n // 2)
@@ -537,6 +545,29 @@ def test_selection_c4_first8_vmap():
         assert np.array_equal(as_np(rs[b]), g["rank"][b][order])
         assert_dist_close(ds[b], g["dist"][b][order])
         assert np.array_equal(as_np(fs[b]), as_np(w.f[b])[order])
+
+
+def test_c4_every_population_against_the_cpu_side():
+    """All 1024 populations of the batched configuration in one call: the ranks of every population against the
+    batched restatement of the reference's loop, and every population's selection against the plain-C checker."""
+    from oracle import c_oracle
+
+    say("c4_every_population")
+    w = workloads.c4()
+    fd = w.f.to(DEV)
+    xd = torch.arange(512, dtype=torch.int32, device=DEV)[None, :, None].expand(1024, 512, 1).contiguous()
+    ranks = as_np(non_dominate_rank(fd))
+    xs, fs, rs, ds = (as_np(t) for t in nd_environmental_selection(xd, fd, w.topk))
+    for lo in range(0, 1024, 64):  # (64 populations: 50 MB for each of the restatement's (B, N, N, M) temporaries)
+        assert np.array_equal(ranks[lo: lo + 64], as_np(er.ranks_by_peeling_batched(w.f[lo: lo + 64]))), lo
+    f_np = as_np(w.f)
+    for b in range(1024):
+        order, rank, dist, _ = c_oracle.select(f_np[b], w.topk)
+        assert np.array_equal(rank, ranks[b]), b
+        assert np.array_equal(xs[b][:, 0].astype(np.int64), order), b
+        assert np.array_equal(rs[b], rank[order]), b
+        assert_dist_close(ds[b], dist[order], f"population {b}")
+        assert np.array_equal(fs[b], f_np[b][order]), b
 
 
 def test_c4_full_batch_one_launch():
