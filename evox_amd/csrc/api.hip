@@ -821,6 +821,18 @@ int evox_hip_workspace_layout(int64_t n, int64_t m, int64_t* out) {
   return 0;
 }
 
+int evox_hip_slot_sort_layout(int64_t n, int64_t m, int64_t* out) {
+  Layout L;
+  if (out == nullptr || !make_layout(n, m, &L)) return kErrBadArg;
+  out[0] = (int64_t)L.key_sorted;
+  out[1] = (int64_t)L.kid_sorted;
+  out[2] = (int64_t)L.xs_sorted;
+  out[3] = (int64_t)L.xs;
+  out[4] = L.npad;
+  out[5] = (int64_t)L.slot_of;
+  return 0;
+}
+
 int evox_hip_set_option(const char* name, int64_t value) {
   if (name == nullptr) return kErrBadArg;
   if (!strcmp(name, "peel_blocks_per_cu") && value >= 1 && value <= 16) {

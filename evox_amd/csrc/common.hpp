@@ -27,6 +27,77 @@ __device__ inline uint32_t ordered_key(float v) {
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+// Maximum, minimum and sum over the sixteen lanes of a group (lanes 16 g .. 16 g + 15), the same in every lane of
+// the group: four rotations inside the DPP row (row_ror 8, 4, 2, 1), no trip through the LDS permute unit.
+__device__ inline unsigned long long row16_rotate(unsigned long long v, int ctrl_index) {
+  unsigned lo = (unsigned)v, hi = (unsigned)(v >> 32);
+  switch (ctrl_index) {  // (the DPP control is an immediate)
+    case 8:
+      lo = __builtin_amdgcn_update_dpp(0, lo, 0x128, 0xf, 0xf, false);
+      hi = __builtin_amdgcn_update_dpp(0, hi, 0x128, 0xf, 0xf, false);
+      break;
+    case 4:
+      lo = __builtin_amdgcn_update_dpp(0, lo, 0x124, 0xf, 0xf, false);
+      hi = __builtin_amdgcn_update_dpp(0, hi, 0x124, 0xf, 0xf, false);
+      break;
+    case 2:
+      lo = __builtin_amdgcn_update_dpp(0, lo, 0x122, 0xf, 0xf, false);
+      hi = __builtin_amdgcn_update_dpp(0, hi, 0x122, 0xf, 0xf, false);
+      break;
+    default:
+      lo = __builtin_amdgcn_update_dpp(0, lo, 0x121, 0xf, 0xf, false);
+      hi = __builtin_amdgcn_update_dpp(0, hi, 0x121, 0xf, 0xf, false);
+      break;
+  }
+  return ((unsigned long long)hi << 32) | lo;
+}
+__device__ inline unsigned long long group16_max(unsigned long long v) {
+#pragma unroll
+  for (int r = 8; r >= 1; r >>= 1) {
+    const unsigned long long o = row16_rotate(v, r);
+    v = o > v ? o : v;
+  }
+  return v;
+}
+__device__ inline unsigned long long group16_min(unsigned long long v) {
+#pragma unroll
+  for (int r = 8; r >= 1; r >>= 1) {
+    const unsigned long long o = row16_rotate(v, r);
+    v = o < v ? o : v;
+  }
+  return v;
+}
+__device__ inline int group16_sum(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x124, 0xf, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x122, 0xf, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x121, 0xf, 0xf, false);
+  return v;
+}
+// Relaxed agent-scope accesses: one location at a time, coherent across the whole device, without
+// the cache-wide write-back / invalidate that an agent-scope fence costs.  Everything that one
+// block writes and another block reads during the kernel (front bitmaps, front sizes, barrier
+// flags) is accessed only through these or through atomics.
+template <class T>
+__device__ inline T coherent_load(const T* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <class T>
+__device__ inline void coherent_store(T* p, T v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// A wait on another workgroup that always ends: false when `spin_limit` polls were not enough.
+template <class Pred>
+__device__ inline bool bounded_wait(Pred done, unsigned spin_limit) {
+  unsigned spins = 0;
+  while (!done()) {
+    if (++spins > spin_limit) return false;
+    __builtin_amdgcn_s_sleep(1);
+  }
+  return true;
+}
+
 // Device control block shared by the peel / crowding / selection kernels of one call.
 struct Ctrl {
   int err;          // 0, or kErrBarrierTimeout when a bounded grid-barrier wait ran out
@@ -39,7 +110,8 @@ struct Ctrl {
   int listed;       // front bitmaps 0 .. listed-1 have been listed and cleared; polled by the barrier master
   int radix_epoch;  // runs of a radix sort kernel so far: each takes a fresh range of barrier generations
   int tail_done;    // the peel kernel has also left the crowding distances and the order of the last front
-  int reserved[6];  // [0], [1]: arrival counters of the barriers inside the kernels that order the last front
+  int reserved[6];  // [0], [1]: arrival counters of the barriers inside the kernels that order the last front;
+                    // [2]: that of the barriers inside the slot sort
   // grid barrier: block 0 publishes (generation << 32 | rows found by all blocks) in `release` and in
   // kReleaseCopies copies of it, one per 128-byte line, so that the waiting blocks do not all poll one
   // address; all-ones means "give up" (a bounded wait ran out).  Every other block publishes

@@ -102,53 +102,6 @@ __device__ inline int wave_max(int v) {
   return __builtin_amdgcn_readlane(v, 63);
 }
 
-// Maximum, minimum and sum over the sixteen lanes of a group (lanes 16 g .. 16 g + 15), the same in every lane of
-// the group: four rotations inside the DPP row (row_ror 8, 4, 2, 1), no trip through the LDS permute unit.
-__device__ inline unsigned long long row16_rotate(unsigned long long v, int ctrl_index) {
-  unsigned lo = (unsigned)v, hi = (unsigned)(v >> 32);
-  switch (ctrl_index) {  // (the DPP control is an immediate)
-    case 8:
-      lo = __builtin_amdgcn_update_dpp(0, lo, 0x128, 0xf, 0xf, false);
-      hi = __builtin_amdgcn_update_dpp(0, hi, 0x128, 0xf, 0xf, false);
-      break;
-    case 4:
-      lo = __builtin_amdgcn_update_dpp(0, lo, 0x124, 0xf, 0xf, false);
-      hi = __builtin_amdgcn_update_dpp(0, hi, 0x124, 0xf, 0xf, false);
-      break;
-    case 2:
-      lo = __builtin_amdgcn_update_dpp(0, lo, 0x122, 0xf, 0xf, false);
-      hi = __builtin_amdgcn_update_dpp(0, hi, 0x122, 0xf, 0xf, false);
-      break;
-    default:
-      lo = __builtin_amdgcn_update_dpp(0, lo, 0x121, 0xf, 0xf, false);
-      hi = __builtin_amdgcn_update_dpp(0, hi, 0x121, 0xf, 0xf, false);
-      break;
-  }
-  return ((unsigned long long)hi << 32) | lo;
-}
-__device__ inline unsigned long long group16_max(unsigned long long v) {
-#pragma unroll
-  for (int r = 8; r >= 1; r >>= 1) {
-    const unsigned long long o = row16_rotate(v, r);
-    v = o > v ? o : v;
-  }
-  return v;
-}
-__device__ inline unsigned long long group16_min(unsigned long long v) {
-#pragma unroll
-  for (int r = 8; r >= 1; r >>= 1) {
-    const unsigned long long o = row16_rotate(v, r);
-    v = o < v ? o : v;
-  }
-  return v;
-}
-__device__ inline int group16_sum(int v) {
-  v += __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false);
-  v += __builtin_amdgcn_update_dpp(0, v, 0x124, 0xf, 0xf, false);
-  v += __builtin_amdgcn_update_dpp(0, v, 0x122, 0xf, 0xf, false);
-  v += __builtin_amdgcn_update_dpp(0, v, 0x121, 0xf, 0xf, false);
-  return v;
-}
 // The cost behind an ordered_key (common.hpp): zero comes back as +0.0, every NaN as the canonical one.
 __device__ inline float cost_of_key(uint32_t key) {
   if (key == 0xFFFFFFFFu) return __uint_as_float(0x7FC00000u);
@@ -308,19 +261,6 @@ __global__ __launch_bounds__(256) void count_from_totals_kernel(const int* __res
 
 // ------------------------------------------------------------ grid barrier
 
-// Relaxed agent-scope accesses: one location at a time, coherent across the whole device, without
-// the cache-wide write-back / invalidate that an agent-scope fence costs.  Everything that one
-// block writes and another block reads during the kernel (front bitmaps, front sizes, barrier
-// flags) is accessed only through these or through atomics.
-template <class T>
-__device__ inline T coherent_load(const T* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-template <class T>
-__device__ inline void coherent_store(T* p, T v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // Grid synchronisation with three roles, all through flag words and bounded polling:
 //   block 0 ("master")   waits for the tally of every sweeping block, adds them up and publishes
 //                        (generation << 32 | total) in `release`: one round trip both synchronises the
@@ -338,16 +278,6 @@ constexpr int kFirstSweeper = 2;
 constexpr int kSharedListingRows = 8192;   // a final front 0 of more rows is listed by many blocks
 constexpr int kSharedListingBlocks = 64;
 constexpr int kFrontBuffers = 8;  // front bitmaps in rotation: the lister may lag the sweepers by 6 fronts
-
-template <class Pred>
-__device__ inline bool bounded_wait(Pred done, unsigned spin_limit) {
-  unsigned spins = 0;
-  while (!done()) {
-    if (++spins > spin_limit) return false;
-    __builtin_amdgcn_s_sleep(1);
-  }
-  return true;
-}
 
 // Sweeper side.  Returns false after a timeout (here or elsewhere); *total_out = size of the new front.
 __device__ inline bool sweeper_barrier(Ctrl* ctrl, unsigned gen, int block_tally, int* total_out, unsigned spin_limit,

@@ -140,7 +140,15 @@ def workspace_views(ws: torch.Tensor, n: int, m: int) -> dict:
         size = torch.empty((), dtype=dtype).element_size()
         return ws[off: off + count_ * size].view(dtype)
 
+    sort = (ctypes.c_int64 * 6)()
+    _lib.call("evox_hip_slot_sort_layout", n, m, sort)
+    npad = sort[4]
     return {
+        "key_sorted": view(sort[0], npad, torch.int64),
+        "kid_sorted": view(sort[1], npad, torch.int32),
+        "xs_sorted": view(sort[2], m * npad, torch.float32).view(m, npad),
+        "xs": view(sort[3], m * npad, torch.float32).view(m, npad),
+        "slot_of": view(sort[5], n, torch.int32),
         "dom": view(dom_off, n * wstride, torch.int64).view(n, wstride),
         "nwords": nwords,
         "count": view(count, n, torch.int32),
@@ -151,4 +159,5 @@ def workspace_views(ws: torch.Tensor, n: int, m: int) -> dict:
         "order": view(order, n, torch.int32),
         "ctrl": view(ctrl, 16, torch.int32),
         "orig_of": view(orig_of, n, torch.int32),
+        "orig_of_padded": view(orig_of, npad, torch.int32),
     }

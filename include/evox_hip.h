@@ -231,6 +231,12 @@ int evox_hip_stage_order(int64_t n, int64_t m, void* workspace, size_t workspace
  * dominates the row in slot s.  Ranks, distances, listings and the order use original row indices. */
 int evox_hip_workspace_layout(int64_t n, int64_t m, int64_t* out11);
 
+/* Byte offsets of what the slot sort leaves, for tests: out[0] row keys by slot (uint64, out[4] entries: all-ones behind
+ * the n-th), out[1] first slot that holds the same key (uint32, out[4] entries), out[2] fitness by slot as a structure of
+ * arrays (float32, objective k at + k * out[4]; NaN behind the n-th row), out[3] fitness by original index, same shape,
+ * out[4] padded row count, out[5] original row index -> slot (int32 n; written for populations of more than 4096 rows). */
+int evox_hip_slot_sort_layout(int64_t n, int64_t m, int64_t* out6);
+
 /* How a population of this shape is peeled, for tools and benchmarks: out[0] = 1 when every sweeping workgroup keeps
  * its rows of the bit matrix in LDS (the matrix fits the LDS of the device; counts and peeling are then one kernel),
  * 0 when rows are rescanned in memory; out[1] = sweeping workgroups of that kernel, out[2] = bytes of LDS of each
