@@ -42,8 +42,8 @@ def _order_preserving_f32(t: torch.Tensor, what: str) -> torch.Tensor:
 
     Dominance only looks at the order of the values within one objective, so fitness of a dtype that
     the kernels do not read (float64, integers) is replaced, objective by objective, by the dense rank
-    of each value among the values of that objective (``torch.unique`` on the device: equal values get
-    equal ranks, -0.0 and 0.0 tie, NaN stays NaN).  Dense ranks below 2**24 are exact in float32.
+    of each value among the values of that objective (a sort on the device: equal values get equal
+    ranks, -0.0 and 0.0 tie, NaN stays NaN).  Dense ranks below 2**24 are exact in float32.
     Used for ranking only: crowding distances depend on the values themselves.
     """
     if t.dtype in (torch.float32, torch.float16, torch.bfloat16):
@@ -52,16 +52,17 @@ def _order_preserving_f32(t: torch.Tensor, what: str) -> torch.Tensor:
         raise TypeError(f"{what} must be a real numeric tensor; got {t.dtype}")
     if t.shape[-2] >= 2**24:
         raise ValueError(f"{what} of dtype {t.dtype} is limited to 2**24 rows per population")
+    # one sort per objective column, all columns and populations in the same calls: in sorted order a value opens
+    # a new rank when it differs from the value before it (-0.0 == 0.0; NaN, sorted last, is put back below)
     flat = t.reshape(-1, t.shape[-2], t.shape[-1])
-    out = torch.empty(flat.shape, dtype=torch.float32, device=t.device)
-    for b in range(flat.size(0)):
-        for k in range(flat.size(2)):
-            col = flat[b, :, k]
-            dense = torch.unique(col, sorted=True, return_inverse=True)[1].to(torch.float32)
-            if col.is_floating_point():
-                dense = torch.where(torch.isnan(col), torch.full_like(dense, float("nan")), dense)
-            out[b, :, k] = dense
-    return out.reshape(t.shape)
+    values, index = torch.sort(flat, dim=1)
+    opens = torch.zeros(flat.shape, dtype=torch.int64, device=t.device)
+    opens[:, 1:, :] = (values[:, 1:, :] != values[:, :-1, :]).to(torch.int64)
+    dense = torch.empty(flat.shape, dtype=torch.float32, device=t.device)
+    dense.scatter_(1, index, opens.cumsum(dim=1).to(torch.float32))
+    if flat.is_floating_point():
+        dense = torch.where(torch.isnan(flat), torch.full_like(dense, float("nan")), dense)
+    return dense.reshape(t.shape)
 
 
 def _rank_one(f: torch.Tensor, out: torch.Tensor) -> None:
