@@ -265,8 +265,7 @@ def sweep_pass_bandwidth(dev, n, m):
     ws = runtime.workspace(n, m, dev)
     s = runtime.stream_handle(dev)
     tail = (ws.data_ptr(), ws.numel(), s)
-    runtime.set_option("peel_witness", 0)
-    try:
+    with runtime.options(peel_witness=0):
         _lib.call("evox_hip_stage_prepare", f.data_ptr(), n, m, f.stride(0), f.stride(1), *tail)
         _lib.call("evox_hip_stage_dominance", n, m, 0, *tail)
         _lib.call("evox_hip_stage_count", n, m, *tail)
@@ -291,9 +290,7 @@ def sweep_pass_bandwidth(dev, n, m):
         slot_of = torch.empty(n, dtype=torch.int64, device=dev)
         slot_of[views["orig_of"].long()] = torch.arange(n, device=dev)
         read = int(((((slot_of >> 6) + 2) & ~1) * 8)[views["rank"] >= 1].sum())
-    finally:
-        runtime.set_option("peel_witness", 1)
-        runtime.release_workspaces()
+    runtime.release_workspaces()
     gbs = read / max(t_one - t_none, 1e-9) / 1e3
     return {"pass_us": t_one - t_none, "kernel_us_with_no_pass": t_none, "bytes": read, "bound": "hbm", "achieved": gbs,
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS}

@@ -68,6 +68,10 @@ _SIGNATURES = {
     "evox_hip_peel_plan": (c_int, [c_int64, c_int64, c_void_p]),
     "evox_hip_read_status": (c_int, [c_void_p, c_void_p, c_void_p]),
     "evox_hip_set_option": (c_int, [c_char_p, c_int64]),
+    "evox_hip_options_create": (c_void_p, []),
+    "evox_hip_options_destroy": (None, [c_void_p]),
+    "evox_hip_options_set": (c_int, [c_void_p, c_char_p, c_int64]),
+    "evox_hip_options_use": (c_int, [c_void_p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

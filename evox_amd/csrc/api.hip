@@ -4,6 +4,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <new>
 
 #include "../../include/evox_hip.h"
 #include "batched.hpp"
@@ -47,6 +48,10 @@ struct Options {
   int prefix_bands = 1;  // stretches of the order-based matrix: 1 = bands of rows counted from row 0, 0 = from each tile's diagonal
 };
 static Options g_opt;
+// The tunables that calls made from this thread use: those handed to evox_hip_options_use, else the process-wide ones.
+static thread_local const Options* t_opt = nullptr;
+static inline const Options& opt() { return t_opt != nullptr ? *t_opt : g_opt; }
+
 
 struct Layout {
   int n, m, npad, nwords, kstride, buckets, prep_blocks;
@@ -242,7 +247,7 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
   const Layout& L = w.L;
   if (src.f == nullptr || src.f2 == nullptr || src.n_first < 0 || src.n_first > L.n) return kErrBadArg;
   const int64_t zero_words = (int64_t)((L.zero_end - L.ctrl) / 4);
-  if (with_sort && L.n <= kSmallSortRows && L.m <= kSmallSortObjectives && (int64_t)L.n * L.m <= kSmallSortValues && g_opt.small_sort) {
+  if (with_sort && L.n <= kSmallSortRows && L.m <= kSmallSortObjectives && (int64_t)L.n * L.m <= kSmallSortValues && opt().small_sort) {
     hipLaunchKernelGGL(small_sort_kernel, dim3(L.npad / kSmallSortGroup), dim3(kSmallSortThreads), sizeof(double) * (size_t)L.npad, s, src.f,
                        src.sr, src.sc, (int)src.n_first, src.f2, src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs),
                        w.at<SortParam>(L.sortparam), w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted),
@@ -281,11 +286,11 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
 // Measured (matrix from the orders against pairwise, us): 49152 x 8: 373 / 373; 65536 x 2: 239 / 227, x 3: 277 / 287,
 // x 4: 305 / 366, x 8: 451 / 637; 100000 x 2: 370 / 558, x 3: 408 / 709; 200000 x 3: 1268 / 2622, x 8: 1624 / 5340.
 static bool prefix_dominance_applies(const Layout& L) {
-  if (g_opt.prefix_min_rows <= 0 || L.m < 2 || L.m > kPrefixMaxObjectives) return false;
+  if (opt().prefix_min_rows <= 0 || L.m < 2 || L.m > kPrefixMaxObjectives) return false;
   // (two objectives are cheap pair by pair: a quarter more rows before the orders pay; nine or more are dear: a
   // quarter fewer -- 49152 x 9: 419 / 563, x 16: 675 / 933; 32768 x 9: 365 / 271, x 16: 622 / 464)
-  const int64_t q = g_opt.prefix_min_rows / 4;
-  const int64_t least = L.m == 2 ? g_opt.prefix_min_rows + q : (L.m >= 9 ? g_opt.prefix_min_rows - q : g_opt.prefix_min_rows);
+  const int64_t q = opt().prefix_min_rows / 4;
+  const int64_t least = L.m == 2 ? opt().prefix_min_rows + q : (L.m >= 9 ? opt().prefix_min_rows - q : opt().prefix_min_rows);
   return L.n >= least && L.n > kRadixMinCandidates && L.n <= kPrefixMaxRows;
 }
 static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s);
@@ -296,7 +301,7 @@ static int stage_dominance(const Ws& w, int variant, hipStream_t s) {
   if (variant == kDomAuto && prefix_dominance_applies(w.L)) return stage_dominance_prefix(w, false, s);
   // (the lower triangle in tiles of 4 words keeps every SIMD busy with several waves; 16 is kept for
   // measurements)
-  const int tile = g_opt.dominance_tile_words;
+  const int tile = opt().dominance_tile_words;
   if (tile >= 16)
     launch_dominance<16>(w, variant, s);
   else if (tile >= 8)
@@ -365,7 +370,7 @@ static int grant_dynamic_lds(const void* kernel, size_t lds) {
 // population does not fit (or the option is off).  Every workgroup takes a compute unit of its own.
 constexpr size_t kLdsPeelBudget = 160 * 1024 - 512;
 static int lds_peel_plan(const Layout& L, size_t* lds_out) {
-  if (!g_opt.peel_lds || L.n > 32768 || L.nwords > kLdsPeelThreads) return 0;  // (the lister keeps original indices in 16 bits and takes a bitmap word per thread)
+  if (!opt().peel_lds || L.n > 32768 || L.nwords > kLdsPeelThreads) return 0;  // (the lister keeps original indices in 16 bits and takes a bitmap word per thread)
   const int most = device_cus() - 1 < 255 ? device_cus() - 1 : 255;  // + the lister; a record holds at least 4 units
   if (most < 8) return 0;
   auto fits = [&](int sweepers) {
@@ -373,7 +378,7 @@ static int lds_peel_plan(const Layout& L, size_t* lds_out) {
     return b != 0 && b <= kLdsPeelBudget;
   };
   if (!fits(most)) return 0;
-  int sweepers = g_opt.peel_lds_blocks;
+  int sweepers = opt().peel_lds_blocks;
   if (sweepers == 0) {
     // by size: about 64 rows per workgroup, at least 32 workgroups
     sweepers = L.n / 64 < 32 ? 32 : L.n / 64;
@@ -396,7 +401,7 @@ static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool
   tail.dist = w.at<float>(L.dist);
   tail.order = w.at<int>(L.order);
   tail.buffer = w.at<unsigned long long>(L.tailbuf);
-  if (order_last_front && g_opt.peel_tail) {
+  if (order_last_front && opt().peel_tail) {
     // a small last front is ordered by the peel kernel itself; its LDS must hold the candidates
     const size_t need = peel_tail_lds_bytes(L.n, L.m);
     if (need != 0 && need <= kLdsPeelBudget) {
@@ -422,7 +427,7 @@ static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool
   hipLaunchKernelGGL(peel_lds_kernel, dim3(sweepers + 1), dim3(kLdsPeelThreads), lds, s, w.at<uint64_t>(L.dom), L.wstride, L.nwords, L.n,
                      w.at<int>(L.orig_of), w.at<int>(L.rank), fill_dist ? w.at<float>(L.dist) : (float*)nullptr,
                      w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
-                     want_perm ? w.at<int>(L.perm) : (int*)nullptr, w.at<int>(L.fstart), w.ctrl(), (int)stop_count, g_opt.spin_limit,
+                     want_perm ? w.at<int>(L.perm) : (int*)nullptr, w.at<int>(L.fstart), w.ctrl(), (int)stop_count, opt().spin_limit,
                      w.at<unsigned long long>(L.records), sweepers, tail);
   EVX_LAUNCH_CHECK();
   return 0;
@@ -438,7 +443,7 @@ static int count_and_peel(const Ws& w, int64_t stop_count, bool want_perm, bool 
   if (may_have_ordered) *may_have_ordered = false;
   if (const int sweepers = lds_peel_plan(w.L, &lds)) {
     if (may_have_ordered)
-      *may_have_ordered = order_last_front && g_opt.peel_tail && peel_tail_lds_bytes(w.L.n, w.L.m) != 0 &&
+      *may_have_ordered = order_last_front && opt().peel_tail && peel_tail_lds_bytes(w.L.n, w.L.m) != 0 &&
                           peel_tail_lds_bytes(w.L.n, w.L.m) <= kLdsPeelBudget;
     return launch_lds_peel(w, stop_count, want_perm, fill_dist, sweepers, lds, s, order_last_front);
   }
@@ -455,7 +460,7 @@ static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream
   // The grid never exceeds what the device holds at once (the blocks wait for one another).
   auto grid_for = [&](size_t lds, int* err) -> int {
     int per_cu = peel_blocks_per_cu(lds, err);
-    if (per_cu > g_opt.peel_blocks_per_cu) per_cu = g_opt.peel_blocks_per_cu;
+    if (per_cu > opt().peel_blocks_per_cu) per_cu = opt().peel_blocks_per_cu;
     int64_t blocks = (int64_t)cus * per_cu;
     if (blocks > kMaxGrid) blocks = kMaxGrid;
     const int64_t wpb = kPeelThreads / 64;
@@ -465,7 +470,7 @@ static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream
   // The witness pass keeps two bitmaps in LDS and at most kWitnessChunks * 64 rows per sweeping
   // wave; populations too large for that use the sweep pass.
   int err = 0;
-  int use_witness = g_opt.peel_witness && 2 * bitmap <= lds_limit;
+  int use_witness = opt().peel_witness && 2 * bitmap <= lds_limit;
   int blocks = 0;
   if (use_witness) {
     blocks = grid_for(2 * bitmap, &err);
@@ -479,12 +484,12 @@ static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream
     if (err) return err;
   }
   if (blocks <= kFirstSweeper) return kErrBadArg;
-  if (use_witness && g_opt.peel_records && L.n <= kRecordsMaxRowsWide) {
+  if (use_witness && opt().peel_records && L.n <= kRecordsMaxRowsWide) {
     // all-to-all records: 1 lister + a power of two of sweeping blocks, all resident at once
     // by size: 64 blocks up to 32768 rows, 128 above (measured at 20000 rows: 221 us per selection with 64
     // blocks, 225 with 128, 228 with 32, 238 with 192; between 1200 and 6000 rows the count hardly matters)
     const int by_size = L.n <= 32768 ? 64 : 128;
-    const int sweepers = cus >= 64 ? (g_opt.peel_record_blocks ? g_opt.peel_record_blocks : by_size) : 16;
+    const int sweepers = cus >= 64 ? (opt().peel_record_blocks ? opt().peel_record_blocks : by_size) : 16;
     const int wpb = kRecThreads / 64;
     const int list_capacity = wpb * ((L.n + sweepers * wpb - 1) / (sweepers * wpb));
     const size_t rec_lds = bitmap + 24 * (size_t)list_capacity;  // queue (8 + 4 + 4) and ranked pairs (2 x 4) per row
@@ -503,7 +508,7 @@ static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream
     hipLaunchKernelGGL(wide ? peel_records_kernel<true> : peel_records_kernel<false>, dim3(sweepers + 1), dim3(kRecThreads), rec_lds, s, w.at<uint64_t>(L.dom), L.wstride,
                        L.nwords, L.n, w.at<int>(L.orig_of), w.at<int>(L.rank), w.at<uint64_t>(L.fronts_slot),
                        w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize), want_perm ? w.at<int>(L.perm) : (int*)nullptr,
-                       w.at<int>(L.fstart), w.ctrl(), (int)stop_count, g_opt.spin_limit, w.at<int>(L.witness),
+                       w.at<int>(L.fstart), w.ctrl(), (int)stop_count, opt().spin_limit, w.at<int>(L.witness),
                        w.at<unsigned long long>(L.records), sweepers, list_capacity);
     EVX_LAUNCH_CHECK();
     return 0;
@@ -514,7 +519,7 @@ static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream
                      L.n, w.at<int>(L.orig_of), w.at<int>(L.count), w.at<int>(L.rank), w.at<uint64_t>(L.fronts_slot),
                      w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
                      want_perm ? w.at<int>(L.perm) : (int*)nullptr, w.at<int>(L.fstart), w.ctrl(), (int)stop_count,
-                     g_opt.spin_limit, w.at<int>(L.witness), use_witness);
+                     opt().spin_limit, w.at<int>(L.witness), use_witness);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -567,7 +572,7 @@ static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
   const Layout& L = w.L;
   const int shift = prefix_bucket_shift(L.n);
   const int buckets = ((L.n - 1) >> shift) + 1;
-  const int bands_wanted = g_opt.prefix_bands;
+  const int bands_wanted = opt().prefix_bands;
   // bands of rows shared by all tiles (their stores then fall into the same rows at about the same time) pay from
   // about 100 000 rows on: 200 000 x 8 1203 -> 1156 us, 100 000 x 8 441 -> 424, but 65536 x 3 181 -> 190
   const int bands = bands_wanted != 0 && L.n >= 98304 ? 1 : 0;
@@ -580,12 +585,12 @@ static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
     const int tiles = (int)round_up((L.nwords + WW * tt - 1) / (WW * tt), 128 / (WW * tt));
     hipLaunchKernelGGL(kernel, dim3(tiles, stretches), dim3(kPrefixThreads), lds, s, w.at<int>(L.pos), w.at<int>(L.scost),
                        w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.kstride, L.wstride, L.nwords, shift, buckets,
-                       chunk, bands, g_opt.prefix_mode, w.at<int>(L.total0), w.at<int>(L.witness0), w.at<SortParam>(L.sortparam));
+                       chunk, bands, opt().prefix_mode, w.at<int>(L.total0), w.at<int>(L.witness0), w.at<SortParam>(L.sortparam));
     EVX_LAUNCH_CHECK();
     return 0;
   };
   // (200 000 x 3: 957 -> 769 us, x 4: 972 -> 797; 100 000 x 3: 319 -> 317; 65536 x 3: 184 -> 220: half as many workgroups)
-  if (TT == 2 && g_opt.prefix_double_tile > 0 && L.n >= g_opt.prefix_double_tile) {
+  if (TT == 2 && opt().prefix_double_tile > 0 && L.n >= opt().prefix_double_tile) {
     if (int e = launch(dominance_prefix_kernel<M, WW, TT>, TT)) return e;
   } else {
     if (int e = launch(dominance_prefix_kernel<M, WW, 1>, 1)) return e;
@@ -611,7 +616,7 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) 
   if (workers + kFirstSweeper < radix_grid(L)) workers = radix_grid(L) - kFirstSweeper;
   hipLaunchKernelGGL(objective_order_kernel, dim3(workers + kFirstSweeper), dim3(kRadixThreads), lds, s, w.at<float>(L.xs), L.npad, L.n,
                      L.m, w.at<int>(L.slot_of), w.at<SortParam>(L.sortparam), w.ctrl(), w.at<int>(L.pos), w.at<int>(L.scost), w.at<int>(L.total0),
-                     w.at<int>(L.witness0), radix_buffers(w), g_opt.spin_limit);
+                     w.at<int>(L.witness0), radix_buffers(w), opt().spin_limit);
   EVX_LAUNCH_CHECK();
   // the barrier words of the control block restart from zero for the kernels that follow (the sort counted its
   // generations from a high base)
@@ -655,7 +660,7 @@ static CrowdArgs crowd_args(const Ws& w, const int* list, bool use_orders, int f
   a.pos = w.at<int>(L.pos);
   a.sorted_cost = w.at<float>(L.scost);
   a.buf = radix_buffers(w);
-  a.spin_limit = g_opt.spin_limit;
+  a.spin_limit = opt().spin_limit;
   a.param = w.at<SortParam>(L.sortparam);
   a.use_orders = use_orders ? 1 : 0;
   a.fused = fused;
@@ -833,41 +838,67 @@ int evox_hip_slot_sort_layout(int64_t n, int64_t m, int64_t* out) {
   return 0;
 }
 
-int evox_hip_set_option(const char* name, int64_t value) {
+static int set_named(Options& o, const char* name, int64_t value) {
   if (name == nullptr) return kErrBadArg;
   if (!strcmp(name, "peel_blocks_per_cu") && value >= 1 && value <= 16) {
-    g_opt.peel_blocks_per_cu = (int)value;
+    o.peel_blocks_per_cu = (int)value;
   } else if (!strcmp(name, "peel_witness") && (value == 0 || value == 1)) {
-    g_opt.peel_witness = (int)value;
+    o.peel_witness = (int)value;
   } else if (!strcmp(name, "peel_record_blocks") && (value == 0 || (value >= 16 && value <= 255))) {
-    g_opt.peel_record_blocks = (int)value;
+    o.peel_record_blocks = (int)value;
   } else if (!strcmp(name, "peel_records") && (value == 0 || value == 1)) {
-    g_opt.peel_records = (int)value;
+    o.peel_records = (int)value;
   } else if (!strcmp(name, "peel_lds") && (value == 0 || value == 1)) {
-    g_opt.peel_lds = (int)value;
+    o.peel_lds = (int)value;
   } else if (!strcmp(name, "tail_merged") && (value == 0 || value == 1)) {
-    g_opt.tail_merged = (int)value;
+    o.tail_merged = (int)value;
   } else if (!strcmp(name, "peel_tail") && (value == 0 || value == 1)) {
-    g_opt.peel_tail = (int)value;
+    o.peel_tail = (int)value;
   } else if (!strcmp(name, "peel_lds_blocks") && (value == 0 || (value >= 8 && value <= 255))) {
-    g_opt.peel_lds_blocks = (int)value;
+    o.peel_lds_blocks = (int)value;
   } else if (!strcmp(name, "spin_limit") && value >= 1 && value <= 0x7FFFFFFFll) {
-    g_opt.spin_limit = (unsigned)value;
+    o.spin_limit = (unsigned)value;
   } else if (!strcmp(name, "dominance_tile_words") && (value == 4 || value == 8 || value == 16)) {
-    g_opt.dominance_tile_words = (int)value;
+    o.dominance_tile_words = (int)value;
   } else if (!strcmp(name, "small_sort") && (value == 0 || value == 1)) {
-    g_opt.small_sort = (int)value;
+    o.small_sort = (int)value;
   } else if (!strcmp(name, "prefix_min_rows") && value >= 0) {
-    g_opt.prefix_min_rows = value;
+    o.prefix_min_rows = value;
   } else if (!strcmp(name, "prefix_double_tile") && value >= 0) {
-    g_opt.prefix_double_tile = value;
+    o.prefix_double_tile = value;
   } else if (!strcmp(name, "prefix_mode") && value >= 1 && value <= 3) {
-    g_opt.prefix_mode = (int)value;
+    o.prefix_mode = (int)value;
   } else if (!strcmp(name, "prefix_bands") && (value == 0 || value == 1)) {
-    g_opt.prefix_bands = (int)value;
+    o.prefix_bands = (int)value;
   } else {
     return kErrBadArg;
   }
+  return 0;
+}
+
+int evox_hip_set_option(const char* name, int64_t value) { return set_named(g_opt, name, value); }
+
+struct evox_hip_options {
+  evx::Options values;
+};
+
+evox_hip_options* evox_hip_options_create(void) {
+  evox_hip_options* h = new (std::nothrow) evox_hip_options;
+  if (h != nullptr) h->values = g_opt;
+  return h;
+}
+
+void evox_hip_options_destroy(evox_hip_options* options) {
+  if (options != nullptr && t_opt == &options->values) t_opt = nullptr;
+  delete options;
+}
+
+int evox_hip_options_set(evox_hip_options* options, const char* name, int64_t value) {
+  return options == nullptr ? kErrBadArg : set_named(options->values, name, value);
+}
+
+int evox_hip_options_use(const evox_hip_options* options) {
+  t_opt = options == nullptr ? nullptr : &options->values;
   return 0;
 }
 
@@ -1054,7 +1085,7 @@ static int argsort_step(const void* key, int kind, int64_t stride, int64_t n, co
   if (workers > cap) workers = cap;
   if (workers < 1) workers = 1;
   hipLaunchKernelGGL(argsort_step_kernel, dim3(workers + kFirstSweeper), dim3(kRadixThreads), kRadixLdsBytes, s, key, kind,
-                     stride, L.n, prev_order, reinterpret_cast<Ctrl*>(base + L.ctrl), b, order_out, g_opt.spin_limit);
+                     stride, L.n, prev_order, reinterpret_cast<Ctrl*>(base + L.ctrl), b, order_out, opt().spin_limit);
   EVX_LAUNCH_CHECK();
   // (an order of -1 everywhere when one of the sort's grid barriers ran out)
   return copy_out(reinterpret_cast<const Ctrl*>(base + L.ctrl), order_out, nullptr, n, kPoisonIndex, s);
@@ -1186,7 +1217,7 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   // (crowd_kernel); with more objectives the last front is usually too large for the peel kernel, and the two
   // stages as kernels of their own, each on the grid that suits it, order it faster than the shared launch does
   // (20 000 x 5, a front of 2532 rows: 245 against 261 us per selection; 20 000 x 8, 7481 rows: 457 against 493).
-  const bool one_ordering_launch = peel_orders && g_opt.tail_merged && L.m <= 3;
+  const bool one_ordering_launch = peel_orders && opt().tail_merged && L.m <= 3;
   if (!one_ordering_launch) {
     if (int e = stage_crowd_sort(w, w.at<int>(L.perm), true, 2, s, peel_orders)) return e;
     if (int e = stage_crowd_finish(w, w.at<int>(L.perm), true, 2, s, peel_orders)) return e;

@@ -1,6 +1,8 @@
 """Host-side plumbing between torch tensors and the C ABI: workspaces, streams, status."""
 
+import contextlib
 import ctypes
+import threading
 import os
 from typing import Dict, Optional, Tuple
 
@@ -127,7 +129,41 @@ def last_status() -> dict:
 
 
 def set_option(name: str, value: int) -> None:
+    """Changes a process-wide tunable (configuration at start-up; see ``options`` for a scoped change)."""
     _lib.call("evox_hip_set_option", name.encode(), int(value))
+
+
+_options_in_use = threading.local()
+
+
+@contextlib.contextmanager
+def options(**tunables):
+    """Tunables for the library calls that this thread makes inside the ``with`` block (the process-wide ones,
+    with the given changes); other threads and the process-wide values are left alone."""
+    lib = _lib.lib()
+    handle = lib.evox_hip_options_create()
+    if not handle:
+        raise MemoryError("evox_hip_options_create")
+    stack = getattr(_options_in_use, "stack", None)
+    if stack is None:
+        stack = _options_in_use.stack = []
+    try:
+        if stack:  # start from the enclosing block's values, not from the process-wide ones
+            for name, value in stack[-1][1].items():
+                _lib.call("evox_hip_options_set", handle, name.encode(), int(value))
+        merged = dict(stack[-1][1]) if stack else {}
+        for name, value in tunables.items():
+            _lib.call("evox_hip_options_set", handle, name.encode(), int(value))
+            merged[name] = int(value)
+        stack.append((handle, merged))
+        _lib.call("evox_hip_options_use", handle)
+        try:
+            yield
+        finally:
+            stack.pop()
+            _lib.call("evox_hip_options_use", stack[-1][0] if stack else None)
+    finally:
+        lib.evox_hip_options_destroy(handle)
 
 
 def workspace_views(ws: torch.Tensor, n: int, m: int) -> dict:

@@ -260,6 +260,18 @@ int evox_hip_read_status(const void* workspace, void* stream, int32_t* host_out8
  * Returns EVOX_HIP_E_BAD_ARG for an unknown name or a value out of range. */
 int evox_hip_set_option(const char* name, int64_t value);
 
+/* The same tunables for the calls of one thread, without touching process-wide state: a set of tunables is created
+ * as a copy of the process-wide ones (NULL when memory runs out), changed by name like evox_hip_set_option, and
+ * handed to evox_hip_options_use, after which every call that THIS thread makes into the library reads its tunables
+ * from there, until the thread hands over another set or NULL (the process-wide ones again).  A set in use must
+ * outlive the calls that read it; destroying the set that the calling thread uses puts that thread back on the
+ * process-wide ones.  evox_hip_set_option remains for configuration at start-up. */
+typedef struct evox_hip_options evox_hip_options;
+evox_hip_options* evox_hip_options_create(void);
+void evox_hip_options_destroy(evox_hip_options* options);
+int evox_hip_options_set(evox_hip_options* options, const char* name, int64_t value);
+int evox_hip_options_use(const evox_hip_options* options);
+
 #ifdef __cplusplus
 }
 #endif

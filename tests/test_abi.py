@@ -89,3 +89,28 @@ def test_argument_validation_without_gpu(handle):
                                                                None, p, 64, None) == _lib.E_WORKSPACE
     assert handle.evox_hip_set_option(b"no_such_option", 1) == _lib.E_BAD_ARG
     assert handle.evox_hip_set_option(b"peel_blocks_per_cu", 2) == 0
+    # tunables for the calls of one thread: created from the process-wide ones, set by name, handed over and taken back
+    opts = handle.evox_hip_options_create()
+    assert opts
+    assert handle.evox_hip_options_set(opts, b"spin_limit", 5) == 0
+    assert handle.evox_hip_options_set(opts, b"spin_limit", 0) == _lib.E_BAD_ARG
+    assert handle.evox_hip_options_set(opts, b"no_such_option", 1) == _lib.E_BAD_ARG
+    assert handle.evox_hip_options_set(None, b"spin_limit", 5) == _lib.E_BAD_ARG
+    assert handle.evox_hip_options_use(opts) == 0 and handle.evox_hip_options_use(None) == 0
+    assert handle.evox_hip_options_use(opts) == 0
+    handle.evox_hip_options_destroy(opts)  # (the set in use: the thread falls back to the process-wide tunables)
+    handle.evox_hip_options_destroy(None)
+
+
+def test_scoped_options_nest_and_restore():
+    from evox_amd import runtime
+
+    with runtime.options(spin_limit=7):
+        with runtime.options(peel_witness=0):
+            assert [d for _, d in runtime._options_in_use.stack] == [{"spin_limit": 7}, {"spin_limit": 7, "peel_witness": 0}]
+        assert len(runtime._options_in_use.stack) == 1
+        with pytest.raises(_lib.EvoxHipError):
+            with runtime.options(no_such_option=1):
+                pass
+        assert len(runtime._options_in_use.stack) == 1
+    assert runtime._options_in_use.stack == []

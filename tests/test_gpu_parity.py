@@ -156,12 +156,11 @@ def test_ranks_across_the_switch_to_the_order_based_matrix(n, m):
         assert np.array_equal(as_np(got[0])[:, 0].astype(np.int64), order)
         assert np.array_equal(as_np(got[2]), rank[order])
         assert_dist_close(got[3], dist[order])
-        runtime.set_option("prefix_min_rows", 0)
-        assert torch.equal(got_rank, non_dominate_rank(f))
-        want = nd_environmental_selection(x, f, n // 2)
+        with runtime.options(prefix_min_rows=0):
+            assert torch.equal(got_rank, non_dominate_rank(f))
+            want = nd_environmental_selection(x, f, n // 2)
         assert all(torch.equal(a, b) for a, b in zip(got, want))
     finally:
-        runtime.set_option("prefix_min_rows", 65536)
         runtime.release_workspaces()
 
 
@@ -209,35 +208,29 @@ def test_matrix_from_objective_orders_equals_the_pairwise_matrix(m):
     nan[4000, m - 1] = float("inf")
     cases["nonfinite"] = nan
     cases["large"] = torch.rand(40000, m, generator=g)
-    try:
-        for name, f in cases.items():
-            say("prefix_matrix", m, name, tuple(f.shape))
-            want_state = {}
-            runtime.set_option("prefix_min_rows", 0)
+    for name, f in cases.items():
+        say("prefix_matrix", m, name, tuple(f.shape))
+        want_state = {}
+        with runtime.options(prefix_min_rows=0):
             want = _matrix_words(f.contiguous(), 0, want_state)
-            # up to four objectives also with both tiles of a 128-byte line in one workgroup (by default from 131072 rows on)
-            for double_from in (131072, 1) if m <= 4 else (131072,):
-                runtime.set_option("prefix_min_rows", 4097)  # (a quarter more rows with two objectives)
-                runtime.set_option("prefix_double_tile", double_from)
+        # up to four objectives also with both tiles of a 128-byte line in one workgroup (by default from 131072 rows on)
+        for double_from in (131072, 1) if m <= 4 else (131072,):
+            with runtime.options(prefix_min_rows=4097, prefix_double_tile=double_from):  # (a quarter more rows with two objectives)
                 got_state = {}
                 got = _matrix_words(f.contiguous(), 0, got_state)
-                assert np.array_equal(got, want), (m, name, double_from, int((got != want).sum()))
-                if double_from == 1:
-                    assert np.array_equal(got_state["count"], want_state["count"]), (m, name)
-            runtime.set_option("prefix_double_tile", 131072)
-            # the counts and front 0 that the count stage derives from what the order-based kernel left behind
-            assert np.array_equal(got_state["count"], want_state["count"]), (m, name)
-            assert np.array_equal(got_state["count"], np.bitwise_count(want).sum(axis=1)), (m, name)
-            assert np.array_equal(got_state["rank"], want_state["rank"]), (m, name)
-            if name in ("ties", "duplicates", "large"):  # and the whole ranking on top of them (the passes start from
-                fd = f.contiguous().to(DEV)              # the highest non-empty word of every row)
-                runtime.set_option("prefix_min_rows", 4097)
+            assert np.array_equal(got, want), (m, name, double_from, int((got != want).sum()))
+            if double_from == 1:
+                assert np.array_equal(got_state["count"], want_state["count"]), (m, name)
+        # the counts and front 0 that the count stage derives from what the order-based kernel left behind
+        assert np.array_equal(got_state["count"], want_state["count"]), (m, name)
+        assert np.array_equal(got_state["count"], np.bitwise_count(want).sum(axis=1)), (m, name)
+        assert np.array_equal(got_state["rank"], want_state["rank"]), (m, name)
+        if name in ("ties", "duplicates", "large"):  # and the whole ranking on top of them (the passes start from
+            fd = f.contiguous().to(DEV)              # the highest non-empty word of every row)
+            with runtime.options(prefix_min_rows=4097):
                 ranks = non_dominate_rank(fd)
-                runtime.set_option("prefix_min_rows", 0)
+            with runtime.options(prefix_min_rows=0):
                 assert torch.equal(ranks, non_dominate_rank(fd)), (m, name)
-    finally:
-        runtime.set_option("prefix_min_rows", 65536)
-        runtime.set_option("prefix_double_tile", 131072)
 
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 8, 11, 16])
@@ -315,9 +308,8 @@ def test_both_slot_sorts_on_small_and_mid_size_inputs(population_path):
     cases.append(("uniform-4097x2", workloads.uniform_population(4097, 2, 0, 22)[0]))
     cases.append(("wide-60x200", workloads.uniform_population(60, 200, 0, 23)[0]))   # keys near 2^40
     cases.append(("wide-40x300", workloads.uniform_population(40, 300, 0, 24)[0]))   # too wide for the one-kernel sort
-    try:
-        for small_sort in (0, 1):
-            runtime.set_option("small_sort", small_sort)
+    for small_sort in (0, 1):
+        with runtime.options(small_sort=small_sort):
             for name, f in cases:
                 want = er.ranks_by_peeling(f)
                 assert np.array_equal(as_np(non_dominate_rank(f.to(DEV))), as_np(want)), (small_sort, name)
@@ -330,8 +322,6 @@ def test_both_slot_sorts_on_small_and_mid_size_inputs(population_path):
                     got = nd_environmental_selection_two_part(f[:h].to(DEV), f[:h].to(DEV), f[h:].to(DEV), f[h:].to(DEV), topk)
                     assert np.array_equal(as_np(got[0]), as_np(f)[as_np(order)], equal_nan=True), (small_sort, name)
                     assert np.array_equal(as_np(got[2]), as_np(picked[2])), (small_sort, name)
-    finally:
-        runtime.set_option("small_sort", 1)
 
 
 def test_rank_strided_and_half_inputs():
@@ -354,13 +344,9 @@ def peel_algorithm(request):
     """The peeling variants: matrix rows resident in LDS (default where the matrix fits), and the three that rescan
     rows in memory: witness pass with the record protocol, witness pass with the master barrier and front
     bitmaps, and the popcount-decrement sweep (master barrier)."""
-    runtime.set_option("peel_lds", 1 if request.param == "lds" else 0)
-    runtime.set_option("peel_witness", 0 if request.param == "sweep" else 1)
-    runtime.set_option("peel_records", 1 if request.param == "witness-records" else 0)
-    yield request.param
-    runtime.set_option("peel_lds", 1)
-    runtime.set_option("peel_witness", 1)
-    runtime.set_option("peel_records", 1)
+    with runtime.options(peel_lds=1 if request.param == "lds" else 0, peel_witness=0 if request.param == "sweep" else 1,
+                         peel_records=1 if request.param == "witness-records" else 0):
+        yield request.param
 
 
 @pytest.mark.parametrize("name", ["C1", "C2", "C2p", "C3"])
@@ -868,8 +854,7 @@ def test_barrier_timeout_is_reported_not_hung():
             return True
         return False
 
-    runtime.set_option("spin_limit", 1)
-    try:
+    with runtime.options(spin_limit=1):
         # with one poll a wait may still succeed when the other blocks are already there: either the result is
         # right and the status clean, or the status carries the error and NO partial result is handed out --
         # every rank -1, every distance NaN, the rows all-ones bytes
@@ -889,8 +874,6 @@ def test_barrier_timeout_is_reported_not_hung():
         dist = crowding_distance(f, None)
         if failed():
             assert np.isnan(as_np(dist)).all()
-    finally:
-        runtime.set_option("spin_limit", 4000000)
     assert np.array_equal(as_np(non_dominate_rank(f)), want)
     assert not failed()
 
@@ -943,13 +926,10 @@ def test_record_protocol_with_other_block_counts():
     say("record_blocks")
     f = workloads.uniform_population(6000, 3, 0, 12)[0]
     want = as_np(er.ranks_by_peeling(f))
-    try:
-        for blocks in (16, 37, 100, 128, 200):
-            runtime.set_option("peel_record_blocks", blocks)
+    for blocks in (16, 37, 100, 128, 200):
+        with runtime.options(peel_lds=0, peel_record_blocks=blocks):
             assert np.array_equal(as_np(non_dominate_rank(f.to(DEV))), want), blocks
             assert runtime.last_status()["error"] == 0
-    finally:
-        runtime.set_option("peel_record_blocks", 0)
 
 
 # ------------------------------------------------------------------ ranks up to the cut front only
