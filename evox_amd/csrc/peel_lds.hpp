@@ -406,25 +406,33 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
   }
   EVX_TRACE(62, 2);
   // the witness of every row: its highest non-empty word (the lanes of a wave see their own LDS writes in order)
+  // Every lane walks down its own row, eight words a step, all rows of the wave side by side (the wave as a whole
+  // on one row after the other cost 2 us here at 20 000 rows: a row's highest dominator lies a few dozen words
+  // below its own slot, rows of similar key sums rarely dominate one another).
   int st_word = -1, st_off = 0;
   uint64_t st_bits = 0ull;
-  for (int k = 0; k < per_wave; ++k) {
-    const int64_t j = first_row + (int64_t)k * row_step;
-    if (j >= n) break;  // wave-uniform
-    const int off = row_off[wave * per_wave + k];
-    int word;
-    uint64_t bits;
-    lds_row_highest(rows_lds + off, row_words((int)j), alive_lds, word, bits);
-    if (lane == k) {
-      st_word = word;
-      st_bits = bits;
-      st_off = off;
-      if (word < 0) {  // no dominator: front 0
-        const int e = atomicAdd(&sh[0], 1);
-        found[2 * e] = (int)j;
-        found[2 * e + 1] = st_orig;
-      }
+  const int my_words = have_row ? row_words((int)my_slot) : 0;
+  if (have_row) st_off = row_off[wave * per_wave + lane];
+  for (int top = my_words - 1; __builtin_amdgcn_ballot_w64(st_word < 0 && top >= 0) != 0ull; top -= 8) {
+    uint64_t v[8], a[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int w = top - q;
+      const bool in = st_word < 0 && w >= 0;
+      v[q] = in ? rows_lds[st_off + w] : 0ull;
+      a[q] = in ? alive_lds[w] : 0ull;
     }
+#pragma unroll
+    for (int q = 7; q >= 0; --q)
+      if ((v[q] & a[q]) != 0ull) {
+        st_word = top - q;
+        st_bits = v[q];
+      }
+  }
+  if (have_row && st_word < 0) {  // no dominator: front 0
+    const int e = atomicAdd(&sh[0], 1);
+    found[2 * e] = (int)my_slot;
+    found[2 * e + 1] = st_orig;
   }
   if (have_row) {
     rank[st_orig] = st_word < 0 ? 0 : kRankUnset;
@@ -561,14 +569,29 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
           }
         }
         lds_barrier();
-        // (cost key, original index) of every candidate in every objective: one round trip to memory
-        for (int idx = tid; idx < nv * m; idx += blockDim.x) {
-          const int k = idx / nv, e = idx - k * nv;
-          const int slot = t_slot[e];
-          const int orig = orig_of[slot];
-          const float c = tail.xs_sorted[(int64_t)k * tail.npad + slot];
-          comp[idx] = ((unsigned long long)ordered_key(c) << 32) | (unsigned)orig;
-          if (k == 0) t_orig[e] = orig;
+        // (cost key, original index) of every candidate in every objective: one round trip to memory (at most
+        // kTailValues = 8 * 512 items: a thread's eight pairs of loads are all in flight together)
+        {
+          constexpr int kPerThread = kTailValues / kLdsPeelThreads;
+          int orig_v[kPerThread];
+          float cost_v[kPerThread];
+#pragma unroll
+          for (int q = 0; q < kPerThread; ++q) {
+            const int idx = tid + q * kLdsPeelThreads;
+            const int idc = idx < nv * m ? idx : 0;
+            const int k = idc / nv, e = idc - k * nv;
+            const int slot = t_slot[e];
+            orig_v[q] = orig_of[slot];
+            cost_v[q] = tail.xs_sorted[(int64_t)k * tail.npad + slot];
+          }
+#pragma unroll
+          for (int q = 0; q < kPerThread; ++q) {
+            const int idx = tid + q * kLdsPeelThreads;
+            if (idx < nv * m) {
+              comp[idx] = ((unsigned long long)ordered_key(cost_v[q]) << 32) | (unsigned)orig_v[q];
+              if (idx < nv) t_orig[idx] = orig_v[q];
+            }
+          }
         }
         lds_barrier();
         EVX_TRACE(61, 1);
@@ -652,11 +675,16 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
           typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
           const int e0 = 4 * tid;
           bool pending0 = e0 < nv, pending1 = e0 + 2 < nv, fine_poll = true;
+          // (both loads of a round are in flight together; the buffer holds kTailRows entries, a multiple of four,
+          // so the second load of a thread whose first is in range stays inside it)
           for (unsigned spins = 0; pending0 || pending1; ++spins) {
+            u32x4 r0, r1;
+            asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1\n\ts_waitcnt vmcnt(0)"
+                         : "=&v"(r0), "=&v"(r1)
+                         : "v"(tail.buffer + e0)
+                         : "memory");
             if (pending0) {
-              u32x4 r;
-              asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(r) : "v"(tail.buffer + e0) : "memory");
-              const unsigned long long a = ((unsigned long long)r.y << 32) | r.x, b = ((unsigned long long)r.w << 32) | r.z;
+              const unsigned long long a = ((unsigned long long)r0.y << 32) | r0.x, b = ((unsigned long long)r0.w << 32) | r0.z;
               if (a != 0ull && (e0 + 1 >= nv || b != 0ull)) {
                 comp[e0] = a;
                 if (e0 + 1 < nv) comp[e0 + 1] = b;
@@ -664,9 +692,7 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
               }
             }
             if (pending1) {
-              u32x4 r;
-              asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(r) : "v"(tail.buffer + e0 + 2) : "memory");
-              const unsigned long long a = ((unsigned long long)r.y << 32) | r.x, b = ((unsigned long long)r.w << 32) | r.z;
+              const unsigned long long a = ((unsigned long long)r1.y << 32) | r1.x, b = ((unsigned long long)r1.w << 32) | r1.z;
               if (a != 0ull && (e0 + 3 >= nv || b != 0ull)) {
                 comp[e0 + 2] = a;
                 if (e0 + 3 < nv) comp[e0 + 3] = b;
@@ -678,11 +704,14 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
               break;
             }
           }
-          if (!fine_poll) coherent_store(&ctrl->err, kErrBarrierTimeout);
+          if (!fine_poll) {
+            coherent_store(&ctrl->err, kErrBarrierTimeout);
+            next_cnts[3] = 1;  // (cleared with the counters of the level that will not come)
+          }
         }
         EVX_TRACE(61, 3);
         lds_barrier();
-        if (coherent_load(&ctrl->err) == 0) {
+        if (next_cnts[3] == 0) {  // every entry has arrived (a wait that gave up, here or elsewhere, ended the polls)
           for (int j = tid >> 4; j < mine_n; j += groups) {
             const int e = sb + j * sweepers;
             const unsigned long long mine = comp[e];
