@@ -13,9 +13,10 @@ from ... import ops
 
 
 def _crowding_distance_f64(costs: torch.Tensor, mask: Optional[torch.Tensor]) -> torch.Tensor:
-    """float64 costs (the default dtype set to float64): the reference's statements (non_dominate.py:209-231), one
-    by one, around this package's ``lexsort`` (the stable argsort kernels; the kernels of the float32 path read
-    4-byte values).  One population."""
+    """float64 costs (the default dtype set to float64) or integer costs: the reference's statements
+    (non_dominate.py:209-231), one by one, around this package's ``lexsort`` (the stable argsort kernels; the
+    kernels of the float32 path read 4-byte floats).  Integer costs are subtracted exactly and divided in the
+    default float dtype, as there.  One population."""
     from ...utils import lexsort
 
     total_len, m = costs.shape
@@ -24,14 +25,15 @@ def _crowding_distance_f64(costs: torch.Tensor, mask: Optional[torch.Tensor]) ->
         mask = torch.ones(total_len, dtype=torch.bool, device=costs.device)
     else:
         num_valid = int(mask.sum())
+    out_dtype = costs.dtype if costs.is_floating_point() else torch.get_default_dtype()
     if total_len == 0:
-        return torch.empty(0, dtype=costs.dtype, device=costs.device)
+        return torch.empty(0, dtype=out_dtype, device=costs.device)
     inverted = (~mask).unsqueeze(1).expand(-1, m).to(costs.dtype)
     rank = lexsort([costs, inverted], dim=0)
     sorted_costs = torch.gather(costs, dim=0, index=rank)
     # (torch.empty in the reference: whatever it holds is either overwritten below or belongs to a row outside
     # the mask)
-    distance = torch.full(costs.size(), -torch.inf, dtype=costs.dtype, device=costs.device)
+    distance = torch.full(costs.size(), -torch.inf, dtype=out_dtype, device=costs.device)
     if num_valid > 0:
         distance_range = sorted_costs[num_valid - 1] - sorted_costs[0]
         if total_len > 2:
@@ -117,14 +119,15 @@ def crowding_distance(costs: torch.Tensor, mask: Optional[torch.Tensor]) -> torc
     objective get ``+inf``; every other selected row gets the sum over objectives of
     ``(next - previous) / (last - first)``; unselected rows get ``-inf``.  The result has torch's
     default float dtype, and, as in the reference (its scatter at :224-225), ``costs`` must have that
-    dtype too.  With the default dtype set to float64 the distances are computed in float64, by the
-    reference's own sequence of statements around this package's ``lexsort``.
+    dtype too.  With the default dtype set to float64 the distances are computed in float64, and integer costs
+    are subtracted exactly and divided in the default float dtype, both by the reference's own sequence of
+    statements around this package's ``lexsort``.
     """
-    if costs.dtype != torch.get_default_dtype():
+    if costs.is_floating_point() and costs.dtype != torch.get_default_dtype():
         raise RuntimeError(
             f"crowding_distance: expected costs.dtype to be the default dtype {torch.get_default_dtype()}, got {costs.dtype}"
         )
-    if costs.dtype == torch.float64:
+    if costs.dtype == torch.float64 or not costs.is_floating_point():
         ops.runtime.require_gpu_tensor(costs, "costs")
         return _per_population(_crowding_distance_f64, costs.dim() - 2, costs, mask)
     return ops.crowding(costs, mask)
@@ -144,7 +147,7 @@ def nd_environmental_selection(x: torch.Tensor, f: torch.Tensor, topk: int) -> T
         raise RuntimeError(
             f"nd_environmental_selection: expected f.dtype to be the default dtype {torch.get_default_dtype()}, got {f.dtype}"
         )
-    if f.dtype == torch.float64:
+    if f.dtype == torch.float64 or not (f.is_floating_point() or f.is_complex() or f.dtype == torch.bool):
         ops.runtime.require_gpu_tensor(f, "f")
         return _per_population(lambda xb, fb: _nd_environmental_selection_f64(xb, fb, int(topk)), f.dim() - 2, x, f)
     return ops.nd_select(x, f, int(topk))

@@ -89,3 +89,38 @@ def test_float64_batched_and_errors(float64_default):
         nd_environmental_selection(x[0].to(DEV), f[0].to(DEV), 0)
     with pytest.raises(RuntimeError):  # float32 costs under a float64 default: the reference's scatter refuses them
         crowding_distance(f[0].float().to(DEV), None)
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32, torch.uint8])
+def test_integer_fitness_crowding_and_selection(dtype):
+    """Integer fitness (the reference accepts it: exact integer differences, divided in the default float dtype,
+    non_dominate.py:218-225), 64-bit values beyond float32's 2**24 included."""
+    g = torch.Generator("cpu").manual_seed(66)
+    if dtype == torch.int64:
+        f = (2**40 + torch.randint(0, 3000, (2500, 3), generator=g)).to(dtype)
+    elif dtype == torch.int32:
+        f = torch.randint(-50, 50, (2500, 2), generator=g, dtype=dtype)
+    else:
+        f = torch.randint(0, 256, (1500, 4), generator=g).to(dtype)
+    fd = f.to(DEV)
+    rank = er.ranks_by_peeling(f)
+    for mask in (None, rank == 0, rank == 2):
+        want = er.crowding(f, mask)
+        got = crowding_distance(fd, None if mask is None else mask.to(DEV))
+        assert got.dtype == torch.float32
+        gw, ww = as_np(got), as_np(want)
+        assert np.array_equal(np.isnan(gw), np.isnan(ww)) and np.array_equal(np.isinf(gw), np.isinf(ww))
+        fin = np.isfinite(ww)
+        np.testing.assert_allclose(gw[fin], ww[fin], rtol=1e-5)
+    x = torch.arange(f.size(0), dtype=torch.int64)[:, None]
+    for k in (1, 700, f.size(0)):
+        want = er.environmental_selection(x, f, k)
+        got = nd_environmental_selection(x.to(DEV), fd, k)
+        assert got[1].dtype == dtype and torch.equal(got[1].cpu(), want[1])
+        assert torch.equal(got[2].cpu(), want[2])
+        gw, ww = as_np(got[3]), as_np(want[3])
+        assert np.array_equal(np.isnan(gw), np.isnan(ww)) and np.array_equal(np.isinf(gw), np.isinf(ww))
+        # the selected rows: equal but for distances that tie within float32 rounding at the cut
+        if not torch.equal(got[0].cpu(), want[0]):
+            assert sorted(as_np(got[0])[:, 0].tolist()) == sorted(as_np(want[0])[:, 0].tolist()) or np.allclose(
+                np.sort(gw[np.isfinite(gw)]), np.sort(ww[np.isfinite(ww)]), rtol=1e-5)
