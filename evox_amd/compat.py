@@ -26,6 +26,7 @@ import torch
 
 from .hype import cal_hv
 from .metrics.hv import hv
+from .utils import lexsort
 from .operators.selection import (
     crowding_distance,
     nd_environmental_selection,
@@ -49,6 +50,8 @@ _TARGETS = (
     "evox.workflows.eval_monitor",
     "evox.metrics.hv",
     "evox.metrics",
+    "evox.utils.jit_fix_operator",
+    "evox.utils",
 )
 _FUNCS = {
     "non_dominate_rank": non_dominate_rank,
@@ -58,6 +61,8 @@ _FUNCS = {
     "tournament_selection": tournament_selection,
     "cal_hv": cal_hv,  # only evox.algorithms.mo.hype holds this name
     "hv": hv,  # the function that evox.metrics and evox.metrics.hv hold (src/evox/metrics/__init__.py:4), not the module
+    # src/evox/utils/jit_fix_operator.py:213-252, held by HypE (hype.py:9, used at :143) and the two selection modules
+    "lexsort": lexsort,
 }
 
 _installed = {}  # "module.name" -> the binding that was found there
@@ -218,7 +223,7 @@ def _patch_callers() -> list:
 
 
 def install_into_evox(patch_callers: bool = False) -> list:
-    """Routes EvoX's selection operators (and HypE's ``cal_hv``, and the ``hv`` metric), wherever a module already
+    """Routes EvoX's selection operators (and ``lexsort``, HypE's ``cal_hv`` and the ``hv`` metric), wherever a module already
     holds them, to the HIP-backed ones for tensors on the GPU; tensors elsewhere keep going to the function that
     was bound there.  With ``patch_callers`` the four callers named in the module docstring are changed as well.
     Returns the list of ``module.name`` bindings (and ``module.Class.method`` callers) that were changed; a second

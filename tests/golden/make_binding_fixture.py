@@ -27,7 +27,7 @@ import evox_amd  # noqa: E402
 from evox_amd import compat  # noqa: E402
 
 NAMES = ("non_dominate_rank", "crowding_distance", "nd_environmental_selection", "tournament_selection_multifit",
-         "tournament_selection", "cal_hv", "hv")
+         "tournament_selection", "cal_hv", "hv", "lexsort")
 
 
 def holders():
@@ -48,6 +48,7 @@ def holders():
         "tournament_selection": ts_module.tournament_selection,
         "cal_hv": hype_module.cal_hv,
         "hv": hv_module.hv,
+        "lexsort": importlib.import_module("evox.utils.jit_fix_operator").lexsort,
     }
     found = []
     for mod_name, module in sorted(sys.modules.items()):
