@@ -497,8 +497,15 @@ def main():
     else:
         peel_bytes = int(row_read[ranked_in_passes].sum()) + passes * nwords * 8
     dom_bytes = n * m * 4 + int(row_read.sum())
+    import ctypes
+
+    from evox_amd import _lib
+
+    plan = (ctypes.c_int64 * 2)()
+    _lib.call("evox_hip_dominance_plan", n, m, plan)
+    tile_slots = 64 * max(int(plan[0]), 2)  # dominator slots of a tile (a wave evaluates 64 rows against whole tiles)
     slots = torch.arange(n, device=rank.device)
-    evaluated_pairs = float(((((slots >> 6) << 6) + 63) // 256 * 256 + 256).clamp(max=nwords * 64).sum())
+    evaluated_pairs = float(((((slots >> 6) << 6) + 63) // tile_slots * tile_slots + tile_slots).clamp(max=nwords * 64).sum())
     # finite populations take the arithmetic form: m subtractions (scalar operand), (m - 1) ORs three at a time,
     # clamp, shift-in; others the compare form: m + 2 mask-writing instructions.  Measured alone, two-operand
     # vector-register instructions issue at about 50 T lane-ops/s and three-operand, min/max and scalar-operand
@@ -506,7 +513,7 @@ def main():
     finite = bool(torch.isfinite(f).all())
     # large finite populations get the matrix from the order of the rows in every objective instead (the library's
     # rule: at least 65536 rows with 3 to 8 objectives, 81920 with 2, 49152 with 9 to 16): no pairwise test is executed at all
-    from_orders = finite and ((3 <= m <= 8 and n >= 65536) or (m == 2 and n >= 81920) or (9 <= m <= 16 and n >= 49152))
+    from_orders = finite and bool(plan[1])
     # (up to three objectives the sign of the OR is shifted in by one v_alignbit_b32 and the word complemented at the end)
     valu_per_pair = (m + (m // 2) + (1 if m <= 3 else 2)) if finite else m + 2
     executed_valu = valu_per_pair * evaluated_pairs
@@ -516,7 +523,7 @@ def main():
     phases = {
         "prepare_and_slot_sort": {"us": times["prepare_us"]},
         # achieved / frac: the VALU lane-instructions this kernel issues per ordered pair of the lower triangle (tiles
-        # of 64 rows x 256 columns on or below the diagonal) over the kernel's time, against the peak of the
+        # of 64 rows x 128 or 256 columns on or below the diagonal) over the kernel's time, against the peak of the
         # instruction kind it uses.  The reference's 2*M*N^2 compares over the same time ride along as a rate only:
         # the kernel does not execute them, so no fraction of a peak is formed from them.
         "dominance": {"us": times["dominance_us"], "kernel_alone_us": dom_us, "bound": "valu",

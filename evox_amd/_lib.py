@@ -66,6 +66,7 @@ _SIGNATURES = {
     "evox_hip_workspace_layout": (c_int, [c_int64, c_int64, c_void_p]),
     "evox_hip_slot_sort_layout": (c_int, [c_int64, c_int64, c_void_p]),
     "evox_hip_peel_plan": (c_int, [c_int64, c_int64, c_void_p]),
+    "evox_hip_dominance_plan": (c_int, [c_int64, c_int64, c_void_p]),
     "evox_hip_read_status": (c_int, [c_void_p, c_void_p, c_void_p]),
     "evox_hip_set_option": (c_int, [c_char_p, c_int64]),
     "evox_hip_options_create": (c_void_p, []),

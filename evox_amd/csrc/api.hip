@@ -37,7 +37,7 @@ struct Options {
   int peel_tail = 1;        // that kernel also orders a small last front (0: always the kernels of finish.hpp)
   int tail_merged = 1;      // after such a peel, ordering (where still needed) and gather share one launch
   unsigned spin_limit = 4000000u;
-  int dominance_tile_words = 4;
+  int dominance_tile_words = 0;  // 0 = by size (2 or 4)
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
   int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 8 objectives (a quarter
                                     // more rows with 2, a quarter fewer with 9 to 16) get their matrix from the per-objective orders (prefix.hpp);
@@ -295,19 +295,30 @@ static bool prefix_dominance_applies(const Layout& L) {
 }
 static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s);
 
+static int dominance_tile_words(const Layout& L) {
+  const int tile = opt().dominance_tile_words;
+  if (tile != 0) return tile;
+  return L.m >= 3 && L.m <= 8 && L.n <= (L.m >= 6 ? 32768 : 24576) ? 2 : 4;
+}
+
 static int stage_dominance(const Ws& w, int variant, hipStream_t s) {
   // (kDomOrdersOnly: the first half of the path below alone, for measurements of the second)
   if (variant == kDomOrdersOnly) return prefix_dominance_applies(w.L) ? stage_dominance_prefix(w, true, s) : kErrBadArg;
   if (variant == kDomAuto && prefix_dominance_applies(w.L)) return stage_dominance_prefix(w, false, s);
-  // (the lower triangle in tiles of 4 words keeps every SIMD busy with several waves; 16 is kept for
-  // measurements)
-  const int tile = opt().dominance_tile_words;
+  // (the lower triangle in tiles of 4 words keeps every SIMD busy with several waves; up to about 24 000 rows of
+  // three to eight objectives tiles of 2 words leave a shorter half-empty tail -- measured, us, tiles of 2 / 4:
+  // 5000 x 3: 6.2 / 8.1, 16 000 x 3: 21.9 / 27.1, 20 000 x 3: 30.6 / 34.1, x 5: 47.7 / 54.3, x 8: 67.5 / 80.9,
+  // 24 000 x 3: 41.7 / 42.7, 28 000 x 3: 51.2 / 51.0, x 8: 118.5 / 127.6, 32 768 x 3: 71.5 / 68.2, 50 000 x 3:
+  // 150.5 / 142.8, 20 000 x 2: 26.5 / 24.4 --; 8 and 16 are kept for measurements)
+  const int tile = dominance_tile_words(w.L);
   if (tile >= 16)
     launch_dominance<16>(w, variant, s);
   else if (tile >= 8)
     launch_dominance<8>(w, variant, s);
-  else
+  else if (tile >= 4)
     launch_dominance<4>(w, variant, s);
+  else
+    launch_dominance<2>(w, variant, s);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -858,7 +869,7 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.peel_lds_blocks = (int)value;
   } else if (!strcmp(name, "spin_limit") && value >= 1 && value <= 0x7FFFFFFFll) {
     o.spin_limit = (unsigned)value;
-  } else if (!strcmp(name, "dominance_tile_words") && (value == 4 || value == 8 || value == 16)) {
+  } else if (!strcmp(name, "dominance_tile_words") && (value == 0 || value == 2 || value == 4 || value == 8 || value == 16)) {
     o.dominance_tile_words = (int)value;
   } else if (!strcmp(name, "small_sort") && (value == 0 || value == 1)) {
     o.small_sort = (int)value;
@@ -1471,6 +1482,14 @@ int evox_hip_calibration_launch(int kind, int64_t blocks, int64_t iterations, fl
   else
     hipLaunchKernelGGL(calibrate_kernel<3>, grid, block, 0, s, scratch_out, (int)iterations, 1.0f, 2.0f);
   EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+int evox_hip_dominance_plan(int64_t n, int64_t m, int64_t* out2) {
+  Layout L;
+  if (out2 == nullptr || !make_layout(n, m, &L)) return kErrBadArg;
+  out2[0] = prefix_dominance_applies(L) ? 0 : dominance_tile_words(L);
+  out2[1] = prefix_dominance_applies(L);
   return 0;
 }
 

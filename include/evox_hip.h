@@ -243,6 +243,12 @@ int evox_hip_slot_sort_layout(int64_t n, int64_t m, int64_t* out6);
  * (both 0 when out[0] is 0).  Depends on the device that is current and on the tunables. */
 int evox_hip_peel_plan(int64_t n, int64_t m, int64_t* out3);
 
+/* How the dominance matrix of a population of this shape is built, for tools and benchmarks: out[1] = 1 when a finite
+ * population gets it from the order of its rows in every objective (no pairwise test; out[0] is then 0), else out[0] =
+ * words of a row that one wave of the pairwise kernel produces (it evaluates whole tiles of 64 rows x 64 out[0] slots on
+ * or below the diagonal).  Depends on the tunables. */
+int evox_hip_dominance_plan(int64_t n, int64_t m, int64_t* out2);
+
 /* Waits for `stream`, then copies the control block's eight leading ints to HOST memory:
  * out[0] error (0 or EVOX_HIP_E_BARRIER_TIMEOUT), out[1] fronts peeled, out[2] last front's rank,
  * out[3] rows in better fronts, out[4] last front's size, out[5] rows taken from it, out[6] sweep passes.
@@ -254,7 +260,7 @@ int evox_hip_read_status(const void* workspace, void* stream, int32_t* host_out8
  * (1 = after such a peel the two ordering stages share one launch, up to three objectives),
  * "peel_blocks_per_cu" (default 2), "peel_witness" (1 = witness pass, 0 = popcount sweep), "peel_records" (1 = record
  * protocol, 0 = master barrier and front bitmaps), "peel_record_blocks" (0 = by size, or 16 .. 255), "spin_limit" (polls before a device-side
- * wait gives up, default 4000000), "dominance_tile_words" (4, 8 or 16, default 4), "small_sort" (1 = one-kernel slot sort up to 4096 rows),
+ * wait gives up, default 4000000), "dominance_tile_words" (0 = by size: 2 or 4; or 2, 4, 8, 16), "small_sort" (1 = one-kernel slot sort up to 4096 rows),
  * "prefix_min_rows" (default 65536: smallest finite population whose matrix is built from the per-objective orders, 0 = never),
  * "prefix_bands" (default 1), "prefix_double_tile" (default 131072 rows, 0 = never), "prefix_mode" (default 3; 1 and 2 build only half of that kernel's output, for measurements).
  * Returns EVOX_HIP_E_BAD_ARG for an unknown name or a value out of range. */
