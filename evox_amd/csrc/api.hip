@@ -449,13 +449,24 @@ static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool
 static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s);
 static int stage_count(const Ws& w, bool fill_dist, hipStream_t s);
 static int count_and_peel(const Ws& w, int64_t stop_count, bool want_perm, bool fill_dist, hipStream_t s,
-                          bool order_last_front = false, bool* may_have_ordered = nullptr) {
+                          bool order_last_front = false, bool* may_have_ordered = nullptr, bool* always_orders = nullptr) {
   size_t lds = 0;
   if (may_have_ordered) *may_have_ordered = false;
+  if (always_orders) *always_orders = false;
   if (const int sweepers = lds_peel_plan(w.L, &lds)) {
-    if (may_have_ordered)
-      *may_have_ordered = order_last_front && opt().peel_tail && peel_tail_lds_bytes(w.L.n, w.L.m) != 0 &&
-                          peel_tail_lds_bytes(w.L.n, w.L.m) <= kLdsPeelBudget;
+    const bool may = order_last_front && opt().peel_tail && peel_tail_lds_bytes(w.L.n, w.L.m) != 0 &&
+                     peel_tail_lds_bytes(w.L.n, w.L.m) <= kLdsPeelBudget;
+    if (may_have_ordered) *may_have_ordered = may;
+    if (always_orders && may) {
+      // Whatever the last front turns out to be, the peel kernel orders it: no front of this population is too
+      // large for it, and no workgroup can have more rows in one front than its record holds (a level with such a
+      // record goes through the bitmaps in memory and leaves the last front to the kernels after it).
+      int units = 2;
+      while (units * 2 * sweepers <= kRecUnits && units < 32) units *= 2;
+      const int waves = kLdsPeelThreads / 64;
+      const int rows_of_a_workgroup = (w.L.n + sweepers * waves - 1) / (sweepers * waves) * waves;
+      *always_orders = peel_tail_applies(w.L.n, w.L.m) && rows_of_a_workgroup <= 2 + 3 * (units - 1);
+    }
     return launch_lds_peel(w, stop_count, want_perm, fill_dist, sweepers, lds, s, order_last_front);
   }
   if (int e = stage_count(w, fill_dist, s)) return e;
@@ -1189,7 +1200,8 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   if (int e = stage_prepare(w, fit, true, s)) return e;
   if (int e = stage_dominance(w, kDomAuto, s)) return e;
   bool peel_orders = false;  // the peel kernel orders a small last front itself (it says so in Ctrl.tail_done)
-  if (int e = count_and_peel(w, topk, true, true, s, true, &peel_orders)) return e;
+  bool peel_always_orders = false;  // ... and here every front is small enough: nothing is left to launch but the gather
+  if (int e = count_and_peel(w, topk, true, true, s, true, &peel_orders, &peel_always_orders)) return e;
   int unit = 1;
   if (x != nullptr) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(x2) | reinterpret_cast<uintptr_t>(out_x) |
@@ -1222,6 +1234,7 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   g.out_dist = out_dist;
   g.out_order = out_order;
   g.ctrl = w.ctrl();
+  g.order_from_peel = peel_always_orders ? 1 : 0;
   // Where the peel kernel may have ordered the last front, the kernels that would order it look at Ctrl.tail_done and
   // return at once.  A launch that does nothing still costs about 4.7 us, so with up to three objectives -- last
   // fronts of a few hundred rows, which the peel kernel orders -- the two ordering stages share one launch
@@ -1229,6 +1242,14 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   // stages as kernels of their own, each on the grid that suits it, order it faster than the shared launch does
   // (20 000 x 5, a front of 2532 rows: 245 against 261 us per selection; 20 000 x 8, 7481 rows: 457 against 493).
   const bool one_ordering_launch = peel_orders && opt().tail_merged && L.m <= 3;
+  if (peel_always_orders) {
+    int blocks = (int)((topk + 3) / 4);
+    const int cap = device_cus() * 8;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(gather_after_peel_kernel, dim3(blocks), dim3(256), 0, s, g);
+    EVX_LAUNCH_CHECK();
+    return 0;
+  }
   if (!one_ordering_launch) {
     if (int e = stage_crowd_sort(w, w.at<int>(L.perm), true, 2, s, peel_orders)) return e;
     if (int e = stage_crowd_finish(w, w.at<int>(L.perm), true, 2, s, peel_orders)) return e;

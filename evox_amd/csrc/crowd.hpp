@@ -132,6 +132,7 @@ struct GatherArgs {
   float* out_dist;
   int* out_order;
   const Ctrl* ctrl;
+  int order_from_peel;  // the host launched nothing that orders the last front: the peel kernel must have (Ctrl.tail_done)
 };
 
 // Called by every thread of `blocks` blocks of 256 threads (`block` = the caller's index among them).
@@ -146,7 +147,7 @@ __device__ inline void gather_body(const GatherArgs& a, int block, int blocks, i
   int* __restrict__ out_rank = a.out_rank;
   float* __restrict__ out_dist = a.out_dist;
   int* __restrict__ out_order = a.out_order;
-  if (a.ctrl->err != 0) {
+  if (a.ctrl->err != 0 || (a.order_from_peel != 0 && a.ctrl->tail_done == 0)) {
     // a device-side wait ran out and `order` was not produced: no partial result leaves the call -- rank -1,
     // distance and fitness NaN, order -1, decision vectors all-ones bytes (NaN as floats)
     const int64_t threads = (int64_t)blocks * blockDim.x, t0 = (int64_t)block * blockDim.x + threadIdx.x;
