@@ -38,6 +38,7 @@ struct Options {
   int tail_merged = 1;      // after such a peel, ordering (where still needed) and gather share one launch
   unsigned spin_limit = 4000000u;
   int dominance_tile_words = 0;  // 0 = by size (2 or 4)
+  int mid_argsort = 1;  // an argsort step of 8193 .. kMidArgsortRows positions in one kernel without waits (0: the radix sort)
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
   int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 8 objectives (a quarter
                                     // more rows with 2, a quarter fewer with 9 to 16) get their matrix from the per-objective orders (prefix.hpp);
@@ -884,6 +885,8 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.dominance_tile_words = (int)value;
   } else if (!strcmp(name, "small_sort") && (value == 0 || value == 1)) {
     o.small_sort = (int)value;
+  } else if (!strcmp(name, "mid_argsort") && (value == 0 || value == 1)) {
+    o.mid_argsort = (int)value;
   } else if (!strcmp(name, "prefix_min_rows") && value >= 0) {
     o.prefix_min_rows = value;
   } else if (!strcmp(name, "prefix_double_tile") && value >= 0) {
@@ -1088,6 +1091,16 @@ static int argsort_step(const void* key, int kind, int64_t stride, int64_t n, co
     if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(small_argsort_kernel), sizeof(double) * (size_t)npad)) return e;
     hipLaunchKernelGGL(small_argsort_kernel, dim3(npad / kSmallArgsortGroup), dim3(kSmallArgsortThreads),
                        sizeof(double) * (size_t)npad, s, key, kind, stride, (int)n, prev_order, order_out);
+    EVX_LAUNCH_CHECK();
+    return 0;
+  }
+  if (n <= kMidArgsortRows && opt().mid_argsort) {
+    // (one workgroup per compute unit, each producing a run of slots; no workgroup waits for another)
+    const size_t lds = sizeof(uint32_t) * (size_t)n;
+    if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(mid_argsort_kernel), lds)) return e;
+    const int per = (int)round_up((n + device_cus() - 1) / device_cus(), 16);
+    hipLaunchKernelGGL(mid_argsort_kernel, dim3((unsigned)((n + per - 1) / per)), dim3(kMidArgsortThreads), lds, s, key, kind, stride,
+                       (int)n, prev_order, per, order_out);
     EVX_LAUNCH_CHECK();
     return 0;
   }

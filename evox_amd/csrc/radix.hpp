@@ -327,6 +327,209 @@ __global__ __launch_bounds__(kSmallArgsortThreads) void small_argsort_kernel(con
   }
 }
 
+// The same step for kSmallArgsortRows < n <= kMidArgsortRows positions, still in one launch with no dependence
+// between workgroups (the radix sort needs three launches and twelve grid barriers: 70 us at 20 000 positions, more
+// than torch's own sort).  Every workgroup reads all keys into LDS (32-bit order-preserving images) and works on
+// composites (image << 15 | position: distinct, below 2^47); it produces a run of `slots_per_block` slots of the
+// result: the histogram of all composites over kMidArgsortBuckets buckets (LDS atomics), its scan, the buckets that
+// hold the wanted slots, their composites collected into a list, every member of the list placed by counting the
+// members below it (sixteen lanes per member).  Keys with few distinct values are the usual case here (ranks, a
+// distance that is -inf for most rows): the buckets cut the composites, so a key held by thousands of positions is
+// spread over many buckets by its position bits.  A group of buckets with more than kMidArgsortList composites is
+// not collected: the workgroup takes the bucket of its next slot alone, and if that is too large as well (a wide
+// range of keys with a crowd on one value) it builds the histogram of that bucket's range, which is narrower by the
+// bucket count each time, down to single composites.  The code is loops, not unrolled passes: a launch starts with
+// a cold instruction cache.
+constexpr int kMidArgsortRows = 24576;  // keys of 4 bytes in LDS beside the tables
+constexpr int kMidArgsortThreads = 1024;
+constexpr int kMidArgsortBuckets = 4096;
+constexpr int kMidArgsortList = 2048;
+constexpr int kMidArgsortIndexBits = 15;
+
+// Exclusive scan, in place, of the kMidArgsortBuckets counts in `hist` by the whole workgroup; returns their sum.
+__device__ inline int mid_argsort_scan(int* hist, int* wave_tot) {
+  constexpr int kPer = kMidArgsortBuckets / kMidArgsortThreads;  // 4 consecutive buckets per thread
+  constexpr int kWaves = kMidArgsortThreads / 64;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int4 c = *reinterpret_cast<const int4*>(hist + tid * kPer);
+  const int mine = c.x + c.y + c.z + c.w;
+  int incl = mine;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
+  }
+  if (lane == 63) wave_tot[wave] = incl;
+  __syncthreads();
+  int run = incl - mine, total = 0;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    if (w < wave) run += wave_tot[w];
+    total += wave_tot[w];
+  }
+  int4 o;
+  o.x = run; run += c.x;
+  o.y = run; run += c.y;
+  o.z = run; run += c.z;
+  o.w = run;
+  *reinterpret_cast<int4*>(hist + tid * kPer) = o;
+  __syncthreads();
+  return total;
+}
+
+__global__ __launch_bounds__(kMidArgsortThreads) void mid_argsort_kernel(const void* __restrict__ key, int kind, int64_t stride, int n,
+                                                                         const int* __restrict__ prev, int slots_per_block,
+                                                                         int* __restrict__ order_out) {
+  extern __shared__ uint32_t mid_keys[];  // n order-preserving images of the keys, in the order of the positions
+  __shared__ __attribute__((aligned(16))) int top_hist[kMidArgsortBuckets];  // first-level starts, kept
+  __shared__ __attribute__((aligned(16))) int sub_hist[kMidArgsortBuckets];  // starts of the level below, rebuilt
+  __shared__ unsigned long long list[kMidArgsortList];
+  constexpr int kWaves = kMidArgsortThreads / 64;
+  __shared__ uint32_t red[2][kWaves];
+  __shared__ int wave_tot[kWaves];
+  __shared__ int found[5];  // bucket of the first wanted slot, its start and end; bucket of the last wanted slot, its end
+  __shared__ int list_count;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr unsigned long long kIndexMask = (1ull << kMidArgsortIndexBits) - 1ull;
+  uint32_t kmin = 0xFFFFFFFFu, kmax = 0u;
+#pragma unroll 4
+  for (int e = tid; e < n; e += kMidArgsortThreads) {
+    const int idx = prev ? prev[e] : e;
+    uint32_t k;
+    if (kind == kKeyFloat32)
+      k = ordered_key(static_cast<const float*>(key)[(int64_t)idx * stride]);
+    else if (kind == kKeyInt32)
+      k = static_cast<const uint32_t*>(key)[(int64_t)idx * stride] ^ 0x80000000u;
+    else
+      k = static_cast<const uint32_t*>(key)[(int64_t)idx * stride];
+    mid_keys[e] = k;
+    kmin = k < kmin ? k : kmin;
+    kmax = k > kmax ? k : kmax;
+  }
+  for (int b = tid; b < kMidArgsortBuckets; b += kMidArgsortThreads) top_hist[b] = 0;
+  if (tid == 0) list_count = 0;
+  if (tid < 5) found[tid] = 0;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const uint32_t a = __shfl_xor(kmin, off), b = __shfl_xor(kmax, off);
+    kmin = a < kmin ? a : kmin;
+    kmax = b > kmax ? b : kmax;
+  }
+  if (lane == 0) {
+    red[0][wave] = kmin;
+    red[1][wave] = kmax;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    kmin = red[0][w] < kmin ? red[0][w] : kmin;
+    kmax = red[1][w] > kmax ? red[1][w] : kmax;
+  }
+  auto composite = [&](int e) { return ((unsigned long long)mid_keys[e] << kMidArgsortIndexBits) | (unsigned long long)e; };
+  auto shift_for = [](unsigned long long span) {
+    int shift = 0;
+    while (shift < 63 && (span >> shift) >= (unsigned long long)kMidArgsortBuckets) ++shift;
+    return shift;
+  };
+  const unsigned long long top_lo = (unsigned long long)kmin << kMidArgsortIndexBits;
+  const unsigned long long top_hi = ((unsigned long long)kmax << kMidArgsortIndexBits) | kIndexMask;
+  const int top_shift = shift_for(top_hi - top_lo);
+  for (int e = tid; e < n; e += kMidArgsortThreads) atomicAdd(&top_hist[(int)((composite(e) - top_lo) >> top_shift)], 1);
+  __syncthreads();
+  mid_argsort_scan(top_hist, wave_tot);  // (the total is n)
+  const int s0 = (int)blockIdx.x * slots_per_block;
+  const int s1 = min(n, s0 + slots_per_block);
+  // level state: the same in every thread
+  unsigned long long lo = top_lo, hi = top_hi;  // the composites of the level: lo .. hi
+  int shift = top_shift, base = 0, total = n;
+  bool at_top = true;
+  int x = s0;
+  // (every round either places slots or narrows the range; the count is a guard against a loop that does neither)
+  for (int rounds = 0; x < s1 && rounds < 8 * kMidArgsortList; ++rounds) {
+    const int* hist = at_top ? top_hist : sub_hist;
+    {
+      // the buckets that hold slot x and the last wanted slot of this level
+      const int q0 = x - base, q1 = min(s1 - 1 - base, total - 1);
+      constexpr int kPer = kMidArgsortBuckets / kMidArgsortThreads;
+#pragma unroll
+      for (int u = 0; u < kPer; ++u) {
+        const int b = u * kMidArgsortThreads + tid;  // (neighbouring lanes read neighbouring words)
+        const int st = hist[b], en = b + 1 < kMidArgsortBuckets ? hist[b + 1] : total;
+        if (st <= q0 && q0 < en) {
+          found[0] = b;
+          found[1] = st;
+          found[2] = en;
+        }
+        if (st <= q1 && q1 < en) {
+          found[3] = b;
+          found[4] = en;
+        }
+      }
+    }
+    __syncthreads();
+    const int b0 = found[0], b0_start = found[1], b0_end = found[2];
+    int b1 = found[3], b1_end = found[4];
+    if (b1_end - b0_start > kMidArgsortList) {
+      if (b0_end - b0_start > kMidArgsortList) {
+        // that bucket alone is too large: the histogram of its range
+        base += b0_start;
+        total = b0_end - b0_start;
+        lo += (unsigned long long)b0 << shift;
+        const unsigned long long span = (1ull << shift) - 1ull < hi - lo ? (1ull << shift) - 1ull : hi - lo;
+        hi = lo + span;
+        shift = shift_for(span);
+        at_top = false;
+        for (int b = tid; b < kMidArgsortBuckets; b += kMidArgsortThreads) sub_hist[b] = 0;
+        __syncthreads();
+        for (int e = tid; e < n; e += kMidArgsortThreads) {
+          const unsigned long long c = composite(e);
+          if (c >= lo && c - lo <= span) atomicAdd(&sub_hist[(int)((c - lo) >> shift)], 1);
+        }
+        __syncthreads();
+        mid_argsort_scan(sub_hist, wave_tot);
+        continue;
+      }
+      b1 = b0;
+      b1_end = b0_end;
+    }
+    {
+      const unsigned long long first = lo + ((unsigned long long)b0 << shift);
+      const unsigned long long width = ((unsigned long long)(b1 - b0 + 1) << shift) - 1ull;  // composites first .. first + width
+      for (int e = tid; e < n; e += kMidArgsortThreads) {
+        const unsigned long long c = composite(e);
+        if (c >= first && c - first <= width && c <= hi) list[atomicAdd(&list_count, 1)] = c;
+      }
+    }
+    __syncthreads();
+    const int members = list_count;  // = b1_end - b0_start
+    // sixteen lanes per member: each counts over a sixteenth of the list, the shares are added inside the DPP row
+    for (int p0 = 0; p0 < members; p0 += kMidArgsortThreads / 16) {
+      const int p = p0 + (tid >> 4), sub = tid & 15;
+      const unsigned long long c = p < members ? list[p] : 0ull;
+      int before = 0;
+#pragma unroll 4
+      for (int q = sub; q < members; q += 16) before += list[q] < c;
+      before = group16_sum(before);
+      const int slot = base + b0_start + before;
+      if (sub == 0 && p < members && slot >= x && slot < s1) {
+        const int e = (int)(c & kIndexMask);
+        order_out[slot] = prev ? prev[e] : e;
+      }
+    }
+    x = base + b1_end;
+    __syncthreads();  // the list and found[] are rewritten
+    if (tid == 0) list_count = 0;
+    if (!at_top) {  // back to the first level for the slots that are left
+      lo = top_lo;
+      hi = top_hi;
+      shift = top_shift;
+      base = 0;
+      total = n;
+      at_top = true;
+    }
+  }
+}
+
 // Many independent steps at once: `batch` sorts of n <= kSmallArgsortRows positions each, sort b reading
 // key[b * batch_stride + idx * stride], prev[b * n + .] and writing order_out[b * n + .].  A workgroup of T
 // threads takes `rows_per_block` sorts at a time (a power of two; T / rows_per_block threads each) with the

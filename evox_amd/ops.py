@@ -113,7 +113,7 @@ torch.library.register_vmap(nd_rank, _nd_rank_vmap)
 
 
 RANK_UNSET = 0x7FFFFFFF
-_SMALL_ARGSORT_ROWS = 8192  # longest one-dimensional sort that takes the counting kernel (no device-side waits)
+_SMALL_ARGSORT_ROWS = 24576  # longest one-dimensional sort whose kernel has no device-side waits (and keeps no control block)
 _ROWS_ARGSORT_MAX = 16384  # longest sort of a batch that runs inside one workgroup
 
 
@@ -467,7 +467,7 @@ def stable_argsort_rows(key: torch.Tensor, kind: int, prev: Optional[torch.Tenso
         stream = runtime.stream_handle(key.device)
         _lib.call("evox_hip_stable_argsort_step_batched", key.data_ptr(), kind, key.stride(0), key.stride(1), batch, n,
                   None if prev is None else prev.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
-        if n > (_ROWS_ARGSORT_MAX if batch >= 2 else _SMALL_ARGSORT_ROWS):
+        if n > _SMALL_ARGSORT_ROWS:
             runtime.note_call(ws, stream)
         else:
             runtime.note_small_kernel_call()

@@ -1117,7 +1117,7 @@ def test_lexsort_matches_numpy_and_the_restatement(population_path):
     from evox_amd.utils import lexsort
 
     g = torch.Generator("cpu").manual_seed(5)
-    for n in (1, 2, 63, 64, 65, 1000, 4097, 8191, 8192, 8193, 70000):
+    for n in (1, 2, 63, 64, 65, 1000, 4097, 8191, 8192, 8193, 12000, 24576, 24577, 70000):
         say("lexsort", n)
         k_f32 = torch.randint(0, 7, (n,), generator=g).float() / 2 - 1
         k_f32[torch.rand(n, generator=g) < 0.05] = float("nan")
@@ -1133,6 +1133,11 @@ def test_lexsort_matches_numpy_and_the_restatement(population_path):
             want = er.chained_stable_argsort([k.float() if k.dtype == torch.float16 else k for k in keys])
             got = lexsort([k.to(DEV) for k in keys])
             assert got.dtype == torch.int64 and torch.equal(got.cpu(), want), (n, [k.dtype for k in keys])
+        # distinct values over a wide range, and the same with a crowd on one value (a distance that is -inf for most rows)
+        k_wide = (torch.rand(n, generator=g) - 0.5) * 1e6
+        k_crowd = torch.where(torch.rand(n, generator=g) < 0.7, torch.full((n,), -float("inf")), k_wide)
+        for keys in ([k_wide], [k_crowd], [k_crowd, k_i32]):
+            assert torch.equal(lexsort([k.to(DEV) for k in keys]).cpu(), er.chained_stable_argsort(keys)), (n, "wide")
         # numpy's lexsort on keys without NaN (same convention: last key primary, stable)
         assert np.array_equal(as_np(lexsort([k_i32.to(DEV), k_u8.to(DEV)])), np.lexsort((as_np(k_i32), as_np(k_u8))))
     # along a dimension of a matrix, as the crowding distance uses it (non_dominate.py:221)
