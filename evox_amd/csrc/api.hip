@@ -172,6 +172,7 @@ template <int M, int IW>
 static void launch_dominance_m(const Ws& w, int variant, hipStream_t s) {
   const Layout& L = w.L;
   dim3 grid((L.npad + 255) / 256, (L.nwords + IW - 1) / IW);
+  if (IW == 2) grid = dim3((L.npad + 127) / 128, (L.nwords + 3) / 4);  // a block = two row groups x two tiles
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, w.at<float>(L.xs_sorted), w.at<uint64_t>(L.key_sorted),
                        w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords,
@@ -299,7 +300,7 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s);
 static int dominance_tile_words(const Layout& L) {
   const int tile = opt().dominance_tile_words;
   if (tile != 0) return tile;
-  return L.m >= 3 && L.m <= 8 && L.n <= (L.m >= 6 ? 32768 : 24576) ? 2 : 4;
+  return L.m >= 2 && L.m <= 8 && L.n <= (L.m >= 6 ? 32768 : 24576) ? 2 : 4;
 }
 
 static int stage_dominance(const Ws& w, int variant, hipStream_t s) {
@@ -307,10 +308,10 @@ static int stage_dominance(const Ws& w, int variant, hipStream_t s) {
   if (variant == kDomOrdersOnly) return prefix_dominance_applies(w.L) ? stage_dominance_prefix(w, true, s) : kErrBadArg;
   if (variant == kDomAuto && prefix_dominance_applies(w.L)) return stage_dominance_prefix(w, false, s);
   // (the lower triangle in tiles of 4 words keeps every SIMD busy with several waves; up to about 24 000 rows of
-  // three to eight objectives tiles of 2 words leave a shorter half-empty tail -- measured, us, tiles of 2 / 4:
-  // 5000 x 3: 6.2 / 8.1, 16 000 x 3: 21.9 / 27.1, 20 000 x 3: 30.6 / 34.1, x 5: 47.7 / 54.3, x 8: 67.5 / 80.9,
-  // 24 000 x 3: 41.7 / 42.7, 28 000 x 3: 51.2 / 51.0, x 8: 118.5 / 127.6, 32 768 x 3: 71.5 / 68.2, 50 000 x 3:
-  // 150.5 / 142.8, 20 000 x 2: 26.5 / 24.4 --; 8 and 16 are kept for measurements)
+  // two to eight objectives tiles of 2 words leave a shorter half-empty tail -- measured, us, tiles of 2 / 4:
+  // 5000 x 3: 5.8 / 7.9, 16 000 x 3: 20.3 / 25.7, 20 000 x 2: 20.6 / 23.1, x 3: 27.6 / 31.3, x 8: 64.3 / 80.8,
+  // 24 000 x 3: 38.8 / 39.8, 28 000 x 3: 49.1 / 48.1, x 8: 110.8 / 132.1, 50 000 x 3: 147.5 / 138.4 --; 8 and 16
+  // are kept for measurements)
   const int tile = dominance_tile_words(w.L);
   if (tile >= 16)
     launch_dominance<16>(w, variant, s);

@@ -401,15 +401,20 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
 
 // The tile of block (bx, by): bx = one of ceil(npad / 256) groups of four 64-row waves, by = one of
 // ceil(nwords / IW) column tiles.
+// With tiles of two words the four waves of a block are two groups of rows times two neighbouring tiles: the two
+// 16-byte pieces of a row then reach the cache from the same block at about the same time and leave it as one
+// 32-byte sector (a block of four row groups and one tile wrote 50 MB for the 25 MB triangle of 20 000 x 3).
 template <int M, int IW, int VARIANT>
 __device__ inline void dominance_tile(int bx, int by, const float* __restrict__ xs, const uint64_t* __restrict__ key,
                                       const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom, int n, int npad,
                                       int64_t wstride, int nwords, const SortParam* __restrict__ param) {
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int j = (bx * 4 + wave) * 64 + lane;
+  // (read from the first lane: the tile's first word depends on it, and the dominators are fetched by scalar loads
+  // only at addresses that the compiler knows to be the same in every lane)
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int j = IW == 2 ? (bx * 2 + (wave >> 1)) * 64 + lane : (bx * 4 + wave) * 64 + lane;
   if (j - lane >= npad) return;  // whole wave past the padded population
-  const int w0 = by * IW;
+  const int w0 = IW == 2 ? (by * 2 + (wave & 1)) * IW : by * IW;
   float xj[M];
 #pragma unroll
   for (int k = 0; k < M; ++k) xj[k] = xs[(int64_t)k * npad + j];
@@ -469,7 +474,8 @@ __device__ inline void dominance_tile(int bx, int by, const float* __restrict__ 
   }
 }
 
-// grid.x = ceil(npad / 256) blocks of four 64-row groups, grid.y = ceil(nwords / IW) column tiles.
+// grid.x = ceil(npad / 256) blocks of four 64-row groups, grid.y = ceil(nwords / IW) column tiles (tiles of two words:
+// ceil(npad / 128) blocks of two groups, ceil(nwords / 4) pairs of tiles).
 template <int M, int IW, int VARIANT>
 __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
                                                         const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom, int n,
