@@ -1140,6 +1140,15 @@ def test_lexsort_matches_numpy_and_the_restatement(population_path):
             assert torch.equal(lexsort([k.to(DEV) for k in keys]).cpu(), er.chained_stable_argsort(keys)), (n, "wide")
         # numpy's lexsort on keys without NaN (same convention: last key primary, stable)
         assert np.array_equal(as_np(lexsort([k_i32.to(DEV), k_u8.to(DEV)])), np.lexsort((as_np(k_i32), as_np(k_u8))))
+    # a strided key of a mid-sized sort, and the same sorts through the radix sort (the tunable that sends them there)
+    base = torch.randint(0, 50, (40000,), generator=g).float()
+    strided = base.to(DEV)[::2]
+    assert strided.stride(0) == 2
+    second = torch.randint(0, 5, (20000,), generator=g, dtype=torch.int32)
+    want = er.chained_stable_argsort([base[::2], second])
+    assert torch.equal(lexsort([strided, second.to(DEV)]).cpu(), want)
+    with runtime.options(mid_argsort=0):
+        assert torch.equal(lexsort([strided, second.to(DEV)]).cpu(), want)
     # along a dimension of a matrix, as the crowding distance uses it (non_dominate.py:221)
     c = torch.rand(300, 4, generator=g)
     m = (torch.rand(300, generator=g) < 0.5).float()[:, None].expand(-1, 4).contiguous()
