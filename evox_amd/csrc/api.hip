@@ -325,7 +325,7 @@ static int stage_dominance(const Ws& w, int variant, hipStream_t s) {
   return 0;
 }
 
-static int stage_count(const Ws& w, bool fill_dist, hipStream_t s) {
+static int stage_count(const Ws& w, bool fill_dist, hipStream_t s, bool need_counts) {
   const Layout& L = w.L;
   int blocks = (L.n + 3) / 4;
   const int cap = device_cus() * 8;
@@ -333,7 +333,7 @@ static int stage_count(const Ws& w, bool fill_dist, hipStream_t s) {
   hipLaunchKernelGGL(count_kernel, dim3(blocks), dim3(256), 0, s, w.at<uint64_t>(L.dom), L.wstride, L.n,
                      w.at<int>(L.orig_of), w.at<int>(L.count), w.at<int>(L.rank), w.at<int>(L.witness),
                      w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
-                     fill_dist ? w.at<float>(L.dist) : (float*)nullptr, w.ctrl(), w.at<SortParam>(L.sortparam));
+                     fill_dist ? w.at<float>(L.dist) : (float*)nullptr, w.ctrl(), w.at<SortParam>(L.sortparam), need_counts ? 1 : 0);
   EVX_LAUNCH_CHECK();
   if (prefix_dominance_applies(L)) {
     // the order-based dominance kernel has left the popcounts: count_kernel above returned at once (the choice is
@@ -449,7 +449,8 @@ static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool
 // Counts and peeling for the entry points: one kernel when the matrix fits the LDS of the device, else the count
 // pass over the matrix followed by a peel kernel that rescans rows in memory.
 static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s);
-static int stage_count(const Ws& w, bool fill_dist, hipStream_t s);
+static int stage_count(const Ws& w, bool fill_dist, hipStream_t s, bool need_counts = true);
+static int peel_pass_plan(const Layout& L, int* blocks_out, int* use_witness_out);
 static int count_and_peel(const Ws& w, int64_t stop_count, bool want_perm, bool fill_dist, hipStream_t s,
                           bool order_last_front = false, bool* may_have_ordered = nullptr, bool* always_orders = nullptr) {
   size_t lds = 0;
@@ -471,13 +472,17 @@ static int count_and_peel(const Ws& w, int64_t stop_count, bool want_perm, bool 
     }
     return launch_lds_peel(w, stop_count, want_perm, fill_dist, sweepers, lds, s, order_last_front);
   }
-  if (int e = stage_count(w, fill_dist, s)) return e;
+  // (the witness passes read of a row only its highest dominator: the count stage then walks every row from the top
+  // as far as that, instead of adding up all of it)
+  int blocks = 0, use_witness = 0;
+  if (int e = peel_pass_plan(w.L, &blocks, &use_witness)) return e;
+  if (int e = stage_count(w, fill_dist, s, use_witness == 0)) return e;
   return stage_peel(w, stop_count, want_perm, s);
 }
 
-static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s) {
-  const Layout& L = w.L;
-  if (stop_count < 1 || stop_count > L.n) return kErrBadArg;
+// Grid of the peel kernels that rescan rows in memory, and whether they use the witness pass (else the sweep pass,
+// which needs the popcounts of the rows).
+static int peel_pass_plan(const Layout& L, int* blocks_out, int* use_witness_out) {
   const size_t lds_limit = 160 * 1024 - 4096;
   const size_t bitmap = sizeof(uint64_t) * (size_t)L.nwords;
   const int cus = device_cus();
@@ -508,6 +513,18 @@ static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream
     if (err) return err;
   }
   if (blocks <= kFirstSweeper) return kErrBadArg;
+  *blocks_out = blocks;
+  *use_witness_out = use_witness;
+  return 0;
+}
+
+static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s) {
+  const Layout& L = w.L;
+  if (stop_count < 1 || stop_count > L.n) return kErrBadArg;
+  const size_t bitmap = sizeof(uint64_t) * (size_t)L.nwords;
+  const int cus = device_cus();
+  int blocks = 0, use_witness = 0;
+  if (int e = peel_pass_plan(L, &blocks, &use_witness)) return e;
   if (use_witness && opt().peel_records && L.n <= kRecordsMaxRowsWide) {
     // all-to-all records: 1 lister + a power of two of sweeping blocks, all resident at once
     // by size: 64 blocks up to 32768 rows, 128 above (measured at 20000 rows: 221 us per selection with 64

@@ -174,17 +174,48 @@ __device__ inline RowScan scan_row(const uint64_t* __restrict__ row, int nw, con
 
 // ------------------------------------------------------------------ counts
 
+// The highest non-empty word of a row (-1: the row is empty) by a walk from its top, 128 words a step, that ends at
+// the first step that finds a bit: the witness passes want nothing else of a row, and in slot order a row's highest
+// dominator lies a few dozen words below its own slot.  `total` is 1 or 0 (dominated or not), not the popcount.
+__device__ inline RowScan scan_row_top(const uint64_t* __restrict__ row, int nw) {
+  const int lane = threadIdx.x & 63;
+  RowScan out;
+  out.total = 0;
+  out.last_word = -1;
+  out.last_bits = 0ull;
+  const int limit = (nw + 1) & ~1;
+  for (int base = limit > 0 ? ((limit - 1) >> 7) << 7 : -1; base >= 0; base -= 128) {  // wave-uniform, from the top
+    const int w = base + 2 * lane;
+    const ulonglong2 v = w < limit ? *reinterpret_cast<const ulonglong2*>(row + w) : make_ulonglong2(0ull, 0ull);
+    const uint64_t seen = __builtin_amdgcn_ballot_w64((v.x | v.y) != 0ull);
+    if (seen != 0ull) {
+      const int top = 63 - __builtin_clzll(seen);
+      const int cand_word = v.y != 0ull ? w + 1 : w;
+      const uint64_t cand_bits = v.y != 0ull ? v.y : v.x;
+      out.total = 1;
+      out.last_word = __builtin_amdgcn_readlane(cand_word, top);
+      const uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)cand_bits, top);
+      const uint32_t hi = __builtin_amdgcn_readlane((int)(uint32_t)(cand_bits >> 32), top);
+      out.last_bits = ((uint64_t)hi << 32) | lo;
+      return out;
+    }
+  }
+  return out;
+}
+
 // One wave per row (slot): popcount of the row = the domination count.  Rows with no dominator
 // are rank 0 and form front 0, published both in slot space (for the passes) and in original-index
 // space (for the listing).  witness[j] = the highest non-empty word of row j (-1 for ranked rows).
 // Also fills the crowding-distance output with -inf when one is given.  Ranks are stored by
-// original index.
+// original index.  need_counts = 0 (the peel that follows uses the witness pass): the rows are walked from the top
+// only as far as their first dominator, and count[j] is 1 or 0.
 __global__ __launch_bounds__(256) void count_kernel(const uint64_t* __restrict__ dom, int64_t wstride, int n,
                                                     const int* __restrict__ orig_of, int* __restrict__ count,
                                                     int* __restrict__ rank, int* __restrict__ witness,
                                                     uint64_t* __restrict__ front0_slot, uint64_t* __restrict__ front0_orig,
                                                     int* __restrict__ fsize, float* __restrict__ dist_fill,
-                                                    const Ctrl* __restrict__ ctrl, const SortParam* __restrict__ param) {
+                                                    const Ctrl* __restrict__ ctrl, const SortParam* __restrict__ param,
+                                                    int need_counts) {
   if (ctrl->err != 0) return;  // the slot tables are not valid: leave front 0 empty, nothing gets peeled
   if (param->totals_valid != 0) return;  // count_from_totals_kernel does the work from what the dominance stage left
   __shared__ int block_found;
@@ -195,7 +226,8 @@ __global__ __launch_bounds__(256) void count_kernel(const uint64_t* __restrict__
   const int waves = gridDim.x * (blockDim.x >> 6);
   int found = 0;
   for (int j = blockIdx.x * (blockDim.x >> 6) + wave_in_block; j < n; j += waves) {
-    const RowScan r = scan_row<false>(dom + (int64_t)j * wstride, row_words(j), nullptr);
+    const RowScan r = need_counts ? scan_row<false>(dom + (int64_t)j * wstride, row_words(j), nullptr)
+                                  : scan_row_top(dom + (int64_t)j * wstride, row_words(j));
     if (lane == 0) {
       const int o = orig_of[j];
       count[j] = r.total;
