@@ -30,7 +30,9 @@ namespace evx {
 constexpr int kFusedFrontRows = 2048;
 constexpr int kFusedFrontValues = 4096;  // candidates x objectives held in LDS: 12 bytes each
 constexpr int kFusedFrontObjectives = 64;
-constexpr size_t kFusedFrontLdsBytes = 12 * (size_t)kFusedFrontValues + 4 * (size_t)kFusedFrontRows + 16 * kFusedFrontObjectives;
+constexpr int kFusedSoloRows = 512;       // up to here one workgroup does it all
+constexpr size_t kFusedFrontLdsBytes =
+    12 * (size_t)kFusedFrontValues + 4 * (size_t)kFusedFrontRows + 16 * kFusedFrontObjectives + 4 * (size_t)kFusedSoloRows;
 
 __device__ inline bool fused_front_applies(int nv, int m) {
   return nv <= kFusedFrontRows && (int64_t)nv * m <= kFusedFrontValues && m <= kFusedFrontObjectives;
@@ -48,9 +50,13 @@ __device__ inline void crowd_small_front(const float* __restrict__ xs, int npad,
   float* cost = reinterpret_cast<float*>(comp + kFusedFrontValues);  // [m][nv]
   int* lst = reinterpret_cast<int*>(cost + kFusedFrontValues);       // [nv]
   unsigned long long* ends = reinterpret_cast<unsigned long long*>(lst + kFusedFrontRows);  // [m][2]: first, last composite
-  for (int e = tid; e < nv; e += blockDim.x) lst[e] = list[e];
+  // A front of a few hundred rows is the work of one workgroup: the others would only repeat its loads and then
+  // make it wait for them at the barrier below.
+  const bool solo = nv <= kFusedSoloRows;
   if (mode == 2)  // the better fronts keep the order in which they are listed
     for (int i = blockIdx.x * blockDim.x + tid; i < start; i += gridDim.x * blockDim.x) order[i] = list_base[i];
+  if (solo && blockIdx.x != 0) return;
+  for (int e = tid; e < nv; e += blockDim.x) lst[e] = list[e];
   __syncthreads();
   for (int i = tid; i < nv * m; i += blockDim.x) {
     const int k = i / nv, e = i - k * nv;
@@ -80,7 +86,8 @@ __device__ inline void crowd_small_front(const float* __restrict__ xs, int npad,
     }
   }
   __syncthreads();
-  const int groups = gridDim.x * (blockDim.x >> 4);
+  const int groups = (solo ? 1 : gridDim.x) * (blockDim.x >> 4);
+  uint32_t* dkey_lds = reinterpret_cast<uint32_t*>(ends + 2 * kFusedFrontObjectives);  // [kFusedSoloRows], solo only
   for (int q = blockIdx.x * (blockDim.x >> 4) + (tid >> 4); q < nv; q += groups) {
     bool boundary = false;
     float acc = 0.0f;
@@ -112,12 +119,21 @@ __device__ inline void crowd_small_front(const float* __restrict__ xs, int npad,
     if (sub == 0) {
       const float d = boundary ? INFINITY : acc;
       dist[lst[q]] = d;
-      if (mode == 2) coherent_store(&dkey[q], ordered_key(-d));
+      if (mode == 2) {
+        if (solo)
+          dkey_lds[q] = ordered_key(-d);
+        else
+          coherent_store(&dkey[q], ordered_key(-d));
+      }
     }
   }
   if (mode != 2) return;
   // every block has stored its distance keys: one counter, bounded wait
   __syncthreads();
+  if (solo) {
+    for (int e = tid; e < nv; e += blockDim.x) comp[e] = ((unsigned long long)dkey_lds[e] << 32) | (unsigned)e;
+    __syncthreads();
+  } else {
   if (tid == 0) {
     __hip_atomic_fetch_add(&ctrl->reserved[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const bool seen = bounded_wait([&] { return coherent_load(&ctrl->reserved[0]) >= (int)gridDim.x || coherent_load(&ctrl->err) != 0; },
@@ -129,6 +145,7 @@ __device__ inline void crowd_small_front(const float* __restrict__ xs, int npad,
   if (scratch[0] == 0) return;
   for (int e = tid; e < nv; e += blockDim.x) comp[e] = ((unsigned long long)coherent_load(&dkey[e]) << 32) | (unsigned)e;
   __syncthreads();
+  }
   for (int q = blockIdx.x * (blockDim.x >> 4) + (tid >> 4); q < nv; q += groups) {
     const unsigned long long mine = comp[q];
     int smaller = 0;
