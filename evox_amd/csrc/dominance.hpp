@@ -13,7 +13,7 @@
 // Work split: lane = j (fitness of 64 rows held in VGPRs), loop over i with x[i, :] fetched by
 // scalar loads (the index is wave-uniform), so every `<=` is one v_cmp_le_f32 with an SGPR operand
 // whose result is a 64-lane mask in an SGPR pair; the per-objective masks are ANDed on the scalar
-// unit.  "any strictly less" is replaced by one integer compare: with key(i) = sum_k ordered_key(x[i,k])
+// unit.  "any strictly less" is replaced by one integer compare: with key(i) = sum_k w_k ordered_key(x[i,k]) (positive weights w_k, key_weight below)
 // and all_k(x[i,k] <= x[j,k]) already true (which rules out NaN on both sides), the rows differ in
 // some objective exactly when key(i) != key(j), because the per-objective keys are ordered the same
 // way as the floats and sum without overflow.  The compare is made on a 32-bit stand-in for the key,
@@ -41,6 +41,14 @@
 
 namespace evx {
 
+// The row key of the bucket sort weighs the objectives differently (3, 5, ..., 17, 3, ...).  Any positive weights
+// keep what the key is for -- a dominator's key is strictly smaller, rows equal in every objective have equal keys
+// -- and unequal ones keep the keys of a population that lies on a plane sum_k x[i,k] = const (normalised
+// objectives, a converged front) apart: the integer image of a float is linear in the float within a binade, so
+// with equal weights all rows whose values share their binades would get the same key, thousands of rows in one
+// bucket.  At most 17 * 65535 * 2^32 < 2^53: no overflow.
+__host__ __device__ inline uint32_t key_weight(int k) { return 2u * (uint32_t)(k & 7) + 3u; }
+
 // One kernel turns the caller's strided (n, m) fitness into structure-of-arrays form in original
 // order (padded with NaN to npad, a multiple of 128 rows) plus the 64-bit row keys, leaves the
 // (min, max) key of each block in `partials` for the slot sort, and clears the state arrays that
@@ -67,7 +75,7 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
                       : i < n     ? f2[(i - n_first) * stride_row2 + k * stride_col2]
                                   : __uint_as_float(0x7FC00000u);
       xs[(int64_t)k * npad + i] = v;
-      s += ordered_key(v);
+      s += (uint64_t)key_weight(k) * ordered_key(v);
       bad |= i < n && !(fabsf(v) <= 3.4028234663852886e38f);  // NaN or infinite
     }
     key[i] = s;

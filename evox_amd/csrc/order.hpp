@@ -1,6 +1,6 @@
 // Relabelling of the population by ascending row key ("slots").
 //
-// key(i) = sum_k ordered_key(x[i,k]) is strictly smaller for a dominator than for the row it
+// key(i) = sum_k w_k ordered_key(x[i,k]) (w_k > 0: key_weight in dominance.hpp) is strictly smaller for a dominator than for the row it
 // dominates (every term is <=, one is <, and NaN rows dominate nothing), so after sorting the rows by
 // (key, original index) every dominance pair has slot(i) < slot(j): the bit matrix built in slot
 // space is strictly lower triangular.  That halves the dominance work, bounds every row scan by the

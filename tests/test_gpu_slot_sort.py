@@ -56,6 +56,8 @@ def _cases():
     z = torch.zeros(8000, 2)
     z[::2] = -0.0
     cases["signed_zeros"] = z
+    simplex = torch.rand(20000, 3, generator=g)  # a converged front of normalised objectives: every row sums to one
+    cases["simplex_20000x3"] = simplex / simplex.sum(dim=1, keepdim=True)
     return cases
 
 
@@ -76,12 +78,13 @@ def test_slot_sort_orders_by_key_then_index(name):
     assert np.all((key[1:] > key[:-1]) | ((key[1:] == key[:-1]) & (orig[1:] > orig[:-1])))
     first = np.flatnonzero(np.concatenate([[True], key[1:] != key[:-1]]))
     assert np.array_equal(got["kid_sorted"][:n], np.repeat(first, np.diff(np.concatenate([first, [n]]))).astype(np.int32))
-    # the keys are the sums of the order-preserving integer images of the values (NaN largest, the zeros equal)
+    # the keys are the weighted sums of the order-preserving integer images of the values (NaN largest, the zeros equal)
     u = as_np(f_cpu).view(np.uint32).astype(np.uint64)
     image = np.where(u >> 31 == 1, (~u) & 0xFFFFFFFF, u | 0x80000000)
     image = np.where(as_np(f_cpu) == 0, np.uint64(0x80000000), image)
     image = np.where(np.isnan(as_np(f_cpu)), np.uint64(0xFFFFFFFF), image)
-    assert np.array_equal(key, image.sum(axis=1)[orig])
+    weights = (2 * (np.arange(m) & 7) + 3).astype(np.uint64)  # unequal, so that rows on a plane sum(x) = const keep apart
+    assert np.array_equal(key, (image * weights).sum(axis=1)[orig])
     # the fitness by slot (with -0.0 stored as +0.0) and by original index, NaN behind the n-th row
     want_sorted = (as_np(f_cpu)[orig] + np.float32(0.0)).T
     assert np.array_equal(got["xs_sorted"][:, :n].view(np.uint32), want_sorted.view(np.uint32))
