@@ -588,7 +588,12 @@ static int radix_grid(const Layout& L) {
 // Grid of the two kernels that order the last front (finish.hpp): the radix grid when a front of this
 // population can exceed kRadixMinCandidates rows (they then synchronise across blocks), else one block
 // per 256 candidates and objective.
+// A last front of more than kRadixMinCandidates rows in a population of at most kMidArgsortRows: its orders come from
+// workgroups that sort in LDS without waiting for each other (finish.hpp), one per compute unit.
+static bool crowd_mid_sort(const Layout& L) { return opt().mid_argsort != 0 && L.n > kRadixMinCandidates && L.n <= kMidArgsortRows; }
+
 static int finish_grid(const Layout& L, int per_candidate_block) {
+  if (crowd_mid_sort(L)) return device_cus();  // (their LDS leaves room for one workgroup per compute unit: all resident)
   if (L.n > kRadixMinCandidates) {
     // The kernels choose on the device: a front of at most kRadixMinCandidates rows is still ordered by counting,
     // one work item per 256 candidates (and objective), and wants as many blocks as it has items -- a population
@@ -705,6 +710,7 @@ static CrowdArgs crowd_args(const Ws& w, const int* list, bool use_orders, int f
   a.param = w.at<SortParam>(L.sortparam);
   a.use_orders = use_orders ? 1 : 0;
   a.fused = fused;
+  a.mid_sort = crowd_mid_sort(L) ? 1 : 0;
   a.dist = w.at<float>(L.dist);
   a.dkey = w.at<uint32_t>(L.dkey);
   a.order = w.at<int>(L.order);
@@ -737,6 +743,7 @@ static size_t crowd_lds_bytes(const Layout& L, int fused) {
   size_t lds = sizeof(uint32_t) * kRadixMinCandidates + sizeof(uint64_t) * kRankTile;
   if (L.n > kRadixMinCandidates && kRadixLdsBytes > lds) lds = kRadixLdsBytes;
   if (fused != 0 && kFusedFrontLdsBytes > lds) lds = kFusedFrontLdsBytes;
+  if (crowd_mid_sort(L) && mid_sort_lds_bytes(L.n) > lds) lds = mid_sort_lds_bytes(L.n);
   return lds;
 }
 
@@ -748,12 +755,20 @@ static int stage_crowd_sort(const Ws& w, const int* list, bool use_orders, int f
   if (use_orders)
     if (int e = stage_front_orders(w, list, s)) return e;
   const size_t lds = crowd_lds_bytes(L, fused);
-  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(crowd_sort_kernel), lds)) return e;
+  const bool mid = crowd_mid_sort(L);
+  if (int e = grant_dynamic_lds(mid ? reinterpret_cast<const void*>(crowd_sort_kernel<kMidArgsortThreads>)
+                                    : reinterpret_cast<const void*>(crowd_sort_kernel<kRadixThreads>), lds))
+    return e;
   // (the fused path ends with a barrier between all blocks: the grid must be resident at once, which a grid of at
   // most two blocks of 256 threads per compute unit is)
   int grid = finish_grid(L, L.m);
   if (fused != 0 && grid > device_cus() * 2) grid = device_cus() * 2;
-  hipLaunchKernelGGL(crowd_sort_kernel, dim3(grid), dim3(kRadixThreads), lds, s, crowd_args(w, list, use_orders, fused), after_peel_tail ? 1 : 0);
+  if (mid)
+    hipLaunchKernelGGL(crowd_sort_kernel<kMidArgsortThreads>, dim3(grid), dim3(kMidArgsortThreads), lds, s,
+                       crowd_args(w, list, use_orders, fused), after_peel_tail ? 1 : 0);
+  else
+    hipLaunchKernelGGL(crowd_sort_kernel<kRadixThreads>, dim3(grid), dim3(kRadixThreads), lds, s, crowd_args(w, list, use_orders, fused),
+                       after_peel_tail ? 1 : 0);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -764,8 +779,16 @@ static int stage_crowd_finish(const Ws& w, const int* list, bool want_order, int
   // (no front of this population is too large for the fused path of crowd_sort_kernel: nothing is left to do)
   if (fused != 0 && L.n <= kFusedFrontRows && (int64_t)L.n * L.m <= kFusedFrontValues && L.m <= kFusedFrontObjectives) return 0;
   const size_t lds = crowd_lds_bytes(L, 0);
-  hipLaunchKernelGGL(crowd_finish_kernel, dim3(finish_grid(L, 1)), dim3(kRadixThreads), lds, s, crowd_args(w, list, false, fused),
-                     want_order ? 1 : 0, after_peel_tail ? 1 : 0);
+  const bool mid = crowd_mid_sort(L);
+  if (int e = grant_dynamic_lds(mid ? reinterpret_cast<const void*>(crowd_finish_kernel<kMidArgsortThreads>)
+                                    : reinterpret_cast<const void*>(crowd_finish_kernel<kRadixThreads>), lds))
+    return e;
+  if (mid)
+    hipLaunchKernelGGL(crowd_finish_kernel<kMidArgsortThreads>, dim3(finish_grid(L, 1)), dim3(kMidArgsortThreads), lds, s,
+                       crowd_args(w, list, false, fused), want_order ? 1 : 0, after_peel_tail ? 1 : 0);
+  else
+    hipLaunchKernelGGL(crowd_finish_kernel<kRadixThreads>, dim3(finish_grid(L, 1)), dim3(kRadixThreads), lds, s,
+                       crowd_args(w, list, false, fused), want_order ? 1 : 0, after_peel_tail ? 1 : 0);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -1114,7 +1137,7 @@ static int argsort_step(const void* key, int kind, int64_t stride, int64_t n, co
   }
   if (n <= kMidArgsortRows && opt().mid_argsort) {
     // (one workgroup per compute unit, each producing a run of slots; no workgroup waits for another)
-    const size_t lds = sizeof(uint32_t) * (size_t)n;
+    const size_t lds = mid_sort_lds_bytes((int)n);
     if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(mid_argsort_kernel), lds)) return e;
     const int per = (int)round_up((n + device_cus() - 1) / device_cus(), 16);
     hipLaunchKernelGGL(mid_argsort_kernel, dim3((unsigned)((n + per - 1) / per)), dim3(kMidArgsortThreads), lds, s, key, kind, stride,
@@ -1297,10 +1320,16 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   // the peel kernel may have ordered the last front: one launch for what is left of the ordering (nothing, then),
   // one for the gather
   const size_t lds = crowd_lds_bytes(L, 2);
-  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(crowd_kernel), lds)) return e;
+  const bool mid = crowd_mid_sort(L);
+  if (int e = grant_dynamic_lds(mid ? reinterpret_cast<const void*>(crowd_kernel<kMidArgsortThreads>)
+                                    : reinterpret_cast<const void*>(crowd_kernel<kRadixThreads>), lds))
+    return e;
   int grid = finish_grid(L, L.m);  // resident at once: at most two blocks of 256 threads per compute unit
   if (grid > device_cus() * 2) grid = device_cus() * 2;
-  hipLaunchKernelGGL(crowd_kernel, dim3(grid), dim3(kRadixThreads), lds, s, crowd_args(w, w.at<int>(L.perm), false, 2));
+  if (mid)
+    hipLaunchKernelGGL(crowd_kernel<kMidArgsortThreads>, dim3(grid), dim3(kMidArgsortThreads), lds, s, crowd_args(w, w.at<int>(L.perm), false, 2));
+  else
+    hipLaunchKernelGGL(crowd_kernel<kRadixThreads>, dim3(grid), dim3(kRadixThreads), lds, s, crowd_args(w, w.at<int>(L.perm), false, 2));
   EVX_LAUNCH_CHECK();
   int blocks = (int)((topk + 3) / 4);
   const int cap = device_cus() * 8;

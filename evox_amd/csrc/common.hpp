@@ -4,6 +4,11 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// Hooks for development builds; they compile to nothing in the library.
+#ifndef EVX_TRACE
+#define EVX_TRACE(level, slot)
+#endif
+
 namespace evx {
 
 constexpr int kWave = 64;
@@ -110,7 +115,7 @@ struct Ctrl {
   int listed;       // front bitmaps 0 .. listed-1 have been listed and cleared; polled by the barrier master
   int radix_epoch;  // runs of a radix sort kernel so far: each takes a fresh range of barrier generations
   int tail_done;    // the peel kernel has also left the crowding distances and the order of the last front
-  int reserved[6];  // [0], [1]: arrival counters of the barriers inside the kernels that order the last front;
+  int reserved[6];  // [0], [1], [3]: arrival counters of the barriers inside the kernels that order the last front;
                     // [2]: that of the barriers inside the slot sort
   // grid barrier: block 0 publishes (generation << 32 | rows found by all blocks) in `release` and in
   // kReleaseCopies copies of it, one per 128-byte line, so that the waiting blocks do not all poll one

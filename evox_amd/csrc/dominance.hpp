@@ -41,13 +41,15 @@
 
 namespace evx {
 
-// The row key of the bucket sort weighs the objectives differently (3, 5, ..., 17, 3, ...).  Any positive weights
-// keep what the key is for -- a dominator's key is strictly smaller, rows equal in every objective have equal keys
-// -- and unequal ones keep the keys of a population that lies on a plane sum_k x[i,k] = const (normalised
+// The row key of the bucket sort weighs the objectives slightly differently (16, 17, ..., 23, 16, ...).  Any positive
+// weights keep what the key is for -- a dominator's key is strictly smaller, rows equal in every objective have equal
+// keys -- and unequal ones keep the keys of a population that lies on a plane sum_k x[i,k] = const (normalised
 // objectives, a converged front) apart: the integer image of a float is linear in the float within a binade, so
 // with equal weights all rows whose values share their binades would get the same key, thousands of rows in one
-// bucket.  At most 17 * 65535 * 2^32 < 2^53: no overflow.
-__host__ __device__ inline uint32_t key_weight(int k) { return 2u * (uint32_t)(k & 7) + 3u; }
+// bucket (weights whose odd parts differ never cancel against the binades' powers of two).  Nearly equal, because the
+// peel counts on rows of large key lying in deep fronts (weights 3, 5, 7 cost it 2 us at 20 000 x 3, weights 4, 5, 6 one).  At most
+// 23 * 65535 * 2^32 < 2^53: no overflow.
+__host__ __device__ inline uint32_t key_weight(int k) { return 16u + (uint32_t)(k & 7); }
 
 // One kernel turns the caller's strided (n, m) fitness into structure-of-arrays form in original
 // order (padded with NaN to npad, a multiple of 128 rows) plus the 64-bit row keys, leaves the

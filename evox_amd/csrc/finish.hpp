@@ -178,10 +178,16 @@ struct CrowdArgs {
   unsigned spin_limit;
   SortParam* param;
   int use_orders, fused;
+  int mid_sort;  // fronts of more than kRadixMinCandidates rows are ordered by mid_argsort_slice (the population has at most kMidArgsortRows)
   float* dist;
   uint32_t* dkey;
   int* order;
 };
+
+// Whether a last front of nv rows is ordered by workgroups that sort in LDS (the same answer in every workgroup).
+__device__ inline bool crowd_mid_applies(const CrowdArgs& a, int nv) {
+  return a.mid_sort != 0 && nv > kRadixMinCandidates && nv <= kMidArgsortRows && blockDim.x == kMidArgsortThreads;
+}
 
 // `epochs`: how many epochs of radix barrier generations the control block's counter moves on when the radix path
 // has run (1 when the kernel ends after this body; the merged tail kernel passes 0 and moves the counter itself).
@@ -225,6 +231,25 @@ __device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int ep
     }
     return;
   }
+  if (crowd_mid_applies(a, nv)) {
+    // a workgroup produces a run of positions of one objective's order from the front's keys in its LDS; nobody waits
+    const MidSortLds T = mid_sort_lds(finish_lds);
+    const int nb = (int)gridDim.x;
+    const int per_objective = nb >= m ? nb / m : 1;  // workgroups that share an objective
+    const int run = ((nv + per_objective - 1) / per_objective + 15) & ~15;
+    for (int item = blockIdx.x; item < per_objective * m; item += nb) {
+      const int k = item % m, s0 = (item / m) * run;
+      if (s0 >= nv) continue;
+      const float* __restrict__ col = xs + (int64_t)k * npad;
+      mid_argsort_slice(
+          T, nv, s0, s0 + run, [&](int e) { return ordered_key(col[list[e]]); },
+          [&](int p, int e) {  // (coherent stores: the distances may be worked out later in this same kernel)
+            coherent_store(&pos[(int64_t)k * kstride + e], p);
+            coherent_store(&sorted_cost[(int64_t)k * kstride + p], col[list[e]]);
+          });
+    }
+    return;
+  }
   // radix sort, one segment per objective (the host gave this launch the radix grid)
   if (blockIdx.x == 0) {
     radix_master(ctrl, gen0, 12, spin_limit, scratch);
@@ -251,8 +276,11 @@ __device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int ep
 }
 
 // after_peel_tail: the peel kernel may have ordered the last front already (Ctrl.tail_done).
-__global__ __launch_bounds__(kRadixThreads) void crowd_sort_kernel(CrowdArgs a, int after_peel_tail) {
-  extern __shared__ uint64_t finish_lds[];
+// T threads: kRadixThreads, or kMidArgsortThreads where CrowdArgs.mid_sort is set (the radix sort, which is written for
+// kRadixThreads, does not run then).
+template <int T>
+__global__ __launch_bounds__(T) void crowd_sort_kernel(CrowdArgs a, int after_peel_tail) {
+  extern __shared__ __attribute__((aligned(16))) uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
   if (after_peel_tail != 0 && a.ctrl->tail_done != 0) return;
@@ -359,6 +387,36 @@ __global__ __launch_bounds__(256) void front_order_place_kernel(const unsigned l
   }
 }
 
+// A barrier of all `target` workgroups of a resident grid on the counter Ctrl.reserved[which] (zero at the start of the
+// call; used once).  False when the bounded wait ran out (Ctrl.err is set then).
+// kBarrierFences: the code on either side exchanges its results (positions, sorted costs, distances, the order) through
+// plain stores and loads, which are coherent between kernels but not between the dies of one kernel: the die's L2 is
+// written back before the workgroup arrives and its caches are dropped after it leaves.  A write-back or an
+// invalidation works on the whole cache, whichever wave asks for it, and costs the same every time (1024 threads
+// of 256 workgroups each asking: 65 us per barrier), so one wave of the workgroup asks, once every wave's own stores
+// have arrived in the L2.  kBarrierCoherent: the data is exchanged through coherent stores and loads, nothing else is done.
+// kBarrierDrop: what arrives was stored coherently (written through), and is read by plain loads afterwards: nothing to
+// write back, but the caches are dropped (every workgroup reads all of it: coherent loads would all go to memory).
+enum BarrierKind { kBarrierFences = 0, kBarrierCoherent = 1, kBarrierDrop = 2 };
+template <int KIND = kBarrierFences>
+__device__ inline bool counter_barrier(Ctrl* ctrl, int which, int target, unsigned spin_limit, int* scratch) {
+  constexpr bool FENCES = KIND == kBarrierFences;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    if (FENCES) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __hip_atomic_fetch_add(&ctrl->reserved[which], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool seen = bounded_wait([&] { return coherent_load(&ctrl->reserved[which]) >= target; }, spin_limit);
+    if (!seen) coherent_store(&ctrl->err, kErrBarrierTimeout);
+    scratch[0] = seen;
+    if (FENCES || KIND == kBarrierDrop) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  }
+  __syncthreads();
+  const bool fine = scratch[0] != 0;
+  __syncthreads();  // scratch is reused
+  return fine;
+}
+
 // Crowding distance of every candidate of the last front (written by original index) and, when
 // `want_order` is set, the selection order: the better fronts as listed, then the `need` candidates
 // that come first by (distance descending, NaN after every number, row index) -- jit_fix_operator.py:246-252
@@ -412,6 +470,30 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
     }
     return;
   }
+  if (crowd_mid_applies(a, nv)) {
+    // distances by stripes; then, for the order, every workgroup takes all distance keys into its LDS and produces a
+    // run of the first `need` positions
+    EVX_TRACE(50, 0);
+    for (int q = blockIdx.x * blockDim.x + threadIdx.x; q < nv; q += gridDim.x * blockDim.x) {
+      const float d = crowding_distance_of<true>(q, nv, m, pos, sorted_cost, kstride);
+      dist[list[q]] = d;
+      coherent_store(&dkey[q], ordered_key(-d));
+    }
+    if (!want_order) return;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < start; i += gridDim.x * blockDim.x) order[i] = list_base[i];
+    EVX_TRACE(50, 1);
+    if (!counter_barrier<kBarrierDrop>(ctrl, 3, (int)gridDim.x, spin_limit, scratch)) return;
+    EVX_TRACE(50, 2);
+    const MidSortLds T = mid_sort_lds(finish_lds);
+    const int run = ((need + (int)gridDim.x - 1) / (int)gridDim.x + 15) & ~15;
+    const int s0 = (int)blockIdx.x * run;
+    if (s0 < need)
+      mid_argsort_slice<52>(
+          T, nv, s0, min(need, s0 + run), [&](int e) { return dkey[e]; },
+          [&](int p, int e) { order[start + p] = list[e]; });
+    EVX_TRACE(50, 3);
+    return;
+  }
   // large front: distances by stripes, then (for the order) a grid barrier and the radix sort of their keys
   if (blockIdx.x == 0) {
     if (want_order) {
@@ -443,8 +525,9 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
   }
 }
 
-__global__ __launch_bounds__(kRadixThreads) void crowd_finish_kernel(CrowdArgs a, int want_order, int after_peel_tail) {
-  extern __shared__ uint64_t finish_lds[];
+template <int T>
+__global__ __launch_bounds__(T) void crowd_finish_kernel(CrowdArgs a, int want_order, int after_peel_tail) {
+  extern __shared__ __attribute__((aligned(16))) uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
   if (after_peel_tail != 0 && a.ctrl->tail_done != 0) return;
@@ -456,23 +539,9 @@ __global__ __launch_bounds__(kRadixThreads) void crowd_finish_kernel(CrowdArgs a
 // still costs as much as a small kernel (about 4.7 us on this device), so the two stages share one launch; they are
 // separated by a counter barrier of all blocks.  Grid: that of crowd_sort_kernel (the radix grid: master, idle
 // block, workers), resident at once.
-__device__ inline bool tail_barrier(Ctrl* ctrl, int target, unsigned spin_limit, int* scratch) {
-  // The bodies on either side exchange their results (positions, sorted costs, distances, the order) through plain
-  // stores and loads, which are coherent between kernels but not between the dies of one kernel: every thread writes
-  // its die's L2 back before it arrives and drops what its caches hold after it leaves.
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    __hip_atomic_fetch_add(&ctrl->reserved[1], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const bool seen = bounded_wait([&] { return coherent_load(&ctrl->reserved[1]) >= target; }, spin_limit);
-    if (!seen) coherent_store(&ctrl->err, kErrBarrierTimeout);
-    scratch[0] = seen;
-  }
-  __syncthreads();
-  const bool fine = scratch[0] != 0;
-  __syncthreads();  // scratch is reused
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-  return fine;
+__device__ inline bool tail_barrier(Ctrl* ctrl, int target, unsigned spin_limit, int* scratch, bool coherent_exchange) {
+  return coherent_exchange ? counter_barrier<kBarrierCoherent>(ctrl, 1, target, spin_limit, scratch)
+                           : counter_barrier<kBarrierFences>(ctrl, 1, target, spin_limit, scratch);
 }
 
 __global__ __launch_bounds__(256) void gather_kernel(GatherArgs g) { gather_body(g, blockIdx.x, gridDim.x, 0); }
@@ -483,15 +552,18 @@ __global__ __launch_bounds__(256) void gather_after_peel_kernel(GatherArgs g) {
   gather_body(g, blockIdx.x, gridDim.x, g.ctrl->err == 0 && g.ctrl->tail_done != 0 ? g.ctrl->worst_start : 0);
 }
 
-__global__ __launch_bounds__(kRadixThreads) void crowd_kernel(CrowdArgs a) {
-  extern __shared__ uint64_t finish_lds[];
+template <int T>
+__global__ __launch_bounds__(T) void crowd_kernel(CrowdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
   Ctrl* ctrl = a.ctrl;
   if (coherent_load(&ctrl->err) != 0 || ctrl->tail_done != 0) return;
   const unsigned gen0 = radix_generation_base(ctrl);
   crowd_sort_body(a, gen0, 0, finish_lds, base, scratch);
-  if (tail_barrier(ctrl, (int)gridDim.x, a.spin_limit, scratch)) crowd_finish_body(a, 1, gen0 + 16u, 0, finish_lds, base, scratch);
+  // (the sorts in LDS hand their tables on through coherent stores)
+  if (tail_barrier(ctrl, (int)gridDim.x, a.spin_limit, scratch, crowd_mid_applies(a, ctrl->nv)))
+    crowd_finish_body(a, 1, gen0 + 16u, 0, finish_lds, base, scratch);
   if (blockIdx.x == 0 && threadIdx.x == 0) ctrl->radix_epoch += 2;  // both bodies may have run a radix sort
 }
 

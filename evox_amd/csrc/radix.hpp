@@ -377,37 +377,60 @@ __device__ inline int mid_argsort_scan(int* hist, int* wave_tot) {
   return total;
 }
 
-__global__ __launch_bounds__(kMidArgsortThreads) void mid_argsort_kernel(const void* __restrict__ key, int kind, int64_t stride, int n,
-                                                                         const int* __restrict__ prev, int slots_per_block,
-                                                                         int* __restrict__ order_out) {
-  extern __shared__ uint32_t mid_keys[];  // n order-preserving images of the keys, in the order of the positions
-  __shared__ __attribute__((aligned(16))) int top_hist[kMidArgsortBuckets];  // first-level starts, kept
-  __shared__ __attribute__((aligned(16))) int sub_hist[kMidArgsortBuckets];  // starts of the level below, rebuilt
-  __shared__ unsigned long long list[kMidArgsortList];
+// The tables of a workgroup that sorts in LDS, carved from `bytes` = mid_sort_lds_bytes(n) of it.
+struct MidSortLds {
+  int* top_hist;             // [kMidArgsortBuckets] first-level starts, kept
+  int* sub_hist;             // [kMidArgsortBuckets] starts of the level below, rebuilt
+  unsigned long long* list;  // [kMidArgsortList]
+  uint32_t* red;             // [2][waves]
+  int* wave_tot;             // [waves]
+  int* found;                // [5] bucket of the first wanted slot, its start and end; bucket of the last wanted slot, its end
+  int* list_count;
+  uint32_t* keys;            // [n] order-preserving images of the keys, in the order of the positions
+};
+constexpr size_t kMidSortTableBytes = 2 * sizeof(int) * kMidArgsortBuckets + sizeof(unsigned long long) * kMidArgsortList + 256;
+__host__ __device__ inline size_t mid_sort_lds_bytes(int n) { return kMidSortTableBytes + sizeof(uint32_t) * (size_t)n; }
+__device__ inline MidSortLds mid_sort_lds(void* lds) {  // (16-byte aligned)
   constexpr int kWaves = kMidArgsortThreads / 64;
-  __shared__ uint32_t red[2][kWaves];
-  __shared__ int wave_tot[kWaves];
-  __shared__ int found[5];  // bucket of the first wanted slot, its start and end; bucket of the last wanted slot, its end
-  __shared__ int list_count;
+  MidSortLds t;
+  t.top_hist = static_cast<int*>(lds);
+  t.sub_hist = t.top_hist + kMidArgsortBuckets;
+  t.list = reinterpret_cast<unsigned long long*>(t.sub_hist + kMidArgsortBuckets);
+  t.red = reinterpret_cast<uint32_t*>(t.list + kMidArgsortList);
+  t.wave_tot = reinterpret_cast<int*>(t.red + 2 * kWaves);
+  t.found = t.wave_tot + kWaves;
+  t.list_count = t.found + 5;
+  t.keys = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(lds) + kMidSortTableBytes);
+  return t;
+}
+
+// Slots s0 .. s1-1 of the stable ascending order of n <= kMidArgsortRows 32-bit keys, by one workgroup of
+// kMidArgsortThreads threads that holds all keys in LDS and waits for no other workgroup: key_of(e) = the key of
+// position e (read once), emit(slot, e) = position e belongs in `slot`.  The keys go into kMidArgsortBuckets buckets
+// by value; the buckets that hold the wanted slots are collected (a bucket too large for the list is cut into buckets
+// of its own range first) and their members placed by counting.  Every thread of the workgroup calls it.
+template <int TRACE = 51, class KeyOf, class Emit>
+__device__ inline void mid_argsort_slice(const MidSortLds& T, int n, int s0, int s1_wanted, KeyOf key_of, Emit emit) {
+  uint32_t* const mid_keys = T.keys;
+  int* const top_hist = T.top_hist;
+  int* const sub_hist = T.sub_hist;
+  unsigned long long* const list = T.list;
+  int* const wave_tot = T.wave_tot;
+  int* const found = T.found;
+  constexpr int kWaves = kMidArgsortThreads / 64;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   constexpr unsigned long long kIndexMask = (1ull << kMidArgsortIndexBits) - 1ull;
   uint32_t kmin = 0xFFFFFFFFu, kmax = 0u;
 #pragma unroll 4
   for (int e = tid; e < n; e += kMidArgsortThreads) {
-    const int idx = prev ? prev[e] : e;
-    uint32_t k;
-    if (kind == kKeyFloat32)
-      k = ordered_key(static_cast<const float*>(key)[(int64_t)idx * stride]);
-    else if (kind == kKeyInt32)
-      k = static_cast<const uint32_t*>(key)[(int64_t)idx * stride] ^ 0x80000000u;
-    else
-      k = static_cast<const uint32_t*>(key)[(int64_t)idx * stride];
+    const uint32_t k = key_of(e);
     mid_keys[e] = k;
     kmin = k < kmin ? k : kmin;
     kmax = k > kmax ? k : kmax;
   }
+  EVX_TRACE(TRACE, 0);
   for (int b = tid; b < kMidArgsortBuckets; b += kMidArgsortThreads) top_hist[b] = 0;
-  if (tid == 0) list_count = 0;
+  if (tid == 0) *T.list_count = 0;
   if (tid < 5) found[tid] = 0;
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
@@ -416,14 +439,14 @@ __global__ __launch_bounds__(kMidArgsortThreads) void mid_argsort_kernel(const v
     kmax = b > kmax ? b : kmax;
   }
   if (lane == 0) {
-    red[0][wave] = kmin;
-    red[1][wave] = kmax;
+    T.red[wave] = kmin;
+    T.red[kWaves + wave] = kmax;
   }
   __syncthreads();
 #pragma unroll
   for (int w = 0; w < kWaves; ++w) {
-    kmin = red[0][w] < kmin ? red[0][w] : kmin;
-    kmax = red[1][w] > kmax ? red[1][w] : kmax;
+    kmin = T.red[w] < kmin ? T.red[w] : kmin;
+    kmax = T.red[kWaves + w] > kmax ? T.red[kWaves + w] : kmax;
   }
   auto composite = [&](int e) { return ((unsigned long long)mid_keys[e] << kMidArgsortIndexBits) | (unsigned long long)e; };
   auto shift_for = [](unsigned long long span) {
@@ -437,8 +460,8 @@ __global__ __launch_bounds__(kMidArgsortThreads) void mid_argsort_kernel(const v
   for (int e = tid; e < n; e += kMidArgsortThreads) atomicAdd(&top_hist[(int)((composite(e) - top_lo) >> top_shift)], 1);
   __syncthreads();
   mid_argsort_scan(top_hist, wave_tot);  // (the total is n)
-  const int s0 = (int)blockIdx.x * slots_per_block;
-  const int s1 = min(n, s0 + slots_per_block);
+  EVX_TRACE(TRACE, 1);
+  const int s1 = min(n, s1_wanted);
   // level state: the same in every thread
   unsigned long long lo = top_lo, hi = top_hi;  // the composites of the level: lo .. hi
   int shift = top_shift, base = 0, total = n;
@@ -469,8 +492,11 @@ __global__ __launch_bounds__(kMidArgsortThreads) void mid_argsort_kernel(const v
     __syncthreads();
     const int b0 = found[0], b0_start = found[1], b0_end = found[2];
     int b1 = found[3], b1_end = found[4];
-    if (b1_end - b0_start > kMidArgsortList) {
-      if (b0_end - b0_start > kMidArgsortList) {
+    // Placing the members of the collected buckets costs their number squared: where the keys crowd into a few buckets
+    // (crowding distances do), a bucket many times larger than the run of slots that is wanted from it is cut up first.
+    const int most = min(kMidArgsortList, max(512, 4 * (s1 - x)));
+    if (b1_end - b0_start > most) {
+      if (b0_end - b0_start > most) {
         // that bucket alone is too large: the histogram of its range
         base += b0_start;
         total = b0_end - b0_start;
@@ -495,13 +521,24 @@ __global__ __launch_bounds__(kMidArgsortThreads) void mid_argsort_kernel(const v
     {
       const unsigned long long first = lo + ((unsigned long long)b0 << shift);
       const unsigned long long width = ((unsigned long long)(b1 - b0 + 1) << shift) - 1ull;  // composites first .. first + width
-      for (int e = tid; e < n; e += kMidArgsortThreads) {
-        const unsigned long long c = composite(e);
-        if (c >= first && c - first <= width && c <= hi) list[atomicAdd(&list_count, 1)] = c;
+      // (one addition to the list's counter per wave, not per member: thousands of them to one LDS word take longer
+      // than everything else in a round)
+      for (int e0 = 0; e0 < n; e0 += kMidArgsortThreads) {
+        const int e = e0 + tid;
+        const unsigned long long c = e < n ? composite(e) : 0ull;
+        const bool take = e < n && c >= first && c - first <= width && c <= hi;
+        const unsigned long long takers = __builtin_amdgcn_ballot_w64(take);
+        if (takers != 0ull) {
+          int at = 0;
+          if (lane == 0) at = atomicAdd(T.list_count, __popcll(takers));
+          at = __shfl(at, 0);
+          if (take) list[at + __popcll(takers & ((1ull << lane) - 1ull))] = c;
+        }
       }
     }
     __syncthreads();
-    const int members = list_count;  // = b1_end - b0_start
+    EVX_TRACE(TRACE, 2);
+    const int members = *T.list_count;  // = b1_end - b0_start
     // sixteen lanes per member: each counts over a sixteenth of the list, the shares are added inside the DPP row
     for (int p0 = 0; p0 < members; p0 += kMidArgsortThreads / 16) {
       const int p = p0 + (tid >> 4), sub = tid & 15;
@@ -511,14 +548,11 @@ __global__ __launch_bounds__(kMidArgsortThreads) void mid_argsort_kernel(const v
       for (int q = sub; q < members; q += 16) before += list[q] < c;
       before = group16_sum(before);
       const int slot = base + b0_start + before;
-      if (sub == 0 && p < members && slot >= x && slot < s1) {
-        const int e = (int)(c & kIndexMask);
-        order_out[slot] = prev ? prev[e] : e;
-      }
+      if (sub == 0 && p < members && slot >= x && slot < s1) emit(slot, (int)(c & kIndexMask));
     }
     x = base + b1_end;
     __syncthreads();  // the list and found[] are rewritten
-    if (tid == 0) list_count = 0;
+    if (tid == 0) *T.list_count = 0;
     if (!at_top) {  // back to the first level for the slots that are left
       lo = top_lo;
       hi = top_hi;
@@ -528,6 +562,25 @@ __global__ __launch_bounds__(kMidArgsortThreads) void mid_argsort_kernel(const v
       at_top = true;
     }
   }
+  __syncthreads();
+  EVX_TRACE(TRACE, 3);
+}
+
+// One step of a lexsort of n <= kMidArgsortRows positions: a workgroup per `slots_per_block` slots of the order.
+// Dynamic LDS: mid_sort_lds_bytes(n).
+__global__ __launch_bounds__(kMidArgsortThreads) void mid_argsort_kernel(const void* __restrict__ key, int kind, int64_t stride, int n,
+                                                                         const int* __restrict__ prev, int slots_per_block,
+                                                                         int* __restrict__ order_out) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];
+  const MidSortLds T = mid_sort_lds(mid_lds);
+  auto key_of = [&](int e) -> uint32_t {
+    const int idx = prev ? prev[e] : e;
+    if (kind == kKeyFloat32) return ordered_key(static_cast<const float*>(key)[(int64_t)idx * stride]);
+    if (kind == kKeyInt32) return static_cast<const uint32_t*>(key)[(int64_t)idx * stride] ^ 0x80000000u;
+    return static_cast<const uint32_t*>(key)[(int64_t)idx * stride];
+  };
+  const int s0 = (int)blockIdx.x * slots_per_block;
+  mid_argsort_slice(T, n, s0, s0 + slots_per_block, key_of, [&](int slot, int e) { order_out[slot] = prev ? prev[e] : e; });
 }
 
 // Many independent steps at once: `batch` sorts of n <= kSmallArgsortRows positions each, sort b reading

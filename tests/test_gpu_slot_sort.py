@@ -83,7 +83,7 @@ def test_slot_sort_orders_by_key_then_index(name):
     image = np.where(u >> 31 == 1, (~u) & 0xFFFFFFFF, u | 0x80000000)
     image = np.where(as_np(f_cpu) == 0, np.uint64(0x80000000), image)
     image = np.where(np.isnan(as_np(f_cpu)), np.uint64(0xFFFFFFFF), image)
-    weights = (2 * (np.arange(m) & 7) + 3).astype(np.uint64)  # unequal, so that rows on a plane sum(x) = const keep apart
+    weights = (16 + (np.arange(m) & 7)).astype(np.uint64)  # unequal, so that rows on a plane sum(x) = const keep apart
     assert np.array_equal(key, (image * weights).sum(axis=1)[orig])
     # the fitness by slot (with -0.0 stored as +0.0) and by original index, NaN behind the n-th row
     want_sorted = (as_np(f_cpu)[orig] + np.float32(0.0)).T
