@@ -413,21 +413,33 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
   uint64_t st_bits = 0ull;
   const int my_words = have_row ? row_words((int)my_slot) : 0;
   if (have_row) st_off = row_off[wave * per_wave + lane];
-  for (int top = my_words - 1; __builtin_amdgcn_ballot_w64(st_word < 0 && top >= 0) != 0ull; top -= 8) {
-    uint64_t v[8], a[8];
+  // (no row is ranked yet, so every bit counts; a row is a whole number of 16-byte pieces, read as such; the words
+  // of a step are ORed together first: a row without dominators -- every row of a converged population -- is walked
+  // to its end, at a third of the instructions that looking at every word would take)
+  for (int top = my_words - 1; __builtin_amdgcn_ballot_w64(st_word < 0 && top >= 0) != 0ull; top -= 16) {
+    ulonglong2 v[8];
+    uint64_t any = 0ull;
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
-      const int w = top - q;
+      const int w = top - 1 - 2 * q;  // the piece holds words w and w + 1
       const bool in = st_word < 0 && w >= 0;
-      v[q] = in ? rows_lds[st_off + w] : 0ull;
-      a[q] = in ? alive_lds[w] : 0ull;
+      v[q] = in ? *reinterpret_cast<const ulonglong2*>(rows_lds + st_off + w) : make_ulonglong2(0ull, 0ull);
+      any |= v[q].x | v[q].y;
     }
+    if (__builtin_amdgcn_ballot_w64(any != 0ull) != 0ull) {
 #pragma unroll
-    for (int q = 7; q >= 0; --q)
-      if ((v[q] & a[q]) != 0ull) {
-        st_word = top - q;
-        st_bits = v[q];
+      for (int q = 7; q >= 0; --q) {
+        const int w = top - 1 - 2 * q;
+        if (v[q].x != 0ull) {
+          st_word = w;
+          st_bits = v[q].x;
+        }
+        if (v[q].y != 0ull) {
+          st_word = w + 1;
+          st_bits = v[q].y;
+        }
       }
+    }
   }
   if (have_row && st_word < 0) {  // no dominator: front 0
     const int e = atomicAdd(&sh[0], 1);
