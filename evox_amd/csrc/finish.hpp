@@ -489,7 +489,13 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
     const int s0 = (int)blockIdx.x * run;
     if (s0 < need)
       mid_argsort_slice<52>(
-          T, nv, s0, min(need, s0 + run), [&](int e) { return dkey[e]; },
+          T, nv, s0, min(need, s0 + run),
+          // (the key of an infinite distance lies far below those of the finite ones, which would leave them a twentieth
+          // of the sorter's buckets: any key below that of -m will do for it, a distance being at most m)
+          [&](int e) {
+            const uint32_t k = dkey[e];
+            return k == 0x007FFFFFu /* ordered_key(-inf) */ ? 0x37FFFFFFu /* ordered_key(-131072) */ : k;
+          },
           [&](int p, int e) { order[start + p] = list[e]; });
     EVX_TRACE(50, 3);
     return;
