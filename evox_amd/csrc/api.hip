@@ -588,9 +588,9 @@ static int radix_grid(const Layout& L) {
 // Grid of the two kernels that order the last front (finish.hpp): the radix grid when a front of this
 // population can exceed kRadixMinCandidates rows (they then synchronise across blocks), else one block
 // per 256 candidates and objective.
-// A last front of more than kRadixMinCandidates rows in a population of at most kMidArgsortRows: its orders come from
+// A last front of more than kMidSortMinCandidates rows in a population of at most kMidArgsortRows: its orders come from
 // workgroups that sort in LDS without waiting for each other (finish.hpp), one per compute unit.
-static bool crowd_mid_sort(const Layout& L) { return opt().mid_argsort != 0 && L.n > kRadixMinCandidates && L.n <= kMidArgsortRows; }
+static bool crowd_mid_sort(const Layout& L) { return opt().mid_argsort != 0 && L.n > kMidSortMinCandidates && L.n <= kMidArgsortRows; }
 
 static int finish_grid(const Layout& L, int per_candidate_block) {
   if (crowd_mid_sort(L)) return device_cus();  // (their LDS leaves room for one workgroup per compute unit: all resident)

@@ -185,8 +185,11 @@ struct CrowdArgs {
 };
 
 // Whether a last front of nv rows is ordered by workgroups that sort in LDS (the same answer in every workgroup).
+// Smaller fronts are ranked by counting, which is quadratic: 2000 candidates x 3 objectives took 67 us that way, on
+// the 24 workgroups that the counting keeps busy.
+constexpr int kMidSortMinCandidates = 1024;
 __device__ inline bool crowd_mid_applies(const CrowdArgs& a, int nv) {
-  return a.mid_sort != 0 && nv > kRadixMinCandidates && nv <= kMidArgsortRows && blockDim.x == kMidArgsortThreads;
+  return a.mid_sort != 0 && nv > kMidSortMinCandidates && nv <= kMidArgsortRows && blockDim.x == kMidArgsortThreads;
 }
 
 // `epochs`: how many epochs of radix barrier generations the control block's counter moves on when the radix path
@@ -213,7 +216,7 @@ __device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int ep
   const int* __restrict__ list = list_base + ctrl->worst_start;
   // a large front of a population whose per-objective orders are at hand is ordered by front_order_*_kernel
   if (nv > kRadixMinCandidates && use_orders && param->orders_valid != 0) return;
-  if (nv <= kRadixMinCandidates) {
+  if (nv <= kRadixMinCandidates && !crowd_mid_applies(a, nv)) {
     // ranking by counting: one work item per (256 candidates, objective)
     const int qblocks = (nv + (int)blockDim.x - 1) / (int)blockDim.x;
     for (int item = blockIdx.x; item < qblocks * m; item += gridDim.x) {
@@ -441,7 +444,7 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
   const int start = ctrl->worst_start;
   const int need = ctrl->need;
   const int* __restrict__ list = list_base + start;
-  if (nv <= kRadixMinCandidates) {
+  if (nv <= kRadixMinCandidates && !crowd_mid_applies(a, nv)) {
     // every block derives the distance keys of all candidates in LDS (a few thousand table look-ups);
     // block 0 also stores the distances
     uint32_t* dkey_lds = reinterpret_cast<uint32_t*>(finish_lds);

@@ -1,4 +1,4 @@
-"""Last fronts of more than 8192 rows in populations of at most 24 576 rows -- a converged population, where most
+"""Last fronts of more than 1024 rows in populations of at most 24 576 rows -- a converged population, where most
 rows are non-dominated -- whose per-objective orders and distance order come from workgroups that sort in LDS: against
 the plain-C checker, against the radix path (option ``mid_argsort`` off), and ``crowding_distance`` on masks of that
 size.  Ties in an objective (equal costs keep their row order), duplicate rows, a NaN objective, the largest
@@ -38,6 +38,11 @@ def _cases():
     cases["two_objectives_9000_smallest_of_the_path"] = (torch.stack([a, -a], dim=1), [4500])
     wide = _simplex(9000, 16, g)
     cases["simplex_9000x16"] = (wide, [4500])
+    cases["simplex_2000x3"] = (_simplex(2000, 3, g), [1, 1000, 2000])
+    cases["simplex_5000x4"] = (_simplex(5000, 4, g), [2500])
+    small = _simplex(3000, 3, g)
+    small[1100:] = small[1100:] * 1.5 + 0.1  # a front of 1100 rows, just above the smallest that is sorted this way
+    cases["front0_1100_of_3000x3"] = (small, [1000])
     return cases
 
 
@@ -64,7 +69,7 @@ def test_large_last_front_against_the_c_checker_and_the_radix_path(name):
     for k in ks:
         got = nd_environmental_selection(x, fd, k)
         st = runtime.last_status()
-        assert st["error"] == 0 and st["last_front_size"] > 8192, st
+        assert st["error"] == 0 and st["last_front_size"] > 1024, st
         _check(f, k, got, name)
         with runtime.options(mid_argsort=0):
             old = nd_environmental_selection(x, fd, k)
