@@ -336,6 +336,17 @@ def next_rows(dev, reps):
         "rank_until_us": event_time_us(lambda: non_dominate_rank_until(f, w.topk + 1), reps),
         "full_rank_us": event_time_us(lambda: non_dominate_rank(f), reps),
     }
+    # a converged population: every row on one front (the unit simplex), so the whole selection is the ordering of that
+    # front by crowding distance -- what a run looks like once the front is found, which uniform fitness never shows
+    for n, m in ((2000, 3), (20000, 3), (20000, 2), (50000, 3)):
+        g = torch.Generator("cpu").manual_seed(5)
+        fc = torch.rand(n, m, generator=g)
+        fc = (fc / fc.sum(dim=1, keepdim=True)).to(dev)
+        xc = torch.rand(n, 16, device=dev)
+        nd_environmental_selection(xc, fc, n // 2)
+        out[f"converged one front N={n} M={m} topk={n // 2}"] = {
+            "us": event_time_us(lambda: nd_environmental_selection(xc, fc, n // 2), reps)}
+        del fc, xc
     # lexsort as a function of its own: HypE's lexsort([-dis, rank]) over the merged population
     full_rank = non_dominate_rank(f)
     key = torch.rand(f.size(0), device=dev)

@@ -25,35 +25,43 @@ namespace evx {
 __global__ __launch_bounds__(1024) void compact_mask_kernel(const uint8_t* __restrict__ mask, int64_t mask_stride, int n,
                                                             int* __restrict__ list, float* __restrict__ dist,
                                                             Ctrl* __restrict__ ctrl) {
+  // A wave takes a run of consecutive rows, 64 at a time: it counts its selected rows (loads that depend on nothing:
+  // several in flight), the runs' counts are added up once, and a second walk writes the list.  (One step of 1024
+  // rows at a time with the running total handed on through LDS cost three barriers and a memory round trip per
+  // step: 21 us for 20 000 rows.)
   __shared__ int wave_tot[16];
-  __shared__ int running;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  if (threadIdx.x == 0) running = 0;
+  const int waves = blockDim.x >> 6;
+  const int per_wave = ((n + waves - 1) / waves + 63) & ~63;
+  const int r0 = wave * per_wave, r1 = min(n, r0 + per_wave);
+  auto selected = [&](int j) { return j < r1 && (mask == nullptr || mask[(int64_t)j * mask_stride] != 0); };
+  int count = 0;
+#pragma unroll 4
+  for (int j0 = r0; j0 < r1; j0 += 64) {
+    const int j = j0 + lane;
+    if (j < r1) dist[j] = -INFINITY;
+    count += __popcll(__builtin_amdgcn_ballot_w64(selected(j)));
+  }
+  if (lane == 0) wave_tot[wave] = count;
   __syncthreads();
-  for (int base = 0; base < n; base += blockDim.x) {
-    const int j = base + threadIdx.x;
-    const bool on = j < n && (mask == nullptr || mask[j * mask_stride] != 0);
-    if (j < n) dist[j] = -INFINITY;
+  int offset = 0, total = 0;
+  for (int w = 0; w < waves; ++w) {
+    if (w < wave) offset += wave_tot[w];
+    total += wave_tot[w];
+  }
+#pragma unroll 4
+  for (int j0 = r0; j0 < r1; j0 += 64) {
+    const int j = j0 + lane;
+    const bool on = selected(j);
     const uint64_t b = __builtin_amdgcn_ballot_w64(on);
-    const int before = __popcll(b & ((1ull << lane) - 1ull));
-    if (lane == 0) wave_tot[wave] = __popcll(b);
-    __syncthreads();
-    int offset = running;
-    for (int w = 0; w < wave; ++w) offset += wave_tot[w];
-    if (on) list[offset + before] = j;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      int t = 0;
-      for (int w = 0; w < (int)(blockDim.x >> 6); ++w) t += wave_tot[w];
-      running += t;
-    }
-    __syncthreads();
+    if (on) list[offset + __popcll(b & ((1ull << lane) - 1ull))] = j;
+    offset += __popcll(b);
   }
   if (threadIdx.x == 0) {
     ctrl->worst_start = 0;
-    ctrl->nv = running;
-    ctrl->need = running;
+    ctrl->nv = total;
+    ctrl->need = total;
   }
 }
 
