@@ -534,7 +534,11 @@ __device__ inline void scan_up_to_four(const uint64_t* const (&rows)[4], const i
   if (cnt > 2 && short_rows) {
     scan_rows_highest<4, 4>(rows, nws, alive_lds, r);
   } else {
-    for (int q0 = 0; q0 < cnt; q0 += 2) {
+    // (unrolled, so that the arrays are indexed by constants: indexed at run time they would live in scratch memory,
+    // a round trip to memory in every rescan)
+#pragma unroll
+    for (int q0 = 0; q0 < 4; q0 += 2) {
+      if (q0 >= cnt) break;
       const uint64_t* const two[2] = {rows[q0], rows[q0 + 1]};
       const int nw2[2] = {nws[q0], nws[q0 + 1]};
       RowScan r2[2];

@@ -86,8 +86,10 @@ __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, in
   int dummy = 0;
   for (int pass = 0; pass < 4; ++pass) {
     const int shift = 8 * pass;
-    const unsigned long long* __restrict__ in = buf.pairs[pass & 1];
-    unsigned long long* __restrict__ out = buf.pairs[(pass + 1) & 1];
+    // (chosen, not indexed: an array indexed at run time lives in scratch memory, which every lane of every kernel that
+    // holds a RadixBuffers then writes when it starts -- 10 MB per launch of the 1024-thread ordering kernel)
+    const unsigned long long* __restrict__ in = (pass & 1) ? buf.pairs[1] : buf.pairs[0];
+    unsigned long long* __restrict__ out = (pass & 1) ? buf.pairs[0] : buf.pairs[1];
     auto fetch = [&](int k, int e) { return pass == 0 ? initial(k, e) : coherent_load(&in[(int64_t)k * buf.kstride + e]); };
     // ---- 1. digit counts of every chunk (kRadixBatch pairs per lane are fetched before any is used: the coherent
     // loads of a wave are then in flight together instead of costing a memory round trip each)
