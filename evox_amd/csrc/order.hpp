@@ -74,8 +74,22 @@ __global__ __launch_bounds__(256) void bucket_hist_kernel(const uint64_t* __rest
   __shared__ unsigned long long lds2[3];
   const SortParam sp = make_sort_param(partials, nparts, buckets, lds2);
   if (blockIdx.x == 0 && threadIdx.x == 0) *param_out = sp;
-  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
-    atomicAdd(&hist[bucket_of(key[i], sp)], 1);
+  const int lane = threadIdx.x & 63;
+  for (int i0 = blockIdx.x * blockDim.x; i0 < n; i0 += gridDim.x * blockDim.x) {
+    const int i = i0 + threadIdx.x;
+    const int b = i < n ? bucket_of(key[i], sp) : -1;
+    // Thousands of equal rows (a penalty value for every infeasible row, say) meet in one bucket: the lanes of a wave
+    // that share a bucket with one of its first three lanes send one addition between them, so that the additions to
+    // a crowded bucket do not queue up one by one (20 000 equal rows: 229 us otherwise).
+    uint64_t todo = __builtin_amdgcn_ballot_w64(b >= 0);
+    for (int round = 0; round < 3 && todo != 0ull; ++round) {
+      const int leader = __builtin_amdgcn_readlane(b, __ffsll((unsigned long long)todo) - 1);
+      const uint64_t same = __builtin_amdgcn_ballot_w64(b == leader) & todo;
+      if (lane == __ffsll((unsigned long long)same) - 1) atomicAdd(&hist[leader], __popcll(same));
+      todo &= ~same;
+    }
+    if ((todo >> lane) & 1ull) atomicAdd(&hist[b], 1);
+  }
 }
 
 // start[b] = exclusive prefix of hist, start[buckets] = n; cursor = copy of start.
@@ -145,13 +159,48 @@ __global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint64_t* __r
                                                              const Ctrl* __restrict__ ctrl) {
   if (ctrl->err != 0) return;
   const SortParam sp = *param;
-  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
-    const uint64_t ki = key[i];
-    const int p = atomicAdd(&cursor[bucket_of(ki, sp)], 1);
-    members[p] = i;
-    member_key[p] = ki;  // beside the index, so that the placing kernel reads a bucket without a dependent load
+  const int lane = threadIdx.x & 63;
+  for (int i0 = blockIdx.x * blockDim.x; i0 < n; i0 += gridDim.x * blockDim.x) {
+    const int i = i0 + threadIdx.x;
+    const uint64_t ki = i < n ? key[i] : 0ull;
+    const int b = i < n ? bucket_of(ki, sp) : -1;
+    // (as in the histogram: the lanes that share a bucket with one of the wave's first three take their places with
+    // one addition between them; the groups are found first and all additions go out together, so that the wave waits
+    // for one round trip to memory, as it did with one addition per lane)
+    uint64_t todo = __builtin_amdgcn_ballot_w64(b >= 0);
+    uint64_t group[3] = {0ull, 0ull, 0ull};
+    int first[3] = {0, 0, 0};
+#pragma unroll
+    for (int round = 0; round < 3; ++round) {
+      if (todo == 0ull) break;
+      const int leader = __builtin_amdgcn_readlane(b, __ffsll((unsigned long long)todo) - 1);
+      group[round] = __builtin_amdgcn_ballot_w64(b == leader) & todo;
+      first[round] = __ffsll((unsigned long long)group[round]) - 1;
+      todo &= ~group[round];
+    }
+    const uint64_t me = 1ull << lane;
+    int count = (todo & me) ? 1 : 0;  // a lane of no group adds for itself
+#pragma unroll
+    for (int round = 0; round < 3; ++round)
+      if (group[round] != 0ull && lane == first[round]) count = __popcll(group[round]);
+    int at = 0;
+    if (count != 0) at = atomicAdd(&cursor[b], count);
+    int p = at;
+#pragma unroll
+    for (int round = 0; round < 3; ++round) {
+      if (group[round] == 0ull) continue;
+      const int base = __builtin_amdgcn_readlane(at, first[round]);
+      if (group[round] & me) p = base + __popcll(group[round] & (me - 1ull));
+    }
+    if (i < n) {
+      members[p] = i;
+      member_key[p] = ki;  // beside the index, so that the placing kernel reads a bucket without a dependent load
+    }
   }
 }
+
+constexpr int kPlaceLarge = 512;  // a bucket of more members goes through LDS once per workgroup, not through memory once per row
+constexpr int kPlaceTile = 1024;  // its members in LDS at a time
 
 // Exact slot of every row: bucket start + number of bucket members that precede it by (key, index).
 // Writes the slot-ordered copies of the fitness (structure of arrays, NaN padding up to npad), of
@@ -165,18 +214,71 @@ __global__ __launch_bounds__(256) void bucket_place_kernel(const float* __restri
                                                            int* __restrict__ slot_of, const Ctrl* __restrict__ ctrl) {
   if (ctrl->err != 0) return;
   const SortParam sp = *param;
+  __shared__ __attribute__((aligned(16))) uint64_t tile[kPlaceTile];
+  __shared__ int next_big;
   // A thread takes the row at its position in the bucket-ordered member list, not the row of its own index: the
   // lanes of a wave then walk through the same one or two buckets (their loads fall into the same lines instead of
   // 64 lists apart) and write neighbouring slots; only the reads of the row's fitness are scattered.
-  for (int t = blockIdx.x * blockDim.x + threadIdx.x; t < npad; t += gridDim.x * blockDim.x) {
+  for (int t0 = blockIdx.x * blockDim.x; t0 < npad; t0 += gridDim.x * blockDim.x) {
+    const int t = t0 + threadIdx.x;
+    // Rows of a bucket of more than kPlaceLarge members (thousands of equal rows: a penalty value for every
+    // infeasible row, say): the workgroup takes the bucket through LDS, a tile at a time, as composites
+    // (key - first key of the bucket) << 32 | row, and every thread counts for its own row: one 64-bit and one 32-bit
+    // comparison per member, the members read eight at a time as 16-byte pieces that all lanes share -- a pass over the
+    // bucket per workgroup instead of one per thread, each of them a chain of memory round trips (20 000 equal
+    // rows: 2.3 ms that way).  (Buckets wider than 2^32 keys keep the walk per thread.)
+    int before = 0, smaller = 0;
+    bool counted = false;
+    int i = 0, b = -1, lo = 0, hi = 0;
+    uint64_t ki = 0ull;
     if (t < n) {
-      const int i = members[t];
-      const uint64_t ki = member_key[t];
-      const int b = bucket_of(ki, sp);
-      const int lo = start[b], hi = start[b + 1];
-      int before = 0, smaller = 0;
+      i = members[t];
+      ki = member_key[t];
+      b = bucket_of(ki, sp);
+      lo = start[b];
+      hi = start[b + 1];
+    }
+    if (sp.shift <= 32) {
+      const bool big = hi - lo > kPlaceLarge;
+      int done_below = -1;  // large buckets up to this one are done (the rows of a workgroup lie in ascending buckets)
+      while (__syncthreads_or(big && b > done_below)) {
+        __syncthreads();
+        if (threadIdx.x == 0) next_big = 0x7FFFFFFF;
+        __syncthreads();
+        if (big && b > done_below) atomicMin(&next_big, b);
+        __syncthreads();
+        const int bb = next_big;
+        if (bb == 0x7FFFFFFF) break;
+        const int blo = start[bb], bhi = start[bb + 1];
+        const uint64_t first_key = sp.kmin + ((uint64_t)bb << sp.shift);
+        const bool mine = big && b == bb;
+        const uint64_t ci = ((ki - first_key) << 32) | (uint32_t)i;
+        const uint32_t ci_key = (uint32_t)(ci >> 32);
+        for (int p0 = blo; p0 < bhi; p0 += kPlaceTile) {
+          __syncthreads();
+          for (int e = threadIdx.x; e < kPlaceTile; e += blockDim.x)
+            tile[e] = p0 + e < bhi ? ((member_key[p0 + e] - first_key) << 32) | (uint32_t)members[p0 + e] : ~0ull;
+          __syncthreads();
+          if (mine) {
+            for (int e0 = 0; e0 < kPlaceTile; e0 += 8) {
+              ulonglong2 c[4];
+#pragma unroll
+              for (int u = 0; u < 4; ++u) c[u] = *reinterpret_cast<const ulonglong2*>(&tile[e0 + 2 * u]);
+#pragma unroll
+              for (int u = 0; u < 4; ++u) {
+                before += (c[u].x < ci ? 1 : 0) + (c[u].y < ci ? 1 : 0);
+                smaller += ((uint32_t)(c[u].x >> 32) < ci_key ? 1 : 0) + ((uint32_t)(c[u].y >> 32) < ci_key ? 1 : 0);
+              }
+            }
+          }
+        }
+        if (mine) counted = true;
+        done_below = bb;
+      }
+    }
+    if (t < n) {
       // eight members at a time, all loads before any use (a bucket of a clustered population holds dozens of rows)
-      for (int p0 = lo; p0 < hi; p0 += 8) {
+      for (int p0 = counted ? hi : lo; p0 < hi; p0 += 8) {
         int e[8];
         uint64_t ke[8];
 #pragma unroll
@@ -198,7 +300,7 @@ __global__ __launch_bounds__(256) void bucket_place_kernel(const float* __restri
       kid_sorted[slot] = (uint32_t)(lo + smaller);  // first slot holding this key: equal ids <=> equal keys
       // -0.0 is stored as +0.0: every comparison reads the same, and differences of equal values are +0.0
       for (int k = 0; k < m; ++k) xs_sorted[(int64_t)k * npad + slot] = xs[(int64_t)k * npad + i] + 0.0f;
-    } else {
+    } else if (t < npad) {
       orig_of[t] = -1;
       key_sorted[t] = ~0ull;
       kid_sorted[t] = (uint32_t)t;

@@ -40,6 +40,8 @@ def _cases():
     two = torch.rand(20000, 3, generator=g)
     two[:9000] = 0.5  # one key with 9000 rows among 11000 distinct ones
     cases["one_large_tie_group"] = two[torch.randperm(20000, generator=g)]
+    cases["tie_group_in_the_first_rows"] = two.clone()  # whole waves of equal rows, then whole waves of distinct ones
+    cases["all_equal_20001x2"] = torch.full((20001, 2), -3.0)  # (the padding behind the last row belongs to half a workgroup)
     ties = torch.randint(0, 3, (30000, 2), generator=g).float()  # five distinct keys
     cases["five_keys_30000x2"] = ties
     cl = torch.rand(25000, 3, generator=g) * 1e-6 + 0.5  # keys within a sliver of the range ...
