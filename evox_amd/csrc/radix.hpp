@@ -509,16 +509,46 @@ __device__ inline void mid_argsort_slice(const MidSortLds& T, int n, int s0, int
         at_top = false;
         for (int b = tid; b < kMidArgsortBuckets; b += kMidArgsortThreads) sub_hist[b] = 0;
         __syncthreads();
-        for (int e = tid; e < n; e += kMidArgsortThreads) {
-          const unsigned long long c = composite(e);
-          if (c >= lo && c - lo <= span) atomicAdd(&sub_hist[(int)((c - lo) >> shift)], 1);
+        for (int e0 = 0; e0 < n; e0 += kMidArgsortThreads) {
+          const int e = e0 + tid;
+          const unsigned long long c = e < n ? composite(e) : 0ull;
+          const bool in = e < n && c >= lo && c - lo <= span;
+          const int b = in ? (int)((c - lo) >> shift) : -1;
+          // (thousands of equal keys -- what makes a bucket too large in the first place -- fall into one bucket of
+          // this level too, and additions to one LDS word are carried out one after the other: where all lanes of the
+          // wave that have a key in the range have the same bucket, one of them adds for all)
+          const uint64_t ins = __builtin_amdgcn_ballot_w64(in);
+          if (ins != 0ull) {
+            const int lead = __ffsll((unsigned long long)ins) - 1;
+            const int b_lead = __builtin_amdgcn_readlane(b, lead);
+            if (__builtin_amdgcn_ballot_w64(in && b == b_lead) == ins) {
+              if (lane == lead) atomicAdd(&sub_hist[b_lead], __popcll(ins));
+            } else if (in) {
+              atomicAdd(&sub_hist[b], 1);
+            }
+          }
         }
         __syncthreads();
         mid_argsort_scan(sub_hist, wave_tot);
         continue;
       }
-      b1 = b0;
-      b1_end = b0_end;
+      // as many buckets from b0 on as the list takes (not b0 alone: where the run of wanted slots ends in a bucket of
+      // thousands of equal keys, every round would place one small bucket): the last bucket that ends in time
+      __syncthreads();  // (everybody has read found[])
+      constexpr int kPer = kMidArgsortBuckets / kMidArgsortThreads;
+#pragma unroll
+      for (int u = 0; u < kPer; ++u) {
+        const int b = u * kMidArgsortThreads + tid;
+        const int en = b + 1 < kMidArgsortBuckets ? hist[b + 1] : total;
+        const int en_next = b + 2 < kMidArgsortBuckets ? hist[b + 2] : total;
+        if (b >= b0 && en - b0_start <= most && (en_next - b0_start > most || b + 1 >= kMidArgsortBuckets)) {
+          found[3] = b;
+          found[4] = en;
+        }
+      }
+      __syncthreads();
+      b1 = found[3];
+      b1_end = found[4];
     }
     {
       const unsigned long long first = lo + ((unsigned long long)b0 << shift);
@@ -555,7 +585,9 @@ __device__ inline void mid_argsort_slice(const MidSortLds& T, int n, int s0, int
     x = base + b1_end;
     __syncthreads();  // the list and found[] are rewritten
     if (tid == 0) *T.list_count = 0;
-    if (!at_top) {  // back to the first level for the slots that are left
+    // back to the first level for the slots that are left, unless the next of them lies in the range of this level too
+    // (its histogram is still there: a run of slots inside thousands of equal keys is cut up once, not once per round)
+    if (!at_top && !(x < base + total)) {
       lo = top_lo;
       hi = top_hi;
       shift = top_shift;
