@@ -371,7 +371,7 @@ static int peel_blocks_per_cu(size_t lds, int* err) {
 }
 
 static int grant_dynamic_lds(const void* kernel, size_t lds) {
-  if (lds > 150 * 1024) return kErrBadArg;
+  if (lds > 160 * 1024) return kErrBadArg;  // (what a workgroup of this device can have)
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
@@ -756,19 +756,24 @@ static int stage_crowd_sort(const Ws& w, const int* list, bool use_orders, int f
     if (int e = stage_front_orders(w, list, s)) return e;
   const size_t lds = crowd_lds_bytes(L, fused);
   const bool mid = crowd_mid_sort(L);
-  if (int e = grant_dynamic_lds(mid ? reinterpret_cast<const void*>(crowd_sort_kernel<kMidArgsortThreads>)
-                                    : reinterpret_cast<const void*>(crowd_sort_kernel<kRadixThreads>), lds))
-    return e;
+  const bool wide = L.n <= kMidArgsortWideRows;  // (which tables of the LDS sorter the population leaves room for)
+  const void* const kernel = !mid ? reinterpret_cast<const void*>(crowd_sort_kernel<kRadixThreads, 0>)
+                             : wide ? reinterpret_cast<const void*>(crowd_sort_kernel<kMidArgsortThreads, 1>)
+                                    : reinterpret_cast<const void*>(crowd_sort_kernel<kMidArgsortThreads, 2>);
+  if (int e = grant_dynamic_lds(kernel, lds)) return e;
   // (the fused path ends with a barrier between all blocks: the grid must be resident at once, which a grid of at
   // most two blocks of 256 threads per compute unit is)
   int grid = finish_grid(L, L.m);
   if (fused != 0 && grid > device_cus() * 2) grid = device_cus() * 2;
-  if (mid)
-    hipLaunchKernelGGL(crowd_sort_kernel<kMidArgsortThreads>, dim3(grid), dim3(kMidArgsortThreads), lds, s,
+  if (mid && wide)
+    hipLaunchKernelGGL((crowd_sort_kernel<kMidArgsortThreads, 1>), dim3(grid), dim3(kMidArgsortThreads), lds, s,
+                       crowd_args(w, list, use_orders, fused), after_peel_tail ? 1 : 0);
+  else if (mid)
+    hipLaunchKernelGGL((crowd_sort_kernel<kMidArgsortThreads, 2>), dim3(grid), dim3(kMidArgsortThreads), lds, s,
                        crowd_args(w, list, use_orders, fused), after_peel_tail ? 1 : 0);
   else
-    hipLaunchKernelGGL(crowd_sort_kernel<kRadixThreads>, dim3(grid), dim3(kRadixThreads), lds, s, crowd_args(w, list, use_orders, fused),
-                       after_peel_tail ? 1 : 0);
+    hipLaunchKernelGGL((crowd_sort_kernel<kRadixThreads, 0>), dim3(grid), dim3(kRadixThreads), lds, s,
+                       crowd_args(w, list, use_orders, fused), after_peel_tail ? 1 : 0);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -780,14 +785,19 @@ static int stage_crowd_finish(const Ws& w, const int* list, bool want_order, int
   if (fused != 0 && L.n <= kFusedFrontRows && (int64_t)L.n * L.m <= kFusedFrontValues && L.m <= kFusedFrontObjectives) return 0;
   const size_t lds = crowd_lds_bytes(L, 0);
   const bool mid = crowd_mid_sort(L);
-  if (int e = grant_dynamic_lds(mid ? reinterpret_cast<const void*>(crowd_finish_kernel<kMidArgsortThreads>)
-                                    : reinterpret_cast<const void*>(crowd_finish_kernel<kRadixThreads>), lds))
-    return e;
-  if (mid)
-    hipLaunchKernelGGL(crowd_finish_kernel<kMidArgsortThreads>, dim3(finish_grid(L, 1)), dim3(kMidArgsortThreads), lds, s,
+  const bool wide = L.n <= kMidArgsortWideRows;
+  const void* const kernel = !mid ? reinterpret_cast<const void*>(crowd_finish_kernel<kRadixThreads, 0>)
+                             : wide ? reinterpret_cast<const void*>(crowd_finish_kernel<kMidArgsortThreads, 1>)
+                                    : reinterpret_cast<const void*>(crowd_finish_kernel<kMidArgsortThreads, 2>);
+  if (int e = grant_dynamic_lds(kernel, lds)) return e;
+  if (mid && wide)
+    hipLaunchKernelGGL((crowd_finish_kernel<kMidArgsortThreads, 1>), dim3(finish_grid(L, 1)), dim3(kMidArgsortThreads), lds, s,
+                       crowd_args(w, list, false, fused), want_order ? 1 : 0, after_peel_tail ? 1 : 0);
+  else if (mid)
+    hipLaunchKernelGGL((crowd_finish_kernel<kMidArgsortThreads, 2>), dim3(finish_grid(L, 1)), dim3(kMidArgsortThreads), lds, s,
                        crowd_args(w, list, false, fused), want_order ? 1 : 0, after_peel_tail ? 1 : 0);
   else
-    hipLaunchKernelGGL(crowd_finish_kernel<kRadixThreads>, dim3(finish_grid(L, 1)), dim3(kRadixThreads), lds, s,
+    hipLaunchKernelGGL((crowd_finish_kernel<kRadixThreads, 0>), dim3(finish_grid(L, 1)), dim3(kRadixThreads), lds, s,
                        crowd_args(w, list, false, fused), want_order ? 1 : 0, after_peel_tail ? 1 : 0);
   EVX_LAUNCH_CHECK();
   return 0;
@@ -1138,10 +1148,17 @@ static int argsort_step(const void* key, int kind, int64_t stride, int64_t n, co
   if (n <= kMidArgsortRows && opt().mid_argsort) {
     // (one workgroup per compute unit, each producing a run of slots; no workgroup waits for another)
     const size_t lds = mid_sort_lds_bytes((int)n);
-    if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(mid_argsort_kernel), lds)) return e;
+    const bool wide = n <= kMidArgsortWideRows;
+    if (int e = grant_dynamic_lds(wide ? reinterpret_cast<const void*>(mid_argsort_kernel<true>)
+                                       : reinterpret_cast<const void*>(mid_argsort_kernel<false>), lds))
+      return e;
     const int per = (int)round_up((n + device_cus() - 1) / device_cus(), 16);
-    hipLaunchKernelGGL(mid_argsort_kernel, dim3((unsigned)((n + per - 1) / per)), dim3(kMidArgsortThreads), lds, s, key, kind, stride,
-                       (int)n, prev_order, per, order_out);
+    if (wide)
+      hipLaunchKernelGGL(mid_argsort_kernel<true>, dim3((unsigned)((n + per - 1) / per)), dim3(kMidArgsortThreads), lds, s, key, kind,
+                         stride, (int)n, prev_order, per, order_out);
+    else
+      hipLaunchKernelGGL(mid_argsort_kernel<false>, dim3((unsigned)((n + per - 1) / per)), dim3(kMidArgsortThreads), lds, s, key, kind,
+                         stride, (int)n, prev_order, per, order_out);
     EVX_LAUNCH_CHECK();
     return 0;
   }
@@ -1321,15 +1338,19 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   // one for the gather
   const size_t lds = crowd_lds_bytes(L, 2);
   const bool mid = crowd_mid_sort(L);
-  if (int e = grant_dynamic_lds(mid ? reinterpret_cast<const void*>(crowd_kernel<kMidArgsortThreads>)
-                                    : reinterpret_cast<const void*>(crowd_kernel<kRadixThreads>), lds))
-    return e;
+  const bool wide = L.n <= kMidArgsortWideRows;
+  const void* const kernel = !mid ? reinterpret_cast<const void*>(crowd_kernel<kRadixThreads, 0>)
+                             : wide ? reinterpret_cast<const void*>(crowd_kernel<kMidArgsortThreads, 1>)
+                                    : reinterpret_cast<const void*>(crowd_kernel<kMidArgsortThreads, 2>);
+  if (int e = grant_dynamic_lds(kernel, lds)) return e;
   int grid = finish_grid(L, L.m);  // resident at once: at most two blocks of 256 threads per compute unit
   if (grid > device_cus() * 2) grid = device_cus() * 2;
-  if (mid)
-    hipLaunchKernelGGL(crowd_kernel<kMidArgsortThreads>, dim3(grid), dim3(kMidArgsortThreads), lds, s, crowd_args(w, w.at<int>(L.perm), false, 2));
+  if (mid && wide)
+    hipLaunchKernelGGL((crowd_kernel<kMidArgsortThreads, 1>), dim3(grid), dim3(kMidArgsortThreads), lds, s, crowd_args(w, w.at<int>(L.perm), false, 2));
+  else if (mid)
+    hipLaunchKernelGGL((crowd_kernel<kMidArgsortThreads, 2>), dim3(grid), dim3(kMidArgsortThreads), lds, s, crowd_args(w, w.at<int>(L.perm), false, 2));
   else
-    hipLaunchKernelGGL(crowd_kernel<kRadixThreads>, dim3(grid), dim3(kRadixThreads), lds, s, crowd_args(w, w.at<int>(L.perm), false, 2));
+    hipLaunchKernelGGL((crowd_kernel<kRadixThreads, 0>), dim3(grid), dim3(kRadixThreads), lds, s, crowd_args(w, w.at<int>(L.perm), false, 2));
   EVX_LAUNCH_CHECK();
   int blocks = (int)((topk + 3) / 4);
   const int cap = device_cus() * 8;

@@ -194,6 +194,9 @@ __device__ inline bool crowd_mid_applies(const CrowdArgs& a, int nv) {
 
 // `epochs`: how many epochs of radix barrier generations the control block's counter moves on when the radix path
 // has run (1 when the kernel ends after this body; the merged tail kernel passes 0 and moves the counter itself).
+// TABLES: 0 = the launch has no LDS sorter (kRadixThreads threads), 1 = its large tables, 2 = its small ones (the host
+// goes by the size of the population).
+template <int TABLES>
 __device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int epochs, uint64_t* finish_lds, int* base, int* scratch) {
   const float* __restrict__ xs = a.xs;
   const int npad = a.npad, m = a.m, kstride = a.kstride, use_orders = a.use_orders, fused = a.fused;
@@ -216,7 +219,7 @@ __device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int ep
   const int* __restrict__ list = list_base + ctrl->worst_start;
   // a large front of a population whose per-objective orders are at hand is ordered by front_order_*_kernel
   if (nv > kRadixMinCandidates && use_orders && param->orders_valid != 0) return;
-  if (nv <= kRadixMinCandidates && !crowd_mid_applies(a, nv)) {
+  if (nv <= kRadixMinCandidates && !(TABLES != 0 && crowd_mid_applies(a, nv))) {
     // ranking by counting: one work item per (256 candidates, objective)
     const int qblocks = (nv + (int)blockDim.x - 1) / (int)blockDim.x;
     for (int item = blockIdx.x; item < qblocks * m; item += gridDim.x) {
@@ -234,9 +237,8 @@ __device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int ep
     }
     return;
   }
-  if (crowd_mid_applies(a, nv)) {
+  if (TABLES != 0 && crowd_mid_applies(a, nv)) {
     // a workgroup produces a run of positions of one objective's order from the front's keys in its LDS; nobody waits
-    const MidSortLds T = mid_sort_lds(finish_lds);
     const int nb = (int)gridDim.x;
     const int per_objective = nb >= m ? nb / m : 1;  // workgroups that share an objective
     const int run = ((nv + per_objective - 1) / per_objective + 15) & ~15;
@@ -244,8 +246,8 @@ __device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int ep
       const int k = item % m, s0 = (item / m) * run;
       if (s0 >= nv) continue;
       const float* __restrict__ col = xs + (int64_t)k * npad;
-      mid_argsort_slice(
-          T, nv, s0, s0 + run, [&](int e) { return ordered_key(col[list[e]]); },
+      mid_argsort_slice<TABLES == 1>(
+          finish_lds, nv, s0, s0 + run, [&](int e) { return ordered_key(col[list[e]]); },
           [&](int p, int e) {  // (coherent stores: the distances may be worked out later in this same kernel)
             coherent_store(&pos[(int64_t)k * kstride + e], p);
             coherent_store(&sorted_cost[(int64_t)k * kstride + p], col[list[e]]);
@@ -281,13 +283,13 @@ __device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int ep
 // after_peel_tail: the peel kernel may have ordered the last front already (Ctrl.tail_done).
 // T threads: kRadixThreads, or kMidArgsortThreads where CrowdArgs.mid_sort is set (the radix sort, which is written for
 // kRadixThreads, does not run then).
-template <int T>
+template <int T, int TABLES>
 __global__ __launch_bounds__(T) void crowd_sort_kernel(CrowdArgs a, int after_peel_tail) {
   extern __shared__ __attribute__((aligned(16))) uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
   if (after_peel_tail != 0 && a.ctrl->tail_done != 0) return;
-  crowd_sort_body(a, radix_generation_base(a.ctrl), 1, finish_lds, base, scratch);
+  crowd_sort_body<TABLES>(a, radix_generation_base(a.ctrl), 1, finish_lds, base, scratch);
 }
 
 // ---- The same per-objective order of a large last front, taken from the orders of the whole population that
@@ -425,6 +427,7 @@ __device__ inline bool counter_barrier(Ctrl* ctrl, int which, int target, unsign
 // that come first by (distance descending, NaN after every number, row index) -- jit_fix_operator.py:246-252
 // applied to non_dominate.py:253.  Same grid rule as crowd_sort_kernel.  Dynamic LDS:
 // kRadixMinCandidates * 4 + kRankTile * 8 bytes.
+template <int TABLES>
 __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, unsigned gen0, int epochs, uint64_t* finish_lds,
                                          int* base, int* scratch) {
   const int m = a.m, kstride = a.kstride, fused = a.fused;
@@ -444,7 +447,7 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
   const int start = ctrl->worst_start;
   const int need = ctrl->need;
   const int* __restrict__ list = list_base + start;
-  if (nv <= kRadixMinCandidates && !crowd_mid_applies(a, nv)) {
+  if (nv <= kRadixMinCandidates && !(TABLES != 0 && crowd_mid_applies(a, nv))) {
     // every block derives the distance keys of all candidates in LDS (a few thousand table look-ups);
     // block 0 also stores the distances
     uint32_t* dkey_lds = reinterpret_cast<uint32_t*>(finish_lds);
@@ -473,7 +476,7 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
     }
     return;
   }
-  if (crowd_mid_applies(a, nv)) {
+  if (TABLES != 0 && crowd_mid_applies(a, nv)) {
     // distances by stripes; then, for the order, every workgroup takes all distance keys into its LDS and produces a
     // run of the first `need` positions
     EVX_TRACE(50, 0);
@@ -487,12 +490,11 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
     EVX_TRACE(50, 1);
     if (!counter_barrier<kBarrierDrop>(ctrl, 3, (int)gridDim.x, spin_limit, scratch)) return;
     EVX_TRACE(50, 2);
-    const MidSortLds T = mid_sort_lds(finish_lds);
     const int run = ((need + (int)gridDim.x - 1) / (int)gridDim.x + 15) & ~15;
     const int s0 = (int)blockIdx.x * run;
     if (s0 < need)
-      mid_argsort_slice<52>(
-          T, nv, s0, min(need, s0 + run),
+      mid_argsort_slice<TABLES == 1, 52>(
+          finish_lds, nv, s0, min(need, s0 + run),
           // (the key of an infinite distance lies far below those of the finite ones, which would leave them a twentieth
           // of the sorter's buckets: any key below that of -m will do for it, a distance being at most m)
           [&](int e) {
@@ -534,13 +536,13 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
   }
 }
 
-template <int T>
+template <int T, int TABLES>
 __global__ __launch_bounds__(T) void crowd_finish_kernel(CrowdArgs a, int want_order, int after_peel_tail) {
   extern __shared__ __attribute__((aligned(16))) uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
   if (after_peel_tail != 0 && a.ctrl->tail_done != 0) return;
-  crowd_finish_body(a, want_order, radix_generation_base(a.ctrl), 1, finish_lds, base, scratch);
+  crowd_finish_body<TABLES>(a, want_order, radix_generation_base(a.ctrl), 1, finish_lds, base, scratch);
 }
 
 // ---- The ordering of the last front in one launch, for populations whose peel kernel orders a small last front
@@ -561,7 +563,7 @@ __global__ __launch_bounds__(256) void gather_after_peel_kernel(GatherArgs g) {
   gather_body(g, blockIdx.x, gridDim.x, g.ctrl->err == 0 && g.ctrl->tail_done != 0 ? g.ctrl->worst_start : 0);
 }
 
-template <int T>
+template <int T, int TABLES>
 __global__ __launch_bounds__(T) void crowd_kernel(CrowdArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint64_t finish_lds[];
   __shared__ int base[256];
@@ -569,10 +571,10 @@ __global__ __launch_bounds__(T) void crowd_kernel(CrowdArgs a) {
   Ctrl* ctrl = a.ctrl;
   if (coherent_load(&ctrl->err) != 0 || ctrl->tail_done != 0) return;
   const unsigned gen0 = radix_generation_base(ctrl);
-  crowd_sort_body(a, gen0, 0, finish_lds, base, scratch);
+  crowd_sort_body<TABLES>(a, gen0, 0, finish_lds, base, scratch);
   // (the sorts in LDS hand their tables on through coherent stores)
-  if (tail_barrier(ctrl, (int)gridDim.x, a.spin_limit, scratch, crowd_mid_applies(a, ctrl->nv)))
-    crowd_finish_body(a, 1, gen0 + 16u, 0, finish_lds, base, scratch);
+  if (tail_barrier(ctrl, (int)gridDim.x, a.spin_limit, scratch, TABLES != 0 && crowd_mid_applies(a, ctrl->nv)))
+    crowd_finish_body<TABLES>(a, 1, gen0 + 16u, 0, finish_lds, base, scratch);
   if (blockIdx.x == 0 && threadIdx.x == 0) ctrl->radix_epoch += 2;  // both bodies may have run a radix sort
 }
 

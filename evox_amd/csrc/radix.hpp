@@ -333,7 +333,7 @@ __global__ __launch_bounds__(kSmallArgsortThreads) void small_argsort_kernel(con
 // between workgroups (the radix sort needs three launches and twelve grid barriers: 70 us at 20 000 positions, more
 // than torch's own sort).  Every workgroup reads all keys into LDS (32-bit order-preserving images) and works on
 // composites (image << 15 | position: distinct, below 2^47); it produces a run of `slots_per_block` slots of the
-// result: the histogram of all composites over kMidArgsortBuckets buckets (LDS atomics), its scan, the buckets that
+// result: the histogram of all composites over 4096 (or 2048) buckets (LDS atomics), its scan, the buckets that
 // hold the wanted slots, their composites collected into a list, every member of the list placed by counting the
 // members below it (sixteen lanes per member).  Keys with few distinct values are the usual case here (ranks, a
 // distance that is -inf for most rows): the buckets cut the composites, so a key held by thousands of positions is
@@ -342,19 +342,31 @@ __global__ __launch_bounds__(kSmallArgsortThreads) void small_argsort_kernel(con
 // range of keys with a crowd on one value) it builds the histogram of that bucket's range, which is narrower by the
 // bucket count each time, down to single composites.  The code is loops, not unrolled passes: a launch starts with
 // a cold instruction cache.
-constexpr int kMidArgsortRows = 24576;  // keys of 4 bytes in LDS beside the tables
+constexpr int kMidArgsortRows = 32768;  // keys of 4 bytes in LDS (128 KB) beside the tables: a merged population of 2 x 16384
 constexpr int kMidArgsortThreads = 1024;
-constexpr int kMidArgsortBuckets = 4096;
-constexpr int kMidArgsortList = 2048;
+// Up to kMidArgsortWideRows keys the tables are 4096 buckets and a list of 2048 (48 KB); above, 2048 buckets and a list
+// of 1536 (28 KB), so that 32768 keys still fit beside them (20 000 keys: 15 us slower with the small tables).
+constexpr int kMidArgsortWideRows = 24576;
 constexpr int kMidArgsortIndexBits = 15;
 
-// Exclusive scan, in place, of the kMidArgsortBuckets counts in `hist` by the whole workgroup; returns their sum.
+// Exclusive scan, in place, of the BUCKETS counts in `hist` by the whole workgroup; returns their sum.
+template <int BUCKETS>
 __device__ inline int mid_argsort_scan(int* hist, int* wave_tot) {
-  constexpr int kPer = kMidArgsortBuckets / kMidArgsortThreads;  // 4 consecutive buckets per thread
+  constexpr int kPer = BUCKETS / kMidArgsortThreads;  // consecutive buckets per thread
+  static_assert(kPer == 2 || kPer == 4, "two or four buckets per thread");
   constexpr int kWaves = kMidArgsortThreads / 64;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int4 c = *reinterpret_cast<const int4*>(hist + tid * kPer);
-  const int mine = c.x + c.y + c.z + c.w;
+  int c[kPer];
+  if constexpr (kPer == 4) {
+    const int4 v = *reinterpret_cast<const int4*>(hist + tid * kPer);
+    c[0] = v.x; c[1] = v.y; c[2] = v.z; c[3] = v.w;
+  } else {
+    const int2 v = *reinterpret_cast<const int2*>(hist + tid * kPer);
+    c[0] = v.x; c[1] = v.y;
+  }
+  int mine = 0;
+#pragma unroll
+  for (int u = 0; u < kPer; ++u) mine += c[u];
   int incl = mine;
 #pragma unroll
   for (int off = 1; off < 64; off <<= 1) {
@@ -369,50 +381,55 @@ __device__ inline int mid_argsort_scan(int* hist, int* wave_tot) {
     if (w < wave) run += wave_tot[w];
     total += wave_tot[w];
   }
-  int4 o;
-  o.x = run; run += c.x;
-  o.y = run; run += c.y;
-  o.z = run; run += c.z;
-  o.w = run;
-  *reinterpret_cast<int4*>(hist + tid * kPer) = o;
+#pragma unroll
+  for (int u = 0; u < kPer; ++u) {
+    hist[tid * kPer + u] = run;
+    run += c[u];
+  }
   __syncthreads();
   return total;
 }
 
 // The tables of a workgroup that sorts in LDS, carved from `bytes` = mid_sort_lds_bytes(n) of it.
 struct MidSortLds {
-  int* top_hist;             // [kMidArgsortBuckets] first-level starts, kept
-  int* sub_hist;             // [kMidArgsortBuckets] starts of the level below, rebuilt
-  unsigned long long* list;  // [kMidArgsortList]
+  int* top_hist;             // [buckets] first-level starts, kept
+  int* sub_hist;             // [buckets] starts of the level below, rebuilt
+  unsigned long long* list;  // [list entries]
   uint32_t* red;             // [2][waves]
   int* wave_tot;             // [waves]
   int* found;                // [5] bucket of the first wanted slot, its start and end; bucket of the last wanted slot, its end
   int* list_count;
   uint32_t* keys;            // [n] order-preserving images of the keys, in the order of the positions
 };
-constexpr size_t kMidSortTableBytes = 2 * sizeof(int) * kMidArgsortBuckets + sizeof(unsigned long long) * kMidArgsortList + 256;
-__host__ __device__ inline size_t mid_sort_lds_bytes(int n) { return kMidSortTableBytes + sizeof(uint32_t) * (size_t)n; }
+__host__ __device__ inline size_t mid_sort_table_bytes(int n) {
+  const int buckets = n <= kMidArgsortWideRows ? 4096 : 2048, list = n <= kMidArgsortWideRows ? 2048 : 1536;
+  return 2 * sizeof(int) * (size_t)buckets + sizeof(unsigned long long) * (size_t)list + 256;
+}
+__host__ __device__ inline size_t mid_sort_lds_bytes(int n) { return mid_sort_table_bytes(n) + sizeof(uint32_t) * (size_t)n; }
+template <int BUCKETS, int LIST>
 __device__ inline MidSortLds mid_sort_lds(void* lds) {  // (16-byte aligned)
   constexpr int kWaves = kMidArgsortThreads / 64;
   MidSortLds t;
   t.top_hist = static_cast<int*>(lds);
-  t.sub_hist = t.top_hist + kMidArgsortBuckets;
-  t.list = reinterpret_cast<unsigned long long*>(t.sub_hist + kMidArgsortBuckets);
-  t.red = reinterpret_cast<uint32_t*>(t.list + kMidArgsortList);
+  t.sub_hist = t.top_hist + BUCKETS;
+  t.list = reinterpret_cast<unsigned long long*>(t.sub_hist + BUCKETS);
+  t.red = reinterpret_cast<uint32_t*>(t.list + LIST);
   t.wave_tot = reinterpret_cast<int*>(t.red + 2 * kWaves);
   t.found = t.wave_tot + kWaves;
   t.list_count = t.found + 5;
-  t.keys = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(lds) + kMidSortTableBytes);
+  t.keys = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(lds) + 2 * sizeof(int) * BUCKETS + sizeof(unsigned long long) * LIST + 256);
   return t;
 }
 
 // Slots s0 .. s1-1 of the stable ascending order of n <= kMidArgsortRows 32-bit keys, by one workgroup of
 // kMidArgsortThreads threads that holds all keys in LDS and waits for no other workgroup: key_of(e) = the key of
-// position e (read once), emit(slot, e) = position e belongs in `slot`.  The keys go into kMidArgsortBuckets buckets
+// position e (read once), emit(slot, e) = position e belongs in `slot`.  The keys go into BUCKETS buckets
 // by value; the buckets that hold the wanted slots are collected (a bucket too large for the list is cut into buckets
 // of its own range first) and their members placed by counting.  Every thread of the workgroup calls it.
-template <int TRACE = 51, class KeyOf, class Emit>
-__device__ inline void mid_argsort_slice(const MidSortLds& T, int n, int s0, int s1_wanted, KeyOf key_of, Emit emit) {
+template <int BUCKETS, int LIST, int TRACE, class KeyOf, class Emit>
+__device__ inline void mid_argsort_slice_sized(void* lds, int n, int s0, int s1_wanted, KeyOf key_of, Emit emit) {
+  constexpr int kMidArgsortBuckets = BUCKETS, kMidArgsortList = LIST;
+  const MidSortLds T = mid_sort_lds<BUCKETS, LIST>(lds);
   uint32_t* const mid_keys = T.keys;
   int* const top_hist = T.top_hist;
   int* const sub_hist = T.sub_hist;
@@ -461,7 +478,7 @@ __device__ inline void mid_argsort_slice(const MidSortLds& T, int n, int s0, int
   const int top_shift = shift_for(top_hi - top_lo);
   for (int e = tid; e < n; e += kMidArgsortThreads) atomicAdd(&top_hist[(int)((composite(e) - top_lo) >> top_shift)], 1);
   __syncthreads();
-  mid_argsort_scan(top_hist, wave_tot);  // (the total is n)
+  mid_argsort_scan<BUCKETS>(top_hist, wave_tot);  // (the total is n)
   EVX_TRACE(TRACE, 1);
   const int s1 = min(n, s1_wanted);
   // level state: the same in every thread
@@ -529,7 +546,7 @@ __device__ inline void mid_argsort_slice(const MidSortLds& T, int n, int s0, int
           }
         }
         __syncthreads();
-        mid_argsort_scan(sub_hist, wave_tot);
+        mid_argsort_scan<BUCKETS>(sub_hist, wave_tot);
         continue;
       }
       // as many buckets from b0 on as the list takes (not b0 alone: where the run of wanted slots ends in a bucket of
@@ -600,13 +617,23 @@ __device__ inline void mid_argsort_slice(const MidSortLds& T, int n, int s0, int
   EVX_TRACE(TRACE, 3);
 }
 
+// WIDE: the large tables (at most kMidArgsortWideRows keys).  `lds` = mid_sort_lds_bytes(most keys the launch may
+// meet) bytes, 16-byte aligned: the host picks WIDE by that number, so that a kernel holds one size of the code.
+template <bool WIDE, int TRACE = 51, class KeyOf, class Emit>
+__device__ inline void mid_argsort_slice(void* lds, int n, int s0, int s1_wanted, KeyOf key_of, Emit emit) {
+  if constexpr (WIDE)
+    mid_argsort_slice_sized<4096, 2048, TRACE>(lds, n, s0, s1_wanted, key_of, emit);
+  else
+    mid_argsort_slice_sized<2048, 1536, TRACE>(lds, n, s0, s1_wanted, key_of, emit);
+}
+
 // One step of a lexsort of n <= kMidArgsortRows positions: a workgroup per `slots_per_block` slots of the order.
 // Dynamic LDS: mid_sort_lds_bytes(n).
+template <bool WIDE>
 __global__ __launch_bounds__(kMidArgsortThreads) void mid_argsort_kernel(const void* __restrict__ key, int kind, int64_t stride, int n,
                                                                          const int* __restrict__ prev, int slots_per_block,
                                                                          int* __restrict__ order_out) {
   extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];
-  const MidSortLds T = mid_sort_lds(mid_lds);
   auto key_of = [&](int e) -> uint32_t {
     const int idx = prev ? prev[e] : e;
     if (kind == kKeyFloat32) return ordered_key(static_cast<const float*>(key)[(int64_t)idx * stride]);
@@ -614,7 +641,7 @@ __global__ __launch_bounds__(kMidArgsortThreads) void mid_argsort_kernel(const v
     return static_cast<const uint32_t*>(key)[(int64_t)idx * stride];
   };
   const int s0 = (int)blockIdx.x * slots_per_block;
-  mid_argsort_slice(T, n, s0, s0 + slots_per_block, key_of, [&](int slot, int e) { order_out[slot] = prev ? prev[e] : e; });
+  mid_argsort_slice<WIDE>(mid_lds, n, s0, s0 + slots_per_block, key_of, [&](int slot, int e) { order_out[slot] = prev ? prev[e] : e; });
 }
 
 // Many independent steps at once: `batch` sorts of n <= kSmallArgsortRows positions each, sort b reading

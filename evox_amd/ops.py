@@ -113,7 +113,7 @@ torch.library.register_vmap(nd_rank, _nd_rank_vmap)
 
 
 RANK_UNSET = 0x7FFFFFFF
-_SMALL_ARGSORT_ROWS = 24576  # longest one-dimensional sort whose kernel has no device-side waits (and keeps no control block)
+_SMALL_ARGSORT_ROWS = 32768  # longest one-dimensional sort whose kernel has no device-side waits (and keeps no control block)
 _ROWS_ARGSORT_MAX = 16384  # longest sort of a batch that runs inside one workgroup
 
 

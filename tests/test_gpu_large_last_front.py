@@ -1,4 +1,4 @@
-"""Last fronts of more than 1024 rows in populations of at most 24 576 rows -- a converged population, where most
+"""Last fronts of more than 1024 rows in populations of at most 32 768 rows -- a converged population, where most
 rows are non-dominated -- whose per-objective orders and distance order come from workgroups that sort in LDS: against
 the plain-C checker, against the radix path (option ``mid_argsort`` off), and ``crowding_distance`` on masks of that
 size.  Ties in an objective (equal costs keep their row order), duplicate rows, a NaN objective, the largest
@@ -27,6 +27,10 @@ def _cases():
     cases = {}
     cases["simplex_20000x3"] = (_simplex(20000, 3, g), [1, 10000, 20000])
     cases["simplex_24576x2"] = (_simplex(24576, 2, g), [12288])
+    cases["simplex_32768x3"] = (_simplex(32768, 3, g), [16384])  # the largest population of the path
+    most = _simplex(26000, 3, g)
+    most[24000:] = most[24000:] * 1.5 + 0.1  # a population that gets the small tables, a front that would fit the large ones
+    cases["front0_24000_of_26000x3"] = (most, [13000])
     cases["simplex_12000x5"] = (_simplex(12000, 5, g), [6000])
     mixed = _simplex(20000, 3, g)
     mixed[14000:] = mixed[14000:] * 1.5 + 0.1  # 30 % of the rows dominated: the cut falls into front 0 of 14 000 rows
