@@ -96,21 +96,18 @@ __device__ inline int rank_by_counting(uint64_t mine, int nv, LoadPair load_pair
 // (next - previous) / (last - first) in sorted order, +inf for a candidate that is first or last in any
 // objective (non_dominate.py:223-229).  Objectives are added in column order starting from the first
 // term, which is what torch's row sum does for the small M of this workload.
-// COHERENT: the tables were written earlier in the same kernel by other workgroups (coherent stores): coherent loads.
-template <bool COHERENT = false>
 __device__ inline float crowding_distance_of(int q, int nv, int m, const int* __restrict__ pos,
                                              const float* __restrict__ sorted_cost, int kstride) {
   bool boundary = false;
   float acc = 0.0f;
   for (int k = 0; k < m; ++k) {
     const float* __restrict__ sc = sorted_cost + (int64_t)k * kstride;
-    auto cost_at = [&](int p) { return COHERENT ? coherent_load(&sc[p]) : sc[p]; };
-    const int p = COHERENT ? coherent_load(&pos[(int64_t)k * kstride + q]) : pos[(int64_t)k * kstride + q];
+    const int p = pos[(int64_t)k * kstride + q];
     if (p == 0 || p == nv - 1) {
       boundary = true;
     } else {
-      const float span = cost_at(nv - 1) - cost_at(0);
-      const float term = (cost_at(p + 1) - cost_at(p - 1)) / span;
+      const float span = sc[nv - 1] - sc[0];
+      const float term = (sc[p + 1] - sc[p - 1]) / span;
       acc = k == 0 ? term : acc + term;
     }
   }

@@ -248,9 +248,9 @@ __device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int ep
       const float* __restrict__ col = xs + (int64_t)k * npad;
       mid_argsort_slice<TABLES == 1>(
           finish_lds, nv, s0, s0 + run, [&](int e) { return ordered_key(col[list[e]]); },
-          [&](int p, int e) {  // (coherent stores: the distances may be worked out later in this same kernel)
-            coherent_store(&pos[(int64_t)k * kstride + e], p);
-            coherent_store(&sorted_cost[(int64_t)k * kstride + p], col[list[e]]);
+          [&](int p, int e) {
+            pos[(int64_t)k * kstride + e] = p;
+            sorted_cost[(int64_t)k * kstride + p] = col[list[e]];
           });
     }
     return;
@@ -394,27 +394,21 @@ __global__ __launch_bounds__(256) void front_order_place_kernel(const unsigned l
 
 // A barrier of all `target` workgroups of a resident grid on the counter Ctrl.reserved[which] (zero at the start of the
 // call; used once).  False when the bounded wait ran out (Ctrl.err is set then).
-// kBarrierFences: the code on either side exchanges its results (positions, sorted costs, distances, the order) through
-// plain stores and loads, which are coherent between kernels but not between the dies of one kernel: the die's L2 is
-// written back before the workgroup arrives and its caches are dropped after it leaves.  A write-back or an
-// invalidation works on the whole cache, whichever wave asks for it, and costs the same every time (1024 threads
-// of 256 workgroups each asking: 65 us per barrier), so one wave of the workgroup asks, once every wave's own stores
-// have arrived in the L2.  kBarrierCoherent: the data is exchanged through coherent stores and loads, nothing else is done.
-// kBarrierDrop: what arrives was stored coherently (written through), and is read by plain loads afterwards: nothing to
-// write back, but the caches are dropped (every workgroup reads all of it: coherent loads would all go to memory).
-enum BarrierKind { kBarrierFences = 0, kBarrierCoherent = 1, kBarrierDrop = 2 };
-template <int KIND = kBarrierFences>
+// The code on either side exchanges its results (positions, sorted costs, distances, the order) through plain stores
+// and loads, which are coherent between kernels but not between the dies of one kernel: the die's L2 is written back
+// before the workgroup arrives and its caches are dropped after it leaves.  A write-back or an invalidation works on
+// the whole cache, whichever wave asks for it, and costs the same every time (1024 threads of 256 workgroups each
+// asking: 65 us per barrier), so one wave of the workgroup asks, once every wave's own stores have arrived in the L2.
 __device__ inline bool counter_barrier(Ctrl* ctrl, int which, int target, unsigned spin_limit, int* scratch) {
-  constexpr bool FENCES = KIND == kBarrierFences;
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (threadIdx.x == 0) {
-    if (FENCES) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __hip_atomic_fetch_add(&ctrl->reserved[which], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const bool seen = bounded_wait([&] { return coherent_load(&ctrl->reserved[which]) >= target; }, spin_limit);
     if (!seen) coherent_store(&ctrl->err, kErrBarrierTimeout);
     scratch[0] = seen;
-    if (FENCES || KIND == kBarrierDrop) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   }
   __syncthreads();
   const bool fine = scratch[0] != 0;
@@ -481,14 +475,14 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
     // run of the first `need` positions
     EVX_TRACE(50, 0);
     for (int q = blockIdx.x * blockDim.x + threadIdx.x; q < nv; q += gridDim.x * blockDim.x) {
-      const float d = crowding_distance_of<true>(q, nv, m, pos, sorted_cost, kstride);
+      const float d = crowding_distance_of(q, nv, m, pos, sorted_cost, kstride);
       dist[list[q]] = d;
-      coherent_store(&dkey[q], ordered_key(-d));
+      dkey[q] = ordered_key(-d);
     }
     if (!want_order) return;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < start; i += gridDim.x * blockDim.x) order[i] = list_base[i];
     EVX_TRACE(50, 1);
-    if (!counter_barrier<kBarrierDrop>(ctrl, 3, (int)gridDim.x, spin_limit, scratch)) return;
+    if (!counter_barrier(ctrl, 3, (int)gridDim.x, spin_limit, scratch)) return;
     EVX_TRACE(50, 2);
     const int run = ((need + (int)gridDim.x - 1) / (int)gridDim.x + 15) & ~15;
     const int s0 = (int)blockIdx.x * run;
@@ -550,9 +544,8 @@ __global__ __launch_bounds__(T) void crowd_finish_kernel(CrowdArgs a, int want_o
 // still costs as much as a small kernel (about 4.7 us on this device), so the two stages share one launch; they are
 // separated by a counter barrier of all blocks.  Grid: that of crowd_sort_kernel (the radix grid: master, idle
 // block, workers), resident at once.
-__device__ inline bool tail_barrier(Ctrl* ctrl, int target, unsigned spin_limit, int* scratch, bool coherent_exchange) {
-  return coherent_exchange ? counter_barrier<kBarrierCoherent>(ctrl, 1, target, spin_limit, scratch)
-                           : counter_barrier<kBarrierFences>(ctrl, 1, target, spin_limit, scratch);
+__device__ inline bool tail_barrier(Ctrl* ctrl, int target, unsigned spin_limit, int* scratch) {
+  return counter_barrier(ctrl, 1, target, spin_limit, scratch);
 }
 
 __global__ __launch_bounds__(256) void gather_kernel(GatherArgs g) { gather_body(g, blockIdx.x, gridDim.x, 0); }
@@ -572,8 +565,7 @@ __global__ __launch_bounds__(T) void crowd_kernel(CrowdArgs a) {
   if (coherent_load(&ctrl->err) != 0 || ctrl->tail_done != 0) return;
   const unsigned gen0 = radix_generation_base(ctrl);
   crowd_sort_body<TABLES>(a, gen0, 0, finish_lds, base, scratch);
-  // (the sorts in LDS hand their tables on through coherent stores)
-  if (tail_barrier(ctrl, (int)gridDim.x, a.spin_limit, scratch, TABLES != 0 && crowd_mid_applies(a, ctrl->nv)))
+  if (tail_barrier(ctrl, (int)gridDim.x, a.spin_limit, scratch))
     crowd_finish_body<TABLES>(a, 1, gen0 + 16u, 0, finish_lds, base, scratch);
   if (blockIdx.x == 0 && threadIdx.x == 0) ctrl->radix_epoch += 2;  // both bodies may have run a radix sort
 }
