@@ -19,6 +19,30 @@
 
 namespace evx {
 
+// A barrier of all `target` workgroups of a resident grid on the counter Ctrl.reserved[which] (zero at the start of the
+// call; used once).  False when the bounded wait ran out (Ctrl.err is set then).
+// The code on either side exchanges its results (positions, sorted costs, distances, the order) through plain stores
+// and loads, which are coherent between kernels but not between the dies of one kernel: the die's L2 is written back
+// before the workgroup arrives and its caches are dropped after it leaves.  A write-back or an invalidation works on
+// the whole cache, whichever wave asks for it, and costs the same every time (1024 threads of 256 workgroups each
+// asking: 65 us per barrier), so one wave of the workgroup asks, once every wave's own stores have arrived in the L2.
+__device__ inline bool counter_barrier(Ctrl* ctrl, int which, int target, unsigned spin_limit, int* scratch) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __hip_atomic_fetch_add(&ctrl->reserved[which], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool seen = bounded_wait([&] { return coherent_load(&ctrl->reserved[which]) >= target; }, spin_limit);
+    if (!seen) coherent_store(&ctrl->err, kErrBarrierTimeout);
+    scratch[0] = seen;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  }
+  __syncthreads();
+  const bool fine = scratch[0] != 0;
+  __syncthreads();  // scratch is reused
+  return fine;
+}
+
 // ---- A small last front in one launch.  With a few hundred candidates the two kernels below cost two launches and
 // three chains of dependent loads (positions, sorted costs, distance keys) for a few microseconds of work.  Here the
 // candidates' (key, candidate) composites and costs of every objective sit in LDS of every workgroup, a candidate is
@@ -123,28 +147,20 @@ __device__ inline void crowd_small_front(const float* __restrict__ xs, int npad,
         if (solo)
           dkey_lds[q] = ordered_key(-d);
         else
-          coherent_store(&dkey[q], ordered_key(-d));
+          dkey[q] = ordered_key(-d);
       }
     }
   }
   if (mode != 2) return;
-  // every block has stored its distance keys: one counter, bounded wait
   __syncthreads();
   if (solo) {
     for (int e = tid; e < nv; e += blockDim.x) comp[e] = ((unsigned long long)dkey_lds[e] << 32) | (unsigned)e;
     __syncthreads();
   } else {
-  if (tid == 0) {
-    __hip_atomic_fetch_add(&ctrl->reserved[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const bool seen = bounded_wait([&] { return coherent_load(&ctrl->reserved[0]) >= (int)gridDim.x || coherent_load(&ctrl->err) != 0; },
-                                   spin_limit);
-    if (!seen) coherent_store(&ctrl->err, kErrBarrierTimeout);
-    scratch[0] = seen && coherent_load(&ctrl->err) == 0;
-  }
-  __syncthreads();
-  if (scratch[0] == 0) return;
-  for (int e = tid; e < nv; e += blockDim.x) comp[e] = ((unsigned long long)coherent_load(&dkey[e]) << 32) | (unsigned)e;
-  __syncthreads();
+    // every block has stored its distance keys
+    if (!counter_barrier(ctrl, 0, (int)gridDim.x, spin_limit, scratch)) return;
+    for (int e = tid; e < nv; e += blockDim.x) comp[e] = ((unsigned long long)dkey[e] << 32) | (unsigned)e;
+    __syncthreads();
   }
   for (int q = blockIdx.x * (blockDim.x >> 4) + (tid >> 4); q < nv; q += groups) {
     const unsigned long long mine = comp[q];
@@ -390,30 +406,6 @@ __global__ __launch_bounds__(256) void front_order_place_kernel(const unsigned l
     }
     running += wave_count[u][0] + wave_count[u][1] + wave_count[u][2] + wave_count[u][3];
   }
-}
-
-// A barrier of all `target` workgroups of a resident grid on the counter Ctrl.reserved[which] (zero at the start of the
-// call; used once).  False when the bounded wait ran out (Ctrl.err is set then).
-// The code on either side exchanges its results (positions, sorted costs, distances, the order) through plain stores
-// and loads, which are coherent between kernels but not between the dies of one kernel: the die's L2 is written back
-// before the workgroup arrives and its caches are dropped after it leaves.  A write-back or an invalidation works on
-// the whole cache, whichever wave asks for it, and costs the same every time (1024 threads of 256 workgroups each
-// asking: 65 us per barrier), so one wave of the workgroup asks, once every wave's own stores have arrived in the L2.
-__device__ inline bool counter_barrier(Ctrl* ctrl, int which, int target, unsigned spin_limit, int* scratch) {
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    __hip_atomic_fetch_add(&ctrl->reserved[which], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const bool seen = bounded_wait([&] { return coherent_load(&ctrl->reserved[which]) >= target; }, spin_limit);
-    if (!seen) coherent_store(&ctrl->err, kErrBarrierTimeout);
-    scratch[0] = seen;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-  }
-  __syncthreads();
-  const bool fine = scratch[0] != 0;
-  __syncthreads();  // scratch is reused
-  return fine;
 }
 
 // Crowding distance of every candidate of the last front (written by original index) and, when
