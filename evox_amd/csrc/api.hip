@@ -591,6 +591,9 @@ static int radix_grid(const Layout& L) {
 // A last front of more than kMidSortMinCandidates rows in a population of at most kMidArgsortRows: its orders come from
 // workgroups that sort in LDS without waiting for each other (finish.hpp), one per compute unit.
 static bool crowd_mid_sort(const Layout& L) { return opt().mid_argsort != 0 && L.n > kMidSortMinCandidates && L.n <= kMidArgsortRows; }
+// A larger population: such a front gets a launch of its own (its kernels have kMidArgsortThreads threads, the radix
+// sort of a larger front kRadixThreads); each of the two returns at once from a front that is the other's.
+static bool crowd_mid_split(const Layout& L) { return opt().mid_argsort != 0 && L.n > kMidArgsortRows; }
 
 static int finish_grid(const Layout& L, int per_candidate_block) {
   if (crowd_mid_sort(L)) return device_cus();  // (their LDS leaves room for one workgroup per compute unit: all resident)
@@ -710,7 +713,7 @@ static CrowdArgs crowd_args(const Ws& w, const int* list, bool use_orders, int f
   a.param = w.at<SortParam>(L.sortparam);
   a.use_orders = use_orders ? 1 : 0;
   a.fused = fused;
-  a.mid_sort = crowd_mid_sort(L) ? 1 : 0;
+  a.mid_sort = crowd_mid_sort(L) ? 1 : (crowd_mid_split(L) ? 3 : 0);
   a.dist = w.at<float>(L.dist);
   a.dkey = w.at<uint32_t>(L.dkey);
   a.order = w.at<int>(L.order);
@@ -754,6 +757,15 @@ static int stage_crowd_sort(const Ws& w, const int* list, bool use_orders, int f
   // those (finish.hpp); the three kernels and the one below choose on the device which of them has work
   if (use_orders)
     if (int e = stage_front_orders(w, list, s)) return e;
+  if (crowd_mid_split(L)) {
+    const size_t mid_lds = mid_sort_lds_bytes(kMidArgsortRows);
+    if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(crowd_sort_kernel<kMidArgsortThreads, 2>), mid_lds)) return e;
+    CrowdArgs a = crowd_args(w, list, use_orders, fused);
+    a.mid_sort = 2;
+    hipLaunchKernelGGL((crowd_sort_kernel<kMidArgsortThreads, 2>), dim3(device_cus()), dim3(kMidArgsortThreads), mid_lds, s, a,
+                       after_peel_tail ? 1 : 0);
+    EVX_LAUNCH_CHECK();
+  }
   const size_t lds = crowd_lds_bytes(L, fused);
   const bool mid = crowd_mid_sort(L);
   const bool wide = L.n <= kMidArgsortWideRows;  // (which tables of the LDS sorter the population leaves room for)
@@ -783,6 +795,15 @@ static int stage_crowd_finish(const Ws& w, const int* list, bool want_order, int
   const Layout& L = w.L;
   // (no front of this population is too large for the fused path of crowd_sort_kernel: nothing is left to do)
   if (fused != 0 && L.n <= kFusedFrontRows && (int64_t)L.n * L.m <= kFusedFrontValues && L.m <= kFusedFrontObjectives) return 0;
+  if (crowd_mid_split(L)) {
+    const size_t mid_lds = mid_sort_lds_bytes(kMidArgsortRows);
+    if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(crowd_finish_kernel<kMidArgsortThreads, 2>), mid_lds)) return e;
+    CrowdArgs a = crowd_args(w, list, false, fused);
+    a.mid_sort = 2;
+    hipLaunchKernelGGL((crowd_finish_kernel<kMidArgsortThreads, 2>), dim3(device_cus()), dim3(kMidArgsortThreads), mid_lds, s, a,
+                       want_order ? 1 : 0, after_peel_tail ? 1 : 0);
+    EVX_LAUNCH_CHECK();
+  }
   const size_t lds = crowd_lds_bytes(L, 0);
   const bool mid = crowd_mid_sort(L);
   const bool wide = L.n <= kMidArgsortWideRows;

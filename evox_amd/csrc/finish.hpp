@@ -194,7 +194,11 @@ struct CrowdArgs {
   unsigned spin_limit;
   SortParam* param;
   int use_orders, fused;
-  int mid_sort;  // fronts of more than kRadixMinCandidates rows are ordered by mid_argsort_slice (the population has at most kMidArgsortRows)
+  // The LDS sorter (mid_argsort_slice) for fronts of kMidSortMinCandidates + 1 to kMidArgsortRows rows: 0 = not used;
+  // 1 = this launch has it beside everything else (kMidArgsortThreads threads, populations up to kMidArgsortRows);
+  // larger populations get two launches: 2 = this one (kMidArgsortThreads threads) orders such a front and nothing
+  // else, 3 = this one (kRadixThreads threads) leaves such a front to the other.
+  int mid_sort;
   float* dist;
   uint32_t* dkey;
   int* order;
@@ -205,7 +209,17 @@ struct CrowdArgs {
 // the 24 workgroups that the counting keeps busy.
 constexpr int kMidSortMinCandidates = 1024;
 __device__ inline bool crowd_mid_applies(const CrowdArgs& a, int nv) {
-  return a.mid_sort != 0 && nv > kMidSortMinCandidates && nv <= kMidArgsortRows && blockDim.x == kMidArgsortThreads;
+  return (a.mid_sort == 1 || a.mid_sort == 2) && nv > kMidSortMinCandidates && nv <= kMidArgsortRows &&
+         blockDim.x == kMidArgsortThreads;
+}
+// Where the work is split over two launches (mid_sort 2 and 3): whether the one with the LDS sorter orders the front
+// by objective (`by_objective`) or by distance.  A front that crowd_small_front takes, or whose per-objective orders
+// are read off those of the population, is not the LDS sorter's.
+__device__ inline bool crowd_mid_takes(const CrowdArgs& a, int nv, bool by_objective) {
+  if (nv <= kMidSortMinCandidates || nv > kMidArgsortRows) return false;
+  if (a.fused != 0 && fused_front_applies(nv, a.m)) return false;
+  if (by_objective && nv > kRadixMinCandidates && a.use_orders != 0 && a.param->orders_valid != 0) return false;
+  return true;
 }
 
 // `epochs`: how many epochs of radix barrier generations the control block's counter moves on when the radix path
@@ -228,6 +242,7 @@ __device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int ep
   int* __restrict__ order = a.order;
   if (coherent_load(&ctrl->err) != 0) return;
   const int nv = ctrl->nv;
+  if (a.mid_sort >= 2 && (a.mid_sort == 2) != crowd_mid_takes(a, nv, true)) return;  // the other launch's front
   if (fused != 0 && fused_front_applies(nv, m)) {  // a small front: distances (and order) right here
     crowd_small_front(xs, npad, list_base, ctrl, m, dist, dkey, order, spin_limit, fused, finish_lds, scratch);
     return;
@@ -429,6 +444,7 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
   int* __restrict__ order = a.order;
   if (coherent_load(&ctrl->err) != 0) return;
   const int nv = ctrl->nv;
+  if (a.mid_sort >= 2 && (a.mid_sort == 2) != crowd_mid_takes(a, nv, false)) return;  // the other launch's front
   if (fused != 0 && fused_front_applies(nv, m)) return;  // crowd_sort_kernel has done it all
   const int start = ctrl->worst_start;
   const int need = ctrl->need;

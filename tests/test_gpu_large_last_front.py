@@ -47,6 +47,16 @@ def _cases():
     small = _simplex(3000, 3, g)
     small[1100:] = small[1100:] * 1.5 + 0.1  # a front of 1100 rows, just above the smallest that is sorted this way
     cases["front0_1100_of_3000x3"] = (small, [1000])
+    # larger populations: the front goes to a launch of its own beside the one that holds the radix sort
+    big = _simplex(40000, 3, g)
+    big[9000:] = big[9000:] * 1.5 + 0.1  # front 0 of 9000 rows, ordered by objective and by distance in LDS
+    cases["front0_9000_of_40000x3"] = (big[torch.randperm(40000, generator=g)], [5000])
+    big2 = _simplex(40000, 4, g)
+    big2[30000:] = big2[30000:] * 1.5 + 0.1  # front 0 of 30 000 rows
+    cases["front0_30000_of_40000x4"] = (big2, [20000])
+    big3 = _simplex(70000, 3, g)
+    big3[20000:] = big3[20000:] * (1.5 + torch.rand(50000, 1, generator=g)) + 0.1  # (a population whose matrix comes from the objective orders)
+    cases["front0_20000_of_70000x3"] = (big3, [12000])
     return cases
 
 
