@@ -93,7 +93,7 @@ def test_large_last_front_against_the_c_checker_and_the_radix_path(name):
     runtime.release_workspaces()
 
 
-@pytest.mark.parametrize("n,m,keep", [(20000, 3, 1.0), (24576, 2, 0.6), (10000, 8, 0.9)])
+@pytest.mark.parametrize("n,m,keep", [(20000, 3, 1.0), (24576, 2, 0.6), (10000, 8, 0.9), (50000, 3, 0.4), (40000, 2, 1.0)])
 def test_crowding_distance_of_a_large_mask(n, m, keep):
     g = torch.Generator("cpu").manual_seed(n + m)
     costs = torch.rand(n, m, generator=g)
