@@ -268,6 +268,30 @@ def nd_select(x: torch.Tensor, f: torch.Tensor, topk: int) -> Tuple[torch.Tensor
         raise IndexError(f"topk must be at least 1; got {topk}")
     if m == 0:
         raise ValueError("fitness must have at least one objective")
+    if bd == 0 and f.dtype is torch.float32 and x.is_contiguous() and f.device.index == torch.cuda.current_device():
+        # One population of float32 fitness on the current device -- what an algorithm's step passes: the same call
+        # without the views and the device guard of the general path below (a third of the time of a selection of
+        # 200 rows is spent on this side of the C ABI).
+        out_x = torch.empty((topk,) + tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
+        out_f = torch.empty((topk, m), dtype=torch.float32, device=f.device)
+        out_rank = torch.empty((topk,), dtype=torch.int32, device=f.device)
+        out_dist = torch.empty((topk,), dtype=torch.float32, device=f.device)
+        es = x.element_size()
+        row_bytes = (x.numel() // n) * es
+        has_x = row_bytes > 0
+        stream = runtime.stream_handle(f.device)
+        if runtime.small_population_kernel_fits(n, m, 1):
+            _lib.call("evox_hip_batched_nd_environmental_selection", x.data_ptr() if has_x else None, row_bytes, row_bytes,
+                      n * row_bytes, f.data_ptr(), 1, n, m, n * f.stride(0), f.stride(0), f.stride(1), topk,
+                      out_x.data_ptr() if has_x else None, out_f.data_ptr(), out_rank.data_ptr(), out_dist.data_ptr(), stream)
+            runtime.note_small_kernel_call()
+        else:
+            ws = runtime.workspace(n, m, f.device)
+            _lib.call("evox_hip_nd_environmental_selection", x.data_ptr() if has_x else None, row_bytes, row_bytes,
+                      f.data_ptr(), n, m, f.stride(0), f.stride(1), topk, out_x.data_ptr() if has_x else None,
+                      out_f.data_ptr(), out_rank.data_ptr(), out_dist.data_ptr(), None, ws.data_ptr(), ws.numel(), stream)
+            runtime.note_call(ws, stream)
+        return out_x, out_f, out_rank, out_dist
     f32 = _as_f32(f, "fitness")
     batch = f.shape[:bd]
     tail = x.shape[bd + 1:]

@@ -36,10 +36,16 @@ def _lone_population_limit(m: int) -> int:
     return 160
 
 
+_batched_max_rows = {}  # objectives -> rows that the one-workgroup kernel takes (asked of the library once)
+
+
 def small_population_kernel_fits(n: int, m: int, batch: int) -> bool:
     if use_small_population_kernel is False:
         return False
-    if not 1 <= n <= int(_lib.lib().evox_hip_batched_max_rows(m)):
+    most = _batched_max_rows.get(m)
+    if most is None:
+        most = _batched_max_rows[m] = int(_lib.lib().evox_hip_batched_max_rows(m))
+    if not 1 <= n <= most:
         return False
     if use_small_population_kernel is True:
         return True
@@ -62,14 +68,21 @@ def stream_handle(device: torch.device) -> int:
     return int(torch.cuda.current_stream(device).cuda_stream)
 
 
+_workspace_need = {}  # (rows, objectives, with the matrix) -> bytes (asked of the library once per shape)
+
+
 def workspace(n: int, m: int, device: torch.device, with_matrix: bool = True) -> torch.Tensor:
     """A uint8 tensor of at least evox_hip_workspace_bytes(n, m) bytes, cached per (device, stream):
     calls on one stream are ordered, so they can share it.  ``with_matrix=False`` asks only for the
     bytes that the entry points without a dominance matrix need."""
-    query = _lib.lib().evox_hip_workspace_bytes if with_matrix else _lib.lib().evox_hip_first_front_workspace_bytes
-    need = int(query(n, m))
-    if need == 0:
-        raise ValueError(f"unsupported population shape n={n}, m={m}")
+    need = _workspace_need.get((n, m, with_matrix))
+    if need is None:
+        query = _lib.lib().evox_hip_workspace_bytes if with_matrix else _lib.lib().evox_hip_first_front_workspace_bytes
+        need = int(query(n, m))
+        if need == 0:
+            raise ValueError(f"unsupported population shape n={n}, m={m}")
+        if len(_workspace_need) < 4096:
+            _workspace_need[(n, m, with_matrix)] = need
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream_handle(device))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < need:
