@@ -59,3 +59,24 @@ def test_random_shapes_against_the_c_checker(seed):
         fin = np.isfinite(want)
         np.testing.assert_allclose(got[fin], want[fin], rtol=1e-5, err_msg=str(what))
     runtime.release_workspaces()
+
+
+def test_more_fronts_than_a_record_tag_counts():
+    """One objective, 71 099 distinct values: a front per row, more fronts than the 16-bit tags of the peel's records
+    count before they wrap.  The rank of a row is the dense rank of its value; the selection is the stable sort."""
+    g = torch.Generator("cpu").manual_seed(3)
+    n = 71099
+    f = torch.rand(n, 1, generator=g)
+    fd = f.to(DEV)
+    from evox_amd.operators.selection import non_dominate_rank
+
+    rank = non_dominate_rank(fd)
+    st = runtime.last_status()
+    want = torch.unique(f[:, 0], return_inverse=True)[1]
+    assert st["error"] == 0 and st["fronts"] == int(want.max()) + 1 > 65536
+    assert torch.equal(rank.cpu().long(), want)
+    x = torch.arange(n, dtype=torch.int32, device=DEV)[:, None]
+    xs, _, rs, _ = nd_environmental_selection(x, fd, n // 2)
+    order = torch.argsort(f[:, 0], stable=True)[: n // 2]
+    assert torch.equal(xs[:, 0].cpu().long(), order) and torch.equal(rs.cpu().long(), want[order])
+    runtime.release_workspaces()
