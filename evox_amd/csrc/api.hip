@@ -1329,9 +1329,9 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   g.order_from_peel = peel_always_orders ? 1 : 0;
   // Where the peel kernel may have ordered the last front, the kernels that would order it look at Ctrl.tail_done and
   // return at once.  A launch that does nothing still costs about 4.7 us, so with up to three objectives -- last
-  // fronts of a few hundred rows, which the peel kernel orders -- the two ordering stages share one launch
-  // (crowd_kernel); with more objectives the last front is usually too large for the peel kernel, and the two
-  // stages as kernels of their own, each on the grid that suits it, order it faster than the shared launch does
+  // fronts of a few hundred rows, which the peel kernel orders -- the two ordering stages and the gather share one
+  // launch (crowd_gather_kernel); with more objectives the last front is usually too large for the peel kernel, and
+  // the two stages as kernels of their own, each on the grid that suits it, order it faster than the shared launch does
   // (20 000 x 5, a front of 2532 rows: 245 against 261 us per selection; 20 000 x 8, 7481 rows: 457 against 493).
   const bool one_ordering_launch = peel_orders && opt().tail_merged && L.m <= 3;
   if (peel_always_orders) {
@@ -1355,28 +1355,24 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
     EVX_LAUNCH_CHECK();
     return 0;
   }
-  // the peel kernel may have ordered the last front: one launch for what is left of the ordering (nothing, then),
-  // one for the gather
+  // the peel kernel may have ordered the last front: one launch for what is left of the ordering (nothing, then) and
+  // the gather
   const size_t lds = crowd_lds_bytes(L, 2);
   const bool mid = crowd_mid_sort(L);
   const bool wide = L.n <= kMidArgsortWideRows;
-  const void* const kernel = !mid ? reinterpret_cast<const void*>(crowd_kernel<kRadixThreads, 0>)
-                             : wide ? reinterpret_cast<const void*>(crowd_kernel<kMidArgsortThreads, 1>)
-                                    : reinterpret_cast<const void*>(crowd_kernel<kMidArgsortThreads, 2>);
+  const void* const kernel = !mid ? reinterpret_cast<const void*>(crowd_gather_kernel<kRadixThreads, 0>)
+                             : wide ? reinterpret_cast<const void*>(crowd_gather_kernel<kMidArgsortThreads, 1>)
+                                    : reinterpret_cast<const void*>(crowd_gather_kernel<kMidArgsortThreads, 2>);
   if (int e = grant_dynamic_lds(kernel, lds)) return e;
   int grid = finish_grid(L, L.m);  // resident at once: at most two blocks of 256 threads per compute unit
   if (grid > device_cus() * 2) grid = device_cus() * 2;
+  const CrowdArgs ca = crowd_args(w, w.at<int>(L.perm), false, 2);
   if (mid && wide)
-    hipLaunchKernelGGL((crowd_kernel<kMidArgsortThreads, 1>), dim3(grid), dim3(kMidArgsortThreads), lds, s, crowd_args(w, w.at<int>(L.perm), false, 2));
+    hipLaunchKernelGGL((crowd_gather_kernel<kMidArgsortThreads, 1>), dim3(grid), dim3(kMidArgsortThreads), lds, s, ca, g);
   else if (mid)
-    hipLaunchKernelGGL((crowd_kernel<kMidArgsortThreads, 2>), dim3(grid), dim3(kMidArgsortThreads), lds, s, crowd_args(w, w.at<int>(L.perm), false, 2));
+    hipLaunchKernelGGL((crowd_gather_kernel<kMidArgsortThreads, 2>), dim3(grid), dim3(kMidArgsortThreads), lds, s, ca, g);
   else
-    hipLaunchKernelGGL((crowd_kernel<kRadixThreads, 0>), dim3(grid), dim3(kRadixThreads), lds, s, crowd_args(w, w.at<int>(L.perm), false, 2));
-  EVX_LAUNCH_CHECK();
-  int blocks = (int)((topk + 3) / 4);
-  const int cap = device_cus() * 8;
-  if (blocks > cap) blocks = cap;
-  hipLaunchKernelGGL(gather_after_peel_kernel, dim3(blocks), dim3(256), 0, s, g);
+    hipLaunchKernelGGL((crowd_gather_kernel<kRadixThreads, 0>), dim3(grid), dim3(kRadixThreads), lds, s, ca, g);
   EVX_LAUNCH_CHECK();
   return 0;
 }

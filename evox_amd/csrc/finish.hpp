@@ -547,11 +547,11 @@ __global__ __launch_bounds__(T) void crowd_finish_kernel(CrowdArgs a, int want_o
   crowd_finish_body<TABLES>(a, want_order, radix_generation_base(a.ctrl), 1, finish_lds, base, scratch);
 }
 
-// ---- The ordering of the last front in one launch, for populations whose peel kernel orders a small last front
-// itself (Ctrl.tail_done says whether it has: then nothing is left to do here).  A launch that finds nothing to do
-// still costs as much as a small kernel (about 4.7 us on this device), so the two stages share one launch; they are
-// separated by a counter barrier of all blocks.  Grid: that of crowd_sort_kernel (the radix grid: master, idle
-// block, workers), resident at once.
+// ---- The ordering of the last front in one launch (crowd_gather_kernel below), for populations whose peel kernel
+// orders a small last front itself (Ctrl.tail_done says whether it has: then nothing is left to order).  A launch
+// that finds nothing to do still costs as much as a small kernel (about 4.7 us on this device), so the two stages
+// share one launch; they are separated by a counter barrier of all blocks.  Grid: that of crowd_sort_kernel (the
+// radix grid: master, idle block, workers), resident at once.
 __device__ inline bool tail_barrier(Ctrl* ctrl, int target, unsigned spin_limit, int* scratch) {
   return counter_barrier(ctrl, 1, target, spin_limit, scratch);
 }
@@ -564,18 +564,32 @@ __global__ __launch_bounds__(256) void gather_after_peel_kernel(GatherArgs g) {
   gather_body(g, blockIdx.x, gridDim.x, g.ctrl->err == 0 && g.ctrl->tail_done != 0 ? g.ctrl->worst_start : 0);
 }
 
+// Both ordering stages and the gather of the selected rows behind them.  When the peel kernel has ordered the last
+// front -- the usual case where this kernel is launched -- the gather is all that is left, and it starts at once: one
+// launch after the peel instead of two or three.  Otherwise the order is complete when every block has passed the
+// second round of the barrier counter that separates the two ordering stages.  After a failed wait the gather writes
+// no rows (it looks at Ctrl.err).
 template <int T, int TABLES>
-__global__ __launch_bounds__(T) void crowd_kernel(CrowdArgs a) {
+__global__ __launch_bounds__(T) void crowd_gather_kernel(CrowdArgs a, GatherArgs g) {
   extern __shared__ __attribute__((aligned(16))) uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
   Ctrl* ctrl = a.ctrl;
-  if (coherent_load(&ctrl->err) != 0 || ctrl->tail_done != 0) return;
+  if (coherent_load(&ctrl->err) != 0) {
+    gather_body(g, blockIdx.x, gridDim.x, 0);
+    return;
+  }
+  if (ctrl->tail_done != 0) {
+    gather_body(g, blockIdx.x, gridDim.x, ctrl->worst_start);
+    return;
+  }
   const unsigned gen0 = radix_generation_base(ctrl);
   crowd_sort_body<TABLES>(a, gen0, 0, finish_lds, base, scratch);
   if (tail_barrier(ctrl, (int)gridDim.x, a.spin_limit, scratch))
     crowd_finish_body<TABLES>(a, 1, gen0 + 16u, 0, finish_lds, base, scratch);
   if (blockIdx.x == 0 && threadIdx.x == 0) ctrl->radix_epoch += 2;  // both bodies may have run a radix sort
+  counter_barrier(ctrl, 1, 2 * (int)gridDim.x, a.spin_limit, scratch);
+  gather_body(g, blockIdx.x, gridDim.x, 0);
 }
 
 }  // namespace evx

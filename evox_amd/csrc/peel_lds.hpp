@@ -115,6 +115,44 @@ __device__ inline void lds_row_highest(const uint64_t* row, int nw, const uint64
   }
 }
 
+// (sort key, original index below 32 768) as one number that a double holds exactly, and the key back out of it.
+__device__ inline double tail_composite(uint32_t key, int orig) {
+  return (double)(((unsigned long long)key << 15) | (unsigned)orig);
+}
+__device__ inline uint32_t tail_composite_key(double c) { return (uint32_t)((unsigned long long)c >> 15); }
+// (as instructions: the compiler's own maximum first makes sure that neither operand is a signalling NaN)
+__device__ inline double max_f64(double a, double b) {
+  double r;
+  asm("v_max_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ inline double min_f64(double a, double b) {
+  double r;
+  asm("v_min_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+// Lanes that share one item of the last front's scans when a workgroup of kLdsPeelThreads has `items` of them.
+__device__ inline int tail_group_lanes(int items) {
+  return items * 64 <= kLdsPeelThreads ? 64 : items * 32 <= kLdsPeelThreads ? 32 : 16;
+}
+__device__ inline double shfl_xor_f64(double v, int off) {
+  const unsigned long long b = (unsigned long long)__double_as_longlong(v);
+  const unsigned long long o = ((unsigned long long)__shfl_xor((unsigned)(b >> 32), off) << 32) | __shfl_xor((unsigned)b, off);
+  return __longlong_as_double((long long)o);
+}
+__device__ inline double group16_max(double v) {
+#pragma unroll
+  for (int r = 8; r >= 1; r >>= 1)
+    v = max_f64(v, __longlong_as_double((long long)row16_rotate((unsigned long long)__double_as_longlong(v), r)));
+  return v;
+}
+__device__ inline double group16_min(double v) {
+#pragma unroll
+  for (int r = 8; r >= 1; r >>= 1)
+    v = min_f64(v, __longlong_as_double((long long)row16_rotate((unsigned long long)__double_as_longlong(v), r)));
+  return v;
+}
+
 // Lists the set bits of a front bitmap of at most blockDim.x words (LDS) in ascending order into perm[base ...].  A
 // thread takes a word; when some word is dense (a front of neighbouring rows: 64 stores from one thread, one after
 // the other, made a level of the listing slower than a level of the peeling) the words are instead taken by whole
@@ -530,9 +568,12 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
       // front `level` is the last one: a small one is ordered right here (the overflow path leaves no slots in v)
       if (tail.mode == 2 && (flags & 1) == 0 && peel_tail_applies(size, tail.m)) {
         const int nv = size, start = ranked, want = stop_count - ranked, m = tail.m;
-        unsigned long long* comp = reinterpret_cast<unsigned long long*>(lds);  // [m][nv], then the distance composites
-        unsigned long long* ends = comp + (size_t)nv * m;                        // [m][2]
-        int* t_slot = reinterpret_cast<int*>(ends + 2 * m);                      // [nv]
+        // Composites (key << 15 | original index: at most 47 bits, the population has at most 32 768 rows) are held
+        // as doubles, which represent them exactly: the vector unit compares doubles and takes their maximum at the
+        // rate of 32-bit values, 64-bit integers at a quarter of it, and the scans below are nothing but comparisons.
+        double* comp = reinterpret_cast<double*>(lds);       // [m][nv], then the distance composites
+        double* ends = comp + (size_t)nv * m;                // [m][2]
+        int* t_slot = reinterpret_cast<int*>(ends + 2 * m);  // [nv]
         int* t_orig = t_slot + nv;                                               // [nv]
         int* rec_cnt = t_orig + nv;                                              // [256] rows per record, then their prefix
         EVX_TRACE(61, 0);
@@ -600,7 +641,7 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
           for (int q = 0; q < kPerThread; ++q) {
             const int idx = tid + q * kLdsPeelThreads;
             if (idx < nv * m) {
-              comp[idx] = ((unsigned long long)ordered_key(cost_v[q]) << 32) | (unsigned)orig_v[q];
+              comp[idx] = tail_composite(ordered_key(cost_v[q]), orig_v[q]);
               if (idx < nv) t_orig[idx] = orig_v[q];
             }
           }
@@ -608,18 +649,16 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
         lds_barrier();
         EVX_TRACE(61, 1);
         for (int k = wave; k < m; k += kWaves) {  // first and last composite of every objective
-          unsigned long long lo = ~0ull, hi = 0ull;
+          double lo = INFINITY, hi = -1.0;
           for (int e = lane; e < nv; e += 64) {
-            const unsigned long long c = comp[k * nv + e];
-            lo = c < lo ? c : lo;
-            hi = c > hi ? c : hi;
+            const double c = comp[k * nv + e];
+            lo = min_f64(lo, c);
+            hi = max_f64(hi, c);
           }
 #pragma unroll
           for (int off = 1; off < 64; off <<= 1) {
-            const unsigned long long a = ((unsigned long long)__shfl_xor((unsigned)(lo >> 32), off) << 32) | __shfl_xor((unsigned)lo, off);
-            const unsigned long long b = ((unsigned long long)__shfl_xor((unsigned)(hi >> 32), off) << 32) | __shfl_xor((unsigned)hi, off);
-            lo = a < lo ? a : lo;
-            hi = b > hi ? b : hi;
+            lo = min_f64(lo, shfl_xor_f64(lo, off));
+            hi = max_f64(hi, shfl_xor_f64(hi, off));
           }
           if (lane == 0) {
             ends[2 * k] = lo;
@@ -628,37 +667,43 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
         }
         lds_barrier();
         EVX_TRACE(59, 0);
-        const int sub = tid & 15;
-        // this workgroup's candidates are e = sb, sb + sweepers, ...; a group of sixteen lanes takes one (candidate,
+        // this workgroup's candidates are e = sb, sb + sweepers, ...; a group of lanes takes one (candidate,
         // objective) pair, so that the objectives of a candidate are scanned side by side, and leaves the term of
-        // the distance (NaN bit pattern 0xFFFFFFFF for "first or last of the objective") in LDS
-        const int groups = kLdsPeelThreads >> 4;
+        // the distance (NaN bit pattern 0xFFFFFFFF for "first or last of the objective") in LDS.  A group is sixteen
+        // lanes, or 32 or 64 when the workgroup has so few pairs that most of its lanes would have nothing to do.
         const int mine_n = sb < nv ? (nv - 1 - sb) / sweepers + 1 : 0;
+        const int gl = tail_group_lanes(mine_n * m);
+        const int sub = tid & (gl - 1);
+        const int groups = kLdsPeelThreads / gl;
         float* term_lds = reinterpret_cast<float*>(rec_cnt + 256);  // [candidates of this workgroup][m]
         constexpr uint32_t kBoundaryTerm = 0xFFFFFFFFu;
-        for (int it = tid >> 4; it < mine_n * m; it += groups) {  // (whole groups leave the loop together)
+        for (int it = tid / gl; it < mine_n * m; it += groups) {  // (whole groups leave the loop together)
           const int j = it / m, k = it - j * m;
           const int e = sb + j * sweepers;
-          const unsigned long long* row = comp + (size_t)k * nv;
-          const unsigned long long mine = row[e];
-          unsigned long long below = 0ull, above = ~0ull;  // no composite is zero or all ones
-          for (int p0 = sub; p0 < nv; p0 += 8 * 16) {  // eight partners per step, their LDS reads in flight together
-            unsigned long long c[8];
+          const double* row = comp + (size_t)k * nv;
+          const double mine = row[e];
+          double below = -1.0, above = INFINITY;  // no composite is negative or infinite
+          for (int p0 = sub; p0 < nv; p0 += 8 * gl) {  // eight partners per step, their LDS reads in flight together
+            double c[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) c[u] = p0 + 16 * u < nv ? row[p0 + 16 * u] : mine;
+            for (int u = 0; u < 8; ++u) c[u] = p0 + gl * u < nv ? row[p0 + gl * u] : mine;
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
-              if (c[u] < mine) below = c[u] > below ? c[u] : below;
-              if (c[u] > mine) above = c[u] < above ? c[u] : above;
+              below = max_f64(below, c[u] < mine ? c[u] : -1.0);
+              above = min_f64(above, c[u] > mine ? c[u] : INFINITY);
             }
           }
           below = group16_max(below);
           above = group16_min(above);
+          for (int off = 16; off < gl; off <<= 1) {
+            below = max_f64(below, shfl_xor_f64(below, off));
+            above = min_f64(above, shfl_xor_f64(above, off));
+          }
           if (sub == 0) {
             float term = __uint_as_float(kBoundaryTerm);  // first or last of this objective (non_dominate.py:226-227)
-            if (below != 0ull && above != ~0ull) {
-              const float span = cost_of_key((uint32_t)(ends[2 * k + 1] >> 32)) - cost_of_key((uint32_t)(ends[2 * k] >> 32));
-              term = (cost_of_key((uint32_t)(above >> 32)) - cost_of_key((uint32_t)(below >> 32))) / span;
+            if (below >= 0.0 && above != INFINITY) {
+              const float span = cost_of_key(tail_composite_key(ends[2 * k + 1])) - cost_of_key(tail_composite_key(ends[2 * k]));
+              term = (cost_of_key(tail_composite_key(above)) - cost_of_key(tail_composite_key(below))) / span;
             }
             term_lds[it] = term;
           }
@@ -698,16 +743,16 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
             if (pending0) {
               const unsigned long long a = ((unsigned long long)r0.y << 32) | r0.x, b = ((unsigned long long)r0.w << 32) | r0.z;
               if (a != 0ull && (e0 + 1 >= nv || b != 0ull)) {
-                comp[e0] = a;
-                if (e0 + 1 < nv) comp[e0 + 1] = b;
+                comp[e0] = tail_composite((uint32_t)(a >> 32), (int)(uint32_t)a);
+                if (e0 + 1 < nv) comp[e0 + 1] = tail_composite((uint32_t)(b >> 32), (int)(uint32_t)b);
                 pending0 = false;
               }
             }
             if (pending1) {
               const unsigned long long a = ((unsigned long long)r1.y << 32) | r1.x, b = ((unsigned long long)r1.w << 32) | r1.z;
               if (a != 0ull && (e0 + 3 >= nv || b != 0ull)) {
-                comp[e0 + 2] = a;
-                if (e0 + 3 < nv) comp[e0 + 3] = b;
+                comp[e0 + 2] = tail_composite((uint32_t)(a >> 32), (int)(uint32_t)a);
+                if (e0 + 3 < nv) comp[e0 + 3] = tail_composite((uint32_t)(b >> 32), (int)(uint32_t)b);
                 pending1 = false;
               }
             }
@@ -724,19 +769,21 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
         EVX_TRACE(61, 3);
         lds_barrier();
         if (next_cnts[3] == 0) {  // every entry has arrived (a wait that gave up, here or elsewhere, ended the polls)
-          for (int j = tid >> 4; j < mine_n; j += groups) {
+          const int gc = tail_group_lanes(mine_n), sub_c = tid & (gc - 1);
+          for (int j = tid / gc; j < mine_n; j += kLdsPeelThreads / gc) {
             const int e = sb + j * sweepers;
-            const unsigned long long mine = comp[e];
+            const double mine = comp[e];
             int smaller = 0;
-            for (int p0 = sub; p0 < nv; p0 += 8 * 16) {
-              unsigned long long c[8];
+            for (int p0 = sub_c; p0 < nv; p0 += 8 * gc) {
+              double c[8];
 #pragma unroll
-              for (int u = 0; u < 8; ++u) c[u] = p0 + 16 * u < nv ? comp[p0 + 16 * u] : ~0ull;
+              for (int u = 0; u < 8; ++u) c[u] = p0 + gc * u < nv ? comp[p0 + gc * u] : INFINITY;
 #pragma unroll
               for (int u = 0; u < 8; ++u) smaller += c[u] < mine;
             }
             smaller = group16_sum(smaller);
-            if (sub == 0 && smaller < want) tail.order[start + smaller] = (int)(unsigned)mine;
+            for (int off = 16; off < gc; off <<= 1) smaller += __shfl_xor(smaller, off);
+            if (sub_c == 0 && smaller < want) tail.order[start + smaller] = t_orig[e];
           }
           if (sb == 0 && tid == 0) ctrl->tail_done = 1;
           EVX_TRACE(60, 0);
