@@ -88,7 +88,7 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->fronts_orig = o; o = align_up(o + sizeof(uint64_t) * kFrontBuffers * kFrontStride * (size_t)L->nwords);
   L->hist = o;        o = align_up(o + sizeof(int) * (size_t)buckets);
   L->scanflags = o;   o = align_up(o + sizeof(unsigned long long) * 64);
-  L->tailbuf = o;     o = align_up(o + (n <= 32768 ? sizeof(unsigned long long) * kTailRows : 0));
+  L->tailbuf = o;     o = align_up(o + (n <= 32768 ? sizeof(unsigned long long) * kTailCopies * kTailRows : 0));
   L->records = o;     o = align_up(o + (n <= 32768 ? sizeof(unsigned long long) * kLdsPeelRecordUnits : (n <= kRecordsMaxRowsWide ? sizeof(unsigned long long) * kRecRing * kRecUnits : 0)));
   L->zero_end = o;
   L->fstart = o;     o = align_up(o + sizeof(int) * (size_t)(n + 2));

@@ -208,6 +208,7 @@ __device__ inline void list_front_words(const uint64_t* front_lds, int nwords, i
 // finish.hpp, except that the costs are read back from their order-preserving keys, under which -0.0 is +0.0 (the
 // sign of a distance of zero can differ) and every NaN is the same NaN.
 constexpr int kTailRows = 2048;        // candidates (four per thread in the poll of the buffer)
+constexpr int kTailCopies = 8;         // of the buffer that every workgroup polls: one per die, like the records
 constexpr int kTailValues = 4096;      // candidates x objectives: 12 bytes of LDS each
 constexpr int kTailObjectives = 64;
 
@@ -229,7 +230,7 @@ struct PeelTail {
   const float* xs_sorted;  // fitness by slot, structure of arrays, columns npad apart
   float* dist;             // by original index
   int* order;              // selection order
-  unsigned long long* buffer;  // kTailRows entries, zero at the start of the call
+  unsigned long long* buffer;  // kTailCopies x kTailRows entries, zero at the start of the call
 };
 
 // Grid: 1 lister + `sweepers` sweeping workgroups of kLdsPeelThreads threads, all resident at once (every workgroup
@@ -723,7 +724,9 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
           }
           const float d = boundary ? INFINITY : acc;
           coherent_store(&tail.dist[t_orig[e]], d);
-          coherent_store(&tail.buffer[e], ((unsigned long long)ordered_key(-d) << 32) | (unsigned)t_orig[e]);
+          const unsigned long long entry = ((unsigned long long)ordered_key(-d) << 32) | (unsigned)t_orig[e];
+#pragma unroll
+          for (int c = 0; c < kTailCopies; ++c) coherent_store(&tail.buffer[c * kTailRows + e], entry);
         }
         EVX_TRACE(61, 2);
         lds_barrier();  // the composites of the objectives are no longer needed
@@ -738,7 +741,7 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
             u32x4 r0, r1;
             asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1\n\ts_waitcnt vmcnt(0)"
                          : "=&v"(r0), "=&v"(r1)
-                         : "v"(tail.buffer + e0)
+                         : "v"(tail.buffer + (blockIdx.x % kTailCopies) * kTailRows + e0)
                          : "memory");
             if (pending0) {
               const unsigned long long a = ((unsigned long long)r0.y << 32) | r0.x, b = ((unsigned long long)r0.w << 32) | r0.z;
