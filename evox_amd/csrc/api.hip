@@ -1,9 +1,10 @@
 // C ABI of libevox_hip.so (declared in include/evox_hip.h): argument checks, workspace layout
 // and kernel launches.  Nothing here allocates device memory or waits for the device, except
-// evox_hip_read_status().
+// evox_hip_read_status(); the selection entry points keep 64 bytes of pinned host memory per device (outcome_slot).
 #include <string.h>
 
 #include <atomic>
+#include <mutex>
 #include <new>
 
 #include "../../include/evox_hip.h"
@@ -36,6 +37,7 @@ struct Options {
   int peel_lds_blocks = 0;  // sweeping workgroups of that kernel, 0 = by size
   int peel_tail = 1;        // that kernel also orders a small last front (0: always the kernels of finish.hpp)
   int tail_merged = 1;      // after such a peel, ordering (where still needed) and gather share one launch
+  int launch_memory = 1;    // ... unless the last selection of this shape had a last front that the peel left alone
   unsigned spin_limit = 4000000u;
   int dominance_tile_words = 0;  // 0 = by size (2 or 4)
   int mid_argsort = 1;  // an argsort step of 8193 .. kMidArgsortRows positions in one kernel without waits (0: the radix sort)
@@ -158,6 +160,42 @@ static int device_cus() {
     cached[dev] = v;
   }
   return cached[dev];
+}
+
+// What the last selections on this device found, for the choice of launches of the next one: sixteen words of pinned
+// host memory per device, which the last kernel of a selection writes (1: the peel kernel ordered the last front, 2: it
+// left it to the ordering kernels) and the host reads at its next call of that shape without waiting for anything --
+// a stale or missing word costs a few microseconds, never a result.  Allocated at the first selection on a device
+// that may allocate (not during a stream capture); null until then and for callers that may not.
+static int* outcome_slot(int64_t n, int64_t m, bool may_allocate, hipStream_t s) {
+  static std::atomic<int*> words[64];
+  static std::atomic<bool> failed[64];
+  static std::mutex mu;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  int* base = words[dev].load(std::memory_order_acquire);
+  if (base == nullptr) {
+    if (!may_allocate || failed[dev].load(std::memory_order_relaxed)) return nullptr;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    base = words[dev].load(std::memory_order_acquire);
+    if (base == nullptr) {
+      void* p = nullptr;
+      if (hipHostMalloc(&p, 64, hipHostMallocDefault) != hipSuccess || p == nullptr) {
+        (void)hipGetLastError();
+        failed[dev].store(true, std::memory_order_relaxed);
+        return nullptr;
+      }
+      memset(p, 0, 64);
+      base = static_cast<int*>(p);
+      words[dev].store(base, std::memory_order_release);
+    }
+  }
+  return base + (int)(((uint64_t)n * 31u + (uint64_t)m) & 15u);
 }
 
 #define EVX_LAUNCH_CHECK()                          \
@@ -947,6 +985,8 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.peel_lds = (int)value;
   } else if (!strcmp(name, "tail_merged") && (value == 0 || value == 1)) {
     o.tail_merged = (int)value;
+  } else if (!strcmp(name, "launch_memory") && (value == 0 || value == 1)) {
+    o.launch_memory = (int)value;
   } else if (!strcmp(name, "peel_tail") && (value == 0 || value == 1)) {
     o.peel_tail = (int)value;
   } else if (!strcmp(name, "peel_lds_blocks") && (value == 0 || (value >= 8 && value <= 255))) {
@@ -1281,7 +1321,7 @@ int evox_hip_stable_argsort_step_batched(const void* key, int kind, int64_t batc
 static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes, const void* x2,
                        int64_t x2_row_stride_bytes, const Fitness& fit, int64_t n, int64_t m, int64_t topk, void* out_x,
                        float* out_f, int32_t* out_rank, float* out_dist, int32_t* out_order, void* ws, size_t ws_bytes,
-                       hipStream_t s) {
+                       hipStream_t s, bool may_allocate) {
   Ws w;
   if (out_f == nullptr || out_rank == nullptr || out_dist == nullptr) return kErrBadArg;
   if ((x == nullptr) != (out_x == nullptr) || (x == nullptr) != (x2 == nullptr)) return kErrBadArg;
@@ -1327,13 +1367,18 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   g.out_order = out_order;
   g.ctrl = w.ctrl();
   g.order_from_peel = peel_always_orders ? 1 : 0;
+  g.outcome = peel_orders && !peel_always_orders && opt().launch_memory ? outcome_slot(n, m, may_allocate, s) : nullptr;
+  const int last_outcome = g.outcome != nullptr ? __atomic_load_n(g.outcome, __ATOMIC_RELAXED) : 0;
   // Where the peel kernel may have ordered the last front, the kernels that would order it look at Ctrl.tail_done and
   // return at once.  A launch that does nothing still costs about 4.7 us, so with up to three objectives -- last
   // fronts of a few hundred rows, which the peel kernel orders -- the two ordering stages and the gather share one
   // launch (crowd_gather_kernel); with more objectives the last front is usually too large for the peel kernel, and
   // the two stages as kernels of their own, each on the grid that suits it, order it faster than the shared launch does
   // (20 000 x 5, a front of 2532 rows: 245 against 261 us per selection; 20 000 x 8, 7481 rows: 457 against 493).
-  const bool one_ordering_launch = peel_orders && opt().tail_merged && L.m <= 3;
+  // What the last selection of this shape found decides where it is known: a population that has converged keeps
+  // last fronts of thousands of rows, which the kernels of their own order 20-30 us faster (20 000 x 3, one front: 166
+  // against 194 us), and a last front that the peel ordered will mostly be followed by another.
+  const bool one_ordering_launch = peel_orders && opt().tail_merged && L.m <= 3 && last_outcome != 2;
   if (peel_always_orders) {
     int blocks = (int)((topk + 3) / 4);
     const int cap = device_cus() * 8;
@@ -1385,7 +1430,7 @@ int evox_hip_nd_environmental_selection(const void* x, int64_t x_row_bytes, int6
                                         size_t ws_bytes, void* stream) {
   if (f == nullptr) return kErrBadArg;
   return select_rows(x, x_row_bytes, x_row_stride_bytes, x, x_row_stride_bytes, one_part(f, n, sr, sc), n, m, topk, out_x,
-                     out_f, out_rank, out_dist, out_order, ws, ws_bytes, (hipStream_t)stream);
+                     out_f, out_rank, out_dist, out_order, ws, ws_bytes, (hipStream_t)stream, true);
 }
 
 int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_row_stride_bytes, const void* x_b,
@@ -1408,7 +1453,7 @@ int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_ro
   if (f_a == nullptr || f_b == nullptr) return kErrBadArg;
   const Fitness fit{f_a, f_a_stride_row, f_a_stride_col, n_a, f_b, f_b_stride_row, f_b_stride_col};
   return select_rows(x_a, x_row_bytes, x_a_row_stride_bytes, x_b, x_b_row_stride_bytes, fit, n_a + n_b, m, topk, out_x, out_f,
-                     out_rank, out_dist, out_order, ws, ws_bytes, (hipStream_t)stream);
+                     out_rank, out_dist, out_order, ws, ws_bytes, (hipStream_t)stream, true);
 }
 
 }  // extern "C"
@@ -1450,7 +1495,7 @@ int evox_hip_nd_environmental_selection_static(const void* x, int64_t x_row_byte
   // every call clears the part of the buffer that must start from zero (stage_prepare), whatever the call before
   // left there
   return select_rows(x, x_row_bytes, x_row_stride_bytes, x, x_row_stride_bytes, one_part(f, n, sr, sc), n, m, topk, out_x,
-                     out_f, out_rank, out_dist, out_order, ws, (size_t)EVOX_HIP_STATIC_SCRATCH_BYTES, (hipStream_t)stream);
+                     out_f, out_rank, out_dist, out_order, ws, (size_t)EVOX_HIP_STATIC_SCRATCH_BYTES, (hipStream_t)stream, false);
 }
 
 int64_t evox_hip_batched_max_rows(int64_t m) { return (m >= 1 && m <= kBatchedMaxObjectives) ? kBatchedMaxRows : 0; }

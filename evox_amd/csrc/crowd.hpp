@@ -141,6 +141,7 @@ struct GatherArgs {
   int* out_order;
   const Ctrl* ctrl;
   int order_from_peel;  // the host launched nothing that orders the last front: the peel kernel must have (Ctrl.tail_done)
+  int* outcome;  // pinned host memory or null: 1 when the peel kernel has ordered the last front of this call, else 2
 };
 
 // Called by every thread of `blocks` blocks of 256 threads (`block` = the caller's index among them).
@@ -169,6 +170,9 @@ __device__ inline void gather_body(const GatherArgs& a, int block, int blocks, i
       for (int64_t b = t0; b < (int64_t)topk * x_row_bytes; b += threads) out_x[b] = 0xFF;
     return;
   }
+  // (for the host's choice of launches at its next call; it reads the word without waiting for anything)
+  if (a.outcome != nullptr && block == 0 && threadIdx.x == 0)
+    __hip_atomic_store(a.outcome, a.ctrl->tail_done != 0 ? 1 : 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   // A row is copied by g lanes, g = the smallest power of two (4 .. 64) that holds the row's units and its m
   // fitness values: short rows share a wave (a row of 400 bytes in 16-byte units took 25 of 64 lanes).
   const int64_t units = (x ? x_row_bytes : 0) / unit;

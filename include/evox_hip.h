@@ -257,7 +257,9 @@ int evox_hip_read_status(const void* workspace, void* stream, int32_t* host_out8
 
 /* Tunables (process-wide): "peel_lds" (1 = populations whose bit matrix fits the LDS of the device are peeled from LDS), "peel_lds_blocks"
  * (0 = by size, or 8 .. 255 sweeping workgroups of that kernel), "peel_tail" (1 = that kernel also orders a small last front), "tail_merged"
- * (1 = after such a peel the two ordering stages share one launch, up to three objectives),
+ * (1 = after such a peel the two ordering stages and the gather share one launch, up to three objectives), "launch_memory" (1 = ... unless
+ * the last selection of that shape on the device had a last front that the peel kernel left to the ordering kernels, which a word of
+ * pinned host memory tells: the library allocates 64 bytes of it per device at the first selection; 0 = never looked at),
  * "peel_blocks_per_cu" (default 2), "peel_witness" (1 = witness pass, 0 = popcount sweep), "peel_records" (1 = record
  * protocol, 0 = master barrier and front bitmaps), "peel_record_blocks" (0 = by size, or 16 .. 255), "spin_limit" (polls before a device-side
  * wait gives up, default 4000000), "dominance_tile_words" (0 = by size: 2 or 4; or 2, 4, 8, 16), "mid_argsort" (1 = an argsort step of 8193 to 32768 positions, and a last front of 1025 to 32768 rows, are ordered by workgroups that sort in LDS without waiting for each other; 0 = the radix sort and ranking by counting), "small_sort" (1 = one-kernel slot sort up to 4096 rows),

@@ -1,0 +1,48 @@
+"""The choice of launches after the peel follows what the last selection of the same shape found (a word of pinned
+host memory that the last kernel of a selection writes).  Whatever it says, stale or not, the results are those of
+the plain-C checker: selections with a small and with a large last front take turns here, so that every call meets
+the word left by a call of the other kind, and a run of equal calls meets its own."""
+
+import numpy as np
+import pytest
+import torch
+
+from evox_amd import runtime
+from evox_amd.operators.selection import nd_environmental_selection
+from oracle import c_oracle
+from tests.cases import as_np
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+
+
+def _check(f, k, got):
+    order, rank, dist, _ = c_oracle.select(as_np(f), k)
+    xs, fs, rs, ds = got
+    assert np.array_equal(as_np(xs)[:, 0].astype(np.int64), order)
+    assert np.array_equal(as_np(rs), rank[order])
+    gd, wd = as_np(ds), dist[order]
+    assert np.array_equal(np.isinf(gd), np.isinf(wd))
+    fin = np.isfinite(wd)
+    np.testing.assert_allclose(gd[fin], wd[fin], rtol=1e-5)
+
+
+@pytest.mark.parametrize("n,m", [(6000, 3), (3000, 2)])
+def test_small_and_large_last_fronts_in_turn(n, m):
+    g = torch.Generator("cpu").manual_seed(n + m)
+    uniform = torch.rand(n, m, generator=g)  # many fronts, the last one small: the peel kernel orders it
+    simplex = torch.rand(n, m, generator=g)
+    simplex = simplex / simplex.sum(dim=1, keepdim=True)  # one front: the ordering kernels have it
+    x = torch.arange(n, dtype=torch.int32, device=DEV)[:, None]
+    sizes = []
+    for f in (uniform, uniform, simplex, simplex, uniform, simplex, uniform, uniform):
+        got = nd_environmental_selection(x, f.to(DEV), n // 2)
+        st = runtime.last_status()
+        assert st["error"] == 0
+        sizes.append(st["last_front_size"])
+        _check(f, n // 2, got)
+    assert min(sizes) < 1024 < max(sizes), sizes  # both kinds of last front were met
+    with runtime.options(launch_memory=0):
+        for f in (simplex, uniform):
+            _check(f, n // 2, nd_environmental_selection(x, f.to(DEV), n // 2))
+    runtime.release_workspaces()
