@@ -45,6 +45,9 @@ _SIGNATURES = {
     "evox_hip_batched_nd_environmental_selection": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                                             c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                                             c_void_p, c_void_p, c_void_p]),
+    "evox_hip_small_nd_environmental_selection_two_part": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64,
+                                                                   c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "evox_hip_tournament_pick": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p,
                                          c_void_p]),
     "evox_hip_argsort_workspace_bytes": (c_size_t, [c_int64]),

@@ -1548,6 +1548,44 @@ int evox_hip_batched_nd_environmental_selection(const void* x, int64_t x_row_byt
   return launch_batched(a, batch, (hipStream_t)stream);
 }
 
+int evox_hip_small_nd_environmental_selection_two_part(const void* x_a, const void* x_b, int64_t x_row_bytes,
+                                                       int64_t x_row_stride_bytes, const float* f_a, int64_t n_a,
+                                                       const float* f_b, int64_t n_b, int64_t m, int64_t stride_row,
+                                                       int64_t stride_col, int64_t topk, void* out_x, float* out_f,
+                                                       int32_t* out_rank, float* out_dist, void* stream) {
+  if (f_a == nullptr || f_b == nullptr || out_f == nullptr || out_rank == nullptr || out_dist == nullptr) return kErrBadArg;
+  if (n_a < 1 || n_b < 1 || n_a + n_b > kBatchedMaxRows || m < 1 || m > kBatchedMaxObjectives) return kErrBadArg;
+  const int64_t n = n_a + n_b;
+  if (topk < 1 || topk > n) return kErrBadArg;
+  if ((x_a == nullptr) != (out_x == nullptr) || (x_a == nullptr) != (x_b == nullptr)) return kErrBadArg;
+  if (x_a != nullptr && (x_row_bytes < 0 || x_row_stride_bytes < 0)) return kErrBadArg;
+  BatchedArgs a = {};
+  a.f = f_a;
+  a.f_stride_row = stride_row;
+  a.f_stride_col = stride_col;
+  a.n = (int)n;
+  a.m = (int)m;
+  a.stop_count = (int)topk;
+  a.n_first = (int)n_a;
+  // row i >= n_a of the population is row i - n_a of part b: f_a + i * stride_row + f_second
+  a.f_second = (f_b - f_a) - n_a * stride_row;
+  a.x = static_cast<const uint8_t*>(x_a);
+  a.x_row_stride = x_row_stride_bytes;
+  a.x_row_bytes = x_row_bytes;
+  a.out_x = static_cast<uint8_t*>(out_x);
+  a.out_f = out_f;
+  a.out_rank = out_rank;
+  a.out_dist = out_dist;
+  a.x_unit = 1;
+  if (x_a != nullptr) {
+    a.x_second = (static_cast<const uint8_t*>(x_b) - static_cast<const uint8_t*>(x_a)) - n_a * x_row_stride_bytes;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(x_a) | reinterpret_cast<uintptr_t>(x_b) | reinterpret_cast<uintptr_t>(out_x) |
+                           (uintptr_t)x_row_bytes | (uintptr_t)x_row_stride_bytes;
+    a.x_unit = (bits % 16 == 0) ? 16 : (bits % 4 == 0) ? 4 : 1;
+  }
+  return launch_batched(a, 1, (hipStream_t)stream);
+}
+
 int evox_hip_tournament_pick(const int64_t* parents, int64_t n_round, int64_t tournament_size, const float* fit,
                              int64_t n_candidates, int64_t n_keys, int64_t stride_row, int64_t stride_col, int64_t* out,
                              void* stream) {

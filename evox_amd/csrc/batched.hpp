@@ -40,6 +40,11 @@ struct BatchedArgs {
   const uint8_t* x;        // (batch, n, row_bytes) raw rows, or null
   int64_t x_stride_b, x_row_stride, x_row_bytes;
   int x_unit;              // 16, 4 or 1: copy granularity that pointers, strides and row size allow
+  // A population given as two tensors with the same strides (parents and offspring): rows from n_first on are read
+  // f_second elements (x: x_second bytes) further on, which is where the second tensor's row 0 lies from row n_first
+  // of the first.  One tensor: all zero.
+  int n_first;
+  int64_t f_second, x_second;
   uint8_t* out_x;          // (batch, topk, row_bytes)
   float* out_f;            // (batch, topk, m)
   int* out_rank;           // (batch, topk)
@@ -112,15 +117,20 @@ __device__ inline int position_by_counting(const uint64_t* tile, int* below, int
 // for the store before it costs a memory round trip per unit.
 template <class T>
 __device__ inline void gather_units(const uint8_t* __restrict__ xb, uint8_t* __restrict__ dst, const int* order,
-                                    int64_t x_row_stride, uint32_t row_units, uint32_t total, int j, int nt) {
+                                    int64_t x_row_stride, uint32_t row_units, uint32_t total, int j, int nt,
+                                    int n_first, int64_t x_second) {
+  auto row_at = [&](uint32_t p) {
+    const int src = order[p];
+    return xb + (int64_t)src * x_row_stride + (src >= n_first ? x_second : 0);
+  };
   for (uint32_t e = j; e < total; e += 4u * nt) {
     const uint32_t e1 = e + nt, e2 = e + 2u * nt, e3 = e + 3u * nt;
     const uint32_t c0 = e, c1 = e1 < total ? e1 : e, c2 = e2 < total ? e2 : e, c3 = e3 < total ? e3 : e;
     const uint32_t p0 = c0 / row_units, p1 = c1 / row_units, p2 = c2 / row_units, p3 = c3 / row_units;
-    const T v0 = *reinterpret_cast<const T*>(xb + (int64_t)order[p0] * x_row_stride + (int64_t)(c0 - p0 * row_units) * sizeof(T));
-    const T v1 = *reinterpret_cast<const T*>(xb + (int64_t)order[p1] * x_row_stride + (int64_t)(c1 - p1 * row_units) * sizeof(T));
-    const T v2 = *reinterpret_cast<const T*>(xb + (int64_t)order[p2] * x_row_stride + (int64_t)(c2 - p2 * row_units) * sizeof(T));
-    const T v3 = *reinterpret_cast<const T*>(xb + (int64_t)order[p3] * x_row_stride + (int64_t)(c3 - p3 * row_units) * sizeof(T));
+    const T v0 = *reinterpret_cast<const T*>(row_at(p0) + (int64_t)(c0 - p0 * row_units) * sizeof(T));
+    const T v1 = *reinterpret_cast<const T*>(row_at(p1) + (int64_t)(c1 - p1 * row_units) * sizeof(T));
+    const T v2 = *reinterpret_cast<const T*>(row_at(p2) + (int64_t)(c2 - p2 * row_units) * sizeof(T));
+    const T v3 = *reinterpret_cast<const T*>(row_at(p3) + (int64_t)(c3 - p3 * row_units) * sizeof(T));
     *reinterpret_cast<T*>(dst + (int64_t)c0 * sizeof(T)) = v0;
     if (e1 < total) *reinterpret_cast<T*>(dst + (int64_t)e1 * sizeof(T)) = v1;
     if (e2 < total) *reinterpret_cast<T*>(dst + (int64_t)e2 * sizeof(T)) = v2;
@@ -159,7 +169,8 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(M <= 12 ? 
   EVX_BATCH_TRACE(0);
   float xj[M];
 #pragma unroll
-  for (int k = 0; k < M; ++k) xj[k] = valid ? f[(int64_t)j * a.f_stride_row + k * a.f_stride_col] : nan;
+  for (int k = 0; k < M; ++k)
+    xj[k] = valid ? f[(int64_t)j * a.f_stride_row + k * a.f_stride_col + (j >= a.n_first ? a.f_second : 0)] : nan;
 
   // ---- dominance: word w of row j = which rows 64 w .. 64 w + 63 dominate row j.  When every value of
   // the population is finite the test is the arithmetic one of dominance.hpp (signs of the differences
@@ -183,11 +194,14 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(M <= 12 ? 
 #pragma unroll
     for (int h = 1; h >= 0; --h) {
       uint32_t acc = 0;
-      if (all_finite && packed_rows && w * 64 + h * 32 + 32 <= n) {
+      const int i0 = w * 64 + h * 32;
+      const int64_t second0 = i0 >= a.n_first ? a.f_second : 0;
+      if (all_finite && packed_rows && i0 + 32 <= n && (i0 + 32 <= a.n_first || i0 >= a.n_first)) {
         // rows of M consecutive floats: GP dominators are GP M consecutive scalars, fetched by wide scalar loads
+        // (the 32 dominators come from one tensor)
 #pragma unroll 1
         for (int g = 32 / GP - 1; g >= 0; --g) {
-          const ConstFloatPtr p = fc + (int64_t)(w * 64 + h * 32 + g * GP) * M;  // wave-uniform
+          const ConstFloatPtr p = fc + (int64_t)(i0 + g * GP) * M + second0;  // wave-uniform
           float v[GP * M];
 #pragma unroll
           for (int e = 0; e < GP * M; ++e) v[e] = p[e];
@@ -206,7 +220,8 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(M <= 12 ? 
           const int ic = i < n ? i : 0;
           uint32_t o = 0u;
 #pragma unroll
-          for (int k = 0; k < M; ++k) o |= __float_as_uint(xz[k] - fc[(int64_t)ic * a.f_stride_row + k * a.f_stride_col]);
+          for (int k = 0; k < M; ++k)
+            o |= __float_as_uint(xz[k] - fc[(int64_t)ic * a.f_stride_row + k * a.f_stride_col + (ic >= a.n_first ? a.f_second : 0)]);
           acc = shift_in_positive(acc, i < n ? o : 0u);
         }
       } else {
@@ -218,7 +233,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(M <= 12 ? 
           uint64_t lt = 0ull;
 #pragma unroll
           for (int k = 0; k < M; ++k) {
-            const float xi = fc[(int64_t)ic * a.f_stride_row + k * a.f_stride_col];
+            const float xi = fc[(int64_t)ic * a.f_stride_row + k * a.f_stride_col + (ic >= a.n_first ? a.f_second : 0)];
             le &= __builtin_amdgcn_ballot_w64(xi <= xj[k]);
             lt |= __builtin_amdgcn_ballot_w64(xi < xj[k]);
           }
@@ -339,13 +354,13 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(M <= 12 ? 
     const int64_t total = row_units * topk;
     if (a.x_unit >= 4 && total < (1ll << 31)) {
       if (a.x_unit == 16)
-        gather_units<uint4>(xb, dst, order, a.x_row_stride, (uint32_t)row_units, (uint32_t)total, j, nt);
+        gather_units<uint4>(xb, dst, order, a.x_row_stride, (uint32_t)row_units, (uint32_t)total, j, nt, a.n_first, a.x_second);
       else
-        gather_units<uint32_t>(xb, dst, order, a.x_row_stride, (uint32_t)row_units, (uint32_t)total, j, nt);
+        gather_units<uint32_t>(xb, dst, order, a.x_row_stride, (uint32_t)row_units, (uint32_t)total, j, nt, a.n_first, a.x_second);
     } else {
       const int waves = nt >> 6;
       for (int p = wave; p < topk; p += waves) {
-        const uint8_t* __restrict__ sp = xb + (int64_t)order[p] * a.x_row_stride;
+        const uint8_t* __restrict__ sp = xb + (int64_t)order[p] * a.x_row_stride + (order[p] >= a.n_first ? a.x_second : 0);
         uint8_t* __restrict__ dp = dst + (int64_t)p * a.x_row_bytes;
         if (a.x_unit == 16) {
           for (int64_t b = lane * 16; b < a.x_row_bytes; b += 64 * 16)

@@ -379,6 +379,23 @@ def nd_select_two_part(x_a: torch.Tensor, f_a: torch.Tensor, x_b: torch.Tensor, 
         raise IndexError(f"topk must be at least 1; got {topk}")
     if m == 0:
         raise ValueError("fitness must have at least one objective")
+    if (n_a > 0 and n_b > 0 and f_a.dtype is torch.float32 and f_a.stride() == f_b.stride() and x_a.is_contiguous()
+            and x_b.is_contiguous() and f_a.device.index == torch.cuda.current_device()
+            and runtime.small_population_kernel_fits(n, m, 1)):
+        # parents and offspring of a run with a few hundred individuals: one launch of the one-workgroup kernel,
+        # which reads both parts where they lie (the pipeline's four launches took half as long again)
+        out_x = torch.empty((topk,) + tuple(x_a.shape[1:]), dtype=x_a.dtype, device=x_a.device)
+        out_f = torch.empty((topk, m), dtype=torch.float32, device=f_a.device)
+        out_rank = torch.empty((topk,), dtype=torch.int32, device=f_a.device)
+        out_dist = torch.empty((topk,), dtype=torch.float32, device=f_a.device)
+        row_bytes = (x_a.numel() // n_a) * x_a.element_size()
+        has_x = row_bytes > 0
+        _lib.call("evox_hip_small_nd_environmental_selection_two_part", x_a.data_ptr() if has_x else None,
+                  x_b.data_ptr() if has_x else None, row_bytes, row_bytes, f_a.data_ptr(), n_a, f_b.data_ptr(), n_b, m,
+                  f_a.stride(0), f_a.stride(1), topk, out_x.data_ptr() if has_x else None, out_f.data_ptr(),
+                  out_rank.data_ptr(), out_dist.data_ptr(), runtime.stream_handle(f_a.device))
+        runtime.note_small_kernel_call()
+        return out_x, out_f, out_rank, out_dist
     fa32, fb32 = _as_f32(f_a, "fitness"), _as_f32(f_b, "fitness")
     tail = x_a.shape[1:]
     out_x = torch.empty(topk, *tail, dtype=x_a.dtype, device=x_a.device)

@@ -135,6 +135,18 @@ int evox_hip_batched_nd_environmental_selection(const void* x, int64_t x_row_byt
                                                 int64_t topk, void* out_x, float* out_f, int32_t* out_rank, float* out_dist,
                                                 void* stream);
 
+/* One small population given in two parts of equal strides (parents and offspring of NSGA-II,
+ * src/evox/algorithms/mo/nsga2.py:99-102, at the population sizes such runs mostly have: a few hundred rows): the
+ * selection of evox_hip_nd_environmental_selection_two_part in the one-workgroup kernel of the entry points above,
+ * one launch and no workspace.  n_a, n_b >= 1, n_a + n_b <= evox_hip_batched_max_rows(m); both fitness parts are
+ * addressed as f[i * stride_row + k * stride_col], both parts of x as rows of x_row_bytes bytes x_row_stride_bytes
+ * apart.  Results equal those of the other entry points on the concatenation. */
+int evox_hip_small_nd_environmental_selection_two_part(const void* x_a, const void* x_b, int64_t x_row_bytes,
+                                                       int64_t x_row_stride_bytes, const float* f_a, int64_t n_a,
+                                                       const float* f_b, int64_t n_b, int64_t m, int64_t stride_row,
+                                                       int64_t stride_col, int64_t topk, void* out_x, float* out_f,
+                                                       int32_t* out_rank, float* out_dist, void* stream);
+
 /* out[r] (int64) = the winner of tournament r: among parents[r * tournament_size + 0 .. tournament_size-1]
  * (int64 candidate indices, values in [0, n_candidates)) the one that sorts first by the LAST key column of
  * fit, ties by the column before it, ..., ties by position in the tournament; NaN after every number.

@@ -87,7 +87,13 @@ def test_argument_validation_without_gpu(handle):
                                                                p, None, p, 64, None) == _lib.E_BAD_ARG  # missing part
     assert handle.evox_hip_nd_environmental_selection_two_part(None, 0, None, 0, 0, p, 5, 3, 1, p, 5, 3, 1, 3, 4, None, p, p, p,
                                                                None, p, 64, None) == _lib.E_WORKSPACE
+    small = handle.evox_hip_small_nd_environmental_selection_two_part
+    assert small(None, None, 0, 0, p, 5, p, 5, 3, 3, 1, 11, None, p, p, p, None) == _lib.E_BAD_ARG  # topk > n_a + n_b
+    assert small(None, None, 0, 0, p, 5, None, 5, 3, 3, 1, 4, None, p, p, p, None) == _lib.E_BAD_ARG  # missing part
+    assert small(None, None, 0, 0, p, 5, p, 0, 3, 3, 1, 4, None, p, p, p, None) == _lib.E_BAD_ARG  # a part without rows
+    assert small(None, None, 0, 0, p, 1000, p, 25, 3, 3, 1, 4, None, p, p, p, None) == _lib.E_BAD_ARG  # more than 1024 rows
     assert handle.evox_hip_set_option(b"no_such_option", 1) == _lib.E_BAD_ARG
+    assert handle.evox_hip_set_option(b"launch_memory", 1) == 0
     assert handle.evox_hip_set_option(b"peel_blocks_per_cu", 2) == 0
     # tunables for the calls of one thread: created from the process-wide ones, set by name, handed over and taken back
     opts = handle.evox_hip_options_create()
