@@ -40,6 +40,7 @@ struct Options {
   int launch_memory = 1;    // ... unless the last selection of this shape had a last front that the peel left alone
   unsigned spin_limit = 4000000u;
   int dominance_tile_words = 0;  // 0 = by size (2 or 4)
+  int dominance_folded = 1;      // tiles of two words: only the blocks at or below the diagonal are launched
   int mid_argsort = 1;  // an argsort step of 8193 .. kMidArgsortRows positions in one kernel without waits (0: the radix sort)
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
   int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 8 objectives (a quarter
@@ -216,6 +217,13 @@ static void launch_dominance_m(const Ws& w, int variant, hipStream_t s) {
                        w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords,
                        w.at<SortParam>(L.sortparam));
   };
+  if (IW == 2 && variant == kDomAuto && opt().dominance_folded) {
+    const int row_blocks = (L.npad + 127) / 128;
+    hipLaunchKernelGGL(dominance_folded_kernel<M>, dim3((row_blocks + 1) / 2, (row_blocks - 1) / 2 + 2), dim3(256), 0, s,
+                       w.at<float>(L.xs_sorted), w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted),
+                       w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords, w.at<SortParam>(L.sortparam), row_blocks);
+    return;
+  }
   switch (variant) {
     case kDomTwoCompares: launch(dominance_kernel<M, IW, kDomTwoCompares>); break;
     case kDomKey64: launch(dominance_kernel<M, IW, kDomKey64>); break;
@@ -995,6 +1003,8 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.spin_limit = (unsigned)value;
   } else if (!strcmp(name, "dominance_tile_words") && (value == 0 || value == 2 || value == 4 || value == 8 || value == 16)) {
     o.dominance_tile_words = (int)value;
+  } else if (!strcmp(name, "dominance_folded") && (value == 0 || value == 1)) {
+    o.dominance_folded = (int)value;
   } else if (!strcmp(name, "small_sort") && (value == 0 || value == 1)) {
     o.small_sort = (int)value;
   } else if (!strcmp(name, "mid_argsort") && (value == 0 || value == 1)) {

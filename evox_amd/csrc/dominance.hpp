@@ -415,7 +415,7 @@ __device__ inline uint32_t dominance_half_word(const float* __restrict__ xs, con
 // 16-byte pieces of a row then reach the cache from the same block at about the same time and leave it as one
 // 32-byte sector (a block of four row groups and one tile wrote 50 MB for the 25 MB triangle of 20 000 x 3).
 template <int M, int IW, int VARIANT>
-__device__ inline void dominance_tile(int bx, int by, const float* __restrict__ xs, const uint64_t* __restrict__ key,
+__device__ __forceinline__ void dominance_tile(int bx, int by, const float* __restrict__ xs, const uint64_t* __restrict__ key,
                                       const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom, int n, int npad,
                                       int64_t wstride, int nwords, const SortParam* __restrict__ param) {
   const int lane = threadIdx.x & 63;
@@ -492,6 +492,25 @@ __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict_
                                                         int npad, int64_t wstride, int nwords,
                                                         const SortParam* __restrict__ param) {
   dominance_tile<M, IW, VARIANT>((int)blockIdx.x, (int)blockIdx.y, xs, key, kid, dom, n, npad, wstride, nwords, param);
+}
+
+// Tiles of two words without the blocks above the diagonal, which are half of the grid above and return at once:
+// row block x (128 rows) needs x / 2 + 1 blocks of tiles, row block row_blocks - 1 - x the rest of about
+// row_blocks / 2 + 2, so the two share column x of a grid of ceil(row_blocks / 2) x ((row_blocks - 1) / 2 + 2) blocks.
+template <int M>
+__global__ __launch_bounds__(256) void dominance_folded_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
+                                                               const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom,
+                                                               int n, int npad, int64_t wstride, int nwords,
+                                                               const SortParam* __restrict__ param, int row_blocks) {
+  const int x = (int)blockIdx.x, y = (int)blockIdx.y;
+  const int own = x / 2 + 1;
+  int bx = x, by = y;
+  if (y >= own) {
+    bx = row_blocks - 1 - x;
+    by = y - own;
+    if (bx <= x || by > bx / 2) return;  // the middle row block has no partner; past the partner's diagonal
+  }
+  dominance_tile<M, 2, kDomAuto>(bx, by, xs, key, kid, dom, n, npad, wstride, nwords, param);
 }
 
 // The same matrix for a population that holds a NaN or an infinity, launched beside the kernels of prefix.hpp,

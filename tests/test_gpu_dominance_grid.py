@@ -1,0 +1,37 @@
+"""The dominance kernel's two grids for tiles of two words -- every block of the rectangle, or only those at or below
+the diagonal, two row blocks sharing a column of the grid -- must leave the same matrix: ranks of the whole population
+against the plain-C checker for both, at row-block counts that are odd, even and too small to fold."""
+
+import numpy as np
+import pytest
+import torch
+
+from evox_amd import runtime
+from evox_amd.operators.selection import non_dominate_rank
+from oracle import c_oracle
+from tests.cases import as_np
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+
+
+# rows -> row blocks of 128: 1, 2, 3, 4, 5, 40, 41, 79, 157 (the pipeline takes a lone population from 897 rows on;
+# smaller ones reach the kernel with the one-workgroup kernel switched off)
+@pytest.mark.parametrize("n", [100, 200, 300, 512, 640, 5100, 5200, 10050, 20000])
+@pytest.mark.parametrize("m", [2, 3, 5])
+def test_folded_and_full_grid_agree_with_the_checker(n, m):
+    g = torch.Generator("cpu").manual_seed(n * 7 + m)
+    f = torch.rand(n, m, generator=g)
+    f[: n // 10] = f[n // 10: 2 * (n // 10)]  # equal rows
+    want, _ = c_oracle.nd_rank(as_np(f))
+    fd = f.to(DEV)
+    runtime.use_small_population_kernel = False
+    try:
+        for folded in (1, 0):
+            with runtime.options(dominance_folded=folded):
+                got = as_np(non_dominate_rank(fd))
+                assert runtime.last_status()["error"] == 0
+            assert np.array_equal(got, want), (n, m, folded)
+    finally:
+        runtime.use_small_population_kernel = None
+    runtime.release_workspaces()
