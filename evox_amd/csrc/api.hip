@@ -217,9 +217,10 @@ static void launch_dominance_m(const Ws& w, int variant, hipStream_t s) {
                        w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords,
                        w.at<SortParam>(L.sortparam));
   };
-  if (IW == 2 && variant == kDomAuto && opt().dominance_folded) {
-    const int row_blocks = (L.npad + 127) / 128;
-    hipLaunchKernelGGL(dominance_folded_kernel<M>, dim3((row_blocks + 1) / 2, (row_blocks - 1) / 2 + 2), dim3(256), 0, s,
+  if ((IW == 2 || IW == 4) && variant == kDomAuto && opt().dominance_folded) {
+    const int row_blocks = IW == 2 ? (L.npad + 127) / 128 : (L.npad + 255) / 256;
+    const int column = IW == 2 ? (row_blocks - 1) / 2 + 2 : row_blocks + 1;
+    hipLaunchKernelGGL((dominance_folded_kernel<M, (IW == 2 ? 2 : 4)>), dim3((row_blocks + 1) / 2, column), dim3(256), 0, s,
                        w.at<float>(L.xs_sorted), w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted),
                        w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords, w.at<SortParam>(L.sortparam), row_blocks);
     return;

@@ -494,23 +494,25 @@ __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict_
   dominance_tile<M, IW, VARIANT>((int)blockIdx.x, (int)blockIdx.y, xs, key, kid, dom, n, npad, wstride, nwords, param);
 }
 
-// Tiles of two words without the blocks above the diagonal, which are half of the grid above and return at once:
-// row block x (128 rows) needs x / 2 + 1 blocks of tiles, row block row_blocks - 1 - x the rest of about
+// The grid without the blocks above the diagonal, which are half of the rectangle above and return at once.  Tiles of
+// two words: row block x (128 rows) needs x / 2 + 1 blocks of tiles, row block row_blocks - 1 - x the rest of about
 // row_blocks / 2 + 2, so the two share column x of a grid of ceil(row_blocks / 2) x ((row_blocks - 1) / 2 + 2) blocks.
-template <int M>
+// Tiles of four words: row block x (256 rows) needs x + 1 tiles, the two together row_blocks + 1.
+template <int M, int IW>
 __global__ __launch_bounds__(256) void dominance_folded_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
                                                                const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom,
                                                                int n, int npad, int64_t wstride, int nwords,
                                                                const SortParam* __restrict__ param, int row_blocks) {
+  static_assert(IW == 2 || IW == 4, "tiles of two or four words");
   const int x = (int)blockIdx.x, y = (int)blockIdx.y;
-  const int own = x / 2 + 1;
+  const int own = IW == 2 ? x / 2 + 1 : x + 1;
   int bx = x, by = y;
   if (y >= own) {
     bx = row_blocks - 1 - x;
     by = y - own;
-    if (bx <= x || by > bx / 2) return;  // the middle row block has no partner; past the partner's diagonal
+    if (bx <= x || by > (IW == 2 ? bx / 2 : bx)) return;  // the middle row block has no partner; past the partner's diagonal
   }
-  dominance_tile<M, 2, kDomAuto>(bx, by, xs, key, kid, dom, n, npad, wstride, nwords, param);
+  dominance_tile<M, IW, kDomAuto>(bx, by, xs, key, kid, dom, n, npad, wstride, nwords, param);
 }
 
 // The same matrix for a population that holds a NaN or an infinity, launched beside the kernels of prefix.hpp,

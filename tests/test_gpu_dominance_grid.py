@@ -1,5 +1,5 @@
-"""The dominance kernel's two grids for tiles of two words -- every block of the rectangle, or only those at or below
-the diagonal, two row blocks sharing a column of the grid -- must leave the same matrix: ranks of the whole population
+"""The dominance kernel's two grids -- every block of the rectangle, or only those at or below
+the diagonal, two row blocks sharing a column of the grid -- must leave the same matrix, with tiles of two words and of four: ranks of the whole population
 against the plain-C checker for both, at row-block counts that are odd, even and too small to fold."""
 
 import numpy as np
@@ -17,7 +17,8 @@ DEV = torch.device("cuda", 0)
 
 # rows -> row blocks of 128: 1, 2, 3, 4, 5, 40, 41, 79, 157 (the pipeline takes a lone population from 897 rows on;
 # smaller ones reach the kernel with the one-workgroup kernel switched off)
-@pytest.mark.parametrize("n", [100, 200, 300, 512, 640, 5100, 5200, 10050, 20000])
+# Tiles of four words (more than 24 576 rows, 32 768 from six objectives on): row blocks of 256, 129 and 157 of them.
+@pytest.mark.parametrize("n", [100, 200, 300, 512, 640, 5100, 5200, 10050, 20000, 33000, 40001])
 @pytest.mark.parametrize("m", [2, 3, 5])
 def test_folded_and_full_grid_agree_with_the_checker(n, m):
     g = torch.Generator("cpu").manual_seed(n * 7 + m)
