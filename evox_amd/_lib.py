@@ -45,6 +45,8 @@ _SIGNATURES = {
     "evox_hip_batched_nd_environmental_selection": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                                             c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                                             c_void_p, c_void_p, c_void_p]),
+    "evox_hip_tournament_pick_keys": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+                                              c_void_p]),
     "evox_hip_small_nd_environmental_selection_two_part": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64,
                                                                    c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                                                    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),

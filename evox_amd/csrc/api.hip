@@ -1612,6 +1612,29 @@ int evox_hip_tournament_pick(const int64_t* parents, int64_t n_round, int64_t to
   return 0;
 }
 
+int evox_hip_tournament_pick_keys(const int64_t* parents, int64_t n_round, int64_t tournament_size, int64_t n_candidates,
+                                  int64_t n_keys, const void* const* keys, const int32_t* kinds, const int64_t* strides,
+                                  int64_t* out, void* stream) {
+  if (parents == nullptr || keys == nullptr || kinds == nullptr || strides == nullptr || out == nullptr) return kErrBadArg;
+  if (n_round < 0 || tournament_size < 1 || tournament_size > 0x7FFFFFFF || n_candidates < 1 || n_keys < 1 || n_keys > 4)
+    return kErrBadArg;
+  TournamentKeys t = {};
+  for (int k = 0; k < (int)n_keys; ++k) {
+    if (keys[k] == nullptr || (kinds[k] != 0 && kinds[k] != 1)) return kErrBadArg;
+    t.key[k] = keys[k];
+    t.kind[k] = kinds[k];
+    t.stride[k] = strides[k];
+  }
+  t.nkeys = (int)n_keys;
+  if (n_round == 0) return 0;
+  int64_t blocks = (n_round + 255) / 256;
+  if (blocks > 65535) blocks = 65535;
+  hipLaunchKernelGGL(tournament_pick_keys_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, parents, n_round,
+                     (int)tournament_size, t, out);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
 size_t evox_hip_hv_workspace_bytes(int64_t n, int64_t n_sample) {
   if (n < 1 || n_sample < 1 || n > 0x7FFFFF00ll || n_sample > 0x7FFFFF00ll) return 0;
   const int point_chunk = hv_chunk_length(n, kHvPointChunk), sample_chunk = hv_chunk_length(n_sample, kHvChunk);

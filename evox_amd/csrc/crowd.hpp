@@ -238,4 +238,42 @@ __global__ __launch_bounds__(256) void tournament_pick_kernel(const int64_t* __r
   }
 }
 
+// The same tournaments on keys that lie in up to four arrays of their own -- what the caller of the reference passes
+// (a list of tensors, which the reference stacks: tournament_selection.py:23) -- so that no stacked copy is made.
+// kind 0: float32; kind 1: int32, compared as the float32 it converts to (the stack's type promotion).
+struct TournamentKeys {
+  const void* key[4];
+  int64_t stride[4];
+  int kind[4];
+  int nkeys;
+};
+
+__device__ inline uint32_t tournament_key_of(const void* base, int kind, int64_t at) {
+  return ordered_key(kind == 0 ? static_cast<const float*>(base)[at] : (float)static_cast<const int*>(base)[at]);
+}
+
+__global__ __launch_bounds__(256) void tournament_pick_keys_kernel(const int64_t* __restrict__ parents, int64_t n_round, int tsize,
+                                                                   TournamentKeys keys, int64_t* __restrict__ out) {
+  for (int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; r < n_round; r += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t* __restrict__ row = parents + r * tsize;
+    int64_t best = row[0];
+    for (int t = 1; t < tsize; ++t) {
+      const int64_t cand = row[t];
+      bool better = false, decided = false;
+#pragma unroll
+      for (int k = 3; k >= 0; --k) {  // (constant indices into the argument struct)
+        if (k >= keys.nkeys || decided) continue;
+        const uint32_t a = tournament_key_of(keys.key[k], keys.kind[k], cand * keys.stride[k]);
+        const uint32_t b = tournament_key_of(keys.key[k], keys.kind[k], best * keys.stride[k]);
+        if (a != b) {
+          better = a < b;
+          decided = true;
+        }
+      }
+      if (better) best = cand;
+    }
+    out[r] = best;
+  }
+}
+
 }  // namespace evx

@@ -19,6 +19,12 @@ def tournament_selection_multifit(n_round: int, fitnesses: List[torch.Tensor], t
     is won by the candidate that sorts first by the LAST tensor of ``fitnesses``, ties by the one
     before it, ..., ties by position in the tournament (NaN last).  The result is squeezed, as there.
     """
+    if ops.tournament_keys_fit(fitnesses):
+        # float32 and int32 vectors -- the crowding distances and ranks that NSGA-II passes: read where they lie
+        # (the stacked copy with its type promotion is two or three more launches than the tournaments themselves)
+        parents = torch.randint(0, fitnesses[0].size(0), (n_round, tournament_size), device=fitnesses[0].device)
+        pick = ops.tournament_pick_keys_direct if ops.plain_eager() else ops.tournament_pick_keys
+        return pick(parents, list(fitnesses)).squeeze()
     fitness_tensor = torch.stack(fitnesses, dim=1)
     num_candidates = fitness_tensor.size(0)
     parents = torch.randint(0, num_candidates, (n_round, tournament_size), device=fitnesses[0].device)

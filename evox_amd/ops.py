@@ -9,9 +9,12 @@ front; the operators themselves accept any number of leading batch dimensions, s
 need no extra registrations.
 """
 
-from typing import Optional, Tuple
+import ctypes
+from typing import List, Optional, Tuple
 
 import torch
+
+from torch.utils._python_dispatch import _get_current_dispatch_mode
 
 from . import _lib, runtime
 
@@ -641,3 +644,67 @@ def _tournament_pick_vmap(info, in_dims, parents, fitness):
 
 
 torch.library.register_vmap(tournament_pick, _tournament_pick_vmap)
+
+
+def tournament_keys_fit(keys) -> bool:
+    """Whether tournament_pick_keys takes this list of key tensors: one to four float32 or int32 vectors of one length
+    on one GPU (anything else goes through the stacked copy and tournament_pick)."""
+    if not 1 <= len(keys) <= 4:
+        return False
+    first = keys[0]
+    return all(isinstance(t, torch.Tensor) and t.is_cuda and t.dim() == 1 and t.dtype in (torch.float32, torch.int32)
+               and t.device == first.device and t.size(0) == first.size(0) for t in keys) and first.size(0) > 0
+
+
+def plain_eager() -> bool:
+    """True when no transform (vmap, grad), tracer (torch.compile, make_fx) or dispatch mode is looking at the call,
+    so that an operator's implementation may be called as the Python function it is: the dispatcher's way to the same
+    function costs about 10 us, a third of a host-bound call like a tournament selection."""
+    try:
+        return (not torch.compiler.is_compiling() and torch._C._functorch.peek_interpreter_stack() is None
+                and _get_current_dispatch_mode() is None)
+    except AttributeError:  # another torch: take the dispatcher
+        return False
+
+
+def tournament_pick_keys_direct(parents: torch.Tensor, keys: List[torch.Tensor]) -> torch.Tensor:
+    """parents (n_round, t) int64 candidate indices, keys: one to four (candidates,) float32 or int32 vectors ->
+    (n_round,) int64 winners, as tournament_pick on torch.stack(keys, dim=1) without making it."""
+    runtime.require_gpu_tensor(parents, "parents")
+    if parents.dim() != 2 or parents.dtype != torch.int64 or not tournament_keys_fit(keys):
+        raise ValueError("parents must be (n_round, tournament_size) int64 and keys one to four float32 or int32 vectors")
+    par = parents.contiguous()
+    out = torch.empty(par.size(0), dtype=torch.int64, device=parents.device)
+    count = len(keys)
+    pointers = (ctypes.c_void_p * count)(*[t.data_ptr() for t in keys])
+    kinds = (ctypes.c_int32 * count)(*[0 if t.dtype is torch.float32 else 1 for t in keys])
+    strides = (ctypes.c_int64 * count)(*[t.stride(0) for t in keys])
+    with torch.cuda.device(parents.device):
+        _lib.call("evox_hip_tournament_pick_keys", par.data_ptr(), par.size(0), par.size(1), keys[0].size(0), count,
+                  ctypes.addressof(pointers), ctypes.addressof(kinds), ctypes.addressof(strides), out.data_ptr(),
+                  runtime.stream_handle(parents.device))
+    return out
+
+
+@torch.library.custom_op("evox_amd::tournament_pick_keys", mutates_args=())
+def tournament_pick_keys(parents: torch.Tensor, keys: List[torch.Tensor]) -> torch.Tensor:
+    """tournament_pick_keys_direct as an operator (traceable, with a batching rule)."""
+    return tournament_pick_keys_direct(parents, keys)
+
+
+@tournament_pick_keys.register_fake
+def _(parents, keys):
+    return parents.new_empty(parents.shape[0])
+
+
+def _tournament_pick_keys_vmap(info, in_dims, parents, keys):
+    # mapped populations: the stacked form, whose batching rule puts all tournaments into one launch
+    parents_dim, keys_dims = in_dims
+    size = info.batch_size
+    moved = [k.movedim(d, 0) if d is not None else k.unsqueeze(0).expand(size, *k.shape) for k, d in zip(keys, keys_dims)]
+    par = parents.movedim(parents_dim, 0) if parents_dim is not None else parents.unsqueeze(0).expand(size, *parents.shape)
+    stacked = torch.stack([k.to(torch.float32) for k in moved], dim=-1)
+    return _tournament_pick_vmap(info, (0, 0), par, stacked)
+
+
+torch.library.register_vmap(tournament_pick_keys, _tournament_pick_keys_vmap)

@@ -158,6 +158,16 @@ int evox_hip_tournament_pick(const int64_t* parents, int64_t n_round, int64_t to
                              int64_t n_candidates, int64_t n_keys, int64_t stride_row, int64_t stride_col, int64_t* out,
                              void* stream);
 
+/* The same tournaments on the caller's list of key tensors as it is, without the stacked copy that
+ * tournament_selection_multifit makes of it (tournament_selection.py:23: torch.stack(fitnesses, dim=1), with int32
+ * ranks promoted to float32 beside float32 distances): keys, kinds and strides are HOST arrays of n_keys (1 .. 4)
+ * entries, read during the call -- keys[k] a device pointer to n_candidates values stride[k] elements apart, kinds[k]
+ * 0 for float32 and 1 for int32 (compared as the float32 it converts to, as after the stack).  The LAST key decides
+ * first, as above. */
+int evox_hip_tournament_pick_keys(const int64_t* parents, int64_t n_round, int64_t tournament_size, int64_t n_candidates,
+                                  int64_t n_keys, const void* const* keys, const int32_t* kinds, const int64_t* strides,
+                                  int64_t* out, void* stream);
+
 /* One step of evox.utils.lexsort (src/evox/utils/jit_fix_operator.py:246-250): order_out = prev_order
  * rearranged by a stable ascending sort of key[prev_order[.]] (NaN after every number, -0.0 and 0.0 tied);
  * prev_order == NULL is the identity (the first key, :246).  Chaining one call per key, in the order of the

@@ -87,6 +87,15 @@ def test_argument_validation_without_gpu(handle):
                                                                p, None, p, 64, None) == _lib.E_BAD_ARG  # missing part
     assert handle.evox_hip_nd_environmental_selection_two_part(None, 0, None, 0, 0, p, 5, 3, 1, p, 5, 3, 1, 3, 4, None, p, p, p,
                                                                None, p, 64, None) == _lib.E_WORKSPACE
+    three = (ctypes.c_void_p * 3)(p, p, None)
+    kinds = (ctypes.c_int32 * 3)(0, 1, 0)
+    strides = (ctypes.c_int64 * 3)(1, 1, 1)
+    by_keys = handle.evox_hip_tournament_pick_keys
+    assert by_keys(p, 4, 2, 10, 5, ctypes.addressof(three), ctypes.addressof(kinds), ctypes.addressof(strides), p, None) == _lib.E_BAD_ARG  # five keys
+    assert by_keys(p, 4, 2, 10, 3, ctypes.addressof(three), ctypes.addressof(kinds), ctypes.addressof(strides), p, None) == _lib.E_BAD_ARG  # a null key
+    kinds[1] = 7
+    assert by_keys(p, 4, 2, 10, 2, ctypes.addressof(three), ctypes.addressof(kinds), ctypes.addressof(strides), p, None) == _lib.E_BAD_ARG  # unknown kind
+    assert by_keys(p, 4, 0, 10, 1, ctypes.addressof(three), ctypes.addressof(kinds), ctypes.addressof(strides), p, None) == _lib.E_BAD_ARG
     small = handle.evox_hip_small_nd_environmental_selection_two_part
     assert small(None, None, 0, 0, p, 5, p, 5, 3, 3, 1, 11, None, p, p, p, None) == _lib.E_BAD_ARG  # topk > n_a + n_b
     assert small(None, None, 0, 0, p, 5, None, 5, 3, 3, 1, 4, None, p, p, p, None) == _lib.E_BAD_ARG  # missing part

@@ -1327,6 +1327,37 @@ def test_tournament_pick_against_oracle(tsize, population_path):
         assert np.array_equal(as_np(ops.tournament_pick(parents.to(DEV), table_t)), want)
 
 
+@pytest.mark.parametrize("tsize", [1, 2, 5])
+def test_tournament_pick_on_a_list_of_keys(tsize, population_path):
+    """The keys as the caller holds them (float32 distances, int32 ranks; strided views; one to four of them) give
+    the winners of the stacked table."""
+    if population_path != "pipeline":
+        pytest.skip("does not depend on the population path")
+    from evox_amd import ops
+
+    for seed, n_cand, n_round in ((1, 1, 5), (2, 6, 64), (3, 50, 3000), (4, 10000, 100000)):
+        say("tournament_keys", tsize, seed, n_cand, n_round)
+        parents, fits = _tournament_case(seed, n_cand, n_round, tsize)
+        want = as_np(er.tournament_winners(parents, fits)).reshape(-1)
+        keys = [k.to(DEV) for k in fits]
+        assert keys[0].dtype == torch.float32 and keys[1].dtype == torch.int32
+        assert np.array_equal(as_np(ops.tournament_pick_keys(parents.to(DEV), keys)), want), (tsize, seed)
+        # every second element of a longer vector: through the stride
+        wide = [torch.stack([k, k + 1], dim=1).reshape(-1)[::2] for k in keys]
+        assert n_cand == 1 or not wide[0].is_contiguous()
+        assert np.array_equal(as_np(ops.tournament_pick_keys(parents.to(DEV), wide)), want)
+        # one, three and four keys against the stacked table
+        g = torch.Generator("cpu").manual_seed(seed)
+        more = [torch.randint(0, 3, (n_cand,), generator=g).float().to(DEV) for _ in range(2)]
+        for chosen in ([keys[1]], [more[0], keys[0], keys[1]], [more[1], more[0], keys[0], keys[1]]):
+            table = torch.stack([k.float() for k in chosen], dim=1)
+            assert torch.equal(ops.tournament_pick_keys(parents.to(DEV), chosen), ops.tournament_pick(parents.to(DEV), table))
+    with pytest.raises(ValueError):
+        ops.tournament_pick_keys(parents.to(DEV), [keys[0].double()])
+    with pytest.raises(ValueError):
+        ops.tournament_pick_keys(parents.to(DEV), [keys[0]] * 5)
+
+
 def test_tournament_selection_multifit_follows_the_generator(population_path):
     """Same seed, same tournaments as the reference draws them (torch.randint on the fitness device),
     so the winners are those the restatement finds for that draw."""
