@@ -587,6 +587,13 @@ def main():
     if measured is not None:
         roofline["traffic"] = measured["bytes"]
         roofline["traffic_source"] = measured["source"]
+    from evox_amd import runtime as _runtime
+    if _runtime.small_population_kernel_fits(n, m, 1):
+        # a population this small is selected by one launch of the one-workgroup kernel (that is what ms_per_step
+        # times); the phases and this object describe the pipeline's kernels on the same rows, timed through the
+        # stage entry points
+        roofline["note"] = ("the timed step is one launch of batched_kernel; phases and roofline are the pipeline's "
+                            "stages on the same population")
 
     out = {
         "metric": "dominance comparisons/sec through nd_environmental_selection (N^2 ordered pairs per step)",
