@@ -43,9 +43,9 @@ struct Options {
   int dominance_folded = 1;      // tiles of two words: only the blocks at or below the diagonal are launched
   int mid_argsort = 1;  // an argsort step of 8193 .. kMidArgsortRows positions in one kernel without waits (0: the radix sort)
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
-  int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 to 8 objectives (a quarter
-                                    // more rows with 2, a quarter fewer with 9 to 16) get their matrix from the per-objective orders (prefix.hpp);
-                                    // 0 = never
+  int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 objectives (a quarter more
+                                    // with 2, fewer with more: half at 8, a quarter at 16 -- prefix_least_rows) get
+                                    // their matrix from the per-objective orders (prefix.hpp); 0 = never
   int64_t prefix_double_tile = 131072;  // order-based matrix, up to four objectives: from this many rows on a workgroup
                                         // takes both tiles of a 128-byte line; 0 = never
   int prefix_mode = 3;  // measurements: 1 = popcounts only, 2 = matrix only
@@ -332,15 +332,22 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
   return 0;
 }
 
-// Measured (matrix from the orders against pairwise, us): 49152 x 8: 373 / 373; 65536 x 2: 239 / 227, x 3: 277 / 287,
-// x 4: 305 / 366, x 8: 451 / 637; 100000 x 2: 370 / 558, x 3: 408 / 709; 200000 x 3: 1268 / 2622, x 8: 1624 / 5340.
+// From how many rows on the matrix comes from the per-objective orders: the pairwise kernel's work grows with the
+// objectives (two compares each per pair), the other's hardly does, and it starts from some 160 us for the orders
+// themselves.  Measured, a whole selection of uniform fitness in us, pairwise / from the orders:
+//   x 3: 60 000 521 / 530;  x 4: 40 000 300 / 337, 50 000 406 / 376;  x 5: 40 000 295 / 335, 50 000 395 / 350;
+//   x 6: 40 000 325 / 343, 50 000 439 / 352;  x 7: 33 000 302 / 315, 40 000 377 / 351;  x 8: 26 000 254 / 312,
+//   33 000 335 / 325, 50 000 584 / 386;  x 9: 20 000 251 / 305, 26 000 342 / 323;  x 10: 20 000 269 / 315, 26 000 363 / 329;
+//   x 12: 16 000 261 / 308, 20 000 312 / 307;  x 14: 16 000 301 / 327, 20 000 363 / 327;  x 16: 12 000 253 / 330,
+//   16 000 342 / 344, 20 000 424 / 352;  x 2 (65 536 rows): 227 / 239, (100 000) 558 / 370.
+// As thirty-seconds of the tunable (65 536 rows for three objectives):
+static int64_t prefix_least_rows(int m) {
+  const int parts = m <= 2 ? 40 : m == 3 ? 32 : m <= 5 ? 22 : m == 6 ? 20 : m == 7 ? 18 : m == 8 ? 16 : m <= 10 ? 12 : m <= 12 ? 10 : m <= 14 ? 9 : 8;
+  return opt().prefix_min_rows / 32 * parts + (opt().prefix_min_rows % 32 != 0 ? 1 : 0);
+}
 static bool prefix_dominance_applies(const Layout& L) {
   if (opt().prefix_min_rows <= 0 || L.m < 2 || L.m > kPrefixMaxObjectives) return false;
-  // (two objectives are cheap pair by pair: a quarter more rows before the orders pay; nine or more are dear: a
-  // quarter fewer -- 49152 x 9: 419 / 563, x 16: 675 / 933; 32768 x 9: 365 / 271, x 16: 622 / 464)
-  const int64_t q = opt().prefix_min_rows / 4;
-  const int64_t least = L.m == 2 ? opt().prefix_min_rows + q : (L.m >= 9 ? opt().prefix_min_rows - q : opt().prefix_min_rows);
-  return L.n >= least && L.n > kRadixMinCandidates && L.n <= kPrefixMaxRows;
+  return L.n >= prefix_least_rows(L.m) && L.n > kRadixMinCandidates && L.n <= kPrefixMaxRows;
 }
 static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s);
 
@@ -1733,7 +1740,7 @@ int evox_hip_peel_plan(int64_t n, int64_t m, int64_t* out3) {
   Layout L;
   if (out3 == nullptr || !make_layout(n, m, &L)) return kErrBadArg;
   size_t lds = 0;
-  const int sweepers = prefix_dominance_applies(L) ? 0 : lds_peel_plan(L, &lds);
+  const int sweepers = lds_peel_plan(L, &lds);
   out3[0] = sweepers != 0;
   out3[1] = sweepers;
   out3[2] = (int64_t)lds;
