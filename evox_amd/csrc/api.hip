@@ -44,7 +44,7 @@ struct Options {
   int mid_argsort = 1;  // an argsort step of 8193 .. kMidArgsortRows positions in one kernel without waits (0: the radix sort)
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
   int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 objectives (a quarter more
-                                    // with 2, fewer with more: half at 8, a quarter at 16 -- prefix_least_rows) get
+                                    // with 2, fewer with more: 28672 at 8, 10240 at 16 -- prefix_least_rows) get
                                     // their matrix from the per-objective orders (prefix.hpp); 0 = never
   int64_t prefix_double_tile = 131072;  // order-based matrix, up to four objectives: from this many rows on a workgroup
                                         // takes both tiles of a 128-byte line; 0 = never
@@ -341,8 +341,12 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
 //   x 12: 16 000 261 / 308, 20 000 312 / 307;  x 14: 16 000 301 / 327, 20 000 363 / 327;  x 16: 12 000 253 / 330,
 //   16 000 342 / 344, 20 000 424 / 352;  x 2 (65 536 rows): 227 / 239, (100 000) 558 / 370.
 // As thirty-seconds of the tunable (65 536 rows for three objectives):
+// Up to kMidArgsortRows rows the orders come from workgroups that sort in LDS and cost 60 to 90 us less:
+//   x 8: 26 000 254 / 261, 32 768 322 / 295;  x 9: 16 000 212 / 224, 20 000 252 / 236;  x 10: 16 000 222 / 231,
+//   20 000 268 / 245;  x 12: 12 000 198 / 210, 16 000 257 / 225;  x 16: 9000 220 / 215, 12 000 259 / 237.
 static int64_t prefix_least_rows(int m) {
-  const int parts = m <= 2 ? 40 : m == 3 ? 32 : m <= 5 ? 22 : m == 6 ? 20 : m == 7 ? 18 : m == 8 ? 16 : m <= 10 ? 12 : m <= 12 ? 10 : m <= 14 ? 9 : 8;
+  int parts = m <= 2 ? 40 : m == 3 ? 32 : m <= 5 ? 22 : m == 6 ? 20 : m == 7 ? 18 : m == 8 ? 16 : m <= 10 ? 12 : m <= 12 ? 10 : m <= 14 ? 9 : 8;
+  if (opt().mid_argsort && m >= 8) parts = m == 8 ? 14 : m <= 10 ? 9 : m <= 12 ? 7 : m <= 14 ? 6 : 5;
   return opt().prefix_min_rows / 32 * parts + (opt().prefix_min_rows % 32 != 0 ? 1 : 0);
 }
 static bool prefix_dominance_applies(const Layout& L) {
@@ -708,8 +712,35 @@ static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
 
 // The matrix of a large finite population from the order of its rows in every objective (prefix.hpp).  The
 // buffers of the crowding stage (radix pairs, pos, scost) are free until then and carry the orders.
+template <int M>
+static int launch_dominance_prefix(const Ws& w, hipStream_t s);
+static int dispatch_dominance_prefix(const Ws& w, hipStream_t s);
+
 static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) {
   const Layout& L = w.L;
+  if (L.n <= kMidArgsortRows && opt().mid_argsort) {
+    // the orders from workgroups that sort in LDS: two launches, no grid barrier (and no barrier words to reset)
+    const size_t sort_lds = mid_sort_lds_bytes(L.n);
+    const bool wide = L.n <= kMidArgsortWideRows;
+    const void* const kernel = wide ? reinterpret_cast<const void*>(objective_order_lds_kernel<true>)
+                                    : reinterpret_cast<const void*>(objective_order_lds_kernel<false>);
+    if (int e = grant_dynamic_lds(kernel, sort_lds)) return e;
+    if (wide)
+      hipLaunchKernelGGL(objective_order_lds_kernel<true>, dim3(device_cus()), dim3(kMidArgsortThreads), sort_lds, s, w.at<float>(L.xs),
+                         L.npad, L.n, L.m, w.at<SortParam>(L.sortparam), w.ctrl(), w.at<int>(L.total0), w.at<int>(L.witness0),
+                         radix_buffers(w));
+    else
+      hipLaunchKernelGGL(objective_order_lds_kernel<false>, dim3(device_cus()), dim3(kMidArgsortThreads), sort_lds, s, w.at<float>(L.xs),
+                         L.npad, L.n, L.m, w.at<SortParam>(L.sortparam), w.ctrl(), w.at<int>(L.total0), w.at<int>(L.witness0),
+                         radix_buffers(w));
+    EVX_LAUNCH_CHECK();
+    int64_t blocks = ((int64_t)L.n * L.m + 255) / 256;
+    if (blocks > device_cus() * 8) blocks = device_cus() * 8;
+    hipLaunchKernelGGL(objective_positions_kernel, dim3((unsigned)blocks), dim3(256), 0, s, L.n, L.m, w.at<int>(L.slot_of),
+                       w.at<SortParam>(L.sortparam), w.ctrl(), w.at<int>(L.pos), w.at<int>(L.scost), radix_buffers(w));
+    EVX_LAUNCH_CHECK();
+    return orders_only ? 0 : dispatch_dominance_prefix(w, s);
+  }
   const size_t lds = kRadixLdsBytes;
   if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(objective_order_kernel), lds)) return e;
   // more workers than one per 1024 rows: every one of them handles its share of all m segments
@@ -727,8 +758,11 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) 
   const int64_t words = (int64_t)((sizeof(Ctrl) + sizeof(unsigned long long) * kMaxGrid - first) / 4);
   hipLaunchKernelGGL(reset_state_kernel, dim3(16), dim3(256), 0, s, reinterpret_cast<uint32_t*>(w.base + L.ctrl + first), words);
   EVX_LAUNCH_CHECK();
-  if (orders_only) return 0;
-  switch (L.m) {
+  return orders_only ? 0 : dispatch_dominance_prefix(w, s);
+}
+
+static int dispatch_dominance_prefix(const Ws& w, hipStream_t s) {
+  switch (w.L.m) {
     case 2: return launch_dominance_prefix<2>(w, s);
     case 3: return launch_dominance_prefix<3>(w, s);
     case 4: return launch_dominance_prefix<4>(w, s);

@@ -122,6 +122,66 @@ __global__ __launch_bounds__(kRadixThreads) void objective_order_kernel(const fl
   if (wb == 0 && threadIdx.x == 0) param->orders_valid = 1;
 }
 
+// The same orders for populations of at most kMidArgsortRows rows, in two launches without a wait between
+// workgroups (the radix sort above spends 160 us on its twelve grid barriers whatever the size): the workgroups share
+// the objectives out, and each produces a run of positions of its objective's order from all keys of that objective
+// in its LDS (mid_argsort_slice); a second kernel derives pos and upper from the sorted pairs.
+// Grid: any (one workgroup per compute unit).  Dynamic LDS: mid_sort_lds_bytes(n).
+template <bool WIDE>
+__global__ __launch_bounds__(kMidArgsortThreads) void objective_order_lds_kernel(const float* __restrict__ xs, int npad, int n, int m,
+                                                                                 const SortParam* __restrict__ param,
+                                                                                 const Ctrl* __restrict__ ctrl,
+                                                                                 int* __restrict__ total0, int* __restrict__ witness0,
+                                                                                 RadixBuffers buf) {
+  extern __shared__ __attribute__((aligned(16))) uint64_t order_sort_lds[];
+  if (param->nonfinite != 0 || ctrl->err != 0) return;
+  for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < n; j += gridDim.x * blockDim.x) {
+    total0[j] = 0;
+    witness0[j] = -1;
+  }
+  const int nb = (int)gridDim.x;
+  const int per_objective = nb >= m ? nb / m : 1;  // workgroups that share an objective
+  const int run = ((n + per_objective - 1) / per_objective + 15) & ~15;
+  for (int item = blockIdx.x; item < per_objective * m; item += nb) {
+    const int k = item % m, s0 = (item / m) * run;
+    if (s0 >= n) continue;
+    const float* __restrict__ col = xs + (int64_t)k * npad;
+    unsigned long long* __restrict__ sorted = buf.pairs[0] + (int64_t)k * buf.kstride;
+    mid_argsort_slice<WIDE>(
+        order_sort_lds, n, s0, s0 + run, [&](int e) { return ordered_key(col[e]); },
+        [&](int p, int e) { sorted[p] = ((unsigned long long)ordered_key(col[e]) << 32) | (unsigned)e; });
+  }
+}
+
+__global__ __launch_bounds__(256) void objective_positions_kernel(int n, int m, const int* __restrict__ slot_of,
+                                                                  SortParam* __restrict__ param, const Ctrl* __restrict__ ctrl,
+                                                                  int* __restrict__ pos, int* __restrict__ upper, RadixBuffers buf) {
+  if (param->nonfinite != 0 || ctrl->err != 0) return;
+  for (int64_t at = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; at < (int64_t)n * m; at += (int64_t)gridDim.x * blockDim.x) {
+    const int k = (int)(at / n), p = (int)(at - (int64_t)k * n);
+    const unsigned long long* __restrict__ sorted = buf.pairs[0] + (int64_t)k * buf.kstride;
+    const unsigned long long pr = sorted[p];
+    const uint32_t key = (uint32_t)(pr >> 32);
+    const int slot = slot_of[(int)(unsigned)(pr & 0xFFFFFFFFull)];
+    int e = p + 1;
+    if (e < n && (uint32_t)(sorted[e] >> 32) == key) {
+      // a run of equal values: its end by bisection (the first position whose key is larger, or n)
+      int lo = p + 2, hi = n;
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if ((uint32_t)(sorted[mid] >> 32) > key)
+          hi = mid;
+        else
+          lo = mid + 1;
+      }
+      e = lo;
+    }
+    pos[(int64_t)k * buf.kstride + slot] = p;
+    upper[(int64_t)k * buf.kstride + slot] = e;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) param->orders_valid = 1;
+}
+
 // The value that the neighbouring lane (lane ^ 1) passes in, by two DPP quad permutations.
 __device__ inline uint64_t pair_exchange(uint64_t v) {
   const int lo = __builtin_amdgcn_mov_dpp((int)(uint32_t)v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]

@@ -137,11 +137,11 @@ def test_dominance_bits_all_m(m):
 
 
 @pytest.mark.parametrize("n,m", [(65535, 3), (65536, 3), (65537, 4), (65664, 8), (81919, 2), (81920, 2), (70001, 10), (49151, 9), (49152, 16), (66000, 17),
-                                 (45055, 5), (45056, 4), (40960, 6), (36863, 7), (32767, 8), (32768, 8), (24575, 9), (24576, 10),
-                                 (20480, 12), (18432, 14), (16383, 16), (16384, 16)])
+                                 (45055, 5), (45056, 4), (40960, 6), (36863, 7), (28671, 8), (28672, 8), (32768, 8), (18431, 9), (18432, 10),
+                                 (14336, 12), (12288, 14), (10239, 16), (10240, 16), (24577, 16)])
 def test_ranks_across_the_switch_to_the_order_based_matrix(n, m):
     """Populations just below and above the size at which the matrix comes from the per-objective orders -- 65 536 rows
-    of three objectives, fewer with more objectives, down to 16 384 of sixteen -- and 65536 rows, where the padded
+    of three objectives, fewer with more objectives, down to 10 240 of sixteen -- and 65536 rows, where the padded
     column length steps off a multiple of 4096: same ranks and same selection whichever kernel builds the matrix, and
     both the ranks and the selection of the plain-C checker."""
     from oracle import c_oracle
