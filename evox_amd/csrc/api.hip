@@ -20,6 +20,7 @@
 #include "peel_lds.hpp"
 #include "prefix.hpp"
 #include "radix.hpp"
+#include "wide.hpp"
 
 namespace evx {
 
@@ -1506,6 +1507,160 @@ int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_ro
   const Fitness fit{f_a, f_a_stride_row, f_a_stride_col, n_a, f_b, f_b_stride_row, f_b_stride_col};
   return select_rows(x_a, x_row_bytes, x_a_row_stride_bytes, x_b, x_b_row_stride_bytes, fit, n_a + n_b, m, topk, out_x, out_f,
                      out_rank, out_dist, out_order, ws, ws_bytes, (hipStream_t)stream, true);
+}
+
+}  // extern "C"
+
+// ---- fitness of 8-byte elements (wide.hpp)
+struct WideLayout {
+  int n, m;
+  size_t ctrl, key_lo, key_hi, key_mask, selected, boundary, ord_a, ord_b, terms, dist, neg_lo, neg_hi, order_a, order_b, sort_ws,
+      sort_bytes, total;
+};
+
+static bool make_wide_layout(int64_t n, int64_t m, WideLayout* L) {
+  if (n < 1 || m < 1 || n > 0x7FFFFF00ll || m > 65535 || n * m > 0x7FFFFFFFll * 16) return false;
+  L->n = (int)n;
+  L->m = (int)m;
+  const size_t nm = (size_t)n * (size_t)m;
+  size_t o = 0;
+  L->ctrl = o;      o = align_up(o + sizeof(WideCtrl));
+  L->key_lo = o;    o = align_up(o + 4 * nm);
+  L->key_hi = o;    o = align_up(o + 4 * nm);
+  L->key_mask = o;  o = align_up(o + 4 * (size_t)n);
+  L->selected = o;  o = align_up(o + (size_t)n);
+  L->boundary = o;  o = align_up(o + 4 * (size_t)n);
+  L->ord_a = o;     o = align_up(o + 4 * nm);
+  L->ord_b = o;     o = align_up(o + 4 * nm);
+  L->terms = o;     o = align_up(o + 8 * nm);
+  L->dist = o;      o = align_up(o + 8 * (size_t)n);
+  L->neg_lo = o;    o = align_up(o + 4 * (size_t)n);
+  L->neg_hi = o;    o = align_up(o + 4 * (size_t)n);
+  L->order_a = o;   o = align_up(o + 4 * (size_t)n);
+  L->order_b = o;   o = align_up(o + 4 * (size_t)n);
+  L->sort_bytes = evox_hip_argsort_workspace_bytes(n);
+  if (L->sort_bytes == 0) return false;
+  L->sort_ws = o;   o = align_up(o + L->sort_bytes);
+  L->total = o;
+  return true;
+}
+
+static int wide_grid(int64_t items) {
+  int64_t blocks = (items + 255) / 256;
+  const int64_t cap = (int64_t)device_cus() * 8;
+  if (blocks > cap) blocks = cap;
+  return (int)(blocks < 1 ? 1 : blocks);
+}
+
+// The crowding distances of the rows selected by the mask, by the rank vector (rank == its largest set value) or all
+// rows, into `dist` (double for out_kind 0, float for 1), and with neg_keys the sort keys of their negatives.
+static int wide_distances(const WideLayout& L, uint8_t* base, const void* costs, int kind, int64_t sr, int64_t sc,
+                          const uint8_t* mask, int64_t mask_stride, const int32_t* rank, void* dist, int out_kind, bool neg_keys,
+                          hipStream_t s) {
+  const int n = L.n, m = L.m;
+  WideCtrl* ctrl = reinterpret_cast<WideCtrl*>(base + L.ctrl);
+  uint32_t* key_lo = reinterpret_cast<uint32_t*>(base + L.key_lo);
+  uint32_t* key_hi = reinterpret_cast<uint32_t*>(base + L.key_hi);
+  int* key_mask = reinterpret_cast<int*>(base + L.key_mask);
+  uint8_t* selected = base + L.selected;
+  int* boundary = reinterpret_cast<int*>(base + L.boundary);
+  int* ord_a = reinterpret_cast<int*>(base + L.ord_a);
+  int* ord_b = reinterpret_cast<int*>(base + L.ord_b);
+  hipLaunchKernelGGL(wide_head_kernel, dim3(1), dim3(1024), 0, s, mask, mask_stride, rank, n, ctrl);
+  EVX_LAUNCH_CHECK();
+  hipLaunchKernelGGL(wide_keys_kernel, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, mask, mask_stride,
+                     rank, ctrl, key_lo, key_hi, key_mask, selected, boundary);
+  EVX_LAUNCH_CHECK();
+  // per objective: by cost (low half, then high half of its ordered image), then selected rows first; ties by row
+  void* sort_ws = base + L.sort_ws;
+  if (int e = evox_hip_stable_argsort_step_batched(key_lo, kKeyUint32, n, 1, m, n, nullptr, ord_a, sort_ws, L.sort_bytes, s)) return e;
+  if (int e = evox_hip_stable_argsort_step_batched(key_hi, kKeyUint32, n, 1, m, n, ord_a, ord_b, sort_ws, L.sort_bytes, s)) return e;
+  const int* order = ord_b;
+  if (mask != nullptr || rank != nullptr) {
+    if (int e = evox_hip_stable_argsort_step_batched(key_mask, kKeyInt32, 0, 1, m, n, ord_b, ord_a, sort_ws, L.sort_bytes, s)) return e;
+    order = ord_a;
+  }
+  uint32_t* neg_lo = neg_keys ? reinterpret_cast<uint32_t*>(base + L.neg_lo) : nullptr;
+  uint32_t* neg_hi = neg_keys ? reinterpret_cast<uint32_t*>(base + L.neg_hi) : nullptr;
+  if (out_kind == 0) {
+    double* terms = reinterpret_cast<double*>(base + L.terms);
+    hipLaunchKernelGGL(wide_terms_kernel<double>, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, order, ctrl,
+                       terms, boundary);
+    EVX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(wide_sum_kernel<double>, dim3(wide_grid(n)), dim3(256), 0, s, terms, selected, boundary, ctrl, n, m,
+                       static_cast<double*>(dist), neg_lo, neg_hi);
+  } else {
+    float* terms = reinterpret_cast<float*>(base + L.terms);
+    hipLaunchKernelGGL(wide_terms_kernel<float>, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, order, ctrl,
+                       terms, boundary);
+    EVX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(wide_sum_kernel<float>, dim3(wide_grid(n)), dim3(256), 0, s, terms, selected, boundary, ctrl, n, m,
+                       static_cast<float*>(dist), neg_lo, neg_hi);
+  }
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+static int gather_rows(const void* src, int64_t row_bytes, int64_t row_stride_bytes, const int* order, int64_t count, void* dst,
+                       hipStream_t s) {
+  if (row_bytes <= 0 || count <= 0) return 0;
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | (uintptr_t)row_bytes | (uintptr_t)row_stride_bytes;
+  const int unit = bits % 16 == 0 ? 16 : bits % 8 == 0 ? 8 : bits % 4 == 0 ? 4 : 1;
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(wide_grid(count * (row_bytes / unit))), dim3(256), 0, s, static_cast<const uint8_t*>(src),
+                     row_bytes, row_stride_bytes, order, count, static_cast<uint8_t*>(dst), unit);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" {
+
+size_t evox_hip_wide_workspace_bytes(int64_t n, int64_t m) {
+  WideLayout L;
+  return make_wide_layout(n, m, &L) ? L.total : 0;
+}
+
+int evox_hip_crowding_distance_wide(const void* costs, int kind, int64_t n, int64_t m, int64_t sr, int64_t sc, const uint8_t* mask,
+                                    int64_t mask_stride, void* dist_out, int out_kind, void* ws, size_t ws_bytes, void* stream) {
+  WideLayout L;
+  if (costs == nullptr || dist_out == nullptr || (kind != kWideFloat64 && kind != kWideInt64) || (out_kind != 0 && out_kind != 1))
+    return kErrBadArg;
+  if (!make_wide_layout(n, m, &L)) return kErrBadArg;
+  if (ws == nullptr || ws_bytes < L.total || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return kErrWorkspace;
+  return wide_distances(L, static_cast<uint8_t*>(ws), costs, kind, sr, sc, mask, mask_stride, nullptr, dist_out, out_kind, false,
+                        (hipStream_t)stream);
+}
+
+int evox_hip_nd_environmental_selection_wide(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes, const void* f_rows,
+                                             int64_t f_row_bytes, int64_t f_row_stride_bytes, const void* costs, int kind, int64_t n,
+                                             int64_t m, int64_t sr, int64_t sc, const int32_t* rank, int64_t topk, void* out_x,
+                                             void* out_f, int32_t* out_rank, void* out_dist, int out_kind, void* ws, size_t ws_bytes,
+                                             void* stream) {
+  WideLayout L;
+  if (costs == nullptr || rank == nullptr || f_rows == nullptr || out_f == nullptr || out_rank == nullptr || out_dist == nullptr)
+    return kErrBadArg;
+  if ((kind != kWideFloat64 && kind != kWideInt64) || (out_kind != 0 && out_kind != 1)) return kErrBadArg;
+  if ((x == nullptr) != (out_x == nullptr) || x_row_bytes < 0 || x_row_stride_bytes < 0 || f_row_bytes < 1 || f_row_stride_bytes < 0)
+    return kErrBadArg;
+  if (!make_wide_layout(n, m, &L) || topk < 1 || topk > n) return kErrBadArg;
+  if (ws == nullptr || ws_bytes < L.total || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return kErrWorkspace;
+  hipStream_t s = (hipStream_t)stream;
+  uint8_t* base = static_cast<uint8_t*>(ws);
+  void* dist = base + L.dist;
+  if (int e = wide_distances(L, base, costs, kind, sr, sc, nullptr, 0, rank, dist, out_kind, true, s)) return e;
+  // rows by rank, then by distance descending (NaN last), then by index: one stable step per key part, least
+  // significant first (src/evox/operators/selection/non_dominate.py:253, src/evox/utils/jit_fix_operator.py:246-250)
+  int* order_a = reinterpret_cast<int*>(base + L.order_a);
+  int* order_b = reinterpret_cast<int*>(base + L.order_b);
+  void* sort_ws = base + L.sort_ws;
+  if (int e = evox_hip_stable_argsort_step(base + L.neg_lo, kKeyUint32, 1, n, nullptr, order_a, sort_ws, L.sort_bytes, s)) return e;
+  if (int e = evox_hip_stable_argsort_step(base + L.neg_hi, kKeyUint32, 1, n, order_a, order_b, sort_ws, L.sort_bytes, s)) return e;
+  if (int e = evox_hip_stable_argsort_step(rank, kKeyInt32, 1, n, order_b, order_a, sort_ws, L.sort_bytes, s)) return e;
+  if (x != nullptr)
+    if (int e = gather_rows(x, x_row_bytes, x_row_stride_bytes, order_a, topk, out_x, s)) return e;
+  if (int e = gather_rows(f_rows, f_row_bytes, f_row_stride_bytes, order_a, topk, out_f, s)) return e;
+  if (int e = gather_rows(rank, 4, 4, order_a, topk, out_rank, s)) return e;
+  const int64_t dist_bytes = out_kind == 0 ? 8 : 4;
+  return gather_rows(dist, dist_bytes, dist_bytes, order_a, topk, out_dist, s);
 }
 
 }  // extern "C"

@@ -252,7 +252,11 @@ __global__ __launch_bounds__(kRadixThreads) void argsort_step_kernel(const void*
   const int workers = gridDim.x - kFirstSweeper;
   const int wb = (int)blockIdx.x - kFirstSweeper;
   auto initial = [&](int, int e) {
-    const int idx = prev ? prev[e] : e;
+    int idx = prev ? prev[e] : e;
+    if (idx < 0) {  // the order of a step whose wait ran out (-1 everywhere): this step fails too, and reads nothing through it
+      coherent_store(&ctrl->err, kErrBarrierTimeout);
+      idx = 0;
+    }
     uint32_t k;
     if (kind == kKeyFloat32)
       k = ordered_key(static_cast<const float*>(key)[(int64_t)idx * stride]);

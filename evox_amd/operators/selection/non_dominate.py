@@ -1,8 +1,9 @@
 """Drop-in replacements for the three selection operators of
 ``evox.operators.selection.non_dominate`` (src/evox/operators/selection/non_dominate.py),
 with the same names, positional arguments, return arity, dtypes and devices.  The work is done by
-hand-written gfx950 kernels reached through the ``evox_amd::`` custom operators; there is no
-PyTorch or CPU implementation behind them.
+hand-written gfx950 kernels reached through the ``evox_amd::`` custom operators, for float32 fitness
+(the kernels of the selection path) as for float64 and integer fitness (kernels that read 8-byte
+values); there is no PyTorch or CPU implementation behind them.
 """
 
 from typing import Optional, Tuple
@@ -10,68 +11,6 @@ from typing import Optional, Tuple
 import torch
 
 from ... import ops
-
-
-def _crowding_distance_f64(costs: torch.Tensor, mask: Optional[torch.Tensor]) -> torch.Tensor:
-    """float64 costs (the default dtype set to float64) or integer costs: the reference's statements
-    (non_dominate.py:209-231), one by one, around this package's ``lexsort`` (the stable argsort kernels; the
-    kernels of the float32 path read 4-byte floats).  Integer costs are subtracted exactly and divided in the
-    default float dtype, as there.  One population."""
-    from ...utils import lexsort
-
-    total_len, m = costs.shape
-    if mask is None:
-        num_valid = total_len
-        mask = torch.ones(total_len, dtype=torch.bool, device=costs.device)
-    else:
-        num_valid = int(mask.sum())
-    out_dtype = costs.dtype if costs.is_floating_point() else torch.get_default_dtype()
-    if total_len == 0:
-        return torch.empty(0, dtype=out_dtype, device=costs.device)
-    inverted = (~mask).unsqueeze(1).expand(-1, m).to(costs.dtype)
-    rank = lexsort([costs, inverted], dim=0)
-    sorted_costs = torch.gather(costs, dim=0, index=rank)
-    # (torch.empty in the reference: whatever it holds is either overwritten below or belongs to a row outside
-    # the mask)
-    distance = torch.full(costs.size(), -torch.inf, dtype=out_dtype, device=costs.device)
-    if num_valid > 0:
-        distance_range = sorted_costs[num_valid - 1] - sorted_costs[0]
-        if total_len > 2:
-            distance = distance.scatter(0, rank[1:-1], (sorted_costs[2:] - sorted_costs[:-2]) / distance_range)
-        distance[rank[0], :] = torch.inf  # (whole rows: first or last in any objective means +inf in all of them)
-        distance[rank[num_valid - 1], :] = torch.inf
-    return torch.where(mask.unsqueeze(1), distance, -torch.inf).sum(dim=1)
-
-
-def _nd_environmental_selection_f64(x: torch.Tensor, f: torch.Tensor, topk: int) -> Tuple[torch.Tensor, ...]:
-    """float64 fitness: the reference's statements (non_dominate.py:249-254) around the ranking kernels (which see
-    the per-objective dense ranks of the values, exact in float32) and this package's ``lexsort``.  The ranking
-    stops at the front that holds the topk-th row: the rows behind it carry the largest int32 and sort last."""
-    from ...utils import lexsort
-
-    n = f.shape[0]
-    if topk > n:
-        raise RuntimeError(f"selected index k out of range: topk={topk} > {n} rows")
-    if topk < 1:
-        raise IndexError(f"index -1 is out of bounds: topk={topk}")
-    rank = ops.nd_rank_until(f, topk)
-    worst_rank = torch.topk(rank, topk, largest=False)[0][-1]
-    mask = rank == worst_rank
-    crowding_dis = _crowding_distance_f64(f, mask)
-    combined_order = lexsort([-crowding_dis, rank])[:topk]
-    return x[combined_order], f[combined_order], rank[combined_order], crowding_dis[combined_order]
-
-
-def _per_population(fn, lead: int, *tensors):
-    """``fn`` over the leading ``lead`` dimensions of the tensors, one population at a time, results stacked."""
-    if lead == 0:
-        return fn(*tensors)
-    batch = tensors[0].shape[:lead]
-    flat = [None if t is None else t.reshape(-1, *t.shape[lead:]) for t in tensors]
-    outs = [fn(*[None if t is None else t[b] for t in flat]) for b in range(flat[0].shape[0])]
-    if isinstance(outs[0], tuple):
-        return tuple(torch.stack([o[i] for o in outs]).reshape(*batch, *outs[0][i].shape) for i in range(len(outs[0])))
-    return torch.stack(outs).reshape(*batch, *outs[0].shape)
 
 
 def non_dominate_rank(x: torch.Tensor) -> torch.Tensor:
@@ -120,16 +59,14 @@ def crowding_distance(costs: torch.Tensor, mask: Optional[torch.Tensor]) -> torc
     ``(next - previous) / (last - first)``; unselected rows get ``-inf``.  The result has torch's
     default float dtype, and, as in the reference (its scatter at :224-225), ``costs`` must have that
     dtype too.  With the default dtype set to float64 the distances are computed in float64, and integer costs
-    are subtracted exactly and divided in the default float dtype, both by the reference's own sequence of
-    statements around this package's ``lexsort``.
+    are subtracted exactly and divided in the default float dtype, by kernels that read 8-byte values.
     """
     if costs.is_floating_point() and costs.dtype != torch.get_default_dtype():
         raise RuntimeError(
             f"crowding_distance: expected costs.dtype to be the default dtype {torch.get_default_dtype()}, got {costs.dtype}"
         )
     if costs.dtype == torch.float64 or not costs.is_floating_point():
-        ops.runtime.require_gpu_tensor(costs, "costs")
-        return _per_population(_crowding_distance_f64, costs.dim() - 2, costs, mask)
+        return ops.crowding_wide(costs, mask)
     return ops.crowding(costs, mask)
 
 
@@ -148,8 +85,7 @@ def nd_environmental_selection(x: torch.Tensor, f: torch.Tensor, topk: int) -> T
             f"nd_environmental_selection: expected f.dtype to be the default dtype {torch.get_default_dtype()}, got {f.dtype}"
         )
     if f.dtype == torch.float64 or not (f.is_floating_point() or f.is_complex() or f.dtype == torch.bool):
-        ops.runtime.require_gpu_tensor(f, "f")
-        return _per_population(lambda xb, fb: _nd_environmental_selection_f64(xb, fb, int(topk)), f.dim() - 2, x, f)
+        return ops.nd_select_wide(x, f, int(topk))
     return ops.nd_select(x, f, int(topk))
 
 
@@ -160,6 +96,11 @@ def nd_environmental_selection_two_part(
 
     Not a name of the reference; it replaces the merge step of its NSGA-II
     (src/evox/algorithms/mo/nsga2.py:99-102), where parents and offspring are concatenated only to be
-    handed to the selection.  Same four results as ``nd_environmental_selection``.
+    handed to the selection.  Same four results as ``nd_environmental_selection``.  Fitness that the two-part
+    kernels do not read (float64, integers, parts of different dtypes) is concatenated after all, with
+    ``torch.cat``'s promotion of the dtypes, and goes the way of ``nd_environmental_selection``.
     """
+    narrow = (torch.float32, torch.float16, torch.bfloat16)
+    if f_a.dtype != f_b.dtype or f_a.dtype not in narrow or x_a.dtype != x_b.dtype:
+        return nd_environmental_selection(torch.cat([x_a, x_b], dim=0), torch.cat([f_a, f_b], dim=0), int(topk))
     return ops.nd_select_two_part(x_a, f_a, x_b, f_b, int(topk))

@@ -252,6 +252,141 @@ def _crowding_vmap(info, in_dims, costs, mask):
 torch.library.register_vmap(crowding, _crowding_vmap)
 
 
+def _wide_costs(t: torch.Tensor, what: str):
+    """Costs of a dtype that the float32 kernels do not read, as the 8-byte elements that the wide kernels read:
+    (tensor, kind of the C ABI, dtype of the distances)."""
+    if t.dtype == torch.float64:
+        return t, 0, torch.float64
+    if t.is_floating_point() or t.is_complex() or t.dtype == torch.bool:
+        raise TypeError(f"{what} must be float64 or an integer tensor here; got {t.dtype}")
+    out_dtype = torch.get_default_dtype()  # integer differences are divided in the default float dtype
+    if out_dtype not in (torch.float32, torch.float64):
+        raise TypeError(f"integer {what} needs a default float dtype of float32 or float64; got {out_dtype}")
+    return t.to(torch.int64), 1, out_dtype
+
+
+@torch.library.custom_op("evox_amd::crowding_wide", mutates_args=())
+def crowding_wide(costs: torch.Tensor, mask: Optional[torch.Tensor]) -> torch.Tensor:
+    """(..., N, M) float64 or integer costs, optional (..., N) bool mask -> (..., N) crowding distance: float64 for
+    float64 costs, torch's default float dtype for integer costs."""
+    runtime.require_gpu_tensor(costs, "costs")
+    if costs.dim() < 2:
+        raise ValueError("costs must have shape (..., N, M)")
+    wide, kind, out_dtype = _wide_costs(costs, "costs")
+    n, m = wide.shape[-2:]
+    out = torch.empty(wide.shape[:-1], dtype=out_dtype, device=costs.device)
+    if mask is not None:
+        runtime.require_gpu_tensor(mask, "mask")
+        if mask.dtype != torch.bool:
+            raise TypeError(f"mask must be a bool tensor; got {mask.dtype}")
+        if mask.shape != out.shape:
+            raise ValueError(f"mask shape {tuple(mask.shape)} does not match costs {tuple(costs.shape)}")
+    if n == 0 or out.numel() == 0:
+        return out
+    if m == 0:
+        raise ValueError("costs must have at least one objective")
+    with torch.cuda.device(costs.device):
+        flat_c = wide.reshape(-1, n, m)
+        flat_out = out.view(-1, n)
+        flat_mask = None if mask is None else mask.reshape(-1, n)
+        stream = runtime.stream_handle(costs.device)
+        ws = runtime.wide_workspace(n, m, costs.device)
+        for b in range(flat_c.size(0)):
+            c = flat_c[b]
+            mk = None if flat_mask is None else flat_mask[b]
+            _lib.call("evox_hip_crowding_distance_wide", c.data_ptr(), kind, n, m, c.stride(0), c.stride(1),
+                      None if mk is None else mk.data_ptr(), 0 if mk is None else mk.stride(0), flat_out[b].data_ptr(),
+                      0 if out_dtype == torch.float64 else 1, ws.data_ptr(), ws.numel(), stream)
+        runtime.note_small_kernel_call()
+    return out
+
+
+@crowding_wide.register_fake
+def _(costs, mask):
+    return costs.new_empty(costs.shape[:-1], dtype=torch.float64 if costs.dtype == torch.float64 else torch.get_default_dtype())
+
+
+def _crowding_wide_vmap(info, in_dims, costs, mask):
+    costs, mask = _batched_first(info, in_dims, (costs, mask))
+    return crowding_wide(costs, mask), 0
+
+
+torch.library.register_vmap(crowding_wide, _crowding_wide_vmap)
+
+
+@torch.library.custom_op("evox_amd::nd_select_wide", mutates_args=())
+def nd_select_wide(x: torch.Tensor, f: torch.Tensor, topk: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """nd_select for float64 or integer fitness: x (..., N, *D), f (..., N, M), topk -> (x, f, rank, crowding distance)
+    of the topk survivors, the distance in float64 for float64 fitness and in the default float dtype for integers."""
+    runtime.require_gpu_tensor(f, "fitness")
+    runtime.require_gpu_tensor(x, "decision vectors")
+    if f.dim() < 2:
+        raise ValueError("fitness must have shape (..., N, M)")
+    bd = f.dim() - 2
+    n, m = f.shape[-2:]
+    if x.dim() < bd + 1 or x.shape[: bd + 1] != f.shape[: bd + 1]:
+        raise ValueError(f"decision vectors {tuple(x.shape)} and fitness {tuple(f.shape)} disagree on the leading dimensions")
+    if x.device != f.device:
+        raise RuntimeError("decision vectors and fitness are on different devices")
+    if topk > n:
+        raise RuntimeError(f"selected index k out of range: topk={topk} exceeds the population size {n}")
+    if topk < 1:
+        raise IndexError(f"topk must be at least 1; got {topk}")
+    if m == 0:
+        raise ValueError("fitness must have at least one objective")
+    wide, kind, out_dtype = _wide_costs(f, "fitness")
+    batch = f.shape[:bd]
+    out_x = torch.empty(*batch, topk, *x.shape[bd + 1:], dtype=x.dtype, device=x.device)
+    out_f = torch.empty(*batch, topk, m, dtype=f.dtype, device=f.device)
+    out_rank = torch.empty(*batch, topk, dtype=torch.int32, device=f.device)
+    out_dist = torch.empty(*batch, topk, dtype=out_dtype, device=f.device)
+    if out_rank.numel() == 0:
+        return out_x, out_f, out_rank, out_dist
+    # the ranks, as far as the front that holds the topk-th row, from the ranking kernels on a float32 image of the
+    # fitness that keeps every comparison (the rows behind that front are marked unset)
+    rank = nd_rank_until(f, topk)
+    with torch.cuda.device(f.device):
+        flat_w = wide.reshape(-1, n, m)
+        flat_f = f.reshape(-1, n, m).contiguous()
+        flat_x = x.reshape(flat_w.size(0), n, -1).contiguous()
+        flat_rank = rank.reshape(-1, n)
+        row_bytes = flat_x.size(-1) * flat_x.element_size()
+        f_row_bytes = m * flat_f.element_size()
+        has_x = row_bytes > 0
+        fo_x = out_x.view(flat_w.size(0), topk, -1)
+        fo_f, fo_r, fo_d = out_f.view(-1, topk, m), out_rank.view(-1, topk), out_dist.view(-1, topk)
+        stream = runtime.stream_handle(f.device)
+        ws = runtime.wide_workspace(n, m, f.device)
+        for b in range(flat_w.size(0)):
+            wb = flat_w[b]
+            _lib.call("evox_hip_nd_environmental_selection_wide", flat_x[b].data_ptr() if has_x else None, row_bytes, row_bytes,
+                      flat_f[b].data_ptr(), f_row_bytes, f_row_bytes, wb.data_ptr(), kind, n, m, wb.stride(0), wb.stride(1),
+                      flat_rank[b].data_ptr(), topk, fo_x[b].data_ptr() if has_x else None, fo_f[b].data_ptr(), fo_r[b].data_ptr(),
+                      fo_d[b].data_ptr(), 0 if out_dtype == torch.float64 else 1, ws.data_ptr(), ws.numel(), stream)
+        runtime.note_small_kernel_call()
+    return out_x, out_f, out_rank, out_dist
+
+
+@nd_select_wide.register_fake
+def _(x, f, topk):
+    bd = f.dim() - 2
+    batch = f.shape[:bd]
+    return (
+        x.new_empty(*batch, topk, *x.shape[bd + 1:]),
+        f.new_empty(*batch, topk, f.shape[-1]),
+        f.new_empty(*batch, topk, dtype=torch.int32),
+        f.new_empty(*batch, topk, dtype=torch.float64 if f.dtype == torch.float64 else torch.get_default_dtype()),
+    )
+
+
+def _nd_select_wide_vmap(info, in_dims, x, f, topk):
+    x, f = _batched_first(info, in_dims[:2], (x, f))
+    return nd_select_wide(x, f, topk), (0, 0, 0, 0)
+
+
+torch.library.register_vmap(nd_select_wide, _nd_select_wide_vmap)
+
+
 @torch.library.custom_op("evox_amd::nd_select", mutates_args=())
 def nd_select(x: torch.Tensor, f: torch.Tensor, topk: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """x (..., N, *D), f (..., N, M), topk -> (x, f, rank, crowding distance) of the topk survivors."""
@@ -620,7 +755,9 @@ def tournament_pick(parents: torch.Tensor, fitness: torch.Tensor) -> torch.Tenso
     runtime.require_gpu_tensor(fitness, "fitness")
     if parents.dim() != 2 or fitness.dim() != 2 or parents.dtype != torch.int64:
         raise ValueError("parents must be (n_round, tournament_size) int64 and fitness (candidates, keys)")
-    fit = _as_f32(fitness, "fitness")
+    # (keys of other dtypes -- float64 distances under a float64 default, integers -- as per-column dense ranks, which
+    # keep every comparison)
+    fit = _order_preserving_f32(fitness, "fitness") if fitness.numel() > 0 else fitness.float()
     par = parents.contiguous()
     out = torch.empty(par.size(0), dtype=torch.int64, device=parents.device)
     with torch.cuda.device(parents.device):

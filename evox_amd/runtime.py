@@ -110,6 +110,21 @@ def sort_workspace(n: int, device: torch.device) -> torch.Tensor:
     return ws
 
 
+def wide_workspace(n: int, m: int, device: torch.device) -> torch.Tensor:
+    """Workspace of the entry points for 8-byte fitness; shares the per-(device, stream) buffer of `workspace`."""
+    need = int(_lib.lib().evox_hip_wide_workspace_bytes(n, m))
+    if need == 0:
+        raise ValueError(f"unsupported population shape n={n}, m={m}")
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_handle(device))
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        _workspaces.pop(key, None)
+        ws = None
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
 def release_workspaces() -> None:
     _workspaces.clear()
 

@@ -75,6 +75,30 @@ int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t
                                const uint8_t* mask, int64_t mask_stride, float* dist_out, void* workspace,
                                size_t workspace_bytes, void* stream);
 
+/* The same distance for costs of 8-byte elements, which the reference also accepts (it computes the differences in
+ * the costs' dtype and the quotients in torch's default float dtype, non_dominate.py:222-225): kind 0 = float64
+ * costs, 1 = int64 costs (exact wrapping differences, divided as floats); out_kind 0 = float64 distances, 1 =
+ * float32 (integer costs under a float32 default).  Strides in elements.  The per-objective orders
+ * (jit_fix_operator.py:246-250) come from the stable argsort steps below on the halves of an order-preserving 64-bit
+ * image of the cost.  Workspace: evox_hip_wide_workspace_bytes(n, m). */
+size_t evox_hip_wide_workspace_bytes(int64_t n, int64_t m);
+int evox_hip_crowding_distance_wide(const void* costs, int kind, int64_t n, int64_t m, int64_t stride_row, int64_t stride_col,
+                                    const uint8_t* mask, int64_t mask_stride, void* dist_out, int out_kind, void* workspace,
+                                    size_t workspace_bytes, void* stream);
+
+/* The selection steps after the ranking for such fitness (non_dominate.py:249-254): given rank (int32, n entries,
+ * EVOX_HIP_RANK_UNSET behind the front that holds the topk-th row, as evox_hip_non_dominate_rank_until leaves them on
+ * any order-preserving float32 image of the fitness), the distances of the rows of the largest set rank (the mask
+ * rank == worst of :250-252), the order by (rank, distance descending with NaN last, row index) and the gathers:
+ * out_x rows of x_row_bytes, out_f rows of f_row_bytes taken from f_rows (the caller's fitness rows as raw bytes, of
+ * whatever dtype they have), out_rank int32, out_dist float64 (out_kind 0) or float32 (1).  costs / kind / strides as
+ * above.  Workspace: evox_hip_wide_workspace_bytes(n, m). */
+int evox_hip_nd_environmental_selection_wide(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes, const void* f_rows,
+                                             int64_t f_row_bytes, int64_t f_row_stride_bytes, const void* costs, int kind,
+                                             int64_t n, int64_t m, int64_t stride_row, int64_t stride_col, const int32_t* rank,
+                                             int64_t topk, void* out_x, void* out_f, int32_t* out_rank, void* out_dist,
+                                             int out_kind, void* workspace, size_t workspace_bytes, void* stream);
+
 /* NSGA-II survivor selection: ranks f, takes the topk best rows by (rank ascending, crowding
  * distance within the last admitted front descending, row index ascending) and gathers them.
  *   x            decision vectors as raw bytes, row i at x + i * x_row_stride_bytes, x_row_bytes each

@@ -124,3 +124,24 @@ def test_integer_fitness_crowding_and_selection(dtype):
         if not torch.equal(got[0].cpu(), want[0]):
             assert sorted(as_np(got[0])[:, 0].tolist()) == sorted(as_np(want[0])[:, 0].tolist()) or np.allclose(
                 np.sort(gw[np.isfinite(gw)]), np.sort(ww[np.isfinite(ww)]), rtol=1e-5)
+
+
+def test_float64_long_sorts_and_vmap(float64_default):
+    """Orders of more than 32 768 positions come from the radix sort, shorter ones from the kernels that sort in
+    LDS; mapped populations go through the same operators."""
+    g = torch.Generator("cpu").manual_seed(67)
+    f = torch.rand(40000, 2, generator=g, dtype=torch.float64)
+    f[::7, 0] = f[3::7, 0][: f[::7].size(0)]  # ties
+    mask = torch.rand(40000, generator=g) < 0.4
+    _close(crowding_distance(f.to(DEV), mask.to(DEV)), er.crowding(f, mask), "40000 rows")
+    _close(crowding_distance(f.to(DEV), None), er.crowding(f, None), "40000 rows, no mask")
+    fb = torch.rand(4, 300, 3, generator=g, dtype=torch.float64)
+    mb = torch.rand(4, 300, generator=g) < 0.5
+    mapped = torch.vmap(crowding_distance)(fb.to(DEV), mb.to(DEV))
+    xb = torch.arange(300, dtype=torch.int64)[None, :, None].repeat(4, 1, 1)
+    sel = torch.vmap(lambda x, f: nd_environmental_selection(x, f, 120))(xb.to(DEV), fb.to(DEV))
+    for b in range(4):
+        _close(mapped[b], er.crowding(fb[b], mb[b]), ("vmap", b))
+        want = er.environmental_selection(xb[b], fb[b], 120)
+        assert torch.equal(sel[0][b].cpu(), want[0]) and torch.equal(sel[2][b].cpu(), want[2])
+        _close(sel[3][b], want[3], ("vmap selection", b))

@@ -79,7 +79,7 @@ def _stand_in_package():
             return evox_amd.ops.tournament_pick(self.draws[self.t % 16], keys)
 
         def evaluate(self, x):
-            return _dtlz(x, self.n_objs)
+            return _dtlz(x, self.n_objs).to(x.dtype)
 
         def step(self):  # nsga2.py:92-102
             mating_pool = self.selection(self.pop_size, [-self.dis, self.rank])
@@ -188,6 +188,31 @@ def test_patched_nsga2_step_leaves_the_same_state(package):
         patched.t += 1
         for got, w in zip((patched.pop, patched.fit, patched.rank, patched.dis), want):
             assert torch.equal(got, w) and got.dtype == w.dtype
+
+
+def test_patched_nsga2_step_with_float64_fitness(package):
+    """A run under a float64 default dtype (float64 population and fitness): the two-part selection hands fitness
+    that its kernels do not read to the selection of the concatenation, as the unpatched step does."""
+    NSGA2 = package["evox.algorithms.mo.nsga2"].NSGA2
+    torch.set_default_dtype(torch.float64)
+    try:
+        evox_amd.install_into_evox()
+        plain = NSGA2(200, 8, 3, seed=9)
+        assert plain.fit.dtype == torch.float64 and plain.dis.dtype == torch.float64
+        states = []
+        for _ in range(3):
+            plain.step()
+            plain.t += 1
+            states.append([t.clone() for t in (plain.pop, plain.fit, plain.rank, plain.dis)])
+        evox_amd.install_into_evox(patch_callers=True)
+        patched = NSGA2(200, 8, 3, seed=9)
+        for want in states:
+            patched.step()
+            patched.t += 1
+            for got, w in zip((patched.pop, patched.fit, patched.rank, patched.dis), want):
+                assert torch.equal(got, w) and got.dtype == w.dtype
+    finally:
+        torch.set_default_dtype(torch.float32)
 
 
 @pytest.mark.parametrize("n,m,pop_size,seed", [(600, 3, 300, 1), (2000, 2, 1000, 2), (5000, 3, 2500, 3), (400, 8, 100, 4)])
