@@ -64,7 +64,9 @@ def parse():
     ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--cpu-sample", type=int, default=0, help="rows of the workload timed on the CPU (0 = all of them)")
-    ap.add_argument("--cpu-runs", type=int, default=1, help="runs of the CPU leg (the median is reported)")
+    ap.add_argument("--cpu-runs", type=int, default=3, help="runs of the CPU leg (the median is reported)")
+    ap.add_argument("--no-off-config", action="store_true",
+                    help="skip the off-config object of the default line (one HBM-bound sweep pass at 200000 x 3)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 512 MiB device copy three times, so that a rocprofv3 --pmc run of this "
                          "command holds a kernel of known traffic next to the selection kernels")
@@ -477,6 +479,13 @@ def main():
     def step():
         return nd_environmental_selection(x, f, w.topk)
 
+    # the first call of the process: kernels not yet loaded, no workspace yet, no record of an earlier selection of
+    # this shape (the library keeps, per device, what the last selections found and picks the launches of the next by it)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    step()
+    torch.cuda.synchronize()
+    first_call_ms = (time.perf_counter() - t0) * 1e3
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -486,6 +495,17 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
+    # the same steps when the library may not look at what earlier selections found (a call whose predecessor was of
+    # another kind pays this launch set)
+    from evox_amd import runtime as _rt
+    with _rt.options(launch_memory=0):
+        step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        ms_without_launch_memory = (time.perf_counter() - t0) / args.steps * 1e3
 
     times, status, rank, slot_of, nwords = stage_profile(w, x, f, max(5, min(args.steps, 30)))
     from_lds = times["peel_from_lds"]
@@ -572,12 +592,16 @@ def main():
         phases["dominance"]["measured_issue_rates_Gops"] = rates
         phases["dominance"]["frac_of_measured_rate"] = (
             phases["dominance"]["achieved"] / (rates["v_add_f32"] if finite else rates["v_cmp_to_sgpr"]))
+    # the kernel that builds the matrix: from the per-objective orders, or pair by pair -- up to eight objectives on
+    # a grid that holds only the blocks at or below the diagonal (tunable dominance_folded, tiles of two or four words)
+    folded = _rt.current_option("dominance_folded", 1) and m <= 8 and int(plan[0]) in (2, 4)
+    dominance_kernel_name = "dominance_prefix_kernel" if from_orders else ("dominance_folded_kernel" if folded else "dominance_kernel")
     dominant = max((k for k in ("dominance", "count", "peel") if k in phases), key=lambda k: phases[k]["us"])
     d = phases[dominant]
     roofline = {
         # populations whose matrix fits the LDS of the device are peeled from there; others up to 262144 rows by the
         # record-protocol kernel, larger ones by peel_kernel
-        "kernel": {"dominance": "dominance_prefix_kernel" if from_orders else "dominance_kernel", "count": "count_kernel",
+        "kernel": {"dominance": dominance_kernel_name, "count": "count_kernel",
                    "peel": "peel_lds_kernel" if from_lds else ("peel_records_kernel" if n <= 262144 else "peel_kernel")}[dominant],
         "bound": "hbm" if d["bound"] == "hbm" else "valu",
         "achieved": d["achieved"], "peak": d["peak"], "unit": d["unit"], "frac": d["frac"], "traffic": None,
@@ -587,8 +611,7 @@ def main():
     if measured is not None:
         roofline["traffic"] = measured["bytes"]
         roofline["traffic_source"] = measured["source"]
-    from evox_amd import runtime as _runtime
-    if _runtime.small_population_kernel_fits(n, m, 1):
+    if _rt.small_population_kernel_fits(n, m, 1):
         # a population this small is selected by one launch of the one-workgroup kernel (that is what ms_per_step
         # times); the phases and this object describe the pipeline's kernels on the same rows, timed through the
         # stage entry points
@@ -612,6 +635,8 @@ def main():
                                f"topk={w.topk}, fitness U[0,1) seed {w.seed}" if w.name in ("C1", "C3") else
                                f"{w.name}: nd_environmental_selection N={n} M={m} topk={w.topk} seed {w.seed}"},
         "latency_ms": ms_per_step,
+        "first_call_ms": first_call_ms,
+        "ms_per_step_without_launch_memory": ms_without_launch_memory,
         "step_us_by_events": times["step_us"],
         "dominance_kernel_comparisons_per_s": pairs / (times["dominance_alone_us"] * 1e-6),
         "dominance_kernel_scalar_compares_per_s": compares / (times["dominance_alone_us"] * 1e-6),
@@ -621,6 +646,15 @@ def main():
     }
     if args.next_rows:
         out["next_rows"] = next_rows(dev, max(5, min(args.steps, 20)))
+    elif args.workload == "C3" and not args.no_off_config:
+        # Not the configuration of the line and not the default formulation: the popcount-decrement sweep pass where a
+        # pass is large enough to be bound by memory bandwidth (at C3 a pass would read 25 MB, 3 us at the peak, and is
+        # bound by the exchange between workgroups instead, which is why the witness pass is the default there)
+        runtime_ws_release = _rt.release_workspaces
+        runtime_ws_release()
+        out["off_config"] = {"sweep pass N=200000 M=3": sweep_pass_bandwidth(dev, 200000, 3),
+                             "note": "off-config and non-default: one pass of the sweep formulation (tunable peel_witness=0) "
+                                     "over a population whose passes are HBM-bound"}
     if not args.no_cpu:
         base = cpu_baseline(w, args.cpu_sample, args.cpu_runs)
         out["cpu_baseline"] = base

@@ -20,6 +20,7 @@
 #include "peel_lds.hpp"
 #include "prefix.hpp"
 #include "radix.hpp"
+#include "slotsort.hpp"
 #include "wide.hpp"
 
 namespace evx {
@@ -44,6 +45,8 @@ struct Options {
   int dominance_folded = 1;      // tiles of two words: only the blocks at or below the diagonal are launched
   int mid_argsort = 1;  // an argsort step of 8193 .. kMidArgsortRows positions in one kernel without waits (0: the radix sort)
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
+  int one_sort = 1;    // populations of kOneSortMinRows .. kOneSortMaxRows rows likewise (slotsort.hpp; 0: bucket sort)
+  int one_sort_cap = kOneSortCap;  // members of a range that kernel places from LDS (smaller values: for tests of the other way)
   int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 objectives (a quarter more
                                     // with 2, fewer with more: 28672 at 8, 10240 at 16 -- prefix_least_rows) get
                                     // their matrix from the per-objective orders (prefix.hpp); 0 = never
@@ -152,16 +155,18 @@ static int open_ws(int64_t n, int64_t m, void* ws, size_t bytes, Ws* out, bool w
   return 0;
 }
 
+// (The small host-side caches below are read and written by whichever threads call into the library: each slot is
+// an atomic that holds a value derived from the device alone, so two threads that fill it at once store the same.)
 static int device_cus() {
-  static int cached[64] = {0};
+  static std::atomic<int> cached[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int v = 0;
+  int v = cached[dev].load(std::memory_order_relaxed);
+  if (v == 0) {
     if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
-    cached[dev] = v;
+    cached[dev].store(v, std::memory_order_relaxed);
   }
-  return cached[dev];
+  return v;
 }
 
 // What the last selections on this device found, for the choice of launches of the next one: sixteen words of pinned
@@ -305,6 +310,20 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
     EVX_LAUNCH_CHECK();
     return 0;
   }
+  if (with_sort && L.n >= kOneSortMinRows && L.n <= kOneSortMaxRows && (int64_t)L.n * L.m <= kOneSortMaxValues && opt().one_sort) {
+    // as many workgroups as compute units, a power of two (each takes one range of the sample's cuts)
+    int grid = kOneSortSamples;
+    while (grid > 8 && grid > device_cus()) grid >>= 1;
+    auto launch = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, dim3(grid), dim3(kOneSortThreads), 0, s, src.f, src.sr, src.sc, (int)src.n_first, src.f2, src.sr2,
+                         src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs), w.at<double>(L.key), w.at<SortParam>(L.sortparam),
+                         w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of),
+                         w.at<int>(L.slot_of), w.at<uint32_t>(L.ctrl), zero_words, opt().one_sort_cap);
+    };
+    launch(one_sort_kernel);
+    EVX_LAUNCH_CHECK();
+    return 0;
+  }
   hipLaunchKernelGGL(prepare_kernel, dim3(L.prep_blocks), dim3(256), 0, s, src.f, src.sr, src.sc, (int)src.n_first, src.f2,
                      src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs), w.at<uint64_t>(L.key),
                      w.at<unsigned long long>(L.partials), w.at<uint32_t>(L.ctrl), zero_words);
@@ -406,35 +425,56 @@ static int stage_count(const Ws& w, bool fill_dist, hipStream_t s, bool need_cou
   return 0;
 }
 
+static int grant_dynamic_lds(const void* kernel, size_t lds);
+
 // Resident blocks per CU of the peel kernel for a dynamic-LDS size (cached: the query is not free).
 // Returns a negative library code or positive hipError_t through *err and 0 on failure.
 static int peel_blocks_per_cu(size_t lds, int* err) {
   struct Entry { size_t lds; int dev; int per_cu; };
   static Entry cache[16];
   static int used = 0;
+  static std::mutex mu;
   int dev = 0;
   (void)hipGetDevice(&dev);
-  for (int i = 0; i < used; ++i)
-    if (cache[i].lds == lds && cache[i].dev == dev) return cache[i].per_cu;
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(peel_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) { *err = (int)e; return 0; }
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    for (int i = 0; i < used; ++i)
+      if (cache[i].lds == lds && cache[i].dev == dev) return cache[i].per_cu;
   }
+  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(peel_kernel), lds)) { *err = e; return 0; }
   int per_cu = 0;
   hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, peel_kernel, kPeelThreads, lds);
   if (e != hipSuccess) { *err = (int)e; return 0; }
   if (per_cu < 1) { *err = kErrBadArg; return 0; }
-  if (used < 16) cache[used++] = Entry{lds, dev, per_cu};
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (used < 16) cache[used++] = Entry{lds, dev, per_cu};
+  }
   return per_cu;
 }
 
+// Grants only ever grow per (kernel, device), and are made one at a time: a thread that was given a large size never
+// finds it taken back by another thread's smaller one between its grant and its launch.
 static int grant_dynamic_lds(const void* kernel, size_t lds) {
   if (lds > 160 * 1024) return kErrBadArg;  // (what a workgroup of this device can have)
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-  }
+  if (lds <= 48 * 1024) return 0;
+  struct Entry { const void* kernel; int dev; size_t lds; };
+  static Entry table[128];
+  static int used = 0;
+  static std::mutex mu;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = -1;
+  std::lock_guard<std::mutex> lock(mu);
+  int at = -1;
+  for (int i = 0; i < used; ++i)
+    if (table[i].kernel == kernel && table[i].dev == dev) at = i;
+  if (at >= 0 && table[at].lds >= lds) return 0;
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return (int)e;
+  if (at >= 0)
+    table[at].lds = lds;
+  else if (used < 128)
+    table[used++] = Entry{kernel, dev, lds};
   return 0;
 }
 
@@ -483,19 +523,21 @@ static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool
   }
   // the attribute belongs to the (kernel, device) pair; every workgroup waits for every other one, so the grid
   // must be resident at once: checked once per device for the largest LDS size
-  static int resident[64] = {0};  // 0 unknown, else workgroups per compute unit + 1
+  static std::atomic<int> resident[64];  // 0 unknown, else workgroups per compute unit + 1
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return kErrBadArg;
-  if (resident[dev] == 0) {
+  int known = resident[dev].load(std::memory_order_acquire);
+  if (known == 0) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(peel_lds_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)kLdsPeelBudget);
     if (e != hipSuccess) return (int)e;
     int per_cu = 0;
     e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, peel_lds_kernel, kLdsPeelThreads, kLdsPeelBudget);
     if (e != hipSuccess) return (int)e;
-    resident[dev] = per_cu + 1;
+    known = per_cu + 1;
+    resident[dev].store(known, std::memory_order_release);
   }
-  if ((int64_t)(resident[dev] - 1) * device_cus() < sweepers + 1) return kErrBadArg;
+  if ((int64_t)(known - 1) * device_cus() < sweepers + 1) return kErrBadArg;
   hipLaunchKernelGGL(peel_lds_kernel, dim3(sweepers + 1), dim3(kLdsPeelThreads), lds, s, w.at<uint64_t>(L.dom), L.wstride, L.nwords, L.n,
                      w.at<int>(L.orig_of), w.at<int>(L.rank), fill_dist ? w.at<float>(L.dist) : (float*)nullptr,
                      w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
@@ -933,13 +975,17 @@ static int launch_batched_m(const BatchedArgs& a, int64_t batch, hipStream_t s) 
   const size_t lds = batched_lds_bytes(nt, M);
   // the attribute belongs to the (kernel, device) pair: remembered per device
   static size_t granted[64] = {0};
+  static std::mutex mu;  // (a smaller grant by another thread must not follow a larger one)
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
-  if (lds > 48 * 1024 && (dev < 0 || lds > granted[dev])) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(batched_kernel<M>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-    if (dev >= 0) granted[dev] = lds;
+  if (lds > 48 * 1024) {
+    std::lock_guard<std::mutex> lock(mu);
+    if (dev < 0 || lds > granted[dev]) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(batched_kernel<M>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return (int)e;
+      if (dev >= 0) granted[dev] = lds;
+    }
   }
   // grid.x carries the batch; very large batches go in slices
   for (int64_t b0 = 0; b0 < batch; b0 += 0x40000000ll) {
@@ -1050,6 +1096,10 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.dominance_folded = (int)value;
   } else if (!strcmp(name, "small_sort") && (value == 0 || value == 1)) {
     o.small_sort = (int)value;
+  } else if (!strcmp(name, "one_sort") && (value == 0 || value == 1)) {
+    o.one_sort = (int)value;
+  } else if (!strcmp(name, "one_sort_cap") && value >= 0 && value <= kOneSortCap) {
+    o.one_sort_cap = (int)value;
   } else if (!strcmp(name, "mid_argsort") && (value == 0 || value == 1)) {
     o.mid_argsort = (int)value;
   } else if (!strcmp(name, "prefix_min_rows") && value >= 0) {
@@ -1937,7 +1987,12 @@ int evox_hip_peel_plan(int64_t n, int64_t m, int64_t* out3) {
 }
 
 int evox_hip_read_status(const void* ws, void* stream, int32_t* host_out8) {
-  if (ws == nullptr || host_out8 == nullptr) return kErrBadArg;
+  if (host_out8 == nullptr) return kErrBadArg;
+  if (ws == nullptr) {  // the library's own scratch memory on the current device (the entry point that takes no workspace)
+    void* own = nullptr;
+    if (int e = static_scratch(&own)) return e;
+    ws = own;
+  }
   // the control block is the first region of the workspace
   hipError_t e = hipMemcpyAsync(host_out8, ws, 8 * sizeof(int32_t), hipMemcpyDeviceToHost, (hipStream_t)stream);
   if (e != hipSuccess) return (int)e;

@@ -116,7 +116,13 @@ torch.library.register_vmap(nd_rank, _nd_rank_vmap)
 
 
 RANK_UNSET = 0x7FFFFFFF
-_SMALL_ARGSORT_ROWS = 32768  # longest one-dimensional sort whose kernel has no device-side waits (and keeps no control block)
+def _argsort_waits(n: int) -> bool:
+    """Whether a one-dimensional argsort step of n positions goes through the radix kernel, whose workgroups wait for
+    each other and report a wait that ran out in a control block: sorts of more than 32 768 positions, and with the
+    tunable ``mid_argsort`` switched off those of more than 8192."""
+    return n > (32768 if runtime.current_option("mid_argsort", 1) else 8192)
+
+
 _ROWS_ARGSORT_MAX = 16384  # longest sort of a batch that runs inside one workgroup
 
 
@@ -608,7 +614,7 @@ def stable_argsort_step(key: torch.Tensor, kind: int, prev: Optional[torch.Tenso
         _lib.call("evox_hip_stable_argsort_step", key.data_ptr(), kind, key.stride(0), n,
                   None if prev is None else prev.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
         # only the radix sort of long keys waits on the device and keeps a control block
-        if n > _SMALL_ARGSORT_ROWS:
+        if _argsort_waits(n):
             runtime.note_call(ws, stream)
         else:
             runtime.note_small_kernel_call()
@@ -646,7 +652,7 @@ def stable_argsort_rows(key: torch.Tensor, kind: int, prev: Optional[torch.Tenso
         stream = runtime.stream_handle(key.device)
         _lib.call("evox_hip_stable_argsort_step_batched", key.data_ptr(), kind, key.stride(0), key.stride(1), batch, n,
                   None if prev is None else prev.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
-        if n > _SMALL_ARGSORT_ROWS:
+        if _argsort_waits(n) and (batch < 2 or n > _ROWS_ARGSORT_MAX):
             runtime.note_call(ws, stream)
         else:
             runtime.note_small_kernel_call()

@@ -156,12 +156,25 @@ def last_status() -> dict:
     return dict(zip(keys, list(out)[:7]))
 
 
+_process_options: Dict[str, int] = {}  # what set_option has changed (the library holds the values themselves)
+
+
 def set_option(name: str, value: int) -> None:
     """Changes a process-wide tunable (configuration at start-up; see ``options`` for a scoped change)."""
     _lib.call("evox_hip_set_option", name.encode(), int(value))
+    _process_options[name] = int(value)
 
 
 _options_in_use = threading.local()
+
+
+def current_option(name: str, default: int) -> int:
+    """The value of a tunable as the calls of this thread see it, where this module has set it (else ``default``,
+    which must be the library's own default)."""
+    stack = getattr(_options_in_use, "stack", None)
+    if stack and name in stack[-1][1]:
+        return stack[-1][1][name]
+    return _process_options.get(name, default)
 
 
 @contextlib.contextmanager

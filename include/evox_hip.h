@@ -8,6 +8,15 @@
  *     and synchronises only in evox_hip_read_status().  (One entry point brings its own scratch memory
  *     instead of taking a workspace: evox_hip_nd_environmental_selection_static.)  All work is enqueued on `stream`
  *     (a hipStream_t passed as void*).
+ *   - What the library keeps between calls, per process: the tunables; per device, small host-side tables of what it
+ *     has asked the runtime once (compute units, resident workgroups, LDS grants); the scratch buffer of the entry
+ *     point named above (EVOX_HIP_STATIC_SCRATCH_BYTES of device memory on every GPU that the process touches,
+ *     whether or not that entry point is ever called: it is part of the device image); and 64 bytes of pinned host
+ *     memory per device, allocated at the first selection, in which the last kernel of a selection notes whether the
+ *     peel kernel ordered the last front -- the next selection of a like shape picks its launches by it (tunable
+ *     "launch_memory"; 0 = never looked at).  Results never depend on any of it; the time of a call can, by a few
+ *     microseconds (a first call, or calls whose last fronts alternate between small and large, take the other set
+ *     of launches).
  *   - Fitness `f` is float32, addressed as f[i * stride_row + k * stride_col] (strides in elements),
  *     minimisation, n rows (individuals) by m columns (objectives).
  *   - The workspace must hold evox_hip_workspace_bytes(n, m) bytes, 256-byte aligned.  Calls that
@@ -295,7 +304,8 @@ int evox_hip_peel_plan(int64_t n, int64_t m, int64_t* out3);
  * or below the diagonal).  Depends on the tunables. */
 int evox_hip_dominance_plan(int64_t n, int64_t m, int64_t* out2);
 
-/* Waits for `stream`, then copies the control block's eight leading ints to HOST memory:
+/* Waits for `stream`, then copies the control block's eight leading ints to HOST memory (workspace == NULL: those of
+ * the library's own scratch buffer on the current device, i.e. of evox_hip_nd_environmental_selection_static):
  * out[0] error (0 or EVOX_HIP_E_BARRIER_TIMEOUT), out[1] fronts peeled, out[2] last front's rank,
  * out[3] rows in better fronts, out[4] last front's size, out[5] rows taken from it, out[6] sweep passes.
  * Returns out[0] when it is non-zero. */

@@ -131,7 +131,7 @@ def test_float64_long_sorts_and_vmap(float64_default):
     LDS; mapped populations go through the same operators."""
     g = torch.Generator("cpu").manual_seed(67)
     f = torch.rand(40000, 2, generator=g, dtype=torch.float64)
-    f[::7, 0] = f[3::7, 0][: f[::7].size(0)]  # ties
+    f[:5000, 0] = f[5000:10000, 0]  # ties
     mask = torch.rand(40000, generator=g) < 0.4
     _close(crowding_distance(f.to(DEV), mask.to(DEV)), er.crowding(f, mask), "40000 rows")
     _close(crowding_distance(f.to(DEV), None), er.crowding(f, None), "40000 rows, no mask")
