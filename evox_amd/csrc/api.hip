@@ -20,7 +20,7 @@
 #include "peel_lds.hpp"
 #include "prefix.hpp"
 #include "radix.hpp"
-#include "slotsort.hpp"
+#include "stepped.hpp"
 #include "wide.hpp"
 
 namespace evx {
@@ -37,6 +37,8 @@ struct Options {
   int peel_records = 1;  // record protocol (all-to-all, no master) for populations up to kRecordsMaxRowsWide
   int peel_lds = 1;      // populations whose lower triangle fits the LDS of the device are peeled from LDS (peel_lds.hpp)
   int peel_lds_blocks = 0;  // sweeping workgroups of that kernel, 0 = by size
+  int peel_stepped = 0;     // 1: the fronts are peeled one launch each by kernels that never wait for each other (stepped.hpp),
+                            // and the last front is ordered likewise; 0: only where the persistent grids cannot be resident
   int peel_tail = 1;        // that kernel also orders a small last front (0: always the kernels of finish.hpp)
   int tail_merged = 1;      // after such a peel, ordering (where still needed) and gather share one launch
   int launch_memory = 1;    // ... unless the last selection of this shape had a last front that the peel left alone
@@ -45,8 +47,6 @@ struct Options {
   int dominance_folded = 1;      // tiles of two words: only the blocks at or below the diagonal are launched
   int mid_argsort = 1;  // an argsort step of 8193 .. kMidArgsortRows positions in one kernel without waits (0: the radix sort)
   int small_sort = 1;  // populations up to kSmallSortRows rows are put in slot order by one kernel (0: bucket sort)
-  int one_sort = 1;    // populations of kOneSortMinRows .. kOneSortMaxRows rows likewise (slotsort.hpp; 0: bucket sort)
-  int one_sort_cap = kOneSortCap;  // members of a range that kernel places from LDS (smaller values: for tests of the other way)
   int64_t prefix_min_rows = 65536;  // finite populations of at least this many rows and 3 objectives (a quarter more
                                     // with 2, fewer with more: 28672 at 8, 10240 at 16 -- prefix_least_rows) get
                                     // their matrix from the per-objective orders (prefix.hpp); 0 = never
@@ -66,10 +66,12 @@ struct Layout {
   int64_t wstride;
   // byte offsets
   size_t ctrl, fsize, fronts_slot, fronts_orig, hist, zero_end, fstart, xs, key, partials, sortparam, bstart, bcursor,
-      scanflags, tailbuf, records, members, member_key, slot_of, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, total0, witness0, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, dom, total;
+      scanflags, tailbuf, records, members, member_key, slot_of, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, total0, witness0, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, wide, wide_bytes, dom, total;
 };
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
+static size_t wide_workspace_need(int64_t n, int64_t m);  // (workspace of the kernels of wide.hpp, defined with them)
+constexpr int kErrNotResident = -100;  // internal: the grid of a persistent kernel would not be resident at once
 
 static bool make_layout(int64_t n, int64_t m, Layout* L) {
   if (n < 1 || m < 1 || n > 0x7FFFFF00ll || m > 65535) return false;
@@ -132,6 +134,10 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->scost = o;      o = align_up(o + sizeof(float) * (size_t)m * L->kstride);
   L->dkey = o;       o = align_up(o + sizeof(uint32_t) * (size_t)L->kstride);
   L->dom = o;        o = align_up(o + sizeof(uint64_t) * (size_t)n * (size_t)L->wstride);
+  // behind the matrix (the entry points that build none need only the bytes before it): the ordering of the last
+  // front by kernels that never wait for each other (the tail of the stepped path)
+  L->wide_bytes = wide_workspace_need(n, m);
+  L->wide = o;       o = align_up(o + L->wide_bytes);
   L->total = o;
   return true;
 }
@@ -146,7 +152,7 @@ struct Ws {
   Ctrl* ctrl() const { return at<Ctrl>(L.ctrl); }
 };
 
-// The bit matrix is the last region: entry points that never build it need only the bytes before it.
+// The bit matrix and what lies behind it are the last regions: entry points that never build it need only the bytes before it.
 static int open_ws(int64_t n, int64_t m, void* ws, size_t bytes, Ws* out, bool with_matrix = true) {
   if (!make_layout(n, m, &out->L)) return kErrBadArg;
   const size_t need = with_matrix ? out->L.total : out->L.dom;
@@ -310,20 +316,6 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
     EVX_LAUNCH_CHECK();
     return 0;
   }
-  if (with_sort && L.n >= kOneSortMinRows && L.n <= kOneSortMaxRows && (int64_t)L.n * L.m <= kOneSortMaxValues && opt().one_sort) {
-    // as many workgroups as compute units, a power of two (each takes one range of the sample's cuts)
-    int grid = kOneSortSamples;
-    while (grid > 8 && grid > device_cus()) grid >>= 1;
-    auto launch = [&](auto kernel) {
-      hipLaunchKernelGGL(kernel, dim3(grid), dim3(kOneSortThreads), 0, s, src.f, src.sr, src.sc, (int)src.n_first, src.f2, src.sr2,
-                         src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs), w.at<double>(L.key), w.at<SortParam>(L.sortparam),
-                         w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of),
-                         w.at<int>(L.slot_of), w.at<uint32_t>(L.ctrl), zero_words, opt().one_sort_cap);
-    };
-    launch(one_sort_kernel);
-    EVX_LAUNCH_CHECK();
-    return 0;
-  }
   hipLaunchKernelGGL(prepare_kernel, dim3(L.prep_blocks), dim3(256), 0, s, src.f, src.sr, src.sc, (int)src.n_first, src.f2,
                      src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs), w.at<uint64_t>(L.key),
                      w.at<unsigned long long>(L.partials), w.at<uint32_t>(L.ctrl), zero_words);
@@ -384,7 +376,8 @@ static int dominance_tile_words(const Layout& L) {
 static int stage_dominance(const Ws& w, int variant, hipStream_t s) {
   // (kDomOrdersOnly: the first half of the path below alone, for measurements of the second)
   if (variant == kDomOrdersOnly) return prefix_dominance_applies(w.L) ? stage_dominance_prefix(w, true, s) : kErrBadArg;
-  if (variant == kDomAuto && prefix_dominance_applies(w.L)) return stage_dominance_prefix(w, false, s);
+  // (the orders of that path come from kernels whose workgroups wait for each other: not with the stepped path)
+  if (variant == kDomAuto && prefix_dominance_applies(w.L) && !opt().peel_stepped) return stage_dominance_prefix(w, false, s);
   // (the lower triangle in tiles of 4 words keeps every SIMD busy with several waves; up to about 24 000 rows of
   // two to eight objectives tiles of 2 words leave a shorter half-empty tail -- measured, us, tiles of 2 / 4:
   // 5000 x 3: 5.8 / 7.9, 16 000 x 3: 20.3 / 25.7, 20 000 x 2: 20.6 / 23.1, x 3: 27.6 / 31.3, x 8: 64.3 / 80.8,
@@ -537,7 +530,7 @@ static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool
     known = per_cu + 1;
     resident[dev].store(known, std::memory_order_release);
   }
-  if ((int64_t)(known - 1) * device_cus() < sweepers + 1) return kErrBadArg;
+  if ((int64_t)(known - 1) * device_cus() < sweepers + 1) return kErrNotResident;
   hipLaunchKernelGGL(peel_lds_kernel, dim3(sweepers + 1), dim3(kLdsPeelThreads), lds, s, w.at<uint64_t>(L.dom), L.wstride, L.nwords, L.n,
                      w.at<int>(L.orig_of), w.at<int>(L.rank), fill_dist ? w.at<float>(L.dist) : (float*)nullptr,
                      w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
@@ -552,8 +545,28 @@ static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool
 static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s);
 static int stage_count(const Ws& w, bool fill_dist, hipStream_t s, bool need_counts = true);
 static int peel_pass_plan(const Layout& L, int* blocks_out, int* use_witness_out);
+static int stage_peel_stepped(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s);
+static int count_and_peel_persistent(const Ws& w, int64_t stop_count, bool want_perm, bool fill_dist, hipStream_t s,
+                                     bool order_last_front, bool* may_have_ordered, bool* always_orders);
+
+// used_stepped: the fronts were peeled one launch each (stepped.hpp) -- asked for by the tunable, or because the grids
+// of the persistent kernels would not be resident at once on this device; the last front is then left to the caller.
 static int count_and_peel(const Ws& w, int64_t stop_count, bool want_perm, bool fill_dist, hipStream_t s,
-                          bool order_last_front = false, bool* may_have_ordered = nullptr, bool* always_orders = nullptr) {
+                          bool order_last_front = false, bool* may_have_ordered = nullptr, bool* always_orders = nullptr,
+                          bool* used_stepped = nullptr) {
+  if (used_stepped) *used_stepped = false;
+  int e = kErrNotResident;
+  if (!opt().peel_stepped) e = count_and_peel_persistent(w, stop_count, want_perm, fill_dist, s, order_last_front, may_have_ordered, always_orders);
+  if (e != kErrNotResident) return e;
+  if (may_have_ordered) *may_have_ordered = false;
+  if (always_orders) *always_orders = false;
+  if (used_stepped) *used_stepped = true;
+  if (int c = stage_count(w, fill_dist, s, true)) return c;
+  return stage_peel_stepped(w, stop_count, want_perm, s);
+}
+
+static int count_and_peel_persistent(const Ws& w, int64_t stop_count, bool want_perm, bool fill_dist, hipStream_t s,
+                                     bool order_last_front, bool* may_have_ordered, bool* always_orders) {
   size_t lds = 0;
   if (may_have_ordered) *may_have_ordered = false;
   if (always_orders) *always_orders = false;
@@ -613,7 +626,7 @@ static int peel_pass_plan(const Layout& L, int* blocks_out, int* use_witness_out
     blocks = grid_for(bitmap, &err);
     if (err) return err;
   }
-  if (blocks <= kFirstSweeper) return kErrBadArg;
+  if (blocks <= kFirstSweeper) return kErrNotResident;
   *blocks_out = blocks;
   *use_witness_out = use_witness;
   return 0;
@@ -663,6 +676,38 @@ static int stage_peel(const Ws& w, int64_t stop_count, bool want_perm, hipStream
                      want_perm ? w.at<int>(L.perm) : (int*)nullptr, w.at<int>(L.fstart), w.ctrl(), (int)stop_count,
                      opt().spin_limit, w.at<int>(L.witness), use_witness);
   EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+// One launch per front, in groups; between groups the host waits for the stream and reads whether the pass that finds
+// the ranking complete has run (the only place where this path waits).  stage_count must have left the full counts.
+constexpr int kStepGroup = 16;
+static int stage_peel_stepped(const Ws& w, int64_t stop_count, bool want_perm, hipStream_t s) {
+  const Layout& L = w.L;
+  if (stop_count < 1 || stop_count > L.n) return kErrBadArg;
+  const size_t lds = sizeof(uint64_t) * (size_t)((L.nwords + 1) & ~1);
+  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(step_pass_kernel), lds)) return e;
+  int sweepers = (L.n + kStepThreads / 64 - 1) / (kStepThreads / 64);
+  const int cap = device_cus() * 8;
+  if (sweepers > cap) sweepers = cap;
+  const int listers = (L.nwords + kStepListWords - 1) / kStepListWords;
+  // (front L.n - 1 is the last that can exist; the pass after a front is the one that sees it complete)
+  for (int64_t level = 1; level <= (int64_t)L.n + 1;) {
+    for (int k = 0; k < kStepGroup && level <= (int64_t)L.n + 1; ++k, ++level) {
+      hipLaunchKernelGGL(step_pass_kernel, dim3(sweepers + listers), dim3(kStepThreads), lds, s, w.at<uint64_t>(L.dom), L.wstride,
+                         L.nwords, L.n, w.at<int>(L.orig_of), w.at<int>(L.count), w.at<int>(L.rank), w.at<uint64_t>(L.fronts_slot),
+                         w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize), w.at<int>(L.fstart),
+                         want_perm ? w.at<int>(L.perm) : (int*)nullptr, w.ctrl(), (int)stop_count, (int)level, sweepers);
+      EVX_LAUNCH_CHECK();
+    }
+    int32_t head[16];
+    hipError_t e = hipMemcpyAsync(head, w.ctrl(), sizeof(head), hipMemcpyDeviceToHost, s);
+    if (e != hipSuccess) return (int)e;
+    e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return (int)e;
+    static_assert(offsetof(Ctrl, reserved) == 40 && sizeof(int32_t) * (10 + kStepDone + 1) <= sizeof(head), "Ctrl.reserved[kStepDone]");
+    if (head[0] != 0 || head[10 + kStepDone] != 0) break;
+  }
   return 0;
 }
 
@@ -1084,6 +1129,8 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.tail_merged = (int)value;
   } else if (!strcmp(name, "launch_memory") && (value == 0 || value == 1)) {
     o.launch_memory = (int)value;
+  } else if (!strcmp(name, "peel_stepped") && (value == 0 || value == 1)) {
+    o.peel_stepped = (int)value;
   } else if (!strcmp(name, "peel_tail") && (value == 0 || value == 1)) {
     o.peel_tail = (int)value;
   } else if (!strcmp(name, "peel_lds_blocks") && (value == 0 || (value >= 8 && value <= 255))) {
@@ -1096,10 +1143,6 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.dominance_folded = (int)value;
   } else if (!strcmp(name, "small_sort") && (value == 0 || value == 1)) {
     o.small_sort = (int)value;
-  } else if (!strcmp(name, "one_sort") && (value == 0 || value == 1)) {
-    o.one_sort = (int)value;
-  } else if (!strcmp(name, "one_sort_cap") && value >= 0 && value <= kOneSortCap) {
-    o.one_sort_cap = (int)value;
   } else if (!strcmp(name, "mid_argsort") && (value == 0 || value == 1)) {
     o.mid_argsort = (int)value;
   } else if (!strcmp(name, "prefix_min_rows") && value >= 0) {
@@ -1420,6 +1463,115 @@ int evox_hip_stable_argsort_step_batched(const void* key, int kind, int64_t batc
 
 }  // extern "C"
 
+// ---- fitness of 8-byte elements (wide.hpp)
+struct WideLayout {
+  int n, m;
+  size_t ctrl, key_lo, key_hi, key_mask, selected, boundary, ord_a, ord_b, terms, dist, neg_lo, neg_hi, order_a, order_b, sort_ws,
+      sort_bytes, total;
+};
+
+static bool make_wide_layout(int64_t n, int64_t m, WideLayout* L) {
+  if (n < 1 || m < 1 || n > 0x7FFFFF00ll || m > 65535 || n * m > 0x7FFFFFFFll * 16) return false;
+  L->n = (int)n;
+  L->m = (int)m;
+  const size_t nm = (size_t)n * (size_t)m;
+  size_t o = 0;
+  L->ctrl = o;      o = align_up(o + sizeof(WideCtrl));
+  L->key_lo = o;    o = align_up(o + 4 * nm);
+  L->key_hi = o;    o = align_up(o + 4 * nm);
+  L->key_mask = o;  o = align_up(o + 4 * (size_t)n);
+  L->selected = o;  o = align_up(o + (size_t)n);
+  L->boundary = o;  o = align_up(o + 4 * (size_t)n);
+  L->ord_a = o;     o = align_up(o + 4 * nm);
+  L->ord_b = o;     o = align_up(o + 4 * nm);
+  L->terms = o;     o = align_up(o + 8 * nm);
+  L->dist = o;      o = align_up(o + 8 * (size_t)n);
+  L->neg_lo = o;    o = align_up(o + 4 * (size_t)n);
+  L->neg_hi = o;    o = align_up(o + 4 * (size_t)n);
+  L->order_a = o;   o = align_up(o + 4 * (size_t)n);
+  L->order_b = o;   o = align_up(o + 4 * (size_t)n);
+  SortLayout sort_layout;
+  if (!make_sort_layout(n, &sort_layout)) return false;
+  L->sort_bytes = sort_layout.total;
+  L->sort_ws = o;   o = align_up(o + L->sort_bytes);
+  L->total = o;
+  return true;
+}
+
+static int wide_grid(int64_t items) {
+  int64_t blocks = (items + 255) / 256;
+  const int64_t cap = (int64_t)device_cus() * 8;
+  if (blocks > cap) blocks = cap;
+  return (int)(blocks < 1 ? 1 : blocks);
+}
+
+// The crowding distances of the rows selected by the mask, by the rank vector (rank == its largest set value) or all
+// rows, into `dist` (double for out_kind 0, float for 1), and with neg_keys the sort keys of their negatives.
+static int wide_distances(const WideLayout& L, uint8_t* base, const void* costs, int kind, int64_t sr, int64_t sc,
+                          const uint8_t* mask, int64_t mask_stride, const int32_t* rank, void* dist, int out_kind, bool neg_keys,
+                          hipStream_t s) {
+  const int n = L.n, m = L.m;
+  WideCtrl* ctrl = reinterpret_cast<WideCtrl*>(base + L.ctrl);
+  uint32_t* key_lo = reinterpret_cast<uint32_t*>(base + L.key_lo);
+  uint32_t* key_hi = reinterpret_cast<uint32_t*>(base + L.key_hi);
+  int* key_mask = reinterpret_cast<int*>(base + L.key_mask);
+  uint8_t* selected = base + L.selected;
+  int* boundary = reinterpret_cast<int*>(base + L.boundary);
+  int* ord_a = reinterpret_cast<int*>(base + L.ord_a);
+  int* ord_b = reinterpret_cast<int*>(base + L.ord_b);
+  hipLaunchKernelGGL(wide_head_kernel, dim3(1), dim3(1024), 0, s, mask, mask_stride, rank, n, ctrl);
+  EVX_LAUNCH_CHECK();
+  hipLaunchKernelGGL(wide_keys_kernel, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, mask, mask_stride,
+                     rank, ctrl, key_lo, key_hi, key_mask, selected, boundary);
+  EVX_LAUNCH_CHECK();
+  // per objective: by cost (low half, then high half of its ordered image), then selected rows first; ties by row
+  void* sort_ws = base + L.sort_ws;
+  if (int e = evox_hip_stable_argsort_step_batched(key_lo, kKeyUint32, n, 1, m, n, nullptr, ord_a, sort_ws, L.sort_bytes, s)) return e;
+  if (int e = evox_hip_stable_argsort_step_batched(key_hi, kKeyUint32, n, 1, m, n, ord_a, ord_b, sort_ws, L.sort_bytes, s)) return e;
+  const int* order = ord_b;
+  if (mask != nullptr || rank != nullptr) {
+    if (int e = evox_hip_stable_argsort_step_batched(key_mask, kKeyInt32, 0, 1, m, n, ord_b, ord_a, sort_ws, L.sort_bytes, s)) return e;
+    order = ord_a;
+  }
+  uint32_t* neg_lo = neg_keys ? reinterpret_cast<uint32_t*>(base + L.neg_lo) : nullptr;
+  uint32_t* neg_hi = neg_keys ? reinterpret_cast<uint32_t*>(base + L.neg_hi) : nullptr;
+  if (out_kind == 0) {
+    double* terms = reinterpret_cast<double*>(base + L.terms);
+    hipLaunchKernelGGL(wide_terms_kernel<double>, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, order, ctrl,
+                       terms, boundary);
+    EVX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(wide_sum_kernel<double>, dim3(wide_grid(n)), dim3(256), 0, s, terms, selected, boundary, ctrl, n, m,
+                       static_cast<double*>(dist), neg_lo, neg_hi);
+  } else {
+    float* terms = reinterpret_cast<float*>(base + L.terms);
+    hipLaunchKernelGGL(wide_terms_kernel<float>, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, order, ctrl,
+                       terms, boundary);
+    EVX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(wide_sum_kernel<float>, dim3(wide_grid(n)), dim3(256), 0, s, terms, selected, boundary, ctrl, n, m,
+                       static_cast<float*>(dist), neg_lo, neg_hi);
+  }
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+static int gather_rows(const void* src, int64_t row_bytes, int64_t row_stride_bytes, const int* order, int64_t count, void* dst,
+                       hipStream_t s) {
+  if (row_bytes <= 0 || count <= 0) return 0;
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | (uintptr_t)row_bytes | (uintptr_t)row_stride_bytes;
+  const int unit = bits % 16 == 0 ? 16 : bits % 8 == 0 ? 8 : bits % 4 == 0 ? 4 : 1;
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(wide_grid(count * (row_bytes / unit))), dim3(256), 0, s, static_cast<const uint8_t*>(src),
+                     row_bytes, row_stride_bytes, order, count, static_cast<uint8_t*>(dst), unit);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+namespace evx {
+static size_t wide_workspace_need(int64_t n, int64_t m) {
+  WideLayout L;
+  return make_wide_layout(n, m, &L) ? L.total : 0;
+}
+}  // namespace evx
+
 // Shared body of the two selection entry points: the population is one part or two.
 static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes, const void* x2,
                        int64_t x2_row_stride_bytes, const Fitness& fit, int64_t n, int64_t m, int64_t topk, void* out_x,
@@ -1436,7 +1588,8 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   if (int e = stage_dominance(w, kDomAuto, s)) return e;
   bool peel_orders = false;  // the peel kernel orders a small last front itself (it says so in Ctrl.tail_done)
   bool peel_always_orders = false;  // ... and here every front is small enough: nothing is left to launch but the gather
-  if (int e = count_and_peel(w, topk, true, true, s, true, &peel_orders, &peel_always_orders)) return e;
+  bool stepped = false;  // the fronts were peeled one launch each: the last front is ordered likewise, by the kernels of wide.hpp
+  if (int e = count_and_peel(w, topk, true, true, s, true, &peel_orders, &peel_always_orders, &stepped)) return e;
   int unit = 1;
   if (x != nullptr) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(x2) | reinterpret_cast<uintptr_t>(out_x) |
@@ -1482,6 +1635,30 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   // last fronts of thousands of rows, which the kernels of their own order 20-30 us faster (20 000 x 3, one front: 166
   // against 194 us), and a last front that the peel ordered will mostly be followed by another.
   const bool one_ordering_launch = peel_orders && opt().tail_merged && L.m <= 3 && last_outcome != 2;
+  if (stepped) {
+    // distances of the rows of the last front (the mask rank == worst), the order by (rank, distance descending, index)
+    // from three stable argsort steps, the gather: the fitness is read from its structure-of-arrays copy
+    WideLayout WL;
+    if (!make_wide_layout(n, m, &WL) || WL.total > L.wide_bytes) return kErrWorkspace;
+    uint8_t* wb = w.base + L.wide;
+    if (int e = wide_distances(WL, wb, w.at<float>(L.xs), kWideFloat32, 1, L.npad, nullptr, 0, w.at<int>(L.rank), w.at<float>(L.dist), 1,
+                               true, s))
+      return e;
+    int* order_a = reinterpret_cast<int*>(wb + WL.order_a);
+    int* order_b = reinterpret_cast<int*>(wb + WL.order_b);
+    void* sort_ws = wb + WL.sort_ws;
+    if (int e = evox_hip_stable_argsort_step(wb + WL.neg_lo, kKeyUint32, 1, n, nullptr, order_a, sort_ws, WL.sort_bytes, s)) return e;
+    if (int e = evox_hip_stable_argsort_step(wb + WL.neg_hi, kKeyUint32, 1, n, order_a, order_b, sort_ws, WL.sort_bytes, s)) return e;
+    if (int e = evox_hip_stable_argsort_step(w.at<int>(L.rank), kKeyInt32, 1, n, order_b, w.at<int>(L.order), sort_ws, WL.sort_bytes, s))
+      return e;
+    g.outcome = nullptr;
+    int blocks = (int)((topk + 3) / 4);
+    const int cap = device_cus() * 8;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(256), 0, s, g);
+    EVX_LAUNCH_CHECK();
+    return 0;
+  }
   if (peel_always_orders) {
     int blocks = (int)((topk + 3) / 4);
     const int cap = device_cus() * 8;
@@ -1560,107 +1737,6 @@ int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_ro
 }
 
 }  // extern "C"
-
-// ---- fitness of 8-byte elements (wide.hpp)
-struct WideLayout {
-  int n, m;
-  size_t ctrl, key_lo, key_hi, key_mask, selected, boundary, ord_a, ord_b, terms, dist, neg_lo, neg_hi, order_a, order_b, sort_ws,
-      sort_bytes, total;
-};
-
-static bool make_wide_layout(int64_t n, int64_t m, WideLayout* L) {
-  if (n < 1 || m < 1 || n > 0x7FFFFF00ll || m > 65535 || n * m > 0x7FFFFFFFll * 16) return false;
-  L->n = (int)n;
-  L->m = (int)m;
-  const size_t nm = (size_t)n * (size_t)m;
-  size_t o = 0;
-  L->ctrl = o;      o = align_up(o + sizeof(WideCtrl));
-  L->key_lo = o;    o = align_up(o + 4 * nm);
-  L->key_hi = o;    o = align_up(o + 4 * nm);
-  L->key_mask = o;  o = align_up(o + 4 * (size_t)n);
-  L->selected = o;  o = align_up(o + (size_t)n);
-  L->boundary = o;  o = align_up(o + 4 * (size_t)n);
-  L->ord_a = o;     o = align_up(o + 4 * nm);
-  L->ord_b = o;     o = align_up(o + 4 * nm);
-  L->terms = o;     o = align_up(o + 8 * nm);
-  L->dist = o;      o = align_up(o + 8 * (size_t)n);
-  L->neg_lo = o;    o = align_up(o + 4 * (size_t)n);
-  L->neg_hi = o;    o = align_up(o + 4 * (size_t)n);
-  L->order_a = o;   o = align_up(o + 4 * (size_t)n);
-  L->order_b = o;   o = align_up(o + 4 * (size_t)n);
-  L->sort_bytes = evox_hip_argsort_workspace_bytes(n);
-  if (L->sort_bytes == 0) return false;
-  L->sort_ws = o;   o = align_up(o + L->sort_bytes);
-  L->total = o;
-  return true;
-}
-
-static int wide_grid(int64_t items) {
-  int64_t blocks = (items + 255) / 256;
-  const int64_t cap = (int64_t)device_cus() * 8;
-  if (blocks > cap) blocks = cap;
-  return (int)(blocks < 1 ? 1 : blocks);
-}
-
-// The crowding distances of the rows selected by the mask, by the rank vector (rank == its largest set value) or all
-// rows, into `dist` (double for out_kind 0, float for 1), and with neg_keys the sort keys of their negatives.
-static int wide_distances(const WideLayout& L, uint8_t* base, const void* costs, int kind, int64_t sr, int64_t sc,
-                          const uint8_t* mask, int64_t mask_stride, const int32_t* rank, void* dist, int out_kind, bool neg_keys,
-                          hipStream_t s) {
-  const int n = L.n, m = L.m;
-  WideCtrl* ctrl = reinterpret_cast<WideCtrl*>(base + L.ctrl);
-  uint32_t* key_lo = reinterpret_cast<uint32_t*>(base + L.key_lo);
-  uint32_t* key_hi = reinterpret_cast<uint32_t*>(base + L.key_hi);
-  int* key_mask = reinterpret_cast<int*>(base + L.key_mask);
-  uint8_t* selected = base + L.selected;
-  int* boundary = reinterpret_cast<int*>(base + L.boundary);
-  int* ord_a = reinterpret_cast<int*>(base + L.ord_a);
-  int* ord_b = reinterpret_cast<int*>(base + L.ord_b);
-  hipLaunchKernelGGL(wide_head_kernel, dim3(1), dim3(1024), 0, s, mask, mask_stride, rank, n, ctrl);
-  EVX_LAUNCH_CHECK();
-  hipLaunchKernelGGL(wide_keys_kernel, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, mask, mask_stride,
-                     rank, ctrl, key_lo, key_hi, key_mask, selected, boundary);
-  EVX_LAUNCH_CHECK();
-  // per objective: by cost (low half, then high half of its ordered image), then selected rows first; ties by row
-  void* sort_ws = base + L.sort_ws;
-  if (int e = evox_hip_stable_argsort_step_batched(key_lo, kKeyUint32, n, 1, m, n, nullptr, ord_a, sort_ws, L.sort_bytes, s)) return e;
-  if (int e = evox_hip_stable_argsort_step_batched(key_hi, kKeyUint32, n, 1, m, n, ord_a, ord_b, sort_ws, L.sort_bytes, s)) return e;
-  const int* order = ord_b;
-  if (mask != nullptr || rank != nullptr) {
-    if (int e = evox_hip_stable_argsort_step_batched(key_mask, kKeyInt32, 0, 1, m, n, ord_b, ord_a, sort_ws, L.sort_bytes, s)) return e;
-    order = ord_a;
-  }
-  uint32_t* neg_lo = neg_keys ? reinterpret_cast<uint32_t*>(base + L.neg_lo) : nullptr;
-  uint32_t* neg_hi = neg_keys ? reinterpret_cast<uint32_t*>(base + L.neg_hi) : nullptr;
-  if (out_kind == 0) {
-    double* terms = reinterpret_cast<double*>(base + L.terms);
-    hipLaunchKernelGGL(wide_terms_kernel<double>, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, order, ctrl,
-                       terms, boundary);
-    EVX_LAUNCH_CHECK();
-    hipLaunchKernelGGL(wide_sum_kernel<double>, dim3(wide_grid(n)), dim3(256), 0, s, terms, selected, boundary, ctrl, n, m,
-                       static_cast<double*>(dist), neg_lo, neg_hi);
-  } else {
-    float* terms = reinterpret_cast<float*>(base + L.terms);
-    hipLaunchKernelGGL(wide_terms_kernel<float>, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, order, ctrl,
-                       terms, boundary);
-    EVX_LAUNCH_CHECK();
-    hipLaunchKernelGGL(wide_sum_kernel<float>, dim3(wide_grid(n)), dim3(256), 0, s, terms, selected, boundary, ctrl, n, m,
-                       static_cast<float*>(dist), neg_lo, neg_hi);
-  }
-  EVX_LAUNCH_CHECK();
-  return 0;
-}
-
-static int gather_rows(const void* src, int64_t row_bytes, int64_t row_stride_bytes, const int* order, int64_t count, void* dst,
-                       hipStream_t s) {
-  if (row_bytes <= 0 || count <= 0) return 0;
-  const uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | (uintptr_t)row_bytes | (uintptr_t)row_stride_bytes;
-  const int unit = bits % 16 == 0 ? 16 : bits % 8 == 0 ? 8 : bits % 4 == 0 ? 4 : 1;
-  hipLaunchKernelGGL(gather_rows_kernel, dim3(wide_grid(count * (row_bytes / unit))), dim3(256), 0, s, static_cast<const uint8_t*>(src),
-                     row_bytes, row_stride_bytes, order, count, static_cast<uint8_t*>(dst), unit);
-  EVX_LAUNCH_CHECK();
-  return 0;
-}
 
 extern "C" {
 

@@ -92,12 +92,36 @@ __device__ inline void coherent_store(T* p, T v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// A wait on another workgroup that always ends: false when `spin_limit` polls were not enough.
+// The bound of a device-side wait (the tunable "spin_limit").  A value up to kPollLimitMax counts failed polls (for
+// tests that force a wait to give up: 1 ends it after the first failed poll, and every kernel still exits normally);
+// a larger value is a time in ticks of the device's constant 100 MHz clock -- 10 ns; the default of 4 000 000 is
+// 40 ms -- so that a wait ends after that time whatever else the device is doing, not after a number of polls whose
+// duration depends on the load.  The clock is read on every 64th failed poll, the first reading starting the time.
+constexpr unsigned kPollLimitMax = 65535u;
+struct WaitBound {
+  unsigned limit;
+  unsigned long long t0;
+  __device__ explicit WaitBound(unsigned l) : limit(l), t0(0ull) {}
+  // after the failed poll number `spins` (counted from 0): must the wait end?
+  __device__ bool expired(unsigned spins) {
+    if (limit <= kPollLimitMax) return spins > limit;
+    if ((spins & 63u) != 0u) return false;
+    const unsigned long long now = (unsigned long long)wall_clock64();
+    if (t0 == 0ull) {
+      t0 = now | 1ull;
+      return false;
+    }
+    return now - t0 > (unsigned long long)limit;
+  }
+};
+
+// A wait on another workgroup that always ends: false when the bound `spin_limit` (WaitBound) ran out.
 template <class Pred>
 __device__ inline bool bounded_wait(Pred done, unsigned spin_limit) {
   unsigned spins = 0;
+  WaitBound bound(spin_limit);
   while (!done()) {
-    if (++spins > spin_limit) return false;
+    if (bound.expired(++spins)) return false;
     __builtin_amdgcn_s_sleep(1);
   }
   return true;

@@ -184,6 +184,17 @@ __device__ inline void gather_body(const GatherArgs& a, int block, int blocks, i
   for (int64_t p = ((int64_t)block * (blockDim.x >> 6) + (threadIdx.x >> 6)) * per_wave + sub; p < topk;
        p += waves * per_wave) {
     const int64_t src = p < listed_until ? a.listed[p] : a.order[p];
+    if (src < 0) {  // an order that a failed sort has poisoned: no row is read through it, the outputs say so
+      if (x)
+        for (int64_t b = lane; b < x_row_bytes; b += g) out_x[p * x_row_bytes + b] = 0xFF;
+      for (int k = lane; k < m; k += g) out_f[p * m + k] = __uint_as_float(0x7FC00000u);
+      if (lane == 0) {
+        out_rank[p] = -1;
+        out_dist[p] = __uint_as_float(0x7FC00000u);
+        if (out_order) out_order[p] = -1;
+      }
+      continue;
+    }
     const bool second = src >= n_first;  // rows of the second part of a two-part population
     if (x) {
       const uint8_t* __restrict__ s = second ? x2 + (src - n_first) * a.x2_row_stride : x + src * a.x_row_stride;

@@ -97,7 +97,7 @@ __global__ __launch_bounds__(256) void bucket_hist_kernel(const uint64_t* __rest
 // bins, publishes (1 << 32 | total) in its flag, adds the totals of the blocks before it as they appear
 // (the flags start at zero), and then scans its own bins.  A block only ever waits for blocks of
 // lower index, which are dispatched before it and wait for nobody above them, so the wait ends; it is
-// bounded all the same (kScanSpinLimit polls), and running out sets the error flag, on which every
+// bounded all the same (kScanSpinLimit ticks of 10 ns), and running out sets the error flag, on which every
 // later kernel of the call returns without touching the half-built tables.
 constexpr unsigned kScanSpinLimit = 1u << 24;
 
@@ -127,8 +127,9 @@ __global__ __launch_bounds__(256) void bucket_scan_kernel(const int* __restrict_
     if (lane < (int)blockIdx.x) {
       unsigned long long f = 0;
       unsigned spins = 0;
+      WaitBound bound(kScanSpinLimit);
       while (((f = __hip_atomic_load(&flags[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) == 0) {
-        if (++spins > kScanSpinLimit) {
+        if (bound.expired(++spins)) {
           __hip_atomic_store(&ctrl->err, kErrBarrierTimeout, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }

@@ -992,6 +992,7 @@ __device__ inline bool poll_record_units(const unsigned long long* gen_units, in
       v[k] = ~0ull;
   }
   bool waiting_listed = listed != nullptr;
+  WaitBound bound(spin_limit);
   for (unsigned spins = 0;; ++spins) {
     int seen_listed = 0;
 #pragma unroll
@@ -1003,7 +1004,7 @@ __device__ inline bool poll_record_units(const unsigned long long* gen_units, in
       if ((pending & (1u << k)) && (unsigned)(v[k] >> 48) == (gen & 0xFFFFu)) pending &= ~(1u << k);
     if (waiting_listed && seen_listed >= listed_needed) waiting_listed = false;
     if (pending == 0u && !waiting_listed) return true;
-    if (spins > spin_limit) return false;
+    if (bound.expired(spins)) return false;
     if ((spins & 63u) == 63u && coherent_load(err) != 0) return false;
   }
 }

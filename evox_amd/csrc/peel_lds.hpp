@@ -69,6 +69,7 @@ __device__ inline bool poll_record_pair(const unsigned long long* gen_units, int
   v[0] = v[1] = ~0ull;                 // units past the last record are never written: they read as "no slot"
   bool waiting = have, waiting_listed = listed != nullptr;
   const unsigned long long* mine = gen_units + (have ? idx : 0);
+  WaitBound bound(spin_limit);
   for (unsigned spins = 0;; ++spins) {
     if (waiting) {
       u32x4 r;
@@ -81,7 +82,7 @@ __device__ inline bool poll_record_pair(const unsigned long long* gen_units, int
     }
     if (waiting_listed && coherent_load(listed) >= listed_needed) waiting_listed = false;
     if (!waiting && !waiting_listed) return true;
-    if (spins > spin_limit) return false;
+    if (bound.expired(spins)) return false;
     if ((spins & 63u) == 63u && coherent_load(err) != 0) return false;
   }
 }
@@ -739,6 +740,7 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
           bool pending0 = e0 < nv, pending1 = e0 + 2 < nv, fine_poll = true;
           // (both loads of a round are in flight together; the buffer holds kTailRows entries, a multiple of four,
           // so the second load of a thread whose first is in range stays inside it)
+          WaitBound bound(spin_limit);
           for (unsigned spins = 0; pending0 || pending1; ++spins) {
             u32x4 r0, r1;
             asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1\n\ts_waitcnt vmcnt(0)"
@@ -761,7 +763,7 @@ __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
                 pending1 = false;
               }
             }
-            if (spins > spin_limit || ((spins & 63u) == 63u && coherent_load(&ctrl->err) != 0)) {
+            if (bound.expired(spins) || ((spins & 63u) == 63u && coherent_load(&ctrl->err) != 0)) {
               fine_poll = false;
               break;
             }

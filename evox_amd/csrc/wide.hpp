@@ -1,4 +1,5 @@
-// Crowding distance and selection order for fitness of 8-byte elements (float64, int64).
+// Crowding distance and selection order for fitness of 8-byte elements (float64, int64), and -- as the tail of the
+// selection path whose kernels never wait for each other (stepped.hpp) -- of float32 fitness.
 //
 // Reference semantics: src/evox/operators/selection/non_dominate.py:198-231 computes the distance in the dtype of the
 // costs (differences) and in torch's default float dtype (the buffer that takes the quotients), so a population of
@@ -18,6 +19,7 @@ namespace evx {
 
 constexpr int kWideFloat64 = 0;  // costs are IEEE doubles
 constexpr int kWideInt64 = 1;    // costs are two's-complement 64-bit integers
+constexpr int kWideFloat32 = 2;  // costs are IEEE floats (differences and quotients in float, as the float32 kernels compute them)
 
 struct WideCtrl {
   int nv;     // rows selected by the mask
@@ -90,8 +92,9 @@ __global__ __launch_bounds__(256) void wide_keys_kernel(const void* __restrict__
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
     const int k = (int)(idx / n), i = (int)(idx - (int64_t)k * n);
     const int64_t at = (int64_t)i * stride_row + (int64_t)k * stride_col;
-    const uint64_t image = kind == kWideFloat64 ? ordered_key64(static_cast<const double*>(costs)[at])
-                                                : ordered_key64(static_cast<const long long*>(costs)[at]);
+    const uint64_t image = kind == kWideFloat64   ? ordered_key64(static_cast<const double*>(costs)[at])
+                           : kind == kWideFloat32 ? ordered_key64((double)static_cast<const float*>(costs)[at])
+                                                  : ordered_key64(static_cast<const long long*>(costs)[at]);
     key_lo[idx] = (uint32_t)image;
     key_hi[idx] = (uint32_t)(image >> 32);
     if (k == 0) {
@@ -107,6 +110,10 @@ template <class Out>
 __device__ inline Out wide_term(const void* costs, int kind, int64_t next, int64_t prev, int64_t last, int64_t first) {
   if (kind == kWideFloat64) {
     const double* c = static_cast<const double*>(costs);
+    return (Out)((c[next] - c[prev]) / (c[last] - c[first]));
+  }
+  if (kind == kWideFloat32) {
+    const float* c = static_cast<const float*>(costs);
     return (Out)((c[next] - c[prev]) / (c[last] - c[first]));
   }
   // integers: exact differences (wrapping, as the integer subtraction of the reference), divided as floats

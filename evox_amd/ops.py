@@ -72,9 +72,12 @@ def _rank_one(f: torch.Tensor, out: torch.Tensor) -> None:
     n, m = f.shape
     ws = runtime.workspace(n, m, f.device)
     stream = runtime.stream_handle(f.device)
-    _lib.call("evox_hip_non_dominate_rank", f.data_ptr(), n, m, f.stride(0), f.stride(1), out.data_ptr(), ws.data_ptr(),
-              ws.numel(), stream)
-    runtime.note_call(ws, stream)
+    def issue():
+        _lib.call("evox_hip_non_dominate_rank", f.data_ptr(), n, m, f.stride(0), f.stride(1), out.data_ptr(), ws.data_ptr(),
+                  ws.numel(), stream)
+        runtime.note_call(ws, stream)
+
+    runtime.checked(issue)
 
 
 @torch.library.custom_op("evox_amd::nd_rank", mutates_args=())
@@ -151,9 +154,13 @@ def nd_rank_until(f: torch.Tensor, count: int) -> torch.Tensor:
         stream = runtime.stream_handle(f.device)
         for b in range(flat_f.size(0)):
             fb = flat_f[b]
-            _lib.call("evox_hip_non_dominate_rank_until", fb.data_ptr(), n, m, fb.stride(0), fb.stride(1), count,
-                      flat_out[b].data_ptr(), ws.data_ptr(), ws.numel(), stream)
-        runtime.note_call(ws, stream)
+
+            def issue():
+                _lib.call("evox_hip_non_dominate_rank_until", fb.data_ptr(), n, m, fb.stride(0), fb.stride(1), count,
+                          flat_out[b].data_ptr(), ws.data_ptr(), ws.numel(), stream)
+                runtime.note_call(ws, stream)
+
+            runtime.checked(issue)
     return out
 
 
@@ -431,10 +438,14 @@ def nd_select(x: torch.Tensor, f: torch.Tensor, topk: int) -> Tuple[torch.Tensor
             runtime.note_small_kernel_call()
         else:
             ws = runtime.workspace(n, m, f.device)
-            _lib.call("evox_hip_nd_environmental_selection", x.data_ptr() if has_x else None, row_bytes, row_bytes,
-                      f.data_ptr(), n, m, f.stride(0), f.stride(1), topk, out_x.data_ptr() if has_x else None,
-                      out_f.data_ptr(), out_rank.data_ptr(), out_dist.data_ptr(), None, ws.data_ptr(), ws.numel(), stream)
-            runtime.note_call(ws, stream)
+
+            def issue():
+                _lib.call("evox_hip_nd_environmental_selection", x.data_ptr() if has_x else None, row_bytes, row_bytes,
+                          f.data_ptr(), n, m, f.stride(0), f.stride(1), topk, out_x.data_ptr() if has_x else None,
+                          out_f.data_ptr(), out_rank.data_ptr(), out_dist.data_ptr(), None, ws.data_ptr(), ws.numel(), stream)
+                runtime.note_call(ws, stream)
+
+            runtime.checked(issue)
         return out_x, out_f, out_rank, out_dist
     f32 = _as_f32(f, "fitness")
     batch = f.shape[:bd]
@@ -468,11 +479,15 @@ def nd_select(x: torch.Tensor, f: torch.Tensor, topk: int) -> Tuple[torch.Tensor
         ws = runtime.workspace(n, m, f.device)
         for b in range(flat_f.size(0)):
             fb, xb = flat_f[b], flat_x[b]
-            _lib.call("evox_hip_nd_environmental_selection", xb.data_ptr() if has_x else None, row_bytes,
-                      xb.stride(0) * xb.element_size(), fb.data_ptr(), n, m, fb.stride(0), fb.stride(1), topk,
-                      fo_x[b].data_ptr() if has_x else None, fo_f[b].data_ptr(), fo_r[b].data_ptr(), fo_d[b].data_ptr(),
-                      None, ws.data_ptr(), ws.numel(), stream)
-        runtime.note_call(ws, stream)
+
+            def issue():
+                _lib.call("evox_hip_nd_environmental_selection", xb.data_ptr() if has_x else None, row_bytes,
+                          xb.stride(0) * xb.element_size(), fb.data_ptr(), n, m, fb.stride(0), fb.stride(1), topk,
+                          fo_x[b].data_ptr() if has_x else None, fo_f[b].data_ptr(), fo_r[b].data_ptr(), fo_d[b].data_ptr(),
+                          None, ws.data_ptr(), ws.numel(), stream)
+                runtime.note_call(ws, stream)
+
+            runtime.checked(issue)
     return out_x, out_f.to(f.dtype), out_rank, out_dist
 
 
@@ -560,12 +575,15 @@ def nd_select_two_part(x_a: torch.Tensor, f_a: torch.Tensor, x_b: torch.Tensor, 
         has_x = row_bytes > 0
         ws = runtime.workspace(n, m, f_a.device)
         stream = runtime.stream_handle(f_a.device)
-        _lib.call("evox_hip_nd_environmental_selection_two_part", xa.data_ptr() if has_x else None, xa.stride(0) * es,
-                  xb.data_ptr() if has_x else None, xb.stride(0) * es, row_bytes, fa32.data_ptr(), n_a, fa32.stride(0),
-                  fa32.stride(1), fb32.data_ptr(), n_b, fb32.stride(0), fb32.stride(1), m, topk,
-                  out_x.data_ptr() if has_x else None, out_f.data_ptr(), out_rank.data_ptr(), out_dist.data_ptr(), None,
-                  ws.data_ptr(), ws.numel(), stream)
-        runtime.note_call(ws, stream)
+        def issue():
+            _lib.call("evox_hip_nd_environmental_selection_two_part", xa.data_ptr() if has_x else None, xa.stride(0) * es,
+                      xb.data_ptr() if has_x else None, xb.stride(0) * es, row_bytes, fa32.data_ptr(), n_a, fa32.stride(0),
+                      fa32.stride(1), fb32.data_ptr(), n_b, fb32.stride(0), fb32.stride(1), m, topk,
+                      out_x.data_ptr() if has_x else None, out_f.data_ptr(), out_rank.data_ptr(), out_dist.data_ptr(), None,
+                      ws.data_ptr(), ws.numel(), stream)
+            runtime.note_call(ws, stream)
+
+        runtime.checked(issue)
     return out_x, out_f.to(f_a.dtype), out_rank, out_dist
 
 

@@ -136,6 +136,23 @@ def note_call(ws: torch.Tensor, stream: int) -> None:
         last_status()
 
 
+# With status checking on, a ranking or selection whose device-side wait ran out (the persistent kernels need all
+# their workgroups resident at once: another kernel may hold the compute units) is issued once more through the
+# kernels that never wait for each other (tunable peel_stepped), instead of raising.
+RETRY_WITHOUT_CORESIDENCY = True
+
+
+def checked(issue) -> None:
+    """``issue()`` enqueues one library call and notes it (``note_call``)."""
+    try:
+        issue()
+    except _lib.EvoxHipError as e:
+        if e.code != _lib.E_BARRIER_TIMEOUT or not RETRY_WITHOUT_CORESIDENCY or current_option("peel_stepped", 0):
+            raise
+        with options(peel_stepped=1):
+            issue()
+
+
 def note_small_kernel_call() -> None:
     """The one-workgroup-per-population kernel has no control block and no device-side waits."""
     global _last

@@ -42,13 +42,15 @@ def test_workspace_size_and_layout(handle):
     assert handle.evox_hip_workspace_bytes(10, 0) == 0
     b = handle.evox_hip_workspace_bytes(20000, 3)
     # dominated by the bit matrix: 20000 rows x 320 words (313 rounded up to a 128-byte multiple)
-    assert 20000 * 320 * 8 <= b <= 20000 * 320 * 8 + 8 * 2**20
+    # (plus the state arrays, the buffers of the last front's sorts and those of the stepped path's ordering)
+    assert 20000 * 320 * 8 <= b <= 20000 * 320 * 8 + 12 * 2**20
     b5 = handle.evox_hip_workspace_bytes(200000, 8)
     assert 5.0e9 < b5 < 5.3e9
     # the first-front entry builds no matrix: a few arrays of n entries
     assert handle.evox_hip_first_front_workspace_bytes(0, 3) == 0
     assert 0 < handle.evox_hip_first_front_workspace_bytes(20000, 3) < 8 * 2**20
-    assert handle.evox_hip_first_front_workspace_bytes(200000, 8) == b5 - 200000 * 3136 * 8
+    # (behind the matrix lie the buffers of the stepped path's ordering of the last front: a few arrays of n * m entries)
+    assert 0 < b5 - 200000 * 3136 * 8 - handle.evox_hip_first_front_workspace_bytes(200000, 8) < 64 * 2**20
     out = (ctypes.c_int64 * 11)()
     assert handle.evox_hip_workspace_layout(20000, 3, out) == 0
     assert out[1] == 320 and out[2] == 314 and out[0] % 256 == 0 and out[9] == 0

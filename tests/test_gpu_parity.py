@@ -342,13 +342,15 @@ def test_rank_strided_and_half_inputs():
     assert np.array_equal(as_np(non_dominate_rank(h.to(DEV))), as_np(er.ranks_by_peeling(h.float())))
 
 
-@pytest.fixture(params=["lds", "witness-records", "witness-master", "sweep"])
+@pytest.fixture(params=["lds", "witness-records", "witness-master", "sweep", "stepped"])
 def peel_algorithm(request):
-    """The peeling variants: matrix rows resident in LDS (default where the matrix fits), and the three that rescan
+    """The peeling variants: matrix rows resident in LDS (default where the matrix fits), the three that rescan
     rows in memory: witness pass with the record protocol, witness pass with the master barrier and front
-    bitmaps, and the popcount-decrement sweep (master barrier)."""
+    bitmaps, and the popcount-decrement sweep (master barrier); and one launch per front by a kernel whose workgroups
+    never wait for each other (with the last front of a selection ordered likewise)."""
     with runtime.options(peel_lds=1 if request.param == "lds" else 0, peel_witness=0 if request.param == "sweep" else 1,
-                         peel_records=1 if request.param == "witness-records" else 0):
+                         peel_records=1 if request.param == "witness-records" else 0,
+                         peel_stepped=1 if request.param == "stepped" else 0):
         yield request.param
 
 

@@ -63,28 +63,13 @@ def _cases():
     return cases
 
 
-# The three ways a population of 4097 to 32768 rows can be sorted: by the one-launch kernel from its LDS lists (the
-# default), by the same kernel counting over all rows (what it does for a range that overflows its list; forced
-# here by a list of no entries, on the smaller cases: it is quadratic), and by the five kernels of the bucket sort.
-@pytest.fixture(params=["default", "counted", "bucket"])
-def sort_path(request):
-    return request.param
-
-
 @pytest.mark.parametrize("name", sorted(_cases()))
-def test_slot_sort_orders_by_key_then_index(name, sort_path):
+def test_slot_sort_orders_by_key_then_index(name):
     f_cpu = _cases()[name]
     f = f_cpu.to(DEV)
     n, m = f.shape
-    one_launch = 4097 <= n <= 32768 and n * m <= 131072
-    if sort_path != "default" and not one_launch:
-        pytest.skip("one path only for this shape")
-    if sort_path == "counted" and n > 12000:
-        pytest.skip("the quadratic way is tested on the smaller cases")
-    tunables = {"counted": {"one_sort_cap": 0}, "bucket": {"one_sort": 0}}.get(sort_path, {})
     try:
-        with runtime.options(**tunables):
-            got = _sorted_arrays(f)
+        got = _sorted_arrays(f)
     finally:
         runtime.release_workspaces()
     # ascending (key, original index); kid = first slot of the key; slot_of = the inverse table
