@@ -21,6 +21,7 @@
 #include "prefix.hpp"
 #include "radix.hpp"
 #include "stepped.hpp"
+#include "two.hpp"
 #include "wide.hpp"
 
 namespace evx {
@@ -39,6 +40,7 @@ struct Options {
   int peel_lds_blocks = 0;  // sweeping workgroups of that kernel, 0 = by size
   int peel_stepped = 0;     // 1: the fronts are peeled one launch each by kernels that never wait for each other (stepped.hpp),
                             // and the last front is ordered likewise; 0: only where the persistent grids cannot be resident
+  int64_t two_min_rows = 4097;  // populations of two objectives and at least this many rows are ranked without a matrix (two.hpp); 0 = never
   int peel_tail = 1;        // that kernel also orders a small last front (0: always the kernels of finish.hpp)
   int tail_merged = 1;      // after such a peel, ordering (where still needed) and gather share one launch
   int launch_memory = 1;    // ... unless the last selection of this shape had a last front that the peel left alone
@@ -66,7 +68,7 @@ struct Layout {
   int64_t wstride;
   // byte offsets
   size_t ctrl, fsize, fronts_slot, fronts_orig, hist, zero_end, fstart, xs, key, partials, sortparam, bstart, bcursor,
-      scanflags, tailbuf, records, members, member_key, slot_of, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, total0, witness0, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, wide, wide_bytes, dom, total;
+      scanflags, tailbuf, records, two_ring, members, member_key, slot_of, xs_sorted, key_sorted, kid_sorted, orig_of, count, witness, total0, witness0, rank, dist, perm, order, rpairs0, rpairs1, rtable, rtotals, pos, scost, dkey, wide, wide_bytes, dom, total;
 };
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
@@ -99,6 +101,8 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->scanflags = o;   o = align_up(o + sizeof(unsigned long long) * 64);
   L->tailbuf = o;     o = align_up(o + (n <= 32768 ? sizeof(unsigned long long) * kTailCopies * kTailRows : 0));
   L->records = o;     o = align_up(o + (n <= 32768 ? sizeof(unsigned long long) * kLdsPeelRecordUnits : (n <= kRecordsMaxRowsWide ? sizeof(unsigned long long) * kRecRing * kRecUnits : 0)));
+  // the hand-over rings of the two-objective ranking (two.hpp)
+  L->two_ring = o;    o = align_up(o + (m == 2 && n <= kTwoMaxRows ? sizeof(unsigned long long) * kTwoRingStride * (size_t)((n + kTwoChunk - 1) / kTwoChunk) : 0));
   L->zero_end = o;
   L->fstart = o;     o = align_up(o + sizeof(int) * (size_t)(n + 2));
   L->xs = o;         o = align_up(o + sizeof(float) * (size_t)m * L->npad);
@@ -304,11 +308,11 @@ struct Fitness {
 
 static Fitness one_part(const float* f, int64_t n, int64_t sr, int64_t sc) { return Fitness{f, sr, sc, n, f, sr, sc}; }
 
-static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStream_t s) {
+static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStream_t s, bool lexicographic = false) {
   const Layout& L = w.L;
   if (src.f == nullptr || src.f2 == nullptr || src.n_first < 0 || src.n_first > L.n) return kErrBadArg;
   const int64_t zero_words = (int64_t)((L.zero_end - L.ctrl) / 4);
-  if (with_sort && L.n <= kSmallSortRows && L.m <= kSmallSortObjectives && (int64_t)L.n * L.m <= kSmallSortValues && opt().small_sort) {
+  if (with_sort && !lexicographic && L.n <= kSmallSortRows && L.m <= kSmallSortObjectives && (int64_t)L.n * L.m <= kSmallSortValues && opt().small_sort) {
     hipLaunchKernelGGL(small_sort_kernel, dim3(L.npad / kSmallSortGroup), dim3(kSmallSortThreads), sizeof(double) * (size_t)L.npad, s, src.f,
                        src.sr, src.sc, (int)src.n_first, src.f2, src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs),
                        w.at<SortParam>(L.sortparam), w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted),
@@ -318,7 +322,7 @@ static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStr
   }
   hipLaunchKernelGGL(prepare_kernel, dim3(L.prep_blocks), dim3(256), 0, s, src.f, src.sr, src.sc, (int)src.n_first, src.f2,
                      src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs), w.at<uint64_t>(L.key),
-                     w.at<unsigned long long>(L.partials), w.at<uint32_t>(L.ctrl), zero_words);
+                     w.at<unsigned long long>(L.partials), w.at<uint32_t>(L.ctrl), zero_words, lexicographic ? 1 : 0);
   EVX_LAUNCH_CHECK();
   if (!with_sort) return 0;
   int blocks = (L.n + 255) / 256;
@@ -1075,6 +1079,9 @@ static int launch_batched(const BatchedArgs& a, int64_t batch, hipStream_t s) {
 
 using namespace evx;
 
+static bool two_applies(const Layout& L);
+static int stage_rank_two(const Ws& w, const Fitness& src, int64_t stop_count, bool fill_dist, int* rank_until, hipStream_t s);
+
 extern "C" {
 
 int evox_hip_abi_version(void) { return EVOX_HIP_ABI_VERSION; }
@@ -1131,6 +1138,8 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.launch_memory = (int)value;
   } else if (!strcmp(name, "peel_stepped") && (value == 0 || value == 1)) {
     o.peel_stepped = (int)value;
+  } else if (!strcmp(name, "two_min_rows") && value >= 0) {
+    o.two_min_rows = value;
   } else if (!strcmp(name, "peel_tail") && (value == 0 || value == 1)) {
     o.peel_tail = (int)value;
   } else if (!strcmp(name, "peel_lds_blocks") && (value == 0 || (value >= 8 && value <= 255))) {
@@ -1246,6 +1255,14 @@ int evox_hip_non_dominate_rank_until(const float* f, int64_t n, int64_t m, int64
   if (rank_out == nullptr || stop_count < 1 || stop_count > n) return kErrBadArg;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   hipStream_t s = (hipStream_t)stream;
+  if (two_applies(w.L)) {
+    int* until = stop_count < n ? w.at<int>(w.L.order) : (int*)nullptr;
+    const int e = stage_rank_two(w, one_part(f, n, sr, sc), stop_count, false, until, s);
+    if (e != kErrNotResident) {
+      if (e) return e;
+      return copy_out(w.ctrl(), rank_out, until != nullptr ? until : w.at<int>(w.L.rank), n, kPoisonIndex, s);
+    }
+  }
   if (int e = stage_prepare(w, one_part(f, n, sr, sc), true, s)) return e;
   if (int e = stage_dominance(w, kDomAuto, s)) return e;
   if (int e = count_and_peel(w, stop_count, false, false, s)) return e;
@@ -1572,6 +1589,47 @@ static size_t wide_workspace_need(int64_t n, int64_t m) {
 }
 }  // namespace evx
 
+// Two objectives without a matrix (two.hpp): the rows sorted by (f1, f2, index), the fronts as rounds of prefix
+// minima handed from workgroup to workgroup, the listing by (rank, index) from one stable argsort of the ranks.
+static bool two_applies(const Layout& L) {
+  return L.m == 2 && opt().two_min_rows > 0 && L.n >= opt().two_min_rows && L.n <= kTwoMaxRows && !opt().peel_stepped;
+}
+
+// Leaves what count_and_peel leaves: ranks by original index (of every row), the listing, the front starts and sizes
+// and the control block's description of the front that holds the stop_count-th row.  rank_until: optionally the
+// ranks with the rows behind that front unset (n ints).
+static int stage_rank_two(const Ws& w, const Fitness& src, int64_t stop_count, bool fill_dist, int* rank_until, hipStream_t s) {
+  const Layout& L = w.L;
+  if (stop_count < 1 || stop_count > L.n) return kErrBadArg;
+  WideLayout WL;
+  if (!make_wide_layout(L.n, L.m, &WL) || WL.total > L.wide_bytes) return kErrWorkspace;
+  if (int e = stage_prepare(w, src, true, s, true)) return e;
+  const int blocks = (L.n + kTwoChunk - 1) / kTwoChunk;
+  // (every workgroup waits for the one before it: resident at once on any device with as many compute units)
+  if (blocks > device_cus() * 2) return kErrNotResident;
+  const float* xs_sorted = w.at<float>(L.xs_sorted);
+  hipLaunchKernelGGL(two_peel_kernel, dim3(blocks), dim3(kTwoThreads), 0, s, xs_sorted, xs_sorted + L.npad, w.at<uint32_t>(L.kid_sorted),
+                     w.at<int>(L.orig_of), L.n, w.at<int>(L.rank), fill_dist ? w.at<float>(L.dist) : (float*)nullptr, w.ctrl(),
+                     w.at<unsigned long long>(L.two_ring), opt().spin_limit);
+  EVX_LAUNCH_CHECK();
+  int grid = (L.n + 255) / 256;
+  if (grid > device_cus() * 8) grid = device_cus() * 8;
+  hipLaunchKernelGGL(two_finish_kernel, dim3(grid), dim3(256), 0, s, w.at<uint32_t>(L.kid_sorted), w.at<int>(L.orig_of), xs_sorted,
+                     xs_sorted + L.npad, L.n, w.at<int>(L.rank), w.ctrl());
+  EVX_LAUNCH_CHECK();
+  uint8_t* wb = w.base + L.wide;
+  if (int e = evox_hip_stable_argsort_step(w.at<int>(L.rank), kKeyInt32, 1, L.n, nullptr, w.at<int>(L.perm), wb + WL.sort_ws,
+                                           WL.sort_bytes, s))
+    return e;
+  hipLaunchKernelGGL(two_bounds_kernel, dim3(grid), dim3(256), 0, s, w.at<int>(L.perm), w.at<int>(L.rank), L.n, w.at<int>(L.fstart),
+                     w.ctrl(), (int)stop_count);
+  EVX_LAUNCH_CHECK();
+  hipLaunchKernelGGL(two_sizes_kernel, dim3(grid), dim3(256), 0, s, w.at<int>(L.perm), w.at<int>(L.rank), L.n, w.at<int>(L.fstart),
+                     w.at<int>(L.fsize), w.ctrl(), rank_until);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
 // Shared body of the two selection entry points: the population is one part or two.
 static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes, const void* x2,
                        int64_t x2_row_stride_bytes, const Fitness& fit, int64_t n, int64_t m, int64_t topk, void* out_x,
@@ -1584,6 +1642,53 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   if (topk < 1 || topk > n) return kErrBadArg;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   const Layout& L = w.L;
+  if (two_applies(L)) {
+    const int e = stage_rank_two(w, fit, topk, true, nullptr, s);
+    if (e != kErrNotResident) {
+      if (e) return e;
+      // the last front by the ordering kernels, then the gather, as after a peel that leaves the last front alone
+      if (int c = stage_crowd_sort(w, w.at<int>(L.perm), false, 2, s, false)) return c;
+      if (int c = stage_crowd_finish(w, w.at<int>(L.perm), true, 2, s, false)) return c;
+      GatherArgs g2 = {};
+      int unit2 = 1;
+      if (x != nullptr) {
+        const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(x2) | reinterpret_cast<uintptr_t>(out_x) |
+                               (uintptr_t)x_row_bytes | (uintptr_t)x_row_stride_bytes | (uintptr_t)x2_row_stride_bytes;
+        unit2 = (bits % 16 == 0) ? 16 : (bits % 4 == 0) ? 4 : 1;
+      }
+      g2.order = w.at<int>(L.order);
+      g2.listed = w.at<int>(L.perm);
+      g2.topk = (int)topk;
+      g2.x = static_cast<const uint8_t*>(x);
+      g2.x_row_stride = x_row_stride_bytes;
+      g2.x_row_bytes = x_row_bytes;
+      g2.out_x = static_cast<uint8_t*>(out_x);
+      g2.unit = unit2;
+      g2.f = fit.f;
+      g2.f_stride_row = fit.sr;
+      g2.f_stride_col = fit.sc;
+      g2.n_first = (int)fit.n_first;
+      g2.x2 = static_cast<const uint8_t*>(x2);
+      g2.x2_row_stride = x2_row_stride_bytes;
+      g2.f2 = fit.f2;
+      g2.f2_stride_row = fit.sr2;
+      g2.f2_stride_col = fit.sc2;
+      g2.m = L.m;
+      g2.out_f = out_f;
+      g2.rank = w.at<int>(L.rank);
+      g2.out_rank = out_rank;
+      g2.dist = w.at<float>(L.dist);
+      g2.out_dist = out_dist;
+      g2.out_order = out_order;
+      g2.ctrl = w.ctrl();
+      int blocks = (int)((topk + 3) / 4);
+      const int cap = device_cus() * 8;
+      if (blocks > cap) blocks = cap;
+      hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(256), 0, s, g2);
+      EVX_LAUNCH_CHECK();
+      return 0;
+    }
+  }
   if (int e = stage_prepare(w, fit, true, s)) return e;
   if (int e = stage_dominance(w, kDomAuto, s)) return e;
   bool peel_orders = false;  // the peel kernel orders a small last front itself (it says so in Ctrl.tail_done)

@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
                                                       int n_first, const float* __restrict__ f2, int64_t stride_row2,
                                                       int64_t stride_col2, int n, int m, int npad, float* __restrict__ xs,
                                                       uint64_t* __restrict__ key, unsigned long long* __restrict__ partials,
-                                                      uint32_t* __restrict__ zero_words, int64_t n_zero_words) {
+                                                      uint32_t* __restrict__ zero_words, int64_t n_zero_words, int lexicographic) {
   __shared__ unsigned long long red[2][4];
   __shared__ int any_bad;
   if (threadIdx.x == 0) any_bad = 0;
@@ -77,7 +77,8 @@ __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ 
                       : i < n     ? f2[(i - n_first) * stride_row2 + k * stride_col2]
                                   : __uint_as_float(0x7FC00000u);
       xs[(int64_t)k * npad + i] = v;
-      s += (uint64_t)key_weight(k) * ordered_key(v);
+      // (two objectives ranked without a matrix, two.hpp: the rows in the order of the first objective, then the second)
+      s = lexicographic ? (s << 32) | ordered_key(v) : s + (uint64_t)key_weight(k) * ordered_key(v);
       bad |= i < n && !(fabsf(v) <= 3.4028234663852886e38f);  // NaN or infinite
     }
     key[i] = s;
