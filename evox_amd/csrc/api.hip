@@ -41,6 +41,9 @@ struct Options {
   int peel_stepped = 0;     // 1: the fronts are peeled one launch each by kernels that never wait for each other (stepped.hpp),
                             // and the last front is ordered likewise; 0: only where the persistent grids cannot be resident
   int64_t two_min_rows = 4097;  // populations of two objectives and at least this many rows are ranked without a matrix (two.hpp); 0 = never
+  int64_t two_min_rows_partial = 24576;  // ... when the ranking may stop at the front that holds a given row (that path always
+                                         // peels every front: measured, us per selection of half the rows, without / with a matrix:
+                                         // 20 000 rows 399 / 361, 50 000 rows 715 / 1181; all ranks: 5000 rows 185 / 332)
   int peel_tail = 1;        // that kernel also orders a small last front (0: always the kernels of finish.hpp)
   int tail_merged = 1;      // after such a peel, ordering (where still needed) and gather share one launch
   int launch_memory = 1;    // ... unless the last selection of this shape had a last front that the peel left alone
@@ -1079,7 +1082,7 @@ static int launch_batched(const BatchedArgs& a, int64_t batch, hipStream_t s) {
 
 using namespace evx;
 
-static bool two_applies(const Layout& L);
+static bool two_applies(const Layout& L, int64_t stop_count);
 static int stage_rank_two(const Ws& w, const Fitness& src, int64_t stop_count, bool fill_dist, int* rank_until, hipStream_t s);
 
 extern "C" {
@@ -1140,6 +1143,9 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.peel_stepped = (int)value;
   } else if (!strcmp(name, "two_min_rows") && value >= 0) {
     o.two_min_rows = value;
+    if (value < o.two_min_rows_partial) o.two_min_rows_partial = value;  // (a lower limit asked for counts for both)
+  } else if (!strcmp(name, "two_min_rows_partial") && value >= 0) {
+    o.two_min_rows_partial = value;
   } else if (!strcmp(name, "peel_tail") && (value == 0 || value == 1)) {
     o.peel_tail = (int)value;
   } else if (!strcmp(name, "peel_lds_blocks") && (value == 0 || (value >= 8 && value <= 255))) {
@@ -1255,7 +1261,7 @@ int evox_hip_non_dominate_rank_until(const float* f, int64_t n, int64_t m, int64
   if (rank_out == nullptr || stop_count < 1 || stop_count > n) return kErrBadArg;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   hipStream_t s = (hipStream_t)stream;
-  if (two_applies(w.L)) {
+  if (two_applies(w.L, stop_count)) {
     int* until = stop_count < n ? w.at<int>(w.L.order) : (int*)nullptr;
     const int e = stage_rank_two(w, one_part(f, n, sr, sc), stop_count, false, until, s);
     if (e != kErrNotResident) {
@@ -1591,8 +1597,9 @@ static size_t wide_workspace_need(int64_t n, int64_t m) {
 
 // Two objectives without a matrix (two.hpp): the rows sorted by (f1, f2, index), the fronts as rounds of prefix
 // minima handed from workgroup to workgroup, the listing by (rank, index) from one stable argsort of the ranks.
-static bool two_applies(const Layout& L) {
-  return L.m == 2 && opt().two_min_rows > 0 && L.n >= opt().two_min_rows && L.n <= kTwoMaxRows && !opt().peel_stepped;
+static bool two_applies(const Layout& L, int64_t stop_count) {
+  const int64_t least = stop_count >= L.n ? opt().two_min_rows : (opt().two_min_rows_partial > opt().two_min_rows ? opt().two_min_rows_partial : opt().two_min_rows);
+  return L.m == 2 && opt().two_min_rows > 0 && L.n >= least && L.n <= kTwoMaxRows && !opt().peel_stepped;
 }
 
 // Leaves what count_and_peel leaves: ranks by original index (of every row), the listing, the front starts and sizes
@@ -1642,7 +1649,7 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   if (topk < 1 || topk > n) return kErrBadArg;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   const Layout& L = w.L;
-  if (two_applies(L)) {
+  if (two_applies(L, topk)) {
     const int e = stage_rank_two(w, fit, topk, true, nullptr, s);
     if (e != kErrNotResident) {
       if (e) return e;

@@ -24,6 +24,8 @@
 
 namespace evx {
 
+// (256 threads x 16 slots, one wave per SIMD, was slower: 1.5 against 0.75 us per round -- the running minimum over a
+// thread's own slots is a chain of dependent instructions that no other wave hides.)
 constexpr int kTwoThreads = 1024;
 constexpr int kTwoPerThread = 4;                             // consecutive slots per thread
 constexpr int kTwoChunk = kTwoThreads * kTwoPerThread;       // slots per workgroup
@@ -56,8 +58,9 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
                                                                int n, int* __restrict__ rank, float* __restrict__ dist_fill,
                                                                Ctrl* __restrict__ ctrl, unsigned long long* __restrict__ ring,
                                                                unsigned spin_limit) {
-  __shared__ uint32_t wave_min_lds[2][kTwoThreads / 64];  // by the parity of the round: a wave may be a round ahead of another's reads
+  __shared__ __attribute__((aligned(16))) uint32_t wave_min_lds[2][kTwoThreads / 64];  // by the parity of the round: a wave may be a round ahead of another's reads
   __shared__ uint32_t in_lds[2];  // the round's incoming minimum; 1 when the workgroup leaves after this round's hand-over
+  __shared__ uint32_t before_lds[kTwoThreads / 64];  // the minimum over the waves before each wave
   __shared__ int ranked_lds;      // rows this workgroup ranked in the round
   if (coherent_load(&ctrl->err) != 0) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -101,6 +104,13 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
     for (int w = 0; w < kTwoThreads / 64; ++w) left += (int)wave_min_lds[1][w];
   __syncthreads();
   bool upstream_ended = b == 0;
+  // (thread 0) the words of the next two rounds are asked for ahead of time: the workgroup before is usually a round
+  // or more ahead, so that a round finds its word there and pays no memory round trip
+  unsigned long long ahead[2] = {0ull, 0ull};
+  if (tid == 0 && !upstream_ended) {
+    ahead[0] = coherent_load(up_ring + 0);
+    ahead[1] = coherent_load(up_ring + (1 % kTwoRing));
+  }
   for (int round = 0;; ++round) {
     const unsigned tag = (unsigned)round + 1u;
     // ---- the minimum of this workgroup's remaining rows
@@ -110,31 +120,45 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
     const uint32_t incl = wave_prefix_min(tmin);
     uint32_t* const wave_min = wave_min_lds[round & 1];
     if (lane == 63) wave_min[wave] = incl;
+    EVX_TRACE(round, 0);
     lds_barrier();
+    EVX_TRACE(round, 1);
+    // the first wave turns the wave minima into what stands before every wave (a prefix minimum over sixteen lanes
+    // of a DPP row) and the minimum of the workgroup
+    uint32_t local = kTwoNone;
+    if (wave == 0) {
+      const uint32_t mine = lane < kTwoThreads / 64 ? wave_min[lane] : kTwoNone;
+      const uint32_t upto = wave_prefix_min(mine);
+      const uint32_t before_wave = (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)upto, 0x138, 0xf, 0xf, false);  // wave_shr:1
+      if (lane < kTwoThreads / 64) before_lds[lane] = before_wave;
+      local = (uint32_t)__builtin_amdgcn_readlane((int)upto, kTwoThreads / 64 - 1);
+    }
     if (tid == 0) {
       left -= ranked_lds;  // what the round before has ranked
       ranked_lds = 0;
-      uint32_t local = kTwoNone;
-      for (int w = 0; w < kTwoThreads / 64; ++w) local = min(local, wave_min[w]);
       // ---- the incoming minimum of the round
       uint32_t in = kTwoNone;
       bool failed = false;
       if (!upstream_ended) {
         const unsigned long long* slot = up_ring + (round % kTwoRing);
-        unsigned long long word = 0;
-        WaitBound bound(spin_limit);
-        for (unsigned spins = 0;; ++spins) {
-          word = coherent_load(slot);
-          if (((unsigned)(word >> 32) & ~kTwoEnd) == tag) break;
-          if (bound.expired(spins) || ((spins & 63u) == 63u && coherent_load(&ctrl->err) != 0)) {
-            failed = true;
-            break;
+        unsigned long long word = ahead[0];
+        ahead[0] = ahead[1];
+        if (((unsigned)(word >> 32) & ~kTwoEnd) != tag) {
+          WaitBound bound(spin_limit);
+          for (unsigned spins = 0;; ++spins) {
+            word = coherent_load(slot);
+            if (((unsigned)(word >> 32) & ~kTwoEnd) == tag) break;
+            if (bound.expired(spins) || ((spins & 63u) == 63u && coherent_load(&ctrl->err) != 0)) {
+              failed = true;
+              break;
+            }
           }
         }
         if (!failed) {
           in = (uint32_t)word;
           if ((unsigned)(word >> 32) & kTwoEnd) upstream_ended = true;  // nothing remains before this workgroup, from this round on
           coherent_store(my_progress, round + 1);
+          if (!upstream_ended) ahead[1] = coherent_load(up_ring + ((round + 2) % kTwoRing));
         }
       }
       // ---- hand on at once: the minimum over the remaining rows up to the end of this workgroup's run.  The stream
@@ -157,11 +181,12 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
       in_lds[0] = in;
       in_lds[1] = failed || ends_here ? 1u : 0u;
     }
+    EVX_TRACE(round, 2);
     lds_barrier();
+    EVX_TRACE(round, 3);
     if (in_lds[1] != 0u) break;  // nothing is left here and before, or a wait ran out
     // ---- exclusive prefix minimum over the remaining rows before each slot, seeded with the incoming one
-    uint32_t before = in_lds[0];
-    for (int w = 0; w < wave; ++w) before = min(before, wave_min[w]);
+    uint32_t before = min(in_lds[0], before_lds[wave]);
     {
       const uint32_t shifted = (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)incl, 0x138, 0xf, 0xf, false);  // wave_shr:1
       before = min(before, shifted);
@@ -177,8 +202,7 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
       }
       before = min(before, mine);
     }
-    ranked = wave_sum(ranked);
-    if (lane == 0 && ranked) atomicAdd(&ranked_lds, ranked);
+    if (ranked) atomicAdd(&ranked_lds, ranked);  // (few threads rank a row in any one round)
     // (the barrier at the head of the next round also closes this round's counting)
   }
 }

@@ -84,7 +84,9 @@ def test_two_objective_populations_against_the_checker(name):
     topk = n // 2
     order, rank, dist, _ = c_oracle.select(f.numpy(), topk)
     x = torch.arange(n, dtype=torch.int32)[:, None]
-    sel = nd_environmental_selection(x.to(DEV), fd, topk)
+    with runtime.options(two_min_rows=1):  # (by default a selection of fewer than 24 576 rows takes the matrix)
+        sel = nd_environmental_selection(x.to(DEV), fd, topk)
+        until = as_np(non_dominate_rank_until(fd, topk + 1))
     assert np.array_equal(as_np(sel[2]), rank[order]), name
     gd, wd = as_np(sel[3]), dist[order]
     fin = np.isfinite(wd)
@@ -93,7 +95,6 @@ def test_two_objective_populations_against_the_checker(name):
     if not np.array_equal(as_np(sel[0])[:, 0], order):
         # rows may only change places where their distances tie within rounding at the cut
         assert sorted(as_np(sel[0])[:, 0].tolist()) == sorted(order.tolist()) or np.allclose(np.sort(gd[fin]), np.sort(wd[fin]), rtol=1e-5), name
-    until = as_np(non_dominate_rank_until(fd, topk + 1))
     worst = np.sort(want)[topk]
     assert np.array_equal(until, np.where(want <= worst, want, 2**31 - 1)), name
 
@@ -103,7 +104,8 @@ def test_two_objectives_in_two_parts_and_with_strides():
     f = (torch.rand(12000, 2, generator=g) * 500).round() / 500
     x = torch.rand(12000, 5, generator=g)
     want = er.environmental_selection(x, f, 5000)
-    got = nd_environmental_selection_two_part(x[:7000].to(DEV), f[:7000].to(DEV), x[7000:].to(DEV), f[7000:].to(DEV), 5000)
+    with runtime.options(two_min_rows=1):
+        got = nd_environmental_selection_two_part(x[:7000].to(DEV), f[:7000].to(DEV), x[7000:].to(DEV), f[7000:].to(DEV), 5000)
     for a, b in zip(got[:3], want[:3]):
         assert torch.equal(a.cpu(), b)
     wide = torch.zeros(12000, 5)
