@@ -152,6 +152,10 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
 struct Ws {
   Layout L;
   uint8_t* base;
+  // several populations of one shape in the same launches (blockIdx.z): `step` bytes from the workspace of one to that
+  // of the next, all laid out alike; 1 and 0 for a single population
+  int batch = 1;
+  int64_t step = 0;
   template <class T>
   T* at(size_t off) const {
     return reinterpret_cast<T*>(base + off);
@@ -229,19 +233,25 @@ static int* outcome_slot(int64_t n, int64_t m, bool may_allocate, hipStream_t s)
 template <int M, int IW>
 static void launch_dominance_m(const Ws& w, int variant, hipStream_t s) {
   const Layout& L = w.L;
-  dim3 grid((L.npad + 255) / 256, (L.nwords + IW - 1) / IW);
-  if (IW == 2) grid = dim3((L.npad + 127) / 128, (L.nwords + 3) / 4);  // a block = two row groups x two tiles
+  dim3 grid((L.npad + 255) / 256, (L.nwords + IW - 1) / IW, w.batch);
+  if (IW == 2) grid = dim3((L.npad + 127) / 128, (L.nwords + 3) / 4, w.batch);  // a block = two row groups x two tiles
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, w.at<float>(L.xs_sorted), w.at<uint64_t>(L.key_sorted),
                        w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords,
-                       w.at<SortParam>(L.sortparam));
+                       w.at<SortParam>(L.sortparam), w.step);
   };
   if ((IW == 2 || IW == 4) && variant == kDomAuto && opt().dominance_folded) {
     const int row_blocks = IW == 2 ? (L.npad + 127) / 128 : (L.npad + 255) / 256;
     const int column = IW == 2 ? (row_blocks - 1) / 2 + 2 : row_blocks + 1;
-    hipLaunchKernelGGL((dominance_folded_kernel<M, (IW == 2 ? 2 : 4)>), dim3((row_blocks + 1) / 2, column), dim3(256), 0, s,
-                       w.at<float>(L.xs_sorted), w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted),
-                       w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords, w.at<SortParam>(L.sortparam), row_blocks);
+    auto folded = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, dim3((row_blocks + 1) / 2, column, w.batch), dim3(256), 0, s, w.at<float>(L.xs_sorted),
+                         w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride,
+                         L.nwords, w.at<SortParam>(L.sortparam), row_blocks, w.step);
+    };
+    if (w.batch > 1)
+      folded(dominance_folded_kernel<M, (IW == 2 ? 2 : 4), true>);
+    else
+      folded(dominance_folded_kernel<M, (IW == 2 ? 2 : 4), false>);
     return;
   }
   switch (variant) {
@@ -269,9 +279,9 @@ static void launch_dominance(const Ws& w, int variant, hipStream_t s) {
       // on the device); the other tile sizes and the check variants, and more objectives, take the generic kernel
       if (IW == 4 && variant == kDomAuto && L.m <= 16) {
         auto wide = [&](auto kernel) {
-          hipLaunchKernelGGL(kernel, dim3((L.npad + 255) / 256, (L.nwords + 3) / 4), dim3(256), 0, s, w.at<float>(L.xs_sorted),
+          hipLaunchKernelGGL(kernel, dim3((L.npad + 255) / 256, (L.nwords + 3) / 4, w.batch), dim3(256), 0, s, w.at<float>(L.xs_sorted),
                              w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad,
-                             L.wstride, L.nwords, w.at<SortParam>(L.sortparam));
+                             L.wstride, L.nwords, w.at<SortParam>(L.sortparam), w.step);
         };
         switch (L.m) {
           case 9: wide(dominance_kernel<9, 4, kDomAuto>); return;
@@ -284,9 +294,9 @@ static void launch_dominance(const Ws& w, int variant, hipStream_t s) {
           default: wide(dominance_kernel<16, 4, kDomAuto>); return;
         }
       }
-      dim3 grid((L.npad + 255) / 256, (L.nwords + IW - 1) / IW);
+      dim3 grid((L.npad + 255) / 256, (L.nwords + IW - 1) / IW, w.batch);
       hipLaunchKernelGGL((dominance_any_m_kernel<IW>), grid, dim3(256), 0, s, w.at<float>(L.xs_sorted),
-                         w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords, L.m);
+                         w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride, L.nwords, L.m, w.step);
     }
   }
 }
@@ -307,46 +317,92 @@ struct Fitness {
   int64_t n_first;
   const float* f2;
   int64_t sr2, sc2;
+  int64_t step = 0, step2 = 0;  // several populations: elements from one population's fitness to the next one's
 };
 
-static Fitness one_part(const float* f, int64_t n, int64_t sr, int64_t sc) { return Fitness{f, sr, sc, n, f, sr, sc}; }
+static Fitness one_part(const float* f, int64_t n, int64_t sr, int64_t sc, int64_t step = 0) {
+  return Fitness{f, sr, sc, n, f, sr, sc, step, step};
+}
 
 static int stage_prepare(const Ws& w, const Fitness& src, bool with_sort, hipStream_t s, bool lexicographic = false) {
   const Layout& L = w.L;
   if (src.f == nullptr || src.f2 == nullptr || src.n_first < 0 || src.n_first > L.n) return kErrBadArg;
   const int64_t zero_words = (int64_t)((L.zero_end - L.ctrl) / 4);
-  if (with_sort && !lexicographic && L.n <= kSmallSortRows && L.m <= kSmallSortObjectives && (int64_t)L.n * L.m <= kSmallSortValues && opt().small_sort) {
-    hipLaunchKernelGGL(small_sort_kernel, dim3(L.npad / kSmallSortGroup), dim3(kSmallSortThreads), sizeof(double) * (size_t)L.npad, s, src.f,
-                       src.sr, src.sc, (int)src.n_first, src.f2, src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs),
-                       w.at<SortParam>(L.sortparam), w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted),
-                       w.at<float>(L.xs_sorted), w.at<int>(L.orig_of), w.at<uint32_t>(L.ctrl), zero_words);
+  // (every workgroup of small_sort_kernel reads its whole population to place sixteen rows: with several populations
+  // in the launch, more workgroups than the device holds at once take turns -- 16 x 4096 rows: 102 us against 10 for
+  // one population, the five launches of the bucket sort 30)
+  const bool many = w.batch > 1;
+  const bool small_sort_pays = w.batch == 1 || (int64_t)w.batch * (L.npad / kSmallSortGroup) <= 2 * device_cus();
+  if (with_sort && !lexicographic && L.n <= kSmallSortRows && L.m <= kSmallSortObjectives && (int64_t)L.n * L.m <= kSmallSortValues &&
+      opt().small_sort && small_sort_pays) {
+    auto launch = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, dim3(L.npad / kSmallSortGroup, 1, w.batch), dim3(kSmallSortThreads), sizeof(double) * (size_t)L.npad, s, src.f,
+                         src.sr, src.sc, (int)src.n_first, src.f2, src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs),
+                         w.at<SortParam>(L.sortparam), w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted),
+                         w.at<float>(L.xs_sorted), w.at<int>(L.orig_of), w.at<uint32_t>(L.ctrl), zero_words, src.step, src.step2, w.step);
+    };
+    if (many)
+      launch(small_sort_kernel<true>);
+    else
+      launch(small_sort_kernel<false>);
     EVX_LAUNCH_CHECK();
     return 0;
   }
-  hipLaunchKernelGGL(prepare_kernel, dim3(L.prep_blocks), dim3(256), 0, s, src.f, src.sr, src.sc, (int)src.n_first, src.f2,
-                     src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs), w.at<uint64_t>(L.key),
-                     w.at<unsigned long long>(L.partials), w.at<uint32_t>(L.ctrl), zero_words, lexicographic ? 1 : 0);
+  auto launch_prepare = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(L.prep_blocks, 1, w.batch), dim3(256), 0, s, src.f, src.sr, src.sc, (int)src.n_first, src.f2,
+                       src.sr2, src.sc2, L.n, L.m, L.npad, w.at<float>(L.xs), w.at<uint64_t>(L.key),
+                       w.at<unsigned long long>(L.partials), w.at<uint32_t>(L.ctrl), zero_words, lexicographic ? 1 : 0, src.step,
+                       src.step2, w.step);
+  };
+  if (many)
+    launch_prepare(prepare_kernel<true>);
+  else
+    launch_prepare(prepare_kernel<false>);
   EVX_LAUNCH_CHECK();
   if (!with_sort) return 0;
   int blocks = (L.n + 255) / 256;
   if (blocks > 2048) blocks = 2048;
-  hipLaunchKernelGGL(bucket_hist_kernel, dim3(blocks), dim3(256), 0, s, w.at<uint64_t>(L.key), L.n,
-                     w.at<unsigned long long>(L.partials), L.prep_blocks, L.buckets, w.at<int>(L.hist),
-                     w.at<SortParam>(L.sortparam));
+  auto launch_hist = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(blocks, 1, w.batch), dim3(256), 0, s, w.at<uint64_t>(L.key), L.n,
+                       w.at<unsigned long long>(L.partials), L.prep_blocks, L.buckets, w.at<int>(L.hist),
+                       w.at<SortParam>(L.sortparam), w.step);
+  };
+  if (many)
+    launch_hist(bucket_hist_kernel<true>);
+  else
+    launch_hist(bucket_hist_kernel<false>);
   EVX_LAUNCH_CHECK();
-  hipLaunchKernelGGL(bucket_scan_kernel, dim3(L.buckets / 1024), dim3(256), 0, s, w.at<int>(L.hist), L.buckets,
-                     w.at<int>(L.bstart), w.at<int>(L.bcursor), w.at<unsigned long long>(L.scanflags), w.ctrl());
+  auto launch_scan = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(L.buckets / 1024, 1, w.batch), dim3(256), 0, s, w.at<int>(L.hist), L.buckets,
+                       w.at<int>(L.bstart), w.at<int>(L.bcursor), w.at<unsigned long long>(L.scanflags), w.ctrl(), w.step);
+  };
+  if (many)
+    launch_scan(bucket_scan_kernel<true>);
+  else
+    launch_scan(bucket_scan_kernel<false>);
   EVX_LAUNCH_CHECK();
-  hipLaunchKernelGGL(bucket_scatter_kernel, dim3(blocks), dim3(256), 0, s, w.at<uint64_t>(L.key), L.n,
-                     w.at<SortParam>(L.sortparam), w.at<int>(L.bcursor), w.at<int>(L.members), w.at<uint64_t>(L.member_key),
-                     w.ctrl());
+  auto launch_scatter = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(blocks, 1, w.batch), dim3(256), 0, s, w.at<uint64_t>(L.key), L.n,
+                       w.at<SortParam>(L.sortparam), w.at<int>(L.bcursor), w.at<int>(L.members), w.at<uint64_t>(L.member_key),
+                       w.ctrl(), w.step);
+  };
+  if (many)
+    launch_scatter(bucket_scatter_kernel<true>);
+  else
+    launch_scatter(bucket_scatter_kernel<false>);
   EVX_LAUNCH_CHECK();
   int pblocks = (L.npad + 255) / 256;
   if (pblocks > 2048) pblocks = 2048;
-  hipLaunchKernelGGL(bucket_place_kernel, dim3(pblocks), dim3(256), 0, s, w.at<float>(L.xs), L.n, L.m,
-                     L.npad, w.at<SortParam>(L.sortparam), w.at<int>(L.bstart), w.at<int>(L.members), w.at<uint64_t>(L.member_key),
-                     w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of), w.at<int>(L.slot_of),
-                     w.ctrl());
+  auto launch_place = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(pblocks, 1, w.batch), dim3(256), 0, s, w.at<float>(L.xs), L.n, L.m,
+                       L.npad, w.at<SortParam>(L.sortparam), w.at<int>(L.bstart), w.at<int>(L.members), w.at<uint64_t>(L.member_key),
+                       w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<float>(L.xs_sorted), w.at<int>(L.orig_of), w.at<int>(L.slot_of),
+                       w.ctrl(), w.step);
+  };
+  if (many)
+    launch_place(bucket_place_kernel<true>);
+  else
+    launch_place(bucket_place_kernel<false>);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -384,7 +440,8 @@ static int stage_dominance(const Ws& w, int variant, hipStream_t s) {
   // (kDomOrdersOnly: the first half of the path below alone, for measurements of the second)
   if (variant == kDomOrdersOnly) return prefix_dominance_applies(w.L) ? stage_dominance_prefix(w, true, s) : kErrBadArg;
   // (the orders of that path come from kernels whose workgroups wait for each other: not with the stepped path)
-  if (variant == kDomAuto && prefix_dominance_applies(w.L) && !opt().peel_stepped) return stage_dominance_prefix(w, false, s);
+  // (nor for several populations in one launch: those orders come from a grid that fills the device)
+  if (variant == kDomAuto && prefix_dominance_applies(w.L) && !opt().peel_stepped && w.batch == 1) return stage_dominance_prefix(w, false, s);
   // (the lower triangle in tiles of 4 words keeps every SIMD busy with several waves; up to about 24 000 rows of
   // two to eight objectives tiles of 2 words leave a shorter half-empty tail -- measured, us, tiles of 2 / 4:
   // 5000 x 3: 5.8 / 7.9, 16 000 x 3: 20.3 / 25.7, 20 000 x 2: 20.6 / 23.1, x 3: 27.6 / 31.3, x 8: 64.3 / 80.8,
@@ -481,8 +538,68 @@ static int grant_dynamic_lds(const void* kernel, size_t lds) {
 // Sweeping workgroups of the LDS-resident peel for this population and the dynamic LDS each needs; 0 when the
 // population does not fit (or the option is off).  Every workgroup takes a compute unit of its own.
 constexpr size_t kLdsPeelBudget = 160 * 1024 - 512;
-static int lds_peel_plan(const Layout& L, size_t* lds_out) {
+
+// Workgroups of peel_lds_kernel that a compute unit holds at once when each has `lds` bytes of dynamic LDS (asked of
+// the runtime once per device and 8 KB step of the size, for the upper end of the step); 0 when the query fails.
+static int lds_peel_per_cu(size_t lds) {
+  static std::atomic<int> cache[64][24];  // 0 unknown, else the answer + 1
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || lds > kLdsPeelBudget) return 0;
+  const int slot = (int)((lds + 8191) / 8192);
+  int known = cache[dev][slot].load(std::memory_order_acquire);
+  if (known == 0) {
+    // (the attribute belongs to the (kernel, device) pair)
+    // (both instances of the kernel: the one for several populations only moves its pointers first)
+    int per_cu = 1 << 30;
+    const size_t upper = (size_t)slot * 8192 < kLdsPeelBudget ? (size_t)slot * 8192 : kLdsPeelBudget;
+    for (const void* kernel : {reinterpret_cast<const void*>(peel_lds_kernel<false>), reinterpret_cast<const void*>(peel_lds_kernel<true>)}) {
+      if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPeelBudget) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+      }
+      int one = 0;
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&one, kernel, kLdsPeelThreads, upper) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+      }
+      if (one < per_cu) per_cu = one;
+    }
+    known = per_cu + 1;
+    cache[dev][slot].store(known, std::memory_order_release);
+  }
+  return known - 1;
+}
+
+// batch > 1: that many populations share the launch, each with this many sweeping workgroups (and its lister); up to
+// four workgroups then share a compute unit where their LDS allows it, and the plan is the one with the most
+// sweeping workgroups per population.
+static int lds_peel_plan(const Layout& L, size_t* lds_out, int batch = 1) {
   if (!opt().peel_lds || L.n > 32768 || L.nwords > kLdsPeelThreads) return 0;  // (the lister keeps original indices in 16 bits and takes a bitmap word per thread)
+  if (batch > 1) {
+    size_t tail_need = opt().peel_tail ? peel_tail_lds_bytes(L.n, L.m) : 0;  // (a small last front is ordered in the kernel's LDS)
+    if (tail_need > kLdsPeelBudget) tail_need = 0;
+    int wanted = opt().peel_lds_blocks;
+    if (wanted == 0) wanted = L.n / 64 < 32 ? 32 : L.n / 64;
+    int best = 0;
+    for (int per_cu = 1; per_cu <= 4; ++per_cu) {
+      const int64_t share = (int64_t)per_cu * device_cus() / batch - 1;
+      const int most = share < 255 ? (int)share : 255;
+      if (most < 8) continue;
+      const size_t limit = (size_t)160 * 1024 / per_cu - 1024;
+      auto fits = [&](int sweepers) {
+        const size_t b = lds_peel_bytes(L.n, L.nwords, sweepers);
+        return b != 0 && b <= limit;
+      };
+      int sweepers = wanted < most ? wanted : most;
+      while (sweepers < most && !fits(sweepers)) sweepers = sweepers + 8 < most ? sweepers + 8 : most;
+      if (!fits(sweepers) || tail_need > limit || sweepers <= best) continue;
+      const size_t lds = lds_peel_bytes(L.n, L.nwords, sweepers);
+      if (lds_peel_per_cu(lds > tail_need ? lds : tail_need) < per_cu) continue;
+      best = sweepers;
+      *lds_out = lds;
+    }
+    return best;
+  }
   const int most = device_cus() - 1 < 255 ? device_cus() - 1 : 255;  // + the lister; a record holds at least 4 units
   if (most < 8) return 0;
   auto fits = [&](int sweepers) {
@@ -521,28 +638,19 @@ static int launch_lds_peel(const Ws& w, int64_t stop_count, bool want_perm, bool
       if (lds < need) lds = need;
     }
   }
-  // the attribute belongs to the (kernel, device) pair; every workgroup waits for every other one, so the grid
-  // must be resident at once: checked once per device for the largest LDS size
-  static std::atomic<int> resident[64];  // 0 unknown, else workgroups per compute unit + 1
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return kErrBadArg;
-  int known = resident[dev].load(std::memory_order_acquire);
-  if (known == 0) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(peel_lds_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)kLdsPeelBudget);
-    if (e != hipSuccess) return (int)e;
-    int per_cu = 0;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, peel_lds_kernel, kLdsPeelThreads, kLdsPeelBudget);
-    if (e != hipSuccess) return (int)e;
-    known = per_cu + 1;
-    resident[dev].store(known, std::memory_order_release);
-  }
-  if ((int64_t)(known - 1) * device_cus() < sweepers + 1) return kErrNotResident;
-  hipLaunchKernelGGL(peel_lds_kernel, dim3(sweepers + 1), dim3(kLdsPeelThreads), lds, s, w.at<uint64_t>(L.dom), L.wstride, L.nwords, L.n,
-                     w.at<int>(L.orig_of), w.at<int>(L.rank), fill_dist ? w.at<float>(L.dist) : (float*)nullptr,
-                     w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
-                     want_perm ? w.at<int>(L.perm) : (int*)nullptr, w.at<int>(L.fstart), w.ctrl(), (int)stop_count, opt().spin_limit,
-                     w.at<unsigned long long>(L.records), sweepers, tail);
+  // every workgroup waits for every other one, so the grid must be resident at once
+  if ((int64_t)lds_peel_per_cu(lds) * device_cus() < (int64_t)(sweepers + 1) * w.batch) return kErrNotResident;
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(sweepers + 1, 1, w.batch), dim3(kLdsPeelThreads), lds, s, w.at<uint64_t>(L.dom), L.wstride, L.nwords, L.n,
+                       w.at<int>(L.orig_of), w.at<int>(L.rank), fill_dist ? w.at<float>(L.dist) : (float*)nullptr,
+                       w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
+                       want_perm ? w.at<int>(L.perm) : (int*)nullptr, w.at<int>(L.fstart), w.ctrl(), (int)stop_count, opt().spin_limit,
+                       w.at<unsigned long long>(L.records), sweepers, tail, w.step);
+  };
+  if (w.batch > 1)
+    launch(peel_lds_kernel<true>);
+  else
+    launch(peel_lds_kernel<false>);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -577,7 +685,7 @@ static int count_and_peel_persistent(const Ws& w, int64_t stop_count, bool want_
   size_t lds = 0;
   if (may_have_ordered) *may_have_ordered = false;
   if (always_orders) *always_orders = false;
-  if (const int sweepers = lds_peel_plan(w.L, &lds)) {
+  if (const int sweepers = lds_peel_plan(w.L, &lds, w.batch)) {
     const bool may = order_last_front && opt().peel_tail && peel_tail_lds_bytes(w.L.n, w.L.m) != 0 &&
                      peel_tail_lds_bytes(w.L.n, w.L.m) <= kLdsPeelBudget;
     if (may_have_ordered) *may_have_ordered = may;
@@ -593,6 +701,7 @@ static int count_and_peel_persistent(const Ws& w, int64_t stop_count, bool want_
     }
     return launch_lds_peel(w, stop_count, want_perm, fill_dist, sweepers, lds, s, order_last_front);
   }
+  if (w.batch > 1) return kErrNotResident;  // (the kernels below take one population per launch)
   // (the witness passes read of a row only its highest dominator: the count stage then walks every row from the top
   // as far as that, instead of adding up all of it)
   int blocks = 0, use_witness = 0;
@@ -766,6 +875,14 @@ static int finish_grid(const Layout& L, int per_candidate_block) {
   return blocks < 1 ? 1 : blocks;
 }
 
+// The grid of one population when `batch` of them share a launch whose workgroups may wait for each other: the device
+// holds `resident` such workgroups at once.
+static int shared_grid(int grid, int resident, int batch) {
+  if (batch <= 1) return grid;
+  const int cap = resident / batch < 1 ? 1 : resident / batch;
+  return grid < cap ? grid : cap;
+}
+
 template <int M>
 static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
   constexpr int WW = M <= kPrefixWideObjectives ? 8 : 4;  // words per tile: what the LDS holds tables for
@@ -900,6 +1017,7 @@ static CrowdArgs crowd_args(const Ws& w, const int* list, bool use_orders, int f
   a.dist = w.at<float>(L.dist);
   a.dkey = w.at<uint32_t>(L.dkey);
   a.order = w.at<int>(L.order);
+  a.ws_step = w.step;
   return a;
 }
 
@@ -935,7 +1053,7 @@ static size_t crowd_lds_bytes(const Layout& L, int fused) {
 
 static int stage_crowd_sort(const Ws& w, const int* list, bool use_orders, int fused, hipStream_t s, bool after_peel_tail = false) {
   const Layout& L = w.L;
-  use_orders = use_orders && prefix_dominance_applies(L);
+  use_orders = use_orders && prefix_dominance_applies(L) && w.batch == 1;
   // a large front of a population whose matrix came from the per-objective orders: its own orders are read off
   // those (finish.hpp); the three kernels and the one below choose on the device which of them has work
   if (use_orders)
@@ -952,23 +1070,31 @@ static int stage_crowd_sort(const Ws& w, const int* list, bool use_orders, int f
   const size_t lds = crowd_lds_bytes(L, fused);
   const bool mid = crowd_mid_sort(L);
   const bool wide = L.n <= kMidArgsortWideRows;  // (which tables of the LDS sorter the population leaves room for)
-  const void* const kernel = !mid ? reinterpret_cast<const void*>(crowd_sort_kernel<kRadixThreads, 0>)
-                             : wide ? reinterpret_cast<const void*>(crowd_sort_kernel<kMidArgsortThreads, 1>)
-                                    : reinterpret_cast<const void*>(crowd_sort_kernel<kMidArgsortThreads, 2>);
+  const bool many = w.batch > 1;
+  auto instance = [&](auto one, auto several) { return many ? reinterpret_cast<const void*>(several) : reinterpret_cast<const void*>(one); };
+  const void* const kernel = !mid   ? instance(crowd_sort_kernel<kRadixThreads, 0, false>, crowd_sort_kernel<kRadixThreads, 0, true>)
+                             : wide ? instance(crowd_sort_kernel<kMidArgsortThreads, 1, false>, crowd_sort_kernel<kMidArgsortThreads, 1, true>)
+                                    : instance(crowd_sort_kernel<kMidArgsortThreads, 2, false>, crowd_sort_kernel<kMidArgsortThreads, 2, true>);
   if (int e = grant_dynamic_lds(kernel, lds)) return e;
   // (the fused path ends with a barrier between all blocks: the grid must be resident at once, which a grid of at
   // most two blocks of 256 threads per compute unit is)
   int grid = finish_grid(L, L.m);
   if (fused != 0 && grid > device_cus() * 2) grid = device_cus() * 2;
-  if (mid && wide)
-    hipLaunchKernelGGL((crowd_sort_kernel<kMidArgsortThreads, 1>), dim3(grid), dim3(kMidArgsortThreads), lds, s,
-                       crowd_args(w, list, use_orders, fused), after_peel_tail ? 1 : 0);
+  grid = shared_grid(grid, mid ? device_cus() : device_cus() * 2, w.batch);
+  const CrowdArgs ca = crowd_args(w, list, use_orders, fused);
+  const int tail_flag = after_peel_tail ? 1 : 0;
+  if (mid && wide && many)
+    hipLaunchKernelGGL((crowd_sort_kernel<kMidArgsortThreads, 1, true>), dim3(grid, 1, w.batch), dim3(kMidArgsortThreads), lds, s, ca, tail_flag);
+  else if (mid && wide)
+    hipLaunchKernelGGL((crowd_sort_kernel<kMidArgsortThreads, 1, false>), dim3(grid), dim3(kMidArgsortThreads), lds, s, ca, tail_flag);
+  else if (mid && many)
+    hipLaunchKernelGGL((crowd_sort_kernel<kMidArgsortThreads, 2, true>), dim3(grid, 1, w.batch), dim3(kMidArgsortThreads), lds, s, ca, tail_flag);
   else if (mid)
-    hipLaunchKernelGGL((crowd_sort_kernel<kMidArgsortThreads, 2>), dim3(grid), dim3(kMidArgsortThreads), lds, s,
-                       crowd_args(w, list, use_orders, fused), after_peel_tail ? 1 : 0);
+    hipLaunchKernelGGL((crowd_sort_kernel<kMidArgsortThreads, 2, false>), dim3(grid), dim3(kMidArgsortThreads), lds, s, ca, tail_flag);
+  else if (many)
+    hipLaunchKernelGGL((crowd_sort_kernel<kRadixThreads, 0, true>), dim3(grid, 1, w.batch), dim3(kRadixThreads), lds, s, ca, tail_flag);
   else
-    hipLaunchKernelGGL((crowd_sort_kernel<kRadixThreads, 0>), dim3(grid), dim3(kRadixThreads), lds, s,
-                       crowd_args(w, list, use_orders, fused), after_peel_tail ? 1 : 0);
+    hipLaunchKernelGGL((crowd_sort_kernel<kRadixThreads, 0, false>), dim3(grid), dim3(kRadixThreads), lds, s, ca, tail_flag);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -990,31 +1116,40 @@ static int stage_crowd_finish(const Ws& w, const int* list, bool want_order, int
   const size_t lds = crowd_lds_bytes(L, 0);
   const bool mid = crowd_mid_sort(L);
   const bool wide = L.n <= kMidArgsortWideRows;
-  const void* const kernel = !mid ? reinterpret_cast<const void*>(crowd_finish_kernel<kRadixThreads, 0>)
-                             : wide ? reinterpret_cast<const void*>(crowd_finish_kernel<kMidArgsortThreads, 1>)
-                                    : reinterpret_cast<const void*>(crowd_finish_kernel<kMidArgsortThreads, 2>);
+  const bool many = w.batch > 1;
+  auto instance = [&](auto one, auto several) { return many ? reinterpret_cast<const void*>(several) : reinterpret_cast<const void*>(one); };
+  const void* const kernel = !mid   ? instance(crowd_finish_kernel<kRadixThreads, 0, false>, crowd_finish_kernel<kRadixThreads, 0, true>)
+                             : wide ? instance(crowd_finish_kernel<kMidArgsortThreads, 1, false>, crowd_finish_kernel<kMidArgsortThreads, 1, true>)
+                                    : instance(crowd_finish_kernel<kMidArgsortThreads, 2, false>, crowd_finish_kernel<kMidArgsortThreads, 2, true>);
   if (int e = grant_dynamic_lds(kernel, lds)) return e;
-  if (mid && wide)
-    hipLaunchKernelGGL((crowd_finish_kernel<kMidArgsortThreads, 1>), dim3(finish_grid(L, 1)), dim3(kMidArgsortThreads), lds, s,
-                       crowd_args(w, list, false, fused), want_order ? 1 : 0, after_peel_tail ? 1 : 0);
+  const int grid = shared_grid(finish_grid(L, 1), mid ? device_cus() : device_cus() * 2, w.batch);
+  const CrowdArgs ca = crowd_args(w, list, false, fused);
+  const int order_flag = want_order ? 1 : 0, tail_flag = after_peel_tail ? 1 : 0;
+  if (mid && wide && many)
+    hipLaunchKernelGGL((crowd_finish_kernel<kMidArgsortThreads, 1, true>), dim3(grid, 1, w.batch), dim3(kMidArgsortThreads), lds, s, ca, order_flag, tail_flag);
+  else if (mid && wide)
+    hipLaunchKernelGGL((crowd_finish_kernel<kMidArgsortThreads, 1, false>), dim3(grid), dim3(kMidArgsortThreads), lds, s, ca, order_flag, tail_flag);
+  else if (mid && many)
+    hipLaunchKernelGGL((crowd_finish_kernel<kMidArgsortThreads, 2, true>), dim3(grid, 1, w.batch), dim3(kMidArgsortThreads), lds, s, ca, order_flag, tail_flag);
   else if (mid)
-    hipLaunchKernelGGL((crowd_finish_kernel<kMidArgsortThreads, 2>), dim3(finish_grid(L, 1)), dim3(kMidArgsortThreads), lds, s,
-                       crowd_args(w, list, false, fused), want_order ? 1 : 0, after_peel_tail ? 1 : 0);
+    hipLaunchKernelGGL((crowd_finish_kernel<kMidArgsortThreads, 2, false>), dim3(grid), dim3(kMidArgsortThreads), lds, s, ca, order_flag, tail_flag);
+  else if (many)
+    hipLaunchKernelGGL((crowd_finish_kernel<kRadixThreads, 0, true>), dim3(grid, 1, w.batch), dim3(kRadixThreads), lds, s, ca, order_flag, tail_flag);
   else
-    hipLaunchKernelGGL((crowd_finish_kernel<kRadixThreads, 0>), dim3(finish_grid(L, 1)), dim3(kRadixThreads), lds, s,
-                       crowd_args(w, list, false, fused), want_order ? 1 : 0, after_peel_tail ? 1 : 0);
+    hipLaunchKernelGGL((crowd_finish_kernel<kRadixThreads, 0, false>), dim3(grid), dim3(kRadixThreads), lds, s, ca, order_flag, tail_flag);
   EVX_LAUNCH_CHECK();
   return 0;
 }
 
 // The copy of a result of 4-byte elements out of the workspace, as the last kernel of an entry point: the result, or
 // `poison` in every element when a device-side wait of the call ran out.
-static int copy_out(const Ctrl* ctrl, void* dst, const void* src, int64_t n, uint32_t poison, hipStream_t s) {
+static int copy_out(const Ctrl* ctrl, void* dst, const void* src, int64_t n, uint32_t poison, hipStream_t s, int batch = 1,
+                    int64_t ws_step = 0) {
   int64_t blocks = (n + 1023) / 1024;
   if (blocks > 1024) blocks = 1024;
   if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL(copy_or_poison_kernel, dim3((unsigned)blocks), dim3(256), 0, s, ctrl, static_cast<const uint32_t*>(src),
-                     static_cast<uint32_t*>(dst), n, poison);
+  hipLaunchKernelGGL(copy_or_poison_kernel, dim3((unsigned)blocks, 1, batch), dim3(256), 0, s, ctrl, static_cast<const uint32_t*>(src),
+                     static_cast<uint32_t*>(dst), n, poison, ws_step);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -1255,24 +1390,42 @@ int evox_hip_stage_order(int64_t n, int64_t m, void* ws, size_t ws_bytes, void* 
   return stage_crowd_finish(w, w.at<int>(w.L.perm), true, 0, (hipStream_t)stream);
 }
 
-int evox_hip_non_dominate_rank_until(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, int64_t stop_count,
-                                     int32_t* rank_out, void* ws, size_t ws_bytes, void* stream) {
+}  // extern "C"
+
+// batch > 1: that many populations of one shape in the same launches (see select_rows); their ranks lie n elements apart.
+static int rank_rows(const Fitness& fit, int64_t n, int64_t m, int64_t stop_count, int32_t* rank_out, void* ws, size_t ws_bytes,
+                     hipStream_t s, int batch = 1, int64_t ws_step = 0) {
   Ws w;
   if (rank_out == nullptr || stop_count < 1 || stop_count > n) return kErrBadArg;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
-  hipStream_t s = (hipStream_t)stream;
-  if (two_applies(w.L, stop_count)) {
+  if (batch > 1) {
+    if (ws_step < (int64_t)w.L.total || (ws_step & 255) != 0 || ws_bytes < (size_t)ws_step * (size_t)batch) return kErrWorkspace;
+    w.batch = batch;
+    w.step = ws_step;
+  }
+  if (batch == 1 && two_applies(w.L, stop_count)) {
     int* until = stop_count < n ? w.at<int>(w.L.order) : (int*)nullptr;
-    const int e = stage_rank_two(w, one_part(f, n, sr, sc), stop_count, false, until, s);
+    const int e = stage_rank_two(w, fit, stop_count, false, until, s);
     if (e != kErrNotResident) {
       if (e) return e;
       return copy_out(w.ctrl(), rank_out, until != nullptr ? until : w.at<int>(w.L.rank), n, kPoisonIndex, s);
     }
   }
-  if (int e = stage_prepare(w, one_part(f, n, sr, sc), true, s)) return e;
+  if (int e = stage_prepare(w, fit, true, s)) return e;
   if (int e = stage_dominance(w, kDomAuto, s)) return e;
-  if (int e = count_and_peel(w, stop_count, false, false, s)) return e;
-  return copy_out(w.ctrl(), rank_out, w.at<int>(w.L.rank), n, kPoisonIndex, s);
+  if (batch > 1) {
+    if (int e = count_and_peel_persistent(w, stop_count, false, false, s, false, nullptr, nullptr)) return e == kErrNotResident ? kErrBadArg : e;
+  } else if (int e = count_and_peel(w, stop_count, false, false, s)) {
+    return e;
+  }
+  return copy_out(w.ctrl(), rank_out, w.at<int>(w.L.rank), n, kPoisonIndex, s, w.batch, w.step);
+}
+
+extern "C" {
+
+int evox_hip_non_dominate_rank_until(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, int64_t stop_count,
+                                     int32_t* rank_out, void* ws, size_t ws_bytes, void* stream) {
+  return rank_rows(one_part(f, n, sr, sc), n, m, stop_count, rank_out, ws, ws_bytes, (hipStream_t)stream);
 }
 
 int evox_hip_non_dominate_rank(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, int32_t* rank_out, void* ws,
@@ -1641,7 +1794,11 @@ static int stage_rank_two(const Ws& w, const Fitness& src, int64_t stop_count, b
 static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes, const void* x2,
                        int64_t x2_row_stride_bytes, const Fitness& fit, int64_t n, int64_t m, int64_t topk, void* out_x,
                        float* out_f, int32_t* out_rank, float* out_dist, int32_t* out_order, void* ws, size_t ws_bytes,
-                       hipStream_t s, bool may_allocate) {
+                       hipStream_t s, bool may_allocate, int batch = 1, int64_t ws_step = 0, int64_t x_step_bytes = 0,
+                       int64_t x2_step_bytes = 0) {
+  // batch > 1: that many populations of one shape in the same launches (the caller has checked that their grids are
+  // resident together: many_populations_plan); their workspaces lie ws_step bytes apart, their decision vectors
+  // x_step_bytes, their fitness fit.step elements, their results topk rows
   Ws w;
   if (out_f == nullptr || out_rank == nullptr || out_dist == nullptr) return kErrBadArg;
   if ((x == nullptr) != (out_x == nullptr) || (x == nullptr) != (x2 == nullptr)) return kErrBadArg;
@@ -1649,66 +1806,19 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   if (topk < 1 || topk > n) return kErrBadArg;
   if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
   const Layout& L = w.L;
-  if (two_applies(L, topk)) {
-    const int e = stage_rank_two(w, fit, topk, true, nullptr, s);
-    if (e != kErrNotResident) {
-      if (e) return e;
-      // the last front by the ordering kernels, then the gather, as after a peel that leaves the last front alone
-      if (int c = stage_crowd_sort(w, w.at<int>(L.perm), false, 2, s, false)) return c;
-      if (int c = stage_crowd_finish(w, w.at<int>(L.perm), true, 2, s, false)) return c;
-      GatherArgs g2 = {};
-      int unit2 = 1;
-      if (x != nullptr) {
-        const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(x2) | reinterpret_cast<uintptr_t>(out_x) |
-                               (uintptr_t)x_row_bytes | (uintptr_t)x_row_stride_bytes | (uintptr_t)x2_row_stride_bytes;
-        unit2 = (bits % 16 == 0) ? 16 : (bits % 4 == 0) ? 4 : 1;
-      }
-      g2.order = w.at<int>(L.order);
-      g2.listed = w.at<int>(L.perm);
-      g2.topk = (int)topk;
-      g2.x = static_cast<const uint8_t*>(x);
-      g2.x_row_stride = x_row_stride_bytes;
-      g2.x_row_bytes = x_row_bytes;
-      g2.out_x = static_cast<uint8_t*>(out_x);
-      g2.unit = unit2;
-      g2.f = fit.f;
-      g2.f_stride_row = fit.sr;
-      g2.f_stride_col = fit.sc;
-      g2.n_first = (int)fit.n_first;
-      g2.x2 = static_cast<const uint8_t*>(x2);
-      g2.x2_row_stride = x2_row_stride_bytes;
-      g2.f2 = fit.f2;
-      g2.f2_stride_row = fit.sr2;
-      g2.f2_stride_col = fit.sc2;
-      g2.m = L.m;
-      g2.out_f = out_f;
-      g2.rank = w.at<int>(L.rank);
-      g2.out_rank = out_rank;
-      g2.dist = w.at<float>(L.dist);
-      g2.out_dist = out_dist;
-      g2.out_order = out_order;
-      g2.ctrl = w.ctrl();
-      int blocks = (int)((topk + 3) / 4);
-      const int cap = device_cus() * 8;
-      if (blocks > cap) blocks = cap;
-      hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(256), 0, s, g2);
-      EVX_LAUNCH_CHECK();
-      return 0;
-    }
+  if (batch > 1) {
+    if (ws_step < (int64_t)L.total || (ws_step & 255) != 0 || ws_bytes < (size_t)ws_step * (size_t)batch) return kErrWorkspace;
+    w.batch = batch;
+    w.step = ws_step;
   }
-  if (int e = stage_prepare(w, fit, true, s)) return e;
-  if (int e = stage_dominance(w, kDomAuto, s)) return e;
-  bool peel_orders = false;  // the peel kernel orders a small last front itself (it says so in Ctrl.tail_done)
-  bool peel_always_orders = false;  // ... and here every front is small enough: nothing is left to launch but the gather
-  bool stepped = false;  // the fronts were peeled one launch each: the last front is ordered likewise, by the kernels of wide.hpp
-  if (int e = count_and_peel(w, topk, true, true, s, true, &peel_orders, &peel_always_orders, &stepped)) return e;
   int unit = 1;
   if (x != nullptr) {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(x2) | reinterpret_cast<uintptr_t>(out_x) |
-                           (uintptr_t)x_row_bytes | (uintptr_t)x_row_stride_bytes | (uintptr_t)x2_row_stride_bytes;
+                           (uintptr_t)x_row_bytes | (uintptr_t)x_row_stride_bytes | (uintptr_t)x2_row_stride_bytes |
+                           (uintptr_t)x_step_bytes | (uintptr_t)x2_step_bytes;
     unit = (bits % 16 == 0) ? 16 : (bits % 4 == 0) ? 4 : 1;
   }
-  GatherArgs g;
+  GatherArgs g = {};
   g.order = w.at<int>(L.order);
   g.listed = w.at<int>(L.perm);
   g.topk = (int)topk;
@@ -1734,8 +1844,48 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   g.out_dist = out_dist;
   g.out_order = out_order;
   g.ctrl = w.ctrl();
+  g.ws_step = w.step;
+  g.x_step = x_step_bytes;
+  g.x2_step = x2_step_bytes;
+  g.f_step = fit.step;
+  g.f2_step = fit.step2;
+  int gather_blocks = (int)((topk + 3) / 4);
+  if (gather_blocks > device_cus() * 8) gather_blocks = device_cus() * 8;
+  const dim3 gather_grid(gather_blocks, 1, w.batch);
+  auto launch_gather = [&](bool after_peel) {
+    if (after_peel && w.batch > 1)
+      hipLaunchKernelGGL(gather_after_peel_kernel<true>, gather_grid, dim3(256), 0, s, g);
+    else if (after_peel)
+      hipLaunchKernelGGL(gather_after_peel_kernel<false>, gather_grid, dim3(256), 0, s, g);
+    else if (w.batch > 1)
+      hipLaunchKernelGGL(gather_kernel<true>, gather_grid, dim3(256), 0, s, g);
+    else
+      hipLaunchKernelGGL(gather_kernel<false>, gather_grid, dim3(256), 0, s, g);
+  };
+  if (batch == 1 && two_applies(L, topk)) {
+    const int e = stage_rank_two(w, fit, topk, true, nullptr, s);
+    if (e != kErrNotResident) {
+      if (e) return e;
+      // the last front by the ordering kernels, then the gather, as after a peel that leaves the last front alone
+      if (int c = stage_crowd_sort(w, w.at<int>(L.perm), false, 2, s, false)) return c;
+      if (int c = stage_crowd_finish(w, w.at<int>(L.perm), true, 2, s, false)) return c;
+      launch_gather(false);
+      EVX_LAUNCH_CHECK();
+      return 0;
+    }
+  }
+  if (int e = stage_prepare(w, fit, true, s)) return e;
+  if (int e = stage_dominance(w, kDomAuto, s)) return e;
+  bool peel_orders = false;  // the peel kernel orders a small last front itself (it says so in Ctrl.tail_done)
+  bool peel_always_orders = false;  // ... and here every front is small enough: nothing is left to launch but the gather
+  bool stepped = false;  // the fronts were peeled one launch each: the last front is ordered likewise, by the kernels of wide.hpp
+  if (batch > 1) {
+    if (int e = count_and_peel_persistent(w, topk, true, true, s, true, &peel_orders, &peel_always_orders)) return e == kErrNotResident ? kErrBadArg : e;
+  } else if (int e = count_and_peel(w, topk, true, true, s, true, &peel_orders, &peel_always_orders, &stepped)) {
+    return e;
+  }
   g.order_from_peel = peel_always_orders ? 1 : 0;
-  g.outcome = peel_orders && !peel_always_orders && opt().launch_memory ? outcome_slot(n, m, may_allocate, s) : nullptr;
+  g.outcome = batch == 1 && peel_orders && !peel_always_orders && opt().launch_memory ? outcome_slot(n, m, may_allocate, s) : nullptr;
   const int last_outcome = g.outcome != nullptr ? __atomic_load_n(g.outcome, __ATOMIC_RELAXED) : 0;
   // Where the peel kernel may have ordered the last front, the kernels that would order it look at Ctrl.tail_done and
   // return at once.  A launch that does nothing still costs about 4.7 us, so with up to three objectives -- last
@@ -1764,31 +1914,22 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
     if (int e = evox_hip_stable_argsort_step(w.at<int>(L.rank), kKeyInt32, 1, n, order_b, w.at<int>(L.order), sort_ws, WL.sort_bytes, s))
       return e;
     g.outcome = nullptr;
-    int blocks = (int)((topk + 3) / 4);
-    const int cap = device_cus() * 8;
-    if (blocks > cap) blocks = cap;
-    hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(256), 0, s, g);
+    launch_gather(false);
     EVX_LAUNCH_CHECK();
     return 0;
   }
   if (peel_always_orders) {
-    int blocks = (int)((topk + 3) / 4);
-    const int cap = device_cus() * 8;
-    if (blocks > cap) blocks = cap;
-    hipLaunchKernelGGL(gather_after_peel_kernel, dim3(blocks), dim3(256), 0, s, g);
+    launch_gather(true);
     EVX_LAUNCH_CHECK();
     return 0;
   }
   if (!one_ordering_launch) {
     if (int e = stage_crowd_sort(w, w.at<int>(L.perm), true, 2, s, peel_orders)) return e;
     if (int e = stage_crowd_finish(w, w.at<int>(L.perm), true, 2, s, peel_orders)) return e;
-    int blocks = (int)((topk + 3) / 4);
-    const int cap = device_cus() * 8;
-    if (blocks > cap) blocks = cap;
     if (peel_orders)
-      hipLaunchKernelGGL(gather_after_peel_kernel, dim3(blocks), dim3(256), 0, s, g);
+      launch_gather(true);
     else
-      hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(256), 0, s, g);
+      launch_gather(false);
     EVX_LAUNCH_CHECK();
     return 0;
   }
@@ -1797,19 +1938,28 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
   const size_t lds = crowd_lds_bytes(L, 2);
   const bool mid = crowd_mid_sort(L);
   const bool wide = L.n <= kMidArgsortWideRows;
-  const void* const kernel = !mid ? reinterpret_cast<const void*>(crowd_gather_kernel<kRadixThreads, 0>)
-                             : wide ? reinterpret_cast<const void*>(crowd_gather_kernel<kMidArgsortThreads, 1>)
-                                    : reinterpret_cast<const void*>(crowd_gather_kernel<kMidArgsortThreads, 2>);
+  const bool many = w.batch > 1;
+  auto instance = [&](auto one, auto several) { return many ? reinterpret_cast<const void*>(several) : reinterpret_cast<const void*>(one); };
+  const void* const kernel = !mid   ? instance(crowd_gather_kernel<kRadixThreads, 0, false>, crowd_gather_kernel<kRadixThreads, 0, true>)
+                             : wide ? instance(crowd_gather_kernel<kMidArgsortThreads, 1, false>, crowd_gather_kernel<kMidArgsortThreads, 1, true>)
+                                    : instance(crowd_gather_kernel<kMidArgsortThreads, 2, false>, crowd_gather_kernel<kMidArgsortThreads, 2, true>);
   if (int e = grant_dynamic_lds(kernel, lds)) return e;
   int grid = finish_grid(L, L.m);  // resident at once: at most two blocks of 256 threads per compute unit
   if (grid > device_cus() * 2) grid = device_cus() * 2;
+  grid = shared_grid(grid, mid ? device_cus() : device_cus() * 2, w.batch);
   const CrowdArgs ca = crowd_args(w, w.at<int>(L.perm), false, 2);
-  if (mid && wide)
-    hipLaunchKernelGGL((crowd_gather_kernel<kMidArgsortThreads, 1>), dim3(grid), dim3(kMidArgsortThreads), lds, s, ca, g);
+  if (mid && wide && many)
+    hipLaunchKernelGGL((crowd_gather_kernel<kMidArgsortThreads, 1, true>), dim3(grid, 1, w.batch), dim3(kMidArgsortThreads), lds, s, ca, g);
+  else if (mid && wide)
+    hipLaunchKernelGGL((crowd_gather_kernel<kMidArgsortThreads, 1, false>), dim3(grid), dim3(kMidArgsortThreads), lds, s, ca, g);
+  else if (mid && many)
+    hipLaunchKernelGGL((crowd_gather_kernel<kMidArgsortThreads, 2, true>), dim3(grid, 1, w.batch), dim3(kMidArgsortThreads), lds, s, ca, g);
   else if (mid)
-    hipLaunchKernelGGL((crowd_gather_kernel<kMidArgsortThreads, 2>), dim3(grid), dim3(kMidArgsortThreads), lds, s, ca, g);
+    hipLaunchKernelGGL((crowd_gather_kernel<kMidArgsortThreads, 2, false>), dim3(grid), dim3(kMidArgsortThreads), lds, s, ca, g);
+  else if (many)
+    hipLaunchKernelGGL((crowd_gather_kernel<kRadixThreads, 0, true>), dim3(grid, 1, w.batch), dim3(kRadixThreads), lds, s, ca, g);
   else
-    hipLaunchKernelGGL((crowd_gather_kernel<kRadixThreads, 0>), dim3(grid), dim3(kRadixThreads), lds, s, ca, g);
+    hipLaunchKernelGGL((crowd_gather_kernel<kRadixThreads, 0, false>), dim3(grid), dim3(kRadixThreads), lds, s, ca, g);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -1846,6 +1996,88 @@ int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_ro
   const Fitness fit{f_a, f_a_stride_row, f_a_stride_col, n_a, f_b, f_b_stride_row, f_b_stride_col};
   return select_rows(x_a, x_row_bytes, x_a_row_stride_bytes, x_b, x_b_row_stride_bytes, fit, n_a + n_b, m, topk, out_x, out_f,
                      out_rank, out_dist, out_order, ws, ws_bytes, (hipStream_t)stream, true);
+}
+
+}  // extern "C"
+
+// ---- Many populations of one shape (more rows than the one-workgroup kernel of batched.hpp takes): the stages of the
+// pipeline run once for `share` populations at a time, population b in the workgroups with blockIdx.z == b on its own
+// copy of the workspace.  The kernels whose workgroups wait for each other get 1 / share of the device each, so that
+// all of them are resident together; that is possible where the peel keeps the matrix in LDS (up to 32 768 rows) and
+// a population's matrix fits the LDS of its share of the compute units.  Reference: the batched loop of
+// src/evox/operators/selection/non_dominate.py:107-125 (torch.vmap of the ranking, utils/op_register.py:26-51).
+static int many_populations_share(const Layout& L, int64_t batch, int64_t stop_count) {
+  if (batch < 2 || opt().peel_stepped || !opt().peel_lds || L.n > 32768) return 0;
+  if (!opt().mid_argsort && L.n > kRadixMinCandidates) return 0;  // (large last fronts would take the radix grid)
+  if (two_applies(L, stop_count)) return 0;
+  int share = 4 * device_cus() / 9;  // at least eight sweeping workgroups and the lister per population, up to four on a compute unit
+  if (share > batch) share = (int)batch;
+  size_t lds = 0;
+  while (share >= 2 && lds_peel_plan(L, &lds, share) == 0) --share;
+  if (share < 2) return 0;
+  const int64_t passes = (batch + share - 1) / share;
+  return (int)((batch + passes - 1) / passes);  // even passes: 30 populations, 28 at a time at most -> 15 + 15
+}
+
+static size_t many_workspace_step(const Layout& L) { return align_up(L.total); }
+
+extern "C" {
+
+/* Workspace for evox_hip_many_*: one copy of the single-population workspace per population that shares a launch. */
+size_t evox_hip_many_workspace_bytes(int64_t batch, int64_t n, int64_t m, int64_t stop_count) {
+  Layout L;
+  if (batch < 1 || !make_layout(n, m, &L)) return 0;
+  const int share = many_populations_share(L, batch, stop_count);
+  return many_workspace_step(L) * (size_t)(share > 1 ? share : 1);
+}
+
+int64_t evox_hip_many_populations_per_launch(int64_t batch, int64_t n, int64_t m, int64_t stop_count) {
+  Layout L;
+  if (batch < 1 || !make_layout(n, m, &L)) return 0;
+  const int share = many_populations_share(L, batch, stop_count);
+  return share > 1 ? share : 1;
+}
+
+int evox_hip_many_non_dominate_rank_until(const float* f, int64_t batch, int64_t n, int64_t m, int64_t stride_batch, int64_t sr,
+                                          int64_t sc, int64_t stop_count, int32_t* rank_out, void* ws, size_t ws_bytes,
+                                          void* stream) {
+  Layout L;
+  if (f == nullptr || rank_out == nullptr || batch < 1 || !make_layout(n, m, &L)) return kErrBadArg;
+  const int share = many_populations_share(L, batch, stop_count);
+  const size_t step = many_workspace_step(L);
+  for (int64_t b0 = 0; b0 < batch;) {
+    const int64_t left = batch - b0;
+    const int count = share > 1 ? (int)(left < share ? left : share) : 1;
+    const Fitness fit = one_part(f + b0 * stride_batch, n, sr, sc, stride_batch);
+    if (int e = rank_rows(fit, n, m, stop_count, rank_out + b0 * n, ws, ws_bytes, (hipStream_t)stream, count, count > 1 ? (int64_t)step : 0))
+      return e;
+    b0 += count;
+  }
+  return 0;
+}
+
+int evox_hip_many_nd_environmental_selection(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes,
+                                             int64_t x_batch_stride_bytes, const float* f, int64_t batch, int64_t n, int64_t m,
+                                             int64_t stride_batch, int64_t sr, int64_t sc, int64_t topk, void* out_x, float* out_f,
+                                             int32_t* out_rank, float* out_dist, void* ws, size_t ws_bytes, void* stream) {
+  Layout L;
+  if (f == nullptr || batch < 1 || !make_layout(n, m, &L) || topk < 1 || topk > n) return kErrBadArg;
+  if ((x == nullptr) != (out_x == nullptr) || (x != nullptr && (x_row_bytes < 0 || x_batch_stride_bytes < 0))) return kErrBadArg;
+  const int share = many_populations_share(L, batch, topk);
+  const size_t step = many_workspace_step(L);
+  for (int64_t b0 = 0; b0 < batch;) {
+    const int64_t left = batch - b0;
+    const int count = share > 1 ? (int)(left < share ? left : share) : 1;
+    const Fitness fit = one_part(f + b0 * stride_batch, n, sr, sc, stride_batch);
+    const uint8_t* xb = x != nullptr ? static_cast<const uint8_t*>(x) + b0 * x_batch_stride_bytes : nullptr;
+    uint8_t* oxb = out_x != nullptr ? static_cast<uint8_t*>(out_x) + b0 * topk * x_row_bytes : nullptr;
+    if (int e = select_rows(xb, x_row_bytes, x_row_stride_bytes, xb, x_row_stride_bytes, fit, n, m, topk, oxb, out_f + b0 * topk * m,
+                            out_rank + b0 * topk, out_dist + b0 * topk, nullptr, ws, ws_bytes, (hipStream_t)stream, true, count,
+                            count > 1 ? (int64_t)step : 0, x_batch_stride_bytes, x_batch_stride_bytes))
+      return e;
+    b0 += count;
+  }
+  return 0;
 }
 
 }  // extern "C"

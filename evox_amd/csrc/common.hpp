@@ -79,6 +79,20 @@ __device__ inline int group16_sum(int v) {
   v += __builtin_amdgcn_update_dpp(0, v, 0x121, 0xf, 0xf, false);
   return v;
 }
+// Several populations in one launch: population b is the workgroups with blockIdx.z == b, and every buffer of the
+// library's workspace that a kernel is given for population 0 lies b * `step` bytes further on for population b (a
+// launch for one population has blockIdx.z == 0 everywhere and passes a step of 0).  A kernel moves the pointers it
+// was given once, at its start; a null pointer ("not wanted") stays null.
+template <class P>
+__device__ __forceinline__ void to_population(int64_t step_bytes, P& p) {
+  if (p != nullptr) p = (P)((char*)p + (int64_t)blockIdx.z * step_bytes);
+}
+template <class P, class... More>
+__device__ __forceinline__ void to_population(int64_t step_bytes, P& p, More&... more) {
+  to_population(step_bytes, p);
+  to_population(step_bytes, more...);
+}
+
 // Relaxed agent-scope accesses: one location at a time, coherent across the whole device, without
 // the cache-wide write-back / invalidate that an agent-scope fence costs.  Everything that one
 // block writes and another block reads during the kernel (front bitmaps, front sizes, barrier

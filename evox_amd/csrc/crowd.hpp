@@ -142,7 +142,24 @@ struct GatherArgs {
   const Ctrl* ctrl;
   int order_from_peel;  // the host launched nothing that orders the last front: the peel kernel must have (Ctrl.tail_done)
   int* outcome;  // pinned host memory or null: 1 when the peel kernel has ordered the last front of this call, else 2
+  // several populations in one launch (blockIdx.z): from one population to the next, bytes between the library's
+  // buffers and between the decision vectors, elements between the fitness; the outputs are topk rows apart
+  int64_t ws_step, x_step, x2_step, f_step, f2_step;
 };
+
+__device__ __forceinline__ void to_population(GatherArgs& g) {
+  to_population(g.ws_step, g.order, g.listed, g.rank, g.dist, g.ctrl);
+  const int64_t b = (int64_t)blockIdx.z;
+  if (g.x != nullptr) g.x += b * g.x_step;
+  if (g.x2 != nullptr) g.x2 += b * g.x2_step;
+  if (g.out_x != nullptr) g.out_x += b * g.topk * g.x_row_bytes;
+  g.f += b * g.f_step;
+  g.f2 += b * g.f2_step;
+  g.out_f += b * g.topk * g.m;
+  g.out_rank += b * g.topk;
+  g.out_dist += b * g.topk;
+  if (g.out_order != nullptr) g.out_order += b * g.topk;
+}
 
 // Called by every thread of `blocks` blocks of 256 threads (`block` = the caller's index among them).
 // listed_until: positions below it take their row from a.listed instead of a.order.

@@ -57,13 +57,22 @@ __host__ __device__ inline uint32_t key_weight(int k) { return 16u + (uint32_t)(
 // later kernels accumulate into.  The third partial of a block says whether it met a NaN or an infinity.
 // The population may come in two parts (rows 0..n_first-1 from f, the rest from f2: parents and
 // offspring that the caller never concatenates, src/evox/algorithms/mo/nsga2.py:99-100).
+// MANY: several populations in the launch, one per blockIdx.z (the instance for one population is compiled without
+// the pointer moves).
+template <bool MANY>
 __global__ __launch_bounds__(256) void prepare_kernel(const float* __restrict__ f, int64_t stride_row, int64_t stride_col,
                                                       int n_first, const float* __restrict__ f2, int64_t stride_row2,
                                                       int64_t stride_col2, int n, int m, int npad, float* __restrict__ xs,
                                                       uint64_t* __restrict__ key, unsigned long long* __restrict__ partials,
-                                                      uint32_t* __restrict__ zero_words, int64_t n_zero_words, int lexicographic) {
+                                                      uint32_t* __restrict__ zero_words, int64_t n_zero_words, int lexicographic,
+                                                      int64_t f_step, int64_t f2_step, int64_t ws_step) {
   __shared__ unsigned long long red[2][4];
   __shared__ int any_bad;
+  if constexpr (MANY) {  // the fitness of population b lies f_step elements behind that of population 0
+    f += (int64_t)blockIdx.z * f_step;
+    f2 += (int64_t)blockIdx.z * f2_step;
+    to_population(ws_step, xs, key, partials, zero_words);
+  }
   if (threadIdx.x == 0) any_bad = 0;
   __syncthreads();
   bool bad = false;
@@ -128,11 +137,17 @@ constexpr int kSmallSortObjectives = 256;  // keys stay below 2^40, composites b
 constexpr int kSmallSortThreads = 1024;
 constexpr int kSmallSortGroup = 16;  // rows placed by one workgroup
 
+template <bool MANY>
 __global__ __launch_bounds__(kSmallSortThreads) void small_sort_kernel(
     const float* __restrict__ f, int64_t stride_row, int64_t stride_col, int n_first, const float* __restrict__ f2,
     int64_t stride_row2, int64_t stride_col2, int n, int m, int npad, float* __restrict__ xs, SortParam* __restrict__ param_out,
     uint64_t* __restrict__ key_sorted, uint32_t* __restrict__ kid_sorted, float* __restrict__ xs_sorted, int* __restrict__ orig_of,
-    uint32_t* __restrict__ zero_words, int64_t n_zero_words) {
+    uint32_t* __restrict__ zero_words, int64_t n_zero_words, int64_t f_step, int64_t f2_step, int64_t ws_step) {
+  if constexpr (MANY) {
+    f += (int64_t)blockIdx.z * f_step;
+    f2 += (int64_t)blockIdx.z * f2_step;
+    to_population(ws_step, xs, param_out, key_sorted, kid_sorted, xs_sorted, orig_of, zero_words);
+  }
   // npad composites, held as doubles (they are below 2^47, so exact): the hardware compares doubles at the
   // rate of 32-bit values, 64-bit integers several times slower; +inf for the padding rows
   extern __shared__ double comp[];
@@ -491,7 +506,8 @@ template <int M, int IW, int VARIANT>
 __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
                                                         const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom, int n,
                                                         int npad, int64_t wstride, int nwords,
-                                                        const SortParam* __restrict__ param) {
+                                                        const SortParam* __restrict__ param, int64_t ws_step) {
+  to_population(ws_step, xs, key, kid, dom, param);
   dominance_tile<M, IW, VARIANT>((int)blockIdx.x, (int)blockIdx.y, xs, key, kid, dom, n, npad, wstride, nwords, param);
 }
 
@@ -499,12 +515,14 @@ __global__ __launch_bounds__(256) void dominance_kernel(const float* __restrict_
 // two words: row block x (128 rows) needs x / 2 + 1 blocks of tiles, row block row_blocks - 1 - x the rest of about
 // row_blocks / 2 + 2, so the two share column x of a grid of ceil(row_blocks / 2) x ((row_blocks - 1) / 2 + 2) blocks.
 // Tiles of four words: row block x (256 rows) needs x + 1 tiles, the two together row_blocks + 1.
-template <int M, int IW>
+template <int M, int IW, bool MANY>
 __global__ __launch_bounds__(256) void dominance_folded_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
                                                                const uint32_t* __restrict__ kid, uint64_t* __restrict__ dom,
                                                                int n, int npad, int64_t wstride, int nwords,
-                                                               const SortParam* __restrict__ param, int row_blocks) {
+                                                               const SortParam* __restrict__ param, int row_blocks,
+                                                               int64_t ws_step) {
   static_assert(IW == 2 || IW == 4, "tiles of two or four words");
+  if constexpr (MANY) to_population(ws_step, xs, key, kid, dom, param);
   const int x = (int)blockIdx.x, y = (int)blockIdx.y;
   const int own = IW == 2 ? x / 2 + 1 : x + 1;
   int bx = x, by = y;
@@ -535,7 +553,8 @@ __global__ __launch_bounds__(256) void dominance_nonfinite_kernel(const float* _
 template <int IW>
 __global__ __launch_bounds__(256) void dominance_any_m_kernel(const float* __restrict__ xs, const uint32_t* __restrict__ kid,
                                                               uint64_t* __restrict__ dom, int n, int npad, int64_t wstride,
-                                                              int nwords, int m) {
+                                                              int nwords, int m, int64_t ws_step) {
+  to_population(ws_step, xs, kid, dom);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int j = (blockIdx.x * 4 + wave) * 64 + lane;

@@ -202,7 +202,13 @@ struct CrowdArgs {
   float* dist;
   uint32_t* dkey;
   int* order;
+  int64_t ws_step;  // several populations in one launch: bytes from one population's buffers to the next one's
 };
+
+__device__ __forceinline__ void to_population(CrowdArgs& a) {
+  to_population(a.ws_step, a.xs, a.list_base, a.ctrl, a.pos, a.sorted_cost, a.buf.pairs[0], a.buf.pairs[1], a.buf.table, a.buf.totals,
+                a.param, a.dist, a.dkey, a.order);
+}
 
 // Whether a last front of nv rows is ordered by workgroups that sort in LDS (the same answer in every workgroup).
 // Smaller fronts are ranked by counting, which is quadratic: 2000 candidates x 3 objectives took 67 us that way, on
@@ -314,11 +320,12 @@ __device__ inline void crowd_sort_body(const CrowdArgs& a, unsigned gen0, int ep
 // after_peel_tail: the peel kernel may have ordered the last front already (Ctrl.tail_done).
 // T threads: kRadixThreads, or kMidArgsortThreads where CrowdArgs.mid_sort is set (the radix sort, which is written for
 // kRadixThreads, does not run then).
-template <int T, int TABLES>
+template <int T, int TABLES, bool MANY = false>
 __global__ __launch_bounds__(T) void crowd_sort_kernel(CrowdArgs a, int after_peel_tail) {
   extern __shared__ __attribute__((aligned(16))) uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
+  if constexpr (MANY) to_population(a);  // several populations in the launch, one per blockIdx.z
   if (after_peel_tail != 0 && a.ctrl->tail_done != 0) return;
   crowd_sort_body<TABLES>(a, radix_generation_base(a.ctrl), 1, finish_lds, base, scratch);
 }
@@ -538,11 +545,12 @@ __device__ inline void crowd_finish_body(const CrowdArgs& a, int want_order, uns
   }
 }
 
-template <int T, int TABLES>
+template <int T, int TABLES, bool MANY = false>
 __global__ __launch_bounds__(T) void crowd_finish_kernel(CrowdArgs a, int want_order, int after_peel_tail) {
   extern __shared__ __attribute__((aligned(16))) uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
+  if constexpr (MANY) to_population(a);
   if (after_peel_tail != 0 && a.ctrl->tail_done != 0) return;
   crowd_finish_body<TABLES>(a, want_order, radix_generation_base(a.ctrl), 1, finish_lds, base, scratch);
 }
@@ -556,11 +564,17 @@ __device__ inline bool tail_barrier(Ctrl* ctrl, int target, unsigned spin_limit,
   return counter_barrier(ctrl, 1, target, spin_limit, scratch);
 }
 
-__global__ __launch_bounds__(256) void gather_kernel(GatherArgs g) { gather_body(g, blockIdx.x, gridDim.x, 0); }
+template <bool MANY>
+__global__ __launch_bounds__(256) void gather_kernel(GatherArgs g) {
+  if constexpr (MANY) to_population(g);
+  gather_body(g, blockIdx.x, gridDim.x, 0);
+}
 
 // listed: the rows of the better fronts as the peel listed them; positions below Ctrl.worst_start take their row
 // from there when the peel kernel has ordered the last front (it then leaves only that front's part of `order`).
+template <bool MANY>
 __global__ __launch_bounds__(256) void gather_after_peel_kernel(GatherArgs g) {
+  if constexpr (MANY) to_population(g);
   gather_body(g, blockIdx.x, gridDim.x, g.ctrl->err == 0 && g.ctrl->tail_done != 0 ? g.ctrl->worst_start : 0);
 }
 
@@ -569,11 +583,15 @@ __global__ __launch_bounds__(256) void gather_after_peel_kernel(GatherArgs g) {
 // launch after the peel instead of two or three.  Otherwise the order is complete when every block has passed the
 // second round of the barrier counter that separates the two ordering stages.  After a failed wait the gather writes
 // no rows (it looks at Ctrl.err).
-template <int T, int TABLES>
+template <int T, int TABLES, bool MANY>
 __global__ __launch_bounds__(T) void crowd_gather_kernel(CrowdArgs a, GatherArgs g) {
   extern __shared__ __attribute__((aligned(16))) uint64_t finish_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
+  if constexpr (MANY) {  // several populations in the launch, one per blockIdx.z
+    to_population(a);
+    to_population(g);
+  }
   Ctrl* ctrl = a.ctrl;
   if (coherent_load(&ctrl->err) != 0) {
     gather_body(g, blockIdx.x, gridDim.x, 0);

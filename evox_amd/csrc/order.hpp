@@ -68,10 +68,15 @@ __device__ inline SortParam make_sort_param(const unsigned long long* __restrict
   return sp;
 }
 
+// (MANY, here and below: several populations in the launch, one per blockIdx.z; the instance for one population is
+// compiled without the pointer moves)
+template <bool MANY>
 __global__ __launch_bounds__(256) void bucket_hist_kernel(const uint64_t* __restrict__ key, int n,
                                                           const unsigned long long* __restrict__ partials, int nparts,
-                                                          int buckets, int* __restrict__ hist, SortParam* __restrict__ param_out) {
+                                                          int buckets, int* __restrict__ hist, SortParam* __restrict__ param_out,
+                                                          int64_t ws_step) {
   __shared__ unsigned long long lds2[3];
+  if constexpr (MANY) to_population(ws_step, key, partials, hist, param_out);
   const SortParam sp = make_sort_param(partials, nparts, buckets, lds2);
   if (blockIdx.x == 0 && threadIdx.x == 0) *param_out = sp;
   const int lane = threadIdx.x & 63;
@@ -101,10 +106,12 @@ __global__ __launch_bounds__(256) void bucket_hist_kernel(const uint64_t* __rest
 // later kernel of the call returns without touching the half-built tables.
 constexpr unsigned kScanSpinLimit = 1u << 24;
 
+template <bool MANY>
 __global__ __launch_bounds__(256) void bucket_scan_kernel(const int* __restrict__ hist, int buckets, int* __restrict__ start,
                                                           int* __restrict__ cursor, unsigned long long* __restrict__ flags,
-                                                          Ctrl* __restrict__ ctrl) {
+                                                          Ctrl* __restrict__ ctrl, int64_t ws_step) {
   __shared__ int wave_tot[4];
+  if constexpr (MANY) to_population(ws_step, hist, start, cursor, flags, ctrl);
   __shared__ int base_lds;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int b0 = blockIdx.x * 1024 + threadIdx.x * 4;
@@ -154,10 +161,12 @@ __global__ __launch_bounds__(256) void bucket_scan_kernel(const int* __restrict_
   if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 255) start[buckets] = run;
 }
 
+template <bool MANY>
 __global__ __launch_bounds__(256) void bucket_scatter_kernel(const uint64_t* __restrict__ key, int n,
                                                              const SortParam* __restrict__ param, int* __restrict__ cursor,
                                                              int* __restrict__ members, uint64_t* __restrict__ member_key,
-                                                             const Ctrl* __restrict__ ctrl) {
+                                                             const Ctrl* __restrict__ ctrl, int64_t ws_step) {
+  if constexpr (MANY) to_population(ws_step, key, param, cursor, members, member_key, ctrl);
   if (ctrl->err != 0) return;
   const SortParam sp = *param;
   const int lane = threadIdx.x & 63;
@@ -206,13 +215,15 @@ constexpr int kPlaceTile = 1024;  // its members in LDS at a time
 // Exact slot of every row: bucket start + number of bucket members that precede it by (key, index).
 // Writes the slot-ordered copies of the fitness (structure of arrays, NaN padding up to npad), of
 // the keys (all-ones padding), the slot -> original index table (-1 padding) and its inverse.
+template <bool MANY>
 __global__ __launch_bounds__(256) void bucket_place_kernel(const float* __restrict__ xs, int n,
                                                            int m, int npad, const SortParam* __restrict__ param,
                                                            const int* __restrict__ start, const int* __restrict__ members,
                                                            const uint64_t* __restrict__ member_key,
                                                            uint64_t* __restrict__ key_sorted, uint32_t* __restrict__ kid_sorted,
                                                            float* __restrict__ xs_sorted, int* __restrict__ orig_of,
-                                                           int* __restrict__ slot_of, const Ctrl* __restrict__ ctrl) {
+                                                           int* __restrict__ slot_of, const Ctrl* __restrict__ ctrl, int64_t ws_step) {
+  if constexpr (MANY) to_population(ws_step, xs, param, start, members, member_key, key_sorted, kid_sorted, xs_sorted, orig_of, slot_of, ctrl);
   if (ctrl->err != 0) return;
   const SortParam sp = *param;
   __shared__ __attribute__((aligned(16))) uint64_t tile[kPlaceTile];

@@ -57,7 +57,11 @@ __global__ __launch_bounds__(256) void reset_state_kernel(uint32_t* __restrict__
 // kernel of an entry point, so that a caller who never reads the status still cannot take a partial result for a
 // result (ranks -1, distances NaN, orders -1).  src == nullptr only poisons.
 __global__ __launch_bounds__(256) void copy_or_poison_kernel(const Ctrl* __restrict__ ctrl, const uint32_t* __restrict__ src,
-                                                             uint32_t* __restrict__ dst, int64_t n, uint32_t poison) {
+                                                             uint32_t* __restrict__ dst, int64_t n, uint32_t poison,
+                                                             int64_t ws_step) {
+  // (several populations in one launch: their results lie n elements apart)
+  to_population(ws_step, ctrl, src);
+  dst += (int64_t)blockIdx.z * n;
   const bool failed = ctrl->err != 0;
   if (!failed && src == nullptr) return;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)

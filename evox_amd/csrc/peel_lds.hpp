@@ -238,14 +238,19 @@ struct PeelTail {
 // waits for every other one).  Dynamic LDS: lds_peel_bytes().  The matrix must be complete in `dom`; rank, the
 // crowding-distance fill, the front sizes and listings and the control block are written as by count_kernel +
 // peel_records_kernel.  Stops as soon as the fronts built so far hold stop_count rows.
+template <bool MANY>  // several populations in the launch, one per blockIdx.z (the other instance is compiled without the pointer moves)
 __global__ __launch_bounds__(kLdsPeelThreads) void peel_lds_kernel(
     const uint64_t* __restrict__ dom, int64_t wstride, int nwords, int n, const int* __restrict__ orig_of,
     int* __restrict__ rank, float* __restrict__ dist_fill, uint64_t* __restrict__ fronts_slot,
     uint64_t* __restrict__ fronts_orig, int* __restrict__ fsize, int* __restrict__ perm, int* __restrict__ fstart,
     Ctrl* __restrict__ ctrl, int stop_count, unsigned spin_limit, unsigned long long* __restrict__ records, int sweepers,
-    PeelTail tail) {
+    PeelTail tail, int64_t ws_step) {
   extern __shared__ __attribute__((aligned(16))) uint64_t lds[];  // the rows are read 16 bytes at a time
   __shared__ int sh[48];
+  if constexpr (MANY) {
+    to_population(ws_step, dom, orig_of, rank, dist_fill, fronts_slot, fronts_orig, fsize, perm, fstart, ctrl, records);
+    to_population(ws_step, tail.xs_sorted, tail.dist, tail.order, tail.buffer);
+  }
   if (coherent_load(&ctrl->err) != 0) return;
   int units = 2;  // per record: the largest power of two up to 32 that gives every sweeper a record
   while (units * 2 * sweepers <= kRecUnits && units < 32) units *= 2;

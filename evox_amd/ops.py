@@ -57,25 +57,49 @@ def _order_preserving_f32(t: torch.Tensor, what: str) -> torch.Tensor:
         raise ValueError(f"{what} of dtype {t.dtype} is limited to 2**24 rows per population")
     # one sort per objective column, all columns and populations in the same calls: in sorted order a value opens
     # a new rank when it differs from the value before it (-0.0 == 0.0; NaN, sorted last, is put back below)
-    flat = t.reshape(-1, t.shape[-2], t.shape[-1])
-    values, index = torch.sort(flat, dim=1)
-    opens = torch.zeros(flat.shape, dtype=torch.int64, device=t.device)
-    opens[:, 1:, :] = (values[:, 1:, :] != values[:, :-1, :]).to(torch.int64)
+    # (every objective as a contiguous row: torch's scan along any other dimension takes milliseconds for 20 000 rows)
+    flat = t.reshape(-1, t.shape[-2], t.shape[-1]).transpose(1, 2).contiguous()
+    values, index = torch.sort(flat, dim=2)
+    opens = torch.zeros(flat.shape, dtype=torch.int32, device=t.device)
+    opens[:, :, 1:] = values[:, :, 1:] != values[:, :, :-1]
     dense = torch.empty(flat.shape, dtype=torch.float32, device=t.device)
-    dense.scatter_(1, index, opens.cumsum(dim=1).to(torch.float32))
+    dense.scatter_(2, index, opens.cumsum(dim=2, dtype=torch.int32).to(torch.float32))
     if flat.is_floating_point():
         dense = torch.where(torch.isnan(flat), torch.full_like(dense, float("nan")), dense)
-    return dense.reshape(t.shape)
+    return dense.transpose(1, 2).reshape(t.shape)
 
 
-def _rank_one(f: torch.Tensor, out: torch.Tensor) -> None:
-    n, m = f.shape
-    ws = runtime.workspace(n, m, f.device)
-    stream = runtime.stream_handle(f.device)
+def _passes(batch: int, per_launch: int):
+    """(first population, populations) of the library calls that rank or select `batch` populations: one call for all
+    of them -- the library then runs its launches for `per_launch` populations at a time -- unless the status of every
+    call is checked, which looks at the control blocks of one pass."""
+    if not runtime.CHECK_STATUS or per_launch >= batch:
+        return [(0, batch)]
+    return [(b0, min(per_launch, batch - b0)) for b0 in range(0, batch, per_launch)]
+
+
+def _rank_many(flat_f: torch.Tensor, flat_out: torch.Tensor, count: int) -> None:
+    """Ranks of (B, N, M) float32 fitness as far as the front that holds the count-th row, into (B, N) int32."""
+    batch, n, m = flat_f.shape
+    if batch == 1:
+        ws = runtime.workspace(n, m, flat_f.device)
+        stream = runtime.stream_handle(flat_f.device)
+
+        def issue_one():
+            _lib.call("evox_hip_non_dominate_rank_until", flat_f.data_ptr(), n, m, flat_f.stride(1), flat_f.stride(2), count,
+                      flat_out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
+            runtime.note_call(ws, stream)
+
+        runtime.checked(issue_one)
+        return
+    stream = runtime.stream_handle(flat_f.device)
+
     def issue():
-        _lib.call("evox_hip_non_dominate_rank", f.data_ptr(), n, m, f.stride(0), f.stride(1), out.data_ptr(), ws.data_ptr(),
-                  ws.numel(), stream)
-        runtime.note_call(ws, stream)
+        ws, per_launch, step = runtime.many_workspace(batch, n, m, count, flat_f.device)
+        for b0, nb in _passes(batch, per_launch):
+            _lib.call("evox_hip_many_non_dominate_rank_until", flat_f[b0].data_ptr(), nb, n, m, flat_f.stride(0), flat_f.stride(1),
+                      flat_f.stride(2), count, flat_out[b0].data_ptr(), ws.data_ptr(), ws.numel(), stream)
+            runtime.note_call(ws, stream, min(per_launch, nb), step)
 
     runtime.checked(issue)
 
@@ -101,8 +125,7 @@ def nd_rank(f: torch.Tensor) -> torch.Tensor:
                       flat_f.stride(1), flat_f.stride(2), flat_out.data_ptr(), runtime.stream_handle(f.device))
             runtime.note_small_kernel_call()
         else:
-            for b in range(flat_f.size(0)):
-                _rank_one(flat_f[b], flat_out[b])
+            _rank_many(flat_f, flat_out, n)
     return out
 
 
@@ -148,19 +171,7 @@ def nd_rank_until(f: torch.Tensor, count: int) -> torch.Tensor:
     if out.numel() == 0:
         return out
     with torch.cuda.device(f.device):
-        flat_f = f32.reshape(-1, n, m)
-        flat_out = out.view(-1, n)
-        ws = runtime.workspace(n, m, f.device)
-        stream = runtime.stream_handle(f.device)
-        for b in range(flat_f.size(0)):
-            fb = flat_f[b]
-
-            def issue():
-                _lib.call("evox_hip_non_dominate_rank_until", fb.data_ptr(), n, m, fb.stride(0), fb.stride(1), count,
-                          flat_out[b].data_ptr(), ws.data_ptr(), ws.numel(), stream)
-                runtime.note_call(ws, stream)
-
-            runtime.checked(issue)
+        _rank_many(f32.reshape(-1, n, m), out.view(-1, n), count)
     return out
 
 
@@ -476,18 +487,19 @@ def nd_select(x: torch.Tensor, f: torch.Tensor, topk: int) -> Tuple[torch.Tensor
                       fo_r.data_ptr(), fo_d.data_ptr(), stream)
             runtime.note_small_kernel_call()
             return out_x, out_f.to(f.dtype), out_rank, out_dist
-        ws = runtime.workspace(n, m, f.device)
-        for b in range(flat_f.size(0)):
-            fb, xb = flat_f[b], flat_x[b]
+        batch_count = flat_f.size(0)
+        es = flat_x.element_size()
 
-            def issue():
-                _lib.call("evox_hip_nd_environmental_selection", xb.data_ptr() if has_x else None, row_bytes,
-                          xb.stride(0) * xb.element_size(), fb.data_ptr(), n, m, fb.stride(0), fb.stride(1), topk,
-                          fo_x[b].data_ptr() if has_x else None, fo_f[b].data_ptr(), fo_r[b].data_ptr(), fo_d[b].data_ptr(),
-                          None, ws.data_ptr(), ws.numel(), stream)
-                runtime.note_call(ws, stream)
+        def issue():
+            ws, per_launch, step = runtime.many_workspace(batch_count, n, m, topk, f.device)
+            for b0, nb in _passes(batch_count, per_launch):
+                _lib.call("evox_hip_many_nd_environmental_selection", flat_x[b0].data_ptr() if has_x else None, row_bytes,
+                          flat_x.stride(1) * es, flat_x.stride(0) * es, flat_f[b0].data_ptr(), nb, n, m, flat_f.stride(0),
+                          flat_f.stride(1), flat_f.stride(2), topk, fo_x[b0].data_ptr() if has_x else None, fo_f[b0].data_ptr(),
+                          fo_r[b0].data_ptr(), fo_d[b0].data_ptr(), ws.data_ptr(), ws.numel(), stream)
+                runtime.note_call(ws, stream, min(per_launch, nb), step)
 
-            runtime.checked(issue)
+        runtime.checked(issue)
     return out_x, out_f.to(f.dtype), out_rank, out_dist
 
 

@@ -125,13 +125,34 @@ def wide_workspace(n: int, m: int, device: torch.device) -> torch.Tensor:
     return ws
 
 
+def many_workspace(batch: int, n: int, m: int, stop_count: int, device: torch.device):
+    """Workspace of the entry points that take many populations of one shape: (tensor, populations per launch, bytes
+    from one population's copy of the workspace to the next); shares the per-(device, stream) buffer of `workspace`.
+    Asked anew at every call: the answer depends on the tunables in use."""
+    lib = _lib.lib()
+    need = int(lib.evox_hip_many_workspace_bytes(batch, n, m, stop_count))
+    per_launch = int(lib.evox_hip_many_populations_per_launch(batch, n, m, stop_count))
+    if need == 0 or per_launch < 1:
+        raise ValueError(f"unsupported population shape n={n}, m={m}")
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_handle(device))
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        _workspaces.pop(key, None)
+        ws = None
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        assert ws.data_ptr() % 256 == 0
+        _workspaces[key] = ws
+    return ws, per_launch, need // per_launch
+
+
 def release_workspaces() -> None:
     _workspaces.clear()
 
 
-def note_call(ws: torch.Tensor, stream: int) -> None:
+def note_call(ws: torch.Tensor, stream: int, copies: int = 1, step: int = 0) -> None:
+    """copies, step: the call used that many copies of the workspace, `step` bytes apart, each with a control block."""
     global _last
-    _last = (ws, stream)
+    _last = (ws, stream, copies, step)
     if CHECK_STATUS:
         last_status()
 
@@ -164,11 +185,12 @@ def last_status() -> dict:
     Calls served by the small-population kernel have no control block: {"error": 0}."""
     if _last is None:
         return {"error": 0}
-    ws, stream = _last
+    ws, stream, copies, step = _last
     out = (ctypes.c_int32 * 8)()
-    code = _lib.lib().evox_hip_read_status(ws.data_ptr(), stream, out)
-    if code != 0:
-        raise _lib.EvoxHipError("evox_hip_read_status", code)
+    for b in reversed(range(copies)):  # (the control block reported is that of the first copy)
+        code = _lib.lib().evox_hip_read_status(ws.data_ptr() + b * step, stream, out)
+        if code != 0:
+            raise _lib.EvoxHipError("evox_hip_read_status", code)
     keys = ("error", "fronts", "worst_rank", "better_rows", "last_front_size", "taken_from_last", "passes")
     return dict(zip(keys, list(out)[:7]))
 

@@ -168,6 +168,27 @@ int evox_hip_batched_nd_environmental_selection(const void* x, int64_t x_row_byt
                                                 int64_t topk, void* out_x, float* out_f, int32_t* out_rank, float* out_dist,
                                                 void* stream);
 
+/* ---- many populations of one shape, of any size (the same reference loop, non_dominate.py:107-125, and
+ * utils/op_register.py:26-51, through which a vmapped caller reaches it -- problems/hpo_wrapper.py:214-223 maps whole
+ * workflows).  The stages of the single-population pipeline run once for several populations at a time, each in
+ * its own workgroups on its own copy of the workspace, wherever the kernels whose workgroups wait for each other
+ * can all be resident with a share of the device each: populations of up to 32 768 rows whose bit matrix fits the
+ * LDS of that share.  evox_hip_many_populations_per_launch says how many share a launch (1: the entry points below
+ * then run the populations one after the other, which is always correct); evox_hip_many_workspace_bytes is the
+ * workspace for it (that many single-population workspaces).  `stop_count` is the topk of the selection, or the
+ * count of evox_hip_non_dominate_rank_until (n: every row is ranked).  Addressing as in evox_hip_batched_*; outputs
+ * are contiguous (batch, ...) arrays; per population the results equal those of the single-population entry points. */
+size_t evox_hip_many_workspace_bytes(int64_t batch, int64_t n, int64_t m, int64_t stop_count);
+int64_t evox_hip_many_populations_per_launch(int64_t batch, int64_t n, int64_t m, int64_t stop_count);
+int evox_hip_many_non_dominate_rank_until(const float* f, int64_t batch, int64_t n, int64_t m, int64_t stride_batch,
+                                          int64_t stride_row, int64_t stride_col, int64_t stop_count, int32_t* rank_out,
+                                          void* workspace, size_t workspace_bytes, void* stream);
+int evox_hip_many_nd_environmental_selection(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes,
+                                             int64_t x_batch_stride_bytes, const float* f, int64_t batch, int64_t n, int64_t m,
+                                             int64_t stride_batch, int64_t stride_row, int64_t stride_col, int64_t topk,
+                                             void* out_x, float* out_f, int32_t* out_rank, float* out_dist, void* workspace,
+                                             size_t workspace_bytes, void* stream);
+
 /* One small population given in two parts of equal strides (parents and offspring of NSGA-II,
  * src/evox/algorithms/mo/nsga2.py:99-102, at the population sizes such runs mostly have: a few hundred rows): the
  * selection of evox_hip_nd_environmental_selection_two_part in the one-workgroup kernel of the entry points above,
