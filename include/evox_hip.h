@@ -145,7 +145,7 @@ int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_ro
  * memory is a buffer of EVOX_HIP_STATIC_SCRATCH_BYTES bytes that is part of the library's device image, one copy per
  * GPU, held until the process ends.  The call allocates and frees nothing.  Results are those of
  * evox_hip_nd_environmental_selection.  A population with evox_hip_workspace_bytes(n, m) >
- * EVOX_HIP_STATIC_SCRATCH_BYTES (about 14 000 rows of 3 objectives, 11 000 of 16) is refused with
+ * EVOX_HIP_STATIC_SCRATCH_BYTES (about 14 000 rows of 3 objectives, 9800 of 16) is refused with
  * EVOX_HIP_E_STATIC_LIMIT.  All calls on one GPU share the buffer: calls on different streams of one GPU that
  * overlap in time race, the caller must order them. */
 #define EVOX_HIP_STATIC_SCRATCH_BYTES (32u << 20)
