@@ -349,6 +349,43 @@ def next_rows(dev, reps):
         out[f"converged one front N={n} M={m} topk={n // 2}"] = {
             "us": event_time_us(lambda: nd_environmental_selection(xc, fc, n // 2), reps)}
         del fc, xc
+    # many populations of more rows than the one-workgroup kernel takes, in one call (the stages of the pipeline run
+    # once for all of them) against one of them alone
+    from evox_amd import runtime
+    for b, n, m in ((16, 4096, 3), (32, 1500, 3), (64, 2000, 2)):
+        g = torch.Generator("cpu").manual_seed(6)
+        fm = torch.rand(b, n, m, generator=g).to(dev)
+        xm = torch.rand(b, n, 16, generator=g).to(dev)
+        nd_environmental_selection(xm, fm, n // 2)
+        nd_environmental_selection(xm[0], fm[0], n // 2)
+        out[f"many populations {b} x ({n}, {m}) topk={n // 2}"] = {
+            "all_in_one_call_us": event_time_us(lambda: nd_environmental_selection(xm, fm, n // 2), reps),
+            "one_alone_us": event_time_us(lambda: nd_environmental_selection(xm[0], fm[0], n // 2), reps)}
+        del fm, xm
+    # two objectives: ranked without a dominance matrix from 4097 rows on (all fronts) / 24576 rows on (up to a cut)
+    for n in (50000, 200000):
+        f2, x2 = workloads.uniform_population(n, 2, 16, 8)
+        f2, x2 = f2.to(dev), x2.to(dev)
+        nd_environmental_selection(x2, f2, n // 2)
+        row = {"selection_us": event_time_us(lambda: nd_environmental_selection(x2, f2, n // 2), max(3, reps // 2), inner=1)}
+        with runtime.options(two_min_rows=0):
+            nd_environmental_selection(x2, f2, n // 2)
+            row["selection_through_the_matrix_us"] = event_time_us(lambda: nd_environmental_selection(x2, f2, n // 2), 3, inner=1)
+        out[f"two objectives N={n} topk={n // 2}"] = row
+        del f2, x2
+    # the selection path whose kernels never wait for each other (one launch per front), and float64 fitness, at C3
+    with runtime.options(peel_stepped=1):
+        nd_environmental_selection(x, f, w.topk)
+        out["launch per front C3"] = {"us": event_time_us(lambda: nd_environmental_selection(x, f, w.topk), max(3, reps // 2), inner=1)}
+    default_dtype = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float64)
+    try:
+        f64, x64 = f.double(), x.double()
+        nd_environmental_selection(x64, f64, w.topk)
+        out["float64 fitness C3"] = {"us": event_time_us(lambda: nd_environmental_selection(x64, f64, w.topk), max(3, reps // 2), inner=1)}
+        del f64, x64
+    finally:
+        torch.set_default_dtype(default_dtype)
     # lexsort as a function of its own: HypE's lexsort([-dis, rank]) over the merged population
     full_rank = non_dominate_rank(f)
     key = torch.rand(f.size(0), device=dev)

@@ -51,6 +51,12 @@ _SIGNATURES = {
     "evox_hip_batched_nd_environmental_selection": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_int64,
                                                             c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                                             c_void_p, c_void_p, c_void_p]),
+    "evox_hip_many_first_front_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
+    "evox_hip_many_first_front_mask": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+                                               c_size_t, c_void_p]),
+    "evox_hip_many_crowding_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
+    "evox_hip_many_crowding_distance": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64,
+                                                c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "evox_hip_many_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
     "evox_hip_many_populations_per_launch": (c_int64, [c_int64, c_int64, c_int64, c_int64]),
     "evox_hip_many_non_dominate_rank_until": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,

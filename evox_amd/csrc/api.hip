@@ -304,9 +304,9 @@ static void launch_dominance(const Ws& w, int variant, hipStream_t s) {
 template <int M>
 static void launch_first_front(const Ws& w, uint8_t* mask, hipStream_t s) {
   const Layout& L = w.L;
-  hipLaunchKernelGGL((first_front_kernel<M>), dim3((L.n + 255) / 256), dim3(256), 0, s, w.at<float>(L.xs_sorted),
+  hipLaunchKernelGGL((first_front_kernel<M>), dim3((L.n + 255) / 256, 1, w.batch), dim3(256), 0, s, w.at<float>(L.xs_sorted),
                      w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<int>(L.orig_of), L.n, L.npad, mask,
-                     w.ctrl(), w.at<SortParam>(L.sortparam));
+                     w.ctrl(), w.at<SortParam>(L.sortparam), w.step);
 }
 
 // Fitness -> structure of arrays + keys, state reset, then the slot sort (order.hpp).
@@ -1438,14 +1438,22 @@ size_t evox_hip_first_front_workspace_bytes(int64_t n, int64_t m) {
   return make_layout(n, m, &L) ? L.dom : 0;
 }
 
-int evox_hip_first_front_mask(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, uint8_t* mask_out, void* ws,
-                              size_t ws_bytes, void* stream) {
+}  // extern "C"
+
+// batch > 1: that many populations of one shape in the same launches, their workspaces (without the matrix) ws_step
+// bytes apart, their masks n bytes.
+static int first_front_rows(const Fitness& fit, int64_t n, int64_t m, uint8_t* mask_out, void* ws, size_t ws_bytes, hipStream_t s,
+                            int batch = 1, int64_t ws_step = 0) {
   Ws w;
   if (mask_out == nullptr) return kErrBadArg;
   if (int e = open_ws(n, m, ws, ws_bytes, &w, false)) return e;
   const Layout& L = w.L;
-  hipStream_t s = (hipStream_t)stream;
-  if (int e = stage_prepare(w, one_part(f, n, sr, sc), true, s)) return e;
+  if (batch > 1) {
+    if (ws_step < (int64_t)L.dom || (ws_step & 255) != 0 || ws_bytes < (size_t)ws_step * (size_t)batch) return kErrWorkspace;
+    w.batch = batch;
+    w.step = ws_step;
+  }
+  if (int e = stage_prepare(w, fit, true, s)) return e;
   switch (L.m) {
     case 1: launch_first_front<1>(w, mask_out, s); break;
     case 2: launch_first_front<2>(w, mask_out, s); break;
@@ -1464,27 +1472,107 @@ int evox_hip_first_front_mask(const float* f, int64_t n, int64_t m, int64_t sr, 
     case 15: launch_first_front<15>(w, mask_out, s); break;
     case 16: launch_first_front<16>(w, mask_out, s); break;
     default:
-      hipLaunchKernelGGL(first_front_any_m_kernel, dim3((L.n + 255) / 256), dim3(256), 0, s, w.at<float>(L.xs_sorted),
-                         w.at<uint32_t>(L.kid_sorted), w.at<int>(L.orig_of), L.n, L.npad, L.m, mask_out, w.ctrl());
+      hipLaunchKernelGGL(first_front_any_m_kernel, dim3((L.n + 255) / 256, 1, w.batch), dim3(256), 0, s, w.at<float>(L.xs_sorted),
+                         w.at<uint32_t>(L.kid_sorted), w.at<int>(L.orig_of), L.n, L.npad, L.m, mask_out, w.ctrl(), w.step);
   }
   EVX_LAUNCH_CHECK();
   return 0;
 }
 
-int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t sr, int64_t sc, const uint8_t* mask,
-                               int64_t mask_stride, float* dist_out, void* ws, size_t ws_bytes, void* stream) {
+// batch > 1: as above; the masks lie mask_step bytes apart, the distances n elements.
+static int crowding_rows(const Fitness& costs, int64_t n, int64_t m, const uint8_t* mask, int64_t mask_stride, int64_t mask_step,
+                         float* dist_out, void* ws, size_t ws_bytes, hipStream_t s, int batch = 1, int64_t ws_step = 0) {
   Ws w;
-  if (costs == nullptr || dist_out == nullptr) return kErrBadArg;
-  if (int e = open_ws(n, m, ws, ws_bytes, &w)) return e;
+  if (costs.f == nullptr || dist_out == nullptr) return kErrBadArg;
+  if (int e = open_ws(n, m, ws, ws_bytes, &w, batch == 1)) return e;
   const Layout& L = w.L;
-  hipStream_t s = (hipStream_t)stream;
-  if (int e = stage_prepare(w, one_part(costs, n, sr, sc), false, s)) return e;
-  hipLaunchKernelGGL(compact_mask_kernel, dim3(1), dim3(1024), 0, s, mask, mask_stride, L.n, w.at<int>(L.perm),
-                     w.at<float>(L.dist), w.ctrl());
+  if (batch > 1) {
+    if (ws_step < (int64_t)L.dom || (ws_step & 255) != 0 || ws_bytes < (size_t)ws_step * (size_t)batch) return kErrWorkspace;
+    w.batch = batch;
+    w.step = ws_step;
+  }
+  if (int e = stage_prepare(w, costs, false, s)) return e;
+  hipLaunchKernelGGL(compact_mask_kernel, dim3(1, 1, w.batch), dim3(1024), 0, s, mask, mask_stride, L.n, w.at<int>(L.perm),
+                     w.at<float>(L.dist), w.ctrl(), mask_step, w.step);
   EVX_LAUNCH_CHECK();
   if (int e = stage_crowd_sort(w, w.at<int>(L.perm), false, 1, s)) return e;
   if (int e = stage_crowd_finish(w, w.at<int>(L.perm), false, 1, s)) return e;
-  return copy_out(w.ctrl(), dist_out, w.at<float>(L.dist), n, kPoisonFloat, s);
+  return copy_out(w.ctrl(), dist_out, w.at<float>(L.dist), n, kPoisonFloat, s, w.batch, w.step);
+}
+
+// Populations that share the launches of a first-front mask or of the crowding distances: their kernels need no
+// matrix, so a copy of the workspace is small; as many as 1 GiB of workspace holds (for the crowding distances:
+// and as the kernels that order a front, whose workgroups wait for each other, can be resident together).
+static int many_small_share(const Layout& L, int64_t batch, bool crowding) {
+  if (batch < 2) return 1;
+  if (crowding && (L.n > kMidArgsortRows || (!opt().mid_argsort && L.n > kRadixMinCandidates))) return 1;
+  int64_t share = (int64_t)(1ull << 30) / (int64_t)align_up(L.dom);
+  if (crowding && share > device_cus() / 2) share = device_cus() / 2;
+  if (share > 32768) share = 32768;
+  if (share > batch) share = batch;
+  if (share < 2) return 1;
+  const int64_t passes = (batch + share - 1) / share;
+  return (int)((batch + passes - 1) / passes);
+}
+
+extern "C" {
+
+int evox_hip_first_front_mask(const float* f, int64_t n, int64_t m, int64_t sr, int64_t sc, uint8_t* mask_out, void* ws,
+                              size_t ws_bytes, void* stream) {
+  return first_front_rows(one_part(f, n, sr, sc), n, m, mask_out, ws, ws_bytes, (hipStream_t)stream);
+}
+
+size_t evox_hip_many_first_front_workspace_bytes(int64_t batch, int64_t n, int64_t m) {
+  Layout L;
+  if (batch < 1 || !make_layout(n, m, &L)) return 0;
+  return align_up(L.dom) * (size_t)many_small_share(L, batch, false);
+}
+
+int evox_hip_many_first_front_mask(const float* f, int64_t batch, int64_t n, int64_t m, int64_t stride_batch, int64_t sr, int64_t sc,
+                                   uint8_t* mask_out, void* ws, size_t ws_bytes, void* stream) {
+  Layout L;
+  if (f == nullptr || mask_out == nullptr || batch < 1 || !make_layout(n, m, &L)) return kErrBadArg;
+  const int share = many_small_share(L, batch, false);
+  for (int64_t b0 = 0; b0 < batch;) {
+    const int64_t left = batch - b0;
+    const int count = (int)(left < share ? left : share);
+    if (int e = first_front_rows(one_part(f + b0 * stride_batch, n, sr, sc, stride_batch), n, m, mask_out + b0 * n, ws, ws_bytes,
+                                 (hipStream_t)stream, count, count > 1 ? (int64_t)align_up(L.dom) : 0))
+      return e;
+    b0 += count;
+  }
+  return 0;
+}
+
+size_t evox_hip_many_crowding_workspace_bytes(int64_t batch, int64_t n, int64_t m) {
+  Layout L;
+  if (batch < 1 || !make_layout(n, m, &L)) return 0;
+  const int share = many_small_share(L, batch, true);
+  return share > 1 ? align_up(L.dom) * (size_t)share : L.total;
+}
+
+int evox_hip_many_crowding_distance(const float* costs, int64_t batch, int64_t n, int64_t m, int64_t stride_batch, int64_t sr,
+                                    int64_t sc, const uint8_t* mask, int64_t mask_batch_stride, int64_t mask_stride, float* dist_out,
+                                    void* ws, size_t ws_bytes, void* stream) {
+  Layout L;
+  if (costs == nullptr || dist_out == nullptr || batch < 1 || !make_layout(n, m, &L)) return kErrBadArg;
+  const int share = many_small_share(L, batch, true);
+  for (int64_t b0 = 0; b0 < batch;) {
+    const int64_t left = batch - b0;
+    const int count = (int)(left < share ? left : share);
+    if (int e = crowding_rows(one_part(costs + b0 * stride_batch, n, sr, sc, stride_batch), n, m,
+                              mask != nullptr ? mask + b0 * mask_batch_stride : nullptr, mask_stride, mask_batch_stride,
+                              dist_out + b0 * n, ws, ws_bytes, (hipStream_t)stream, count, count > 1 ? (int64_t)align_up(L.dom) : 0))
+      return e;
+    b0 += count;
+  }
+  return 0;
+}
+
+int evox_hip_crowding_distance(const float* costs, int64_t n, int64_t m, int64_t sr, int64_t sc, const uint8_t* mask,
+                               int64_t mask_stride, float* dist_out, void* ws, size_t ws_bytes, void* stream) {
+  if (costs == nullptr) return kErrBadArg;
+  return crowding_rows(one_part(costs, n, sr, sc), n, m, mask, mask_stride, 0, dist_out, ws, ws_bytes, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -22,9 +22,12 @@ namespace evx {
 
 // Stable compaction of a boolean mask into an ascending list (one block; n is at most a few 10^5).
 // mask == nullptr selects every row.  Also fills dist with -inf and publishes nv in ctrl.
+// (Several populations in the launch, one per blockIdx.z: their masks lie mask_step bytes apart.)
 __global__ __launch_bounds__(1024) void compact_mask_kernel(const uint8_t* __restrict__ mask, int64_t mask_stride, int n,
                                                             int* __restrict__ list, float* __restrict__ dist,
-                                                            Ctrl* __restrict__ ctrl) {
+                                                            Ctrl* __restrict__ ctrl, int64_t mask_step, int64_t ws_step) {
+  if (mask != nullptr) mask += (int64_t)blockIdx.z * mask_step;
+  to_population(ws_step, list, dist, ctrl);
   // A wave takes a run of consecutive rows, 64 at a time: it counts its selected rows (loads that depend on nothing:
   // several in flight), the runs' counts are added up once, and a second walk writes the list.  (One step of 1024
   // rows at a time with the running total handed on through LDS cost three barriers and a memory round trip per

@@ -602,7 +602,11 @@ template <int M>
 __global__ __launch_bounds__(256) void first_front_kernel(const float* __restrict__ xs, const uint64_t* __restrict__ key,
                                                           const uint32_t* __restrict__ kid, const int* __restrict__ orig_of,
                                                           int n, int npad, uint8_t* __restrict__ mask,
-                                                          const Ctrl* __restrict__ ctrl, const SortParam* __restrict__ param) {
+                                                          const Ctrl* __restrict__ ctrl, const SortParam* __restrict__ param,
+                                                          int64_t ws_step) {
+  // (several populations in the launch, one per blockIdx.z: their masks lie n bytes apart)
+  to_population(ws_step, xs, key, kid, orig_of, ctrl, param);
+  mask += (int64_t)blockIdx.z * n;
   const int lane = threadIdx.x & 63;
   const int j = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 64 + lane;
   if (ctrl->err != 0) {  // the slot sort failed, nothing is valid: no row is reported (the status carries the error)
@@ -636,7 +640,10 @@ __global__ __launch_bounds__(256) void first_front_kernel(const float* __restric
 // Any number of objectives (used above 8).
 __global__ __launch_bounds__(256) void first_front_any_m_kernel(const float* __restrict__ xs, const uint32_t* __restrict__ kid,
                                                                 const int* __restrict__ orig_of, int n, int npad, int m,
-                                                                uint8_t* __restrict__ mask, const Ctrl* __restrict__ ctrl) {
+                                                                uint8_t* __restrict__ mask, const Ctrl* __restrict__ ctrl,
+                                                                int64_t ws_step) {
+  to_population(ws_step, xs, kid, orig_of, ctrl);
+  mask += (int64_t)blockIdx.z * n;
   const int lane = threadIdx.x & 63;
   const int j = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 64 + lane;
   if (ctrl->err != 0) {

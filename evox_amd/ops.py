@@ -203,12 +203,15 @@ def nd_first_front(f: torch.Tensor) -> torch.Tensor:
     with torch.cuda.device(f.device):
         flat_f = f32.reshape(-1, n, m)
         flat_out = out.view(-1, n)
-        ws = runtime.workspace(n, m, f.device, with_matrix=False)
         stream = runtime.stream_handle(f.device)
-        for b in range(flat_f.size(0)):
-            fb = flat_f[b]
-            _lib.call("evox_hip_first_front_mask", fb.data_ptr(), n, m, fb.stride(0), fb.stride(1), flat_out[b].data_ptr(),
+        if flat_f.size(0) == 1:
+            ws = runtime.workspace(n, m, f.device, with_matrix=False)
+            _lib.call("evox_hip_first_front_mask", flat_f.data_ptr(), n, m, flat_f.stride(1), flat_f.stride(2), flat_out.data_ptr(),
                       ws.data_ptr(), ws.numel(), stream)
+        else:
+            ws = runtime.sized_workspace(int(_lib.lib().evox_hip_many_first_front_workspace_bytes(flat_f.size(0), n, m)), f.device)
+            _lib.call("evox_hip_many_first_front_mask", flat_f.data_ptr(), flat_f.size(0), n, m, flat_f.stride(0), flat_f.stride(1),
+                      flat_f.stride(2), flat_out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
         runtime.note_call(ws, stream)
     return out
 
@@ -249,13 +252,17 @@ def crowding(costs: torch.Tensor, mask: Optional[torch.Tensor]) -> torch.Tensor:
         flat_out = out.view(-1, n)
         flat_mask = None if mask is None else mask.reshape(-1, n)
         stream = runtime.stream_handle(costs.device)
-        ws = runtime.workspace(n, m, costs.device)
-        for b in range(flat_c.size(0)):
-            c = flat_c[b]
-            mk = None if flat_mask is None else flat_mask[b]
-            _lib.call("evox_hip_crowding_distance", c.data_ptr(), n, m, c.stride(0), c.stride(1),
-                      None if mk is None else mk.data_ptr(), 0 if mk is None else mk.stride(0), flat_out[b].data_ptr(),
-                      ws.data_ptr(), ws.numel(), stream)
+        if flat_c.size(0) == 1:
+            ws = runtime.workspace(n, m, costs.device)
+            _lib.call("evox_hip_crowding_distance", flat_c.data_ptr(), n, m, flat_c.stride(1), flat_c.stride(2),
+                      None if flat_mask is None else flat_mask.data_ptr(), 0 if flat_mask is None else flat_mask.stride(1),
+                      flat_out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
+        else:
+            ws = runtime.sized_workspace(int(_lib.lib().evox_hip_many_crowding_workspace_bytes(flat_c.size(0), n, m)), costs.device)
+            _lib.call("evox_hip_many_crowding_distance", flat_c.data_ptr(), flat_c.size(0), n, m, flat_c.stride(0), flat_c.stride(1),
+                      flat_c.stride(2), None if flat_mask is None else flat_mask.data_ptr(),
+                      0 if flat_mask is None else flat_mask.stride(0), 0 if flat_mask is None else flat_mask.stride(1),
+                      flat_out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
         runtime.note_call(ws, stream)
     return out
 

@@ -125,6 +125,21 @@ def wide_workspace(n: int, m: int, device: torch.device) -> torch.Tensor:
     return ws
 
 
+def sized_workspace(need: int, device: torch.device) -> torch.Tensor:
+    """The per-(device, stream) buffer of `workspace`, at least `need` bytes."""
+    if need <= 0:
+        raise ValueError("unsupported population shape")
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_handle(device))
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        _workspaces.pop(key, None)
+        ws = None
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        assert ws.data_ptr() % 256 == 0
+        _workspaces[key] = ws
+    return ws
+
+
 def many_workspace(batch: int, n: int, m: int, stop_count: int, device: torch.device):
     """Workspace of the entry points that take many populations of one shape: (tensor, populations per launch, bytes
     from one population's copy of the workspace to the next); shares the per-(device, stream) buffer of `workspace`.

@@ -189,6 +189,19 @@ int evox_hip_many_nd_environmental_selection(const void* x, int64_t x_row_bytes,
                                              void* out_x, float* out_f, int32_t* out_rank, float* out_dist, void* workspace,
                                              size_t workspace_bytes, void* stream);
 
+/* The first-front mask and the crowding distances of many populations of one shape (evox_hip_first_front_mask and
+ * evox_hip_crowding_distance under vmap / leading batch dimensions): the same launches for all of them where the
+ * workspace for it (the query beside each) stays below 1 GiB, else in passes.  Masks and distances are contiguous
+ * (batch, n) arrays; the optional input mask of the crowding distances is addressed as
+ * mask[b * mask_batch_stride + i * mask_stride] (bytes). */
+size_t evox_hip_many_first_front_workspace_bytes(int64_t batch, int64_t n, int64_t m);
+int evox_hip_many_first_front_mask(const float* f, int64_t batch, int64_t n, int64_t m, int64_t stride_batch, int64_t stride_row,
+                                   int64_t stride_col, uint8_t* mask_out, void* workspace, size_t workspace_bytes, void* stream);
+size_t evox_hip_many_crowding_workspace_bytes(int64_t batch, int64_t n, int64_t m);
+int evox_hip_many_crowding_distance(const float* costs, int64_t batch, int64_t n, int64_t m, int64_t stride_batch,
+                                    int64_t stride_row, int64_t stride_col, const uint8_t* mask, int64_t mask_batch_stride,
+                                    int64_t mask_stride, float* dist_out, void* workspace, size_t workspace_bytes, void* stream);
+
 /* One small population given in two parts of equal strides (parents and offspring of NSGA-II,
  * src/evox/algorithms/mo/nsga2.py:99-102, at the population sizes such runs mostly have: a few hundred rows): the
  * selection of evox_hip_nd_environmental_selection_two_part in the one-workgroup kernel of the entry points above,

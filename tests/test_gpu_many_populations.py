@@ -150,3 +150,41 @@ def test_a_wait_that_runs_out_poisons_every_population():
     for b in range(8):
         want, _fronts = c_oracle.nd_rank(f[b])
         assert np.array_equal(as_np(again[b]), as_np(want))
+
+
+@pytest.mark.parametrize("batch,n,m,kind", [(5, 3000, 3, "ties"), (12, 1500, 2, "uniform"), (3, 40000, 3, "uniform"),
+                                            (4, 9000, 8, "one_front"), (2, 2000, 17, "ties"), (70, 1100, 3, "fronts")])
+def test_first_front_and_crowding_of_many_populations(batch, n, m, kind):
+    """The first-front mask and the crowding distances under leading batch dimensions: one set of launches for all
+    populations, the same results as population by population."""
+    from evox_amd.operators.selection import crowding_distance, non_dominated_mask
+    from oracle import eager_restatement as er
+
+    f, _ = _populations(batch, n, m, 300 + batch + n + m, kind)
+    fd = f.to(DEV)
+    first = non_dominated_mask(fd)
+    assert first.shape == (batch, n) and first.dtype == torch.bool
+    g = torch.Generator("cpu").manual_seed(batch)
+    mask = torch.rand(batch, n, generator=g) < 0.3
+    mask[0] = False  # an empty selection
+    mask[batch - 1] = True
+    maskd = mask.to(DEV)
+    dist_all = crowding_distance(fd, None)
+    dist_masked = crowding_distance(fd, maskd)
+    dist_front = crowding_distance(fd, first)
+    assert runtime.last_status()["error"] == 0
+    for b in range(batch):
+        assert torch.equal(first[b], non_dominated_mask(fd[b])), b
+        for got, mk in ((dist_all, None), (dist_masked, maskd[b]), (dist_front, first[b])):
+            assert np.array_equal(as_np(got[b]), as_np(crowding_distance(fd[b], mk)), equal_nan=True), b
+    for b in range(0, batch, max(1, batch // 2)):
+        want_first = as_np(c_oracle.nd_rank(f[b])[0]) == 0
+        assert np.array_equal(as_np(first[b]), want_first), b
+        want = as_np(er.crowding(f[b], mask[b]))
+        got = as_np(dist_masked[b])
+        fin = np.isfinite(want)
+        assert np.array_equal(np.isfinite(got), fin) and np.array_equal(got[~fin], want[~fin], equal_nan=True), b
+        np.testing.assert_allclose(got[fin], want[fin], rtol=1e-5)
+    # a mask that is a strided view, populations along the second dimension
+    mapped = torch.vmap(crowding_distance, in_dims=(1, 1))(fd.permute(1, 0, 2).contiguous(), maskd.t().contiguous())
+    assert np.array_equal(as_np(mapped), as_np(dist_masked), equal_nan=True)
