@@ -22,6 +22,7 @@
 #include "radix.hpp"
 #include "stepped.hpp"
 #include "two.hpp"
+#include "two_small.hpp"
 #include "wide.hpp"
 
 namespace evx {
@@ -40,6 +41,8 @@ struct Options {
   int peel_lds_blocks = 0;  // sweeping workgroups of that kernel, 0 = by size
   int peel_stepped = 0;     // 1: the fronts are peeled one launch each by kernels that never wait for each other (stepped.hpp),
                             // and the last front is ordered likewise; 0: only where the persistent grids cannot be resident
+  int64_t two_small_min_rows = 128;  // populations of two objectives and at least this many rows (at most 4096) that go to a
+                                   // one-workgroup kernel take the one without a matrix (two_small.hpp); 0 = never
   int64_t two_min_rows = 4097;  // populations of two objectives and at least this many rows are ranked without a matrix (two.hpp); 0 = never
   int64_t two_min_rows_partial = 24576;  // ... when the ranking may stop at the front that holds a given row (that path always
                                          // peels every front: measured, us per selection of half the rows, without / with a matrix:
@@ -1191,7 +1194,34 @@ static int launch_batched_m(const BatchedArgs& a, int64_t batch, hipStream_t s) 
   return 0;
 }
 
+// Two objectives: one workgroup per population without a matrix (two_small.hpp), for up to kTwoSmallRows rows.
+static int launch_two_small(const BatchedArgs& a, int64_t batch, hipStream_t s) {
+  if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(two_small_kernel), kTwoSmallLdsBytes)) return e;
+  for (int64_t b0 = 0; b0 < batch; b0 += 0x40000000ll) {
+    BatchedArgs part = a;
+    const int64_t nb = batch - b0 < 0x40000000ll ? batch - b0 : 0x40000000ll;
+    part.f += b0 * a.f_stride_b;
+    if (part.rank_all) part.rank_all += b0 * a.n;
+    if (part.x) part.x += b0 * a.x_stride_b;
+    if (part.out_x) part.out_x += b0 * a.stop_count * a.x_row_bytes;
+    if (part.out_f) part.out_f += b0 * a.stop_count * a.m;
+    if (part.out_rank) part.out_rank += b0 * a.stop_count;
+    if (part.out_dist) part.out_dist += b0 * a.stop_count;
+    hipLaunchKernelGGL(two_small_kernel, dim3((unsigned)nb), dim3(kTwoSmallThreads), kTwoSmallLdsBytes, s, part);
+    EVX_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+// Rows that the one-workgroup kernels take: the matrix kernel up to kBatchedMaxRows, two objectives up to kTwoSmallRows.
+static int64_t batched_rows_limit(int64_t m) {
+  if (m < 1 || m > kBatchedMaxObjectives) return 0;
+  return m == 2 && opt().two_small_min_rows > 0 ? kTwoSmallRows : kBatchedMaxRows;
+}
+
 static int launch_batched(const BatchedArgs& a, int64_t batch, hipStream_t s) {
+  if (a.m == 2 && opt().two_small_min_rows > 0 && (a.n >= opt().two_small_min_rows || a.n > kBatchedMaxRows))
+    return launch_two_small(a, batch, s);
   switch (a.m) {
     case 1: return launch_batched_m<1>(a, batch, s);
     case 2: return launch_batched_m<2>(a, batch, s);
@@ -1276,6 +1306,8 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.launch_memory = (int)value;
   } else if (!strcmp(name, "peel_stepped") && (value == 0 || value == 1)) {
     o.peel_stepped = (int)value;
+  } else if (!strcmp(name, "two_small_min_rows") && value >= 0) {
+    o.two_small_min_rows = value;
   } else if (!strcmp(name, "two_min_rows") && value >= 0) {
     o.two_min_rows = value;
     if (value < o.two_min_rows_partial) o.two_min_rows_partial = value;  // (a lower limit asked for counts for both)
@@ -2263,11 +2295,11 @@ int evox_hip_nd_environmental_selection_static(const void* x, int64_t x_row_byte
                      out_f, out_rank, out_dist, out_order, ws, (size_t)EVOX_HIP_STATIC_SCRATCH_BYTES, (hipStream_t)stream, false);
 }
 
-int64_t evox_hip_batched_max_rows(int64_t m) { return (m >= 1 && m <= kBatchedMaxObjectives) ? kBatchedMaxRows : 0; }
+int64_t evox_hip_batched_max_rows(int64_t m) { return batched_rows_limit(m); }
 
 int evox_hip_batched_non_dominate_rank(const float* f, int64_t batch, int64_t n, int64_t m, int64_t stride_batch,
                                        int64_t stride_row, int64_t stride_col, int32_t* rank_out, void* stream) {
-  if (f == nullptr || rank_out == nullptr || batch < 1 || n < 1 || n > kBatchedMaxRows || m < 1 || m > kBatchedMaxObjectives) return kErrBadArg;
+  if (f == nullptr || rank_out == nullptr || batch < 1 || n < 1 || n > batched_rows_limit(m)) return kErrBadArg;
   BatchedArgs a = {};
   a.f = f;
   a.f_stride_b = stride_batch;
@@ -2286,7 +2318,7 @@ int evox_hip_batched_nd_environmental_selection(const void* x, int64_t x_row_byt
                                                 int64_t topk, void* out_x, float* out_f, int32_t* out_rank, float* out_dist,
                                                 void* stream) {
   if (f == nullptr || out_f == nullptr || out_rank == nullptr || out_dist == nullptr) return kErrBadArg;
-  if (batch < 1 || n < 1 || n > kBatchedMaxRows || m < 1 || m > kBatchedMaxObjectives || topk < 1 || topk > n) return kErrBadArg;
+  if (batch < 1 || n < 1 || n > batched_rows_limit(m) || topk < 1 || topk > n) return kErrBadArg;
   if ((x == nullptr) != (out_x == nullptr) || (x != nullptr && (x_row_bytes < 0 || x_row_stride_bytes < 0))) return kErrBadArg;
   BatchedArgs a = {};
   a.f = f;
@@ -2319,7 +2351,7 @@ int evox_hip_small_nd_environmental_selection_two_part(const void* x_a, const vo
                                                        int64_t stride_col, int64_t topk, void* out_x, float* out_f,
                                                        int32_t* out_rank, float* out_dist, void* stream) {
   if (f_a == nullptr || f_b == nullptr || out_f == nullptr || out_rank == nullptr || out_dist == nullptr) return kErrBadArg;
-  if (n_a < 1 || n_b < 1 || n_a + n_b > kBatchedMaxRows || m < 1 || m > kBatchedMaxObjectives) return kErrBadArg;
+  if (n_a < 1 || n_b < 1 || n_a + n_b > batched_rows_limit(m)) return kErrBadArg;
   const int64_t n = n_a + n_b;
   if (topk < 1 || topk > n) return kErrBadArg;
   if ((x_a == nullptr) != (out_x == nullptr) || (x_a == nullptr) != (x_b == nullptr)) return kErrBadArg;

@@ -115,8 +115,8 @@ __device__ inline int position_by_counting(const uint64_t* tile, int* below, int
 // The selected rows of x as one flat array of units of type T (4 or 16 bytes): unit e of the output is unit
 // e % row_units of input row order[e / row_units].  Four units per thread are in flight: a load that waits
 // for the store before it costs a memory round trip per unit.
-template <class T>
-__device__ inline void gather_units(const uint8_t* __restrict__ xb, uint8_t* __restrict__ dst, const int* order,
+template <class T, class Index>
+__device__ inline void gather_units(const uint8_t* __restrict__ xb, uint8_t* __restrict__ dst, const Index* order,
                                     int64_t x_row_stride, uint32_t row_units, uint32_t total, int j, int nt,
                                     int n_first, int64_t x_second) {
   auto row_at = [&](uint32_t p) {

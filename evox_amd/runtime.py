@@ -42,6 +42,12 @@ _batched_max_rows = {}  # objectives -> rows that the one-workgroup kernel takes
 def small_population_kernel_fits(n: int, m: int, batch: int) -> bool:
     if use_small_population_kernel is False:
         return False
+    if m == 2:
+        # (two objectives have a one-workgroup kernel of their own, which takes up to 4096 rows and beats the pipeline
+        # at every size; a tunable switches it off, so the library is asked every time)
+        most = int(_lib.lib().evox_hip_batched_max_rows(m))
+        return 1 <= n <= most and (most > 1024 or use_small_population_kernel is True or batch >= 4
+                                   or n <= _lone_population_limit(m) * (1 if batch == 1 else 2))
     most = _batched_max_rows.get(m)
     if most is None:
         most = _batched_max_rows[m] = int(_lib.lib().evox_hip_batched_max_rows(m))

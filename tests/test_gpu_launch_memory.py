@@ -16,6 +16,13 @@ pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda", 0)
 
 
+@pytest.fixture(autouse=True)
+def through_the_pipeline():
+    runtime.use_small_population_kernel = False  # (the one-workgroup kernels have no such choice to make)
+    yield
+    runtime.use_small_population_kernel = None
+
+
 def _check(f, k, got):
     order, rank, dist, _ = c_oracle.select(as_np(f), k)
     xs, fs, rs, ds = got
