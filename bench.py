@@ -362,7 +362,7 @@ def next_rows(dev, reps):
             "all_in_one_call_us": event_time_us(lambda: nd_environmental_selection(xm, fm, n // 2), reps),
             "one_alone_us": event_time_us(lambda: nd_environmental_selection(xm[0], fm[0], n // 2), reps)}
         del fm, xm
-    # two objectives: ranked without a dominance matrix from 4097 rows on (all fronts) / 24576 rows on (up to a cut)
+    # two objectives: ranked without a dominance matrix from 4097 rows on
     for n in (50000, 200000):
         f2, x2 = workloads.uniform_population(n, 2, 16, 8)
         f2, x2 = f2.to(dev), x2.to(dev)

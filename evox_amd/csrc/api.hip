@@ -44,9 +44,9 @@ struct Options {
   int64_t two_small_min_rows = 128;  // populations of two objectives and at least this many rows (at most 4096) that go to a
                                    // one-workgroup kernel take the one without a matrix (two_small.hpp); 0 = never
   int64_t two_min_rows = 4097;  // populations of two objectives and at least this many rows are ranked without a matrix (two.hpp); 0 = never
-  int64_t two_min_rows_partial = 24576;  // ... when the ranking may stop at the front that holds a given row (that path always
-                                         // peels every front: measured, us per selection of half the rows, without / with a matrix:
-                                         // 20 000 rows 399 / 361, 50 000 rows 715 / 1181; all ranks: 5000 rows 185 / 332)
+  int64_t two_min_rows_partial = 4097;  // ... when the ranking may stop at the front that holds a given row (measured, us per
+                                        // selection of half the rows, without / with a matrix: 5000 rows 110 / 178, 20 000 rows
+                                        // 218 / 362, 50 000 rows 324 / 1181; all ranks: 5000 rows 140 / 332)
   int peel_tail = 1;        // that kernel also orders a small last front (0: always the kernels of finish.hpp)
   int tail_merged = 1;      // after such a peel, ordering (where still needed) and gather share one launch
   int launch_memory = 1;    // ... unless the last selection of this shape had a last front that the peel left alone
@@ -1633,8 +1633,9 @@ static bool make_sort_layout(int64_t n, SortLayout* L) {
   return true;
 }
 
+// key_cap: see argsort_step_kernel (device memory or null; only the sort of more than kMidArgsortRows keys looks at it).
 static int argsort_step(const void* key, int kind, int64_t stride, int64_t n, const int32_t* prev_order, int32_t* order_out,
-                        void* ws, size_t ws_bytes, void* stream) {
+                        void* ws, size_t ws_bytes, void* stream, const int* key_cap = nullptr) {
   SortLayout L;
   if (key == nullptr || order_out == nullptr || kind < 0 || kind > 2) return kErrBadArg;
   if (!make_sort_layout(n, &L)) return kErrBadArg;
@@ -1681,7 +1682,7 @@ static int argsort_step(const void* key, int kind, int64_t stride, int64_t n, co
   if (workers > cap) workers = cap;
   if (workers < 1) workers = 1;
   hipLaunchKernelGGL(argsort_step_kernel, dim3(workers + kFirstSweeper), dim3(kRadixThreads), kRadixLdsBytes, s, key, kind,
-                     stride, L.n, prev_order, reinterpret_cast<Ctrl*>(base + L.ctrl), b, order_out, opt().spin_limit);
+                     stride, L.n, prev_order, reinterpret_cast<Ctrl*>(base + L.ctrl), b, order_out, opt().spin_limit, key_cap);
   EVX_LAUNCH_CHECK();
   // (an order of -1 everywhere when one of the sort's grid barriers ran out)
   return copy_out(reinterpret_cast<const Ctrl*>(base + L.ctrl), order_out, nullptr, n, kPoisonIndex, s);
@@ -1890,7 +1891,7 @@ static int stage_rank_two(const Ws& w, const Fitness& src, int64_t stop_count, b
   const float* xs_sorted = w.at<float>(L.xs_sorted);
   hipLaunchKernelGGL(two_peel_kernel, dim3(blocks), dim3(kTwoThreads), 0, s, xs_sorted, xs_sorted + L.npad, w.at<uint32_t>(L.kid_sorted),
                      w.at<int>(L.orig_of), L.n, w.at<int>(L.rank), fill_dist ? w.at<float>(L.dist) : (float*)nullptr, w.ctrl(),
-                     w.at<unsigned long long>(L.two_ring), opt().spin_limit);
+                     w.at<unsigned long long>(L.two_ring), opt().spin_limit, (int)stop_count);
   EVX_LAUNCH_CHECK();
   int grid = (L.n + 255) / 256;
   if (grid > device_cus() * 8) grid = device_cus() * 8;
@@ -1898,8 +1899,8 @@ static int stage_rank_two(const Ws& w, const Fitness& src, int64_t stop_count, b
                      xs_sorted + L.npad, L.n, w.at<int>(L.rank), w.ctrl());
   EVX_LAUNCH_CHECK();
   uint8_t* wb = w.base + L.wide;
-  if (int e = evox_hip_stable_argsort_step(w.at<int>(L.rank), kKeyInt32, 1, L.n, nullptr, w.at<int>(L.perm), wb + WL.sort_ws,
-                                           WL.sort_bytes, s))
+  if (int e = argsort_step(w.at<int>(L.rank), kKeyInt32, 1, L.n, nullptr, w.at<int>(L.perm), wb + WL.sort_ws, WL.sort_bytes, s,
+                           &w.ctrl()->reserved[kTwoRounds]))
     return e;
   hipLaunchKernelGGL(two_bounds_kernel, dim3(grid), dim3(256), 0, s, w.at<int>(L.perm), w.at<int>(L.rank), L.n, w.at<int>(L.fstart),
                      w.ctrl(), (int)stop_count);

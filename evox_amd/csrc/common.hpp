@@ -154,7 +154,8 @@ struct Ctrl {
   int radix_epoch;  // runs of a radix sort kernel so far: each takes a fresh range of barrier generations
   int tail_done;    // the peel kernel has also left the crowding distances and the order of the last front
   int reserved[6];  // [0], [1], [3]: arrival counters of the barriers inside the kernels that order the last front;
-                    // [2]: that of the barriers inside the slot sort; [5]: the level that the launch-per-front
+                    // [2]: that of the barriers inside the slot sort; [4]: the rounds that the last workgroup of
+                    // the two-objective ranking went through (two.hpp); [5]: the level that the launch-per-front
                     // path has finished (stepped.hpp)
   // grid barrier: block 0 publishes (generation << 32 | rows found by all blocks) in `release` and in
   // kReleaseCopies copies of it, one per 128-byte line, so that the waiting blocks do not all poll one

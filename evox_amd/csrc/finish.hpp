@@ -54,7 +54,7 @@ __device__ inline bool counter_barrier(Ctrl* ctrl, int which, int target, unsign
 constexpr int kFusedFrontRows = 2048;
 constexpr int kFusedFrontValues = 4096;  // candidates x objectives held in LDS: 12 bytes each
 constexpr int kFusedFrontObjectives = 64;
-constexpr int kFusedSoloRows = 512;       // up to here one workgroup does it all
+constexpr int kFusedSoloRows = 128;       // up to here one workgroup does it all (450 rows of two objectives in one workgroup: 100 us, in 29: 20)
 constexpr size_t kFusedFrontLdsBytes =
     12 * (size_t)kFusedFrontValues + 4 * (size_t)kFusedFrontRows + 16 * kFusedFrontObjectives + 4 * (size_t)kFusedSoloRows;
 
@@ -77,9 +77,13 @@ __device__ inline void crowd_small_front(const float* __restrict__ xs, int npad,
   // A front of a few hundred rows is the work of one workgroup: the others would only repeat its loads and then
   // make it wait for them at the barrier below.
   const bool solo = nv <= kFusedSoloRows;
+  // ... and a front of up to kFusedFrontRows rows that of as many workgroups as have sixteen candidates each: the
+  // barrier below costs every workgroup that arrives a write-back and an invalidation of its die's cache (the 512
+  // workgroups of the grid of a population of 200 000 rows: 100 us for a front of 600 rows)
+  const int active = solo ? 1 : min((int)gridDim.x, (nv + (int)(blockDim.x >> 4) - 1) / (int)(blockDim.x >> 4));
   if (mode == 2)  // the better fronts keep the order in which they are listed
     for (int i = blockIdx.x * blockDim.x + tid; i < start; i += gridDim.x * blockDim.x) order[i] = list_base[i];
-  if (solo && blockIdx.x != 0) return;
+  if ((int)blockIdx.x >= active) return;
   for (int e = tid; e < nv; e += blockDim.x) lst[e] = list[e];
   __syncthreads();
   for (int i = tid; i < nv * m; i += blockDim.x) {
@@ -110,7 +114,7 @@ __device__ inline void crowd_small_front(const float* __restrict__ xs, int npad,
     }
   }
   __syncthreads();
-  const int groups = (solo ? 1 : gridDim.x) * (blockDim.x >> 4);
+  const int groups = active * (blockDim.x >> 4);
   uint32_t* dkey_lds = reinterpret_cast<uint32_t*>(ends + 2 * kFusedFrontObjectives);  // [kFusedSoloRows], solo only
   for (int q = blockIdx.x * (blockDim.x >> 4) + (tid >> 4); q < nv; q += groups) {
     bool boundary = false;
@@ -158,7 +162,7 @@ __device__ inline void crowd_small_front(const float* __restrict__ xs, int npad,
     __syncthreads();
   } else {
     // every block has stored its distance keys
-    if (!counter_barrier(ctrl, 0, (int)gridDim.x, spin_limit, scratch)) return;
+    if (!counter_barrier(ctrl, 0, active, spin_limit, scratch)) return;
     for (int e = tid; e < nv; e += blockDim.x) comp[e] = ((unsigned long long)dkey[e] << 32) | (unsigned)e;
     __syncthreads();
   }

@@ -38,7 +38,8 @@ struct RadixBuffers {
 };
 
 // Sorts `nseg` segments of nv pairs; pair e of segment k is initial(k, e) (candidate order), the
-// result is left in buf.pairs[0] (four passes: initial -> pairs[1] -> pairs[0] -> pairs[1] -> pairs[0]).
+// result is left in buf.pairs[0] (four passes: initial -> pairs[1] -> pairs[0] -> pairs[1] -> pairs[0]; `passes` = 2
+// where every key is below 65536: the same in all blocks, and the master runs three barriers per pass).
 // Must be called by every thread of every block with blockIdx.x >= kFirstSweeper; block 0 must run
 // radix_master().  `lds` = kRadixLdsBytes of LDS; `base` = LDS, 256 ints; `scratch` as for the barrier.
 //
@@ -51,7 +52,8 @@ constexpr size_t kRadixLdsBytes = sizeof(int) * 6 * 256 + sizeof(unsigned long l
 
 template <class Initial>
 __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, int nv, Initial initial, Ctrl* ctrl,
-                                           unsigned gen0, unsigned spin_limit, int* lds, int* base, int* scratch) {
+                                           unsigned gen0, unsigned spin_limit, int* lds, int* base, int* scratch,
+                                           int passes = 4) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int tid = threadIdx.x;  // blockDim.x == 256
@@ -84,7 +86,7 @@ __device__ inline bool radix_sort_segments(const RadixBuffers& buf, int nseg, in
   };
   unsigned gen = gen0;
   int dummy = 0;
-  for (int pass = 0; pass < 4; ++pass) {
+  for (int pass = 0; pass < passes; ++pass) {
     const int shift = 8 * pass;
     // (chosen, not indexed: an array indexed at run time lives in scratch memory, which every lane of every kernel that
     // holds a RadixBuffers then writes when it starts -- 10 MB per launch of the 1024-thread ordering kernel)
@@ -232,19 +234,26 @@ __device__ inline unsigned radix_generation_base(const Ctrl* ctrl) { return 0x80
 //     sorted_indices = sorted_indices.gather(dim, step)
 // -- and the first step with prev == nullptr (the identity).  The caller chains one launch per key.
 // kind 0: float32 keys, 1: int32 keys, 2: uint32 keys; `stride` in elements.
+// key_cap (device memory, or null): int32 keys that are not negative are sorted as min(key, *key_cap) -- two passes
+// instead of four where the cap is below 65536 (the ranks of a population, whose number of fronts an earlier kernel
+// has left there; rows without a rank stand behind all others either way).
 enum KeyKind { kKeyFloat32 = 0, kKeyInt32 = 1, kKeyUint32 = 2 };
 
 __global__ __launch_bounds__(kRadixThreads) void argsort_step_kernel(const void* __restrict__ key, int kind, int64_t stride,
                                                                      int n, const int* __restrict__ prev,
                                                                      Ctrl* __restrict__ ctrl, RadixBuffers buf,
-                                                                     int* __restrict__ order_out, unsigned spin_limit) {
+                                                                     int* __restrict__ order_out, unsigned spin_limit,
+                                                                     const int* __restrict__ key_cap) {
   extern __shared__ int radix_lds[];
   __shared__ int base[256];
   __shared__ int scratch[kRadixThreads];
   if (coherent_load(&ctrl->err) != 0) return;
   const unsigned gen0 = radix_generation_base(ctrl);
+  const bool capped = key_cap != nullptr && kind == kKeyInt32;
+  const uint32_t cap = capped ? (uint32_t)*key_cap : 0xFFFFFFFFu;
+  const int passes = capped && cap < 65536u ? 2 : 4;
   if (blockIdx.x == 0) {
-    radix_master(ctrl, gen0, 12, spin_limit, scratch);
+    radix_master(ctrl, gen0, 3 * passes, spin_limit, scratch);
     if (threadIdx.x == 0) ctrl->radix_epoch += 1;  // nobody reads it again in this kernel
     return;
   }
@@ -260,13 +269,15 @@ __global__ __launch_bounds__(kRadixThreads) void argsort_step_kernel(const void*
     uint32_t k;
     if (kind == kKeyFloat32)
       k = ordered_key(static_cast<const float*>(key)[(int64_t)idx * stride]);
+    else if (capped)
+      k = min(static_cast<const uint32_t*>(key)[(int64_t)idx * stride], cap);
     else if (kind == kKeyInt32)
       k = static_cast<const uint32_t*>(key)[(int64_t)idx * stride] ^ 0x80000000u;
     else
       k = static_cast<const uint32_t*>(key)[(int64_t)idx * stride];
     return ((unsigned long long)k << 32) | (unsigned)idx;
   };
-  if (!radix_sort_segments(buf, 1, n, initial, ctrl, gen0, spin_limit, radix_lds, base, scratch)) return;
+  if (!radix_sort_segments(buf, 1, n, initial, ctrl, gen0, spin_limit, radix_lds, base, scratch, passes)) return;
   for (int p = wb * blockDim.x + threadIdx.x; p < n; p += workers * blockDim.x)
     order_out[p] = (int)(unsigned)(coherent_load(&buf.pairs[0][p]) & 0xFFFFFFFFull);
 }

@@ -9,32 +9,67 @@
 // objective is no larger: the front of what remains is the set of strict prefix minima of the second objective.
 // Each round of the peeling is therefore one prefix-minimum scan, O(n) work and no n^2 anywhere, where the matrix
 // formulation pays n^2 / 2 pair tests and a pass over bit rows per front (two objectives give many thin fronts:
-// 380 of them at 200 000 rows).
+// 880 of them at 200 000 rows).
 //
 // The scan of a round runs through the workgroups like a bucket brigade: workgroup b owns a run of slots, receives
-// the minimum over the remaining rows before its run from workgroup b - 1, hands min(that, its own minimum) on to
-// workgroup b + 1 AT ONCE -- before its own scan -- and then ranks its rows.  A round costs a workgroup one scan in
-// registers and LDS, and the rounds of different workgroups overlap: F fronts over B workgroups take about F + B
-// hand-overs, not F * B.  A workgroup only ever waits for the one before it (and, when it is a whole ring of rounds
-// ahead, for the one after it); all waits are bounded.  Rows holding a NaN neither dominate nor are dominated: rank 0,
-// and they take no part.
+// the minimum over the remaining rows before its run from workgroup b - 1 and hands min(that, its own minimum) on to
+// workgroup b + 1.  The rounds of different workgroups overlap: F fronts over B workgroups take F rounds of the last
+// workgroup plus what the B hand-overs put between the first workgroup's start and the last one's, not F * B.  A
+// workgroup only ever waits for the one before it (and, when it is a whole ring of rounds ahead, for the one after
+// it); all waits are bounded.  Rows holding a NaN neither dominate nor are dominated: rank 0, and they take no part.
+//
+// A round inside a workgroup is ONE barrier: every wave leaves the prefix minimum of its rows in LDS, and behind the
+// barrier every wave reads the sixteen wave minima and the incoming minimum and ranks its own rows.  Everything that
+// talks to other workgroups happens beside that, in single lanes of different waves, because a wave waits for its
+// memory operations in the order of their issue (a load that has to see another workgroup's store takes over a
+// microsecond -- two rounds -- and a write-through store as long):
+//   * the word of round q is asked for kTwoAhead rounds ahead by the first lane of wave q mod kTwoAhead and taken
+//     in -- tag checked, polled for if it is late -- right behind the barrier of round q - 1, so that it lies in LDS
+//     at the barrier of round q.  These waves issue no store inside the loop (the ranks stay in registers until the
+//     kernel ends), so the only thing such a lane ever waits for is its own load of kTwoAhead rounds ago;
+//   * the first lane of the last wave publishes: behind the barrier of round r it counts what round r - 1 ranked,
+//     stores the word of round r for the next workgroup and the progress counter for the one before, and decides
+//     whether the workgroup is done (seen by all waves behind the next barrier).  It loads nothing but, once every
+//     ring of rounds, the progress of the workgroup after.
+// A workgroup whose words come late polls for them and thereby falls behind the one before it, until it is far enough
+// behind for its words to be there when it asks (about kTwoAhead rounds and the time a store takes to be seen: 3 to
+// 5 us per workgroup of the chain).  A round takes 0.65 us -- instruction issue: sixteen waves of some eighty
+// instructions on four SIMDs; half as many waves with twice the rows each take as long, since one or two waves per
+// SIMD wait nine clocks for every dependent instruction instead of four -- where the two barriers and the one
+// thread between them of an earlier form of this kernel took 1.25.  Falling back on purpose (a sleep after the first
+// late word) and asking three, four or six rounds ahead were measured and are slower.
 #pragma once
 
 #include "peel.hpp"
 
 namespace evx {
 
-// (256 threads x 16 slots, one wave per SIMD, was slower: 1.5 against 0.75 us per round -- the running minimum over a
-// thread's own slots is a chain of dependent instructions that no other wave hides.)
 constexpr int kTwoThreads = 1024;
-constexpr int kTwoPerThread = 4;                             // consecutive slots per thread
-constexpr int kTwoChunk = kTwoThreads * kTwoPerThread;       // slots per workgroup
+constexpr int kTwoWaves = kTwoThreads / 64;
+constexpr int kTwoChunk = 4096;                              // slots per workgroup
+constexpr int kTwoPerThread = kTwoChunk / kTwoThreads;       // consecutive slots per thread
 constexpr int kTwoMaxBlocks = 256;
 constexpr int64_t kTwoMaxRows = (int64_t)kTwoChunk * kTwoMaxBlocks;
 constexpr int kTwoRing = 256;                                // rounds of a workgroup's outgoing stream that are kept
 constexpr int kTwoRingStride = kTwoRing + 16;                // words per workgroup: the ring, then its progress counter on a line of its own
+constexpr int kTwoAhead = 2;                                 // rounds between asking for a word and taking it in; as many waves take turns
+constexpr int kTwoPublisher = kTwoThreads - 64;              // the thread that stores
+constexpr int kTwoRounds = 4;                                // Ctrl.reserved[kTwoRounds]: the rounds of the last workgroup (every rank up to the cut is below it)
 constexpr uint32_t kTwoNone = 0xFFFFFFFFu;                   // "no remaining row": larger than every image of a number
-constexpr unsigned kTwoEnd = 0x80000000u;                    // in a word's tag: nothing remains in this workgroup or before it
+// A word of a ring: the minimum in the low half; in the high half bit 31 "nothing remains in this workgroup or before
+// it", bits 30:29 the generation of the ring slot (1..3, 0 = never written: the ring starts zeroed), bits 28:0 the
+// number of rows that this workgroup and those before it have ranked in the rounds before the word's round.
+constexpr unsigned kTwoEnd = 0x80000000u;
+constexpr unsigned kTwoTagShift = 29;
+constexpr unsigned kTwoCountMask = (1u << kTwoTagShift) - 1u;
+__device__ inline unsigned two_tag(int round) { return (unsigned)((round / kTwoRing) % 3) + 1u; }
+__device__ inline unsigned two_tag_of(unsigned long long word) { return ((unsigned)(word >> 32) >> kTwoTagShift) & 3u; }
+static_assert(kTwoMaxRows <= (int64_t)kTwoCountMask, "the count of ranked rows must fit its field");
+static_assert(kTwoAhead <= kTwoWaves - 1 && kTwoAhead < kTwoRing, "the lanes that load and the lane that stores sit in different waves");
+static_assert(kTwoWaves <= 16, "the wave minima are reduced inside rows of sixteen lanes");
+// flags of an incoming word as the waves see it in LDS
+constexpr uint32_t kTwoInEnded = 1u;  // nothing remains before this workgroup, from this round on
+constexpr uint32_t kTwoInStop = 2u;   // leave now: a wait ran out, or enough rows are ranked everywhere
 
 // Inclusive prefix minimum over the lanes of a wave (DPP row shifts and row broadcasts).
 __device__ inline uint32_t wave_prefix_min(uint32_t x) {
@@ -49,30 +84,57 @@ __device__ inline uint32_t wave_prefix_min(uint32_t x) {
   return v;
 }
 
+// What a receiving lane asks for ahead of time -- the word of its next round and the "enough" flag -- lands in
+// the accumulation registers a0..a2, which the compiler uses for nothing in this kernel.  Asked for into ordinary
+// registers, the loads would be followed at the end of the loop body by the compiler's copies of those registers
+// and the wait that a copy needs: a memory round trip in every round.
+__device__ __forceinline__ void two_ask(const unsigned long long* word, const int* flag) {
+  asm volatile("global_load_dwordx2 a[0:1], %0, off sc1\n\tglobal_load_dword a2, %1, off sc1" ::"v"(word), "v"(flag) : "memory", "a0", "a1", "a2");
+}
+__device__ __forceinline__ void two_take(unsigned long long* word, int* flag) {
+  unsigned lo, hi, en;
+  asm volatile("s_waitcnt vmcnt(0)\n\tv_accvgpr_read_b32 %0, a0\n\tv_accvgpr_read_b32 %1, a1\n\tv_accvgpr_read_b32 %2, a2"
+               : "=v"(lo), "=v"(hi), "=v"(en)::"memory");
+  *word = ((unsigned long long)hi << 32) | lo;
+  *flag = (int)en;
+}
+
 // Grid: ceil(n / kTwoChunk) workgroups of kTwoThreads.  xs1_sorted / xs2_sorted: the objectives by slot (rows sorted by
 // (f1, f2, index)); kid: first slot of the slot's key.  Writes the rank of every row that is the first of its key
-// (by original index), rank 0 for rows holding a NaN, and the -inf fill of the distances; every front is peeled.
+// (by original index), rank 0 for rows holding a NaN, and the -inf fill of the distances.  stop_count >= n: every front
+// is peeled.  stop_count < n: the peeling may end once the fronts so far hold stop_count rows -- the last workgroup,
+// which sees the count of all workgroups a round late, raises a flag that the others find a few rounds later;
+// rows not ranked by then are left at kRankUnset, and a front after the one that holds the stop_count-th row may be
+// ranked in part.  Only first rows of a key count (copies and rows with a NaN do not): the peeling never ends before
+// the stop_count-th row has its rank, and goes through all fronts where copies make up the difference.
 // ring: gridDim.x * kTwoRingStride words, zero at the start of the call.
 __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __restrict__ xs1_sorted, const float* __restrict__ xs2_sorted,
                                                                const uint32_t* __restrict__ kid, const int* __restrict__ orig_of,
                                                                int n, int* __restrict__ rank, float* __restrict__ dist_fill,
                                                                Ctrl* __restrict__ ctrl, unsigned long long* __restrict__ ring,
-                                                               unsigned spin_limit) {
-  __shared__ __attribute__((aligned(16))) uint32_t wave_min_lds[2][kTwoThreads / 64];  // by the parity of the round: a wave may be a round ahead of another's reads
-  __shared__ uint32_t in_lds[2];  // the round's incoming minimum; 1 when the workgroup leaves after this round's hand-over
-  __shared__ uint32_t before_lds[kTwoThreads / 64];  // the minimum over the waves before each wave
-  __shared__ int ranked_lds;      // rows this workgroup ranked in the round
+                                                               unsigned spin_limit, int stop_count) {
+  __shared__ __attribute__((aligned(16))) uint32_t wave_min_lds[2][16];  // by the parity of the round; entries from kTwoWaves on stay "none"
+  // by the parity of the round: incoming minimum, rows ranked before this workgroup, flags (these three from the
+  // round's receiver), "the workgroup leaves behind this round's barrier" (from the publisher)
+  __shared__ __attribute__((aligned(16))) uint32_t in_lds[2][4];
+  __shared__ int ranked_lds[2];    // rows this workgroup ranked in a round, by the parity of the round
+  __shared__ int unranked_lds[kTwoWaves];
   if (coherent_load(&ctrl->err) != 0) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int b = blockIdx.x;
   const bool last_block = b == (int)gridDim.x - 1;
   unsigned long long* my_ring = ring + (size_t)b * kTwoRingStride;
   const unsigned long long* up_ring = ring + (size_t)(b > 0 ? b - 1 : 0) * kTwoRingStride;
   int* my_progress = reinterpret_cast<int*>(my_ring + kTwoRing);  // rounds of the stream before that this workgroup has taken in
   const int* down_progress = reinterpret_cast<const int*>(ring + (size_t)(last_block ? b : b + 1) * kTwoRingStride + kTwoRing);
+  // "enough rows are ranked": in the spare words behind the last workgroup's ring (whose progress counter nobody reads)
+  int* const enough_flag = reinterpret_cast<int*>(ring + (size_t)(gridDim.x - 1) * kTwoRingStride + kTwoRing + 8);
+  const bool may_stop = stop_count < n;
   // ---- this thread's slots
   uint32_t v[kTwoPerThread];
-  int orig[kTwoPerThread];
+  int orig[kTwoPerThread];   // -1: the slot takes no part
+  int rk[kTwoPerThread];
   int unranked = 0;
   {
     const int s0 = b * kTwoChunk + tid * kTwoPerThread;
@@ -80,7 +142,8 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
     for (int e = 0; e < kTwoPerThread; ++e) {
       const int s = s0 + e;
       v[e] = kTwoNone;
-      orig[e] = 0;
+      orig[e] = -1;
+      rk[e] = kRankUnset;
       if (s < n) {
         const float a1 = xs1_sorted[s], a2 = xs2_sorted[s];
         const int o = orig_of[s];
@@ -95,116 +158,168 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
       }
     }
   }
-  if (tid == 0) ranked_lds = 0;
-  unranked = wave_sum(unranked);
-  if (lane == 0) wave_min_lds[1][wave] = (uint32_t)unranked;
-  __syncthreads();
-  int left = 0;  // (thread 0 keeps the count of this workgroup's unranked rows)
-  if (tid == 0)
-    for (int w = 0; w < kTwoThreads / 64; ++w) left += (int)wave_min_lds[1][w];
-  __syncthreads();
-  bool upstream_ended = b == 0;
-  // (thread 0) the words of the next two rounds are asked for ahead of time: the workgroup before is usually a round
-  // or more ahead, so that a round finds its word there and pays no memory round trip
-  unsigned long long ahead[2] = {0ull, 0ull};
-  if (tid == 0 && !upstream_ended) {
-    ahead[0] = coherent_load(up_ring + 0);
-    ahead[1] = coherent_load(up_ring + (1 % kTwoRing));
+  if (tid == 0) {
+    ranked_lds[0] = 0;
+    ranked_lds[1] = 0;
+    in_lds[0][3] = 0u;
+    in_lds[1][3] = 0u;
   }
-  for (int round = 0;; ++round) {
-    const unsigned tag = (unsigned)round + 1u;
-    // ---- the minimum of this workgroup's remaining rows
+  if (tid < 32) wave_min_lds[tid >> 4][tid & 15] = kTwoNone;
+  unranked = wave_sum(unranked);
+  if (lane == 0) unranked_lds[wave] = unranked;
+  __syncthreads();
+  const bool publisher = tid == kTwoPublisher;
+  const bool receiver = lane == 0 && wave < kTwoAhead;  // takes in the words of the rounds q with q mod kTwoAhead == wave
+  // (publisher) rows of this workgroup without a rank, rows ranked so far by this workgroup, the progress of the
+  // workgroup after this one as last read
+  int left = 0, done_here = 0, down_seen = 0;
+  if (publisher)
+    for (int w = 0; w < kTwoWaves; ++w) left += unranked_lds[w];
+  const bool lower = (lane & 15) < wave;  // this lane's entry of the wave minima belongs to a wave before this one
+  // (receivers) the round whose word is asked for
+  int my_round = wave;
+  if (receiver && (b > 0 || may_stop)) two_ask(up_ring + my_round, enough_flag);
+  // Takes in the word of round q (the caller is the receiver of that round; before: the flags and the count that
+  // round q - 1 saw) and leaves it in LDS for the barrier of round q.
+  auto receive = [&](int q, uint32_t flags_before, uint32_t count_before) {
+    uint32_t in = kTwoNone, count = count_before, flags = flags_before & kTwoInEnded;
+    if (!(flags & kTwoInEnded) || may_stop) {
+      unsigned long long word;
+      int flag_seen;
+      two_take(&word, &flag_seen);
+      bool enough = may_stop && flag_seen != 0;
+      bool failed = false;
+      if (!enough && !(flags & kTwoInEnded)) {
+        const unsigned tag = two_tag(q);
+        if (two_tag_of(word) != tag) {  // late: the workgroup before is not far enough ahead (yet)
+          const unsigned long long* slot = up_ring + (q % kTwoRing);
+          WaitBound bound(spin_limit);
+          for (unsigned spins = 0;; ++spins) {
+            word = coherent_load(slot);
+            if (two_tag_of(word) == tag) break;
+            if (may_stop && (spins & 3u) == 3u && coherent_load(enough_flag) != 0) {  // (the workgroup before may have left on it)
+              enough = true;
+              break;
+            }
+            if (bound.expired(spins) || ((spins & 63u) == 63u && coherent_load(&ctrl->err) != 0)) {
+              failed = true;
+              break;
+            }
+          }
+        }
+        if (!failed && !enough) {
+          in = (uint32_t)word;
+          count = (unsigned)(word >> 32) & kTwoCountMask;
+          if ((unsigned)(word >> 32) & kTwoEnd) flags |= kTwoInEnded;
+        }
+      }
+      if (failed) coherent_store(&ctrl->err, kErrBarrierTimeout);
+      if (failed || enough) flags |= kTwoInStop;
+      my_round = q + kTwoAhead;
+      if (!(flags & kTwoInStop) && (!(flags & kTwoInEnded) || may_stop)) two_ask(up_ring + (my_round % kTwoRing), enough_flag);
+    }
+    in_lds[q & 1][0] = in;
+    in_lds[q & 1][1] = count;
+    in_lds[q & 1][2] = flags;
+  };
+  if (tid == 0) receive(0, b == 0 ? kTwoInEnded : 0u, 0u);
+  int round = 0;
+  for (;; ++round) {
+    const int par = round & 1;
+    // ---- the minimum of this thread's remaining rows, of the wave's rows up to this lane
     uint32_t tmin = kTwoNone;
 #pragma unroll
     for (int e = 0; e < kTwoPerThread; ++e) tmin = min(tmin, v[e]);
     const uint32_t incl = wave_prefix_min(tmin);
-    uint32_t* const wave_min = wave_min_lds[round & 1];
-    if (lane == 63) wave_min[wave] = incl;
+    if (lane == 63) wave_min_lds[par][wave] = incl;
     EVX_TRACE(round, 0);
     lds_barrier();
     EVX_TRACE(round, 1);
-    // the first wave turns the wave minima into what stands before every wave (a prefix minimum over sixteen lanes
-    // of a DPP row) and the minimum of the workgroup
-    uint32_t local = kTwoNone;
-    if (wave == 0) {
-      const uint32_t mine = lane < kTwoThreads / 64 ? wave_min[lane] : kTwoNone;
-      const uint32_t upto = wave_prefix_min(mine);
-      const uint32_t before_wave = (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)upto, 0x138, 0xf, 0xf, false);  // wave_shr:1
-      if (lane < kTwoThreads / 64) before_lds[lane] = before_wave;
-      local = (uint32_t)__builtin_amdgcn_readlane((int)upto, kTwoThreads / 64 - 1);
-    }
-    if (tid == 0) {
-      left -= ranked_lds;  // what the round before has ranked
-      ranked_lds = 0;
-      // ---- the incoming minimum of the round
-      uint32_t in = kTwoNone;
-      bool failed = false;
-      if (!upstream_ended) {
-        const unsigned long long* slot = up_ring + (round % kTwoRing);
-        unsigned long long word = ahead[0];
-        ahead[0] = ahead[1];
-        if (((unsigned)(word >> 32) & ~kTwoEnd) != tag) {
-          WaitBound bound(spin_limit);
-          for (unsigned spins = 0;; ++spins) {
-            word = coherent_load(slot);
-            if (((unsigned)(word >> 32) & ~kTwoEnd) == tag) break;
-            if (bound.expired(spins) || ((spins & 63u) == 63u && coherent_load(&ctrl->err) != 0)) {
-              failed = true;
-              break;
-            }
-          }
-        }
-        if (!failed) {
-          in = (uint32_t)word;
-          if ((unsigned)(word >> 32) & kTwoEnd) upstream_ended = true;  // nothing remains before this workgroup, from this round on
-          coherent_store(my_progress, round + 1);
-          if (!upstream_ended) ahead[1] = coherent_load(up_ring + ((round + 2) % kTwoRing));
-        }
-      }
-      // ---- hand on at once: the minimum over the remaining rows up to the end of this workgroup's run.  The stream
-      // ends with the round in which neither this workgroup nor those before it have a row left.
-      const bool ends_here = upstream_ended && left == 0;
-      if (!failed && !last_block) {
-        if (round >= kTwoRing) {  // (the slot still holds round - kTwoRing: has the next workgroup taken it in?)
-          WaitBound bound(spin_limit);
-          for (unsigned spins = 0; coherent_load(down_progress) < round - kTwoRing + 1; ++spins) {
-            if (bound.expired(spins) || ((spins & 63u) == 63u && coherent_load(&ctrl->err) != 0)) {
-              failed = true;
-              break;
-            }
-          }
-        }
-        if (!failed)
-          coherent_store(my_ring + (round % kTwoRing), ((unsigned long long)(tag | (ends_here ? kTwoEnd : 0u)) << 32) | min(in, local));
-      }
-      if (failed) coherent_store(&ctrl->err, kErrBarrierTimeout);
-      in_lds[0] = in;
-      in_lds[1] = failed || ends_here ? 1u : 0u;
-    }
-    EVX_TRACE(round, 2);
-    lds_barrier();
-    EVX_TRACE(round, 3);
-    if (in_lds[1] != 0u) break;  // nothing is left here and before, or a wait ran out
-    // ---- exclusive prefix minimum over the remaining rows before each slot, seeded with the incoming one
-    uint32_t before = min(in_lds[0], before_lds[wave]);
-    {
-      const uint32_t shifted = (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)incl, 0x138, 0xf, 0xf, false);  // wave_shr:1
-      before = min(before, shifted);
-    }
-    int ranked = 0;
+    const uint4 in_word = *reinterpret_cast<const uint4*>(in_lds[par]);
+    const uint32_t wave_min = wave_min_lds[par][lane & 15];
+    const uint32_t in = in_word.x, count_in = in_word.y, flags = in_word.z;
+    if (((flags & kTwoInStop) | in_word.w) != 0u) break;  // (the same for every wave: written before the barrier)
+    // ---- what stands before this wave: the minimum over the wave minima of the waves before, reduced inside every
+    // row of sixteen lanes (all lanes get it)
+    uint32_t before = lower ? wave_min : kTwoNone;
+    before = min(before, (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)before, 0x128, 0xf, 0xf, false));  // row_ror:8
+    before = min(before, (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)before, 0x124, 0xf, 0xf, false));  // row_ror:4
+    before = min(before, (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)before, 0x122, 0xf, 0xf, false));  // row_ror:2
+    before = min(before, (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)before, 0x121, 0xf, 0xf, false));  // row_ror:1
+    before = min(before, in);
+    before = min(before, (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)incl, 0x138, 0xf, 0xf, false));  // wave_shr:1
+    // ---- the rows that are strict prefix minima form the front of this round
+    int ranked = 0;  // (of the whole wave)
 #pragma unroll
     for (int e = 0; e < kTwoPerThread; ++e) {
-      const uint32_t mine = v[e];
-      if (mine < before) {  // a strict prefix minimum: no remaining row before it is no worse in both objectives
-        rank[orig[e]] = round;
-        v[e] = kTwoNone;
-        ++ranked;
-      }
-      before = min(before, mine);
+      const uint32_t mine_e = v[e];
+      const bool front = mine_e < before;  // no remaining row before it is no worse in both objectives
+      ranked += __popcll(__builtin_amdgcn_ballot_w64(front));
+      rk[e] = front ? round : rk[e];
+      v[e] = front ? kTwoNone : mine_e;
+      before = min(before, mine_e);
     }
-    if (ranked) atomicAdd(&ranked_lds, ranked);  // (few threads rank a row in any one round)
-    // (the barrier at the head of the next round also closes this round's counting)
+    if (ranked != 0 && lane == 0) atomicAdd(&ranked_lds[par], ranked);  // (read behind the next barrier)
+    EVX_TRACE(round, 2);
+    if (wave == kTwoPublisher / 64) {
+      // the minimum of the workgroup
+      uint32_t local = wave_min;
+      local = min(local, (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)local, 0x128, 0xf, 0xf, false));  // row_ror:8
+      local = min(local, (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)local, 0x124, 0xf, 0xf, false));  // row_ror:4
+      local = min(local, (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)local, 0x122, 0xf, 0xf, false));  // row_ror:2
+      local = min(local, (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)local, 0x121, 0xf, 0xf, false));  // row_ror:1
+      if (publisher) {
+        const int before_round = ranked_lds[par ^ 1];  // what round - 1 has ranked
+        ranked_lds[par ^ 1] = 0;
+        left -= before_round;
+        done_here += before_round;
+        const int done = (int)count_in + done_here;
+        const bool ended_before = (flags & kTwoInEnded) != 0u;
+        // the stream ends with the round in which neither this workgroup nor those before it have a row left
+        const bool ends_here = ended_before && left == 0;
+        bool stop_next = ends_here;
+        if (last_block) {
+          if (may_stop && done >= stop_count) {  // enough rows ranked everywhere, as of the round before this one
+            coherent_store(enough_flag, 1);
+            stop_next = true;
+          }
+        } else {
+          bool go = true;
+          if (round >= kTwoRing && down_seen < round - kTwoRing + 1) {  // (the slot still holds round - kTwoRing: has the next workgroup taken it in?)
+            WaitBound bound(spin_limit);
+            for (unsigned spins = 0;; ++spins) {
+              down_seen = coherent_load(down_progress);
+              if (down_seen >= round - kTwoRing + 1) break;
+              if (may_stop && (spins & 3u) == 3u && coherent_load(enough_flag) != 0) {
+                go = false;
+                break;
+              }
+              if (bound.expired(spins) || ((spins & 63u) == 63u && coherent_load(&ctrl->err) != 0)) {
+                coherent_store(&ctrl->err, kErrBarrierTimeout);
+                go = false;
+                break;
+              }
+            }
+          }
+          if (go)
+            coherent_store(my_ring + (round % kTwoRing),
+                           ((unsigned long long)((ends_here ? kTwoEnd : 0u) | (two_tag(round) << kTwoTagShift) | (unsigned)done) << 32) | min(in, local));
+          else
+            stop_next = true;
+        }
+        if (!ended_before) coherent_store(my_progress, round + 1);
+        in_lds[par ^ 1][3] = stop_next ? 1u : 0u;
+      }
+    }
+    if (receiver && wave == (round + 1) % kTwoAhead) receive(round + 1, flags, count_in);
+    EVX_TRACE(round, 3);
   }
+  if (last_block && publisher) ctrl->reserved[kTwoRounds] = round;  // (for the sort of the ranks: how many bits they have)
+  // ---- the ranks, kept in registers so far; rows that no round has reached (the peeling ended early, or a wait ran
+  // out) stay unset
+#pragma unroll
+  for (int e = 0; e < kTwoPerThread; ++e)
+    if (orig[e] >= 0) rank[orig[e]] = rk[e];
 }
 
 // After the brigade: the rows of a key take the rank of the key's first row.
@@ -221,9 +336,11 @@ __global__ __launch_bounds__(256) void two_finish_kernel(const uint32_t* __restr
   }
 }
 
-// After the listing (perm = rows by (rank, original index), every row ranked, the ranks 0 .. F - 1 all present):
-// where every front starts, and -- the peeling having gone through all fronts -- the front that holds the
-// stop_count-th row, as the control block describes it for the kernels that order it.
+// After the listing (perm = rows by (rank, original index) up to the cut front and beyond; behind the fronts that every
+// workgroup has been through, rows of later fronts and rows without a rank follow in no particular order): where every
+// front starts, and the front that holds the stop_count-th row, as the control block
+// describes it for the kernels that order it.  Every front up to that one is complete; later ones may be ranked in
+// part, their starts mean nothing.
 __global__ __launch_bounds__(256) void two_bounds_kernel(const int* __restrict__ perm, const int* __restrict__ rank, int n,
                                                          int* __restrict__ fstart, Ctrl* __restrict__ ctrl, int stop_count) {
   if (ctrl->err != 0) return;
@@ -231,8 +348,9 @@ __global__ __launch_bounds__(256) void two_bounds_kernel(const int* __restrict__
   for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < n; p += gridDim.x * blockDim.x) {
     const int r = rank[perm[p]];
     const int r_before = p > 0 ? rank[perm[p - 1]] : -1;
-    if (r != r_before) {  // position p opens front r
-      fstart[r] = p;
+    if (r != r_before) {  // position p opens front r and closes front r_before
+      if (r != kRankUnset) fstart[r] = p;
+      if (r_before == worst) fstart[worst + 1] = p;  // (whatever follows the cut front: the next one, a later one ranked in part, rows without a rank)
       if (r == worst) {
         ctrl->worst = worst;
         ctrl->nfronts = worst + 1;
@@ -241,7 +359,7 @@ __global__ __launch_bounds__(256) void two_bounds_kernel(const int* __restrict__
         ctrl->need = stop_count - p;
       }
     }
-    if (p == n - 1) fstart[r + 1] = n;
+    if (p == n - 1 && r != kRankUnset) fstart[r + 1] = n;
   }
 }
 
@@ -250,8 +368,9 @@ __global__ __launch_bounds__(256) void two_sizes_kernel(const int* __restrict__ 
                                                         const int* __restrict__ fstart, int* __restrict__ fsize,
                                                         Ctrl* __restrict__ ctrl, int* __restrict__ rank_until_out) {
   if (ctrl->err != 0) return;
-  const int fronts = rank[perm[n - 1]] + 1;
   const int worst = ctrl->worst;
+  const int last = rank[perm[n - 1]];
+  const int fronts = last == kRankUnset ? worst + 1 : last + 1;
   for (int r = blockIdx.x * blockDim.x + threadIdx.x; r < fronts; r += gridDim.x * blockDim.x) {
     fsize[r] = fstart[r + 1] - fstart[r];
     if (r == worst) ctrl->nv = fstart[r + 1] - fstart[r];

@@ -84,7 +84,7 @@ def test_two_objective_populations_against_the_checker(name):
     topk = n // 2
     order, rank, dist, _ = c_oracle.select(f.numpy(), topk)
     x = torch.arange(n, dtype=torch.int32)[:, None]
-    with runtime.options(two_min_rows=1):  # (by default a selection of fewer than 24 576 rows takes the matrix)
+    with runtime.options(two_min_rows=1):  # (by default a population of up to 4096 rows takes the matrix, or the one-workgroup kernel)
         sel = nd_environmental_selection(x.to(DEV), fd, topk)
         until = as_np(non_dominate_rank_until(fd, topk + 1))
     assert np.array_equal(as_np(sel[2]), rank[order]), name
@@ -111,3 +111,84 @@ def test_two_objectives_in_two_parts_and_with_strides():
     wide = torch.zeros(12000, 5)
     wide[:, 1:4:2] = f
     assert np.array_equal(as_np(non_dominate_rank(wide.to(DEV)[:, 1:4:2])), as_np(er.ranks_by_peeling(f)))
+
+
+def _stop_cases():
+    g = torch.Generator("cpu").manual_seed(2224)
+    out = {}
+    # the first workgroup holds a chain of 4096 rows (its own front each), the others two fronts: the fronts so far hold
+    # the rows asked for after two rounds, while the first workgroup has thousands of rounds before it
+    t = torch.arange(4096, dtype=torch.float32)
+    chain = torch.stack([t * 1e-3, 100.0 + t], dim=1)
+    a = torch.rand(12000, generator=g)
+    rest = torch.stack([10.0 + a, 1.0 - a + (torch.rand(12000, generator=g) < 0.5).float() * 2.0], dim=1)
+    out["chain_in_the_first_workgroup"] = torch.cat([chain, rest])
+    # every row four times: only the first copy of a row counts while the peeling looks for its end, so it goes on
+    # beyond the front that holds the rows asked for
+    u = torch.rand(5000, 2, generator=g)
+    out["every_row_four_times"] = u.repeat(4, 1)[torch.randperm(20000, generator=g)]
+    # few fronts, all of them large: the cut falls into the first rounds of a chain of ten workgroups
+    b = torch.rand(40000, generator=g)
+    out["five_lines"] = torch.stack([b, 1.0 - b + torch.randint(0, 5, (40000,), generator=g).float()], dim=1)
+    # more rounds than the ring of hand-over words holds, three times over
+    c = torch.rand(9000, 2, generator=g)
+    out["many_fronts"] = c + torch.arange(9000)[:, None].float().div(9).floor() * 0.01
+    out["uniform_60000"] = torch.rand(60000, 2, generator=g)
+    return out
+
+
+STOPS = _stop_cases()
+
+
+@pytest.mark.parametrize("name", sorted(STOPS))
+def test_the_peeling_may_end_at_the_cut(name):
+    """Selections and ranks up to a cut, where the chain of workgroups stops peeling once the fronts so far hold the rows
+    asked for: every stop count gives the checker's ranks up to its cut front and the same selection as all ranks do."""
+    f = STOPS[name]
+    n = f.size(0)
+    fd = f.to(DEV)
+    want, _fronts = c_oracle.nd_rank(f)
+    want = as_np(want)
+    assert np.array_equal(as_np(non_dominate_rank(fd)), want), name
+    x = torch.arange(n, dtype=torch.int32)[:, None].to(DEV)
+    for topk in (1, 7, n // 10, n // 2, n - 1, n):
+        until = as_np(non_dominate_rank_until(fd, topk))
+        worst = np.sort(want)[topk - 1]
+        assert np.array_equal(until, np.where(want <= worst, want, 2**31 - 1)), (name, topk)
+        if n > 30000 and topk != n // 2:  # (the checker's selection of that many rows takes seconds)
+            continue
+        sel = nd_environmental_selection(x, fd, topk)
+        status = runtime.last_status()
+        assert status["error"] == 0 and status["fronts"] == worst + 1, (name, topk, status)
+        order, rank, dist, _ = c_oracle.select(f.numpy(), topk)
+        order, rank, dist = as_np(order)[:topk], as_np(rank), as_np(dist)
+        assert np.array_equal(as_np(sel[2]), rank[order]), (name, topk)
+        gd, wd = as_np(sel[3]), dist[order]
+        fin = np.isfinite(wd)
+        assert np.array_equal(np.isfinite(gd), fin), (name, topk)
+        np.testing.assert_allclose(gd[fin], wd[fin], rtol=1e-5, err_msg=f"{name} {topk}")
+        got_rows = as_np(sel[0])[:, 0]
+        if not np.array_equal(got_rows, order):  # rows may only change places where their distances tie within rounding
+            assert np.allclose(np.sort(gd[fin]), np.sort(wd[fin]), rtol=1e-5), (name, topk)
+            assert np.array_equal(np.sort(got_rows[rank[got_rows] < worst]), np.sort(order[rank[order] < worst])), (name, topk)
+
+
+def test_a_wait_that_runs_out_in_the_chain_is_reported():
+    f = torch.rand(60000, 2, generator=torch.Generator("cpu").manual_seed(2225))
+    fd = f.to(DEV)
+    x = torch.arange(60000, dtype=torch.float32)[:, None].to(DEV)
+    with runtime.options(spin_limit=1):
+        rank = non_dominate_rank(fd)
+        with pytest.raises(Exception):
+            runtime.last_status()
+        sel = nd_environmental_selection(x, fd, 30000)
+    torch.cuda.synchronize()
+    assert (as_np(rank) == -1).all() and (as_np(sel[2]) == -1).all() and np.isnan(as_np(sel[3])).all()
+    # ... and with the status checked, the call comes through on the kernels that never wait
+    runtime.CHECK_STATUS = True
+    try:
+        with runtime.options(spin_limit=1):
+            again = non_dominate_rank(fd)
+    finally:
+        runtime.CHECK_STATUS = False
+    assert np.array_equal(as_np(again), as_np(c_oracle.nd_rank(f)[0]))
