@@ -1,0 +1,75 @@
+"""What the compiler made of the kernels, read from the metadata of the built library (the gfx950 code object inside
+libevox_hip.so; no GPU needed).
+
+``two_peel_kernel`` (csrc/two.hpp) keeps loads in flight across rounds in the accumulation registers a0..a2, which it
+names in inline asm.  That is only sound while the compiler uses no accumulation register of its own in that kernel
+(it would, to spill vector registers): the kernel must report exactly three of them and no scratch memory, and no
+other kernel of the library may report any.
+"""
+
+import os
+import struct
+
+import msgpack
+import pytest
+
+from evox_amd.build import LIB_PATH, build_library
+
+MAGIC = b"__CLANG_OFFLOAD_BUNDLE__"
+
+
+def _gfx950_code_object(blob: bytes) -> bytes:
+    start = blob.find(MAGIC)
+    assert start >= 0, "no offload bundle in the library"
+    (entries,) = struct.unpack_from("<Q", blob, start + len(MAGIC))
+    at = start + len(MAGIC) + 8
+    for _ in range(entries):
+        offset, size, triple_size = struct.unpack_from("<QQQ", blob, at)
+        at += 24
+        triple = blob[at:at + triple_size].decode()
+        at += triple_size
+        if "gfx950" in triple:
+            return blob[start + offset:start + offset + size]
+    raise AssertionError("no gfx950 code object in the library")
+
+
+def _kernels(elf: bytes):
+    assert elf[:4] == b"\x7fELF"
+    (section_table,) = struct.unpack_from("<Q", elf, 0x28)
+    entry_size, count, _names = struct.unpack_from("<HHH", elf, 0x3A)
+    for s in range(count):
+        _name, kind, _flags, _addr, offset, size = struct.unpack_from("<IIQQQQ", elf, section_table + s * entry_size)
+        if kind != 7:  # SHT_NOTE
+            continue
+        at, end = offset, offset + size
+        while at < end:
+            name_size, desc_size, note_type = struct.unpack_from("<III", elf, at)
+            at += 12 + ((name_size + 3) & ~3)
+            desc = elf[at:at + desc_size]
+            at += (desc_size + 3) & ~3
+            if note_type == 32:  # NT_AMDGPU_METADATA
+                return msgpack.unpackb(desc, raw=False)["amdhsa.kernels"]
+    raise AssertionError("no kernel metadata in the code object")
+
+
+@pytest.fixture(scope="module")
+def kernels():
+    if not os.path.exists(LIB_PATH):
+        build_library()
+    with open(LIB_PATH, "rb") as fh:
+        return _kernels(_gfx950_code_object(fh.read()))
+
+
+def test_only_the_chain_kernel_uses_accumulation_registers_and_only_its_own_three(kernels):
+    with_agprs = {k[".name"]: k[".agpr_count"] for k in kernels if k.get(".agpr_count", 0)}
+    assert len(with_agprs) == 1, with_agprs
+    (name, count), = with_agprs.items()
+    assert "two_peel_kernel" in name and count == 3, with_agprs
+    chain = next(k for k in kernels if "two_peel_kernel" in k[".name"])
+    assert chain[".private_segment_fixed_size"] == 0  # nothing spilled
+    assert chain[".max_flat_workgroup_size"] == 1024
+
+
+def test_every_kernel_is_built_for_wave64(kernels):
+    assert len(kernels) > 100
+    assert all(k[".wavefront_size"] == 64 for k in kernels)
