@@ -192,3 +192,27 @@ def test_a_wait_that_runs_out_in_the_chain_is_reported():
     finally:
         runtime.CHECK_STATUS = False
     assert np.array_equal(as_np(again), as_np(c_oracle.nd_rank(f)[0]))
+
+
+def test_half_a_million_rows_on_a_grid():
+    """The points (i, j) of a 707 x 707 grid: the rank of a point is i + j (1413 fronts, 123 workgroups in the chain,
+    five rings of hand-over words), which no checker has to compute."""
+    side = 707
+    n = side * side
+    i, j = np.divmod(np.arange(n), side)
+    perm = np.random.default_rng(side).permutation(n)
+    f = torch.from_numpy(np.stack([i, j], 1).astype(np.float32)[perm])
+    want = (i + j)[perm]
+    fd = f.to(DEV)
+    assert np.array_equal(as_np(non_dominate_rank(fd)), want)
+    assert runtime.last_status()["error"] == 0
+    x = torch.arange(n, dtype=torch.float32, device=DEV)[:, None]
+    for topk in (1000, n // 2):
+        worst = np.sort(want)[topk - 1]
+        assert np.array_equal(as_np(non_dominate_rank_until(fd, topk)), np.where(want <= worst, want, 2**31 - 1)), topk
+        sel = nd_environmental_selection(x, fd, topk)
+        status = runtime.last_status()
+        assert status["error"] == 0 and status["fronts"] == worst + 1, status
+        rows = as_np(sel[0])[:, 0].astype(np.int64)
+        assert len(np.unique(rows)) == topk and np.array_equal(as_np(sel[2]), want[rows]), topk
+        assert np.array_equal(np.sort(rows[want[rows] < worst]), np.flatnonzero(want < worst)), topk
