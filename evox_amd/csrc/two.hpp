@@ -20,24 +20,26 @@
 //
 // A round inside a workgroup is ONE barrier: every wave leaves the prefix minimum of its rows in LDS, and behind the
 // barrier every wave reads the sixteen wave minima and the incoming minimum and ranks its own rows.  Everything that
-// talks to other workgroups happens beside that, in single lanes of different waves, because a wave waits for its
-// memory operations in the order of their issue (a load that has to see another workgroup's store takes over a
-// microsecond -- two rounds -- and a write-through store as long):
-//   * the word of round q is asked for kTwoAhead rounds ahead by the first lane of wave q mod kTwoAhead and taken
-//     in -- tag checked, polled for if it is late -- right behind the barrier of round q - 1, so that it lies in LDS
-//     at the barrier of round q.  These waves issue no store inside the loop (the ranks stay in registers until the
-//     kernel ends), so the only thing such a lane ever waits for is its own load of kTwoAhead rounds ago;
+// talks to other workgroups happens beside that, in single lanes of two waves, because a wave waits for its memory
+// operations in the order of their issue (a load that has to see another workgroup's store takes half a
+// microsecond, most of a round, and a write-through store longer):
+//   * the first wave holds no rows.  Right behind the barrier of round q - 1 its first lane loads the word of round q
+//     -- tag checked, loaded again while it is not there -- and leaves it in LDS for the barrier of round q; the load
+//     takes as long as the other waves rank their rows.  This wave stores nothing;
 //   * the first lane of the last wave publishes: behind the barrier of round r it counts what round r - 1 ranked,
 //     stores the word of round r for the next workgroup and the progress counter for the one before, and decides
 //     whether the workgroup is done (seen by all waves behind the next barrier).  It loads nothing but, once every
-//     ring of rounds, the progress of the workgroup after.
-// A workgroup whose words come late polls for them and thereby falls behind the one before it, until it is far enough
-// behind for its words to be there when it asks (about kTwoAhead rounds and the time a store takes to be seen: 3 to
-// 5 us per workgroup of the chain).  A round takes 0.65 us -- instruction issue: sixteen waves of some eighty
-// instructions on four SIMDs; half as many waves with twice the rows each take as long, since one or two waves per
-// SIMD wait nine clocks for every dependent instruction instead of four -- where the two barriers and the one
-// thread between them of an earlier form of this kernel took 1.25.  Falling back on purpose (a sleep after the first
-// late word) and asking three, four or six rounds ahead were measured and are slower.
+//     ring of rounds, the progress of the workgroup after.  The ranks stay in registers until the kernel ends, so the
+//     other waves store nothing inside the loop either.
+// A workgroup runs about 1.3 us behind the one before it (the time a stored word takes to be seen and loaded).  A
+// round takes 0.65 us -- instruction issue: fifteen waves of some eighty instructions on four SIMDs; half as many
+// waves with twice the rows each take as long, since one or two waves per SIMD wait nine clocks for every dependent
+// instruction instead of four -- where the two barriers and the one thread between them of an earlier form of this
+// kernel took 1.25: that thread waited for its own write-through stores and for loads issued a round earlier.
+// Measured and no faster: words asked for one to six rounds ahead (into accumulation registers, so that the compiler
+// places no wait at the end of the loop body), by the wave without rows or by lanes of waves that also hold rows (a
+// word that is not there yet costs such a wave a second load on top of its rows: 0.85 us per round); falling back on
+// purpose (a sleep after the first late word).
 #pragma once
 
 #include "peel.hpp"
@@ -46,13 +48,12 @@ namespace evx {
 
 constexpr int kTwoThreads = 1024;
 constexpr int kTwoWaves = kTwoThreads / 64;
-constexpr int kTwoChunk = 4096;                              // slots per workgroup
-constexpr int kTwoPerThread = kTwoChunk / kTwoThreads;       // consecutive slots per thread
+constexpr int kTwoPerThread = 4;                             // consecutive slots per thread
+constexpr int kTwoChunk = (kTwoThreads - 64) * kTwoPerThread;  // slots per workgroup: the first wave holds none
 constexpr int kTwoMaxBlocks = 256;
 constexpr int64_t kTwoMaxRows = (int64_t)kTwoChunk * kTwoMaxBlocks;
 constexpr int kTwoRing = 256;                                // rounds of a workgroup's outgoing stream that are kept
 constexpr int kTwoRingStride = kTwoRing + 16;                // words per workgroup: the ring, then its progress counter on a line of its own
-constexpr int kTwoAhead = 2;                                 // rounds between asking for a word and taking it in; as many waves take turns
 constexpr int kTwoPublisher = kTwoThreads - 64;              // the thread that stores
 constexpr int kTwoRounds = 4;                                // Ctrl.reserved[kTwoRounds]: the rounds of the last workgroup (every rank up to the cut is below it)
 constexpr uint32_t kTwoNone = 0xFFFFFFFFu;                   // "no remaining row": larger than every image of a number
@@ -65,7 +66,6 @@ constexpr unsigned kTwoCountMask = (1u << kTwoTagShift) - 1u;
 __device__ inline unsigned two_tag(int round) { return (unsigned)((round / kTwoRing) % 3) + 1u; }
 __device__ inline unsigned two_tag_of(unsigned long long word) { return ((unsigned)(word >> 32) >> kTwoTagShift) & 3u; }
 static_assert(kTwoMaxRows <= (int64_t)kTwoCountMask, "the count of ranked rows must fit its field");
-static_assert(kTwoAhead <= kTwoWaves - 1 && kTwoAhead < kTwoRing, "the lanes that load and the lane that stores sit in different waves");
 static_assert(kTwoWaves <= 16, "the wave minima are reduced inside rows of sixteen lanes");
 // flags of an incoming word as the waves see it in LDS
 constexpr uint32_t kTwoInEnded = 1u;  // nothing remains before this workgroup, from this round on
@@ -82,21 +82,6 @@ __device__ inline uint32_t wave_prefix_min(uint32_t x) {
   v = min(v, (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)v, 0x142, 0xa, 0xf, false));  // row_bcast:15
   v = min(v, (uint32_t)__builtin_amdgcn_update_dpp((int)kTwoNone, (int)v, 0x143, 0xc, 0xf, false));  // row_bcast:31
   return v;
-}
-
-// What a receiving lane asks for ahead of time -- the word of its next round and the "enough" flag -- lands in
-// the accumulation registers a0..a2, which the compiler uses for nothing in this kernel.  Asked for into ordinary
-// registers, the loads would be followed at the end of the loop body by the compiler's copies of those registers
-// and the wait that a copy needs: a memory round trip in every round.
-__device__ __forceinline__ void two_ask(const unsigned long long* word, const int* flag) {
-  asm volatile("global_load_dwordx2 a[0:1], %0, off sc1\n\tglobal_load_dword a2, %1, off sc1" ::"v"(word), "v"(flag) : "memory", "a0", "a1", "a2");
-}
-__device__ __forceinline__ void two_take(unsigned long long* word, int* flag) {
-  unsigned lo, hi, en;
-  asm volatile("s_waitcnt vmcnt(0)\n\tv_accvgpr_read_b32 %0, a0\n\tv_accvgpr_read_b32 %1, a1\n\tv_accvgpr_read_b32 %2, a2"
-               : "=v"(lo), "=v"(hi), "=v"(en)::"memory");
-  *word = ((unsigned long long)hi << 32) | lo;
-  *flag = (int)en;
 }
 
 // Grid: ceil(n / kTwoChunk) workgroups of kTwoThreads.  xs1_sorted / xs2_sorted: the objectives by slot (rows sorted by
@@ -137,14 +122,14 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
   int rk[kTwoPerThread];
   int unranked = 0;
   {
-    const int s0 = b * kTwoChunk + tid * kTwoPerThread;
+    const int s0 = b * kTwoChunk + (tid - 64) * kTwoPerThread;
 #pragma unroll
     for (int e = 0; e < kTwoPerThread; ++e) {
       const int s = s0 + e;
       v[e] = kTwoNone;
       orig[e] = -1;
       rk[e] = kRankUnset;
-      if (s < n) {
+      if (wave > 0 && s < n) {
         const float a1 = xs1_sorted[s], a2 = xs2_sorted[s];
         const int o = orig_of[s];
         if (dist_fill) dist_fill[o] = -INFINITY;
@@ -164,35 +149,31 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
     in_lds[0][3] = 0u;
     in_lds[1][3] = 0u;
   }
-  if (tid < 32) wave_min_lds[tid >> 4][tid & 15] = kTwoNone;
+  if (tid < 32) wave_min_lds[tid >> 4][tid & 15] = kTwoNone;  // (the first wave's entries stay that way)
   unranked = wave_sum(unranked);
   if (lane == 0) unranked_lds[wave] = unranked;
   __syncthreads();
   const bool publisher = tid == kTwoPublisher;
-  const bool receiver = lane == 0 && wave < kTwoAhead;  // takes in the words of the rounds q with q mod kTwoAhead == wave
+  const bool receiver = tid == 0;
   // (publisher) rows of this workgroup without a rank, rows ranked so far by this workgroup, the progress of the
   // workgroup after this one as last read
   int left = 0, done_here = 0, down_seen = 0;
   if (publisher)
     for (int w = 0; w < kTwoWaves; ++w) left += unranked_lds[w];
   const bool lower = (lane & 15) < wave;  // this lane's entry of the wave minima belongs to a wave before this one
-  // (receivers) the round whose word is asked for
-  int my_round = wave;
-  if (receiver && (b > 0 || may_stop)) two_ask(up_ring + my_round, enough_flag);
-  // Takes in the word of round q (the caller is the receiver of that round; before: the flags and the count that
-  // round q - 1 saw) and leaves it in LDS for the barrier of round q.
+  // Takes in the word of round q (before: the flags and the count that round q - 1 saw) and leaves it in LDS for the
+  // barrier of round q.
   auto receive = [&](int q, uint32_t flags_before, uint32_t count_before) {
     uint32_t in = kTwoNone, count = count_before, flags = flags_before & kTwoInEnded;
     if (!(flags & kTwoInEnded) || may_stop) {
-      unsigned long long word;
-      int flag_seen;
-      two_take(&word, &flag_seen);
-      bool enough = may_stop && flag_seen != 0;
+      const unsigned long long* slot = up_ring + (q % kTwoRing);
+      // (the word and the flag in flight together)
+      unsigned long long word = (flags & kTwoInEnded) ? 0ull : coherent_load(slot);
+      bool enough = may_stop && coherent_load(enough_flag) != 0;
       bool failed = false;
       if (!enough && !(flags & kTwoInEnded)) {
         const unsigned tag = two_tag(q);
-        if (two_tag_of(word) != tag) {  // late: the workgroup before is not far enough ahead (yet)
-          const unsigned long long* slot = up_ring + (q % kTwoRing);
+        if (two_tag_of(word) != tag) {  // not there yet: the workgroup before is less than a store and a load ahead
           WaitBound bound(spin_limit);
           for (unsigned spins = 0;; ++spins) {
             word = coherent_load(slot);
@@ -215,30 +196,36 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
       }
       if (failed) coherent_store(&ctrl->err, kErrBarrierTimeout);
       if (failed || enough) flags |= kTwoInStop;
-      my_round = q + kTwoAhead;
-      if (!(flags & kTwoInStop) && (!(flags & kTwoInEnded) || may_stop)) two_ask(up_ring + (my_round % kTwoRing), enough_flag);
     }
     in_lds[q & 1][0] = in;
     in_lds[q & 1][1] = count;
     in_lds[q & 1][2] = flags;
   };
-  if (tid == 0) receive(0, b == 0 ? kTwoInEnded : 0u, 0u);
+  if (receiver) receive(0, b == 0 ? kTwoInEnded : 0u, 0u);
   int round = 0;
   for (;; ++round) {
     const int par = round & 1;
     // ---- the minimum of this thread's remaining rows, of the wave's rows up to this lane
-    uint32_t tmin = kTwoNone;
+    uint32_t incl = kTwoNone;
+    if (wave > 0) {
+      uint32_t tmin = kTwoNone;
 #pragma unroll
-    for (int e = 0; e < kTwoPerThread; ++e) tmin = min(tmin, v[e]);
-    const uint32_t incl = wave_prefix_min(tmin);
-    if (lane == 63) wave_min_lds[par][wave] = incl;
+      for (int e = 0; e < kTwoPerThread; ++e) tmin = min(tmin, v[e]);
+      incl = wave_prefix_min(tmin);
+      if (lane == 63) wave_min_lds[par][wave] = incl;
+    }
     EVX_TRACE(round, 0);
     lds_barrier();
     EVX_TRACE(round, 1);
     const uint4 in_word = *reinterpret_cast<const uint4*>(in_lds[par]);
-    const uint32_t wave_min = wave_min_lds[par][lane & 15];
     const uint32_t in = in_word.x, count_in = in_word.y, flags = in_word.z;
     if (((flags & kTwoInStop) | in_word.w) != 0u) break;  // (the same for every wave: written before the barrier)
+    if (wave == 0) {  // the wave without rows: the word of the next round
+      if (receiver) receive(round + 1, flags, count_in);
+      EVX_TRACE(round, 3);
+      continue;
+    }
+    const uint32_t wave_min = wave_min_lds[par][lane & 15];
     // ---- what stands before this wave: the minimum over the wave minima of the waves before, reduced inside every
     // row of sixteen lanes (all lanes get it)
     uint32_t before = lower ? wave_min : kTwoNone;
@@ -311,8 +298,6 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
         in_lds[par ^ 1][3] = stop_next ? 1u : 0u;
       }
     }
-    if (receiver && wave == (round + 1) % kTwoAhead) receive(round + 1, flags, count_in);
-    EVX_TRACE(round, 3);
   }
   if (last_block && publisher) ctrl->reserved[kTwoRounds] = round;  // (for the sort of the ranks: how many bits they have)
   // ---- the ranks, kept in registers so far; rows that no round has reached (the peeling ended early, or a wait ran

@@ -195,7 +195,7 @@ def test_a_wait_that_runs_out_in_the_chain_is_reported():
 
 
 def test_half_a_million_rows_on_a_grid():
-    """The points (i, j) of a 707 x 707 grid: the rank of a point is i + j (1413 fronts, 123 workgroups in the chain,
+    """The points (i, j) of a 707 x 707 grid: the rank of a point is i + j (1413 fronts, 131 workgroups in the chain,
     five rings of hand-over words), which no checker has to compute."""
     side = 707
     n = side * side
