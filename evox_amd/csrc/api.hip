@@ -6,6 +6,7 @@
 #include <atomic>
 #include <mutex>
 #include <new>
+#include <type_traits>
 
 #include "../../include/evox_hip.h"
 #include "batched.hpp"
@@ -194,7 +195,9 @@ static int device_cus() {
 // left it to the ordering kernels) and the host reads at its next call of that shape without waiting for anything --
 // a stale or missing word costs a few microseconds, never a result.  Allocated at the first selection on a device
 // that may allocate (not during a stream capture); null until then and for callers that may not.
-static int* outcome_slot(int64_t n, int64_t m, bool may_allocate, hipStream_t s) {
+// salt: 0 for the selections of 4-byte fitness, 1 for those whose last front is ordered by the kernels of wide.hpp
+// (there the word says whether that front was small, 1, or large, 2).
+static int* outcome_slot(int64_t n, int64_t m, bool may_allocate, hipStream_t s, int salt = 0) {
   static std::atomic<int*> words[64];
   static std::atomic<bool> failed[64];
   static std::mutex mu;
@@ -222,7 +225,7 @@ static int* outcome_slot(int64_t n, int64_t m, bool may_allocate, hipStream_t s)
       words[dev].store(base, std::memory_order_release);
     }
   }
-  return base + (int)(((uint64_t)n * 31u + (uint64_t)m) & 15u);
+  return base + (int)(((uint64_t)n * 31u + (uint64_t)m + (uint64_t)salt * 7u) & 15u);
 }
 
 #define EVX_LAUNCH_CHECK()                          \
@@ -1763,8 +1766,8 @@ int evox_hip_stable_argsort_step_batched(const void* key, int kind, int64_t batc
 // ---- fitness of 8-byte elements (wide.hpp)
 struct WideLayout {
   int n, m;
-  size_t ctrl, key_lo, key_hi, key_mask, selected, boundary, ord_a, ord_b, terms, dist, neg_lo, neg_hi, order_a, order_b, sort_ws,
-      sort_bytes, total;
+  size_t ctrl, key_lo, key_hi, key_mask, selected, boundary, ord_a, ord_b, terms, dist, neg_lo, neg_hi, order_a, order_b, front_dkey,
+      front_ends, sort_ws, sort_bytes, total;
 };
 
 static bool make_wide_layout(int64_t n, int64_t m, WideLayout* L) {
@@ -1787,6 +1790,8 @@ static bool make_wide_layout(int64_t n, int64_t m, WideLayout* L) {
   L->neg_hi = o;    o = align_up(o + 4 * (size_t)n);
   L->order_a = o;   o = align_up(o + 4 * (size_t)n);
   L->order_b = o;   o = align_up(o + 4 * (size_t)n);
+  L->front_dkey = o; o = align_up(o + 8 * (size_t)n);
+  L->front_ends = o; o = align_up(o + 8 * (size_t)m);
   SortLayout sort_layout;
   if (!make_sort_layout(n, &sort_layout)) return false;
   L->sort_bytes = sort_layout.total;
@@ -1806,7 +1811,7 @@ static int wide_grid(int64_t items) {
 // rows, into `dist` (double for out_kind 0, float for 1), and with neg_keys the sort keys of their negatives.
 static int wide_distances(const WideLayout& L, uint8_t* base, const void* costs, int kind, int64_t sr, int64_t sc,
                           const uint8_t* mask, int64_t mask_stride, const int32_t* rank, void* dist, int out_kind, bool neg_keys,
-                          hipStream_t s) {
+                          hipStream_t s, int* outcome = nullptr) {
   const int n = L.n, m = L.m;
   WideCtrl* ctrl = reinterpret_cast<WideCtrl*>(base + L.ctrl);
   uint32_t* key_lo = reinterpret_cast<uint32_t*>(base + L.key_lo);
@@ -1838,15 +1843,55 @@ static int wide_distances(const WideLayout& L, uint8_t* base, const void* costs,
                        terms, boundary);
     EVX_LAUNCH_CHECK();
     hipLaunchKernelGGL(wide_sum_kernel<double>, dim3(wide_grid(n)), dim3(256), 0, s, terms, selected, boundary, ctrl, n, m,
-                       static_cast<double*>(dist), neg_lo, neg_hi);
+                       static_cast<double*>(dist), neg_lo, neg_hi, outcome);
   } else {
     float* terms = reinterpret_cast<float*>(base + L.terms);
     hipLaunchKernelGGL(wide_terms_kernel<float>, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, order, ctrl,
                        terms, boundary);
     EVX_LAUNCH_CHECK();
     hipLaunchKernelGGL(wide_sum_kernel<float>, dim3(wide_grid(n)), dim3(256), 0, s, terms, selected, boundary, ctrl, n, m,
-                       static_cast<float*>(dist), neg_lo, neg_hi);
+                       static_cast<float*>(dist), neg_lo, neg_hi, outcome);
   }
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+// Whether the selection of a population of n rows orders its last front without sorting the costs
+// (wide_select_direct): up to kWideDirectRows rows, unless the last selection of this shape found a front of more
+// than kWideDirectFront rows -- that path's work grows with the square of the front.
+static bool wide_direct_applies(int64_t n, const int* outcome) {
+  return n <= kWideDirectRows && (outcome == nullptr || __atomic_load_n(outcome, __ATOMIC_RELAXED) != 2);
+}
+
+// The distances of the rows of the last front (rank == the largest rank set) and the selection order of all rows by
+// (rank, distance descending, row index), for populations of up to kWideDirectRows rows: one stable argsort step of
+// the ranks lists the rows, the kernels of wide.hpp do the rest without sorting the costs.
+static int wide_select_direct(const WideLayout& L, uint8_t* base, const void* costs, int kind, int64_t sr, int64_t sc,
+                              const int32_t* rank, void* dist, int out_kind, int* order_out, hipStream_t s, int* outcome) {
+  const int n = L.n, m = L.m;
+  WideCtrl* ctrl = reinterpret_cast<WideCtrl*>(base + L.ctrl);
+  int* listing = reinterpret_cast<int*>(base + L.order_b);
+  uint64_t* key = reinterpret_cast<uint64_t*>(base + L.terms);
+  uint64_t* dkey = reinterpret_cast<uint64_t*>(base + L.front_dkey);
+  int* ends = reinterpret_cast<int*>(base + L.front_ends);
+  hipLaunchKernelGGL(wide_head_kernel, dim3(1), dim3(1024), 0, s, (const uint8_t*)nullptr, (int64_t)0, rank, n, ctrl);
+  EVX_LAUNCH_CHECK();
+  if (int e = evox_hip_stable_argsort_step(rank, kKeyInt32, 1, n, nullptr, listing, base + L.sort_ws, L.sort_bytes, s)) return e;
+  // (sixteen lanes per candidate; the grid is sized for a front of all rows, which the kernels find out on the device)
+  const int pair_grid = wide_grid((int64_t)n * 16);
+  auto launch = [&](auto* typed_dist) {
+    using Out = std::remove_pointer_t<decltype(typed_dist)>;
+    hipLaunchKernelGGL(wide_front_keys_kernel<Out>, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, listing,
+                       ctrl, key, ends, typed_dist);
+    hipLaunchKernelGGL(wide_front_dist_kernel<Out>, dim3(pair_grid), dim3(256), 0, s, costs, kind, sr, sc, n, m, listing, ctrl, key,
+                       ends, typed_dist, dkey);
+  };
+  if (out_kind == 0)
+    launch(static_cast<double*>(dist));
+  else
+    launch(static_cast<float*>(dist));
+  EVX_LAUNCH_CHECK();
+  hipLaunchKernelGGL(wide_front_order_kernel, dim3(pair_grid), dim3(256), 0, s, listing, ctrl, dkey, n, order_out, outcome);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -2024,8 +2069,18 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
     WideLayout WL;
     if (!make_wide_layout(n, m, &WL) || WL.total > L.wide_bytes) return kErrWorkspace;
     uint8_t* wb = w.base + L.wide;
+    int* const wide_outcome = opt().launch_memory ? outcome_slot(n, m, may_allocate, s, 1) : nullptr;
+    if (wide_direct_applies(n, wide_outcome)) {
+      if (int e = wide_select_direct(WL, wb, w.at<float>(L.xs), kWideFloat32, 1, L.npad, w.at<int>(L.rank), w.at<float>(L.dist), 1,
+                                     w.at<int>(L.order), s, wide_outcome))
+        return e;
+      g.outcome = nullptr;
+      launch_gather(false);
+      EVX_LAUNCH_CHECK();
+      return 0;
+    }
     if (int e = wide_distances(WL, wb, w.at<float>(L.xs), kWideFloat32, 1, L.npad, nullptr, 0, w.at<int>(L.rank), w.at<float>(L.dist), 1,
-                               true, s))
+                               true, s, wide_outcome))
       return e;
     int* order_a = reinterpret_cast<int*>(wb + WL.order_a);
     int* order_b = reinterpret_cast<int*>(wb + WL.order_b);
@@ -2237,15 +2292,20 @@ int evox_hip_nd_environmental_selection_wide(const void* x, int64_t x_row_bytes,
   hipStream_t s = (hipStream_t)stream;
   uint8_t* base = static_cast<uint8_t*>(ws);
   void* dist = base + L.dist;
-  if (int e = wide_distances(L, base, costs, kind, sr, sc, nullptr, 0, rank, dist, out_kind, true, s)) return e;
-  // rows by rank, then by distance descending (NaN last), then by index: one stable step per key part, least
-  // significant first (src/evox/operators/selection/non_dominate.py:253, src/evox/utils/jit_fix_operator.py:246-250)
   int* order_a = reinterpret_cast<int*>(base + L.order_a);
   int* order_b = reinterpret_cast<int*>(base + L.order_b);
-  void* sort_ws = base + L.sort_ws;
-  if (int e = evox_hip_stable_argsort_step(base + L.neg_lo, kKeyUint32, 1, n, nullptr, order_a, sort_ws, L.sort_bytes, s)) return e;
-  if (int e = evox_hip_stable_argsort_step(base + L.neg_hi, kKeyUint32, 1, n, order_a, order_b, sort_ws, L.sort_bytes, s)) return e;
-  if (int e = evox_hip_stable_argsort_step(rank, kKeyInt32, 1, n, order_b, order_a, sort_ws, L.sort_bytes, s)) return e;
+  int* const outcome = opt().launch_memory ? outcome_slot(n, m, true, s, 1) : nullptr;
+  if (wide_direct_applies(n, outcome)) {
+    if (int e = wide_select_direct(L, base, costs, kind, sr, sc, rank, dist, out_kind, order_a, s, outcome)) return e;
+  } else {
+    if (int e = wide_distances(L, base, costs, kind, sr, sc, nullptr, 0, rank, dist, out_kind, true, s, outcome)) return e;
+    // rows by rank, then by distance descending (NaN last), then by index: one stable step per key part, least
+    // significant first (src/evox/operators/selection/non_dominate.py:253, src/evox/utils/jit_fix_operator.py:246-250)
+    void* sort_ws = base + L.sort_ws;
+    if (int e = evox_hip_stable_argsort_step(base + L.neg_lo, kKeyUint32, 1, n, nullptr, order_a, sort_ws, L.sort_bytes, s)) return e;
+    if (int e = evox_hip_stable_argsort_step(base + L.neg_hi, kKeyUint32, 1, n, order_a, order_b, sort_ws, L.sort_bytes, s)) return e;
+    if (int e = evox_hip_stable_argsort_step(rank, kKeyInt32, 1, n, order_b, order_a, sort_ws, L.sort_bytes, s)) return e;
+  }
   if (x != nullptr)
     if (int e = gather_rows(x, x_row_bytes, x_row_stride_bytes, order_a, topk, out_x, s)) return e;
   if (int e = gather_rows(f_rows, f_row_bytes, f_row_stride_bytes, order_a, topk, out_f, s)) return e;

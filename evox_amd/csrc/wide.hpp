@@ -21,11 +21,18 @@ constexpr int kWideFloat64 = 0;  // costs are IEEE doubles
 constexpr int kWideInt64 = 1;    // costs are two's-complement 64-bit integers
 constexpr int kWideFloat32 = 2;  // costs are IEEE floats (differences and quotients in float, as the float32 kernels compute them)
 
+// (see the kernels that order a last front without sorting the costs, below)
+constexpr int kWideDirectRows = 24576;
+// Beyond a front of this many rows the sorts are the faster way (direct: 160 us at 8192 candidates of three objectives,
+// 950 at 20 000); the host goes by what the last selection of the shape found (`outcome`: pinned host memory or
+// null; 1 = a front up to this size, 2 = a larger one), and either way handles a front of any size.
+constexpr int kWideDirectFront = 8192;
+
 struct WideCtrl {
   int nv;     // rows selected by the mask
   int worst;  // with a rank vector: the largest rank that is not EVOX_HIP_RANK_UNSET (the mask is rank == worst)
   int err;    // an order came back poisoned (a sort's bounded device-side wait ran out): the results are poisoned too
-  int pad;
+  int start;  // with a rank vector: the rows of the fronts before that one
 };
 
 // Order-preserving map double -> uint64 with torch's sort conventions: -0.0 and +0.0 share a key, every NaN maps to
@@ -63,18 +70,31 @@ __global__ __launch_bounds__(1024) void wide_head_kernel(const uint8_t* __restri
     worst = worst_lds;
     __syncthreads();
   }
-  int count = 0;
-  for (int i = threadIdx.x; i < n; i += blockDim.x)
+  int count = 0, better = 0;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
     count += rank != nullptr ? (rank[i] == worst) : (mask != nullptr ? (mask[(int64_t)i * mask_stride] != 0) : 1);
+    better += rank != nullptr && rank[i] < worst ? 1 : 0;
+  }
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) count += __shfl_xor(count, off);
-  if (lane == 0) red[wave] = count;
+  for (int off = 32; off > 0; off >>= 1) {
+    count += __shfl_xor(count, off);
+    better += __shfl_xor(better, off);
+  }
+  __shared__ int red_better[16];
+  if (lane == 0) {
+    red[wave] = count;
+    red_better[wave] = better;
+  }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int v = 1; v < (int)(blockDim.x >> 6); ++v) count += red[v];
+    for (int v = 1; v < (int)(blockDim.x >> 6); ++v) {
+      count += red[v];
+      better += red_better[v];
+    }
     ctrl->nv = count;
     ctrl->worst = worst;
     ctrl->err = 0;
+    ctrl->start = better;
   }
 }
 
@@ -159,8 +179,10 @@ template <class Out>
 __global__ __launch_bounds__(256) void wide_sum_kernel(const Out* __restrict__ terms, const uint8_t* __restrict__ selected,
                                                        const int* __restrict__ boundary, const WideCtrl* __restrict__ ctrl, int n,
                                                        int m, Out* __restrict__ dist, uint32_t* __restrict__ neg_lo,
-                                                       uint32_t* __restrict__ neg_hi) {
+                                                       uint32_t* __restrict__ neg_hi, int* __restrict__ outcome) {
   const bool failed = ctrl->err != 0;
+  if (outcome != nullptr && blockIdx.x == 0 && threadIdx.x == 0)
+    __hip_atomic_store(outcome, ctrl->nv > kWideDirectFront ? 2 : 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
     Out d;
     if (failed) {
@@ -179,6 +201,176 @@ __global__ __launch_bounds__(256) void wide_sum_kernel(const Out* __restrict__ t
       neg_lo[i] = (uint32_t)image;
       neg_hi[i] = (uint32_t)(image >> 32);
     }
+  }
+}
+
+// ---- The same distances and the selection order without a sort of the costs, for populations of up to
+// kWideDirectRows rows.  `listing` holds the rows by (rank, row index) -- one stable argsort step of the ranks -- so
+// the rows of the last front are listing[start .. start + nv) in index order: candidate q of the front.  A candidate's
+// neighbours in an objective's order (non_dominate.py:221-225: by cost, ties by row index) are the largest composite
+// (ordered image of the cost, candidate number) below its own and the smallest above; sixteen lanes look for them
+// among all candidates, as crowd_small_front (finish.hpp) does for 4-byte costs held in LDS.  The work grows with the
+// square of the front -- 10 us for a front of some hundred rows, where the sorts of all n rows by every objective take
+// twelve launches of 40 us at 20 000 rows, and about as long as those sorts when all 20 000 rows are one front.
+
+__device__ inline uint64_t wide_image(const void* costs, int kind, int64_t at) {
+  return kind == kWideFloat64   ? ordered_key64(static_cast<const double*>(costs)[at])
+         : kind == kWideFloat32 ? ordered_key64((double)static_cast<const float*>(costs)[at])
+                                : ordered_key64(static_cast<const long long*>(costs)[at]);
+}
+
+// key[k][q] (columns n apart) of every candidate; dist = -inf for every row (the candidates' are written afterwards);
+// and, by workgroup k < m (or every gridDim.x-th objective), the candidates that stand first and last in objective
+// k's order: ends[2k], ends[2k + 1].
+template <class Out>
+__global__ __launch_bounds__(256) void wide_front_keys_kernel(const void* __restrict__ costs, int kind, int64_t stride_row,
+                                                              int64_t stride_col, int n, int m, const int* __restrict__ listing,
+                                                              const WideCtrl* __restrict__ ctrl, uint64_t* __restrict__ key,
+                                                              int* __restrict__ ends, Out* __restrict__ dist) {
+  __shared__ uint64_t lo_key[4], hi_key[4];
+  __shared__ int lo_at[4], hi_at[4];
+  const int nv = ctrl->nv, start = ctrl->start;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) dist[i] = (Out)(-INFINITY);
+  const int64_t total = (int64_t)nv * m;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+    const int k = (int)(idx / nv), q = (int)(idx - (int64_t)k * nv);
+    const int row = listing[start + q];
+    key[(int64_t)k * n + q] = row < 0 ? ~0ull : wide_image(costs, kind, (int64_t)row * stride_row + (int64_t)k * stride_col);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int k = blockIdx.x; k < m; k += gridDim.x) {
+    uint64_t lo = ~0ull, hi = 0ull;
+    int lo_q = -1, hi_q = -1;  // (ascending q per thread: the first of equal images stays first, the last one last)
+    for (int q = threadIdx.x; q < nv; q += blockDim.x) {
+      const int row = listing[start + q];
+      const uint64_t image = row < 0 ? ~0ull : wide_image(costs, kind, (int64_t)row * stride_row + (int64_t)k * stride_col);
+      if (lo_q < 0 || image < lo) lo = image, lo_q = q;
+      if (hi_q < 0 || image >= hi) hi = image, hi_q = q;
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const uint64_t other_lo = ((uint64_t)__shfl_xor((unsigned)(lo >> 32), off) << 32) | (unsigned)__shfl_xor((unsigned)lo, off);
+      const uint64_t other_hi = ((uint64_t)__shfl_xor((unsigned)(hi >> 32), off) << 32) | (unsigned)__shfl_xor((unsigned)hi, off);
+      const int other_lo_q = __shfl_xor(lo_q, off), other_hi_q = __shfl_xor(hi_q, off);
+      if (other_lo_q >= 0 && (lo_q < 0 || other_lo < lo || (other_lo == lo && other_lo_q < lo_q))) lo = other_lo, lo_q = other_lo_q;
+      if (other_hi_q >= 0 && (hi_q < 0 || other_hi > hi || (other_hi == hi && other_hi_q > hi_q))) hi = other_hi, hi_q = other_hi_q;
+    }
+    __syncthreads();  // (the arrays are reused from objective to objective)
+    if (lane == 0) {
+      lo_key[wave] = lo;
+      lo_at[wave] = lo_q;
+      hi_key[wave] = hi;
+      hi_at[wave] = hi_q;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      for (int v = 1; v < (int)(blockDim.x >> 6); ++v) {
+        if (lo_at[v] >= 0 && (lo_q < 0 || lo_key[v] < lo || (lo_key[v] == lo && lo_at[v] < lo_q))) lo = lo_key[v], lo_q = lo_at[v];
+        if (hi_at[v] >= 0 && (hi_q < 0 || hi_key[v] > hi || (hi_key[v] == hi && hi_at[v] > hi_q))) hi = hi_key[v], hi_q = hi_at[v];
+      }
+      ends[2 * k] = lo_q;
+      ends[2 * k + 1] = hi_q;
+    }
+  }
+}
+
+// The distance of every candidate (written by row) and the ordered image of its negative (by candidate number).
+template <class Out>
+__global__ __launch_bounds__(256) void wide_front_dist_kernel(const void* __restrict__ costs, int kind, int64_t stride_row,
+                                                              int64_t stride_col, int n, int m, const int* __restrict__ listing,
+                                                              WideCtrl* __restrict__ ctrl, const uint64_t* __restrict__ key,
+                                                              const int* __restrict__ ends, Out* __restrict__ dist,
+                                                              uint64_t* __restrict__ dkey) {
+  const int nv = ctrl->nv, start = ctrl->start;
+  const int sub = threadIdx.x & 15;
+  const int groups = (int)(gridDim.x * (blockDim.x >> 4));
+  for (int q = (int)(blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4)); q < nv; q += groups) {
+    const int row = listing[start + q];
+    bool boundary = false;
+    Out acc = (Out)0;
+    for (int k = 0; k < m; ++k) {
+      const uint64_t* __restrict__ col = key + (int64_t)k * n;
+      const uint64_t mine = col[q];
+      uint64_t below = 0ull, above = ~0ull;
+      int below_q = -1, above_q = -1;
+      for (int e0 = sub; e0 < nv; e0 += 4 * 16) {  // four partners per step, their loads in flight together
+        uint64_t c[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) c[u] = e0 + 16 * u < nv ? col[e0 + 16 * u] : mine;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int e = e0 + 16 * u;  // (e ascends within a lane)
+          const bool before = c[u] < mine || (c[u] == mine && e < q);
+          const bool after = c[u] > mine || (c[u] == mine && e > q);
+          if (e < nv && before && (below_q < 0 || c[u] >= below)) below = c[u], below_q = e;  // the last of the largest
+          if (e < nv && after && (above_q < 0 || c[u] < above)) above = c[u], above_q = e;    // the first of the smallest
+        }
+      }
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1) {
+        const uint64_t ob = ((uint64_t)__shfl_xor((unsigned)(below >> 32), off) << 32) | (unsigned)__shfl_xor((unsigned)below, off);
+        const uint64_t oa = ((uint64_t)__shfl_xor((unsigned)(above >> 32), off) << 32) | (unsigned)__shfl_xor((unsigned)above, off);
+        const int obq = __shfl_xor(below_q, off), oaq = __shfl_xor(above_q, off);
+        if (obq >= 0 && (below_q < 0 || ob > below || (ob == below && obq > below_q))) below = ob, below_q = obq;
+        if (oaq >= 0 && (above_q < 0 || oa < above || (oa == above && oaq < above_q))) above = oa, above_q = oaq;
+      }
+      if (below_q < 0 || above_q < 0) {
+        boundary = true;  // first or last of this objective (non_dominate.py:226-227)
+      } else if (row >= 0) {
+        const int64_t c0 = (int64_t)k * stride_col;
+        const Out term = wide_term<Out>(costs, kind, (int64_t)listing[start + above_q] * stride_row + c0,
+                                        (int64_t)listing[start + below_q] * stride_row + c0,
+                                        (int64_t)listing[start + ends[2 * k + 1]] * stride_row + c0,
+                                        (int64_t)listing[start + ends[2 * k]] * stride_row + c0);
+        acc = k == 0 ? term : acc + term;
+      }
+    }
+    if (sub == 0) {
+      if (row < 0) {  // a poisoned listing
+        ctrl->err = 1;
+        dkey[q] = ~0ull;
+      } else {
+        const Out d = boundary ? (Out)INFINITY : acc;
+        dist[row] = d;
+        dkey[q] = ordered_key64(-(double)d);
+      }
+    }
+  }
+}
+
+// The selection order: the fronts before the last one as listed, the candidates by (distance descending, NaN last,
+// row index), what the ranking left without a rank behind them as listed.  Every entry -1 when something was poisoned.
+__global__ __launch_bounds__(256) void wide_front_order_kernel(const int* __restrict__ listing, const WideCtrl* __restrict__ ctrl,
+                                                               const uint64_t* __restrict__ dkey, int n, int* __restrict__ order,
+                                                               int* __restrict__ outcome) {
+  const int nv = ctrl->nv, start = ctrl->start;
+  const bool failed = ctrl->err != 0;
+  if (outcome != nullptr && blockIdx.x == 0 && threadIdx.x == 0)
+    __hip_atomic_store(outcome, nv > kWideDirectFront ? 2 : 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
+    if (failed)
+      order[i] = -1;
+    else if (i < start || i >= start + nv)
+      order[i] = listing[i];
+  if (failed) return;
+  const int sub = threadIdx.x & 15;
+  const int groups = (int)(gridDim.x * (blockDim.x >> 4));
+  for (int q = (int)(blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4)); q < nv; q += groups) {
+    const uint64_t mine = dkey[q];
+    int smaller = 0;
+    for (int e0 = sub; e0 < nv; e0 += 4 * 16) {
+      uint64_t c[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) c[u] = e0 + 16 * u < nv ? dkey[e0 + 16 * u] : ~0ull;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int e = e0 + 16 * u;
+        smaller += e < nv && (c[u] < mine || (c[u] == mine && e < q)) ? 1 : 0;
+      }
+    }
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) smaller += __shfl_xor(smaller, off);
+    if (sub == 0) order[start + smaller] = listing[start + q];
   }
 }
 

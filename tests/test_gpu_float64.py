@@ -145,3 +145,51 @@ def test_float64_long_sorts_and_vmap(float64_default):
         want = er.environmental_selection(xb[b], fb[b], 120)
         assert torch.equal(sel[0][b].cpu(), want[0]) and torch.equal(sel[2][b].cpu(), want[2])
         _close(sel[3][b], want[3], ("vmap selection", b))
+
+
+def test_float64_selection_either_side_of_the_direct_limit(float64_default):
+    """Up to 24 576 rows the last front's distances and order come from kernels that look for every candidate's
+    neighbours among the candidates (whatever the size of the front: here one front of all rows, ties included);
+    above, from sorts of all rows.  The larger populations hold values that float32 represents exactly, so that the C
+    checker (float32) gives their ranks and, to float32's rounding, their distances."""
+    from oracle import c_oracle
+
+    g = torch.Generator("cpu").manual_seed(68)
+    a = (torch.rand(6000, generator=g, dtype=torch.float64) * 900).round() / 900  # one front with duplicates
+    f = torch.stack([a, 1.0 - a], dim=1)
+    x = torch.arange(6000, dtype=torch.int64)[:, None]
+    for k in (1, 3000, 6000):
+        want = er.environmental_selection(x, f, k)
+        got = nd_environmental_selection(x.to(DEV), f.to(DEV), k)
+        assert torch.equal(got[2].cpu(), want[2]), k
+        _close(got[3], want[3], ("one front", k))
+        if not torch.equal(got[0].cpu(), want[0]):  # (equal distances at the cut may change places only among themselves)
+            gw, ww = as_np(got[3]), as_np(want[3])
+            assert np.array_equal(np.sort(gw[np.isfinite(gw)]), np.sort(ww[np.isfinite(ww)])), k
+    # a front beyond what those kernels are meant for: the first selection of the shape goes through them all the same,
+    # the next ones through the sorts (the library remembers what the last selection of a shape found)
+    a = torch.rand(12000, generator=g, dtype=torch.float64)
+    f = torch.stack([a, 1.0 - a], dim=1)
+    x = torch.arange(12000, dtype=torch.int64)[:, None]
+    want = er.environmental_selection(x, f, 7000)
+    for call in range(3):
+        got = nd_environmental_selection(x.to(DEV), f.to(DEV), 7000)
+        assert torch.equal(got[0].cpu(), want[0]) and torch.equal(got[2].cpu(), want[2]), call
+        _close(got[3], want[3], ("one front of 12000", call))
+    for n, m in ((24576, 2), (30000, 3)):
+        f32 = torch.rand(n, m, generator=g)
+        k = n // 2
+        order, rank, dist, _ = c_oracle.select(f32.numpy(), k)
+        order, rank, dist = as_np(order)[:k], as_np(rank), as_np(dist)
+        got = nd_environmental_selection(torch.arange(n, dtype=torch.int64, device=DEV)[:, None], f32.double().to(DEV), k)
+        assert got[3].dtype == torch.float64
+        rows = as_np(got[0])[:, 0]
+        assert np.array_equal(as_np(got[2]), rank[rows]) and np.array_equal(np.sort(rank[rows]), np.sort(rank[order])), (n, m)
+        worst = rank[order].max()
+        assert np.array_equal(np.sort(rows[rank[rows] < worst]), np.sort(order[rank[order] < worst])), (n, m)
+        gd, wd = as_np(got[3]), dist[rows]
+        fin = np.isfinite(wd)
+        assert np.array_equal(np.isfinite(gd), fin), (n, m)
+        np.testing.assert_allclose(gd[fin], wd[fin], rtol=1e-4, err_msg=str((n, m)))  # (the checker's sums are float32)
+        cut = rank[rows] == worst  # taken from the cut front by descending distance
+        assert (gd[cut][:-1] >= gd[cut][1:]).all(), (n, m)
