@@ -2260,6 +2260,21 @@ int evox_hip_many_nd_environmental_selection(const void* x, int64_t x_row_bytes,
 
 extern "C" {
 
+int evox_hip_dense_rank_rows(const void* sorted, int kind, const int64_t* index, int64_t batch, int64_t n, int64_t m, float* out,
+                             void* stream) {
+  if (sorted == nullptr || index == nullptr || out == nullptr || (kind != kWideFloat64 && kind != kWideInt64)) return kErrBadArg;
+  if (batch < 1 || n < 1 || m < 1 || n >= (1ll << 24) || batch * m > 0x7FFFFFFFll) return kErrBadArg;
+  hipStream_t s = (hipStream_t)stream;
+  if (kind == kWideFloat64)
+    hipLaunchKernelGGL(dense_rank_kernel<double>, dim3((unsigned)(batch * m)), dim3(kDenseRankThreads), 0, s,
+                       static_cast<const double*>(sorted), index, (int)n, (int)m, out);
+  else
+    hipLaunchKernelGGL(dense_rank_kernel<long long>, dim3((unsigned)(batch * m)), dim3(kDenseRankThreads), 0, s,
+                       static_cast<const long long*>(sorted), index, (int)n, (int)m, out);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
 size_t evox_hip_wide_workspace_bytes(int64_t n, int64_t m) {
   WideLayout L;
   return make_wide_layout(n, m, &L) ? L.total : 0;

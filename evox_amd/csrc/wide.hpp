@@ -374,6 +374,62 @@ __global__ __launch_bounds__(256) void wide_front_order_kernel(const int* __rest
   }
 }
 
+// ---- The dense ranks of the values of one objective, from their sorted order: what the ranking kernels, which read
+// 4-byte floats, get in place of 8-byte fitness (dominance only looks at the order of the values inside an objective).
+// One workgroup per sorted row: sorted[row][p] ascending (NaN last), index[row][p] the place the value came from;
+// out[(b * n + index) * m + k] for row = b * m + k gets the number of distinct values before it (-0.0 and 0.0 are one
+// value), as a float -- exact below 2^24 -- and NaN where the value is NaN.
+constexpr int kDenseRankThreads = 1024;
+constexpr int kDenseRankPer = 4;
+
+template <class T>
+__global__ __launch_bounds__(kDenseRankThreads) void dense_rank_kernel(const T* __restrict__ sorted, const int64_t* __restrict__ index,
+                                                                       int n, int m, float* __restrict__ out) {
+  __shared__ int wave_total[kDenseRankThreads / 64];
+  __shared__ int carry_lds;
+  const int row = blockIdx.x, b = row / m, k = row - b * m;
+  const T* __restrict__ v = sorted + (int64_t)row * n;
+  const int64_t* __restrict__ at = index + (int64_t)row * n;
+  float* __restrict__ dst = out + (int64_t)b * n * m + k;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0) carry_lds = 0;
+  __syncthreads();
+  for (int base = 0; base < n; base += kDenseRankThreads * kDenseRankPer) {
+    const int p0 = base + (int)threadIdx.x * kDenseRankPer;
+    int opens[kDenseRankPer];
+    T mine[kDenseRankPer];
+    T before = p0 > 0 && p0 - 1 < n ? v[p0 - 1] : T(0);
+    int sum = 0;
+#pragma unroll
+    for (int e = 0; e < kDenseRankPer; ++e) {
+      const int p = p0 + e;
+      mine[e] = p < n ? v[p] : T(0);
+      opens[e] = p > 0 && p < n && mine[e] != before ? 1 : 0;  // (a NaN differs from everything, itself included)
+      sum += opens[e];
+      before = mine[e];
+    }
+    int incl = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(incl, off);
+      if (lane >= off) incl += up;
+    }
+    if (lane == 63) wave_total[wave] = incl;
+    __syncthreads();
+    int rank = carry_lds + incl - sum;
+    for (int w = 0; w < wave; ++w) rank += wave_total[w];
+#pragma unroll
+    for (int e = 0; e < kDenseRankPer; ++e) {
+      const int p = p0 + e;
+      rank += opens[e];
+      if (p < n) dst[at[p] * m] = mine[e] != mine[e] ? NAN : (float)rank;
+    }
+    __syncthreads();
+    if (threadIdx.x == kDenseRankThreads - 1) carry_lds = rank;  // (the last thread's last rank: everything so far)
+    __syncthreads();
+  }
+}
+
 // dst row r = src row order[r] (raw bytes), for r < count, `unit` bytes at a time; all-ones bytes for a row of a
 // poisoned order (-1).
 __global__ __launch_bounds__(256) void gather_rows_kernel(const uint8_t* __restrict__ src, int64_t row_bytes,

@@ -60,6 +60,14 @@ def _order_preserving_f32(t: torch.Tensor, what: str) -> torch.Tensor:
     # (every objective as a contiguous row: torch's scan along any other dimension takes milliseconds for 20 000 rows)
     flat = t.reshape(-1, t.shape[-2], t.shape[-1]).transpose(1, 2).contiguous()
     values, index = torch.sort(flat, dim=2)
+    if flat.dtype in (torch.float64, torch.int64) and flat.is_cuda:
+        # the rest in one kernel: a value opens a new rank when it differs from the one before it, the ranks go back to
+        # the rows that the values came from
+        dense = torch.empty(flat.size(0), flat.size(2), flat.size(1), dtype=torch.float32, device=t.device)
+        with torch.cuda.device(t.device):
+            _lib.call("evox_hip_dense_rank_rows", values.data_ptr(), 0 if flat.dtype == torch.float64 else 1, index.data_ptr(),
+                      flat.size(0), flat.size(2), flat.size(1), dense.data_ptr(), runtime.stream_handle(t.device))
+        return dense.reshape(t.shape)
     opens = torch.zeros(flat.shape, dtype=torch.int32, device=t.device)
     opens[:, :, 1:] = values[:, :, 1:] != values[:, :, :-1]
     dense = torch.empty(flat.shape, dtype=torch.float32, device=t.device)

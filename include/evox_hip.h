@@ -96,6 +96,16 @@ int evox_hip_crowding_distance_wide(const void* costs, int kind, int64_t n, int6
                                     const uint8_t* mask, int64_t mask_stride, void* dist_out, int out_kind, void* workspace,
                                     size_t workspace_bytes, void* stream);
 
+/* The float32 image of such fitness that the ranking entry points take: dominance (non_dominate.py:6-26) only looks
+ * at the order of the values inside an objective, so the ranks of fitness of any ordered dtype are the ranks of its
+ * per-objective dense ranks.  sorted: (batch, m, n) values of kind 0 = float64 or 1 = int64, every row ascending
+ * with NaN last; index: (batch, m, n) int64, the row that each value came from (what a sort of every objective
+ * returns).  out: (batch, n, m) float32: the number of distinct values of the objective below the row's (-0.0 and
+ * 0.0 are one value), NaN where the value is NaN; n below 2^24.  Nothing of this shape exists in the reference, which
+ * compares the values themselves (:20-24); it stands in for those comparisons. */
+int evox_hip_dense_rank_rows(const void* sorted, int kind, const int64_t* index, int64_t batch, int64_t n, int64_t m,
+                             float* out, void* stream);
+
 /* The selection steps after the ranking for such fitness (non_dominate.py:249-254): given rank (int32, n entries,
  * EVOX_HIP_RANK_UNSET behind the front that holds the topk-th row, as evox_hip_non_dominate_rank_until leaves them on
  * any order-preserving float32 image of the fitness), the distances of the rows of the largest set rank (the mask

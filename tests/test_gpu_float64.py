@@ -193,3 +193,35 @@ def test_float64_selection_either_side_of_the_direct_limit(float64_default):
         np.testing.assert_allclose(gd[fin], wd[fin], rtol=1e-4, err_msg=str((n, m)))  # (the checker's sums are float32)
         cut = rank[rows] == worst  # taken from the cut front by descending distance
         assert (gd[cut][:-1] >= gd[cut][1:]).all(), (n, m)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.int64])
+def test_dense_rank_image(dtype):
+    """The float32 image that the ranking takes in place of 8-byte fitness: per objective, the number of distinct
+    values below a row's value (one kernel behind a sort of every objective), against numpy."""
+    from evox_amd import ops
+
+    g = torch.Generator("cpu").manual_seed(69)
+    for shape in ((1, 1), (5, 2), (4097, 3), (3, 50000, 2), (2, 2, 700, 4)):
+        if dtype == torch.float64:
+            f = (torch.rand(*shape, generator=g, dtype=torch.float64) * 50).round() / 50
+            flat = f.view(-1)
+            if flat.numel() > 40:
+                flat[3], flat[11] = 0.0, -0.0
+                flat[5], flat[20] = float("nan"), float("nan")
+                flat[7], flat[9] = float("inf"), -float("inf")
+                flat[13] = 1.0 + 2.0**-40  # not a float32 value
+        else:
+            f = torch.randint(-(2**40), 2**40, shape, generator=g, dtype=torch.int64)
+            f.view(-1)[::3] //= 2**38  # ties
+        got = as_np(ops._order_preserving_f32(f.to(DEV), "fitness"))
+        assert got.dtype == np.float32 and got.shape == tuple(shape)
+        cols = f.numpy().reshape(-1, shape[-2], shape[-1])
+        for b in range(cols.shape[0]):
+            for k in range(shape[-1]):
+                col = cols[b][:, k]
+                want = np.full(col.shape, np.nan, dtype=np.float32)
+                ok = ~np.isnan(col) if dtype == torch.float64 else np.ones(col.shape, bool)
+                values = np.unique(col[ok] + 0.0 if dtype == torch.float64 else col[ok])  # (-0.0 + 0.0 == 0.0)
+                want[ok] = np.searchsorted(values, col[ok]).astype(np.float32)
+                assert np.array_equal(got.reshape(cols.shape)[b][:, k], want, equal_nan=True), (shape, b, k)
