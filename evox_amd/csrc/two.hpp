@@ -50,7 +50,7 @@ constexpr int kTwoThreads = 1024;
 constexpr int kTwoWaves = kTwoThreads / 64;
 constexpr int kTwoPerThread = 4;                             // consecutive slots per thread
 constexpr int kTwoChunk = (kTwoThreads - 64) * kTwoPerThread;  // slots per workgroup: the first wave holds none
-constexpr int kTwoMaxBlocks = 256;
+constexpr int kTwoMaxBlocks = 512;  // (two workgroups of 1024 threads per compute unit)
 constexpr int64_t kTwoMaxRows = (int64_t)kTwoChunk * kTwoMaxBlocks;
 constexpr int kTwoRing = 256;                                // rounds of a workgroup's outgoing stream that are kept
 constexpr int kTwoRingStride = kTwoRing + 16;                // words per workgroup: the ring, then its progress counter on a line of its own
