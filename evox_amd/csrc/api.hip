@@ -1896,17 +1896,6 @@ static int wide_select_direct(const WideLayout& L, uint8_t* base, const void* co
   return 0;
 }
 
-static int gather_rows(const void* src, int64_t row_bytes, int64_t row_stride_bytes, const int* order, int64_t count, void* dst,
-                       hipStream_t s) {
-  if (row_bytes <= 0 || count <= 0) return 0;
-  const uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | (uintptr_t)row_bytes | (uintptr_t)row_stride_bytes;
-  const int unit = bits % 16 == 0 ? 16 : bits % 8 == 0 ? 8 : bits % 4 == 0 ? 4 : 1;
-  hipLaunchKernelGGL(gather_rows_kernel, dim3(wide_grid(count * (row_bytes / unit))), dim3(256), 0, s, static_cast<const uint8_t*>(src),
-                     row_bytes, row_stride_bytes, order, count, static_cast<uint8_t*>(dst), unit);
-  EVX_LAUNCH_CHECK();
-  return 0;
-}
-
 namespace evx {
 static size_t wide_workspace_need(int64_t n, int64_t m) {
   WideLayout L;
@@ -2321,12 +2310,30 @@ int evox_hip_nd_environmental_selection_wide(const void* x, int64_t x_row_bytes,
     if (int e = evox_hip_stable_argsort_step(base + L.neg_hi, kKeyUint32, 1, n, order_a, order_b, sort_ws, L.sort_bytes, s)) return e;
     if (int e = evox_hip_stable_argsort_step(rank, kKeyInt32, 1, n, order_b, order_a, sort_ws, L.sort_bytes, s)) return e;
   }
-  if (x != nullptr)
-    if (int e = gather_rows(x, x_row_bytes, x_row_stride_bytes, order_a, topk, out_x, s)) return e;
-  if (int e = gather_rows(f_rows, f_row_bytes, f_row_stride_bytes, order_a, topk, out_f, s)) return e;
-  if (int e = gather_rows(rank, 4, 4, order_a, topk, out_rank, s)) return e;
+  // the four gathers in one launch
+  GatherParts parts;
+  parts.parts = 0;
+  parts.first[0] = 0;
+  auto add_part = [&](const void* src, int64_t row_bytes, int64_t row_stride_bytes, void* dst) {
+    if (row_bytes <= 0) return;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | (uintptr_t)row_bytes | (uintptr_t)row_stride_bytes;
+    const int unit = bits % 16 == 0 ? 16 : bits % 8 == 0 ? 8 : bits % 4 == 0 ? 4 : 1;
+    const int p = parts.parts++;
+    parts.src[p] = static_cast<const uint8_t*>(src);
+    parts.dst[p] = static_cast<uint8_t*>(dst);
+    parts.row_bytes[p] = row_bytes;
+    parts.row_stride_bytes[p] = row_stride_bytes;
+    parts.unit[p] = unit;
+    parts.first[p + 1] = parts.first[p] + topk * (row_bytes / unit);
+  };
+  if (x != nullptr) add_part(x, x_row_bytes, x_row_stride_bytes, out_x);
+  add_part(f_rows, f_row_bytes, f_row_stride_bytes, out_f);
+  add_part(rank, 4, 4, out_rank);
   const int64_t dist_bytes = out_kind == 0 ? 8 : 4;
-  return gather_rows(dist, dist_bytes, dist_bytes, order_a, topk, out_dist, s);
+  add_part(dist, dist_bytes, dist_bytes, out_dist);
+  hipLaunchKernelGGL(gather_parts_kernel, dim3(wide_grid(parts.first[parts.parts])), dim3(256), 0, s, parts, order_a, topk);
+  EVX_LAUNCH_CHECK();
+  return 0;
 }
 
 }  // extern "C"

@@ -430,22 +430,33 @@ __global__ __launch_bounds__(kDenseRankThreads) void dense_rank_kernel(const T* 
   }
 }
 
-// dst row r = src row order[r] (raw bytes), for r < count, `unit` bytes at a time; all-ones bytes for a row of a
-// poisoned order (-1).
-__global__ __launch_bounds__(256) void gather_rows_kernel(const uint8_t* __restrict__ src, int64_t row_bytes,
-                                                          int64_t row_stride_bytes, const int* __restrict__ order, int64_t count,
-                                                          uint8_t* __restrict__ dst, int unit) {
-  const int64_t per_row = row_bytes / unit;
-  const int64_t total = count * per_row;
-  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t r = idx / per_row, u = idx - r * per_row;
+// Up to four gathers of rows by one order in one launch (decision vectors, fitness rows, ranks, distances of a
+// selection): dst row r = src row order[r] (raw bytes) for r < count, unit[p] bytes at a time; all-ones bytes for a row
+// of a poisoned order (-1).  Part p copies rows of row_bytes[p] bytes.
+struct GatherParts {
+  const uint8_t* src[4];
+  uint8_t* dst[4];
+  int64_t row_bytes[4], row_stride_bytes[4];
+  int64_t first[5];  // the work items (count x units per row) of part p are first[p] .. first[p + 1]
+  int unit[4];
+  int parts;
+};
+
+__global__ __launch_bounds__(256) void gather_parts_kernel(GatherParts g, const int* __restrict__ order, int64_t count) {
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < g.first[g.parts]; idx += (int64_t)gridDim.x * blockDim.x) {
+    int p = 0;
+    while (p + 1 < g.parts && idx >= g.first[p + 1]) ++p;
+    const int unit = g.unit[p];
+    const int64_t per_row = g.row_bytes[p] / unit;
+    const int64_t local = idx - g.first[p];
+    const int64_t r = local / per_row, u = local - r * per_row;
     const int row = order[r];
-    uint8_t* to = dst + r * row_bytes + u * unit;
+    uint8_t* to = g.dst[p] + r * g.row_bytes[p] + u * unit;
     if (row < 0) {
       for (int b = 0; b < unit; ++b) to[b] = 0xFF;
       continue;
     }
-    const uint8_t* from = src + (int64_t)row * row_stride_bytes + u * unit;
+    const uint8_t* from = g.src[p] + (int64_t)row * g.row_stride_bytes[p] + u * unit;
     if (unit == 16)
       *reinterpret_cast<uint4*>(to) = *reinterpret_cast<const uint4*>(from);
     else if (unit == 8)
