@@ -2174,12 +2174,16 @@ int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_ro
 static int many_populations_share(const Layout& L, int64_t batch, int64_t stop_count) {
   if (batch < 2 || opt().peel_stepped || !opt().peel_lds || L.n > 32768) return 0;
   if (!opt().mid_argsort && L.n > kRadixMinCandidates) return 0;  // (large last fronts would take the radix grid)
-  if (two_applies(L, stop_count)) return 0;
   int share = 4 * device_cus() / 9;  // at least eight sweeping workgroups and the lister per population, up to four on a compute unit
   if (share > batch) share = (int)batch;
   size_t lds = 0;
   while (share >= 2 && lds_peel_plan(L, &lds, share) == 0) --share;
   if (share < 2) return 0;
+  // Two objectives above the one-workgroup kernel's rows: a population alone goes through the chain of workgroups
+  // without a matrix (two.hpp), which takes one population at a time; several together are faster through the
+  // matrix kernels that they share (16 x 5000 x 2: 258 us against 1663 one after the other, 64 x 6000 x 2: 1.08
+  // against 6.99 ms, 16 x 10 000 x 2: 1.27 against 2.63 ms) unless few of them fit a launch.
+  if (two_applies(L, stop_count) && share < 4 && L.n > 12288) return 0;
   const int64_t passes = (batch + share - 1) / share;
   return (int)((batch + passes - 1) / passes);  // even passes: 30 populations, 28 at a time at most -> 15 + 15
 }

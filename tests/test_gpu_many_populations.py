@@ -49,6 +49,9 @@ SHAPES = [  # batch, n, m, kind
     (16, 4096, 3, "uniform"), (5, 2000, 2, "ties"), (7, 1500, 5, "fronts"), (30, 1100, 3, "uniform"), (2, 9000, 8, "uniform"),
     (4, 3000, 16, "ties"), (3, 1300, 17, "uniform"), (6, 2500, 3, "one_front"), (9, 5000, 4, "fronts"), (3, 20000, 3, "uniform"),
     (12, 1025, 1, "ties"), (2, 12000, 3, "one_front"),
+    # two objectives above the rows of the one-workgroup kernel: alone they go through the chain of workgroups,
+    # together through the kernels that they share
+    (6, 5000, 2, "ties"), (3, 9000, 2, "fronts"),
 ]
 
 
