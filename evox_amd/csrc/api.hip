@@ -1251,6 +1251,7 @@ static int launch_batched(const BatchedArgs& a, int64_t batch, hipStream_t s) {
 using namespace evx;
 
 static bool two_applies(const Layout& L, int64_t stop_count);
+static int many_two_share(const Layout& L, int64_t batch, int64_t stop_count);
 static int stage_rank_two(const Ws& w, const Fitness& src, int64_t stop_count, bool fill_dist, int* rank_until, hipStream_t s);
 
 extern "C" {
@@ -1438,12 +1439,12 @@ static int rank_rows(const Fitness& fit, int64_t n, int64_t m, int64_t stop_coun
     w.batch = batch;
     w.step = ws_step;
   }
-  if (batch == 1 && two_applies(w.L, stop_count)) {
+  if (batch == 1 ? two_applies(w.L, stop_count) : many_two_share(w.L, batch, stop_count) >= batch) {
     int* until = stop_count < n ? w.at<int>(w.L.order) : (int*)nullptr;
     const int e = stage_rank_two(w, fit, stop_count, false, until, s);
-    if (e != kErrNotResident) {
-      if (e) return e;
-      return copy_out(w.ctrl(), rank_out, until != nullptr ? until : w.at<int>(w.L.rank), n, kPoisonIndex, s);
+    if (e != kErrNotResident || batch > 1) {
+      if (e) return e == kErrNotResident ? kErrBadArg : e;
+      return copy_out(w.ctrl(), rank_out, until != nullptr ? until : w.at<int>(w.L.rank), n, kPoisonIndex, s, w.batch, w.step);
     }
   }
   if (int e = stage_prepare(w, fit, true, s)) return e;
@@ -1691,6 +1692,40 @@ static int argsort_step(const void* key, int kind, int64_t stride, int64_t n, co
   return copy_out(reinterpret_cast<const Ctrl*>(base + L.ctrl), order_out, nullptr, n, kPoisonIndex, s);
 }
 
+// One stable argsort step of int32 keys for each of `batch` populations in one launch (n <= kMidArgsortRows, the
+// kernels that never wait): keys key_step bytes apart, orders order_step bytes apart.
+static int argsort_step_many(const void* key, int64_t n, int batch, int64_t key_step, int32_t* order_out, int64_t order_step,
+                             hipStream_t s) {
+  if (n <= kSmallArgsortRows) {
+    const int npad = ((int)n + 127) & ~127;
+    if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(small_argsort_kernel), sizeof(double) * (size_t)npad)) return e;
+    hipLaunchKernelGGL(small_argsort_kernel, dim3(npad / kSmallArgsortGroup, batch), dim3(kSmallArgsortThreads),
+                       sizeof(double) * (size_t)npad, s, key, (int)kKeyInt32, (int64_t)1, (int)n, (const int*)nullptr, order_out, key_step,
+                       order_step);
+    EVX_LAUNCH_CHECK();
+    return 0;
+  }
+  if (n > kMidArgsortRows) return kErrBadArg;
+  const size_t lds = mid_sort_lds_bytes((int)n);
+  const bool wide = n <= kMidArgsortWideRows;
+  if (int e = grant_dynamic_lds(wide ? reinterpret_cast<const void*>(mid_argsort_kernel<true>)
+                                     : reinterpret_cast<const void*>(mid_argsort_kernel<false>), lds))
+    return e;
+  // (a population's share of the compute units, at least sixteen workgroups)
+  int blocks = device_cus() / batch;
+  if (blocks < 16) blocks = 16;
+  const int per = (int)round_up((n + blocks - 1) / blocks, 16);
+  const dim3 grid((unsigned)((n + per - 1) / per), (unsigned)batch);
+  if (wide)
+    hipLaunchKernelGGL(mid_argsort_kernel<true>, grid, dim3(kMidArgsortThreads), lds, s, key, (int)kKeyInt32, (int64_t)1, (int)n,
+                       (const int*)nullptr, per, order_out, key_step, order_step);
+  else
+    hipLaunchKernelGGL(mid_argsort_kernel<false>, grid, dim3(kMidArgsortThreads), lds, s, key, (int)kKeyInt32, (int64_t)1, (int)n,
+                       (const int*)nullptr, per, order_out, key_step, order_step);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
 // `batch` sorts of n <= kSmallArgsortRows positions in one launch: a workgroup per sort, or several sorts per
 // workgroup when they are short.
 template <int T, int R>
@@ -1910,6 +1945,18 @@ static bool two_applies(const Layout& L, int64_t stop_count) {
   return L.m == 2 && opt().two_min_rows > 0 && L.n >= least && L.n <= kTwoMaxRows && !opt().peel_stepped;
 }
 
+// Several populations at once take that path when their argsort of the ranks is one of the kernels that never wait
+// and all their chains are resident together: how many of `batch` share a launch (0: none).
+static int many_two_share(const Layout& L, int64_t batch, int64_t stop_count) {
+  if (batch < 2 || !two_applies(L, stop_count) || L.n > kMidArgsortRows || !opt().mid_argsort) return 0;
+  const int blocks = (L.n + kTwoChunk - 1) / kTwoChunk;
+  int share = device_cus() * 2 / blocks;
+  if (share > batch) share = (int)batch;
+  if (share < 2) return 0;
+  const int64_t passes = (batch + share - 1) / share;
+  return (int)((batch + passes - 1) / passes);
+}
+
 // Leaves what count_and_peel leaves: ranks by original index (of every row), the listing, the front starts and sizes
 // and the control block's description of the front that holds the stop_count-th row.  rank_until: optionally the
 // ranks with the rows behind that front unset (n ints).
@@ -1921,26 +1968,32 @@ static int stage_rank_two(const Ws& w, const Fitness& src, int64_t stop_count, b
   if (int e = stage_prepare(w, src, true, s, true)) return e;
   const int blocks = (L.n + kTwoChunk - 1) / kTwoChunk;
   // (every workgroup waits for the one before it: resident at once on any device with as many compute units)
-  if (blocks > device_cus() * 2) return kErrNotResident;
+  if ((int64_t)blocks * w.batch > device_cus() * 2) return kErrNotResident;
   const float* xs_sorted = w.at<float>(L.xs_sorted);
-  hipLaunchKernelGGL(two_peel_kernel, dim3(blocks), dim3(kTwoThreads), 0, s, xs_sorted, xs_sorted + L.npad, w.at<uint32_t>(L.kid_sorted),
-                     w.at<int>(L.orig_of), L.n, w.at<int>(L.rank), fill_dist ? w.at<float>(L.dist) : (float*)nullptr, w.ctrl(),
-                     w.at<unsigned long long>(L.two_ring), opt().spin_limit, (int)stop_count);
+  hipLaunchKernelGGL(two_peel_kernel, dim3(blocks, 1, w.batch), dim3(kTwoThreads), 0, s, xs_sorted, xs_sorted + L.npad,
+                     w.at<uint32_t>(L.kid_sorted), w.at<int>(L.orig_of), L.n, w.at<int>(L.rank),
+                     fill_dist ? w.at<float>(L.dist) : (float*)nullptr, w.ctrl(), w.at<unsigned long long>(L.two_ring), opt().spin_limit,
+                     (int)stop_count, w.step);
   EVX_LAUNCH_CHECK();
   int grid = (L.n + 255) / 256;
   if (grid > device_cus() * 8) grid = device_cus() * 8;
-  hipLaunchKernelGGL(two_finish_kernel, dim3(grid), dim3(256), 0, s, w.at<uint32_t>(L.kid_sorted), w.at<int>(L.orig_of), xs_sorted,
-                     xs_sorted + L.npad, L.n, w.at<int>(L.rank), w.ctrl());
+  grid = shared_grid(grid, device_cus() * 8, w.batch);
+  hipLaunchKernelGGL(two_finish_kernel, dim3(grid, 1, w.batch), dim3(256), 0, s, w.at<uint32_t>(L.kid_sorted), w.at<int>(L.orig_of),
+                     xs_sorted, xs_sorted + L.npad, L.n, w.at<int>(L.rank), w.ctrl(), w.step);
   EVX_LAUNCH_CHECK();
-  uint8_t* wb = w.base + L.wide;
-  if (int e = argsort_step(w.at<int>(L.rank), kKeyInt32, 1, L.n, nullptr, w.at<int>(L.perm), wb + WL.sort_ws, WL.sort_bytes, s,
-                           &w.ctrl()->reserved[kTwoRounds]))
-    return e;
-  hipLaunchKernelGGL(two_bounds_kernel, dim3(grid), dim3(256), 0, s, w.at<int>(L.perm), w.at<int>(L.rank), L.n, w.at<int>(L.fstart),
-                     w.ctrl(), (int)stop_count);
+  if (w.batch > 1) {
+    if (int e = argsort_step_many(w.at<int>(L.rank), L.n, w.batch, w.step, w.at<int>(L.perm), w.step, s)) return e;
+  } else {
+    uint8_t* wb = w.base + L.wide;
+    if (int e = argsort_step(w.at<int>(L.rank), kKeyInt32, 1, L.n, nullptr, w.at<int>(L.perm), wb + WL.sort_ws, WL.sort_bytes, s,
+                             &w.ctrl()->reserved[kTwoRounds]))
+      return e;
+  }
+  hipLaunchKernelGGL(two_bounds_kernel, dim3(grid, 1, w.batch), dim3(256), 0, s, w.at<int>(L.perm), w.at<int>(L.rank), L.n,
+                     w.at<int>(L.fstart), w.ctrl(), (int)stop_count, w.step);
   EVX_LAUNCH_CHECK();
-  hipLaunchKernelGGL(two_sizes_kernel, dim3(grid), dim3(256), 0, s, w.at<int>(L.perm), w.at<int>(L.rank), L.n, w.at<int>(L.fstart),
-                     w.at<int>(L.fsize), w.ctrl(), rank_until);
+  hipLaunchKernelGGL(two_sizes_kernel, dim3(grid, 1, w.batch), dim3(256), 0, s, w.at<int>(L.perm), w.at<int>(L.rank), L.n,
+                     w.at<int>(L.fstart), w.at<int>(L.fsize), w.ctrl(), rank_until, w.step);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -2017,10 +2070,10 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
     else
       hipLaunchKernelGGL(gather_kernel<false>, gather_grid, dim3(256), 0, s, g);
   };
-  if (batch == 1 && two_applies(L, topk)) {
+  if (batch == 1 ? two_applies(L, topk) : many_two_share(L, batch, topk) >= batch) {
     const int e = stage_rank_two(w, fit, topk, true, nullptr, s);
-    if (e != kErrNotResident) {
-      if (e) return e;
+    if (e != kErrNotResident || batch > 1) {
+      if (e) return e == kErrNotResident ? kErrBadArg : e;
       // the last front by the ordering kernels, then the gather, as after a peel that leaves the last front alone
       if (int c = stage_crowd_sort(w, w.at<int>(L.perm), false, 2, s, false)) return c;
       if (int c = stage_crowd_finish(w, w.at<int>(L.perm), true, 2, s, false)) return c;
@@ -2172,6 +2225,7 @@ int evox_hip_nd_environmental_selection_two_part(const void* x_a, int64_t x_a_ro
 // a population's matrix fits the LDS of its share of the compute units.  Reference: the batched loop of
 // src/evox/operators/selection/non_dominate.py:107-125 (torch.vmap of the ranking, utils/op_register.py:26-51).
 static int many_populations_share(const Layout& L, int64_t batch, int64_t stop_count) {
+  if (const int two = many_two_share(L, batch, stop_count)) return two;  // every population a chain of workgroups (two.hpp)
   if (batch < 2 || opt().peel_stepped || !opt().peel_lds || L.n > 32768) return 0;
   if (!opt().mid_argsort && L.n > kRadixMinCandidates) return 0;  // (large last fronts would take the radix grid)
   int share = 4 * device_cus() / 9;  // at least eight sweeping workgroups and the lister per population, up to four on a compute unit
@@ -2179,10 +2233,8 @@ static int many_populations_share(const Layout& L, int64_t batch, int64_t stop_c
   size_t lds = 0;
   while (share >= 2 && lds_peel_plan(L, &lds, share) == 0) --share;
   if (share < 2) return 0;
-  // Two objectives above the one-workgroup kernel's rows: a population alone goes through the chain of workgroups
-  // without a matrix (two.hpp), which takes one population at a time; several together are faster through the
-  // matrix kernels that they share (16 x 5000 x 2: 258 us against 1663 one after the other, 64 x 6000 x 2: 1.08
-  // against 6.99 ms, 16 x 10 000 x 2: 1.27 against 2.63 ms) unless few of them fit a launch.
+  // (two objectives where many_two_share does not apply -- the LDS sorter switched off: several populations are still
+  // faster through the matrix kernels that they share than one after the other, unless few of them fit a launch)
   if (two_applies(L, stop_count) && share < 4 && L.n > 12288) return 0;
   const int64_t passes = (batch + share - 1) / share;
   return (int)((batch + passes - 1) / passes);  // even passes: 30 populations, 28 at a time at most -> 15 + 15

@@ -291,10 +291,15 @@ constexpr int kSmallArgsortRows = 8192;  // measured per step: 30 us up to 8192 
 constexpr int kSmallArgsortThreads = 1024;
 constexpr int kSmallArgsortGroup = 16;
 
+// (blockIdx.y: one of several such steps in the launch, their keys key_step bytes and their orders order_step bytes apart)
 __global__ __launch_bounds__(kSmallArgsortThreads) void small_argsort_kernel(const void* __restrict__ key, int kind, int64_t stride,
                                                                              int n, const int* __restrict__ prev,
-                                                                             int* __restrict__ order_out) {
+                                                                             int* __restrict__ order_out, int64_t key_step = 0,
+                                                                             int64_t order_step = 0) {
   extern __shared__ double argsort_comp[];  // n rounded up to a multiple of 128 entries, +inf past n
+  key = static_cast<const char*>(key) + (int64_t)blockIdx.y * key_step;
+  order_out = reinterpret_cast<int*>(reinterpret_cast<char*>(order_out) + (int64_t)blockIdx.y * order_step);
+  if (prev != nullptr) prev = reinterpret_cast<const int*>(reinterpret_cast<const char*>(prev) + (int64_t)blockIdx.y * order_step);
   __shared__ int share[16 * (64 / kSmallArgsortGroup)][kSmallArgsortGroup];
   const int npad = (n + 127) & ~127;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -647,8 +652,13 @@ __device__ inline void mid_argsort_slice(void* lds, int n, int s0, int s1_wanted
 template <bool WIDE>
 __global__ __launch_bounds__(kMidArgsortThreads) void mid_argsort_kernel(const void* __restrict__ key, int kind, int64_t stride, int n,
                                                                          const int* __restrict__ prev, int slots_per_block,
-                                                                         int* __restrict__ order_out) {
+                                                                         int* __restrict__ order_out, int64_t key_step = 0,
+                                                                         int64_t order_step = 0) {
   extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];
+  // (blockIdx.y: one of several such steps in the launch, their keys key_step bytes and their orders order_step bytes apart)
+  key = static_cast<const char*>(key) + (int64_t)blockIdx.y * key_step;
+  order_out = reinterpret_cast<int*>(reinterpret_cast<char*>(order_out) + (int64_t)blockIdx.y * order_step);
+  if (prev != nullptr) prev = reinterpret_cast<const int*>(reinterpret_cast<const char*>(prev) + (int64_t)blockIdx.y * order_step);
   auto key_of = [&](int e) -> uint32_t {
     const int idx = prev ? prev[e] : e;
     if (kind == kKeyFloat32) return ordered_key(static_cast<const float*>(key)[(int64_t)idx * stride]);

@@ -92,12 +92,14 @@ __device__ inline uint32_t wave_prefix_min(uint32_t x) {
 // rows not ranked by then are left at kRankUnset, and a front after the one that holds the stop_count-th row may be
 // ranked in part.  Only first rows of a key count (copies and rows with a NaN do not): the peeling never ends before
 // the stop_count-th row has its rank, and goes through all fronts where copies make up the difference.
-// ring: gridDim.x * kTwoRingStride words, zero at the start of the call.
+// ring: gridDim.x * kTwoRingStride words, zero at the start of the call.  blockIdx.z: one of several populations in the
+// launch, whose buffers lie ws_step bytes apart (each population a chain of gridDim.x workgroups of its own).
 __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __restrict__ xs1_sorted, const float* __restrict__ xs2_sorted,
                                                                const uint32_t* __restrict__ kid, const int* __restrict__ orig_of,
                                                                int n, int* __restrict__ rank, float* __restrict__ dist_fill,
                                                                Ctrl* __restrict__ ctrl, unsigned long long* __restrict__ ring,
-                                                               unsigned spin_limit, int stop_count) {
+                                                               unsigned spin_limit, int stop_count, int64_t ws_step) {
+  to_population(ws_step, xs1_sorted, xs2_sorted, kid, orig_of, rank, dist_fill, ctrl, ring);
   __shared__ __attribute__((aligned(16))) uint32_t wave_min_lds[2][16];  // by the parity of the round; entries from kTwoWaves on stay "none"
   // by the parity of the round: incoming minimum, rows ranked before this workgroup, flags (these three from the
   // round's receiver), "the workgroup leaves behind this round's barrier" (from the publisher)
@@ -310,7 +312,8 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
 // After the brigade: the rows of a key take the rank of the key's first row.
 __global__ __launch_bounds__(256) void two_finish_kernel(const uint32_t* __restrict__ kid, const int* __restrict__ orig_of,
                                                          const float* __restrict__ xs1_sorted, const float* __restrict__ xs2_sorted,
-                                                         int n, int* __restrict__ rank, const Ctrl* __restrict__ ctrl) {
+                                                         int n, int* __restrict__ rank, const Ctrl* __restrict__ ctrl, int64_t ws_step) {
+  to_population(ws_step, kid, orig_of, xs1_sorted, xs2_sorted, rank, ctrl);
   if (ctrl->err != 0) return;
   for (int s = blockIdx.x * blockDim.x + threadIdx.x; s < n; s += gridDim.x * blockDim.x) {
     const int first = (int)kid[s];
@@ -327,7 +330,8 @@ __global__ __launch_bounds__(256) void two_finish_kernel(const uint32_t* __restr
 // describes it for the kernels that order it.  Every front up to that one is complete; later ones may be ranked in
 // part, their starts mean nothing.
 __global__ __launch_bounds__(256) void two_bounds_kernel(const int* __restrict__ perm, const int* __restrict__ rank, int n,
-                                                         int* __restrict__ fstart, Ctrl* __restrict__ ctrl, int stop_count) {
+                                                         int* __restrict__ fstart, Ctrl* __restrict__ ctrl, int stop_count, int64_t ws_step) {
+  to_population(ws_step, perm, rank, fstart, ctrl);
   if (ctrl->err != 0) return;
   const int worst = rank[perm[stop_count - 1]];
   for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < n; p += gridDim.x * blockDim.x) {
@@ -351,7 +355,8 @@ __global__ __launch_bounds__(256) void two_bounds_kernel(const int* __restrict__
 // ... and the sizes of the fronts, from their starts (one small launch behind the one above).
 __global__ __launch_bounds__(256) void two_sizes_kernel(const int* __restrict__ perm, const int* __restrict__ rank, int n,
                                                         const int* __restrict__ fstart, int* __restrict__ fsize,
-                                                        Ctrl* __restrict__ ctrl, int* __restrict__ rank_until_out) {
+                                                        Ctrl* __restrict__ ctrl, int* __restrict__ rank_until_out, int64_t ws_step) {
+  to_population(ws_step, perm, rank, fstart, fsize, ctrl, rank_until_out);  // (the ranks up to the cut lie in the workspaces too)
   if (ctrl->err != 0) return;
   const int worst = ctrl->worst;
   const int last = rank[perm[n - 1]];

@@ -191,3 +191,27 @@ def test_first_front_and_crowding_of_many_populations(batch, n, m, kind):
     # a mask that is a strided view, populations along the second dimension
     mapped = torch.vmap(crowding_distance, in_dims=(1, 1))(fd.permute(1, 0, 2).contiguous(), maskd.t().contiguous())
     assert np.array_equal(as_np(mapped), as_np(dist_masked), equal_nan=True)
+
+
+def test_chains_of_two_objective_populations_share_a_launch_and_report_a_wait_that_runs_out():
+    """Two objectives above 4096 rows: every population is a chain of workgroups of its own, all chains in one launch."""
+    assert _per_launch(16, 10000, 2, 5000) == 16 and _per_launch(300, 5000, 2, 5000) > 100
+    f, x = _populations(5, 6000, 2, 11, "fronts")
+    fd, xd = f.to(DEV), x.to(DEV)
+    with runtime.options(spin_limit=1):
+        rank = non_dominate_rank(fd)
+        with pytest.raises(_lib.EvoxHipError):
+            runtime.last_status()
+        got = nd_environmental_selection(xd, fd, 3000)
+    torch.cuda.synchronize()
+    for b in range(5):
+        r = as_np(rank[b])
+        if not (r == -1).all():  # (a chain of two workgroups may come through: the second one's first load can succeed)
+            assert np.array_equal(r, as_np(c_oracle.nd_rank(f[b])[0])), b
+        assert (as_np(got[2][b]) == -1).all() == bool(np.isnan(as_np(got[3][b])).all()), b
+    assert (as_np(rank) == -1).all(axis=1).any()
+    with runtime.options(two_min_rows=0):  # the matrix kernels for the same batch
+        other = nd_environmental_selection(xd, fd, 3000)
+    good = nd_environmental_selection(xd, fd, 3000)
+    for a, c in zip(good, other):
+        assert np.array_equal(as_np(a), as_np(c), equal_nan=True)
