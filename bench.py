@@ -352,7 +352,7 @@ def next_rows(dev, reps):
     # many populations of more rows than the one-workgroup kernel takes, in one call (the stages of the pipeline run
     # once for all of them) against one of them alone
     from evox_amd import runtime
-    for b, n, m in ((16, 4096, 3), (32, 1500, 3), (64, 2000, 2)):
+    for b, n, m in ((16, 4096, 3), (32, 1500, 3), (64, 2000, 2), (16, 10000, 2)):
         g = torch.Generator("cpu").manual_seed(6)
         fm = torch.rand(b, n, m, generator=g).to(dev)
         xm = torch.rand(b, n, 16, generator=g).to(dev)
