@@ -1914,11 +1914,12 @@ static int wide_select_direct(const WideLayout& L, uint8_t* base, const void* co
   if (int e = evox_hip_stable_argsort_step(rank, kKeyInt32, 1, n, nullptr, listing, base + L.sort_ws, L.sort_bytes, s)) return e;
   // (sixteen lanes per candidate; the grid is sized for a front of all rows, which the kernels find out on the device)
   const int pair_grid = wide_grid((int64_t)n * 16);
+  const int dist_grid = (n + 15) / 16;  // (a group of lanes per row, n <= kWideDirectRows)
   auto launch = [&](auto* typed_dist) {
     using Out = std::remove_pointer_t<decltype(typed_dist)>;
     hipLaunchKernelGGL(wide_front_keys_kernel<Out>, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, listing,
                        ctrl, key, ends, typed_dist);
-    hipLaunchKernelGGL(wide_front_dist_kernel<Out>, dim3(pair_grid), dim3(256), 0, s, costs, kind, sr, sc, n, m, listing, ctrl, key,
+    hipLaunchKernelGGL(wide_front_dist_kernel<Out>, dim3(dist_grid), dim3(256), 0, s, costs, kind, sr, sc, n, m, listing, ctrl, key,
                        ends, typed_dist, dkey);
   };
   if (out_kind == 0)

@@ -275,65 +275,79 @@ __global__ __launch_bounds__(256) void wide_front_keys_kernel(const void* __rest
 }
 
 // The distance of every candidate (written by row) and the ordered image of its negative (by candidate number).
+// Grid: a group of sixteen lanes per row of the population (ceil(n / 16) workgroups of 256 threads); the groups
+// beyond the front have nothing to do.  A front of up to kWideStagedFront rows has the images of an objective staged in
+// the LDS of every workgroup that holds candidates (otherwise every step of the search is a round trip to the L2:
+// 25 us for a front of 600 rows).
+constexpr int kWideStagedFront = 4096;
+
 template <class Out>
 __global__ __launch_bounds__(256) void wide_front_dist_kernel(const void* __restrict__ costs, int kind, int64_t stride_row,
                                                               int64_t stride_col, int n, int m, const int* __restrict__ listing,
                                                               WideCtrl* __restrict__ ctrl, const uint64_t* __restrict__ key,
                                                               const int* __restrict__ ends, Out* __restrict__ dist,
                                                               uint64_t* __restrict__ dkey) {
+  __shared__ uint64_t staged[kWideStagedFront];
   const int nv = ctrl->nv, start = ctrl->start;
+  if ((int)(blockIdx.x * (blockDim.x >> 4)) >= nv) return;  // (the whole workgroup)
   const int sub = threadIdx.x & 15;
-  const int groups = (int)(gridDim.x * (blockDim.x >> 4));
-  for (int q = (int)(blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4)); q < nv; q += groups) {
-    const int row = listing[start + q];
-    bool boundary = false;
-    Out acc = (Out)0;
-    for (int k = 0; k < m; ++k) {
-      const uint64_t* __restrict__ col = key + (int64_t)k * n;
-      const uint64_t mine = col[q];
-      uint64_t below = 0ull, above = ~0ull;
-      int below_q = -1, above_q = -1;
-      for (int e0 = sub; e0 < nv; e0 += 4 * 16) {  // four partners per step, their loads in flight together
-        uint64_t c[4];
+  const int q = (int)(blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4));
+  const bool mine_exists = q < nv;
+  const bool stage = nv <= kWideStagedFront;
+  const int row = mine_exists ? listing[start + q] : -1;
+  bool boundary = false;
+  Out acc = (Out)0;
+  for (int k = 0; k < m; ++k) {
+    const uint64_t* __restrict__ col = key + (int64_t)k * n;
+    if (stage) {
+      __syncthreads();  // (the searches of the objective before are over)
+      for (int e = threadIdx.x; e < nv; e += blockDim.x) staged[e] = col[e];
+      __syncthreads();
+    }
+    if (!mine_exists) continue;
+    const uint64_t mine = stage ? staged[q] : col[q];
+    uint64_t below = 0ull, above = ~0ull;
+    int below_q = -1, above_q = -1;
+    for (int e0 = sub; e0 < nv; e0 += 4 * 16) {  // four partners per step, their loads in flight together
+      uint64_t c[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) c[u] = e0 + 16 * u < nv ? col[e0 + 16 * u] : mine;
+      for (int u = 0; u < 4; ++u) c[u] = e0 + 16 * u < nv ? (stage ? staged[e0 + 16 * u] : col[e0 + 16 * u]) : mine;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int e = e0 + 16 * u;  // (e ascends within a lane)
-          const bool before = c[u] < mine || (c[u] == mine && e < q);
-          const bool after = c[u] > mine || (c[u] == mine && e > q);
-          if (e < nv && before && (below_q < 0 || c[u] >= below)) below = c[u], below_q = e;  // the last of the largest
-          if (e < nv && after && (above_q < 0 || c[u] < above)) above = c[u], above_q = e;    // the first of the smallest
-        }
-      }
-#pragma unroll
-      for (int off = 1; off < 16; off <<= 1) {
-        const uint64_t ob = ((uint64_t)__shfl_xor((unsigned)(below >> 32), off) << 32) | (unsigned)__shfl_xor((unsigned)below, off);
-        const uint64_t oa = ((uint64_t)__shfl_xor((unsigned)(above >> 32), off) << 32) | (unsigned)__shfl_xor((unsigned)above, off);
-        const int obq = __shfl_xor(below_q, off), oaq = __shfl_xor(above_q, off);
-        if (obq >= 0 && (below_q < 0 || ob > below || (ob == below && obq > below_q))) below = ob, below_q = obq;
-        if (oaq >= 0 && (above_q < 0 || oa < above || (oa == above && oaq < above_q))) above = oa, above_q = oaq;
-      }
-      if (below_q < 0 || above_q < 0) {
-        boundary = true;  // first or last of this objective (non_dominate.py:226-227)
-      } else if (row >= 0) {
-        const int64_t c0 = (int64_t)k * stride_col;
-        const Out term = wide_term<Out>(costs, kind, (int64_t)listing[start + above_q] * stride_row + c0,
-                                        (int64_t)listing[start + below_q] * stride_row + c0,
-                                        (int64_t)listing[start + ends[2 * k + 1]] * stride_row + c0,
-                                        (int64_t)listing[start + ends[2 * k]] * stride_row + c0);
-        acc = k == 0 ? term : acc + term;
+      for (int u = 0; u < 4; ++u) {
+        const int e = e0 + 16 * u;  // (e ascends within a lane)
+        const bool before = c[u] < mine || (c[u] == mine && e < q);
+        const bool after = c[u] > mine || (c[u] == mine && e > q);
+        if (e < nv && before && (below_q < 0 || c[u] >= below)) below = c[u], below_q = e;  // the last of the largest
+        if (e < nv && after && (above_q < 0 || c[u] < above)) above = c[u], above_q = e;    // the first of the smallest
       }
     }
-    if (sub == 0) {
-      if (row < 0) {  // a poisoned listing
-        ctrl->err = 1;
-        dkey[q] = ~0ull;
-      } else {
-        const Out d = boundary ? (Out)INFINITY : acc;
-        dist[row] = d;
-        dkey[q] = ordered_key64(-(double)d);
-      }
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+      const uint64_t ob = ((uint64_t)__shfl_xor((unsigned)(below >> 32), off) << 32) | (unsigned)__shfl_xor((unsigned)below, off);
+      const uint64_t oa = ((uint64_t)__shfl_xor((unsigned)(above >> 32), off) << 32) | (unsigned)__shfl_xor((unsigned)above, off);
+      const int obq = __shfl_xor(below_q, off), oaq = __shfl_xor(above_q, off);
+      if (obq >= 0 && (below_q < 0 || ob > below || (ob == below && obq > below_q))) below = ob, below_q = obq;
+      if (oaq >= 0 && (above_q < 0 || oa < above || (oa == above && oaq < above_q))) above = oa, above_q = oaq;
+    }
+    if (below_q < 0 || above_q < 0) {
+      boundary = true;  // first or last of this objective (non_dominate.py:226-227)
+    } else if (row >= 0) {
+      const int64_t c0 = (int64_t)k * stride_col;
+      const Out term = wide_term<Out>(costs, kind, (int64_t)listing[start + above_q] * stride_row + c0,
+                                      (int64_t)listing[start + below_q] * stride_row + c0,
+                                      (int64_t)listing[start + ends[2 * k + 1]] * stride_row + c0,
+                                      (int64_t)listing[start + ends[2 * k]] * stride_row + c0);
+      acc = k == 0 ? term : acc + term;
+    }
+  }
+  if (mine_exists && sub == 0) {
+    if (row < 0) {  // a poisoned listing
+      ctrl->err = 1;
+      dkey[q] = ~0ull;
+    } else {
+      const Out d = boundary ? (Out)INFINITY : acc;
+      dist[row] = d;
+      dkey[q] = ordered_key64(-(double)d);
     }
   }
 }
@@ -380,7 +394,7 @@ __global__ __launch_bounds__(256) void wide_front_order_kernel(const int* __rest
 // out[(b * n + index) * m + k] for row = b * m + k gets the number of distinct values before it (-0.0 and 0.0 are one
 // value), as a float -- exact below 2^24 -- and NaN where the value is NaN.
 constexpr int kDenseRankThreads = 1024;
-constexpr int kDenseRankPer = 4;
+constexpr int kDenseRankPer = 16;  // (four: 25 us for 20 000 values a row, the passes over 4096 values each being chains of barriers; sixteen: see below)
 
 template <class T>
 __global__ __launch_bounds__(kDenseRankThreads) void dense_rank_kernel(const T* __restrict__ sorted, const int64_t* __restrict__ index,
