@@ -101,8 +101,8 @@ __global__ __launch_bounds__(kTwoThreads) void two_peel_kernel(const float* __re
                                                                unsigned spin_limit, int stop_count, int64_t ws_step) {
   to_population(ws_step, xs1_sorted, xs2_sorted, kid, orig_of, rank, dist_fill, ctrl, ring);
   __shared__ __attribute__((aligned(16))) uint32_t wave_min_lds[2][16];  // by the parity of the round; entries from kTwoWaves on stay "none"
-  // by the parity of the round: incoming minimum, rows ranked before this workgroup, flags (these three from the
-  // round's receiver), "the workgroup leaves behind this round's barrier" (from the publisher)
+  // by the parity of the round: incoming minimum, rows ranked before this workgroup, flags (these three from the lane
+  // that loads), "the workgroup leaves behind this round's barrier" (from the lane that publishes)
   __shared__ __attribute__((aligned(16))) uint32_t in_lds[2][4];
   __shared__ int ranked_lds[2];    // rows this workgroup ranked in a round, by the parity of the round
   __shared__ int unranked_lds[kTwoWaves];

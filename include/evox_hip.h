@@ -185,7 +185,8 @@ int evox_hip_batched_nd_environmental_selection(const void* x, int64_t x_row_byt
  * workflows).  The stages of the single-population pipeline run once for several populations at a time, each in
  * its own workgroups on its own copy of the workspace, wherever the kernels whose workgroups wait for each other
  * can all be resident with a share of the device each: populations of up to 32 768 rows whose bit matrix fits the
- * LDS of that share.  evox_hip_many_populations_per_launch says how many share a launch (1: the entry points below
+ * LDS of that share; of two objectives and more than 4096 rows, as many as have their chains of workgroups resident
+ * together (two per compute unit, a workgroup to 3840 rows).  evox_hip_many_populations_per_launch says how many share a launch (1: the entry points below
  * then run the populations one after the other, which is always correct); evox_hip_many_workspace_bytes is the
  * workspace for it (that many single-population workspaces).  `stop_count` is the topk of the selection, or the
  * count of evox_hip_non_dominate_rank_until (n: every row is ranked).  Addressing as in evox_hip_batched_*; outputs
