@@ -33,6 +33,10 @@ _SIGNATURES = {
     "evox_hip_wide_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "evox_hip_crowding_distance_wide": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p,
                                                 c_int, c_void_p, c_size_t, c_void_p]),
+    "evox_hip_many_nd_environmental_selection_wide": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64,
+                                                              c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                                              c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                                              c_void_p, c_size_t, c_void_p]),
     "evox_hip_dense_rank_rows": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "evox_hip_nd_environmental_selection_wide": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int,
                                                          c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p,

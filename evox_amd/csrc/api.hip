@@ -1902,32 +1902,80 @@ static bool wide_direct_applies(int64_t n, const int* outcome) {
 // (rank, distance descending, row index), for populations of up to kWideDirectRows rows: one stable argsort step of
 // the ranks lists the rows, the kernels of wide.hpp do the rest without sorting the costs.
 static int wide_select_direct(const WideLayout& L, uint8_t* base, const void* costs, int kind, int64_t sr, int64_t sc,
-                              const int32_t* rank, void* dist, int out_kind, int* order_out, hipStream_t s, int* outcome) {
+                              const int32_t* rank, void* dist, int out_kind, int* order_out, hipStream_t s, int* outcome,
+                              int batch = 1, int64_t ws_step = 0, int64_t cost_step = 0) {
+  // batch > 1: that many populations in the same launches, their workspaces ws_step bytes, their costs cost_step bytes and
+  // their rank vectors n entries apart (dist and order_out lie in the workspaces)
   const int n = L.n, m = L.m;
   WideCtrl* ctrl = reinterpret_cast<WideCtrl*>(base + L.ctrl);
   int* listing = reinterpret_cast<int*>(base + L.order_b);
   uint64_t* key = reinterpret_cast<uint64_t*>(base + L.terms);
   uint64_t* dkey = reinterpret_cast<uint64_t*>(base + L.front_dkey);
   int* ends = reinterpret_cast<int*>(base + L.front_ends);
-  hipLaunchKernelGGL(wide_head_kernel, dim3(1), dim3(1024), 0, s, (const uint8_t*)nullptr, (int64_t)0, rank, n, ctrl);
+  hipLaunchKernelGGL(wide_head_kernel, dim3(1, 1, batch), dim3(1024), 0, s, (const uint8_t*)nullptr, (int64_t)0, rank, n, ctrl, ws_step);
   EVX_LAUNCH_CHECK();
-  if (int e = evox_hip_stable_argsort_step(rank, kKeyInt32, 1, n, nullptr, listing, base + L.sort_ws, L.sort_bytes, s)) return e;
-  // (sixteen lanes per candidate; the grid is sized for a front of all rows, which the kernels find out on the device)
-  const int pair_grid = wide_grid((int64_t)n * 16);
+  if (batch > 1) {
+    if (int e = argsort_step_many(rank, n, batch, (int64_t)n * 4, listing, ws_step, s)) return e;
+  } else if (int e = evox_hip_stable_argsort_step(rank, kKeyInt32, 1, n, nullptr, listing, base + L.sort_ws, L.sort_bytes, s)) {
+    return e;
+  }
+  // (sixteen lanes per candidate; the grids are sized for a front of all rows, which the kernels find out on the device)
+  const int pair_grid = shared_grid(wide_grid((int64_t)n * 16), device_cus() * 8, batch);
+  const int keys_grid = shared_grid(wide_grid((int64_t)n * m), device_cus() * 8, batch);
   const int dist_grid = (n + 15) / 16;  // (a group of lanes per row, n <= kWideDirectRows)
   auto launch = [&](auto* typed_dist) {
     using Out = std::remove_pointer_t<decltype(typed_dist)>;
-    hipLaunchKernelGGL(wide_front_keys_kernel<Out>, dim3(wide_grid((int64_t)n * m)), dim3(256), 0, s, costs, kind, sr, sc, n, m, listing,
-                       ctrl, key, ends, typed_dist);
-    hipLaunchKernelGGL(wide_front_dist_kernel<Out>, dim3(dist_grid), dim3(256), 0, s, costs, kind, sr, sc, n, m, listing, ctrl, key,
-                       ends, typed_dist, dkey);
+    hipLaunchKernelGGL(wide_front_keys_kernel<Out>, dim3(keys_grid < m ? m : keys_grid, 1, batch), dim3(256), 0, s, costs, kind, sr, sc, n,
+                       m, listing, ctrl, key, ends, typed_dist, ws_step, cost_step);
+    hipLaunchKernelGGL(wide_front_dist_kernel<Out>, dim3(dist_grid, 1, batch), dim3(256), 0, s, costs, kind, sr, sc, n, m, listing, ctrl,
+                       key, ends, typed_dist, dkey, ws_step, cost_step);
   };
   if (out_kind == 0)
     launch(static_cast<double*>(dist));
   else
     launch(static_cast<float*>(dist));
   EVX_LAUNCH_CHECK();
-  hipLaunchKernelGGL(wide_front_order_kernel, dim3(pair_grid), dim3(256), 0, s, listing, ctrl, dkey, n, order_out, outcome);
+  hipLaunchKernelGGL(wide_front_order_kernel, dim3(pair_grid, 1, batch), dim3(256), 0, s, listing, ctrl, dkey, n, order_out, outcome, ws_step);
+  EVX_LAUNCH_CHECK();
+  return 0;
+}
+
+// The gathers of a selection by `order` in one launch: x (if any), the fitness rows, the ranks and the distances.
+struct WideGather {
+  const void* x;
+  int64_t x_row_bytes, x_row_stride_bytes, x_step;
+  const void* f_rows;
+  int64_t f_row_bytes, f_row_stride_bytes, f_step;
+  const int32_t* rank;
+  const void* dist;
+  int64_t dist_bytes, dist_step;
+  void *out_x, *out_f, *out_rank, *out_dist;
+};
+static int wide_gather(const WideGather& a, const int* order, int64_t order_step, int64_t n, int64_t topk, int batch, hipStream_t s) {
+  GatherParts parts;
+  parts.parts = 0;
+  parts.first[0] = 0;
+  auto add_part = [&](const void* src, int64_t row_bytes, int64_t row_stride_bytes, int64_t src_step, void* dst) {
+    if (row_bytes <= 0) return;
+    uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | (uintptr_t)row_bytes | (uintptr_t)row_stride_bytes;
+    if (batch > 1) bits |= (uintptr_t)src_step | (uintptr_t)(topk * row_bytes);
+    const int unit = bits % 16 == 0 ? 16 : bits % 8 == 0 ? 8 : bits % 4 == 0 ? 4 : 1;
+    const int p = parts.parts++;
+    parts.src[p] = static_cast<const uint8_t*>(src);
+    parts.dst[p] = static_cast<uint8_t*>(dst);
+    parts.row_bytes[p] = row_bytes;
+    parts.row_stride_bytes[p] = row_stride_bytes;
+    parts.src_step[p] = src_step;
+    parts.dst_step[p] = topk * row_bytes;
+    parts.unit[p] = unit;
+    parts.first[p + 1] = parts.first[p] + topk * (row_bytes / unit);
+  };
+  if (a.x != nullptr) add_part(a.x, a.x_row_bytes, a.x_row_stride_bytes, a.x_step, a.out_x);
+  add_part(a.f_rows, a.f_row_bytes, a.f_row_stride_bytes, a.f_step, a.out_f);
+  add_part(a.rank, 4, 4, n * 4, a.out_rank);
+  add_part(a.dist, a.dist_bytes, a.dist_bytes, a.dist_step, a.out_dist);
+  const int grid = shared_grid(wide_grid(parts.first[parts.parts]), device_cus() * 8, batch);
+  hipLaunchKernelGGL(gather_parts_kernel, dim3(grid, 1, batch), dim3(256), 0, s, parts, order, topk, order_step);
   EVX_LAUNCH_CHECK();
   return 0;
 }
@@ -2367,30 +2415,53 @@ int evox_hip_nd_environmental_selection_wide(const void* x, int64_t x_row_bytes,
     if (int e = evox_hip_stable_argsort_step(base + L.neg_hi, kKeyUint32, 1, n, order_a, order_b, sort_ws, L.sort_bytes, s)) return e;
     if (int e = evox_hip_stable_argsort_step(rank, kKeyInt32, 1, n, order_b, order_a, sort_ws, L.sort_bytes, s)) return e;
   }
-  // the four gathers in one launch
-  GatherParts parts;
-  parts.parts = 0;
-  parts.first[0] = 0;
-  auto add_part = [&](const void* src, int64_t row_bytes, int64_t row_stride_bytes, void* dst) {
-    if (row_bytes <= 0) return;
-    const uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | (uintptr_t)row_bytes | (uintptr_t)row_stride_bytes;
-    const int unit = bits % 16 == 0 ? 16 : bits % 8 == 0 ? 8 : bits % 4 == 0 ? 4 : 1;
-    const int p = parts.parts++;
-    parts.src[p] = static_cast<const uint8_t*>(src);
-    parts.dst[p] = static_cast<uint8_t*>(dst);
-    parts.row_bytes[p] = row_bytes;
-    parts.row_stride_bytes[p] = row_stride_bytes;
-    parts.unit[p] = unit;
-    parts.first[p + 1] = parts.first[p] + topk * (row_bytes / unit);
-  };
-  if (x != nullptr) add_part(x, x_row_bytes, x_row_stride_bytes, out_x);
-  add_part(f_rows, f_row_bytes, f_row_stride_bytes, out_f);
-  add_part(rank, 4, 4, out_rank);
   const int64_t dist_bytes = out_kind == 0 ? 8 : 4;
-  add_part(dist, dist_bytes, dist_bytes, out_dist);
-  hipLaunchKernelGGL(gather_parts_kernel, dim3(wide_grid(parts.first[parts.parts])), dim3(256), 0, s, parts, order_a, topk);
-  EVX_LAUNCH_CHECK();
-  return 0;
+  const WideGather gather = {x, x_row_bytes, x_row_stride_bytes, 0, f_rows, f_row_bytes, f_row_stride_bytes, 0, rank, dist, dist_bytes, 0,
+                             out_x, out_f, out_rank, out_dist};
+  return wide_gather(gather, order_a, 0, n, topk, 1, s);
+}
+
+int evox_hip_many_nd_environmental_selection_wide(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes, int64_t x_batch_stride_bytes,
+                                                  const void* f_rows, int64_t f_row_bytes, int64_t f_row_stride_bytes,
+                                                  int64_t f_batch_stride_bytes, const void* costs, int kind, int64_t batch, int64_t n,
+                                                  int64_t m, int64_t stride_batch, int64_t sr, int64_t sc, const int32_t* rank,
+                                                  int64_t topk, void* out_x, void* out_f, int32_t* out_rank, void* out_dist,
+                                                  int out_kind, void* ws, size_t ws_bytes, void* stream) {
+  WideLayout L;
+  if (batch < 1 || !make_wide_layout(n, m, &L) || topk < 1 || topk > n) return kErrBadArg;
+  if ((kind != kWideFloat64 && kind != kWideInt64) || (out_kind != 0 && out_kind != 1)) return kErrBadArg;
+  const int64_t step = (int64_t)align_up(L.total);
+  const int64_t dist_bytes = out_kind == 0 ? 8 : 4;
+  hipStream_t s = (hipStream_t)stream;
+  int* const outcome = opt().launch_memory ? outcome_slot(n, m, true, s, 1) : nullptr;
+  const int64_t x_out_step = topk * x_row_bytes, f_out_step = topk * f_row_bytes;
+  const bool together = batch > 1 && wide_direct_applies(n, outcome) && (n <= kSmallArgsortRows || opt().mid_argsort) &&
+                        ws_bytes >= (size_t)step * (size_t)batch && batch <= 65535;
+  if (!together) {  // one population after the other, each through the single-population entry point
+    for (int64_t b = 0; b < batch; ++b) {
+      const int e = evox_hip_nd_environmental_selection_wide(
+          x ? static_cast<const char*>(x) + b * x_batch_stride_bytes : nullptr, x_row_bytes, x_row_stride_bytes,
+          static_cast<const char*>(f_rows) + b * f_batch_stride_bytes, f_row_bytes, f_row_stride_bytes,
+          static_cast<const char*>(costs) + b * stride_batch * 8, kind, n, m, sr, sc, rank + b * n, topk,
+          out_x ? static_cast<char*>(out_x) + b * x_out_step : nullptr, static_cast<char*>(out_f) + b * f_out_step, out_rank + b * topk,
+          static_cast<char*>(out_dist) + b * topk * dist_bytes, out_kind, ws, ws_bytes, stream);
+      if (e) return e;
+    }
+    return 0;
+  }
+  if (costs == nullptr || rank == nullptr || f_rows == nullptr || out_f == nullptr || out_rank == nullptr || out_dist == nullptr)
+    return kErrBadArg;
+  if ((x == nullptr) != (out_x == nullptr) || x_row_bytes < 0 || x_row_stride_bytes < 0 || f_row_bytes < 1 || f_row_stride_bytes < 0)
+    return kErrBadArg;
+  if (ws == nullptr || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return kErrWorkspace;
+  uint8_t* base = static_cast<uint8_t*>(ws);
+  void* dist = base + L.dist;
+  int* order = reinterpret_cast<int*>(base + L.order_a);
+  if (int e = wide_select_direct(L, base, costs, kind, sr, sc, rank, dist, out_kind, order, s, outcome, (int)batch, step, stride_batch * 8))
+    return e;
+  const WideGather gather = {x, x_row_bytes, x_row_stride_bytes, x_batch_stride_bytes, f_rows, f_row_bytes, f_row_stride_bytes,
+                             f_batch_stride_bytes, rank, dist, dist_bytes, step, out_x, out_f, out_rank, out_dist};
+  return wide_gather(gather, order, step, n, topk, (int)batch, s);
 }
 
 }  // extern "C"

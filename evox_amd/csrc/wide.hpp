@@ -47,9 +47,13 @@ __device__ inline uint64_t ordered_key64(long long v) { return (uint64_t)v ^ 0x8
 
 // One workgroup: the number of selected rows, and with a rank vector the rank that selects them.
 // mask: a byte per row (stride in bytes), or null; rank: int32 per row, or null (then the mask, or every row).
+// blockIdx.z: one of several populations (rank vectors n entries apart, control blocks ws_step bytes apart).
 __global__ __launch_bounds__(1024) void wide_head_kernel(const uint8_t* __restrict__ mask, int64_t mask_stride,
-                                                         const int* __restrict__ rank, int n, WideCtrl* __restrict__ ctrl) {
+                                                         const int* __restrict__ rank, int n, WideCtrl* __restrict__ ctrl,
+                                                         int64_t ws_step = 0) {
   __shared__ int red[16];
+  if (rank != nullptr) rank += (int64_t)blockIdx.z * n;
+  ctrl = reinterpret_cast<WideCtrl*>(reinterpret_cast<char*>(ctrl) + (int64_t)blockIdx.z * ws_step);
   __shared__ int worst_lds;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int worst = -1;
@@ -226,8 +230,12 @@ template <class Out>
 __global__ __launch_bounds__(256) void wide_front_keys_kernel(const void* __restrict__ costs, int kind, int64_t stride_row,
                                                               int64_t stride_col, int n, int m, const int* __restrict__ listing,
                                                               const WideCtrl* __restrict__ ctrl, uint64_t* __restrict__ key,
-                                                              int* __restrict__ ends, Out* __restrict__ dist) {
+                                                              int* __restrict__ ends, Out* __restrict__ dist, int64_t ws_step = 0,
+                                                              int64_t cost_step = 0) {
   __shared__ uint64_t lo_key[4], hi_key[4];
+  // (blockIdx.z: one of several populations, their buffers ws_step bytes and their costs cost_step bytes apart)
+  to_population(ws_step, listing, ctrl, key, ends, dist);
+  costs = static_cast<const char*>(costs) + (int64_t)blockIdx.z * cost_step;
   __shared__ int lo_at[4], hi_at[4];
   const int nv = ctrl->nv, start = ctrl->start;
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) dist[i] = (Out)(-INFINITY);
@@ -286,8 +294,11 @@ __global__ __launch_bounds__(256) void wide_front_dist_kernel(const void* __rest
                                                               int64_t stride_col, int n, int m, const int* __restrict__ listing,
                                                               WideCtrl* __restrict__ ctrl, const uint64_t* __restrict__ key,
                                                               const int* __restrict__ ends, Out* __restrict__ dist,
-                                                              uint64_t* __restrict__ dkey) {
+                                                              uint64_t* __restrict__ dkey, int64_t ws_step = 0,
+                                                              int64_t cost_step = 0) {
   __shared__ uint64_t staged[kWideStagedFront];
+  to_population(ws_step, listing, ctrl, key, ends, dist, dkey);
+  costs = static_cast<const char*>(costs) + (int64_t)blockIdx.z * cost_step;
   const int nv = ctrl->nv, start = ctrl->start;
   if ((int)(blockIdx.x * (blockDim.x >> 4)) >= nv) return;  // (the whole workgroup)
   const int sub = threadIdx.x & 15;
@@ -356,10 +367,11 @@ __global__ __launch_bounds__(256) void wide_front_dist_kernel(const void* __rest
 // row index), what the ranking left without a rank behind them as listed.  Every entry -1 when something was poisoned.
 __global__ __launch_bounds__(256) void wide_front_order_kernel(const int* __restrict__ listing, const WideCtrl* __restrict__ ctrl,
                                                                const uint64_t* __restrict__ dkey, int n, int* __restrict__ order,
-                                                               int* __restrict__ outcome) {
+                                                               int* __restrict__ outcome, int64_t ws_step = 0) {
+  to_population(ws_step, listing, ctrl, dkey, order);
   const int nv = ctrl->nv, start = ctrl->start;
   const bool failed = ctrl->err != 0;
-  if (outcome != nullptr && blockIdx.x == 0 && threadIdx.x == 0)
+  if (outcome != nullptr && blockIdx.x == 0 && blockIdx.z == 0 && threadIdx.x == 0)
     __hip_atomic_store(outcome, nv > kWideDirectFront ? 2 : 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
     if (failed)
@@ -452,11 +464,18 @@ struct GatherParts {
   uint8_t* dst[4];
   int64_t row_bytes[4], row_stride_bytes[4];
   int64_t first[5];  // the work items (count x units per row) of part p are first[p] .. first[p + 1]
+  int64_t src_step[4], dst_step[4];  // several populations in the launch (blockIdx.z): bytes from one to the next
   int unit[4];
   int parts;
 };
 
-__global__ __launch_bounds__(256) void gather_parts_kernel(GatherParts g, const int* __restrict__ order, int64_t count) {
+__global__ __launch_bounds__(256) void gather_parts_kernel(GatherParts g, const int* __restrict__ order, int64_t count,
+                                                           int64_t order_step = 0) {
+  order = reinterpret_cast<const int*>(reinterpret_cast<const char*>(order) + (int64_t)blockIdx.z * order_step);
+  for (int p = 0; p < g.parts; ++p) {
+    g.src[p] += (int64_t)blockIdx.z * g.src_step[p];
+    g.dst[p] += (int64_t)blockIdx.z * g.dst_step[p];
+  }
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < g.first[g.parts]; idx += (int64_t)gridDim.x * blockDim.x) {
     int p = 0;
     while (p + 1 < g.parts && idx >= g.first[p + 1]) ++p;

@@ -395,13 +395,29 @@ def nd_select_wide(x: torch.Tensor, f: torch.Tensor, topk: int) -> Tuple[torch.T
         fo_x = out_x.view(flat_w.size(0), topk, -1)
         fo_f, fo_r, fo_d = out_f.view(-1, topk, m), out_rank.view(-1, topk), out_dist.view(-1, topk)
         stream = runtime.stream_handle(f.device)
-        ws = runtime.wide_workspace(n, m, f.device)
-        for b in range(flat_w.size(0)):
-            wb = flat_w[b]
-            _lib.call("evox_hip_nd_environmental_selection_wide", flat_x[b].data_ptr() if has_x else None, row_bytes, row_bytes,
-                      flat_f[b].data_ptr(), f_row_bytes, f_row_bytes, wb.data_ptr(), kind, n, m, wb.stride(0), wb.stride(1),
-                      flat_rank[b].data_ptr(), topk, fo_x[b].data_ptr() if has_x else None, fo_f[b].data_ptr(), fo_r[b].data_ptr(),
-                      fo_d[b].data_ptr(), 0 if out_dtype == torch.float64 else 1, ws.data_ptr(), ws.numel(), stream)
+        count = flat_w.size(0)
+        if count == 1:
+            ws = runtime.wide_workspace(n, m, f.device)
+            wb = flat_w[0]
+            _lib.call("evox_hip_nd_environmental_selection_wide", flat_x.data_ptr() if has_x else None, row_bytes, row_bytes,
+                      flat_f.data_ptr(), f_row_bytes, f_row_bytes, wb.data_ptr(), kind, n, m, wb.stride(0), wb.stride(1),
+                      flat_rank.data_ptr(), topk, fo_x.data_ptr() if has_x else None, fo_f.data_ptr(), fo_r.data_ptr(),
+                      fo_d.data_ptr(), 0 if out_dtype == torch.float64 else 1, ws.data_ptr(), ws.numel(), stream)
+        else:
+            # all populations in the same launches where the library can (it takes them one after the other otherwise);
+            # at most 1 GiB of workspace copies at a time
+            one = (int(_lib.lib().evox_hip_wide_workspace_bytes(n, m)) + 255) // 256 * 256
+            per_call = max(1, min(count, (1 << 30) // max(one, 1)))
+            flat_rank = flat_rank.contiguous()
+            for b0 in range(0, count, per_call):
+                nb = min(per_call, count - b0)
+                ws = runtime.wide_workspace(n, m, f.device, nb)
+                wb = flat_w[b0:b0 + nb]
+                _lib.call("evox_hip_many_nd_environmental_selection_wide", flat_x[b0].data_ptr() if has_x else None, row_bytes, row_bytes,
+                          n * row_bytes, flat_f[b0].data_ptr(), f_row_bytes, f_row_bytes, n * f_row_bytes, wb.data_ptr(), kind, nb, n, m,
+                          wb.stride(0), wb.stride(1), wb.stride(2), flat_rank[b0].data_ptr(), topk,
+                          fo_x[b0].data_ptr() if has_x else None, fo_f[b0].data_ptr(), fo_r[b0].data_ptr(), fo_d[b0].data_ptr(),
+                          0 if out_dtype == torch.float64 else 1, ws.data_ptr(), ws.numel(), stream)
         runtime.note_small_kernel_call()
     return out_x, out_f, out_rank, out_dist
 

@@ -116,11 +116,14 @@ def sort_workspace(n: int, device: torch.device) -> torch.Tensor:
     return ws
 
 
-def wide_workspace(n: int, m: int, device: torch.device) -> torch.Tensor:
-    """Workspace of the entry points for 8-byte fitness; shares the per-(device, stream) buffer of `workspace`."""
+def wide_workspace(n: int, m: int, device: torch.device, copies: int = 1) -> torch.Tensor:
+    """Workspace of the entry points for 8-byte fitness (`copies` of it, each rounded up to 256 bytes, for as many
+    populations in the same launches); shares the per-(device, stream) buffer of `workspace`."""
     need = int(_lib.lib().evox_hip_wide_workspace_bytes(n, m))
     if need == 0:
         raise ValueError(f"unsupported population shape n={n}, m={m}")
+    if copies > 1:
+        need = ((need + 255) // 256 * 256) * copies
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream_handle(device))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < need:

@@ -119,6 +119,20 @@ int evox_hip_nd_environmental_selection_wide(const void* x, int64_t x_row_bytes,
                                              int64_t topk, void* out_x, void* out_f, int32_t* out_rank, void* out_dist,
                                              int out_kind, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same for `batch` populations of one shape in the same launches (what a vmapped caller of the reference's
+ * nd_environmental_selection gets, utils/op_register.py:26-51): x, f_rows and costs of population b lie
+ * x_batch_stride_bytes, f_batch_stride_bytes and stride_batch elements further; rank is (batch, n), the outputs are
+ * contiguous (batch, topk, ...) arrays.  workspace: batch copies of evox_hip_wide_workspace_bytes(n, m), each rounded
+ * up to a multiple of 256 bytes; with a smaller one (at least one copy), more than 24 576 rows, or after a selection
+ * of the shape whose last front held more than 8192 rows, the populations are taken one after the other. */
+int evox_hip_many_nd_environmental_selection_wide(const void* x, int64_t x_row_bytes, int64_t x_row_stride_bytes,
+                                                  int64_t x_batch_stride_bytes, const void* f_rows, int64_t f_row_bytes,
+                                                  int64_t f_row_stride_bytes, int64_t f_batch_stride_bytes, const void* costs,
+                                                  int kind, int64_t batch, int64_t n, int64_t m, int64_t stride_batch,
+                                                  int64_t stride_row, int64_t stride_col, const int32_t* rank, int64_t topk,
+                                                  void* out_x, void* out_f, int32_t* out_rank, void* out_dist, int out_kind,
+                                                  void* workspace, size_t workspace_bytes, void* stream);
+
 /* NSGA-II survivor selection: ranks f, takes the topk best rows by (rank ascending, crowding
  * distance within the last admitted front descending, row index ascending) and gathers them.
  *   x            decision vectors as raw bytes, row i at x + i * x_row_stride_bytes, x_row_bytes each

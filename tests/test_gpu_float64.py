@@ -225,3 +225,29 @@ def test_dense_rank_image(dtype):
                 values = np.unique(col[ok] + 0.0 if dtype == torch.float64 else col[ok])  # (-0.0 + 0.0 == 0.0)
                 want[ok] = np.searchsorted(values, col[ok]).astype(np.float32)
                 assert np.array_equal(got.reshape(cols.shape)[b][:, k], want, equal_nan=True), (shape, b, k)
+
+
+def test_batches_of_8_byte_fitness_share_their_launches(float64_default):
+    """Several populations of float64 or int64 fitness in one call: the same as one population at a time."""
+    g = torch.Generator("cpu").manual_seed(70)
+    f64 = (torch.rand(5, 3000, 3, generator=g, dtype=torch.float64) * 300).round() / 300
+    f64[1, 7, 2] = float("nan")
+    f64[2, :, 1] = 1.0 - f64[2, :, 0]
+    f64[3] = f64[3, :1]  # every row the same
+    i64 = torch.randint(-(2**40), 2**40, (3, 9000, 2), generator=g, dtype=torch.int64)
+    for f, k in ((f64, 1200), (f64, 3000), (i64, 4000)):
+        batch, n = f.shape[:2]
+        x = torch.rand(batch, n, 3, generator=g, dtype=torch.float64)
+        fd, xd = f.to(DEV), x.to(DEV)
+        got = nd_environmental_selection(xd, fd, k)
+        for b in range(batch):
+            alone = nd_environmental_selection(xd[b], fd[b], k)
+            for part, (a, c) in enumerate(zip(got, alone)):
+                assert a[b].dtype == c.dtype and np.array_equal(as_np(a[b]), as_np(c), equal_nan=True), (f.dtype, k, b, part)
+    # no decision columns, populations along another dimension
+    none = nd_environmental_selection(torch.empty(5, 3000, 0, device=DEV), f64.to(DEV), 1200)
+    want = nd_environmental_selection(torch.zeros(5, 3000, 1, device=DEV), f64.to(DEV), 1200)
+    assert none[0].shape == (5, 1200, 0) and torch.equal(none[2], want[2]) and np.array_equal(as_np(none[3]), as_np(want[3]), equal_nan=True)
+    mapped = torch.vmap(lambda a, c: nd_environmental_selection(a, c, 1200), in_dims=(1, 1))(
+        torch.zeros(3000, 5, 1, device=DEV), f64.permute(1, 0, 2).contiguous().to(DEV))
+    assert torch.equal(mapped[2], want[2]) and np.array_equal(as_np(mapped[1]), as_np(want[1]), equal_nan=True)
