@@ -203,6 +203,20 @@ def stage_profile(w, x, f, reps):
         times["dominance_orders_us"] = event_time_us(orders, reps)
     except _lib.EvoxHipError:
         times["dominance_orders_us"] = None
+    if times["dominance_orders_us"] is not None:
+        # The selection entry point may have that stage count the dominators first and build the matrix only when front 0
+        # holds fewer rows than are kept (tunable prefix_count_first; the stage entry points always do both at once):
+        # the stage with the counts alone, and the whole step with the choice switched off
+        with runtime.options(prefix_mode=1):
+            dom()
+            times["dominance_counts_only_us"] = event_time_us(dom, reps)
+        with runtime.options(prefix_count_first=0):
+            whole()
+            times["step_matrix_always_us"] = event_time_us(whole, reps)
+        # (the prefixes above are made of the stage entry points: the rest of the step is what follows them in a step
+        # that launches the same kernels)
+        times["order_and_gather_us"] = times["step_matrix_always_us"] - t_peel
+        prep(); dom()
     upto_peel()
     runtime.note_call(ws, s)
     status = runtime.last_status()
@@ -587,6 +601,8 @@ def main():
     executed_valu = valu_per_pair * evaluated_pairs
     executed_peak = VALU_FP32_PEAK_GOPS if finite else VALU_CMP_PEAK_GOPS
     count_bytes = int(row_read.sum()) + n * 12
+    if from_orders:  # the totals that the dominance kernel left, four words per row in, four out; no row is read
+        count_bytes = n * 32
     dom_us = times["dominance_alone_us"]  # the kernel by itself, back to back; "us" is its share of the step
     phases = {
         "prepare_and_slot_sort": {"us": times["prepare_us"]},
@@ -619,6 +635,27 @@ def main():
                                "prefix_kernel_us": kernel_us, "bound": "hbm", "achieved": dom_bytes / kernel_us / 1e3,
                                "peak": HBM_PEAK_GBS, "unit": "GB/s", "executed_form": "objective orders",
                                "reference_compares_rate_Gcompare_s": compares / dom_us / 1e3}
+        # The selection itself counts first where its last two calls found the rows they keep in front 0 (and the peel
+        # is not the one that holds the matrix in LDS): the matrix is then never written, and the kernel's launch is
+        # bound by its table look-ups in LDS -- the bytes it has to move are the orders it reads and the two words per
+        # row it leaves
+        front0 = int((rank == 0).sum())
+        counted_first = (not from_lds and front0 >= w.topk and bool(_rt.current_option("prefix_count_first", 1))
+                         and bool(_rt.current_option("launch_memory", 1)) and "dominance_counts_only_us" in times)
+        phases["dominance"]["front0_rows"] = front0
+        phases["dominance"]["counted_first_in_the_step"] = counted_first
+        if "dominance_counts_only_us" in times:
+            counts_kernel_us = times["dominance_counts_only_us"] - (times.get("dominance_orders_us") or 0.0)
+            counts_bytes = n * m * 8 + n * 4 + n * 8
+            phases["dominance"]["counts_only"] = {
+                "stage_us": times["dominance_counts_only_us"], "prefix_kernel_us": counts_kernel_us, "bytes": counts_bytes,
+                "achieved": counts_bytes / counts_kernel_us / 1e3, "unit": "GB/s",
+                "note": "no matrix written: bound by the look-ups in the tables that the workgroups keep in LDS"}
+            phases["dominance"]["step_us_with_the_matrix_always"] = times["step_matrix_always_us"]
+        if counted_first:
+            phases["dominance"]["note"] = ("`us`, kernel_alone_us, prefix_kernel_us, achieved and frac are those of the launch "
+                                           "that builds the matrix (stage entry point); the timed step ran the kernel for "
+                                           "the counts alone (counts_only) and skipped the matrix")
     for p in phases.values():
         if "achieved" in p:
             p["frac"] = p["achieved"] / p["peak"]
@@ -644,8 +681,19 @@ def main():
         "achieved": d["achieved"], "peak": d["peak"], "unit": d["unit"], "frac": d["frac"], "traffic": None,
         "kernel_us": d.get("prefix_kernel_us", d.get("kernel_alone_us", d["us"])),
     }
+    if dominant == "dominance" and d.get("counted_first_in_the_step"):
+        c = d["counts_only"]
+        roofline.update({"achieved": c["achieved"], "frac": c["achieved"] / HBM_PEAK_GBS, "kernel_us": c["prefix_kernel_us"],
+                         "traffic": None,
+                         "note": ("the step ran this kernel for the row totals alone (front 0 held every row kept, so the "
+                                  "matrix was not built): " + c["note"] + "; matrix_launch is the same kernel when it "
+                                  "also writes the matrix"),
+                         "matrix_launch": {"achieved": d["achieved"], "frac": d["frac"], "kernel_us": d["prefix_kernel_us"]}})
     measured = profile_traffic(args.workload, roofline["kernel"])
-    if measured is not None:
+    if measured is not None and "matrix_launch" in roofline:  # (the committed counters are those of the launch with the matrix)
+        roofline["matrix_launch"]["traffic"] = measured["bytes"]
+        roofline["matrix_launch"]["traffic_source"] = measured["source"]
+    elif measured is not None:
         roofline["traffic"] = measured["bytes"]
         roofline["traffic_source"] = measured["source"]
     if _rt.small_population_kernel_fits(n, m, 1):

@@ -63,6 +63,8 @@ struct Options {
                                         // takes both tiles of a 128-byte line; 0 = never
   int prefix_mode = 3;  // measurements: 1 = popcounts only, 2 = matrix only
   int prefix_bands = 1;  // stretches of the order-based matrix: 1 = bands of rows counted from row 0, 0 = from each tile's diagonal
+  int prefix_count_first = 1;  // a selection whose last two of this shape found all they keep in front 0 has the order-based
+                               // kernel count dominators first and build the matrix only if front 0 falls short; 0 = never
 };
 static Options g_opt;
 // The tunables that calls made from this thread use: those handed to evox_hip_options_use, else the process-wide ones.
@@ -160,6 +162,9 @@ struct Ws {
   // of the next, all laid out alike; 1 and 0 for a single population
   int batch = 1;
   int64_t step = 0;
+  // above zero: the order-based dominance kernel has only counted so far; the count stage launches it again for the
+  // matrix, and that launch does nothing when front 0 holds this many rows
+  mutable int64_t matrix_unless = 0;
   template <class T>
   T* at(size_t off) const {
     return reinterpret_cast<T*>(base + off);
@@ -196,7 +201,8 @@ static int device_cus() {
 // a stale or missing word costs a few microseconds, never a result.  Allocated at the first selection on a device
 // that may allocate (not during a stream capture); null until then and for callers that may not.
 // salt: 0 for the selections of 4-byte fitness, 1 for those whose last front is ordered by the kernels of wide.hpp
-// (there the word says whether that front was small, 1, or large, 2).
+// (there the word says whether that front was small, 1, or large, 2), 2 for whether front 0 alone held what was kept
+// (GatherArgs::front0_note).
 static int* outcome_slot(int64_t n, int64_t m, bool may_allocate, hipStream_t s, int salt = 0) {
   static std::atomic<int*> words[64];
   static std::atomic<bool> failed[64];
@@ -434,7 +440,8 @@ static bool prefix_dominance_applies(const Layout& L) {
   if (opt().prefix_min_rows <= 0 || L.m < 2 || L.m > kPrefixMaxObjectives) return false;
   return L.n >= prefix_least_rows(L.m) && L.n > kRadixMinCandidates && L.n <= kPrefixMaxRows;
 }
-static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s);
+static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s, int64_t count_first = 0);
+static int dispatch_dominance_prefix(const Ws& w, hipStream_t s, int phase = 0);
 
 static int dominance_tile_words(const Layout& L) {
   const int tile = opt().dominance_tile_words;
@@ -442,12 +449,13 @@ static int dominance_tile_words(const Layout& L) {
   return L.m >= 2 && L.m <= 8 && L.n <= (L.m >= 6 ? 32768 : 24576) ? 2 : 4;
 }
 
-static int stage_dominance(const Ws& w, int variant, hipStream_t s) {
+// count_first: above zero, the caller keeps that many rows and expects front 0 to hold them (see Ws::matrix_unless).
+static int stage_dominance(const Ws& w, int variant, hipStream_t s, int64_t count_first = 0) {
   // (kDomOrdersOnly: the first half of the path below alone, for measurements of the second)
   if (variant == kDomOrdersOnly) return prefix_dominance_applies(w.L) ? stage_dominance_prefix(w, true, s) : kErrBadArg;
   // (the orders of that path come from kernels whose workgroups wait for each other: not with the stepped path)
   // (nor for several populations in one launch: those orders come from a grid that fills the device)
-  if (variant == kDomAuto && prefix_dominance_applies(w.L) && !opt().peel_stepped && w.batch == 1) return stage_dominance_prefix(w, false, s);
+  if (variant == kDomAuto && prefix_dominance_applies(w.L) && !opt().peel_stepped && w.batch == 1) return stage_dominance_prefix(w, false, s, count_first);
   // (the lower triangle in tiles of 4 words keeps every SIMD busy with several waves; up to about 24 000 rows of
   // two to eight objectives tiles of 2 words leave a shorter half-empty tail -- measured, us, tiles of 2 / 4:
   // 5000 x 3: 5.8 / 7.9, 16 000 x 3: 20.3 / 25.7, 20 000 x 2: 20.6 / 23.1, x 3: 27.6 / 31.3, x 8: 64.3 / 80.8,
@@ -484,6 +492,10 @@ static int stage_count(const Ws& w, bool fill_dist, hipStream_t s, bool need_cou
                        w.at<int>(L.witness), w.at<uint64_t>(L.fronts_slot), w.at<uint64_t>(L.fronts_orig), w.at<int>(L.fsize),
                        fill_dist ? w.at<float>(L.dist) : (float*)nullptr, w.ctrl(), w.at<SortParam>(L.sortparam));
     EVX_LAUNCH_CHECK();
+    if (w.matrix_unless > 0) {  // the size of front 0 is known now: the matrix, if anybody is going to read it
+      if (int e = dispatch_dominance_prefix(w, s, 2)) return e;
+      w.matrix_unless = 0;
+    }
   }
   return 0;
 }
@@ -889,8 +901,10 @@ static int shared_grid(int grid, int resident, int batch) {
   return grid < cap ? grid : cap;
 }
 
+// phase 0: totals and matrix in one launch (or what the tunable prefix_mode asks for); 1: the totals alone, and the
+// pairwise kernel for a population that is not finite; 2: the matrix alone, unless front 0 holds w.matrix_unless rows.
 template <int M>
-static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
+static int launch_dominance_prefix(const Ws& w, hipStream_t s, int phase) {
   constexpr int WW = M <= kPrefixWideObjectives ? 8 : 4;  // words per tile: what the LDS holds tables for
   // up to four objectives the tables of two tiles fit: a workgroup then builds whole 128-byte lines of the matrix
   constexpr int TT = M <= 4 ? 2 : 1;
@@ -910,7 +924,8 @@ static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
     const int tiles = (int)round_up((L.nwords + WW * tt - 1) / (WW * tt), 128 / (WW * tt));
     hipLaunchKernelGGL(kernel, dim3(tiles, stretches), dim3(kPrefixThreads), lds, s, w.at<int>(L.pos), w.at<int>(L.scost),
                        w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.kstride, L.wstride, L.nwords, shift, buckets,
-                       chunk, bands, opt().prefix_mode, w.at<int>(L.total0), w.at<int>(L.witness0), w.at<SortParam>(L.sortparam));
+                       chunk, bands, phase == 0 ? opt().prefix_mode : phase, w.at<int>(L.total0), w.at<int>(L.witness0),
+                       w.at<SortParam>(L.sortparam), phase == 2 ? w.at<int>(L.fsize) : (const int*)nullptr, (int)w.matrix_unless);
     EVX_LAUNCH_CHECK();
     return 0;
   };
@@ -920,6 +935,7 @@ static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
   } else {
     if (int e = launch(dominance_prefix_kernel<M, WW, 1>, 1)) return e;
   }
+  if (phase == 2) return 0;
   // a population with a NaN or an infinity: the pairwise kernel, on a grid that costs nothing when it has nothing to do
   hipLaunchKernelGGL(dominance_nonfinite_kernel<M>, dim3(device_cus() * 8), dim3(256), 0, s, w.at<float>(L.xs_sorted),
                      w.at<uint64_t>(L.key_sorted), w.at<uint32_t>(L.kid_sorted), w.at<uint64_t>(L.dom), L.n, L.npad, L.wstride,
@@ -931,11 +947,15 @@ static int launch_dominance_prefix(const Ws& w, hipStream_t s) {
 // The matrix of a large finite population from the order of its rows in every objective (prefix.hpp).  The
 // buffers of the crowding stage (radix pairs, pos, scost) are free until then and carry the orders.
 template <int M>
-static int launch_dominance_prefix(const Ws& w, hipStream_t s);
-static int dispatch_dominance_prefix(const Ws& w, hipStream_t s);
+static int launch_dominance_prefix(const Ws& w, hipStream_t s, int phase);
 
-static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) {
+static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s, int64_t count_first) {
   const Layout& L = w.L;
+  // (the count stage launches the second phase: the peel that keeps the matrix in LDS has no count stage)
+  size_t unused = 0;
+  const int phase = count_first > 0 && !orders_only && opt().prefix_count_first && opt().prefix_mode == 3 &&
+                            lds_peel_plan(L, &unused, 1) == 0 ? 1 : 0;
+  if (phase == 1) w.matrix_unless = count_first;
   if (L.n <= kMidArgsortRows && opt().mid_argsort) {
     // the orders from workgroups that sort in LDS: two launches, no grid barrier (and no barrier words to reset)
     const size_t sort_lds = mid_sort_lds_bytes(L.n);
@@ -957,7 +977,7 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) 
     hipLaunchKernelGGL(objective_positions_kernel, dim3((unsigned)blocks), dim3(256), 0, s, L.n, L.m, w.at<int>(L.slot_of),
                        w.at<SortParam>(L.sortparam), w.ctrl(), w.at<int>(L.pos), w.at<int>(L.scost), radix_buffers(w));
     EVX_LAUNCH_CHECK();
-    return orders_only ? 0 : dispatch_dominance_prefix(w, s);
+    return orders_only ? 0 : dispatch_dominance_prefix(w, s, phase);
   }
   const size_t lds = kRadixLdsBytes;
   if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(objective_order_kernel), lds)) return e;
@@ -976,26 +996,26 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s) 
   const int64_t words = (int64_t)((sizeof(Ctrl) + sizeof(unsigned long long) * kMaxGrid - first) / 4);
   hipLaunchKernelGGL(reset_state_kernel, dim3(16), dim3(256), 0, s, reinterpret_cast<uint32_t*>(w.base + L.ctrl + first), words);
   EVX_LAUNCH_CHECK();
-  return orders_only ? 0 : dispatch_dominance_prefix(w, s);
+  return orders_only ? 0 : dispatch_dominance_prefix(w, s, phase);
 }
 
-static int dispatch_dominance_prefix(const Ws& w, hipStream_t s) {
+static int dispatch_dominance_prefix(const Ws& w, hipStream_t s, int phase) {
   switch (w.L.m) {
-    case 2: return launch_dominance_prefix<2>(w, s);
-    case 3: return launch_dominance_prefix<3>(w, s);
-    case 4: return launch_dominance_prefix<4>(w, s);
-    case 5: return launch_dominance_prefix<5>(w, s);
-    case 6: return launch_dominance_prefix<6>(w, s);
-    case 7: return launch_dominance_prefix<7>(w, s);
-    case 8: return launch_dominance_prefix<8>(w, s);
-    case 9: return launch_dominance_prefix<9>(w, s);
-    case 10: return launch_dominance_prefix<10>(w, s);
-    case 11: return launch_dominance_prefix<11>(w, s);
-    case 12: return launch_dominance_prefix<12>(w, s);
-    case 13: return launch_dominance_prefix<13>(w, s);
-    case 14: return launch_dominance_prefix<14>(w, s);
-    case 15: return launch_dominance_prefix<15>(w, s);
-    case 16: return launch_dominance_prefix<16>(w, s);
+    case 2: return launch_dominance_prefix<2>(w, s, phase);
+    case 3: return launch_dominance_prefix<3>(w, s, phase);
+    case 4: return launch_dominance_prefix<4>(w, s, phase);
+    case 5: return launch_dominance_prefix<5>(w, s, phase);
+    case 6: return launch_dominance_prefix<6>(w, s, phase);
+    case 7: return launch_dominance_prefix<7>(w, s, phase);
+    case 8: return launch_dominance_prefix<8>(w, s, phase);
+    case 9: return launch_dominance_prefix<9>(w, s, phase);
+    case 10: return launch_dominance_prefix<10>(w, s, phase);
+    case 11: return launch_dominance_prefix<11>(w, s, phase);
+    case 12: return launch_dominance_prefix<12>(w, s, phase);
+    case 13: return launch_dominance_prefix<13>(w, s, phase);
+    case 14: return launch_dominance_prefix<14>(w, s, phase);
+    case 15: return launch_dominance_prefix<15>(w, s, phase);
+    case 16: return launch_dominance_prefix<16>(w, s, phase);
     default: return kErrBadArg;
   }
 }
@@ -1339,6 +1359,8 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.prefix_mode = (int)value;
   } else if (!strcmp(name, "prefix_bands") && (value == 0 || value == 1)) {
     o.prefix_bands = (int)value;
+  } else if (!strcmp(name, "prefix_count_first") && (value == 0 || value == 1)) {
+    o.prefix_count_first = (int)value;
   } else {
     return kErrBadArg;
   }
@@ -2132,7 +2154,18 @@ static int select_rows(const void* x, int64_t x_row_bytes, int64_t x_row_stride_
     }
   }
   if (int e = stage_prepare(w, fit, true, s)) return e;
-  if (int e = stage_dominance(w, kDomAuto, s)) return e;
+  // A population that keeps filling what is kept from front 0 alone (many objectives, or converged) has no use for
+  // the matrix: where the order-based kernel would build it, the word of the launch memory says what the last two
+  // selections of the shape found, and the kernel counts first when both had enough in front 0 (200 000 x 8, half
+  // kept: the stage 0.98 -> 0.80 ms; a wrong guess costs a second launch, 0.92 ms, once).
+  int64_t count_first = 0;
+  if (batch == 1 && opt().launch_memory && opt().prefix_count_first && prefix_dominance_applies(L) && !opt().peel_stepped) {
+    g.front0_note = outcome_slot(n, m, may_allocate, s, 2);
+    g.front0_size = w.at<int>(L.fsize);
+    g.front0_enough = (int)topk;
+    if (g.front0_note != nullptr && __atomic_load_n(g.front0_note, __ATOMIC_RELAXED) == 3) count_first = topk;
+  }
+  if (int e = stage_dominance(w, kDomAuto, s, count_first)) return e;
   bool peel_orders = false;  // the peel kernel orders a small last front itself (it says so in Ctrl.tail_done)
   bool peel_always_orders = false;  // ... and here every front is small enough: nothing is left to launch but the gather
   bool stepped = false;  // the fronts were peeled one launch each: the last front is ordered likewise, by the kernels of wide.hpp

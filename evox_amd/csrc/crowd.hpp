@@ -145,6 +145,11 @@ struct GatherArgs {
   const Ctrl* ctrl;
   int order_from_peel;  // the host launched nothing that orders the last front: the peel kernel must have (Ctrl.tail_done)
   int* outcome;  // pinned host memory or null: 1 when the peel kernel has ordered the last front of this call, else 2
+  // pinned host memory or null: whether front 0 (front0_size rows) held the front0_enough rows that this call keeps --
+  // 2: no, 1: yes, 3: yes, and at the call that wrote the word before as well
+  int* front0_note;
+  const int* front0_size;
+  int front0_enough;
   // several populations in one launch (blockIdx.z): from one population to the next, bytes between the library's
   // buffers and between the decision vectors, elements between the fitness; the outputs are topk rows apart
   int64_t ws_step, x_step, x2_step, f_step, f2_step;
@@ -193,6 +198,11 @@ __device__ inline void gather_body(const GatherArgs& a, int block, int blocks, i
   // (for the host's choice of launches at its next call; it reads the word without waiting for anything)
   if (a.outcome != nullptr && block == 0 && threadIdx.x == 0)
     __hip_atomic_store(a.outcome, a.ctrl->tail_done != 0 ? 1 : 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  if (a.front0_note != nullptr && block == 0 && threadIdx.x == 0) {
+    const int before = __hip_atomic_load(a.front0_note, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    const int now = *a.front0_size >= a.front0_enough ? (before == 1 || before == 3 ? 3 : 1) : 2;
+    __hip_atomic_store(a.front0_note, now, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
   // A row is copied by g lanes, g = the smallest power of two (4 .. 64) that holds the row's units and its m
   // fitness values: short rows share a wave (a row of 400 bytes in 16-byte units took 25 of 64 lanes).
   const int64_t units = (x ? x_row_bytes : 0) / unit;

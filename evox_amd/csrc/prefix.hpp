@@ -233,19 +233,22 @@ __device__ inline void quad_transpose_pieces(uint64_t (&d)[8], int lane) {
 // tile have no word there).  Dynamic LDS: TT * prefix_lds_bytes(M, WW, buckets).  Writes the words of its tiles in
 // every row of the stretch and adds their popcount to total0[row]; witness0[row] = the highest non-empty word so far
 // (both start from objective_order_kernel's 0 and -1).  Sets param->totals_valid.  mode: bit 0 = the row totals,
-// bit 1 = the matrix.
+// bit 1 = the matrix.  unless_front0 (null: always run): the size of front 0, known from a launch with mode 1 and the
+// count stage; when it holds `enough` rows nobody will read the matrix, and the launch (mode 2) does nothing.
 template <int M, int WW, int TT>
 __global__ __launch_bounds__(kPrefixThreads) void dominance_prefix_kernel(const int* __restrict__ pos, const int* __restrict__ upper,
                                                                           const uint32_t* __restrict__ kid,
                                                                           uint64_t* __restrict__ dom, int n, int kstride,
                                                                           int64_t wstride, int nwords, int shift, int buckets,
                                                                           int chunk, int bands, int mode, int* __restrict__ total0,
-                                                                          int* __restrict__ witness0, SortParam* __restrict__ param) {
+                                                                          int* __restrict__ witness0, SortParam* __restrict__ param,
+                                                                          const int* __restrict__ unless_front0, int enough) {
   constexpr int TS = 64 * WW, T = kPrefixThreads;
   constexpr int TPL = 16 / (WW * TT);  // workgroups that share a 128-byte line of the matrix
   constexpr int MPL = TS / 64;  // members of the tile per lane when a wave walks through them
   extern __shared__ uint64_t prefix_lds[];
   if (param->nonfinite != 0) return;
+  if (unless_front0 != nullptr && *unless_front0 >= enough) return;
   if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) param->totals_valid = 1;  // for the count stage
   // Workgroups go to the eight dies in turn (linear index modulo 8), and a die has its own L2.  The tiles
   // that share the 128-byte lines of the matrix are given to consecutive workgroups of one die, which run

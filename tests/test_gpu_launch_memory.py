@@ -53,3 +53,45 @@ def test_small_and_large_last_fronts_in_turn(n, m):
         for f in (simplex, uniform):
             _check(f, n // 2, nd_environmental_selection(x, f.to(DEV), n // 2))
     runtime.release_workspaces()
+
+
+def test_counting_first_follows_what_front_0_held():
+    """40 000 rows of eight objectives get their matrix from the per-objective orders.  After two selections that
+    found every row they keep in front 0, the next one counts dominators first and builds the matrix only if front 0
+    falls short: populations with a large and with a small front 0, and one with an infinity, take turns, so that
+    every kind of call meets every state of the word."""
+    n, m, k = 40000, 8, 5000
+    g = torch.Generator("cpu").manual_seed(408)
+    wide = torch.rand(n, m, generator=g)  # thousands of rows in front 0
+    deep = torch.rand(n, m, generator=g) + (torch.arange(n) % 64)[:, None].float()  # a few hundred
+    holed = wide.clone()
+    holed[torch.randperm(n, generator=g)[:200], 3] = float("inf")
+    want = {}
+    x = torch.arange(n, dtype=torch.int32, device=DEV)[:, None]
+    front0 = {}
+    for name, f in (("wide", wide), ("deep", deep), ("holed", holed)):
+        want[name] = c_oracle.select(as_np(f), k)
+        front0[name] = int((want[name][1] == 0).sum())
+    assert front0["wide"] >= k > front0["deep"], front0
+
+    def run(name, f):
+        print("count first:", name, flush=True)
+        xs, fs, rs, ds = nd_environmental_selection(x, f.to(DEV), k)
+        assert runtime.last_status()["error"] == 0
+        order, rank, dist, _ = want[name]
+        assert np.array_equal(as_np(xs)[:, 0].astype(np.int64), order), name
+        assert np.array_equal(as_np(rs), rank[order]), name
+        gd, wd = as_np(ds), dist[order]
+        assert np.array_equal(np.isinf(gd), np.isinf(wd)), name
+        fin = np.isfinite(wd)
+        np.testing.assert_allclose(gd[fin], wd[fin], rtol=1e-4)
+
+    turns = ["wide", "wide", "wide", "wide", "deep", "deep", "wide", "wide", "holed", "wide", "wide", "wide", "holed",
+             "deep", "wide"]
+    table = {"wide": wide, "deep": deep, "holed": holed}
+    for name in turns:
+        run(name, table[name])
+    with runtime.options(prefix_count_first=0):
+        for name in ("wide", "wide", "wide", "deep"):
+            run(name, table[name])
+    runtime.release_workspaces()
