@@ -28,16 +28,18 @@ FP32_VECTOR_PEAK_GFLOPS = 157300.0
 
 
 
-def profile_traffic(workload, kernel):
+def profile_traffic(workload, kernel, variant=None):
     """HBM bytes per launch of `kernel` as the committed counter summary of this workload holds them
     (profiles/<workload>_selection_hbm_traffic.md: FETCH_SIZE and WRITE_SIZE runs of this script, scaled by what the
-    same counters read for a 512 MiB copy); None where the summary has no row for the kernel."""
+    same counters read for a 512 MiB copy); None where the summary has no row for the kernel.  variant: words after
+    the kernel's name in a summary that lists the kinds of launches of one kernel apart (else the first row counts)."""
     path = os.path.join(ROOT, "profiles", f"{workload.lower()}_selection_hbm_traffic.md")
     if not os.path.exists(path):
         return None
     for line in open(path):
         cells = [c.strip() for c in line.strip().strip("|").split("|")]
-        if len(cells) == 6 and cells[0].startswith("evx::" + kernel) and cells[0][len("evx::" + kernel):][:1] in ("", "<"):
+        if (len(cells) == 6 and cells[0].startswith("evx::" + kernel) and cells[0][len("evx::" + kernel):][:1] in ("", "<")
+                and (variant is None or variant in cells[0])):
             try:
                 return {"bytes": (float(cells[4]) + float(cells[5])) * 1e6, "read_MB": float(cells[4]),
                         "written_MB": float(cells[5]), "source": os.path.relpath(path, ROOT)}
@@ -690,9 +692,13 @@ def main():
                                   "also writes the matrix"),
                          "matrix_launch": {"achieved": d["achieved"], "frac": d["frac"], "kernel_us": d["prefix_kernel_us"]}})
     measured = profile_traffic(args.workload, roofline["kernel"])
-    if measured is not None and "matrix_launch" in roofline:  # (the committed counters are those of the launch with the matrix)
+    if measured is not None and "matrix_launch" in roofline:  # (the first row is that of the launches with the matrix)
         roofline["matrix_launch"]["traffic"] = measured["bytes"]
         roofline["matrix_launch"]["traffic_source"] = measured["source"]
+        alone = profile_traffic(args.workload, roofline["kernel"], "row totals alone")
+        if alone is not None:
+            roofline["traffic"] = alone["bytes"]
+            roofline["traffic_source"] = alone["source"]
     elif measured is not None:
         roofline["traffic"] = measured["bytes"]
         roofline["traffic_source"] = measured["source"]

@@ -14,10 +14,12 @@
  *     whether or not that entry point is ever called: it is part of the device image); and 64 bytes of pinned host
  *     memory per device, allocated at the first selection, in which the last kernel of a selection notes whether the
  *     peel kernel ordered the last front (for a selection of 8-byte fitness: whether its last front held more than
- *     8192 rows) -- the next selection of a like shape picks its launches by it (tunable "launch_memory"; 0 = never
- *     looked at).  Results never depend on any of it; the time of a call can, by a few microseconds (a first call, or
- *     calls whose last fronts alternate between small and large, take the other set of launches; with 8-byte fitness
- *     and a front of all of 20 000 rows the other set costs 0.7 ms more, once).
+ *     8192 rows; for a large population whose matrix comes from the per-objective orders: whether front 0 held
+ *     every row kept) -- the next selection of a like shape picks its launches by it (tunable "launch_memory"; 0 =
+ *     never looked at).  Results never depend on any of it; the time of a call can, by a few microseconds (a first
+ *     call, or calls whose last fronts alternate between small and large, take the other set of launches; with 8-byte
+ *     fitness and a front of all of 20 000 rows the other set costs 0.7 ms more, once; so does, at 200 000 rows of
+ *     eight objectives, the first selection with a short front 0 after two or more with a full one).
  *   - Fitness `f` is float32, addressed as f[i * stride_row + k * stride_col] (strides in elements),
  *     minimisation, n rows (individuals) by m columns (objectives).
  *   - The workspace must hold evox_hip_workspace_bytes(n, m) bytes, 256-byte aligned.  Calls that
