@@ -95,3 +95,44 @@ def test_counting_first_follows_what_front_0_held():
         for name in ("wide", "wide", "wide", "deep"):
             run(name, table[name])
     runtime.release_workspaces()
+
+
+def test_a_graph_captured_while_counting_first_builds_the_matrix_when_a_replay_needs_it():
+    """Captured after selections that found all they keep in front 0, a selection holds the launch for the row
+    totals, the count stage and the guarded launch for the matrix: a replay on a population with a short front 0
+    must build the matrix on the device's own decision (the host plays no part in a replay)."""
+    n, m, k = 40000, 8, 5000
+    g = torch.Generator("cpu").manual_seed(409)
+    wide = torch.rand(n, m, generator=g)
+    deep = torch.rand(n, m, generator=g) + (torch.arange(n) % 64)[:, None].float()
+    want = {"wide": c_oracle.select(as_np(wide), k), "deep": c_oracle.select(as_np(deep), k)}
+    assert int((want["wide"][1] == 0).sum()) >= k > int((want["deep"][1] == 0).sum())
+    x = torch.arange(n, dtype=torch.int32, device=DEV)[:, None]
+    f_static = wide.to(DEV).clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):  # the word of the launch memory says "twice in a row" from the second call on
+            nd_environmental_selection(x, f_static, k)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = nd_environmental_selection(x, f_static, k)
+    for name in ("wide", "deep", "deep", "wide", "deep"):
+        print("replay:", name, flush=True)
+        f_static.copy_((wide if name == "wide" else deep).to(DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        xs, fs, rs, ds = [t.clone() for t in out]
+        nd_environmental_selection(x, wide.to(DEV), k)  # eager work between the replays
+        torch.cuda.synchronize()
+        order, rank, dist, _ = want[name]
+        assert np.array_equal(as_np(xs)[:, 0].astype(np.int64), order), name
+        assert np.array_equal(as_np(rs), rank[order]), name
+        gd, wd = as_np(ds), dist[order]
+        assert np.array_equal(np.isinf(gd), np.isinf(wd)), name
+        fin = np.isfinite(wd)
+        np.testing.assert_allclose(gd[fin], wd[fin], rtol=1e-4)
+    del graph
+    runtime.release_workspaces()
