@@ -63,6 +63,9 @@ struct Options {
                                         // takes both tiles of a 128-byte line; 0 = never
   int prefix_mode = 3;  // measurements: 1 = popcounts only, 2 = matrix only
   int prefix_bands = 1;  // stretches of the order-based matrix: 1 = bands of rows counted from row 0, 0 = from each tile's diagonal
+  int order_stream = 1;  // the per-objective orders of more than 32768 rows come from workgroups that sort shares of
+                         // them in LDS (0: from the radix sort whose workgroups wait for each other)
+  int order_stream_capacity = 16384;  // entries that such a workgroup sorts at once (tests make it small: shares in pieces)
   int prefix_count_first = 1;  // a selection whose last two of this shape found all they keep in front 0 has the order-based
                                // kernel count dominators first and build the matrix only if front 0 falls short; 0 = never
 };
@@ -979,6 +982,28 @@ static int stage_dominance_prefix(const Ws& w, bool orders_only, hipStream_t s, 
     EVX_LAUNCH_CHECK();
     return orders_only ? 0 : dispatch_dominance_prefix(w, s, phase);
   }
+  // shares of one objective's order that the streaming kernel would cut: as many as give every compute unit a
+  // workgroup, if shares of kOrderStreamShare rows need no more than that
+  const int stream_parts = device_cus() / L.m;
+  if (opt().order_stream && L.n > kOrderStreamSample && L.n <= kOrderStreamMaxRows && (L.npad & 3) == 0 && stream_parts >= 1 &&
+      stream_parts <= kOrderStreamSample && (int64_t)stream_parts * kOrderStreamShare >= L.n) {
+    // larger populations likewise, by workgroups that read their objective's keys once and sort their share of the
+    // order in LDS -- while those shares stay small: 40 000 x 8 the orders in 52 instead of 127 us, 65 536 x 3 57 / 90,
+    // 100 000 x 8 105 / 144, 200 000 x 3 120 / 147; 200 000 x 8 (shares of 6250 rows) 201 / 185: the radix sort below
+    const size_t stream_lds = sizeof(double) * kOrderStreamCapacity;
+    if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(objective_order_stream_kernel), stream_lds)) return e;
+    const int parts = stream_parts;
+    hipLaunchKernelGGL(objective_order_stream_kernel, dim3(L.m * parts), dim3(kOrderStreamThreads), stream_lds, s, w.at<float>(L.xs),
+                       L.npad, L.n, L.m, parts, opt().order_stream_capacity, w.at<SortParam>(L.sortparam), w.ctrl(),
+                       w.at<int>(L.total0), w.at<int>(L.witness0), radix_buffers(w));
+    EVX_LAUNCH_CHECK();
+    int64_t blocks = ((int64_t)L.n * L.m + 255) / 256;
+    if (blocks > device_cus() * 8) blocks = device_cus() * 8;
+    hipLaunchKernelGGL(objective_positions_kernel, dim3((unsigned)blocks), dim3(256), 0, s, L.n, L.m, w.at<int>(L.slot_of),
+                       w.at<SortParam>(L.sortparam), w.ctrl(), w.at<int>(L.pos), w.at<int>(L.scost), radix_buffers(w));
+    EVX_LAUNCH_CHECK();
+    return orders_only ? 0 : dispatch_dominance_prefix(w, s, phase);
+  }
   const size_t lds = kRadixLdsBytes;
   if (int e = grant_dynamic_lds(reinterpret_cast<const void*>(objective_order_kernel), lds)) return e;
   // more workers than one per 1024 rows: every one of them handles its share of all m segments
@@ -1359,6 +1384,10 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.prefix_mode = (int)value;
   } else if (!strcmp(name, "prefix_bands") && (value == 0 || value == 1)) {
     o.prefix_bands = (int)value;
+  } else if (!strcmp(name, "order_stream") && (value == 0 || value == 1)) {
+    o.order_stream = (int)value;
+  } else if (!strcmp(name, "order_stream_capacity") && value >= 1 && value <= kOrderStreamCapacity) {
+    o.order_stream_capacity = (int)value;
   } else if (!strcmp(name, "prefix_count_first") && (value == 0 || value == 1)) {
     o.prefix_count_first = (int)value;
   } else {

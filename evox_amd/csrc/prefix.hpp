@@ -153,6 +153,168 @@ __global__ __launch_bounds__(kMidArgsortThreads) void objective_order_lds_kernel
   }
 }
 
+// The same orders for larger populations, still without a wait between workgroups: the workgroups share the
+// objectives out, `parts` to each, and a workgroup produces a run of consecutive positions of its objective's order.
+// Rows are composites (key << 20 | original index: distinct, below 2^52).  Every workgroup of an objective sorts the
+// same kOrderStreamSample composites (rows n i / sample) and takes the composites between two of them as its share,
+// which makes `parts` shares of about n / parts rows whatever the values are, equal ones included; it then reads the
+// objective's keys once, counts the composites below its share (where its run starts) and collects those inside it in
+// LDS, sorts them there (the bitonic network of radix.hpp over doubles 2^52 + composite, which order like the
+// composites) and writes the run.  A share that does not fit `capacity` entries -- rows arranged so that the sample
+// misses where they crowd -- is taken in pieces: the largest stretch of composites from the share's start that fits is
+// found by bisection over the composites, a pass over the keys per step, as often as it takes.
+// Where the time goes (200 000 x 8 in 32 shares of 6250 rows, 154 us): the sort of the sample 23 us, the pass over the
+// keys 34 + 20 for storing what it collects, the sort of the share 77 (padded to 8192; 35 when padded to 4096) -- the
+// network's passes are what this costs, which is why the host takes this kernel only while shares of at most
+// kOrderStreamShare rows leave it no more workgroups than the device has compute units.
+// Grid: m * parts workgroups of kOrderStreamThreads.  Dynamic LDS: 8 * kOrderStreamCapacity bytes.  n <= 2^20.
+constexpr int kOrderStreamThreads = 1024;
+constexpr int kOrderStreamCapacity = 16384;
+constexpr int kOrderStreamSample = 2048;
+constexpr int kOrderStreamMaxRows = 1 << 20;
+constexpr int kOrderStreamShare = 3200;  // rows of a share, at most, that the host aims at: sorted as 4096 entries
+
+__global__ __launch_bounds__(kOrderStreamThreads) void objective_order_stream_kernel(const float* __restrict__ xs, int npad, int n, int m,
+                                                                                     int parts, int capacity,
+                                                                                     const SortParam* __restrict__ param,
+                                                                                     const Ctrl* __restrict__ ctrl,
+                                                                                     int* __restrict__ total0, int* __restrict__ witness0,
+                                                                                     RadixBuffers buf) {
+  extern __shared__ __attribute__((aligned(16))) double order_stream_comp[];
+  __shared__ int taken;           // composites of the present pass that lie in its range
+  __shared__ int below_of[16];    // per wave: composites below the range
+  if (param->nonfinite != 0 || ctrl->err != 0) return;
+  for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < n; j += gridDim.x * blockDim.x) {
+    total0[j] = 0;
+    witness0[j] = -1;
+  }
+  double* const comp = order_stream_comp;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int k = (int)blockIdx.x % m, part = (int)blockIdx.x / m;
+  if (part >= parts) return;
+  const float* __restrict__ col = xs + (int64_t)k * npad;
+  unsigned long long* __restrict__ sorted = buf.pairs[0] + (int64_t)k * buf.kstride;
+  constexpr unsigned long long kBias = 0x4330000000000000ull;  // the bits of 2^52 as a double
+  constexpr unsigned long long kEnd = 1ull << 52;               // above every composite
+  auto composite = [&](int e) { return ((unsigned long long)ordered_key(col[e]) << 20) | (unsigned long long)(unsigned)e; };
+
+  // ---- the share: between two members of the sorted sample
+  for (int i = tid; i < kOrderStreamSample; i += kOrderStreamThreads)
+    comp[bitonic_slot(i)] = __longlong_as_double((long long)(kBias | composite((int)(((int64_t)i * n) / kOrderStreamSample))));
+  __syncthreads();
+  bitonic_sort_lds(comp, kOrderStreamSample);
+  auto sample_at = [&](int i) { return (unsigned long long)__double_as_longlong(comp[bitonic_slot(i)]) & (kEnd - 1ull); };
+  unsigned long long lo = part == 0 ? 0ull : sample_at((int)(((int64_t)part * kOrderStreamSample) / parts));
+  const unsigned long long end = part == parts - 1 ? kEnd : sample_at((int)(((int64_t)(part + 1) * kOrderStreamSample) / parts));
+  __syncthreads();  // (the sample is overwritten from here on)
+
+  // One pass over the objective's keys: the composites in [from, to) are counted (the return value) and, with `collect`,
+  // the first `capacity` of them stored; *below = the composites smaller than `from`.
+  auto pass = [&](unsigned long long from, unsigned long long to, bool collect, int* below) {
+    if (tid == 0) taken = 0;
+    __syncthreads();
+    const unsigned long long span = to - from;
+    int under = 0;  // (wave-uniform)
+    // (a wave takes 256 keys a step and fetches the keys of kAhead steps before it looks at the first of them)
+    constexpr int kAhead = 8;
+    for (int g0 = 256 * wave; g0 < n; g0 += kAhead * 4 * kOrderStreamThreads) {  // (wave-uniform)
+      float4 q[kAhead];
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) {
+        const int e0 = g0 + a * 4 * kOrderStreamThreads + 4 * lane;
+        q[a] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (e0 + 3 < n) {
+          q[a] = *reinterpret_cast<const float4*>(col + e0);
+        } else if (e0 < n) {
+          q[a].x = col[e0];
+          if (e0 + 1 < n) q[a].y = col[e0 + 1];
+          if (e0 + 2 < n) q[a].z = col[e0 + 2];
+        }
+      }
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) {
+        const int b0 = g0 + a * 4 * kOrderStreamThreads;
+        if (b0 >= n) break;  // (wave-uniform)
+        const int e0 = b0 + 4 * lane;
+        const float v[4] = {q[a].x, q[a].y, q[a].z, q[a].w};
+        unsigned long long c[4];
+        uint64_t in[4];
+        int here = 0;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          c[u] = ((unsigned long long)ordered_key(v[u]) << 20) | (unsigned long long)(unsigned)(e0 + u);
+          const bool live = e0 + u < n;
+          in[u] = __builtin_amdgcn_ballot_w64(live && c[u] - from < span);
+          under += __popcll(__builtin_amdgcn_ballot_w64(live && c[u] < from));
+          here += __popcll(in[u]);
+        }
+        if (here != 0) {  // (wave-uniform)
+          int at = 0;
+          if (lane == 0) at = atomicAdd(&taken, here);
+          at = __builtin_amdgcn_readfirstlane(at);
+          if (collect) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const int mine = at + __popcll(in[u] & ((1ull << lane) - 1ull));
+              if (((in[u] >> lane) & 1ull) != 0ull && mine < capacity)
+                comp[bitonic_slot(mine)] = __longlong_as_double((long long)(kBias | c[u]));
+              at += __popcll(in[u]);
+            }
+          }
+        }
+      }
+    }
+    if (lane == 0) below_of[wave] = under;
+    __syncthreads();
+    if (below != nullptr) {
+      int sum = 0;
+#pragma unroll
+      for (int w = 0; w < kOrderStreamThreads / 64; ++w) sum += below_of[w];
+      *below = sum;
+    }
+    const int count = taken;
+    __syncthreads();  // (everybody has read the counters before the next pass clears them)
+    return count;
+  };
+
+  int run_start = 0;
+  bool first = true;
+  while (lo < end) {  // (the same in every thread)
+    unsigned long long hi = end;
+    int below = 0;
+    int count = pass(lo, hi, true, &below);
+    if (first) run_start = below;
+    first = false;
+    if (count > capacity) {
+      // [lo, fits) holds at most one composite; [lo, over) too many
+      unsigned long long fits = lo + 1ull, over = hi;
+      while (over - fits > 1ull) {
+        const unsigned long long mid = fits + (over - fits) / 2ull;
+        if (pass(lo, mid, false, nullptr) <= capacity)
+          fits = mid;
+        else
+          over = mid;
+      }
+      hi = fits;
+      count = pass(lo, hi, true, nullptr);
+    }
+    if (count > 0) {
+      int padded = kRowsBitonicMin;
+      while (padded < count) padded <<= 1;
+      for (int e = count + tid; e < padded; e += kOrderStreamThreads) comp[bitonic_slot(e)] = (double)INFINITY;
+      __syncthreads();
+      bitonic_sort_lds(comp, padded);
+      for (int e = tid; e < count; e += kOrderStreamThreads) {
+        const unsigned long long c = (unsigned long long)__double_as_longlong(comp[bitonic_slot(e)]) & (kEnd - 1ull);
+        sorted[run_start + e] = ((c >> 20) << 32) | (c & 0xFFFFFull);
+      }
+      __syncthreads();
+    }
+    run_start += count;
+    lo = hi;
+  }
+}
+
 __global__ __launch_bounds__(256) void objective_positions_kernel(int n, int m, const int* __restrict__ slot_of,
                                                                   SortParam* __restrict__ param, const Ctrl* __restrict__ ctrl,
                                                                   int* __restrict__ pos, int* __restrict__ upper, RadixBuffers buf) {

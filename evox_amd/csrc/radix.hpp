@@ -770,6 +770,46 @@ __device__ inline void bitonic_pass(double* comp, int npad, int k, int low_log) 
   }
 }
 
+// Sorts comp[bitonic_slot(0 .. npad-1)] ascending in place: npad a power of two from kRowsBitonicMin on, the entries
+// distinct or +inf.  Every thread of the workgroup calls it, after a barrier that follows the last write of an entry;
+// it ends with a barrier.
+__device__ inline void bitonic_sort_lds(double* comp, int npad) {
+  // phases 2, 4 and 8: eight neighbours sorted in registers, every second run of eight descending
+  for (int u = threadIdx.x; u < (npad >> 3); u += blockDim.x) {
+    const int base = u << 3;
+    const int flip = (base & 8) ? 7 : 0;
+    double v[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) v[c] = comp[bitonic_slot(base + (c ^ flip))];
+    compare_exchange(v[0], v[1]); compare_exchange(v[3], v[2]); compare_exchange(v[4], v[5]); compare_exchange(v[7], v[6]);
+    compare_exchange(v[0], v[2]); compare_exchange(v[1], v[3]); compare_exchange(v[6], v[4]); compare_exchange(v[7], v[5]);
+    compare_exchange(v[0], v[1]); compare_exchange(v[2], v[3]); compare_exchange(v[5], v[4]); compare_exchange(v[7], v[6]);
+#pragma unroll
+    for (int d = 4; d > 0; d >>= 1)
+#pragma unroll
+      for (int c = 0; c < 8; ++c)
+        if ((c & d) == 0) compare_exchange(v[c], v[c | d]);
+#pragma unroll
+    for (int c = 0; c < 8; ++c) comp[bitonic_slot(base + (c ^ flip))] = v[c];
+  }
+  __syncthreads();
+  for (int k = 16, top = 3; k <= npad; k <<= 1, ++top) {  // top = the highest index bit that phase k pairs
+    int low_log = (top / 3) * 3;
+    const int first = top - low_log + 1;
+    if (first == 1)
+      bitonic_pass<1>(comp, npad, k, low_log);
+    else if (first == 2)
+      bitonic_pass<2>(comp, npad, k, low_log);
+    else
+      bitonic_pass<3>(comp, npad, k, low_log);
+    __syncthreads();
+    for (low_log -= 3; low_log >= 0; low_log -= 3) {
+      bitonic_pass<3>(comp, npad, k, low_log);
+      __syncthreads();
+    }
+  }
+}
+
 __global__ __launch_bounds__(1024) void rows_bitonic_argsort_kernel(const void* __restrict__ key, int kind, int64_t batch_stride,
                                                                     int64_t stride, int64_t batch, int n, int npad,
                                                                     const int* __restrict__ prev, int* __restrict__ order_out) {
@@ -794,40 +834,7 @@ __global__ __launch_bounds__(1024) void rows_bitonic_argsort_kernel(const void* 
       comp[bitonic_slot(e)] = c;
     }
     __syncthreads();
-    // phases 2, 4 and 8: eight neighbours sorted in registers, every second run of eight descending
-    for (int u = threadIdx.x; u < (npad >> 3); u += blockDim.x) {
-      const int base = u << 3;
-      const int flip = (base & 8) ? 7 : 0;
-      double v[8];
-#pragma unroll
-      for (int c = 0; c < 8; ++c) v[c] = comp[bitonic_slot(base + (c ^ flip))];
-      compare_exchange(v[0], v[1]); compare_exchange(v[3], v[2]); compare_exchange(v[4], v[5]); compare_exchange(v[7], v[6]);
-      compare_exchange(v[0], v[2]); compare_exchange(v[1], v[3]); compare_exchange(v[6], v[4]); compare_exchange(v[7], v[5]);
-      compare_exchange(v[0], v[1]); compare_exchange(v[2], v[3]); compare_exchange(v[5], v[4]); compare_exchange(v[7], v[6]);
-#pragma unroll
-      for (int d = 4; d > 0; d >>= 1)
-#pragma unroll
-        for (int c = 0; c < 8; ++c)
-          if ((c & d) == 0) compare_exchange(v[c], v[c | d]);
-#pragma unroll
-      for (int c = 0; c < 8; ++c) comp[bitonic_slot(base + (c ^ flip))] = v[c];
-    }
-    __syncthreads();
-    for (int k = 16, top = 3; k <= npad; k <<= 1, ++top) {  // top = the highest index bit that phase k pairs
-      int low_log = (top / 3) * 3;
-      const int first = top - low_log + 1;
-      if (first == 1)
-        bitonic_pass<1>(comp, npad, k, low_log);
-      else if (first == 2)
-        bitonic_pass<2>(comp, npad, k, low_log);
-      else
-        bitonic_pass<3>(comp, npad, k, low_log);
-      __syncthreads();
-      for (low_log -= 3; low_log >= 0; low_log -= 3) {
-        bitonic_pass<3>(comp, npad, k, low_log);
-        __syncthreads();
-      }
-    }
+    bitonic_sort_lds(comp, npad);
     for (int e = threadIdx.x; e < n; e += blockDim.x) {
       const int pos = (int)((uint64_t)comp[bitonic_slot(e)] & 16383ull);
       order_out[row * n + e] = prev_row ? prev_row[pos] : pos;

@@ -236,6 +236,60 @@ def test_matrix_from_objective_orders_equals_the_pairwise_matrix(m):
                 assert torch.equal(ranks, non_dominate_rank(fd)), (m, name)
 
 
+@pytest.mark.parametrize("m", [2, 3, 5, 8, 16])
+def test_objective_orders_of_more_than_32768_rows(m):
+    """Above 32 768 rows the per-objective orders come from workgroups that read their objective's keys once and sort a
+    share of the order in LDS (the shares are cut between members of a sorted sample).  The matrix built from them
+    must be that of the radix sort's orders, word for word: uniform values, few distinct values, a constant objective,
+    values with the period of the sample, and a crowd of equal values that the sample does not see (a share too large
+    for the workgroup's LDS, taken in pieces); then the same with room for 700 entries only, so that every share is
+    taken in pieces."""
+    n = 36000
+    g = torch.Generator("cpu").manual_seed(800 + m)
+    cases = {}
+    cases["uniform"] = torch.rand(n, m, generator=g)
+    cases["few_values"] = torch.randint(0, 7, (n, m), generator=g).float()
+    const = torch.rand(n, m, generator=g)
+    const[:, 0] = 3.0
+    cases["constant_objective"] = const
+    period = torch.rand(n, m, generator=g)
+    period[:, m - 1] = (torch.arange(n) % 2048).float()  # (the sample takes every (n / 2048)-th row)
+    cases["periodic"] = period
+    hidden = torch.zeros(n, m)
+    hidden[:, 0] = torch.rand(n, generator=g)
+    seen = (torch.arange(2048) * n) // 2048  # the rows of the sample: the only ones that differ in the last objective
+    hidden[seen, m - 1] = 1.0 + torch.rand(2048, generator=g)
+    cases["crowd_hidden_from_the_sample"] = hidden
+    for name, f in cases.items():
+        say("stream_orders", m, name)
+        with runtime.options(prefix_min_rows=4097, order_stream=0):
+            want_state = {}
+            want = _matrix_words(f.contiguous(), 0, want_state)
+        for capacity in (16384, 700):
+            with runtime.options(prefix_min_rows=4097, order_stream=1, order_stream_capacity=capacity):
+                got_state = {}
+                got = _matrix_words(f.contiguous(), 0, got_state)
+            assert np.array_equal(got, want), (m, name, capacity, int((got != want).sum()))
+            assert np.array_equal(got_state["count"], want_state["count"]), (m, name, capacity)
+            assert np.array_equal(got_state["rank"], want_state["rank"]), (m, name, capacity)
+        del want, got
+    # the sorted pairs stay behind for the ordering of a large last front: a selection out of one front
+    from oracle import c_oracle
+
+    front = cases["uniform"] / cases["uniform"].sum(dim=1, keepdim=True)
+    order, rank, dist, _ = c_oracle.select(as_np(front), n // 2)
+    x = torch.arange(n, dtype=torch.int32, device=DEV)[:, None]
+    for capacity in (16384, 700):
+        with runtime.options(prefix_min_rows=4097, order_stream_capacity=capacity):
+            xs, fs, rs, ds = nd_environmental_selection(x, front.to(DEV), n // 2)
+        assert runtime.last_status()["error"] == 0
+        assert np.array_equal(as_np(rs), rank[order])
+        assert_dist_close(ds, dist[order], "stream orders")
+        if m in (2, 3, 8):
+            assert np.array_equal(as_np(xs)[:, 0].astype(np.int64), order)
+    runtime.release_workspaces()
+
+
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 8, 11, 16])
 def test_dominance_arithmetic_form_corner_values(m):
     """A population of finite values takes the arithmetic form of the dominance test (signs of differences):
