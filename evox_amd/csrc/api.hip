@@ -63,6 +63,8 @@ struct Options {
                                         // takes both tiles of a 128-byte line; 0 = never
   int prefix_mode = 3;  // measurements: 1 = popcounts only, 2 = matrix only
   int prefix_bands = 1;  // stretches of the order-based matrix: 1 = bands of rows counted from row 0, 0 = from each tile's diagonal
+  int batched_stage = 1;  // the one-workgroup kernel reads its dominators from a copy of the fitness in LDS when the populations
+                          // have at most 256 rows and are no more than the device has compute units (0: by scalar loads always)
   int order_stream = 1;  // the per-objective orders of more than 32768 rows come from workgroups that sort shares of
                          // them in LDS (0: from the radix sort whose workgroups wait for each other)
   int order_stream_capacity = 16384;  // entries that such a workgroup sorts at once (tests make it small: shares in pieces)
@@ -1210,7 +1212,10 @@ constexpr uint32_t kPoisonFloat = 0x7FC00000u;  // NaN as a distance
 template <int M>
 static int launch_batched_m(const BatchedArgs& a, int64_t batch, hipStream_t s) {
   const int nt = (int)round_up(a.n, 64);
-  const size_t lds = batched_lds_bytes(nt, M);
+  // (few populations of at most 256 rows: every workgroup has a compute unit, and every wave a SIMD, to itself -- 200 x 3:
+  // the matrix in 7.5 instead of 12 us; with two waves to a SIMD the scalar loads win: 512 x 3 14 against 16.5 us)
+  const bool stage = batch <= device_cus() && nt <= 256 && M <= 8 && opt().batched_stage;
+  const size_t lds = batched_lds_bytes(nt, M) + (stage ? batched_stage_bytes(nt, M) : 0);
   // the attribute belongs to the (kernel, device) pair: remembered per device
   static size_t granted[64] = {0};
   static std::mutex mu;  // (a smaller grant by another thread must not follow a larger one)
@@ -1228,6 +1233,7 @@ static int launch_batched_m(const BatchedArgs& a, int64_t batch, hipStream_t s) 
   // grid.x carries the batch; very large batches go in slices
   for (int64_t b0 = 0; b0 < batch; b0 += 0x40000000ll) {
     BatchedArgs part = a;
+    part.stage_fitness = stage ? 1 : 0;
     const int64_t nb = batch - b0 < 0x40000000ll ? batch - b0 : 0x40000000ll;
     part.f += b0 * a.f_stride_b;
     if (part.rank_all) part.rank_all += b0 * a.n;
@@ -1384,6 +1390,8 @@ static int set_named(Options& o, const char* name, int64_t value) {
     o.prefix_mode = (int)value;
   } else if (!strcmp(name, "prefix_bands") && (value == 0 || value == 1)) {
     o.prefix_bands = (int)value;
+  } else if (!strcmp(name, "batched_stage") && (value == 0 || value == 1)) {
+    o.batched_stage = (int)value;
   } else if (!strcmp(name, "order_stream") && (value == 0 || value == 1)) {
     o.order_stream = (int)value;
   } else if (!strcmp(name, "order_stream_capacity") && value >= 1 && value <= kOrderStreamCapacity) {

@@ -49,6 +49,11 @@ struct BatchedArgs {
   float* out_f;            // (batch, topk, m)
   int* out_rank;           // (batch, topk)
   float* out_dist;         // (batch, topk)
+  // 1: the launch has batched_stage_bytes(nt, m) more dynamic LDS, behind the layout below, and the dominators of the
+  // arithmetic test are read from a copy of the fitness there (few small populations: a wave that has its SIMD to
+  // itself waits out every scalar load in full, 0.35 us per eight dominators; reads from LDS return in order and are
+  // issued ahead); 0: from memory by scalar loads, which is faster once waves share a SIMD -- the LDS has one port
+  int stage_fitness;
 };
 
 // Number of elements of `tile` (nv entries, (key << 32 | index) pairs) that are smaller than `mine`.
@@ -80,6 +85,9 @@ __host__ __device__ inline int batched_row_stride(int nt, int m) {
 __host__ __device__ inline size_t batched_lds_bytes(int nt, int m) {
   return sizeof(uint64_t) * ((size_t)nt * batched_row_stride(nt, m) + 32) + sizeof(int) * (size_t)nt;
 }
+// The copy of the fitness for BatchedArgs::stage_fitness: rows of the objectives rounded up to a multiple of four.
+__host__ __device__ inline int batched_stage_stride(int m) { return (m + 3) & ~3; }
+__host__ __device__ inline size_t batched_stage_bytes(int nt, int m) { return sizeof(float) * (size_t)nt * batched_stage_stride(m); }
 
 // Position of every candidate among the nv (key << 32 | index) pairs of `tile`, by counting the smaller
 // ones; the count of candidate q is split over `parts` threads (q + nvq * part, nvq = nv rounded up to whole
@@ -182,6 +190,15 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(M <= 12 ? 
     finite_row &= !valid || fabsf(xj[k]) <= 3.4028234663852886e38f;
     xz[k] = xj[k] + 0.0f;
   }
+  constexpr int MS = (M + 3) & ~3;
+  // (behind the layout above, 16-byte aligned; the address is formed where it is used: one register less to keep)
+  auto stage_of = [&]() { return reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(lds64) + batched_lds_bytes(nt, M)); };
+  constexpr bool kMayStage = M <= 8;  // (with more objectives the extra path costs the kernel a register it does not have)
+  if (kMayStage && a.stage_fitness) {
+    float* const stage = stage_of();
+#pragma unroll
+    for (int k = 0; k < M; ++k) stage[j * MS + k] = xj[k];
+  }
   const bool all_finite = __syncthreads_and(finite_row) != 0;
   const bool packed_rows = a.f_stride_col == 1 && a.f_stride_row == M;
   constexpr int GP = M <= 8 ? 8 : 4;  // dominators per group of scalar loads (at most 64 scalars)
@@ -196,7 +213,23 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(M <= 12 ? 
       uint32_t acc = 0;
       const int i0 = w * 64 + h * 32;
       const int64_t second0 = i0 >= a.n_first ? a.f_second : 0;
-      if (all_finite && packed_rows && i0 + 32 <= n && (i0 + 32 <= a.n_first || i0 >= a.n_first)) {
+      if (kMayStage && all_finite && a.stage_fitness) {
+        // (rows from n on hold NaN: a lane's test against them is discarded)
+#pragma unroll 8
+        for (int t = 31; t >= 0; --t) {
+          const int i = i0 + t;  // wave-uniform
+          float v[MS];
+#pragma unroll
+          for (int q = 0; q < MS / 4; ++q) {
+            const float4 piece = *reinterpret_cast<const float4*>(stage_of() + i * MS + 4 * q);
+            v[4 * q] = piece.x; v[4 * q + 1] = piece.y; v[4 * q + 2] = piece.z; v[4 * q + 3] = piece.w;
+          }
+          uint32_t o = 0u;
+#pragma unroll
+          for (int k = 0; k < M; ++k) o |= __float_as_uint(xz[k] - v[k]);
+          acc = shift_in_positive(acc, i < n ? o : 0u);
+        }
+      } else if (all_finite && packed_rows && i0 + 32 <= n && (i0 + 32 <= a.n_first || i0 >= a.n_first)) {
         // rows of M consecutive floats: GP dominators are GP M consecutive scalars, fetched by wide scalar loads
         // (the 32 dominators come from one tensor)
 #pragma unroll 1

@@ -383,6 +383,7 @@ int evox_hip_read_status(const void* workspace, void* stream, int32_t* host_out8
  * protocol, 0 = master barrier and front bitmaps), "peel_record_blocks" (0 = by size, or 16 .. 255), "spin_limit" (the bound of every device-side wait: a value above 65535 is a time in units of 10 ns on the device's constant clock, default 4000000 = 40 ms; a value up to 65535 counts failed polls, for tests that force a wait to give up), "two_small_min_rows" (default 128: from this many rows on, a population of two objectives that goes to a one-workgroup kernel takes the one without a dominance matrix, which also raises evox_hip_batched_max_rows(2) to 4096; 0 = never), "two_min_rows" (default 4097: smallest population of two objectives that is ranked without a dominance matrix -- rows sorted by (f1, f2, index), every front the strict prefix minima of f2 among the rows that remain; 0 = never) and "two_min_rows_partial" (default 4097: the same where the ranking may stop at a front, as in a selection; there the peeling ends once the fronts so far hold the rows asked for), "peel_stepped" (0 = the fronts are peeled by one persistent kernel where its grid can be resident at once, 1 = always by one launch per front and the last front by kernels that never wait for each other: slower, needs no co-residency, and waits for the stream between groups of sixteen launches), "dominance_tile_words" (0 = by size: 2 or 4; or 2, 4, 8, 16), "dominance_folded" (1 = only the blocks at or below the diagonal are launched; 0 = the whole rectangle), "mid_argsort" (1 = an argsort step of 8193 to 32768 positions, and a last front of 1025 to 32768 rows, are ordered by workgroups that sort in LDS without waiting for each other; 0 = the radix sort and ranking by counting), "small_sort" (1 = one-kernel slot sort up to 4096 rows),
  * "prefix_min_rows" (default 65536: smallest finite population of three objectives whose matrix is built from the per-objective orders -- a quarter more rows with two, fewer with more: 28672 at eight, 10240 at sixteen; 0 = never),
  * "prefix_bands" (default 1), "prefix_double_tile" (default 131072 rows, 0 = never), "prefix_mode" (default 3; 1 and 2 build only half of that kernel's output, for measurements),
+ * "batched_stage" (default 1: the one-workgroup kernel reads the dominators of populations of at most 256 rows and eight objectives from a copy of the fitness in LDS when the launch holds no more populations than the device has compute units; 0 = by scalar loads from memory always),
  * "order_stream" (default 1: for more than 32768 rows those orders come from workgroups that read their objective's keys once and sort a share of the order in LDS, without waiting for each other, while shares of 3200 rows need no more workgroups than the device has compute units -- up to 102400 rows of eight objectives; 0 = from the radix sort, whose workgroups wait for each other twelve times), "order_stream_capacity" (default 16384, 1 .. 16384: entries that such a workgroup sorts at once; a larger share is taken in pieces -- tests make it small),
  * "prefix_count_first" (default 1: a selection of such a population whose last two of the same shape on the device found all the rows they keep in front 0 -- told by a word of the pinned host memory of "launch_memory" -- has that kernel count the dominators of every row first and build the matrix, in a second launch, only if front 0 falls short this time; 0 = always both at once).
  * Returns EVOX_HIP_E_BAD_ARG for an unknown name or a value out of range. */

@@ -67,6 +67,13 @@ def test_the_chain_kernel_spills_nothing(kernels):
     assert chain[".max_flat_workgroup_size"] == 1024
 
 
+def test_the_one_workgroup_kernels_spill_nothing(kernels):
+    """Their registers are capped for eight waves per SIMD up to twelve objectives; a path added to them must fit."""
+    small = [k for k in kernels if "batched_kernel" in k[".name"] or "two_small_kernel" in k[".name"]]
+    assert len(small) == 17
+    assert {k[".name"]: k[".private_segment_fixed_size"] for k in small if k[".private_segment_fixed_size"]} == {}
+
+
 def test_every_kernel_is_built_for_wave64(kernels):
     assert len(kernels) > 100
     assert all(k[".wavefront_size"] == 64 for k in kernels)
