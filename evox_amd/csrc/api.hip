@@ -114,7 +114,7 @@ static bool make_layout(int64_t n, int64_t m, Layout* L) {
   L->hist = o;        o = align_up(o + sizeof(int) * (size_t)buckets);
   L->scanflags = o;   o = align_up(o + sizeof(unsigned long long) * 64);
   L->tailbuf = o;     o = align_up(o + (n <= 32768 ? sizeof(unsigned long long) * kTailCopies * kTailRows : 0));
-  L->records = o;     o = align_up(o + (n <= 32768 ? sizeof(unsigned long long) * kLdsPeelRecordUnits : (n <= kRecordsMaxRowsWide ? sizeof(unsigned long long) * kRecRing * kRecUnits : 0)));
+  L->records = o;     o = align_up(o + (n <= 32768 ? sizeof(unsigned long long) * kLdsPeelRecordUnits : (n <= kRecordsMaxRowsWide ? sizeof(unsigned long long) * kRecRing * (n > kRecordsMaxRows ? kRecUnitsWide : kRecUnits) : 0)));
   // the hand-over rings of the two-objective ranking (two.hpp)
   L->two_ring = o;    o = align_up(o + (m == 2 && n <= kTwoMaxRows ? sizeof(unsigned long long) * kTwoRingStride * (size_t)((n + kTwoChunk - 1) / kTwoChunk) : 0));
   L->zero_end = o;

@@ -928,6 +928,11 @@ constexpr int kRecThreads = 512;
 constexpr int kRecUnits = 1024;  // units of one generation = sweepers x units per record
 constexpr int kRecRing = 8;      // == kFrontBuffers: a generation's record slot and bitmap buffer recycle together
 constexpr int kRecLoads = kRecUnits / kRecThreads;
+// Populations of 65 535 rows and more (the wide layout: two slots per unit) have fronts of thousands of rows, and a
+// workgroup whose rows of a front do not fit its record sends everybody to the bitmaps in memory for that pass
+// (200 000 x 3: 2000 rows a front, 128 sweepers with room for 15 each).  Their generations hold four times the
+// units: room for 63 rows per workgroup.
+constexpr int kRecUnitsWide = 4 * kRecUnits;
 constexpr uint32_t kRecOverflowNarrow = 0x8000u;  // in the count field: the rows are in the bitmaps, not in the record
 static_assert(kRecRing == kFrontBuffers, "records and bitmaps are recycled by the same counter");
 
@@ -982,6 +987,7 @@ struct RecFormat {
 // another block has given up.  Only what is still missing is loaded again: a block's uncached loads are
 // served one after the other, so every extra polling load delays the one that matters (two rounds in
 // flight at once, or records four times this size, each cost more than a microsecond per pass).
+template <int kRecLoads>
 __device__ inline bool poll_record_units(const unsigned long long* gen_units, int used_units, unsigned gen,
                                          unsigned long long (&v)[kRecLoads], const int* listed, int listed_needed,
                                          const int* err, unsigned spin_limit) {
@@ -1025,6 +1031,8 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
                                          // of the rows just ranked
   __shared__ int sh[32];
   if (coherent_load(&ctrl->err) != 0) return;
+  constexpr int kRecUnits = WIDE ? evx::kRecUnitsWide : evx::kRecUnits;  // (units of a generation, in this kernel)
+  constexpr int kRecLoads = kRecUnits / kRecThreads;
   int units = 1;  // per record: the largest power of two that gives every sweeper a record
   while (units * 2 * sweepers <= kRecUnits) units *= 2;
   const int tid = threadIdx.x;
@@ -1033,6 +1041,11 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
     // ---- lister
     uint64_t* front_lds = rec_lds;
     int ranked = 0;
+    // The bitmaps of a front in memory are written by the count stage (front 0) and by sweepers whose rows of a front
+    // did not fit their record; nobody else touches them, so those of a front whose records all fitted are still
+    // clear.  (Clearing them whatever they held made the lister the slowest block from 65 535 rows on: two stores
+    // per 128-byte line of two buffers, 17 of its 21 us per front at 200 000 rows, and the sweepers wait for it.)
+    bool prev_written = true;
     for (int level = 0;; ++level) {
       int size = 0;
       if (level == 0) {
@@ -1049,6 +1062,7 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
         __syncthreads();
         size = sh[1];
       } else {
+        EVX_TRACE(level, 0);
         for (int w = tid; w < nwords; w += blockDim.x) front_lds[w] = 0ull;
         if (tid == 0) {
           sh[1] = 0;
@@ -1062,23 +1076,34 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
           coherent_store(&ctrl->err, kErrBarrierTimeout);
           atomicOr(&sh[2], 2);
         } else {
+          // (the original indices of all slots of this thread's units are fetched together: one after the other, with
+          // the addition to the bitmap in between, they were a memory round trip each)
+          constexpr int kFields = RecFormat<WIDE>::kFields;
+          int slots[kRecLoads * kFields];
 #pragma unroll
           for (int k = 0; k < kRecLoads; ++k) {
+#pragma unroll
+            for (int q = 0; q < kFields; ++q) slots[k * kFields + q] = -1;
             if (tid + k * kRecThreads >= sweepers * units) continue;  // past the last record
             const int i = (tid + k * kRecThreads) & (units - 1);
+            int at = 0;
             RecFormat<WIDE>::read(
                 v[k], i == 0,
                 [&](int count, bool overflow) {
                   atomicAdd(&sh[1], count);
                   if (overflow) atomicOr(&sh[2], 1);
                 },
-                [&](int slot) {
-                  const int o = orig_of[slot];
-                  atomicOr(reinterpret_cast<unsigned long long*>(&front_lds[o >> 6]), 1ull << (o & 63));
-                });
+                [&](int slot) { slots[k * kFields + at++] = slot; });
           }
+          int origs[kRecLoads * kFields];
+#pragma unroll
+          for (int e = 0; e < kRecLoads * kFields; ++e) origs[e] = slots[e] >= 0 ? orig_of[slots[e]] : -1;
+#pragma unroll
+          for (int e = 0; e < kRecLoads * kFields; ++e)
+            if (origs[e] >= 0) atomicOr(reinterpret_cast<unsigned long long*>(&front_lds[origs[e] >> 6]), 1ull << (origs[e] & 63));
         }
         __syncthreads();
+        EVX_TRACE(level, 1);
         if (sh[2] & 2) return;
         size = sh[1];
         if (sh[2] & 1) {
@@ -1086,19 +1111,24 @@ __global__ __launch_bounds__(kRecThreads) void peel_records_kernel(
           for (int w = tid; w < nwords; w += blockDim.x) front_lds[w] |= coherent_load(&cur[(int64_t)w * kFrontStride]);
         }
         // every sweeper has published generation `level`, so it has finished with the bitmaps of front level-1
-        uint64_t* prev_slot = fronts_slot + (int64_t)((level - 1) % kFrontBuffers) * nwords * kFrontStride;
-        uint64_t* prev_orig = fronts_orig + (int64_t)((level - 1) % kFrontBuffers) * nwords * kFrontStride;
-        for (int w = tid; w < nwords; w += blockDim.x) {
-          coherent_store(&prev_slot[(int64_t)w * kFrontStride], (uint64_t)0);
-          coherent_store(&prev_orig[(int64_t)w * kFrontStride], (uint64_t)0);
+        if (prev_written) {
+          uint64_t* prev_slot = fronts_slot + (int64_t)((level - 1) % kFrontBuffers) * nwords * kFrontStride;
+          uint64_t* prev_orig = fronts_orig + (int64_t)((level - 1) % kFrontBuffers) * nwords * kFrontStride;
+          for (int w = tid; w < nwords; w += blockDim.x) {
+            coherent_store(&prev_slot[(int64_t)w * kFrontStride], (uint64_t)0);
+            coherent_store(&prev_orig[(int64_t)w * kFrontStride], (uint64_t)0);
+          }
         }
+        prev_written = (sh[2] & 1) != 0;
       }
       __syncthreads();  // also waits for the clearing stores of this block's waves
+      EVX_TRACE(level, 2);
       if (tid == 0) coherent_store(&ctrl->listed, level);  // records <= level consumed, bitmaps < level cleared
       const bool last = size <= 0 || ranked + size >= stop_count;
       // a front 0 that ends the peel is listed by the sweepers together (see peel_kernel)
       const bool shared_listing = level == 0 && last && size > kSharedListingRows;
       if (perm && !shared_listing) list_front(front_lds, nwords, perm, ranked, sh + 8);
+      EVX_TRACE(level, 3);
       if (tid == 0) {
         fstart[level] = ranked;
         if (level > 0) fsize[level] = size;

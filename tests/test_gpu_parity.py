@@ -961,9 +961,46 @@ def test_fronts_of_thousands_of_rows(peel_algorithm):
         assert_dist_close(ds, dist[order], f"big fronts topk {topk}")
 
 
+def test_large_fronts_between_small_ones_above_65534_rows(population_path):
+    """70 000 rows of three objectives in layers that dominate one another: a front of 9000 rows (more than the
+    records of the sweeping workgroups carry: it goes through the bitmaps in memory), then the thin fronts of 15 000
+    uniform rows (records only: their bitmaps are never written and are not cleared either), a front of 12 000, thin
+    fronts again, and so on.  Ranks and the selection against the plain-C checker."""
+    if population_path != "pipeline":
+        pytest.skip("single large populations always take the pipeline")
+    from oracle import c_oracle
+
+    say("large_and_small_fronts")
+    g = torch.Generator("cpu").manual_seed(4242)
+
+    def simplex(rows):
+        u = torch.rand(rows, 3, generator=g)
+        return u / u.sum(dim=1, keepdim=True)
+
+    parts = [simplex(9000), 2.0 + torch.rand(15000, 3, generator=g), 10.0 + simplex(12000), 20.0 + torch.rand(14000, 3, generator=g),
+             30.0 + simplex(8500), 40.0 + torch.rand(11500, 3, generator=g)]
+    f = torch.cat(parts)[torch.randperm(70000, generator=g)].contiguous()
+    n = f.size(0)
+    want_rank, fronts = c_oracle.nd_rank(as_np(f))
+    assert fronts > 40
+    fd = f.to(DEV)
+    assert np.array_equal(as_np(non_dominate_rank(fd)), want_rank)
+    st = runtime.last_status()
+    assert st["error"] == 0 and st["fronts"] == fronts
+    x = torch.arange(n, dtype=torch.int32, device=DEV)[:, None]
+    for topk in (30000, 69000):
+        order, rank, dist, _ = c_oracle.select(as_np(f), topk)
+        xs, fs, rs, ds = nd_environmental_selection(x, fd, topk)
+        assert runtime.last_status()["error"] == 0
+        assert np.array_equal(as_np(xs)[:, 0].astype(np.int64), order), topk
+        assert np.array_equal(as_np(rs), rank[order])
+        assert_dist_close(ds, dist[order], f"large and small fronts topk {topk}")
+    runtime.release_workspaces()
+
+
 def test_rank_at_the_protocol_boundary(population_path):
-    """65534 rows is the largest population that the record protocol peels (16-bit slots), 65535 the first
-    one that goes to the master protocol: both against the plain-C checker."""
+    """65534 rows is the largest population whose records hold three 16-bit slots a unit, 65535 the first one with
+    two 24-bit slots: both against the plain-C checker."""
     if population_path != "pipeline":
         pytest.skip("single large populations always take the pipeline")
     from oracle import c_oracle
