@@ -187,10 +187,13 @@ __device__ inline void two_small_pass(const uint32_t* key_in, const uint16_t* pa
   EVX_PASS_TRACE(9);
 }
 
-// `passes` passes from the lowest digit up (1 .. 4); returns through the references where the result lies.
+// `passes` passes from the lowest digit up (1 .. 4); returns through the references where the result lies.  vary: the
+// bits in which any two keys differ (or more bits); a digit in which no two keys differ needs no pass -- objectives
+// that take few values, such as counts or multiples of a step, leave the low bits of their float32 images alike.
 __device__ inline void two_small_sort(uint32_t*& key_a, uint16_t*& pay_a, uint32_t*& key_b, uint16_t*& pay_b, int count, int passes,
-                                      uint32_t* cnt, uint32_t* part, uint32_t* lanes_a) {
+                                      uint32_t* cnt, uint32_t* part, uint32_t* lanes_a, uint32_t vary = 0xFFFFFFFFu) {
   for (int p = 0; p < passes; ++p) {
+    if (((vary >> (8 * p)) & 255u) == 0u) continue;  // (the same in every thread)
     two_small_pass(key_a, pay_a, key_b, pay_b, count, 8 * p, cnt, part, lanes_a);
     uint32_t* tk = key_a;
     key_a = key_b;
@@ -207,6 +210,7 @@ __global__ __launch_bounds__(kTwoSmallThreads) void two_small_kernel(BatchedArgs
   __shared__ __attribute__((aligned(16))) uint32_t wave_min[2][16];
   __shared__ __attribute__((aligned(16))) uint32_t part[16];
   __shared__ uint32_t round_count[3];
+  __shared__ uint32_t vary_bits[2];  // bits in which the keys of f1 / of f2 differ from those of row 0
   __shared__ __attribute__((aligned(16))) uint32_t wave_first[16];
   uint32_t* key_a = reinterpret_cast<uint32_t*>(two_small_lds);
   uint32_t* key_b = key_a + kTwoSmallRows;
@@ -241,20 +245,43 @@ __global__ __launch_bounds__(kTwoSmallThreads) void two_small_kernel(BatchedArgs
     for (int i = tid; i < 2 * kTwoSmallRows / 4; i += kTwoSmallThreads)
       reinterpret_cast<uint4*>(seen)[i] = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty);
     int nan_f1 = 0;
-    uint32_t mine1[kTwoSmallPer];
+    uint32_t mine1[kTwoSmallPer], mine2[kTwoSmallPer];
+    if (tid < 2) vary_bits[tid] = 0u;
 #pragma unroll
     for (int r = 0; r < kTwoSmallPer; ++r) {
       const int i = tid + kTwoSmallThreads * r;
       mine1[r] = kEmpty;
+      mine2[r] = kEmpty;
       if (i < n) {
         const uint32_t a1 = ordered_key(fitness_at(i, 0)), a2 = ordered_key(fitness_at(i, 1));
         k1[i] = a1;
         k2[i] = a2;
         mine1[r] = a1;
+        mine2[r] = a2;
         nan_f1 += a1 == kEmpty ? 1 : 0;  // (the key of a NaN is the table's mark for a free word: counted instead)
       }
     }
     __syncthreads();
+    {
+      const uint32_t ref1 = k1[0], ref2 = k2[0];
+      uint32_t v1 = 0u, v2 = 0u;
+#pragma unroll
+      for (int r = 0; r < kTwoSmallPer; ++r) {
+        if (tid + kTwoSmallThreads * r < n) {
+          v1 |= mine1[r] ^ ref1;
+          v2 |= mine2[r] ^ ref2;
+        }
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        v1 |= (uint32_t)__shfl_xor((int)v1, off);
+        v2 |= (uint32_t)__shfl_xor((int)v2, off);
+      }
+      if (lane == 0) {
+        if (v1) atomicOr(&vary_bits[0], v1);
+        if (v2) atomicOr(&vary_bits[1], v2);
+      }
+    }
 #pragma unroll
     for (int r = 0; r < kTwoSmallPer; ++r) {
       if (mine1[r] == kEmpty) continue;
@@ -280,12 +307,12 @@ __global__ __launch_bounds__(kTwoSmallThreads) void two_small_kernel(BatchedArgs
   }
   __syncthreads();
   EVX_BATCH_TRACE(1);
-  two_small_sort(key_a, pay_a, key_b, pay_b, n, 4, cnt, part, lanes_a);
+  two_small_sort(key_a, pay_a, key_b, pay_b, n, 4, cnt, part, lanes_a, vary_bits[twin ? 1 : 0]);
   EVX_BATCH_TRACE(2);
   if (twin) {
     for (int s = tid; s < n; s += kTwoSmallThreads) key_a[s] = k1[pay_a[s]];
     __syncthreads();
-    two_small_sort(key_a, pay_a, key_b, pay_b, n, 4, cnt, part, lanes_a);
+    two_small_sort(key_a, pay_a, key_b, pay_b, n, 4, cnt, part, lanes_a, vary_bits[0]);
   }
   for (int s = tid; s < n; s += kTwoSmallThreads) lexi[s] = pay_a[s];
   __syncthreads();
