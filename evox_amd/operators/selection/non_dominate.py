@@ -12,6 +12,22 @@ import torch
 
 from ... import ops
 
+_functorch_level = torch._C._functorch.maybe_current_level
+_is_compiling = torch.compiler.is_compiling
+
+
+def _plain(op, *tensors):
+    """``op`` itself, or -- for plain tensors outside ``torch.compile`` and ``vmap`` / ``grad`` transforms -- the
+    function that the custom operator wraps: what the operator would run after four layers of dispatch, a fifth
+    of the time of a selection of 200 rows.  Tensor subclasses (fake tensors, functional wrappers) and tensors that
+    require a gradient keep to the operator."""
+    for t in tensors:
+        if type(t) is not torch.Tensor or t.requires_grad:
+            return op
+    if _is_compiling() or _functorch_level() is not None:
+        return op
+    return op._init_fn
+
 
 def non_dominate_rank(x: torch.Tensor) -> torch.Tensor:
     """Non-domination rank of every row of ``x`` (minimisation).
@@ -23,7 +39,7 @@ def non_dominate_rank(x: torch.Tensor) -> torch.Tensor:
     accepted, as in the reference: float32 (and float16 / bfloat16, widened exactly) goes to the kernels
     as it is, other dtypes through per-objective dense ranks, which keep every comparison.
     """
-    return ops.nd_rank(x)
+    return _plain(ops.nd_rank, x)(x)
 
 
 def non_dominate_rank_until(x: torch.Tensor, count: int) -> torch.Tensor:
@@ -86,7 +102,7 @@ def nd_environmental_selection(x: torch.Tensor, f: torch.Tensor, topk: int) -> T
         )
     if f.dtype == torch.float64 or not (f.is_floating_point() or f.is_complex() or f.dtype == torch.bool):
         return ops.nd_select_wide(x, f, int(topk))
-    return ops.nd_select(x, f, int(topk))
+    return _plain(ops.nd_select, x, f)(x, f, int(topk))
 
 
 def nd_environmental_selection_two_part(
@@ -103,4 +119,4 @@ def nd_environmental_selection_two_part(
     narrow = (torch.float32, torch.float16, torch.bfloat16)
     if f_a.dtype != f_b.dtype or f_a.dtype not in narrow or x_a.dtype != x_b.dtype:
         return nd_environmental_selection(torch.cat([x_a, x_b], dim=0), torch.cat([f_a, f_b], dim=0), int(topk))
-    return ops.nd_select_two_part(x_a, f_a, x_b, f_b, int(topk))
+    return _plain(ops.nd_select_two_part, x_a, f_a, x_b, f_b)(x_a, f_a, x_b, f_b, int(topk))

@@ -70,7 +70,14 @@ def require_gpu_tensor(t: torch.Tensor, what: str) -> None:
         )
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_handle(device: torch.device) -> int:
+    """The hipStream_t of torch's current stream on ``device`` (asked of torch directly where it offers that: the
+    Stream object costs 1.5 us more to build)."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return int(torch.cuda.current_stream(device).cuda_stream)
 
 
