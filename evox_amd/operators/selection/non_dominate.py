@@ -12,21 +12,16 @@ import torch
 
 from ... import ops
 
-_functorch_level = torch._C._functorch.maybe_current_level
-_is_compiling = torch.compiler.is_compiling
-
 
 def _plain(op, *tensors):
-    """``op`` itself, or -- for plain tensors outside ``torch.compile`` and ``vmap`` / ``grad`` transforms -- the
-    function that the custom operator wraps: what the operator would run after four layers of dispatch, a fifth
-    of the time of a selection of 200 rows.  Tensor subclasses (fake tensors, functional wrappers) and tensors that
-    require a gradient keep to the operator."""
+    """``op`` itself, or -- for plain tensors with no transform, tracer or dispatch mode looking at the call
+    (``ops.plain_eager``) -- the function that the custom operator wraps: what the operator would run after four
+    layers of dispatch, a fifth of the time of a selection of 200 rows.  Tensor subclasses (fake tensors, functional
+    wrappers) and tensors that require a gradient keep to the operator."""
     for t in tensors:
         if type(t) is not torch.Tensor or t.requires_grad:
             return op
-    if _is_compiling() or _functorch_level() is not None:
-        return op
-    return op._init_fn
+    return op._init_fn if ops.plain_eager() else op
 
 
 def non_dominate_rank(x: torch.Tensor) -> torch.Tensor:
@@ -52,7 +47,7 @@ def non_dominate_rank_until(x: torch.Tensor, count: int) -> torch.Tensor:
     (src/evox/algorithms/mo/hype.py:135-138) -- which read the same ``worst`` and ``keep`` from the
     truncated ranks without the fronts behind the cut ever being peeled.
     """
-    return ops.nd_rank_until(x, int(count))
+    return _plain(ops.nd_rank_until, x)(x, int(count))
 
 
 def non_dominated_mask(x: torch.Tensor) -> torch.Tensor:
@@ -63,7 +58,7 @@ def non_dominated_mask(x: torch.Tensor) -> torch.Tensor:
     history only to keep the rows of rank 0.  No dominance matrix is built, so memory stays linear in
     ``N`` and a history of millions of rows can be filtered.
     """
-    return ops.nd_first_front(x)
+    return _plain(ops.nd_first_front, x)(x)
 
 
 def crowding_distance(costs: torch.Tensor, mask: Optional[torch.Tensor]) -> torch.Tensor:
@@ -83,7 +78,7 @@ def crowding_distance(costs: torch.Tensor, mask: Optional[torch.Tensor]) -> torc
         )
     if costs.dtype == torch.float64 or not costs.is_floating_point():
         return ops.crowding_wide(costs, mask)
-    return ops.crowding(costs, mask)
+    return _plain(ops.crowding, costs, *(() if mask is None else (mask,)))(costs, mask)
 
 
 def nd_environmental_selection(x: torch.Tensor, f: torch.Tensor, topk: int) -> Tuple[torch.Tensor, ...]:
