@@ -21,7 +21,7 @@ def _plain(op, *tensors):
     for t in tensors:
         if type(t) is not torch.Tensor or t.requires_grad:
             return op
-    return op._init_fn if ops.plain_eager() else op
+    return getattr(op, "_init_fn", op) if ops.plain_eager() else op  # (another torch may not keep it there: the operator then)
 
 
 def non_dominate_rank(x: torch.Tensor) -> torch.Tensor:
